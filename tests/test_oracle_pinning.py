@@ -1,0 +1,426 @@
+"""Pins the CPU oracle against independent facts (library routines, closed forms,
+autograd of the textbook expressions, brute force) before anything is compared
+with it.  The reference holds no golden vectors for this path."""
+import math
+import zlib
+
+import numpy as np
+import pytest
+import scipy.special as sp
+import torch
+
+from oracle import oracle as orc
+
+RNG = np.random.default_rng(7)
+
+
+def _seed(*parts):
+    return zlib.crc32(repr(parts).encode())
+
+
+# ---------------------------------------------------------------- special functions
+
+def test_digamma_trigamma_lgamma_against_scipy():
+    x = np.concatenate([RNG.uniform(0.05, 12.0, 4000), RNG.uniform(12.0, 500.0, 500),
+                        [0.05, 0.5, 1.0, 2.0, 9.999, 10.0, 10.001, 1e6]])
+    assert np.allclose(orc.special("digamma", x), sp.digamma(x), rtol=1e-12, atol=1e-12)
+    # the reference's trigamma series (6 recurrence steps + 4-term tail) is itself only 1e-8 accurate
+    assert np.allclose(orc.special("trigamma", x), sp.polygamma(1, x), rtol=2e-8, atol=0)
+    assert np.allclose(orc.special("lgamma", x), sp.gammaln(x), rtol=1e-13, atol=1e-13)
+
+
+def test_special_known_values_and_recurrences():
+    assert abs(orc.special("digamma", [1.0])[0] + np.euler_gamma) < 1e-14
+    assert abs(orc.special("digamma", [10.0])[0] - 2.2517525890667211) < 1e-15
+    assert abs(orc.special("trigamma", [1.0])[0] - math.pi ** 2 / 6) < 1e-8
+    x = RNG.uniform(0.05, 30.0, 1000)
+    assert np.allclose(orc.special("digamma", x + 1) - orc.special("digamma", x), 1 / x, rtol=0, atol=1e-12)
+    assert np.allclose(orc.special("trigamma", x + 1) - orc.special("trigamma", x), -1 / x ** 2, rtol=1e-7, atol=1e-9)
+    n = np.arange(1, 20, dtype=np.float64)
+    assert np.allclose(orc.special("lgamma", n), [math.log(math.factorial(int(k) - 1)) for k in n], atol=1e-12)
+    # negative arguments: reflection branch of the reference series
+    xn = np.array([-0.5, -1.5, -2.25, 0.25, 0.4])
+    assert np.allclose(orc.special("digamma", xn), sp.digamma(xn), rtol=1e-12)
+    assert np.allclose(orc.special("trigamma", xn),
+                       torch.polygamma(1, torch.tensor(xn, dtype=torch.float64)).numpy(), rtol=1e-7)
+    assert np.isinf(orc.special("digamma", [0.0])[0]) and np.isnan(orc.special("digamma", [-2.0])[0])
+
+
+def test_f32_special_close_to_f64():
+    x = RNG.uniform(0.05, 40.0, 2000)
+    for name, tol in (("digamma", 3e-6), ("trigamma", 3e-6), ("lgamma", 3e-6)):
+        a = orc.special(name, x.astype(np.float32), np.float32).astype(np.float64)
+        b = orc.special(name, x.astype(np.float32).astype(np.float64))
+        assert np.all(np.abs(a - b) <= tol * np.maximum(1.0, np.abs(b))), name
+
+
+# ---------------------------------------------------------------- forward closed forms
+
+def _halves(e):
+    d = e.shape[-1] // 2
+    return e[..., :d], e[..., d:]
+
+
+def closed_form(kind, e, q1, q2):
+    """Textbook expressions with numpy broadcasting on [be,ne,De] x [bc,nc,D]."""
+    if kind == "l1":
+        return np.abs(e - q1).sum(-1)
+    if kind == "l2":
+        return ((e - q1) ** 2).sum(-1)
+    if kind == "box_out":
+        return np.maximum(np.abs(e - q1) - q2, 0).sum(-1)
+    if kind == "box_in":
+        return np.abs(np.minimum(np.abs(e - q1), q2)).sum(-1)
+    if kind == "rotate":
+        a, b = _halves(e)
+        return np.sqrt((a - q1) ** 2 + (b - q2) ** 2 + 1e-20).sum(-1)
+    if kind == "complex":
+        a, b = _halves(e)
+        return (a * q1 + b * q2).sum(-1)
+    if kind == "distmult":
+        return (e * q1).sum(-1)
+    if kind == "beta_l2":
+        a, b = _halves(e)
+        return 0.5 * ((a - q1) ** 2 + (b - q2) ** 2).sum(-1)
+    if kind == "beta_kl":
+        a, b = _halves(e)
+        sp_, sq = a + b, q1 + q2
+        t = (sp.gammaln(q1) + sp.gammaln(q2) + sp.gammaln(sp_) - sp.gammaln(a) - sp.gammaln(b) - sp.gammaln(sq)
+             + (a - q1) * sp.digamma(a) + (b - q2) * sp.digamma(b) + (sq - sp_) * sp.digamma(sp_))
+        return t.sum(-1)
+    if kind == "beta_fisher_approx":
+        a, b = _halves(e)
+        ta, tb, tab = sp.polygamma(1, a), sp.polygamma(1, b), -sp.polygamma(1, a + b)
+        da, db = a - q1, b - q2
+        return 0.5 * ((ta + tab) * da ** 2 + 2 * tab * da * db + (tb + tab) * db ** 2).sum(-1)
+    raise KeyError(kind)
+
+
+def make_inputs(kind, be, ne, bc, nc, dim, rng, positive=False):
+    mul = 2 if kind in orc.TWO_HALVES else 1
+    if kind.startswith("beta"):
+        f = lambda *s: np.clip(1 + np.where((x := rng.standard_normal(s)) > 0, x, np.expm1(x)), 0.05, 1e9)
+    else:
+        f = lambda *s: rng.standard_normal(s)
+    e = f(be, ne, dim * mul)
+    q1 = f(bc, nc, dim)
+    q2 = None if kind in orc.ONE_QUERY else f(bc, nc, dim)
+    if kind.startswith("box") and positive:
+        q2 = np.abs(q2)
+    return e, q1, q2
+
+
+LAYOUTS = [  # (be, ne, bc, nc): every caller situation the operator must accept
+    (6, 5, 6, 1),   # per-query negatives
+    (1, 7, 4, 1),   # shared negatives
+    (5, 1, 5, 1),   # positives
+    (1, 9, 1, 1),   # eval against all entities
+    (4, 1, 4, 6),   # reverse queries (ne=1 < nc)
+    (6, 1, 1, 5),   # the reference's smoke-test layout
+    (6, 4, 3, 2),   # both sides broadcast by modulo
+]
+
+
+@pytest.mark.parametrize("kind", list(orc.KINDS))
+@pytest.mark.parametrize("layout", LAYOUTS)
+def test_forward_matches_closed_form(kind, layout):
+    be, ne, bc, nc = layout
+    rng = np.random.default_rng(_seed(kind, layout))
+    e, q1, q2 = make_inputs(kind, be, ne, bc, nc, 11, rng)
+    got = orc.dist_forward(kind, e, q1, q2)
+    bsize, num = max(be, bc), max(ne, nc)
+    # modulo broadcast rule of the launch loop, spelled out by brute force
+    ii, jj = np.meshgrid(np.arange(bsize), np.arange(num), indexing="ij")
+    eb = e[ii % be, jj % ne]
+    q1b = q1[ii % bc, jj % nc]
+    q2b = None if q2 is None else q2[ii % bc, jj % nc]
+    want = closed_form(kind, eb, q1b, q2b)
+    tol = 3e-8 if "fisher" in kind else 1e-11
+    assert np.allclose(got, want, rtol=tol, atol=tol)
+
+
+def test_beta_kl_is_torch_kl_beta_beta():
+    rng = np.random.default_rng(3)
+    e, q1, q2 = make_inputs("beta_kl", 8, 6, 8, 1, 16, rng)
+    from torch.distributions import Beta
+    from torch.distributions.kl import _kl_beta_beta
+    a, b = _halves(torch.from_numpy(e))
+    kl = _kl_beta_beta(Beta(a, b), Beta(torch.from_numpy(q1), torch.from_numpy(q2))).sum(-1).numpy()
+    assert np.allclose(orc.dist_forward("beta_kl", e, q1, q2), kl, rtol=1e-11, atol=1e-11)
+    assert np.all(kl > -1e-9)
+
+
+# ---------------------------------------------------------------- backward
+
+def torch_form(kind, e, q1, q2):
+    if kind == "l1":
+        return (e - q1).abs().sum(-1)
+    if kind == "l2":
+        return ((e - q1) ** 2).sum(-1)
+    if kind == "box_out":
+        return torch.relu((e - q1).abs() - q2).sum(-1)
+    if kind == "box_in":
+        return torch.minimum((e - q1).abs(), q2).abs().sum(-1)
+    a, b = torch.chunk(e, 2, dim=-1) if kind in orc.TWO_HALVES else (e, None)
+    if kind == "rotate":
+        return torch.sqrt((a - q1) ** 2 + (b - q2) ** 2 + 1e-20).sum(-1)
+    if kind == "complex":
+        return (a * q1 + b * q2).sum(-1)
+    if kind == "distmult":
+        return (e * q1).sum(-1)
+    if kind == "beta_l2":
+        return 0.5 * ((a - q1) ** 2 + (b - q2) ** 2).sum(-1)
+    if kind == "beta_kl":
+        sp_, sq = a + b, q1 + q2
+        return (torch.lgamma(q1) + torch.lgamma(q2) + torch.lgamma(sp_) - torch.lgamma(a) - torch.lgamma(b)
+                - torch.lgamma(sq) + (a - q1) * torch.digamma(a) + (b - q2) * torch.digamma(b)
+                + (sq - sp_) * torch.digamma(sp_)).sum(-1)
+    if kind == "beta_fisher_approx":
+        with torch.no_grad():  # the reference treats the trigamma weights as constants
+            ta, tb, tab = a.polygamma(1), b.polygamma(1), -(a + b).polygamma(1)
+        da, db = a - q1, b - q2
+        return 0.5 * ((ta + tab) * da ** 2 + 2 * tab * da * db + (tb + tab) * db ** 2).sum(-1)
+    raise KeyError(kind)
+
+
+@pytest.mark.parametrize("kind", list(orc.KINDS))
+@pytest.mark.parametrize("layout", LAYOUTS)
+def test_backward_matches_autograd(kind, layout):
+    be, ne, bc, nc = layout
+    rng = np.random.default_rng(_seed("b", kind, layout))
+    e, q1, q2 = make_inputs(kind, be, ne, bc, nc, 9, rng)
+    bsize, num = max(be, bc), max(ne, nc)
+    gout = rng.standard_normal((bsize, num))
+    te = torch.tensor(e, requires_grad=True)
+    t1 = torch.tensor(q1, requires_grad=True)
+    t2 = None if q2 is None else torch.tensor(q2, requires_grad=True)
+    ii, jj = torch.meshgrid(torch.arange(bsize), torch.arange(num), indexing="ij")
+    out = torch_form(kind, te[ii % be, jj % ne], t1[ii % bc, jj % nc], None if t2 is None else t2[ii % bc, jj % nc])
+    (out * torch.from_numpy(gout)).sum().backward()
+    gent, gq1, gq2 = orc.dist_backward(kind, gout, e, q1, q2)
+    tol = 3e-7 if kind.startswith("beta") else 1e-10
+    assert np.allclose(gent, te.grad.numpy(), rtol=tol, atol=tol)
+    assert np.allclose(gq1, t1.grad.numpy(), rtol=tol, atol=tol)
+    if q2 is not None:
+        assert np.allclose(gq2, t2.grad.numpy(), rtol=tol, atol=tol)
+
+
+@pytest.mark.parametrize("kind", ["l2", "rotate", "beta_kl", "box_out", "box_in"])
+def test_backward_matches_finite_differences(kind):
+    rng = np.random.default_rng(11)
+    e, q1, q2 = make_inputs(kind, 3, 2, 3, 1, 5, rng, positive=True)
+    gout = rng.standard_normal((3, 2))
+    gent, gq1, gq2 = orc.dist_backward(kind, gout, e, q1, q2)
+    h = 1e-6
+
+    def loss(e_, a_, b_):
+        return float((orc.dist_forward(kind, e_, a_, b_) * gout).sum())
+
+    for arr, grad in ((e, gent), (q1, gq1), (q2, gq2)):
+        if arr is None:
+            continue
+        flat = arr.reshape(-1)
+        for k in rng.choice(flat.size, size=min(12, flat.size), replace=False):
+            old = flat[k]
+            flat[k] = old + h
+            up = loss(e, q1, q2)
+            flat[k] = old - h
+            dn = loss(e, q1, q2)
+            flat[k] = old
+            assert abs((up - dn) / (2 * h) - grad.reshape(-1)[k]) < 2e-5
+
+
+def test_tie_conventions_follow_the_kernel():
+    one = lambda *v: np.array(v, dtype=np.float64).reshape(1, 1, -1)
+    g = np.array([[2.0]])
+    # l1 at e == c: sign(0) = -1
+    gent, gq, _ = orc.dist_backward("l1", g, one(0.5), one(0.5))
+    assert gent.item() == -2.0 and gq.item() == 2.0
+    # box_out at |e-c| - o == 0 passes gradient (>=); e-c = 0.25 > 0
+    gent, gc, go = orc.dist_backward("box_out", g, one(1.0), one(0.75), one(0.25))
+    assert (gent.item(), gc.item(), go.item()) == (2.0, -2.0, -2.0)
+    # box_out inside the box: no gradient at all
+    gent, gc, go = orc.dist_backward("box_out", g, one(1.0), one(0.75), one(0.5))
+    assert (gent.item(), gc.item(), go.item()) == (0.0, 0.0, 0.0)
+    # box_out with e == c and o == 0: relu argument is 0 -> passes, sign(0) = -1
+    gent, gc, go = orc.dist_backward("box_out", g, one(1.0), one(1.0), one(0.0))
+    assert (gent.item(), gc.item(), go.item()) == (-2.0, 2.0, -2.0)
+    # box_in tie |e-c| == o goes to the offset branch
+    gent, gc, go = orc.dist_backward("box_in", g, one(1.0), one(0.75), one(0.25))
+    assert (gent.item(), gc.item(), go.item()) == (0.0, 0.0, 2.0)
+    # box_in inside: gradient to entity / center with inner sign
+    gent, gc, go = orc.dist_backward("box_in", g, one(0.5), one(0.75), one(0.5))
+    assert (gent.item(), gc.item(), go.item()) == (-2.0, 2.0, 0.0)
+    # box_in with negative offset: min(...) <= 0 -> outer sign -1, offset branch
+    gent, gc, go = orc.dist_backward("box_in", g, one(1.0), one(0.75), one(-0.5))
+    assert (gent.item(), gc.item(), go.item()) == (0.0, 0.0, -2.0)
+    assert orc.dist_forward("box_in", one(1.0), one(0.75), one(-0.5)).item() == 0.5
+    # box_in with e == c (min = 0 -> outer sign -1, inner sign(0) = -1)
+    gent, gc, go = orc.dist_backward("box_in", g, one(1.0), one(1.0), one(0.5))
+    assert (gent.item(), gc.item(), go.item()) == (2.0, -2.0, 0.0)
+    # rotate at zero distance: eps inside the root keeps everything finite and zero
+    gent, gr, gi = orc.dist_backward("rotate", g, one(0.3, 0.4), one(0.3), one(0.4))
+    assert np.all(gent == 0) and gr.item() == 0 and gi.item() == 0
+    assert abs(orc.dist_forward("rotate", one(0.3, 0.4), one(0.3), one(0.4)).item() - 1e-10) < 1e-16
+
+
+# ---------------------------------------------------------------- gather / merge / Adam
+
+def test_gather_and_regularizer():
+    t = RNG.standard_normal((50, 6))
+    idx = RNG.integers(0, 50, size=(7, 5))
+    assert np.array_equal(orc.gather(t, idx), t[idx.reshape(-1)])
+    with pytest.raises(IndexError):
+        orc.gather(t, np.array([50]))
+    with pytest.raises(IndexError):
+        orc.gather(t, np.array([-1]))
+    x = RNG.standard_normal(100) * 3
+    assert np.array_equal(orc.regularizer(x), np.clip(x + 1, 0.05, 1e9))
+
+
+@pytest.mark.parametrize("p,n", [(1, 5), (64, 4), (1000, 50), (1000, 10 ** 9), (17, 1)])
+def test_merge_indices_is_numpy_unique(p, n):
+    idx = RNG.integers(0, n, size=p)
+    uniq, inverse, order, seg = orc.merge_indices(idx)
+    u2, inv2 = np.unique(idx, return_inverse=True)
+    assert np.array_equal(uniq, u2) and np.array_equal(inverse, inv2)
+    assert np.array_equal(order, np.argsort(idx, kind="stable"))
+    assert seg[0] == 0 and seg[-1] == p and np.all(np.diff(seg) > 0)
+    assert np.array_equal(np.diff(seg), np.bincount(inv2))
+    assert np.all(np.diff(uniq) > 0)
+
+
+def test_merge_indices_empty():
+    uniq, inverse, order, seg = orc.merge_indices(np.zeros(0, dtype=np.int64))
+    assert uniq.size == 0 and seg.tolist() == [0]
+
+
+def test_merge_grads_is_add_at():
+    idx = RNG.integers(0, 30, size=400)
+    g = RNG.standard_normal((400, 7))
+    uniq, inverse, _, _ = orc.merge_indices(idx)
+    want = np.zeros((uniq.size, 7))
+    np.add.at(want, inverse, g)
+    assert np.allclose(orc.merge_grads(g, inverse, uniq.size), want, rtol=1e-13, atol=1e-13)
+
+
+def test_adam_equals_torch_adam_when_every_row_is_touched():
+    n, d, lr = 12, 5, 1e-2
+    w0 = RNG.standard_normal((n, d))
+    w, m, v = w0.copy(), np.zeros((n, d)), np.zeros((n, d))
+    tw = torch.tensor(w0.copy(), requires_grad=True)
+    opt = torch.optim.Adam([tw], lr=lr, betas=(0.9, 0.999), eps=1e-8)
+    for step in range(1, 6):
+        g = RNG.standard_normal((n, d))
+        perm = RNG.permutation(n)
+        orc.adam_rows(w, m, v, np.sort(perm), g, lr, step)
+        tw.grad = torch.tensor(g)
+        opt.step()
+        assert np.allclose(w, tw.detach().numpy(), rtol=1e-12, atol=1e-12)
+    st = opt.state[tw]
+    assert np.allclose(m, st["exp_avg"].numpy(), rtol=1e-12)
+    assert np.allclose(v, st["exp_avg_sq"].numpy(), rtol=1e-12)
+
+
+def test_adam_is_lazy_and_uses_the_global_step():
+    n, d, lr = 10, 4, 1e-3
+    w = RNG.standard_normal((n, d))
+    m, v = np.zeros((n, d)), np.zeros((n, d))
+    w0 = w.copy()
+    g = RNG.standard_normal((2, d))
+    # first touch happens at global step 3: bias correction uses t = 3, not 1
+    orc.adam_rows(w, m, v, np.array([2, 7]), g, lr, step=3)
+    untouched = [r for r in range(n) if r not in (2, 7)]
+    assert np.array_equal(w[untouched], w0[untouched])
+    assert not m[untouched].any() and not v[untouched].any()
+    m1, v1 = 0.1 * g, 0.001 * g * g
+    denom = np.sqrt(v1) / math.sqrt(1 - 0.999 ** 3) + 1e-8
+    want = w0[[2, 7]] - lr / (1 - 0.9 ** 3) * m1 / denom
+    assert np.allclose(w[[2, 7]], want, rtol=1e-13)
+    assert np.allclose(m[[2, 7]], m1, rtol=1e-13) and np.allclose(v[[2, 7]], v1, rtol=1e-13)
+    # a touched row with an exactly zero gradient still moves by momentum
+    wb = w.copy()
+    orc.adam_rows(w, m, v, np.array([2]), np.zeros((1, d)), lr, step=4)
+    assert np.all(w[2] != wb[2]) and np.array_equal(w[7], wb[7])
+
+
+def test_adam_squeeze_variant_closed_form():
+    n, d, lr = 6, 8, 1e-3
+    w = RNG.standard_normal((n, d))
+    m, v = np.zeros((n, d)), np.full((n, 1), 0.25)
+    w0 = w.copy()
+    g = RNG.standard_normal((1, d))
+    orc.adam_rows(w, m, v, np.array([4]), g, lr, step=2, squeeze=True)
+    v1 = 0.999 * 0.25 + 0.001 * np.mean(g * g)
+    assert abs(v[4, 0] - v1) < 1e-15 and np.all(v[[0, 1, 2, 3, 5]] == 0.25)
+    want = w0[4] - lr / (1 - 0.9 ** 2) * (0.1 * g[0]) / (math.sqrt(v1) / math.sqrt(1 - 0.999 ** 2) + 1e-8)
+    assert np.allclose(w[4], want, rtol=1e-13)
+
+
+# ---------------------------------------------------------------- composition
+
+def test_scores_match_native_cal_logit_forms():
+    rng = np.random.default_rng(5)
+    b, k, d = 4, 6, 10
+    rows = rng.standard_normal((b, k, d))
+    c, o = rng.standard_normal((b, 1, d)), np.abs(rng.standard_normal((b, 1, d)))
+    delta = np.abs(rows - c)
+    want = 24 - np.maximum(delta - o, 0).sum(-1) - 0.02 * np.minimum(delta, o).sum(-1)
+    assert np.allclose(orc.score_forward("box", rows, c, o, 24.0, 0.02), want, rtol=1e-12)
+    assert np.allclose(orc.score_forward("l2", rows, c, None, 12.0), 12 - np.linalg.norm(rows - c, axis=-1), rtol=1e-12)
+    assert np.allclose(orc.score_forward("l1", rows, c, None, 12.0), 12 - np.abs(rows - c).sum(-1), rtol=1e-12)
+    rows2 = rng.standard_normal((b, k, 2 * d))
+    re, im = rng.standard_normal((b, 1, d)), rng.standard_normal((b, 1, d))
+    want = 9 - np.sqrt((rows2[..., :d] - re) ** 2 + (rows2[..., d:] - im) ** 2).sum(-1)
+    assert np.allclose(orc.score_forward("rotate", rows2, re, im, 9.0), want, rtol=1e-12)
+
+
+def test_score_backward_matches_autograd_l2_and_box():
+    rng = np.random.default_rng(6)
+    b, k, d = 3, 5, 7
+    rows = rng.standard_normal((b, k, d))
+    c, o = rng.standard_normal((b, 1, d)), np.abs(rng.standard_normal((b, 1, d)))
+    gs = rng.standard_normal((b, k))
+    tr, tc, to = (torch.tensor(x, requires_grad=True) for x in (rows, c, o))
+    s = 12 - torch.linalg.norm(tr - tc, dim=-1)
+    (s * torch.from_numpy(gs)).sum().backward()
+    gr, gc, _ = orc.score_backward("l2", gs, rows, c)
+    assert np.allclose(gr, tr.grad.numpy(), rtol=1e-11) and np.allclose(gc, tc.grad.numpy(), rtol=1e-11)
+    tr.grad = tc.grad = None
+    delta = (tr - tc).abs()
+    s = 24 - torch.relu(delta - to).sum(-1) - 0.02 * torch.minimum(delta, to).sum(-1)
+    (s * torch.from_numpy(gs)).sum().backward()
+    gr, gc, go = orc.score_backward("box", gs, rows, c, o, cen=0.02)
+    assert np.allclose(gr, tr.grad.numpy(), rtol=1e-11, atol=1e-14)
+    assert np.allclose(gc, tc.grad.numpy(), rtol=1e-11, atol=1e-14)
+    assert np.allclose(go, to.grad.numpy(), rtol=1e-11, atol=1e-14)
+
+
+def test_train_step_equals_dense_autograd_pipeline():
+    """gather -> score -> backward -> merge -> Adam equals autograd through table[idx]
+    followed by a dense Adam restricted to the touched rows."""
+    rng = np.random.default_rng(8)
+    n, d, b, k = 40, 6, 5, 9
+    table = rng.uniform(-0.07, 0.07, (n, d))
+    m, v = np.zeros((n, d)), np.zeros((n, d))
+    c, o = rng.uniform(-0.07, 0.07, (b, 1, d)), np.abs(rng.uniform(-0.07, 0.07, (b, 1, d)))
+    idx = rng.integers(0, n, (b, k))
+    gs = rng.standard_normal((b, k))
+    tt = torch.tensor(table.copy(), requires_grad=True)
+    rows = tt[torch.from_numpy(idx)]
+    delta = (rows - torch.from_numpy(c)).abs()
+    s = 24 - torch.relu(delta - torch.from_numpy(o)).sum(-1) - 0.02 * torch.minimum(delta, torch.from_numpy(o)).sum(-1)
+    (s * torch.from_numpy(gs)).sum().backward()
+    t0 = table.copy()
+    res = orc.train_step("box", table, m, v, idx, c, o, gs, 24.0, 0.02, 1e-4, 1)
+    assert np.allclose(res["score"], s.detach().numpy(), rtol=1e-12)
+    dense = np.zeros((n, d))
+    dense[res["uniq"]] = res["merged"]
+    assert np.allclose(dense, tt.grad.numpy(), rtol=1e-11, atol=1e-14)
+    touched = np.zeros(n, bool)
+    touched[idx.reshape(-1)] = True
+    assert np.array_equal(np.flatnonzero(touched), res["uniq"])
+    assert np.array_equal(table[~touched], t0[~touched])
+    g = tt.grad.numpy()[touched]
+    want = t0[touched] - 1e-4 / 0.1 * (0.1 * g) / (np.sqrt(0.001 * g * g) / math.sqrt(0.001) + 1e-8)
+    assert np.allclose(table[touched], want, rtol=1e-11)
