@@ -1,0 +1,26 @@
+// Host-side helpers shared by the translation units of libsmore_amd.so.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstddef>
+#include <cstdint>
+#include <cstdio>
+
+#include "../../include/smore_amd.h"
+
+namespace smx {
+
+constexpr int kWave = 64;  // gfx950 wavefront
+
+// Records the message returned by smx_last_error() and hands back `code`.
+int fail(int code, const char* fmt, ...);
+
+// Checks the launch that just happened on this thread.
+int check_launch(const char* what);
+
+inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+}  // namespace smx

@@ -1,0 +1,49 @@
+"""Helpers shared by the parity tests."""
+import zlib
+
+import numpy as np
+
+from oracle import oracle as orc
+
+# Floating-point bar of the scoring path: 1e-5 relative, fp32.  An element is compared
+# against max(|reference element|, RMS of the reference tensor): sums over many signed
+# terms can cancel to values far below the tensor's scale, where a pure elementwise
+# relative bound would ask for more digits than fp32 addition has.
+REL_F32 = 1e-5
+REL_F64 = 1e-10
+
+
+def seed(*parts):
+    return zlib.crc32(repr(parts).encode())
+
+
+def assert_close(got, ref, rel, what=""):
+    got = np.asarray(got, dtype=np.float64)
+    ref = np.asarray(ref, dtype=np.float64)
+    assert got.shape == ref.shape, (what, got.shape, ref.shape)
+    assert np.all(np.isfinite(got)) or not np.all(np.isfinite(ref)), f"{what}: non-finite output"
+    scale = float(np.sqrt(np.mean(ref ** 2))) if ref.size else 0.0
+    bound = rel * np.maximum(np.abs(ref), scale) + 1e-300
+    err = np.abs(got - ref)
+    bad = err > bound
+    if bad.any():
+        k = np.argmax(err / bound)
+        raise AssertionError(
+            f"{what}: {bad.sum()} of {ref.size} elements off; worst got={got.reshape(-1)[k]!r} "
+            f"ref={ref.reshape(-1)[k]!r} err/bound={(err / bound).reshape(-1)[k]:.3g} scale={scale:.3g}")
+
+
+def make_inputs(kind, be, ne, bc, nc, dim, rng, scale=1.0):
+    """Random operands of one dense operator call (float64 numpy)."""
+    mul = 2 if kind in orc.TWO_HALVES else 1
+    if kind.startswith("beta"):
+        def f(*s):
+            x = rng.standard_normal(s)
+            return np.clip(1 + np.where(x > 0, x, np.expm1(x)), 0.05, 1e9)
+    else:
+        def f(*s):
+            return rng.standard_normal(s) * scale
+    e = f(be, ne, dim * mul)
+    q1 = f(bc, nc, dim)
+    q2 = None if kind in orc.ONE_QUERY else f(bc, nc, dim)
+    return e, q1, q2
