@@ -81,6 +81,108 @@ int smx_dist_backward_f64(int kind, void* stream, const double* gout, const doub
                           double* gq2, size_t bsize, size_t num, size_t be, size_t ne, size_t bc,
                           size_t nc, size_t dim);
 
+/* ---- gather-fused scoring -------------------------------------------------
+ * One training step scores every (query b, negative k) pair against the entity
+ * row table[idx[b,k]].  These entry points fuse what the reference runs as
+ * separate steps, without materialising the gathered [B,K,row] tensor:
+ *   rows = table[idx]            smore/common/embedding/embed_rw.py:74-75
+ *                                (EmbedLookupFunc.forward, embed_optimizer.py:51-61)
+ *   clamp(rows + add, lo, hi)    smore/common/modules.py:29-36 (BetaE only)
+ *   dist forward / backward      smore/common/torchext/common_kernel.h:33-123
+ *   logit = gamma - dist         custom_cal_logit of smore/models/{vec,box,rotate,beta}.py
+ *   table [n_rows, dim*mul] fp32   idx [B,K] int64   q1, q2 [B, dim]   score [B,K]
+ * idx == NULL means `table` already holds the B*K rows in pair order (the
+ * dense [B,K,row] layout of the reference operators).
+ * An id outside [0, n_rows) sets *err_flag (device int, may be NULL) to 1 and
+ * row 0 is read in its place; the caller decides when to look at the flag. */
+typedef struct smx_score_params {
+  float gamma;   /* margin: logit = gamma - distance */
+  float cen;     /* BOX: weight of the inside distance */
+  int reg_on;    /* apply clamp(e + reg_add, reg_lo, reg_hi) to entity values */
+  float reg_add;
+  float reg_lo;
+  float reg_hi;
+} smx_score_params;
+
+int smx_score_forward(int model, void* stream, const float* table, size_t n_rows, const int64_t* idx,
+                      const float* q1, const float* q2, float* score, size_t B, size_t K, size_t dim,
+                      const smx_score_params* params, int* err_flag);
+
+/* Query-side gradient of sum(gscore * score): gq1, gq2 [B, dim] are overwritten.
+ * `score` is the tensor smx_score_forward wrote (L2 needs it for the chain
+ * rule of the square root).  Replaces dist_backward_query_kernel
+ * (common_kernel.h:92-123) plus the autograd nodes between it and the logit. */
+int smx_score_backward_query(int model, void* stream, const float* table, size_t n_rows,
+                             const int64_t* idx, const float* q1, const float* q2,
+                             const float* score, const float* gscore, float* gq1, float* gq2,
+                             size_t B, size_t K, size_t dim, const smx_score_params* params);
+
+/* ---- segment plan ----------------------------------------------------------
+ * Groups the P = B*K pairs of a step by entity id on the device.  Replaces
+ * merge_grad_indices (smore/common/embedding/embed_optimizer.py:39-42), i.e.
+ * torch.unique(ids, return_inverse=True) run on the host.  Integer outputs are
+ * bit-exact by contract:
+ *   order[P]       pair positions grouped by id; inside an id ascending (stable)
+ *   sorted_ids[P]  idx[order[.]] as 32-bit ids (read as unsigned)
+ *   seg_of_pos[P]  segment number of every sorted position
+ *   uniq[P]        first n_uniq entries: the distinct ids, ascending (= torch.unique)
+ *   seg_start[P+1] first n_uniq+1 entries: start of each segment in order[]
+ *   inverse[P]     position of idx[p] in uniq (= return_inverse), may be NULL
+ *   n_uniq         device int: number of distinct ids
+ * All arrays are caller-allocated device memory.  workspace: at least
+ * smx_plan_workspace_bytes(P, n_rows) bytes, 256-byte aligned.  Needs n_rows <= 2^32. */
+size_t smx_plan_workspace_bytes(size_t n_pairs, size_t n_rows);
+int smx_plan_build(void* stream, const int64_t* idx, size_t n_pairs, size_t n_rows, void* workspace,
+                   size_t workspace_bytes, int32_t* order, int32_t* sorted_ids, int32_t* seg_of_pos,
+                   int64_t* uniq, int32_t* seg_start, int64_t* inverse, int32_t* n_uniq,
+                   int* err_flag);
+
+typedef struct smx_plan_view {
+  const int32_t* order;
+  const int32_t* sorted_ids;
+  const int32_t* seg_of_pos;
+  const int32_t* seg_start;
+  size_t n_pairs;
+} smx_plan_view;
+
+/* Lazy Adam of the sparse row optimizer: AdamEmbedOptimizer.update_step
+ * (smore/common/embedding/embed_optimizer.py:208-252).  `step` is the global
+ * counter after apply_grad incremented it (:156), so the first update has
+ * step = 1.  eps is smore/common/consts.py:20 in the reference. */
+typedef struct smx_adam_params {
+  double lr;    /* hyper-parameters are doubles, as the Python floats of the reference are: */
+  double beta1; /* 1 - beta is formed in double and only then rounded to fp32             */
+  double beta2;
+  double eps;
+  long step;
+} smx_adam_params;
+
+/* ---- entity-side backward, segment sum and row update in one pass ----------
+ * For every distinct id u of the plan: g[u,:] = sum over the pairs of segment u
+ * of d(sum gscore*score)/d(entity row), summed in the plan's order (fixed, no
+ * atomics).  Then, as requested:
+ *   merged != NULL   merged[u,:] = g[u,:]        ([n_uniq, dim*mul], caller-sized for P rows
+ *                                                 or fewer if it knows n_uniq)
+ *   m, v, adam given table[id], m[id], v[id] are updated by lazy Adam in place;
+ *                    rows of ids not in the plan are not touched.
+ * Replaces dist_backward_ent_kernel (common_kernel.h:59-89), EmbedLookupFunc.backward
+ * (embed_optimizer.py:63-66), merge_grad_list (:45-48) and update_step (:208-252).
+ * workspace: smx_entity_workspace_bytes(P, dim*mul) bytes, 256-byte aligned. */
+size_t smx_entity_workspace_bytes(size_t n_pairs, size_t row_len);
+int smx_score_backward_entity(int model, void* stream, const smx_plan_view* plan, float* table,
+                              size_t n_rows, const float* q1, const float* q2, const float* score,
+                              const float* gscore, size_t B, size_t K, size_t dim,
+                              const smx_score_params* params, float* merged, float* m, float* v,
+                              const smx_adam_params* adam, void* workspace, size_t workspace_bytes);
+
+/* Same pass for gradient rows that already exist in memory (what autograd hands
+ * EmbedLookupFunc.backward): grad_rows [P, row_len] in pair order.  Replaces
+ * merge_grad_list (embed_optimizer.py:45-48) and, when m, v, adam are given,
+ * update_step (:208-252) on `table`. */
+int smx_rows_backward(void* stream, const smx_plan_view* plan, const float* grad_rows,
+                      size_t row_len, float* merged, float* table, float* m, float* v,
+                      const smx_adam_params* adam, void* workspace, size_t workspace_bytes);
+
 #ifdef __cplusplus
 }
 #endif

@@ -29,7 +29,35 @@ SIGNATURES = {
     "smx_dist_forward_f64": (_i, _DENSE_FWD),
     "smx_dist_backward_f32": (_i, _DENSE_BWD),
     "smx_dist_backward_f64": (_i, _DENSE_BWD),
+    # model, stream, table, n_rows, idx, q1, q2, score, B, K, dim, params, err_flag
+    "smx_score_forward": (_i, [_i, _vp, _vp, _sz, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _vp, _vp]),
+    # model, stream, table, n_rows, idx, q1, q2, score, gscore, gq1, gq2, B, K, dim, params
+    "smx_score_backward_query": (_i, [_i, _vp, _vp, _sz, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _vp]),
+    "smx_plan_workspace_bytes": (_sz, [_sz, _sz]),
+    # stream, idx, n_pairs, n_rows, ws, ws_bytes, order, sorted_ids, seg_of_pos, uniq, seg_start, inverse, n_uniq, err
+    "smx_plan_build": (_i, [_vp, _vp, _sz, _sz, _vp, _sz, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "smx_entity_workspace_bytes": (_sz, [_sz, _sz]),
+    # model, stream, plan, table, n_rows, q1, q2, score, gscore, B, K, dim, params, merged, m, v, adam, ws, ws_bytes
+    "smx_score_backward_entity": (_i, [_i, _vp, _vp, _vp, _sz, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _vp, _vp, _vp, _vp,
+                                       _vp, _vp, _sz]),
+    # stream, plan, grad_rows, row_len, merged, table, m, v, adam, ws, ws_bytes
+    "smx_rows_backward": (_i, [_vp, _vp, _vp, _sz, _vp, _vp, _vp, _vp, _vp, _vp, _sz]),
 }
+
+
+class ScoreParams(ctypes.Structure):
+    """smx_score_params of include/smore_amd.h."""
+    _fields_ = [("gamma", _f), ("cen", _f), ("reg_on", _i), ("reg_add", _f), ("reg_lo", _f), ("reg_hi", _f)]
+
+
+class AdamParams(ctypes.Structure):
+    """smx_adam_params of include/smore_amd.h."""
+    _fields_ = [("lr", _d), ("beta1", _d), ("beta2", _d), ("eps", _d), ("step", _l)]
+
+
+class PlanView(ctypes.Structure):
+    """smx_plan_view of include/smore_amd.h."""
+    _fields_ = [("order", _vp), ("sorted_ids", _vp), ("seg_of_pos", _vp), ("seg_start", _vp), ("n_pairs", _sz)]
 
 _lib = None
 

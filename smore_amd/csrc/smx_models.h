@@ -1,0 +1,172 @@
+// Score models of the gather-fused path: logit = gamma - distance, one struct per
+// model, built from the per-feature terms in smx_functors.h.
+//
+//   model      logit                                   reference call site
+//   L1         gamma - sum |e-q|                        smore/models/vec.py:85-90
+//   L2         gamma - sqrt(sum (e-q)^2)                smore/common/torchext/dist_func/l2_dist.py:59-62
+//   BOX        gamma - d_out - cen * d_in               smore/models/box.py:157-164
+//   ROTATE     gamma - sum sqrt(dre^2 + dim^2 + 1e-20)  smore/models/rotate.py:137-142
+//   BETA_KL    gamma - sum KL(Beta(e) || Beta(q))       smore/models/beta.py:303-308
+//
+// A model exposes
+//   fwd(e1,e2,q,acc0,acc1)      add one feature's term(s) to the accumulators
+//   score(acc0,acc1,p)          logit from the reduced accumulators
+//   coef(g,score,p,c0,c1)       d logit-loss / d accumulator, from the upstream
+//                               gradient g of the logit and the saved logit
+//   bwd_e / bwd_q               add one feature's gradient w.r.t. entity / query
+// Optional entity prologue (BetaE): e' = clamp(e + add, lo, hi)
+// (smore/common/modules.py:29-36 applied at smore/models/kg_reasoning.py:352);
+// its backward passes gradient where lo <= e + add <= hi.
+#pragma once
+#include "smx_functors.h"
+
+namespace smx {
+
+enum Model : int { mL1 = 0, mL2 = 1, mBox = 2, mRotate = 3, mBetaKL = 4, mNumModels = 5 };
+
+__host__ __device__ constexpr int model_mul(int m) { return (m == mRotate || m == mBetaKL) ? 2 : 1; }
+__host__ __device__ constexpr int model_nq(int m) { return (m == mL1 || m == mL2) ? 1 : 2; }
+
+struct ScoreParams {
+  float gamma;
+  float cen;      // weight of the inside distance (BOX only)
+  int reg_on;     // entity prologue on/off
+  float reg_add, reg_lo, reg_hi;
+};
+
+__device__ __forceinline__ float reg_apply(float e, const ScoreParams& p) {
+  if (!p.reg_on) return e;
+  const float v = e + p.reg_add;
+  return fminf(fmaxf(v, p.reg_lo), p.reg_hi);
+}
+__device__ __forceinline__ float reg_mask(float e_raw, float g, const ScoreParams& p) {
+  if (!p.reg_on) return g;
+  const float v = e_raw + p.reg_add;
+  return (v >= p.reg_lo && v <= p.reg_hi) ? g : 0.0f;
+}
+
+// per-feature query registers kept by a lane for the whole tile
+struct QPair {
+  float a, b;
+};
+
+template <int M> struct ModelOps;
+
+template <> struct ModelOps<mL1> {
+  using Q = QPair;
+  static __device__ __forceinline__ Q prep(float q1, float) { return {q1, 0.f}; }
+  static __device__ __forceinline__ void fwd(float e1, float, const Q& q, float& a0, float&) {
+    a0 += Term<kL1, float>::fwd(e1, 0.f, q.a, 0.f);
+  }
+  static __device__ __forceinline__ float score(float a0, float, const ScoreParams& p) { return p.gamma - a0; }
+  static __device__ __forceinline__ void coef(float g, float, const ScoreParams&, float& c0, float& c1) {
+    c0 = -g;
+    c1 = 0.f;
+  }
+  static __device__ __forceinline__ void bwd_e(float c0, float, float e1, float, const Q& q, float& ge1, float&) {
+    float s1 = 0, s2 = 0, s3 = 0;
+    Term<kL1, float>::bwd(c0, e1, 0.f, q.a, 0.f, ge1, s1, s2, s3);
+  }
+  static __device__ __forceinline__ void bwd_q(float c0, float, float e1, float, const Q& q, float& gq1, float&) {
+    float s1 = 0, s2 = 0, s3 = 0;
+    Term<kL1, float>::bwd(c0, e1, 0.f, q.a, 0.f, s1, s2, gq1, s3);
+  }
+};
+
+template <> struct ModelOps<mL2> {
+  using Q = QPair;
+  static __device__ __forceinline__ Q prep(float q1, float) { return {q1, 0.f}; }
+  static __device__ __forceinline__ void fwd(float e1, float, const Q& q, float& a0, float&) {
+    a0 += Term<kL2, float>::fwd(e1, 0.f, q.a, 0.f);
+  }
+  static __device__ __forceinline__ float score(float a0, float, const ScoreParams& p) { return p.gamma - sqrtf(a0); }
+  // d(gamma - sqrt(d2)) / d d2 = -1 / (2 sqrt(d2)), and sqrt(d2) = gamma - score.  At d2 == 0 the
+  // coefficient is infinite, as autograd of torch.sqrt makes it in the reference.
+  static __device__ __forceinline__ void coef(float g, float s, const ScoreParams& p, float& c0, float& c1) {
+    c0 = -g / (2.0f * (p.gamma - s));
+    c1 = 0.f;
+  }
+  static __device__ __forceinline__ void bwd_e(float c0, float, float e1, float, const Q& q, float& ge1, float&) {
+    float s1 = 0, s2 = 0, s3 = 0;
+    Term<kL2, float>::bwd(c0, e1, 0.f, q.a, 0.f, ge1, s1, s2, s3);
+  }
+  static __device__ __forceinline__ void bwd_q(float c0, float, float e1, float, const Q& q, float& gq1, float&) {
+    float s1 = 0, s2 = 0, s3 = 0;
+    Term<kL2, float>::bwd(c0, e1, 0.f, q.a, 0.f, s1, s2, gq1, s3);
+  }
+};
+
+// acc0 = outside distance, acc1 = inside distance; one row read serves both.
+template <> struct ModelOps<mBox> {
+  using Q = QPair;  // a = center, b = offset
+  static __device__ __forceinline__ Q prep(float q1, float q2) { return {q1, q2}; }
+  static __device__ __forceinline__ void fwd(float e1, float, const Q& q, float& a0, float& a1) {
+    a0 += Term<kBoxOut, float>::fwd(e1, 0.f, q.a, q.b);
+    a1 += Term<kBoxIn, float>::fwd(e1, 0.f, q.a, q.b);
+  }
+  static __device__ __forceinline__ float score(float a0, float a1, const ScoreParams& p) {
+    return p.gamma - a0 - p.cen * a1;
+  }
+  static __device__ __forceinline__ void coef(float g, float, const ScoreParams& p, float& c0, float& c1) {
+    c0 = -g;
+    c1 = -p.cen * g;
+  }
+  static __device__ __forceinline__ void bwd_e(float c0, float c1, float e1, float, const Q& q, float& ge1, float&) {
+    float s1 = 0, s2 = 0, s3 = 0;
+    Term<kBoxOut, float>::bwd(c0, e1, 0.f, q.a, q.b, ge1, s1, s2, s3);
+    Term<kBoxIn, float>::bwd(c1, e1, 0.f, q.a, q.b, ge1, s1, s2, s3);
+  }
+  static __device__ __forceinline__ void bwd_q(float c0, float c1, float e1, float, const Q& q, float& gc, float& go) {
+    float s1 = 0, s2 = 0;
+    Term<kBoxOut, float>::bwd(c0, e1, 0.f, q.a, q.b, s1, s2, gc, go);
+    Term<kBoxIn, float>::bwd(c1, e1, 0.f, q.a, q.b, s1, s2, gc, go);
+  }
+};
+
+template <> struct ModelOps<mRotate> {
+  using Q = QPair;  // a = re, b = im
+  static __device__ __forceinline__ Q prep(float q1, float q2) { return {q1, q2}; }
+  static __device__ __forceinline__ void fwd(float e1, float e2, const Q& q, float& a0, float&) {
+    a0 += Term<kRotate, float>::fwd(e1, e2, q.a, q.b);
+  }
+  static __device__ __forceinline__ float score(float a0, float, const ScoreParams& p) { return p.gamma - a0; }
+  static __device__ __forceinline__ void coef(float g, float, const ScoreParams&, float& c0, float& c1) {
+    c0 = -g;
+    c1 = 0.f;
+  }
+  static __device__ __forceinline__ void bwd_e(float c0, float, float e1, float e2, const Q& q, float& ge1, float& ge2) {
+    float s1 = 0, s2 = 0;
+    Term<kRotate, float>::bwd(c0, e1, e2, q.a, q.b, ge1, ge2, s1, s2);
+  }
+  static __device__ __forceinline__ void bwd_q(float c0, float, float e1, float e2, const Q& q, float& g1, float& g2) {
+    float s1 = 0, s2 = 0;
+    Term<kRotate, float>::bwd(c0, e1, e2, q.a, q.b, s1, s2, g1, g2);
+  }
+};
+
+template <> struct ModelOps<mBetaKL> {
+  using Q = QPair;  // a = alpha, b = beta of the query
+  static __device__ __forceinline__ Q prep(float q1, float q2) { return {q1, q2}; }
+  static __device__ __forceinline__ void fwd(float e1, float e2, const Q& q, float& a0, float&) {
+    a0 += Term<kBetaKL, float>::fwd(e1, e2, q.a, q.b);
+  }
+  static __device__ __forceinline__ float score(float a0, float, const ScoreParams& p) { return p.gamma - a0; }
+  static __device__ __forceinline__ void coef(float g, float, const ScoreParams&, float& c0, float& c1) {
+    c0 = -g;
+    c1 = 0.f;
+  }
+  static __device__ __forceinline__ void bwd_e(float c0, float, float e1, float e2, const Q& q, float& ge1, float& ge2) {
+    const float se = e1 + e2, sq = q.a + q.b;
+    const float common = (sq - se) * trigamma(se);
+    ge1 += c0 * ((e1 - q.a) * trigamma(e1) + common);
+    ge2 += c0 * ((e2 - q.b) * trigamma(e2) + common);
+  }
+  static __device__ __forceinline__ void bwd_q(float c0, float, float e1, float e2, const Q& q, float& g1, float& g2) {
+    const float se = e1 + e2, sq = q.a + q.b;
+    const float common = digamma(se) - digamma(sq);
+    g1 += c0 * (digamma(q.a) - digamma(e1) + common);
+    g2 += c0 * (digamma(q.b) - digamma(e2) + common);
+  }
+};
+
+}  // namespace smx

@@ -1,0 +1,139 @@
+// Segment plan: groups the (query, negative) pairs of one step by entity id.
+//
+// Replaces merge_grad_indices (smore/common/embedding/embed_optimizer.py:39-42),
+// i.e. torch.unique(ids, return_inverse=True), which the reference runs on the
+// host CPU, with a device pipeline:
+//   keys  = (uint32) idx[p]                      narrow + range check
+//   sort  (key, p) by key                        LSD radix sort, stable, only the
+//                                                bits an id below n_rows can have
+//   heads = key[p] != key[p-1]                   segment boundaries
+//   scan  heads                                  segment number of every position
+//   emit  uniq, seg_start, inverse, n_uniq
+// The sort is stable, so inside a segment pairs stay in ascending pair order:
+// every later reduction over a segment has one fixed summation order.
+#include <cstring>
+
+#include <rocprim/device/device_radix_sort.hpp>
+#include <rocprim/device/device_scan.hpp>
+#include <rocprim/iterator/counting_iterator.hpp>
+
+#include "smx_common.h"
+
+namespace smx {
+
+__global__ __launch_bounds__(256) void plan_keys_kernel(const long long* __restrict__ idx, unsigned* __restrict__ keys,
+                                                        int n, unsigned long long n_rows, int* err) {
+  const int p = blockIdx.x * blockDim.x + threadIdx.x;
+  if (p >= n) return;
+  long long id = idx[p];
+  if ((unsigned long long)id >= n_rows) {
+    if (err) *err = 1;
+    id = 0;
+  }
+  keys[p] = (unsigned)id;
+}
+
+__global__ __launch_bounds__(256) void plan_heads_kernel(const int* __restrict__ sorted_ids, unsigned* __restrict__ heads,
+                                                         int n) {
+  const int p = blockIdx.x * blockDim.x + threadIdx.x;
+  if (p >= n) return;
+  heads[p] = (p == 0 || sorted_ids[p] != sorted_ids[p - 1]) ? 1u : 0u;
+}
+
+__global__ __launch_bounds__(256) void plan_emit_kernel(const int* __restrict__ sorted_ids, const int* __restrict__ order,
+                                                        const unsigned* __restrict__ seg_incl, int* __restrict__ seg_of_pos,
+                                                        long long* __restrict__ uniq, int* __restrict__ seg_start,
+                                                        long long* __restrict__ inverse, int* __restrict__ n_uniq, int n) {
+  const int p = blockIdx.x * blockDim.x + threadIdx.x;
+  if (p >= n) return;
+  const int seg = (int)seg_incl[p] - 1;
+  seg_of_pos[p] = seg;
+  if (p == 0 || sorted_ids[p] != sorted_ids[p - 1]) {
+    uniq[seg] = (long long)(unsigned)sorted_ids[p];
+    seg_start[seg] = p;
+  }
+  if (inverse) inverse[order[p]] = seg;
+  if (p == n - 1) {
+    *n_uniq = seg + 1;
+    seg_start[seg + 1] = n;
+  }
+}
+
+static unsigned key_bits(size_t n_rows) {
+  unsigned bits = 1;
+  while (bits < 32 && (1ull << bits) < n_rows) ++bits;
+  return bits;
+}
+
+struct PlanScratch {
+  size_t keys_off, heads_off, scan_off, temp_off, temp_bytes, total;
+};
+
+static hipError_t plan_scratch(size_t n, size_t n_rows, PlanScratch* s) {
+  size_t sort_bytes = 0, scan_bytes = 0;
+  unsigned* kp = nullptr;
+  int* ip = nullptr;
+  hipError_t e = rocprim::radix_sort_pairs(nullptr, sort_bytes, kp, kp, rocprim::counting_iterator<int>(0), ip, n, 0,
+                                           key_bits(n_rows), (hipStream_t)0);
+  if (e != hipSuccess) return e;
+  e = rocprim::inclusive_scan(nullptr, scan_bytes, kp, kp, n, rocprim::plus<unsigned>(), (hipStream_t)0);
+  if (e != hipSuccess) return e;
+  auto up = [](size_t x) { return (x + 255) & ~(size_t)255; };
+  s->keys_off = 0;
+  s->heads_off = up(n * sizeof(unsigned));
+  s->scan_off = s->heads_off + up(n * sizeof(unsigned));
+  s->temp_off = s->scan_off + up(n * sizeof(unsigned));
+  s->temp_bytes = up(sort_bytes > scan_bytes ? sort_bytes : scan_bytes);
+  s->total = s->temp_off + s->temp_bytes;
+  return hipSuccess;
+}
+
+}  // namespace smx
+
+extern "C" {
+
+size_t smx_plan_workspace_bytes(size_t n_pairs, size_t n_rows) {
+  smx::PlanScratch s;
+  if (n_pairs == 0) return 256;
+  if (smx::plan_scratch(n_pairs, n_rows, &s) != hipSuccess) return 0;
+  return s.total;
+}
+
+int smx_plan_build(void* stream, const int64_t* idx, size_t n_pairs, size_t n_rows, void* workspace,
+                   size_t workspace_bytes, int32_t* order, int32_t* sorted_ids, int32_t* seg_of_pos, int64_t* uniq,
+                   int32_t* seg_start, int64_t* inverse, int32_t* n_uniq, int* err_flag) {
+  using namespace smx;
+  if (!idx || !order || !sorted_ids || !seg_of_pos || !uniq || !seg_start || !n_uniq || !workspace)
+    return fail(SMX_ERR_ARG, "null pointer in plan build");
+  if (n_pairs == 0 || n_pairs > 0x7fffffffull) return fail(SMX_ERR_SHAPE, "pair count %zu out of range", n_pairs);
+  if (n_rows == 0 || n_rows > 0x100000000ull) return fail(SMX_ERR_SHAPE, "entity count %zu needs ids wider than 32 bits", n_rows);
+  PlanScratch s;
+  if (plan_scratch(n_pairs, n_rows, &s) != hipSuccess) return fail(SMX_ERR_HIP, "rocprim size query failed");
+  if (workspace_bytes < s.total)
+    return fail(SMX_ERR_WORKSPACE, "plan workspace too small: %zu < %zu", workspace_bytes, s.total);
+  if (reinterpret_cast<uintptr_t>(workspace) & 255u) return fail(SMX_ERR_ARG, "workspace must be 256-byte aligned");
+  hipStream_t st = as_stream(stream);
+  char* ws = static_cast<char*>(workspace);
+  unsigned* keys = reinterpret_cast<unsigned*>(ws + s.keys_off);
+  unsigned* heads = reinterpret_cast<unsigned*>(ws + s.heads_off);
+  unsigned* scan = reinterpret_cast<unsigned*>(ws + s.scan_off);
+  void* temp = ws + s.temp_off;
+  const int n = (int)n_pairs;
+  const unsigned blocks = (unsigned)((n_pairs + 255) / 256);
+
+  hipLaunchKernelGGL(plan_keys_kernel, dim3(blocks), dim3(256), 0, st, reinterpret_cast<const long long*>(idx), keys, n,
+                     (unsigned long long)n_rows, err_flag);
+  size_t tb = s.temp_bytes;
+  hipError_t e = rocprim::radix_sort_pairs(temp, tb, keys, reinterpret_cast<unsigned*>(sorted_ids),
+                                           rocprim::counting_iterator<int>(0), order, n_pairs, 0, key_bits(n_rows), st);
+  if (e != hipSuccess) return fail(SMX_ERR_HIP, "radix sort: %s", hipGetErrorString(e));
+  hipLaunchKernelGGL(plan_heads_kernel, dim3(blocks), dim3(256), 0, st, sorted_ids, heads, n);
+  tb = s.temp_bytes;
+  e = rocprim::inclusive_scan(temp, tb, heads, scan, n_pairs, rocprim::plus<unsigned>(), st);
+  if (e != hipSuccess) return fail(SMX_ERR_HIP, "scan: %s", hipGetErrorString(e));
+  hipLaunchKernelGGL(plan_emit_kernel, dim3(blocks), dim3(256), 0, st, sorted_ids, order, scan, seg_of_pos,
+                     reinterpret_cast<long long*>(uniq), seg_start, reinterpret_cast<long long*>(inverse), n_uniq, n);
+  return check_launch("plan build");
+}
+
+}  // extern "C"

@@ -1,0 +1,380 @@
+// Gather-fused scoring, forward and query-side backward (fp32).
+//
+// Replaces, in one pass each, the sequence the reference runs per training
+// step for the negative samples (smore/models/kg_reasoning.py:301-307,349-355):
+//   rows = table[idx]                      smore/common/embedding/embed_rw.py:74-75
+//   [optional clamp(rows + 1, .05, 1e9)]   smore/common/modules.py:29-36
+//   d = dist(rows, query)                  smore/common/torchext/common_kernel.h:33-56
+//   logit = gamma - d                      custom_cal_logit of smore/models/*.py
+// and, backward, the query-gradient kernel common_kernel.h:92-123.  The
+// [B,K,D] gathered tensor is never materialised: a wavefront reads each entity
+// row straight from the table with 16-byte loads (one float4 column per lane).
+//
+// Work split.  forward: workgroup = (query b, tile of negatives); the query
+// row(s) are staged once in LDS, every lane then keeps the features it owns in
+// registers for the whole tile; the four wavefronts take turns on the tile's
+// rows, several rows in flight per wavefront.  backward: one workgroup per
+// query walks all K negatives, wavefront partial sums are combined through LDS
+// in wavefront order, so the gradient has a fixed summation order.
+#include "smx_common.h"
+#include "smx_models.h"
+#include "smx_wave.h"
+
+namespace smx {
+
+template <int VEC> struct Pack {
+  float v[VEC];
+};
+
+template <int VEC>
+__device__ __forceinline__ Pack<VEC> load_pack(const float* __restrict__ base, int col) {
+  Pack<VEC> r;
+  if constexpr (VEC == 4) {
+    const float4 t = reinterpret_cast<const float4*>(base)[col];
+    r.v[0] = t.x;
+    r.v[1] = t.y;
+    r.v[2] = t.z;
+    r.v[3] = t.w;
+  } else {
+    r.v[0] = base[col];
+  }
+  return r;
+}
+
+// Loads the features a lane owns of the staged query into registers.
+template <int M, int VEC, int NIT>
+__device__ __forceinline__ void load_query_regs(const float* lds, int dim, int ncol, int lane,
+                                                typename ModelOps<M>::Q (&q)[NIT][VEC]) {
+#pragma unroll
+  for (int it = 0; it < NIT; ++it) {
+    const int c = lane + 64 * it;
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) {
+      const float a = c < ncol ? lds[c * VEC + v] : 0.f;
+      const float b = (model_nq(M) == 2 && c < ncol) ? lds[dim + c * VEC + v] : 0.f;
+      q[it][v] = ModelOps<M>::prep(a, b);
+    }
+  }
+}
+
+template <int M>
+__device__ __forceinline__ void stage_query(float* lds, const float* __restrict__ q1, const float* __restrict__ q2,
+                                            size_t b, int dim) {
+  for (int d = threadIdx.x; d < dim; d += blockDim.x) {
+    lds[d] = q1[b * dim + d];
+    if (model_nq(M) == 2) lds[dim + d] = q2[b * dim + d];
+  }
+  __syncthreads();
+}
+
+// Row pointer of pair (b,k): through idx when given, else the dense [B*K, row_len] layout.
+__device__ __forceinline__ const float* pair_row(const float* __restrict__ table, const long long* __restrict__ idx,
+                                                 size_t pair, size_t row_len, unsigned long long n_rows, int lane,
+                                                 int* err) {
+  long long row = idx ? idx[pair] : (long long)pair;
+  if ((unsigned long long)row >= n_rows) {  // out-of-range id: flag it, read row 0 instead of faulting
+    if (err && lane == 0) *err = 1;
+    row = 0;
+  }
+  return table + (size_t)row * row_len;
+}
+
+template <int M, int VEC, int NIT, int RIF>
+__global__ __launch_bounds__(256) void score_forward_kernel(const float* __restrict__ table,
+                                                            const long long* __restrict__ idx,
+                                                            const float* __restrict__ q1, const float* __restrict__ q2,
+                                                            float* __restrict__ score, int K, int ncol, int tiles,
+                                                            int tile_k, unsigned long long n_rows, ScoreParams p,
+                                                            int* err) {
+  constexpr int MUL = model_mul(M);
+  extern __shared__ float lds[];
+  const int b = blockIdx.x / tiles;
+  const int tile = blockIdx.x - b * tiles;
+  const int lane = threadIdx.x & 63;
+  const int wave = uniform(threadIdx.x >> 6);
+  const int dim = ncol * VEC;
+  const size_t row_len = (size_t)dim * MUL;
+
+  stage_query<M>(lds, q1, q2, b, dim);
+  typename ModelOps<M>::Q q[NIT][VEC];
+  load_query_regs<M, VEC, NIT>(lds, dim, ncol, lane, q);
+
+  const int k0 = tile * tile_k;
+  const int k1 = min(K, k0 + tile_k);
+  for (int kb = k0 + wave * RIF; kb < k1; kb += 4 * RIF) {
+    Pack<VEC> e1[RIF][NIT], e2[RIF][NIT];
+#pragma unroll
+    for (int r = 0; r < RIF; ++r) {
+      const int k = kb + r;
+      if (k < k1) {
+        const float* pe = pair_row(table, idx, (size_t)b * K + k, row_len, n_rows, lane, err);
+#pragma unroll
+        for (int it = 0; it < NIT; ++it) {
+          const int c = lane + 64 * it;
+          if (c < ncol) {
+            e1[r][it] = load_pack<VEC>(pe, c);
+            if (MUL == 2) e2[r][it] = load_pack<VEC>(pe + dim, c);
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < RIF; ++r) {
+      const int k = kb + r;
+      if (k < k1) {
+        float a0 = 0.f, a1 = 0.f;
+#pragma unroll
+        for (int it = 0; it < NIT; ++it) {
+          const int c = lane + 64 * it;
+          if (c < ncol) {
+#pragma unroll
+            for (int v = 0; v < VEC; ++v) {
+              const float x1 = reg_apply(e1[r][it].v[v], p);
+              const float x2 = MUL == 2 ? reg_apply(e2[r][it].v[v], p) : 0.f;
+              ModelOps<M>::fwd(x1, x2, q[it][v], a0, a1);
+            }
+          }
+        }
+        a0 = wave_sum_f32(a0);
+        if (M == mBox) a1 = wave_sum_f32(a1);
+        if (lane == 0) score[(size_t)b * K + k] = ModelOps<M>::score(a0, a1, p);
+      }
+    }
+  }
+}
+
+template <int M, int VEC, int NIT, int RIF, int NW>
+__global__ __launch_bounds__(NW * 64) void score_backward_query_kernel(
+    const float* __restrict__ table, const long long* __restrict__ idx, const float* __restrict__ q1,
+    const float* __restrict__ q2, const float* __restrict__ score, const float* __restrict__ gscore,
+    float* __restrict__ gq1, float* __restrict__ gq2, int K, int ncol, unsigned long long n_rows, ScoreParams p) {
+  constexpr int MUL = model_mul(M);
+  constexpr int NQ = model_nq(M);
+  extern __shared__ float lds[];
+  const int b = blockIdx.x;
+  const int lane = threadIdx.x & 63;
+  const int wave = uniform(threadIdx.x >> 6);
+  const int dim = ncol * VEC;
+  const size_t row_len = (size_t)dim * MUL;
+
+  stage_query<M>(lds, q1, q2, b, dim);
+  typename ModelOps<M>::Q q[NIT][VEC];
+  load_query_regs<M, VEC, NIT>(lds, dim, ncol, lane, q);
+
+  float g1[NIT][VEC], g2[NIT][VEC];
+#pragma unroll
+  for (int it = 0; it < NIT; ++it)
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) g1[it][v] = g2[it][v] = 0.f;
+
+  for (int kb = wave * RIF; kb < K; kb += NW * RIF) {
+    Pack<VEC> e1[RIF][NIT], e2[RIF][NIT];
+    float c0[RIF], c1[RIF];
+#pragma unroll
+    for (int r = 0; r < RIF; ++r) {
+      const int k = kb + r;
+      if (k < K) {
+        const size_t pair = (size_t)b * K + k;
+        const float* pe = pair_row(table, idx, pair, row_len, n_rows, lane, nullptr);
+        ModelOps<M>::coef(gscore[pair], score[pair], p, c0[r], c1[r]);
+#pragma unroll
+        for (int it = 0; it < NIT; ++it) {
+          const int c = lane + 64 * it;
+          if (c < ncol) {
+            e1[r][it] = load_pack<VEC>(pe, c);
+            if (MUL == 2) e2[r][it] = load_pack<VEC>(pe + dim, c);
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < RIF; ++r) {
+      if (kb + r < K) {
+#pragma unroll
+        for (int it = 0; it < NIT; ++it) {
+          if (lane + 64 * it < ncol) {
+#pragma unroll
+            for (int v = 0; v < VEC; ++v) {
+              const float x1 = reg_apply(e1[r][it].v[v], p);
+              const float x2 = MUL == 2 ? reg_apply(e2[r][it].v[v], p) : 0.f;
+              ModelOps<M>::bwd_q(c0[r], c1[r], x1, x2, q[it][v], g1[it][v], g2[it][v]);
+            }
+          }
+        }
+      }
+    }
+  }
+
+  // wavefront partials -> LDS -> fixed-order sum over wavefronts
+  float* part = lds + NQ * dim;  // [NW][NQ][dim]
+#pragma unroll
+  for (int it = 0; it < NIT; ++it) {
+    const int c = lane + 64 * it;
+    if (c < ncol) {
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) {
+        part[(wave * NQ + 0) * dim + c * VEC + v] = g1[it][v];
+        if (NQ == 2) part[(wave * NQ + 1) * dim + c * VEC + v] = g2[it][v];
+      }
+    }
+  }
+  __syncthreads();
+  for (int d = threadIdx.x; d < dim; d += NW * 64) {
+    float s1 = 0.f, s2 = 0.f;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) {
+      s1 += part[(w * NQ + 0) * dim + d];
+      if (NQ == 2) s2 += part[(w * NQ + 1) * dim + d];
+    }
+    gq1[(size_t)b * dim + d] = s1;
+    if (NQ == 2) gq2[(size_t)b * dim + d] = s2;
+  }
+}
+
+// ---- host dispatch ---------------------------------------------------------------------------
+
+struct ScoreShape {
+  int vec, nit, ncol;
+};
+
+// Picks the column width: float4 columns when rows are 16-byte aligned, single floats otherwise.
+static int pick_shape(size_t dim, int mul, const void* table, const void* qa, const void* qb, ScoreShape* s) {
+  const bool vec4 = dim % 4 == 0 && aligned16(table) && aligned16(qa) && (!qb || aligned16(qb));
+  (void)mul;
+  s->vec = vec4 ? 4 : 1;
+  const size_t ncol = dim / s->vec;
+  if (ncol > 512) return fail(SMX_ERR_SHAPE, "dim %zu not supported by the fused path (at most %d)", dim, 512 * s->vec);
+  s->ncol = (int)ncol;
+  const int need = (int)((ncol + 63) / 64);
+  s->nit = need <= 1 ? 1 : (need <= 2 ? 2 : (need <= 4 ? 4 : 8));
+  return SMX_OK;
+}
+
+static ScoreParams to_params(const smx_score_params* p) {
+  ScoreParams r;
+  r.gamma = p->gamma;
+  r.cen = p->cen;
+  r.reg_on = p->reg_on;
+  r.reg_add = p->reg_add;
+  r.reg_lo = p->reg_lo;
+  r.reg_hi = p->reg_hi;
+  return r;
+}
+
+constexpr int rows_in_flight(int nit, int mul) {
+  const int r = 8 / (nit * mul);
+  return r < 1 ? 1 : (r > 4 ? 4 : r);
+}
+
+template <int M, int VEC, int NIT>
+static int launch_forward(hipStream_t st, const float* table, const int64_t* idx, const float* q1, const float* q2,
+                          float* score, size_t B, size_t K, int ncol, size_t n_rows, const ScoreParams& p, int* err) {
+  constexpr int RIF = rows_in_flight(NIT, model_mul(M));
+  int tile_k = 128;
+  while (tile_k > 4 * RIF && B * ((K + tile_k - 1) / tile_k) < 4096) tile_k /= 2;
+  const int tiles = (int)((K + tile_k - 1) / tile_k);
+  const size_t lds = (size_t)model_nq(M) * ncol * VEC * sizeof(float);
+  hipLaunchKernelGGL((score_forward_kernel<M, VEC, NIT, RIF>), dim3((unsigned)(B * tiles)), dim3(256), lds, st, table,
+                     reinterpret_cast<const long long*>(idx), q1, q2, score, (int)K, ncol, tiles, tile_k,
+                     (unsigned long long)n_rows, p, err);
+  return check_launch("score forward");
+}
+
+template <int M, int VEC, int NIT, int NW>
+static int launch_backward_query(hipStream_t st, const float* table, const int64_t* idx, const float* q1,
+                                 const float* q2, const float* score, const float* gscore, float* gq1, float* gq2,
+                                 size_t B, size_t K, int ncol, size_t n_rows, const ScoreParams& p) {
+  constexpr int RIF = rows_in_flight(NIT, model_mul(M));
+  const size_t lds = (size_t)(NW + 1) * model_nq(M) * ncol * VEC * sizeof(float);
+  hipLaunchKernelGGL((score_backward_query_kernel<M, VEC, NIT, RIF, NW>), dim3((unsigned)B), dim3(NW * 64), lds, st,
+                     table, reinterpret_cast<const long long*>(idx), q1, q2, score, gscore, gq1, gq2, (int)K, ncol,
+                     (unsigned long long)n_rows, p);
+  return check_launch("score backward (query)");
+}
+
+template <int M, int VEC, int NIT>
+static int pick_waves_backward_query(hipStream_t st, const float* table, const int64_t* idx, const float* q1,
+                                     const float* q2, const float* score, const float* gscore, float* gq1, float* gq2,
+                                     size_t B, size_t K, int ncol, size_t n_rows, const ScoreParams& p) {
+  const size_t per_wave = (size_t)model_nq(M) * ncol * VEC * sizeof(float);
+  if (9 * per_wave <= 60 * 1024)
+    return launch_backward_query<M, VEC, NIT, 8>(st, table, idx, q1, q2, score, gscore, gq1, gq2, B, K, ncol, n_rows, p);
+  if (5 * per_wave <= 60 * 1024)
+    return launch_backward_query<M, VEC, NIT, 4>(st, table, idx, q1, q2, score, gscore, gq1, gq2, B, K, ncol, n_rows, p);
+  return launch_backward_query<M, VEC, NIT, 2>(st, table, idx, q1, q2, score, gscore, gq1, gq2, B, K, ncol, n_rows, p);
+}
+
+#define SMX_DISPATCH_NIT(M, VEC, nit, CALL) \
+  switch (nit) {                            \
+    case 1: return CALL(M, VEC, 1);         \
+    case 2: return CALL(M, VEC, 2);         \
+    case 4: return CALL(M, VEC, 4);         \
+    default: return CALL(M, VEC, 8);        \
+  }
+
+#define SMX_DISPATCH_SHAPE(M, shape, CALL)       \
+  if ((shape).vec == 4) {                        \
+    SMX_DISPATCH_NIT(M, 4, (shape).nit, CALL)    \
+  } else {                                       \
+    SMX_DISPATCH_NIT(M, 1, (shape).nit, CALL)    \
+  }
+
+#define SMX_DISPATCH_MODEL(model, shape, CALL)            \
+  switch (model) {                                        \
+    case mL1: SMX_DISPATCH_SHAPE(mL1, shape, CALL)        \
+    case mL2: SMX_DISPATCH_SHAPE(mL2, shape, CALL)        \
+    case mBox: SMX_DISPATCH_SHAPE(mBox, shape, CALL)      \
+    case mRotate: SMX_DISPATCH_SHAPE(mRotate, shape, CALL) \
+    case mBetaKL: SMX_DISPATCH_SHAPE(mBetaKL, shape, CALL) \
+  }
+
+static int check_score_args(int model, const float* table, const float* q1, const float* q2, size_t B, size_t K,
+                            size_t dim, const smx_score_params* params) {
+  if (model < 0 || model >= mNumModels) return fail(SMX_ERR_KIND, "unknown score model %d", model);
+  if (!table || !q1 || !params || (model_nq(model) == 2 && !q2)) return fail(SMX_ERR_ARG, "null pointer");
+  if (B == 0 || K == 0 || dim == 0) return fail(SMX_ERR_SHAPE, "empty dimension");
+  if (B > 0x7fffffffull || K > 0x7fffffffull || B * K > 0x7fffffffull)
+    return fail(SMX_ERR_SHAPE, "more than 2^31-1 pairs in one call");
+  return SMX_OK;
+}
+
+}  // namespace smx
+
+extern "C" {
+
+int smx_score_forward(int model, void* stream, const float* table, size_t n_rows, const int64_t* idx,
+                      const float* q1, const float* q2, float* score, size_t B, size_t K, size_t dim,
+                      const smx_score_params* params, int* err_flag) {
+  using namespace smx;
+  if (int rc = check_score_args(model, table, q1, q2, B, K, dim, params)) return rc;
+  if (!score) return fail(SMX_ERR_ARG, "null score pointer");
+  if (!idx) n_rows = B * K;
+  ScoreShape shape;
+  if (int rc = pick_shape(dim, model_mul(model), table, q1, model_nq(model) == 2 ? q2 : nullptr, &shape)) return rc;
+  const ScoreParams p = to_params(params);
+  hipStream_t st = as_stream(stream);
+#define CALL(M, VEC, NIT) launch_forward<M, VEC, NIT>(st, table, idx, q1, q2, score, B, K, shape.ncol, n_rows, p, err_flag)
+  SMX_DISPATCH_MODEL(model, shape, CALL)
+#undef CALL
+  return fail(SMX_ERR_KIND, "unknown score model %d", model);
+}
+
+int smx_score_backward_query(int model, void* stream, const float* table, size_t n_rows, const int64_t* idx,
+                             const float* q1, const float* q2, const float* score, const float* gscore, float* gq1,
+                             float* gq2, size_t B, size_t K, size_t dim, const smx_score_params* params) {
+  using namespace smx;
+  if (int rc = check_score_args(model, table, q1, q2, B, K, dim, params)) return rc;
+  if (!score || !gscore || !gq1 || (model_nq(model) == 2 && !gq2)) return fail(SMX_ERR_ARG, "null pointer");
+  if (!idx) n_rows = B * K;
+  ScoreShape shape;
+  if (int rc = pick_shape(dim, model_mul(model), table, q1, model_nq(model) == 2 ? q2 : nullptr, &shape)) return rc;
+  const ScoreParams p = to_params(params);
+  hipStream_t st = as_stream(stream);
+#define CALL(M, VEC, NIT) \
+  pick_waves_backward_query<M, VEC, NIT>(st, table, idx, q1, q2, score, gscore, gq1, gq2, B, K, shape.ncol, n_rows, p)
+  SMX_DISPATCH_MODEL(model, shape, CALL)
+#undef CALL
+  return fail(SMX_ERR_KIND, "unknown score model %d", model);
+}
+
+}  // extern "C"

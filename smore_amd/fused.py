@@ -1,0 +1,192 @@
+"""Gather-fused scoring, segment plan and fused entity backward + sparse Adam.
+
+Thin tensor-level front end of the fused entry points of libsmore_amd.so.  The
+reference runs this as separate tensor programs: table[idx]
+(smore/common/embedding/embed_rw.py:74-75), the distance operator
+(smore/common/torchext/dist_func/*.py), gamma - dist (custom_cal_logit of
+smore/models/*.py), and, after loss.backward(), unique / scatter-sum / Adam
+(smore/common/embedding/embed_optimizer.py:39-48, 155-163, 208-252).
+"""
+import ctypes
+
+import torch
+
+from . import _lib
+
+MODELS = {"l1": 0, "l2": 1, "box": 2, "rotate": 3, "beta_kl": 4}
+TWO_HALVES = ("rotate", "beta_kl")
+ONE_QUERY = ("l1", "l2")
+
+
+def _stream(t):
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _ptr(t):
+    return None if t is None else t.data_ptr()
+
+
+def _f32(t, name):
+    if t is None:
+        return
+    if t.dtype != torch.float32 or not t.is_contiguous() or t.device.type != "cuda":
+        raise _lib.SmxError(f"{name} must be a contiguous fp32 device tensor")
+
+
+def score_params(gamma, cen=0.0, regularizer=None):
+    """regularizer: None or (base_add, min_val, max_val) as in smore/common/modules.py:29-36."""
+    if regularizer is None:
+        return _lib.ScoreParams(gamma, cen, 0, 0.0, 0.0, 0.0)
+    add, lo, hi = regularizer
+    return _lib.ScoreParams(gamma, cen, 1, add, lo, hi)
+
+
+def new_error_flag(device):
+    """Device int the kernels set to 1 when they meet an entity id outside the table."""
+    return torch.zeros(1, dtype=torch.int32, device=device)
+
+
+def _dims(model, table, idx, q1, q2):
+    if model not in MODELS:
+        raise _lib.SmxError(f"unknown score model {model}")
+    _f32(table, "table")
+    _f32(q1, "q1")
+    _f32(q2, "q2")
+    if (q2 is None) != (model in ONE_QUERY):
+        raise _lib.SmxError(f"model {model} takes {'one' if model in ONE_QUERY else 'two'} query tensor(s)")
+    mul = 2 if model in TWO_HALVES else 1
+    b, dim = q1.shape[0], q1.shape[-1]
+    if q1.numel() != b * dim or (q2 is not None and q2.shape != q1.shape):
+        raise _lib.SmxError("query tensors must be [B, dim] (or [B, 1, dim])")
+    if table.dim() != 2 or table.shape[1] != dim * mul:
+        raise _lib.SmxError(f"table row length {tuple(table.shape)} does not match dim {dim} x {mul}")
+    if idx is not None:
+        if idx.dtype != torch.int64 or not idx.is_contiguous() or idx.device != table.device:
+            raise _lib.SmxError("idx must be a contiguous int64 tensor on the table's device")
+        if idx.dim() != 2 or idx.shape[0] != b:
+            raise _lib.SmxError("idx must be [B, K]")
+        k = idx.shape[1]
+    else:
+        if table.shape[0] % b:
+            raise _lib.SmxError("dense rows must be [B*K, row]")
+        k = table.shape[0] // b
+    return b, k, dim
+
+
+def score_forward(model, table, idx, q1, q2, params, err_flag=None):
+    """logit[b,k] = gamma - dist(table[idx[b,k]], q[b]).  idx None: table is the dense [B*K, row] rows."""
+    b, k, dim = _dims(model, table, idx, q1, q2)
+    score = torch.empty((b, k), dtype=torch.float32, device=table.device)
+    with torch.cuda.device(table.device):
+        _lib.call("smx_score_forward", MODELS[model], _stream(table), _ptr(table), table.shape[0], _ptr(idx),
+                  _ptr(q1), _ptr(q2), _ptr(score), b, k, dim, ctypes.byref(params), _ptr(err_flag))
+    return score
+
+
+def score_backward_query(model, table, idx, q1, q2, score, gscore, params):
+    """Gradients of sum(gscore * score) w.r.t. q1 (and q2)."""
+    b, k, dim = _dims(model, table, idx, q1, q2)
+    _f32(score, "score")
+    _f32(gscore, "gscore")
+    gq1 = torch.empty_like(q1)
+    gq2 = None if q2 is None else torch.empty_like(q2)
+    with torch.cuda.device(table.device):
+        _lib.call("smx_score_backward_query", MODELS[model], _stream(table), _ptr(table), table.shape[0], _ptr(idx),
+                  _ptr(q1), _ptr(q2), _ptr(score), _ptr(gscore), _ptr(gq1), _ptr(gq2), b, k, dim,
+                  ctypes.byref(params))
+    return gq1, gq2
+
+
+class SegmentPlan:
+    """Device-resident result of grouping one step's pairs by entity id (see smx_plan_build)."""
+
+    def __init__(self, n_pairs, n_rows, device, want_inverse):
+        i32 = dict(dtype=torch.int32, device=device)
+        self.n_pairs, self.n_rows = n_pairs, n_rows
+        self.order = torch.empty(n_pairs, **i32)
+        self.sorted_ids = torch.empty(n_pairs, **i32)
+        self.seg_of_pos = torch.empty(n_pairs, **i32)
+        self.seg_start = torch.empty(n_pairs + 1, **i32)
+        self.uniq_buf = torch.empty(n_pairs, dtype=torch.int64, device=device)
+        self.inverse = torch.empty(n_pairs, dtype=torch.int64, device=device) if want_inverse else None
+        self.n_uniq_dev = torch.zeros(1, **i32)
+        self._n_uniq = None
+
+    @property
+    def n_uniq(self):
+        """Number of distinct ids (first use synchronises with the device)."""
+        if self._n_uniq is None:
+            self._n_uniq = int(self.n_uniq_dev.item())
+        return self._n_uniq
+
+    @property
+    def uniq(self):
+        return self.uniq_buf[: self.n_uniq]
+
+    def view(self):
+        return _lib.PlanView(_ptr(self.order), _ptr(self.sorted_ids), _ptr(self.seg_of_pos), _ptr(self.seg_start),
+                             self.n_pairs)
+
+
+def _workspace(nbytes, device):
+    return torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)
+
+
+def build_plan(idx, n_rows, want_inverse=False, err_flag=None):
+    """Sorts the pairs of idx (any shape, int64, device) by entity id; see SegmentPlan."""
+    if idx.dtype != torch.int64 or idx.device.type != "cuda":
+        raise _lib.SmxError("idx must be an int64 device tensor")
+    flat = idx.reshape(-1).contiguous()
+    n = flat.numel()
+    plan = SegmentPlan(n, n_rows, flat.device, want_inverse)
+    with torch.cuda.device(flat.device):
+        nbytes = _lib.load().smx_plan_workspace_bytes(n, n_rows)
+        if nbytes == 0:
+            raise _lib.SmxError("smx_plan_workspace_bytes failed")
+        ws = _workspace(nbytes, flat.device)
+        _lib.call("smx_plan_build", _stream(flat), _ptr(flat), n, n_rows, _ptr(ws), ws.numel(), _ptr(plan.order),
+                  _ptr(plan.sorted_ids), _ptr(plan.seg_of_pos), _ptr(plan.uniq_buf), _ptr(plan.seg_start),
+                  _ptr(plan.inverse), _ptr(plan.n_uniq_dev), _ptr(err_flag))
+    return plan
+
+
+def adam_params(lr, step, beta1=0.9, beta2=0.999, eps=1e-8):
+    return _lib.AdamParams(lr, beta1, beta2, eps, int(step))
+
+
+def score_backward_entity(model, plan, table, q1, q2, score, gscore, params, merged=None, m=None, v=None, adam=None):
+    """Segmented entity gradient of sum(gscore * score); writes merged [>=U, row] and/or applies lazy Adam
+    to table, m, v in place (all of the table's shape)."""
+    b, dim = q1.shape[0], q1.shape[-1]
+    k = plan.n_pairs // b
+    if model not in MODELS:
+        raise _lib.SmxError(f"unknown score model {model}")
+    for t, name in ((table, "table"), (q1, "q1"), (q2, "q2"), (score, "score"), (gscore, "gscore"),
+                    (merged, "merged"), (m, "m"), (v, "v")):
+        _f32(t, name)
+    row_len = table.shape[1]
+    for s in (m, v):
+        if s is not None and s.shape != table.shape:
+            raise _lib.SmxError("Adam state must have the table's shape")
+    if merged is not None and (merged.dim() != 2 or merged.shape[1] != row_len):
+        raise _lib.SmxError("merged must be [n_uniq or more, row]")
+    with torch.cuda.device(table.device):
+        ws = _workspace(_lib.load().smx_entity_workspace_bytes(plan.n_pairs, row_len), table.device)
+        view = plan.view()
+        _lib.call("smx_score_backward_entity", MODELS[model], _stream(table), ctypes.byref(view), _ptr(table),
+                  table.shape[0], _ptr(q1), _ptr(q2), _ptr(score), _ptr(gscore), b, k, dim, ctypes.byref(params),
+                  _ptr(merged), _ptr(m), _ptr(v), None if adam is None else ctypes.byref(adam), _ptr(ws), ws.numel())
+
+
+def rows_backward(plan, grad_rows, merged=None, table=None, m=None, v=None, adam=None):
+    """Segment sum of materialised gradient rows [P, row] (pair order) and optional lazy Adam."""
+    for t, name in ((grad_rows, "grad_rows"), (merged, "merged"), (table, "table"), (m, "m"), (v, "v")):
+        _f32(t, name)
+    if grad_rows.dim() != 2 or grad_rows.shape[0] != plan.n_pairs:
+        raise _lib.SmxError("grad_rows must be [P, row]")
+    row_len = grad_rows.shape[1]
+    with torch.cuda.device(grad_rows.device):
+        ws = _workspace(_lib.load().smx_entity_workspace_bytes(plan.n_pairs, row_len), grad_rows.device)
+        view = plan.view()
+        _lib.call("smx_rows_backward", _stream(grad_rows), ctypes.byref(view), _ptr(grad_rows), row_len, _ptr(merged),
+                  _ptr(table), _ptr(m), _ptr(v), None if adam is None else ctypes.byref(adam), _ptr(ws), ws.numel())

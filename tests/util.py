@@ -17,13 +17,18 @@ def seed(*parts):
     return zlib.crc32(repr(parts).encode())
 
 
-def assert_close(got, ref, rel, what=""):
+def assert_close(got, ref, rel, what="", sum_abs=None):
+    """sum_abs: for results that are sums of many signed terms, the sum of the terms' magnitudes;
+    one fp32 ulp of it (2^-24 * sum_abs) is added to the bound -- the floor any fp32 summation
+    order has once a long segment cancels to far below its terms."""
     got = np.asarray(got, dtype=np.float64)
     ref = np.asarray(ref, dtype=np.float64)
     assert got.shape == ref.shape, (what, got.shape, ref.shape)
     assert np.all(np.isfinite(got)) or not np.all(np.isfinite(ref)), f"{what}: non-finite output"
     scale = float(np.sqrt(np.mean(ref ** 2))) if ref.size else 0.0
     bound = rel * np.maximum(np.abs(ref), scale) + 1e-300
+    if sum_abs is not None:
+        bound = bound + 2.0 ** -24 * np.asarray(sum_abs, dtype=np.float64)
     err = np.abs(got - ref)
     bad = err > bound
     if bad.any():
