@@ -1,0 +1,278 @@
+"""Benchmark of the scoring hot path on one MI355X.
+
+One "step" = one pass of the hot path over one batch of seeded synthetic input that is already
+resident in HBM: segment plan -> gather-fused score forward -> query backward -> segmented entity
+backward (+ fused sparse Adam where the workload has an optimizer).  Prints ONE JSON line.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 5] [--no-cpu-baseline]
+
+Workloads are the five configurations of BASELINE.json; the default (5) is the one the metric is
+quoted on: box distance + fused sparse Adam on an 86,054,151 x 200 table with Zipf(1.1) ids.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E bandwidth
+
+CONFIGS = {
+    1: dict(name="cfg1-l2-15k", model="l2", n=15_000, dim=200, b=512, k=128, r=0.07, gamma=12.0, cen=0.0,
+            zipf=None, adam=False),
+    2: dict(name="cfg2-box-1m", model="box", n=1_000_000, dim=400, b=1024, k=512, r=0.035, gamma=24.0, cen=0.02,
+            zipf=None, adam=False),
+    3: dict(name="cfg3-rotate-2.5m", model="rotate", n=2_500_000, dim=500, b=1024, k=1024, r=0.028, gamma=9.0,
+            cen=0.0, zipf=None, adam=False),
+    4: dict(name="cfg4-betakl-1m", model="beta_kl", n=1_000_000, dim=400, b=512, k=512, r=None, gamma=60.0, cen=0.0,
+            zipf=None, adam=False),
+    5: dict(name="cfg5-box-adam-86m-zipf1.1", model="box", n=86_054_151, dim=200, b=4096, k=1024, r=0.07, gamma=24.0,
+            cen=0.02, zipf=1.1, adam=True, lr=1e-4),
+}
+
+
+def row_len(cfg):
+    return cfg["dim"] * (2 if cfg["model"] in ("rotate", "beta_kl") else 1)
+
+
+def n_query_tensors(cfg):
+    return 1 if cfg["model"] in ("l1", "l2") else 2
+
+
+def zipf_ids(n, shape, s, gen, device):
+    """Inverse-CDF Zipf(s) over ranks 1..n on a seeded uniform; rank r maps to id r-1 (id 0 hottest)."""
+    import torch
+    w = torch.arange(1, n + 1, dtype=torch.float64, device=device).pow_(-s)
+    cdf = torch.cumsum(w, 0)
+    cdf /= cdf[-1].clone()
+    del w
+    u = torch.rand(shape, dtype=torch.float64, device=device, generator=gen)
+    ids = torch.searchsorted(cdf, u.reshape(-1)).clamp_(max=n - 1).reshape(shape)
+    return ids.contiguous()
+
+
+def make_inputs(cfg, device, seed):
+    import torch
+    gen = torch.Generator(device=device)
+    gen.manual_seed(seed)
+    n, dim, b, k = cfg["n"], cfg["dim"], cfg["b"], cfg["k"]
+    rl = row_len(cfg)
+    if cfg["model"] == "beta_kl":
+        def beta(*shape):
+            x = torch.randn(shape, device=device, generator=gen)
+            return torch.clamp(1 + torch.nn.functional.elu(x), 0.05, 1e9)
+        table, q1, q2 = beta(n, rl), beta(b, dim), beta(b, dim)
+    else:
+        r = cfg["r"]
+        table = torch.empty((n, rl), device=device).uniform_(-r, r, generator=gen)
+        q1 = torch.empty((b, dim), device=device).uniform_(-r, r, generator=gen)
+        q2 = None
+        if n_query_tensors(cfg) == 2:
+            q2 = torch.empty((b, dim), device=device).uniform_(-r, r, generator=gen)
+            if cfg["model"] == "box":
+                q2 = q2.abs_()
+    if cfg["zipf"] is None:
+        idx = torch.randint(0, n, (b, k), device=device, generator=gen, dtype=torch.int64)
+    else:
+        idx = zipf_ids(n, (b, k), cfg["zipf"], gen, device)
+    gscore = torch.randn((b, k), device=device, generator=gen)
+    return table, q1, q2, idx, gscore
+
+
+def algorithmic_bytes(cfg, n_uniq, streaming=False):
+    """Compulsory-traffic model of one step: every distinct touched row crosses
+    HBM once forward and once backward; Adam reads and writes w, m, v of every touched row; ids, scores
+    and upstream gradients once; query tensors read twice and their gradients written once."""
+    p = cfg["b"] * cfg["k"]
+    rows = p if streaming else n_uniq
+    de = row_len(cfg)
+    total = 4 * de * 2 * rows
+    if cfg["adam"]:
+        total += 6 * 4 * de * n_uniq
+    total += p * (8 + 4 + 4)
+    total += 3 * 4 * cfg["b"] * cfg["dim"] * n_query_tensors(cfg)
+    return total
+
+
+def entity_kernel_bytes(cfg, n_uniq):
+    """Algorithmic bytes of the entity pass alone: one read of every distinct row, the upstream gradient of
+    every pair, and (with the optimizer) read + write of w, m, v of every distinct row."""
+    p = cfg["b"] * cfg["k"]
+    de = row_len(cfg)
+    return 4 * de * n_uniq + (6 * 4 * de * n_uniq if cfg["adam"] else 4 * de * n_uniq) + 4 * p
+
+
+class Step:
+    """One pass of the hot path; phases are bracketed by events on the stream the kernels run on."""
+    PHASES = ("plan", "forward", "backward_query", "backward_entity")
+
+    def __init__(self, cfg, table, q1, q2, idx, gscore):
+        import torch
+        from smore_amd import fused
+        self.fused, self.torch = fused, torch
+        self.cfg, self.table, self.q1, self.q2, self.idx, self.gscore = cfg, table, q1, q2, idx, gscore
+        self.params = fused.score_params(cfg["gamma"], cfg["cen"])
+        self.m = torch.zeros_like(table) if cfg["adam"] else None
+        self.v = torch.zeros_like(table) if cfg["adam"] else None
+        self.merged = None
+        self.step_no = 0
+        self.err = fused.new_error_flag(table.device)
+        self.plan = None
+
+    def run(self, events=None):
+        f, cfg = self.fused, self.cfg
+        mark = (lambda i: events[i].record()) if events is not None else (lambda i: None)
+        self.step_no += 1
+        mark(0)
+        plan = f.build_plan(self.idx, cfg["n"], err_flag=self.err)
+        mark(1)
+        score = f.score_forward(cfg["model"], self.table, self.idx, self.q1, self.q2, self.params, self.err)
+        mark(2)
+        gq = f.score_backward_query(cfg["model"], self.table, self.idx, self.q1, self.q2, score, self.gscore,
+                                    self.params)
+        mark(3)
+        if cfg["adam"]:
+            f.score_backward_entity(cfg["model"], plan, self.table, self.q1, self.q2, score, self.gscore, self.params,
+                                    m=self.m, v=self.v, adam=f.adam_params(cfg["lr"], self.step_no))
+        else:
+            if self.merged is None:
+                self.merged = self.torch.empty((plan.n_uniq, self.table.shape[1]), device=self.table.device)
+            f.score_backward_entity(cfg["model"], plan, self.table, self.q1, self.q2, score, self.gscore, self.params,
+                                    merged=self.merged)
+        mark(4)
+        self.plan = plan
+        return score, gq
+
+
+def cpu_baseline(cfg, seed):
+    """Times the CPU oracle (fp32 build, OpenMP) on a bounded sample of the same workload: same row length,
+    K, id distribution and optimizer, fewer queries and -- for the 86M-row table -- fewer rows."""
+    import numpy as np
+    from oracle import oracle as orc
+    cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+    rng = np.random.default_rng(seed)
+    n = min(cfg["n"], 2_000_000)
+    b = min(cfg["b"], 256)
+    k, dim, rl = cfg["k"], cfg["dim"], row_len(cfg)
+    f32 = np.float32
+    if cfg["model"] == "beta_kl":
+        def beta(*s):
+            x = rng.standard_normal(s, dtype=f32)
+            return np.clip(1 + np.where(x > 0, x, np.expm1(x)), 0.05, 1e9).astype(f32)
+        table, q1, q2 = beta(n, rl), beta(b, 1, dim), beta(b, 1, dim)
+    else:
+        r = cfg["r"]
+        table = rng.uniform(-r, r, (n, rl)).astype(f32)
+        q1 = rng.uniform(-r, r, (b, 1, dim)).astype(f32)
+        q2 = None
+        if n_query_tensors(cfg) == 2:
+            q2 = rng.uniform(-r, r, (b, 1, dim)).astype(f32)
+            if cfg["model"] == "box":
+                q2 = np.abs(q2)
+    if cfg["zipf"] is None:
+        idx = rng.integers(0, n, (b, k))
+    else:
+        w = np.arange(1, n + 1, dtype=np.float64) ** -cfg["zipf"]
+        cdf = np.cumsum(w)
+        cdf /= cdf[-1]
+        idx = np.minimum(np.searchsorted(cdf, rng.random((b, k))), n - 1)
+    gs = rng.standard_normal((b, k)).astype(f32)
+    m = np.zeros_like(table) if cfg["adam"] else None
+    v = np.zeros_like(table) if cfg["adam"] else None
+    times = []
+    for step in range(1, 4):
+        t0 = time.perf_counter()
+        orc.train_step(cfg["model"], table, m, v, idx, q1, q2, gs, cfg["gamma"], cfg["cen"], cfg.get("lr", 0.0), step,
+                       dtype=f32, apply_adam=cfg["adam"])
+        times.append(time.perf_counter() - t0)
+    best = sorted(times)[len(times) // 2]
+    return {
+        "value": b * k / best, "unit": "pairs/s", "cores": cores, "kind": "port",
+        "sample": f"oracle fp32 (C, OpenMP x{cores}), same model/K/D/id distribution, B={b}, N={n}, "
+                  f"median of {len(times)} steps of {best * 1e3:.0f} ms",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--config", type=int, default=5, choices=sorted(CONFIGS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--seed", type=int, default=None)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
+
+    import torch
+    from smore_amd import _lib
+    _lib.load()  # fails loudly if the HIP library is not built
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+    device = torch.device("cuda:0")
+    cfg = CONFIGS[args.config]
+    seed = args.seed if args.seed is not None else 20240 + args.config
+
+    table, q1, q2, idx, gscore = make_inputs(cfg, device, seed)
+    step = Step(cfg, table, q1, q2, idx, gscore)
+    for _ in range(args.warmup):
+        step.run()
+    torch.cuda.synchronize()
+    n_uniq = step.plan.n_uniq
+    if step.err.item() != 0:
+        sys.exit("entity id out of range in the synthetic batch")
+
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(5)] for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for s in range(args.steps):
+        step.run(ev[s])
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+
+    phase_ms = {name: sum(e[i].elapsed_time(e[i + 1]) for e in ev) / args.steps for i, name in enumerate(Step.PHASES)}
+    ms_per_step = wall * 1e3 / args.steps
+    pairs = cfg["b"] * cfg["k"]
+    algo = algorithmic_bytes(cfg, n_uniq)
+    algo_stream = algorithmic_bytes(cfg, n_uniq, streaming=True)
+    ent_bytes = entity_kernel_bytes(cfg, n_uniq)
+    ent_gbps = ent_bytes / (phase_ms["backward_entity"] * 1e-3) / 1e9
+
+    out = {
+        "metric": "scored (query,neg) pairs/sec fwd+bwd+opt; achieved HBM GB/s vs peak",
+        "value": pairs / (ms_per_step * 1e-3),
+        "unit": "pairs/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": cfg["name"], "model": None, "N": cfg["n"], "row_len": row_len(cfg), "B": cfg["b"],
+                   "K": cfg["k"], "ids": "zipf(1.1)" if cfg["zipf"] else "uniform", "optimizer": "sparse adam" if
+                   cfg["adam"] else None, "seed": seed, "distinct_ids": n_uniq},
+        "roofline": {
+            "bound": "hbm", "kernel": "entity_tile_kernel (+fixup): segmented entity gradient" +
+                     (" + fused sparse Adam" if cfg["adam"] else ""),
+            "achieved": ent_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": ent_gbps / HBM_PEAK_GBPS,
+            "traffic": None, "algorithmic_bytes": ent_bytes, "avg_ms": phase_ms["backward_entity"],
+        },
+        "step_hbm": {
+            "algorithmic_bytes": algo, "achieved_GBps": algo / (ms_per_step * 1e-3) / 1e9,
+            "frac_of_peak": algo / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+            "streaming_bytes": algo_stream,
+            "streaming_GBps": algo_stream / (ms_per_step * 1e-3) / 1e9,
+        },
+        "phase_ms": phase_ms,
+    }
+    del out["config"]["model"]
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(cfg, seed)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()
