@@ -142,6 +142,8 @@ typedef struct smx_plan_view {
   const int32_t* sorted_ids;
   const int32_t* seg_of_pos;
   const int32_t* seg_start;
+  const int64_t* uniq;
+  const int32_t* n_uniq; /* device scalar */
   size_t n_pairs;
 } smx_plan_view;
 

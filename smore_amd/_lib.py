@@ -57,7 +57,8 @@ class AdamParams(ctypes.Structure):
 
 class PlanView(ctypes.Structure):
     """smx_plan_view of include/smore_amd.h."""
-    _fields_ = [("order", _vp), ("sorted_ids", _vp), ("seg_of_pos", _vp), ("seg_start", _vp), ("n_pairs", _sz)]
+    _fields_ = [("order", _vp), ("sorted_ids", _vp), ("seg_of_pos", _vp), ("seg_start", _vp), ("uniq", _vp),
+                ("n_uniq", _vp), ("n_pairs", _sz)]
 
 _lib = None
 

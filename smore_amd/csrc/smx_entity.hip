@@ -46,8 +46,11 @@ struct EntityArgs {
   const int* sorted_ids;
   const int* seg_of_pos;
   const int* seg_start;
+  const long long* uniq;
+  const int* n_uniq;
   int n_pairs;
-  int tile;  // sorted positions per tile, multiple of 64
+  int tile;        // sorted positions per tile of the long-segment pass, multiple of 64
+  int short_max;   // segments of at most this many pairs are finished by one wavefront
   // source: score model
   const float* q1;
   const float* q2;
@@ -55,6 +58,8 @@ struct EntityArgs {
   const float* gscore;
   int K;
   ScoreParams p;
+  float* meta_c;  // [P] upstream coefficient of every sorted position
+  int* meta_b;    // [P] query number of every sorted position
   // source: gradient rows
   const float* grad_rows;
   // entity table (read for the model sources, updated when adam_on)
@@ -97,30 +102,91 @@ __device__ __forceinline__ void st(float* __restrict__ base, int col, const floa
   }
 }
 
-// Finishes one entity row: optional clamp mask, optional merged-gradient store, optional Adam.
-// g1/g2 are the lane's columns of the summed gradient of the first / second half row.
-template <int SRC, int VEC, int NIT>
+// The lane's columns of one table row (both halves for the two-half models).
+template <int MUL, int VEC, int NIT> struct RowRegs {
+  Pack2<VEC> h[MUL][NIT];
+};
+
+template <int MUL, int VEC, int NIT>
+__device__ __forceinline__ void load_row(RowRegs<MUL, VEC, NIT>& r, const float* __restrict__ base, int half, int ncol,
+                                         int lane) {
+#pragma unroll
+  for (int h = 0; h < MUL; ++h)
+#pragma unroll
+    for (int it = 0; it < NIT; ++it) r.h[h][it] = ld<VEC>(base + h * half, min(lane + 64 * it, ncol - 1));
+}
+
+// Coefficient on the second accumulator (BOX: inside distance) from the first.
+template <int SRC>
+__device__ __forceinline__ float second_coef(float c0, const ScoreParams& p) {
+  return SRC == mBox ? p.cen * c0 : 0.f;
+}
+
+// Adds the gradient of one run -- pairs of one segment that share query b, coefficients already
+// summed into c0 -- to the lane's accumulators.
+template <int SRC, int VEC, int NIT, bool REG>
+__device__ __forceinline__ void add_run(const EntityArgs& A, int lane, int b, float c0,
+                                        const RowRegs<src_mul(SRC), VEC, NIT>& e, float (&g1)[NIT][VEC],
+                                        float (&g2)[NIT][VEC]) {
+  if constexpr (SRC != kSrcRows) {
+    constexpr int MUL = src_mul(SRC);
+    const int half = A.ncol * VEC;
+    const float c1 = second_coef<SRC>(c0, A.p);
+    const float* pq1 = A.q1 + (size_t)b * half;
+    const float* pq2 = model_nq(SRC) == 2 ? A.q2 + (size_t)b * half : pq1;
+    Pack2<VEC> qa[NIT], qb[NIT];
+#pragma unroll
+    for (int it = 0; it < NIT; ++it) {
+      const int c = min(lane + 64 * it, A.ncol - 1);
+      qa[it] = ld<VEC>(pq1, c);
+      if (model_nq(SRC) == 2) qb[it] = ld<VEC>(pq2, c);
+    }
+#pragma unroll
+    for (int it = 0; it < NIT; ++it) {
+#pragma unroll
+      for (int x = 0; x < VEC; ++x) {
+        const typename ModelOps<SRC>::Q q = ModelOps<SRC>::prep(qa[it].v[x], model_nq(SRC) == 2 ? qb[it].v[x] : 0.f);
+        const float x1 = REG ? reg_apply(e.h[0][it].v[x], A.p) : e.h[0][it].v[x];
+        const float x2 = MUL == 2 ? (REG ? reg_apply(e.h[MUL - 1][it].v[x], A.p) : e.h[MUL - 1][it].v[x]) : 0.f;
+        ModelOps<SRC>::bwd_e(c0, c1, x1, x2, q, g1[it][x], g2[it][x]);
+      }
+    }
+  }
+}
+
+// Adds one materialised gradient row.
+template <int VEC, int NIT>
+__device__ __forceinline__ void add_grad_row(const EntityArgs& A, int lane, int pair, float (&g1)[NIT][VEC]) {
+  const float* pg = A.grad_rows + (size_t)pair * A.ncol * VEC;
+  Pack2<VEC> r[NIT];
+#pragma unroll
+  for (int it = 0; it < NIT; ++it) r[it] = ld<VEC>(pg, min(lane + 64 * it, A.ncol - 1));
+#pragma unroll
+  for (int it = 0; it < NIT; ++it)
+#pragma unroll
+    for (int x = 0; x < VEC; ++x) g1[it][x] += r[it].v[x];
+}
+
+// Finishes one entity row: clamp mask, merged-gradient store, Adam.  g1/g2 are the lane's columns of
+// the summed gradient of the first / second half row; w, m0, v0 the row's current weights and moments
+// (w is always valid for the model sources -- it is the entity row the gradient was computed from).
+template <int SRC, int VEC, int NIT, bool REG>
 __device__ __forceinline__ void finish_row(const EntityArgs& A, int lane, unsigned row_id, int seg,
-                                           float (&g1)[NIT][VEC], float (&g2)[NIT][VEC]) {
+                                           float (&g1)[NIT][VEC], float (&g2)[NIT][VEC],
+                                           const RowRegs<src_mul(SRC), VEC, NIT>& w,
+                                           const RowRegs<src_mul(SRC), VEC, NIT>& m0,
+                                           const RowRegs<src_mul(SRC), VEC, NIT>& v0) {
   constexpr int MUL = src_mul(SRC);
   const int half = A.ncol * VEC;
   const size_t row_len = (size_t)half * MUL;
-  float* w = A.table + (size_t)row_id * row_len;
-  if (SRC != kSrcRows && A.p.reg_on) {
+  if (REG) {
 #pragma unroll
-    for (int it = 0; it < NIT; ++it) {
-      const int c = lane + 64 * it;
-      if (c < A.ncol) {
-        const Pack2<VEC> e1 = ld<VEC>(w, c);
+    for (int it = 0; it < NIT; ++it)
 #pragma unroll
-        for (int x = 0; x < VEC; ++x) g1[it][x] = reg_mask(e1.v[x], g1[it][x], A.p);
-        if (MUL == 2) {
-          const Pack2<VEC> e2 = ld<VEC>(w + half, c);
-#pragma unroll
-          for (int x = 0; x < VEC; ++x) g2[it][x] = reg_mask(e2.v[x], g2[it][x], A.p);
-        }
+      for (int x = 0; x < VEC; ++x) {
+        g1[it][x] = reg_mask(w.h[0][it].v[x], g1[it][x], A.p);
+        if (MUL == 2) g2[it][x] = reg_mask(w.h[MUL - 1][it].v[x], g2[it][x], A.p);
       }
-    }
   }
   if (A.merged) {
     float* out = A.merged + (size_t)seg * row_len;
@@ -134,29 +200,27 @@ __device__ __forceinline__ void finish_row(const EntityArgs& A, int lane, unsign
     }
   }
   if (A.adam_on) {
-    float* mm = A.m + (size_t)row_id * row_len;
-    float* vv = A.v + (size_t)row_id * row_len;
+    float* pw = A.table + (size_t)row_id * row_len;
+    float* pm = A.m + (size_t)row_id * row_len;
+    float* pv = A.v + (size_t)row_id * row_len;
 #pragma unroll
     for (int h = 0; h < MUL; ++h) {
 #pragma unroll
       for (int it = 0; it < NIT; ++it) {
         const int c = lane + 64 * it;
         if (c < A.ncol) {
-          const Pack2<VEC> w0 = ld<VEC>(w + h * half, c);
-          const Pack2<VEC> m0 = ld<VEC>(mm + h * half, c);
-          const Pack2<VEC> v0 = ld<VEC>(vv + h * half, c);
           float wn[VEC], mn[VEC], vn[VEC];
 #pragma unroll
           for (int x = 0; x < VEC; ++x) {
             const float g = h == 0 ? g1[it][x] : g2[it][x];
-            mn[x] = m0.v[x] * A.a.beta1 + g * A.a.omb1;
-            vn[x] = v0.v[x] * A.a.beta2 + g * g * A.a.omb2;
+            mn[x] = m0.h[h][it].v[x] * A.a.beta1 + g * A.a.omb1;
+            vn[x] = v0.h[h][it].v[x] * A.a.beta2 + g * g * A.a.omb2;
             const float denom = sqrtf(vn[x]) * A.a.inv_sqrt_bc2 + A.a.eps;
-            wn[x] = w0.v[x] + A.a.step_size * mn[x] / denom;
+            wn[x] = w.h[h][it].v[x] + A.a.step_size * mn[x] / denom;
           }
-          st<VEC>(w + h * half, c, wn);
-          st<VEC>(mm + h * half, c, mn);
-          st<VEC>(vv + h * half, c, vn);
+          st<VEC>(pw + h * half, c, wn);
+          st<VEC>(pm + h * half, c, mn);
+          st<VEC>(pv + h * half, c, vn);
         }
       }
     }
@@ -179,7 +243,90 @@ __device__ __forceinline__ void store_partial(const EntityArgs& A, float* buf, i
   }
 }
 
-template <int SRC, int VEC, int NIT>
+template <int VEC, int NIT>
+__device__ __forceinline__ void zero_acc(float (&g1)[NIT][VEC], float (&g2)[NIT][VEC]) {
+#pragma unroll
+  for (int it = 0; it < NIT; ++it)
+#pragma unroll
+    for (int x = 0; x < VEC; ++x) g1[it][x] = g2[it][x] = 0.f;
+}
+
+// Sorted copy of what the entity pass needs per pair, so that the pass reads it contiguously:
+// meta_c[pos] = d loss / d distance of the pair at sorted position pos, meta_b[pos] = its query.
+template <int SRC>
+__global__ __launch_bounds__(256) void entity_meta_kernel(EntityArgs A) {
+  const int pos = blockIdx.x * blockDim.x + threadIdx.x;
+  if (pos >= A.n_pairs) return;
+  if constexpr (SRC != kSrcRows) {
+    const int pair = A.order[pos];
+    float c0, c1;
+    ModelOps<SRC>::coef(A.gscore[pair], A.score[pair], A.p, c0, c1);
+    A.meta_c[pos] = c0;
+    A.meta_b[pos] = pair / A.K;
+  }
+}
+
+// Walks `len` sorted positions starting at `first` that all belong to one segment and adds their
+// gradient to g1/g2: run by run for the model sources, row by row for materialised gradients.
+template <int SRC, int VEC, int NIT, bool REG>
+__device__ __forceinline__ void add_positions(const EntityArgs& A, int lane, int first, int len,
+                                              const RowRegs<src_mul(SRC), VEC, NIT>& e, float (&g1)[NIT][VEC],
+                                              float (&g2)[NIT][VEC]) {
+  for (int base = 0; base < len; base += 64) {
+    const int n = min(64, len - base);
+    const int pos = first + base + min(lane, n - 1);
+    if constexpr (SRC == kSrcRows) {
+      const int my_pair = A.order[pos];
+      for (int j = 0; j < n; ++j) add_grad_row<VEC, NIT>(A, lane, __builtin_amdgcn_readlane(my_pair, j), g1);
+    } else {
+      const float my_c = A.meta_c[pos];
+      const int my_b = A.meta_b[pos];
+      int j = 0;
+      while (j < n) {
+        const int bj = __builtin_amdgcn_readlane(my_b, j);
+        float c0 = 0.f;
+        do {  // pairs that share query bj: the gradient is linear in the coefficient, sum it first
+          c0 += __int_as_float(__builtin_amdgcn_readlane(__float_as_int(my_c), j));
+          ++j;
+        } while (j < n && __builtin_amdgcn_readlane(my_b, j) == bj);
+        add_run<SRC, VEC, NIT, REG>(A, lane, bj, c0, e, g1, g2);
+      }
+    }
+  }
+}
+
+// Short segments (at most A.short_max pairs): one wavefront per segment, grid-stride over segments.
+template <int SRC, int VEC, int NIT, bool REG>
+__global__ __launch_bounds__(256) void entity_segment_kernel(EntityArgs A) {
+  constexpr int MUL = src_mul(SRC);
+  const int lane = threadIdx.x & 63;
+  const int wave = uniform(threadIdx.x >> 6);
+  const int n_waves = gridDim.x * 4;
+  const int n_uniq = *A.n_uniq;
+  const int half = A.ncol * VEC;
+  const size_t row_len = (size_t)half * MUL;
+  for (int u = blockIdx.x * 4 + wave; u < n_uniq; u += n_waves) {
+    const int s0 = A.seg_start[u], s1 = A.seg_start[u + 1];
+    if (s1 - s0 > A.short_max) continue;
+    const unsigned row_id = (unsigned)A.uniq[u];
+    RowRegs<MUL, VEC, NIT> e, m0, v0;
+    if (SRC != kSrcRows || A.adam_on) load_row<MUL, VEC, NIT>(e, A.table + (size_t)row_id * row_len, half, A.ncol, lane);
+    if (A.adam_on) {
+      load_row<MUL, VEC, NIT>(m0, A.m + (size_t)row_id * row_len, half, A.ncol, lane);
+      load_row<MUL, VEC, NIT>(v0, A.v + (size_t)row_id * row_len, half, A.ncol, lane);
+    }
+    float g1[NIT][VEC], g2[NIT][VEC];
+    zero_acc<VEC, NIT>(g1, g2);
+    add_positions<SRC, VEC, NIT, REG>(A, lane, s0, s1 - s0, e, g1, g2);
+    finish_row<SRC, VEC, NIT, REG>(A, lane, row_id, u, g1, g2, e, m0, v0);
+  }
+}
+
+// Long segments: the sorted pair list is cut into fixed tiles, one wavefront per tile.  The part of a
+// long segment inside the tile is summed; a segment that lies wholly inside the tile is finished here,
+// otherwise the sum goes to the tile's tail row (segment continues past the tile end) or head row
+// (segment came in from the left and ends here).
+template <int SRC, int VEC, int NIT, bool REG>
 __global__ __launch_bounds__(256) void entity_tile_kernel(EntityArgs A) {
   constexpr int MUL = src_mul(SRC);
   const int lane = threadIdx.x & 63;
@@ -191,112 +338,48 @@ __global__ __launch_bounds__(256) void entity_tile_kernel(EntityArgs A) {
   const int half = A.ncol * VEC;
   const size_t row_len = (size_t)half * MUL;
 
-  float g1[NIT][VEC], g2[NIT][VEC];
-  Pack2<VEC> e1[NIT], e2[NIT];
-  int cur_seg = -1;
-  unsigned cur_id = 0;
-
-  auto zero_acc = [&]() {
-#pragma unroll
-    for (int it = 0; it < NIT; ++it)
-#pragma unroll
-      for (int x = 0; x < VEC; ++x) g1[it][x] = g2[it][x] = 0.f;
-  };
-  auto flush = [&]() {
-    const bool open_left = A.seg_start[cur_seg] < p0;
-    const bool closed_right = A.seg_start[cur_seg + 1] <= p1;
-    if (!closed_right)
-      store_partial<SRC, VEC, NIT>(A, A.tail, t, lane, g1, g2);
-    else if (open_left)
-      store_partial<SRC, VEC, NIT>(A, A.head, t, lane, g1, g2);
-    else
-      finish_row<SRC, VEC, NIT>(A, lane, cur_id, cur_seg, g1, g2);
-  };
-
+  // most tiles hold short segments only: find that out with one parallel look and leave
+  bool any_long = false;
   for (int base = p0; base < p1; base += 64) {
-    const int pos = base + lane;
-    const bool valid = pos < p1;
-    const int my_seg = valid ? A.seg_of_pos[pos] : -1;
-    const int my_id = valid ? A.sorted_ids[pos] : 0;
-    const int my_pair = valid ? A.order[pos] : 0;
-    float my_c0 = 0.f, my_c1 = 0.f;
-    int my_b = 0;
-    if (SRC != kSrcRows) {
-      if (valid) {
-        if constexpr (SRC != kSrcRows) ModelOps<SRC>::coef(A.gscore[my_pair], A.score[my_pair], A.p, my_c0, my_c1);
-        my_b = my_pair / A.K;
-      }
-    }
-    const int n = min(64, p1 - base);
-    int j = 0;
-    while (j < n) {
-      const int sj = __builtin_amdgcn_readlane(my_seg, j);
-      if (sj != cur_seg) {
-        if (cur_seg >= 0) flush();
-        cur_seg = sj;
-        cur_id = (unsigned)__builtin_amdgcn_readlane(my_id, j);
-        zero_acc();
-        if (SRC != kSrcRows) {
-          const float* pe = A.table + (size_t)cur_id * row_len;
-#pragma unroll
-          for (int it = 0; it < NIT; ++it) {
-            const int c = lane + 64 * it;
-            if (c < A.ncol) {
-              e1[it] = ld<VEC>(pe, c);
-              if (MUL == 2) e2[it] = ld<VEC>(pe + half, c);
-            }
-          }
-        }
-      }
-      if constexpr (SRC == kSrcRows) {
-        const int pj = __builtin_amdgcn_readlane(my_pair, j);
-        const float* pg = A.grad_rows + (size_t)pj * row_len;
-#pragma unroll
-        for (int it = 0; it < NIT; ++it) {
-          const int c = lane + 64 * it;
-          if (c < A.ncol) {
-            const Pack2<VEC> r = ld<VEC>(pg, c);
-#pragma unroll
-            for (int x = 0; x < VEC; ++x) g1[it][x] += r.v[x];
-          }
-        }
-        ++j;
-      } else {
-        const int bj = __builtin_amdgcn_readlane(my_b, j);
-        float c0 = 0.f, c1 = 0.f;
-        do {  // pairs of this segment that share query bj: sum their coefficients first
-          c0 += __int_as_float(__builtin_amdgcn_readlane(__float_as_int(my_c0), j));
-          c1 += __int_as_float(__builtin_amdgcn_readlane(__float_as_int(my_c1), j));
-          ++j;
-        } while (j < n && __builtin_amdgcn_readlane(my_seg, j) == sj && __builtin_amdgcn_readlane(my_b, j) == bj);
-        const float* pq1 = A.q1 + (size_t)bj * half;
-        const float* pq2 = model_nq(SRC) == 2 ? A.q2 + (size_t)bj * half : pq1;
-#pragma unroll
-        for (int it = 0; it < NIT; ++it) {
-          const int c = lane + 64 * it;
-          if (c < A.ncol) {
-            const Pack2<VEC> a = ld<VEC>(pq1, c);
-            Pack2<VEC> b = a;
-            if (model_nq(SRC) == 2) b = ld<VEC>(pq2, c);
-#pragma unroll
-            for (int x = 0; x < VEC; ++x) {
-              const typename ModelOps<SRC>::Q q = ModelOps<SRC>::prep(a.v[x], b.v[x]);
-              const float x1 = reg_apply(e1[it].v[x], A.p);
-              const float x2 = MUL == 2 ? reg_apply(e2[it].v[x], A.p) : 0.f;
-              ModelOps<SRC>::bwd_e(c0, c1, x1, x2, q, g1[it][x], g2[it][x]);
-            }
-          }
-        }
-      }
-    }
+    const int q = min(base + lane, p1 - 1);
+    const int sg = A.seg_of_pos[q];
+    any_long |= __ballot(A.seg_start[sg + 1] - A.seg_start[sg] > A.short_max) != 0ull;
   }
-  if (cur_seg >= 0) flush();
+  if (!any_long) return;
+
+  int pos = p0;
+  while (pos < p1) {
+    const int seg = A.seg_of_pos[pos];
+    const int s0 = A.seg_start[seg], s1 = A.seg_start[seg + 1];
+    const int end = min(s1, p1);
+    if (s1 - s0 > A.short_max) {
+      const unsigned row_id = (unsigned)A.sorted_ids[pos];
+      const bool whole = s0 >= p0 && s1 <= p1;
+      RowRegs<MUL, VEC, NIT> e, m0, v0;
+      if (SRC != kSrcRows || (whole && A.adam_on))
+        load_row<MUL, VEC, NIT>(e, A.table + (size_t)row_id * row_len, half, A.ncol, lane);
+      if (whole && A.adam_on) {
+        load_row<MUL, VEC, NIT>(m0, A.m + (size_t)row_id * row_len, half, A.ncol, lane);
+        load_row<MUL, VEC, NIT>(v0, A.v + (size_t)row_id * row_len, half, A.ncol, lane);
+      }
+      float g1[NIT][VEC], g2[NIT][VEC];
+      zero_acc<VEC, NIT>(g1, g2);
+      add_positions<SRC, VEC, NIT, REG>(A, lane, pos, end - pos, e, g1, g2);
+      if (whole)
+        finish_row<SRC, VEC, NIT, REG>(A, lane, row_id, seg, g1, g2, e, m0, v0);
+      else if (s1 > p1)
+        store_partial<SRC, VEC, NIT>(A, A.tail, t, lane, g1, g2);
+      else
+        store_partial<SRC, VEC, NIT>(A, A.head, t, lane, g1, g2);
+    }
+    pos = end;
+  }
 }
 
-// One workgroup per tile whose first segment came in from the left and ends inside the tile:
+// One workgroup per tile whose first segment is long, came in from the left and ends inside the tile:
 // adds that segment's partial rows (tails of the tiles it crossed, then this tile's head) in tile
 // order and finishes the row.  Every other workgroup leaves at once.
-template <int SRC, int VEC, int NIT, int NW>
+template <int SRC, int VEC, int NIT, int NW, bool REG>
 __global__ __launch_bounds__(NW * 64) void entity_fixup_kernel(EntityArgs A) {
   constexpr int MUL = src_mul(SRC);
   extern __shared__ float lds[];
@@ -306,7 +389,7 @@ __global__ __launch_bounds__(NW * 64) void entity_fixup_kernel(EntityArgs A) {
   const int p1 = min(A.n_pairs, p0 + A.tile);
   const int seg = A.seg_of_pos[p0];
   const int s0 = A.seg_start[seg], s1 = A.seg_start[seg + 1];
-  if (!(s0 < p0 && s1 <= p1)) return;  // uniform over the workgroup
+  if (!(s0 < p0 && s1 <= p1 && s1 - s0 > A.short_max)) return;  // uniform over the workgroup
   const int lane = threadIdx.x & 63;
   const int wave = uniform(threadIdx.x >> 6);
   const int half = A.ncol * VEC;
@@ -317,79 +400,95 @@ __global__ __launch_bounds__(NW * 64) void entity_fixup_kernel(EntityArgs A) {
   const int j0 = wave * per_wave;
   const int j1 = min(n_parts, j0 + per_wave);
 
+  // four interleaved partial sums per wavefront keep four row loads in flight; they are folded in a
+  // fixed order, so the result depends only on the tiling
+  float acc[4][MUL][NIT][VEC];
+#pragma unroll
+  for (int k = 0; k < 4; ++k)
+#pragma unroll
+    for (int h = 0; h < MUL; ++h)
+#pragma unroll
+      for (int it = 0; it < NIT; ++it)
+#pragma unroll
+        for (int x = 0; x < VEC; ++x) acc[k][h][it][x] = 0.f;
+  for (int j = j0; j < j1; j += 4) {
+    RowRegs<MUL, VEC, NIT> r[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int tj = ts + min(j + k, j1 - 1);
+      load_row<MUL, VEC, NIT>(r[k], (tj < t ? A.tail : A.head) + (size_t)tj * row_len, half, A.ncol, lane);
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      if (j + k < j1) {
+#pragma unroll
+        for (int h = 0; h < MUL; ++h)
+#pragma unroll
+          for (int it = 0; it < NIT; ++it)
+#pragma unroll
+            for (int x = 0; x < VEC; ++x) acc[k][h][it][x] += r[k].h[h][it].v[x];
+      }
+    }
+  }
   float g1[NIT][VEC], g2[NIT][VEC];
 #pragma unroll
   for (int it = 0; it < NIT; ++it)
 #pragma unroll
-    for (int x = 0; x < VEC; ++x) g1[it][x] = g2[it][x] = 0.f;
-  for (int j = j0; j < j1; ++j) {
-    const int tj = ts + j;
-    const float* src = (tj < t ? A.tail : A.head) + (size_t)tj * row_len;
-#pragma unroll
-    for (int it = 0; it < NIT; ++it) {
-      const int c = lane + 64 * it;
-      if (c < A.ncol) {
-        const Pack2<VEC> r1 = ld<VEC>(src, c);
-#pragma unroll
-        for (int x = 0; x < VEC; ++x) g1[it][x] += r1.v[x];
-        if (MUL == 2) {
-          const Pack2<VEC> r2 = ld<VEC>(src + half, c);
-#pragma unroll
-          for (int x = 0; x < VEC; ++x) g2[it][x] += r2.v[x];
-        }
-      }
+    for (int x = 0; x < VEC; ++x) {
+      g1[it][x] = (acc[0][0][it][x] + acc[1][0][it][x]) + (acc[2][0][it][x] + acc[3][0][it][x]);
+      g2[it][x] = MUL == 2 ? (acc[0][MUL - 1][it][x] + acc[1][MUL - 1][it][x]) +
+                                 (acc[2][MUL - 1][it][x] + acc[3][MUL - 1][it][x])
+                           : 0.f;
     }
-  }
   // combine the wavefront sums in wavefront order
-  if (wave > 0) {
-    float* mine = lds + (size_t)(wave - 1) * row_len;
-#pragma unroll
-    for (int it = 0; it < NIT; ++it) {
-      const int c = lane + 64 * it;
-      if (c < A.ncol) {
-        st<VEC>(mine, c, g1[it]);
-        if (MUL == 2) st<VEC>(mine + half, c, g2[it]);
-      }
-    }
-  }
+  if (wave > 0) store_partial<SRC, VEC, NIT>(A, lds, wave - 1, lane, g1, g2);
   __syncthreads();
   if (wave == 0) {
     for (int w = 1; w < NW; ++w) {
-      const float* other = lds + (size_t)(w - 1) * row_len;
+      RowRegs<MUL, VEC, NIT> o;
+      load_row<MUL, VEC, NIT>(o, lds + (size_t)(w - 1) * row_len, half, A.ncol, lane);
 #pragma unroll
-      for (int it = 0; it < NIT; ++it) {
-        const int c = lane + 64 * it;
-        if (c < A.ncol) {
-          const Pack2<VEC> r1 = ld<VEC>(other, c);
+      for (int it = 0; it < NIT; ++it)
 #pragma unroll
-          for (int x = 0; x < VEC; ++x) g1[it][x] += r1.v[x];
-          if (MUL == 2) {
-            const Pack2<VEC> r2 = ld<VEC>(other + half, c);
-#pragma unroll
-            for (int x = 0; x < VEC; ++x) g2[it][x] += r2.v[x];
-          }
+        for (int x = 0; x < VEC; ++x) {
+          g1[it][x] += o.h[0][it].v[x];
+          if (MUL == 2) g2[it][x] += o.h[MUL - 1][it].v[x];
         }
-      }
     }
-    finish_row<SRC, VEC, NIT>(A, lane, (unsigned)A.sorted_ids[p0], seg, g1, g2);
+    const unsigned row_id = (unsigned)A.sorted_ids[p0];
+    RowRegs<MUL, VEC, NIT> e, m0, v0;
+    if (REG || A.adam_on) load_row<MUL, VEC, NIT>(e, A.table + (size_t)row_id * row_len, half, A.ncol, lane);
+    if (A.adam_on) {
+      load_row<MUL, VEC, NIT>(m0, A.m + (size_t)row_id * row_len, half, A.ncol, lane);
+      load_row<MUL, VEC, NIT>(v0, A.v + (size_t)row_id * row_len, half, A.ncol, lane);
+    }
+    finish_row<SRC, VEC, NIT, REG>(A, lane, row_id, seg, g1, g2, e, m0, v0);
   }
 }
 
 // ---- host side -------------------------------------------------------------------------------
 
-static int choose_tile(size_t n_pairs) {
-  // aim at >= 16k tiles so every CU holds several wavefronts; long tiles keep partial rows few
-  size_t tile = ((n_pairs / 16384) + 63) / 64 * 64;
-  if (tile < 64) tile = 64;
-  if (tile > 256) tile = 256;
-  return (int)tile;
+constexpr int kTile = 256;      // sorted positions per tile of the long-segment pass
+constexpr int kShortMax = 64;   // longest segment one wavefront finishes on its own
+
+static size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
+
+struct EntityScratch {
+  size_t tail_off, head_off, meta_c_off, meta_b_off, total;
+};
+
+static EntityScratch entity_scratch(size_t n_pairs, size_t row_len) {
+  const size_t tiles = (n_pairs + kTile - 1) / kTile;
+  EntityScratch s;
+  s.tail_off = 0;
+  s.head_off = align256(tiles * row_len * sizeof(float));
+  s.meta_c_off = s.head_off + align256(tiles * row_len * sizeof(float));
+  s.meta_b_off = s.meta_c_off + align256(n_pairs * sizeof(float));
+  s.total = s.meta_b_off + align256(n_pairs * sizeof(int));
+  return s;
 }
 
-static size_t entity_ws_bytes(size_t n_pairs, size_t row_len) {
-  const size_t tile = (size_t)choose_tile(n_pairs);
-  const size_t tiles = (n_pairs + tile - 1) / tile;
-  return 2 * tiles * row_len * sizeof(float) + 256;
-}
+static size_t entity_ws_bytes(size_t n_pairs, size_t row_len) { return entity_scratch(n_pairs, row_len).total; }
 
 static AdamConsts adam_consts(const smx_adam_params* a) {
   AdamConsts c;
@@ -405,33 +504,55 @@ static AdamConsts adam_consts(const smx_adam_params* a) {
   return c;
 }
 
-template <int SRC, int VEC, int NIT>
-static int launch_entity(hipStream_t st, const EntityArgs& A) {
-  const int tiles = (A.n_pairs + A.tile - 1) / A.tile;
-  hipLaunchKernelGGL((entity_tile_kernel<SRC, VEC, NIT>), dim3((unsigned)((tiles + 3) / 4)), dim3(256), 0, st, A);
-  constexpr int NW = 8;
-  const size_t lds = (size_t)(NW - 1) * A.ncol * VEC * src_mul(SRC) * sizeof(float);
-  hipLaunchKernelGGL((entity_fixup_kernel<SRC, VEC, NIT, NW>), dim3((unsigned)tiles), dim3(NW * 64), lds, st, A);
+template <int SRC, int VEC, int NIT, bool REG>
+static int launch_entity_reg(hipStream_t st, const EntityArgs& A) {
+  const unsigned tiles = (unsigned)((A.n_pairs + A.tile - 1) / A.tile);
+  if (SRC != kSrcRows)
+    hipLaunchKernelGGL((entity_meta_kernel<SRC>), dim3((unsigned)((A.n_pairs + 255) / 256)), dim3(256), 0, st, A);
+  // short segments: a fixed grid of wavefronts strides over the segment list (its length lives on the device)
+  unsigned seg_blocks = (unsigned)((A.n_pairs + 3) / 4);
+  if (seg_blocks > 256u * 8u) seg_blocks = 256u * 8u;
+  hipLaunchKernelGGL((entity_segment_kernel<SRC, VEC, NIT, REG>), dim3(seg_blocks), dim3(256), 0, st, A);
+  hipLaunchKernelGGL((entity_tile_kernel<SRC, VEC, NIT, REG>), dim3((tiles + 3) / 4), dim3(256), 0, st, A);
+  const size_t row_bytes = (size_t)A.ncol * VEC * src_mul(SRC) * sizeof(float);
+  if (15 * row_bytes <= 60 * 1024)
+    hipLaunchKernelGGL((entity_fixup_kernel<SRC, VEC, NIT, 16, REG>), dim3(tiles), dim3(16 * 64), 15 * row_bytes, st, A);
+  else
+    hipLaunchKernelGGL((entity_fixup_kernel<SRC, VEC, NIT, 4, REG>), dim3(tiles), dim3(4 * 64), 3 * row_bytes, st, A);
   return check_launch("entity backward");
 }
 
+template <int SRC, int VEC, int NIT>
+static int launch_entity(hipStream_t st, const EntityArgs& A) {
+  if constexpr (SRC == mBetaKL) {
+    if (A.p.reg_on) return launch_entity_reg<SRC, VEC, NIT, true>(st, A);
+  }
+  return launch_entity_reg<SRC, VEC, NIT, false>(st, A);
+}
+
 static int fill_plan(EntityArgs* A, const smx_plan_view* plan, void* workspace, size_t workspace_bytes, size_t row_len) {
-  if (!plan || !plan->order || !plan->sorted_ids || !plan->seg_of_pos || !plan->seg_start)
+  if (!plan || !plan->order || !plan->sorted_ids || !plan->seg_of_pos || !plan->seg_start || !plan->uniq ||
+      !plan->n_uniq)
     return fail(SMX_ERR_ARG, "incomplete segment plan");
   if (plan->n_pairs == 0 || plan->n_pairs > 0x7fffffffull) return fail(SMX_ERR_SHAPE, "pair count out of range");
-  const size_t need = entity_ws_bytes(plan->n_pairs, row_len);
-  if (!workspace || workspace_bytes < need)
-    return fail(SMX_ERR_WORKSPACE, "entity workspace too small: %zu < %zu", workspace_bytes, need);
+  const EntityScratch sc = entity_scratch(plan->n_pairs, row_len);
+  if (!workspace || workspace_bytes < sc.total)
+    return fail(SMX_ERR_WORKSPACE, "entity workspace too small: %zu < %zu", workspace_bytes, sc.total);
   if (reinterpret_cast<uintptr_t>(workspace) & 255u) return fail(SMX_ERR_ARG, "workspace must be 256-byte aligned");
   A->order = plan->order;
   A->sorted_ids = plan->sorted_ids;
   A->seg_of_pos = plan->seg_of_pos;
   A->seg_start = plan->seg_start;
+  A->uniq = reinterpret_cast<const long long*>(plan->uniq);
+  A->n_uniq = plan->n_uniq;
   A->n_pairs = (int)plan->n_pairs;
-  A->tile = choose_tile(plan->n_pairs);
-  const size_t tiles = (plan->n_pairs + A->tile - 1) / A->tile;
-  A->tail = static_cast<float*>(workspace);
-  A->head = A->tail + tiles * row_len;
+  A->tile = kTile;
+  A->short_max = kShortMax;
+  char* ws = static_cast<char*>(workspace);
+  A->tail = reinterpret_cast<float*>(ws + sc.tail_off);
+  A->head = reinterpret_cast<float*>(ws + sc.head_off);
+  A->meta_c = reinterpret_cast<float*>(ws + sc.meta_c_off);
+  A->meta_b = reinterpret_cast<int*>(ws + sc.meta_b_off);
   return SMX_OK;
 }
 
@@ -463,6 +584,8 @@ int smx_score_backward_entity(int model, void* stream, const smx_plan_view* plan
   if (!table || !q1 || !score || !gscore || !params || (model_nq(model) == 2 && !q2))
     return fail(SMX_ERR_ARG, "null pointer");
   if (B == 0 || K == 0 || dim == 0 || n_rows == 0) return fail(SMX_ERR_SHAPE, "empty dimension");
+  if (params->reg_on && model != mBetaKL)
+    return fail(SMX_ERR_ARG, "the entity clamp prologue exists for the beta_kl model only");
   if (!merged && !m) return fail(SMX_ERR_ARG, "nothing to do: neither merged gradient nor Adam requested");
   EntityArgs A{};
   const size_t row_len = dim * model_mul(model);

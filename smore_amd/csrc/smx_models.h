@@ -9,8 +9,9 @@
 //   BETA_KL    gamma - sum KL(Beta(e) || Beta(q))       smore/models/beta.py:303-308
 //
 // A model exposes
-//   fwd(e1,e2,q,acc0,acc1)      add one feature's term(s) to the accumulators
-//   score(acc0,acc1,p)          logit from the reduced accumulators
+//   fwd(e1,e2,q,acc0,acc1)      add one feature's term(s) to the lane's accumulators
+//   fold(acc0,acc1,p)           the lane's single value to be summed over the wavefront
+//   score(sum,p)                logit from that sum
 //   coef(g,score,p,c0,c1)       d logit-loss / d accumulator, from the upstream
 //                               gradient g of the logit and the saved logit
 //   bwd_e / bwd_q               add one feature's gradient w.r.t. entity / query
@@ -58,7 +59,8 @@ template <> struct ModelOps<mL1> {
   static __device__ __forceinline__ void fwd(float e1, float, const Q& q, float& a0, float&) {
     a0 += Term<kL1, float>::fwd(e1, 0.f, q.a, 0.f);
   }
-  static __device__ __forceinline__ float score(float a0, float, const ScoreParams& p) { return p.gamma - a0; }
+  static __device__ __forceinline__ float fold(float a0, float, const ScoreParams&) { return a0; }
+  static __device__ __forceinline__ float score(float folded, const ScoreParams& p) { return p.gamma - folded; }
   static __device__ __forceinline__ void coef(float g, float, const ScoreParams&, float& c0, float& c1) {
     c0 = -g;
     c1 = 0.f;
@@ -79,7 +81,8 @@ template <> struct ModelOps<mL2> {
   static __device__ __forceinline__ void fwd(float e1, float, const Q& q, float& a0, float&) {
     a0 += Term<kL2, float>::fwd(e1, 0.f, q.a, 0.f);
   }
-  static __device__ __forceinline__ float score(float a0, float, const ScoreParams& p) { return p.gamma - sqrtf(a0); }
+  static __device__ __forceinline__ float fold(float a0, float, const ScoreParams&) { return a0; }
+  static __device__ __forceinline__ float score(float folded, const ScoreParams& p) { return p.gamma - sqrtf(folded); }
   // d(gamma - sqrt(d2)) / d d2 = -1 / (2 sqrt(d2)), and sqrt(d2) = gamma - score.  At d2 == 0 the
   // coefficient is infinite, as autograd of torch.sqrt makes it in the reference.
   static __device__ __forceinline__ void coef(float g, float s, const ScoreParams& p, float& c0, float& c1) {
@@ -104,9 +107,8 @@ template <> struct ModelOps<mBox> {
     a0 += Term<kBoxOut, float>::fwd(e1, 0.f, q.a, q.b);
     a1 += Term<kBoxIn, float>::fwd(e1, 0.f, q.a, q.b);
   }
-  static __device__ __forceinline__ float score(float a0, float a1, const ScoreParams& p) {
-    return p.gamma - a0 - p.cen * a1;
-  }
+  static __device__ __forceinline__ float fold(float a0, float a1, const ScoreParams& p) { return a0 + p.cen * a1; }
+  static __device__ __forceinline__ float score(float folded, const ScoreParams& p) { return p.gamma - folded; }
   static __device__ __forceinline__ void coef(float g, float, const ScoreParams& p, float& c0, float& c1) {
     c0 = -g;
     c1 = -p.cen * g;
@@ -129,7 +131,8 @@ template <> struct ModelOps<mRotate> {
   static __device__ __forceinline__ void fwd(float e1, float e2, const Q& q, float& a0, float&) {
     a0 += Term<kRotate, float>::fwd(e1, e2, q.a, q.b);
   }
-  static __device__ __forceinline__ float score(float a0, float, const ScoreParams& p) { return p.gamma - a0; }
+  static __device__ __forceinline__ float fold(float a0, float, const ScoreParams&) { return a0; }
+  static __device__ __forceinline__ float score(float folded, const ScoreParams& p) { return p.gamma - folded; }
   static __device__ __forceinline__ void coef(float g, float, const ScoreParams&, float& c0, float& c1) {
     c0 = -g;
     c1 = 0.f;
@@ -150,7 +153,8 @@ template <> struct ModelOps<mBetaKL> {
   static __device__ __forceinline__ void fwd(float e1, float e2, const Q& q, float& a0, float&) {
     a0 += Term<kBetaKL, float>::fwd(e1, e2, q.a, q.b);
   }
-  static __device__ __forceinline__ float score(float a0, float, const ScoreParams& p) { return p.gamma - a0; }
+  static __device__ __forceinline__ float fold(float a0, float, const ScoreParams&) { return a0; }
+  static __device__ __forceinline__ float score(float folded, const ScoreParams& p) { return p.gamma - folded; }
   static __device__ __forceinline__ void coef(float g, float, const ScoreParams&, float& c0, float& c1) {
     c0 = -g;
     c1 = 0.f;

@@ -67,19 +67,37 @@ __device__ __forceinline__ void stage_query(float* lds, const float* __restrict_
   __syncthreads();
 }
 
-// Row pointer of pair (b,k): through idx when given, else the dense [B*K, row_len] layout.
+// Entity row of pair `pair`: through idx when given, else the dense [B*K, row_len] layout.  The id is
+// wave-uniform, so the range check and the 64-bit row offset stay on the scalar unit.  An id outside
+// the table is replaced by row 0 and remembered in `bad`.
 __device__ __forceinline__ const float* pair_row(const float* __restrict__ table, const long long* __restrict__ idx,
-                                                 size_t pair, size_t row_len, unsigned long long n_rows, int lane,
-                                                 int* err) {
+                                                 size_t pair, size_t row_len, unsigned long long n_rows, int& bad) {
   long long row = idx ? idx[pair] : (long long)pair;
-  if ((unsigned long long)row >= n_rows) {  // out-of-range id: flag it, read row 0 instead of faulting
-    if (err && lane == 0) *err = 1;
+  if ((unsigned long long)row >= n_rows) {
+    bad = 1;
     row = 0;
   }
   return table + (size_t)row * row_len;
 }
 
-template <int M, int VEC, int NIT, int RIF>
+// Loads the columns a lane owns of RIF rows.  Column and row numbers are clamped instead of
+// predicated, so the loads form one straight-line batch that stays in flight together; lanes
+// beyond the row end re-read its last column (same cache line) and are masked in the arithmetic.
+template <int MUL, int VEC, int NIT, int RIF>
+__device__ __forceinline__ void load_rows(const float* const (&pe)[RIF], int dim, int ncol, int lane,
+                                          Pack<VEC> (&e1)[RIF][NIT], Pack<VEC> (&e2)[RIF][NIT]) {
+#pragma unroll
+  for (int r = 0; r < RIF; ++r) {
+#pragma unroll
+    for (int it = 0; it < NIT; ++it) {
+      const int c = min(lane + 64 * it, ncol - 1);
+      e1[r][it] = load_pack<VEC>(pe[r], c);
+      if (MUL == 2) e2[r][it] = load_pack<VEC>(pe[r] + dim, c);
+    }
+  }
+}
+
+template <int M, int VEC, int NIT, int RIF, bool REG>
 __global__ __launch_bounds__(256) void score_forward_kernel(const float* __restrict__ table,
                                                             const long long* __restrict__ idx,
                                                             const float* __restrict__ q1, const float* __restrict__ q2,
@@ -101,49 +119,37 @@ __global__ __launch_bounds__(256) void score_forward_kernel(const float* __restr
 
   const int k0 = tile * tile_k;
   const int k1 = min(K, k0 + tile_k);
+  int bad = 0;
   for (int kb = k0 + wave * RIF; kb < k1; kb += 4 * RIF) {
+    const float* pe[RIF];
+#pragma unroll
+    for (int r = 0; r < RIF; ++r)
+      pe[r] = pair_row(table, idx, (size_t)b * K + min(kb + r, k1 - 1), row_len, n_rows, bad);
     Pack<VEC> e1[RIF][NIT], e2[RIF][NIT];
+    load_rows<MUL, VEC, NIT, RIF>(pe, dim, ncol, lane, e1, e2);
 #pragma unroll
     for (int r = 0; r < RIF; ++r) {
-      const int k = kb + r;
-      if (k < k1) {
-        const float* pe = pair_row(table, idx, (size_t)b * K + k, row_len, n_rows, lane, err);
+      float a0 = 0.f, a1 = 0.f;
 #pragma unroll
-        for (int it = 0; it < NIT; ++it) {
-          const int c = lane + 64 * it;
-          if (c < ncol) {
-            e1[r][it] = load_pack<VEC>(pe, c);
-            if (MUL == 2) e2[r][it] = load_pack<VEC>(pe + dim, c);
+      for (int it = 0; it < NIT; ++it) {
+        if (lane + 64 * it < ncol) {
+#pragma unroll
+          for (int v = 0; v < VEC; ++v) {
+            const float x1 = REG ? reg_apply(e1[r][it].v[v], p) : e1[r][it].v[v];
+            const float x2 = MUL == 2 ? (REG ? reg_apply(e2[r][it].v[v], p) : e2[r][it].v[v]) : 0.f;
+            ModelOps<M>::fwd(x1, x2, q[it][v], a0, a1);
           }
         }
       }
-    }
-#pragma unroll
-    for (int r = 0; r < RIF; ++r) {
-      const int k = kb + r;
-      if (k < k1) {
-        float a0 = 0.f, a1 = 0.f;
-#pragma unroll
-        for (int it = 0; it < NIT; ++it) {
-          const int c = lane + 64 * it;
-          if (c < ncol) {
-#pragma unroll
-            for (int v = 0; v < VEC; ++v) {
-              const float x1 = reg_apply(e1[r][it].v[v], p);
-              const float x2 = MUL == 2 ? reg_apply(e2[r][it].v[v], p) : 0.f;
-              ModelOps<M>::fwd(x1, x2, q[it][v], a0, a1);
-            }
-          }
-        }
-        a0 = wave_sum_f32(a0);
-        if (M == mBox) a1 = wave_sum_f32(a1);
-        if (lane == 0) score[(size_t)b * K + k] = ModelOps<M>::score(a0, a1, p);
-      }
+      // the logit is linear in the accumulators: fold them per lane, reduce once
+      const float folded = wave_sum_f32(ModelOps<M>::fold(a0, a1, p));
+      if (lane == 0 && kb + r < k1) score[(size_t)b * K + kb + r] = ModelOps<M>::score(folded, p);
     }
   }
+  if (bad && err && lane == 0) *err = 1;
 }
 
-template <int M, int VEC, int NIT, int RIF, int NW>
+template <int M, int VEC, int NIT, int RIF, int NW, bool REG>
 __global__ __launch_bounds__(NW * 64) void score_backward_query_kernel(
     const float* __restrict__ table, const long long* __restrict__ idx, const float* __restrict__ q1,
     const float* __restrict__ q2, const float* __restrict__ score, const float* __restrict__ gscore,
@@ -167,38 +173,29 @@ __global__ __launch_bounds__(NW * 64) void score_backward_query_kernel(
 #pragma unroll
     for (int v = 0; v < VEC; ++v) g1[it][v] = g2[it][v] = 0.f;
 
+  int bad = 0;
   for (int kb = wave * RIF; kb < K; kb += NW * RIF) {
-    Pack<VEC> e1[RIF][NIT], e2[RIF][NIT];
+    const float* pe[RIF];
     float c0[RIF], c1[RIF];
 #pragma unroll
     for (int r = 0; r < RIF; ++r) {
-      const int k = kb + r;
-      if (k < K) {
-        const size_t pair = (size_t)b * K + k;
-        const float* pe = pair_row(table, idx, pair, row_len, n_rows, lane, nullptr);
-        ModelOps<M>::coef(gscore[pair], score[pair], p, c0[r], c1[r]);
-#pragma unroll
-        for (int it = 0; it < NIT; ++it) {
-          const int c = lane + 64 * it;
-          if (c < ncol) {
-            e1[r][it] = load_pack<VEC>(pe, c);
-            if (MUL == 2) e2[r][it] = load_pack<VEC>(pe + dim, c);
-          }
-        }
-      }
+      const size_t pair = (size_t)b * K + min(kb + r, K - 1);
+      pe[r] = pair_row(table, idx, pair, row_len, n_rows, bad);
+      ModelOps<M>::coef(gscore[pair], score[pair], p, c0[r], c1[r]);
+      if (kb + r >= K) c0[r] = c1[r] = 0.f;  // rows past the end contribute nothing
     }
+    Pack<VEC> e1[RIF][NIT], e2[RIF][NIT];
+    load_rows<MUL, VEC, NIT, RIF>(pe, dim, ncol, lane, e1, e2);
 #pragma unroll
     for (int r = 0; r < RIF; ++r) {
-      if (kb + r < K) {
 #pragma unroll
-        for (int it = 0; it < NIT; ++it) {
-          if (lane + 64 * it < ncol) {
+      for (int it = 0; it < NIT; ++it) {
+        if (lane + 64 * it < ncol) {
 #pragma unroll
-            for (int v = 0; v < VEC; ++v) {
-              const float x1 = reg_apply(e1[r][it].v[v], p);
-              const float x2 = MUL == 2 ? reg_apply(e2[r][it].v[v], p) : 0.f;
-              ModelOps<M>::bwd_q(c0[r], c1[r], x1, x2, q[it][v], g1[it][v], g2[it][v]);
-            }
+          for (int v = 0; v < VEC; ++v) {
+            const float x1 = REG ? reg_apply(e1[r][it].v[v], p) : e1[r][it].v[v];
+            const float x2 = MUL == 2 ? (REG ? reg_apply(e2[r][it].v[v], p) : e2[r][it].v[v]) : 0.f;
+            ModelOps<M>::bwd_q(c0[r], c1[r], x1, x2, q[it][v], g1[it][v], g2[it][v]);
           }
         }
       }
@@ -266,18 +263,27 @@ constexpr int rows_in_flight(int nit, int mul) {
   return r < 1 ? 1 : (r > 4 ? 4 : r);
 }
 
-template <int M, int VEC, int NIT>
-static int launch_forward(hipStream_t st, const float* table, const int64_t* idx, const float* q1, const float* q2,
+template <int M, int VEC, int NIT, bool REG>
+static int launch_forward_reg(hipStream_t st, const float* table, const int64_t* idx, const float* q1, const float* q2,
                           float* score, size_t B, size_t K, int ncol, size_t n_rows, const ScoreParams& p, int* err) {
   constexpr int RIF = rows_in_flight(NIT, model_mul(M));
   int tile_k = 128;
   while (tile_k > 4 * RIF && B * ((K + tile_k - 1) / tile_k) < 4096) tile_k /= 2;
   const int tiles = (int)((K + tile_k - 1) / tile_k);
   const size_t lds = (size_t)model_nq(M) * ncol * VEC * sizeof(float);
-  hipLaunchKernelGGL((score_forward_kernel<M, VEC, NIT, RIF>), dim3((unsigned)(B * tiles)), dim3(256), lds, st, table,
+  hipLaunchKernelGGL((score_forward_kernel<M, VEC, NIT, RIF, REG>), dim3((unsigned)(B * tiles)), dim3(256), lds, st, table,
                      reinterpret_cast<const long long*>(idx), q1, q2, score, (int)K, ncol, tiles, tile_k,
                      (unsigned long long)n_rows, p, err);
   return check_launch("score forward");
+}
+
+template <int M, int VEC, int NIT>
+static int launch_forward(hipStream_t st, const float* table, const int64_t* idx, const float* q1, const float* q2,
+                          float* score, size_t B, size_t K, int ncol, size_t n_rows, const ScoreParams& p, int* err) {
+  if constexpr (M == mBetaKL) {
+    if (p.reg_on) return launch_forward_reg<M, VEC, NIT, true>(st, table, idx, q1, q2, score, B, K, ncol, n_rows, p, err);
+  }
+  return launch_forward_reg<M, VEC, NIT, false>(st, table, idx, q1, q2, score, B, K, ncol, n_rows, p, err);
 }
 
 template <int M, int VEC, int NIT, int NW>
@@ -286,8 +292,16 @@ static int launch_backward_query(hipStream_t st, const float* table, const int64
                                  size_t B, size_t K, int ncol, size_t n_rows, const ScoreParams& p) {
   constexpr int RIF = rows_in_flight(NIT, model_mul(M));
   const size_t lds = (size_t)(NW + 1) * model_nq(M) * ncol * VEC * sizeof(float);
-  hipLaunchKernelGGL((score_backward_query_kernel<M, VEC, NIT, RIF, NW>), dim3((unsigned)B), dim3(NW * 64), lds, st,
-                     table, reinterpret_cast<const long long*>(idx), q1, q2, score, gscore, gq1, gq2, (int)K, ncol,
+  if constexpr (M == mBetaKL) {
+    if (p.reg_on) {
+      hipLaunchKernelGGL((score_backward_query_kernel<M, VEC, NIT, RIF, NW, true>), dim3((unsigned)B), dim3(NW * 64),
+                         lds, st, table, reinterpret_cast<const long long*>(idx), q1, q2, score, gscore, gq1, gq2,
+                         (int)K, ncol, (unsigned long long)n_rows, p);
+      return check_launch("score backward (query)");
+    }
+  }
+  hipLaunchKernelGGL((score_backward_query_kernel<M, VEC, NIT, RIF, NW, false>), dim3((unsigned)B), dim3(NW * 64), lds,
+                     st, table, reinterpret_cast<const long long*>(idx), q1, q2, score, gscore, gq1, gq2, (int)K, ncol,
                      (unsigned long long)n_rows, p);
   return check_launch("score backward (query)");
 }
@@ -335,6 +349,8 @@ static int check_score_args(int model, const float* table, const float* q1, cons
   if (B == 0 || K == 0 || dim == 0) return fail(SMX_ERR_SHAPE, "empty dimension");
   if (B > 0x7fffffffull || K > 0x7fffffffull || B * K > 0x7fffffffull)
     return fail(SMX_ERR_SHAPE, "more than 2^31-1 pairs in one call");
+  if (params->reg_on && model != mBetaKL)
+    return fail(SMX_ERR_ARG, "the entity clamp prologue exists for the beta_kl model only");
   return SMX_OK;
 }
 

@@ -125,7 +125,7 @@ class SegmentPlan:
 
     def view(self):
         return _lib.PlanView(_ptr(self.order), _ptr(self.sorted_ids), _ptr(self.seg_of_pos), _ptr(self.seg_start),
-                             self.n_pairs)
+                             _ptr(self.uniq_buf), _ptr(self.n_uniq_dev), self.n_pairs)
 
 
 def _workspace(nbytes, device):
