@@ -185,6 +185,11 @@ int smx_rows_backward(void* stream, const smx_plan_view* plan, const float* grad
                       size_t row_len, float* merged, float* table, float* m, float* v,
                       const smx_adam_params* adam, void* workspace, size_t workspace_bytes);
 
+/* Plain row lookup out[k,:] = table[idx[k],:] (smore/common/embedding/embed_rw.py:74-75, the GPU
+ * branch of EmbeddingReadOnly.read) for callers that need the rows themselves. */
+int smx_gather_rows(void* stream, const float* table, size_t n_rows, size_t row_len,
+                    const int64_t* idx, size_t n, float* out, int* err_flag);
+
 #ifdef __cplusplus
 }
 #endif

@@ -41,6 +41,8 @@ SIGNATURES = {
     "smx_score_backward_entity": (_i, [_i, _vp, _vp, _vp, _sz, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _vp, _vp, _vp, _vp,
                                        _vp, _vp, _sz]),
     # stream, plan, grad_rows, row_len, merged, table, m, v, adam, ws, ws_bytes
+    # stream, table, n_rows, row_len, idx, n, out, err
+    "smx_gather_rows": (_i, [_vp, _vp, _sz, _sz, _vp, _sz, _vp, _vp]),
     "smx_rows_backward": (_i, [_vp, _vp, _vp, _sz, _vp, _vp, _vp, _vp, _vp, _vp, _sz]),
 }
 

@@ -1,0 +1,642 @@
+// Entity-side backward: segmented gradient reduction with the sparse Adam row
+// update fused into the same pass.  No float atomics anywhere; every sum has a
+// fixed order, so two runs on the same inputs give the same bits.
+//
+// Replaces, per training step,
+//   dist_backward_ent_kernel              smore/common/torchext/common_kernel.h:59-89
+//   EmbedLookupFunc.backward / accumulate smore/common/embedding/embed_optimizer.py:63-66,146-148
+//   merge_grad_list (scatter-sum)         embed_optimizer.py:45-48
+//   AdamEmbedOptimizer.update_step        embed_optimizer.py:208-252
+// The reference materialises a [P, row] gradient tensor, scatter-adds it into
+// [U, row] and then runs ~20 row-sized tensor passes for Adam.  Here the sorted
+// pair list of the segment plan is cut into fixed tiles; one wavefront walks a
+// tile, recomputes each pair's entity gradient from (entity row, query row,
+// upstream gradient) in registers -- or, for gradients that autograd already
+// materialised, reads the pair's gradient row -- and sums it per segment.
+//   * a segment that lies inside one tile is finished on the spot: the lanes
+//     holding its gradient read w, m, v of that entity row, apply Adam, and
+//     write the three rows back;
+//   * a segment crossing a tile edge leaves one partial row per tile (tail: it
+//     continues past the tile end; head: it came in from the left and ends
+//     here); a second kernel adds the partials of such a segment in tile order
+//     and then finishes it the same way.
+// Consecutive pairs of a segment that belong to the same query (common when
+// ids repeat inside one query's negatives) share one gradient evaluation: the
+// derivative is linear in the upstream coefficient, so coefficients are summed
+// first.
+#pragma once
+#include "smx_common.h"
+#include "smx_models.h"
+#include "smx_wave.h"
+
+namespace smx {
+
+constexpr int kSrcRows = 100;  // source = materialised gradient rows instead of a score model
+
+__host__ __device__ constexpr int src_mul(int s) { return s == kSrcRows ? 1 : model_mul(s); }
+
+struct AdamConsts {
+  float beta1, beta2, omb1, omb2, eps, step_size, inv_sqrt_bc2;
+};
+
+struct EntityArgs {
+  // plan
+  const int* order;
+  const int* sorted_ids;
+  const int* seg_of_pos;
+  const int* seg_start;
+  const long long* uniq;
+  const int* n_uniq;
+  int n_pairs;
+  int tile;        // sorted positions per tile of the long-segment pass, multiple of 64
+  int short_max;   // segments of at most this many pairs are finished by one wavefront
+  // source: score model
+  const float* q1;
+  const float* q2;
+  const float* score;
+  const float* gscore;
+  int K;
+  ScoreParams p;
+  float* meta_c;  // [P] upstream coefficient of every sorted position
+  int* meta_b;    // [P] query number of every sorted position
+  // source: gradient rows
+  const float* grad_rows;
+  // entity table (read for the model sources, updated when adam_on)
+  float* table;
+  float* m;
+  float* v;
+  int adam_on;
+  AdamConsts a;
+  float* merged;  // [U, row_len] or null
+  float* tail;    // [tiles, row_len]
+  float* head;    // [tiles, row_len]
+  int ncol;       // columns per half row (model sources) or per row (gradient rows)
+};
+
+template <int VEC> struct Pack2 {
+  float v[VEC];
+};
+
+template <int VEC>
+__device__ __forceinline__ Pack2<VEC> ld(const float* __restrict__ base, int col) {
+  Pack2<VEC> r;
+  if constexpr (VEC == 4) {
+    const float4 t = reinterpret_cast<const float4*>(base)[col];
+    r.v[0] = t.x;
+    r.v[1] = t.y;
+    r.v[2] = t.z;
+    r.v[3] = t.w;
+  } else {
+    r.v[0] = base[col];
+  }
+  return r;
+}
+
+template <int VEC>
+__device__ __forceinline__ void st(float* __restrict__ base, int col, const float (&x)[VEC]) {
+  if constexpr (VEC == 4) {
+    reinterpret_cast<float4*>(base)[col] = make_float4(x[0], x[1], x[2], x[3]);
+  } else {
+    base[col] = x[0];
+  }
+}
+
+// The lane's columns of one table row (both halves for the two-half models).
+template <int MUL, int VEC, int NIT> struct RowRegs {
+  Pack2<VEC> h[MUL][NIT];
+};
+
+template <int MUL, int VEC, int NIT>
+__device__ __forceinline__ void load_row(RowRegs<MUL, VEC, NIT>& r, const float* __restrict__ base, int half, int ncol,
+                                         int lane) {
+#pragma unroll
+  for (int h = 0; h < MUL; ++h)
+#pragma unroll
+    for (int it = 0; it < NIT; ++it) r.h[h][it] = ld<VEC>(base + h * half, min(lane + 64 * it, ncol - 1));
+}
+
+// Coefficient on the second accumulator (BOX: inside distance) from the first.
+template <int SRC>
+__device__ __forceinline__ float second_coef(float c0, const ScoreParams& p) {
+  return SRC == mBox ? p.cen * c0 : 0.f;
+}
+
+
+// ---- runs -------------------------------------------------------------------------------------
+// A "run" is a stretch of consecutive sorted positions of one segment that belong to the same
+// query.  The gradient of a pair is linear in its upstream coefficient, so the coefficients of a
+// run are summed first and the run costs one gradient evaluation.  Runs are handled R at a time:
+// the query rows of all R runs are requested before any of them is used, which keeps R (x2) row
+// loads in flight per wavefront.  For materialised gradients a "run" is one pair and the row
+// requested is that pair's gradient row.
+
+template <int R> struct RunSet {
+  int key[R];    // query number (model sources) or pair number (gradient rows)
+  float c[R];    // summed coefficient (model sources)
+  int n;         // valid runs
+};
+
+// Collects up to R runs from window lanes [j, j_end); my_key / my_c hold one sorted position per lane.
+template <int SRC, int R>
+__device__ __forceinline__ void collect_runs(RunSet<R>& rs, int& j, int j_end, int my_key, float my_c) {
+  rs.n = 0;
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    rs.key[r] = 0;
+    rs.c[r] = 0.f;
+    if (j < j_end) {  // wave-uniform
+      rs.n = r + 1;
+      rs.key[r] = __builtin_amdgcn_readlane(my_key, j);
+      if constexpr (SRC == kSrcRows) {
+        ++j;
+      } else {
+        do {
+          rs.c[r] += __int_as_float(__builtin_amdgcn_readlane(__float_as_int(my_c), j));
+          ++j;
+        } while (j < j_end && __builtin_amdgcn_readlane(my_key, j) == rs.key[r]);
+      }
+    }
+  }
+}
+
+template <int SRC, int VEC, int NIT, int R> struct RunRows {
+  Pack2<VEC> a[R][NIT];
+  Pack2<VEC> b[R][NIT];
+};
+
+// Requests the rows the runs need: query row(s) for the model sources, the gradient row otherwise.
+template <int SRC, int VEC, int NIT, int R>
+__device__ __forceinline__ void request_runs(const EntityArgs& A, int lane, const RunSet<R>& rs,
+                                             RunRows<SRC, VEC, NIT, R>& rr) {
+  const int half = A.ncol * VEC;
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    if (r < rs.n) {
+      if constexpr (SRC == kSrcRows) {
+        const float* pg = A.grad_rows + (size_t)rs.key[r] * half;
+#pragma unroll
+        for (int it = 0; it < NIT; ++it) rr.a[r][it] = ld<VEC>(pg, min(lane + 64 * it, A.ncol - 1));
+      } else {
+        const float* pq1 = A.q1 + (size_t)rs.key[r] * half;
+#pragma unroll
+        for (int it = 0; it < NIT; ++it) rr.a[r][it] = ld<VEC>(pq1, min(lane + 64 * it, A.ncol - 1));
+        if constexpr (model_nq(SRC) == 2) {
+          const float* pq2 = A.q2 + (size_t)rs.key[r] * half;
+#pragma unroll
+          for (int it = 0; it < NIT; ++it) rr.b[r][it] = ld<VEC>(pq2, min(lane + 64 * it, A.ncol - 1));
+        }
+      }
+    }
+  }
+}
+
+// Adds the gradient of the runs to the lane's accumulators.
+template <int SRC, int VEC, int NIT, bool REG, int R>
+__device__ __forceinline__ void apply_runs(const EntityArgs& A, const RunSet<R>& rs,
+                                           const RunRows<SRC, VEC, NIT, R>& rr,
+                                           const RowRegs<src_mul(SRC), VEC, NIT>& e, float (&g1)[NIT][VEC],
+                                           float (&g2)[NIT][VEC]) {
+  constexpr int MUL = src_mul(SRC);
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    if (r < rs.n) {
+#pragma unroll
+      for (int it = 0; it < NIT; ++it) {
+#pragma unroll
+        for (int x = 0; x < VEC; ++x) {
+          if constexpr (SRC == kSrcRows) {
+            g1[it][x] += rr.a[r][it].v[x];
+          } else {
+            const float c0 = rs.c[r];
+            const float c1 = second_coef<SRC>(c0, A.p);
+            const typename ModelOps<SRC>::Q q =
+                ModelOps<SRC>::prep(rr.a[r][it].v[x], model_nq(SRC) == 2 ? rr.b[r][it].v[x] : 0.f);
+            const float x1 = REG ? reg_apply(e.h[0][it].v[x], A.p) : e.h[0][it].v[x];
+            const float x2 = MUL == 2 ? (REG ? reg_apply(e.h[MUL - 1][it].v[x], A.p) : e.h[MUL - 1][it].v[x]) : 0.f;
+            ModelOps<SRC>::bwd_e(c0, c1, x1, x2, q, g1[it][x], g2[it][x]);
+          }
+        }
+      }
+    }
+  }
+}
+
+// One sorted position per lane: the window [base, base+64) of the per-position inputs.
+template <int SRC>
+__device__ __forceinline__ void load_window(const EntityArgs& A, int lane, int base, int& my_key, float& my_c) {
+  const int pos = min(base + lane, A.n_pairs - 1);
+  if constexpr (SRC == kSrcRows) {
+    my_key = A.order[pos];
+    my_c = 0.f;
+  } else {
+    my_key = A.meta_b[pos];
+    my_c = A.meta_c[pos];
+  }
+}
+
+// Finishes one entity row: clamp mask, merged-gradient store, Adam.  g1/g2 are the lane's columns of
+// the summed gradient of the first / second half row; w, m0, v0 the row's current weights and moments
+// (w is always valid for the model sources -- it is the entity row the gradient was computed from).
+template <int SRC, int VEC, int NIT, bool REG>
+__device__ __forceinline__ void finish_row(const EntityArgs& A, int lane, unsigned row_id, int seg,
+                                           float (&g1)[NIT][VEC], float (&g2)[NIT][VEC],
+                                           const RowRegs<src_mul(SRC), VEC, NIT>& w,
+                                           const RowRegs<src_mul(SRC), VEC, NIT>& m0,
+                                           const RowRegs<src_mul(SRC), VEC, NIT>& v0) {
+  constexpr int MUL = src_mul(SRC);
+  const int half = A.ncol * VEC;
+  const size_t row_len = (size_t)half * MUL;
+  if (REG) {
+#pragma unroll
+    for (int it = 0; it < NIT; ++it)
+#pragma unroll
+      for (int x = 0; x < VEC; ++x) {
+        g1[it][x] = reg_mask(w.h[0][it].v[x], g1[it][x], A.p);
+        if (MUL == 2) g2[it][x] = reg_mask(w.h[MUL - 1][it].v[x], g2[it][x], A.p);
+      }
+  }
+  if (A.merged) {
+    float* out = A.merged + (size_t)seg * row_len;
+#pragma unroll
+    for (int it = 0; it < NIT; ++it) {
+      const int c = lane + 64 * it;
+      if (c < A.ncol) {
+        st<VEC>(out, c, g1[it]);
+        if (MUL == 2) st<VEC>(out + half, c, g2[it]);
+      }
+    }
+  }
+  if (A.adam_on) {
+    float* pw = A.table + (size_t)row_id * row_len;
+    float* pm = A.m + (size_t)row_id * row_len;
+    float* pv = A.v + (size_t)row_id * row_len;
+#pragma unroll
+    for (int h = 0; h < MUL; ++h) {
+#pragma unroll
+      for (int it = 0; it < NIT; ++it) {
+        const int c = lane + 64 * it;
+        if (c < A.ncol) {
+          float wn[VEC], mn[VEC], vn[VEC];
+#pragma unroll
+          for (int x = 0; x < VEC; ++x) {
+            const float g = h == 0 ? g1[it][x] : g2[it][x];
+            mn[x] = m0.h[h][it].v[x] * A.a.beta1 + g * A.a.omb1;
+            vn[x] = v0.h[h][it].v[x] * A.a.beta2 + g * g * A.a.omb2;
+            const float denom = sqrtf(vn[x]) * A.a.inv_sqrt_bc2 + A.a.eps;
+            wn[x] = w.h[h][it].v[x] + A.a.step_size * mn[x] / denom;
+          }
+          st<VEC>(pw + h * half, c, wn);
+          st<VEC>(pm + h * half, c, mn);
+          st<VEC>(pv + h * half, c, vn);
+        }
+      }
+    }
+  }
+}
+
+template <int SRC, int VEC, int NIT>
+__device__ __forceinline__ void store_partial(const EntityArgs& A, float* buf, int t, int lane,
+                                              const float (&g1)[NIT][VEC], const float (&g2)[NIT][VEC]) {
+  constexpr int MUL = src_mul(SRC);
+  const int half = A.ncol * VEC;
+  float* out = buf + (size_t)t * half * MUL;
+#pragma unroll
+  for (int it = 0; it < NIT; ++it) {
+    const int c = lane + 64 * it;
+    if (c < A.ncol) {
+      st<VEC>(out, c, g1[it]);
+      if (MUL == 2) st<VEC>(out + half, c, g2[it]);
+    }
+  }
+}
+
+template <int VEC, int NIT>
+__device__ __forceinline__ void zero_acc(float (&g1)[NIT][VEC], float (&g2)[NIT][VEC]) {
+#pragma unroll
+  for (int it = 0; it < NIT; ++it)
+#pragma unroll
+    for (int x = 0; x < VEC; ++x) g1[it][x] = g2[it][x] = 0.f;
+}
+
+// Sorted copy of what the entity pass needs per pair, so that the pass reads it contiguously:
+// meta_c[pos] = d loss / d distance of the pair at sorted position pos, meta_b[pos] = its query.
+template <int SRC>
+__global__ __launch_bounds__(256) void entity_meta_kernel(EntityArgs A) {
+  const int pos = blockIdx.x * blockDim.x + threadIdx.x;
+  if (pos >= A.n_pairs) return;
+  if constexpr (SRC != kSrcRows) {
+    const int pair = A.order[pos];
+    float c0, c1;
+    ModelOps<SRC>::coef(A.gscore[pair], A.score[pair], A.p, c0, c1);
+    A.meta_c[pos] = c0;
+    A.meta_b[pos] = pair / A.K;
+  }
+}
+
+
+constexpr int kRunsShort = 2;  // runs in flight per wavefront in the short-segment kernel
+constexpr int kRunsLong = 4;   // ... in the long-segment kernel
+
+template <int MUL, int VEC, int NIT> struct RowState {
+  RowRegs<MUL, VEC, NIT> e, m, v;
+};
+
+template <int SRC, int VEC, int NIT>
+__device__ __forceinline__ void request_state(const EntityArgs& A, int lane, unsigned row_id,
+                                              RowState<src_mul(SRC), VEC, NIT>& s) {
+  constexpr int MUL = src_mul(SRC);
+  const int half = A.ncol * VEC;
+  const size_t off = (size_t)row_id * half * MUL;
+  if (SRC != kSrcRows || A.adam_on) load_row<MUL, VEC, NIT>(s.e, A.table + off, half, A.ncol, lane);
+  if (A.adam_on) {
+    load_row<MUL, VEC, NIT>(s.m, A.m + off, half, A.ncol, lane);
+    load_row<MUL, VEC, NIT>(s.v, A.v + off, half, A.ncol, lane);
+  }
+}
+
+// Short segments (at most A.short_max pairs).  The sorted pair list is cut into chunks of 64
+// positions and a fixed grid of wavefronts strides over the chunks; a wavefront owns the short
+// segments that START in its chunk, so its work is bounded by 64 + short_max pairs however the
+// segment lengths are distributed.  The lanes fetch the chunk's per-position inputs at once; the
+// wavefront then finishes one segment after the other, and while it works on one it already has
+// the next one's w, m, v rows on the way (two register sets used in turn).
+template <int SRC, int VEC, int NIT, bool REG>
+__global__ __launch_bounds__(256) void entity_segment_kernel(EntityArgs A) {
+  constexpr int MUL = src_mul(SRC);
+  constexpr int R = kRunsShort;
+  const int lane = threadIdx.x & 63;
+  const int wave = uniform(threadIdx.x >> 6);
+  const int n_waves = gridDim.x * 4;
+  const int n_chunks = (A.n_pairs + 63) / 64;
+
+  for (int chunk = blockIdx.x * 4 + wave; chunk < n_chunks; chunk += n_waves) {
+    const int base = chunk * 64;
+    const int n_here = min(64, A.n_pairs - base);
+    const int pos = base + min(lane, n_here - 1);
+    const int my_seg = A.seg_of_pos[pos];
+    const int my_s0 = A.seg_start[my_seg];
+    const int my_s1 = A.seg_start[my_seg + 1];
+    unsigned long long todo = __ballot(lane < n_here && my_s0 == pos && my_s1 - my_s0 <= A.short_max);
+    if (todo == 0ull) continue;
+    const int my_id = A.sorted_ids[pos];
+
+    int win_base = base;
+    int my_key;
+    float my_c;
+    load_window<SRC>(A, lane, win_base, my_key, my_c);
+
+    // finishes the segment that starts at lane i of the chunk from row state `cur`; requests the rows
+    // of the segment starting at lane `nxt` (if any) into `ahead` right after this segment's first
+    // run rows are requested
+    auto process = [&](int i, const RowState<MUL, VEC, NIT>& cur, int nxt, RowState<MUL, VEC, NIT>& ahead) {
+      const int s0 = base + i;
+      const int s1 = __builtin_amdgcn_readlane(my_s1, i);
+      const unsigned row_id = (unsigned)__builtin_amdgcn_readlane(my_id, i);
+      const int seg = __builtin_amdgcn_readlane(my_seg, i);
+      if (s1 > win_base + 64) {  // the segment runs past the window: restart the window at its first pair
+        win_base = s0;
+        load_window<SRC>(A, lane, win_base, my_key, my_c);
+      }
+      float g1[NIT][VEC], g2[NIT][VEC];
+      zero_acc<VEC, NIT>(g1, g2);
+      int j = s0 - win_base;
+      const int j_end = s1 - win_base;
+      RunSet<R> rs;
+      RunRows<SRC, VEC, NIT, R> rr;
+      collect_runs<SRC, R>(rs, j, j_end, my_key, my_c);
+      request_runs<SRC, VEC, NIT, R>(A, lane, rs, rr);
+      if (nxt >= 0) request_state<SRC, VEC, NIT>(A, lane, (unsigned)__builtin_amdgcn_readlane(my_id, nxt), ahead);
+      apply_runs<SRC, VEC, NIT, REG, R>(A, rs, rr, cur.e, g1, g2);
+      while (j < j_end) {
+        collect_runs<SRC, R>(rs, j, j_end, my_key, my_c);
+        request_runs<SRC, VEC, NIT, R>(A, lane, rs, rr);
+        apply_runs<SRC, VEC, NIT, REG, R>(A, rs, rr, cur.e, g1, g2);
+      }
+      finish_row<SRC, VEC, NIT, REG>(A, lane, row_id, seg, g1, g2, cur.e, cur.m, cur.v);
+    };
+    auto pop = [&]() {  // lane of the next short segment start in the chunk, -1 when none is left
+      if (todo == 0ull) return -1;
+      const int i = __builtin_ctzll(todo);
+      todo &= todo - 1;
+      return i;
+    };
+
+    RowState<MUL, VEC, NIT> sa, sb;
+    int i = pop();
+    request_state<SRC, VEC, NIT>(A, lane, (unsigned)__builtin_amdgcn_readlane(my_id, i), sa);
+    while (true) {
+      const int k = pop();
+      process(i, sa, k, sb);
+      if (k < 0) break;
+      i = pop();
+      process(k, sb, i, sa);
+      if (i < 0) break;
+    }
+  }
+}
+
+// Long segments: the sorted pair list is cut into fixed tiles, one wavefront per tile.  The part of a
+// long segment inside the tile is summed; a segment that lies wholly inside the tile is finished here,
+// otherwise the sum goes to the tile's tail row (segment continues past the tile end) or head row
+// (segment came in from the left and ends here).
+template <int SRC, int VEC, int NIT, bool REG>
+__global__ __launch_bounds__(256) void entity_tile_kernel(EntityArgs A) {
+  constexpr int MUL = src_mul(SRC);
+  constexpr int R = kRunsLong;
+  const int lane = threadIdx.x & 63;
+  const int wave = uniform(threadIdx.x >> 6);
+  const int t = blockIdx.x * 4 + wave;
+  const int p0 = t * A.tile;
+  if (p0 >= A.n_pairs) return;  // whole wavefront leaves; no workgroup barrier is used below
+  const int p1 = min(A.n_pairs, p0 + A.tile);
+
+  // most tiles hold short segments only: find that out with one parallel look and leave
+  bool any_long = false;
+  for (int base = p0; base < p1; base += 64) {
+    const int q = min(base + lane, p1 - 1);
+    const int sg = A.seg_of_pos[q];
+    any_long |= __ballot(A.seg_start[sg + 1] - A.seg_start[sg] > A.short_max) != 0ull;
+  }
+  if (!any_long) return;
+
+  int pos = p0;
+  while (pos < p1) {
+    const int seg = A.seg_of_pos[pos];
+    const int s0 = A.seg_start[seg], s1 = A.seg_start[seg + 1];
+    const int end = min(s1, p1);
+    if (s1 - s0 > A.short_max) {
+      const unsigned row_id = (unsigned)A.sorted_ids[pos];
+      const bool whole = s0 >= p0 && s1 <= p1;
+      RowState<MUL, VEC, NIT> st;
+      if (whole) {
+        request_state<SRC, VEC, NIT>(A, lane, row_id, st);
+      } else if (SRC != kSrcRows) {
+        load_row<MUL, VEC, NIT>(st.e, A.table + (size_t)row_id * A.ncol * VEC * MUL, A.ncol * VEC, A.ncol, lane);
+      }
+      float g1[NIT][VEC], g2[NIT][VEC];
+      zero_acc<VEC, NIT>(g1, g2);
+      for (int base = pos; base < end; base += 64) {
+        int my_key;
+        float my_c;
+        load_window<SRC>(A, lane, base, my_key, my_c);
+        int j = 0;
+        const int j_end = min(64, end - base);
+        while (j < j_end) {
+          RunSet<R> rs;
+          RunRows<SRC, VEC, NIT, R> rr;
+          collect_runs<SRC, R>(rs, j, j_end, my_key, my_c);
+          request_runs<SRC, VEC, NIT, R>(A, lane, rs, rr);
+          apply_runs<SRC, VEC, NIT, REG, R>(A, rs, rr, st.e, g1, g2);
+        }
+      }
+      if (whole)
+        finish_row<SRC, VEC, NIT, REG>(A, lane, row_id, seg, g1, g2, st.e, st.m, st.v);
+      else if (s1 > p1)
+        store_partial<SRC, VEC, NIT>(A, A.tail, t, lane, g1, g2);
+      else
+        store_partial<SRC, VEC, NIT>(A, A.head, t, lane, g1, g2);
+    }
+    pos = end;
+  }
+}
+
+// One workgroup per tile whose first segment is long, came in from the left and ends inside the tile:
+// adds that segment's partial rows (tails of the tiles it crossed, then this tile's head) in tile
+// order and finishes the row.  Every other workgroup leaves at once.
+template <int SRC, int VEC, int NIT, int NW, bool REG>
+__global__ __launch_bounds__(NW * 64) void entity_fixup_kernel(EntityArgs A) {
+  constexpr int MUL = src_mul(SRC);
+  extern __shared__ float lds[];
+  const int t = blockIdx.x;
+  const int p0 = t * A.tile;
+  if (p0 == 0 || p0 >= A.n_pairs) return;
+  const int p1 = min(A.n_pairs, p0 + A.tile);
+  const int seg = A.seg_of_pos[p0];
+  const int s0 = A.seg_start[seg], s1 = A.seg_start[seg + 1];
+  if (!(s0 < p0 && s1 <= p1 && s1 - s0 > A.short_max)) return;  // uniform over the workgroup
+  const int lane = threadIdx.x & 63;
+  const int wave = uniform(threadIdx.x >> 6);
+  const int half = A.ncol * VEC;
+  const size_t row_len = (size_t)half * MUL;
+  const int ts = s0 / A.tile;
+  const int n_parts = t - ts + 1;
+  const int per_wave = (n_parts + NW - 1) / NW;
+  const int j0 = wave * per_wave;
+  const int j1 = min(n_parts, j0 + per_wave);
+
+  // a few interleaved partial sums per wavefront keep several row loads in flight; they are folded
+  // in a fixed order, so the result depends only on the tiling
+  constexpr int ILP = NIT * MUL <= 2 ? 4 : (NIT * MUL <= 4 ? 2 : 1);
+  float acc[ILP][MUL][NIT][VEC];
+#pragma unroll
+  for (int k = 0; k < ILP; ++k)
+#pragma unroll
+    for (int h = 0; h < MUL; ++h)
+#pragma unroll
+      for (int it = 0; it < NIT; ++it)
+#pragma unroll
+        for (int x = 0; x < VEC; ++x) acc[k][h][it][x] = 0.f;
+  for (int j = j0; j < j1; j += ILP) {
+    RowRegs<MUL, VEC, NIT> r[ILP];
+#pragma unroll
+    for (int k = 0; k < ILP; ++k) {
+      const int tj = ts + min(j + k, j1 - 1);
+      load_row<MUL, VEC, NIT>(r[k], (tj < t ? A.tail : A.head) + (size_t)tj * row_len, half, A.ncol, lane);
+    }
+#pragma unroll
+    for (int k = 0; k < ILP; ++k) {
+      if (j + k < j1) {
+#pragma unroll
+        for (int h = 0; h < MUL; ++h)
+#pragma unroll
+          for (int it = 0; it < NIT; ++it)
+#pragma unroll
+            for (int x = 0; x < VEC; ++x) acc[k][h][it][x] += r[k].h[h][it].v[x];
+      }
+    }
+  }
+  float g1[NIT][VEC], g2[NIT][VEC];
+#pragma unroll
+  for (int it = 0; it < NIT; ++it)
+#pragma unroll
+    for (int x = 0; x < VEC; ++x) {
+      float s1 = acc[0][0][it][x], s2 = acc[0][MUL - 1][it][x];
+#pragma unroll
+      for (int k = 1; k < ILP; ++k) {
+        s1 += acc[k][0][it][x];
+        s2 += acc[k][MUL - 1][it][x];
+      }
+      g1[it][x] = s1;
+      g2[it][x] = MUL == 2 ? s2 : 0.f;
+    }
+  // combine the wavefront sums in wavefront order
+  if (wave > 0) store_partial<SRC, VEC, NIT>(A, lds, wave - 1, lane, g1, g2);
+  __syncthreads();
+  if (wave == 0) {
+    for (int w = 1; w < NW; ++w) {
+      RowRegs<MUL, VEC, NIT> o;
+      load_row<MUL, VEC, NIT>(o, lds + (size_t)(w - 1) * row_len, half, A.ncol, lane);
+#pragma unroll
+      for (int it = 0; it < NIT; ++it)
+#pragma unroll
+        for (int x = 0; x < VEC; ++x) {
+          g1[it][x] += o.h[0][it].v[x];
+          if (MUL == 2) g2[it][x] += o.h[MUL - 1][it].v[x];
+        }
+    }
+    const unsigned row_id = (unsigned)A.sorted_ids[p0];
+    RowRegs<MUL, VEC, NIT> e, m0, v0;
+    if (REG || A.adam_on) load_row<MUL, VEC, NIT>(e, A.table + (size_t)row_id * row_len, half, A.ncol, lane);
+    if (A.adam_on) {
+      load_row<MUL, VEC, NIT>(m0, A.m + (size_t)row_id * row_len, half, A.ncol, lane);
+      load_row<MUL, VEC, NIT>(v0, A.v + (size_t)row_id * row_len, half, A.ncol, lane);
+    }
+    finish_row<SRC, VEC, NIT, REG>(A, lane, row_id, seg, g1, g2, e, m0, v0);
+  }
+}
+
+template <int SRC, int VEC, int NIT, bool REG>
+int launch_entity_reg(hipStream_t st, const EntityArgs& A) {
+  const unsigned tiles = (unsigned)((A.n_pairs + A.tile - 1) / A.tile);
+  if (SRC != kSrcRows)
+    hipLaunchKernelGGL((entity_meta_kernel<SRC>), dim3((unsigned)((A.n_pairs + 255) / 256)), dim3(256), 0, st, A);
+  // short segments: a fixed grid of wavefronts strides over the segment list (its length lives on the device)
+  unsigned seg_blocks = (unsigned)((A.n_pairs + 3) / 4);
+  if (seg_blocks > 256u * 8u) seg_blocks = 256u * 8u;
+  hipLaunchKernelGGL((entity_segment_kernel<SRC, VEC, NIT, REG>), dim3(seg_blocks), dim3(256), 0, st, A);
+  hipLaunchKernelGGL((entity_tile_kernel<SRC, VEC, NIT, REG>), dim3((tiles + 3) / 4), dim3(256), 0, st, A);
+  const size_t row_bytes = (size_t)A.ncol * VEC * src_mul(SRC) * sizeof(float);
+  if (15 * row_bytes <= 60 * 1024)
+    hipLaunchKernelGGL((entity_fixup_kernel<SRC, VEC, NIT, 16, REG>), dim3(tiles), dim3(16 * 64), 15 * row_bytes, st, A);
+  else
+    hipLaunchKernelGGL((entity_fixup_kernel<SRC, VEC, NIT, 4, REG>), dim3(tiles), dim3(4 * 64), 3 * row_bytes, st, A);
+  return check_launch("entity backward");
+}
+
+template <int SRC, int VEC, int NIT>
+int launch_entity(hipStream_t st, const EntityArgs& A) {
+  if constexpr (SRC == mBetaKL) {
+    if (A.p.reg_on) return launch_entity_reg<SRC, VEC, NIT, true>(st, A);
+  }
+  return launch_entity_reg<SRC, VEC, NIT, false>(st, A);
+}
+
+// Instantiated once per source in its own translation unit (smx_entity_inst_*.hip).
+template <int SRC>
+int entity_dispatch(hipStream_t st, const EntityArgs& A, int vec, int nit) {
+  if (vec == 4) {
+    switch (nit) {
+      case 1: return launch_entity<SRC, 4, 1>(st, A);
+      case 2: return launch_entity<SRC, 4, 2>(st, A);
+      case 4: return launch_entity<SRC, 4, 4>(st, A);
+      default: return launch_entity<SRC, 4, 8>(st, A);
+    }
+  }
+  switch (nit) {
+    case 1: return launch_entity<SRC, 1, 1>(st, A);
+    case 2: return launch_entity<SRC, 1, 2>(st, A);
+    default: return launch_entity<SRC, 1, 4>(st, A);
+  }
+}
+
+}  // namespace smx

@@ -147,11 +147,21 @@ template <> struct ModelOps<mRotate> {
   }
 };
 
+// Out-of-line copies of the special functions for the fused kernels: their bodies are long, and the
+// fused kernels evaluate them inside fully unrolled register loops.
+static __device__ __noinline__ float digamma_call(float x) { return digamma(x); }
+static __device__ __noinline__ float trigamma_call(float x) { return trigamma(x); }
+static __device__ __noinline__ float lgamma_call(float x) { return m_lgamma(x); }
+
+// KL(Beta(e1,e2) || Beta(q.a,q.b)); same formulas as Term<kBetaKL, float>.
 template <> struct ModelOps<mBetaKL> {
   using Q = QPair;  // a = alpha, b = beta of the query
   static __device__ __forceinline__ Q prep(float q1, float q2) { return {q1, q2}; }
-  static __device__ __forceinline__ void fwd(float e1, float e2, const Q& q, float& a0, float&) {
-    a0 += Term<kBetaKL, float>::fwd(e1, e2, q.a, q.b);
+  static __device__ __forceinline__ void fwd(float ea, float eb, const Q& q, float& a0, float&) {
+    const float se = ea + eb, sq = q.a + q.b;
+    const float t1 = lgamma_call(q.a) + lgamma_call(q.b) + lgamma_call(se);
+    const float t2 = lgamma_call(ea) + lgamma_call(eb) + lgamma_call(sq);
+    a0 += t1 - t2 + (ea - q.a) * digamma_call(ea) + (eb - q.b) * digamma_call(eb) + (sq - se) * digamma_call(se);
   }
   static __device__ __forceinline__ float fold(float a0, float, const ScoreParams&) { return a0; }
   static __device__ __forceinline__ float score(float folded, const ScoreParams& p) { return p.gamma - folded; }
@@ -161,15 +171,15 @@ template <> struct ModelOps<mBetaKL> {
   }
   static __device__ __forceinline__ void bwd_e(float c0, float, float e1, float e2, const Q& q, float& ge1, float& ge2) {
     const float se = e1 + e2, sq = q.a + q.b;
-    const float common = (sq - se) * trigamma(se);
-    ge1 += c0 * ((e1 - q.a) * trigamma(e1) + common);
-    ge2 += c0 * ((e2 - q.b) * trigamma(e2) + common);
+    const float common = (sq - se) * trigamma_call(se);
+    ge1 += c0 * ((e1 - q.a) * trigamma_call(e1) + common);
+    ge2 += c0 * ((e2 - q.b) * trigamma_call(e2) + common);
   }
   static __device__ __forceinline__ void bwd_q(float c0, float, float e1, float e2, const Q& q, float& g1, float& g2) {
     const float se = e1 + e2, sq = q.a + q.b;
-    const float common = digamma(se) - digamma(sq);
-    g1 += c0 * (digamma(q.a) - digamma(e1) + common);
-    g2 += c0 * (digamma(q.b) - digamma(e2) + common);
+    const float common = digamma_call(se) - digamma_call(sq);
+    g1 += c0 * (digamma_call(q.a) - digamma_call(e1) + common);
+    g2 += c0 * (digamma_call(q.b) - digamma_call(e2) + common);
   }
 };
 

@@ -137,3 +137,52 @@ int smx_plan_build(void* stream, const int64_t* idx, size_t n_pairs, size_t n_ro
 }
 
 }  // extern "C"
+
+// ---- row gather -------------------------------------------------------------------------------
+// out[k,:] = table[idx[k],:], one wavefront per row with 16-byte column loads when alignment allows.
+// The plain lookup of the reference (smore/common/embedding/embed_rw.py:74-75) for callers that
+// need the rows themselves (positives, anchors) rather than a fused score.
+namespace smx {
+
+template <int VEC>
+__global__ __launch_bounds__(256) void gather_rows_kernel(const float* __restrict__ table,
+                                                          const long long* __restrict__ idx, float* __restrict__ out,
+                                                          int n, int ncol, unsigned long long n_rows, int* err) {
+  const int lane = threadIdx.x & 63;
+  const int k = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (k >= n) return;
+  long long row = idx[k];
+  if ((unsigned long long)row >= n_rows) {
+    if (err && lane == 0) *err = 1;
+    row = 0;
+  }
+  const size_t row_len = (size_t)ncol * VEC;
+  for (int c = lane; c < ncol; c += 64) {
+    if (VEC == 4)
+      reinterpret_cast<float4*>(out + (size_t)k * row_len)[c] =
+          reinterpret_cast<const float4*>(table + (size_t)row * row_len)[c];
+    else
+      out[(size_t)k * row_len + c] = table[(size_t)row * row_len + c];
+  }
+}
+
+}  // namespace smx
+
+extern "C" int smx_gather_rows(void* stream, const float* table, size_t n_rows, size_t row_len, const int64_t* idx,
+                               size_t n, float* out, int* err_flag) {
+  using namespace smx;
+  if (!table || !idx || !out) return fail(SMX_ERR_ARG, "null pointer in gather");
+  if (n == 0 || n > 0x7fffffffull || row_len == 0 || row_len > 0x7fffffffull)
+    return fail(SMX_ERR_SHAPE, "gather size out of range");
+  hipStream_t st = as_stream(stream);
+  const unsigned blocks = (unsigned)((n + 3) / 4);
+  if (row_len % 4 == 0 && aligned16(table) && aligned16(out))
+    hipLaunchKernelGGL(gather_rows_kernel<4>, dim3(blocks), dim3(256), 0, st, table,
+                       reinterpret_cast<const long long*>(idx), out, (int)n, (int)(row_len / 4),
+                       (unsigned long long)n_rows, err_flag);
+  else
+    hipLaunchKernelGGL(gather_rows_kernel<1>, dim3(blocks), dim3(256), 0, st, table,
+                       reinterpret_cast<const long long*>(idx), out, (int)n, (int)row_len, (unsigned long long)n_rows,
+                       err_flag);
+  return check_launch("gather rows");
+}

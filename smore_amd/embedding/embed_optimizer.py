@@ -1,0 +1,226 @@
+"""Sparse row optimizer for the entity table (surface of smore/common/embedding/embed_optimizer.py).
+
+Same driver protocol as the reference (training/train_process.py:172-220):
+    opt.zero_grad(); rows = sp_embed(ids, name) ... loss.backward(); opt.apply_grad(lr)
+and one addition, the gather-fused scorer
+    logit = opt.score_negatives(model, ids[B,K], q1, q2, gamma, cen)
+which stands for  gamma - dist(regularizer(sp_embed(ids).view(B,K,-1)), query)  without ever
+building the [B,K,row] tensor.  Everything after loss.backward() -- unique-merge of ids
+(embed_optimizer.py:39-42), segment sum of gradient rows (:45-48) and the lazy Adam update
+(:208-252) -- runs as the segment plan and the fused entity pass of libsmore_amd.so.
+"""
+from abc import ABC, abstractmethod
+
+import torch
+import torch.nn as nn
+
+from .. import _lib, fused
+from .sparse_embed import SparseEmbedding
+
+
+def merge_grad_indices(idx_list, n_rows):
+    """torch.unique(cat(idx_list), return_inverse=True) on the device (embed_optimizer.py:39-42).
+    Returns (merged_indices, inverse_indices, plan)."""
+    flat = torch.cat([i.reshape(-1) for i in idx_list], dim=0)
+    plan = fused.build_plan(flat, n_rows, want_inverse=True)
+    return plan.uniq, plan.inverse, plan
+
+
+def merge_grad_list(grad_list, plan):
+    """Segment sum of the concatenated gradient rows (embed_optimizer.py:45-48, reduce='sum')."""
+    grads = torch.cat(grad_list, dim=0).contiguous()
+    merged = torch.empty((plan.n_uniq, grads.shape[1]), dtype=torch.float32, device=grads.device)
+    fused.rows_backward(plan, grads, merged=merged)
+    return merged
+
+
+class EmbedLookupFunc(torch.autograd.Function):
+    """rows = table[indices]; backward hands (indices, grad_rows) to the optimizer
+    (embed_optimizer.py:51-66)."""
+
+    @staticmethod
+    def forward(ctx, embed_opt, dummy_tensor, indices, name):
+        ctx.embed_opt = embed_opt
+        ctx.indices = indices
+        ctx.idx_fwd = embed_opt.n_fwd
+        embed_opt.n_fwd += 1
+        with torch.no_grad():
+            table = embed_opt.sparse_embed.embedding.detach()
+            return fused.gather_rows(table, indices.to(table.device), embed_opt.err_flag)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        ctx.embed_opt.accumulate_grad(ctx.indices, grad_output, ctx.idx_fwd)
+        return None, None, None, None
+
+
+class _FusedScoreFunc(torch.autograd.Function):
+    """logit[b,k] = gamma - dist(table[ids[b,k]], q[b]); the entity gradient is not returned to
+    autograd but recorded with the optimizer, which reduces it per entity in apply_grad."""
+
+    @staticmethod
+    def forward(ctx, embed_opt, dummy_tensor, model, ids, params, q1, q2):
+        table = embed_opt.sparse_embed.embedding.detach()
+        with torch.no_grad():
+            score = fused.score_forward(model, table, ids, q1, q2, params, embed_opt.err_flag)
+        ctx.embed_opt, ctx.model, ctx.ids, ctx.params = embed_opt, model, ids, params
+        ctx.save_for_backward(q1.detach(), q2.detach() if q2 is not None else None, score)
+        ctx.idx_fwd = embed_opt.n_fwd
+        embed_opt.n_fwd += 1
+        return score
+
+    @staticmethod
+    def backward(ctx, gscore):
+        q1, q2, score = ctx.saved_tensors
+        opt = ctx.embed_opt
+        table = opt.sparse_embed.embedding.detach()
+        with torch.no_grad():
+            gscore = gscore.contiguous()
+            gq1, gq2 = fused.score_backward_query(ctx.model, table, ctx.ids, q1, q2, score, gscore, ctx.params)
+        opt.accumulate_fused(ctx.model, ctx.ids, q1, q2, score, gscore, ctx.params, ctx.idx_fwd)
+        return None, None, None, None, None, gq1, gq2
+
+
+class EmbeddingOptimizer(ABC):
+    """Base driver (embed_optimizer.py:69-163).  `args` needs .optim_mode, a tuple or tuple string
+    (mode, name, device, squeeze, queue) as in the reference, and .share_optim_stats."""
+
+    def __init__(self, args, sp_embed, gpu_id=0):
+        assert isinstance(sp_embed, SparseEmbedding)
+        self.args = args
+        self.sparse_embed = sp_embed
+        sp_embed.fwd_delegate = self.forward
+        self.dummy_tensor = nn.Parameter(torch.randn(1, 1))
+        self.grad_list, self.fused_list, self.has_grad_list = [], [], []
+        self.n_fwd = 0
+        self.step = 0
+        self.gpu_id = gpu_id
+        mode = args.optim_mode
+        if isinstance(mode, str):
+            mode = tuple(x.strip() for x in mode.strip("()").split(","))
+        self.optim_mode = mode
+        self.optimizer_name = mode[1]
+        self.squeeze = str(mode[3]).lower() in ("true", "1") if len(mode) > 3 else False
+        self.share_optim_stats = getattr(args, "share_optim_stats", True)
+        if sp_embed.embedding.device.type != "cuda":
+            raise _lib.SmxError("the entity table must live on the GPU (no CPU-table mode in this build)")
+        self.err_flag = fused.new_error_flag(sp_embed.embedding.device)
+        self.prepare_state()
+
+    # -- hooks of the concrete optimizer
+    @abstractmethod
+    def prepare_state(self):
+        ...
+
+    @abstractmethod
+    def update_from_plan(self, plan, grad_rows, lr):
+        """Segment-sum grad_rows [P,row] over plan and update the table rows of plan.uniq."""
+
+    @abstractmethod
+    def update_fused(self, plan, rec, lr):
+        """Same for one fused record whose entity gradient is recomputed on the fly."""
+
+    # -- protocol of the training loop
+    def zero_grad(self):
+        self.grad_list, self.fused_list, self.has_grad_list = [], [], []
+        self.n_fwd = 0
+
+    def share_memory(self):
+        pass  # state is device memory of one process
+
+    def accumulate_grad(self, indices, grad_submat, fwd_idx):
+        self.grad_list.append((indices, grad_submat))
+        self.has_grad_list.append(fwd_idx)
+
+    def accumulate_fused(self, model, ids, q1, q2, score, gscore, params, fwd_idx):
+        self.fused_list.append(dict(model=model, ids=ids, q1=q1, q2=q2, score=score, gscore=gscore, params=params))
+        self.has_grad_list.append(fwd_idx)
+
+    def forward(self, indices, name=None):
+        if indices is None:
+            mat = self.sparse_embed.embedding
+        else:
+            mat = EmbedLookupFunc.apply(self, self.dummy_tensor, indices, name)
+        mat.job_handle = self.sparse_embed.dummy_job
+        return mat
+
+    def score_negatives(self, model, ids, q1, q2=None, gamma=0.0, cen=0.0, regularizer=None):
+        """Gather-fused logits [B,K]; q1/q2 are [B,dim] or [B,1,dim] and receive gradients."""
+        table = self.sparse_embed.embedding
+        ids = ids.to(table.device).contiguous()
+        b = ids.shape[0]
+        q1c = q1.reshape(b, -1).contiguous()
+        q2c = None if q2 is None else q2.reshape(b, -1).contiguous()
+        params = fused.score_params(gamma, cen, regularizer)
+        return _FusedScoreFunc.apply(self, self.dummy_tensor, model, ids, params, q1c, q2c)
+
+    def check_ids(self):
+        """Raises if any lookup since the last check met an id outside the table (synchronises)."""
+        if int(self.err_flag.item()) != 0:
+            self.err_flag.zero_()
+            raise IndexError("entity id out of range in a sparse lookup")
+
+    def apply_grad(self, lr):
+        self.step += 1  # counts calls, also those without gradients (embed_optimizer.py:156)
+        if not self.grad_list and not self.fused_list:
+            return
+        n_rows = self.sparse_embed.num_rows
+        with torch.no_grad():
+            if len(self.fused_list) == 1 and not self.grad_list:
+                rec = self.fused_list[0]
+                plan = fused.build_plan(rec["ids"], n_rows, err_flag=self.err_flag)
+                self.update_fused(plan, rec, lr)
+                return
+            idx_list = [i.reshape(-1).to(self.sparse_embed.device) for i, _ in self.grad_list]
+            grad_list = [g.reshape(g.shape[0] if g.dim() == 2 else -1, g.shape[-1]).contiguous().float()
+                         for _, g in self.grad_list]
+            table = self.sparse_embed.embedding.detach()
+            for rec in self.fused_list:  # reduce each fused record to (distinct ids, summed rows) first
+                plan = fused.build_plan(rec["ids"], n_rows, err_flag=self.err_flag)
+                merged = torch.empty((plan.n_uniq, table.shape[1]), dtype=torch.float32, device=table.device)
+                fused.score_backward_entity(rec["model"], plan, table, rec["q1"], rec["q2"], rec["score"],
+                                            rec["gscore"], rec["params"], merged=merged)
+                idx_list.append(plan.uniq)
+                grad_list.append(merged)
+            flat = torch.cat(idx_list, dim=0)
+            plan = fused.build_plan(flat, n_rows, err_flag=self.err_flag)
+            self.update_from_plan(plan, torch.cat(grad_list, dim=0).contiguous(), lr)
+
+
+class AdamEmbedOptimizer(EmbeddingOptimizer):
+    """Lazy Adam with one global step counter (embed_optimizer.py:188-252).  State buffers carry the
+    reference's names, state_sum_fo / state_sum_sq, on the SparseEmbedding, so they are part of its
+    state_dict like there."""
+    beta1, beta2, eps = 0.9, 0.999, 1e-8  # embed_optimizer.py:209-210, consts.py:20
+
+    def prepare_state(self):
+        emb = self.sparse_embed
+        if self.squeeze:
+            raise NotImplementedError("squeezed second moment ([N,1]) is not built yet")
+        for name in ("state_sum_fo", "state_sum_sq"):
+            if not hasattr(emb, name):
+                emb.register_tensor(name, torch.zeros_like(emb.embedding.detach()))
+
+    def _adam(self, lr):
+        return fused.adam_params(lr, self.step, self.beta1, self.beta2, self.eps)
+
+    def update_from_plan(self, plan, grad_rows, lr):
+        emb = self.sparse_embed
+        fused.rows_backward(plan, grad_rows, table=emb.embedding.detach(), m=emb.state_sum_fo, v=emb.state_sum_sq,
+                            adam=self._adam(lr))
+
+    def update_fused(self, plan, rec, lr):
+        emb = self.sparse_embed
+        fused.score_backward_entity(rec["model"], plan, emb.embedding.detach(), rec["q1"], rec["q2"], rec["score"],
+                                    rec["gscore"], rec["params"], m=emb.state_sum_fo, v=emb.state_sum_sq,
+                                    adam=self._adam(lr))
+
+
+def get_optim_class(args):
+    """embed_optimizer.py:352-364; only Adam is built so far."""
+    mode = args.optim_mode
+    if isinstance(mode, str):
+        mode = tuple(x.strip() for x in mode.strip("()").split(","))
+    if mode[1] == "adam":
+        return AdamEmbedOptimizer
+    raise NotImplementedError(f"sparse optimizer '{mode[1]}' is not built yet")

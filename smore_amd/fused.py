@@ -97,6 +97,20 @@ def score_backward_query(model, table, idx, q1, q2, score, gscore, params):
     return gq1, gq2
 
 
+def gather_rows(table, idx, err_flag=None):
+    """rows = table[idx] (idx any shape, flattened) -> [idx.numel(), row]."""
+    _f32(table, "table")
+    if idx.dtype != torch.int64 or idx.device != table.device:
+        raise _lib.SmxError("idx must be an int64 tensor on the table's device")
+    flat = idx.reshape(-1).contiguous()
+    out = torch.empty((flat.numel(), table.shape[1]), dtype=torch.float32, device=table.device)
+    if flat.numel():
+        with torch.cuda.device(table.device):
+            _lib.call("smx_gather_rows", _stream(table), _ptr(table), table.shape[0], table.shape[1], _ptr(flat),
+                      flat.numel(), _ptr(out), _ptr(err_flag))
+    return out
+
+
 class SegmentPlan:
     """Device-resident result of grouping one step's pairs by entity id (see smx_plan_build)."""
 

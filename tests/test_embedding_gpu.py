@@ -1,0 +1,165 @@
+"""The sparse-embedding driver protocol (zero_grad -> lookups/scores -> backward -> apply_grad) on the
+HIP path, against the CPU oracle's float64 pipeline."""
+import types
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle as orc
+from tests.util import REL_F32, assert_close
+
+pytestmark = pytest.mark.gpu
+
+
+def _setup(n, d, seed):
+    from smore_amd.embedding.embed_optimizer import AdamEmbedOptimizer
+    from smore_amd.embedding.sparse_embed import SparseEmbedding
+    torch.manual_seed(seed)
+    emb = SparseEmbedding(n, d).cuda()
+    emb.init_params(-0.07, 0.07)
+    args = types.SimpleNamespace(optim_mode="(aggr,adam,gpu,False,5)", share_optim_stats=True)
+    opt = AdamEmbedOptimizer(args, emb, 0)
+    return emb, opt
+
+
+def test_lookup_and_plain_gradients_match_oracle():
+    """positives + negatives through plain lookups and the autograd box operators, one Adam step."""
+    from smore_amd.torchext import ext_ops
+    n, d, b, k, lr = 300, 32, 6, 9, 1e-3
+    emb, opt = _setup(n, d, 1)
+    w0 = emb.embedding.detach().cpu().numpy().astype(np.float64)
+    rng = np.random.default_rng(2)
+    pos = torch.tensor(rng.integers(0, n, b), device="cuda")
+    neg = torch.tensor(rng.integers(0, n, (b, k)), device="cuda")
+    c = torch.tensor(rng.uniform(-0.07, 0.07, (b, 1, d)), dtype=torch.float32, device="cuda", requires_grad=True)
+    o = torch.tensor(np.abs(rng.uniform(-0.07, 0.07, (b, 1, d))), dtype=torch.float32, device="cuda", requires_grad=True)
+    gp = torch.tensor(rng.standard_normal((b, 1)), dtype=torch.float32, device="cuda")
+    gn = torch.tensor(rng.standard_normal((b, k)), dtype=torch.float32, device="cuda")
+
+    opt.zero_grad()
+    rows_p = emb(pos, "positive_entity")
+    rows_n = emb(neg.view(-1), "negative_entity")
+    assert rows_p.shape == (b, d) and rows_n.shape == (b * k, d)
+    rows_p.job_handle.sync()
+    assert torch.equal(rows_p, emb.embedding.detach()[pos])
+
+    def logit(rows):
+        return 24 - ext_ops.box_dist_out(rows, c, o) - 0.02 * ext_ops.box_dist_in(rows, c, o)
+
+    lp = logit(rows_p.unsqueeze(1))
+    ln = logit(rows_n.view(b, k, -1))
+    ((lp * gp).sum() + (ln * gn).sum()).backward()
+    opt.apply_grad(lr)
+    opt.check_ids()
+
+    # oracle: same pipeline in float64
+    cn, on = c.detach().cpu().numpy().astype(np.float64), o.detach().cpu().numpy().astype(np.float64)
+    gpn, gnn = gp.cpu().numpy().astype(np.float64), gn.cpu().numpy().astype(np.float64)
+    pos_n, neg_n = pos.cpu().numpy(), neg.cpu().numpy()
+    rp = orc.gather(w0, pos_n).reshape(b, 1, d)
+    rn = orc.gather(w0, neg_n).reshape(b, k, d)
+    assert_close(lp.detach().cpu().numpy(), orc.score_forward("box", rp, cn, on, 24.0, 0.02), REL_F32, "pos logit")
+    assert_close(ln.detach().cpu().numpy(), orc.score_forward("box", rn, cn, on, 24.0, 0.02), REL_F32, "neg logit")
+    g_rp, gc_p, go_p = orc.score_backward("box", gpn, rp, cn, on, 0.02)
+    g_rn, gc_n, go_n = orc.score_backward("box", gnn, rn, cn, on, 0.02)
+    assert_close(c.grad.cpu().numpy(), gc_p + gc_n, REL_F32, "center grad")
+    assert_close(o.grad.cpu().numpy(), go_p + go_n, REL_F32, "offset grad")
+    all_idx = np.concatenate([pos_n.reshape(-1), neg_n.reshape(-1)])
+    all_g = np.concatenate([g_rp.reshape(b, d), g_rn.reshape(b * k, d)])
+    uniq, inverse, _, _ = orc.merge_indices(all_idx)
+    merged = orc.merge_grads(all_g, inverse, uniq.size)
+    w, m, v = w0.copy(), np.zeros_like(w0), np.zeros_like(w0)
+    orc.adam_rows(w, m, v, uniq, merged, lr, 1)
+    got = emb.embedding.detach().cpu().numpy()
+    touched = np.zeros(n, bool)
+    touched[uniq] = True
+    err = np.abs(got - w)[touched]
+    assert (err > 1e-5 * np.maximum(np.abs(w[touched]), 0.04)).mean() < 1e-3 and err.max() < lr
+    assert np.array_equal(got[~touched], w0[~touched].astype(np.float32))
+    assert_close(emb.state_sum_fo.cpu().numpy()[touched], m[touched], REL_F32, "first moment")
+
+
+def test_fused_scorer_alone_and_mixed_with_plain_lookup():
+    """score_negatives (gather-fused) gives the same step as plain lookups + autograd operators,
+    both alone and when a plain positive lookup shares the step."""
+    from smore_amd.torchext import ext_ops
+    n, d, b, k, lr = 500, 64, 8, 16, 1e-3
+    rng = np.random.default_rng(3)
+    pos_n = rng.integers(0, n, b)
+    neg_n = rng.integers(0, n // 10, (b, k))  # few distinct ids: long segments
+    cn = rng.uniform(-0.07, 0.07, (b, 1, d)).astype(np.float32)
+    on = np.abs(rng.uniform(-0.07, 0.07, (b, 1, d))).astype(np.float32)
+    gp_n = rng.standard_normal((b, 1)).astype(np.float32)
+    gn_n = rng.standard_normal((b, k)).astype(np.float32)
+
+    def run(fused_neg, with_pos):
+        emb, opt = _setup(n, d, 5)
+        c = torch.tensor(cn, device="cuda", requires_grad=True)
+        o = torch.tensor(on, device="cuda", requires_grad=True)
+        pos, neg = torch.tensor(pos_n, device="cuda"), torch.tensor(neg_n, device="cuda")
+        for step in range(2):
+            opt.zero_grad()
+            c.grad = o.grad = None
+            loss = 0
+            if with_pos:
+                rp = emb(pos, "positive_entity").unsqueeze(1)
+                lp = 24 - ext_ops.box_dist_out(rp, c, o) - 0.02 * ext_ops.box_dist_in(rp, c, o)
+                loss = loss + (lp * torch.tensor(gp_n, device="cuda")).sum()
+            if fused_neg:
+                ln = opt.score_negatives("box", neg, c, o, gamma=24.0, cen=0.02)
+            else:
+                rn = emb(neg.view(-1), "negative_entity").view(b, k, -1)
+                ln = 24 - ext_ops.box_dist_out(rn, c, o) - 0.02 * ext_ops.box_dist_in(rn, c, o)
+            loss = loss + (ln * torch.tensor(gn_n, device="cuda")).sum()
+            loss.backward()
+            opt.apply_grad(lr)
+        opt.check_ids()
+        return (emb.embedding.detach().cpu().numpy(), emb.state_sum_fo.cpu().numpy(), emb.state_sum_sq.cpu().numpy(),
+                c.grad.cpu().numpy(), o.grad.cpu().numpy(), ln.detach().cpu().numpy())
+
+    for with_pos in (False, True):
+        a = run(True, with_pos)
+        r = run(False, with_pos)
+        assert_close(a[5], r[5], REL_F32, "logits")
+        assert_close(a[3], r[3], REL_F32, "center grad")
+        assert_close(a[4], r[4], REL_F32, "offset grad")
+        assert_close(a[1], r[1], 5 * REL_F32, "first moment")
+        err = np.abs(a[0] - r[0])
+        assert (err > 1e-5 * np.maximum(np.abs(r[0]), 0.04)).mean() < 1e-3 and err.max() < 2 * lr
+
+
+def test_step_counter_and_empty_steps():
+    emb, opt = _setup(50, 8, 7)
+    opt.zero_grad()
+    opt.apply_grad(1e-3)  # no gradients: the counter still advances (embed_optimizer.py:156-158)
+    assert opt.step == 1
+    w0 = emb.embedding.detach().clone()
+    opt.zero_grad()
+    rows = emb(torch.tensor([3, 3, 7], device="cuda"), "x")
+    (rows.sum() * 2.0).backward()
+    opt.apply_grad(1e-2)
+    assert opt.step == 2
+    w = emb.embedding.detach()
+    changed = (w != w0).any(dim=1).nonzero().flatten().tolist()
+    assert changed == [3, 7]
+    # bias correction uses the global step (2), not the row's own first touch
+    g = np.array([4.0, 2.0])  # row 3 was looked up twice
+    m1, v1 = 0.1 * g, 0.001 * g * g
+    want = -1e-2 / (1 - 0.9 ** 2) * m1 / (np.sqrt(v1) / np.sqrt(1 - 0.999 ** 2) + 1e-8)
+    got = (w - w0)[[3, 7], 0].cpu().numpy()
+    assert np.allclose(got, want, rtol=1e-4)
+
+
+def test_out_of_range_lookup_is_reported():
+    emb, opt = _setup(20, 8, 9)
+    opt.zero_grad()
+    emb(torch.tensor([1, 25], device="cuda"), "x")
+    with pytest.raises(IndexError):
+        opt.check_ids()
+
+
+def test_state_buffers_are_in_the_state_dict():
+    emb, _ = _setup(20, 8, 11)
+    sd = emb.state_dict()
+    assert {"embedding", "state_sum_fo", "state_sum_sq"} <= set(sd)
