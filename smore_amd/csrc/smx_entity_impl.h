@@ -57,8 +57,6 @@ struct EntityArgs {
   const float* gscore;
   int K;
   ScoreParams p;
-  float* meta_c;  // [P] upstream coefficient of every sorted position
-  int* meta_b;    // [P] query number of every sorted position
   // source: gradient rows
   const float* grad_rows;
   // entity table (read for the model sources, updated when adam_on)
@@ -229,8 +227,10 @@ __device__ __forceinline__ void load_window(const EntityArgs& A, int lane, int b
     my_key = A.order[pos];
     my_c = 0.f;
   } else {
-    my_key = A.meta_b[pos];
-    my_c = A.meta_c[pos];
+    const int pair = A.order[pos];
+    float c1;
+    ModelOps<SRC>::coef(A.gscore[pair], A.score[pair], A.p, my_c, c1);
+    my_key = pair / A.K;
   }
 }
 
@@ -317,22 +317,6 @@ __device__ __forceinline__ void zero_acc(float (&g1)[NIT][VEC], float (&g2)[NIT]
 #pragma unroll
     for (int x = 0; x < VEC; ++x) g1[it][x] = g2[it][x] = 0.f;
 }
-
-// Sorted copy of what the entity pass needs per pair, so that the pass reads it contiguously:
-// meta_c[pos] = d loss / d distance of the pair at sorted position pos, meta_b[pos] = its query.
-template <int SRC>
-__global__ __launch_bounds__(256) void entity_meta_kernel(EntityArgs A) {
-  const int pos = blockIdx.x * blockDim.x + threadIdx.x;
-  if (pos >= A.n_pairs) return;
-  if constexpr (SRC != kSrcRows) {
-    const int pair = A.order[pos];
-    float c0, c1;
-    ModelOps<SRC>::coef(A.gscore[pair], A.score[pair], A.p, c0, c1);
-    A.meta_c[pos] = c0;
-    A.meta_b[pos] = pair / A.K;
-  }
-}
-
 
 constexpr int kRunsShort = 2;  // runs in flight per wavefront in the short-segment kernel
 constexpr int kRunsLong = 4;   // ... in the long-segment kernel
@@ -598,8 +582,6 @@ __global__ __launch_bounds__(NW * 64) void entity_fixup_kernel(EntityArgs A) {
 template <int SRC, int VEC, int NIT, bool REG>
 int launch_entity_reg(hipStream_t st, const EntityArgs& A) {
   const unsigned tiles = (unsigned)((A.n_pairs + A.tile - 1) / A.tile);
-  if (SRC != kSrcRows)
-    hipLaunchKernelGGL((entity_meta_kernel<SRC>), dim3((unsigned)((A.n_pairs + 255) / 256)), dim3(256), 0, st, A);
   // short segments: a fixed grid of wavefronts strides over the segment list (its length lives on the device)
   unsigned seg_blocks = (unsigned)((A.n_pairs + 3) / 4);
   if (seg_blocks > 256u * 8u) seg_blocks = 256u * 8u;

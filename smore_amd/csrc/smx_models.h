@@ -53,6 +53,12 @@ struct QPair {
 
 template <int M> struct ModelOps;
 
+// Hook applied once to a lane's accumulated query gradient before it leaves the registers
+// (identity unless a model defers part of its derivative, as BOX does).
+template <int M>
+__device__ __forceinline__ void finish_query_grad(const typename ModelOps<M>::Q& q, float& g1, float& g2,
+                                                  const ScoreParams& p);
+
 template <> struct ModelOps<mL1> {
   using Q = QPair;
   static __device__ __forceinline__ Q prep(float q1, float) { return {q1, 0.f}; }
@@ -99,13 +105,26 @@ template <> struct ModelOps<mL2> {
   }
 };
 
-// acc0 = outside distance, acc1 = inside distance; one row read serves both.
+// Query2box: acc0 = outside distance, acc1 = inside distance; one row read serves both.
+//
+// With d = e - c, a = |d|, the terms of smore/common/torchext/dist_kernel.h:58-105 are
+//   out = relu(a - o) = a - min(a, o)      (bit-identical: a - o when a > o, else a - a = 0)
+//   in  = |min(a, o)|
+// and their derivatives, with "outside" := (a - o >= 0), c0 / c1 the coefficients on out / in:
+//   outside:  d/de = s_out c0,  d/dc = -s_out c0,  d/do = -c0 + sgn(o) c1   s_out = (d > 0 ? 1 : -1), sgn(o) = (o > 0 ? 1 : -1)
+//   inside :  d/de = s_in  c1,  d/dc = -s_in  c1,  d/do = 0                 s_in  = (d >= 0 ? 1 : -1)
+// (inside means a < o, so min(a,o) = a, the outer sign of the reference is -1 exactly when a == 0,
+// where its inner sign is -1 too: the product is +1 there and sgn(d) elsewhere, i.e. s_in.)
+// The offset gradient of a whole query is therefore (sgn(o) cen - 1) * sum over outside pairs of
+// c0, so the loop only accumulates that sum and the factor is applied once at the end.
 template <> struct ModelOps<mBox> {
   using Q = QPair;  // a = center, b = offset
   static __device__ __forceinline__ Q prep(float q1, float q2) { return {q1, q2}; }
   static __device__ __forceinline__ void fwd(float e1, float, const Q& q, float& a0, float& a1) {
-    a0 += Term<kBoxOut, float>::fwd(e1, 0.f, q.a, q.b);
-    a1 += Term<kBoxIn, float>::fwd(e1, 0.f, q.a, q.b);
+    const float a = fabsf(e1 - q.a);
+    const float mn = fminf(a, q.b);
+    a0 += a - mn;
+    a1 += fabsf(mn);
   }
   static __device__ __forceinline__ float fold(float a0, float a1, const ScoreParams& p) { return a0 + p.cen * a1; }
   static __device__ __forceinline__ float score(float folded, const ScoreParams& p) { return p.gamma - folded; }
@@ -113,15 +132,26 @@ template <> struct ModelOps<mBox> {
     c0 = -g;
     c1 = -p.cen * g;
   }
-  static __device__ __forceinline__ void bwd_e(float c0, float c1, float e1, float, const Q& q, float& ge1, float&) {
-    float s1 = 0, s2 = 0, s3 = 0;
-    Term<kBoxOut, float>::bwd(c0, e1, 0.f, q.a, q.b, ge1, s1, s2, s3);
-    Term<kBoxIn, float>::bwd(c1, e1, 0.f, q.a, q.b, ge1, s1, s2, s3);
+  // gradient of the entity feature; the center's is its negative
+  static __device__ __forceinline__ float de(float c0, float c1, float e1, const Q& q, bool& outside) {
+    const float d = e1 - q.a;
+    outside = fabsf(d) - q.b >= 0.f;
+    const float w = outside ? c0 : c1;
+    const bool positive = outside ? (d > 0.f) : (d >= 0.f);
+    return positive ? w : -w;
   }
+  static __device__ __forceinline__ void bwd_e(float c0, float c1, float e1, float, const Q& q, float& ge1, float&) {
+    bool outside;
+    ge1 += de(c0, c1, e1, q, outside);
+  }
+  // gc accumulates the center gradient; go accumulates sum(c0 over outside pairs), see finish_q
   static __device__ __forceinline__ void bwd_q(float c0, float c1, float e1, float, const Q& q, float& gc, float& go) {
-    float s1 = 0, s2 = 0;
-    Term<kBoxOut, float>::bwd(c0, e1, 0.f, q.a, q.b, s1, s2, gc, go);
-    Term<kBoxIn, float>::bwd(c1, e1, 0.f, q.a, q.b, s1, s2, gc, go);
+    bool outside;
+    gc -= de(c0, c1, e1, q, outside);
+    go += outside ? c0 : 0.f;
+  }
+  static __device__ __forceinline__ void finish_q(const Q& q, float&, float& go, const ScoreParams& p) {
+    go *= (q.b > 0.f ? p.cen : -p.cen) - 1.0f;
   }
 };
 
@@ -182,5 +212,11 @@ template <> struct ModelOps<mBetaKL> {
     g2 += c0 * (digamma_call(q.b) - digamma_call(e2) + common);
   }
 };
+
+template <int M>
+__device__ __forceinline__ void finish_query_grad(const typename ModelOps<M>::Q& q, float& g1, float& g2,
+                                                  const ScoreParams& p) {
+  if constexpr (M == mBox) ModelOps<mBox>::finish_q(q, g1, g2, p);
+}
 
 }  // namespace smx

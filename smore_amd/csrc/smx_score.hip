@@ -12,8 +12,8 @@
 //
 // Work split.  forward: workgroup = (query b, tile of negatives); the query
 // row(s) are staged once in LDS, every lane then keeps the features it owns in
-// registers for the whole tile; the four wavefronts take turns on the tile's
-// rows, several rows in flight per wavefront.  backward: one workgroup per
+// registers for the whole tile; each of the four wavefronts streams its
+// quarter of the tile's rows, two batches of rows in flight at a time.  backward: one workgroup per
 // query walks all K negatives, wavefront partial sums are combined through LDS
 // in wavefront order, so the gradient has a fixed summation order.
 #include "smx_common.h"
@@ -67,33 +67,73 @@ __device__ __forceinline__ void stage_query(float* lds, const float* __restrict_
   __syncthreads();
 }
 
-// Entity row of pair `pair`: through idx when given, else the dense [B*K, row_len] layout.  The id is
-// wave-uniform, so the range check and the 64-bit row offset stay on the scalar unit.  An id outside
-// the table is replaced by row 0 and remembered in `bad`.
-__device__ __forceinline__ const float* pair_row(const float* __restrict__ table, const long long* __restrict__ idx,
-                                                 size_t pair, size_t row_len, unsigned long long n_rows, int& bad) {
+// ---- streaming the rows of up to 64 pairs through a wavefront -----------------------------------
+// The lanes first fetch, in one coalesced load, the ids of the pairs the wavefront is about to
+// process (pair j of the batch lives in lane j) and turn them into row offsets.  The row loop then
+// needs no memory access to find a row: the offset comes out of lane j with two v_readlane, so the
+// only loads in the loop are the rows themselves.  Rows are requested RIF at a time into two
+// register sets used in turn: while set A is consumed, set B is already on its way.  All loads are
+// unconditional (indices are clamped) so that they issue as one batch and stay in flight together.
+
+struct PairBatch {
+  unsigned off_lo, off_hi;  // this lane's pair: offset of its entity row in floats
+};
+
+__device__ __forceinline__ PairBatch load_pair_batch(const long long* __restrict__ idx, size_t first_pair, int cnt,
+                                                     int lane, size_t row_len, unsigned long long n_rows, int& bad) {
+  const size_t pair = first_pair + min(lane, cnt - 1);
   long long row = idx ? idx[pair] : (long long)pair;
-  if ((unsigned long long)row >= n_rows) {
+  if ((unsigned long long)row >= n_rows) {  // id outside the table: remember it, read row 0 instead
     bad = 1;
     row = 0;
   }
-  return table + (size_t)row * row_len;
+  const unsigned long long off = (unsigned long long)row * row_len;
+  return {(unsigned)off, (unsigned)(off >> 32)};
 }
 
-// Loads the columns a lane owns of RIF rows.  Column and row numbers are clamped instead of
-// predicated, so the loads form one straight-line batch that stays in flight together; lanes
-// beyond the row end re-read its last column (same cache line) and are masked in the arithmetic.
+__device__ __forceinline__ const float* batch_row(const float* __restrict__ table, const PairBatch& pb, int j) {
+  const unsigned lo = (unsigned)__builtin_amdgcn_readlane((int)pb.off_lo, j);
+  const unsigned hi = (unsigned)__builtin_amdgcn_readlane((int)pb.off_hi, j);
+  return table + (((unsigned long long)hi << 32) | lo);
+}
+
+template <int MUL, int VEC, int NIT, int RIF> struct RowSet {
+  Pack<VEC> e1[RIF][NIT];
+  Pack<VEC> e2[RIF][NIT];
+};
+
+// Requests rows j0 .. j0+RIF-1 of the batch (clamped to cnt-1).
 template <int MUL, int VEC, int NIT, int RIF>
-__device__ __forceinline__ void load_rows(const float* const (&pe)[RIF], int dim, int ncol, int lane,
-                                          Pack<VEC> (&e1)[RIF][NIT], Pack<VEC> (&e2)[RIF][NIT]) {
+__device__ __forceinline__ void request_rows(RowSet<MUL, VEC, NIT, RIF>& rs, const float* __restrict__ table,
+                                             const PairBatch& pb, int j0, int cnt, int dim, int ncol, int lane) {
 #pragma unroll
   for (int r = 0; r < RIF; ++r) {
+    const float* pe = batch_row(table, pb, min(j0 + r, cnt - 1));
 #pragma unroll
     for (int it = 0; it < NIT; ++it) {
       const int c = min(lane + 64 * it, ncol - 1);
-      e1[r][it] = load_pack<VEC>(pe[r], c);
-      if (MUL == 2) e2[r][it] = load_pack<VEC>(pe[r] + dim, c);
+      rs.e1[r][it] = load_pack<VEC>(pe, c);
+      if (MUL == 2) rs.e2[r][it] = load_pack<VEC>(pe + dim, c);
     }
+  }
+}
+
+// Streams the cnt (<= 64) rows of a batch through `consume(j, e1, e2)`, j ascending.
+template <int MUL, int VEC, int NIT, int RIF, class Consume>
+__device__ __forceinline__ void stream_batch(const float* __restrict__ table, const PairBatch& pb, int cnt, int dim,
+                                             int ncol, int lane, Consume&& consume) {
+  RowSet<MUL, VEC, NIT, RIF> a, b;
+  const int last = ((cnt - 1) / RIF) * RIF;  // first row of the last group
+  request_rows<MUL, VEC, NIT, RIF>(a, table, pb, 0, cnt, dim, ncol, lane);
+  for (int j0 = 0; j0 < cnt; j0 += 2 * RIF) {
+    request_rows<MUL, VEC, NIT, RIF>(b, table, pb, min(j0 + RIF, last), cnt, dim, ncol, lane);
+#pragma unroll
+    for (int r = 0; r < RIF; ++r)
+      if (j0 + r < cnt) consume(j0 + r, a.e1[r], a.e2[r]);
+    request_rows<MUL, VEC, NIT, RIF>(a, table, pb, min(j0 + 2 * RIF, last), cnt, dim, ncol, lane);
+#pragma unroll
+    for (int r = 0; r < RIF; ++r)
+      if (j0 + RIF + r < cnt) consume(j0 + RIF + r, b.e1[r], b.e2[r]);
   }
 }
 
@@ -113,40 +153,39 @@ __global__ __launch_bounds__(256) void score_forward_kernel(const float* __restr
   const int dim = ncol * VEC;
   const size_t row_len = (size_t)dim * MUL;
 
+  // this wavefront's share of the tile: per_wave (<= 64) consecutive negatives
+  const int per_wave = tile_k / 4;
+  const int kw0 = tile * tile_k + wave * per_wave;
+  const int cnt = min(per_wave, K - kw0);
+  int bad = 0;
+  PairBatch pb{0u, 0u};
+  if (cnt > 0) pb = load_pair_batch(idx, (size_t)b * K + kw0, cnt, lane, row_len, n_rows, bad);
+
   stage_query<M>(lds, q1, q2, b, dim);
   typename ModelOps<M>::Q q[NIT][VEC];
   load_query_regs<M, VEC, NIT>(lds, dim, ncol, lane, q);
+  if (cnt <= 0) return;
 
-  const int k0 = tile * tile_k;
-  const int k1 = min(K, k0 + tile_k);
-  int bad = 0;
-  for (int kb = k0 + wave * RIF; kb < k1; kb += 4 * RIF) {
-    const float* pe[RIF];
+  float* out = score + (size_t)b * K + kw0;
+  stream_batch<MUL, VEC, NIT, RIF>(table, pb, cnt, dim, ncol, lane,
+                                   [&](int j, const Pack<VEC>(&e1)[NIT], const Pack<VEC>(&e2)[NIT]) {
+    float a0 = 0.f, a1 = 0.f;
 #pragma unroll
-    for (int r = 0; r < RIF; ++r)
-      pe[r] = pair_row(table, idx, (size_t)b * K + min(kb + r, k1 - 1), row_len, n_rows, bad);
-    Pack<VEC> e1[RIF][NIT], e2[RIF][NIT];
-    load_rows<MUL, VEC, NIT, RIF>(pe, dim, ncol, lane, e1, e2);
+    for (int it = 0; it < NIT; ++it) {
+      if (lane + 64 * it < ncol) {
 #pragma unroll
-    for (int r = 0; r < RIF; ++r) {
-      float a0 = 0.f, a1 = 0.f;
-#pragma unroll
-      for (int it = 0; it < NIT; ++it) {
-        if (lane + 64 * it < ncol) {
-#pragma unroll
-          for (int v = 0; v < VEC; ++v) {
-            const float x1 = REG ? reg_apply(e1[r][it].v[v], p) : e1[r][it].v[v];
-            const float x2 = MUL == 2 ? (REG ? reg_apply(e2[r][it].v[v], p) : e2[r][it].v[v]) : 0.f;
-            ModelOps<M>::fwd(x1, x2, q[it][v], a0, a1);
-          }
+        for (int v = 0; v < VEC; ++v) {
+          const float x1 = REG ? reg_apply(e1[it].v[v], p) : e1[it].v[v];
+          const float x2 = MUL == 2 ? (REG ? reg_apply(e2[it].v[v], p) : e2[it].v[v]) : 0.f;
+          ModelOps<M>::fwd(x1, x2, q[it][v], a0, a1);
         }
       }
-      // the logit is linear in the accumulators: fold them per lane, reduce once
-      const float folded = wave_sum_f32(ModelOps<M>::fold(a0, a1, p));
-      if (lane == 0 && kb + r < k1) score[(size_t)b * K + kb + r] = ModelOps<M>::score(folded, p);
     }
-  }
-  if (bad && err && lane == 0) *err = 1;
+    // the logit is linear in the accumulators: fold them per lane, reduce once
+    const float folded = wave_sum_f32(ModelOps<M>::fold(a0, a1, p));
+    if (lane == 0) out[j] = ModelOps<M>::score(folded, p);
+  });
+  if (__ballot(bad != 0) != 0ull && err && lane == 0) *err = 1;
 }
 
 template <int M, int VEC, int NIT, int RIF, int NW, bool REG>
@@ -173,34 +212,40 @@ __global__ __launch_bounds__(NW * 64) void score_backward_query_kernel(
 #pragma unroll
     for (int v = 0; v < VEC; ++v) g1[it][v] = g2[it][v] = 0.f;
 
+  // this wavefront's share of the query's negatives: a contiguous range, walked in batches of 64
+  const int per_wave = (K + NW - 1) / NW;
+  const int kw0 = wave * per_wave;
+  const int kw1 = min(K, kw0 + per_wave);
   int bad = 0;
-  for (int kb = wave * RIF; kb < K; kb += NW * RIF) {
-    const float* pe[RIF];
-    float c0[RIF], c1[RIF];
-#pragma unroll
-    for (int r = 0; r < RIF; ++r) {
-      const size_t pair = (size_t)b * K + min(kb + r, K - 1);
-      pe[r] = pair_row(table, idx, pair, row_len, n_rows, bad);
-      ModelOps<M>::coef(gscore[pair], score[pair], p, c0[r], c1[r]);
-      if (kb + r >= K) c0[r] = c1[r] = 0.f;  // rows past the end contribute nothing
-    }
-    Pack<VEC> e1[RIF][NIT], e2[RIF][NIT];
-    load_rows<MUL, VEC, NIT, RIF>(pe, dim, ncol, lane, e1, e2);
-#pragma unroll
-    for (int r = 0; r < RIF; ++r) {
+  for (int kb = kw0; kb < kw1; kb += 64) {
+    const int cnt = min(64, kw1 - kb);
+    const size_t first = (size_t)b * K + kb;
+    const PairBatch pb = load_pair_batch(idx, first, cnt, lane, row_len, n_rows, bad);
+    const size_t mine = first + min(lane, cnt - 1);
+    float my_c0, my_c1;
+    ModelOps<M>::coef(gscore[mine], score[mine], p, my_c0, my_c1);
+    stream_batch<MUL, VEC, NIT, RIF>(table, pb, cnt, dim, ncol, lane,
+                                     [&](int j, const Pack<VEC>(&e1)[NIT], const Pack<VEC>(&e2)[NIT]) {
+      const float c0 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(my_c0), j));
+      const float c1 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(my_c1), j));
 #pragma unroll
       for (int it = 0; it < NIT; ++it) {
         if (lane + 64 * it < ncol) {
 #pragma unroll
           for (int v = 0; v < VEC; ++v) {
-            const float x1 = REG ? reg_apply(e1[r][it].v[v], p) : e1[r][it].v[v];
-            const float x2 = MUL == 2 ? (REG ? reg_apply(e2[r][it].v[v], p) : e2[r][it].v[v]) : 0.f;
-            ModelOps<M>::bwd_q(c0[r], c1[r], x1, x2, q[it][v], g1[it][v], g2[it][v]);
+            const float x1 = REG ? reg_apply(e1[it].v[v], p) : e1[it].v[v];
+            const float x2 = MUL == 2 ? (REG ? reg_apply(e2[it].v[v], p) : e2[it].v[v]) : 0.f;
+            ModelOps<M>::bwd_q(c0, c1, x1, x2, q[it][v], g1[it][v], g2[it][v]);
           }
         }
       }
-    }
+    });
   }
+
+#pragma unroll
+  for (int it = 0; it < NIT; ++it)
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) finish_query_grad<M>(q[it][v], g1[it][v], g2[it][v], p);
 
   // wavefront partials -> LDS -> fixed-order sum over wavefronts
   float* part = lds + NQ * dim;  // [NW][NQ][dim]
@@ -258,17 +303,18 @@ static ScoreParams to_params(const smx_score_params* p) {
   return r;
 }
 
+// rows requested per batch; two batches are in flight at a time
 constexpr int rows_in_flight(int nit, int mul) {
-  const int r = 8 / (nit * mul);
-  return r < 1 ? 1 : (r > 4 ? 4 : r);
+  const int r = 4 / (nit * mul);
+  return r < 1 ? 1 : r;
 }
 
 template <int M, int VEC, int NIT, bool REG>
 static int launch_forward_reg(hipStream_t st, const float* table, const int64_t* idx, const float* q1, const float* q2,
                           float* score, size_t B, size_t K, int ncol, size_t n_rows, const ScoreParams& p, int* err) {
   constexpr int RIF = rows_in_flight(NIT, model_mul(M));
-  int tile_k = 128;
-  while (tile_k > 4 * RIF && B * ((K + tile_k - 1) / tile_k) < 4096) tile_k /= 2;
+  int tile_k = 256;  // 64 negatives per wavefront; smaller tiles when the grid would not fill the chip
+  while (tile_k > 4 * RIF && (B * ((K + tile_k - 1) / tile_k) < 8192 || (size_t)tile_k / 2 >= K)) tile_k /= 2;
   const int tiles = (int)((K + tile_k - 1) / tile_k);
   const size_t lds = (size_t)model_nq(M) * ncol * VEC * sizeof(float);
   hipLaunchKernelGGL((score_forward_kernel<M, VEC, NIT, RIF, REG>), dim3((unsigned)(B * tiles)), dim3(256), lds, st, table,

@@ -238,3 +238,35 @@ def test_argument_errors():
     with pytest.raises(_lib.SmxError):
         fused.score_backward_entity("l1", plan, t, q, None, torch.zeros(2, 3, device="cuda"),
                                     torch.zeros(2, 3, device="cuda"), fused.score_params(1.0))  # nothing requested
+
+
+def test_box_tie_conventions_through_the_fused_path():
+    """The fused box kernels use a rearranged derivative; at ties it must still give the values of
+    the reference functors (dist_kernel.h:68-104): sign(0) = -1 outside, gradient passes at
+    |e-c| == o, e == c inside the box, negative offsets."""
+    from smore_amd import fused
+    cases = [  # e, c, o
+        (1.0, 0.75, 0.25), (1.0, 0.75, 0.5), (1.0, 1.0, 0.0), (0.5, 0.75, 0.5), (1.0, 0.75, -0.5),
+        (1.0, 1.0, 0.5), (0.25, 0.75, 0.25), (1.0, 1.0, -0.5), (0.75, 1.0, 0.0),
+    ]
+    n = len(cases)
+    table = np.array([[e] * 4 for e, _, _ in cases], dtype=np.float64)      # one entity row per case
+    q1 = np.array([[c] * 4 for _, c, _ in cases], dtype=np.float64)          # one query per case
+    q2 = np.array([[o] * 4 for _, _, o in cases], dtype=np.float64)
+    idx = np.arange(n, dtype=np.int64)[:, None]                              # pair (i, i)
+    gs = np.full((n, 1), 2.0)
+    params = fused.score_params(24.0, 0.5)
+    t_table, t_q1, t_q2, t_gs = dev(table), dev(q1), dev(q2), dev(gs)
+    t_idx = torch.tensor(idx, device="cuda")
+    score = fused.score_forward("box", t_table, t_idx, t_q1, t_q2, params)
+    rows = table[:, None, :]
+    want = orc.score_forward("box", rows, q1[:, None], q2[:, None], 24.0, 0.5)
+    assert np.array_equal(score.cpu().numpy().astype(np.float64), want)
+    g_rows, g_c, g_o = orc.score_backward("box", gs, rows, q1[:, None], q2[:, None], 0.5)
+    gq1, gq2 = fused.score_backward_query("box", t_table, t_idx, t_q1, t_q2, score, t_gs, params)
+    assert np.array_equal(gq1.cpu().numpy().astype(np.float64), g_c[:, 0])
+    assert np.array_equal(gq2.cpu().numpy().astype(np.float64), g_o[:, 0])
+    plan = fused.build_plan(t_idx, n)
+    merged = torch.empty((n, 4), device="cuda")
+    fused.score_backward_entity("box", plan, t_table, t_q1, t_q2, score, t_gs, params, merged=merged)
+    assert np.array_equal(merged.cpu().numpy().astype(np.float64), g_rows[:, 0])
