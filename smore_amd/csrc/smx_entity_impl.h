@@ -246,6 +246,16 @@ __device__ __forceinline__ void finish_row(const EntityArgs& A, int lane, unsign
   constexpr int MUL = src_mul(SRC);
   const int half = A.ncol * VEC;
   const size_t row_len = (size_t)half * MUL;
+  if constexpr (SRC != kSrcRows) {
+#pragma unroll
+    for (int it = 0; it < NIT; ++it)
+#pragma unroll
+      for (int x = 0; x < VEC; ++x) {
+        const float x1 = REG ? reg_apply(w.h[0][it].v[x], A.p) : w.h[0][it].v[x];
+        const float x2 = MUL == 2 ? (REG ? reg_apply(w.h[MUL - 1][it].v[x], A.p) : w.h[MUL - 1][it].v[x]) : 0.f;
+        finish_entity_grad<SRC>(x1, x2, g1[it][x], g2[it][x]);
+      }
+  }
   if (REG) {
 #pragma unroll
     for (int it = 0; it < NIT; ++it)
@@ -570,7 +580,8 @@ __global__ __launch_bounds__(NW * 64) void entity_fixup_kernel(EntityArgs A) {
     }
     const unsigned row_id = (unsigned)A.sorted_ids[p0];
     RowRegs<MUL, VEC, NIT> e, m0, v0;
-    if (REG || A.adam_on) load_row<MUL, VEC, NIT>(e, A.table + (size_t)row_id * row_len, half, A.ncol, lane);
+    if (REG || A.adam_on || SRC == mBetaKL)
+      load_row<MUL, VEC, NIT>(e, A.table + (size_t)row_id * row_len, half, A.ncol, lane);
     if (A.adam_on) {
       load_row<MUL, VEC, NIT>(m0, A.m + (size_t)row_id * row_len, half, A.ncol, lane);
       load_row<MUL, VEC, NIT>(v0, A.v + (size_t)row_id * row_len, half, A.ncol, lane);

@@ -177,21 +177,39 @@ template <> struct ModelOps<mRotate> {
   }
 };
 
-// Out-of-line copies of the special functions for the fused kernels: their bodies are long, and the
-// fused kernels evaluate them inside fully unrolled register loops.
-static __device__ __noinline__ float digamma_call(float x) { return digamma(x); }
-static __device__ __noinline__ float trigamma_call(float x) { return trigamma(x); }
-static __device__ __noinline__ float lgamma_call(float x) { return m_lgamma(x); }
+// BetaE: KL(Beta(ea,eb) || Beta(qa,qb)) of smore/common/torchext/dist_kernel.h:207-266, regrouped into an
+// entity part and a query part so that everything that depends on one side only is evaluated once:
+//   KL = [lgG(qa)+lgG(qb)-lgG(sq)] + [lgG(se)-lgG(ea)-lgG(eb)] + (ea-qa)psi(ea) + (eb-qb)psi(eb) + (sq-se)psi(se)
+//   dKL/dqa = [psi(qa) - psi(sq)] - psi(ea) + psi(se)                       (same with b)
+//   dKL/dea = (ea-qa) psi'(ea) + (sq-se) psi'(se)                            (same with b)
+// The bracketed query terms are per (query, feature) constants held in the lane's query registers.
+// For the entity gradient the trigammas depend on the entity only, and (ea-qa) + (eb-qb) = se - sq,
+// so a segment accumulates S1 = sum c (ea-qa), S2 = sum c (eb-qb) and applies
+//   g_a = psi'(ea) S1 - psi'(se) (S1+S2),  g_b = psi'(eb) S2 - psi'(se) (S1+S2)
+// once when the segment is finished.
+struct QBeta {
+  float a, b;  // alpha, beta of the query
+  float k;     // forward: lgG(qa)+lgG(qb)-lgG(sq); query backward: psi(qa)-psi(sq)
+  float l;     // query backward: psi(qb)-psi(sq)
+};
 
-// KL(Beta(e1,e2) || Beta(q.a,q.b)); same formulas as Term<kBetaKL, float>.
 template <> struct ModelOps<mBetaKL> {
-  using Q = QPair;  // a = alpha, b = beta of the query
-  static __device__ __forceinline__ Q prep(float q1, float q2) { return {q1, q2}; }
+  using Q = QBeta;
+  static __device__ __forceinline__ Q prep(float q1, float q2) { return {q1, q2, 0.f, 0.f}; }
+  static __device__ __forceinline__ Q prep_fwd(float q1, float q2) {
+    float lb, pa, pb, ps;
+    beta_terms(q1, q2, lb, pa, pb, ps);
+    return {q1, q2, -lb, 0.f};
+  }
+  static __device__ __forceinline__ Q prep_bwd_q(float q1, float q2) {
+    float pa, pb, ps;
+    digamma3(q1, q2, pa, pb, ps);
+    return {q1, q2, pa - ps, pb - ps};
+  }
   static __device__ __forceinline__ void fwd(float ea, float eb, const Q& q, float& a0, float&) {
-    const float se = ea + eb, sq = q.a + q.b;
-    const float t1 = lgamma_call(q.a) + lgamma_call(q.b) + lgamma_call(se);
-    const float t2 = lgamma_call(ea) + lgamma_call(eb) + lgamma_call(sq);
-    a0 += t1 - t2 + (ea - q.a) * digamma_call(ea) + (eb - q.b) * digamma_call(eb) + (sq - se) * digamma_call(se);
+    float lb, pa, pb, ps;
+    beta_terms(ea, eb, lb, pa, pb, ps);
+    a0 += (q.k + lb) + (ea - q.a) * pa + (eb - q.b) * pb + ((q.a + q.b) - (ea + eb)) * ps;
   }
   static __device__ __forceinline__ float fold(float a0, float, const ScoreParams&) { return a0; }
   static __device__ __forceinline__ float score(float folded, const ScoreParams& p) { return p.gamma - folded; }
@@ -199,19 +217,44 @@ template <> struct ModelOps<mBetaKL> {
     c0 = -g;
     c1 = 0.f;
   }
-  static __device__ __forceinline__ void bwd_e(float c0, float, float e1, float e2, const Q& q, float& ge1, float& ge2) {
-    const float se = e1 + e2, sq = q.a + q.b;
-    const float common = (sq - se) * trigamma_call(se);
-    ge1 += c0 * ((e1 - q.a) * trigamma_call(e1) + common);
-    ge2 += c0 * ((e2 - q.b) * trigamma_call(e2) + common);
+  // accumulates S1, S2 (see above); finish_e turns them into the gradient
+  static __device__ __forceinline__ void bwd_e(float c0, float, float e1, float e2, const Q& q, float& s1, float& s2) {
+    s1 += c0 * (e1 - q.a);
+    s2 += c0 * (e2 - q.b);
+  }
+  static __device__ __forceinline__ void finish_e(float e1, float e2, float& g1, float& g2) {
+    float ta, tb, ts;
+    trigamma3(e1, e2, ta, tb, ts);
+    const float common = ts * (g1 + g2);
+    g1 = ta * g1 - common;
+    g2 = tb * g2 - common;
   }
   static __device__ __forceinline__ void bwd_q(float c0, float, float e1, float e2, const Q& q, float& g1, float& g2) {
-    const float se = e1 + e2, sq = q.a + q.b;
-    const float common = digamma_call(se) - digamma_call(sq);
-    g1 += c0 * (digamma_call(q.a) - digamma_call(e1) + common);
-    g2 += c0 * (digamma_call(q.b) - digamma_call(e2) + common);
+    float pa, pb, ps;
+    digamma3(e1, e2, pa, pb, ps);
+    g1 += c0 * (q.k - pa + ps);
+    g2 += c0 * (q.l - pb + ps);
   }
 };
+
+// Query registers for the forward / the query-backward kernel (models without side constants use prep).
+template <int M>
+__device__ __forceinline__ typename ModelOps<M>::Q prep_forward(float q1, float q2) {
+  if constexpr (M == mBetaKL) return ModelOps<M>::prep_fwd(q1, q2);
+  else return ModelOps<M>::prep(q1, q2);
+}
+template <int M>
+__device__ __forceinline__ typename ModelOps<M>::Q prep_backward_query(float q1, float q2) {
+  if constexpr (M == mBetaKL) return ModelOps<M>::prep_bwd_q(q1, q2);
+  else return ModelOps<M>::prep(q1, q2);
+}
+
+// Hook applied once per finished entity row to the summed accumulators (identity unless a model
+// defers part of its derivative, as BETA_KL does).  e1 / e2 are the (regularised) entity values.
+template <int M>
+__device__ __forceinline__ void finish_entity_grad(float e1, float e2, float& g1, float& g2) {
+  if constexpr (M == mBetaKL) ModelOps<mBetaKL>::finish_e(e1, e2, g1, g2);
+}
 
 template <int M>
 __device__ __forceinline__ void finish_query_grad(const typename ModelOps<M>::Q& q, float& g1, float& g2,

@@ -42,7 +42,7 @@ __device__ __forceinline__ Pack<VEC> load_pack(const float* __restrict__ base, i
 }
 
 // Loads the features a lane owns of the staged query into registers.
-template <int M, int VEC, int NIT>
+template <int M, int VEC, int NIT, bool FWD>
 __device__ __forceinline__ void load_query_regs(const float* lds, int dim, int ncol, int lane,
                                                 typename ModelOps<M>::Q (&q)[NIT][VEC]) {
 #pragma unroll
@@ -50,9 +50,10 @@ __device__ __forceinline__ void load_query_regs(const float* lds, int dim, int n
     const int c = lane + 64 * it;
 #pragma unroll
     for (int v = 0; v < VEC; ++v) {
-      const float a = c < ncol ? lds[c * VEC + v] : 0.f;
-      const float b = (model_nq(M) == 2 && c < ncol) ? lds[dim + c * VEC + v] : 0.f;
-      q[it][v] = ModelOps<M>::prep(a, b);
+      const int cc = min(c, ncol - 1);  // lanes past the row end hold a copy of the last column
+      const float a = lds[cc * VEC + v];
+      const float b = model_nq(M) == 2 ? lds[dim + cc * VEC + v] : 0.f;
+      q[it][v] = FWD ? prep_forward<M>(a, b) : prep_backward_query<M>(a, b);
     }
   }
 }
@@ -163,7 +164,7 @@ __global__ __launch_bounds__(256) void score_forward_kernel(const float* __restr
 
   stage_query<M>(lds, q1, q2, b, dim);
   typename ModelOps<M>::Q q[NIT][VEC];
-  load_query_regs<M, VEC, NIT>(lds, dim, ncol, lane, q);
+  load_query_regs<M, VEC, NIT, true>(lds, dim, ncol, lane, q);
   if (cnt <= 0) return;
 
   float* out = score + (size_t)b * K + kw0;
@@ -204,7 +205,7 @@ __global__ __launch_bounds__(NW * 64) void score_backward_query_kernel(
 
   stage_query<M>(lds, q1, q2, b, dim);
   typename ModelOps<M>::Q q[NIT][VEC];
-  load_query_regs<M, VEC, NIT>(lds, dim, ncol, lane, q);
+  load_query_regs<M, VEC, NIT, false>(lds, dim, ncol, lane, q);
 
   float g1[NIT][VEC], g2[NIT][VEC];
 #pragma unroll
