@@ -21,6 +21,13 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E bandwidth
 
+# Entity-pass traffic per launch in bytes (L2<->fabric, reads + writes), measured with two
+# `rocprofv3 --pmc` runs (FETCH_SIZE, WRITE_SIZE) and scaled by what the same counters read for a plain
+# row copy of known size (`bench.py --calibrate-copy`: FETCH_SIZE x1.942, WRITE_SIZE x1.000).  A counter
+# cannot be read from inside this process, so the figures are those of the profile summary
+# pmc_traffic_<workload>.md kept with the other rocprofv3 summaries; workloads not profiled report null.
+MEASURED_ENTITY_TRAFFIC = {"cfg5-box-adam-86m-zipf1.1": 6.90e9}
+
 CONFIGS = {
     1: dict(name="cfg1-l2-15k", model="l2", n=15_000, dim=200, b=512, k=128, r=0.07, gamma=12.0, cen=0.0,
             zipf=None, adam=False),
@@ -156,7 +163,7 @@ def cpu_baseline(cfg, seed):
     cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
     rng = np.random.default_rng(seed)
     n = min(cfg["n"], 2_000_000)
-    b = min(cfg["b"], 256)
+    b = min(cfg["b"], 1024)
     k, dim, rl = cfg["k"], cfg["dim"], row_len(cfg)
     f32 = np.float32
     if cfg["model"] == "beta_kl":
@@ -184,7 +191,7 @@ def cpu_baseline(cfg, seed):
     m = np.zeros_like(table) if cfg["adam"] else None
     v = np.zeros_like(table) if cfg["adam"] else None
     times = []
-    for step in range(1, 4):
+    for step in range(1, 6):
         t0 = time.perf_counter()
         orc.train_step(cfg["model"], table, m, v, idx, q1, q2, gs, cfg["gamma"], cfg["cen"], cfg.get("lr", 0.0), step,
                        dtype=f32, apply_adam=cfg["adam"])
@@ -205,6 +212,9 @@ def main():
     ap.add_argument("--config", type=int, default=5, choices=sorted(CONFIGS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--seed", type=int, default=None)
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="run only a plain row copy of known size (1 GiB read + 1 GiB written per launch) through "
+                         "smx_gather_rows; under rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE this gives the counters' scale")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
@@ -215,6 +225,18 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a GPU")
     device = torch.device("cuda:0")
+    if args.calibrate_copy:
+        from smore_amd import fused
+        rows, row_len_ = (1 << 30) // 800, 200  # 800-byte rows as in the headline workload
+        src = torch.rand((rows, row_len_), device=device)
+        ident = torch.arange(rows, device=device)
+        for _ in range(5):
+            out = fused.gather_rows(src, ident)
+        torch.cuda.synchronize()
+        assert torch.equal(out, src)
+        print(json.dumps({"calibration": "smx_gather_rows identity copy", "bytes_read": rows * 800 + rows * 8,
+                          "bytes_written": rows * 800, "launches": 5}))
+        return
     cfg = CONFIGS[args.config]
     seed = args.seed if args.seed is not None else 20240 + args.config
 
@@ -255,10 +277,11 @@ def main():
                    "K": cfg["k"], "ids": "zipf(1.1)" if cfg["zipf"] else "uniform", "optimizer": "sparse adam" if
                    cfg["adam"] else None, "seed": seed, "distinct_ids": n_uniq},
         "roofline": {
-            "bound": "hbm", "kernel": "entity_tile_kernel (+fixup): segmented entity gradient" +
-                     (" + fused sparse Adam" if cfg["adam"] else ""),
+            "bound": "hbm",
+            "kernel": "entity pass (one C-ABI call = entity_segment_kernel + entity_tile_kernel + entity_fixup_kernel): "
+                      "segmented entity gradient" + (" + fused sparse Adam" if cfg["adam"] else ""),
             "achieved": ent_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": ent_gbps / HBM_PEAK_GBPS,
-            "traffic": None, "algorithmic_bytes": ent_bytes, "avg_ms": phase_ms["backward_entity"],
+            "traffic": MEASURED_ENTITY_TRAFFIC.get(cfg["name"]), "algorithmic_bytes": ent_bytes, "avg_ms": phase_ms["backward_entity"],
         },
         "step_hbm": {
             "algorithmic_bytes": algo, "achieved_GBps": algo / (ms_per_step * 1e-3) / 1e9,

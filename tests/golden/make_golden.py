@@ -1,0 +1,58 @@
+"""Writes the golden fixtures in this directory from the CPU oracle (float64).
+
+The reference holds no vectors for this path (its tests print numbers), and its implementation is
+CUDA-only, so the fixtures are produced by the oracle after it has been pinned against library
+routines and closed forms (tests/test_oracle_pinning.py).  They freeze one tiny training step per
+score model -- inputs, scores, query gradients, the integer segment plan, merged entity gradients
+and the table / Adam moments after two steps -- so that a later change of the oracle or of the HIP
+path that alters any result is caught against data, not against the same formula.
+
+    python tests/golden/make_golden.py        # rewrites tests/golden/step_*.npz
+"""
+import os
+import sys
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.dirname(os.path.dirname(HERE)))
+from oracle import oracle as orc  # noqa: E402
+
+GAMMA = {"l1": 12.0, "l2": 12.0, "box": 24.0, "rotate": 9.0, "beta_kl": 60.0}
+
+
+def make(model, seed):
+    rng = np.random.default_rng(seed)
+    n, b, k, dim, lr, cen = 48, 4, 6, 8, 1e-3, 0.02
+    mul = 2 if model in ("rotate", "beta_kl") else 1
+    f32 = lambda x: x.astype(np.float32).astype(np.float64)
+    if model == "beta_kl":
+        beta = lambda *s: np.clip(1 + rng.standard_normal(s), 0.05, 1e9)
+        table, q1, q2 = beta(n, dim * mul), beta(b, dim), beta(b, dim)
+    else:
+        table = rng.uniform(-0.07, 0.07, (n, dim * mul))
+        q1 = rng.uniform(-0.07, 0.07, (b, dim))
+        q2 = None if model in ("l1", "l2") else np.abs(rng.uniform(-0.07, 0.07, (b, dim)))
+    table, q1 = f32(table), f32(q1)
+    q2 = None if q2 is None else f32(q2)
+    idx = rng.integers(0, n // 3, (b, k)).astype(np.int64)  # repeats on purpose
+    gs = f32(rng.standard_normal((b, k)))
+    w, m, v = table.copy(), np.zeros_like(table), np.zeros_like(table)
+    o1 = q1[:, None]
+    o2 = None if q2 is None else q2[:, None]
+    first = orc.train_step(model, w, m, v, idx, o1, o2, gs, GAMMA[model], cen, lr, 1)
+    orc.train_step(model, w, m, v, idx, o1, o2, gs, GAMMA[model], cen, lr, 2)
+    out = dict(table=table, q1=q1, idx=idx, gs=gs, gamma=GAMMA[model], cen=cen, lr=lr,
+               score=first["score"], gq1=first["gq1"][:, 0], uniq=first["uniq"], inverse=first["inverse"],
+               order=first["order"], seg_start=first["seg_start"], merged=first["merged"],
+               w_after=w, m_after=m, v_after=v)
+    if q2 is not None:
+        out["q2"] = q2
+        out["gq2"] = first["gq2"][:, 0]
+    np.savez_compressed(os.path.join(HERE, f"step_{model}.npz"), **out)
+
+
+if __name__ == "__main__":
+    for i, model in enumerate(GAMMA):
+        make(model, 100 + i)
+    print("wrote", sorted(f for f in os.listdir(HERE) if f.endswith(".npz")))
