@@ -21,12 +21,12 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E bandwidth
 
-# Entity-pass traffic per launch in bytes (L2<->fabric, reads + writes), measured with two
+# Traffic of the backward call per launch in bytes (L2<->fabric, reads + writes), measured with two
 # `rocprofv3 --pmc` runs (FETCH_SIZE, WRITE_SIZE) and scaled by what the same counters read for a plain
 # row copy of known size (`bench.py --calibrate-copy`: FETCH_SIZE x1.942, WRITE_SIZE x1.000).  A counter
 # cannot be read from inside this process, so the figures are those of the profile summary
 # pmc_traffic_<workload>.md kept with the other rocprofv3 summaries; workloads not profiled report null.
-MEASURED_ENTITY_TRAFFIC = {"cfg5-box-adam-86m-zipf1.1": 6.90e9}
+MEASURED_BACKWARD_TRAFFIC = {}
 
 CONFIGS = {
     1: dict(name="cfg1-l2-15k", model="l2", n=15_000, dim=200, b=512, k=128, r=0.07, gamma=12.0, cen=0.0,
@@ -105,17 +105,19 @@ def algorithmic_bytes(cfg, n_uniq, streaming=False):
     return total
 
 
-def entity_kernel_bytes(cfg, n_uniq):
-    """Algorithmic bytes of the entity pass alone: one read of every distinct row, the upstream gradient of
-    every pair, and (with the optimizer) read + write of w, m, v of every distinct row."""
+def backward_bytes(cfg, n_uniq):
+    """Algorithmic bytes of the backward call (query gradients + entity pass): the backward share of the step
+    model above -- every distinct row once, Adam's read + write of w, m, v (or, without optimizer, the merged
+    gradient rows written), the upstream gradient of every pair, queries read and their gradients written."""
     p = cfg["b"] * cfg["k"]
     de = row_len(cfg)
-    return 4 * de * n_uniq + (6 * 4 * de * n_uniq if cfg["adam"] else 4 * de * n_uniq) + 4 * p
+    rows = 4 * de * n_uniq + (6 * 4 * de * n_uniq if cfg["adam"] else 4 * de * n_uniq)
+    return rows + 4 * p + 2 * 4 * cfg["b"] * cfg["dim"] * n_query_tensors(cfg)
 
 
 class Step:
     """One pass of the hot path; phases are bracketed by events on the stream the kernels run on."""
-    PHASES = ("plan", "forward", "backward_query", "backward_entity")
+    PHASES = ("plan", "forward", "backward")
 
     def __init__(self, cfg, table, q1, q2, idx, gscore):
         import torch
@@ -139,18 +141,15 @@ class Step:
         mark(1)
         score = f.score_forward(cfg["model"], self.table, self.idx, self.q1, self.q2, self.params, self.err)
         mark(2)
-        gq = f.score_backward_query(cfg["model"], self.table, self.idx, self.q1, self.q2, score, self.gscore,
-                                    self.params)
-        mark(3)
         if cfg["adam"]:
-            f.score_backward_entity(cfg["model"], plan, self.table, self.q1, self.q2, score, self.gscore, self.params,
-                                    m=self.m, v=self.v, adam=f.adam_params(cfg["lr"], self.step_no))
+            gq = f.score_backward_fused(cfg["model"], plan, self.table, self.idx, self.q1, self.q2, score, self.gscore,
+                                        self.params, m=self.m, v=self.v, adam=f.adam_params(cfg["lr"], self.step_no))
         else:
             if self.merged is None:
                 self.merged = self.torch.empty((plan.n_uniq, self.table.shape[1]), device=self.table.device)
-            f.score_backward_entity(cfg["model"], plan, self.table, self.q1, self.q2, score, self.gscore, self.params,
-                                    merged=self.merged)
-        mark(4)
+            gq = f.score_backward_fused(cfg["model"], plan, self.table, self.idx, self.q1, self.q2, score, self.gscore,
+                                        self.params, merged=self.merged)
+        mark(3)
         self.plan = plan
         return score, gq
 
@@ -249,7 +248,7 @@ def main():
     if step.err.item() != 0:
         sys.exit("entity id out of range in the synthetic batch")
 
-    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(5)] for _ in range(args.steps)]
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(args.steps)]
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for s in range(args.steps):
@@ -262,8 +261,8 @@ def main():
     pairs = cfg["b"] * cfg["k"]
     algo = algorithmic_bytes(cfg, n_uniq)
     algo_stream = algorithmic_bytes(cfg, n_uniq, streaming=True)
-    ent_bytes = entity_kernel_bytes(cfg, n_uniq)
-    ent_gbps = ent_bytes / (phase_ms["backward_entity"] * 1e-3) / 1e9
+    ent_bytes = backward_bytes(cfg, n_uniq)
+    ent_gbps = ent_bytes / (phase_ms["backward"] * 1e-3) / 1e9
 
     out = {
         "metric": "scored (query,neg) pairs/sec fwd+bwd+opt; achieved HBM GB/s vs peak",
@@ -278,10 +277,11 @@ def main():
                    cfg["adam"] else None, "seed": seed, "distinct_ids": n_uniq},
         "roofline": {
             "bound": "hbm",
-            "kernel": "entity pass (one C-ABI call = entity_segment_kernel + entity_tile_kernel + entity_fixup_kernel): "
-                      "segmented entity gradient" + (" + fused sparse Adam" if cfg["adam"] else ""),
+            "kernel": "backward (one C-ABI call, smx_score_backward_fused = score_backward_query_kernel + "
+                      "entity_segment_kernel + entity_tile_kernel + entity_fixup_kernel): query gradients, segmented "
+                      "entity gradient" + (" + fused sparse Adam" if cfg["adam"] else " (merged rows)"),
             "achieved": ent_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": ent_gbps / HBM_PEAK_GBPS,
-            "traffic": MEASURED_ENTITY_TRAFFIC.get(cfg["name"]), "algorithmic_bytes": ent_bytes, "avg_ms": phase_ms["backward_entity"],
+            "traffic": MEASURED_BACKWARD_TRAFFIC.get(cfg["name"]), "algorithmic_bytes": ent_bytes, "avg_ms": phase_ms["backward"],
         },
         "step_hbm": {
             "algorithmic_bytes": algo, "achieved_GBps": algo / (ms_per_step * 1e-3) / 1e9,

@@ -128,14 +128,16 @@ int smx_score_backward_query(int model, void* stream, const float* table, size_t
  *   uniq[P]        first n_uniq entries: the distinct ids, ascending (= torch.unique)
  *   seg_start[P+1] first n_uniq+1 entries: start of each segment in order[]
  *   inverse[P]     position of idx[p] in uniq (= return_inverse), may be NULL
+ *   pair_seg[P]    per pair: sign bit + segment number when the pair is alone in its segment (its
+ *                  id occurs once in the step), 0 otherwise; may be NULL
  *   n_uniq         device int: number of distinct ids
  * All arrays are caller-allocated device memory.  workspace: at least
  * smx_plan_workspace_bytes(P, n_rows) bytes, 256-byte aligned.  Needs n_rows <= 2^32. */
 size_t smx_plan_workspace_bytes(size_t n_pairs, size_t n_rows);
 int smx_plan_build(void* stream, const int64_t* idx, size_t n_pairs, size_t n_rows, void* workspace,
                    size_t workspace_bytes, int32_t* order, int32_t* sorted_ids, int32_t* seg_of_pos,
-                   int64_t* uniq, int32_t* seg_start, int64_t* inverse, int32_t* n_uniq,
-                   int* err_flag);
+                   int64_t* uniq, int32_t* seg_start, int64_t* inverse, int32_t* pair_seg,
+                   int32_t* n_uniq, int* err_flag);
 
 typedef struct smx_plan_view {
   const int32_t* order;
@@ -143,7 +145,8 @@ typedef struct smx_plan_view {
   const int32_t* seg_of_pos;
   const int32_t* seg_start;
   const int64_t* uniq;
-  const int32_t* n_uniq; /* device scalar */
+  const int32_t* n_uniq;   /* device scalar */
+  const int32_t* pair_seg; /* may be NULL where the one-pair fast path is not used */
   size_t n_pairs;
 } smx_plan_view;
 
@@ -176,6 +179,23 @@ int smx_score_backward_entity(int model, void* stream, const smx_plan_view* plan
                               const float* gscore, size_t B, size_t K, size_t dim,
                               const smx_score_params* params, float* merged, float* m, float* v,
                               const smx_adam_params* adam, void* workspace, size_t workspace_bytes);
+
+/* Everything after the loss in one call: query gradients, and every entity row of the step finished
+ * (merged gradient row and/or lazy Adam on w, m, v), as smx_score_backward_query followed by
+ * smx_score_backward_entity would do -- except that rows of ids occurring once in the step are
+ * finished by the query-gradient kernel itself, which already holds the query in registers and has
+ * just read the entity row; the entity pass then skips them.  The plan must have been built with
+ * pair_seg.  Same results as the two separate calls up to fp32 rounding (the one-pair rows are computed
+ * by a different kernel, so a multiply-add may be contracted differently).
+ * workspace as for smx_score_backward_entity.  No counterpart as one function in the reference:
+ * it stands for dist_backward (extlib_cuda.cpp:230-262) + EmbedLookupFunc.backward +
+ * EmbeddingOptimizer.apply_grad (embed_optimizer.py:63-66,155-163). */
+int smx_score_backward_fused(int model, void* stream, const smx_plan_view* plan, float* table,
+                             size_t n_rows, const int64_t* idx, const float* q1, const float* q2,
+                             const float* score, const float* gscore, float* gq1, float* gq2,
+                             size_t B, size_t K, size_t dim, const smx_score_params* params,
+                             float* merged, float* m, float* v, const smx_adam_params* adam,
+                             void* workspace, size_t workspace_bytes);
 
 /* Same pass for gradient rows that already exist in memory (what autograd hands
  * EmbedLookupFunc.backward): grad_rows [P, row_len] in pair order.  Replaces

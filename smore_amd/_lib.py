@@ -34,12 +34,17 @@ SIGNATURES = {
     # model, stream, table, n_rows, idx, q1, q2, score, gscore, gq1, gq2, B, K, dim, params
     "smx_score_backward_query": (_i, [_i, _vp, _vp, _sz, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _vp]),
     "smx_plan_workspace_bytes": (_sz, [_sz, _sz]),
-    # stream, idx, n_pairs, n_rows, ws, ws_bytes, order, sorted_ids, seg_of_pos, uniq, seg_start, inverse, n_uniq, err
-    "smx_plan_build": (_i, [_vp, _vp, _sz, _sz, _vp, _sz, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
+    # stream, idx, n_pairs, n_rows, ws, ws_bytes, order, sorted_ids, seg_of_pos, uniq, seg_start, inverse, pair_seg,
+    # n_uniq, err
+    "smx_plan_build": (_i, [_vp, _vp, _sz, _sz, _vp, _sz, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "smx_entity_workspace_bytes": (_sz, [_sz, _sz]),
     # model, stream, plan, table, n_rows, q1, q2, score, gscore, B, K, dim, params, merged, m, v, adam, ws, ws_bytes
     "smx_score_backward_entity": (_i, [_i, _vp, _vp, _vp, _sz, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _vp, _vp, _vp, _vp,
                                        _vp, _vp, _sz]),
+    # model, stream, plan, table, n_rows, idx, q1, q2, score, gscore, gq1, gq2, B, K, dim, params, merged, m, v,
+    # adam, ws, ws_bytes
+    "smx_score_backward_fused": (_i, [_i, _vp, _vp, _vp, _sz, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _vp,
+                                      _vp, _vp, _vp, _vp, _vp, _sz]),
     # stream, plan, grad_rows, row_len, merged, table, m, v, adam, ws, ws_bytes
     # stream, table, n_rows, row_len, idx, n, out, err
     "smx_gather_rows": (_i, [_vp, _vp, _sz, _sz, _vp, _sz, _vp, _vp]),
@@ -60,7 +65,7 @@ class AdamParams(ctypes.Structure):
 class PlanView(ctypes.Structure):
     """smx_plan_view of include/smore_amd.h."""
     _fields_ = [("order", _vp), ("sorted_ids", _vp), ("seg_of_pos", _vp), ("seg_start", _vp), ("uniq", _vp),
-                ("n_uniq", _vp), ("n_pairs", _sz)]
+                ("n_uniq", _vp), ("pair_seg", _vp), ("n_pairs", _sz)]
 
 _lib = None
 

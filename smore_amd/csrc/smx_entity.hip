@@ -57,20 +57,6 @@ static EntityScratch entity_scratch(size_t n_pairs, size_t row_len) {
 
 static size_t entity_ws_bytes(size_t n_pairs, size_t row_len) { return entity_scratch(n_pairs, row_len).total; }
 
-static AdamConsts adam_consts(const smx_adam_params* a) {
-  AdamConsts c;
-  const double bc1 = 1.0 - std::pow(a->beta1, (double)a->step);
-  const double bc2 = 1.0 - std::pow(a->beta2, (double)a->step);
-  c.beta1 = (float)a->beta1;
-  c.beta2 = (float)a->beta2;
-  c.omb1 = (float)(1.0 - a->beta1);
-  c.omb2 = (float)(1.0 - a->beta2);
-  c.eps = (float)a->eps;
-  c.step_size = (float)(-a->lr / bc1);
-  c.inv_sqrt_bc2 = (float)(1.0 / std::sqrt(bc2));
-  return c;
-}
-
 static int fill_plan(EntityArgs* A, const smx_plan_view* plan, void* workspace, size_t workspace_bytes, size_t row_len) {
   if (!plan || !plan->order || !plan->sorted_ids || !plan->seg_of_pos || !plan->seg_start || !plan->uniq ||
       !plan->n_uniq)
@@ -95,6 +81,11 @@ static int fill_plan(EntityArgs* A, const smx_plan_view* plan, void* workspace, 
   return SMX_OK;
 }
 
+int entity_backward(int model, void* stream, const smx_plan_view* plan, float* table, size_t n_rows, const float* q1,
+                    const float* q2, const float* score, const float* gscore, size_t B, size_t K, size_t dim,
+                    const smx_score_params* params, float* merged, float* m, float* v, const smx_adam_params* adam,
+                    void* workspace, size_t workspace_bytes, int skip_single);
+
 static int fill_adam(EntityArgs* A, float* m, float* v, const smx_adam_params* adam) {
   A->adam_on = 0;
   A->m = m;
@@ -103,7 +94,7 @@ static int fill_adam(EntityArgs* A, float* m, float* v, const smx_adam_params* a
     if (!m || !v || !adam) return fail(SMX_ERR_ARG, "Adam needs m, v and parameters together");
     if (adam->step < 1) return fail(SMX_ERR_ARG, "Adam step counter starts at 1");
     A->adam_on = 1;
-    A->a = adam_consts(adam);
+    A->a = make_adam_consts(adam);
   }
   return SMX_OK;
 }
@@ -118,7 +109,18 @@ int smx_score_backward_entity(int model, void* stream, const smx_plan_view* plan
                               const float* q1, const float* q2, const float* score, const float* gscore, size_t B,
                               size_t K, size_t dim, const smx_score_params* params, float* merged, float* m, float* v,
                               const smx_adam_params* adam, void* workspace, size_t workspace_bytes) {
-  using namespace smx;
+  return smx::entity_backward(model, stream, plan, table, n_rows, q1, q2, score, gscore, B, K, dim, params, merged, m,
+                              v, adam, workspace, workspace_bytes, 0);
+}
+
+}  // extern "C"
+
+namespace smx {
+
+int entity_backward(int model, void* stream, const smx_plan_view* plan, float* table, size_t n_rows, const float* q1,
+                    const float* q2, const float* score, const float* gscore, size_t B, size_t K, size_t dim,
+                    const smx_score_params* params, float* merged, float* m, float* v, const smx_adam_params* adam,
+                    void* workspace, size_t workspace_bytes, int skip_single) {
   if (model < 0 || model >= mNumModels) return fail(SMX_ERR_KIND, "unknown score model %d", model);
   if (!table || !q1 || !score || !gscore || !params || (model_nq(model) == 2 && !q2))
     return fail(SMX_ERR_ARG, "null pointer");
@@ -148,6 +150,7 @@ int smx_score_backward_entity(int model, void* stream, const smx_plan_view* plan
   A.table = table;
   A.merged = merged;
   A.ncol = (int)ncol;
+  A.skip_single = skip_single;
   hipStream_t st = as_stream(stream);
   switch (model) {
     case mL1: return entity_dispatch<mL1>(st, A, vec, nit);
@@ -158,6 +161,10 @@ int smx_score_backward_entity(int model, void* stream, const smx_plan_view* plan
   }
   return fail(SMX_ERR_KIND, "unknown score model %d", model);
 }
+
+}  // namespace smx
+
+extern "C" {
 
 int smx_rows_backward(void* stream, const smx_plan_view* plan, const float* grad_rows, size_t row_len, float* merged,
                       float* table, float* m, float* v, const smx_adam_params* adam, void* workspace,

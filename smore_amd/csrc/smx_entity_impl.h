@@ -27,19 +27,12 @@
 #pragma once
 #include "smx_common.h"
 #include "smx_models.h"
+#include "smx_rowupdate.h"
 #include "smx_wave.h"
 
 namespace smx {
 
-constexpr int kSrcRows = 100;  // source = materialised gradient rows instead of a score model
-
-__host__ __device__ constexpr int src_mul(int s) { return s == kSrcRows ? 1 : model_mul(s); }
-
-struct AdamConsts {
-  float beta1, beta2, omb1, omb2, eps, step_size, inv_sqrt_bc2;
-};
-
-struct EntityArgs {
+struct EntityArgs : RowSink {
   // plan
   const int* order;
   const int* sorted_ids;
@@ -56,64 +49,13 @@ struct EntityArgs {
   const float* score;
   const float* gscore;
   int K;
-  ScoreParams p;
   // source: gradient rows
   const float* grad_rows;
-  // entity table (read for the model sources, updated when adam_on)
-  float* table;
-  float* m;
-  float* v;
-  int adam_on;
-  AdamConsts a;
-  float* merged;  // [U, row_len] or null
-  float* tail;    // [tiles, row_len]
+  float* tail;    // [tiles, row_len] partial rows of long segments
   float* head;    // [tiles, row_len]
-  int ncol;       // columns per half row (model sources) or per row (gradient rows)
+  int skip_single;  // segments of one pair were already finished by the query-backward kernel
 };
 
-template <int VEC> struct Pack2 {
-  float v[VEC];
-};
-
-template <int VEC>
-__device__ __forceinline__ Pack2<VEC> ld(const float* __restrict__ base, int col) {
-  Pack2<VEC> r;
-  if constexpr (VEC == 4) {
-    const float4 t = reinterpret_cast<const float4*>(base)[col];
-    r.v[0] = t.x;
-    r.v[1] = t.y;
-    r.v[2] = t.z;
-    r.v[3] = t.w;
-  } else {
-    r.v[0] = base[col];
-  }
-  return r;
-}
-
-template <int VEC>
-__device__ __forceinline__ void st(float* __restrict__ base, int col, const float (&x)[VEC]) {
-  if constexpr (VEC == 4) {
-    reinterpret_cast<float4*>(base)[col] = make_float4(x[0], x[1], x[2], x[3]);
-  } else {
-    base[col] = x[0];
-  }
-}
-
-// The lane's columns of one table row (both halves for the two-half models).
-template <int MUL, int VEC, int NIT> struct RowRegs {
-  Pack2<VEC> h[MUL][NIT];
-};
-
-template <int MUL, int VEC, int NIT>
-__device__ __forceinline__ void load_row(RowRegs<MUL, VEC, NIT>& r, const float* __restrict__ base, int half, int ncol,
-                                         int lane) {
-#pragma unroll
-  for (int h = 0; h < MUL; ++h)
-#pragma unroll
-    for (int it = 0; it < NIT; ++it) r.h[h][it] = ld<VEC>(base + h * half, min(lane + 64 * it, ncol - 1));
-}
-
-// Coefficient on the second accumulator (BOX: inside distance) from the first.
 template <int SRC>
 __device__ __forceinline__ float second_coef(float c0, const ScoreParams& p) {
   return SRC == mBox ? p.cen * c0 : 0.f;
@@ -234,76 +176,6 @@ __device__ __forceinline__ void load_window(const EntityArgs& A, int lane, int b
   }
 }
 
-// Finishes one entity row: clamp mask, merged-gradient store, Adam.  g1/g2 are the lane's columns of
-// the summed gradient of the first / second half row; w, m0, v0 the row's current weights and moments
-// (w is always valid for the model sources -- it is the entity row the gradient was computed from).
-template <int SRC, int VEC, int NIT, bool REG>
-__device__ __forceinline__ void finish_row(const EntityArgs& A, int lane, unsigned row_id, int seg,
-                                           float (&g1)[NIT][VEC], float (&g2)[NIT][VEC],
-                                           const RowRegs<src_mul(SRC), VEC, NIT>& w,
-                                           const RowRegs<src_mul(SRC), VEC, NIT>& m0,
-                                           const RowRegs<src_mul(SRC), VEC, NIT>& v0) {
-  constexpr int MUL = src_mul(SRC);
-  const int half = A.ncol * VEC;
-  const size_t row_len = (size_t)half * MUL;
-  if constexpr (SRC != kSrcRows) {
-#pragma unroll
-    for (int it = 0; it < NIT; ++it)
-#pragma unroll
-      for (int x = 0; x < VEC; ++x) {
-        const float x1 = REG ? reg_apply(w.h[0][it].v[x], A.p) : w.h[0][it].v[x];
-        const float x2 = MUL == 2 ? (REG ? reg_apply(w.h[MUL - 1][it].v[x], A.p) : w.h[MUL - 1][it].v[x]) : 0.f;
-        finish_entity_grad<SRC>(x1, x2, g1[it][x], g2[it][x]);
-      }
-  }
-  if (REG) {
-#pragma unroll
-    for (int it = 0; it < NIT; ++it)
-#pragma unroll
-      for (int x = 0; x < VEC; ++x) {
-        g1[it][x] = reg_mask(w.h[0][it].v[x], g1[it][x], A.p);
-        if (MUL == 2) g2[it][x] = reg_mask(w.h[MUL - 1][it].v[x], g2[it][x], A.p);
-      }
-  }
-  if (A.merged) {
-    float* out = A.merged + (size_t)seg * row_len;
-#pragma unroll
-    for (int it = 0; it < NIT; ++it) {
-      const int c = lane + 64 * it;
-      if (c < A.ncol) {
-        st<VEC>(out, c, g1[it]);
-        if (MUL == 2) st<VEC>(out + half, c, g2[it]);
-      }
-    }
-  }
-  if (A.adam_on) {
-    float* pw = A.table + (size_t)row_id * row_len;
-    float* pm = A.m + (size_t)row_id * row_len;
-    float* pv = A.v + (size_t)row_id * row_len;
-#pragma unroll
-    for (int h = 0; h < MUL; ++h) {
-#pragma unroll
-      for (int it = 0; it < NIT; ++it) {
-        const int c = lane + 64 * it;
-        if (c < A.ncol) {
-          float wn[VEC], mn[VEC], vn[VEC];
-#pragma unroll
-          for (int x = 0; x < VEC; ++x) {
-            const float g = h == 0 ? g1[it][x] : g2[it][x];
-            mn[x] = m0.h[h][it].v[x] * A.a.beta1 + g * A.a.omb1;
-            vn[x] = v0.h[h][it].v[x] * A.a.beta2 + g * g * A.a.omb2;
-            const float denom = sqrtf(vn[x]) * A.a.inv_sqrt_bc2 + A.a.eps;
-            wn[x] = w.h[h][it].v[x] + A.a.step_size * mn[x] / denom;
-          }
-          st<VEC>(pw + h * half, c, wn);
-          st<VEC>(pm + h * half, c, mn);
-          st<VEC>(pv + h * half, c, vn);
-        }
-      }
-    }
-  }
-}
-
 template <int SRC, int VEC, int NIT>
 __device__ __forceinline__ void store_partial(const EntityArgs& A, float* buf, int t, int lane,
                                               const float (&g1)[NIT][VEC], const float (&g2)[NIT][VEC]) {
@@ -331,23 +203,6 @@ __device__ __forceinline__ void zero_acc(float (&g1)[NIT][VEC], float (&g2)[NIT]
 constexpr int kRunsShort = 2;  // runs in flight per wavefront in the short-segment kernel
 constexpr int kRunsLong = 4;   // ... in the long-segment kernel
 
-template <int MUL, int VEC, int NIT> struct RowState {
-  RowRegs<MUL, VEC, NIT> e, m, v;
-};
-
-template <int SRC, int VEC, int NIT>
-__device__ __forceinline__ void request_state(const EntityArgs& A, int lane, unsigned row_id,
-                                              RowState<src_mul(SRC), VEC, NIT>& s) {
-  constexpr int MUL = src_mul(SRC);
-  const int half = A.ncol * VEC;
-  const size_t off = (size_t)row_id * half * MUL;
-  if (SRC != kSrcRows || A.adam_on) load_row<MUL, VEC, NIT>(s.e, A.table + off, half, A.ncol, lane);
-  if (A.adam_on) {
-    load_row<MUL, VEC, NIT>(s.m, A.m + off, half, A.ncol, lane);
-    load_row<MUL, VEC, NIT>(s.v, A.v + off, half, A.ncol, lane);
-  }
-}
-
 // Short segments (at most A.short_max pairs).  The sorted pair list is cut into chunks of 64
 // positions and a fixed grid of wavefronts strides over the chunks; a wavefront owns the short
 // segments that START in its chunk, so its work is bounded by 64 + short_max pairs however the
@@ -370,7 +225,9 @@ __global__ __launch_bounds__(256) void entity_segment_kernel(EntityArgs A) {
     const int my_seg = A.seg_of_pos[pos];
     const int my_s0 = A.seg_start[my_seg];
     const int my_s1 = A.seg_start[my_seg + 1];
-    unsigned long long todo = __ballot(lane < n_here && my_s0 == pos && my_s1 - my_s0 <= A.short_max);
+    const int my_len = my_s1 - my_s0;
+    unsigned long long todo =
+        __ballot(lane < n_here && my_s0 == pos && my_len <= A.short_max && !(A.skip_single && my_len == 1));
     if (todo == 0ull) continue;
     const int my_id = A.sorted_ids[pos];
 

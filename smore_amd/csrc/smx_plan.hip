@@ -22,9 +22,11 @@
 namespace smx {
 
 __global__ __launch_bounds__(256) void plan_keys_kernel(const long long* __restrict__ idx, unsigned* __restrict__ keys,
-                                                        int n, unsigned long long n_rows, int* err) {
+                                                        int* __restrict__ pair_seg, int n, unsigned long long n_rows,
+                                                        int* err) {
   const int p = blockIdx.x * blockDim.x + threadIdx.x;
   if (p >= n) return;
+  if (pair_seg) pair_seg[p] = 0;  // "not alone"; the emit kernel overwrites the entries of one-pair segments
   long long id = idx[p];
   if ((unsigned long long)id >= n_rows) {
     if (err) *err = 1;
@@ -43,16 +45,20 @@ __global__ __launch_bounds__(256) void plan_heads_kernel(const int* __restrict__
 __global__ __launch_bounds__(256) void plan_emit_kernel(const int* __restrict__ sorted_ids, const int* __restrict__ order,
                                                         const unsigned* __restrict__ seg_incl, int* __restrict__ seg_of_pos,
                                                         long long* __restrict__ uniq, int* __restrict__ seg_start,
-                                                        long long* __restrict__ inverse, int* __restrict__ n_uniq, int n) {
+                                                        long long* __restrict__ inverse, int* __restrict__ pair_seg,
+                                                        int* __restrict__ n_uniq, int n) {
   const int p = blockIdx.x * blockDim.x + threadIdx.x;
   if (p >= n) return;
   const int seg = (int)seg_incl[p] - 1;
   seg_of_pos[p] = seg;
-  if (p == 0 || sorted_ids[p] != sorted_ids[p - 1]) {
+  const bool head = p == 0 || sorted_ids[p] != sorted_ids[p - 1];
+  if (head) {
     uniq[seg] = (long long)(unsigned)sorted_ids[p];
     seg_start[seg] = p;
   }
   if (inverse) inverse[order[p]] = seg;
+  if (pair_seg && head && (p == n - 1 || sorted_ids[p + 1] != sorted_ids[p]))
+    pair_seg[order[p]] = seg | (int)0x80000000;  // this pair is its segment: sign bit + segment number
   if (p == n - 1) {
     *n_uniq = seg + 1;
     seg_start[seg + 1] = n;
@@ -101,7 +107,7 @@ size_t smx_plan_workspace_bytes(size_t n_pairs, size_t n_rows) {
 
 int smx_plan_build(void* stream, const int64_t* idx, size_t n_pairs, size_t n_rows, void* workspace,
                    size_t workspace_bytes, int32_t* order, int32_t* sorted_ids, int32_t* seg_of_pos, int64_t* uniq,
-                   int32_t* seg_start, int64_t* inverse, int32_t* n_uniq, int* err_flag) {
+                   int32_t* seg_start, int64_t* inverse, int32_t* pair_seg, int32_t* n_uniq, int* err_flag) {
   using namespace smx;
   if (!idx || !order || !sorted_ids || !seg_of_pos || !uniq || !seg_start || !n_uniq || !workspace)
     return fail(SMX_ERR_ARG, "null pointer in plan build");
@@ -121,8 +127,8 @@ int smx_plan_build(void* stream, const int64_t* idx, size_t n_pairs, size_t n_ro
   const int n = (int)n_pairs;
   const unsigned blocks = (unsigned)((n_pairs + 255) / 256);
 
-  hipLaunchKernelGGL(plan_keys_kernel, dim3(blocks), dim3(256), 0, st, reinterpret_cast<const long long*>(idx), keys, n,
-                     (unsigned long long)n_rows, err_flag);
+  hipLaunchKernelGGL(plan_keys_kernel, dim3(blocks), dim3(256), 0, st, reinterpret_cast<const long long*>(idx), keys,
+                     pair_seg, n, (unsigned long long)n_rows, err_flag);
   size_t tb = s.temp_bytes;
   hipError_t e = rocprim::radix_sort_pairs(temp, tb, keys, reinterpret_cast<unsigned*>(sorted_ids),
                                            rocprim::counting_iterator<int>(0), order, n_pairs, 0, key_bits(n_rows), st);
@@ -132,7 +138,8 @@ int smx_plan_build(void* stream, const int64_t* idx, size_t n_pairs, size_t n_ro
   e = rocprim::inclusive_scan(temp, tb, heads, scan, n_pairs, rocprim::plus<unsigned>(), st);
   if (e != hipSuccess) return fail(SMX_ERR_HIP, "scan: %s", hipGetErrorString(e));
   hipLaunchKernelGGL(plan_emit_kernel, dim3(blocks), dim3(256), 0, st, sorted_ids, order, scan, seg_of_pos,
-                     reinterpret_cast<long long*>(uniq), seg_start, reinterpret_cast<long long*>(inverse), n_uniq, n);
+                     reinterpret_cast<long long*>(uniq), seg_start, reinterpret_cast<long long*>(inverse), pair_seg, n_uniq,
+                     n);
   return check_launch("plan build");
 }
 

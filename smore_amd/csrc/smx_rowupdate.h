@@ -1,0 +1,181 @@
+// Finishing one entity row: the pieces shared by the entity pass (smx_entity_impl.h) and by the
+// query-backward kernel when it finishes one-pair segments itself (smx_score_impl.h).
+//
+// "Finishing" = turning the summed accumulators of a segment into the row's gradient (model hook,
+// clamp mask), storing it as a merged-gradient row and/or applying the lazy Adam update of
+// smore/common/embedding/embed_optimizer.py:208-252 to the w, m, v rows in place.
+#pragma once
+#include <cmath>
+
+#include "../../include/smore_amd.h"
+#include "smx_models.h"
+
+namespace smx {
+
+constexpr int kSrcRows = 100;  // source = materialised gradient rows instead of a score model
+
+__host__ __device__ constexpr int src_mul(int s) { return s == kSrcRows ? 1 : model_mul(s); }
+
+struct AdamConsts {
+  float beta1, beta2, omb1, omb2, eps, step_size, inv_sqrt_bc2;
+};
+
+inline AdamConsts make_adam_consts(const smx_adam_params* a) {
+  AdamConsts c;
+  const double bc1 = 1.0 - std::pow(a->beta1, (double)a->step);
+  const double bc2 = 1.0 - std::pow(a->beta2, (double)a->step);
+  c.beta1 = (float)a->beta1;
+  c.beta2 = (float)a->beta2;
+  c.omb1 = (float)(1.0 - a->beta1);
+  c.omb2 = (float)(1.0 - a->beta2);
+  c.eps = (float)a->eps;
+  c.step_size = (float)(-a->lr / bc1);
+  c.inv_sqrt_bc2 = (float)(1.0 / std::sqrt(bc2));
+  return c;
+}
+
+// Where finished rows go.
+struct RowSink {
+  float* table;   // entity table: read for the model sources, updated when adam_on
+  float* m;
+  float* v;
+  float* merged;  // [U, row_len] or null
+  int adam_on;
+  AdamConsts a;
+  ScoreParams p;
+  int ncol;       // columns per half row (model sources) or per row (gradient rows)
+};
+
+template <int VEC> struct Pack2 {
+  float v[VEC];
+};
+
+template <int VEC>
+__device__ __forceinline__ Pack2<VEC> ld(const float* __restrict__ base, int col) {
+  Pack2<VEC> r;
+  if constexpr (VEC == 4) {
+    const float4 t = reinterpret_cast<const float4*>(base)[col];
+    r.v[0] = t.x;
+    r.v[1] = t.y;
+    r.v[2] = t.z;
+    r.v[3] = t.w;
+  } else {
+    r.v[0] = base[col];
+  }
+  return r;
+}
+
+template <int VEC>
+__device__ __forceinline__ void st(float* __restrict__ base, int col, const float (&x)[VEC]) {
+  if constexpr (VEC == 4) {
+    reinterpret_cast<float4*>(base)[col] = make_float4(x[0], x[1], x[2], x[3]);
+  } else {
+    base[col] = x[0];
+  }
+}
+
+// The lane's columns of one table row (both halves for the two-half models).
+template <int MUL, int VEC, int NIT> struct RowRegs {
+  Pack2<VEC> h[MUL][NIT];
+};
+
+template <int MUL, int VEC, int NIT>
+__device__ __forceinline__ void load_row(RowRegs<MUL, VEC, NIT>& r, const float* __restrict__ base, int half, int ncol,
+                                         int lane) {
+#pragma unroll
+  for (int h = 0; h < MUL; ++h)
+#pragma unroll
+    for (int it = 0; it < NIT; ++it) r.h[h][it] = ld<VEC>(base + h * half, min(lane + 64 * it, ncol - 1));
+}
+
+// Coefficient on the second accumulator (BOX: inside distance) from the first.
+// Finishes one entity row: clamp mask, merged-gradient store, Adam.  g1/g2 are the lane's columns of
+// the summed gradient of the first / second half row; w, m0, v0 the row's current weights and moments
+// (w is always valid for the model sources -- it is the entity row the gradient was computed from).
+// ADAM_STATIC: the caller knows at compile time that Adam is on (its m0 / v0 are loaded); otherwise the
+// run-time flag A.adam_on decides.
+template <int SRC, int VEC, int NIT, bool REG, bool ADAM_STATIC = false>
+__device__ __forceinline__ void finish_row(const RowSink& A, int lane, unsigned row_id, int seg,
+                                           float (&g1)[NIT][VEC], float (&g2)[NIT][VEC],
+                                           const RowRegs<src_mul(SRC), VEC, NIT>& w,
+                                           const RowRegs<src_mul(SRC), VEC, NIT>& m0,
+                                           const RowRegs<src_mul(SRC), VEC, NIT>& v0) {
+  constexpr int MUL = src_mul(SRC);
+  const int half = A.ncol * VEC;
+  const size_t row_len = (size_t)half * MUL;
+  if constexpr (SRC != kSrcRows) {
+#pragma unroll
+    for (int it = 0; it < NIT; ++it)
+#pragma unroll
+      for (int x = 0; x < VEC; ++x) {
+        const float x1 = REG ? reg_apply(w.h[0][it].v[x], A.p) : w.h[0][it].v[x];
+        const float x2 = MUL == 2 ? (REG ? reg_apply(w.h[MUL - 1][it].v[x], A.p) : w.h[MUL - 1][it].v[x]) : 0.f;
+        finish_entity_grad<SRC>(x1, x2, g1[it][x], g2[it][x]);
+      }
+  }
+  if (REG) {
+#pragma unroll
+    for (int it = 0; it < NIT; ++it)
+#pragma unroll
+      for (int x = 0; x < VEC; ++x) {
+        g1[it][x] = reg_mask(w.h[0][it].v[x], g1[it][x], A.p);
+        if (MUL == 2) g2[it][x] = reg_mask(w.h[MUL - 1][it].v[x], g2[it][x], A.p);
+      }
+  }
+  if (A.merged) {
+    float* out = A.merged + (size_t)seg * row_len;
+#pragma unroll
+    for (int it = 0; it < NIT; ++it) {
+      const int c = lane + 64 * it;
+      if (c < A.ncol) {
+        st<VEC>(out, c, g1[it]);
+        if (MUL == 2) st<VEC>(out + half, c, g2[it]);
+      }
+    }
+  }
+  if (ADAM_STATIC || A.adam_on) {
+    float* pw = A.table + (size_t)row_id * row_len;
+    float* pm = A.m + (size_t)row_id * row_len;
+    float* pv = A.v + (size_t)row_id * row_len;
+#pragma unroll
+    for (int h = 0; h < MUL; ++h) {
+#pragma unroll
+      for (int it = 0; it < NIT; ++it) {
+        const int c = lane + 64 * it;
+        if (c < A.ncol) {
+          float wn[VEC], mn[VEC], vn[VEC];
+#pragma unroll
+          for (int x = 0; x < VEC; ++x) {
+            const float g = h == 0 ? g1[it][x] : g2[it][x];
+            mn[x] = m0.h[h][it].v[x] * A.a.beta1 + g * A.a.omb1;
+            vn[x] = v0.h[h][it].v[x] * A.a.beta2 + g * g * A.a.omb2;
+            const float denom = sqrtf(vn[x]) * A.a.inv_sqrt_bc2 + A.a.eps;
+            wn[x] = w.h[h][it].v[x] + A.a.step_size * mn[x] / denom;
+          }
+          st<VEC>(pw + h * half, c, wn);
+          st<VEC>(pm + h * half, c, mn);
+          st<VEC>(pv + h * half, c, vn);
+        }
+      }
+    }
+  }
+}
+
+template <int MUL, int VEC, int NIT> struct RowState {
+  RowRegs<MUL, VEC, NIT> e, m, v;
+};
+
+template <int SRC, int VEC, int NIT>
+__device__ __forceinline__ void request_state(const RowSink& A, int lane, unsigned row_id,
+                                              RowState<src_mul(SRC), VEC, NIT>& s) {
+  constexpr int MUL = src_mul(SRC);
+  const int half = A.ncol * VEC;
+  const size_t off = (size_t)row_id * half * MUL;
+  if (SRC != kSrcRows || A.adam_on) load_row<MUL, VEC, NIT>(s.e, A.table + off, half, A.ncol, lane);
+  if (A.adam_on) {
+    load_row<MUL, VEC, NIT>(s.m, A.m + off, half, A.ncol, lane);
+    load_row<MUL, VEC, NIT>(s.v, A.v + off, half, A.ncol, lane);
+  }
+}
+
+}  // namespace smx

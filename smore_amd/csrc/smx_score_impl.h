@@ -1,0 +1,429 @@
+// Gather-fused scoring, forward and query-side backward (fp32).
+//
+// Replaces, in one pass each, the sequence the reference runs per training
+// step for the negative samples (smore/models/kg_reasoning.py:301-307,349-355):
+//   rows = table[idx]                      smore/common/embedding/embed_rw.py:74-75
+//   [optional clamp(rows + 1, .05, 1e9)]   smore/common/modules.py:29-36
+//   d = dist(rows, query)                  smore/common/torchext/common_kernel.h:33-56
+//   logit = gamma - d                      custom_cal_logit of smore/models/*.py
+// and, backward, the query-gradient kernel common_kernel.h:92-123.  The
+// [B,K,D] gathered tensor is never materialised: a wavefront reads each entity
+// row straight from the table with 16-byte loads (one float4 column per lane).
+//
+// Work split.  forward: workgroup = (query b, tile of negatives); the query
+// row(s) are staged once in LDS, every lane then keeps the features it owns in
+// registers for the whole tile; each of the four wavefronts streams its
+// quarter of the tile's rows, two batches of rows in flight at a time.  backward: one workgroup per
+// query walks all K negatives, wavefront partial sums are combined through LDS
+// in wavefront order, so the gradient has a fixed summation order.
+#pragma once
+#include "smx_common.h"
+#include "smx_models.h"
+#include "smx_rowupdate.h"
+#include "smx_wave.h"
+
+namespace smx {
+
+struct ScoreArgs {
+  const float* table;
+  const long long* idx;  // null: `table` holds the B*K rows in pair order
+  const float* q1;
+  const float* q2;
+  float* score_out;      // forward
+  const float* score;    // backward: the logits the forward wrote
+  const float* gscore;
+  float* gq1;
+  float* gq2;
+  int B, K, ncol;
+  unsigned long long n_rows;
+  ScoreParams p;
+  int* err;
+  const int* pair_seg;   // one-pair segments finished by the query backward (SINGLES kernels)
+  RowSink sink;
+};
+
+template <int VEC> struct Pack {
+  float v[VEC];
+};
+
+template <int VEC>
+__device__ __forceinline__ Pack<VEC> load_pack(const float* __restrict__ base, int col) {
+  Pack<VEC> r;
+  if constexpr (VEC == 4) {
+    const float4 t = reinterpret_cast<const float4*>(base)[col];
+    r.v[0] = t.x;
+    r.v[1] = t.y;
+    r.v[2] = t.z;
+    r.v[3] = t.w;
+  } else {
+    r.v[0] = base[col];
+  }
+  return r;
+}
+
+// Loads the features a lane owns of the staged query into registers.
+template <int M, int VEC, int NIT, bool FWD>
+__device__ __forceinline__ void load_query_regs(const float* lds, int dim, int ncol, int lane,
+                                                typename ModelOps<M>::Q (&q)[NIT][VEC]) {
+#pragma unroll
+  for (int it = 0; it < NIT; ++it) {
+    const int c = lane + 64 * it;
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) {
+      const int cc = min(c, ncol - 1);  // lanes past the row end hold a copy of the last column
+      const float a = lds[cc * VEC + v];
+      const float b = model_nq(M) == 2 ? lds[dim + cc * VEC + v] : 0.f;
+      q[it][v] = FWD ? prep_forward<M>(a, b) : prep_backward_query<M>(a, b);
+    }
+  }
+}
+
+template <int M>
+__device__ __forceinline__ void stage_query(float* lds, const float* __restrict__ q1, const float* __restrict__ q2,
+                                            size_t b, int dim) {
+  for (int d = threadIdx.x; d < dim; d += blockDim.x) {
+    lds[d] = q1[b * dim + d];
+    if (model_nq(M) == 2) lds[dim + d] = q2[b * dim + d];
+  }
+  __syncthreads();
+}
+
+// ---- streaming the rows of up to 64 pairs through a wavefront -----------------------------------
+// The lanes first fetch, in one coalesced load, the ids of the pairs the wavefront is about to
+// process (pair j of the batch lives in lane j) and turn them into row offsets.  The row loop then
+// needs no memory access to find a row: the offset comes out of lane j with two v_readlane, so the
+// only loads in the loop are the rows themselves.  Rows are requested RIF at a time into two
+// register sets used in turn: while set A is consumed, set B is already on its way.  All loads are
+// unconditional (indices are clamped) so that they issue as one batch and stay in flight together.
+
+struct PairBatch {
+  unsigned off_lo, off_hi;  // this lane's pair: offset of its entity row in floats
+  unsigned row;             // ... and the row number (low 32 bits)
+};
+
+__device__ __forceinline__ PairBatch load_pair_batch(const long long* __restrict__ idx, size_t first_pair, int cnt,
+                                                     int lane, size_t row_len, unsigned long long n_rows, int& bad) {
+  const size_t pair = first_pair + min(lane, cnt - 1);
+  long long row = idx ? idx[pair] : (long long)pair;
+  if ((unsigned long long)row >= n_rows) {  // id outside the table: remember it, read row 0 instead
+    bad = 1;
+    row = 0;
+  }
+  const unsigned long long off = (unsigned long long)row * row_len;
+  return {(unsigned)off, (unsigned)(off >> 32), (unsigned)row};
+}
+
+__device__ __forceinline__ unsigned long long batch_off(const PairBatch& pb, int j) {
+  const unsigned lo = (unsigned)__builtin_amdgcn_readlane((int)pb.off_lo, j);
+  const unsigned hi = (unsigned)__builtin_amdgcn_readlane((int)pb.off_hi, j);
+  return ((unsigned long long)hi << 32) | lo;
+}
+__device__ __forceinline__ const float* batch_row(const float* __restrict__ table, const PairBatch& pb, int j) {
+  return table + batch_off(pb, j);
+}
+
+template <int MUL, int VEC, int NIT, int RIF> struct RowSet {
+  Pack<VEC> e1[RIF][NIT];
+  Pack<VEC> e2[RIF][NIT];
+};
+
+// Requests rows j0 .. j0+RIF-1 of the batch (clamped to cnt-1).
+template <int MUL, int VEC, int NIT, int RIF>
+__device__ __forceinline__ void request_rows(RowSet<MUL, VEC, NIT, RIF>& rs, const float* __restrict__ table,
+                                             const PairBatch& pb, int j0, int cnt, int dim, int ncol, int lane) {
+#pragma unroll
+  for (int r = 0; r < RIF; ++r) {
+    const float* pe = batch_row(table, pb, min(j0 + r, cnt - 1));
+#pragma unroll
+    for (int it = 0; it < NIT; ++it) {
+      const int c = min(lane + 64 * it, ncol - 1);
+      rs.e1[r][it] = load_pack<VEC>(pe, c);
+      if (MUL == 2) rs.e2[r][it] = load_pack<VEC>(pe + dim, c);
+    }
+  }
+}
+
+// Streams the cnt (<= 64) rows of a batch through `consume(j, e1, e2)`, j ascending.
+template <int MUL, int VEC, int NIT, int RIF, class Consume>
+__device__ __forceinline__ void stream_batch(const float* __restrict__ table, const PairBatch& pb, int cnt, int dim,
+                                             int ncol, int lane, Consume&& consume) {
+  RowSet<MUL, VEC, NIT, RIF> a, b;
+  const int last = ((cnt - 1) / RIF) * RIF;  // first row of the last group
+  request_rows<MUL, VEC, NIT, RIF>(a, table, pb, 0, cnt, dim, ncol, lane);
+  for (int j0 = 0; j0 < cnt; j0 += 2 * RIF) {
+    request_rows<MUL, VEC, NIT, RIF>(b, table, pb, min(j0 + RIF, last), cnt, dim, ncol, lane);
+#pragma unroll
+    for (int r = 0; r < RIF; ++r)
+      if (j0 + r < cnt) consume(j0 + r, a.e1[r], a.e2[r]);
+    request_rows<MUL, VEC, NIT, RIF>(a, table, pb, min(j0 + 2 * RIF, last), cnt, dim, ncol, lane);
+#pragma unroll
+    for (int r = 0; r < RIF; ++r)
+      if (j0 + RIF + r < cnt) consume(j0 + RIF + r, b.e1[r], b.e2[r]);
+  }
+}
+
+template <int M, int VEC, int NIT, int RIF, bool REG>
+__global__ __launch_bounds__(256) void score_forward_kernel(ScoreArgs A, int tiles, int tile_k) {
+  const float* __restrict__ table = A.table;
+  const long long* __restrict__ idx = A.idx;
+  const float* __restrict__ q1 = A.q1;
+  const float* __restrict__ q2 = A.q2;
+  float* __restrict__ score = A.score_out;
+  const int K = A.K, ncol = A.ncol;
+  const unsigned long long n_rows = A.n_rows;
+  const ScoreParams p = A.p;
+  int* err = A.err;
+  constexpr int MUL = model_mul(M);
+  extern __shared__ float lds[];
+  const int b = blockIdx.x / tiles;
+  const int tile = blockIdx.x - b * tiles;
+  const int lane = threadIdx.x & 63;
+  const int wave = uniform(threadIdx.x >> 6);
+  const int dim = ncol * VEC;
+  const size_t row_len = (size_t)dim * MUL;
+
+  // this wavefront's share of the tile: per_wave (<= 64) consecutive negatives
+  const int per_wave = tile_k / 4;
+  const int kw0 = tile * tile_k + wave * per_wave;
+  const int cnt = min(per_wave, K - kw0);
+  int bad = 0;
+  PairBatch pb{0u, 0u};
+  if (cnt > 0) pb = load_pair_batch(idx, (size_t)b * K + kw0, cnt, lane, row_len, n_rows, bad);
+
+  stage_query<M>(lds, q1, q2, b, dim);
+  typename ModelOps<M>::Q q[NIT][VEC];
+  load_query_regs<M, VEC, NIT, true>(lds, dim, ncol, lane, q);
+  if (cnt <= 0) return;
+
+  float* out = score + (size_t)b * K + kw0;
+  stream_batch<MUL, VEC, NIT, RIF>(table, pb, cnt, dim, ncol, lane,
+                                   [&](int j, const Pack<VEC>(&e1)[NIT], const Pack<VEC>(&e2)[NIT]) {
+    float a0 = 0.f, a1 = 0.f;
+#pragma unroll
+    for (int it = 0; it < NIT; ++it) {
+      if (lane + 64 * it < ncol) {
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) {
+          const float x1 = REG ? reg_apply(e1[it].v[v], p) : e1[it].v[v];
+          const float x2 = MUL == 2 ? (REG ? reg_apply(e2[it].v[v], p) : e2[it].v[v]) : 0.f;
+          ModelOps<M>::fwd(x1, x2, q[it][v], a0, a1);
+        }
+      }
+    }
+    // the logit is linear in the accumulators: fold them per lane, reduce once
+    const float folded = wave_sum_f32(ModelOps<M>::fold(a0, a1, p));
+    if (lane == 0) out[j] = ModelOps<M>::score(folded, p);
+  });
+  if (__ballot(bad != 0) != 0ull && err && lane == 0) *err = 1;
+}
+
+// SINGLES: the plan marks pairs whose entity occurs once in the step.  Such a segment needs no
+// reduction, and this kernel already holds the pair's query in registers and has just read its entity
+// row, so it finishes the row here (merged-gradient row and/or Adam on w, m, v) instead of leaving it
+// to the entity pass, which would have to fetch the query rows and the entity row again.
+// SINGLES: 0 = leave every segment to the entity pass, 1 = finish one-pair segments here as merged-gradient
+// rows, 2 = ... with Adam on w, m, v (and the merged row if asked for).
+template <int M, int VEC, int NIT, int RIF, int NW, bool REG, int SINGLES>
+__global__ __launch_bounds__(NW * 64) void score_backward_query_kernel(ScoreArgs A) {
+  const float* __restrict__ table = A.table;
+  const long long* __restrict__ idx = A.idx;
+  const float* __restrict__ q1 = A.q1;
+  const float* __restrict__ q2 = A.q2;
+  const float* __restrict__ score = A.score;
+  const float* __restrict__ gscore = A.gscore;
+  float* __restrict__ gq1 = A.gq1;
+  float* __restrict__ gq2 = A.gq2;
+  const int K = A.K, ncol = A.ncol;
+  const unsigned long long n_rows = A.n_rows;
+  const ScoreParams p = A.p;
+  constexpr int MUL = model_mul(M);
+  constexpr int NQ = model_nq(M);
+  extern __shared__ float lds[];
+  const int b = blockIdx.x;
+  const int lane = threadIdx.x & 63;
+  const int wave = uniform(threadIdx.x >> 6);
+  const int dim = ncol * VEC;
+  const size_t row_len = (size_t)dim * MUL;
+
+  stage_query<M>(lds, q1, q2, b, dim);
+  typename ModelOps<M>::Q q[NIT][VEC];
+  load_query_regs<M, VEC, NIT, false>(lds, dim, ncol, lane, q);
+
+  float g1[NIT][VEC], g2[NIT][VEC];
+#pragma unroll
+  for (int it = 0; it < NIT; ++it)
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) g1[it][v] = g2[it][v] = 0.f;
+
+  // this wavefront's share of the query's negatives: a contiguous range, walked in batches of 64
+  const int per_wave = (K + NW - 1) / NW;
+  const int kw0 = wave * per_wave;
+  const int kw1 = min(K, kw0 + per_wave);
+  int bad = 0;
+  for (int kb = kw0; kb < kw1; kb += 64) {
+    const int cnt = min(64, kw1 - kb);
+    const size_t first = (size_t)b * K + kb;
+    const PairBatch pb = load_pair_batch(idx, first, cnt, lane, row_len, n_rows, bad);
+    const size_t mine = first + min(lane, cnt - 1);
+    float my_c0, my_c1;
+    ModelOps<M>::coef(gscore[mine], score[mine], p, my_c0, my_c1);
+    stream_batch<MUL, VEC, NIT, RIF>(table, pb, cnt, dim, ncol, lane,
+                                     [&](int j, const Pack<VEC>(&e1)[NIT], const Pack<VEC>(&e2)[NIT]) {
+      const float c0 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(my_c0), j));
+      const float c1 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(my_c1), j));
+#pragma unroll
+      for (int it = 0; it < NIT; ++it) {
+        if (lane + 64 * it < ncol) {
+#pragma unroll
+          for (int v = 0; v < VEC; ++v) {
+            const float x1 = REG ? reg_apply(e1[it].v[v], p) : e1[it].v[v];
+            const float x2 = MUL == 2 ? (REG ? reg_apply(e2[it].v[v], p) : e2[it].v[v]) : 0.f;
+            ModelOps<M>::bwd_q(c0, c1, x1, x2, q[it][v], g1[it][v], g2[it][v]);
+          }
+        }
+      }
+    });
+
+    if constexpr (SINGLES != 0) {
+      // One row at a time per wavefront: with the registers this keeps free the kernel runs at full
+      // occupancy, and the other wavefronts of the CU cover the latency of the row loads.
+      const int my_ps = A.pair_seg[mine];
+      unsigned long long todo = __ballot(lane < cnt && my_ps < 0);
+      while (todo != 0ull) {
+        const int j = __builtin_ctzll(todo);
+        todo &= todo - 1;
+        const unsigned long long off = batch_off(pb, j);
+        RowRegs<MUL, VEC, NIT> e, m0, v0;
+        load_row<MUL, VEC, NIT>(e, table + off, dim, ncol, lane);
+        if constexpr (SINGLES == 2) {
+          load_row<MUL, VEC, NIT>(m0, A.sink.m + off, dim, ncol, lane);
+          load_row<MUL, VEC, NIT>(v0, A.sink.v + off, dim, ncol, lane);
+        }
+        const float c0 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(my_c0), j));
+        const float c1 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(my_c1), j));
+        const int seg = __builtin_amdgcn_readlane(my_ps, j) & 0x7fffffff;
+        const unsigned row = (unsigned)__builtin_amdgcn_readlane((int)pb.row, j);
+        float ge1[NIT][VEC], ge2[NIT][VEC];
+#pragma unroll
+        for (int it = 0; it < NIT; ++it)
+#pragma unroll
+          for (int v = 0; v < VEC; ++v) {
+            ge1[it][v] = ge2[it][v] = 0.f;
+            const float x1 = REG ? reg_apply(e.h[0][it].v[v], p) : e.h[0][it].v[v];
+            const float x2 = MUL == 2 ? (REG ? reg_apply(e.h[MUL - 1][it].v[v], p) : e.h[MUL - 1][it].v[v]) : 0.f;
+            ModelOps<M>::bwd_e(c0, c1, x1, x2, q[it][v], ge1[it][v], ge2[it][v]);
+          }
+        finish_row<M, VEC, NIT, REG, SINGLES == 2>(A.sink, lane, row, seg, ge1, ge2, e, m0, v0);
+      }
+    }
+  }
+
+#pragma unroll
+  for (int it = 0; it < NIT; ++it)
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) finish_query_grad<M>(q[it][v], g1[it][v], g2[it][v], p);
+
+  // wavefront partials -> LDS -> fixed-order sum over wavefronts
+  float* part = lds + NQ * dim;  // [NW][NQ][dim]
+#pragma unroll
+  for (int it = 0; it < NIT; ++it) {
+    const int c = lane + 64 * it;
+    if (c < ncol) {
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) {
+        part[(wave * NQ + 0) * dim + c * VEC + v] = g1[it][v];
+        if (NQ == 2) part[(wave * NQ + 1) * dim + c * VEC + v] = g2[it][v];
+      }
+    }
+  }
+  __syncthreads();
+  for (int d = threadIdx.x; d < dim; d += NW * 64) {
+    float s1 = 0.f, s2 = 0.f;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) {
+      s1 += part[(w * NQ + 0) * dim + d];
+      if (NQ == 2) s2 += part[(w * NQ + 1) * dim + d];
+    }
+    gq1[(size_t)b * dim + d] = s1;
+    if (NQ == 2) gq2[(size_t)b * dim + d] = s2;
+  }
+}
+
+// rows requested per batch; two batches are in flight at a time
+constexpr int rows_in_flight(int nit, int mul) {
+  const int r = 4 / (nit * mul);
+  return r < 1 ? 1 : r;
+}
+
+template <int M, int VEC, int NIT, bool REG>
+int launch_forward_reg(hipStream_t st, const ScoreArgs& A) {
+  constexpr int RIF = rows_in_flight(NIT, model_mul(M));
+  const size_t B = (size_t)A.B, K = (size_t)A.K;
+  int tile_k = 256;  // 64 negatives per wavefront; smaller tiles when the grid would not fill the chip
+  while (tile_k > 4 * RIF && (B * ((K + tile_k - 1) / tile_k) < 8192 || (size_t)tile_k / 2 >= K)) tile_k /= 2;
+  const int tiles = (int)((K + tile_k - 1) / tile_k);
+  const size_t lds = (size_t)model_nq(M) * A.ncol * VEC * sizeof(float);
+  hipLaunchKernelGGL((score_forward_kernel<M, VEC, NIT, RIF, REG>), dim3((unsigned)(B * tiles)), dim3(256), lds, st, A,
+                     tiles, tile_k);
+  return check_launch("score forward");
+}
+
+template <int M, int VEC, int NIT, int NW, bool REG>
+int launch_backward_query_reg(hipStream_t st, const ScoreArgs& A) {
+  constexpr int RIF = rows_in_flight(NIT, model_mul(M));
+  const size_t lds = (size_t)(NW + 1) * model_nq(M) * A.ncol * VEC * sizeof(float);
+  if (A.pair_seg && A.sink.adam_on)
+    hipLaunchKernelGGL((score_backward_query_kernel<M, VEC, NIT, RIF, NW, REG, 2>), dim3((unsigned)A.B),
+                       dim3(NW * 64), lds, st, A);
+  else if (A.pair_seg)
+    hipLaunchKernelGGL((score_backward_query_kernel<M, VEC, NIT, RIF, NW, REG, 1>), dim3((unsigned)A.B),
+                       dim3(NW * 64), lds, st, A);
+  else
+    hipLaunchKernelGGL((score_backward_query_kernel<M, VEC, NIT, RIF, NW, REG, 0>), dim3((unsigned)A.B),
+                       dim3(NW * 64), lds, st, A);
+  return check_launch("score backward (query)");
+}
+
+template <int M, int VEC, int NIT>
+int launch_score(hipStream_t st, const ScoreArgs& A, bool forward) {
+  const bool reg = M == mBetaKL && A.p.reg_on;
+  if (forward) {
+    if constexpr (M == mBetaKL) {
+      if (reg) return launch_forward_reg<M, VEC, NIT, true>(st, A);
+    }
+    return launch_forward_reg<M, VEC, NIT, false>(st, A);
+  }
+  // wavefronts per query: as many as the LDS combine buffer allows
+  const size_t per_wave = (size_t)model_nq(M) * A.ncol * VEC * sizeof(float);
+  const int nw = 9 * per_wave <= 60 * 1024 ? 8 : (5 * per_wave <= 60 * 1024 ? 4 : 2);
+  if constexpr (M == mBetaKL) {
+    if (reg) {
+      if (nw == 8) return launch_backward_query_reg<M, VEC, NIT, 8, true>(st, A);
+      if (nw == 4) return launch_backward_query_reg<M, VEC, NIT, 4, true>(st, A);
+      return launch_backward_query_reg<M, VEC, NIT, 2, true>(st, A);
+    }
+  }
+  if (nw == 8) return launch_backward_query_reg<M, VEC, NIT, 8, false>(st, A);
+  if (nw == 4) return launch_backward_query_reg<M, VEC, NIT, 4, false>(st, A);
+  return launch_backward_query_reg<M, VEC, NIT, 2, false>(st, A);
+}
+
+// Instantiated once per model in its own translation unit (smx_score_inst_*.hip).
+template <int M>
+int score_dispatch(hipStream_t st, const ScoreArgs& A, int vec, int nit, bool forward) {
+  if (vec == 4) {
+    switch (nit) {
+      case 1: return launch_score<M, 4, 1>(st, A, forward);
+      case 2: return launch_score<M, 4, 2>(st, A, forward);
+      case 4: return launch_score<M, 4, 4>(st, A, forward);
+      default: return launch_score<M, 4, 8>(st, A, forward);
+    }
+  }
+  switch (nit) {
+    case 1: return launch_score<M, 1, 1>(st, A, forward);
+    case 2: return launch_score<M, 1, 2>(st, A, forward);
+    default: return launch_score<M, 1, 4>(st, A, forward);
+  }
+}
+
+}  // namespace smx

@@ -123,6 +123,7 @@ class SegmentPlan:
         self.seg_start = torch.empty(n_pairs + 1, **i32)
         self.uniq_buf = torch.empty(n_pairs, dtype=torch.int64, device=device)
         self.inverse = torch.empty(n_pairs, dtype=torch.int64, device=device) if want_inverse else None
+        self.pair_seg = torch.empty(n_pairs, **i32)
         self.n_uniq_dev = torch.zeros(1, **i32)
         self._n_uniq = None
 
@@ -139,7 +140,7 @@ class SegmentPlan:
 
     def view(self):
         return _lib.PlanView(_ptr(self.order), _ptr(self.sorted_ids), _ptr(self.seg_of_pos), _ptr(self.seg_start),
-                             _ptr(self.uniq_buf), _ptr(self.n_uniq_dev), self.n_pairs)
+                             _ptr(self.uniq_buf), _ptr(self.n_uniq_dev), _ptr(self.pair_seg), self.n_pairs)
 
 
 def _workspace(nbytes, device):
@@ -160,7 +161,7 @@ def build_plan(idx, n_rows, want_inverse=False, err_flag=None):
         ws = _workspace(nbytes, flat.device)
         _lib.call("smx_plan_build", _stream(flat), _ptr(flat), n, n_rows, _ptr(ws), ws.numel(), _ptr(plan.order),
                   _ptr(plan.sorted_ids), _ptr(plan.seg_of_pos), _ptr(plan.uniq_buf), _ptr(plan.seg_start),
-                  _ptr(plan.inverse), _ptr(plan.n_uniq_dev), _ptr(err_flag))
+                  _ptr(plan.inverse), _ptr(plan.pair_seg), _ptr(plan.n_uniq_dev), _ptr(err_flag))
     return plan
 
 
@@ -190,6 +191,32 @@ def score_backward_entity(model, plan, table, q1, q2, score, gscore, params, mer
         _lib.call("smx_score_backward_entity", MODELS[model], _stream(table), ctypes.byref(view), _ptr(table),
                   table.shape[0], _ptr(q1), _ptr(q2), _ptr(score), _ptr(gscore), b, k, dim, ctypes.byref(params),
                   _ptr(merged), _ptr(m), _ptr(v), None if adam is None else ctypes.byref(adam), _ptr(ws), ws.numel())
+
+
+def score_backward_fused(model, plan, table, idx, q1, q2, score, gscore, params, merged=None, m=None, v=None,
+                         adam=None):
+    """Query gradients and all entity rows of the step in one call (see smx_score_backward_fused).
+    Returns (gq1, gq2); merged / table, m, v are written in place as in score_backward_entity."""
+    b, k, dim = _dims(model, table, idx, q1, q2)
+    for t, name in ((score, "score"), (gscore, "gscore"), (merged, "merged"), (m, "m"), (v, "v")):
+        _f32(t, name)
+    if plan.n_pairs != b * k:
+        raise _lib.SmxError("plan does not belong to these ids")
+    for s in (m, v):
+        if s is not None and s.shape != table.shape:
+            raise _lib.SmxError("Adam state must have the table's shape")
+    if merged is not None and (merged.dim() != 2 or merged.shape[1] != table.shape[1]):
+        raise _lib.SmxError("merged must be [n_uniq or more, row]")
+    gq1 = torch.empty_like(q1)
+    gq2 = None if q2 is None else torch.empty_like(q2)
+    with torch.cuda.device(table.device):
+        ws = _workspace(_lib.load().smx_entity_workspace_bytes(plan.n_pairs, table.shape[1]), table.device)
+        view = plan.view()
+        _lib.call("smx_score_backward_fused", MODELS[model], _stream(table), ctypes.byref(view), _ptr(table),
+                  table.shape[0], _ptr(idx), _ptr(q1), _ptr(q2), _ptr(score), _ptr(gscore), _ptr(gq1), _ptr(gq2),
+                  b, k, dim, ctypes.byref(params), _ptr(merged), _ptr(m), _ptr(v),
+                  None if adam is None else ctypes.byref(adam), _ptr(ws), ws.numel())
+    return gq1, gq2
 
 
 def rows_backward(plan, grad_rows, merged=None, table=None, m=None, v=None, adam=None):

@@ -92,6 +92,16 @@ def run_case(model, n, b, k, dim, zipf=None, cen=0.02, adam_steps=2, lr=1e-3):
     assert_close(merged.cpu().numpy(), o_merged, REL_F32, f"{model} merged entity grad", sum_abs=o_abs)
     assert torch.equal(t_table, dev(table)), "table must not change without Adam"
 
+    # one-call backward (one-pair segments finished by the query-gradient kernel): same values up to the
+    # rounding of a contracted multiply-add (the two kernels are compiled separately)
+    merged3 = torch.full_like(merged, float("nan"))
+    f1, f2 = fused.score_backward_fused(model, plan, t_table, t_idx, t_q1, t_q2, score, t_gs, params, merged=merged3)
+    assert_close(f1.cpu().numpy(), gq1.cpu().numpy(), 1e-6, f"{model} gq1, one-call backward")
+    if gq2 is not None:
+        assert_close(f2.cpu().numpy(), gq2.cpu().numpy(), 1e-6, f"{model} gq2, one-call backward")
+    assert_close(merged3.cpu().numpy(), merged.cpu().numpy(), 1e-6, f"{model} merged, one-call backward")
+    assert (plan.pair_seg < 0).sum().item() == int((np.diff(seg_start) == 1).sum())
+
     # same sum from materialised gradient rows
     merged2 = torch.full_like(merged, float("nan"))
     fused.rows_backward(plan, dev(o_rows.reshape(b * k, -1)), merged=merged2)
@@ -111,8 +121,14 @@ def run_case(model, n, b, k, dim, zipf=None, cen=0.02, adam_steps=2, lr=1e-3):
         fused.score_backward_entity(model, plan, t_table, t_q1, t_q2, sc, t_gs, params, merged=merged)
         w_s, m_s, v_s = (x.cpu().numpy().astype(np.float64) for x in (t_table, t_m, t_v))
         orc.adam_rows(w_s, m_s, v_s, uniq, merged.cpu().numpy().astype(np.float64), lr, step)
+        c_table, c_m, c_v = t_table.clone(), t_m.clone(), t_v.clone()
         fused.score_backward_entity(model, plan, t_table, t_q1, t_q2, sc, t_gs, params, m=t_m, v=t_v,
                                     adam=fused.adam_params(lr, step))
+        fused.score_backward_fused(model, plan, c_table, t_idx, t_q1, t_q2, sc, t_gs, params, m=c_m, v=c_v,
+                                   adam=fused.adam_params(lr, step))
+        for got, ref, what in ((c_table, t_table, "w"), (c_m, t_m, "m"), (c_v, t_v, "v")):
+            assert_close(got.cpu().numpy()[touched], ref.cpu().numpy()[touched], 2e-6, f"{model} one-call backward: {what}")
+            assert torch.equal(got[torch.tensor(~touched, device="cuda")], ref[torch.tensor(~touched, device="cuda")])
         assert_close(t_table.cpu().numpy()[touched], w_s[touched], REL_F32, f"{model} Adam step {step}: w")
         assert_close(t_m.cpu().numpy()[touched], m_s[touched], REL_F32, f"{model} Adam step {step}: m")
         assert_close(t_v.cpu().numpy()[touched], v_s[touched], REL_F32, f"{model} Adam step {step}: v")
@@ -270,3 +286,35 @@ def test_box_tie_conventions_through_the_fused_path():
     merged = torch.empty((n, 4), device="cuda")
     fused.score_backward_entity("box", plan, t_table, t_q1, t_q2, score, t_gs, params, merged=merged)
     assert np.array_equal(merged.cpu().numpy().astype(np.float64), g_rows[:, 0])
+
+
+def test_one_call_backward_with_many_queries_takes_the_one_pair_shortcut():
+    """With query tensors above 4 MiB the one-call backward finishes one-pair segments in the
+    query-gradient kernel; results must still equal the two separate calls."""
+    from smore_amd import fused
+    rng = np.random.default_rng(12)
+    n, b, k, dim = 60000, 4200, 6, 128   # 4200 x 2 x 128 floats = 4.3 MB of queries
+    table, q1, q2, idx, gs = make_problem("box", n, b, k, dim, rng)
+    t_table, t_q1, t_q2, t_gs = dev(table), dev(q1), dev(q2), dev(gs)
+    t_idx = torch.tensor(idx, device="cuda")
+    params = fused.score_params(24.0, 0.02)
+    plan = fused.build_plan(t_idx, n)
+    assert 0.3 < (plan.pair_seg < 0).float().mean().item() < 0.9
+    score = fused.score_forward("box", t_table, t_idx, t_q1, t_q2, params)
+    gq1, gq2 = fused.score_backward_query("box", t_table, t_idx, t_q1, t_q2, score, t_gs, params)
+    w_a, m_a, v_a = t_table.clone(), torch.zeros_like(t_table), torch.zeros_like(t_table)
+    w_b, m_b, v_b = t_table.clone(), torch.zeros_like(t_table), torch.zeros_like(t_table)
+    fused.score_backward_entity("box", plan, w_a, t_q1, t_q2, score, t_gs, params, m=m_a, v=v_a,
+                                adam=fused.adam_params(1e-3, 1))
+    f1, f2 = fused.score_backward_fused("box", plan, w_b, t_idx, t_q1, t_q2, score, t_gs, params, m=m_b, v=v_b,
+                                        adam=fused.adam_params(1e-3, 1))
+    assert_close(f1.cpu().numpy(), gq1.cpu().numpy(), 1e-6, "gq1")
+    assert_close(f2.cpu().numpy(), gq2.cpu().numpy(), 1e-6, "gq2")
+    assert_close(m_b.cpu().numpy(), m_a.cpu().numpy(), 2e-6, "m")
+    assert_close(v_b.cpu().numpy(), v_a.cpu().numpy(), 2e-6, "v")
+    assert_close(w_b.cpu().numpy(), w_a.cpu().numpy(), 2e-6, "w")
+    merged_a = torch.empty((plan.n_uniq, dim), device="cuda")
+    merged_b = torch.full_like(merged_a, float("nan"))
+    fused.score_backward_entity("box", plan, t_table, t_q1, t_q2, score, t_gs, params, merged=merged_a)
+    fused.score_backward_fused("box", plan, t_table, t_idx, t_q1, t_q2, score, t_gs, params, merged=merged_b)
+    assert_close(merged_b.cpu().numpy(), merged_a.cpu().numpy(), 1e-6, "merged")
