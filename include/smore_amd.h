@@ -150,17 +150,28 @@ typedef struct smx_plan_view {
   size_t n_pairs;
 } smx_plan_view;
 
-/* Lazy Adam of the sparse row optimizer: AdamEmbedOptimizer.update_step
- * (smore/common/embedding/embed_optimizer.py:208-252).  `step` is the global
- * counter after apply_grad incremented it (:156), so the first update has
- * step = 1.  eps is smore/common/consts.py:20 in the reference. */
-typedef struct smx_adam_params {
+/* Row optimizers of smore/common/embedding/embed_optimizer.py, all lazy (touched rows only):
+ *   ADAM    AdamEmbedOptimizer.update_step :208-252 (global step counter, eps = common/consts.py:20)
+ *   SGD     SGDEmbedOptimizer.update_step :174-178
+ *   ADAGRAD AdaGradEmbedOptimizer.update_step :327-349
+ *   RMSPROP RMSpropEmbedOptimizer.update_step :271-309 (its alpha = 0.99 goes in beta2)
+ * `step` is the counter after apply_grad incremented it (:156): the first update has step = 1.
+ * squeeze != 0: the second-moment state v is one float per row ([N] / [N,1]) fed by the row mean of
+ * g*g (optim_mode[3] of the reference, :220-221, :237-238, :336-337).  State tables: ADAM uses m and v,
+ * ADAGRAD / RMSPROP use v only (m may be NULL), SGD none. */
+#define SMX_OPT_ADAM 1
+#define SMX_OPT_SGD 2
+#define SMX_OPT_ADAGRAD 3
+#define SMX_OPT_RMSPROP 4
+typedef struct smx_opt_params {
   double lr;    /* hyper-parameters are doubles, as the Python floats of the reference are: */
   double beta1; /* 1 - beta is formed in double and only then rounded to fp32             */
   double beta2;
   double eps;
   long step;
-} smx_adam_params;
+  int kind;     /* SMX_OPT_* */
+  int squeeze;
+} smx_opt_params;
 
 /* ---- entity-side backward, segment sum and row update in one pass ----------
  * For every distinct id u of the plan: g[u,:] = sum over the pairs of segment u
@@ -168,8 +179,9 @@ typedef struct smx_adam_params {
  * atomics).  Then, as requested:
  *   merged != NULL   merged[u,:] = g[u,:]        ([n_uniq, dim*mul], caller-sized for P rows
  *                                                 or fewer if it knows n_uniq)
- *   m, v, adam given table[id], m[id], v[id] are updated by lazy Adam in place;
- *                    rows of ids not in the plan are not touched.
+ *   adam given       table[id] and the optimizer's state rows m[id], v[id] are updated in place
+ *                    (see smx_opt_params for which state a kind uses); rows of ids not in the
+ *                    plan are not touched.
  * Replaces dist_backward_ent_kernel (common_kernel.h:59-89), EmbedLookupFunc.backward
  * (embed_optimizer.py:63-66), merge_grad_list (:45-48) and update_step (:208-252).
  * workspace: smx_entity_workspace_bytes(P, dim*mul) bytes, 256-byte aligned. */
@@ -178,7 +190,7 @@ int smx_score_backward_entity(int model, void* stream, const smx_plan_view* plan
                               size_t n_rows, const float* q1, const float* q2, const float* score,
                               const float* gscore, size_t B, size_t K, size_t dim,
                               const smx_score_params* params, float* merged, float* m, float* v,
-                              const smx_adam_params* adam, void* workspace, size_t workspace_bytes);
+                              const smx_opt_params* adam, void* workspace, size_t workspace_bytes);
 
 /* Everything after the loss in one call: query gradients, and every entity row of the step finished
  * (merged gradient row and/or lazy Adam on w, m, v), as smx_score_backward_query followed by
@@ -194,7 +206,7 @@ int smx_score_backward_fused(int model, void* stream, const smx_plan_view* plan,
                              size_t n_rows, const int64_t* idx, const float* q1, const float* q2,
                              const float* score, const float* gscore, float* gq1, float* gq2,
                              size_t B, size_t K, size_t dim, const smx_score_params* params,
-                             float* merged, float* m, float* v, const smx_adam_params* adam,
+                             float* merged, float* m, float* v, const smx_opt_params* adam,
                              void* workspace, size_t workspace_bytes);
 
 /* Same pass for gradient rows that already exist in memory (what autograd hands
@@ -203,7 +215,7 @@ int smx_score_backward_fused(int model, void* stream, const smx_plan_view* plan,
  * update_step (:208-252) on `table`. */
 int smx_rows_backward(void* stream, const smx_plan_view* plan, const float* grad_rows,
                       size_t row_len, float* merged, float* table, float* m, float* v,
-                      const smx_adam_params* adam, void* workspace, size_t workspace_bytes);
+                      const smx_opt_params* adam, void* workspace, size_t workspace_bytes);
 
 /* Plain row lookup out[k,:] = table[idx[k],:] (smore/common/embedding/embed_rw.py:74-75, the GPU
  * branch of EmbeddingReadOnly.read) for callers that need the rows themselves. */

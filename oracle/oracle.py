@@ -26,6 +26,8 @@ function is pinned by an independent check in tests/test_oracle_pinning.py:
   adam_rows                 torch.optim.Adam when every row is touched each
                             step; untouched rows bit-identical; hand-computed
                             first step; squeeze variant by closed form
+  sgd / adagrad / rmsprop   torch.optim.SGD / Adagrad / RMSprop(alpha=0.99) when
+                            every row is touched; squeeze variants by closed form
   score / train_step        composition only (gamma - dist, chain rule of sqrt)
 """
 import ctypes
@@ -193,6 +195,30 @@ def adam_rows(w, m, v, uniq, merged, lr, step, beta1=0.9, beta2=0.999, eps=1e-8,
         _p(w), _p(m), _p(v), _p(uniq), _p(merged), _sz(uniq.size), _sz(w.shape[1]),
         ctypes.c_double(lr), ctypes.c_double(beta1), ctypes.c_double(beta2), ctypes.c_double(eps),
         ctypes.c_long(int(step)), ctypes.c_int(1 if squeeze else 0))
+
+
+def sgd_rows(w, uniq, merged, lr):
+    sfx, _ = _sfx(w.dtype)
+    uniq, merged = _c(uniq, np.int64), _c(merged, w.dtype)
+    getattr(lib(), f"orc_sgd_rows_{sfx}")(_p(w), _p(uniq), _p(merged), _sz(uniq.size), _sz(w.shape[1]),
+                                          ctypes.c_double(lr))
+
+
+def adagrad_rows(w, state, uniq, merged, lr, eps=1e-8, squeeze=False):
+    sfx, _ = _sfx(w.dtype)
+    uniq, merged = _c(uniq, np.int64), _c(merged, w.dtype)
+    assert state.flags.c_contiguous and state.dtype == w.dtype
+    getattr(lib(), f"orc_adagrad_rows_{sfx}")(_p(w), _p(state), _p(uniq), _p(merged), _sz(uniq.size), _sz(w.shape[1]),
+                                              ctypes.c_double(lr), ctypes.c_double(eps), ctypes.c_int(int(squeeze)))
+
+
+def rmsprop_rows(w, state, uniq, merged, lr, alpha=0.99, eps=1e-8, squeeze=False):
+    sfx, _ = _sfx(w.dtype)
+    uniq, merged = _c(uniq, np.int64), _c(merged, w.dtype)
+    assert state.flags.c_contiguous and state.dtype == w.dtype
+    getattr(lib(), f"orc_rmsprop_rows_{sfx}")(_p(w), _p(state), _p(uniq), _p(merged), _sz(uniq.size), _sz(w.shape[1]),
+                                              ctypes.c_double(lr), ctypes.c_double(alpha), ctypes.c_double(eps),
+                                              ctypes.c_int(int(squeeze)))
 
 
 # ---- composition: the score of each model and one training step -------------------------------

@@ -57,9 +57,12 @@ class ScoreParams(ctypes.Structure):
     _fields_ = [("gamma", _f), ("cen", _f), ("reg_on", _i), ("reg_add", _f), ("reg_lo", _f), ("reg_hi", _f)]
 
 
-class AdamParams(ctypes.Structure):
-    """smx_adam_params of include/smore_amd.h."""
-    _fields_ = [("lr", _d), ("beta1", _d), ("beta2", _d), ("eps", _d), ("step", _l)]
+OPT_KINDS = {"adam": 1, "sgd": 2, "adagrad": 3, "rmsprop": 4}
+
+
+class OptParams(ctypes.Structure):
+    """smx_opt_params of include/smore_amd.h."""
+    _fields_ = [("lr", _d), ("beta1", _d), ("beta2", _d), ("eps", _d), ("step", _l), ("kind", _i), ("squeeze", _i)]
 
 
 class PlanView(ctypes.Structure):

@@ -83,18 +83,21 @@ static int fill_plan(EntityArgs* A, const smx_plan_view* plan, void* workspace, 
 
 int entity_backward(int model, void* stream, const smx_plan_view* plan, float* table, size_t n_rows, const float* q1,
                     const float* q2, const float* score, const float* gscore, size_t B, size_t K, size_t dim,
-                    const smx_score_params* params, float* merged, float* m, float* v, const smx_adam_params* adam,
+                    const smx_score_params* params, float* merged, float* m, float* v, const smx_opt_params* adam,
                     void* workspace, size_t workspace_bytes, int skip_single);
 
-static int fill_adam(EntityArgs* A, float* m, float* v, const smx_adam_params* adam) {
+static int fill_adam(EntityArgs* A, float* m, float* v, const smx_opt_params* opt) {
   A->adam_on = 0;
+  A->squeeze = 0;
   A->m = m;
   A->v = v;
-  if (m || v || adam) {
-    if (!m || !v || !adam) return fail(SMX_ERR_ARG, "Adam needs m, v and parameters together");
-    if (adam->step < 1) return fail(SMX_ERR_ARG, "Adam step counter starts at 1");
-    A->adam_on = 1;
-    A->a = make_adam_consts(adam);
+  if (opt) {
+    if (const char* msg = check_opt_params(opt, m, v)) return fail(SMX_ERR_ARG, "%s", msg);
+    A->adam_on = opt->kind;
+    A->squeeze = opt->squeeze ? 1 : 0;
+    A->a = make_adam_consts(opt);
+  } else if (m || v) {
+    return fail(SMX_ERR_ARG, "optimizer state given without optimizer parameters");
   }
   return SMX_OK;
 }
@@ -108,7 +111,7 @@ size_t smx_entity_workspace_bytes(size_t n_pairs, size_t row_len) { return smx::
 int smx_score_backward_entity(int model, void* stream, const smx_plan_view* plan, float* table, size_t n_rows,
                               const float* q1, const float* q2, const float* score, const float* gscore, size_t B,
                               size_t K, size_t dim, const smx_score_params* params, float* merged, float* m, float* v,
-                              const smx_adam_params* adam, void* workspace, size_t workspace_bytes) {
+                              const smx_opt_params* adam, void* workspace, size_t workspace_bytes) {
   return smx::entity_backward(model, stream, plan, table, n_rows, q1, q2, score, gscore, B, K, dim, params, merged, m,
                               v, adam, workspace, workspace_bytes, 0);
 }
@@ -119,7 +122,7 @@ namespace smx {
 
 int entity_backward(int model, void* stream, const smx_plan_view* plan, float* table, size_t n_rows, const float* q1,
                     const float* q2, const float* score, const float* gscore, size_t B, size_t K, size_t dim,
-                    const smx_score_params* params, float* merged, float* m, float* v, const smx_adam_params* adam,
+                    const smx_score_params* params, float* merged, float* m, float* v, const smx_opt_params* adam,
                     void* workspace, size_t workspace_bytes, int skip_single) {
   if (model < 0 || model >= mNumModels) return fail(SMX_ERR_KIND, "unknown score model %d", model);
   if (!table || !q1 || !score || !gscore || !params || (model_nq(model) == 2 && !q2))
@@ -127,14 +130,14 @@ int entity_backward(int model, void* stream, const smx_plan_view* plan, float* t
   if (B == 0 || K == 0 || dim == 0 || n_rows == 0) return fail(SMX_ERR_SHAPE, "empty dimension");
   if (params->reg_on && model != mBetaKL)
     return fail(SMX_ERR_ARG, "the entity clamp prologue exists for the beta_kl model only");
-  if (!merged && !m) return fail(SMX_ERR_ARG, "nothing to do: neither merged gradient nor Adam requested");
+  if (!merged && !adam) return fail(SMX_ERR_ARG, "nothing to do: neither merged gradient nor an optimizer requested");
   EntityArgs A{};
   const size_t row_len = dim * model_mul(model);
   if (int rc = fill_plan(&A, plan, workspace, workspace_bytes, row_len)) return rc;
   if (plan->n_pairs != B * K) return fail(SMX_ERR_SHAPE, "plan holds %zu pairs, call has %zu", plan->n_pairs, B * K);
   if (int rc = fill_adam(&A, m, v, adam)) return rc;
   const bool vec4 = dim % 4 == 0 && aligned16(table) && aligned16(q1) && (!q2 || aligned16(q2)) &&
-                    (!merged || aligned16(merged)) && (!m || (aligned16(m) && aligned16(v)));
+                    (!merged || aligned16(merged)) && (!m || aligned16(m)) && (!v || (adam && adam->squeeze) || aligned16(v));
   const int vec = vec4 ? 4 : 1;
   const size_t ncol = dim / vec;
   if (ncol > 512) return fail(SMX_ERR_SHAPE, "dim %zu not supported by the fused path", dim);
@@ -167,17 +170,17 @@ int entity_backward(int model, void* stream, const smx_plan_view* plan, float* t
 extern "C" {
 
 int smx_rows_backward(void* stream, const smx_plan_view* plan, const float* grad_rows, size_t row_len, float* merged,
-                      float* table, float* m, float* v, const smx_adam_params* adam, void* workspace,
+                      float* table, float* m, float* v, const smx_opt_params* adam, void* workspace,
                       size_t workspace_bytes) {
   using namespace smx;
   if (!grad_rows || row_len == 0) return fail(SMX_ERR_ARG, "null gradient rows");
-  if (!merged && !m) return fail(SMX_ERR_ARG, "nothing to do: neither merged gradient nor Adam requested");
+  if (!merged && !adam) return fail(SMX_ERR_ARG, "nothing to do: neither merged gradient nor an optimizer requested");
   EntityArgs A{};
   if (int rc = fill_plan(&A, plan, workspace, workspace_bytes, row_len)) return rc;
   if (int rc = fill_adam(&A, m, v, adam)) return rc;
   if (A.adam_on && !table) return fail(SMX_ERR_ARG, "Adam needs the weight table");
   const bool vec4 = row_len % 4 == 0 && aligned16(grad_rows) && (!merged || aligned16(merged)) &&
-                    (!A.adam_on || (aligned16(table) && aligned16(m) && aligned16(v)));
+                    (!A.adam_on || (aligned16(table) && (!m || aligned16(m)) && (!v || A.squeeze || aligned16(v))));
   const int vec = vec4 ? 4 : 1;
   const size_t ncol = row_len / vec;
   if (ncol > 512) return fail(SMX_ERR_SHAPE, "row length %zu not supported by the fused path", row_len);

@@ -439,10 +439,9 @@ __global__ __launch_bounds__(NW * 64) void entity_fixup_kernel(EntityArgs A) {
     RowRegs<MUL, VEC, NIT> e, m0, v0;
     if (REG || A.adam_on || SRC == mBetaKL)
       load_row<MUL, VEC, NIT>(e, A.table + (size_t)row_id * row_len, half, A.ncol, lane);
-    if (A.adam_on) {
-      load_row<MUL, VEC, NIT>(m0, A.m + (size_t)row_id * row_len, half, A.ncol, lane);
+    if (A.adam_on == kOptAdam) load_row<MUL, VEC, NIT>(m0, A.m + (size_t)row_id * row_len, half, A.ncol, lane);
+    if (A.adam_on && A.adam_on != kOptSgd && !A.squeeze)
       load_row<MUL, VEC, NIT>(v0, A.v + (size_t)row_id * row_len, half, A.ncol, lane);
-    }
     finish_row<SRC, VEC, NIT, REG>(A, lane, row_id, seg, g1, g2, e, m0, v0);
   }
 }

@@ -9,6 +9,7 @@
 
 #include "../../include/smore_amd.h"
 #include "smx_models.h"
+#include "smx_wave.h"
 
 namespace smx {
 
@@ -16,14 +17,24 @@ constexpr int kSrcRows = 100;  // source = materialised gradient rows instead of
 
 __host__ __device__ constexpr int src_mul(int s) { return s == kSrcRows ? 1 : model_mul(s); }
 
+// Row optimizers of smore/common/embedding/embed_optimizer.py (all lazy: touched rows only).
+//   Adam     :208-252   m' = b1 m + (1-b1) g, v' = b2 v + (1-b2) g2, w += -(lr/bc1) m' / (sqrt(v')/sqrt(bc2) + eps)
+//   SGD      :174-178   w += -lr g
+//   AdaGrad  :327-349   v' = v + g2,                w += -lr g / (sqrt(v') + eps)
+//   RMSprop  :271-309   v' = a v + (1-a) g2,        w += -lr g / (sqrt(v') + eps)        (a = beta2 field)
+// g2 = g*g per feature, or with `squeeze` the row mean of g*g, v then being one value per row.
+enum OptKind : int { kOptNone = 0, kOptAdam = SMX_OPT_ADAM, kOptSgd = SMX_OPT_SGD, kOptAdagrad = SMX_OPT_ADAGRAD,
+                     kOptRmsprop = SMX_OPT_RMSPROP };
+
 struct AdamConsts {
   float beta1, beta2, omb1, omb2, eps, step_size, inv_sqrt_bc2;
 };
 
-inline AdamConsts make_adam_consts(const smx_adam_params* a) {
+inline AdamConsts make_adam_consts(const smx_opt_params* a) {
   AdamConsts c;
-  const double bc1 = 1.0 - std::pow(a->beta1, (double)a->step);
-  const double bc2 = 1.0 - std::pow(a->beta2, (double)a->step);
+  const bool adam = a->kind == SMX_OPT_ADAM;
+  const double bc1 = adam ? 1.0 - std::pow(a->beta1, (double)a->step) : 1.0;
+  const double bc2 = adam ? 1.0 - std::pow(a->beta2, (double)a->step) : 1.0;
   c.beta1 = (float)a->beta1;
   c.beta2 = (float)a->beta2;
   c.omb1 = (float)(1.0 - a->beta1);
@@ -34,13 +45,23 @@ inline AdamConsts make_adam_consts(const smx_adam_params* a) {
   return c;
 }
 
+// 0 when the parameters are usable, else a message for the caller
+inline const char* check_opt_params(const smx_opt_params* a, const void* m, const void* v) {
+  if (a->kind < SMX_OPT_ADAM || a->kind > SMX_OPT_RMSPROP) return "unknown optimizer kind";
+  if (a->kind == SMX_OPT_ADAM && a->step < 1) return "Adam step counter starts at 1";
+  if (a->kind == SMX_OPT_ADAM && !m) return "Adam needs the first-moment table m";
+  if (a->kind != SMX_OPT_SGD && !v) return "this optimizer needs the state table v";
+  return nullptr;
+}
+
 // Where finished rows go.
 struct RowSink {
-  float* table;   // entity table: read for the model sources, updated when adam_on
-  float* m;
-  float* v;
+  float* table;   // entity table: read for the model sources, updated when an optimizer is on
+  float* m;       // Adam first moment [N, row]
+  float* v;       // second moment / squared-gradient state: [N, row], or [N] with squeeze
   float* merged;  // [U, row_len] or null
-  int adam_on;
+  int adam_on;    // OptKind; 0 = no optimizer (name kept from the Adam-only version)
+  int squeeze;
   AdamConsts a;
   ScoreParams p;
   int ncol;       // columns per half row (model sources) or per row (gradient rows)
@@ -134,9 +155,23 @@ __device__ __forceinline__ void finish_row(const RowSink& A, int lane, unsigned 
     }
   }
   if (ADAM_STATIC || A.adam_on) {
+    const int kind = A.adam_on;
     float* pw = A.table + (size_t)row_id * row_len;
     float* pm = A.m + (size_t)row_id * row_len;
     float* pv = A.v + (size_t)row_id * row_len;
+    float g2_row = 0.f, v_row = 0.f;
+    if (A.squeeze && kind != kOptSgd) {  // one second-moment value per row, fed by the row mean of g*g
+      float part = 0.f;
+#pragma unroll
+      for (int it = 0; it < NIT; ++it)
+        if (lane + 64 * it < A.ncol) {
+#pragma unroll
+          for (int x = 0; x < VEC; ++x) part += g1[it][x] * g1[it][x] + (MUL == 2 ? g2[it][x] * g2[it][x] : 0.f);
+        }
+      g2_row = wave_sum_f32(part) / (float)row_len;
+      v_row = A.v[row_id];
+    }
+    float v_new_row = 0.f;
 #pragma unroll
     for (int h = 0; h < MUL; ++h) {
 #pragma unroll
@@ -147,17 +182,29 @@ __device__ __forceinline__ void finish_row(const RowSink& A, int lane, unsigned 
 #pragma unroll
           for (int x = 0; x < VEC; ++x) {
             const float g = h == 0 ? g1[it][x] : g2[it][x];
-            mn[x] = m0.h[h][it].v[x] * A.a.beta1 + g * A.a.omb1;
-            vn[x] = v0.h[h][it].v[x] * A.a.beta2 + g * g * A.a.omb2;
-            const float denom = sqrtf(vn[x]) * A.a.inv_sqrt_bc2 + A.a.eps;
-            wn[x] = w.h[h][it].v[x] + A.a.step_size * mn[x] / denom;
+            const float gg = A.squeeze ? g2_row : g * g;
+            const float v_old = A.squeeze ? v_row : v0.h[h][it].v[x];
+            if (kind == kOptAdam) {
+              mn[x] = m0.h[h][it].v[x] * A.a.beta1 + g * A.a.omb1;
+              vn[x] = v_old * A.a.beta2 + gg * A.a.omb2;
+              wn[x] = w.h[h][it].v[x] + A.a.step_size * mn[x] / (sqrtf(vn[x]) * A.a.inv_sqrt_bc2 + A.a.eps);
+            } else if (kind == kOptSgd) {
+              mn[x] = vn[x] = 0.f;
+              wn[x] = w.h[h][it].v[x] + A.a.step_size * g;
+            } else {
+              mn[x] = 0.f;
+              vn[x] = kind == kOptAdagrad ? v_old + gg : v_old * A.a.beta2 + gg * A.a.omb2;
+              wn[x] = w.h[h][it].v[x] + A.a.step_size * g / (sqrtf(vn[x]) + A.a.eps);
+            }
+            v_new_row = vn[x];
           }
           st<VEC>(pw + h * half, c, wn);
-          st<VEC>(pm + h * half, c, mn);
-          st<VEC>(pv + h * half, c, vn);
+          if (kind == kOptAdam) st<VEC>(pm + h * half, c, mn);
+          if (kind != kOptSgd && !A.squeeze) st<VEC>(pv + h * half, c, vn);
         }
       }
     }
+    if (A.squeeze && kind != kOptSgd && lane == 0) A.v[row_id] = v_new_row;
   }
 }
 
@@ -172,10 +219,8 @@ __device__ __forceinline__ void request_state(const RowSink& A, int lane, unsign
   const int half = A.ncol * VEC;
   const size_t off = (size_t)row_id * half * MUL;
   if (SRC != kSrcRows || A.adam_on) load_row<MUL, VEC, NIT>(s.e, A.table + off, half, A.ncol, lane);
-  if (A.adam_on) {
-    load_row<MUL, VEC, NIT>(s.m, A.m + off, half, A.ncol, lane);
-    load_row<MUL, VEC, NIT>(s.v, A.v + off, half, A.ncol, lane);
-  }
+  if (A.adam_on == kOptAdam) load_row<MUL, VEC, NIT>(s.m, A.m + off, half, A.ncol, lane);
+  if (A.adam_on && A.adam_on != kOptSgd && !A.squeeze) load_row<MUL, VEC, NIT>(s.v, A.v + off, half, A.ncol, lane);
 }
 
 }  // namespace smx

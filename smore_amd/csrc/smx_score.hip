@@ -29,7 +29,7 @@ extern template int score_dispatch<mBetaKL>(hipStream_t, const ScoreArgs&, int, 
 // defined in smx_entity.hip
 int entity_backward(int model, void* stream, const smx_plan_view* plan, float* table, size_t n_rows, const float* q1,
                     const float* q2, const float* score, const float* gscore, size_t B, size_t K, size_t dim,
-                    const smx_score_params* params, float* merged, float* m, float* v, const smx_adam_params* adam,
+                    const smx_score_params* params, float* merged, float* m, float* v, const smx_opt_params* adam,
                     void* workspace, size_t workspace_bytes, int skip_single);
 
 static int dispatch_model(int model, hipStream_t st, const ScoreArgs& A, int vec, int nit, bool forward) {
@@ -112,19 +112,21 @@ int smx_score_backward_fused(int model, void* stream, const smx_plan_view* plan,
                              const int64_t* idx, const float* q1, const float* q2, const float* score,
                              const float* gscore, float* gq1, float* gq2, size_t B, size_t K, size_t dim,
                              const smx_score_params* params, float* merged, float* m, float* v,
-                             const smx_adam_params* adam, void* workspace, size_t workspace_bytes) {
+                             const smx_opt_params* adam, void* workspace, size_t workspace_bytes) {
   using namespace smx;
   ScoreArgs A;
   int vec, nit;
   if (!idx) return fail(SMX_ERR_ARG, "the fused backward needs the id tensor");
   if (!plan || !plan->pair_seg) return fail(SMX_ERR_ARG, "the fused backward needs a plan built with pair_seg");
   if (plan->n_pairs != B * K) return fail(SMX_ERR_SHAPE, "plan holds %zu pairs, call has %zu", plan->n_pairs, B * K);
-  if (!merged && !m) return fail(SMX_ERR_ARG, "nothing to do: neither merged gradient nor Adam requested");
-  if ((m || v || adam) && !(m && v && adam)) return fail(SMX_ERR_ARG, "Adam needs m, v and parameters together");
-  if (adam && adam->step < 1) return fail(SMX_ERR_ARG, "Adam step counter starts at 1");
+  if (!merged && !adam) return fail(SMX_ERR_ARG, "nothing to do: neither merged gradient nor an optimizer requested");
+  if (!adam && (m || v)) return fail(SMX_ERR_ARG, "optimizer state given without optimizer parameters");
+  if (adam)
+    if (const char* msg = check_opt_params(adam, m, v)) return fail(SMX_ERR_ARG, "%s", msg);
   // the same column width must suit the query-backward kernel and the entity pass
   if (int rc = fill_args(&A, &vec, &nit, model, table, n_rows, idx, q1, q2, B, K, dim, params, merged, m)) return rc;
-  if (vec == 4 && v && !aligned16(v)) return fail(SMX_ERR_ARG, "v must be 16-byte aligned like m");
+  if (vec == 4 && v && !(adam && adam->squeeze) && !aligned16(v))
+    return fail(SMX_ERR_ARG, "v must be 16-byte aligned like the table");
   if (!score || !gscore || !gq1 || (model_nq(model) == 2 && !gq2)) return fail(SMX_ERR_ARG, "null pointer");
   A.score = score;
   A.gscore = gscore;
@@ -140,7 +142,8 @@ int smx_score_backward_fused(int model, void* stream, const smx_plan_view* plan,
   A.sink.m = m;
   A.sink.v = v;
   A.sink.merged = merged;
-  A.sink.adam_on = adam ? 1 : 0;
+  A.sink.adam_on = adam ? adam->kind : 0;
+  A.sink.squeeze = (adam && adam->squeeze) ? 1 : 0;
   if (adam) A.sink.a = make_adam_consts(adam);
   A.sink.p = A.p;
   A.sink.ncol = A.ncol;

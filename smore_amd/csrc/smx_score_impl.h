@@ -296,8 +296,8 @@ __global__ __launch_bounds__(NW * 64) void score_backward_query_kernel(ScoreArgs
         RowRegs<MUL, VEC, NIT> e, m0, v0;
         load_row<MUL, VEC, NIT>(e, table + off, dim, ncol, lane);
         if constexpr (SINGLES == 2) {
-          load_row<MUL, VEC, NIT>(m0, A.sink.m + off, dim, ncol, lane);
-          load_row<MUL, VEC, NIT>(v0, A.sink.v + off, dim, ncol, lane);
+          if (A.sink.adam_on == kOptAdam) load_row<MUL, VEC, NIT>(m0, A.sink.m + off, dim, ncol, lane);
+          if (A.sink.adam_on != kOptSgd && !A.sink.squeeze) load_row<MUL, VEC, NIT>(v0, A.sink.v + off, dim, ncol, lane);
         }
         const float c0 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(my_c0), j));
         const float c1 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(my_c1), j));

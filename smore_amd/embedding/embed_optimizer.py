@@ -187,40 +187,71 @@ class EmbeddingOptimizer(ABC):
             self.update_from_plan(plan, torch.cat(grad_list, dim=0).contiguous(), lr)
 
 
-class AdamEmbedOptimizer(EmbeddingOptimizer):
-    """Lazy Adam with one global step counter (embed_optimizer.py:188-252).  State buffers carry the
-    reference's names, state_sum_fo / state_sum_sq, on the SparseEmbedding, so they are part of its
-    state_dict like there."""
-    beta1, beta2, eps = 0.9, 0.999, 1e-8  # embed_optimizer.py:209-210, consts.py:20
+class _RowOptimizer(EmbeddingOptimizer):
+    """Shared body of the concrete optimizers: state buffers live on the SparseEmbedding under the
+    reference's names (so they are part of its state_dict, embed_optimizer.py:190-197, 257-262,
+    314-320) and every update is one fused pass over the plan."""
+    kind = None            # key of fused.opt_params
+    first_moment = None    # buffer name of the [N,row] first moment (Adam only)
+    second_moment = None   # buffer name of the squared-gradient state, [N,row] or [N,1] with squeeze
+    eps = 1e-8             # common/consts.py:20
 
     def prepare_state(self):
         emb = self.sparse_embed
-        if self.squeeze:
-            raise NotImplementedError("squeezed second moment ([N,1]) is not built yet")
-        for name in ("state_sum_fo", "state_sum_sq"):
-            if not hasattr(emb, name):
-                emb.register_tensor(name, torch.zeros_like(emb.embedding.detach()))
+        table = emb.embedding.detach()
+        if self.first_moment and not hasattr(emb, self.first_moment):
+            emb.register_tensor(self.first_moment, torch.zeros_like(table))
+        if self.second_moment and not hasattr(emb, self.second_moment):
+            shape = (table.shape[0], 1) if self.squeeze else tuple(table.shape)
+            emb.register_tensor(self.second_moment, torch.zeros(shape, dtype=table.dtype, device=table.device))
 
-    def _adam(self, lr):
-        return fused.adam_params(lr, self.step, self.beta1, self.beta2, self.eps)
+    def _state(self):
+        emb = self.sparse_embed
+        m = getattr(emb, self.first_moment) if self.first_moment else None
+        v = getattr(emb, self.second_moment) if self.second_moment else None
+        return m, v
+
+    def _params(self, lr):
+        return fused.opt_params(self.kind, lr, step=self.step, squeeze=self.squeeze, eps=self.eps)
 
     def update_from_plan(self, plan, grad_rows, lr):
-        emb = self.sparse_embed
-        fused.rows_backward(plan, grad_rows, table=emb.embedding.detach(), m=emb.state_sum_fo, v=emb.state_sum_sq,
-                            adam=self._adam(lr))
+        m, v = self._state()
+        fused.rows_backward(plan, grad_rows, table=self.sparse_embed.embedding.detach(), m=m, v=v,
+                            adam=self._params(lr))
 
     def update_fused(self, plan, rec, lr):
-        emb = self.sparse_embed
-        fused.score_backward_entity(rec["model"], plan, emb.embedding.detach(), rec["q1"], rec["q2"], rec["score"],
-                                    rec["gscore"], rec["params"], m=emb.state_sum_fo, v=emb.state_sum_sq,
-                                    adam=self._adam(lr))
+        m, v = self._state()
+        fused.score_backward_entity(rec["model"], plan, self.sparse_embed.embedding.detach(), rec["q1"], rec["q2"],
+                                    rec["score"], rec["gscore"], rec["params"], m=m, v=v, adam=self._params(lr))
+
+
+class AdamEmbedOptimizer(_RowOptimizer):
+    """Lazy Adam with one global step counter, betas (0.9, 0.999) (embed_optimizer.py:188-252)."""
+    kind, first_moment, second_moment = "adam", "state_sum_fo", "state_sum_sq"
+
+
+class SGDEmbedOptimizer(_RowOptimizer):
+    """embed_optimizer.py:166-178."""
+    kind = "sgd"
+
+
+class AdaGradEmbedOptimizer(_RowOptimizer):
+    """embed_optimizer.py:312-349."""
+    kind, second_moment = "adagrad", "state_sum"
+
+
+class RMSpropEmbedOptimizer(_RowOptimizer):
+    """embed_optimizer.py:255-309 (alpha = 0.99)."""
+    kind, second_moment = "rmsprop", "state_sum"
 
 
 def get_optim_class(args):
-    """embed_optimizer.py:352-364; only Adam is built so far."""
+    """embed_optimizer.py:352-364."""
     mode = args.optim_mode
     if isinstance(mode, str):
         mode = tuple(x.strip() for x in mode.strip("()").split(","))
-    if mode[1] == "adam":
-        return AdamEmbedOptimizer
-    raise NotImplementedError(f"sparse optimizer '{mode[1]}' is not built yet")
+    classes = {"adam": AdamEmbedOptimizer, "rmsprop": RMSpropEmbedOptimizer, "adagrad": AdaGradEmbedOptimizer,
+               "sgd": SGDEmbedOptimizer}
+    if mode[1] not in classes:
+        raise NotImplementedError(mode[1])
+    return classes[mode[1]]

@@ -165,8 +165,26 @@ def build_plan(idx, n_rows, want_inverse=False, err_flag=None):
     return plan
 
 
-def adam_params(lr, step, beta1=0.9, beta2=0.999, eps=1e-8):
-    return _lib.AdamParams(lr, beta1, beta2, eps, int(step))
+def adam_params(lr, step, beta1=0.9, beta2=0.999, eps=1e-8, squeeze=False):
+    return _lib.OptParams(lr, beta1, beta2, eps, int(step), _lib.OPT_KINDS["adam"], int(bool(squeeze)))
+
+
+def opt_params(kind, lr, step=1, squeeze=False, eps=1e-8, alpha=0.99):
+    """Parameters of a row optimizer: kind in {adam, sgd, adagrad, rmsprop} (see smx_opt_params)."""
+    if kind == "adam":
+        return adam_params(lr, step, eps=eps, squeeze=squeeze)
+    if kind not in _lib.OPT_KINDS:
+        raise _lib.SmxError(f"unknown optimizer {kind}")
+    return _lib.OptParams(lr, 0.0, alpha, eps, int(step), _lib.OPT_KINDS[kind], int(bool(squeeze)))
+
+
+def _check_state(table, m, v, opt):
+    if m is not None and m.shape != table.shape:
+        raise _lib.SmxError("the first-moment table must have the entity table's shape")
+    if v is not None:
+        want = table.shape[0] if (opt is not None and opt.squeeze) else table.numel()
+        if v.numel() != want:
+            raise _lib.SmxError("the second-moment table must be [N, row], or [N] / [N,1] with squeeze")
 
 
 def score_backward_entity(model, plan, table, q1, q2, score, gscore, params, merged=None, m=None, v=None, adam=None):
@@ -180,9 +198,7 @@ def score_backward_entity(model, plan, table, q1, q2, score, gscore, params, mer
                     (merged, "merged"), (m, "m"), (v, "v")):
         _f32(t, name)
     row_len = table.shape[1]
-    for s in (m, v):
-        if s is not None and s.shape != table.shape:
-            raise _lib.SmxError("Adam state must have the table's shape")
+    _check_state(table, m, v, adam)
     if merged is not None and (merged.dim() != 2 or merged.shape[1] != row_len):
         raise _lib.SmxError("merged must be [n_uniq or more, row]")
     with torch.cuda.device(table.device):
@@ -202,9 +218,7 @@ def score_backward_fused(model, plan, table, idx, q1, q2, score, gscore, params,
         _f32(t, name)
     if plan.n_pairs != b * k:
         raise _lib.SmxError("plan does not belong to these ids")
-    for s in (m, v):
-        if s is not None and s.shape != table.shape:
-            raise _lib.SmxError("Adam state must have the table's shape")
+    _check_state(table, m, v, adam)
     if merged is not None and (merged.dim() != 2 or merged.shape[1] != table.shape[1]):
         raise _lib.SmxError("merged must be [n_uniq or more, row]")
     gq1 = torch.empty_like(q1)
@@ -226,6 +240,8 @@ def rows_backward(plan, grad_rows, merged=None, table=None, m=None, v=None, adam
     if grad_rows.dim() != 2 or grad_rows.shape[0] != plan.n_pairs:
         raise _lib.SmxError("grad_rows must be [P, row]")
     row_len = grad_rows.shape[1]
+    if table is not None:
+        _check_state(table, m, v, adam)
     with torch.cuda.device(grad_rows.device):
         ws = _workspace(_lib.load().smx_entity_workspace_bytes(plan.n_pairs, row_len), grad_rows.device)
         view = plan.view()

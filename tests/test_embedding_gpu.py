@@ -163,3 +163,46 @@ def test_state_buffers_are_in_the_state_dict():
     emb, _ = _setup(20, 8, 11)
     sd = emb.state_dict()
     assert {"embedding", "state_sum_fo", "state_sum_sq"} <= set(sd)
+
+
+@pytest.mark.parametrize("name", ["adam", "sgd", "adagrad", "rmsprop"])
+@pytest.mark.parametrize("squeeze", [False, True])
+def test_row_optimizers_match_oracle(name, squeeze):
+    """Every optimizer of the reference (and its squeezed second moment), three steps of plain lookups."""
+    from smore_amd.embedding import embed_optimizer as eo
+    from smore_amd.embedding.sparse_embed import SparseEmbedding
+    torch.manual_seed(3)
+    n, d, lr = 120, 24, 1e-2
+    emb = SparseEmbedding(n, d).cuda()
+    emb.init_params(-0.5, 0.5)
+    args = types.SimpleNamespace(optim_mode=f"(aggr,{name},gpu,{squeeze},5)", share_optim_stats=True)
+    opt = eo.get_optim_class(args)(args, emb, 0)
+    assert opt.squeeze == squeeze
+    w = emb.embedding.detach().cpu().numpy().astype(np.float64)
+    m = np.zeros_like(w)
+    v = np.zeros((n, 1)) if squeeze else np.zeros_like(w)
+    rng = np.random.default_rng(4)
+    for step in range(1, 4):
+        ids = rng.integers(0, n, 80)
+        coef = rng.standard_normal((80, d))
+        opt.zero_grad()
+        rows = emb(torch.tensor(ids, device="cuda"), "x")
+        (rows * torch.tensor(coef, dtype=torch.float32, device="cuda")).sum().backward()
+        opt.apply_grad(lr)
+        uniq, inverse, _, _ = orc.merge_indices(ids)
+        merged = orc.merge_grads(coef.astype(np.float32).astype(np.float64), inverse, uniq.size)
+        if name == "adam":
+            orc.adam_rows(w, m, v, uniq, merged, lr, step, squeeze=squeeze)
+        elif name == "sgd":
+            orc.sgd_rows(w, uniq, merged, lr)
+        elif name == "adagrad":
+            orc.adagrad_rows(w, v, uniq, merged, lr, squeeze=squeeze)
+        else:
+            orc.rmsprop_rows(w, v, uniq, merged, lr, squeeze=squeeze)
+    assert_close(emb.embedding.detach().cpu().numpy(), w, 2e-5, f"{name} weights")
+    if name != "sgd":
+        state = emb.state_sum_sq if name == "adam" else emb.state_sum
+        assert state.shape == ((n, 1) if squeeze else (n, d))
+        assert_close(state.cpu().numpy(), v, 2e-5, f"{name} second moment")
+    if name == "adam":
+        assert_close(emb.state_sum_fo.cpu().numpy(), m, 2e-5, "adam first moment")

@@ -318,3 +318,53 @@ def test_one_call_backward_with_many_queries_takes_the_one_pair_shortcut():
     fused.score_backward_entity("box", plan, t_table, t_q1, t_q2, score, t_gs, params, merged=merged_a)
     fused.score_backward_fused("box", plan, t_table, t_idx, t_q1, t_q2, score, t_gs, params, merged=merged_b)
     assert_close(merged_b.cpu().numpy(), merged_a.cpu().numpy(), 1e-6, "merged")
+
+
+@pytest.mark.parametrize("kind", ["adam", "sgd", "adagrad", "rmsprop"])
+@pytest.mark.parametrize("squeeze", [False, True])
+def test_fused_entity_pass_with_every_optimizer(kind, squeeze):
+    """Gather-fused entity backward + row update for each optimizer kind, long and short segments,
+    both through the entity pass alone and through the one-call backward."""
+    from smore_amd import fused
+    rng = np.random.default_rng(21)
+    n, b, k, dim, lr = 600, 24, 128, 48, 1e-2
+    table, q1, q2, idx, gs = make_problem("box", n, b, k, dim, rng, zipf=1.2)
+    t_q1, t_q2, t_gs = dev(q1), dev(q2), dev(gs)
+    t_idx = torch.tensor(idx, device="cuda")
+    params = fused.score_params(24.0, 0.02)
+    plan = fused.build_plan(t_idx, n, want_inverse=True)
+    uniq, inverse, _, _ = orc.merge_indices(idx)
+    for one_call in (False, True):
+        t_w = dev(table)
+        t_m = torch.zeros_like(t_w) if kind == "adam" else None
+        t_v = None if kind == "sgd" else (torch.zeros((n, 1), device="cuda") if squeeze else torch.zeros_like(t_w))
+        w, m = table.copy(), np.zeros_like(table)
+        v = np.zeros((n, 1)) if squeeze else np.zeros_like(table)
+        for step in (1, 2):
+            score = fused.score_forward("box", t_w, t_idx, t_q1, t_q2, params)
+            merged = torch.empty((uniq.size, dim), device="cuda")
+            fused.score_backward_entity("box", plan, t_w, t_q1, t_q2, score, t_gs, params, merged=merged)
+            g = merged.cpu().numpy().astype(np.float64)  # the device's own merged gradient isolates the update rule
+            w_s, m_s, v_s = t_w.cpu().numpy().astype(np.float64), None, None
+            if t_m is not None:
+                m_s = t_m.cpu().numpy().astype(np.float64)
+            if t_v is not None:
+                v_s = t_v.cpu().numpy().astype(np.float64)
+            if kind == "adam":
+                orc.adam_rows(w_s, m_s, v_s, uniq, g, lr, step, squeeze=squeeze)
+            elif kind == "sgd":
+                orc.sgd_rows(w_s, uniq, g, lr)
+            elif kind == "adagrad":
+                orc.adagrad_rows(w_s, v_s, uniq, g, lr, squeeze=squeeze)
+            else:
+                orc.rmsprop_rows(w_s, v_s, uniq, g, lr, squeeze=squeeze)
+            op = fused.opt_params(kind, lr, step=step, squeeze=squeeze)
+            if one_call:
+                fused.score_backward_fused("box", plan, t_w, t_idx, t_q1, t_q2, score, t_gs, params, m=t_m, v=t_v, adam=op)
+            else:
+                fused.score_backward_entity("box", plan, t_w, t_q1, t_q2, score, t_gs, params, m=t_m, v=t_v, adam=op)
+            assert_close(t_w.cpu().numpy(), w_s, REL_F32, f"{kind} w step {step}")
+            if t_v is not None:
+                assert_close(t_v.cpu().numpy(), v_s, REL_F32, f"{kind} v step {step}")
+            if t_m is not None:
+                assert_close(t_m.cpu().numpy(), m_s, REL_F32, f"{kind} m step {step}")

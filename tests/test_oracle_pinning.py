@@ -357,6 +357,46 @@ def test_adam_squeeze_variant_closed_form():
     assert np.allclose(w[4], want, rtol=1e-13)
 
 
+@pytest.mark.parametrize("name", ["sgd", "adagrad", "rmsprop"])
+def test_other_row_optimizers_equal_torch_when_every_row_is_touched(name):
+    n, d, lr = 9, 5, 1e-2
+    w0 = RNG.standard_normal((n, d))
+    w, state = w0.copy(), np.zeros((n, d))
+    tw = torch.tensor(w0.copy(), requires_grad=True)
+    opt = {"sgd": lambda: torch.optim.SGD([tw], lr=lr),
+           "adagrad": lambda: torch.optim.Adagrad([tw], lr=lr, eps=1e-8),
+           "rmsprop": lambda: torch.optim.RMSprop([tw], lr=lr, alpha=0.99, eps=1e-8)}[name]()
+    for _ in range(4):
+        g = RNG.standard_normal((n, d))
+        if name == "sgd":
+            orc.sgd_rows(w, np.arange(n), g, lr)
+        elif name == "adagrad":
+            orc.adagrad_rows(w, state, np.arange(n), g, lr)
+        else:
+            orc.rmsprop_rows(w, state, np.arange(n), g, lr)
+        tw.grad = torch.tensor(g)
+        opt.step()
+        assert np.allclose(w, tw.detach().numpy(), rtol=1e-12, atol=1e-12)
+
+
+def test_other_row_optimizers_are_lazy_and_squeeze_by_closed_form():
+    n, d, lr = 7, 6, 1e-2
+    w0 = RNG.standard_normal((n, d))
+    g = RNG.standard_normal((2, d))
+    rows = np.array([1, 4])
+    gm = (g * g).mean(1, keepdims=True)
+    w, st = w0.copy(), np.full((n, 1), 0.5)
+    orc.adagrad_rows(w, st, rows, g, lr, squeeze=True)
+    assert np.allclose(st[rows], 0.5 + gm, rtol=1e-14) and np.all(st[[0, 2, 3, 5, 6]] == 0.5)
+    assert np.allclose(w[rows], w0[rows] - lr * g / (np.sqrt(0.5 + gm) + 1e-8), rtol=1e-13)
+    assert np.array_equal(w[[0, 2, 3, 5, 6]], w0[[0, 2, 3, 5, 6]])
+    w, st = w0.copy(), np.full((n, 1), 0.5)
+    orc.rmsprop_rows(w, st, rows, g, lr, squeeze=True)
+    s1 = 0.99 * 0.5 + 0.01 * gm
+    assert np.allclose(st[rows], s1, rtol=1e-14)
+    assert np.allclose(w[rows], w0[rows] - lr * g / (np.sqrt(s1) + 1e-8), rtol=1e-13)
+
+
 # ---------------------------------------------------------------- composition
 
 def test_scores_match_native_cal_logit_forms():
