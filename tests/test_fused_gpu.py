@@ -368,3 +368,56 @@ def test_fused_entity_pass_with_every_optimizer(kind, squeeze):
                 assert_close(t_v.cpu().numpy(), v_s, REL_F32, f"{kind} v step {step}")
             if t_m is not None:
                 assert_close(t_m.cpu().numpy(), m_s, REL_F32, f"{kind} m step {step}")
+
+
+@pytest.mark.parametrize("shape", [
+    (7, 1, 1, 4),        # a single pair
+    (50, 9, 1, 16),      # K = 1: the positives layout [B,1]
+    (50, 1, 333, 16),    # one query, ragged K
+    (1, 5, 70, 8),       # a table of one row: one segment holds every pair
+    (100000, 3, 65, 4),  # every id distinct with high probability: only one-pair segments
+    (64, 2, 3, 2048),    # the widest row the fused path takes (8 float4 columns per lane)
+    (64, 2, 3, 252),     # widest unaligned-friendly scalar row is 256; 252 is float4-aligned
+    (30, 2, 5, 255),     # scalar columns, four per lane
+])
+def test_fused_edge_shapes(shape):
+    n, b, k, dim = shape
+    run_case("box", n, b, k, dim, adam_steps=1)
+    run_case("l2", n, b, k, dim, adam_steps=1)
+
+
+def test_one_giant_segment_and_all_long_segments():
+    """Every pair hits one of three ids: nothing but long segments, many tiles each."""
+    from smore_amd import fused
+    rng = np.random.default_rng(31)
+    n, b, k, dim = 3, 40, 500, 32
+    table, q1, q2, idx, gs = make_problem("rotate", n, b, k, dim, rng)
+    t_table, t_q1, t_q2, t_gs = dev(table), dev(q1), dev(q2), dev(gs)
+    t_idx = torch.tensor(idx, device="cuda")
+    params = fused.score_params(9.0)
+    plan = fused.build_plan(t_idx, n, want_inverse=True)
+    assert plan.n_uniq == 3
+    score = fused.score_forward("rotate", t_table, t_idx, t_q1, t_q2, params)
+    merged = torch.empty((3, 2 * dim), device="cuda")
+    fused.score_backward_entity("rotate", plan, t_table, t_q1, t_q2, score, t_gs, params, merged=merged)
+    rows = orc.gather(table, idx).reshape(b, k, -1)
+    g_rows, _, _ = orc.score_backward("rotate", gs, rows, q1[:, None], q2[:, None])
+    uniq, inverse, _, _ = orc.merge_indices(idx)
+    want = orc.merge_grads(g_rows.reshape(b * k, -1), inverse, 3)
+    sum_abs = orc.merge_grads(np.abs(g_rows).reshape(b * k, -1), inverse, 3)
+    assert_close(merged.cpu().numpy(), want, REL_F32, "giant segments", sum_abs=sum_abs)
+
+
+def test_unsupported_rows_are_refused_not_mangled():
+    from smore_amd import _lib, fused
+    idx = torch.zeros(2, 3, dtype=torch.int64, device="cuda")
+    for dim in (2052, 257):  # too wide for float4 columns / for scalar columns
+        t = torch.zeros(10, dim, device="cuda")
+        q = torch.zeros(2, dim, device="cuda")
+        with pytest.raises(_lib.SmxError):
+            fused.score_forward("l1", t, idx, q, None, fused.score_params(1.0))
+    with pytest.raises(_lib.SmxError):  # regulariser prologue is a BetaE feature
+        fused.score_forward("l1", torch.zeros(10, 8, device="cuda"), idx, torch.zeros(2, 8, device="cuda"), None,
+                            fused.score_params(1.0, regularizer=(1.0, 0.05, 1e9)))
+    with pytest.raises(_lib.SmxError):  # empty batch
+        fused.build_plan(torch.zeros(0, dtype=torch.int64, device="cuda"), 10)
