@@ -186,8 +186,8 @@ __device__ __forceinline__ void store_partial(const EntityArgs& A, float* buf, i
   for (int it = 0; it < NIT; ++it) {
     const int c = lane + 64 * it;
     if (c < A.ncol) {
-      st<VEC>(out, c, g1[it]);
-      if (MUL == 2) st<VEC>(out + half, c, g2[it]);
+      st<VEC, true>(out, c, g1[it]);
+      if (MUL == 2) st<VEC, true>(out + half, c, g2[it]);
     }
   }
 }
@@ -392,7 +392,7 @@ __global__ __launch_bounds__(NW * 64) void entity_fixup_kernel(EntityArgs A) {
 #pragma unroll
     for (int k = 0; k < ILP; ++k) {
       const int tj = ts + min(j + k, j1 - 1);
-      load_row<MUL, VEC, NIT>(r[k], (tj < t ? A.tail : A.head) + (size_t)tj * row_len, half, A.ncol, lane);
+      load_row<MUL, VEC, NIT, true>(r[k], (tj < t ? A.tail : A.head) + (size_t)tj * row_len, half, A.ncol, lane);
     }
 #pragma unroll
     for (int k = 0; k < ILP; ++k) {
@@ -438,10 +438,10 @@ __global__ __launch_bounds__(NW * 64) void entity_fixup_kernel(EntityArgs A) {
     const unsigned row_id = (unsigned)A.sorted_ids[p0];
     RowRegs<MUL, VEC, NIT> e, m0, v0;
     if (REG || A.adam_on || SRC == mBetaKL)
-      load_row<MUL, VEC, NIT>(e, A.table + (size_t)row_id * row_len, half, A.ncol, lane);
-    if (A.adam_on == kOptAdam) load_row<MUL, VEC, NIT>(m0, A.m + (size_t)row_id * row_len, half, A.ncol, lane);
+      load_row<MUL, VEC, NIT, true>(e, A.table + (size_t)row_id * row_len, half, A.ncol, lane);
+    if (A.adam_on == kOptAdam) load_row<MUL, VEC, NIT, true>(m0, A.m + (size_t)row_id * row_len, half, A.ncol, lane);
     if (A.adam_on && A.adam_on != kOptSgd && !A.squeeze)
-      load_row<MUL, VEC, NIT>(v0, A.v + (size_t)row_id * row_len, half, A.ncol, lane);
+      load_row<MUL, VEC, NIT, true>(v0, A.v + (size_t)row_id * row_len, half, A.ncol, lane);
     finish_row<SRC, VEC, NIT, REG>(A, lane, row_id, seg, g1, g2, e, m0, v0);
   }
 }

@@ -120,9 +120,17 @@ template <> struct ModelOps<mL2> {
 template <> struct ModelOps<mBox> {
   using Q = QPair;  // a = center, b = offset
   static __device__ __forceinline__ Q prep(float q1, float q2) { return {q1, q2}; }
+  // min(|d|, o) as the one hardware instruction (fminf semantics for NaN); the compiler's own fminf
+  // re-canonicalises the loop-invariant offset for every row
+  static __device__ __forceinline__ float min_abs(float d, float o) {
+    float mn;
+    asm("v_min_f32_e64 %0, |%1|, %2" : "=v"(mn) : "v"(d), "v"(o));
+    return mn;
+  }
   static __device__ __forceinline__ void fwd(float e1, float, const Q& q, float& a0, float& a1) {
-    const float a = fabsf(e1 - q.a);
-    const float mn = fminf(a, q.b);
+    const float d = e1 - q.a;
+    const float a = fabsf(d);
+    const float mn = min_abs(d, q.b);
     a0 += a - mn;
     a1 += fabsf(mn);
   }
@@ -133,12 +141,15 @@ template <> struct ModelOps<mBox> {
     c1 = -p.cen * g;
   }
   // gradient of the entity feature; the center's is its negative
+  // Written as three selects on three compares: that is what the hardware does in one instruction each
+  // (v_cmp + v_cndmask with a sign modifier).  |d| >= o decides the same as |d| - o >= 0 for finite
+  // operands (a difference of two distinct floats never rounds to zero).
   static __device__ __forceinline__ float de(float c0, float c1, float e1, const Q& q, bool& outside) {
     const float d = e1 - q.a;
-    outside = fabsf(d) - q.b >= 0.f;
-    const float w = outside ? c0 : c1;
-    const bool positive = outside ? (d > 0.f) : (d >= 0.f);
-    return positive ? w : -w;
+    outside = fabsf(d) >= q.b;
+    const float r_out = d > 0.f ? c0 : -c0;
+    const float r_in = d >= 0.f ? c1 : -c1;
+    return outside ? r_out : r_in;
   }
   static __device__ __forceinline__ void bwd_e(float c0, float c1, float e1, float, const Q& q, float& ge1, float&) {
     bool outside;

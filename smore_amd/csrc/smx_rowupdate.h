@@ -71,27 +71,41 @@ template <int VEC> struct Pack2 {
   float v[VEC];
 };
 
-template <int VEC>
+// STREAM marks data that crosses the chip once per step (optimizer state, rows of one-off partial
+// sums, the updated rows written back): loaded and stored with the non-temporal hint, it does not push
+// the rows that are reused (queries, popular entities) out of the L2.
+typedef float vec4f __attribute__((ext_vector_type(4)));
+
+template <int VEC, bool STREAM = false>
 __device__ __forceinline__ Pack2<VEC> ld(const float* __restrict__ base, int col) {
   Pack2<VEC> r;
   if constexpr (VEC == 4) {
-    const float4 t = reinterpret_cast<const float4*>(base)[col];
+    const vec4f* p = reinterpret_cast<const vec4f*>(base) + col;
+    const vec4f t = STREAM ? __builtin_nontemporal_load(p) : *p;
     r.v[0] = t.x;
     r.v[1] = t.y;
     r.v[2] = t.z;
     r.v[3] = t.w;
   } else {
-    r.v[0] = base[col];
+    r.v[0] = STREAM ? __builtin_nontemporal_load(base + col) : base[col];
   }
   return r;
 }
 
-template <int VEC>
+template <int VEC, bool STREAM = false>
 __device__ __forceinline__ void st(float* __restrict__ base, int col, const float (&x)[VEC]) {
   if constexpr (VEC == 4) {
-    reinterpret_cast<float4*>(base)[col] = make_float4(x[0], x[1], x[2], x[3]);
+    vec4f t;
+    t.x = x[0];
+    t.y = x[1];
+    t.z = x[2];
+    t.w = x[3];
+    vec4f* p = reinterpret_cast<vec4f*>(base) + col;
+    if (STREAM) __builtin_nontemporal_store(t, p);
+    else *p = t;
   } else {
-    base[col] = x[0];
+    if (STREAM) __builtin_nontemporal_store(x[0], base + col);
+    else base[col] = x[0];
   }
 }
 
@@ -100,13 +114,13 @@ template <int MUL, int VEC, int NIT> struct RowRegs {
   Pack2<VEC> h[MUL][NIT];
 };
 
-template <int MUL, int VEC, int NIT>
+template <int MUL, int VEC, int NIT, bool STREAM = false>
 __device__ __forceinline__ void load_row(RowRegs<MUL, VEC, NIT>& r, const float* __restrict__ base, int half, int ncol,
                                          int lane) {
 #pragma unroll
   for (int h = 0; h < MUL; ++h)
 #pragma unroll
-    for (int it = 0; it < NIT; ++it) r.h[h][it] = ld<VEC>(base + h * half, min(lane + 64 * it, ncol - 1));
+    for (int it = 0; it < NIT; ++it) r.h[h][it] = ld<VEC, STREAM>(base + h * half, min(lane + 64 * it, ncol - 1));
 }
 
 // Coefficient on the second accumulator (BOX: inside distance) from the first.
@@ -149,8 +163,8 @@ __device__ __forceinline__ void finish_row(const RowSink& A, int lane, unsigned 
     for (int it = 0; it < NIT; ++it) {
       const int c = lane + 64 * it;
       if (c < A.ncol) {
-        st<VEC>(out, c, g1[it]);
-        if (MUL == 2) st<VEC>(out + half, c, g2[it]);
+        st<VEC, true>(out, c, g1[it]);
+        if (MUL == 2) st<VEC, true>(out + half, c, g2[it]);
       }
     }
   }
@@ -198,9 +212,9 @@ __device__ __forceinline__ void finish_row(const RowSink& A, int lane, unsigned 
             }
             v_new_row = vn[x];
           }
-          st<VEC>(pw + h * half, c, wn);
-          if (kind == kOptAdam) st<VEC>(pm + h * half, c, mn);
-          if (kind != kOptSgd && !A.squeeze) st<VEC>(pv + h * half, c, vn);
+          st<VEC, true>(pw + h * half, c, wn);
+          if (kind == kOptAdam) st<VEC, true>(pm + h * half, c, mn);
+          if (kind != kOptSgd && !A.squeeze) st<VEC, true>(pv + h * half, c, vn);
         }
       }
     }
@@ -218,9 +232,9 @@ __device__ __forceinline__ void request_state(const RowSink& A, int lane, unsign
   constexpr int MUL = src_mul(SRC);
   const int half = A.ncol * VEC;
   const size_t off = (size_t)row_id * half * MUL;
-  if (SRC != kSrcRows || A.adam_on) load_row<MUL, VEC, NIT>(s.e, A.table + off, half, A.ncol, lane);
-  if (A.adam_on == kOptAdam) load_row<MUL, VEC, NIT>(s.m, A.m + off, half, A.ncol, lane);
-  if (A.adam_on && A.adam_on != kOptSgd && !A.squeeze) load_row<MUL, VEC, NIT>(s.v, A.v + off, half, A.ncol, lane);
+  if (SRC != kSrcRows || A.adam_on) load_row<MUL, VEC, NIT, true>(s.e, A.table + off, half, A.ncol, lane);
+  if (A.adam_on == kOptAdam) load_row<MUL, VEC, NIT, true>(s.m, A.m + off, half, A.ncol, lane);
+  if (A.adam_on && A.adam_on != kOptSgd && !A.squeeze) load_row<MUL, VEC, NIT, true>(s.v, A.v + off, half, A.ncol, lane);
 }
 
 }  // namespace smx

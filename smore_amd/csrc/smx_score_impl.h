@@ -90,11 +90,14 @@ __device__ __forceinline__ void stage_query(float* lds, const float* __restrict_
 
 // ---- streaming the rows of up to 64 pairs through a wavefront -----------------------------------
 // The lanes first fetch, in one coalesced load, the ids of the pairs the wavefront is about to
-// process (pair j of the batch lives in lane j) and turn them into row offsets.  The row loop then
-// needs no memory access to find a row: the offset comes out of lane j with two v_readlane, so the
-// only loads in the loop are the rows themselves.  Rows are requested RIF at a time into two
-// register sets used in turn: while set A is consumed, set B is already on its way.  All loads are
-// unconditional (indices are clamped) so that they issue as one batch and stay in flight together.
+// process (pair j of the batch lives in lane j), turn them into row addresses and park them, with the
+// pair's two gradient coefficients in the backward kernel, in a 64-entry slab of LDS that belongs to
+// the wavefront.  The row loop then finds a row with one LDS read at a uniform address (a broadcast,
+// no bank conflicts) instead of v_readlane + scalar address arithmetic per row: the loop is bound by
+// instruction issue, and every vector or scalar instruction it does not need is time.  Rows are
+// requested RIF at a time into two register sets used in turn: while set A is consumed, set B is
+// already on its way.  All loads are unconditional so that they issue as one batch and stay in
+// flight together: entries past the batch's end repeat its last pair.
 
 struct PairBatch {
   unsigned off_lo, off_hi;  // this lane's pair: offset of its entity row in floats
@@ -118,8 +121,51 @@ __device__ __forceinline__ unsigned long long batch_off(const PairBatch& pb, int
   const unsigned hi = (unsigned)__builtin_amdgcn_readlane((int)pb.off_hi, j);
   return ((unsigned long long)hi << 32) | lo;
 }
-__device__ __forceinline__ const float* batch_row(const float* __restrict__ table, const PairBatch& pb, int j) {
-  return table + batch_off(pb, j);
+
+constexpr int kSlabDwords = 64 * 4;  // per wavefront: 64 entries of {address lo, address hi, c0, c1}
+
+// Orders a wavefront's own LDS writes before its later LDS reads (other lanes' entries).
+__device__ __forceinline__ void slab_fence() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+__device__ __forceinline__ void stage_pairs(unsigned* slab, int lane, const float* __restrict__ table,
+                                            const PairBatch& pb, float c0, float c1) {
+  slab_fence();  // reads of the previous batch are done
+  const unsigned long long addr =
+      (unsigned long long)(table + (((unsigned long long)pb.off_hi << 32) | pb.off_lo));
+  *reinterpret_cast<uint4*>(slab + 4 * lane) =
+      make_uint4((unsigned)addr, (unsigned)(addr >> 32), __float_as_uint(c0), __float_as_uint(c1));
+  slab_fence();
+}
+
+// The address comes back from LDS as an integer; the pointer made from it is declared global so that
+// the row loads are global_load (a generic pointer would make them flat_load, which also counts
+// against the LDS wait counter).
+typedef const __attribute__((address_space(1))) float* GlobalRow;
+__device__ __forceinline__ GlobalRow slab_row(const unsigned* slab, int j) {
+  const uint2 a = *reinterpret_cast<const uint2*>(slab + 4 * j);
+  return reinterpret_cast<GlobalRow>(((unsigned long long)a.y << 32) | a.x);
+}
+template <int VEC>
+__device__ __forceinline__ Pack<VEC> load_pack(GlobalRow base, int col) {
+  Pack<VEC> r;
+  if constexpr (VEC == 4) {
+    typedef float vec4 __attribute__((ext_vector_type(4)));
+    const vec4 t = reinterpret_cast<const __attribute__((address_space(1))) vec4*>(base)[col];
+    r.v[0] = t.x;
+    r.v[1] = t.y;
+    r.v[2] = t.z;
+    r.v[3] = t.w;
+  } else {
+    r.v[0] = base[col];
+  }
+  return r;
+}
+__device__ __forceinline__ float2 slab_coef(const unsigned* slab, int j) {
+  return *reinterpret_cast<const float2*>(slab + 4 * j + 2);
 }
 
 template <int MUL, int VEC, int NIT, int RIF> struct RowSet {
@@ -127,13 +173,13 @@ template <int MUL, int VEC, int NIT, int RIF> struct RowSet {
   Pack<VEC> e2[RIF][NIT];
 };
 
-// Requests rows j0 .. j0+RIF-1 of the batch (clamped to cnt-1).
+// Requests rows g0 .. g0+RIF-1 of the batch; g0 is a multiple of RIF, so the entries exist.
 template <int MUL, int VEC, int NIT, int RIF>
-__device__ __forceinline__ void request_rows(RowSet<MUL, VEC, NIT, RIF>& rs, const float* __restrict__ table,
-                                             const PairBatch& pb, int j0, int cnt, int dim, int ncol, int lane) {
+__device__ __forceinline__ void request_rows(RowSet<MUL, VEC, NIT, RIF>& rs, const unsigned* slab, int g0, int dim,
+                                             int ncol, int lane) {
 #pragma unroll
   for (int r = 0; r < RIF; ++r) {
-    const float* pe = batch_row(table, pb, min(j0 + r, cnt - 1));
+    const GlobalRow pe = slab_row(slab, g0 + r);
 #pragma unroll
     for (int it = 0; it < NIT; ++it) {
       const int c = min(lane + 64 * it, ncol - 1);
@@ -143,19 +189,20 @@ __device__ __forceinline__ void request_rows(RowSet<MUL, VEC, NIT, RIF>& rs, con
   }
 }
 
-// Streams the cnt (<= 64) rows of a batch through `consume(j, e1, e2)`, j ascending.
+// Streams the cnt (<= 64) rows of a staged batch through `consume(j, e1, e2)`, j ascending.
 template <int MUL, int VEC, int NIT, int RIF, class Consume>
-__device__ __forceinline__ void stream_batch(const float* __restrict__ table, const PairBatch& pb, int cnt, int dim,
-                                             int ncol, int lane, Consume&& consume) {
+__device__ __forceinline__ void stream_batch(const unsigned* slab, int cnt, int dim, int ncol, int lane,
+                                             Consume&& consume) {
+  static_assert(64 % RIF == 0, "a group of rows must not straddle the end of the slab");
   RowSet<MUL, VEC, NIT, RIF> a, b;
   const int last = ((cnt - 1) / RIF) * RIF;  // first row of the last group
-  request_rows<MUL, VEC, NIT, RIF>(a, table, pb, 0, cnt, dim, ncol, lane);
+  request_rows<MUL, VEC, NIT, RIF>(a, slab, 0, dim, ncol, lane);
   for (int j0 = 0; j0 < cnt; j0 += 2 * RIF) {
-    request_rows<MUL, VEC, NIT, RIF>(b, table, pb, min(j0 + RIF, last), cnt, dim, ncol, lane);
+    request_rows<MUL, VEC, NIT, RIF>(b, slab, min(j0 + RIF, last), dim, ncol, lane);
 #pragma unroll
     for (int r = 0; r < RIF; ++r)
       if (j0 + r < cnt) consume(j0 + r, a.e1[r], a.e2[r]);
-    request_rows<MUL, VEC, NIT, RIF>(a, table, pb, min(j0 + 2 * RIF, last), cnt, dim, ncol, lane);
+    request_rows<MUL, VEC, NIT, RIF>(a, slab, min(j0 + 2 * RIF, last), dim, ncol, lane);
 #pragma unroll
     for (int r = 0; r < RIF; ++r)
       if (j0 + RIF + r < cnt) consume(j0 + RIF + r, b.e1[r], b.e2[r]);
@@ -194,25 +241,29 @@ __global__ __launch_bounds__(256) void score_forward_kernel(ScoreArgs A, int til
   typename ModelOps<M>::Q q[NIT][VEC];
   load_query_regs<M, VEC, NIT, true>(lds, dim, ncol, lane, q);
   if (cnt <= 0) return;
+  unsigned* slab = reinterpret_cast<unsigned*>(lds + model_nq(M) * dim) + wave * kSlabDwords;
+  stage_pairs(slab, lane, table, pb, 0.f, 0.f);
 
   float* out = score + (size_t)b * K + kw0;
-  stream_batch<MUL, VEC, NIT, RIF>(table, pb, cnt, dim, ncol, lane,
+  stream_batch<MUL, VEC, NIT, RIF>(slab, cnt, dim, ncol, lane,
                                    [&](int j, const Pack<VEC>(&e1)[NIT], const Pack<VEC>(&e2)[NIT]) {
-    float a0 = 0.f, a1 = 0.f;
+    // lanes past the row end hold a copy of the last column: they compute along and are dropped here.
+    // The logit is linear in the accumulators: fold them per lane, reduce once.
+    float mine = 0.f;
 #pragma unroll
     for (int it = 0; it < NIT; ++it) {
-      if (lane + 64 * it < ncol) {
+      float a0 = 0.f, a1 = 0.f;
 #pragma unroll
-        for (int v = 0; v < VEC; ++v) {
-          const float x1 = REG ? reg_apply(e1[it].v[v], p) : e1[it].v[v];
-          const float x2 = MUL == 2 ? (REG ? reg_apply(e2[it].v[v], p) : e2[it].v[v]) : 0.f;
-          ModelOps<M>::fwd(x1, x2, q[it][v], a0, a1);
-        }
+      for (int v = 0; v < VEC; ++v) {
+        const float x1 = REG ? reg_apply(e1[it].v[v], p) : e1[it].v[v];
+        const float x2 = MUL == 2 ? (REG ? reg_apply(e2[it].v[v], p) : e2[it].v[v]) : 0.f;
+        ModelOps<M>::fwd(x1, x2, q[it][v], a0, a1);
       }
+      const float f = ModelOps<M>::fold(a0, a1, p);
+      mine += lane + 64 * it < ncol ? f : 0.f;
     }
-    // the logit is linear in the accumulators: fold them per lane, reduce once
-    const float folded = wave_sum_f32(ModelOps<M>::fold(a0, a1, p));
-    if (lane == 0) out[j] = ModelOps<M>::score(folded, p);
+    const float folded = wave_sum_last_f32(mine);
+    if (lane == 63) out[j] = ModelOps<M>::score(folded, p);
   });
   if (__ballot(bad != 0) != 0ull && err && lane == 0) *err = 1;
 }
@@ -254,6 +305,8 @@ __global__ __launch_bounds__(NW * 64) void score_backward_query_kernel(ScoreArgs
   for (int it = 0; it < NIT; ++it)
 #pragma unroll
     for (int v = 0; v < VEC; ++v) g1[it][v] = g2[it][v] = 0.f;
+  // LDS: query | per-wavefront partial sums | per-wavefront pair slabs
+  unsigned* slab = reinterpret_cast<unsigned*>(lds + (NW + 1) * NQ * dim) + wave * kSlabDwords;
 
   // this wavefront's share of the query's negatives: a contiguous range, walked in batches of 64
   const int per_wave = (K + NW - 1) / NW;
@@ -267,19 +320,18 @@ __global__ __launch_bounds__(NW * 64) void score_backward_query_kernel(ScoreArgs
     const size_t mine = first + min(lane, cnt - 1);
     float my_c0, my_c1;
     ModelOps<M>::coef(gscore[mine], score[mine], p, my_c0, my_c1);
-    stream_batch<MUL, VEC, NIT, RIF>(table, pb, cnt, dim, ncol, lane,
+    stage_pairs(slab, lane, table, pb, my_c0, my_c1);
+    // lanes past the row end hold a copy of the last column: what they accumulate is never stored
+    stream_batch<MUL, VEC, NIT, RIF>(slab, cnt, dim, ncol, lane,
                                      [&](int j, const Pack<VEC>(&e1)[NIT], const Pack<VEC>(&e2)[NIT]) {
-      const float c0 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(my_c0), j));
-      const float c1 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(my_c1), j));
+      const float2 c = slab_coef(slab, j);
 #pragma unroll
       for (int it = 0; it < NIT; ++it) {
-        if (lane + 64 * it < ncol) {
 #pragma unroll
-          for (int v = 0; v < VEC; ++v) {
-            const float x1 = REG ? reg_apply(e1[it].v[v], p) : e1[it].v[v];
-            const float x2 = MUL == 2 ? (REG ? reg_apply(e2[it].v[v], p) : e2[it].v[v]) : 0.f;
-            ModelOps<M>::bwd_q(c0, c1, x1, x2, q[it][v], g1[it][v], g2[it][v]);
-          }
+        for (int v = 0; v < VEC; ++v) {
+          const float x1 = REG ? reg_apply(e1[it].v[v], p) : e1[it].v[v];
+          const float x2 = MUL == 2 ? (REG ? reg_apply(e2[it].v[v], p) : e2[it].v[v]) : 0.f;
+          ModelOps<M>::bwd_q(c.x, c.y, x1, x2, q[it][v], g1[it][v], g2[it][v]);
         }
       }
     });
@@ -296,8 +348,8 @@ __global__ __launch_bounds__(NW * 64) void score_backward_query_kernel(ScoreArgs
         RowRegs<MUL, VEC, NIT> e, m0, v0;
         load_row<MUL, VEC, NIT>(e, table + off, dim, ncol, lane);
         if constexpr (SINGLES == 2) {
-          if (A.sink.adam_on == kOptAdam) load_row<MUL, VEC, NIT>(m0, A.sink.m + off, dim, ncol, lane);
-          if (A.sink.adam_on != kOptSgd && !A.sink.squeeze) load_row<MUL, VEC, NIT>(v0, A.sink.v + off, dim, ncol, lane);
+          if (A.sink.adam_on == kOptAdam) load_row<MUL, VEC, NIT, true>(m0, A.sink.m + off, dim, ncol, lane);
+          if (A.sink.adam_on != kOptSgd && !A.sink.squeeze) load_row<MUL, VEC, NIT, true>(v0, A.sink.v + off, dim, ncol, lane);
         }
         const float c0 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(my_c0), j));
         const float c1 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(my_c1), j));
@@ -362,7 +414,7 @@ int launch_forward_reg(hipStream_t st, const ScoreArgs& A) {
   int tile_k = 256;  // 64 negatives per wavefront; smaller tiles when the grid would not fill the chip
   while (tile_k > 4 * RIF && (B * ((K + tile_k - 1) / tile_k) < 8192 || (size_t)tile_k / 2 >= K)) tile_k /= 2;
   const int tiles = (int)((K + tile_k - 1) / tile_k);
-  const size_t lds = (size_t)model_nq(M) * A.ncol * VEC * sizeof(float);
+  const size_t lds = ((size_t)model_nq(M) * A.ncol * VEC + 4 * kSlabDwords) * sizeof(float);
   hipLaunchKernelGGL((score_forward_kernel<M, VEC, NIT, RIF, REG>), dim3((unsigned)(B * tiles)), dim3(256), lds, st, A,
                      tiles, tile_k);
   return check_launch("score forward");
@@ -371,7 +423,7 @@ int launch_forward_reg(hipStream_t st, const ScoreArgs& A) {
 template <int M, int VEC, int NIT, int NW, bool REG>
 int launch_backward_query_reg(hipStream_t st, const ScoreArgs& A) {
   constexpr int RIF = rows_in_flight(NIT, model_mul(M));
-  const size_t lds = (size_t)(NW + 1) * model_nq(M) * A.ncol * VEC * sizeof(float);
+  const size_t lds = ((size_t)(NW + 1) * model_nq(M) * A.ncol * VEC + NW * kSlabDwords) * sizeof(float);
   if (A.pair_seg && A.sink.adam_on)
     hipLaunchKernelGGL((score_backward_query_kernel<M, VEC, NIT, RIF, NW, REG, 2>), dim3((unsigned)A.B),
                        dim3(NW * 64), lds, st, A);

@@ -26,6 +26,24 @@ __device__ __forceinline__ float wave_sum_f32(float v) {
   return ((r0 + r1) + r2) + r3;
 }
 
+// Sum over the 64 lanes, valid in lane 63 only: the four row sums are combined with two more DPP
+// steps (row_bcast:15 into rows 1 and 3, row_bcast:31 into rows 2 and 3) instead of being read out
+// into scalars, six vector instructions in all.  Order: (r2 + r3) + (r0 + r1).
+__device__ __forceinline__ float wave_sum_last_f32(float v) {
+  v += dpp_move<0xB1>(v);
+  v += dpp_move<0x4E>(v);
+  v += dpp_move<0x141>(v);
+  v += dpp_move<0x140>(v);
+  // rows outside row_mask keep their value; written as the fused instruction (the compiler expands the
+  // builtin form into mov 0 + mov_dpp + add); the s_nop cover the VALU-write -> DPP-read wait states
+  asm("s_nop 1\n\t"
+      "v_add_f32_dpp %0, %0, %0 row_bcast:15 row_mask:0xa bank_mask:0xf\n\t"
+      "s_nop 1\n\t"
+      "v_add_f32_dpp %0, %0, %0 row_bcast:31 row_mask:0xc bank_mask:0xf"
+      : "+v"(v));
+  return v;
+}
+
 // Makes a value the compiler cannot prove wave-uniform into a scalar.
 __device__ __forceinline__ int uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
 
