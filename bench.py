@@ -119,7 +119,7 @@ class Step:
     """One pass of the hot path; phases are bracketed by events on the stream the kernels run on."""
     PHASES = ("plan", "forward", "backward")
 
-    def __init__(self, cfg, table, q1, q2, idx, gscore):
+    def __init__(self, cfg, table, q1, q2, idx, gscore, sign_codes=True):
         import torch
         from smore_amd import fused
         self.fused, self.torch = fused, torch
@@ -130,6 +130,8 @@ class Step:
         self.merged = None
         self.step_no = 0
         self.err = fused.new_error_flag(table.device)
+        # box: the forward leaves two bits per feature for the backward (None for models without sign codes)
+        self.codes = fused.new_codes(cfg["model"], table, idx, q1) if sign_codes else None
         self.plan = None
 
     def run(self, events=None):
@@ -139,16 +141,18 @@ class Step:
         mark(0)
         plan = f.build_plan(self.idx, cfg["n"], err_flag=self.err)
         mark(1)
-        score = f.score_forward(cfg["model"], self.table, self.idx, self.q1, self.q2, self.params, self.err)
+        score = f.score_forward(cfg["model"], self.table, self.idx, self.q1, self.q2, self.params, self.err,
+                                codes=self.codes)
         mark(2)
         if cfg["adam"]:
             gq = f.score_backward_fused(cfg["model"], plan, self.table, self.idx, self.q1, self.q2, score, self.gscore,
-                                        self.params, m=self.m, v=self.v, adam=f.adam_params(cfg["lr"], self.step_no))
+                                        self.params, m=self.m, v=self.v, adam=f.adam_params(cfg["lr"], self.step_no),
+                                        codes=self.codes)
         else:
             if self.merged is None:
                 self.merged = self.torch.empty((plan.n_uniq, self.table.shape[1]), device=self.table.device)
             gq = f.score_backward_fused(cfg["model"], plan, self.table, self.idx, self.q1, self.q2, score, self.gscore,
-                                        self.params, merged=self.merged)
+                                        self.params, merged=self.merged, codes=self.codes)
         mark(3)
         self.plan = plan
         return score, gq
@@ -210,6 +214,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--config", type=int, default=5, choices=sorted(CONFIGS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-sign-codes", action="store_true",
+                    help="box: do not save sign codes in the forward; the backward re-reads entity and query rows")
     ap.add_argument("--seed", type=int, default=None)
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run only a plain row copy of known size (1 GiB read + 1 GiB written per launch) through "
@@ -240,7 +246,7 @@ def main():
     seed = args.seed if args.seed is not None else 20240 + args.config
 
     table, q1, q2, idx, gscore = make_inputs(cfg, device, seed)
-    step = Step(cfg, table, q1, q2, idx, gscore)
+    step = Step(cfg, table, q1, q2, idx, gscore, sign_codes=not args.no_sign_codes)
     for _ in range(args.warmup):
         step.run()
     torch.cuda.synchronize()

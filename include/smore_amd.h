@@ -104,9 +104,19 @@ typedef struct smx_score_params {
   float reg_hi;
 } smx_score_params;
 
+/* Sign codes (optional, what autograd would call a saved tensor).  For the box model the derivative
+ * of a pair's distance w.r.t. each feature is +-c0 or +-c1, decided by comparisons the forward pass
+ * makes anyway.  Given a `codes` buffer of smx_score_codes_bytes(model, B*K, dim) bytes (16-byte
+ * aligned), the forward leaves those decisions there, two bits per feature; handed to
+ * smx_score_backward_fused, they replace every read of entity and query rows for the gradient -- the
+ * same decisions, hence the same bits as recomputing them, as long as table and queries are unchanged
+ * between the two calls.  smx_score_codes_bytes is 0 for models or row lengths without codes (pass
+ * codes = NULL then). */
+size_t smx_score_codes_bytes(int model, size_t n_pairs, size_t dim);
+
 int smx_score_forward(int model, void* stream, const float* table, size_t n_rows, const int64_t* idx,
                       const float* q1, const float* q2, float* score, size_t B, size_t K, size_t dim,
-                      const smx_score_params* params, int* err_flag);
+                      const smx_score_params* params, int* err_flag, void* codes, size_t codes_bytes);
 
 /* Query-side gradient of sum(gscore * score): gq1, gq2 [B, dim] are overwritten.
  * `score` is the tensor smx_score_forward wrote (L2 needs it for the chain
@@ -199,15 +209,23 @@ int smx_score_backward_entity(int model, void* stream, const smx_plan_view* plan
  * just read the entity row; the entity pass then skips them.  The plan must have been built with
  * pair_seg.  Same results as the two separate calls up to fp32 rounding (the one-pair rows are computed
  * by a different kernel, so a multiply-add may be contracted differently).
- * workspace as for smx_score_backward_entity.  No counterpart as one function in the reference:
+ * workspace: smx_fused_workspace_bytes (below).  No counterpart as one function in the reference:
  * it stands for dist_backward (extlib_cuda.cpp:230-262) + EmbedLookupFunc.backward +
  * EmbeddingOptimizer.apply_grad (embed_optimizer.py:63-66,155-163). */
+/* Workspace of smx_score_backward_fused: smx_entity_workspace_bytes(P, dim*mul) plus, for models whose
+ * entity derivative is a choice of sign and coefficient (box), room for the per-pair sign codes the
+ * query-gradient kernel leaves for the entity pass (64 bytes per pair and 256 floats of dim).  With
+ * only smx_entity_workspace_bytes the call works too and the entity pass reads the query rows.
+ * fwd_codes (may be NULL): the codes smx_score_forward wrote for these same pairs; the workspace then
+ * needs no room for codes. */
+size_t smx_fused_workspace_bytes(int model, size_t n_pairs, size_t dim);
 int smx_score_backward_fused(int model, void* stream, const smx_plan_view* plan, float* table,
                              size_t n_rows, const int64_t* idx, const float* q1, const float* q2,
                              const float* score, const float* gscore, float* gq1, float* gq2,
                              size_t B, size_t K, size_t dim, const smx_score_params* params,
                              float* merged, float* m, float* v, const smx_opt_params* adam,
-                             void* workspace, size_t workspace_bytes);
+                             void* workspace, size_t workspace_bytes,
+                             const void* fwd_codes, size_t fwd_codes_bytes);
 
 /* Same pass for gradient rows that already exist in memory (what autograd hands
  * EmbedLookupFunc.backward): grad_rows [P, row_len] in pair order.  Replaces

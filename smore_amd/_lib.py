@@ -29,8 +29,9 @@ SIGNATURES = {
     "smx_dist_forward_f64": (_i, _DENSE_FWD),
     "smx_dist_backward_f32": (_i, _DENSE_BWD),
     "smx_dist_backward_f64": (_i, _DENSE_BWD),
-    # model, stream, table, n_rows, idx, q1, q2, score, B, K, dim, params, err_flag
-    "smx_score_forward": (_i, [_i, _vp, _vp, _sz, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _vp, _vp]),
+    "smx_score_codes_bytes": (_sz, [_i, _sz, _sz]),
+    # model, stream, table, n_rows, idx, q1, q2, score, B, K, dim, params, err_flag, codes, codes_bytes
+    "smx_score_forward": (_i, [_i, _vp, _vp, _sz, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _vp, _vp, _vp, _sz]),
     # model, stream, table, n_rows, idx, q1, q2, score, gscore, gq1, gq2, B, K, dim, params
     "smx_score_backward_query": (_i, [_i, _vp, _vp, _sz, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _vp]),
     "smx_plan_workspace_bytes": (_sz, [_sz, _sz]),
@@ -38,13 +39,14 @@ SIGNATURES = {
     # n_uniq, err
     "smx_plan_build": (_i, [_vp, _vp, _sz, _sz, _vp, _sz, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "smx_entity_workspace_bytes": (_sz, [_sz, _sz]),
+    "smx_fused_workspace_bytes": (_sz, [_i, _sz, _sz]),
     # model, stream, plan, table, n_rows, q1, q2, score, gscore, B, K, dim, params, merged, m, v, adam, ws, ws_bytes
     "smx_score_backward_entity": (_i, [_i, _vp, _vp, _vp, _sz, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _vp, _vp, _vp, _vp,
                                        _vp, _vp, _sz]),
     # model, stream, plan, table, n_rows, idx, q1, q2, score, gscore, gq1, gq2, B, K, dim, params, merged, m, v,
-    # adam, ws, ws_bytes
+    # adam, ws, ws_bytes, fwd_codes, fwd_codes_bytes
     "smx_score_backward_fused": (_i, [_i, _vp, _vp, _vp, _sz, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _vp,
-                                      _vp, _vp, _vp, _vp, _vp, _sz]),
+                                      _vp, _vp, _vp, _vp, _vp, _sz, _vp, _sz]),
     # stream, plan, grad_rows, row_len, merged, table, m, v, adam, ws, ws_bytes
     # stream, table, n_rows, row_len, idx, n, out, err
     "smx_gather_rows": (_i, [_vp, _vp, _sz, _sz, _vp, _sz, _vp, _vp]),

@@ -55,7 +55,16 @@ static EntityScratch entity_scratch(size_t n_pairs, size_t row_len) {
   return s;
 }
 
-static size_t entity_ws_bytes(size_t n_pairs, size_t row_len) { return entity_scratch(n_pairs, row_len).total; }
+size_t entity_ws_bytes(size_t n_pairs, size_t row_len) { return entity_scratch(n_pairs, row_len).total; }
+
+// Sign codes: one byte per lane and column group of 64 lanes; the groups are those of the float4 layout
+// when dim allows it (rows that are then not 16-byte aligned get no codes), of single floats otherwise.
+size_t code_bytes_per_pair(size_t dim) {
+  const size_t ncol = dim % 4 == 0 ? dim / 4 : dim;
+  size_t groups = (ncol + 63) / 64, g = 1;
+  while (g < groups) g *= 2;
+  return g * 64;
+}
 
 static int fill_plan(EntityArgs* A, const smx_plan_view* plan, void* workspace, size_t workspace_bytes, size_t row_len) {
   if (!plan || !plan->order || !plan->sorted_ids || !plan->seg_of_pos || !plan->seg_start || !plan->uniq ||
@@ -84,7 +93,8 @@ static int fill_plan(EntityArgs* A, const smx_plan_view* plan, void* workspace, 
 int entity_backward(int model, void* stream, const smx_plan_view* plan, float* table, size_t n_rows, const float* q1,
                     const float* q2, const float* score, const float* gscore, size_t B, size_t K, size_t dim,
                     const smx_score_params* params, float* merged, float* m, float* v, const smx_opt_params* adam,
-                    void* workspace, size_t workspace_bytes, int skip_single);
+                    void* workspace, size_t workspace_bytes, int skip_single, const unsigned char* codes, int codes_vec,
+                    int codes_nit);
 
 static int fill_adam(EntityArgs* A, float* m, float* v, const smx_opt_params* opt) {
   A->adam_on = 0;
@@ -108,12 +118,20 @@ extern "C" {
 
 size_t smx_entity_workspace_bytes(size_t n_pairs, size_t row_len) { return smx::entity_ws_bytes(n_pairs, row_len); }
 
+size_t smx_fused_workspace_bytes(int model, size_t n_pairs, size_t dim) {
+  using namespace smx;
+  if (model < 0 || model >= mNumModels) return 0;
+  size_t total = entity_ws_bytes(n_pairs, dim * model_mul(model));
+  if (model_coded(model)) total += align256(n_pairs * code_bytes_per_pair(dim));
+  return total;
+}
+
 int smx_score_backward_entity(int model, void* stream, const smx_plan_view* plan, float* table, size_t n_rows,
                               const float* q1, const float* q2, const float* score, const float* gscore, size_t B,
                               size_t K, size_t dim, const smx_score_params* params, float* merged, float* m, float* v,
                               const smx_opt_params* adam, void* workspace, size_t workspace_bytes) {
   return smx::entity_backward(model, stream, plan, table, n_rows, q1, q2, score, gscore, B, K, dim, params, merged, m,
-                              v, adam, workspace, workspace_bytes, 0);
+                              v, adam, workspace, workspace_bytes, 0, nullptr, 0, 0);
 }
 
 }  // extern "C"
@@ -123,7 +141,8 @@ namespace smx {
 int entity_backward(int model, void* stream, const smx_plan_view* plan, float* table, size_t n_rows, const float* q1,
                     const float* q2, const float* score, const float* gscore, size_t B, size_t K, size_t dim,
                     const smx_score_params* params, float* merged, float* m, float* v, const smx_opt_params* adam,
-                    void* workspace, size_t workspace_bytes, int skip_single) {
+                    void* workspace, size_t workspace_bytes, int skip_single, const unsigned char* codes, int codes_vec,
+                    int codes_nit) {
   if (model < 0 || model >= mNumModels) return fail(SMX_ERR_KIND, "unknown score model %d", model);
   if (!table || !q1 || !score || !gscore || !params || (model_nq(model) == 2 && !q2))
     return fail(SMX_ERR_ARG, "null pointer");
@@ -154,6 +173,10 @@ int entity_backward(int model, void* stream, const smx_plan_view* plan, float* t
   A.merged = merged;
   A.ncol = (int)ncol;
   A.skip_single = skip_single;
+  if (codes) {
+    if (vec != codes_vec || nit != codes_nit) return fail(SMX_ERR_ARG, "sign codes were written for another column layout");
+    A.codes = codes;
+  }
   hipStream_t st = as_stream(stream);
   switch (model) {
     case mL1: return entity_dispatch<mL1>(st, A, vec, nit);

@@ -54,6 +54,8 @@ struct EntityArgs : RowSink {
   float* tail;    // [tiles, row_len] partial rows of long segments
   float* head;    // [tiles, row_len]
   int skip_single;  // segments of one pair were already finished by the query-backward kernel
+  // sign codes written by the query-backward kernel, [n_pairs][NIT*64] bytes, or null (CODED kernels)
+  const unsigned char* codes;
 };
 
 template <int SRC>
@@ -72,21 +74,25 @@ __device__ __forceinline__ float second_coef(float c0, const ScoreParams& p) {
 
 template <int R> struct RunSet {
   int key[R];    // query number (model sources) or pair number (gradient rows)
+  int pair[R];   // first pair of the run (CODED: where its sign codes are)
   float c[R];    // summed coefficient (model sources)
   int n;         // valid runs
 };
 
 // Collects up to R runs from window lanes [j, j_end); my_key / my_c hold one sorted position per lane.
-template <int SRC, int R>
-__device__ __forceinline__ void collect_runs(RunSet<R>& rs, int& j, int j_end, int my_key, float my_c) {
+template <int SRC, int R, bool CODED = false>
+__device__ __forceinline__ void collect_runs(RunSet<R>& rs, int& j, int j_end, int my_key, float my_c,
+                                             int my_pair = 0) {
   rs.n = 0;
 #pragma unroll
   for (int r = 0; r < R; ++r) {
     rs.key[r] = 0;
+    rs.pair[r] = 0;
     rs.c[r] = 0.f;
     if (j < j_end) {  // wave-uniform
       rs.n = r + 1;
       rs.key[r] = __builtin_amdgcn_readlane(my_key, j);
+      if constexpr (CODED) rs.pair[r] = __builtin_amdgcn_readlane(my_pair, j);
       if constexpr (SRC == kSrcRows) {
         ++j;
       } else {
@@ -102,17 +108,22 @@ __device__ __forceinline__ void collect_runs(RunSet<R>& rs, int& j, int j_end, i
 template <int SRC, int VEC, int NIT, int R> struct RunRows {
   Pack2<VEC> a[R][NIT];
   Pack2<VEC> b[R][NIT];
+  unsigned code[R][NIT];  // CODED: the lane's code byte per column group
 };
 
 // Requests the rows the runs need: query row(s) for the model sources, the gradient row otherwise.
-template <int SRC, int VEC, int NIT, int R>
+template <int SRC, int VEC, int NIT, int R, bool CODED = false>
 __device__ __forceinline__ void request_runs(const EntityArgs& A, int lane, const RunSet<R>& rs,
                                              RunRows<SRC, VEC, NIT, R>& rr) {
   const int half = A.ncol * VEC;
 #pragma unroll
   for (int r = 0; r < R; ++r) {
     if (r < rs.n) {
-      if constexpr (SRC == kSrcRows) {
+      if constexpr (CODED) {
+        const unsigned char* pc = A.codes + (size_t)rs.pair[r] * (NIT * 64) + lane;
+#pragma unroll
+        for (int it = 0; it < NIT; ++it) rr.code[r][it] = pc[64 * it];
+      } else if constexpr (SRC == kSrcRows) {
         const float* pg = A.grad_rows + (size_t)rs.key[r] * half;
 #pragma unroll
         for (int it = 0; it < NIT; ++it) rr.a[r][it] = ld<VEC>(pg, min(lane + 64 * it, A.ncol - 1));
@@ -131,7 +142,7 @@ __device__ __forceinline__ void request_runs(const EntityArgs& A, int lane, cons
 }
 
 // Adds the gradient of the runs to the lane's accumulators.
-template <int SRC, int VEC, int NIT, bool REG, int R>
+template <int SRC, int VEC, int NIT, bool REG, int R, bool CODED = false>
 __device__ __forceinline__ void apply_runs(const EntityArgs& A, const RunSet<R>& rs,
                                            const RunRows<SRC, VEC, NIT, R>& rr,
                                            const RowRegs<src_mul(SRC), VEC, NIT>& e, float (&g1)[NIT][VEC],
@@ -144,7 +155,9 @@ __device__ __forceinline__ void apply_runs(const EntityArgs& A, const RunSet<R>&
       for (int it = 0; it < NIT; ++it) {
 #pragma unroll
         for (int x = 0; x < VEC; ++x) {
-          if constexpr (SRC == kSrcRows) {
+          if constexpr (CODED) {
+            ModelOps<SRC>::bwd_e_coded(rs.c[r], second_coef<SRC>(rs.c[r], A.p), rr.code[r][it], VEC - 1 - x, g1[it][x]);
+          } else if constexpr (SRC == kSrcRows) {
             g1[it][x] += rr.a[r][it].v[x];
           } else {
             const float c0 = rs.c[r];
@@ -163,13 +176,14 @@ __device__ __forceinline__ void apply_runs(const EntityArgs& A, const RunSet<R>&
 
 // One sorted position per lane: the window [base, base+64) of the per-position inputs.
 template <int SRC>
-__device__ __forceinline__ void load_window(const EntityArgs& A, int lane, int base, int& my_key, float& my_c) {
+__device__ __forceinline__ void load_window(const EntityArgs& A, int lane, int base, int& my_key, float& my_c,
+                                            int& my_pair) {
   const int pos = min(base + lane, A.n_pairs - 1);
   if constexpr (SRC == kSrcRows) {
-    my_key = A.order[pos];
+    my_key = my_pair = A.order[pos];
     my_c = 0.f;
   } else {
-    const int pair = A.order[pos];
+    const int pair = my_pair = A.order[pos];
     float c1;
     ModelOps<SRC>::coef(A.gscore[pair], A.score[pair], A.p, my_c, c1);
     my_key = pair / A.K;
@@ -200,8 +214,10 @@ __device__ __forceinline__ void zero_acc(float (&g1)[NIT][VEC], float (&g2)[NIT]
     for (int x = 0; x < VEC; ++x) g1[it][x] = g2[it][x] = 0.f;
 }
 
-constexpr int kRunsShort = 2;  // runs in flight per wavefront in the short-segment kernel
-constexpr int kRunsLong = 4;   // ... in the long-segment kernel
+// runs in flight per wavefront in the short-segment kernel / the long-segment kernel; with sign codes
+// a run costs one byte per lane instead of two row loads, so more of them fit
+constexpr int runs_short(bool coded) { return coded ? 4 : 2; }
+constexpr int runs_long(bool coded) { return coded ? 8 : 4; }
 
 // Short segments (at most A.short_max pairs).  The sorted pair list is cut into chunks of 64
 // positions and a fixed grid of wavefronts strides over the chunks; a wavefront owns the short
@@ -209,10 +225,10 @@ constexpr int kRunsLong = 4;   // ... in the long-segment kernel
 // segment lengths are distributed.  The lanes fetch the chunk's per-position inputs at once; the
 // wavefront then finishes one segment after the other, and while it works on one it already has
 // the next one's w, m, v rows on the way (two register sets used in turn).
-template <int SRC, int VEC, int NIT, bool REG>
+template <int SRC, int VEC, int NIT, bool REG, bool CODED = false>
 __global__ __launch_bounds__(256) void entity_segment_kernel(EntityArgs A) {
   constexpr int MUL = src_mul(SRC);
-  constexpr int R = kRunsShort;
+  constexpr int R = runs_short(CODED);
   const int lane = threadIdx.x & 63;
   const int wave = uniform(threadIdx.x >> 6);
   const int n_waves = gridDim.x * 4;
@@ -232,9 +248,9 @@ __global__ __launch_bounds__(256) void entity_segment_kernel(EntityArgs A) {
     const int my_id = A.sorted_ids[pos];
 
     int win_base = base;
-    int my_key;
+    int my_key, my_pair;
     float my_c;
-    load_window<SRC>(A, lane, win_base, my_key, my_c);
+    load_window<SRC>(A, lane, win_base, my_key, my_c, my_pair);
 
     // finishes the segment that starts at lane i of the chunk from row state `cur`; requests the rows
     // of the segment starting at lane `nxt` (if any) into `ahead` right after this segment's first
@@ -246,7 +262,7 @@ __global__ __launch_bounds__(256) void entity_segment_kernel(EntityArgs A) {
       const int seg = __builtin_amdgcn_readlane(my_seg, i);
       if (s1 > win_base + 64) {  // the segment runs past the window: restart the window at its first pair
         win_base = s0;
-        load_window<SRC>(A, lane, win_base, my_key, my_c);
+        load_window<SRC>(A, lane, win_base, my_key, my_c, my_pair);
       }
       float g1[NIT][VEC], g2[NIT][VEC];
       zero_acc<VEC, NIT>(g1, g2);
@@ -254,14 +270,14 @@ __global__ __launch_bounds__(256) void entity_segment_kernel(EntityArgs A) {
       const int j_end = s1 - win_base;
       RunSet<R> rs;
       RunRows<SRC, VEC, NIT, R> rr;
-      collect_runs<SRC, R>(rs, j, j_end, my_key, my_c);
-      request_runs<SRC, VEC, NIT, R>(A, lane, rs, rr);
+      collect_runs<SRC, R, CODED>(rs, j, j_end, my_key, my_c, my_pair);
+      request_runs<SRC, VEC, NIT, R, CODED>(A, lane, rs, rr);
       if (nxt >= 0) request_state<SRC, VEC, NIT>(A, lane, (unsigned)__builtin_amdgcn_readlane(my_id, nxt), ahead);
-      apply_runs<SRC, VEC, NIT, REG, R>(A, rs, rr, cur.e, g1, g2);
+      apply_runs<SRC, VEC, NIT, REG, R, CODED>(A, rs, rr, cur.e, g1, g2);
       while (j < j_end) {
-        collect_runs<SRC, R>(rs, j, j_end, my_key, my_c);
-        request_runs<SRC, VEC, NIT, R>(A, lane, rs, rr);
-        apply_runs<SRC, VEC, NIT, REG, R>(A, rs, rr, cur.e, g1, g2);
+        collect_runs<SRC, R, CODED>(rs, j, j_end, my_key, my_c, my_pair);
+        request_runs<SRC, VEC, NIT, R, CODED>(A, lane, rs, rr);
+        apply_runs<SRC, VEC, NIT, REG, R, CODED>(A, rs, rr, cur.e, g1, g2);
       }
       finish_row<SRC, VEC, NIT, REG>(A, lane, row_id, seg, g1, g2, cur.e, cur.m, cur.v);
     };
@@ -290,10 +306,10 @@ __global__ __launch_bounds__(256) void entity_segment_kernel(EntityArgs A) {
 // long segment inside the tile is summed; a segment that lies wholly inside the tile is finished here,
 // otherwise the sum goes to the tile's tail row (segment continues past the tile end) or head row
 // (segment came in from the left and ends here).
-template <int SRC, int VEC, int NIT, bool REG>
+template <int SRC, int VEC, int NIT, bool REG, bool CODED = false>
 __global__ __launch_bounds__(256) void entity_tile_kernel(EntityArgs A) {
   constexpr int MUL = src_mul(SRC);
-  constexpr int R = kRunsLong;
+  constexpr int R = runs_long(CODED);
   const int lane = threadIdx.x & 63;
   const int wave = uniform(threadIdx.x >> 6);
   const int t = blockIdx.x * 4 + wave;
@@ -321,23 +337,23 @@ __global__ __launch_bounds__(256) void entity_tile_kernel(EntityArgs A) {
       RowState<MUL, VEC, NIT> st;
       if (whole) {
         request_state<SRC, VEC, NIT>(A, lane, row_id, st);
-      } else if (SRC != kSrcRows) {
+      } else if (SRC != kSrcRows && !CODED) {
         load_row<MUL, VEC, NIT>(st.e, A.table + (size_t)row_id * A.ncol * VEC * MUL, A.ncol * VEC, A.ncol, lane);
       }
       float g1[NIT][VEC], g2[NIT][VEC];
       zero_acc<VEC, NIT>(g1, g2);
       for (int base = pos; base < end; base += 64) {
-        int my_key;
+        int my_key, my_pair;
         float my_c;
-        load_window<SRC>(A, lane, base, my_key, my_c);
+        load_window<SRC>(A, lane, base, my_key, my_c, my_pair);
         int j = 0;
         const int j_end = min(64, end - base);
         while (j < j_end) {
           RunSet<R> rs;
           RunRows<SRC, VEC, NIT, R> rr;
-          collect_runs<SRC, R>(rs, j, j_end, my_key, my_c);
-          request_runs<SRC, VEC, NIT, R>(A, lane, rs, rr);
-          apply_runs<SRC, VEC, NIT, REG, R>(A, rs, rr, st.e, g1, g2);
+          collect_runs<SRC, R, CODED>(rs, j, j_end, my_key, my_c, my_pair);
+          request_runs<SRC, VEC, NIT, R, CODED>(A, lane, rs, rr);
+          apply_runs<SRC, VEC, NIT, REG, R, CODED>(A, rs, rr, st.e, g1, g2);
         }
       }
       if (whole)
@@ -452,8 +468,17 @@ int launch_entity_reg(hipStream_t st, const EntityArgs& A) {
   // short segments: a fixed grid of wavefronts strides over the segment list (its length lives on the device)
   unsigned seg_blocks = (unsigned)((A.n_pairs + 3) / 4);
   if (seg_blocks > 256u * 8u) seg_blocks = 256u * 8u;
-  hipLaunchKernelGGL((entity_segment_kernel<SRC, VEC, NIT, REG>), dim3(seg_blocks), dim3(256), 0, st, A);
-  hipLaunchKernelGGL((entity_tile_kernel<SRC, VEC, NIT, REG>), dim3((tiles + 3) / 4), dim3(256), 0, st, A);
+  bool coded = false;
+  if constexpr (SRC != kSrcRows && model_coded(SRC) && !REG) coded = A.codes != nullptr;
+  if (coded) {
+    if constexpr (SRC != kSrcRows && model_coded(SRC) && !REG) {
+      hipLaunchKernelGGL((entity_segment_kernel<SRC, VEC, NIT, REG, true>), dim3(seg_blocks), dim3(256), 0, st, A);
+      hipLaunchKernelGGL((entity_tile_kernel<SRC, VEC, NIT, REG, true>), dim3((tiles + 3) / 4), dim3(256), 0, st, A);
+    }
+  } else {
+    hipLaunchKernelGGL((entity_segment_kernel<SRC, VEC, NIT, REG>), dim3(seg_blocks), dim3(256), 0, st, A);
+    hipLaunchKernelGGL((entity_tile_kernel<SRC, VEC, NIT, REG>), dim3((tiles + 3) / 4), dim3(256), 0, st, A);
+  }
   const size_t row_bytes = (size_t)A.ncol * VEC * src_mul(SRC) * sizeof(float);
   if (15 * row_bytes <= 60 * 1024)
     hipLaunchKernelGGL((entity_fixup_kernel<SRC, VEC, NIT, 16, REG>), dim3(tiles), dim3(16 * 64), 15 * row_bytes, st, A);

@@ -27,6 +27,8 @@ enum Model : int { mL1 = 0, mL2 = 1, mBox = 2, mRotate = 3, mBetaKL = 4, mNumMod
 
 __host__ __device__ constexpr int model_mul(int m) { return (m == mRotate || m == mBetaKL) ? 2 : 1; }
 __host__ __device__ constexpr int model_nq(int m) { return (m == mL1 || m == mL2) ? 1 : 2; }
+// models whose entity derivative can be kept as sign codes (ModelOps<M>::bwd_q_coded / bwd_e_coded)
+__host__ __device__ constexpr bool model_coded(int m) { return m == mBox; }
 
 struct ScoreParams {
   float gamma;
@@ -163,6 +165,64 @@ template <> struct ModelOps<mBox> {
   }
   static __device__ __forceinline__ void finish_q(const Q& q, float&, float& go, const ScoreParams& p) {
     go *= (q.b > 0.f ? p.cen : -p.cen) - 1.0f;
+  }
+
+  // ---- sign codes ----
+  // The derivative of a pair's distance w.r.t. one entity feature is +-c0 or +-c1: two bits say which
+  // (lower bit: outside, upper bit: negative; the features of a column are pushed in ascending order, so the
+  // last one sits in bits 0-1 and feature x of VEC at position VEC-1-x).  The query-gradient kernel, which makes these decisions anyway,
+  // can leave them behind, one byte per four features; the entity pass then sums  +-c  straight from
+  // the codes and needs neither the query rows nor the comparisons -- same decisions, same bits.
+  // push2: code = 4 * code + 2 * (lane's bit of hi) + (lane's bit of lo): two v_addc with the masks as
+  // carry-in.  The s_nop covers the wait states a VALU read of an SGPR needs after a VALU compare
+  // wrote it (the assembler does not look into inline asm).
+  static __device__ __forceinline__ unsigned push2(unsigned code, unsigned long long hi, unsigned long long lo) {
+    unsigned long long carry;
+    asm("s_nop 1\n\t"
+        "v_addc_co_u32_e64 %0, %1, %0, %0, %2\n\t"
+        "v_addc_co_u32_e64 %0, %1, %0, %0, %3"
+        : "+v"(code), "=&s"(carry)
+        : "s"(hi), "s"(lo));
+    return code;
+  }
+  // As bwd_q, and pushes this feature's two bits onto `code`.
+  static __device__ __forceinline__ void bwd_q_coded(float c0, float c1, float e1, const Q& q, float& gc, float& go,
+                                                     unsigned& code) {
+    const float d = e1 - q.a;
+    const bool outside = fabsf(d) >= q.b, gt = d > 0.f, ge = d >= 0.f;
+    const float r_out = gt ? c0 : -c0;
+    const float r_in = ge ? c1 : -c1;
+    gc -= outside ? r_out : r_in;
+    go += outside ? c0 : 0.f;
+    const unsigned long long T = __ballot(outside), GT = __ballot(gt), GE = __ballot(ge);
+    code = push2(code, ~((T & GT) | (~T & GE)), T);
+  }
+  // As fwd, and pushes this feature's two bits onto `code`: the forward pass
+  // can leave the codes too, and then the whole backward works from them without the entity rows.
+  static __device__ __forceinline__ void fwd_coded(float e1, const Q& q, float& a0, float& a1, unsigned& code) {
+    const float d = e1 - q.a;
+    const float a = fabsf(d);
+    const float mn = min_abs(d, q.b);
+    a0 += a - mn;
+    a1 += fabsf(mn);
+    const unsigned long long T = __ballot(a >= q.b), GT = __ballot(d > 0.f), GE = __ballot(d >= 0.f);
+    code = push2(code, ~((T & GT) | (~T & GE)), T);
+  }
+  // Query side from a code byte: gc -= derivative of the feature at position x, go += c0 where the pair is outside.
+  static __device__ __forceinline__ void bwd_q_from_code(float c0, float c1, unsigned code, int x, float& gc,
+                                                         float& go) {
+    const unsigned t = (unsigned)__builtin_amdgcn_sbfe((int)code, 2 * x, 1);  // 0 or ~0
+    const float w = __uint_as_float((__float_as_uint(c0) & t) | (__float_as_uint(c1) & ~t));
+    const unsigned sign = (code << (30 - 2 * x)) & 0x80000000u;
+    gc -= __uint_as_float(__float_as_uint(w) ^ sign);
+    go += __uint_as_float(__float_as_uint(c0) & t);
+  }
+  // ge += derivative of the feature at position x of the lane's code byte
+  static __device__ __forceinline__ void bwd_e_coded(float c0, float c1, unsigned code, int x, float& ge) {
+    const unsigned t = (unsigned)__builtin_amdgcn_sbfe((int)code, 2 * x, 1);  // 0 or ~0
+    const float w = __uint_as_float((__float_as_uint(c0) & t) | (__float_as_uint(c1) & ~t));
+    const unsigned sign = (code << (30 - 2 * x)) & 0x80000000u;
+    ge += __uint_as_float(__float_as_uint(w) ^ sign);
   }
 };
 

@@ -30,7 +30,21 @@ extern template int score_dispatch<mBetaKL>(hipStream_t, const ScoreArgs&, int, 
 int entity_backward(int model, void* stream, const smx_plan_view* plan, float* table, size_t n_rows, const float* q1,
                     const float* q2, const float* score, const float* gscore, size_t B, size_t K, size_t dim,
                     const smx_score_params* params, float* merged, float* m, float* v, const smx_opt_params* adam,
-                    void* workspace, size_t workspace_bytes, int skip_single);
+                    void* workspace, size_t workspace_bytes, int skip_single, const unsigned char* codes, int codes_vec,
+                    int codes_nit);
+size_t entity_ws_bytes(size_t n_pairs, size_t row_len);
+size_t code_bytes_per_pair(size_t dim);
+
+// Sign codes are laid out for float4 columns when dim is a multiple of 4, single floats otherwise, and
+// exist for rows of up to 512 floats.  Returns null when (vec, nit) of this call fits that layout and
+// the buffer has the size smx_score_codes_bytes gives, else what is wrong.
+static const char* codes_mismatch(int model, size_t n_pairs, size_t dim, int vec, int nit, size_t codes_bytes) {
+  if (!model_coded(model)) return "this model has no sign codes";
+  if (vec != (dim % 4 == 0 ? 4 : 1)) return "sign codes need 16-byte aligned rows when dim is a multiple of 4";
+  if (nit > 2) return "sign codes exist for rows of up to 512 floats";
+  if (codes_bytes != n_pairs * code_bytes_per_pair(dim)) return "codes buffer is not smx_score_codes_bytes() long";
+  return nullptr;
+}
 
 static int dispatch_model(int model, hipStream_t st, const ScoreArgs& A, int vec, int nit, bool forward) {
   switch (model) {
@@ -80,14 +94,26 @@ static int fill_args(ScoreArgs* A, int* vec, int* nit, int model, const float* t
 
 extern "C" {
 
+size_t smx_score_codes_bytes(int model, size_t n_pairs, size_t dim) {
+  using namespace smx;
+  if (model < 0 || model >= mNumModels || !model_coded(model)) return 0;
+  const size_t per_pair = code_bytes_per_pair(dim);
+  return per_pair > 2 * 64 ? 0 : n_pairs * per_pair;
+}
+
 int smx_score_forward(int model, void* stream, const float* table, size_t n_rows, const int64_t* idx,
                       const float* q1, const float* q2, float* score, size_t B, size_t K, size_t dim,
-                      const smx_score_params* params, int* err_flag) {
+                      const smx_score_params* params, int* err_flag, void* codes, size_t codes_bytes) {
   using namespace smx;
   ScoreArgs A;
   int vec, nit;
   if (int rc = fill_args(&A, &vec, &nit, model, table, n_rows, idx, q1, q2, B, K, dim, params, nullptr, nullptr)) return rc;
   if (!score) return fail(SMX_ERR_ARG, "null score pointer");
+  if (codes) {
+    if (const char* msg = codes_mismatch(model, B * K, dim, vec, nit, codes_bytes)) return fail(SMX_ERR_ARG, "%s", msg);
+    if (reinterpret_cast<uintptr_t>(codes) & 15u) return fail(SMX_ERR_ARG, "codes must be 16-byte aligned");
+    A.codes = static_cast<unsigned char*>(codes);
+  }
   A.score_out = score;
   A.err = err_flag;
   return dispatch_model(model, as_stream(stream), A, vec, nit, true);
@@ -112,7 +138,8 @@ int smx_score_backward_fused(int model, void* stream, const smx_plan_view* plan,
                              const int64_t* idx, const float* q1, const float* q2, const float* score,
                              const float* gscore, float* gq1, float* gq2, size_t B, size_t K, size_t dim,
                              const smx_score_params* params, float* merged, float* m, float* v,
-                             const smx_opt_params* adam, void* workspace, size_t workspace_bytes) {
+                             const smx_opt_params* adam, void* workspace, size_t workspace_bytes,
+                             const void* fwd_codes, size_t fwd_codes_bytes) {
   using namespace smx;
   ScoreArgs A;
   int vec, nit;
@@ -147,9 +174,29 @@ int smx_score_backward_fused(int model, void* stream, const smx_plan_view* plan,
   if (adam) A.sink.a = make_adam_consts(adam);
   A.sink.p = A.p;
   A.sink.ncol = A.ncol;
+  // Sign codes (models that have them): when the entity pass would fetch query rows from beyond the L2,
+  // the query-gradient kernel leaves each pair's derivative decisions in the workspace behind the
+  // entity pass's own scratch, and the entity pass reads those instead of the query rows.  Used when
+  // the caller's workspace has the room (smx_fused_workspace_bytes).
+  const unsigned char* codes = nullptr;
+  if (fwd_codes) {
+    // the forward pass left the codes: neither the query-gradient kernel nor the entity pass needs the
+    // entity rows or the query rows for the derivative
+    if (const char* msg = codes_mismatch(model, B * K, dim, vec, nit, fwd_codes_bytes)) return fail(SMX_ERR_ARG, "%s", msg);
+    if (reinterpret_cast<uintptr_t>(fwd_codes) & 15u) return fail(SMX_ERR_ARG, "codes must be 16-byte aligned");
+    A.codes_in = static_cast<const unsigned char*>(fwd_codes);
+    codes = A.codes_in;
+  } else if (model_coded(model) && singles_here && workspace && nit <= 2) {  // rows of up to 512 floats
+    const size_t base = entity_ws_bytes(B * K, dim * model_mul(model));
+    const size_t need = (size_t)B * K * nit * 64;
+    if (workspace_bytes >= base + need) {
+      A.codes = static_cast<unsigned char*>(workspace) + base;
+      codes = A.codes;
+    }
+  }
   if (int rc = dispatch_model(model, as_stream(stream), A, vec, nit, false)) return rc;
   return entity_backward(model, stream, plan, table, n_rows, q1, q2, score, gscore, B, K, dim, params, merged, m, v,
-                         adam, workspace, workspace_bytes, singles_here ? 1 : 0);
+                         adam, workspace, workspace_bytes, singles_here ? 1 : 0, codes, vec, nit);
 }
 
 }  // extern "C"

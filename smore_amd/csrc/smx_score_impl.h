@@ -39,6 +39,8 @@ struct ScoreArgs {
   ScoreParams p;
   int* err;
   const int* pair_seg;   // one-pair segments finished by the query backward (SINGLES kernels)
+  unsigned char* codes;  // [B*K][NIT*64] sign codes written by this kernel (forward or query backward), or null
+  const unsigned char* codes_in;  // query backward: codes the forward left; the entity rows are then not read
   RowSink sink;
 };
 
@@ -209,7 +211,29 @@ __device__ __forceinline__ void stream_batch(const unsigned* slab, int cnt, int 
   }
 }
 
-template <int M, int VEC, int NIT, int RIF, bool REG>
+// Sign codes on their way to memory: a wavefront parks each pair's NIT x 64 code bytes in its LDS
+// stage and, every 16 pairs (and after the last one), writes the stage out with 16-byte stores -- the
+// 16 pairs are contiguous in the code array as well.
+constexpr int kStagePairs = 16;
+template <int NIT>
+__device__ __forceinline__ void flush_codes(const unsigned char* stage, unsigned char* codes, size_t first_pair, int j,
+                                            int cnt, int lane) {
+  if ((j & (kStagePairs - 1)) == kStagePairs - 1 || j == cnt - 1) {
+    slab_fence();
+    typedef unsigned vec4u __attribute__((ext_vector_type(4)));
+    const int rows_here = (j & (kStagePairs - 1)) + 1;
+    vec4u* out = reinterpret_cast<vec4u*>(codes + (first_pair + (j & ~(kStagePairs - 1))) * (size_t)(NIT * 64));
+#pragma unroll
+    for (int i = 0; i < NIT; ++i) {
+      const int chunk = lane + 64 * i;
+      if (chunk * 16 < rows_here * NIT * 64)
+        __builtin_nontemporal_store(reinterpret_cast<const vec4u*>(stage)[chunk], out + chunk);
+    }
+    slab_fence();
+  }
+}
+
+template <int M, int VEC, int NIT, int RIF, bool REG, bool CODED = false>
 __global__ __launch_bounds__(256) void score_forward_kernel(ScoreArgs A, int tiles, int tile_k) {
   const float* __restrict__ table = A.table;
   const long long* __restrict__ idx = A.idx;
@@ -245,6 +269,8 @@ __global__ __launch_bounds__(256) void score_forward_kernel(ScoreArgs A, int til
   stage_pairs(slab, lane, table, pb, 0.f, 0.f);
 
   float* out = score + (size_t)b * K + kw0;
+  unsigned char* stage =
+      reinterpret_cast<unsigned char*>(lds + model_nq(M) * dim + 4 * kSlabDwords) + wave * (kStagePairs * NIT * 64);
   stream_batch<MUL, VEC, NIT, RIF>(slab, cnt, dim, ncol, lane,
                                    [&](int j, const Pack<VEC>(&e1)[NIT], const Pack<VEC>(&e2)[NIT]) {
     // lanes past the row end hold a copy of the last column: they compute along and are dropped here.
@@ -253,17 +279,25 @@ __global__ __launch_bounds__(256) void score_forward_kernel(ScoreArgs A, int til
 #pragma unroll
     for (int it = 0; it < NIT; ++it) {
       float a0 = 0.f, a1 = 0.f;
+      if constexpr (CODED) {
+        unsigned code = 0;
 #pragma unroll
-      for (int v = 0; v < VEC; ++v) {
-        const float x1 = REG ? reg_apply(e1[it].v[v], p) : e1[it].v[v];
-        const float x2 = MUL == 2 ? (REG ? reg_apply(e2[it].v[v], p) : e2[it].v[v]) : 0.f;
-        ModelOps<M>::fwd(x1, x2, q[it][v], a0, a1);
+        for (int v = 0; v < VEC; ++v) ModelOps<M>::fwd_coded(e1[it].v[v], q[it][v], a0, a1, code);
+        stage[(j & (kStagePairs - 1)) * (NIT * 64) + 64 * it + lane] = (unsigned char)code;
+      } else {
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) {
+          const float x1 = REG ? reg_apply(e1[it].v[v], p) : e1[it].v[v];
+          const float x2 = MUL == 2 ? (REG ? reg_apply(e2[it].v[v], p) : e2[it].v[v]) : 0.f;
+          ModelOps<M>::fwd(x1, x2, q[it][v], a0, a1);
+        }
       }
       const float f = ModelOps<M>::fold(a0, a1, p);
       mine += lane + 64 * it < ncol ? f : 0.f;
     }
     const float folded = wave_sum_last_f32(mine);
     if (lane == 63) out[j] = ModelOps<M>::score(folded, p);
+    if constexpr (CODED) flush_codes<NIT>(stage, A.codes, (size_t)b * K + kw0, j, cnt, lane);
   });
   if (__ballot(bad != 0) != 0ull && err && lane == 0) *err = 1;
 }
@@ -274,7 +308,11 @@ __global__ __launch_bounds__(256) void score_forward_kernel(ScoreArgs A, int til
 // to the entity pass, which would have to fetch the query rows and the entity row again.
 // SINGLES: 0 = leave every segment to the entity pass, 1 = finish one-pair segments here as merged-gradient
 // rows, 2 = ... with Adam on w, m, v (and the merged row if asked for).
-template <int M, int VEC, int NIT, int RIF, int NW, bool REG, int SINGLES>
+// CODES (models with sign codes): 1 = also writes every pair's derivative decisions, one byte per lane
+// and column group, for the entity pass to use in place of the query rows; 2 = the forward pass left
+// the codes: the query gradient is summed from them and the entity rows are not read at all (except
+// those of the one-pair segments finished here).
+template <int M, int VEC, int NIT, int RIF, int NW, bool REG, int SINGLES, int CODES = 0>
 __global__ __launch_bounds__(NW * 64) void score_backward_query_kernel(ScoreArgs A) {
   const float* __restrict__ table = A.table;
   const long long* __restrict__ idx = A.idx;
@@ -307,6 +345,8 @@ __global__ __launch_bounds__(NW * 64) void score_backward_query_kernel(ScoreArgs
     for (int v = 0; v < VEC; ++v) g1[it][v] = g2[it][v] = 0.f;
   // LDS: query | per-wavefront partial sums | per-wavefront pair slabs
   unsigned* slab = reinterpret_cast<unsigned*>(lds + (NW + 1) * NQ * dim) + wave * kSlabDwords;
+  unsigned char* stage =
+      reinterpret_cast<unsigned char*>(lds + (NW + 1) * NQ * dim + NW * kSlabDwords) + wave * (kStagePairs * NIT * 64);
 
   // this wavefront's share of the query's negatives: a contiguous range, walked in batches of 64
   const int per_wave = (K + NW - 1) / NW;
@@ -320,52 +360,118 @@ __global__ __launch_bounds__(NW * 64) void score_backward_query_kernel(ScoreArgs
     const size_t mine = first + min(lane, cnt - 1);
     float my_c0, my_c1;
     ModelOps<M>::coef(gscore[mine], score[mine], p, my_c0, my_c1);
+    if constexpr (CODES == 2) {
+      // 8 pairs' code bytes requested at a time, two sets used in turn
+      constexpr int CB = 8;
+      const unsigned char* pc = A.codes_in + first * (size_t)(NIT * 64) + lane;
+      unsigned ca[CB][NIT], cb[CB][NIT];
+      auto request = [&](unsigned (&c)[CB][NIT], int j0) {
+#pragma unroll
+        for (int r = 0; r < CB; ++r) {
+          const int j = min(j0 + r, cnt - 1);
+#pragma unroll
+          for (int it = 0; it < NIT; ++it) c[r][it] = pc[(size_t)j * (NIT * 64) + 64 * it];
+        }
+      };
+      auto consume = [&](const unsigned (&c)[CB][NIT], int j0) {
+#pragma unroll
+        for (int r = 0; r < CB; ++r) {
+          if (j0 + r < cnt) {
+            const float c0 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(my_c0), j0 + r));
+            const float c1 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(my_c1), j0 + r));
+#pragma unroll
+            for (int it = 0; it < NIT; ++it)
+#pragma unroll
+              for (int v = 0; v < VEC; ++v)
+                ModelOps<M>::bwd_q_from_code(c0, c1, c[r][it], VEC - 1 - v, g1[it][v], g2[it][v]);
+          }
+        }
+      };
+      request(ca, 0);
+      for (int j0 = 0; j0 < cnt; j0 += 2 * CB) {
+        request(cb, j0 + CB);
+        consume(ca, j0);
+        request(ca, j0 + 2 * CB);
+        consume(cb, j0 + CB);
+      }
+    } else {
     stage_pairs(slab, lane, table, pb, my_c0, my_c1);
     // lanes past the row end hold a copy of the last column: what they accumulate is never stored
     stream_batch<MUL, VEC, NIT, RIF>(slab, cnt, dim, ncol, lane,
                                      [&](int j, const Pack<VEC>(&e1)[NIT], const Pack<VEC>(&e2)[NIT]) {
       const float2 c = slab_coef(slab, j);
+      if constexpr (CODES == 1) {
+        // the pair's code bytes go to the wavefront's LDS stage, see flush_codes
+        unsigned char* mine_b = stage + (j & (kStagePairs - 1)) * (NIT * 64) + lane;
 #pragma unroll
-      for (int it = 0; it < NIT; ++it) {
+        for (int it = 0; it < NIT; ++it) {
+          unsigned code = 0;
 #pragma unroll
-        for (int v = 0; v < VEC; ++v) {
-          const float x1 = REG ? reg_apply(e1[it].v[v], p) : e1[it].v[v];
-          const float x2 = MUL == 2 ? (REG ? reg_apply(e2[it].v[v], p) : e2[it].v[v]) : 0.f;
-          ModelOps<M>::bwd_q(c.x, c.y, x1, x2, q[it][v], g1[it][v], g2[it][v]);
+          for (int v = 0; v < VEC; ++v)
+            ModelOps<M>::bwd_q_coded(c.x, c.y, e1[it].v[v], q[it][v], g1[it][v], g2[it][v], code);
+          mine_b[64 * it] = (unsigned char)code;
+        }
+        flush_codes<NIT>(stage, A.codes, first, j, cnt, lane);
+      } else {
+#pragma unroll
+        for (int it = 0; it < NIT; ++it) {
+#pragma unroll
+          for (int v = 0; v < VEC; ++v) {
+            const float x1 = REG ? reg_apply(e1[it].v[v], p) : e1[it].v[v];
+            const float x2 = MUL == 2 ? (REG ? reg_apply(e2[it].v[v], p) : e2[it].v[v]) : 0.f;
+            ModelOps<M>::bwd_q(c.x, c.y, x1, x2, q[it][v], g1[it][v], g2[it][v]);
+          }
         }
       }
     });
+    }
 
     if constexpr (SINGLES != 0) {
-      // One row at a time per wavefront: with the registers this keeps free the kernel runs at full
-      // occupancy, and the other wavefronts of the CU cover the latency of the row loads.
+      // S rows at a time per wavefront (their w, m, v loads are all requested before the first is
+      // used): the row sets of the streaming loop are dead here, so this costs no extra registers, and
+      // it divides the memory latency each one-pair row would otherwise expose by S.
+      constexpr int S = NIT * MUL == 1 ? 3 : (NIT * MUL == 2 ? 2 : 1);
       const int my_ps = A.pair_seg[mine];
       unsigned long long todo = __ballot(lane < cnt && my_ps < 0);
       while (todo != 0ull) {
-        const int j = __builtin_ctzll(todo);
-        todo &= todo - 1;
-        const unsigned long long off = batch_off(pb, j);
-        RowRegs<MUL, VEC, NIT> e, m0, v0;
-        load_row<MUL, VEC, NIT>(e, table + off, dim, ncol, lane);
-        if constexpr (SINGLES == 2) {
-          if (A.sink.adam_on == kOptAdam) load_row<MUL, VEC, NIT, true>(m0, A.sink.m + off, dim, ncol, lane);
-          if (A.sink.adam_on != kOptSgd && !A.sink.squeeze) load_row<MUL, VEC, NIT, true>(v0, A.sink.v + off, dim, ncol, lane);
-        }
-        const float c0 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(my_c0), j));
-        const float c1 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(my_c1), j));
-        const int seg = __builtin_amdgcn_readlane(my_ps, j) & 0x7fffffff;
-        const unsigned row = (unsigned)__builtin_amdgcn_readlane((int)pb.row, j);
-        float ge1[NIT][VEC], ge2[NIT][VEC];
+        int js[S];
+        RowRegs<MUL, VEC, NIT> e[S], m0[S], v0[S];
 #pragma unroll
-        for (int it = 0; it < NIT; ++it)
-#pragma unroll
-          for (int v = 0; v < VEC; ++v) {
-            ge1[it][v] = ge2[it][v] = 0.f;
-            const float x1 = REG ? reg_apply(e.h[0][it].v[v], p) : e.h[0][it].v[v];
-            const float x2 = MUL == 2 ? (REG ? reg_apply(e.h[MUL - 1][it].v[v], p) : e.h[MUL - 1][it].v[v]) : 0.f;
-            ModelOps<M>::bwd_e(c0, c1, x1, x2, q[it][v], ge1[it][v], ge2[it][v]);
+        for (int s = 0; s < S; ++s) {
+          js[s] = todo != 0ull ? __builtin_ctzll(todo) : -1;
+          if (js[s] >= 0) {  // wave-uniform
+            todo &= todo - 1;
+            const unsigned long long off = batch_off(pb, js[s]);
+            load_row<MUL, VEC, NIT>(e[s], table + off, dim, ncol, lane);
+            if constexpr (SINGLES == 2) {
+              if (A.sink.adam_on == kOptAdam) load_row<MUL, VEC, NIT, true>(m0[s], A.sink.m + off, dim, ncol, lane);
+              if (A.sink.adam_on != kOptSgd && !A.sink.squeeze)
+                load_row<MUL, VEC, NIT, true>(v0[s], A.sink.v + off, dim, ncol, lane);
+            }
           }
-        finish_row<M, VEC, NIT, REG, SINGLES == 2>(A.sink, lane, row, seg, ge1, ge2, e, m0, v0);
+        }
+#pragma unroll
+        for (int s = 0; s < S; ++s) {
+          if (js[s] >= 0) {
+            const int j = js[s];
+            const float c0 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(my_c0), j));
+            const float c1 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(my_c1), j));
+            const int seg = __builtin_amdgcn_readlane(my_ps, j) & 0x7fffffff;
+            const unsigned row = (unsigned)__builtin_amdgcn_readlane((int)pb.row, j);
+            float ge1[NIT][VEC], ge2[NIT][VEC];
+#pragma unroll
+            for (int it = 0; it < NIT; ++it)
+#pragma unroll
+              for (int v = 0; v < VEC; ++v) {
+                ge1[it][v] = ge2[it][v] = 0.f;
+                const float x1 = REG ? reg_apply(e[s].h[0][it].v[v], p) : e[s].h[0][it].v[v];
+                const float x2 =
+                    MUL == 2 ? (REG ? reg_apply(e[s].h[MUL - 1][it].v[v], p) : e[s].h[MUL - 1][it].v[v]) : 0.f;
+                ModelOps<M>::bwd_e(c0, c1, x1, x2, q[it][v], ge1[it][v], ge2[it][v]);
+              }
+            finish_row<M, VEC, NIT, REG, SINGLES == 2>(A.sink, lane, row, seg, ge1, ge2, e[s], m0[s], v0[s]);
+          }
+        }
       }
     }
   }
@@ -415,6 +521,13 @@ int launch_forward_reg(hipStream_t st, const ScoreArgs& A) {
   while (tile_k > 4 * RIF && (B * ((K + tile_k - 1) / tile_k) < 8192 || (size_t)tile_k / 2 >= K)) tile_k /= 2;
   const int tiles = (int)((K + tile_k - 1) / tile_k);
   const size_t lds = ((size_t)model_nq(M) * A.ncol * VEC + 4 * kSlabDwords) * sizeof(float);
+  if constexpr (model_coded(M) && !REG) {
+    if (A.codes) {
+      hipLaunchKernelGGL((score_forward_kernel<M, VEC, NIT, RIF, REG, true>), dim3((unsigned)(B * tiles)), dim3(256),
+                         lds + 4 * kStagePairs * NIT * 64, st, A, tiles, tile_k);
+      return check_launch("score forward (coded)");
+    }
+  }
   hipLaunchKernelGGL((score_forward_kernel<M, VEC, NIT, RIF, REG>), dim3((unsigned)(B * tiles)), dim3(256), lds, st, A,
                      tiles, tile_k);
   return check_launch("score forward");
@@ -424,6 +537,30 @@ template <int M, int VEC, int NIT, int NW, bool REG>
 int launch_backward_query_reg(hipStream_t st, const ScoreArgs& A) {
   constexpr int RIF = rows_in_flight(NIT, model_mul(M));
   const size_t lds = ((size_t)(NW + 1) * model_nq(M) * A.ncol * VEC + NW * kSlabDwords) * sizeof(float);
+  if constexpr (model_coded(M) && !REG) {
+    if (A.codes_in) {
+      if (A.pair_seg && A.sink.adam_on)
+        hipLaunchKernelGGL((score_backward_query_kernel<M, VEC, NIT, RIF, NW, REG, 2, 2>), dim3((unsigned)A.B),
+                           dim3(NW * 64), lds, st, A);
+      else if (A.pair_seg)
+        hipLaunchKernelGGL((score_backward_query_kernel<M, VEC, NIT, RIF, NW, REG, 1, 2>), dim3((unsigned)A.B),
+                           dim3(NW * 64), lds, st, A);
+      else
+        hipLaunchKernelGGL((score_backward_query_kernel<M, VEC, NIT, RIF, NW, REG, 0, 2>), dim3((unsigned)A.B),
+                           dim3(NW * 64), lds, st, A);
+      return check_launch("score backward (query, from codes)");
+    }
+    if (A.codes && A.pair_seg) {
+      const size_t lds_coded = lds + (size_t)NW * kStagePairs * NIT * 64;
+      if (A.sink.adam_on)
+        hipLaunchKernelGGL((score_backward_query_kernel<M, VEC, NIT, RIF, NW, REG, 2, 1>), dim3((unsigned)A.B),
+                           dim3(NW * 64), lds_coded, st, A);
+      else
+        hipLaunchKernelGGL((score_backward_query_kernel<M, VEC, NIT, RIF, NW, REG, 1, 1>), dim3((unsigned)A.B),
+                           dim3(NW * 64), lds_coded, st, A);
+      return check_launch("score backward (query, coded)");
+    }
+  }
   if (A.pair_seg && A.sink.adam_on)
     hipLaunchKernelGGL((score_backward_query_kernel<M, VEC, NIT, RIF, NW, REG, 2>), dim3((unsigned)A.B),
                        dim3(NW * 64), lds, st, A);

@@ -73,13 +73,25 @@ def _dims(model, table, idx, q1, q2):
     return b, k, dim
 
 
-def score_forward(model, table, idx, q1, q2, params, err_flag=None):
-    """logit[b,k] = gamma - dist(table[idx[b,k]], q[b]).  idx None: table is the dense [B*K, row] rows."""
+def new_codes(model, table, idx, q1):
+    """Buffer for the sign codes of one step (see smx_score_codes_bytes), or None when the model or the
+    row length has none.  Pass it to score_forward and, unchanged, to score_backward_fused."""
+    if model not in MODELS:
+        raise _lib.SmxError(f"unknown score model {model}")
+    n_pairs = idx.numel() if idx is not None else table.shape[0]
+    nbytes = _lib.load().smx_score_codes_bytes(MODELS[model], n_pairs, q1.shape[-1])
+    return torch.empty(nbytes, dtype=torch.uint8, device=table.device) if nbytes else None
+
+
+def score_forward(model, table, idx, q1, q2, params, err_flag=None, codes=None):
+    """logit[b,k] = gamma - dist(table[idx[b,k]], q[b]).  idx None: table is the dense [B*K, row] rows.
+    codes: buffer from new_codes() that receives the step's sign codes."""
     b, k, dim = _dims(model, table, idx, q1, q2)
     score = torch.empty((b, k), dtype=torch.float32, device=table.device)
     with torch.cuda.device(table.device):
         _lib.call("smx_score_forward", MODELS[model], _stream(table), _ptr(table), table.shape[0], _ptr(idx),
-                  _ptr(q1), _ptr(q2), _ptr(score), b, k, dim, ctypes.byref(params), _ptr(err_flag))
+                  _ptr(q1), _ptr(q2), _ptr(score), b, k, dim, ctypes.byref(params), _ptr(err_flag),
+                  _ptr(codes), 0 if codes is None else codes.numel())
     return score
 
 
@@ -210,9 +222,12 @@ def score_backward_entity(model, plan, table, q1, q2, score, gscore, params, mer
 
 
 def score_backward_fused(model, plan, table, idx, q1, q2, score, gscore, params, merged=None, m=None, v=None,
-                         adam=None):
+                         adam=None, sign_codes=True, codes=None):
     """Query gradients and all entity rows of the step in one call (see smx_score_backward_fused).
-    Returns (gq1, gq2); merged / table, m, v are written in place as in score_backward_entity."""
+    Returns (gq1, gq2); merged / table, m, v are written in place as in score_backward_entity.
+    codes: the buffer score_forward filled for these pairs (table and queries unchanged since).
+    sign_codes=False gives the call only the entity pass's own workspace, which keeps the box model on
+    the path that re-reads the query rows (same results; for tests and comparison)."""
     b, k, dim = _dims(model, table, idx, q1, q2)
     for t, name in ((score, "score"), (gscore, "gscore"), (merged, "merged"), (m, "m"), (v, "v")):
         _f32(t, name)
@@ -224,12 +239,16 @@ def score_backward_fused(model, plan, table, idx, q1, q2, score, gscore, params,
     gq1 = torch.empty_like(q1)
     gq2 = None if q2 is None else torch.empty_like(q2)
     with torch.cuda.device(table.device):
-        ws = _workspace(_lib.load().smx_entity_workspace_bytes(plan.n_pairs, table.shape[1]), table.device)
+        ws_bytes = _lib.load().smx_fused_workspace_bytes(MODELS[model], plan.n_pairs, dim) \
+            if sign_codes and codes is None else \
+            _lib.load().smx_entity_workspace_bytes(plan.n_pairs, table.shape[1])
+        ws = _workspace(ws_bytes, table.device)
         view = plan.view()
         _lib.call("smx_score_backward_fused", MODELS[model], _stream(table), ctypes.byref(view), _ptr(table),
                   table.shape[0], _ptr(idx), _ptr(q1), _ptr(q2), _ptr(score), _ptr(gscore), _ptr(gq1), _ptr(gq2),
                   b, k, dim, ctypes.byref(params), _ptr(merged), _ptr(m), _ptr(v),
-                  None if adam is None else ctypes.byref(adam), _ptr(ws), ws.numel())
+                  None if adam is None else ctypes.byref(adam), _ptr(ws), ws.numel(),
+                  _ptr(codes), 0 if codes is None else codes.numel())
     return gq1, gq2
 
 

@@ -320,6 +320,106 @@ def test_one_call_backward_with_many_queries_takes_the_one_pair_shortcut():
     assert_close(merged_b.cpu().numpy(), merged_a.cpu().numpy(), 1e-6, "merged")
 
 
+@pytest.mark.parametrize("dim", [128, 400, 30])
+def test_sign_codes_give_the_bits_of_the_query_row_path(dim):
+    """With many queries the box backward leaves per-pair sign codes for the entity pass
+    (smx_fused_workspace_bytes); without the extra workspace the entity pass re-reads the query rows.
+    Both sum the same +-c terms in the same order: the merged rows must be equal bit for bit, long
+    segments, repeated (entity, query) pairs and all."""
+    from smore_amd import fused
+    rng = np.random.default_rng(dim)
+    b = (4 << 20) // (2 * 4 * dim) + 64
+    n, k = 3000, 6
+    table, q1, q2, idx, gs = make_problem("box", n, b, k, dim, rng, zipf=1.2)
+    idx[::3, 1] = idx[::3, 0]            # the same entity twice under one query
+    t_table, t_q1, t_q2, t_gs = dev(table), dev(q1), dev(q2), dev(gs)
+    t_idx = torch.tensor(idx, device="cuda")
+    params = fused.score_params(24.0, 0.02)
+    plan = fused.build_plan(t_idx, n)
+    score = fused.score_forward("box", t_table, t_idx, t_q1, t_q2, params)
+    saved = fused.new_codes("box", t_table, t_idx, t_q1)
+    assert saved is not None and saved.numel() == b * k * 64 * (2 if dim == 400 else 1)
+    score_saving = fused.score_forward("box", t_table, t_idx, t_q1, t_q2, params, codes=saved)
+    assert torch.equal(score_saving, score)
+    out = {}
+    for codes in (False, True, "forward"):
+        merged = torch.full((plan.n_uniq, dim), float("nan"), device="cuda")
+        g1, g2 = fused.score_backward_fused("box", plan, t_table, t_idx, t_q1, t_q2, score, t_gs, params,
+                                            merged=merged, sign_codes=codes is True,
+                                            codes=saved if codes == "forward" else None)
+        out[codes] = (merged.cpu().numpy(), g1.cpu().numpy(), g2.cpu().numpy())
+    for how in (True, "forward"):
+        assert np.array_equal(out[how][0], out[False][0]), how
+        assert_close(out[how][1], out[False][1], 1e-6, "gq1")
+        assert_close(out[how][2], out[False][2], 1e-6, "gq2")
+    # Adam from the forward's codes against Adam from the recomputed derivative
+    state = {}
+    for how in (False, "forward"):
+        w, m, v = t_table.clone(), torch.zeros_like(t_table), torch.zeros_like(t_table)
+        fused.score_backward_fused("box", plan, w, t_idx, t_q1, t_q2, score, t_gs, params, m=m, v=v,
+                                   adam=fused.adam_params(1e-3, 1), sign_codes=False,
+                                   codes=saved if how == "forward" else None)
+        state[how] = (w.cpu().numpy(), m.cpu().numpy(), v.cpu().numpy())
+    for a, b_, what in zip(state["forward"], state[False], "wmv"):
+        assert_close(a, b_, 2e-6, what)
+    g_rows, _, _ = orc.score_backward("box", gs, table[idx], q1[:, None], q2[:, None], 0.02)
+    uniq, inv = np.unique(idx.reshape(-1), return_inverse=True)
+    want = np.zeros((len(uniq), dim))
+    np.add.at(want, inv, g_rows.reshape(-1, dim))
+    sum_abs = np.zeros((len(uniq), dim))
+    np.add.at(sum_abs, inv, np.abs(g_rows.reshape(-1, dim)))
+    assert_close(out[True][0], want, REL_F32, "merged vs oracle", sum_abs=sum_abs)
+
+
+def test_sign_codes_keep_the_tie_conventions():
+    """Ties (e == c, |e - c| == o, negative offsets) through the coded path: every pair of the tie table,
+    under enough queries for the codes to be used, must give the oracle's rows exactly."""
+    from smore_amd import fused
+    cases = [  # e, c, o
+        (1.0, 0.75, 0.25), (1.0, 0.75, 0.5), (1.0, 1.0, 0.0), (0.5, 0.75, 0.5), (1.0, 0.75, -0.5),
+        (1.0, 1.0, 0.5), (0.25, 0.75, 0.25), (1.0, 1.0, -0.5), (0.75, 1.0, 0.0), (-0.0, 0.0, 0.0), (0.0, -0.0, 0.5),
+    ]
+    nc = len(cases)
+    reps = (4 << 20) // (2 * 4 * 4 * nc) + 8
+    b = nc * reps
+    table = np.array([[e] * 4 for e, _, _ in cases], dtype=np.float64)
+    q1 = np.tile(np.array([[c] * 4 for _, c, _ in cases], dtype=np.float64), (reps, 1))
+    q2 = np.tile(np.array([[o] * 4 for _, _, o in cases], dtype=np.float64), (reps, 1))
+    idx = np.tile(np.arange(nc, dtype=np.int64), reps)[:, None]            # query i meets entity i % nc
+    gs = np.random.default_rng(3).integers(1, 4, (b, 1)).astype(np.float64)  # small integers: sums are exact
+    params = fused.score_params(24.0, 0.5)
+    t_table, t_q1, t_q2, t_gs = dev(table), dev(q1), dev(q2), dev(gs)
+    t_idx = torch.tensor(idx, device="cuda")
+    plan = fused.build_plan(t_idx, nc)
+    score = fused.score_forward("box", t_table, t_idx, t_q1, t_q2, params)
+    g_rows, g_c, g_o = orc.score_backward("box", gs, table[idx], q1[:, None], q2[:, None], 0.5)
+    want = np.zeros((nc, 4))
+    np.add.at(want, idx.reshape(-1), g_rows.reshape(-1, 4))
+    saved = fused.new_codes("box", t_table, t_idx, t_q1)
+    assert torch.equal(fused.score_forward("box", t_table, t_idx, t_q1, t_q2, params, codes=saved), score)
+    for codes in (None, saved):   # codes made by the query-gradient kernel / by the forward
+        merged = torch.empty((nc, 4), device="cuda")
+        g1, g2 = fused.score_backward_fused("box", plan, t_table, t_idx, t_q1, t_q2, score, t_gs, params,
+                                            merged=merged, codes=codes)
+        assert np.array_equal(merged.cpu().numpy().astype(np.float64), want)
+        assert np.array_equal(g1.cpu().numpy().astype(np.float64), g_c[:, 0])
+        assert np.array_equal(g2.cpu().numpy().astype(np.float64), g_o[:, 0])
+
+
+def test_sign_codes_are_refused_where_they_do_not_exist():
+    from smore_amd import fused
+    t = torch.zeros(10, 8, device="cuda")
+    q = torch.zeros(2, 8, device="cuda")
+    idx = torch.zeros(2, 3, dtype=torch.int64, device="cuda")
+    assert fused.new_codes("l2", t, idx, q) is None
+    assert fused.new_codes("box", torch.zeros(10, 2048, device="cuda"), idx, torch.zeros(2, 2048, device="cuda")) is None
+    buf = torch.zeros(2 * 3 * 64, dtype=torch.uint8, device="cuda")
+    with pytest.raises(Exception, match="no sign codes"):
+        fused.score_forward("l2", t, idx, q, None, fused.score_params(1.0), codes=buf)
+    with pytest.raises(Exception, match="smx_score_codes_bytes"):
+        fused.score_forward("box", t, idx, q, q, fused.score_params(1.0), codes=buf[:64])
+
+
 @pytest.mark.parametrize("kind", ["adam", "sgd", "adagrad", "rmsprop"])
 @pytest.mark.parametrize("squeeze", [False, True])
 def test_fused_entity_pass_with_every_optimizer(kind, squeeze):
