@@ -163,7 +163,10 @@ int smx_score_backward_fused(int model, void* stream, const smx_plan_view* plan,
   // fetch their query rows from beyond the L2: that is when the query tensors of the step are larger
   // than one XCD's 4 MiB L2 (measured: faster for 4096 queries x 2 x 200 floats, slower for 1024
   // queries x 2 x 400 or 500).  Otherwise every segment goes through the entity pass.
-  const bool singles_here = (size_t)B * dim * model_nq(model) * sizeof(float) > ((size_t)4 << 20);
+  // Without an optimizer the one-pair rows cost the query-gradient kernel one store each (nothing to
+  // fetch), so they are always finished there.
+  const bool q_beyond_l2 = (size_t)B * dim * model_nq(model) * sizeof(float) > ((size_t)4 << 20);
+  const bool singles_here = !adam || q_beyond_l2;
   A.pair_seg = singles_here ? plan->pair_seg : nullptr;
   A.sink.table = table;
   A.sink.m = m;
@@ -186,7 +189,7 @@ int smx_score_backward_fused(int model, void* stream, const smx_plan_view* plan,
     if (reinterpret_cast<uintptr_t>(fwd_codes) & 15u) return fail(SMX_ERR_ARG, "codes must be 16-byte aligned");
     A.codes_in = static_cast<const unsigned char*>(fwd_codes);
     codes = A.codes_in;
-  } else if (model_coded(model) && singles_here && workspace && nit <= 2) {  // rows of up to 512 floats
+  } else if (model_coded(model) && q_beyond_l2 && workspace && nit <= 2) {  // rows of up to 512 floats
     const size_t base = entity_ws_bytes(B * K, dim * model_mul(model));
     const size_t need = (size_t)B * K * nit * 64;
     if (workspace_bytes >= base + need) {

@@ -360,6 +360,15 @@ __global__ __launch_bounds__(NW * 64) void score_backward_query_kernel(ScoreArgs
     const size_t mine = first + min(lane, cnt - 1);
     float my_c0, my_c1;
     ModelOps<M>::coef(gscore[mine], score[mine], p, my_c0, my_c1);
+    int my_ps = 0;
+    unsigned long long singles = 0ull;  // pairs of the batch that are a segment of their own
+    if constexpr (SINGLES != 0) {
+      my_ps = A.pair_seg[mine];
+      singles = __ballot(lane < cnt && my_ps < 0);
+    }
+    // Without optimizer state to fetch, such a pair's row is finished the moment it streams by: its entity
+    // row and query are in registers, the merged-gradient row is one more store.
+    constexpr bool kInStream = SINGLES == 1 && CODES != 2;
     if constexpr (CODES == 2) {
       // 8 pairs' code bytes requested at a time, two sets used in turn
       constexpr int CB = 8;
@@ -423,16 +432,35 @@ __global__ __launch_bounds__(NW * 64) void score_backward_query_kernel(ScoreArgs
           }
         }
       }
+      if constexpr (kInStream) {
+        if ((singles >> j) & 1ull) {  // wave-uniform
+          RowRegs<MUL, VEC, NIT> w, none;
+          float ge1[NIT][VEC], ge2[NIT][VEC];
+#pragma unroll
+          for (int it = 0; it < NIT; ++it)
+#pragma unroll
+            for (int v = 0; v < VEC; ++v) {
+              w.h[0][it].v[v] = e1[it].v[v];
+              if (MUL == 2) w.h[MUL - 1][it].v[v] = e2[it].v[v];
+              ge1[it][v] = ge2[it][v] = 0.f;
+              const float x1 = REG ? reg_apply(e1[it].v[v], p) : e1[it].v[v];
+              const float x2 = MUL == 2 ? (REG ? reg_apply(e2[it].v[v], p) : e2[it].v[v]) : 0.f;
+              ModelOps<M>::bwd_e(c.x, c.y, x1, x2, q[it][v], ge1[it][v], ge2[it][v]);
+            }
+          const int seg = __builtin_amdgcn_readlane(my_ps, j) & 0x7fffffff;
+          const unsigned row = (unsigned)__builtin_amdgcn_readlane((int)pb.row, j);
+          finish_row<M, VEC, NIT, REG, false>(A.sink, lane, row, seg, ge1, ge2, w, none, none);
+        }
+      }
     });
     }
 
-    if constexpr (SINGLES != 0) {
+    if constexpr (SINGLES != 0 && !kInStream) {
       // S rows at a time per wavefront (their w, m, v loads are all requested before the first is
       // used): the row sets of the streaming loop are dead here, so this costs no extra registers, and
       // it divides the memory latency each one-pair row would otherwise expose by S.
       constexpr int S = NIT * MUL == 1 ? 3 : (NIT * MUL == 2 ? 2 : 1);
-      const int my_ps = A.pair_seg[mine];
-      unsigned long long todo = __ballot(lane < cnt && my_ps < 0);
+      unsigned long long todo = singles;
       while (todo != 0ull) {
         int js[S];
         RowRegs<MUL, VEC, NIT> e[S], m0[S], v0[S];
