@@ -462,20 +462,37 @@ __global__ __launch_bounds__(NW * 64) void entity_fixup_kernel(EntityArgs A) {
   }
 }
 
+// Workgroups of 256 threads of `kernel` the current device keeps resident (asked once per kernel).
+template <class K>
+unsigned resident_blocks(K kernel) {
+  static unsigned cached = 0;  // one value per instantiation, i.e. per kernel
+  if (cached == 0) {
+    int dev = 0, cus = 0, per_cu = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+        hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, 256, 0) != hipSuccess || cus <= 0 || per_cu <= 0)
+      return 256u * 8u;
+    cached = (unsigned)cus * (unsigned)per_cu;
+  }
+  return cached;
+}
+
 template <int SRC, int VEC, int NIT, bool REG>
 int launch_entity_reg(hipStream_t st, const EntityArgs& A) {
   const unsigned tiles = (unsigned)((A.n_pairs + A.tile - 1) / A.tile);
   // short segments: a fixed grid of wavefronts strides over the segment list (its length lives on the device)
-  unsigned seg_blocks = (unsigned)((A.n_pairs + 3) / 4);
-  if (seg_blocks > 256u * 8u) seg_blocks = 256u * 8u;
+  // (as many workgroups as the chip holds at once: a second wave of workgroups would run half empty)
+  const unsigned want_blocks = (unsigned)((A.n_pairs + 255) / 256);
   bool coded = false;
   if constexpr (SRC != kSrcRows && model_coded(SRC) && !REG) coded = A.codes != nullptr;
   if (coded) {
     if constexpr (SRC != kSrcRows && model_coded(SRC) && !REG) {
+      const unsigned seg_blocks = min(want_blocks, resident_blocks(entity_segment_kernel<SRC, VEC, NIT, REG, true>));
       hipLaunchKernelGGL((entity_segment_kernel<SRC, VEC, NIT, REG, true>), dim3(seg_blocks), dim3(256), 0, st, A);
       hipLaunchKernelGGL((entity_tile_kernel<SRC, VEC, NIT, REG, true>), dim3((tiles + 3) / 4), dim3(256), 0, st, A);
     }
   } else {
+    const unsigned seg_blocks = min(want_blocks, resident_blocks(entity_segment_kernel<SRC, VEC, NIT, REG>));
     hipLaunchKernelGGL((entity_segment_kernel<SRC, VEC, NIT, REG>), dim3(seg_blocks), dim3(256), 0, st, A);
     hipLaunchKernelGGL((entity_tile_kernel<SRC, VEC, NIT, REG>), dim3((tiles + 3) / 4), dim3(256), 0, st, A);
   }

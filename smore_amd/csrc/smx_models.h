@@ -208,21 +208,24 @@ template <> struct ModelOps<mBox> {
     const unsigned long long T = __ballot(a >= q.b), GT = __ballot(d > 0.f), GE = __ballot(d >= 0.f);
     code = push2(code, ~((T & GT) | (~T & GE)), T);
   }
+  // (t ? c0 : c1) with its sign flipped when the feature's "negative" bit is set: two three-input bit
+  // operations (v_bitop3_b32; table index = src0 << 2 | src1 << 1 | src2).
+  static __device__ __forceinline__ float signed_pick(float c0, float c1, unsigned t, unsigned code, int x) {
+    const unsigned w = __builtin_amdgcn_bitop3_b32(t, __float_as_uint(c0), __float_as_uint(c1), 0xCA);  // t ? c0 : c1
+    const unsigned top = code << (30 - 2 * x);                                    // "negative" bit in bit 31
+    return __uint_as_float(__builtin_amdgcn_bitop3_b32(w, top, 0x80000000u, 0x78));  // w ^ (top & sign bit)
+  }
   // Query side from a code byte: gc -= derivative of the feature at position x, go += c0 where the pair is outside.
   static __device__ __forceinline__ void bwd_q_from_code(float c0, float c1, unsigned code, int x, float& gc,
                                                          float& go) {
     const unsigned t = (unsigned)__builtin_amdgcn_sbfe((int)code, 2 * x, 1);  // 0 or ~0
-    const float w = __uint_as_float((__float_as_uint(c0) & t) | (__float_as_uint(c1) & ~t));
-    const unsigned sign = (code << (30 - 2 * x)) & 0x80000000u;
-    gc -= __uint_as_float(__float_as_uint(w) ^ sign);
+    gc -= signed_pick(c0, c1, t, code, x);
     go += __uint_as_float(__float_as_uint(c0) & t);
   }
   // ge += derivative of the feature at position x of the lane's code byte
   static __device__ __forceinline__ void bwd_e_coded(float c0, float c1, unsigned code, int x, float& ge) {
     const unsigned t = (unsigned)__builtin_amdgcn_sbfe((int)code, 2 * x, 1);  // 0 or ~0
-    const float w = __uint_as_float((__float_as_uint(c0) & t) | (__float_as_uint(c1) & ~t));
-    const unsigned sign = (code << (30 - 2 * x)) & 0x80000000u;
-    ge += __uint_as_float(__float_as_uint(w) ^ sign);
+    ge += signed_pick(c0, c1, t, code, x);
   }
 };
 
