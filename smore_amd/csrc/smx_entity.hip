@@ -43,7 +43,7 @@ constexpr int kShortMax = 64;   // longest segment one wavefront finishes on its
 static size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
 
 struct EntityScratch {
-  size_t tail_off, head_off, total;
+  size_t tail_off, head_off, fix_off, total;
 };
 
 static EntityScratch entity_scratch(size_t n_pairs, size_t row_len) {
@@ -51,7 +51,8 @@ static EntityScratch entity_scratch(size_t n_pairs, size_t row_len) {
   EntityScratch s;
   s.tail_off = 0;
   s.head_off = align256(tiles * row_len * sizeof(float));
-  s.total = s.head_off + align256(tiles * row_len * sizeof(float));
+  s.fix_off = s.head_off + align256(tiles * row_len * sizeof(float));
+  s.total = s.fix_off + align256(tiles);
   return s;
 }
 
@@ -87,6 +88,7 @@ static int fill_plan(EntityArgs* A, const smx_plan_view* plan, void* workspace, 
   char* ws = static_cast<char*>(workspace);
   A->tail = reinterpret_cast<float*>(ws + sc.tail_off);
   A->head = reinterpret_cast<float*>(ws + sc.head_off);
+  A->fix = reinterpret_cast<unsigned char*>(ws + sc.fix_off);
   return SMX_OK;
 }
 

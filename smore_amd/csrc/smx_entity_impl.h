@@ -53,6 +53,7 @@ struct EntityArgs : RowSink {
   const float* grad_rows;
   float* tail;    // [tiles, row_len] partial rows of long segments
   float* head;    // [tiles, row_len]
+  unsigned char* fix;  // [tiles] 1 where the fix-up pass has a segment to finish (written by the tile pass)
   int skip_single;  // segments of one pair were already finished by the query-backward kernel
   // sign codes written by the query-backward kernel, [n_pairs][NIT*64] bytes, or null (CODED kernels)
   const unsigned char* codes;
@@ -316,6 +317,11 @@ __global__ __launch_bounds__(256) void entity_tile_kernel(EntityArgs A) {
   const int p0 = t * A.tile;
   if (p0 >= A.n_pairs) return;  // whole wavefront leaves; no workgroup barrier is used below
   const int p1 = min(A.n_pairs, p0 + A.tile);
+  {  // does a long segment that came in from the left end inside this tile?  The fix-up pass finishes it.
+    const int sg = A.seg_of_pos[p0];
+    const int b0 = A.seg_start[sg], b1 = A.seg_start[sg + 1];
+    if (lane == 0) A.fix[t] = (p0 > 0 && b0 < p0 && b1 <= p1 && b1 - b0 > A.short_max) ? 1 : 0;
+  }
 
   // most tiles hold short segments only: find that out with one parallel look and leave
   bool any_long = false;
@@ -376,11 +382,9 @@ __global__ __launch_bounds__(NW * 64) void entity_fixup_kernel(EntityArgs A) {
   extern __shared__ float lds[];
   const int t = blockIdx.x;
   const int p0 = t * A.tile;
-  if (p0 == 0 || p0 >= A.n_pairs) return;
-  const int p1 = min(A.n_pairs, p0 + A.tile);
+  if (p0 == 0 || p0 >= A.n_pairs || A.fix[t] == 0) return;  // uniform over the workgroup; one byte decides
   const int seg = A.seg_of_pos[p0];
-  const int s0 = A.seg_start[seg], s1 = A.seg_start[seg + 1];
-  if (!(s0 < p0 && s1 <= p1 && s1 - s0 > A.short_max)) return;  // uniform over the workgroup
+  const int s0 = A.seg_start[seg];
   const int lane = threadIdx.x & 63;
   const int wave = uniform(threadIdx.x >> 6);
   const int half = A.ncol * VEC;
@@ -393,7 +397,7 @@ __global__ __launch_bounds__(NW * 64) void entity_fixup_kernel(EntityArgs A) {
 
   // a few interleaved partial sums per wavefront keep several row loads in flight; they are folded
   // in a fixed order, so the result depends only on the tiling
-  constexpr int ILP = NIT * MUL <= 2 ? 4 : (NIT * MUL <= 4 ? 2 : 1);
+  constexpr int ILP = NIT * MUL == 1 ? 8 : (NIT * MUL == 2 ? 4 : (NIT * MUL <= 4 ? 2 : 1));
   float acc[ILP][MUL][NIT][VEC];
 #pragma unroll
   for (int k = 0; k < ILP; ++k)
@@ -497,8 +501,8 @@ int launch_entity_reg(hipStream_t st, const EntityArgs& A) {
     hipLaunchKernelGGL((entity_tile_kernel<SRC, VEC, NIT, REG>), dim3((tiles + 3) / 4), dim3(256), 0, st, A);
   }
   const size_t row_bytes = (size_t)A.ncol * VEC * src_mul(SRC) * sizeof(float);
-  if (15 * row_bytes <= 60 * 1024)
-    hipLaunchKernelGGL((entity_fixup_kernel<SRC, VEC, NIT, 16, REG>), dim3(tiles), dim3(16 * 64), 15 * row_bytes, st, A);
+  if (7 * row_bytes <= 60 * 1024)
+    hipLaunchKernelGGL((entity_fixup_kernel<SRC, VEC, NIT, 8, REG>), dim3(tiles), dim3(8 * 64), 7 * row_bytes, st, A);
   else
     hipLaunchKernelGGL((entity_fixup_kernel<SRC, VEC, NIT, 4, REG>), dim3(tiles), dim3(4 * 64), 3 * row_bytes, st, A);
   return check_launch("entity backward");
