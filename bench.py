@@ -26,7 +26,7 @@ HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E bandwidth
 # row copy of known size (`bench.py --calibrate-copy`: FETCH_SIZE x1.942, WRITE_SIZE x1.000).  A counter
 # cannot be read from inside this process, so the figures are those of the profile summary
 # pmc_traffic_<workload>.md kept with the other rocprofv3 summaries; workloads not profiled report null.
-MEASURED_BACKWARD_TRAFFIC = {"cfg5-box-adam-86m-zipf1.1": 7.53e9}
+MEASURED_BACKWARD_TRAFFIC = {"cfg5-box-adam-86m-zipf1.1": 4.84e9}
 
 CONFIGS = {
     1: dict(name="cfg1-l2-15k", model="l2", n=15_000, dim=200, b=512, k=128, r=0.07, gamma=12.0, cen=0.0,
@@ -285,9 +285,10 @@ def main():
             "bound": "hbm",
             "kernel": "backward (one C-ABI call, smx_score_backward_fused = score_backward_query_kernel + "
                       "entity_segment_kernel + entity_tile_kernel + entity_fixup_kernel): query gradients, segmented "
-                      "entity gradient" + (" + fused sparse Adam" if cfg["adam"] else " (merged rows)"),
+                      "entity gradient" + (" + fused sparse Adam" if cfg["adam"] else " (merged rows)") +
+                      ("; works from the sign codes the forward saved" if step.codes is not None else ""),
             "achieved": ent_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": ent_gbps / HBM_PEAK_GBPS,
-            "traffic": MEASURED_BACKWARD_TRAFFIC.get(cfg["name"]), "algorithmic_bytes": ent_bytes, "avg_ms": phase_ms["backward"],
+            "traffic": MEASURED_BACKWARD_TRAFFIC.get(cfg["name"]) if step.codes is not None else None, "algorithmic_bytes": ent_bytes, "avg_ms": phase_ms["backward"],
         },
         "step_hbm": {
             "algorithmic_bytes": algo, "achieved_GBps": algo / (ms_per_step * 1e-3) / 1e9,
