@@ -119,3 +119,39 @@ def test_full_size_workload(cfg_id):
         # (torch.randn does return a few exact zeros among 4M samples)
         assert u - touched_m.numel() <= int((gs == 0).sum().item())
         assert changed.numel() > 0.9 * u  # a row sum can stay put when its +-lr moves cancel
+
+    # ---- the path bench.py times, as a second step on the state the first one left: forward that saves the
+    # sign codes (box) + one-call backward (query gradients, entity pass, optimizer), against the separate
+    # calls (query gradients) and the oracle (sampled entities)
+    if cfg["adam"]:
+        codes = fused.new_codes(model, table, idx, q1)
+        score2 = fused.score_forward(model, table, idx, q1, q2, params, err, codes=codes)
+        assert torch.equal(score2, fused.score_forward(model, table, idx, q1, q2, params, err))
+        r1, r2 = fused.score_backward_query(model, table, idx, q1, q2, score2, gs, params)
+        eids = [int(plan.uniq[j]) for j in sample_u]
+        before = {e_: (table[e_].clone(), m[e_].clone(), v[e_].clone()) for e_ in eids}
+        f1, f2 = fused.score_backward_fused(model, plan, table, idx, q1, q2, score2, gs, params, m=m, v=v,
+                                            adam=fused.adam_params(cfg["lr"], 2), codes=codes)
+        assert_close(f1.cpu().numpy(), r1.cpu().numpy(), 1e-6, "one-call gq1")
+        if q2 is not None:
+            assert_close(f2.cpu().numpy(), r2.cpu().numpy(), 1e-6, "one-call gq2")
+        for j, eid in zip(sample_u, eids):
+            pairs = plan.order[seg_np[j]: seg_np[j + 1]].long()
+            pb = (pairs // k).cpu().numpy()
+            if len(pb) > 20000:
+                continue
+            w1, m1, v1 = (x.cpu().numpy().astype(np.float64) for x in before[eid])
+            e = w1[None, None, :].repeat(len(pb), 0)
+            a1 = q1[pb].cpu().numpy().astype(np.float64)[:, None]
+            a2 = None if q2 is None else q2[pb].cpu().numpy().astype(np.float64)[:, None]
+            og = gs.reshape(-1)[pairs].cpu().numpy().astype(np.float64)[:, None]
+            g_rows, _, _ = orc.score_backward(model, og, e, a1, a2, cfg["cen"])
+            want, sum_abs = g_rows.sum(axis=(0, 1)), np.abs(g_rows).sum(axis=(0, 1))
+            got_m = m[eid].cpu().numpy().astype(np.float64)
+            assert_close(got_m, 0.9 * m1 + 0.1 * want, REL_F32, f"step 2 first moment of entity {eid}",
+                         sum_abs=0.1 * sum_abs + 0.9 * np.abs(m1))
+            wn, mn, vn = w1[None].copy(), m1[None].copy(), v1[None].copy()
+            orc.adam_rows(wn, mn, vn, np.array([0]), ((got_m - 0.9 * m1) / 0.1)[None], cfg["lr"], 2)
+            assert_close(table[eid].cpu().numpy(), wn[0], REL_F32, f"step 2 weights of entity {eid}")
+            assert_close(v[eid].cpu().numpy(), vn[0], REL_F32, f"step 2 second moment of entity {eid}",
+                         sum_abs=np.full_like(w1, 1e-12))
