@@ -145,10 +145,15 @@ class EmbeddingOptimizer(ABC):
         return mat
 
     def score_negatives(self, model, ids, q1, q2=None, gamma=0.0, cen=0.0, regularizer=None):
-        """Gather-fused logits [B,K]; q1/q2 are [B,dim] or [B,1,dim] and receive gradients."""
+        """Gather-fused logits [B,K]; q1/q2 are [B,dim] or [B,1,dim] and receive gradients.
+        ids [B,K], or [1,K] for negatives shared by all queries of the batch (the --share_negative
+        layout, online_sampler.py:155-157): every query then scores the same K entities."""
         table = self.sparse_embed.embedding
-        ids = ids.to(table.device).contiguous()
-        b = ids.shape[0]
+        b = q1.shape[0]
+        ids = ids.to(table.device)
+        if ids.dim() == 2 and ids.shape[0] == 1 and b > 1:
+            ids = ids.expand(b, ids.shape[1])
+        ids = ids.contiguous()
         q1c = q1.reshape(b, -1).contiguous()
         q2c = None if q2 is None else q2.reshape(b, -1).contiguous()
         params = fused.score_params(gamma, cen, regularizer)

@@ -129,6 +129,43 @@ def test_fused_scorer_alone_and_mixed_with_plain_lookup():
         assert (err > 1e-5 * np.maximum(np.abs(r[0]), 0.04)).mean() < 1e-3 and err.max() < 2 * lr
 
 
+def test_shared_negatives_with_mask_match_the_dense_operators():
+    """--share_negative layout: ids [1,K] scored by every query, logits multiplied by the is_negative_mat
+    mask (train_process.py:195-196); fused scorer against plain lookup + broadcasting dense operators."""
+    from smore_amd.torchext import ext_ops
+    n, d, b, k, lr = 400, 48, 7, 33, 1e-3
+    rng = np.random.default_rng(11)
+    neg_n = rng.integers(0, n, (1, k))
+    cn = rng.uniform(-0.07, 0.07, (b, 1, d)).astype(np.float32)
+    on = np.abs(rng.uniform(-0.07, 0.07, (b, 1, d))).astype(np.float32)
+    mask_n = (rng.random((b, k)) > 0.2).astype(np.float32)
+    gn_n = rng.standard_normal((b, k)).astype(np.float32)
+
+    def run(fused_neg):
+        emb, opt = _setup(n, d, 7)
+        c = torch.tensor(cn, device="cuda", requires_grad=True)
+        o = torch.tensor(on, device="cuda", requires_grad=True)
+        neg = torch.tensor(neg_n, device="cuda")
+        opt.zero_grad()
+        if fused_neg:
+            ln = opt.score_negatives("box", neg, c, o, gamma=24.0, cen=0.02)
+        else:
+            rn = emb(neg.view(-1), "negative_entity").view(1, k, -1)      # [1,K,D] against [B,1,D] queries
+            ln = 24 - ext_ops.box_dist_out(rn, c, o) - 0.02 * ext_ops.box_dist_in(rn, c, o)
+        assert ln.shape == (b, k)
+        ((ln * torch.tensor(mask_n, device="cuda")) * torch.tensor(gn_n, device="cuda")).sum().backward()
+        opt.apply_grad(lr)
+        opt.check_ids()
+        return (ln.detach().cpu().numpy(), c.grad.cpu().numpy(), o.grad.cpu().numpy(), emb.state_sum_fo.cpu().numpy(),
+                emb.embedding.detach().cpu().numpy())
+
+    a, r = run(True), run(False)
+    for x, y, what in zip(a[:4], r[:4], ("logits", "center grad", "offset grad", "first moment")):
+        assert_close(x, y, 5 * REL_F32, what)
+    # masked-out pairs still touch their rows: every listed id has moved (momentum), nothing else has
+    assert np.abs(a[4] - r[4]).max() < 2 * lr
+
+
 def test_step_counter_and_empty_steps():
     emb, opt = _setup(50, 8, 7)
     opt.zero_grad()
