@@ -235,6 +235,22 @@ int smx_rows_backward(void* stream, const smx_plan_view* plan, const float* grad
                       size_t row_len, float* merged, float* table, float* m, float* v,
                       const smx_opt_params* adam, void* workspace, size_t workspace_bytes);
 
+/* ---- sample loss ---------------------------------------------------------------------------
+ * The loss between the scoring forward and its backward (smore/training/train_process.py:194-213)
+ * and its gradient in one pass over the [B,K] negative logits:
+ *   x = neg * mask (mask = is_negative_mat, may be NULL)
+ *   s_b = sum_k softmax(x * temperature)_k logsigmoid(-x_k)   (temperature > 0; weights not differentiated, :197-199)
+ *       | mean_k logsigmoid(-x_k)                             (temperature == 0, :200-201)
+ *   pos_loss = -sum_b W_b logsigmoid(pos_b),  neg_loss = -sum_b W_b s_b,
+ *   W_b = weight_b / sum(weight) (subsampling_weight, :203-207) or 1/B when weight is NULL (:208-211).
+ * out_loss[2] (device) = {pos_loss, neg_loss}; gpos [B], gneg [B,K] = d((pos_loss + neg_loss) * scale) / d logit,
+ * scale = 1/2/world_size (:213): gneg is the upstream gradient smx_score_backward_* consumes.
+ * workspace: smx_sample_loss_workspace_bytes(B). */
+size_t smx_sample_loss_workspace_bytes(size_t B);
+int smx_sample_loss(void* stream, const float* pos, const float* neg, const float* mask,
+                    const float* weight, size_t B, size_t K, double temperature, double scale,
+                    float* out_loss, float* gpos, float* gneg, void* workspace, size_t workspace_bytes);
+
 /* Plain row lookup out[k,:] = table[idx[k],:] (smore/common/embedding/embed_rw.py:74-75, the GPU
  * branch of EmbeddingReadOnly.read) for callers that need the rows themselves. */
 int smx_gather_rows(void* stream, const float* table, size_t n_rows, size_t row_len,

@@ -221,6 +221,23 @@ def rmsprop_rows(w, state, uniq, merged, lr, alpha=0.99, eps=1e-8, squeeze=False
                                               ctypes.c_int(int(squeeze)))
 
 
+def sample_loss(pos, neg, mask=None, weight=None, temperature=0.0, scale=0.5, dtype=np.float64):
+    """Sample loss of train_process.py:194-213 and its gradient w.r.t. the logits.
+    Returns (pos_loss, neg_loss, gpos [B], gneg [B,K]); the gradients are those of (pos_loss + neg_loss) * scale."""
+    sfx, _ = _sfx(dtype)
+    pos, neg = _c(pos, dtype).reshape(-1), _c(neg, dtype)
+    b, k = neg.shape
+    assert pos.size == b
+    mask = None if mask is None else _c(mask, dtype)
+    weight = None if weight is None else _c(weight, dtype).reshape(-1)
+    out, gpos, gneg = np.zeros(2, dtype), np.zeros(b, dtype), np.zeros((b, k), dtype)
+    getattr(lib(), f"orc_sample_loss_{sfx}")(_p(pos), _p(neg), _p(mask) if mask is not None else None,
+                                             _p(weight) if weight is not None else None, _sz(b), _sz(k),
+                                             ctypes.c_double(temperature), ctypes.c_double(scale), _p(out), _p(gpos),
+                                             _p(gneg))
+    return float(out[0]), float(out[1]), gpos, gneg
+
+
 # ---- composition: the score of each model and one training step -------------------------------
 
 MODELS = ("l1", "l2", "box", "rotate", "beta_kl")

@@ -464,3 +464,44 @@ def test_train_step_equals_dense_autograd_pipeline():
     g = tt.grad.numpy()[touched]
     want = t0[touched] - 1e-4 / 0.1 * (0.1 * g) / (np.sqrt(0.001 * g * g) / math.sqrt(0.001) + 1e-8)
     assert np.allclose(table[touched], want, rtol=1e-11)
+
+
+@pytest.mark.parametrize("temperature", [0.0, 0.7])
+@pytest.mark.parametrize("weighted", [False, True])
+@pytest.mark.parametrize("masked", [False, True])
+def test_sample_loss_is_the_torch_expression_of_the_training_step(temperature, weighted, masked):
+    """orc.sample_loss against torch autograd of the expression as train_process.py:194-213 writes it
+    (F.softmax(...).detach() * F.logsigmoid(-x), weighted or plain means, / 2 / world_size)."""
+    import torch.nn.functional as F
+    rng = np.random.default_rng(17)
+    b, k, world = 6, 11, 4
+    pos, neg = rng.standard_normal(b) * 4, rng.standard_normal((b, k)) * 4
+    neg[0, 0], pos[1] = 60.0, -70.0                      # saturated sigmoids
+    mask = (rng.random((b, k)) > 0.3).astype(np.float64)
+    w = rng.random(b) + 0.1
+    tp, tn = torch.tensor(pos, requires_grad=True), torch.tensor(neg, requires_grad=True)
+    x = tn * torch.tensor(mask) if masked else tn
+    if temperature > 0:
+        s = (F.softmax(x * temperature, dim=1).detach() * F.logsigmoid(-x)).sum(dim=1)
+    else:
+        s = F.logsigmoid(-x).mean(dim=1)
+    p = F.logsigmoid(tp)
+    if weighted:
+        tw = torch.tensor(w)
+        pl, nl = -(tw * p).sum() / tw.sum(), -(tw * s).sum() / tw.sum()
+    else:
+        pl, nl = -p.mean(), -s.mean()
+    ((pl + nl) / 2 / world).backward()
+    got = orc.sample_loss(pos, neg, mask if masked else None, w if weighted else None, temperature, 0.5 / world)
+    assert abs(got[0] - pl.item()) < 1e-12 and abs(got[1] - nl.item()) < 1e-12
+    assert np.allclose(got[2], tp.grad.numpy(), rtol=1e-12, atol=1e-15)
+    assert np.allclose(got[3], tn.grad.numpy(), rtol=1e-12, atol=1e-15)
+
+
+def test_sample_loss_known_values():
+    """All logits 0: logsigmoid(0) = -ln 2, sigmoid(0) = 1/2, softmax uniform."""
+    b, k = 3, 5
+    for t in (0.0, 2.0):
+        pl, nl, gp, gn = orc.sample_loss(np.zeros(b), np.zeros((b, k)), temperature=t, scale=0.5)
+        assert abs(pl - math.log(2)) < 1e-15 and abs(nl - math.log(2)) < 1e-15
+        assert np.allclose(gp, -0.5 / b * 0.5) and np.allclose(gn, 0.5 / b / k * 0.5)
