@@ -251,6 +251,28 @@ int smx_sample_loss(void* stream, const float* pos, const float* neg, const floa
                     const float* weight, size_t B, size_t K, double temperature, double scale,
                     float* out_loss, float* gpos, float* gneg, void* workspace, size_t workspace_bytes);
 
+/* ---- evaluation against all entities --------------------------------------------------------
+ * Filtered ranks of a query's answers among all n_rows entities (the test_all branch of
+ * smore/training/train_process.py:112-160: logits of every entity, argsort, ranks of easy + hard
+ * answers, minus the answers ranked before) without materialising or sorting the logit row: the
+ * table is streamed once per two queries and every non-answer entity is counted against the answers
+ * it ranks before.  Equal scores: the lower entity id ranks first.
+ *   ans_id [B, A] int64, ans_count [B] int32: ans_count[b] <= A valid answers (easy and hard alike) per query.
+ * smx_rank_answer_keys: ans_score [B, A] = the answers' logits, ans_key [B, A] = their order keys
+ *   (larger key = ranked earlier; 0 in unused slots).
+ * smx_rank_scan: ans_id / ans_key must be sorted by key, descending, within each query (unused slots
+ *   last); filtered_rank [B, A] int64, 1-based, in that order (0 in unused slots).
+ * workspace: smx_rank_workspace_bytes(B, A).  At most 2048 answers per query, n_rows <= 2^32. */
+size_t smx_rank_workspace_bytes(size_t B, size_t A);
+int smx_rank_answer_keys(int model, void* stream, const float* table, size_t n_rows, const float* q1,
+                         const float* q2, size_t B, size_t dim, const smx_score_params* params,
+                         const int64_t* ans_id, const int32_t* ans_count, size_t A, float* ans_score,
+                         uint64_t* ans_key);
+int smx_rank_scan(int model, void* stream, const float* table, size_t n_rows, const float* q1,
+                  const float* q2, size_t B, size_t dim, const smx_score_params* params,
+                  const int64_t* ans_id, const uint64_t* ans_key, const int32_t* ans_count, size_t A,
+                  int64_t* filtered_rank, void* workspace, size_t workspace_bytes);
+
 /* Plain row lookup out[k,:] = table[idx[k],:] (smore/common/embedding/embed_rw.py:74-75, the GPU
  * branch of EmbeddingReadOnly.read) for callers that need the rows themselves. */
 int smx_gather_rows(void* stream, const float* table, size_t n_rows, size_t row_len,

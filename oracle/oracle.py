@@ -238,6 +238,22 @@ def sample_loss(pos, neg, mask=None, weight=None, temperature=0.0, scale=0.5, dt
     return float(out[0]), float(out[1]), gpos, gneg
 
 
+def filtered_ranks(scores, easy, hard):
+    """Filtered ranks (1-based) of one query's answers among all entities, train_process.py:124-145:
+    ranking = position in the descending argsort of the logits (equal logits: lower id first), and an
+    answer's filtered rank is its position minus the number of answers (easy or hard) placed before it.
+    scores [N]; easy, hard: disjoint id sequences.  Returns (ranks of hard, ranks of easy) in the given order."""
+    scores = np.asarray(scores)
+    order = np.argsort(-scores, kind="stable")
+    ranking = np.empty(scores.shape[0], dtype=np.int64)
+    ranking[order] = np.arange(scores.shape[0])
+    ans = np.array(list(easy) + list(hard), dtype=np.int64)
+    pos = ranking[ans] if ans.size else np.zeros(0, np.int64)
+    before = (pos[None, :] < pos[:, None]).sum(axis=1) if ans.size else pos
+    filt = pos - before + 1
+    return filt[len(easy):], filt[: len(easy)]
+
+
 # ---- composition: the score of each model and one training step -------------------------------
 
 MODELS = ("l1", "l2", "box", "rotate", "beta_kl")

@@ -48,6 +48,11 @@ SIGNATURES = {
     "smx_score_backward_fused": (_i, [_i, _vp, _vp, _vp, _sz, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _vp,
                                       _vp, _vp, _vp, _vp, _vp, _sz, _vp, _sz]),
     # stream, plan, grad_rows, row_len, merged, table, m, v, adam, ws, ws_bytes
+    "smx_rank_workspace_bytes": (_sz, [_sz, _sz]),
+    # model, stream, table, n_rows, q1, q2, B, dim, params, ans_id, ans_count, A, ans_score, ans_key
+    "smx_rank_answer_keys": (_i, [_i, _vp, _vp, _sz, _vp, _vp, _sz, _sz, _vp, _vp, _vp, _sz, _vp, _vp]),
+    # model, stream, table, n_rows, q1, q2, B, dim, params, ans_id, ans_key, ans_count, A, rank, ws, ws_bytes
+    "smx_rank_scan": (_i, [_i, _vp, _vp, _sz, _vp, _vp, _sz, _sz, _vp, _vp, _vp, _vp, _sz, _vp, _vp, _sz]),
     "smx_sample_loss_workspace_bytes": (_sz, [_sz]),
     # stream, pos, neg, mask, weight, B, K, temperature, scale, out_loss, gpos, gneg, ws, ws_bytes
     "smx_sample_loss": (_i, [_vp, _vp, _vp, _vp, _vp, _sz, _sz, ctypes.c_double, ctypes.c_double, _vp, _vp, _vp, _vp, _sz]),

@@ -1,0 +1,95 @@
+// Host side of the all-entity ranking (see smx_rank_impl.h).
+#include "smx_rank_impl.h"
+
+namespace smx {
+
+extern template int rank_dispatch<mL1>(hipStream_t, const RankArgs&, int, int, bool);
+extern template int rank_dispatch<mL2>(hipStream_t, const RankArgs&, int, int, bool);
+extern template int rank_dispatch<mBox>(hipStream_t, const RankArgs&, int, int, bool);
+extern template int rank_dispatch<mRotate>(hipStream_t, const RankArgs&, int, int, bool);
+extern template int rank_dispatch<mBetaKL>(hipStream_t, const RankArgs&, int, int, bool);
+
+constexpr size_t kRankMaxAnswers = 2048;  // per query; bins and keys of a pass live in LDS (2 x 2049 x 4 + 2 x 2048 x 8 bytes)
+
+static size_t rank_ws_bytes(size_t B, size_t A) { return (B * (A + 1) * sizeof(unsigned) + 255) & ~(size_t)255; }
+
+static int rank_common(RankArgs* R, int* vec, int* nit, int model, const float* table, size_t n_rows, const float* q1,
+                       const float* q2, size_t B, size_t dim, const smx_score_params* params, const int64_t* ans_id,
+                       const int32_t* ans_count, size_t A) {
+  if (model < 0 || model >= mNumModels) return fail(SMX_ERR_KIND, "unknown score model %d", model);
+  if (!table || !q1 || !params || !ans_id || !ans_count || (model_nq(model) == 2 && !q2))
+    return fail(SMX_ERR_ARG, "null pointer");
+  if (B == 0 || dim == 0 || n_rows == 0 || A == 0) return fail(SMX_ERR_SHAPE, "empty dimension");
+  if (n_rows > 0x100000000ull) return fail(SMX_ERR_SHAPE, "entity count %zu needs ids wider than 32 bits", n_rows);
+  if (A > kRankMaxAnswers) return fail(SMX_ERR_SHAPE, "at most %zu answers per query", kRankMaxAnswers);
+  if (B > 0x7fffffffull / (A + 1)) return fail(SMX_ERR_SHAPE, "too many queries");
+  if (params->reg_on && model != mBetaKL)
+    return fail(SMX_ERR_ARG, "the entity clamp prologue exists for the beta_kl model only");
+  const bool vec4 = dim % 4 == 0 && aligned16(table) && aligned16(q1) && (model_nq(model) == 1 || aligned16(q2));
+  *vec = vec4 ? 4 : 1;
+  const size_t ncol = dim / *vec;
+  const int need = (int)((ncol + 63) / 64);
+  *nit = need <= 1 ? 1 : (need <= 2 ? 2 : (need <= 4 ? 4 : 8));
+  if (ncol > 512 || (*vec == 1 && *nit > 4))
+    return fail(SMX_ERR_SHAPE, "dim %zu not supported (at most 2048 aligned or 256 unaligned floats)", dim);
+  *R = RankArgs{};
+  R->table = table;
+  R->q1 = q1;
+  R->q2 = q2;
+  R->B = (int)B;
+  R->ncol = (int)ncol;
+  R->n_rows = n_rows;
+  R->p = ScoreParams{params->gamma, params->cen, params->reg_on, params->reg_add, params->reg_lo, params->reg_hi};
+  R->ans_id = reinterpret_cast<const long long*>(ans_id);
+  R->ans_count = ans_count;
+  R->A = (int)A;
+  return SMX_OK;
+}
+
+static int rank_run(int model, hipStream_t st, const RankArgs& R, int vec, int nit, bool keys_only) {
+  switch (model) {
+    case mL1: return rank_dispatch<mL1>(st, R, vec, nit, keys_only);
+    case mL2: return rank_dispatch<mL2>(st, R, vec, nit, keys_only);
+    case mBox: return rank_dispatch<mBox>(st, R, vec, nit, keys_only);
+    case mRotate: return rank_dispatch<mRotate>(st, R, vec, nit, keys_only);
+    case mBetaKL: return rank_dispatch<mBetaKL>(st, R, vec, nit, keys_only);
+  }
+  return fail(SMX_ERR_KIND, "unknown score model %d", model);
+}
+
+}  // namespace smx
+
+extern "C" {
+
+size_t smx_rank_workspace_bytes(size_t B, size_t A) { return smx::rank_ws_bytes(B, A); }
+
+int smx_rank_answer_keys(int model, void* stream, const float* table, size_t n_rows, const float* q1, const float* q2,
+                         size_t B, size_t dim, const smx_score_params* params, const int64_t* ans_id,
+                         const int32_t* ans_count, size_t A, float* ans_score, uint64_t* ans_key) {
+  using namespace smx;
+  RankArgs R;
+  int vec, nit;
+  if (int rc = rank_common(&R, &vec, &nit, model, table, n_rows, q1, q2, B, dim, params, ans_id, ans_count, A)) return rc;
+  if (!ans_score || !ans_key) return fail(SMX_ERR_ARG, "null output pointer");
+  R.score_out = ans_score;
+  R.key_out = reinterpret_cast<unsigned long long*>(ans_key);
+  return rank_run(model, as_stream(stream), R, vec, nit, true);
+}
+
+int smx_rank_scan(int model, void* stream, const float* table, size_t n_rows, const float* q1, const float* q2, size_t B,
+                  size_t dim, const smx_score_params* params, const int64_t* ans_id, const uint64_t* ans_key,
+                  const int32_t* ans_count, size_t A, int64_t* filtered_rank, void* workspace, size_t workspace_bytes) {
+  using namespace smx;
+  RankArgs R;
+  int vec, nit;
+  if (int rc = rank_common(&R, &vec, &nit, model, table, n_rows, q1, q2, B, dim, params, ans_id, ans_count, A)) return rc;
+  if (!ans_key || !filtered_rank || !workspace) return fail(SMX_ERR_ARG, "null pointer");
+  if (workspace_bytes < rank_ws_bytes(B, A))
+    return fail(SMX_ERR_WORKSPACE, "rank workspace too small: %zu < %zu", workspace_bytes, rank_ws_bytes(B, A));
+  R.ans_key = reinterpret_cast<const unsigned long long*>(ans_key);
+  R.bins = static_cast<unsigned*>(workspace);
+  R.rank_out = reinterpret_cast<long long*>(filtered_rank);
+  return rank_run(model, as_stream(stream), R, vec, nit, false);
+}
+
+}  // extern "C"

@@ -1,0 +1,296 @@
+// Evaluation against all entities: filtered ranks of a query's answers without materialising or
+// sorting the [1,N] logit row.
+//
+// Replaces, for the test_all case of smore/training/train_process.py:112-160,
+//   negative_logit = model(None, all_entity_idx, ...)      score of every entity (kg_reasoning.py:349-355)
+//   argsort(descending) -> ranking -> ranking[answers] -> sort -> minus arange -> +1   (filtered setting)
+// The filtered rank of an answer is 1 + the number of NON-answer entities ranked before it.  So the
+// table is streamed once, in order; a wavefront scores a row against the queries of the pass and
+// finds, with one 64-bit compare per 64 answers, how many of the query's answers the entity does not
+// beat; that number indexes a histogram (integer atomics: exact, order-free).  A prefix sum over the
+// histogram gives every answer its count.  Order of equal scores: the lower entity id ranks first
+// (one of the orders an unstable argsort may produce).  "Beats" is one unsigned compare of
+// (sortable(score) << 32 | ~id) keys; the answers' keys come from the same scoring function.
+#pragma once
+#include "smx_common.h"
+#include "smx_models.h"
+#include "smx_wave.h"
+
+namespace smx {
+
+constexpr int kRankQueries = 2;  // queries scored per pass over the table
+
+struct RankArgs {
+  const float* table;
+  const float* q1;
+  const float* q2;
+  int b0, B;            // queries [b0, b0 + kRankQueries) of B are handled by this launch
+  int ncol;
+  unsigned long long n_rows;
+  ScoreParams p;
+  // answers, per query A slots (the first ans_count[b] are valid), sorted by key descending for the scan
+  const long long* ans_id;           // [B, A]
+  const unsigned long long* ans_key; // [B, A]   (scan)
+  unsigned long long* key_out;       // [B, A]   (answer-key kernel)
+  float* score_out;                  // [B, A]   (answer-key kernel)
+  const int* ans_count;              // [B]
+  int A;
+  unsigned* bins;                    // [B, A + 1]
+  long long* rank_out;               // [B, A]
+};
+
+__device__ __forceinline__ unsigned sortable_bits(float s) {
+  const unsigned u = __float_as_uint(s);
+  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);  // ascending in the float order (-0 < +0)
+}
+__device__ __forceinline__ unsigned long long rank_key(float score, unsigned long long id) {
+  return ((unsigned long long)sortable_bits(score) << 32) | (unsigned)(~(unsigned)id);
+}
+
+// Score of one row against one staged query; the value is valid in lane 63.
+template <int M, int VEC, int NIT, bool REG>
+__device__ __forceinline__ float row_score(const float (&e1)[NIT][VEC], const float (&e2)[NIT][VEC],
+                                           const typename ModelOps<M>::Q (&q)[NIT][VEC], int ncol, int lane,
+                                           const ScoreParams& p) {
+  constexpr int MUL = model_mul(M);
+  float mine = 0.f;
+#pragma unroll
+  for (int it = 0; it < NIT; ++it) {
+    float a0 = 0.f, a1 = 0.f;
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) {
+      const float x1 = REG ? reg_apply(e1[it][v], p) : e1[it][v];
+      const float x2 = MUL == 2 ? (REG ? reg_apply(e2[it][v], p) : e2[it][v]) : 0.f;
+      ModelOps<M>::fwd(x1, x2, q[it][v], a0, a1);
+    }
+    const float f = ModelOps<M>::fold(a0, a1, p);
+    mine += lane + 64 * it < ncol ? f : 0.f;
+  }
+  return ModelOps<M>::score(wave_sum_last_f32(mine), p);
+}
+
+template <int VEC, int NIT, int MUL>
+__device__ __forceinline__ void load_entity(const float* __restrict__ row, int dim, int ncol, int lane,
+                                            float (&e1)[NIT][VEC], float (&e2)[NIT][VEC]) {
+#pragma unroll
+  for (int it = 0; it < NIT; ++it) {
+    const int c = min(lane + 64 * it, ncol - 1);
+    if constexpr (VEC == 4) {
+      const float4 a = reinterpret_cast<const float4*>(row)[c];
+      e1[it][0] = a.x; e1[it][1] = a.y; e1[it][2] = a.z; e1[it][3] = a.w;
+      if (MUL == 2) {
+        const float4 b = reinterpret_cast<const float4*>(row + dim)[c];
+        e2[it][0] = b.x; e2[it][1] = b.y; e2[it][2] = b.z; e2[it][3] = b.w;
+      }
+    } else {
+      e1[it][0] = row[c];
+      if (MUL == 2) e2[it][0] = row[dim + c];
+    }
+  }
+}
+
+template <int M, int VEC, int NIT>
+__device__ __forceinline__ void load_rank_query(const float* __restrict__ q1, const float* __restrict__ q2, int b,
+                                                int dim, int ncol, int lane,
+                                                typename ModelOps<M>::Q (&q)[NIT][VEC]) {
+#pragma unroll
+  for (int it = 0; it < NIT; ++it) {
+    const int c = min(lane + 64 * it, ncol - 1);
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) {
+      const float a = q1[(size_t)b * dim + c * VEC + v];
+      const float bb = model_nq(M) == 2 ? q2[(size_t)b * dim + c * VEC + v] : 0.f;
+      q[it][v] = prep_forward<M>(a, bb);
+    }
+  }
+}
+
+// Keys (and scores) of the answers: one wavefront per (query, answer slot).
+template <int M, int VEC, int NIT, bool REG>
+__global__ __launch_bounds__(256) void rank_answer_keys_kernel(RankArgs A) {
+  constexpr int MUL = model_mul(M);
+  const int lane = threadIdx.x & 63;
+  const int slot = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (slot >= A.B * A.A) return;
+  const int b = slot / A.A, j = slot - b * A.A;
+  const int dim = A.ncol * VEC;
+  const bool valid = j < A.ans_count[b];
+  unsigned long long id = valid ? (unsigned long long)A.ans_id[slot] : 0ull;
+  if (id >= A.n_rows) id = 0;  // the host wrapper has already refused such ids
+  typename ModelOps<M>::Q q[NIT][VEC];
+  load_rank_query<M, VEC, NIT>(A.q1, A.q2, b, dim, A.ncol, lane, q);
+  float e1[NIT][VEC], e2[NIT][VEC];
+  load_entity<VEC, NIT, MUL>(A.table + id * (size_t)dim * MUL, dim, A.ncol, lane, e1, e2);
+  const float s = row_score<M, VEC, NIT, REG>(e1, e2, q, A.ncol, lane, A.p);
+  if (lane == 63) {
+    A.score_out[slot] = valid ? s : 0.f;
+    A.key_out[slot] = valid ? rank_key(s, id) : 0ull;  // key 0 sorts last and is never counted
+  }
+}
+
+// The scan.  LDS: bins [kRankQueries][A + 1].
+template <int M, int VEC, int NIT, bool REG>
+__global__ __launch_bounds__(256) void rank_scan_kernel(RankArgs A) {
+  constexpr int MUL = model_mul(M);
+  constexpr int NB = kRankQueries;
+  constexpr int RIF = NIT * MUL <= 2 ? 4 : (NIT * MUL <= 4 ? 2 : 1);
+  extern __shared__ unsigned lds_bins[];  // bins [NB][A + 1], then (8-byte aligned) the answers' keys [NB][A]
+  const int lane = threadIdx.x & 63;
+  const int wave = uniform(threadIdx.x >> 6);
+  const int dim = A.ncol * VEC;
+  const size_t row_len = (size_t)dim * MUL;
+  const int A1 = A.A + 1;
+  unsigned long long* lds_keys = reinterpret_cast<unsigned long long*>(lds_bins + ((NB * A1 + 1) & ~1));
+  for (int i = threadIdx.x; i < NB * A1; i += 256) lds_bins[i] = 0u;
+  for (int i = threadIdx.x; i < NB * A.A; i += 256) {
+    const int x = i / A.A, j = i - x * A.A;
+    const int b = min(A.b0 + x, A.B - 1);
+    lds_keys[i] = j < A.ans_count[b] ? A.ans_key[(size_t)b * A.A + j] : 0ull;
+  }
+  __syncthreads();
+
+  typename ModelOps<M>::Q q[NB][NIT][VEC];
+  int count[NB], qb[NB];
+#pragma unroll
+  for (int x = 0; x < NB; ++x) {
+    qb[x] = min(A.b0 + x, A.B - 1);  // a pass past the last query repeats it; its histogram is dropped
+    count[x] = A.ans_count[qb[x]];
+    load_rank_query<M, VEC, NIT>(A.q1, A.q2, qb[x], dim, A.ncol, lane, q[x]);
+  }
+  const int chunks = (A.A + 63) / 64;
+
+  // wavefronts walk the table together: group g of RIF consecutive rows belongs to wavefront g mod n_waves
+  const unsigned long long n_waves = (unsigned long long)gridDim.x * 4ull;
+  const unsigned long long wid = (unsigned long long)blockIdx.x * 4ull + wave;
+  const unsigned long long groups = (A.n_rows + RIF - 1) / RIF;
+  float ea1[RIF][NIT][VEC], ea2[RIF][NIT][VEC], eb1[RIF][NIT][VEC], eb2[RIF][NIT][VEC];
+  auto request = [&](float (&x1)[RIF][NIT][VEC], float (&x2)[RIF][NIT][VEC], unsigned long long g) {
+#pragma unroll
+    for (int r = 0; r < RIF; ++r) {
+      unsigned long long row = g * RIF + r;
+      if (row >= A.n_rows) row = A.n_rows - 1;
+      load_entity<VEC, NIT, MUL>(A.table + row * row_len, dim, A.ncol, lane, x1[r], x2[r]);
+    }
+  };
+  auto consume = [&](const float (&x1)[RIF][NIT][VEC], const float (&x2)[RIF][NIT][VEC], unsigned long long g) {
+#pragma unroll
+    for (int r = 0; r < RIF; ++r) {
+      const unsigned long long row = g * RIF + r;
+      if (row < A.n_rows) {  // wave-uniform
+#pragma unroll
+        for (int x = 0; x < NB; ++x) {
+          const float s = row_score<M, VEC, NIT, REG>(x1[r], x2[r], q[x], A.ncol, lane, A.p);
+          const float su = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(s), 63));
+          const unsigned long long key = rank_key(su, row);
+          int not_beaten = 0;
+          bool is_answer = false;
+          for (int c = 0; c < chunks; ++c) {
+            const int j = c * 64 + lane;
+            const bool live = j < count[x];
+            const unsigned long long ak = live ? lds_keys[x * A.A + j] : 0ull;
+            not_beaten += __popcll(__ballot(live && !(key > ak)));
+            is_answer |= __ballot(live && ((unsigned)~(unsigned)ak == (unsigned)row)) != 0ull;
+          }
+          if (!is_answer && lane == 0) atomicAdd(&lds_bins[x * A1 + not_beaten], 1u);
+        }
+      }
+    }
+  };
+  unsigned long long g = wid;
+  if (g < groups) request(ea1, ea2, g);
+  while (g < groups) {
+    const unsigned long long g1 = g + n_waves, g2 = g + 2 * n_waves;
+    if (g1 < groups) request(eb1, eb2, g1);
+    consume(ea1, ea2, g);
+    if (g1 >= groups) break;
+    if (g2 < groups) request(ea1, ea2, g2);
+    consume(eb1, eb2, g1);
+    g = g2;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int x = 0; x < NB; ++x) {
+    if (A.b0 + x < A.B) {
+      for (int i = threadIdx.x; i < A1; i += 256) {
+        const unsigned v = lds_bins[x * A1 + i];
+        if (v) atomicAdd(&A.bins[(size_t)(A.b0 + x) * A1 + i], v);
+      }
+    }
+  }
+}
+
+static __global__ __launch_bounds__(256) void rank_clear_kernel(unsigned* bins, size_t n) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) bins[i] = 0u;
+}
+
+// filtered rank of answer j (in key order) = 1 + sum of the bins 0..j; one workgroup per query
+static __global__ __launch_bounds__(256) void rank_finish_kernel(RankArgs A) {
+  const int b = blockIdx.x;
+  const int A1 = A.A + 1;
+  if (threadIdx.x == 0) {
+    unsigned long long run = 0;
+    const int n = A.ans_count[b];
+    for (int j = 0; j < A.A; ++j) {
+      run += A.bins[(size_t)b * A1 + j];
+      A.rank_out[(size_t)b * A.A + j] = j < n ? (long long)(run + 1ull) : 0ll;
+    }
+  }
+}
+
+template <int M, int VEC, int NIT, bool REG>
+int launch_rank_reg(hipStream_t st, RankArgs A, bool keys_only) {
+  if (keys_only) {
+    const unsigned blocks = (unsigned)(((size_t)A.B * A.A + 3) / 4);
+    hipLaunchKernelGGL((rank_answer_keys_kernel<M, VEC, NIT, REG>), dim3(blocks), dim3(256), 0, st, A);
+    return check_launch("rank answer keys");
+  }
+  const size_t n_bins = (size_t)A.B * (A.A + 1);
+  hipLaunchKernelGGL(rank_clear_kernel, dim3((unsigned)((n_bins + 255) / 256)), dim3(256), 0, st, A.bins, n_bins);
+  int dev = 0, cus = 256, per_cu = 2;
+  const size_t lds = (((size_t)kRankQueries * (A.A + 1) + 1) & ~(size_t)1) * sizeof(unsigned) +
+                     (size_t)kRankQueries * A.A * sizeof(unsigned long long);
+  if (hipGetDevice(&dev) == hipSuccess) {
+    (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, rank_scan_kernel<M, VEC, NIT, REG>, 256, lds) != hipSuccess ||
+        per_cu < 1)
+      per_cu = 2;
+  }
+  unsigned blocks = (unsigned)cus * (unsigned)per_cu;
+  const unsigned long long want = (A.n_rows + 15) / 16;
+  if (want < blocks) blocks = (unsigned)(want ? want : 1);
+  for (int b0 = 0; b0 < A.B; b0 += kRankQueries) {
+    A.b0 = b0;
+    hipLaunchKernelGGL((rank_scan_kernel<M, VEC, NIT, REG>), dim3(blocks), dim3(256), lds, st, A);
+  }
+  hipLaunchKernelGGL(rank_finish_kernel, dim3((unsigned)A.B), dim3(256), 0, st, A);
+  return check_launch("rank scan");
+}
+
+template <int M, int VEC, int NIT>
+int launch_rank(hipStream_t st, const RankArgs& A, bool keys_only) {
+  if constexpr (M == mBetaKL) {
+    if (A.p.reg_on) return launch_rank_reg<M, VEC, NIT, true>(st, A, keys_only);
+  }
+  return launch_rank_reg<M, VEC, NIT, false>(st, A, keys_only);
+}
+
+// Instantiated once per model in its own translation unit (smx_rank_inst_*.hip).
+template <int M>
+int rank_dispatch(hipStream_t st, const RankArgs& A, int vec, int nit, bool keys_only) {
+  if (vec == 4) {
+    switch (nit) {
+      case 1: return launch_rank<M, 4, 1>(st, A, keys_only);
+      case 2: return launch_rank<M, 4, 2>(st, A, keys_only);
+      case 4: return launch_rank<M, 4, 4>(st, A, keys_only);
+      default: return launch_rank<M, 4, 8>(st, A, keys_only);
+    }
+  }
+  switch (nit) {
+    case 1: return launch_rank<M, 1, 1>(st, A, keys_only);
+    case 2: return launch_rank<M, 1, 2>(st, A, keys_only);
+    default: return launch_rank<M, 1, 4>(st, A, keys_only);
+  }
+}
+
+}  // namespace smx

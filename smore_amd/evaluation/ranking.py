@@ -1,0 +1,71 @@
+"""Filtered ranks of the answers of a batch of queries among ALL entities, as test_step_mp computes
+them (smore/training/train_process.py:112-160), on the streaming HIP scan instead of
+`argsort` over the [1, nentity] logit row."""
+import ctypes
+
+import torch
+
+from .. import _lib
+from ..fused import MODELS, _dims, _ptr, _stream, _workspace
+
+_TOP = -(1 << 63)  # flips the top bit: unsigned key order -> signed int64 order
+
+
+def filtered_ranks(model, table, q1, q2, params, easy_answers, hard_answers):
+    """model: score model name; table [N,row]; q1/q2 [B,dim] (q2 None for l1/l2); params from
+    fused.score_params (gamma, cen, regularizer); easy_answers / hard_answers: per query a sequence of
+    entity ids (disjoint, train_process.py:139).  Returns per query a pair of int64 tensors (device):
+    the filtered ranks (1-based) of its hard answers, in the order given, and of its easy answers."""
+    b = q1.shape[0]
+    if len(easy_answers) != b or len(hard_answers) != b:
+        raise _lib.SmxError("one answer list per query is needed")
+    n = table.shape[0]
+    lists = [list(e) + list(h) for e, h in zip(easy_answers, hard_answers)]
+    a = max(1, max(len(x) for x in lists))
+    ids = torch.zeros((b, a), dtype=torch.int64)
+    for i, x in enumerate(lists):
+        if x:
+            row = torch.as_tensor(x, dtype=torch.int64)
+            if int(row.min()) < 0 or int(row.max()) >= n:
+                raise IndexError("answer id outside the entity table")
+            if row.unique().numel() != row.numel():
+                raise _lib.SmxError("an entity is listed twice among the answers of one query")
+            ids[i, : len(x)] = row
+    counts = torch.tensor([len(x) for x in lists], dtype=torch.int32)
+    dev = table.device
+    ids, counts = ids.to(dev), counts.to(dev)
+    q1c = q1.reshape(b, -1).contiguous()
+    q2c = None if q2 is None else q2.reshape(b, -1).contiguous()
+    _, _, dim = _dims(model, table, ids, q1c, q2c)
+    scores = torch.empty((b, a), dtype=torch.float32, device=dev)
+    keys = torch.empty((b, a), dtype=torch.int64, device=dev)  # holds the unsigned 64-bit keys bit for bit
+    ranks = torch.empty((b, a), dtype=torch.int64, device=dev)
+    lib = _lib.load()
+    with torch.cuda.device(dev):
+        _lib.call("smx_rank_answer_keys", MODELS[model], _stream(table), _ptr(table), n, _ptr(q1c), _ptr(q2c), b, dim,
+                  ctypes.byref(params), _ptr(ids), _ptr(counts), a, _ptr(scores), _ptr(keys))
+        order = torch.argsort(keys ^ _TOP, dim=1, descending=True, stable=True)
+        ids_sorted = torch.gather(ids, 1, order).contiguous()
+        keys_sorted = torch.gather(keys, 1, order).contiguous()
+        ws = _workspace(lib.smx_rank_workspace_bytes(b, a), dev)
+        _lib.call("smx_rank_scan", MODELS[model], _stream(table), _ptr(table), n, _ptr(q1c), _ptr(q2c), b, dim,
+                  ctypes.byref(params), _ptr(ids_sorted), _ptr(keys_sorted), _ptr(counts), a, _ptr(ranks), _ptr(ws),
+                  ws.numel())
+    back = torch.empty_like(ranks)
+    back.scatter_(1, order, ranks)  # rank of the answer in the slot it was given in
+    out = []
+    for i, (e, h) in enumerate(zip(easy_answers, hard_answers)):
+        ne, nh = len(e), len(h)
+        out.append((back[i, ne: ne + nh], back[i, :ne]))
+    return out
+
+
+def ranking_metrics(hard_ranks):
+    """MRR, HITS1/3/10 and HITS1max of one query from the filtered ranks of its hard answers
+    (train_process.py:146-152); an empty tensor gives zeros, as the reference does for a query whose
+    answer is not among the candidates."""
+    if hard_ranks.numel() == 0:
+        return dict(MRR=0.0, HITS1=0.0, HITS3=0.0, HITS10=0.0, HITS1max=0.0)
+    r = hard_ranks.to(torch.float32)
+    return dict(MRR=float((1.0 / r).mean()), HITS1=float((r <= 1).float().mean()), HITS3=float((r <= 3).float().mean()),
+                HITS10=float((r <= 10).float().mean()), HITS1max=float(r.min() == 1))

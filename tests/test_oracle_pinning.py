@@ -505,3 +505,33 @@ def test_sample_loss_known_values():
         pl, nl, gp, gn = orc.sample_loss(np.zeros(b), np.zeros((b, k)), temperature=t, scale=0.5)
         assert abs(pl - math.log(2)) < 1e-15 and abs(nl - math.log(2)) < 1e-15
         assert np.allclose(gp, -0.5 / b * 0.5) and np.allclose(gn, 0.5 / b / k * 0.5)
+
+
+def test_filtered_ranks_follow_the_evaluation_loop():
+    """orc.filtered_ranks against (1) the tensor recipe of train_process.py:124-145 restated with torch
+    (argsort, scatter of arange, sort of the answers' ranks, minus arange, +1, hard mask) on tie-free
+    scores, and (2) the definition 1 + #non-answers with a larger score."""
+    rng = np.random.default_rng(23)
+    n = 400
+    scores = rng.permutation(n).astype(np.float64) * 0.37 - 20     # tie-free
+    easy, hard = [5, 17, 300, 42], [7, 399, 0, 123, 250]
+    got_h, got_e = orc.filtered_ranks(scores, easy, hard)
+    logit = torch.tensor(scores)[None]
+    argsort = torch.argsort(logit, dim=1, descending=True)
+    ranking = argsort.clone().to(torch.float)
+    ranking = ranking.scatter_(1, argsort, torch.arange(n).to(torch.float).repeat(1, 1))
+    cur = ranking[0, easy + hard]
+    cur, indices = torch.sort(cur)
+    masks = indices >= len(easy)
+    cur = cur - torch.arange(len(easy) + len(hard)).to(torch.float) + 1
+    assert sorted(got_h.tolist()) == cur[masks].to(torch.int64).tolist()
+    is_ans = np.zeros(n, bool)
+    is_ans[easy + hard] = True
+    for a, r in zip(hard + easy, list(got_h) + list(got_e)):
+        assert r == 1 + int(((scores > scores[a]) & ~is_ans).sum())
+    # equal logits: the lower id ranks first
+    tied = np.zeros(6)
+    h, e = orc.filtered_ranks(tied, [], [4])
+    assert h.tolist() == [5] and e.size == 0
+    h, _ = orc.filtered_ranks(tied, [1], [4, 0])
+    assert h.tolist() == [3, 1]      # position 4, two answers (ids 0 and 1) before it

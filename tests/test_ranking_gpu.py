@@ -1,0 +1,107 @@
+"""All-entity filtered ranking (smx_rank_answer_keys + smx_rank_scan) against the CPU oracle."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle as orc
+from tests.test_fused_gpu import GAMMA, dev, make_problem
+
+pytestmark = pytest.mark.gpu
+
+
+def _scores64(model, table, q1, q2, cen):
+    """float64 logits of every entity for every query, [B, N]"""
+    b = q1.shape[0]
+    rows = np.broadcast_to(table[None], (b,) + table.shape)
+    return orc.score_forward(model, rows, q1[:, None], None if q2 is None else q2[:, None], GAMMA[model], cen)
+
+
+def test_integer_valued_l1_ranks_are_exact_ties_included():
+    """Small integer coordinates: every fp32 sum is exact, scores tie in large numbers, and the ranks
+    must be exactly those of the stable descending order."""
+    from smore_amd import fused
+    from smore_amd.evaluation import filtered_ranks
+    rng = np.random.default_rng(0)
+    n, d, b = 5000, 16, 3
+    table = rng.integers(-3, 4, (n, d)).astype(np.float64)
+    q1 = rng.integers(-3, 4, (b, d)).astype(np.float64)
+    easy = [[3, 77, 4000], [], [11]]
+    hard = [[9, 2500, 4999, 0], [123], list(range(100, 180))]      # 80 answers: two compare chunks
+    params = fused.score_params(GAMMA["l1"], 0.0)
+    got = filtered_ranks("l1", dev(table), dev(q1), None, params, easy, hard)
+    scores = _scores64("l1", table, q1, None, 0.0)
+    assert len(np.unique(scores[0])) < n // 10                       # plenty of exact ties
+    for i in range(b):
+        want_h, want_e = orc.filtered_ranks(scores[i], easy[i], hard[i])
+        assert got[i][0].cpu().numpy().tolist() == want_h.tolist()
+        assert got[i][1].cpu().numpy().tolist() == want_e.tolist()
+
+
+@pytest.mark.parametrize("model,dim", [("box", 200), ("l2", 64), ("rotate", 100), ("beta_kl", 40), ("box", 30)])
+def test_ranks_lie_in_the_interval_fp32_allows(model, dim):
+    """Random floats: an entity whose logit is within fp32 error of an answer's may fall on either side;
+    every rank must lie between the counts with the tolerance subtracted and added."""
+    from smore_amd import fused
+    from smore_amd.evaluation import filtered_ranks, ranking_metrics
+    rng = np.random.default_rng(dim)
+    n, b = 20000, 5
+    table, q1, q2, _, _ = make_problem(model, n, b, 1, dim, rng)
+    easy = [rng.choice(n, size=s, replace=False).tolist() for s in (0, 3, 10, 1, 64)]
+    hard = []
+    for e, s in zip(easy, (1, 5, 70, 0, 130)):
+        pool = np.setdiff1d(np.arange(n), np.array(e, dtype=np.int64))
+        hard.append(rng.choice(pool, size=s, replace=False).tolist())
+    params = fused.score_params(GAMMA[model], 0.02)
+    got = filtered_ranks(model, dev(table), dev(q1), dev(q2), params, easy, hard)
+    scores = _scores64(model, table, q1, q2, 0.02)
+    for i in range(b):
+        is_ans = np.zeros(n, bool)
+        is_ans[easy[i] + hard[i]] = True
+        tol = 2e-5 * max(1.0, np.abs(scores[i]).max())
+        others = np.sort(scores[i][~is_ans])
+        for ids, ranks in ((hard[i], got[i][0]), (easy[i], got[i][1])):
+            r = ranks.cpu().numpy()
+            assert r.shape == (len(ids),)
+            for a, ra in zip(ids, r):
+                lo = 1 + (others.size - np.searchsorted(others, scores[i][a] + tol, side="right"))
+                hi = 1 + (others.size - np.searchsorted(others, scores[i][a] - tol, side="left"))
+                assert lo <= ra <= hi, (model, i, a, ra, lo, hi)
+        m = ranking_metrics(got[i][0])
+        if hard[i]:
+            rr = got[i][0].cpu().numpy().astype(np.float64)
+            assert abs(m["MRR"] - (1 / rr).mean()) < 1e-6 and m["HITS10"] == (rr <= 10).mean()
+        else:
+            assert m == dict(MRR=0.0, HITS1=0.0, HITS3=0.0, HITS10=0.0, HITS1max=0.0)
+
+
+def test_planted_best_entity_and_duplicates_of_it():
+    """An entity equal to the box centre inside the box has distance 0: it ranks first; copies of it at
+    higher ids rank right behind it, in id order."""
+    from smore_amd import fused
+    from smore_amd.evaluation import filtered_ranks
+    rng = np.random.default_rng(4)
+    n, d = 3000, 64
+    table, q1, q2, _, _ = make_problem("box", n, 1, 1, d, rng)
+    for i in (10, 500, 2999):
+        table[i] = q1[0]
+    params = fused.score_params(24.0, 0.02)
+    got = filtered_ranks("box", dev(table), dev(q1), dev(q2), params, [[]], [[500]])
+    assert got[0][0].tolist() == [2]                                # entity 10 ties and has the lower id
+    got = filtered_ranks("box", dev(table), dev(q1), dev(q2), params, [[10]], [[2999, 500]])
+    assert got[0][0].tolist() == [1, 1] and got[0][1].tolist() == [1]  # filtered: answers do not count
+
+
+def test_ranking_argument_errors():
+    from smore_amd import _lib, fused
+    from smore_amd.evaluation import filtered_ranks
+    t = torch.zeros(50, 8, device="cuda")
+    q = torch.zeros(1, 8, device="cuda")
+    p = fused.score_params(1.0)
+    with pytest.raises(IndexError):
+        filtered_ranks("l1", t, q, None, p, [[]], [[50]])
+    with pytest.raises(_lib.SmxError):
+        filtered_ranks("l1", t, q, None, p, [[3]], [[3]])
+    with pytest.raises(_lib.SmxError):
+        filtered_ranks("l1", t, q, None, p, [[]], [[1], [2]])
+    with pytest.raises(_lib.SmxError, match="answers per query"):
+        filtered_ranks("l1", torch.zeros(4000, 8, device="cuda"), q, None, p, [[]], [list(range(2049))])
