@@ -207,6 +207,39 @@ def cpu_baseline(cfg, seed):
     }
 
 
+def rank_scan_bench(cfg, device, seed, steps, warmup):
+    """Evaluation against all entities: one pass over the table per two queries; the roofline is the
+    table streamed once, 4 * row_len * N bytes."""
+    import torch
+    from smore_amd import fused
+    from smore_amd.evaluation import filtered_ranks
+    table, q1, q2, idx, _ = make_inputs(cfg, device, seed)
+    q1, q2 = q1[:2].contiguous(), None if q2 is None else q2[:2].contiguous()
+    params = fused.score_params(cfg["gamma"], cfg["cen"])
+    hard = [idx[b, :16].unique().tolist() for b in range(2)]
+    easy = [[], []]
+    for _ in range(warmup):
+        ranks = filtered_ranks(cfg["model"], table, q1, q2, params, easy, hard)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        ranks = filtered_ranks(cfg["model"], table, q1, q2, params, easy, hard)
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / steps
+    nbytes = 4 * row_len(cfg) * cfg["n"]
+    print(json.dumps({
+        "metric": "all-entity evaluation scan: entities ranked per second (2 queries per pass)",
+        "value": cfg["n"] / (ms * 1e-3), "unit": "entities/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+        "ms_per_step": ms, "higher_is_better": True, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": cfg["name"] + "-rank-scan", "N": cfg["n"], "row_len": row_len(cfg), "queries": 2,
+                   "answers_per_query": [len(h) for h in hard]},
+        "roofline": {"bound": "hbm", "kernel": "rank_scan_kernel (table streamed once)", "achieved": nbytes / (ms * 1e-3) / 1e9,
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+                     "traffic": None},
+        "first_ranks": [r[0][:4].tolist() for r in ranks],
+    }))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -217,6 +250,9 @@ def main():
     ap.add_argument("--no-sign-codes", action="store_true",
                     help="box: do not save sign codes in the forward; the backward re-reads entity and query rows")
     ap.add_argument("--seed", type=int, default=None)
+    ap.add_argument("--rank-scan", action="store_true",
+                    help="time the all-entity evaluation scan (filtered ranks of 16 answers for 2 queries) on the "
+                         "config's table instead of the training step; prints its own JSON line")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run only a plain row copy of known size (1 GiB read + 1 GiB written per launch) through "
                          "smx_gather_rows; under rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE this gives the counters' scale")
@@ -244,6 +280,9 @@ def main():
         return
     cfg = CONFIGS[args.config]
     seed = args.seed if args.seed is not None else 20240 + args.config
+    if args.rank_scan:
+        rank_scan_bench(cfg, device, seed, args.steps, args.warmup)
+        return
 
     table, q1, q2, idx, gscore = make_inputs(cfg, device, seed)
     step = Step(cfg, table, q1, q2, idx, gscore, sign_codes=not args.no_sign_codes)
