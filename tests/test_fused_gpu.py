@@ -371,6 +371,40 @@ def test_sign_codes_give_the_bits_of_the_query_row_path(dim):
     assert_close(out[True][0], want, REL_F32, "merged vs oracle", sum_abs=sum_abs)
 
 
+@pytest.mark.parametrize("b,k,dim", [(3, 37, 200), (5, 100, 64), (2, 1, 8), (1, 300, 6), (9, 17, 512), (4, 65, 31)])
+def test_forward_codes_on_odd_shapes(b, k, dim):
+    """Codes saved by the forward for batch shapes that do not fill the 16-pair staging groups, the
+    64-pair batches or the float4 columns; the backward from codes against the recomputing backward."""
+    from smore_amd import fused
+    rng = np.random.default_rng(b * 100 + k)
+    n = 50
+    table, q1, q2, idx, gs = make_problem("box", n, b, k, dim, rng)
+    t_table, t_q1, t_q2, t_gs = dev(table), dev(q1), dev(q2), dev(gs)
+    t_idx = torch.tensor(idx, device="cuda")
+    params = fused.score_params(24.0, 0.02)
+    plan = fused.build_plan(t_idx, n)
+    saved = fused.new_codes("box", t_table, t_idx, t_q1)
+    score = fused.score_forward("box", t_table, t_idx, t_q1, t_q2, params, codes=saved)
+    assert torch.equal(score, fused.score_forward("box", t_table, t_idx, t_q1, t_q2, params))
+    res = {}
+    for how in ("recompute", "codes"):
+        merged = torch.full((plan.n_uniq, dim), float("nan"), device="cuda")
+        g1, g2 = fused.score_backward_fused("box", plan, t_table, t_idx, t_q1, t_q2, score, t_gs, params,
+                                            merged=merged, sign_codes=False, codes=saved if how == "codes" else None)
+        res[how] = (merged.cpu().numpy(), g1.cpu().numpy(), g2.cpu().numpy())
+    assert np.array_equal(res["codes"][0], res["recompute"][0])
+    assert_close(res["codes"][1], res["recompute"][1], 1e-6, "gq1")
+    assert_close(res["codes"][2], res["recompute"][2], 1e-6, "gq2")
+    w, m, v = t_table.clone(), torch.zeros_like(t_table), torch.zeros_like(t_table)
+    w2, m2, v2 = t_table.clone(), torch.zeros_like(t_table), torch.zeros_like(t_table)
+    fused.score_backward_fused("box", plan, w, t_idx, t_q1, t_q2, score, t_gs, params, m=m, v=v,
+                               adam=fused.adam_params(1e-3, 1), codes=saved)
+    fused.score_backward_fused("box", plan, w2, t_idx, t_q1, t_q2, score, t_gs, params, m=m2, v=v2,
+                               adam=fused.adam_params(1e-3, 1), sign_codes=False)
+    assert_close(m.cpu().numpy(), m2.cpu().numpy(), 2e-6, "m")
+    assert_close(w.cpu().numpy(), w2.cpu().numpy(), 2e-6, "w")
+
+
 def test_sign_codes_keep_the_tie_conventions():
     """Ties (e == c, |e - c| == o, negative offsets) through the coded path: every pair of the tie table,
     under enough queries for the codes to be used, must give the oracle's rows exactly."""
