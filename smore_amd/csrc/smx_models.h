@@ -199,14 +199,19 @@ template <> struct ModelOps<mBox> {
   }
   // As fwd, and pushes this feature's two bits onto `code`: the forward pass
   // can leave the codes too, and then the whole backward works from them without the entity rows.
-  static __device__ __forceinline__ void fwd_coded(float e1, const Q& q, float& a0, float& a1, unsigned& code) {
+  // neg_thr (per query feature, loop-invariant): the "negative" decision  outside ? d <= 0 : d < 0  is
+  // d < neg_thr with neg_thr = 0 where the offset is positive (d == 0 is then inside the box) and the
+  // smallest positive float where it is not (d == 0 is then outside, and d < that means d <= 0): one
+  // compare instead of two compares and three mask operations.
+  static __device__ __forceinline__ float neg_threshold(const Q& q) { return q.b > 0.f ? 0.f : __uint_as_float(1u); }
+  static __device__ __forceinline__ void fwd_coded(float e1, const Q& q, float neg_thr, float& a0, float& a1,
+                                                   unsigned& code) {
     const float d = e1 - q.a;
     const float a = fabsf(d);
     const float mn = min_abs(d, q.b);
     a0 += a - mn;
     a1 += fabsf(mn);
-    const unsigned long long T = __ballot(a >= q.b), GT = __ballot(d > 0.f), GE = __ballot(d >= 0.f);
-    code = push2(code, ~((T & GT) | (~T & GE)), T);
+    code = push2(code, __ballot(d < neg_thr), __ballot(a >= q.b));
   }
   // (t ? c0 : c1) with its sign flipped when the feature's "negative" bit is set: two three-input bit
   // operations (v_bitop3_b32; table index = src0 << 2 | src1 << 1 | src2).

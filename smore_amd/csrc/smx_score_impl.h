@@ -268,6 +268,13 @@ __global__ __launch_bounds__(256) void score_forward_kernel(ScoreArgs A, int til
   unsigned* slab = reinterpret_cast<unsigned*>(lds + model_nq(M) * dim) + wave * kSlabDwords;
   stage_pairs(slab, lane, table, pb, 0.f, 0.f);
 
+  float neg_thr[NIT][VEC];
+  if constexpr (CODED) {
+#pragma unroll
+    for (int it = 0; it < NIT; ++it)
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) neg_thr[it][v] = ModelOps<M>::neg_threshold(q[it][v]);
+  }
   float* out = score + (size_t)b * K + kw0;
   unsigned char* stage =
       reinterpret_cast<unsigned char*>(lds + model_nq(M) * dim + 4 * kSlabDwords) + wave * (kStagePairs * NIT * 64);
@@ -282,7 +289,7 @@ __global__ __launch_bounds__(256) void score_forward_kernel(ScoreArgs A, int til
       if constexpr (CODED) {
         unsigned code = 0;
 #pragma unroll
-        for (int v = 0; v < VEC; ++v) ModelOps<M>::fwd_coded(e1[it].v[v], q[it][v], a0, a1, code);
+        for (int v = 0; v < VEC; ++v) ModelOps<M>::fwd_coded(e1[it].v[v], q[it][v], neg_thr[it][v], a0, a1, code);
         stage[(j & (kStagePairs - 1)) * (NIT * 64) + 64 * it + lane] = (unsigned char)code;
       } else {
 #pragma unroll
