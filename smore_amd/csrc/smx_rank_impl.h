@@ -128,11 +128,10 @@ __global__ __launch_bounds__(256) void rank_answer_keys_kernel(RankArgs A) {
   }
 }
 
-// The scan.  LDS: bins [kRankQueries][A + 1].
-template <int M, int VEC, int NIT, bool REG>
+// The scan for NB (1 or 2) queries.  LDS: bins [NB][A + 1], keys [NB][A].
+template <int M, int VEC, int NIT, bool REG, int NB>
 __global__ __launch_bounds__(256) void rank_scan_kernel(RankArgs A) {
   constexpr int MUL = model_mul(M);
-  constexpr int NB = kRankQueries;
   constexpr int RIF = NIT * MUL <= 2 ? 4 : (NIT * MUL <= 4 ? 2 : 1);
   extern __shared__ unsigned lds_bins[];  // bins [NB][A + 1], then (8-byte aligned) the answers' keys [NB][A]
   const int lane = threadIdx.x & 63;
@@ -158,6 +157,10 @@ __global__ __launch_bounds__(256) void rank_scan_kernel(RankArgs A) {
     load_rank_query<M, VEC, NIT>(A.q1, A.q2, qb[x], dim, A.ncol, lane, q[x]);
   }
   const int chunks = (A.A + 63) / 64;
+  // the first 64 answers' keys stay in registers (most queries have no more); further chunks come from LDS
+  unsigned long long first_keys[NB];
+#pragma unroll
+  for (int x = 0; x < NB; ++x) first_keys[x] = lane < count[x] ? lds_keys[x * A.A + lane] : 0ull;
 
   // wavefronts walk the table together: group g of RIF consecutive rows belongs to wavefront g mod n_waves
   const unsigned long long n_waves = (unsigned long long)gridDim.x * 4ull;
@@ -182,9 +185,9 @@ __global__ __launch_bounds__(256) void rank_scan_kernel(RankArgs A) {
           const float s = row_score<M, VEC, NIT, REG>(x1[r], x2[r], q[x], A.ncol, lane, A.p);
           const float su = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(s), 63));
           const unsigned long long key = rank_key(su, row);
-          int not_beaten = 0;
-          bool is_answer = false;
-          for (int c = 0; c < chunks; ++c) {
+          int not_beaten = __popcll(__ballot(lane < count[x] && !(key > first_keys[x])));
+          bool is_answer = __ballot(lane < count[x] && ((unsigned)~(unsigned)first_keys[x] == (unsigned)row)) != 0ull;
+          for (int c = 1; c < chunks; ++c) {
             const int j = c * 64 + lane;
             const bool live = j < count[x];
             const unsigned long long ak = live ? lds_keys[x * A.A + j] : 0ull;
@@ -247,21 +250,30 @@ int launch_rank_reg(hipStream_t st, RankArgs A, bool keys_only) {
   }
   const size_t n_bins = (size_t)A.B * (A.A + 1);
   hipLaunchKernelGGL(rank_clear_kernel, dim3((unsigned)((n_bins + 255) / 256)), dim3(256), 0, st, A.bins, n_bins);
-  int dev = 0, cus = 256, per_cu = 2;
-  const size_t lds = (((size_t)kRankQueries * (A.A + 1) + 1) & ~(size_t)1) * sizeof(unsigned) +
-                     (size_t)kRankQueries * A.A * sizeof(unsigned long long);
-  if (hipGetDevice(&dev) == hipSuccess) {
-    (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, rank_scan_kernel<M, VEC, NIT, REG>, 256, lds) != hipSuccess ||
-        per_cu < 1)
-      per_cu = 2;
-  }
-  unsigned blocks = (unsigned)cus * (unsigned)per_cu;
-  const unsigned long long want = (A.n_rows + 15) / 16;
-  if (want < blocks) blocks = (unsigned)(want ? want : 1);
+  int dev = 0, cus = 256;
+  if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+  auto lds_bytes = [&](int nb) {
+    return (((size_t)nb * (A.A + 1) + 1) & ~(size_t)1) * sizeof(unsigned) + (size_t)nb * A.A * sizeof(unsigned long long);
+  };
+  auto grid_for = [&](auto kernel, size_t lds) {
+    int per_cu = 2;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, 256, lds) != hipSuccess || per_cu < 1) per_cu = 2;
+    unsigned blocks = (unsigned)cus * (unsigned)per_cu;
+    const unsigned long long want = (A.n_rows + 15) / 16;
+    if (want < blocks) blocks = (unsigned)(want ? want : 1);
+    return blocks;
+  };
   for (int b0 = 0; b0 < A.B; b0 += kRankQueries) {
     A.b0 = b0;
-    hipLaunchKernelGGL((rank_scan_kernel<M, VEC, NIT, REG>), dim3(blocks), dim3(256), lds, st, A);
+    if (A.B - b0 >= 2) {
+      const size_t lds = lds_bytes(2);
+      hipLaunchKernelGGL((rank_scan_kernel<M, VEC, NIT, REG, 2>), dim3(grid_for(rank_scan_kernel<M, VEC, NIT, REG, 2>, lds)),
+                         dim3(256), lds, st, A);
+    } else {
+      const size_t lds = lds_bytes(1);
+      hipLaunchKernelGGL((rank_scan_kernel<M, VEC, NIT, REG, 1>), dim3(grid_for(rank_scan_kernel<M, VEC, NIT, REG, 1>, lds)),
+                         dim3(256), lds, st, A);
+    }
   }
   hipLaunchKernelGGL(rank_finish_kernel, dim3((unsigned)A.B), dim3(256), 0, st, A);
   return check_launch("rank scan");
