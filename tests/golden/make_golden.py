@@ -7,7 +7,10 @@ score model -- inputs, scores, query gradients, the integer segment plan, merged
 and the table / Adam moments after two steps -- so that a later change of the oracle or of the HIP
 path that alters any result is caught against data, not against the same formula.
 
-    python tests/golden/make_golden.py        # rewrites tests/golden/step_*.npz
+loss.npz and ranking.npz do the same for the sample loss (train_process.py:194-213) and for the filtered
+ranks of the all-entity evaluation (train_process.py:112-160).
+
+    python tests/golden/make_golden.py        # rewrites tests/golden/*.npz
 """
 import os
 import sys
@@ -52,7 +55,38 @@ def make(model, seed):
     np.savez_compressed(os.path.join(HERE, f"step_{model}.npz"), **out)
 
 
+def make_loss(seed):
+    rng = np.random.default_rng(seed)
+    b, k = 5, 9
+    f32 = lambda x: x.astype(np.float32).astype(np.float64)
+    pos, neg = f32(rng.standard_normal(b) * 3), f32(rng.standard_normal((b, k)) * 3)
+    mask = (rng.random((b, k)) > 0.3).astype(np.float64)
+    weight = f32(rng.random(b) + 0.1)
+    out = dict(pos=pos, neg=neg, mask=mask, weight=weight, temperature=0.8, scale=0.25)
+    for name, (m, w, t) in dict(plain=(None, None, 0.0), full=(mask, weight, 0.8)).items():
+        pl, nl, gp, gn = orc.sample_loss(pos, neg, m, w, t, 0.25)
+        out.update({f"{name}_pos_loss": pl, f"{name}_neg_loss": nl, f"{name}_gpos": gp, f"{name}_gneg": gn})
+    np.savez_compressed(os.path.join(HERE, "loss.npz"), **out)
+
+
+def make_ranking(seed):
+    """Integer-valued L1 problem: every fp32 sum is exact, so the ranks are the same in any precision."""
+    rng = np.random.default_rng(seed)
+    n, d, b = 600, 8, 2
+    table = rng.integers(-3, 4, (n, d)).astype(np.float64)
+    q1 = rng.integers(-3, 4, (b, d)).astype(np.float64)
+    easy = np.array([[4, 99, 300], [17, 18, 500]], dtype=np.int64)
+    hard = np.array([[7, 250, 599, 0], [1, 2, 3, 400]], dtype=np.int64)
+    rows = np.broadcast_to(table[None], (b, n, d))
+    scores = orc.score_forward("l1", rows, q1[:, None], None, GAMMA["l1"], 0.0)
+    hr, er = zip(*(orc.filtered_ranks(scores[i], easy[i].tolist(), hard[i].tolist()) for i in range(b)))
+    np.savez_compressed(os.path.join(HERE, "ranking.npz"), table=table, q1=q1, easy=easy, hard=hard, gamma=GAMMA["l1"],
+                        scores=scores, hard_ranks=np.array(hr), easy_ranks=np.array(er))
+
+
 if __name__ == "__main__":
     for i, model in enumerate(GAMMA):
         make(model, 100 + i)
+    make_loss(200)
+    make_ranking(300)
     print("wrote", sorted(f for f in os.listdir(HERE) if f.endswith(".npz")))

@@ -1,4 +1,4 @@
-"""Committed golden fixtures (tests/golden/step_*.npz): the oracle must reproduce them on the CPU,
+"""Committed golden fixtures (tests/golden/*.npz): the oracle must reproduce them on the CPU,
 the HIP path on the GPU."""
 import glob
 import os
@@ -9,7 +9,7 @@ import pytest
 from oracle import oracle as orc
 from tests.util import REL_F32, assert_close
 
-GOLDEN = sorted(glob.glob(os.path.join(os.path.dirname(__file__), "golden", "step_*.npz")))
+GOLDEN = sorted(glob.glob(os.path.join(os.path.dirname(__file__), "golden", "step_*.npz")))  # one per score model
 
 
 def _load(path):
@@ -74,3 +74,72 @@ def test_hip_path_reproduces_fixture(path):
     assert_close(m.cpu().numpy(), d["m_after"], 5 * REL_F32, "m after two steps")
     err = np.abs(table.cpu().numpy() - d["w_after"])
     assert err.max() < 2 * float(d["lr"]) and (err > 1e-5 * np.maximum(np.abs(d["w_after"]), 0.04)).mean() < 0.01
+
+
+@pytest.mark.gpu
+def test_timed_path_reproduces_the_box_fixture():
+    """Forward that saves sign codes + one-call backward (what bench.py times) on the box fixture."""
+    import torch
+    from smore_amd import fused
+    _, d = _load(os.path.join(os.path.dirname(__file__), "golden", "step_box.npz"))
+    dev = lambda a: torch.tensor(a, dtype=torch.float32, device="cuda")
+    table, q1, q2, gs = dev(d["table"]), dev(d["q1"]), dev(d["q2"]), dev(d["gs"])
+    idx = torch.tensor(d["idx"], device="cuda")
+    params = fused.score_params(float(d["gamma"]), float(d["cen"]))
+    plan = fused.build_plan(idx, table.shape[0])
+    codes = fused.new_codes("box", table, idx, q1)
+    score = fused.score_forward("box", table, idx, q1, q2, params, codes=codes)
+    assert_close(score.cpu().numpy(), d["score"], REL_F32, "score")
+    merged = torch.empty((plan.n_uniq, table.shape[1]), device="cuda")
+    gq1, gq2 = fused.score_backward_fused("box", plan, table, idx, q1, q2, score, gs, params, merged=merged, codes=codes)
+    assert_close(gq1.cpu().numpy(), d["gq1"], REL_F32, "gq1")
+    assert_close(gq2.cpu().numpy(), d["gq2"], REL_F32, "gq2")
+    assert_close(merged.cpu().numpy(), d["merged"], REL_F32, "merged")
+    m, v = torch.zeros_like(table), torch.zeros_like(table)
+    for step in (1, 2):
+        score = fused.score_forward("box", table, idx, q1, q2, params, codes=codes)
+        fused.score_backward_fused("box", plan, table, idx, q1, q2, score, gs, params, m=m, v=v,
+                                   adam=fused.adam_params(float(d["lr"]), step), codes=codes)
+    assert_close(m.cpu().numpy(), d["m_after"], 5 * REL_F32, "m after two steps")
+    err = np.abs(table.cpu().numpy() - d["w_after"])
+    assert err.max() < 2 * float(d["lr"]) and (err > 1e-5 * np.maximum(np.abs(d["w_after"]), 0.04)).mean() < 0.01
+
+
+def _golden(name):
+    return dict(np.load(os.path.join(os.path.dirname(__file__), "golden", name), allow_pickle=False))
+
+
+def test_oracle_reproduces_loss_and_ranking_fixtures():
+    d = _golden("loss.npz")
+    for name, (m, w, t) in dict(plain=(None, None, 0.0), full=(d["mask"], d["weight"], float(d["temperature"]))).items():
+        pl, nl, gp, gn = orc.sample_loss(d["pos"], d["neg"], m, w, t, float(d["scale"]))
+        assert abs(pl - float(d[f"{name}_pos_loss"])) < 1e-13 and abs(nl - float(d[f"{name}_neg_loss"])) < 1e-13
+        assert np.allclose(gp, d[f"{name}_gpos"], rtol=1e-12, atol=0) and np.allclose(gn, d[f"{name}_gneg"], rtol=1e-12, atol=0)
+    r = _golden("ranking.npz")
+    for i in range(r["q1"].shape[0]):
+        h, e = orc.filtered_ranks(r["scores"][i], r["easy"][i].tolist(), r["hard"][i].tolist())
+        assert np.array_equal(h, r["hard_ranks"][i]) and np.array_equal(e, r["easy_ranks"][i])
+
+
+@pytest.mark.gpu
+def test_hip_path_reproduces_loss_and_ranking_fixtures():
+    import torch
+    from smore_amd import fused
+    from smore_amd.evaluation import filtered_ranks
+    from smore_amd.training import sample_loss
+    dev = lambda a: torch.tensor(a, dtype=torch.float32, device="cuda")
+    d = _golden("loss.npz")
+    for name, (m, w, t) in dict(plain=(None, None, 0.0), full=(d["mask"], d["weight"], float(d["temperature"]))).items():
+        tp, tn = dev(d["pos"]).requires_grad_(), dev(d["neg"]).requires_grad_()
+        loss, pl, nl = sample_loss(tp, tn, None if m is None else dev(m), None if w is None else dev(w), t, world_size=2)
+        loss.backward()
+        assert abs(pl.item() - float(d[f"{name}_pos_loss"])) <= REL_F32 * abs(float(d[f"{name}_pos_loss"]))
+        assert abs(nl.item() - float(d[f"{name}_neg_loss"])) <= REL_F32 * abs(float(d[f"{name}_neg_loss"]))
+        assert_close(tp.grad.cpu().numpy(), d[f"{name}_gpos"], REL_F32, "gpos")
+        assert_close(tn.grad.cpu().numpy(), d[f"{name}_gneg"], REL_F32, "gneg")
+    r = _golden("ranking.npz")
+    got = filtered_ranks("l1", dev(r["table"]), dev(r["q1"]), None, fused.score_params(float(r["gamma"])),
+                         [x.tolist() for x in r["easy"]], [x.tolist() for x in r["hard"]])
+    for i, (h, e) in enumerate(got):
+        assert h.cpu().numpy().tolist() == r["hard_ranks"][i].tolist()
+        assert e.cpu().numpy().tolist() == r["easy_ranks"][i].tolist()
