@@ -1,54 +1,79 @@
-"""Sparse entity table (surface of smore/common/embedding/sparse_embed.py:26-67).
+"""Entity table kept in HBM, with the calling surface of smore/common/embedding/sparse_embed.py:26-67.
 
-The table and, once an optimizer is attached, its moment buffers live in HBM for the whole run; row
-lookups go through `fwd_delegate` when an EmbeddingOptimizer has installed itself, exactly like the
-reference, so model code keeps calling `entity_embedding(ids, name)`.
+Model code of the reference talks to the table through three things only: `entity_embedding(ids, name)`
+returns rows carrying a `.job_handle` whose `.sync()` it may call, `entity_embedding(None)` returns the
+whole table (evaluation against all entities), and an `EmbeddingOptimizer` may install itself as
+`fwd_delegate` to take the lookups over (embed_optimizer.py:116-121).  This class keeps exactly that
+contract; the rows themselves come from the HIP gather, and the optimizer state the optimizers register
+(`register_tensor`) becomes part of the module's state_dict under the reference's buffer names.
 """
 import torch
-import torch.nn as nn
+from torch import nn
 
-from .. import fused
+from .. import _lib, fused
 
 
 class DummyJob:
-    """Completed-job handle: the in-HBM lookup has nothing to wait for (embed_rw.py DummyJob)."""
+    """Handle of a lookup that is already complete (the role of embed_rw.py's DummyJob): rows gathered
+    on the device are ordered by the stream, so there is nothing for the caller to wait for."""
+
+    __slots__ = ()
 
     def sync(self):
         return None
 
 
+_DONE = DummyJob()
+
+
 class SparseEmbedding(nn.Module):
+    """[num_rows, num_cols] fp32 table whose rows are read by id and updated sparsely.
+
+    Attributes used by callers: `embedding` (the nn.Parameter), `num_rows`, `fwd_delegate`, `dummy_job`,
+    `device`, `shape`."""
 
     def __init__(self, num_rows, num_cols):
         super().__init__()
-        self.num_rows = num_rows
-        self.embedding = nn.Parameter(torch.zeros(num_rows, num_cols))
-        self.fwd_delegate = None
-        self.dummy_job = DummyJob()
+        if num_rows < 0 or num_cols <= 0:
+            raise ValueError(f"bad table shape {num_rows} x {num_cols}")
+        self.num_rows = int(num_rows)
+        self.dummy_job = _DONE
+        self.fwd_delegate = None  # set by EmbeddingOptimizer.__init__
+        self.embedding = nn.Parameter(torch.zeros((self.num_rows, int(num_cols)), dtype=torch.float32))
 
-    @property
-    def device(self):
-        return self.embedding.device
+    # ---- what callers ask about the table
+    shape = property(lambda self: self.embedding.shape)
+    device = property(lambda self: self.embedding.device)
 
-    @property
-    def shape(self):
-        return self.embedding.shape
+    def extra_repr(self):
+        return f"rows={self.num_rows}, cols={self.embedding.shape[1]}, device={self.embedding.device}"
 
+    # ---- set-up
     def init_params(self, lb, ub):
-        nn.init.uniform_(tensor=self.embedding, a=lb, b=ub)
+        """Uniform initial values in [lb, ub) (the reference's embedding_range)."""
+        with torch.no_grad():
+            self.embedding.uniform_(lb, ub)
 
     def register_tensor(self, name, tensor_obj):
+        """Optimizer state that must be saved and moved with the table (e.g. state_sum_fo / state_sum_sq)."""
+        if tensor_obj.shape[0] != self.num_rows:
+            raise _lib.SmxError(f"{name}: one state row per table row is needed")
         self.register_buffer(name, tensor_obj)
 
+    # ---- lookups
+    def _rows(self, indices):
+        table = self.embedding.detach()
+        with torch.no_grad():
+            return fused.gather_rows(table, indices.to(table.device))
+
     def forward(self, indices, name=None):
-        if self.num_rows == 0:
+        """Rows `indices` of the table (`None`: the table itself), tagged with a finished job handle.
+        With an optimizer attached the lookup is the optimizer's (it records what to update)."""
+        if not self.num_rows:
             return None
-        if self.fwd_delegate is not None:
-            return self.fwd_delegate(indices, name)
-        if indices is None:
-            mat = self.embedding
-        else:
-            with torch.no_grad():
-                mat = fused.gather_rows(self.embedding.detach(), indices.to(self.embedding.device))
-        mat.job_handle = self.dummy_job
-        return mat
+        delegate = self.fwd_delegate
+        if delegate is not None:
+            return delegate(indices, name)
+        out = self.embedding if indices is None else self._rows(indices)
+        out.job_handle = self.dummy_job
+        return out
