@@ -121,11 +121,14 @@ int smx_score_forward(int model, void* stream, const float* table, size_t n_rows
 /* Query-side gradient of sum(gscore * score): gq1, gq2 [B, dim] are overwritten.
  * `score` is the tensor smx_score_forward wrote (L2 needs it for the chain
  * rule of the square root).  Replaces dist_backward_query_kernel
- * (common_kernel.h:92-123) plus the autograd nodes between it and the logit. */
+ * (common_kernel.h:92-123) plus the autograd nodes between it and the logit.
+ * fwd_codes (may be NULL): the sign codes smx_score_forward wrote for these pairs; the kernel then
+ * reads them instead of the entity rows. */
 int smx_score_backward_query(int model, void* stream, const float* table, size_t n_rows,
                              const int64_t* idx, const float* q1, const float* q2,
                              const float* score, const float* gscore, float* gq1, float* gq2,
-                             size_t B, size_t K, size_t dim, const smx_score_params* params);
+                             size_t B, size_t K, size_t dim, const smx_score_params* params,
+                             const void* fwd_codes, size_t fwd_codes_bytes);
 
 /* ---- segment plan ----------------------------------------------------------
  * Groups the P = B*K pairs of a step by entity id on the device.  Replaces
@@ -194,13 +197,15 @@ typedef struct smx_opt_params {
  *                    plan are not touched.
  * Replaces dist_backward_ent_kernel (common_kernel.h:59-89), EmbedLookupFunc.backward
  * (embed_optimizer.py:63-66), merge_grad_list (:45-48) and update_step (:208-252).
- * workspace: smx_entity_workspace_bytes(P, dim*mul) bytes, 256-byte aligned. */
+ * workspace: smx_entity_workspace_bytes(P, dim*mul) bytes, 256-byte aligned.
+ * fwd_codes (may be NULL): the forward's sign codes; they replace the reads of the query rows. */
 size_t smx_entity_workspace_bytes(size_t n_pairs, size_t row_len);
 int smx_score_backward_entity(int model, void* stream, const smx_plan_view* plan, float* table,
                               size_t n_rows, const float* q1, const float* q2, const float* score,
                               const float* gscore, size_t B, size_t K, size_t dim,
                               const smx_score_params* params, float* merged, float* m, float* v,
-                              const smx_opt_params* adam, void* workspace, size_t workspace_bytes);
+                              const smx_opt_params* adam, void* workspace, size_t workspace_bytes,
+                              const void* fwd_codes, size_t fwd_codes_bytes);
 
 /* Everything after the loss in one call: query gradients, and every entity row of the step finished
  * (merged gradient row and/or lazy Adam on w, m, v), as smx_score_backward_query followed by

@@ -32,17 +32,19 @@ SIGNATURES = {
     "smx_score_codes_bytes": (_sz, [_i, _sz, _sz]),
     # model, stream, table, n_rows, idx, q1, q2, score, B, K, dim, params, err_flag, codes, codes_bytes
     "smx_score_forward": (_i, [_i, _vp, _vp, _sz, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _vp, _vp, _vp, _sz]),
-    # model, stream, table, n_rows, idx, q1, q2, score, gscore, gq1, gq2, B, K, dim, params
-    "smx_score_backward_query": (_i, [_i, _vp, _vp, _sz, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _vp]),
+    # model, stream, table, n_rows, idx, q1, q2, score, gscore, gq1, gq2, B, K, dim, params, fwd_codes, bytes
+    "smx_score_backward_query": (_i, [_i, _vp, _vp, _sz, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _vp, _vp,
+                                      _sz]),
     "smx_plan_workspace_bytes": (_sz, [_sz, _sz]),
     # stream, idx, n_pairs, n_rows, ws, ws_bytes, order, sorted_ids, seg_of_pos, uniq, seg_start, inverse, pair_seg,
     # n_uniq, err
     "smx_plan_build": (_i, [_vp, _vp, _sz, _sz, _vp, _sz, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "smx_entity_workspace_bytes": (_sz, [_sz, _sz]),
     "smx_fused_workspace_bytes": (_sz, [_i, _sz, _sz]),
-    # model, stream, plan, table, n_rows, q1, q2, score, gscore, B, K, dim, params, merged, m, v, adam, ws, ws_bytes
+    # model, stream, plan, table, n_rows, q1, q2, score, gscore, B, K, dim, params, merged, m, v, adam, ws, ws_bytes,
+    # fwd_codes, bytes
     "smx_score_backward_entity": (_i, [_i, _vp, _vp, _vp, _sz, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _vp, _vp, _vp, _vp,
-                                       _vp, _vp, _sz]),
+                                       _vp, _vp, _sz, _vp, _sz]),
     # model, stream, plan, table, n_rows, idx, q1, q2, score, gscore, gq1, gq2, B, K, dim, params, merged, m, v,
     # adam, ws, ws_bytes, fwd_codes, fwd_codes_bytes
     "smx_score_backward_fused": (_i, [_i, _vp, _vp, _vp, _sz, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _vp,

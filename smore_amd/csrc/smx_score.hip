@@ -149,12 +149,18 @@ int smx_score_forward(int model, void* stream, const float* table, size_t n_rows
 
 int smx_score_backward_query(int model, void* stream, const float* table, size_t n_rows, const int64_t* idx,
                              const float* q1, const float* q2, const float* score, const float* gscore, float* gq1,
-                             float* gq2, size_t B, size_t K, size_t dim, const smx_score_params* params) {
+                             float* gq2, size_t B, size_t K, size_t dim, const smx_score_params* params,
+                             const void* fwd_codes, size_t fwd_codes_bytes) {
   using namespace smx;
   ScoreArgs A;
   int vec, nit;
   if (int rc = fill_args(&A, &vec, &nit, model, table, n_rows, idx, q1, q2, B, K, dim, params, nullptr, nullptr)) return rc;
   if (!score || !gscore || !gq1 || (model_nq(model) == 2 && !gq2)) return fail(SMX_ERR_ARG, "null pointer");
+  if (fwd_codes) {
+    if (const char* msg = codes_mismatch(model, B * K, dim, vec, nit, fwd_codes_bytes)) return fail(SMX_ERR_ARG, "%s", msg);
+    if (reinterpret_cast<uintptr_t>(fwd_codes) & 15u) return fail(SMX_ERR_ARG, "codes must be 16-byte aligned");
+    A.codes_in = static_cast<const unsigned char*>(fwd_codes);
+  }
   A.score = score;
   A.gscore = gscore;
   A.gq1 = gq1;

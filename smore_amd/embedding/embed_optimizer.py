@@ -62,8 +62,10 @@ class _FusedScoreFunc(torch.autograd.Function):
     def forward(ctx, embed_opt, dummy_tensor, model, ids, params, q1, q2):
         table = embed_opt.sparse_embed.embedding.detach()
         with torch.no_grad():
-            score = fused.score_forward(model, table, ids, q1, q2, params, embed_opt.err_flag)
-        ctx.embed_opt, ctx.model, ctx.ids, ctx.params = embed_opt, model, ids, params
+            # box: the forward leaves 2-bit sign codes from which both backward passes work (None otherwise)
+            codes = fused.new_codes(model, table, ids, q1) if table.shape[1] % 4 == 0 else None
+            score = fused.score_forward(model, table, ids, q1, q2, params, embed_opt.err_flag, codes=codes)
+        ctx.embed_opt, ctx.model, ctx.ids, ctx.params, ctx.codes = embed_opt, model, ids, params, codes
         ctx.save_for_backward(q1.detach(), q2.detach() if q2 is not None else None, score)
         ctx.idx_fwd = embed_opt.n_fwd
         embed_opt.n_fwd += 1
@@ -76,8 +78,9 @@ class _FusedScoreFunc(torch.autograd.Function):
         table = opt.sparse_embed.embedding.detach()
         with torch.no_grad():
             gscore = gscore.contiguous()
-            gq1, gq2 = fused.score_backward_query(ctx.model, table, ctx.ids, q1, q2, score, gscore, ctx.params)
-        opt.accumulate_fused(ctx.model, ctx.ids, q1, q2, score, gscore, ctx.params, ctx.idx_fwd)
+            gq1, gq2 = fused.score_backward_query(ctx.model, table, ctx.ids, q1, q2, score, gscore, ctx.params,
+                                                  codes=ctx.codes)
+        opt.accumulate_fused(ctx.model, ctx.ids, q1, q2, score, gscore, ctx.params, ctx.idx_fwd, ctx.codes)
         return None, None, None, None, None, gq1, gq2
 
 
@@ -132,8 +135,9 @@ class EmbeddingOptimizer(ABC):
         self.grad_list.append((indices, grad_submat))
         self.has_grad_list.append(fwd_idx)
 
-    def accumulate_fused(self, model, ids, q1, q2, score, gscore, params, fwd_idx):
-        self.fused_list.append(dict(model=model, ids=ids, q1=q1, q2=q2, score=score, gscore=gscore, params=params))
+    def accumulate_fused(self, model, ids, q1, q2, score, gscore, params, fwd_idx, codes=None):
+        self.fused_list.append(dict(model=model, ids=ids, q1=q1, q2=q2, score=score, gscore=gscore, params=params,
+                                    codes=codes))
         self.has_grad_list.append(fwd_idx)
 
     def forward(self, indices, name=None):
@@ -184,7 +188,7 @@ class EmbeddingOptimizer(ABC):
                 plan = fused.build_plan(rec["ids"], n_rows, err_flag=self.err_flag)
                 merged = torch.empty((plan.n_uniq, table.shape[1]), dtype=torch.float32, device=table.device)
                 fused.score_backward_entity(rec["model"], plan, table, rec["q1"], rec["q2"], rec["score"],
-                                            rec["gscore"], rec["params"], merged=merged)
+                                            rec["gscore"], rec["params"], merged=merged, codes=rec["codes"])
                 idx_list.append(plan.uniq)
                 grad_list.append(merged)
             flat = torch.cat(idx_list, dim=0)
@@ -227,7 +231,8 @@ class _RowOptimizer(EmbeddingOptimizer):
     def update_fused(self, plan, rec, lr):
         m, v = self._state()
         fused.score_backward_entity(rec["model"], plan, self.sparse_embed.embedding.detach(), rec["q1"], rec["q2"],
-                                    rec["score"], rec["gscore"], rec["params"], m=m, v=v, adam=self._params(lr))
+                                    rec["score"], rec["gscore"], rec["params"], m=m, v=v, adam=self._params(lr),
+                                    codes=rec["codes"])
 
 
 class AdamEmbedOptimizer(_RowOptimizer):

@@ -95,8 +95,8 @@ def score_forward(model, table, idx, q1, q2, params, err_flag=None, codes=None):
     return score
 
 
-def score_backward_query(model, table, idx, q1, q2, score, gscore, params):
-    """Gradients of sum(gscore * score) w.r.t. q1 (and q2)."""
+def score_backward_query(model, table, idx, q1, q2, score, gscore, params, codes=None):
+    """Gradients of sum(gscore * score) w.r.t. q1 (and q2).  codes: what score_forward saved (optional)."""
     b, k, dim = _dims(model, table, idx, q1, q2)
     _f32(score, "score")
     _f32(gscore, "gscore")
@@ -105,7 +105,7 @@ def score_backward_query(model, table, idx, q1, q2, score, gscore, params):
     with torch.cuda.device(table.device):
         _lib.call("smx_score_backward_query", MODELS[model], _stream(table), _ptr(table), table.shape[0], _ptr(idx),
                   _ptr(q1), _ptr(q2), _ptr(score), _ptr(gscore), _ptr(gq1), _ptr(gq2), b, k, dim,
-                  ctypes.byref(params))
+                  ctypes.byref(params), _ptr(codes), 0 if codes is None else codes.numel())
     return gq1, gq2
 
 
@@ -199,9 +199,10 @@ def _check_state(table, m, v, opt):
             raise _lib.SmxError("the second-moment table must be [N, row], or [N] / [N,1] with squeeze")
 
 
-def score_backward_entity(model, plan, table, q1, q2, score, gscore, params, merged=None, m=None, v=None, adam=None):
+def score_backward_entity(model, plan, table, q1, q2, score, gscore, params, merged=None, m=None, v=None, adam=None,
+                          codes=None):
     """Segmented entity gradient of sum(gscore * score); writes merged [>=U, row] and/or applies lazy Adam
-    to table, m, v in place (all of the table's shape)."""
+    to table, m, v in place (all of the table's shape).  codes: what score_forward saved (optional)."""
     b, dim = q1.shape[0], q1.shape[-1]
     k = plan.n_pairs // b
     if model not in MODELS:
@@ -218,7 +219,8 @@ def score_backward_entity(model, plan, table, q1, q2, score, gscore, params, mer
         view = plan.view()
         _lib.call("smx_score_backward_entity", MODELS[model], _stream(table), ctypes.byref(view), _ptr(table),
                   table.shape[0], _ptr(q1), _ptr(q2), _ptr(score), _ptr(gscore), b, k, dim, ctypes.byref(params),
-                  _ptr(merged), _ptr(m), _ptr(v), None if adam is None else ctypes.byref(adam), _ptr(ws), ws.numel())
+                  _ptr(merged), _ptr(m), _ptr(v), None if adam is None else ctypes.byref(adam), _ptr(ws), ws.numel(),
+                  _ptr(codes), 0 if codes is None else codes.numel())
 
 
 def score_backward_fused(model, plan, table, idx, q1, q2, score, gscore, params, merged=None, m=None, v=None,

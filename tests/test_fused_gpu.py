@@ -395,6 +395,13 @@ def test_forward_codes_on_odd_shapes(b, k, dim):
     assert np.array_equal(res["codes"][0], res["recompute"][0])
     assert_close(res["codes"][1], res["recompute"][1], 1e-6, "gq1")
     assert_close(res["codes"][2], res["recompute"][2], 1e-6, "gq2")
+    # the two separate entry points accept the forward's codes too
+    s1, s2 = fused.score_backward_query("box", t_table, t_idx, t_q1, t_q2, score, t_gs, params, codes=saved)
+    assert_close(s1.cpu().numpy(), res["recompute"][1], 1e-6, "gq1 (separate call, codes)")
+    assert_close(s2.cpu().numpy(), res["recompute"][2], 1e-6, "gq2 (separate call, codes)")
+    merged_s = torch.full((plan.n_uniq, dim), float("nan"), device="cuda")
+    fused.score_backward_entity("box", plan, t_table, t_q1, t_q2, score, t_gs, params, merged=merged_s, codes=saved)
+    assert np.array_equal(merged_s.cpu().numpy(), res["recompute"][0])
     w, m, v = t_table.clone(), torch.zeros_like(t_table), torch.zeros_like(t_table)
     w2, m2, v2 = t_table.clone(), torch.zeros_like(t_table), torch.zeros_like(t_table)
     fused.score_backward_fused("box", plan, w, t_idx, t_q1, t_q2, score, t_gs, params, m=m, v=v,
