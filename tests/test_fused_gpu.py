@@ -562,3 +562,39 @@ def test_unsupported_rows_are_refused_not_mangled():
                             fused.score_params(1.0, regularizer=(1.0, 0.05, 1e9)))
     with pytest.raises(_lib.SmxError):  # empty batch
         fused.build_plan(torch.zeros(0, dtype=torch.int64, device="cuda"), 10)
+
+
+def test_second_stream_backward_gives_the_bits_of_the_serial_one(monkeypatch):
+    """Steps of a million pairs or more with the forward's codes and an optimizer run the entity pass on
+    the library's second stream beside the query-gradient kernel.  Same kernels, same data, disjoint
+    rows: the results must be bit-identical to the one-stream order, and repeatable."""
+    import bench
+    from smore_amd import fused
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(7)
+    n, b, k, dim = 2_000_000, 1100, 1024, 200
+    table = torch.empty((n, dim), device="cuda").uniform_(-0.07, 0.07, generator=gen)
+    q1 = torch.empty((b, dim), device="cuda").uniform_(-0.07, 0.07, generator=gen)
+    q2 = torch.empty((b, dim), device="cuda").uniform_(0.0, 0.07, generator=gen)
+    idx = bench.zipf_ids(n, (b, k), 1.1, gen, torch.device("cuda"))
+    gs = torch.randn((b, k), device="cuda", generator=gen)
+    params = fused.score_params(24.0, 0.02)
+    plan = fused.build_plan(idx, n)
+    codes = fused.new_codes("box", table, idx, q1)
+    score = fused.score_forward("box", table, idx, q1, q2, params, codes=codes)
+    results = []
+    for serial in ("1", None, None):
+        if serial:
+            monkeypatch.setenv("SMX_SERIAL_BACKWARD", serial)
+        else:
+            monkeypatch.delenv("SMX_SERIAL_BACKWARD", raising=False)
+        w, m, v = table.clone(), torch.zeros_like(table), torch.zeros_like(table)
+        g1, g2 = fused.score_backward_fused("box", plan, w, idx, q1, q2, score, gs, params, m=m, v=v,
+                                            adam=fused.adam_params(1e-4, 1), codes=codes)
+        torch.cuda.synchronize()
+        results.append((g1, g2, w, m, v))
+    for other in results[1:]:
+        for a, c in zip(results[0], other):
+            assert torch.equal(a, c)
+    touched = (results[0][3].abs().sum(dim=1) != 0).sum().item()
+    assert abs(touched - plan.n_uniq) <= int((gs == 0).sum().item())
