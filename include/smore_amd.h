@@ -104,7 +104,8 @@ typedef struct smx_score_params {
   float reg_hi;
 } smx_score_params;
 
-/* Sign codes (optional, what autograd would call a saved tensor).  For the box model the derivative
+/* Sign codes (optional, what autograd would call a saved tensor).  For the box model (and, with one
+ * decision per feature, L1) the derivative
  * of a pair's distance w.r.t. each feature is +-c0 or +-c1, decided by comparisons the forward pass
  * makes anyway.  Given a `codes` buffer of smx_score_codes_bytes(model, B*K, dim) bytes (16-byte
  * aligned), the forward leaves those decisions there, two bits per feature; handed to

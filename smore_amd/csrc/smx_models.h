@@ -28,7 +28,7 @@ enum Model : int { mL1 = 0, mL2 = 1, mBox = 2, mRotate = 3, mBetaKL = 4, mNumMod
 __host__ __device__ constexpr int model_mul(int m) { return (m == mRotate || m == mBetaKL) ? 2 : 1; }
 __host__ __device__ constexpr int model_nq(int m) { return (m == mL1 || m == mL2) ? 1 : 2; }
 // models whose entity derivative can be kept as sign codes (ModelOps<M>::bwd_q_coded / bwd_e_coded)
-__host__ __device__ constexpr bool model_coded(int m) { return m == mBox; }
+__host__ __device__ constexpr bool model_coded(int m) { return m == mBox || m == mL1; }
 
 struct ScoreParams {
   float gamma;
@@ -61,6 +61,26 @@ template <int M>
 __device__ __forceinline__ void finish_query_grad(const typename ModelOps<M>::Q& q, float& g1, float& g2,
                                                   const ScoreParams& p);
 
+// ---- sign codes -----------------------------------------------------------------------------
+// Models whose entity derivative is a choice among a few values (L1: +-c0; box: +-c0, +-c1) can keep
+// that choice as two bits per feature -- lower bit "outside" (box only), upper bit "negative" -- one
+// byte per float4 column; the features of a column are pushed in ascending order, so the last one
+// sits in bits 0-1 and feature x of VEC at position VEC-1-x.
+// push2: code = 4 * code + 2 * (lane's bit of hi) + (lane's bit of lo): two v_addc with the masks as
+// carry-in.  The s_nop covers the wait states a VALU read of an SGPR needs after a VALU compare
+// wrote it (the assembler does not look into inline asm).
+__device__ __forceinline__ unsigned push2(unsigned code, unsigned long long hi, unsigned long long lo) {
+  unsigned long long carry;
+  asm("s_nop 1\n\t"
+      "v_addc_co_u32_e64 %0, %1, %0, %0, %2\n\t"
+      "v_addc_co_u32_e64 %0, %1, %0, %0, %3"
+      : "+v"(code), "=&s"(carry)
+      : "s"(hi), "s"(lo));
+  return code;
+}
+// the "negative" bit of position x as a sign-bit mask
+__device__ __forceinline__ unsigned code_sign(unsigned code, int x) { return (code << (30 - 2 * x)) & 0x80000000u; }
+
 template <> struct ModelOps<mL1> {
   using Q = QPair;
   static __device__ __forceinline__ Q prep(float q1, float) { return {q1, 0.f}; }
@@ -80,6 +100,26 @@ template <> struct ModelOps<mL1> {
   static __device__ __forceinline__ void bwd_q(float c0, float, float e1, float, const Q& q, float& gq1, float&) {
     float s1 = 0, s2 = 0, s3 = 0;
     Term<kL1, float>::bwd(c0, e1, 0.f, q.a, 0.f, s1, s2, gq1, s3);
+  }
+  // sign codes: the derivative is c0 where e - q > 0 and -c0 elsewhere (sign(0) = -1, dist_kernel.h:141)
+  static __device__ __forceinline__ float neg_threshold(const Q&) { return 0.f; }
+  static __device__ __forceinline__ void fwd_coded(float e1, const Q& q, float, float& a0, float&, unsigned& code) {
+    const float d = e1 - q.a;
+    a0 += fabsf(d);
+    code = push2(code, __ballot(!(d > 0.f)), 0ull);
+  }
+  static __device__ __forceinline__ void bwd_q_coded(float c0, float, float e1, const Q& q, float& gq1, float&,
+                                                     unsigned& code) {
+    const float d = e1 - q.a;
+    const bool pos = d > 0.f;
+    gq1 -= pos ? c0 : -c0;
+    code = push2(code, __ballot(!pos), 0ull);
+  }
+  static __device__ __forceinline__ void bwd_q_from_code(float c0, float, unsigned code, int x, float& gq1, float&) {
+    gq1 -= __uint_as_float(__float_as_uint(c0) ^ code_sign(code, x));
+  }
+  static __device__ __forceinline__ void bwd_e_coded(float c0, float, unsigned code, int x, float& ge) {
+    ge += __uint_as_float(__float_as_uint(c0) ^ code_sign(code, x));
   }
 };
 
@@ -168,23 +208,10 @@ template <> struct ModelOps<mBox> {
   }
 
   // ---- sign codes ----
-  // The derivative of a pair's distance w.r.t. one entity feature is +-c0 or +-c1: two bits say which
-  // (lower bit: outside, upper bit: negative; the features of a column are pushed in ascending order, so the
-  // last one sits in bits 0-1 and feature x of VEC at position VEC-1-x).  The query-gradient kernel, which makes these decisions anyway,
-  // can leave them behind, one byte per four features; the entity pass then sums  +-c  straight from
-  // the codes and needs neither the query rows nor the comparisons -- same decisions, same bits.
-  // push2: code = 4 * code + 2 * (lane's bit of hi) + (lane's bit of lo): two v_addc with the masks as
-  // carry-in.  The s_nop covers the wait states a VALU read of an SGPR needs after a VALU compare
-  // wrote it (the assembler does not look into inline asm).
-  static __device__ __forceinline__ unsigned push2(unsigned code, unsigned long long hi, unsigned long long lo) {
-    unsigned long long carry;
-    asm("s_nop 1\n\t"
-        "v_addc_co_u32_e64 %0, %1, %0, %0, %2\n\t"
-        "v_addc_co_u32_e64 %0, %1, %0, %0, %3"
-        : "+v"(code), "=&s"(carry)
-        : "s"(hi), "s"(lo));
-    return code;
-  }
+  // The derivative of a pair's distance w.r.t. one entity feature is +-c0 or +-c1: two bits say which.
+  // The kernels that make these decisions anyway (forward, or the query-gradient kernel) can leave
+  // them behind, one byte per four features; the entity pass then sums  +-c  straight from the codes
+  // and needs neither the query rows nor the comparisons -- same decisions, same bits.
   // As bwd_q, and pushes this feature's two bits onto `code`.
   static __device__ __forceinline__ void bwd_q_coded(float c0, float c1, float e1, const Q& q, float& gc, float& go,
                                                      unsigned& code) {

@@ -598,3 +598,61 @@ def test_second_stream_backward_gives_the_bits_of_the_serial_one(monkeypatch):
             assert torch.equal(a, c)
     touched = (results[0][3].abs().sum(dim=1) != 0).sum().item()
     assert abs(touched - plan.n_uniq) <= int((gs == 0).sum().item())
+
+
+@pytest.mark.parametrize("b,k,dim", [(6, 50, 128), (3, 7, 30), (40, 300, 200)])
+def test_l1_sign_codes(b, k, dim):
+    """L1 keeps one decision per feature (e - q > 0, ties go to -1): forward-saved codes, codes written by the
+    query-gradient kernel, and the recomputing path give the same merged rows bit for bit; ties included."""
+    from smore_amd import fused
+    rng = np.random.default_rng(k)
+    n = 40
+    table, q1, _, idx, gs = make_problem("l1", n, b, k, dim, rng)
+    table[3] = q1[0]                      # exact ties: entity 3 equals query 0 ...
+    idx[0, :3] = 3                        # ... and they meet
+    t_table, t_q1, t_gs = dev(table), dev(q1), dev(gs)
+    t_idx = torch.tensor(idx, device="cuda")
+    params = fused.score_params(12.0)
+    plan = fused.build_plan(t_idx, n)
+    saved = fused.new_codes("l1", t_table, t_idx, t_q1)
+    assert saved is not None
+    score = fused.score_forward("l1", t_table, t_idx, t_q1, None, params, codes=saved)
+    assert torch.equal(score, fused.score_forward("l1", t_table, t_idx, t_q1, None, params))
+    out = {}
+    for how in ("recompute", "forward"):
+        merged = torch.full((plan.n_uniq, dim), float("nan"), device="cuda")
+        g1, _ = fused.score_backward_fused("l1", plan, t_table, t_idx, t_q1, None, score, t_gs, params, merged=merged,
+                                           sign_codes=False, codes=saved if how == "forward" else None)
+        out[how] = (merged.cpu().numpy(), g1.cpu().numpy())
+    assert np.array_equal(out["forward"][0], out["recompute"][0])
+    assert_close(out["forward"][1], out["recompute"][1], 1e-6, "gq1")
+    g_rows, g_q, _ = orc.score_backward("l1", gs, table[idx], q1[:, None], None, 0.0)
+    uniq, inv = np.unique(idx.reshape(-1), return_inverse=True)
+    want = np.zeros((len(uniq), dim))
+    np.add.at(want, inv, g_rows.reshape(-1, dim))
+    sum_abs = np.zeros((len(uniq), dim))
+    np.add.at(sum_abs, inv, np.abs(g_rows.reshape(-1, dim)))
+    assert_close(out["forward"][0], want, REL_F32, "merged vs oracle", sum_abs=sum_abs)
+    assert_close(out["forward"][1], g_q[:, 0], REL_F32, "gq1 vs oracle")
+
+
+def test_l1_codes_written_by_the_query_gradient_kernel():
+    """More than 4 MiB of L1 queries: without forward codes the one-call backward writes the codes itself
+    for the entity pass; merged rows must equal the recomputing path's bit for bit."""
+    from smore_amd import fused
+    rng = np.random.default_rng(2)
+    n, b, k, dim = 500, 8300, 3, 128
+    table, q1, _, idx, gs = make_problem("l1", n, b, k, dim, rng, zipf=1.1)
+    t_table, t_q1, t_gs = dev(table), dev(q1), dev(gs)
+    t_idx = torch.tensor(idx, device="cuda")
+    params = fused.score_params(12.0)
+    plan = fused.build_plan(t_idx, n)
+    score = fused.score_forward("l1", t_table, t_idx, t_q1, None, params)
+    out = []
+    for codes in (False, True):
+        merged = torch.full((plan.n_uniq, dim), float("nan"), device="cuda")
+        g1, _ = fused.score_backward_fused("l1", plan, t_table, t_idx, t_q1, None, score, t_gs, params, merged=merged,
+                                           sign_codes=codes)
+        out.append((merged.cpu().numpy(), g1.cpu().numpy()))
+    assert np.array_equal(out[0][0], out[1][0])
+    assert_close(out[1][1], out[0][1], 1e-6, "gq1")
