@@ -376,6 +376,9 @@ __global__ __launch_bounds__(NW * 64) void score_backward_query_kernel(ScoreArgs
     // Without optimizer state to fetch, such a pair's row is finished the moment it streams by: its entity
     // row and query are in registers, the merged-gradient row is one more store.
     constexpr bool kInStream = SINGLES == 1 && CODES != 2;
+    // With the forward's codes and no optimizer the merged-gradient row of such a pair is a function of its
+    // code bytes and coefficients alone: it is stored as the codes stream by, and the entity row is never read.
+    constexpr bool kFromCodes = SINGLES == 1 && CODES == 2;
     if constexpr (CODES == 2) {
       // 8 pairs' code bytes requested at a time, two sets used in turn
       constexpr int CB = 8;
@@ -400,6 +403,22 @@ __global__ __launch_bounds__(NW * 64) void score_backward_query_kernel(ScoreArgs
 #pragma unroll
               for (int v = 0; v < VEC; ++v)
                 ModelOps<M>::bwd_q_from_code(c0, c1, c[r][it], VEC - 1 - v, g1[it][v], g2[it][v]);
+            if constexpr (kFromCodes) {
+              if ((singles >> (j0 + r)) & 1ull) {  // wave-uniform
+                RowRegs<MUL, VEC, NIT> none;
+                float ge1[NIT][VEC], ge2[NIT][VEC];
+#pragma unroll
+                for (int it = 0; it < NIT; ++it)
+#pragma unroll
+                  for (int v = 0; v < VEC; ++v) {
+                    none.h[0][it].v[v] = 0.f;
+                    ge1[it][v] = ge2[it][v] = 0.f;
+                    ModelOps<M>::bwd_e_coded(c0, c1, c[r][it], VEC - 1 - v, ge1[it][v]);
+                  }
+                const int seg = __builtin_amdgcn_readlane(my_ps, j0 + r) & 0x7fffffff;
+                finish_row<M, VEC, NIT, REG, false>(A.sink, lane, 0u, seg, ge1, ge2, none, none, none);
+              }
+            }
           }
         }
       };
@@ -462,7 +481,7 @@ __global__ __launch_bounds__(NW * 64) void score_backward_query_kernel(ScoreArgs
     });
     }
 
-    if constexpr (SINGLES != 0 && !kInStream) {
+    if constexpr (SINGLES != 0 && !kInStream && !kFromCodes) {
       // S rows at a time per wavefront (their w, m, v loads are all requested before the first is
       // used): the row sets of the streaming loop are dead here, so this costs no extra registers, and
       // it divides the memory latency each one-pair row would otherwise expose by S.
