@@ -151,17 +151,31 @@ class EmbeddingOptimizer(ABC):
     def score_negatives(self, model, ids, q1, q2=None, gamma=0.0, cen=0.0, regularizer=None):
         """Gather-fused logits [B,K]; q1/q2 are [B,dim] or [B,1,dim] and receive gradients.
         ids [B,K], or [1,K] for negatives shared by all queries of the batch (the --share_negative
-        layout, online_sampler.py:155-157): every query then scores the same K entities."""
+        layout, online_sampler.py:155-157): every query then scores the same K entities.
+        Union queries: q1/q2 of shape [B,U,dim] or [B,U,1,dim] (the merged branch embeddings of
+        kg_reasoning.py:326) give max over the U branches of each branch's logit, as the last line of
+        every custom_cal_logit does (box.py:163, vec.py:89, rotate.py:141, beta.py:307)."""
         table = self.sparse_embed.embedding
         b = q1.shape[0]
+        dim = q1.shape[-1]
+        branches = q1.numel() // (b * dim)
+        if q2 is not None and q2.shape != q1.shape:
+            raise _lib.SmxError("the two query tensors must have the same shape")
         ids = ids.to(table.device)
-        if ids.dim() == 2 and ids.shape[0] == 1 and b > 1:
+        if ids.dim() != 2:
+            raise _lib.SmxError("ids must be [B,K] or [1,K]")
+        if ids.shape[0] == 1 and b > 1:
             ids = ids.expand(b, ids.shape[1])
+        if branches > 1:  # every branch of a query scores that query's negatives
+            ids = ids.repeat_interleave(branches, dim=0)
         ids = ids.contiguous()
-        q1c = q1.reshape(b, -1).contiguous()
-        q2c = None if q2 is None else q2.reshape(b, -1).contiguous()
+        q1c = q1.reshape(b * branches, dim).contiguous()
+        q2c = None if q2 is None else q2.reshape(b * branches, dim).contiguous()
         params = fused.score_params(gamma, cen, regularizer)
-        return _FusedScoreFunc.apply(self, self.dummy_tensor, model, ids, params, q1c, q2c)
+        logit = _FusedScoreFunc.apply(self, self.dummy_tensor, model, ids, params, q1c, q2c)
+        if branches > 1:
+            logit = torch.max(logit.view(b, branches, -1), dim=1)[0]
+        return logit
 
     def check_ids(self):
         """Raises if any lookup since the last check met an id outside the table (synchronises)."""

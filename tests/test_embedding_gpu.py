@@ -166,6 +166,50 @@ def test_shared_negatives_with_mask_match_the_dense_operators():
     assert np.abs(a[4] - r[4]).max() < 2 * lr
 
 
+@pytest.mark.parametrize("model", ["box", "l1", "rotate"])
+def test_union_branches_take_the_max_like_custom_cal_logit(model):
+    """Union queries [B,U,1,D]: logit = max over the U branches (box.py:163); fused scorer against plain
+    lookup + the dense operators' 4-D query form + torch.max.  Only the winning branch gets gradient."""
+    from smore_amd.torchext import ext_ops
+    n, d, b, u, k, lr = 300, 40, 5, 3, 21, 1e-3
+    row = 2 * d if model == "rotate" else d
+    rng = np.random.default_rng(5)
+    neg_n = rng.integers(0, n, (b, k))
+    q1n = rng.uniform(-0.07, 0.07, (b, u, 1, d)).astype(np.float32)
+    q2n = np.abs(rng.uniform(-0.07, 0.07, (b, u, 1, d))).astype(np.float32)
+    gn_n = rng.standard_normal((b, k)).astype(np.float32)
+
+    def run(fused_neg):
+        emb, opt = _setup(n, row, 7)
+        q1 = torch.tensor(q1n, device="cuda", requires_grad=True)
+        q2 = torch.tensor(q2n, device="cuda", requires_grad=True) if model != "l1" else None
+        neg = torch.tensor(neg_n, device="cuda")
+        opt.zero_grad()
+        if fused_neg:
+            ln = opt.score_negatives(model, neg, q1, q2, gamma=24.0, cen=0.02)
+        else:
+            rn = emb(neg.view(-1), "negative_entity").view(b, k, -1)
+            if model == "box":
+                ln = 24 - ext_ops.box_dist_out(rn, q1, q2) - 0.02 * ext_ops.box_dist_in(rn, q1, q2)
+            elif model == "l1":
+                ln = 24 - ext_ops.l1_dist(rn, q1)
+            else:
+                ln = 24 - ext_ops.rotate_dist(rn, q1, q2)
+            assert ln.shape == (b, u, k)
+            ln = torch.max(ln, dim=1)[0]
+        assert ln.shape == (b, k)
+        (ln * torch.tensor(gn_n, device="cuda")).sum().backward()
+        opt.apply_grad(lr)
+        opt.check_ids()
+        grads = [q1.grad.cpu().numpy()] + ([q2.grad.cpu().numpy()] if q2 is not None else [])
+        return [ln.detach().cpu().numpy()] + grads + [emb.state_sum_fo.cpu().numpy()]
+
+    a, r = run(True), run(False)
+    for x, y in zip(a, r):
+        assert_close(x, y, 5 * REL_F32, model)
+    assert np.abs(a[1]).sum() > 0
+
+
 def test_step_counter_and_empty_steps():
     emb, opt = _setup(50, 8, 7)
     opt.zero_grad()
