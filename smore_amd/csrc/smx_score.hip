@@ -42,6 +42,7 @@ size_t code_bytes_per_pair(size_t dim);
 struct SideStream {
   hipStream_t stream = nullptr;
   hipEvent_t fork = nullptr, join = nullptr;
+  std::mutex in_use;  // held while one call records, waits on and re-records the two events
 };
 static SideStream* side_stream() {
   static std::mutex mu;
@@ -243,6 +244,8 @@ int smx_score_backward_fused(int model, void* stream, const smx_plan_view* plan,
     SideStream* side = side_stream();
     if (!side) return fail(SMX_ERR_HIP, "cannot create the side stream");
     hipStream_t st = as_stream(stream);
+    // two host threads on one device share the stream and its events: one fork .. join sequence at a time
+    std::lock_guard<std::mutex> one_call(side->in_use);
     if (hipEventRecord(side->fork, st) != hipSuccess || hipStreamWaitEvent(side->stream, side->fork, 0) != hipSuccess)
       return fail(SMX_ERR_HIP, "fork to the side stream failed");
     int rc = dispatch_model(model, st, A, vec, nit, false);
