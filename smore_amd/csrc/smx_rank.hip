@@ -20,7 +20,7 @@ static int rank_common(RankArgs* R, int* vec, int* nit, int model, const float* 
   if (!table || !q1 || !params || !ans_id || !ans_count || (model_nq(model) == 2 && !q2))
     return fail(SMX_ERR_ARG, "null pointer");
   if (B == 0 || dim == 0 || n_rows == 0 || A == 0) return fail(SMX_ERR_SHAPE, "empty dimension");
-  if (n_rows > 0x100000000ull) return fail(SMX_ERR_SHAPE, "entity count %zu needs ids wider than 32 bits", n_rows);
+  if (n_rows > 0xfffffff8ull) return fail(SMX_ERR_SHAPE, "entity count %zu needs ids wider than 32 bits", n_rows);
   if (A > kRankMaxAnswers) return fail(SMX_ERR_SHAPE, "at most %zu answers per query", kRankMaxAnswers);
   if (B > 0x7fffffffull / (A + 1)) return fail(SMX_ERR_SHAPE, "too many queries");
   if (params->reg_on && model != mBetaKL)

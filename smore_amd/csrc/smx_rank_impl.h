@@ -69,22 +69,26 @@ __device__ __forceinline__ float row_score(const float (&e1)[NIT][VEC], const fl
   return ModelOps<M>::score(wave_sum_last_f32(mine), p);
 }
 
-template <int VEC, int NIT, int MUL>
+// STREAM: the row is read once in a pass over the whole table (non-temporal load).
+template <int VEC, int NIT, int MUL, bool STREAM = false>
 __device__ __forceinline__ void load_entity(const float* __restrict__ row, int dim, int ncol, int lane,
                                             float (&e1)[NIT][VEC], float (&e2)[NIT][VEC]) {
+  typedef float vec4f __attribute__((ext_vector_type(4)));
 #pragma unroll
   for (int it = 0; it < NIT; ++it) {
     const int c = min(lane + 64 * it, ncol - 1);
     if constexpr (VEC == 4) {
-      const float4 a = reinterpret_cast<const float4*>(row)[c];
+      const vec4f* pa = reinterpret_cast<const vec4f*>(row) + c;
+      const vec4f a = STREAM ? __builtin_nontemporal_load(pa) : *pa;
       e1[it][0] = a.x; e1[it][1] = a.y; e1[it][2] = a.z; e1[it][3] = a.w;
       if (MUL == 2) {
-        const float4 b = reinterpret_cast<const float4*>(row + dim)[c];
+        const vec4f* pb = reinterpret_cast<const vec4f*>(row + dim) + c;
+        const vec4f b = STREAM ? __builtin_nontemporal_load(pb) : *pb;
         e2[it][0] = b.x; e2[it][1] = b.y; e2[it][2] = b.z; e2[it][3] = b.w;
       }
     } else {
-      e1[it][0] = row[c];
-      if (MUL == 2) e2[it][0] = row[dim + c];
+      e1[it][0] = STREAM ? __builtin_nontemporal_load(row + c) : row[c];
+      if (MUL == 2) e2[it][0] = STREAM ? __builtin_nontemporal_load(row + dim + c) : row[dim + c];
     }
   }
 }
@@ -157,59 +161,80 @@ __global__ __launch_bounds__(256) void rank_scan_kernel(RankArgs A) {
     load_rank_query<M, VEC, NIT>(A.q1, A.q2, qb[x], dim, A.ncol, lane, q[x]);
   }
   const int chunks = (A.A + 63) / 64;
-  // the first 64 answers' keys stay in registers (most queries have no more); further chunks come from LDS
-  unsigned long long first_keys[NB];
+  // The first 64 answers' keys stay in registers (most queries have no more); further chunks come from LDS.
+  // live[x]: lanes that hold one of them.  my_id[x]: that answer's entity id.
+  unsigned long long first_keys[NB], live[NB];
+  unsigned my_id[NB];
+  // tally[x], lane L: rows so far that beat exactly L of query x's answers (the common cases: L = 0 is
+  // every entity ranked below all answers).  Rows that beat 64 or more go to the LDS histogram directly.
+  unsigned tally[NB];
 #pragma unroll
-  for (int x = 0; x < NB; ++x) first_keys[x] = lane < count[x] ? lds_keys[x * A.A + lane] : 0ull;
+  for (int x = 0; x < NB; ++x) {
+    first_keys[x] = lane < count[x] ? lds_keys[x * A.A + lane] : 0ull;
+    live[x] = count[x] >= 64 ? ~0ull : ((1ull << count[x]) - 1ull);
+    my_id[x] = (unsigned)~(unsigned)first_keys[x];
+    tally[x] = 0u;
+  }
 
-  // wavefronts walk the table together: group g of RIF consecutive rows belongs to wavefront g mod n_waves
-  const unsigned long long n_waves = (unsigned long long)gridDim.x * 4ull;
-  const unsigned long long wid = (unsigned long long)blockIdx.x * 4ull + wave;
-  const unsigned long long groups = (A.n_rows + RIF - 1) / RIF;
+  // Wavefronts walk the table together: group g of RIF consecutive rows belongs to wavefront g mod n_waves.
+  // Group and row numbers are 32-bit scalars (the host refuses tables of 2^32 - 8 rows or more).  Requests
+  // are unconditional -- past the end they repeat the last group -- and rows past the end are scored and
+  // then dropped, so that no branch separates a request from the use of the rows requested before it:
+  // the counters the compiler waits on then leave the newest RIF loads in flight.
+  const unsigned n_waves = gridDim.x * 4u;
+  const unsigned wid = blockIdx.x * 4u + (unsigned)wave;
+  const unsigned n_rows32 = (unsigned)A.n_rows;
+  const unsigned groups = (n_rows32 + RIF - 1) / RIF;
   float ea1[RIF][NIT][VEC], ea2[RIF][NIT][VEC], eb1[RIF][NIT][VEC], eb2[RIF][NIT][VEC];
-  auto request = [&](float (&x1)[RIF][NIT][VEC], float (&x2)[RIF][NIT][VEC], unsigned long long g) {
+  auto request = [&](float (&x1)[RIF][NIT][VEC], float (&x2)[RIF][NIT][VEC], unsigned g) {
+    g = min(g, groups - 1);
 #pragma unroll
     for (int r = 0; r < RIF; ++r) {
-      unsigned long long row = g * RIF + r;
-      if (row >= A.n_rows) row = A.n_rows - 1;
-      load_entity<VEC, NIT, MUL>(A.table + row * row_len, dim, A.ncol, lane, x1[r], x2[r]);
+      const unsigned row = min(g * RIF + r, n_rows32 - 1);
+      load_entity<VEC, NIT, MUL, true>(A.table + row * row_len, dim, A.ncol, lane, x1[r], x2[r]);
     }
   };
-  auto consume = [&](const float (&x1)[RIF][NIT][VEC], const float (&x2)[RIF][NIT][VEC], unsigned long long g) {
+  auto consume = [&](const float (&x1)[RIF][NIT][VEC], const float (&x2)[RIF][NIT][VEC], unsigned g) {
 #pragma unroll
     for (int r = 0; r < RIF; ++r) {
-      const unsigned long long row = g * RIF + r;
-      if (row < A.n_rows) {  // wave-uniform
+      const unsigned id = g * RIF + r;  // entity id of the row
 #pragma unroll
-        for (int x = 0; x < NB; ++x) {
-          const float s = row_score<M, VEC, NIT, REG>(x1[r], x2[r], q[x], A.ncol, lane, A.p);
-          const float su = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(s), 63));
-          const unsigned long long key = rank_key(su, row);
-          int not_beaten = __popcll(__ballot(lane < count[x] && !(key > first_keys[x])));
-          bool is_answer = __ballot(lane < count[x] && ((unsigned)~(unsigned)first_keys[x] == (unsigned)row)) != 0ull;
-          for (int c = 1; c < chunks; ++c) {
-            const int j = c * 64 + lane;
-            const bool live = j < count[x];
-            const unsigned long long ak = live ? lds_keys[x * A.A + j] : 0ull;
-            not_beaten += __popcll(__ballot(live && !(key > ak)));
-            is_answer |= __ballot(live && ((unsigned)~(unsigned)ak == (unsigned)row)) != 0ull;
-          }
-          if (!is_answer && lane == 0) atomicAdd(&lds_bins[x * A1 + not_beaten], 1u);
+      for (int x = 0; x < NB; ++x) {
+        const float s = row_score<M, VEC, NIT, REG>(x1[r], x2[r], q[x], A.ncol, lane, A.p);
+        const float su = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(s), 63));
+        const unsigned long long key = rank_key(su, id);
+        int not_beaten = __popcll(__ballot(!(key > first_keys[x])) & live[x]);
+        bool skip = id >= n_rows32 || (__ballot(my_id[x] == id) & live[x]) != 0ull;  // past the end, or an answer
+        for (int c = 1; c < chunks; ++c) {
+          const int j = c * 64 + lane;
+          const bool in_list = j < count[x];
+          const unsigned long long ak = in_list ? lds_keys[x * A.A + j] : 0ull;
+          not_beaten += __popcll(__ballot(in_list && !(key > ak)));
+          skip |= __ballot(in_list && ((unsigned)~(unsigned)ak == id)) != 0ull;
         }
+        const int beaten = skip ? -1 : count[x] - not_beaten;  // wave-uniform; -1 matches no lane
+        tally[x] += lane == beaten ? 1u : 0u;
+        if (beaten >= 64 && lane == 0) atomicAdd(&lds_bins[x * A1 + not_beaten], 1u);
       }
     }
   };
-  unsigned long long g = wid;
-  if (g < groups) request(ea1, ea2, g);
-  while (g < groups) {
-    const unsigned long long g1 = g + n_waves, g2 = g + 2 * n_waves;
-    if (g1 < groups) request(eb1, eb2, g1);
-    consume(ea1, ea2, g);
-    if (g1 >= groups) break;
-    if (g2 < groups) request(ea1, ea2, g2);
-    consume(eb1, eb2, g1);
-    g = g2;
+  if (wid < groups) {
+    unsigned g = wid;
+    request(ea1, ea2, g);
+    while (true) {
+      // (group numbers stay below 2^30 + 2 * n_waves: no wrap-around)
+      request(eb1, eb2, g + n_waves);
+      consume(ea1, ea2, g);
+      if (g + n_waves >= groups) break;
+      request(ea1, ea2, g + 2 * n_waves);
+      consume(eb1, eb2, g + n_waves);
+      if (g + 2 * n_waves >= groups) break;
+      g += 2 * n_waves;
+    }
   }
+#pragma unroll
+  for (int x = 0; x < NB; ++x)
+    if (lane <= count[x] && tally[x] != 0u) atomicAdd(&lds_bins[x * A1 + (count[x] - lane)], tally[x]);
   __syncthreads();
 #pragma unroll
   for (int x = 0; x < NB; ++x) {

@@ -179,15 +179,21 @@ template <int MUL, int VEC, int NIT, int RIF> struct RowSet {
 template <int MUL, int VEC, int NIT, int RIF>
 __device__ __forceinline__ void request_rows(RowSet<MUL, VEC, NIT, RIF>& rs, const unsigned* slab, int g0, int dim,
                                              int ncol, int lane) {
+  GlobalRow pe[RIF];
+#pragma unroll
+  for (int r = 0; r < RIF; ++r) pe[r] = slab_row(slab, g0 + r);
 #pragma unroll
   for (int r = 0; r < RIF; ++r) {
-    const GlobalRow pe = slab_row(slab, g0 + r);
 #pragma unroll
     for (int it = 0; it < NIT; ++it) {
       const int c = min(lane + 64 * it, ncol - 1);
-      rs.e1[r][it] = load_pack<VEC>(pe, c);
-      if (MUL == 2) rs.e2[r][it] = load_pack<VEC>(pe + dim, c);
+      rs.e1[r][it] = load_pack<VEC>(pe[r], c);
+      if (MUL == 2) rs.e2[r][it] = load_pack<VEC>(pe[r] + dim, c);
     }
+    // Rows are used in the order r = 0, 1, ..: their loads must be issued in that order everywhere (the
+    // scheduler is otherwise free to reverse them in the loop prologue), or the wait for row 0 at the top
+    // of the streaming loop becomes a wait for every load in flight.
+    __builtin_amdgcn_sched_barrier(0);
   }
 }
 
