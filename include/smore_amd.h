@@ -261,7 +261,7 @@ int smx_sample_loss(void* stream, const float* pos, const float* neg, const floa
  * Filtered ranks of a query's answers among all n_rows entities (the test_all branch of
  * smore/training/train_process.py:112-160: logits of every entity, argsort, ranks of easy + hard
  * answers, minus the answers ranked before) without materialising or sorting the logit row: the
- * table is streamed once per two queries and every non-answer entity is counted against the answers
+ * table is streamed once per one, two or four queries (as many as the row length allows) and every non-answer entity is counted against the answers
  * it ranks before.  Equal scores: the lower entity id ranks first.
  *   ans_id [B, A] int64, ans_count [B] int32: ans_count[b] <= A valid answers (easy and hard alike) per query.
  * smx_rank_answer_keys: ans_score [B, A] = the answers' logits, ans_key [B, A] = their order keys

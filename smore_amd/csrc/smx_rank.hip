@@ -9,7 +9,7 @@ extern template int rank_dispatch<mBox>(hipStream_t, const RankArgs&, int, int, 
 extern template int rank_dispatch<mRotate>(hipStream_t, const RankArgs&, int, int, bool);
 extern template int rank_dispatch<mBetaKL>(hipStream_t, const RankArgs&, int, int, bool);
 
-constexpr size_t kRankMaxAnswers = 2048;  // per query; bins and keys of a pass live in LDS (2 x 2049 x 4 + 2 x 2048 x 8 bytes)
+constexpr size_t kRankMaxAnswers = 2048;  // per query; bins and keys of a pass live in LDS (per query of the pass 2049 x 4 + 2048 x 8 bytes)
 
 static size_t rank_ws_bytes(size_t B, size_t A) { return (B * (A + 1) * sizeof(unsigned) + 255) & ~(size_t)255; }
 

@@ -18,13 +18,13 @@
 
 namespace smx {
 
-constexpr int kRankQueries = 2;  // queries scored per pass over the table
+constexpr int kRankQueries = 4;  // most queries scored per pass over the table (short rows; 2 for long ones)
 
 struct RankArgs {
   const float* table;
   const float* q1;
   const float* q2;
-  int b0, B;            // queries [b0, b0 + kRankQueries) of B are handled by this launch
+  int b0, B;            // queries [b0, b0 + NB) of B are handled by this launch (NB: see rank_scan_kernel)
   int ncol;
   unsigned long long n_rows;
   ScoreParams p;
@@ -132,7 +132,7 @@ __global__ __launch_bounds__(256) void rank_answer_keys_kernel(RankArgs A) {
   }
 }
 
-// The scan for NB (1 or 2) queries.  LDS: bins [NB][A + 1], keys [NB][A].
+// The scan for NB (1, 2 or 4) queries.  LDS: bins [NB][A + 1], keys [NB][A].
 template <int M, int VEC, int NIT, bool REG, int NB>
 __global__ __launch_bounds__(256) void rank_scan_kernel(RankArgs A) {
   constexpr int MUL = model_mul(M);
@@ -288,16 +288,30 @@ int launch_rank_reg(hipStream_t st, RankArgs A, bool keys_only) {
     if (want < blocks) blocks = (unsigned)(want ? want : 1);
     return blocks;
   };
-  for (int b0 = 0; b0 < A.B; b0 += kRankQueries) {
+  // Queries per pass: the row is fetched once for all of them, and the kernel turns from bandwidth-bound
+  // to issue-bound between one and two.  Four when the rows are short enough for four queries' registers
+  // and the answers' keys and histograms of four queries fit 48 KB of LDS.
+  constexpr bool kFourFit = NIT * model_mul(M) <= 2;
+  for (int b0 = 0; b0 < A.B;) {
     A.b0 = b0;
-    if (A.B - b0 >= 2) {
+    const int left = A.B - b0;
+    if (kFourFit && left >= 4 && lds_bytes(4) <= (size_t)48 << 10) {
+      if constexpr (kFourFit) {
+        const size_t lds = lds_bytes(4);
+        hipLaunchKernelGGL((rank_scan_kernel<M, VEC, NIT, REG, 4>),
+                           dim3(grid_for(rank_scan_kernel<M, VEC, NIT, REG, 4>, lds)), dim3(256), lds, st, A);
+      }
+      b0 += 4;
+    } else if (left >= 2) {
       const size_t lds = lds_bytes(2);
       hipLaunchKernelGGL((rank_scan_kernel<M, VEC, NIT, REG, 2>), dim3(grid_for(rank_scan_kernel<M, VEC, NIT, REG, 2>, lds)),
                          dim3(256), lds, st, A);
+      b0 += 2;
     } else {
       const size_t lds = lds_bytes(1);
       hipLaunchKernelGGL((rank_scan_kernel<M, VEC, NIT, REG, 1>), dim3(grid_for(rank_scan_kernel<M, VEC, NIT, REG, 1>, lds)),
                          dim3(256), lds, st, A);
+      b0 += 1;
     }
   }
   hipLaunchKernelGGL(rank_finish_kernel, dim3((unsigned)A.B), dim3(256), 0, st, A);

@@ -22,11 +22,12 @@ def test_integer_valued_l1_ranks_are_exact_ties_included():
     from smore_amd import fused
     from smore_amd.evaluation import filtered_ranks
     rng = np.random.default_rng(0)
-    n, d, b = 5000, 16, 3
+    n, d, b = 5000, 16, 7   # passes of four, two and one queries
     table = rng.integers(-3, 4, (n, d)).astype(np.float64)
     q1 = rng.integers(-3, 4, (b, d)).astype(np.float64)
-    easy = [[3, 77, 4000], [], [11]]
-    hard = [[9, 2500, 4999, 0], [123], list(range(100, 180))]      # 80 answers: two compare chunks
+    easy = [[3, 77, 4000], [], [11], [5], [], [1, 2, 3], [4998]]
+    hard = [[9, 2500, 4999, 0], [123], list(range(100, 180)),       # 80 answers: two compare chunks
+            list(range(200, 270)), [42], [4999], [0, 17]]
     params = fused.score_params(GAMMA["l1"], 0.0)
     got = filtered_ranks("l1", dev(table), dev(q1), None, params, easy, hard)
     scores = _scores64("l1", table, q1, None, 0.0)
