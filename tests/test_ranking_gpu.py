@@ -92,6 +92,23 @@ def test_planted_best_entity_and_duplicates_of_it():
     assert got[0][0].tolist() == [1, 1] and got[0][1].tolist() == [1]  # filtered: answers do not count
 
 
+@pytest.mark.parametrize("n", [1, 2, 3, 5, 9])
+def test_tables_shorter_than_one_request_group(n):
+    """Fewer rows than a wavefront requests at a time: the repeated last rows must not be counted."""
+    from smore_amd import fused
+    from smore_amd.evaluation import filtered_ranks
+    rng = np.random.default_rng(n)
+    d = 12
+    table = rng.integers(-3, 4, (n, d)).astype(np.float64)
+    q1 = rng.integers(-3, 4, (2, d)).astype(np.float64)
+    hard = [[n - 1], [0]]
+    got = filtered_ranks("l1", dev(table), dev(q1), None, fused.score_params(GAMMA["l1"], 0.0), [[], []], hard)
+    scores = _scores64("l1", table, q1, None, 0.0)
+    for i in range(2):
+        want_h, _ = orc.filtered_ranks(scores[i], [], hard[i])
+        assert got[i][0].cpu().numpy().tolist() == want_h.tolist()
+
+
 def test_ranking_argument_errors():
     from smore_amd import _lib, fused
     from smore_amd.evaluation import filtered_ranks
