@@ -91,7 +91,7 @@ def make_inputs(cfg, device, seed):
 
 
 def algorithmic_bytes(cfg, n_uniq, streaming=False):
-    """Compulsory-traffic model of one step (BASELINE.md section 2): every distinct touched row crosses
+    """Compulsory-traffic model of one step: every distinct touched row crosses
     HBM once forward and once backward; Adam reads and writes w, m, v of every touched row; ids, scores
     and upstream gradients once; query tensors read twice and their gradients written once."""
     p = cfg["b"] * cfg["k"]
