@@ -199,7 +199,11 @@ typedef struct smx_opt_params {
  * Replaces dist_backward_ent_kernel (common_kernel.h:59-89), EmbedLookupFunc.backward
  * (embed_optimizer.py:63-66), merge_grad_list (:45-48) and update_step (:208-252).
  * workspace: smx_entity_workspace_bytes(P, dim*mul) bytes, 256-byte aligned.
- * fwd_codes (may be NULL): the forward's sign codes; they replace the reads of the query rows. */
+ * fwd_codes (may be NULL): the forward's sign codes; they replace the reads of the query rows.
+ * With them, an optimizer, no merged output and a step of a million pairs or more whose queries
+ * exceed one L2, the call finishes ids that occur once in a pair-ordered kernel on `stream` and
+ * reduces the others on the library's second stream beside it (joined to `stream` before return);
+ * the rows get the same bits either way. */
 size_t smx_entity_workspace_bytes(size_t n_pairs, size_t row_len);
 int smx_score_backward_entity(int model, void* stream, const smx_plan_view* plan, float* table,
                               size_t n_rows, const float* q1, const float* q2, const float* score,

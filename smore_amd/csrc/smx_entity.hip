@@ -128,28 +128,6 @@ size_t smx_fused_workspace_bytes(int model, size_t n_pairs, size_t dim) {
   return total;
 }
 
-int smx_score_backward_entity(int model, void* stream, const smx_plan_view* plan, float* table, size_t n_rows,
-                              const float* q1, const float* q2, const float* score, const float* gscore, size_t B,
-                              size_t K, size_t dim, const smx_score_params* params, float* merged, float* m, float* v,
-                              const smx_opt_params* adam, void* workspace, size_t workspace_bytes,
-                              const void* fwd_codes, size_t fwd_codes_bytes) {
-  using namespace smx;
-  int codes_vec = 0, codes_nit = 0;
-  if (fwd_codes) {
-    // the layout smx_score_codes_bytes promises; entity_backward refuses the call if its own column
-    // layout (alignment of merged / m / v included) turns out different
-    if (model < 0 || model >= mNumModels || !model_coded(model)) return fail(SMX_ERR_ARG, "this model has no sign codes");
-    if (fwd_codes_bytes != B * K * code_bytes_per_pair(dim) || code_bytes_per_pair(dim) > 2 * 64)
-      return fail(SMX_ERR_ARG, "codes buffer is not smx_score_codes_bytes() long");
-    if (reinterpret_cast<uintptr_t>(fwd_codes) & 15u) return fail(SMX_ERR_ARG, "codes must be 16-byte aligned");
-    codes_vec = dim % 4 == 0 ? 4 : 1;
-    codes_nit = (int)(code_bytes_per_pair(dim) / 64);
-  }
-  return entity_backward(model, stream, plan, table, n_rows, q1, q2, score, gscore, B, K, dim, params, merged, m, v,
-                         adam, workspace, workspace_bytes, 0, static_cast<const unsigned char*>(fwd_codes), codes_vec,
-                         codes_nit);
-}
-
 }  // extern "C"
 
 namespace smx {

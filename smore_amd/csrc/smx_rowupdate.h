@@ -188,7 +188,10 @@ __device__ __forceinline__ void finish_row(const RowSink& A, int lane, unsigned 
       for (int it = 0; it < NIT; ++it)
         if (lane + 64 * it < A.ncol) {
 #pragma unroll
-          for (int x = 0; x < VEC; ++x) part += g1[it][x] * g1[it][x] + (MUL == 2 ? g2[it][x] * g2[it][x] : 0.f);
+          for (int x = 0; x < VEC; ++x) {
+            part = __builtin_fmaf(g1[it][x], g1[it][x], part);
+            if (MUL == 2) part = __builtin_fmaf(g2[it][x], g2[it][x], part);
+          }
         }
       g2_row = wave_sum_f32(part) / (float)row_len;
       v_row = A.v[row_id];
@@ -206,17 +209,21 @@ __device__ __forceinline__ void finish_row(const RowSink& A, int lane, unsigned 
             const float g = h == 0 ? g1[it][x] : g2[it][x];
             const float gg = A.squeeze ? g2_row : g * g;
             const float v_old = A.squeeze ? v_row : v0.h[h][it].v[x];
+            // Every multiply-add is written as the fused operation it is meant to be: left to the
+            // compiler's contraction, the kernels that share this function round a*b + c*d differently
+            // from one another, and the same row would get different bits depending on which one finishes it.
             if (kind == kOptAdam) {
-              mn[x] = m0.h[h][it].v[x] * A.a.beta1 + g * A.a.omb1;
-              vn[x] = v_old * A.a.beta2 + gg * A.a.omb2;
-              wn[x] = w.h[h][it].v[x] + A.a.step_size * mn[x] * hw_rcp(hw_sqrt(vn[x]) * A.a.inv_sqrt_bc2 + A.a.eps);
+              mn[x] = __builtin_fmaf(m0.h[h][it].v[x], A.a.beta1, g * A.a.omb1);
+              vn[x] = __builtin_fmaf(v_old, A.a.beta2, gg * A.a.omb2);
+              const float denom = __builtin_fmaf(hw_sqrt(vn[x]), A.a.inv_sqrt_bc2, A.a.eps);
+              wn[x] = __builtin_fmaf(A.a.step_size * mn[x], hw_rcp(denom), w.h[h][it].v[x]);
             } else if (kind == kOptSgd) {
               mn[x] = vn[x] = 0.f;
-              wn[x] = w.h[h][it].v[x] + A.a.step_size * g;
+              wn[x] = __builtin_fmaf(A.a.step_size, g, w.h[h][it].v[x]);
             } else {
               mn[x] = 0.f;
-              vn[x] = kind == kOptAdagrad ? v_old + gg : v_old * A.a.beta2 + gg * A.a.omb2;
-              wn[x] = w.h[h][it].v[x] + A.a.step_size * g * hw_rcp(hw_sqrt(vn[x]) + A.a.eps);
+              vn[x] = kind == kOptAdagrad ? v_old + gg : __builtin_fmaf(v_old, A.a.beta2, gg * A.a.omb2);
+              wn[x] = __builtin_fmaf(A.a.step_size * g, hw_rcp(hw_sqrt(vn[x]) + A.a.eps), w.h[h][it].v[x]);
             }
             v_new_row = vn[x];
           }

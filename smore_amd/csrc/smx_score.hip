@@ -87,6 +87,26 @@ static int dispatch_model(int model, hipStream_t st, const ScoreArgs& A, int vec
   return fail(SMX_ERR_KIND, "unknown score model %d", model);
 }
 
+// Where the rows finished by the query-gradient kernel go: table / optimizer state and/or merged rows.
+static void fill_sink(ScoreArgs* A, float* table, float* m, float* v, float* merged, const smx_opt_params* adam) {
+  A->sink.table = table;
+  A->sink.m = m;
+  A->sink.v = v;
+  A->sink.merged = merged;
+  A->sink.adam_on = adam ? adam->kind : 0;
+  A->sink.squeeze = (adam && adam->squeeze) ? 1 : 0;
+  if (adam) A->sink.a = make_adam_consts(adam);
+  A->sink.p = A->p;
+  A->sink.ncol = A->ncol;
+}
+
+// The step's query tensors do not fit one XCD's 4 MiB L2: the entity pass would fetch a one-pair
+// segment's query rows from beyond it (measured: finishing such segments in the pair-ordered kernel is
+// faster for 4096 queries x 2 x 200 floats, slower for 1024 queries x 2 x 400 or 500).
+static bool queries_beyond_l2(int model, size_t B, size_t dim) {
+  return B * dim * model_nq(model) * sizeof(float) > ((size_t)4 << 20);
+}
+
 // Common argument checks; fills the shape fields of A and picks the column width: float4 columns when
 // rows are 16-byte aligned, single floats otherwise.
 static int fill_args(ScoreArgs* A, int* vec, int* nit, int model, const float* table, size_t n_rows,
@@ -170,6 +190,64 @@ int smx_score_backward_query(int model, void* stream, const float* table, size_t
   return dispatch_model(model, as_stream(stream), A, vec, nit, false);
 }
 
+int smx_score_backward_entity(int model, void* stream, const smx_plan_view* plan, float* table, size_t n_rows,
+                              const float* q1, const float* q2, const float* score, const float* gscore, size_t B,
+                              size_t K, size_t dim, const smx_score_params* params, float* merged, float* m, float* v,
+                              const smx_opt_params* adam, void* workspace, size_t workspace_bytes,
+                              const void* fwd_codes, size_t fwd_codes_bytes) {
+  using namespace smx;
+  int codes_vec = 0, codes_nit = 0;
+  if (fwd_codes) {
+    // the layout smx_score_codes_bytes promises; entity_backward refuses the call if its own column
+    // layout (alignment of merged / m / v included) turns out different
+    if (model < 0 || model >= mNumModels || !model_coded(model)) return fail(SMX_ERR_ARG, "this model has no sign codes");
+    if (fwd_codes_bytes != B * K * code_bytes_per_pair(dim) || code_bytes_per_pair(dim) > 2 * 64)
+      return fail(SMX_ERR_ARG, "codes buffer is not smx_score_codes_bytes() long");
+    if (reinterpret_cast<uintptr_t>(fwd_codes) & 15u) return fail(SMX_ERR_ARG, "codes must be 16-byte aligned");
+    codes_vec = dim % 4 == 0 ? 4 : 1;
+    codes_nit = (int)(code_bytes_per_pair(dim) / 64);
+  }
+  const unsigned char* codes = static_cast<const unsigned char*>(fwd_codes);
+  // Large steps with the forward's codes and an optimizer: the one-pair segments (most of the touched
+  // rows of a skewed or sparse id stream) go through the pair-ordered kernel on the caller's stream while
+  // the entity pass reduces the others on the library's second stream -- the same division of work and
+  // the same arithmetic per row as in smx_score_backward_fused, minus the query gradient.
+  const bool split = fwd_codes && adam && !merged && plan && plan->pair_seg && plan->uniq && score && gscore &&
+                     queries_beyond_l2(model, B, dim) && B * K >= ((size_t)1 << 20) && plan->n_pairs == B * K &&
+                     workspace && workspace_bytes >= entity_ws_bytes(B * K, dim * model_mul(model)) &&
+                     !std::getenv("SMX_SERIAL_BACKWARD");
+  if (split) {
+    ScoreArgs A;
+    int vec, nit;
+    if (const char* msg = check_opt_params(adam, m, v)) return fail(SMX_ERR_ARG, "%s", msg);
+    if (int rc = fill_args(&A, &vec, &nit, model, table, n_rows, nullptr, q1, q2, B, K, dim, params, nullptr, m)) return rc;
+    const bool v_ok = !(vec == 4 && v && !adam->squeeze && !aligned16(v));
+    if (vec == codes_vec && nit == codes_nit && v_ok) {
+      A.n_rows = n_rows;
+      A.score = score;
+      A.gscore = gscore;
+      A.pair_seg = plan->pair_seg;
+      A.uniq = reinterpret_cast<const long long*>(plan->uniq);
+      fill_sink(&A, table, m, v, nullptr, adam);
+      SideStream* side = side_stream();
+      if (!side) return fail(SMX_ERR_HIP, "cannot create the side stream");
+      hipStream_t st = as_stream(stream);
+      std::lock_guard<std::mutex> one_call(side->in_use);
+      if (hipEventRecord(side->fork, st) != hipSuccess || hipStreamWaitEvent(side->stream, side->fork, 0) != hipSuccess)
+        return fail(SMX_ERR_HIP, "fork to the side stream failed");
+      int rc = dispatch_model(model, st, A, vec, nit, false);  // gq1 == null: one-pair segments only
+      if (rc == SMX_OK)
+        rc = entity_backward(model, side->stream, plan, table, n_rows, q1, q2, score, gscore, B, K, dim, params, nullptr,
+                             m, v, adam, workspace, workspace_bytes, 1, codes, codes_vec, codes_nit);
+      if (hipEventRecord(side->join, side->stream) != hipSuccess || hipStreamWaitEvent(st, side->join, 0) != hipSuccess)
+        return fail(SMX_ERR_HIP, "join with the side stream failed");
+      return rc;
+    }
+  }
+  return entity_backward(model, stream, plan, table, n_rows, q1, q2, score, gscore, B, K, dim, params, merged, m, v,
+                         adam, workspace, workspace_bytes, 0, codes, codes_vec, codes_nit);
+}
+
 int smx_score_backward_fused(int model, void* stream, const smx_plan_view* plan, float* table, size_t n_rows,
                              const int64_t* idx, const float* q1, const float* q2, const float* score,
                              const float* gscore, float* gq1, float* gq2, size_t B, size_t K, size_t dim,
@@ -201,18 +279,10 @@ int smx_score_backward_fused(int model, void* stream, const smx_plan_view* plan,
   // queries x 2 x 400 or 500).  Otherwise every segment goes through the entity pass.
   // Without an optimizer the one-pair rows cost the query-gradient kernel one store each (nothing to
   // fetch), so they are always finished there.
-  const bool q_beyond_l2 = (size_t)B * dim * model_nq(model) * sizeof(float) > ((size_t)4 << 20);
+  const bool q_beyond_l2 = queries_beyond_l2(model, B, dim);
   const bool singles_here = !adam || q_beyond_l2;
   A.pair_seg = singles_here ? plan->pair_seg : nullptr;
-  A.sink.table = table;
-  A.sink.m = m;
-  A.sink.v = v;
-  A.sink.merged = merged;
-  A.sink.adam_on = adam ? adam->kind : 0;
-  A.sink.squeeze = (adam && adam->squeeze) ? 1 : 0;
-  if (adam) A.sink.a = make_adam_consts(adam);
-  A.sink.p = A.p;
-  A.sink.ncol = A.ncol;
+  fill_sink(&A, table, m, v, merged, adam);
   // Sign codes (models that have them): when the entity pass would fetch query rows from beyond the L2,
   // the query-gradient kernel leaves each pair's derivative decisions in the workspace behind the
   // entity pass's own scratch, and the entity pass reads those instead of the query rows.  Used when

@@ -39,6 +39,7 @@ struct ScoreArgs {
   ScoreParams p;
   int* err;
   const int* pair_seg;   // one-pair segments finished by the query backward (SINGLES kernels)
+  const long long* uniq; // plan's id list: row of a one-pair segment when the kernel runs without the id tensor (GQ = false)
   unsigned char* codes;  // [B*K][NIT*64] sign codes written by this kernel (forward or query backward), or null
   const unsigned char* codes_in;  // query backward: codes the forward left; the entity rows are then not read
   RowSink sink;
@@ -325,8 +326,13 @@ __global__ __launch_bounds__(256) void score_forward_kernel(ScoreArgs A, int til
 // and column group, for the entity pass to use in place of the query rows; 2 = the forward pass left
 // the codes: the query gradient is summed from them and the entity rows are not read at all (except
 // those of the one-pair segments finished here).
-template <int M, int VEC, int NIT, int RIF, int NW, bool REG, int SINGLES, int CODES = 0>
+// GQ = false: only the one-pair segments are finished (optimizer on w, m, v); no query gradient, no
+// other pair is touched.  The pairs' rows then come from the plan (uniq[segment]), not from the id tensor:
+// this is the half of the work that smx_score_backward_entity hands to this kernel when the query
+// gradients were taken earlier (autograd's backward) and the update comes later (apply_grad).
+template <int M, int VEC, int NIT, int RIF, int NW, bool REG, int SINGLES, int CODES = 0, bool GQ = true>
 __global__ __launch_bounds__(NW * 64) void score_backward_query_kernel(ScoreArgs A) {
+  static_assert(GQ || (SINGLES == 2 && CODES == 0), "the one-pair-only form exists with an optimizer");
   const float* __restrict__ table = A.table;
   const long long* __restrict__ idx = A.idx;
   const float* __restrict__ q1 = A.q1;
@@ -369,23 +375,33 @@ __global__ __launch_bounds__(NW * 64) void score_backward_query_kernel(ScoreArgs
   for (int kb = kw0; kb < kw1; kb += 64) {
     const int cnt = min(64, kw1 - kb);
     const size_t first = (size_t)b * K + kb;
-    const PairBatch pb = load_pair_batch(idx, first, cnt, lane, row_len, n_rows, bad);
     const size_t mine = first + min(lane, cnt - 1);
-    float my_c0, my_c1;
-    ModelOps<M>::coef(gscore[mine], score[mine], p, my_c0, my_c1);
     int my_ps = 0;
     unsigned long long singles = 0ull;  // pairs of the batch that are a segment of their own
     if constexpr (SINGLES != 0) {
       my_ps = A.pair_seg[mine];
       singles = __ballot(lane < cnt && my_ps < 0);
     }
+    PairBatch pb;
+    if constexpr (GQ) {
+      pb = load_pair_batch(idx, first, cnt, lane, row_len, n_rows, bad);
+    } else {
+      if (singles == 0ull) continue;  // wave-uniform
+      const unsigned long long row = my_ps < 0 ? (unsigned long long)A.uniq[my_ps & 0x7fffffff] : 0ull;
+      const unsigned long long off = row * row_len;
+      pb = PairBatch{(unsigned)off, (unsigned)(off >> 32), (unsigned)row};
+    }
+    float my_c0, my_c1;
+    ModelOps<M>::coef(gscore[mine], score[mine], p, my_c0, my_c1);
     // Without optimizer state to fetch, such a pair's row is finished the moment it streams by: its entity
     // row and query are in registers, the merged-gradient row is one more store.
     constexpr bool kInStream = SINGLES == 1 && CODES != 2;
     // With the forward's codes and no optimizer the merged-gradient row of such a pair is a function of its
     // code bytes and coefficients alone: it is stored as the codes stream by, and the entity row is never read.
     constexpr bool kFromCodes = SINGLES == 1 && CODES == 2;
-    if constexpr (CODES == 2) {
+    if constexpr (!GQ) {
+      // nothing streams: only the rows of the one-pair segments below
+    } else if constexpr (CODES == 2) {
       // 8 pairs' code bytes requested at a time, two sets used in turn
       constexpr int CB = 8;
       const unsigned char* pc = A.codes_in + first * (size_t)(NIT * 64) + lane;
@@ -536,6 +552,7 @@ __global__ __launch_bounds__(NW * 64) void score_backward_query_kernel(ScoreArgs
     }
   }
 
+  if constexpr (!GQ) return;
 #pragma unroll
   for (int it = 0; it < NIT; ++it)
 #pragma unroll
@@ -597,6 +614,16 @@ template <int M, int VEC, int NIT, int NW, bool REG>
 int launch_backward_query_reg(hipStream_t st, const ScoreArgs& A) {
   constexpr int RIF = rows_in_flight(NIT, model_mul(M));
   const size_t lds = ((size_t)(NW + 1) * model_nq(M) * A.ncol * VEC + NW * kSlabDwords) * sizeof(float);
+  if (!A.gq1) {  // one-pair segments only; built for the shapes that have sign codes
+    if constexpr (model_coded(M) && !REG && NW == 8 && NIT <= 2) {
+      if (A.pair_seg && A.uniq && A.sink.adam_on) {
+        hipLaunchKernelGGL((score_backward_query_kernel<M, VEC, NIT, RIF, NW, REG, 2, 0, false>), dim3((unsigned)A.B),
+                           dim3(NW * 64), lds, st, A);
+        return check_launch("score backward (one-pair segments)");
+      }
+    }
+    return fail(SMX_ERR_ARG, "the one-pair-segment pass is not available for this model and shape");
+  }
   if constexpr (model_coded(M) && !REG) {
     if (A.codes_in) {
       if (A.pair_seg && A.sink.adam_on)

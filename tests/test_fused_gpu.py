@@ -600,6 +600,51 @@ def test_second_stream_backward_gives_the_bits_of_the_serial_one(monkeypatch):
     assert abs(touched - plan.n_uniq) <= int((gs == 0).sum().item())
 
 
+def test_deferred_entity_pass_matches_the_one_call_backward(monkeypatch):
+    """The autograd flow takes the query gradients first and updates the rows later, in
+    score_backward_entity.  For large steps with the forward's codes that call hands the one-pair
+    segments to the pair-ordered kernel and runs the entity pass beside it: table, m and v must come
+    out bit-identical to the one-call backward and to the one-stream order."""
+    import bench
+    from smore_amd import fused
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(11)
+    n, b, k, dim = 1_500_000, 2800, 384, 200          # queries 4.5 MB (> one L2), 1.07 M pairs
+    table = torch.empty((n, dim), device="cuda").uniform_(-0.07, 0.07, generator=gen)
+    q1 = torch.empty((b, dim), device="cuda").uniform_(-0.07, 0.07, generator=gen)
+    q2 = torch.empty((b, dim), device="cuda").uniform_(0.0, 0.07, generator=gen)
+    idx = bench.zipf_ids(n, (b, k), 1.1, gen, torch.device("cuda"))
+    gs = torch.randn((b, k), device="cuda", generator=gen)
+    params = fused.score_params(24.0, 0.02)
+    plan = fused.build_plan(idx, n)
+    codes = fused.new_codes("box", table, idx, q1)
+    score = fused.score_forward("box", table, idx, q1, q2, params, codes=codes)
+    for squeeze in (False, True):
+        def state():
+            v_shape = (n, 1) if squeeze else (n, dim)
+            return table.clone(), torch.zeros_like(table), torch.zeros(v_shape, device="cuda")
+        opt = fused.adam_params(1e-4, 1, squeeze=squeeze)
+        monkeypatch.delenv("SMX_SERIAL_BACKWARD", raising=False)
+        w0, m0, v0 = state()
+        g1, g2 = fused.score_backward_fused("box", plan, w0, idx, q1, q2, score, gs, params, m=m0, v=v0, adam=opt,
+                                            codes=codes)
+        outcomes = []
+        for serial in (None, "1", None):
+            if serial:
+                monkeypatch.setenv("SMX_SERIAL_BACKWARD", serial)
+            else:
+                monkeypatch.delenv("SMX_SERIAL_BACKWARD", raising=False)
+            w, m, v = state()
+            d1, d2 = fused.score_backward_query("box", table, idx, q1, q2, score, gs, params, codes=codes)
+            fused.score_backward_entity("box", plan, w, q1, q2, score, gs, params, m=m, v=v, adam=opt, codes=codes)
+            torch.cuda.synchronize()
+            outcomes.append((d1, d2, w, m, v))
+        for got in outcomes:
+            for a, c, what in zip((g1, g2, w0, m0, v0), got, ("gq1", "gq2", "table", "m", "v")):
+                assert torch.equal(a, c), (what, squeeze)
+        assert (m0.abs().sum(dim=1) != 0).sum().item() > 0.9 * plan.n_uniq
+
+
 @pytest.mark.parametrize("b,k,dim", [(6, 50, 128), (3, 7, 30), (40, 300, 200)])
 def test_l1_sign_codes(b, k, dim):
     """L1 keeps one decision per feature (e - q > 0, ties go to -1): forward-saved codes, codes written by the
