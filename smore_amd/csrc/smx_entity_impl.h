@@ -152,6 +152,10 @@ __device__ __forceinline__ void apply_runs(const EntityArgs& A, const RunSet<R>&
 #pragma unroll
   for (int r = 0; r < R; ++r) {
     if (r < rs.n) {
+      float c_run = rs.c[r];
+      if constexpr (!CODED && SRC == mL2)
+        c_run = l2_pair_coef<VEC, NIT>(c_run, A.ncol, (int)(threadIdx.x & 63), [&](int it, int x) { return e.h[0][it].v[x]; },
+                                       [&](int it, int x) { return rr.a[r][it].v[x]; });
 #pragma unroll
       for (int it = 0; it < NIT; ++it) {
 #pragma unroll
@@ -161,7 +165,7 @@ __device__ __forceinline__ void apply_runs(const EntityArgs& A, const RunSet<R>&
           } else if constexpr (SRC == kSrcRows) {
             g1[it][x] += rr.a[r][it].v[x];
           } else {
-            const float c0 = rs.c[r];
+            const float c0 = c_run;
             const float c1 = second_coef<SRC>(c0, A.p);
             const typename ModelOps<SRC>::Q q =
                 ModelOps<SRC>::prep(rr.a[r][it].v[x], model_nq(SRC) == 2 ? rr.b[r][it].v[x] : 0.f);

@@ -131,10 +131,11 @@ template <> struct ModelOps<mL2> {
   }
   static __device__ __forceinline__ float fold(float a0, float, const ScoreParams&) { return a0; }
   static __device__ __forceinline__ float score(float folded, const ScoreParams& p) { return p.gamma - sqrtf(folded); }
-  // d(gamma - sqrt(d2)) / d d2 = -1 / (2 sqrt(d2)), and sqrt(d2) = gamma - score.  At d2 == 0 the
-  // coefficient is infinite, as autograd of torch.sqrt makes it in the reference.
-  static __device__ __forceinline__ void coef(float g, float s, const ScoreParams& p, float& c0, float& c1) {
-    c0 = -g / (2.0f * (p.gamma - s));
+  // d(gamma - sqrt(d2)) / d d2 = -1 / (2 sqrt(d2)): the kernels multiply this upstream part by the
+  // pair's own 1 / (2 sqrt(d2)), see l2_pair_coef.  At d2 == 0 the coefficient is infinite, as autograd
+  // of torch.sqrt makes it in the reference.
+  static __device__ __forceinline__ void coef(float g, float, const ScoreParams&, float& c0, float& c1) {
+    c0 = -g;
     c1 = 0.f;
   }
   static __device__ __forceinline__ void bwd_e(float c0, float, float e1, float, const Q& q, float& ge1, float&) {

@@ -53,6 +53,25 @@ inline AdamConsts make_adam_consts(const smx_opt_params* a) {
 __device__ __forceinline__ float hw_sqrt(float x) { return __builtin_amdgcn_sqrtf(x); }
 __device__ __forceinline__ float hw_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
 
+// L2 only.  score = gamma - sqrt(d2), so d score / d d2 = -1 / (2 sqrt(d2)).  The reference divides by the
+// square root autograd saved (l2_dist.py:59,62); recovering it as gamma - score would add half an ulp of
+// gamma to the distance, a relative error of 5e-7 / distance.  The backward kernels hold the pair's entity
+// row and query in registers anyway, so they sum d2 again, in the forward's order, and divide by its root.
+// c_raw: the upstream part of the coefficient (-gscore).  e(it, v), q(it, v): the lane's features.
+template <int VEC, int NIT, class GetE, class GetQ>
+__device__ __forceinline__ float l2_pair_coef(float c_raw, int ncol, int lane, GetE&& e, GetQ&& q) {
+  float mine = 0.f;
+#pragma unroll
+  for (int it = 0; it < NIT; ++it) {
+    float a0 = 0.f;
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) a0 += Term<kL2, float>::fwd(e(it, v), 0.f, q(it, v), 0.f);
+    mine += lane + 64 * it < ncol ? a0 : 0.f;
+  }
+  const float d2 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(wave_sum_last_f32(mine)), 63));
+  return c_raw / (2.0f * sqrtf(d2));
+}
+
 // 0 when the parameters are usable, else a message for the caller
 inline const char* check_opt_params(const smx_opt_params* a, const void* m, const void* v) {
   if (a->kind < SMX_OPT_ADAM || a->kind > SMX_OPT_RMSPROP) return "unknown optimizer kind";

@@ -456,7 +456,10 @@ __global__ __launch_bounds__(NW * 64) void score_backward_query_kernel(ScoreArgs
     // lanes past the row end hold a copy of the last column: what they accumulate is never stored
     stream_batch<MUL, VEC, NIT, RIF>(slab, cnt, dim, ncol, lane,
                                      [&](int j, const Pack<VEC>(&e1)[NIT], const Pack<VEC>(&e2)[NIT]) {
-      const float2 c = slab_coef(slab, j);
+      float2 c = slab_coef(slab, j);
+      if constexpr (M == mL2)
+        c.x = l2_pair_coef<VEC, NIT>(c.x, ncol, lane, [&](int it, int v) { return e1[it].v[v]; },
+                                     [&](int it, int v) { return q[it][v].a; });
       if constexpr (CODES == 1) {
         // the pair's code bytes go to the wavefront's LDS stage, see flush_codes
         unsigned char* mine_b = stage + (j & (kStagePairs - 1)) * (NIT * 64) + lane;
@@ -530,8 +533,11 @@ __global__ __launch_bounds__(NW * 64) void score_backward_query_kernel(ScoreArgs
         for (int s = 0; s < S; ++s) {
           if (js[s] >= 0) {
             const int j = js[s];
-            const float c0 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(my_c0), j));
+            float c0 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(my_c0), j));
             const float c1 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(my_c1), j));
+            if constexpr (M == mL2)
+              c0 = l2_pair_coef<VEC, NIT>(c0, ncol, lane, [&](int it, int v) { return e[s].h[0][it].v[v]; },
+                                          [&](int it, int v) { return q[it][v].a; });
             const int seg = __builtin_amdgcn_readlane(my_ps, j) & 0x7fffffff;
             const unsigned row = (unsigned)__builtin_amdgcn_readlane((int)pb.row, j);
             float ge1[NIT][VEC], ge2[NIT][VEC];

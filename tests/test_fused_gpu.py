@@ -155,6 +155,28 @@ def test_fused_step_matches_oracle(model, shape):
     run_case(model, n, b, k, dim)
 
 
+def _sweep_cases(count=20):
+    """Seeded random shapes: few ids (long segments) to many, K below / across / above the 64-pair batch,
+    dims on and off the float4 path and across the 256- and 512-float column groups."""
+    rng = np.random.default_rng(20240)
+    models = list(GAMMA)
+    cases = []
+    for i in range(count):
+        dim = int(rng.choice([4, 12, 31, 64, 100, 200, 260, 400, 516]))
+        if dim % 4 and dim > 256:
+            dim -= dim % 4
+        b, k = int(rng.integers(1, 12)), int(rng.choice([1, 3, 63, 64, 65, 130, 257]))
+        n = int(rng.choice([7, 50, 600, 20000]))
+        cases.append((models[i % len(models)], n, b, k, dim, None if i % 3 else 1.1))
+    return cases
+
+
+@pytest.mark.parametrize("case", _sweep_cases(), ids=lambda c: "-".join(str(x) for x in c))
+def test_fused_step_random_shapes(case):
+    model, n, b, k, dim, zipf = case
+    run_case(model, n, b, k, dim, zipf=zipf, adam_steps=1)
+
+
 @pytest.mark.parametrize("model", ["box", "rotate"])
 def test_segments_crossing_many_tiles(model):
     """Zipf ids with a head id that owns ~20% of 16k pairs: segments span many tiles of the
