@@ -111,7 +111,7 @@ def run_case(model, n, b, k, dim, zipf=None, cen=0.02, adam_steps=2, lr=1e-3):
     # gradient cancels to ~eps its update is ill-conditioned, so (a) the Adam arithmetic is checked step
     # by step from the device's own state and merged gradient, to the 1e-5 bar, and (b) the end-to-end
     # trajectory against the float64 oracle is checked to 1e-5 on all but a sliver of such elements,
-    # which must still be within one learning-rate step.
+    # which must still be within two learning-rate steps (an Adam step is at most lr long, in either direction).
     w_o, m_o, v_o = table.copy(), np.zeros_like(table), np.zeros_like(table)
     t_m, t_v = torch.zeros_like(t_table), torch.zeros_like(t_table)
     touched = np.zeros(n, bool)
@@ -136,7 +136,7 @@ def run_case(model, n, b, k, dim, zipf=None, cen=0.02, adam_steps=2, lr=1e-3):
     got_w = t_table.cpu().numpy()
     err = np.abs(got_w - w_o)[touched]
     tol = REL_F32 * np.maximum(np.abs(w_o[touched]), np.sqrt(np.mean(w_o[touched] ** 2)))
-    assert (err > tol).mean() < 1e-3 and err.max() < lr * adam_steps, (err.max(), (err > tol).mean())
+    assert (err > tol).mean() < 1e-3 and err.max() < 2 * lr * adam_steps, (err.max(), (err > tol).mean())
     assert_close(t_m.cpu().numpy()[touched], m_o[touched], 5 * REL_F32, f"{model} m trajectory")
     assert np.array_equal(got_w[~touched], table[~touched].astype(np.float32)), "untouched rows must stay bit-identical"
     assert not t_m.cpu().numpy()[~touched].any() and not t_v.cpu().numpy()[~touched].any()
