@@ -157,7 +157,7 @@ __global__ __launch_bounds__(256) void rank_scan_kernel(RankArgs A) {
 #pragma unroll
   for (int x = 0; x < NB; ++x) {
     qb[x] = min(A.b0 + x, A.B - 1);  // a pass past the last query repeats it; its histogram is dropped
-    count[x] = A.ans_count[qb[x]];
+    count[x] = min(max(A.ans_count[qb[x]], 0), A.A);  // a count beyond the slots would index past the LDS arrays
     load_rank_query<M, VEC, NIT>(A.q1, A.q2, qb[x], dim, A.ncol, lane, q[x]);
   }
   const int chunks = (A.A + 63) / 64;
