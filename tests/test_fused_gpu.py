@@ -177,6 +177,45 @@ def test_fused_step_random_shapes(case):
     run_case(model, n, b, k, dim, zipf=zipf, adam_steps=1)
 
 
+def test_rotate_zero_modulus_features_follow_the_eps_convention():
+    """Features where entity and query coincide: the modulus is sqrt(0 + 1e-20) and its derivative
+    0 * rsqrt(1e-20) = 0 (cuda_math_ext.h:100-118) -- finite, no NaN, on the fused and the dense path."""
+    from smore_amd import fused
+    from smore_amd import extlib_hip as ext
+    rng = np.random.default_rng(2)
+    n, b, k, dim = 30, 3, 9, 24
+    table, q1, q2, idx, gs = make_problem("rotate", n, b, k, dim, rng)
+    table[5, :dim] = q1[0]; table[5, dim:] = q2[0]          # entity 5 equals query 0 in every feature
+    table[6, :7] = q1[1, :7]; table[6, dim:dim + 7] = q2[1, :7]   # entity 6 equals query 1 in seven of them
+    idx[0, :2] = 5
+    idx[1, 3] = 6
+    params = fused.score_params(GAMMA["rotate"], 0.0)
+    t_table, t_q1, t_q2, t_gs, t_idx = dev(table), dev(q1), dev(q2), dev(gs), torch.tensor(idx, device="cuda")
+    score = fused.score_forward("rotate", t_table, t_idx, t_q1, t_q2, params)
+    rows = orc.gather(table, idx).reshape(b, k, -1)
+    want = orc.score_forward("rotate", rows, q1[:, None], q2[:, None], GAMMA["rotate"], 0.0)
+    assert_close(score.cpu().numpy(), want, REL_F32, "rotate score with zero-modulus features")
+    assert abs(GAMMA["rotate"] - score[0, 0].item() - dim * 1e-10) < 1e-12 + 1e-6 * dim * 1e-10 + 1e-6  # gamma - dim * sqrt(eps)
+    gq1, gq2 = fused.score_backward_query("rotate", t_table, t_idx, t_q1, t_q2, score, t_gs, params)
+    o_rows, o_g1, o_g2 = orc.score_backward("rotate", gs, rows, q1[:, None], q2[:, None], 0.0)
+    assert torch.isfinite(gq1).all() and torch.isfinite(gq2).all()
+    assert_close(gq1.cpu().numpy(), o_g1[:, 0], REL_F32, "gq1")
+    assert_close(gq2.cpu().numpy(), o_g2[:, 0], REL_F32, "gq2")
+    plan = fused.build_plan(t_idx, n)
+    merged = torch.empty((plan.n_uniq, 2 * dim), device="cuda")
+    fused.score_backward_entity("rotate", plan, t_table, t_q1, t_q2, score, t_gs, params, merged=merged)
+    assert torch.isfinite(merged).all()
+    uniq, inverse, _, _ = orc.merge_indices(idx)
+    o_merged = orc.merge_grads(o_rows.reshape(b * k, -1), inverse, uniq.size)
+    o_abs = orc.merge_grads(np.abs(o_rows).reshape(b * k, -1), inverse, uniq.size)
+    assert_close(merged.cpu().numpy(), o_merged, REL_F32, "merged", sum_abs=o_abs)
+    # the dense operator on the same rows
+    t_rows = dev(rows)
+    dst = torch.empty((b, k), device="cuda")
+    ext.dist_forward("rotate", t_rows, t_q1[:, None].contiguous(), t_q2[:, None].contiguous(), dst, True)
+    assert_close(dst.cpu().numpy(), GAMMA["rotate"] - want, REL_F32, "dense rotate distance")
+
+
 @pytest.mark.parametrize("model", ["box", "rotate"])
 def test_segments_crossing_many_tiles(model):
     """Zipf ids with a head id that owns ~20% of 16k pairs: segments span many tiles of the
