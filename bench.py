@@ -207,6 +207,42 @@ def cpu_baseline(cfg, seed):
     }
 
 
+def measure_ceilings(device, row_bytes, full=False):
+    """What plain kernels sustain on this GPU (GB/s of bytes moved, reads + writes), from the library's
+    probe kernels on two 4 GiB scratch buffers: streaming read, copy, and rows of the workload's length
+    read at random positions.  full: also plain-load read, in-place update, fill, non-temporal rows."""
+    import ctypes
+    import torch
+    from smore_amd import _lib
+    nbytes = 4 << 30
+    a = torch.zeros(nbytes, dtype=torch.uint8, device=device)
+    b = torch.zeros(nbytes, dtype=torch.uint8, device=device)
+    sink = torch.zeros(1, device=device)
+    row_bytes = min(1024, max(16, row_bytes - row_bytes % 16))
+    n_reads = (2 << 30) // row_bytes
+    kinds = [("read", 0, nbytes), ("copy", 2, 2 * nbytes), ("random_rows", 5, n_reads * row_bytes)]
+    if full:
+        kinds += [("read_plain_loads", 1, nbytes), ("update_in_place", 3, 2 * nbytes), ("fill", 4, nbytes),
+                  ("random_rows_nontemporal", 6, n_reads * row_bytes)]
+    out = {"row_bytes": row_bytes}
+    stream = ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+    for name, kind, moved in kinds:
+        def launch():
+            _lib.call("smx_probe_bandwidth", kind, stream, ctypes.c_void_p(a.data_ptr()), ctypes.c_void_p(b.data_ptr()),
+                      nbytes, row_bytes, n_reads, ctypes.c_void_p(sink.data_ptr()))
+        launch()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(3):
+            launch()
+        e1.record()
+        e1.synchronize()
+        out[name + "_GBps"] = round(3 * moved / (e0.elapsed_time(e1) * 1e-3) / 1e9, 1)
+    del a, b
+    torch.cuda.empty_cache()
+    return out
+
+
 def rank_scan_bench(cfg, device, seed, steps, warmup, nq):
     """Evaluation against all entities: one pass over the table per four queries (rows of up to 512
     floats), two, or one, as the library's launcher chooses; the roofline is the table streamed once per
@@ -262,6 +298,9 @@ def main():
                          "config's table instead of the training step; prints its own JSON line")
     ap.add_argument("--rank-queries", type=int, default=1,
                     help="queries per call of the evaluation scan (the reference evaluates one query at a time)")
+    ap.add_argument("--ceilings", action="store_true",
+                    help="run only the bandwidth probes (read, copy, update, fill, random rows of the config's row "
+                         "length, plain and non-temporal) and print them as one JSON line")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run only a plain row copy of known size (1 GiB read + 1 GiB written per launch) through "
                          "smx_gather_rows; under rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE this gives the counters' scale")
@@ -289,6 +328,10 @@ def main():
         return
     cfg = CONFIGS[args.config]
     seed = args.seed if args.seed is not None else 20240 + args.config
+    if args.ceilings:
+        print(json.dumps({"measured_ceilings": measure_ceilings(device, 4 * row_len(cfg), full=True),
+                          "nominal_peak_GBps": HBM_PEAK_GBPS}))
+        return
     if args.rank_scan:
         rank_scan_bench(cfg, device, seed, args.steps, args.warmup, args.rank_queries)
         return
@@ -346,6 +389,11 @@ def main():
         },
         "phase_ms": phase_ms,
     }
+    # what plain kernels sustain on this GPU for the step's access shapes, measured now with the library's
+    # probes (after the timed region); a step that writes w, m, v back is a copy-like mix of reads and writes
+    out["measured_ceilings"] = measure_ceilings(device, 4 * row_len(cfg))
+    out["step_hbm"]["frac_of_measured_copy"] = out["step_hbm"]["achieved_GBps"] / out["measured_ceilings"]["copy_GBps"]
+    out["roofline"]["frac_of_measured_copy"] = ent_gbps / out["measured_ceilings"]["copy_GBps"]
     del out["config"]["model"]
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(cfg, seed)

@@ -283,6 +283,23 @@ int smx_rank_scan(int model, void* stream, const float* table, size_t n_rows, co
                   const int64_t* ans_id, const uint64_t* ans_key, const int32_t* ans_count, size_t A,
                   int64_t* filtered_rank, void* workspace, size_t workspace_bytes);
 
+/* ---- bandwidth probes (measurement only) --------------------------------------------------------
+ * No counterpart in the reference.  One launch of a kernel that does nothing but move memory in one of
+ * the access shapes of this path, for bench.py to time: what the box sustains, next to the nominal peak.
+ *   READ_NT / READ   stream `bytes` of a (non-temporal / plain loads)
+ *   COPY             a -> b          UPDATE  a = 2 a in place          FILL  a = constant
+ *   ROWS / ROWS_NT   n_reads rows of row_bytes (16..1024, multiple of 16) at pseudo-random positions of a
+ * sink: one device float the read probes may write (keeps their loads alive); never meaningful. */
+#define SMX_PROBE_READ_NT 0
+#define SMX_PROBE_READ 1
+#define SMX_PROBE_COPY 2
+#define SMX_PROBE_UPDATE 3
+#define SMX_PROBE_FILL 4
+#define SMX_PROBE_ROWS 5
+#define SMX_PROBE_ROWS_NT 6
+int smx_probe_bandwidth(int kind, void* stream, void* a, void* b, size_t bytes, size_t row_bytes,
+                        size_t n_reads, float* sink);
+
 /* Plain row lookup out[k,:] = table[idx[k],:] (smore/common/embedding/embed_rw.py:74-75, the GPU
  * branch of EmbeddingReadOnly.read) for callers that need the rows themselves. */
 int smx_gather_rows(void* stream, const float* table, size_t n_rows, size_t row_len,

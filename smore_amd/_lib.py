@@ -29,6 +29,8 @@ SIGNATURES = {
     "smx_dist_forward_f64": (_i, _DENSE_FWD),
     "smx_dist_backward_f32": (_i, _DENSE_BWD),
     "smx_dist_backward_f64": (_i, _DENSE_BWD),
+    # kind, stream, a, b, bytes, row_bytes, n_reads, sink
+    "smx_probe_bandwidth": (_i, [_i, _vp, _vp, _vp, _sz, _sz, _sz, _vp]),
     "smx_score_codes_bytes": (_sz, [_i, _sz, _sz]),
     # model, stream, table, n_rows, idx, q1, q2, score, B, K, dim, params, err_flag, codes, codes_bytes
     "smx_score_forward": (_i, [_i, _vp, _vp, _sz, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _vp, _vp, _vp, _sz]),
