@@ -203,7 +203,8 @@ typedef struct smx_opt_params {
  * With them, an optimizer, no merged output and a step of a million pairs or more whose queries
  * exceed one L2, the call finishes ids that occur once in a pair-ordered kernel on `stream` and
  * reduces the others on the library's second stream beside it (joined to `stream` before return);
- * the rows get the same bits either way. */
+ * the rows get the same bits either way.  (Environment: SMX_SERIAL_BACKWARD=1 keeps this call and
+ * smx_score_backward_fused on the caller's stream alone -- for per-kernel profiling.) */
 size_t smx_entity_workspace_bytes(size_t n_pairs, size_t row_len);
 int smx_score_backward_entity(int model, void* stream, const smx_plan_view* plan, float* table,
                               size_t n_rows, const float* q1, const float* q2, const float* score,
