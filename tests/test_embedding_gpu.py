@@ -246,6 +246,39 @@ def test_state_buffers_are_in_the_state_dict():
     assert {"embedding", "state_sum_fo", "state_sum_sq"} <= set(sd)
 
 
+def test_checkpoint_round_trip_resumes_the_same_trajectory():
+    """model.state_dict() carries the table and the optimizer moments under the reference's names
+    (train_process.py:252-262 saves exactly that); a fresh module that loads it continues bit for bit."""
+    import io
+    n, d, b, k, lr = 200, 16, 4, 12, 1e-3
+    rng = np.random.default_rng(8)
+    ids = [torch.tensor(rng.integers(0, n, (b, k)), device="cuda") for _ in range(3)]
+    c = torch.tensor(rng.uniform(-0.07, 0.07, (b, 1, d)), dtype=torch.float32, device="cuda")
+    o = torch.tensor(np.abs(rng.uniform(-0.07, 0.07, (b, 1, d))), dtype=torch.float32, device="cuda")
+    g = torch.tensor(rng.standard_normal((b, k)), dtype=torch.float32, device="cuda")
+
+    def train(emb, opt, steps):
+        for i in steps:
+            opt.zero_grad()
+            (opt.score_negatives("box", ids[i], c, o, gamma=24.0, cen=0.02) * g).sum().backward()
+            opt.apply_grad(lr)
+
+    emb, opt = _setup(n, d, 5)
+    train(emb, opt, [0, 1])
+    blob = io.BytesIO()
+    torch.save({"model_state_dict": emb.state_dict()}, blob)
+    train(emb, opt, [2])
+
+    emb2, opt2 = _setup(n, d, 99)                      # different initial values, overwritten by the load
+    blob.seek(0)
+    missing, unexpected = emb2.load_state_dict(torch.load(blob, weights_only=True)["model_state_dict"], strict=False)
+    assert not missing and not unexpected
+    opt2.step = 2                                      # the step counter lives with the trainer, as in the reference
+    train(emb2, opt2, [2])
+    for name in ("embedding", "state_sum_fo", "state_sum_sq"):
+        assert torch.equal(emb.state_dict()[name], emb2.state_dict()[name]), name
+
+
 @pytest.mark.parametrize("name", ["adam", "sgd", "adagrad", "rmsprop"])
 @pytest.mark.parametrize("squeeze", [False, True])
 def test_row_optimizers_match_oracle(name, squeeze):
