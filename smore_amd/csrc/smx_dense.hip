@@ -3,16 +3,22 @@
 // These are the layout-general kernels behind smx_dist_forward_* /
 // smx_dist_backward_*: entity [be,ne,dim*mul] against query [bc,nc,dim] with
 // the modulo broadcast rule of the replaced launch loops
-// (smore/common/torchext/common_kernel.h:41-49, 73-81, 108-115).  The
-// per-query-negatives layout with 16-byte aligned fp32 rows is routed to the
-// vectorised kernels in smx_score.hip instead.
+// (smore/common/torchext/common_kernel.h:41-49, 73-81, 108-115).
 //
+// General kernels (any layout, fp32 and fp64):
 // forward : one wavefront per output element, lanes stride the feature axis,
 //           xor-butterfly reduction over 64 lanes.
 // backward: one workgroup per row of the side being differentiated; each
 //           thread owns features d, d+blockDim, ... and walks that row's jobs
 //           in ascending job order, so every sum has a fixed order and no
 //           atomics are needed.
+//
+// Per-query kernels (fp32, 16-byte aligned rows, entity [B,N,dim*mul] against query [B,1,dim]: the
+// layout of the models' negatives [B,K] and positives [B,1], kg_reasoning.py:342-355): the query lives
+// in LDS / registers, every entity row is read once with 16-byte loads, and the backward writes the
+// row gradient and accumulates the query gradient in the same pass.
+#include <type_traits>
+
 #include "smx_common.h"
 #include "smx_functors.h"
 
@@ -101,6 +107,171 @@ __global__ __launch_bounds__(128) void dense_backward_kernel(const T* __restrict
   }
 }
 
+// ---- per-query layout, fp32 -------------------------------------------------------------------
+typedef float dvec4 __attribute__((ext_vector_type(4)));
+constexpr int kPqBwdWaves = 8;
+
+template <int K>
+__device__ __forceinline__ float pq_row_terms(const dvec4* __restrict__ pe, const float* lds, int ncol, int dim, int lane) {
+  constexpr int MUL = kind_mul(K), NQ = kind_nq(K);
+  float s = 0.f;
+  for (int c = lane; c < ncol; c += kWave) {
+    const dvec4 e1 = pe[c];
+    const dvec4 e2 = MUL == 2 ? pe[c + ncol] : dvec4{0.f, 0.f, 0.f, 0.f};
+    const dvec4 a = reinterpret_cast<const dvec4*>(lds)[c];
+    const dvec4 b = NQ == 2 ? reinterpret_cast<const dvec4*>(lds + dim)[c] : dvec4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int x = 0; x < 4; ++x) s += Term<K, float>::fwd(e1[x], e2[x], a[x], b[x]);
+  }
+  return s;
+}
+
+// One workgroup per (query, tile of rows); its four wavefronts take the tile's rows two at a time.
+template <int K>
+__global__ __launch_bounds__(256) void dense_pq_forward_kernel(const float* __restrict__ ent, const float* __restrict__ q1,
+                                                               const float* __restrict__ q2, float* __restrict__ dst,
+                                                               int num, int dim, int tiles, int rows_per_tile) {
+  constexpr int MUL = kind_mul(K), NQ = kind_nq(K);
+  extern __shared__ float lds[];  // q1[dim] | q2[dim]
+  const int b = blockIdx.x / tiles, tile = blockIdx.x - b * tiles;
+  for (int d = threadIdx.x; d < dim; d += 256) {
+    lds[d] = q1[(size_t)b * dim + d];
+    if (NQ == 2) lds[dim + d] = q2[(size_t)b * dim + d];
+  }
+  __syncthreads();
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  const int ncol = dim / 4;
+  const int k1 = min(num, (tile + 1) * rows_per_tile);
+  const size_t row_len = (size_t)dim * MUL;
+  for (int k = tile * rows_per_tile + wave; k < k1; k += 8) {
+    const size_t r0 = (size_t)b * num + k;
+    const bool two = k + 4 < k1;
+    const size_t r1 = two ? r0 + 4 : r0;
+    float s0 = pq_row_terms<K>(reinterpret_cast<const dvec4*>(ent + r0 * row_len), lds, ncol, dim, lane);
+    float s1 = pq_row_terms<K>(reinterpret_cast<const dvec4*>(ent + r1 * row_len), lds, ncol, dim, lane);
+    s0 = wave_sum(s0);
+    s1 = wave_sum(s1);
+    if (lane == 0) {
+      dst[r0] = s0;
+      if (two) dst[r1] = s1;
+    }
+  }
+}
+
+// One workgroup of eight wavefronts per query.  Lane l owns the 16-byte columns l, l+64, ... of the row
+// (NIT of them); wavefront w takes rows w, w+8, ...  For every row it writes the row's gradient and adds
+// the row's contribution to its query-gradient registers; the eight partial query gradients are summed
+// through LDS in wavefront order, so the result does not depend on timing.
+template <int K, int NIT>
+__global__ __launch_bounds__(kPqBwdWaves * kWave) void dense_pq_backward_kernel(
+    const float* __restrict__ gout, const float* __restrict__ ent, const float* __restrict__ q1,
+    const float* __restrict__ q2, float* __restrict__ gent, float* __restrict__ gq1, float* __restrict__ gq2, int num,
+    int dim) {
+  constexpr int MUL = kind_mul(K), NQ = kind_nq(K);
+  extern __shared__ float lds[];  // [waves][NQ][dim]
+  const int b = blockIdx.x;
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  const int ncol = dim / 4;
+  const size_t row_len = (size_t)dim * MUL;
+  const dvec4 zero = {0.f, 0.f, 0.f, 0.f};
+  dvec4 qa[NIT], qb[NIT], acc1[NIT], acc2[NIT];
+#pragma unroll
+  for (int it = 0; it < NIT; ++it) {
+    const int c = min(lane + kWave * it, ncol - 1);
+    qa[it] = reinterpret_cast<const dvec4*>(q1 + (size_t)b * dim)[c];
+    qb[it] = NQ == 2 ? reinterpret_cast<const dvec4*>(q2 + (size_t)b * dim)[c] : zero;
+    acc1[it] = acc2[it] = zero;
+  }
+  for (int k = wave; k < num; k += kPqBwdWaves) {
+    const size_t r = (size_t)b * num + k;
+    const float g = gout[r];
+    const dvec4* pe = reinterpret_cast<const dvec4*>(ent + r * row_len);
+    dvec4* pg = reinterpret_cast<dvec4*>(gent + r * row_len);
+    dvec4 e1[NIT], e2[NIT];
+#pragma unroll
+    for (int it = 0; it < NIT; ++it) {
+      const int c = min(lane + kWave * it, ncol - 1);
+      e1[it] = pe[c];
+      e2[it] = MUL == 2 ? pe[c + ncol] : zero;
+    }
+#pragma unroll
+    for (int it = 0; it < NIT; ++it) {
+      const int c = lane + kWave * it;
+      if (c < ncol) {
+        dvec4 ge1 = zero, ge2 = zero;
+#pragma unroll
+        for (int x = 0; x < 4; ++x) {
+          float a1 = 0.f, a2 = 0.f, b1 = acc1[it][x], b2 = acc2[it][x];
+          Term<K, float>::bwd(g, e1[it][x], e2[it][x], qa[it][x], qb[it][x], a1, a2, b1, b2);
+          ge1[x] = a1;
+          ge2[x] = a2;
+          acc1[it][x] = b1;
+          acc2[it][x] = b2;
+        }
+        __builtin_nontemporal_store(ge1, pg + c);
+        if (MUL == 2) __builtin_nontemporal_store(ge2, pg + c + ncol);
+      }
+    }
+  }
+#pragma unroll
+  for (int it = 0; it < NIT; ++it) {
+    const int c = lane + kWave * it;
+    if (c < ncol) {
+      reinterpret_cast<dvec4*>(lds + (size_t)(wave * NQ + 0) * dim)[c] = acc1[it];
+      if (NQ == 2) reinterpret_cast<dvec4*>(lds + (size_t)(wave * NQ + 1) * dim)[c] = acc2[it];
+    }
+  }
+  __syncthreads();
+  for (int d = threadIdx.x; d < dim; d += kPqBwdWaves * kWave) {
+    float s1 = 0.f, s2 = 0.f;
+#pragma unroll
+    for (int w = 0; w < kPqBwdWaves; ++w) {
+      s1 += lds[(size_t)(w * NQ + 0) * dim + d];
+      if (NQ == 2) s2 += lds[(size_t)(w * NQ + 1) * dim + d];
+    }
+    gq1[(size_t)b * dim + d] = s1;
+    if (NQ == 2) gq2[(size_t)b * dim + d] = s2;
+  }
+}
+
+// entity [B,N,.] against query [B,1,.], float4-able, and small enough for the kernels above
+static bool pq_layout(const Layout& L, int kind, const void* a, const void* b, const void* c, const void* d,
+                      const void* e, const void* f, const void* g) {
+  if (L.be != L.bsize || L.bc != L.bsize || L.ne != L.num || L.nc != 1) return false;
+  if (L.dim % 4 != 0 || L.dim > 1024 || L.bsize * L.num > 0x7fffffffull || L.num > 0x7fffffffull) return false;
+  (void)kind;
+  return aligned16(a) && aligned16(b) && aligned16(c) && aligned16(d) && aligned16(e) && aligned16(f) && aligned16(g);
+}
+
+template <int K>
+static int forward_pq(hipStream_t st, const float* ent, const float* q1, const float* q2, float* dst, const Layout& L) {
+  // enough workgroups to fill the chip, at least eight rows each when there are that many
+  int rows_per_tile = (int)L.num;
+  while (rows_per_tile > 8 && L.bsize * ((L.num + rows_per_tile - 1) / rows_per_tile) < 8192) rows_per_tile = (rows_per_tile + 1) / 2;
+  const int tiles = (int)((L.num + rows_per_tile - 1) / rows_per_tile);
+  if (L.bsize * (size_t)tiles > 0x7fffffffull) return -1;
+  const size_t lds = (size_t)kind_nq(K) * L.dim * sizeof(float);
+  hipLaunchKernelGGL((dense_pq_forward_kernel<K>), dim3((unsigned)(L.bsize * tiles)), dim3(256), lds, st, ent, q1, q2, dst,
+                     (int)L.num, (int)L.dim, tiles, rows_per_tile);
+  return check_launch("dist forward (per-query layout)");
+}
+
+template <int K>
+static int backward_pq(hipStream_t st, const float* gout, const float* ent, const float* q1, const float* q2, float* gent,
+                       float* gq1, float* gq2, const Layout& L) {
+  const size_t lds = (size_t)kPqBwdWaves * kind_nq(K) * L.dim * sizeof(float);
+  const dim3 grid((unsigned)L.bsize), block(kPqBwdWaves * kWave);
+  const int num = (int)L.num, dim = (int)L.dim;
+  const size_t ncol = L.dim / 4;
+  if (ncol <= 64)
+    hipLaunchKernelGGL((dense_pq_backward_kernel<K, 1>), grid, block, lds, st, gout, ent, q1, q2, gent, gq1, gq2, num, dim);
+  else if (ncol <= 128)
+    hipLaunchKernelGGL((dense_pq_backward_kernel<K, 2>), grid, block, lds, st, gout, ent, q1, q2, gent, gq1, gq2, num, dim);
+  else
+    hipLaunchKernelGGL((dense_pq_backward_kernel<K, 4>), grid, block, lds, st, gout, ent, q1, q2, gent, gq1, gq2, num, dim);
+  return check_launch("dist backward (per-query layout)");
+}
+
 static int check_layout(const Layout& L) {
   if (L.bsize == 0 || L.num == 0 || L.dim == 0 || L.be == 0 || L.ne == 0 || L.bc == 0 || L.nc == 0)
     return fail(SMX_ERR_SHAPE, "empty dimension in dist layout");
@@ -142,6 +313,17 @@ int dense_forward(int kind, void* stream, const T* ent, const T* q1, const T* q2
   if (int rc = check_layout(L)) return rc;
   if (!ent || !q1 || !dst || (kind_nq(kind) == 2 && !q2)) return fail(SMX_ERR_ARG, "null tensor pointer");
   hipStream_t st = as_stream(stream);
+  if constexpr (std::is_same<T, float>::value) {
+    if (pq_layout(L, kind, ent, q1, q2, dst, nullptr, nullptr, nullptr)) {
+      switch (kind) {
+#define X(KK) \
+  case KK:    \
+    return forward_pq<KK>(st, ent, q1, q2, dst, L);
+        SMX_FOR_EACH_KIND(X)
+#undef X
+      }
+    }
+  }
   switch (kind) {
 #define X(KK) \
   case KK:    \
@@ -161,6 +343,17 @@ int dense_backward(int kind, void* stream, const T* gout, const T* ent, const T*
   if (!gout || !ent || !q1 || !gent || !gq1 || (kind_nq(kind) == 2 && (!q2 || !gq2)))
     return fail(SMX_ERR_ARG, "null tensor pointer");
   hipStream_t st = as_stream(stream);
+  if constexpr (std::is_same<T, float>::value) {
+    if (pq_layout(L, kind, gout, ent, q1, q2, gent, gq1, gq2)) {
+      switch (kind) {
+#define X(KK) \
+  case KK:    \
+    return backward_pq<KK>(st, gout, ent, q1, q2, gent, gq1, gq2, L);
+        SMX_FOR_EACH_KIND(X)
+#undef X
+      }
+    }
+  }
   switch (kind) {
 #define X(KK) \
   case KK:    \
