@@ -149,6 +149,31 @@ template <typename T> struct Term<kBetaKL, T> {
   }
 };
 
+// fp32: the same closed forms on the shared fast evaluations of smx_math.h (one call per Beta
+// distribution gives its three digammas or trigammas and its log-Beta term without a data-dependent loop).
+template <> struct Term<kBetaKL, float> {
+  static __device__ __forceinline__ float fwd(float ea, float eb, float qa, float qb) {
+    float lbe, pa, pb, ps, lbq, ua, ub, us;
+    beta_terms(ea, eb, lbe, pa, pb, ps);   // lbe = lgamma(se) - lgamma(ea) - lgamma(eb)
+    beta_terms(qa, qb, lbq, ua, ub, us);   // only lbq is used
+    return (lbe - lbq) + (ea - qa) * pa + (eb - qb) * pb + ((qa + qb) - (ea + eb)) * ps;
+  }
+  static __device__ __forceinline__ void bwd(float g, float ea, float eb, float qa, float qb, float& gea, float& geb,
+                                             float& gqa, float& gqb) {
+    const float se = ea + eb, sq = qa + qb;
+    float ta, tb, ts, pa, pb, ps, ua, ub, us;
+    trigamma3(ea, eb, ta, tb, ts);
+    digamma3(ea, eb, pa, pb, ps);
+    digamma3(qa, qb, ua, ub, us);
+    const float common_e = (sq - se) * ts;
+    gea += g * ((ea - qa) * ta + common_e);
+    geb += g * ((eb - qb) * tb + common_e);
+    const float common_q = ps - us;
+    gqa += g * (ua - pa + common_q);
+    gqb += g * (ub - pb + common_q);
+  }
+};
+
 // dist_kernel.h:269-287
 template <typename T> struct Term<kBetaL2, T> {
   static __device__ __forceinline__ T fwd(T e1, T e2, T q1, T q2) {
@@ -176,6 +201,27 @@ template <typename T> struct Term<kBetaFisher, T> {
     const T da = ea - qa, db = eb - qb;
     const T m = nab * (da + db);
     const T gl = g * (pa * da + m), gr = g * (pb * db + m);
+    gea += gl;
+    geb += gr;
+    gqa -= gl;
+    gqb -= gr;
+  }
+};
+
+template <> struct Term<kBetaFisher, float> {
+  static __device__ __forceinline__ float fwd(float ea, float eb, float qa, float qb) {
+    float pa, pb, ps;
+    trigamma3(ea, eb, pa, pb, ps);
+    const float nab = -ps, da = ea - qa, db = eb - qb;
+    return 0.5f * (da * da * (pa + nab) + 2 * nab * da * db + db * db * (pb + nab));
+  }
+  static __device__ __forceinline__ void bwd(float g, float ea, float eb, float qa, float qb, float& gea, float& geb,
+                                             float& gqa, float& gqb) {
+    float pa, pb, ps;
+    trigamma3(ea, eb, pa, pb, ps);
+    const float nab = -ps, da = ea - qa, db = eb - qb;
+    const float m = nab * (da + db);
+    const float gl = g * (pa * da + m), gr = g * (pb * db + m);
     gea += gl;
     geb += gr;
     gqa -= gl;
