@@ -127,7 +127,7 @@ __device__ __forceinline__ float pq_row_terms(const dvec4* __restrict__ pe, cons
 }
 
 // One workgroup per (query, tile of rows); its four wavefronts take the tile's rows two at a time.
-template <int K>
+template <int K, bool SHARED = false>
 __global__ __launch_bounds__(256) void dense_pq_forward_kernel(const float* __restrict__ ent, const float* __restrict__ q1,
                                                                const float* __restrict__ q2, float* __restrict__ dst,
                                                                int num, int dim, int tiles, int rows_per_tile) {
@@ -147,8 +147,9 @@ __global__ __launch_bounds__(256) void dense_pq_forward_kernel(const float* __re
     const size_t r0 = (size_t)b * num + k;
     const bool two = k + 4 < k1;
     const size_t r1 = two ? r0 + 4 : r0;
-    float s0 = pq_row_terms<K>(reinterpret_cast<const dvec4*>(ent + r0 * row_len), lds, ncol, dim, lane);
-    float s1 = pq_row_terms<K>(reinterpret_cast<const dvec4*>(ent + r1 * row_len), lds, ncol, dim, lane);
+    const size_t e0 = SHARED ? (size_t)k : r0, e1 = SHARED ? (size_t)(two ? k + 4 : k) : r1;  // entity rows
+    float s0 = pq_row_terms<K>(reinterpret_cast<const dvec4*>(ent + e0 * row_len), lds, ncol, dim, lane);
+    float s1 = pq_row_terms<K>(reinterpret_cast<const dvec4*>(ent + e1 * row_len), lds, ncol, dim, lane);
     s0 = wave_sum(s0);
     s1 = wave_sum(s1);
     if (lane == 0) {
@@ -162,7 +163,9 @@ __global__ __launch_bounds__(256) void dense_pq_forward_kernel(const float* __re
 // (NIT of them); wavefront w takes rows w, w+8, ...  For every row it writes the row's gradient and adds
 // the row's contribution to its query-gradient registers; the eight partial query gradients are summed
 // through LDS in wavefront order, so the result does not depend on timing.
-template <int K, int NIT>
+// SHARED: the entity rows are the same [1,N,.] for every query (--share_negative, online_sampler.py:155-157);
+// this kernel then gives the query gradients only, and dense_shared_entity_backward_kernel the rows'.
+template <int K, int NIT, bool SHARED = false>
 __global__ __launch_bounds__(kPqBwdWaves * kWave) void dense_pq_backward_kernel(
     const float* __restrict__ gout, const float* __restrict__ ent, const float* __restrict__ q1,
     const float* __restrict__ q2, float* __restrict__ gent, float* __restrict__ gq1, float* __restrict__ gq2, int num,
@@ -185,8 +188,9 @@ __global__ __launch_bounds__(kPqBwdWaves * kWave) void dense_pq_backward_kernel(
   for (int k = wave; k < num; k += kPqBwdWaves) {
     const size_t r = (size_t)b * num + k;
     const float g = gout[r];
-    const dvec4* pe = reinterpret_cast<const dvec4*>(ent + r * row_len);
-    dvec4* pg = reinterpret_cast<dvec4*>(gent + r * row_len);
+    const size_t er = SHARED ? (size_t)k : r;
+    const dvec4* pe = reinterpret_cast<const dvec4*>(ent + er * row_len);
+    dvec4* pg = reinterpret_cast<dvec4*>(gent + er * row_len);
     dvec4 e1[NIT], e2[NIT];
 #pragma unroll
     for (int it = 0; it < NIT; ++it) {
@@ -208,8 +212,10 @@ __global__ __launch_bounds__(kPqBwdWaves * kWave) void dense_pq_backward_kernel(
           acc1[it][x] = b1;
           acc2[it][x] = b2;
         }
-        __builtin_nontemporal_store(ge1, pg + c);
-        if (MUL == 2) __builtin_nontemporal_store(ge2, pg + c + ncol);
+        if (!SHARED) {
+          __builtin_nontemporal_store(ge1, pg + c);
+          if (MUL == 2) __builtin_nontemporal_store(ge2, pg + c + ncol);
+        }
       }
     }
   }
@@ -234,6 +240,101 @@ __global__ __launch_bounds__(kPqBwdWaves * kWave) void dense_pq_backward_kernel(
   }
 }
 
+// Shared entity rows: gradient of row j = sum over the queries i of gout[i,j] * d term / d e.  One
+// workgroup per row, the row in registers; wavefront w takes queries w, w+8, ... in ascending order and
+// the eight partial sums are combined through LDS in wavefront order.
+template <int K, int NIT>
+__global__ __launch_bounds__(kPqBwdWaves * kWave) void dense_shared_entity_backward_kernel(
+    const float* __restrict__ gout, const float* __restrict__ ent, const float* __restrict__ q1,
+    const float* __restrict__ q2, float* __restrict__ gent, int bsize, int num, int dim) {
+  constexpr int MUL = kind_mul(K), NQ = kind_nq(K);
+  extern __shared__ float lds[];  // [waves][MUL][dim]
+  const int j = blockIdx.x;
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  const int ncol = dim / 4;
+  const size_t row_len = (size_t)dim * MUL;
+  const dvec4 zero = {0.f, 0.f, 0.f, 0.f};
+  dvec4 e1[NIT], e2[NIT], acc1[NIT], acc2[NIT];
+  const dvec4* pe = reinterpret_cast<const dvec4*>(ent + (size_t)j * row_len);
+#pragma unroll
+  for (int it = 0; it < NIT; ++it) {
+    const int c = min(lane + kWave * it, ncol - 1);
+    e1[it] = pe[c];
+    e2[it] = MUL == 2 ? pe[c + ncol] : zero;
+    acc1[it] = acc2[it] = zero;
+  }
+  for (int i = wave; i < bsize; i += kPqBwdWaves) {
+    const float g = gout[(size_t)i * num + j];
+    const dvec4* pa = reinterpret_cast<const dvec4*>(q1 + (size_t)i * dim);
+    const dvec4* pb = reinterpret_cast<const dvec4*>(q2 + (size_t)i * dim);
+    dvec4 qa[NIT], qb[NIT];
+#pragma unroll
+    for (int it = 0; it < NIT; ++it) {
+      const int c = min(lane + kWave * it, ncol - 1);
+      qa[it] = pa[c];
+      qb[it] = NQ == 2 ? pb[c] : zero;
+    }
+#pragma unroll
+    for (int it = 0; it < NIT; ++it) {
+#pragma unroll
+      for (int x = 0; x < 4; ++x) {
+        float a1 = acc1[it][x], a2 = acc2[it][x], s1 = 0.f, s2 = 0.f;
+        Term<K, float>::bwd(g, e1[it][x], e2[it][x], qa[it][x], qb[it][x], a1, a2, s1, s2);
+        acc1[it][x] = a1;
+        acc2[it][x] = a2;
+      }
+    }
+  }
+#pragma unroll
+  for (int it = 0; it < NIT; ++it) {
+    const int c = lane + kWave * it;
+    if (c < ncol) {
+      reinterpret_cast<dvec4*>(lds + (size_t)(wave * MUL + 0) * dim)[c] = acc1[it];
+      if (MUL == 2) reinterpret_cast<dvec4*>(lds + (size_t)(wave * MUL + 1) * dim)[c] = acc2[it];
+    }
+  }
+  __syncthreads();
+  for (int d = threadIdx.x; d < dim * MUL; d += kPqBwdWaves * kWave) {
+    const int h = d / dim, dd = d - h * dim;
+    float sum = 0.f;
+#pragma unroll
+    for (int w = 0; w < kPqBwdWaves; ++w) sum += lds[(size_t)(w * MUL + h) * dim + dd];
+    gent[(size_t)j * row_len + d] = sum;
+  }
+}
+
+// entity [1,N,.] shared by the queries [B,1,.]
+static bool shared_layout(const Layout& L, const void* a, const void* b, const void* c, const void* d, const void* e,
+                          const void* f, const void* g) {
+  if (L.be != 1 || L.bc != L.bsize || L.ne != L.num || L.nc != 1 || L.bsize < 2) return false;
+  if (L.dim % 4 != 0 || L.dim > 1024 || L.bsize * L.num > 0x7fffffffull) return false;
+  return aligned16(a) && aligned16(b) && aligned16(c) && aligned16(d) && aligned16(e) && aligned16(f) && aligned16(g);
+}
+
+template <int K>
+static int backward_shared(hipStream_t st, const float* gout, const float* ent, const float* q1, const float* q2,
+                           float* gent, float* gq1, float* gq2, const Layout& L) {
+  const dim3 block(kPqBwdWaves * kWave);
+  const int num = (int)L.num, dim = (int)L.dim, bsize = (int)L.bsize;
+  const size_t ncol = L.dim / 4;
+  const size_t lds_q = (size_t)kPqBwdWaves * kind_nq(K) * L.dim * sizeof(float);
+  const size_t lds_e = (size_t)kPqBwdWaves * kind_mul(K) * L.dim * sizeof(float);
+#define SMX_SHARED_LAUNCH(NIT_)                                                                                        \
+  hipLaunchKernelGGL((dense_pq_backward_kernel<K, NIT_, true>), dim3((unsigned)L.bsize), block, lds_q, st, gout, ent, q1, \
+                     q2, gent, gq1, gq2, num, dim);                                                                    \
+  hipLaunchKernelGGL((dense_shared_entity_backward_kernel<K, NIT_>), dim3((unsigned)L.num), block, lds_e, st, gout, ent,  \
+                     q1, q2, gent, bsize, num, dim);
+  if (ncol <= 64) {
+    SMX_SHARED_LAUNCH(1)
+  } else if (ncol <= 128) {
+    SMX_SHARED_LAUNCH(2)
+  } else {
+    SMX_SHARED_LAUNCH(4)
+  }
+#undef SMX_SHARED_LAUNCH
+  return check_launch("dist backward (shared entity rows)");
+}
+
 // entity [B,N,.] against query [B,1,.], float4-able, and small enough for the kernels above
 static bool pq_layout(const Layout& L, int kind, const void* a, const void* b, const void* c, const void* d,
                       const void* e, const void* f, const void* g) {
@@ -243,7 +344,7 @@ static bool pq_layout(const Layout& L, int kind, const void* a, const void* b, c
   return aligned16(a) && aligned16(b) && aligned16(c) && aligned16(d) && aligned16(e) && aligned16(f) && aligned16(g);
 }
 
-template <int K>
+template <int K, bool SHARED = false>
 static int forward_pq(hipStream_t st, const float* ent, const float* q1, const float* q2, float* dst, const Layout& L) {
   // enough workgroups to fill the chip, at least eight rows each when there are that many
   int rows_per_tile = (int)L.num;
@@ -251,7 +352,7 @@ static int forward_pq(hipStream_t st, const float* ent, const float* q1, const f
   const int tiles = (int)((L.num + rows_per_tile - 1) / rows_per_tile);
   if (L.bsize * (size_t)tiles > 0x7fffffffull) return -1;
   const size_t lds = (size_t)kind_nq(K) * L.dim * sizeof(float);
-  hipLaunchKernelGGL((dense_pq_forward_kernel<K>), dim3((unsigned)(L.bsize * tiles)), dim3(256), lds, st, ent, q1, q2, dst,
+  hipLaunchKernelGGL((dense_pq_forward_kernel<K, SHARED>), dim3((unsigned)(L.bsize * tiles)), dim3(256), lds, st, ent, q1, q2, dst,
                      (int)L.num, (int)L.dim, tiles, rows_per_tile);
   return check_launch("dist forward (per-query layout)");
 }
@@ -324,6 +425,17 @@ int dense_forward(int kind, void* stream, const T* ent, const T* q1, const T* q2
       }
     }
   }
+  if constexpr (std::is_same<T, float>::value) {
+    if (shared_layout(L, ent, q1, q2, dst, nullptr, nullptr, nullptr)) {
+      switch (kind) {
+#define X(KK) \
+  case KK:    \
+    return forward_pq<KK, true>(st, ent, q1, q2, dst, L);
+        SMX_FOR_EACH_KIND(X)
+#undef X
+      }
+    }
+  }
   switch (kind) {
 #define X(KK) \
   case KK:    \
@@ -349,6 +461,17 @@ int dense_backward(int kind, void* stream, const T* gout, const T* ent, const T*
 #define X(KK) \
   case KK:    \
     return backward_pq<KK>(st, gout, ent, q1, q2, gent, gq1, gq2, L);
+        SMX_FOR_EACH_KIND(X)
+#undef X
+      }
+    }
+  }
+  if constexpr (std::is_same<T, float>::value) {
+    if (shared_layout(L, gout, ent, q1, q2, gent, gq1, gq2)) {
+      switch (kind) {
+#define X(KK) \
+  case KK:    \
+    return backward_shared<KK>(st, gout, ent, q1, q2, gent, gq1, gq2, L);
         SMX_FOR_EACH_KIND(X)
 #undef X
       }
