@@ -205,9 +205,11 @@ class EmbeddingOptimizer(ABC):
                                             rec["gscore"], rec["params"], merged=merged, codes=rec["codes"])
                 idx_list.append(plan.uniq)
                 grad_list.append(merged)
-            flat = torch.cat(idx_list, dim=0)
+            # (a single record is used as it is: torch.cat would copy its gradient rows)
+            flat = idx_list[0] if len(idx_list) == 1 else torch.cat(idx_list, dim=0)
+            rows = grad_list[0] if len(grad_list) == 1 else torch.cat(grad_list, dim=0)
             plan = fused.build_plan(flat, n_rows, err_flag=self.err_flag)
-            self.update_from_plan(plan, torch.cat(grad_list, dim=0).contiguous(), lr)
+            self.update_from_plan(plan, rows.contiguous(), lr)
 
 
 class _RowOptimizer(EmbeddingOptimizer):
