@@ -252,10 +252,11 @@ __global__ __launch_bounds__(256) void gather_rows_kernel(const float* __restric
   }
   const size_t row_len = (size_t)ncol * VEC;
   for (int c = lane; c < ncol; c += 64) {
-    if (VEC == 4)
-      reinterpret_cast<float4*>(out + (size_t)k * row_len)[c] =
-          reinterpret_cast<const float4*>(table + (size_t)row * row_len)[c];
-    else
+    if (VEC == 4) {  // the copy is written once and read by a later kernel: non-temporal store
+      typedef float gvec4 __attribute__((ext_vector_type(4)));
+      __builtin_nontemporal_store(reinterpret_cast<const gvec4*>(table + (size_t)row * row_len)[c],
+                                  reinterpret_cast<gvec4*>(out + (size_t)k * row_len) + c);
+    } else
       out[(size_t)k * row_len + c] = table[(size_t)row * row_len + c];
   }
 }
