@@ -57,6 +57,34 @@ def test_dense_forward_backward(kind, layout, dtype):
             assert_close(g2.cpu().numpy(), o2, rel, f"{kind} gq2 dim={dim}")
 
 
+@pytest.mark.parametrize("kind", list(orc.KINDS))
+@pytest.mark.parametrize("layout", [(6, 9, 6, 1), (1, 11, 5, 1), (4, 1, 4, 1)])
+def test_long_rows_in_the_per_query_and_shared_layouts(kind, layout):
+    """Rows of two and four 256-float column groups (and one just past the vector kernels' 1024-float limit)
+    in the layouts that have their own fp32 kernels: per-query negatives, shared negatives, positives."""
+    from smore_amd import extlib_hip as ext
+    be, ne, bc, nc = layout
+    for dim in (260, 400, 516, 1000, 1024, 1028):
+        rng = np.random.default_rng(seed(kind, layout, dim))
+        e, q1, q2 = make_inputs(kind, be, ne, bc, nc, dim, rng)
+        bsize, num = max(be, bc), max(ne, nc)
+        gout = rng.standard_normal((bsize, num))
+        e, q1, gout = (x.astype(np.float32).astype(np.float64) for x in (e, q1, gout))
+        q2 = None if q2 is None else q2.astype(np.float32).astype(np.float64)
+        te, t1, t2, tg = (_dev(x, torch.float32) for x in (e, q1, q2, gout))
+        dst = torch.full((bsize, num), float("nan"), device="cuda")
+        ext.dist_forward(kind, te, t1, t2, dst, t2 is not None)
+        assert_close(dst.cpu().numpy(), orc.dist_forward(kind, e, q1, q2), REL_F32, f"{kind} fwd dim={dim}")
+        ge, g1 = torch.full_like(te, float("nan")), torch.full_like(t1, float("nan"))
+        g2 = None if t2 is None else torch.full_like(t2, float("nan"))
+        ext.dist_backward(kind, tg, te, t1, t2, ge, g1, g2, t2 is not None)
+        oe, o1, o2 = orc.dist_backward(kind, gout, e, q1, q2)
+        assert_close(ge.cpu().numpy(), oe, REL_F32, f"{kind} gent dim={dim}")
+        assert_close(g1.cpu().numpy(), o1, REL_F32, f"{kind} gq1 dim={dim}")
+        if t2 is not None:
+            assert_close(g2.cpu().numpy(), o2, REL_F32, f"{kind} gq2 dim={dim}")
+
+
 def test_tie_conventions_on_device():
     from smore_amd import extlib_hip as ext
     cases = [  # kind, e, c, o, expected (ge, gc, go) for gout = 2
