@@ -210,6 +210,44 @@ def test_union_branches_take_the_max_like_custom_cal_logit(model):
     assert np.abs(a[1]).sum() > 0
 
 
+def test_positives_as_column_zero_of_the_fused_call():
+    """One score_negatives call on [positive | negatives] ids gives both logit blocks and keeps apply_grad on
+    its one-record path; same logits, query gradients and table update as a plain positive lookup through
+    the dense operators plus a fused call for the negatives (two records merged into one Adam step)."""
+    from smore_amd.torchext import ext_ops
+    n, d, b, k, lr = 500, 32, 6, 17, 1e-3
+    rng = np.random.default_rng(21)
+    pos_n, neg_n = rng.integers(0, n, (b, 1)), rng.integers(0, n, (b, k))
+    neg_n[0, 0] = pos_n[0, 0]                       # an entity that is both a positive and a negative
+    cn = rng.uniform(-0.07, 0.07, (b, 1, d)).astype(np.float32)
+    on = np.abs(rng.uniform(-0.07, 0.07, (b, 1, d))).astype(np.float32)
+    gp, gn = rng.standard_normal((b, 1)).astype(np.float32), rng.standard_normal((b, k)).astype(np.float32)
+
+    def run(one_call):
+        emb, opt = _setup(n, d, 7)
+        c = torch.tensor(cn, device="cuda", requires_grad=True)
+        o = torch.tensor(on, device="cuda", requires_grad=True)
+        pos, neg = torch.tensor(pos_n, device="cuda"), torch.tensor(neg_n, device="cuda")
+        opt.zero_grad()
+        if one_call:
+            logits = opt.score_negatives("box", torch.cat([pos, neg], dim=1), c, o, gamma=24.0, cen=0.02)
+            lp, ln = logits[:, :1], logits[:, 1:]
+        else:
+            rp = emb(pos.view(-1), "positive_entity").unsqueeze(1)
+            lp = 24 - ext_ops.box_dist_out(rp, c, o) - 0.02 * ext_ops.box_dist_in(rp, c, o)
+            ln = opt.score_negatives("box", neg, c, o, gamma=24.0, cen=0.02)
+        ((lp * torch.tensor(gp, device="cuda")).sum() + (ln * torch.tensor(gn, device="cuda")).sum()).backward()
+        opt.apply_grad(lr)
+        opt.check_ids()
+        return [x.detach().cpu().numpy() for x in (lp, ln, c.grad, o.grad, emb.state_sum_fo, emb.state_sum_sq)] + \
+            [emb.embedding.detach().cpu().numpy()]
+
+    a, r = run(True), run(False)
+    for x, y, what in zip(a[:6], r[:6], ("positive logit", "negative logits", "center grad", "offset grad", "m", "v")):
+        assert_close(x, y, 5 * REL_F32, what)
+    assert np.abs(a[6] - r[6]).max() < 2 * lr
+
+
 def test_step_counter_and_empty_steps():
     emb, opt = _setup(50, 8, 7)
     opt.zero_grad()
