@@ -16,7 +16,8 @@
 // Per-query kernels (fp32, 16-byte aligned rows, entity [B,N,dim*mul] against query [B,1,dim]: the
 // layout of the models' negatives [B,K] and positives [B,1], kg_reasoning.py:342-355): the query lives
 // in LDS / registers, every entity row is read once with 16-byte loads, and the backward writes the
-// row gradient and accumulates the query gradient in the same pass.
+// row gradient and accumulates the query gradient in the same pass.  Shared negatives [1,N,.] and the
+// reverse layout (entity [B,1,.] against query [B,N,.]) have kernels of the same build.
 #include <type_traits>
 
 #include "smx_common.h"
@@ -335,6 +336,147 @@ static int backward_shared(hipStream_t st, const float* gout, const float* ent, 
   return check_launch("dist backward (shared entity rows)");
 }
 
+// ---- reverse layout, fp32: entity [B,1,.] against query [B,N,.] -------------------------------------
+// (inverse queries: the tail entity is projected back through the relations and compared with one query
+// row per candidate, kg_reasoning.py:252-263).  The mirror image of the per-query kernels: the entity row
+// is the one that stays (LDS / registers), the query rows stream by, the query gradient is per row and the
+// entity gradient is the sum over the rows.
+template <int K>
+__global__ __launch_bounds__(256) void dense_rev_forward_kernel(const float* __restrict__ ent, const float* __restrict__ q1,
+                                                                const float* __restrict__ q2, float* __restrict__ dst,
+                                                                int num, int dim, int tiles, int rows_per_tile) {
+  constexpr int MUL = kind_mul(K), NQ = kind_nq(K);
+  extern __shared__ float lds[];  // e1[dim] | e2[dim]
+  const int b = blockIdx.x / tiles, tile = blockIdx.x - b * tiles;
+  for (int d = threadIdx.x; d < dim * MUL; d += 256) lds[d] = ent[(size_t)b * dim * MUL + d];
+  __syncthreads();
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  const int ncol = dim / 4;
+  const int k1 = min(num, (tile + 1) * rows_per_tile);
+  const dvec4 zero = {0.f, 0.f, 0.f, 0.f};
+  for (int k = tile * rows_per_tile + wave; k < k1; k += 4) {
+    const size_t r = (size_t)b * num + k;
+    const dvec4* pa = reinterpret_cast<const dvec4*>(q1 + r * dim);
+    const dvec4* pb = reinterpret_cast<const dvec4*>(q2 + r * dim);
+    float sum = 0.f;
+    for (int c = lane; c < ncol; c += kWave) {
+      const dvec4 e1 = reinterpret_cast<const dvec4*>(lds)[c];
+      const dvec4 e2 = MUL == 2 ? reinterpret_cast<const dvec4*>(lds + dim)[c] : zero;
+      const dvec4 a = pa[c];
+      const dvec4 bq = NQ == 2 ? pb[c] : zero;
+#pragma unroll
+      for (int x = 0; x < 4; ++x) sum += Term<K, float>::fwd(e1[x], e2[x], a[x], bq[x]);
+    }
+    sum = wave_sum(sum);
+    if (lane == 0) dst[r] = sum;
+  }
+}
+
+template <int K, int NIT>
+__global__ __launch_bounds__(kPqBwdWaves * kWave) void dense_rev_backward_kernel(
+    const float* __restrict__ gout, const float* __restrict__ ent, const float* __restrict__ q1,
+    const float* __restrict__ q2, float* __restrict__ gent, float* __restrict__ gq1, float* __restrict__ gq2, int num,
+    int dim) {
+  constexpr int MUL = kind_mul(K), NQ = kind_nq(K);
+  extern __shared__ float lds[];  // [waves][MUL][dim]
+  const int b = blockIdx.x;
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  const int ncol = dim / 4;
+  const size_t row_len = (size_t)dim * MUL;
+  const dvec4 zero = {0.f, 0.f, 0.f, 0.f};
+  dvec4 e1[NIT], e2[NIT], acc1[NIT], acc2[NIT];
+  const dvec4* pe = reinterpret_cast<const dvec4*>(ent + (size_t)b * row_len);
+#pragma unroll
+  for (int it = 0; it < NIT; ++it) {
+    const int c = min(lane + kWave * it, ncol - 1);
+    e1[it] = pe[c];
+    e2[it] = MUL == 2 ? pe[c + ncol] : zero;
+    acc1[it] = acc2[it] = zero;
+  }
+  for (int k = wave; k < num; k += kPqBwdWaves) {
+    const size_t r = (size_t)b * num + k;
+    const float g = gout[r];
+    const dvec4* pa = reinterpret_cast<const dvec4*>(q1 + r * dim);
+    const dvec4* pb = reinterpret_cast<const dvec4*>(q2 + r * dim);
+    dvec4 qa[NIT], qb[NIT];
+#pragma unroll
+    for (int it = 0; it < NIT; ++it) {
+      const int c = min(lane + kWave * it, ncol - 1);
+      qa[it] = pa[c];
+      qb[it] = NQ == 2 ? pb[c] : zero;
+    }
+#pragma unroll
+    for (int it = 0; it < NIT; ++it) {
+      const int c = lane + kWave * it;
+      if (c < ncol) {
+        dvec4 g1 = zero, g2 = zero;
+#pragma unroll
+        for (int x = 0; x < 4; ++x) {
+          float a1 = acc1[it][x], a2 = acc2[it][x], s1 = 0.f, s2 = 0.f;
+          Term<K, float>::bwd(g, e1[it][x], e2[it][x], qa[it][x], qb[it][x], a1, a2, s1, s2);
+          acc1[it][x] = a1;
+          acc2[it][x] = a2;
+          g1[x] = s1;
+          g2[x] = s2;
+        }
+        __builtin_nontemporal_store(g1, reinterpret_cast<dvec4*>(gq1 + r * dim) + c);
+        if (NQ == 2) __builtin_nontemporal_store(g2, reinterpret_cast<dvec4*>(gq2 + r * dim) + c);
+      }
+    }
+  }
+#pragma unroll
+  for (int it = 0; it < NIT; ++it) {
+    const int c = lane + kWave * it;
+    if (c < ncol) {
+      reinterpret_cast<dvec4*>(lds + (size_t)(wave * MUL + 0) * dim)[c] = acc1[it];
+      if (MUL == 2) reinterpret_cast<dvec4*>(lds + (size_t)(wave * MUL + 1) * dim)[c] = acc2[it];
+    }
+  }
+  __syncthreads();
+  for (int d = threadIdx.x; d < dim * MUL; d += kPqBwdWaves * kWave) {
+    const int h = d / dim, dd = d - h * dim;
+    float sum = 0.f;
+#pragma unroll
+    for (int w = 0; w < kPqBwdWaves; ++w) sum += lds[(size_t)(w * MUL + h) * dim + dd];
+    gent[(size_t)b * row_len + d] = sum;
+  }
+}
+
+// entity [B,1,.] against query [B,N,.]
+static bool reverse_layout(const Layout& L, const void* a, const void* b, const void* c, const void* d, const void* e,
+                           const void* f, const void* g) {
+  if (L.be != L.bsize || L.bc != L.bsize || L.ne != 1 || L.nc != L.num || L.num < 2) return false;
+  if (L.dim % 4 != 0 || L.dim > 1024 || L.bsize * L.num > 0x7fffffffull) return false;
+  return aligned16(a) && aligned16(b) && aligned16(c) && aligned16(d) && aligned16(e) && aligned16(f) && aligned16(g);
+}
+
+template <int K>
+static int forward_rev(hipStream_t st, const float* ent, const float* q1, const float* q2, float* dst, const Layout& L) {
+  int rows_per_tile = (int)L.num;
+  while (rows_per_tile > 8 && L.bsize * ((L.num + rows_per_tile - 1) / rows_per_tile) < 8192) rows_per_tile = (rows_per_tile + 1) / 2;
+  const int tiles = (int)((L.num + rows_per_tile - 1) / rows_per_tile);
+  const size_t lds = (size_t)kind_mul(K) * L.dim * sizeof(float);
+  hipLaunchKernelGGL((dense_rev_forward_kernel<K>), dim3((unsigned)(L.bsize * tiles)), dim3(256), lds, st, ent, q1, q2, dst,
+                     (int)L.num, (int)L.dim, tiles, rows_per_tile);
+  return check_launch("dist forward (reverse layout)");
+}
+
+template <int K>
+static int backward_rev(hipStream_t st, const float* gout, const float* ent, const float* q1, const float* q2, float* gent,
+                        float* gq1, float* gq2, const Layout& L) {
+  const size_t lds = (size_t)kPqBwdWaves * kind_mul(K) * L.dim * sizeof(float);
+  const dim3 grid((unsigned)L.bsize), block(kPqBwdWaves * kWave);
+  const int num = (int)L.num, dim = (int)L.dim;
+  const size_t ncol = L.dim / 4;
+  if (ncol <= 64)
+    hipLaunchKernelGGL((dense_rev_backward_kernel<K, 1>), grid, block, lds, st, gout, ent, q1, q2, gent, gq1, gq2, num, dim);
+  else if (ncol <= 128)
+    hipLaunchKernelGGL((dense_rev_backward_kernel<K, 2>), grid, block, lds, st, gout, ent, q1, q2, gent, gq1, gq2, num, dim);
+  else
+    hipLaunchKernelGGL((dense_rev_backward_kernel<K, 4>), grid, block, lds, st, gout, ent, q1, q2, gent, gq1, gq2, num, dim);
+  return check_launch("dist backward (reverse layout)");
+}
+
 // entity [B,N,.] against query [B,1,.], float4-able, and small enough for the kernels above
 static bool pq_layout(const Layout& L, int kind, const void* a, const void* b, const void* c, const void* d,
                       const void* e, const void* f, const void* g) {
@@ -435,6 +577,15 @@ int dense_forward(int kind, void* stream, const T* ent, const T* q1, const T* q2
 #undef X
       }
     }
+    if (reverse_layout(L, ent, q1, q2, dst, nullptr, nullptr, nullptr)) {
+      switch (kind) {
+#define X(KK) \
+  case KK:    \
+    return forward_rev<KK>(st, ent, q1, q2, dst, L);
+        SMX_FOR_EACH_KIND(X)
+#undef X
+      }
+    }
   }
   switch (kind) {
 #define X(KK) \
@@ -472,6 +623,15 @@ int dense_backward(int kind, void* stream, const T* gout, const T* ent, const T*
 #define X(KK) \
   case KK:    \
     return backward_shared<KK>(st, gout, ent, q1, q2, gent, gq1, gq2, L);
+        SMX_FOR_EACH_KIND(X)
+#undef X
+      }
+    }
+    if (reverse_layout(L, gout, ent, q1, q2, gent, gq1, gq2)) {
+      switch (kind) {
+#define X(KK) \
+  case KK:    \
+    return backward_rev<KK>(st, gout, ent, q1, q2, gent, gq1, gq2, L);
         SMX_FOR_EACH_KIND(X)
 #undef X
       }

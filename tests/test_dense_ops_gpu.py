@@ -58,10 +58,10 @@ def test_dense_forward_backward(kind, layout, dtype):
 
 
 @pytest.mark.parametrize("kind", list(orc.KINDS))
-@pytest.mark.parametrize("layout", [(6, 9, 6, 1), (1, 11, 5, 1), (4, 1, 4, 1)])
+@pytest.mark.parametrize("layout", [(6, 9, 6, 1), (1, 11, 5, 1), (4, 1, 4, 1), (5, 1, 5, 10)])
 def test_long_rows_in_the_per_query_and_shared_layouts(kind, layout):
     """Rows of two and four 256-float column groups (and one just past the vector kernels' 1024-float limit)
-    in the layouts that have their own fp32 kernels: per-query negatives, shared negatives, positives."""
+    in the layouts that have their own fp32 kernels: per-query negatives, shared negatives, positives, reverse."""
     from smore_amd import extlib_hip as ext
     be, ne, bc, nc = layout
     for dim in (260, 400, 516, 1000, 1024, 1028):
