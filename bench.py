@@ -23,10 +23,10 @@ HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E bandwidth
 
 # Traffic of the backward call per launch in bytes (L2<->fabric, reads + writes), measured with two
 # `rocprofv3 --pmc` runs (FETCH_SIZE, WRITE_SIZE) and scaled by what the same counters read for a plain
-# row copy of known size (`bench.py --calibrate-copy`: FETCH_SIZE x1.942, WRITE_SIZE x1.000).  A counter
+# row copy of known size (`bench.py --calibrate-copy`: FETCH_SIZE x1.942, WRITE_SIZE x0.986).  A counter
 # cannot be read from inside this process, so the figures are those of the profile summary
 # pmc_traffic_<workload>.md kept with the other rocprofv3 summaries; workloads not profiled report null.
-MEASURED_BACKWARD_TRAFFIC = {"cfg5-box-adam-86m-zipf1.1": 4.84e9}
+MEASURED_BACKWARD_TRAFFIC = {"cfg5-box-adam-86m-zipf1.1": 4.82e9}
 
 CONFIGS = {
     1: dict(name="cfg1-l2-15k", model="l2", n=15_000, dim=200, b=512, k=128, r=0.07, gamma=12.0, cen=0.0,
