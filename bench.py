@@ -391,9 +391,12 @@ def main():
     }
     # what plain kernels sustain on this GPU for the step's access shapes, measured now with the library's
     # probes (after the timed region); a step that writes w, m, v back is a copy-like mix of reads and writes
-    out["measured_ceilings"] = measure_ceilings(device, 4 * row_len(cfg))
-    out["step_hbm"]["frac_of_measured_copy"] = out["step_hbm"]["achieved_GBps"] / out["measured_ceilings"]["copy_GBps"]
-    out["roofline"]["frac_of_measured_copy"] = ent_gbps / out["measured_ceilings"]["copy_GBps"]
+    try:
+        out["measured_ceilings"] = measure_ceilings(device, 4 * row_len(cfg))
+        out["step_hbm"]["frac_of_measured_copy"] = out["step_hbm"]["achieved_GBps"] / out["measured_ceilings"]["copy_GBps"]
+        out["roofline"]["frac_of_measured_copy"] = ent_gbps / out["measured_ceilings"]["copy_GBps"]
+    except torch.OutOfMemoryError:  # no room left for the two 4 GiB probe buffers: the step's figures stand alone
+        out["measured_ceilings"] = None
     del out["config"]["model"]
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(cfg, seed)
