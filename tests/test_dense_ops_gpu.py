@@ -85,6 +85,50 @@ def test_long_rows_in_the_per_query_and_shared_layouts(kind, layout):
             assert_close(g2.cpu().numpy(), o2, REL_F32, f"{kind} gq2 dim={dim}")
 
 
+def _random_layouts(count=48):
+    """Seeded random broadcast layouts (each axis equal, or one side a multiple of the other), dims on and
+    off the 16-byte path, both precisions: exercises the choice between the layout-specific and the general
+    kernels."""
+    rng = np.random.default_rng(77)
+    kinds = list(orc.KINDS)
+    cases = []
+    for i in range(count):
+        def pair():
+            a, m = int(rng.choice([1, 2, 3, 5, 8, 33])), int(rng.choice([1, 1, 2, 3]))
+            return (a, a * m) if rng.random() < 0.5 else (a * m, a)
+        (be, bc), (ne, nc) = pair(), pair()
+        dim = int(rng.choice([1, 3, 4, 16, 63, 64, 200, 257, 400, 1000]))
+        cases.append((kinds[i % len(kinds)], be, ne, bc, nc, dim, "f32" if i % 3 else "f64"))
+    return cases
+
+
+@pytest.mark.parametrize("case", _random_layouts(), ids=lambda c: "-".join(str(x) for x in c))
+def test_random_broadcast_layouts(case):
+    from smore_amd import extlib_hip as ext
+    kind, be, ne, bc, nc, dim, prec = case
+    dtype = torch.float32 if prec == "f32" else torch.float64
+    rng = np.random.default_rng(seed(*case))
+    e, q1, q2 = make_inputs(kind, be, ne, bc, nc, dim, rng)
+    bsize, num = max(be, bc), max(ne, nc)
+    gout = rng.standard_normal((bsize, num))
+    if dtype == torch.float32:
+        e, q1, gout = (x.astype(np.float32).astype(np.float64) for x in (e, q1, gout))
+        q2 = None if q2 is None else q2.astype(np.float32).astype(np.float64)
+    te, t1, t2, tg = (_dev(x, dtype) for x in (e, q1, q2, gout))
+    rel = REL_F32 if dtype == torch.float32 else (1e-9 if kind.startswith("beta") else REL_F64)
+    dst = torch.full((bsize, num), float("nan"), dtype=dtype, device="cuda")
+    ext.dist_forward(kind, te, t1, t2, dst, t2 is not None)
+    assert_close(dst.cpu().numpy(), orc.dist_forward(kind, e, q1, q2), rel, "forward")
+    ge, g1 = torch.full_like(te, float("nan")), torch.full_like(t1, float("nan"))
+    g2 = None if t2 is None else torch.full_like(t2, float("nan"))
+    ext.dist_backward(kind, tg, te, t1, t2, ge, g1, g2, t2 is not None)
+    oe, o1, o2 = orc.dist_backward(kind, gout, e, q1, q2)
+    assert_close(ge.cpu().numpy(), oe, 4 * rel, "gent")
+    assert_close(g1.cpu().numpy(), o1, 4 * rel, "gq1")
+    if t2 is not None:
+        assert_close(g2.cpu().numpy(), o2, 4 * rel, "gq2")
+
+
 def test_tie_conventions_on_device():
     from smore_amd import extlib_hip as ext
     cases = [  # kind, e, c, o, expected (ge, gc, go) for gout = 2
