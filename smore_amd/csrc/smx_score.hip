@@ -212,9 +212,13 @@ int smx_score_backward_entity(int model, void* stream, const smx_plan_view* plan
   // rows of a skewed or sparse id stream) go through the pair-ordered kernel on the caller's stream while
   // the entity pass reduces the others on the library's second stream -- the same division of work and
   // the same arithmetic per row as in smx_score_backward_fused, minus the query gradient.
-  const bool split = fwd_codes && adam && !merged && plan && plan->pair_seg && plan->uniq && score && gscore &&
+  // (everything the entity pass would refuse is checked here first, so that a refused call has not
+  // already updated the one-pair rows)
+  const bool split = fwd_codes && adam && !merged && plan && plan->pair_seg && plan->uniq && plan->order &&
+                     plan->sorted_ids && plan->seg_of_pos && plan->seg_start && plan->n_uniq && score && gscore &&
                      queries_beyond_l2(model, B, dim) && B * K >= ((size_t)1 << 20) && plan->n_pairs == B * K &&
-                     workspace && workspace_bytes >= entity_ws_bytes(B * K, dim * model_mul(model)) &&
+                     workspace && !(reinterpret_cast<uintptr_t>(workspace) & 255u) &&
+                     workspace_bytes >= entity_ws_bytes(B * K, dim * model_mul(model)) &&
                      !std::getenv("SMX_SERIAL_BACKWARD");
   if (split) {
     ScoreArgs A;
