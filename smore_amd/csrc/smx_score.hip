@@ -273,6 +273,14 @@ int smx_score_backward_fused(int model, void* stream, const smx_plan_view* plan,
   if (vec == 4 && v && !(adam && adam->squeeze) && !aligned16(v))
     return fail(SMX_ERR_ARG, "v must be 16-byte aligned like the table");
   if (!score || !gscore || !gq1 || (model_nq(model) == 2 && !gq2)) return fail(SMX_ERR_ARG, "null pointer");
+  // what the entity pass would refuse, before the query-gradient kernel has touched any row
+  if (!plan->order || !plan->sorted_ids || !plan->seg_of_pos || !plan->seg_start || !plan->uniq || !plan->n_uniq)
+    return fail(SMX_ERR_ARG, "incomplete segment plan");
+  if (!workspace || (reinterpret_cast<uintptr_t>(workspace) & 255u))
+    return fail(SMX_ERR_ARG, "workspace must be given and 256-byte aligned");
+  if (workspace_bytes < entity_ws_bytes(B * K, dim * model_mul(model)))
+    return fail(SMX_ERR_WORKSPACE, "fused workspace too small: %zu < %zu", workspace_bytes,
+                entity_ws_bytes(B * K, dim * model_mul(model)));
   A.score = score;
   A.gscore = gscore;
   A.gq1 = gq1;
