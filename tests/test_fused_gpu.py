@@ -68,9 +68,12 @@ def run_case(model, n, b, k, dim, zipf=None, cen=0.02, adam_steps=2, lr=1e-3):
     # query backward
     gq1, gq2 = fused.score_backward_query(model, t_table, t_idx, t_q1, t_q2, score, t_gs, params)
     o_rows, o_g1, o_g2 = orc.score_backward(model, gs, rows, o_q1, o_q2, cen)
-    assert_close(gq1.cpu().numpy(), o_g1[:, 0, :], REL_F32, f"{model} gq1")
+    # a query gradient is a sum over K signed terms of size <= |g_k| (unit-bounded derivatives of l1, l2, box,
+    # rotate): when it cancels, one fp32 ulp of sum |g_k| is the floor of any summation order
+    q_abs = None if model == "beta_kl" else np.abs(gs).sum(axis=1)[:, None] * np.ones((1, dim))
+    assert_close(gq1.cpu().numpy(), o_g1[:, 0, :], REL_F32, f"{model} gq1", sum_abs=q_abs)
     if q2 is not None:
-        assert_close(gq2.cpu().numpy(), o_g2[:, 0, :], REL_F32, f"{model} gq2")
+        assert_close(gq2.cpu().numpy(), o_g2[:, 0, :], REL_F32, f"{model} gq2", sum_abs=q_abs)
 
     # plan: integers are bit-exact
     plan = fused.build_plan(t_idx, n, want_inverse=True, err_flag=err)
