@@ -389,6 +389,16 @@ def main():
         },
         "phase_ms": phase_ms,
     }
+    if cfg["adam"] and step.codes is not None:
+        # the same backward with its kernels one after the other on one stream (the library's profiling
+        # switch): the figure the per-kernel durations of a rocprofv3 trace of that mode add up to
+        os.environ["SMX_SERIAL_BACKWARD"] = "1"
+        ev2 = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(5)]
+        for e in ev2:
+            step.run(e)
+        torch.cuda.synchronize()
+        del os.environ["SMX_SERIAL_BACKWARD"]
+        out["roofline"]["one_stream_avg_ms"] = sum(e[2].elapsed_time(e[3]) for e in ev2) / len(ev2)
     # what plain kernels sustain on this GPU for the step's access shapes, measured now with the library's
     # probes (after the timed region); a step that writes w, m, v back is a copy-like mix of reads and writes
     try:
