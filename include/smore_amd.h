@@ -262,6 +262,19 @@ int smx_sample_loss(void* stream, const float* pos, const float* neg, const floa
                     const float* weight, size_t B, size_t K, double temperature, double scale,
                     float* out_loss, float* gpos, float* gneg, void* workspace, size_t workspace_bytes);
 
+/* The same pass for callers that cannot allocate or pass a workspace: code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the reference.  The
+ * 2 B + 1 floats of scratch live in a static device array of the library (one copy per device, 512 KiB,
+ * held until the process ends); the call allocates nothing and gives the same bits as smx_sample_loss.
+ * At most SMX_SAMPLE_LOSS_STATIC_MAX_QUERIES queries per call (more: SMX_ERR_SHAPE).  Every call on
+ * a device shares that device's array: calls that overlap on one device (two streams, two threads)
+ * race; calls on one stream are ordered.  The first call on a device asks the runtime for the array's
+ * address (hipGetSymbolAddress), so make it before a stream capture begins. */
+#define SMX_SAMPLE_LOSS_STATIC_MAX_QUERIES 65536
+int smx_sample_loss_static(void* stream, const float* pos, const float* neg, const float* mask,
+                           const float* weight, size_t B, size_t K, double temperature, double scale,
+                           float* out_loss, float* gpos, float* gneg);
+
 /* ---- evaluation against all entities --------------------------------------------------------
  * Filtered ranks of a query's answers among all n_rows entities (the test_all branch of
  * smore/training/train_process.py:112-160: logits of every entity, argsort, ranks of easy + hard

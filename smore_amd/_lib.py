@@ -60,6 +60,8 @@ SIGNATURES = {
     "smx_sample_loss_workspace_bytes": (_sz, [_sz]),
     # stream, pos, neg, mask, weight, B, K, temperature, scale, out_loss, gpos, gneg, ws, ws_bytes
     "smx_sample_loss": (_i, [_vp, _vp, _vp, _vp, _vp, _sz, _sz, ctypes.c_double, ctypes.c_double, _vp, _vp, _vp, _vp, _sz]),
+    # stream, pos, neg, mask, weight, B, K, temperature, scale, out_loss, gpos, gneg
+    "smx_sample_loss_static": (_i, [_vp, _vp, _vp, _vp, _vp, _sz, _sz, ctypes.c_double, ctypes.c_double, _vp, _vp, _vp]),
     # stream, table, n_rows, row_len, idx, n, out, err
     "smx_gather_rows": (_i, [_vp, _vp, _sz, _sz, _vp, _sz, _vp, _vp]),
     "smx_rows_backward": (_i, [_vp, _vp, _vp, _sz, _vp, _vp, _vp, _vp, _vp, _vp, _sz]),

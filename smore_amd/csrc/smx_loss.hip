@@ -8,6 +8,7 @@
 // consumes -- autograd is not needed between the two.  One workgroup per query; every reduction has
 // a fixed order (DPP inside a wavefront, wavefront order across the workgroup, query order at the end).
 #include <cmath>
+#include <mutex>
 
 #include "smx_common.h"
 #include "smx_wave.h"
@@ -109,6 +110,55 @@ __global__ __launch_bounds__(256) void loss_finish_kernel(LossArgs A) {
 
 static size_t loss_ws_bytes(size_t B) { return ((2 * B + 1) * sizeof(float) + 255) & ~(size_t)255; }
 
+// Scratch of smx_sample_loss_static: the per-query partial losses and the weight sum that smx_sample_loss
+// keeps in the caller's workspace.  One copy per device, held until the process ends.
+constexpr size_t kStaticLossMaxB = SMX_SAMPLE_LOSS_STATIC_MAX_QUERIES;
+static __device__ __align__(256) float scratch[2 * kStaticLossMaxB + 64];
+
+// The array's name is a host-side stand-in: its device address is asked for once per device, with that
+// device current, and kept.
+static float* static_scratch() {
+  static std::mutex mu;
+  static float* per_device[64] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return nullptr;
+  std::lock_guard<std::mutex> lock(mu);
+  if (!per_device[dev]) {
+    float* ptr = nullptr;
+    if (hipGetSymbolAddress(reinterpret_cast<void**>(&ptr), HIP_SYMBOL(scratch)) != hipSuccess) return nullptr;
+    per_device[dev] = ptr;
+  }
+  return per_device[dev];
+}
+
+// Argument checks and launches shared by the two entry points; `buf` holds 2 B + 1 floats.
+static int launch_loss(void* stream, const float* pos, const float* neg, const float* mask, const float* weight,
+                       size_t B, size_t K, double temperature, double scale, float* out_loss, float* gpos, float* gneg,
+                       float* buf) {
+  if (!pos || !neg || !out_loss || !gpos || !gneg || !buf) return fail(SMX_ERR_ARG, "null pointer in sample loss");
+  if (B == 0 || K == 0 || B > 0x7fffffffull || K > 0x7fffffffull) return fail(SMX_ERR_SHAPE, "empty or oversized batch");
+  if (!(temperature >= 0.0)) return fail(SMX_ERR_ARG, "adversarial temperature must be >= 0 (0 = plain mean)");
+  LossArgs A{};
+  A.pos = pos;
+  A.neg = neg;
+  A.mask = mask;
+  A.weight = weight;
+  A.B = (int)B;
+  A.K = (int)K;
+  A.temperature = (float)temperature;
+  A.scale = (float)scale;
+  A.per_query = buf;
+  A.wsum = buf + 2 * B;
+  A.out_loss = out_loss;
+  A.gpos = gpos;
+  A.gneg = gneg;
+  hipStream_t st = as_stream(stream);
+  if (weight) hipLaunchKernelGGL(loss_weight_sum_kernel, dim3(1), dim3(256), 0, st, A);
+  hipLaunchKernelGGL(loss_rows_kernel, dim3((unsigned)B), dim3(256), 0, st, A);
+  hipLaunchKernelGGL(loss_finish_kernel, dim3(1), dim3(256), 0, st, A);
+  return check_launch("sample loss");
+}
+
 }  // namespace smx
 
 extern "C" {
@@ -119,30 +169,24 @@ int smx_sample_loss(void* stream, const float* pos, const float* neg, const floa
                     size_t B, size_t K, double temperature, double scale, float* out_loss, float* gpos, float* gneg,
                     void* workspace, size_t workspace_bytes) {
   using namespace smx;
-  if (!pos || !neg || !out_loss || !gpos || !gneg || !workspace) return fail(SMX_ERR_ARG, "null pointer in sample loss");
-  if (B == 0 || K == 0 || B > 0x7fffffffull || K > 0x7fffffffull) return fail(SMX_ERR_SHAPE, "empty or oversized batch");
-  if (!(temperature >= 0.0)) return fail(SMX_ERR_ARG, "adversarial temperature must be >= 0 (0 = plain mean)");
+  if (!workspace) return fail(SMX_ERR_ARG, "null pointer in sample loss");
   if (workspace_bytes < loss_ws_bytes(B))
     return fail(SMX_ERR_WORKSPACE, "loss workspace too small: %zu < %zu", workspace_bytes, loss_ws_bytes(B));
-  LossArgs A{};
-  A.pos = pos;
-  A.neg = neg;
-  A.mask = mask;
-  A.weight = weight;
-  A.B = (int)B;
-  A.K = (int)K;
-  A.temperature = (float)temperature;
-  A.scale = (float)scale;
-  A.per_query = static_cast<float*>(workspace);
-  A.wsum = A.per_query + 2 * B;
-  A.out_loss = out_loss;
-  A.gpos = gpos;
-  A.gneg = gneg;
-  hipStream_t st = as_stream(stream);
-  if (weight) hipLaunchKernelGGL(loss_weight_sum_kernel, dim3(1), dim3(256), 0, st, A);
-  hipLaunchKernelGGL(loss_rows_kernel, dim3((unsigned)B), dim3(256), 0, st, A);
-  hipLaunchKernelGGL(loss_finish_kernel, dim3(1), dim3(256), 0, st, A);
-  return check_launch("sample loss");
+  return launch_loss(stream, pos, neg, mask, weight, B, K, temperature, scale, out_loss, gpos, gneg,
+                     static_cast<float*>(workspace));
+}
+
+int smx_sample_loss_static(void* stream, const float* pos, const float* neg, const float* mask, const float* weight,
+                           size_t B, size_t K, double temperature, double scale, float* out_loss, float* gpos,
+                           float* gneg) {
+  using namespace smx;
+  if (B > kStaticLossMaxB)
+    return fail(SMX_ERR_SHAPE, "smx_sample_loss_static takes at most %zu queries per call, got %zu", kStaticLossMaxB, B);
+  float* buf = static_scratch();
+  if (!buf) return fail(SMX_ERR_HIP, "cannot get the device address of the library's scratch array");
+  // every float of the scratch this call reads (2 B partial losses, the weight sum when weights are given)
+  // is written by its own kernels first: nothing has to start at zero
+  return launch_loss(stream, pos, neg, mask, weight, B, K, temperature, scale, out_loss, gpos, gneg, buf);
 }
 
 }  // extern "C"
