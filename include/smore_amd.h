@@ -94,7 +94,9 @@ int smx_dist_backward_f64(int kind, void* stream, const double* gout, const doub
  * idx == NULL means `table` already holds the B*K rows in pair order (the
  * dense [B,K,row] layout of the reference operators).
  * An id outside [0, n_rows) sets *err_flag (device int, may be NULL) to 1 and
- * row 0 is read in its place; the caller decides when to look at the flag. */
+ * row 0 is read in its place for the score and the query gradient; the caller
+ * decides when to look at the flag.  No table row is ever updated for such a
+ * pair (see smx_plan_build). */
 typedef struct smx_score_params {
   float gamma;   /* margin: logit = gamma - distance */
   float cen;     /* BOX: weight of the inside distance */
@@ -146,7 +148,14 @@ int smx_score_backward_query(int model, void* stream, const float* table, size_t
  *                  id occurs once in the step), 0 otherwise; may be NULL
  *   n_uniq         device int: number of distinct ids
  * All arrays are caller-allocated device memory.  workspace: at least
- * smx_plan_workspace_bytes(P, n_rows) bytes, 256-byte aligned.  Needs n_rows <= 2^32. */
+ * smx_plan_workspace_bytes(P, n_rows) bytes (ask with the device current that the build will run on),
+ * 256-byte aligned.  Needs n_rows < 2^32.
+ * The build is kernel launches only (an LSD radix sort written for this shape, then one pass that numbers
+ * the segments): no library call, no memset, so it can be recorded into a HIP graph with the rest of a step.
+ * Ids outside [0, n_rows) set *err_flag = 1 and sort behind every valid id as one last segment that is not
+ * counted in n_uniq, is skipped by the entity pass and is never a one-pair segment: no row is updated for
+ * them (inverse[] holds n_uniq for such pairs).  *err_flag = 2: a workgroup of the sort gave up waiting for
+ * another one (bounded wait, never seen in practice); the plan must then not be used. */
 size_t smx_plan_workspace_bytes(size_t n_pairs, size_t n_rows);
 int smx_plan_build(void* stream, const int64_t* idx, size_t n_pairs, size_t n_rows, void* workspace,
                    size_t workspace_bytes, int32_t* order, int32_t* sorted_ids, int32_t* seg_of_pos,
@@ -185,7 +194,17 @@ typedef struct smx_opt_params {
   long step;
   int kind;     /* SMX_OPT_* */
   int squeeze;
+  /* NULL, or device memory with the two per-step constants smx_opt_step_consts() computes; the kernels
+   * then read them at run time instead of taking them from lr / step above.  A launch recorded into a
+   * HIP graph freezes its arguments: with this buffer (rewritten by the caller between replays) a
+   * captured step follows the learning-rate schedule and Adam's bias correction; without it every
+   * replay repeats the lr and step of the capture. */
+  const float* step_consts_dev;
 } smx_opt_params;
+
+/* out2[0] = -lr / (1 - beta1^step), out2[1] = 1 / sqrt(1 - beta2^step) for ADAM (embed_optimizer.py:241-249),
+ * { -lr, 1 } for the other kinds: the contents of smx_opt_params.step_consts_dev.  Host-only. */
+int smx_opt_step_consts(const smx_opt_params* opt, float* out2);
 
 /* ---- entity-side backward, segment sum and row update in one pass ----------
  * For every distinct id u of the plan: g[u,:] = sum over the pairs of segment u

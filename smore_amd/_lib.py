@@ -42,6 +42,7 @@ SIGNATURES = {
     # n_uniq, err
     "smx_plan_build": (_i, [_vp, _vp, _sz, _sz, _vp, _sz, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "smx_entity_workspace_bytes": (_sz, [_sz, _sz]),
+    "smx_opt_step_consts": (_i, [_vp, _vp]),
     "smx_fused_workspace_bytes": (_sz, [_i, _sz, _sz]),
     # model, stream, plan, table, n_rows, q1, q2, score, gscore, B, K, dim, params, merged, m, v, adam, ws, ws_bytes,
     # fwd_codes, bytes
@@ -78,7 +79,8 @@ OPT_KINDS = {"adam": 1, "sgd": 2, "adagrad": 3, "rmsprop": 4}
 
 class OptParams(ctypes.Structure):
     """smx_opt_params of include/smore_amd.h."""
-    _fields_ = [("lr", _d), ("beta1", _d), ("beta2", _d), ("eps", _d), ("step", _l), ("kind", _i), ("squeeze", _i)]
+    _fields_ = [("lr", _d), ("beta1", _d), ("beta2", _d), ("eps", _d), ("step", _l), ("kind", _i), ("squeeze", _i),
+                ("step_consts_dev", _vp)]
 
 
 class PlanView(ctypes.Structure):

@@ -108,6 +108,7 @@ static int fill_adam(EntityArgs* A, float* m, float* v, const smx_opt_params* op
     A->adam_on = opt->kind;
     A->squeeze = opt->squeeze ? 1 : 0;
     A->a = make_adam_consts(opt);
+    A->step_dev = opt->step_consts_dev;
   } else if (m || v) {
     return fail(SMX_ERR_ARG, "optimizer state given without optimizer parameters");
   }
@@ -119,6 +120,15 @@ static int fill_adam(EntityArgs* A, float* m, float* v, const smx_opt_params* op
 extern "C" {
 
 size_t smx_entity_workspace_bytes(size_t n_pairs, size_t row_len) { return smx::entity_ws_bytes(n_pairs, row_len); }
+
+int smx_opt_step_consts(const smx_opt_params* opt, float* out2) {
+  using namespace smx;
+  if (!opt || !out2) return fail(SMX_ERR_ARG, "null pointer");
+  if (opt->kind < SMX_OPT_ADAM || opt->kind > SMX_OPT_RMSPROP) return fail(SMX_ERR_ARG, "unknown optimizer kind");
+  if (opt->kind == SMX_OPT_ADAM && opt->step < 1) return fail(SMX_ERR_ARG, "Adam step counter starts at 1");
+  step_consts(opt, out2);
+  return SMX_OK;
+}
 
 size_t smx_fused_workspace_bytes(int model, size_t n_pairs, size_t dim) {
   using namespace smx;

@@ -238,6 +238,7 @@ __global__ __launch_bounds__(256) void entity_segment_kernel(EntityArgs A) {
   const int wave = uniform(threadIdx.x >> 6);
   const int n_waves = gridDim.x * 4;
   const int n_chunks = (A.n_pairs + 63) / 64;
+  const int n_valid = *A.n_uniq;  // a last segment beyond this one holds the pairs whose id is outside the table: skipped
 
   for (int chunk = blockIdx.x * 4 + wave; chunk < n_chunks; chunk += n_waves) {
     const int base = chunk * 64;
@@ -248,7 +249,8 @@ __global__ __launch_bounds__(256) void entity_segment_kernel(EntityArgs A) {
     const int my_s1 = A.seg_start[my_seg + 1];
     const int my_len = my_s1 - my_s0;
     unsigned long long todo =
-        __ballot(lane < n_here && my_s0 == pos && my_len <= A.short_max && !(A.skip_single && my_len == 1));
+        __ballot(lane < n_here && my_s0 == pos && my_len <= A.short_max && !(A.skip_single && my_len == 1) &&
+                 my_seg < n_valid);
     if (todo == 0ull) continue;
     const int my_id = A.sorted_ids[pos];
 
@@ -321,10 +323,11 @@ __global__ __launch_bounds__(256) void entity_tile_kernel(EntityArgs A) {
   const int p0 = t * A.tile;
   if (p0 >= A.n_pairs) return;  // whole wavefront leaves; no workgroup barrier is used below
   const int p1 = min(A.n_pairs, p0 + A.tile);
+  const int n_valid = *A.n_uniq;  // the segment of ids outside the table, if there is one, is number n_valid: skipped
   {  // does a long segment that came in from the left end inside this tile?  The fix-up pass finishes it.
     const int sg = A.seg_of_pos[p0];
     const int b0 = A.seg_start[sg], b1 = A.seg_start[sg + 1];
-    if (lane == 0) A.fix[t] = (p0 > 0 && b0 < p0 && b1 <= p1 && b1 - b0 > A.short_max) ? 1 : 0;
+    if (lane == 0) A.fix[t] = (p0 > 0 && b0 < p0 && b1 <= p1 && b1 - b0 > A.short_max && sg < n_valid) ? 1 : 0;
   }
 
   // most tiles hold short segments only: find that out with one parallel look and leave
@@ -332,7 +335,7 @@ __global__ __launch_bounds__(256) void entity_tile_kernel(EntityArgs A) {
   for (int base = p0; base < p1; base += 64) {
     const int q = min(base + lane, p1 - 1);
     const int sg = A.seg_of_pos[q];
-    any_long |= __ballot(A.seg_start[sg + 1] - A.seg_start[sg] > A.short_max) != 0ull;
+    any_long |= __ballot(A.seg_start[sg + 1] - A.seg_start[sg] > A.short_max && sg < n_valid) != 0ull;
   }
   if (!any_long) return;
 
@@ -341,7 +344,7 @@ __global__ __launch_bounds__(256) void entity_tile_kernel(EntityArgs A) {
     const int seg = A.seg_of_pos[pos];
     const int s0 = A.seg_start[seg], s1 = A.seg_start[seg + 1];
     const int end = min(s1, p1);
-    if (s1 - s0 > A.short_max) {
+    if (s1 - s0 > A.short_max && seg < n_valid) {
       const unsigned row_id = (unsigned)A.sorted_ids[pos];
       const bool whole = s0 >= p0 && s1 <= p1;
       RowState<MUL, VEC, NIT> st;

@@ -2,185 +2,656 @@
 //
 // Replaces merge_grad_indices (smore/common/embedding/embed_optimizer.py:39-42),
 // i.e. torch.unique(ids, return_inverse=True), which the reference runs on the
-// host CPU, with a device pipeline:
-//   keys  = (uint32) idx[p]                      narrow + range check
-//   sort  (key, p) by key                        LSD radix sort, stable, only the
-//                                                bits an id below n_rows can have
-//   count heads (key[p] != key[p-1]) per span of 2048 positions, prefix over the spans,
-//   emit  seg_of_pos, uniq, seg_start, inverse, n_uniq
-// The sort is stable, so inside a segment pairs stay in ascending pair order:
-// every later reduction over a segment has one fixed summation order.
+// host CPU, with a device pipeline of six kernel launches and nothing else (no
+// library sort, no memset: the whole build can be recorded into a HIP graph):
+//   hist    one read of the ids: range check, digit histograms of every radix pass per workgroup,
+//           zero fill of the tables the later kernels count in
+//   sum     digit counts of every pass over the whole input
+//   pass    x (key bits / digit bits): stable LSD radix pass over (id, pair) as one 64-bit element
+//   emit    segment heads, segment numbers, uniq, seg_start, inverse, pair_seg, n_uniq
+// The sort is written for this shape: keys are entity ids (only the bits an id below n_rows can
+// have are sorted, 27 for 86M rows = three 9-bit passes), the payload is the pair index and is
+// also the tie-break, so inside a segment pairs stay in ascending pair order and every later
+// reduction over a segment has one fixed summation order.
+//
+// A radix pass handles a tile of up to 16384 elements per workgroup of 1024 threads: elements are
+// kept in registers, ranked per wavefront with ballot matching (stable: lane order inside a round,
+// rounds in order, wavefronts in order), the tile's digit counts are published and the counts of
+// the tiles before it are read back ("look-back"; tiles take their number from a ticket counter,
+// so a tile only ever waits for tiles that are already running), the tile is reordered in LDS and
+// written out in digit runs.  Waiting is bounded: a tile that would wait too long gives up, marks
+// the plan invalid (*err_flag = 2) and every kernel still ends.
+//
+// An id outside [0, n_rows) sets *err_flag = 1 and gets the key n_rows: such pairs sort behind
+// every valid id, form a last segment of their own that is not counted in n_uniq and that the
+// entity pass skips, and are never marked as one-pair segments -- no table row is updated for them.
 #include <cstring>
-
-#include <rocprim/device/device_radix_sort.hpp>
-#include <rocprim/iterator/counting_iterator.hpp>
+#include <mutex>
 
 #include "smx_common.h"
 
 namespace smx {
 
-__global__ __launch_bounds__(256) void plan_keys_kernel(const long long* __restrict__ idx, unsigned* __restrict__ keys,
-                                                        int* __restrict__ pair_seg, int n, unsigned long long n_rows,
-                                                        int* err) {
-  const int p = blockIdx.x * blockDim.x + threadIdx.x;
-  if (p >= n) return;
-  if (pair_seg) pair_seg[p] = 0;  // "not alone"; the emit kernel overwrites the entries of one-pair segments
-  long long id = idx[p];
+constexpr int kSortMaxRounds = 16;          // elements per thread and tile
+constexpr int kSortMaxDigitBits = 10;
+constexpr int kGroup = 16;                  // look-back fan-in: tiles per group, groups per super-block, ...
+constexpr unsigned kReady = 0x80000000u;    // published words: flag | 31-bit count
+constexpr unsigned kCount = 0x7fffffffu;
+constexpr unsigned kSpinLimit = 1u << 22;   // polls before a waiting tile gives up
+constexpr int kAuxThreads = 1024;           // workgroup size of the hist, sum and emit kernels
+constexpr int kAuxWaves = kAuxThreads / 64;
+constexpr int kHistBlocks = 256;
+constexpr int kHistBatch = 8;               // ids a thread of the hist kernel requests at a time
+constexpr int kEmitIters = 16;              // sorted positions per thread of the emit kernel
+constexpr int kEmitTile = kAuxThreads * kEmitIters;
+constexpr int kEmitSuper = 256;             // emit tiles whose head counts one wavefront reads back at once
+
+__device__ __forceinline__ unsigned ld_agent(const unsigned* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void st_agent(unsigned* p, unsigned v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Waits until the word at p carries the ready flag; v is what was last read there.  Bounded: after
+// kSpinLimit polls the caller gets a ready word with count 0 and the plan is marked invalid.
+__device__ __forceinline__ unsigned wait_ready(const unsigned* p, unsigned v, unsigned* abort_flag, int* err) {
+  unsigned spins = 0;
+  while (!(v & kReady)) {
+    __builtin_amdgcn_s_sleep(1);
+    v = ld_agent(p);
+    if (++spins > kSpinLimit) {
+      st_agent(abort_flag, 1u);
+      if (err) *err = 2;
+      return kReady;
+    }
+  }
+  return v;
+}
+
+// Orders a wavefront's own LDS writes before its later LDS reads (other lanes' entries).
+__device__ __forceinline__ void wave_lds_fence() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// Exclusive prefix, in thread order, of one value per thread of a workgroup of NW wavefronts; *total
+// (may be null) gets the sum.  tmp: NW words of LDS.
+template <int NW>
+__device__ __forceinline__ unsigned block_excl_scan(unsigned v, unsigned* tmp, unsigned* total) {
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  unsigned inc = v;
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    const unsigned t = __shfl_up(inc, off);
+    if (lane >= off) inc += t;
+  }
+  __syncthreads();  // tmp may still be read from an earlier scan
+  if (lane == 63) tmp[w] = inc;
+  __syncthreads();
+  unsigned before = 0, all = 0;
+#pragma unroll
+  for (int i = 0; i < NW; ++i) {
+    const unsigned t = tmp[i];
+    before += i < w ? t : 0u;
+    all += t;
+  }
+  if (total) *total = all;
+  return before + inc - v;
+}
+
+__device__ __forceinline__ unsigned clamp_id(long long id, unsigned long long n_rows, int& bad) {
   if ((unsigned long long)id >= n_rows) {
-    if (err) *err = 1;
-    id = 0;
+    bad = 1;
+    return (unsigned)n_rows;
   }
-  keys[p] = (unsigned)id;
+  return (unsigned)id;
 }
 
-// Segment numbering without a device-wide scan primitive: every workgroup owns kPlanSpan consecutive
-// sorted positions.  plan_count counts the segment heads of each span, plan_offsets (one workgroup)
-// turns the counts into the number of the first segment of each span, and plan_emit recounts its span
-// with a running prefix and writes the plan.  No workgroup waits for another one.
-constexpr int kPlanIters = 8;
-constexpr int kPlanSpan = 256 * kPlanIters;
-
-__device__ __forceinline__ bool is_head(const int* __restrict__ sorted_ids, int p, int n) {
-  return p < n && (p == 0 || sorted_ids[p] != sorted_ids[p - 1]);
-}
-
-__global__ __launch_bounds__(256) void plan_count_kernel(const int* __restrict__ sorted_ids, int n,
-                                                         unsigned* __restrict__ span_heads) {
-  __shared__ unsigned per_wave[4];
-  const int base = blockIdx.x * kPlanSpan;
-  unsigned cnt = 0;
+// Lanes of the wavefront (among those of `live`) whose `bits`-bit digit equals this lane's: one ballot
+// per bit, combined with a three-input bit operation per half (same & ~(has ^ mine)).
+__device__ __forceinline__ unsigned long long match_digit(unsigned d, int bits, unsigned long long live) {
+  unsigned lo = (unsigned)live, hi = (unsigned)(live >> 32);
 #pragma unroll
-  for (int it = 0; it < kPlanIters; ++it)
-    cnt += (unsigned)__popcll(__ballot(is_head(sorted_ids, base + it * 256 + (int)threadIdx.x, n)));
-  if ((threadIdx.x & 63) == 0) per_wave[threadIdx.x >> 6] = cnt;
-  __syncthreads();
-  if (threadIdx.x == 0) span_heads[blockIdx.x] = per_wave[0] + per_wave[1] + per_wave[2] + per_wave[3];
-}
-
-// exclusive prefix of span_heads -> span_first; also the segment count and the end marker of seg_start
-__global__ __launch_bounds__(1024) void plan_offsets_kernel(const unsigned* __restrict__ span_heads,
-                                                            unsigned* __restrict__ span_first, int spans,
-                                                            int* __restrict__ n_uniq, int* __restrict__ seg_start, int n) {
-  __shared__ unsigned buf[1024];
-  __shared__ unsigned carry;
-  if (threadIdx.x == 0) carry = 0;
-  __syncthreads();
-  for (int base = 0; base < spans; base += 1024) {
-    const int i = base + (int)threadIdx.x;
-    const unsigned mine = i < spans ? span_heads[i] : 0u;
-    buf[threadIdx.x] = mine;
-    __syncthreads();
-    for (int step = 1; step < 1024; step <<= 1) {  // Hillis-Steele inclusive scan
-      const unsigned add = threadIdx.x >= (unsigned)step ? buf[threadIdx.x - step] : 0u;
-      __syncthreads();
-      buf[threadIdx.x] += add;
-      __syncthreads();
+  for (int b = 0; b < kSortMaxDigitBits; ++b) {
+    if (b < bits) {  // uniform
+      const unsigned mine = (unsigned)__builtin_amdgcn_sbfe((int)d, b, 1);  // 0 or ~0
+      const unsigned long long has = __ballot(mine != 0u);
+      lo = __builtin_amdgcn_bitop3_b32(lo, (unsigned)has, mine, 0x90);
+      hi = __builtin_amdgcn_bitop3_b32(hi, (unsigned)(has >> 32), mine, 0x90);
     }
-    if (i < spans) span_first[i] = carry + buf[threadIdx.x] - mine;
-    __syncthreads();
-    if (threadIdx.x == 1023) carry += buf[1023];
-    __syncthreads();
   }
-  if (threadIdx.x == 0) {
-    *n_uniq = (int)carry;
-    seg_start[carry] = n;
-  }
+  return ((unsigned long long)hi << 32) | lo;
+}
+__device__ __forceinline__ unsigned lanes_below(unsigned long long m) {
+  return __builtin_amdgcn_mbcnt_hi((unsigned)(m >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)m, 0u));
 }
 
-__global__ __launch_bounds__(256) void plan_emit_kernel(const int* __restrict__ sorted_ids, const int* __restrict__ order,
-                                                        const unsigned* __restrict__ span_first,
-                                                        int* __restrict__ seg_of_pos, long long* __restrict__ uniq,
-                                                        int* __restrict__ seg_start, long long* __restrict__ inverse,
-                                                        int* __restrict__ pair_seg, int n) {
-  __shared__ unsigned counts[kPlanIters][4];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int base = blockIdx.x * kPlanSpan;
-  bool head[kPlanIters];
-  unsigned below[kPlanIters];  // heads at lower lanes of this wavefront in the same iteration
-#pragma unroll
-  for (int it = 0; it < kPlanIters; ++it) {
-    head[it] = is_head(sorted_ids, base + it * 256 + (int)threadIdx.x, n);
-    const unsigned long long b = __ballot(head[it]);
-    below[it] = (unsigned)__popcll(b & ((1ull << lane) - 1ull));
-    if (lane == 0) counts[it][wave] = (unsigned)__popcll(b);
-  }
+// ---- hist -------------------------------------------------------------------------------------
+// block_hist[block][pass][digit]: how many ids of the block's share have that digit in that pass.
+// Ids are skewed (a few entities collect most pairs, and the high digits of small ids are all zero):
+// lanes that share the first lane's digit are counted with one LDS atomic for all of them.
+__global__ __launch_bounds__(kAuxThreads) void sort_hist_kernel(const long long* __restrict__ idx, int n,
+                                                                unsigned long long n_rows, int passes, int dbits,
+                                                                unsigned* __restrict__ block_hist,
+                                                                unsigned* __restrict__ zero_from, size_t zero_words,
+                                                                int* __restrict__ pair_seg, int* err) {
+  extern __shared__ unsigned lds_hist[];  // [passes][bins]
+  const int bins = 1 << dbits;
+  const unsigned mask = (unsigned)bins - 1u;
+  const int lane = threadIdx.x & 63;
+  for (int i = threadIdx.x; i < passes * bins; i += kAuxThreads) lds_hist[i] = 0;
+  for (size_t i = (size_t)blockIdx.x * kAuxThreads + threadIdx.x; i < zero_words; i += (size_t)gridDim.x * kAuxThreads)
+    zero_from[i] = 0;
   __syncthreads();
-  unsigned running = span_first[blockIdx.x];
+  int bad = 0;
+  const size_t span = (size_t)kAuxThreads * kHistBatch;
+  for (size_t base = (size_t)blockIdx.x * span; base < (size_t)n; base += (size_t)gridDim.x * span) {
+    long long id[kHistBatch];
 #pragma unroll
-  for (int it = 0; it < kPlanIters; ++it) {
-    unsigned before = running;
-#pragma unroll
-    for (int w = 0; w < 4; ++w) {
-      if (w < wave) before += counts[it][w];
-      running += counts[it][w];
+    for (int u = 0; u < kHistBatch; ++u) {  // all requests of the batch before the first use
+      const size_t p = base + (size_t)u * kAuxThreads + threadIdx.x;
+      id[u] = p < (size_t)n ? idx[p] : 0;
     }
-    const int p = base + it * 256 + (int)threadIdx.x;
-    if (p < n) {
-      const int seg = (int)(before + below[it] + (head[it] ? 1u : 0u)) - 1;
-      seg_of_pos[p] = seg;
-      if (head[it]) {
-        uniq[seg] = (long long)(unsigned)sorted_ids[p];
-        seg_start[seg] = p;
+#pragma unroll
+    for (int u = 0; u < kHistBatch; ++u) {
+      const size_t p = base + (size_t)u * kAuxThreads + threadIdx.x;
+      const bool valid = p < (size_t)n;
+      const unsigned key = clamp_id(id[u], n_rows, bad);
+      for (int s = 0; s < passes; ++s) {
+        const unsigned d = (key >> (s * dbits)) & mask;
+        const unsigned long long live = __ballot(valid);
+        if (live == 0ull) break;  // uniform
+        const unsigned d0 = (unsigned)__builtin_amdgcn_readlane((int)d, __builtin_ctzll(live));
+        const unsigned long long like_first = __ballot(valid && d == d0);
+        if (valid) {
+          if (d != d0) atomicAdd(&lds_hist[s * bins + d], 1u);
+          else if (lane == __builtin_ctzll(like_first)) atomicAdd(&lds_hist[s * bins + d], (unsigned)__popcll(like_first));
+        }
       }
-      if (inverse) inverse[order[p]] = seg;
-      if (pair_seg && head[it] && (p == n - 1 || sorted_ids[p + 1] != sorted_ids[p]))
-        pair_seg[order[p]] = seg | (int)0x80000000;  // this pair is its segment: sign bit + segment number
+      if (valid && pair_seg) pair_seg[p] = 0;  // "not alone"; the emit kernel overwrites the entries of one-pair segments
+    }
+  }
+  if (bad && err) *err = 1;
+  __syncthreads();
+  for (int i = threadIdx.x; i < passes * bins; i += kAuxThreads)
+    block_hist[(size_t)blockIdx.x * passes * bins + i] = lds_hist[i];
+}
+
+// digit_count[pass][digit] = sum over the hist workgroups; one workgroup per (pass, 64 digits), its
+// sixteen wavefronts share the hist workgroups among them, so every thread has a few independent loads.
+__global__ __launch_bounds__(kAuxThreads) void sort_sum_kernel(const unsigned* __restrict__ block_hist, int blocks,
+                                                               int passes, int dbits,
+                                                               unsigned* __restrict__ digit_count) {
+  __shared__ unsigned part[kAuxWaves][64];
+  const int bins = 1 << dbits;
+  const int groups = (bins + 63) / 64;
+  const int s = blockIdx.x / groups;
+  const int d = (blockIdx.x - s * groups) * 64 + (threadIdx.x & 63);
+  const int w = threadIdx.x >> 6;
+  unsigned sum = 0;
+  if (d < bins) {
+    for (int b0 = w; b0 < blocks; b0 += kAuxWaves * 8) {
+      unsigned v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int b = b0 + u * kAuxWaves;
+        v[u] = b < blocks ? block_hist[((size_t)b * passes + s) * bins + d] : 0u;
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) sum += v[u];
+    }
+  }
+  part[w][threadIdx.x & 63] = sum;
+  __syncthreads();
+  if (w == 0 && d < bins) {
+    unsigned all = 0;
+#pragma unroll
+    for (int i = 0; i < kAuxWaves; ++i) all += part[i][threadIdx.x];
+    digit_count[s * bins + d] = all;
+  }
+}
+
+// ---- one radix pass -----------------------------------------------------------------------------
+struct SortPassArgs {
+  const long long* idx;             // IN_IDX: the ids; the payload is the position
+  const unsigned long long* in;     // else: (key << 32 | payload) elements of the previous pass
+  unsigned long long* out;          // packed output, or
+  unsigned* out_keys;               // OUT_SPLIT: sorted ids and
+  int* out_vals;                    //            pair positions as two arrays
+  int n;
+  int rounds;                       // elements per thread; a tile has rounds * NW * 64 elements
+  int shift, dbits;
+  size_t stage_bytes;               // LDS bytes of the region shared by the per-wavefront counters and the staged tile
+  const unsigned* digit_count;      // [bins] of this pass: elements per digit in the whole input
+  // look-back tables, each word = ready flag | count per digit:
+  unsigned* level[3];               // [tiles / 16^l][bins], l = 0: one tile, 1: a group of 16 tiles, 2: 256 tiles
+  unsigned* pre;                    // [tiles / 4096][bins]: everything up to the end of a stretch of 4096 tiles
+  unsigned* ticket;
+  unsigned* abort_flag;
+  unsigned long long n_rows;
+  int* err;
+};
+
+// Digits are owned by threads: thread t owns digit t (and t + threads when there are more digits
+// than threads).
+template <int NW, int MAXR, bool IN_IDX, bool OUT_SPLIT>
+__global__ __launch_bounds__(NW * 64, (MAXR <= 8 ? 8 : 4)) void sort_pass_kernel(SortPassArgs A) {
+  constexpr int NT = NW * 64;
+  constexpr int PER = (1 << kSortMaxDigitBits) / NT > 1 ? (1 << kSortMaxDigitBits) / NT : 1;  // digits per thread, at most
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int bins = 1 << A.dbits;
+  const unsigned mask = (unsigned)bins - 1u;
+  unsigned* counters = reinterpret_cast<unsigned*>(smem);                     // [waves][bins] while ranking
+  unsigned long long* stage = reinterpret_cast<unsigned long long*>(smem);    // [tile] afterwards
+  unsigned* local_base = reinterpret_cast<unsigned*>(smem + A.stage_bytes);   // [bins]
+  unsigned* run_base = local_base + bins;                                     // [bins]
+  unsigned* tmp = run_base + bins;                                            // 32 words
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+  const int R = A.rounds;
+
+  if (tid == 0) tmp[20] = atomicAdd(A.ticket, 1u);
+  for (int d = lane; d < bins; d += 64) counters[w * bins + d] = 0;  // the wavefront's own row
+  __syncthreads();
+  const unsigned tile = tmp[20];
+  const size_t tile_base = (size_t)tile * R * NT;
+  const size_t wave_base = tile_base + (size_t)w * R * 64;
+  const size_t n = (size_t)A.n;
+
+  // 1. the tile's elements: wavefront w owns R * 64 consecutive ones, round r is 64 consecutive
+  unsigned long long e[MAXR];
+  int bad = 0;
+#pragma unroll
+  for (int r = 0; r < MAXR; ++r) {
+    e[r] = ~0ull;
+    if (r < R) {
+      const size_t pos = wave_base + (size_t)r * 64 + lane;
+      if (pos < n) {
+        if constexpr (IN_IDX)
+          e[r] = ((unsigned long long)clamp_id(A.idx[pos], A.n_rows, bad) << 32) | (unsigned)pos;
+        else
+          e[r] = A.in[pos];
+      }
+    }
+  }
+  (void)bad;  // the hist kernel has already reported ids outside the table
+
+  // 2. rank inside the wavefront: position among the wavefront's elements with the same digit
+  unsigned rank[MAXR];
+#pragma unroll
+  for (int r = 0; r < MAXR; ++r) {
+    rank[r] = 0;
+    if (r < R) {  // uniform
+      const bool valid = wave_base + (size_t)r * 64 + lane < n;
+      const unsigned d = ((unsigned)(e[r] >> 32) >> A.shift) & mask;
+      const unsigned long long same = match_digit(d, A.dbits, __ballot(valid));
+      const unsigned below = lanes_below(same);
+      unsigned prev = 0;
+      if (valid) prev = counters[w * bins + d];
+      wave_lds_fence();  // every lane has read before the first lane of each digit writes
+      if (valid && below == 0) counters[w * bins + d] = prev + (unsigned)__popcll(same);
+      wave_lds_fence();
+      rank[r] = prev + below;
+    }
+  }
+  __syncthreads();
+
+  // 3. per digit: the tile's count (published), and the wavefronts' rows turned into exclusive prefixes
+  unsigned mine[PER], lb[PER], db[PER];
+#pragma unroll
+  for (int u = 0; u < PER; ++u) {
+    const int d = tid + u * NT;
+    mine[u] = 0;
+    if (d < bins) {
+      unsigned run = 0;
+#pragma unroll
+      for (int ww = 0; ww < NW; ++ww) {
+        const unsigned t = counters[ww * bins + d];
+        counters[ww * bins + d] = run;
+        run += t;
+      }
+      mine[u] = run;
+      st_agent(&A.level[0][(size_t)tile * bins + d], run | kReady);
+    }
+  }
+  // position of a digit's first element inside the reordered tile, and in the whole output
+  {
+    unsigned carry_l = 0, carry_g = 0;
+#pragma unroll
+    for (int u = 0; u < PER; ++u) {  // digits [u * NT, (u + 1) * NT) in thread order
+      const int d = tid + u * NT;
+      unsigned tl = 0, tg = 0;
+      lb[u] = carry_l + block_excl_scan<NW>(mine[u], tmp, &tl);
+      db[u] = carry_g + block_excl_scan<NW>(d < bins ? A.digit_count[d] : 0u, tmp, &tg);
+      carry_l += tl;
+      carry_g += tg;
+    }
+  }
+
+  // 4. look-back: elements with a digit in the tiles before this one.  Tiles form groups of 16, groups
+  // form super-blocks of 16 groups, and so on: a thread fetches, per level, at most 15 independent words
+  // (the units of that level before its own inside the next-larger unit), and the last tile of a unit
+  // publishes the unit's total as soon as it has it.  Beyond 4096 tiles a chain of prefixes takes over.
+#pragma unroll
+  for (int u = 0; u < PER; ++u) {
+    const int d = tid + u * NT;
+    if (d < bins) {
+      unsigned before = 0;
+      unsigned unit = tile;  // my unit's number at this level
+#pragma unroll
+      for (int l = 0; l < 3; ++l) {
+        const unsigned first = unit & ~(unsigned)(kGroup - 1);
+        const unsigned* tab = A.level[l] + d;
+        unsigned v[kGroup - 1];
+#pragma unroll
+        for (int j = 0; j < kGroup - 1; ++j) v[j] = first + j < unit ? ld_agent(tab + (size_t)(first + j) * bins) : kReady;
+        unsigned here = 0;
+#pragma unroll
+        for (int j = 0; j < kGroup - 1; ++j) {
+          if (first + j < unit) v[j] = wait_ready(tab + (size_t)(first + j) * bins, v[j], A.abort_flag, A.err);
+          here += v[j] & kCount;
+        }
+        before += here;
+        // the last tile of a unit of the next level publishes that unit's total: everything before me
+        // inside it (levels up to here) plus my own count
+        const unsigned span = 1u << (4 * (l + 1));
+        if ((tile & (span - 1)) == span - 1) {
+          if (l < 2) st_agent(A.level[l + 1] + (size_t)(tile / span) * bins + d, ((before + mine[u]) & kCount) | kReady);
+        }
+        unit >>= 4;
+      }
+      if (tile >= 4096u) {
+        const unsigned* p = &A.pre[(size_t)(tile / 4096u - 1) * bins + d];
+        before += wait_ready(p, ld_agent(p), A.abort_flag, A.err) & kCount;
+      }
+      if ((tile & 4095u) == 4095u) st_agent(&A.pre[(size_t)(tile / 4096u) * bins + d], ((before + mine[u]) & kCount) | kReady);
+      local_base[d] = lb[u];
+      run_base[d] = db[u] + before - lb[u];  // + position in the reordered tile = global position
+    }
+  }
+  if (tid == 0) tmp[21] = ld_agent(A.abort_flag);
+  __syncthreads();
+  if (tmp[21]) return;  // a tile gave up waiting: positions are not trustworthy, write nothing
+
+  // 5. position of every element in the tile reordered by digit
+#pragma unroll
+  for (int r = 0; r < MAXR; ++r) {
+    if (r < R) {
+      const unsigned d = ((unsigned)(e[r] >> 32) >> A.shift) & mask;
+      if (wave_base + (size_t)r * 64 + lane < n) rank[r] += local_base[d] + counters[w * bins + d];
+    }
+  }
+  __syncthreads();  // the counters are dead: their LDS becomes the staged tile
+#pragma unroll
+  for (int r = 0; r < MAXR; ++r) {
+    if (r < R) {
+      if (wave_base + (size_t)r * 64 + lane < n) stage[rank[r]] = e[r];
+    }
+  }
+  __syncthreads();
+
+  // 6. write the tile out in digit runs
+  const size_t left = n - tile_base;  // tile_base < n: the grid has ceil(n / tile) tiles
+  const int here = (int)(left < (size_t)R * NT ? left : (size_t)R * NT);
+  for (int j = tid; j < here; j += NT) {
+    const unsigned long long el = stage[j];
+    const unsigned d = ((unsigned)(el >> 32) >> A.shift) & mask;
+    const unsigned pos = run_base[d] + (unsigned)j;
+    if constexpr (OUT_SPLIT) {
+      A.out_keys[pos] = (unsigned)(el >> 32);
+      A.out_vals[pos] = (int)(unsigned)el;
+    } else {
+      A.out[pos] = el;
     }
   }
 }
 
-static unsigned key_bits(size_t n_rows) {
+// ---- emit ---------------------------------------------------------------------------------------
+struct EmitArgs {
+  const unsigned* sorted_ids;
+  const int* order;
+  int n;
+  unsigned long long n_rows;
+  int* seg_of_pos;
+  long long* uniq;
+  int* seg_start;
+  long long* inverse;  // may be null
+  int* pair_seg;       // may be null
+  int* n_uniq;
+  unsigned* agg;       // [tiles]: ready flag | segment heads in the tile
+  unsigned* pre;       // [tiles / kEmitSuper]: ready flag | heads up to the end of a super-block
+  unsigned* ticket;
+  unsigned* abort_flag;
+  int* err;
+};
+
+// Consecutive lanes own consecutive sorted positions (kEmitIters rows of 1024 per tile).  Segment
+// numbers need the number of segment heads before the tile: look-back over the tiles' head counts as
+// in the radix passes, one value per tile, read by the first wavefront.
+__global__ __launch_bounds__(kAuxThreads) void plan_emit_kernel(EmitArgs A) {
+  __shared__ unsigned counts[kEmitIters * kAuxWaves];  // heads per (iteration, wavefront), then their exclusive prefix
+  __shared__ unsigned tmp[32];
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+  if (tid == 0) tmp[20] = atomicAdd(A.ticket, 1u);
+  __syncthreads();
+  const unsigned tile = tmp[20];
+  const long long n = A.n;
+  const long long base = (long long)tile * kEmitTile;
+
+  unsigned key[kEmitIters];
+  unsigned heads = 0, singles = 0;  // bit it: my position of iteration it starts a segment / is a whole segment
+  unsigned char below[kEmitIters];  // heads at lower lanes of my wavefront in the same iteration
+#pragma unroll
+  for (int it = 0; it < kEmitIters; ++it) {
+    const long long p = base + it * kAuxThreads + tid;
+    key[it] = p < n ? A.sorted_ids[p] : 0u;
+    const unsigned prev = (p > 0 && p < n) ? A.sorted_ids[p - 1] : 0u;
+    const unsigned next = p + 1 < n ? A.sorted_ids[p + 1] : 0u;
+    const bool head = p < n && (p == 0 || prev != key[it]);
+    const bool single = head && (p == n - 1 || next != key[it]) && (unsigned long long)key[it] < A.n_rows;
+    heads |= (head ? 1u : 0u) << it;
+    singles |= (single ? 1u : 0u) << it;
+    const unsigned long long b = __ballot(head);
+    below[it] = (unsigned char)lanes_below(b);
+    if (lane == 0) counts[it * kAuxWaves + w] = (unsigned)__popcll(b);
+  }
+  __syncthreads();
+  // exclusive prefix over the (iteration, wavefront) counts, in that order: 256 values, four per lane
+  if (w == 0) {
+    unsigned c[4], s = 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      c[i] = counts[lane * 4 + i];
+      s += c[i];
+    }
+    unsigned inc = s;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+      const unsigned t = __shfl_up(inc, off);
+      if (lane >= off) inc += t;
+    }
+    unsigned run = inc - s;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      counts[lane * 4 + i] = run;
+      run += c[i];
+    }
+    const unsigned total = (unsigned)__builtin_amdgcn_readlane((int)inc, 63);
+    if (lane == 0) st_agent(&A.agg[tile], total | kReady);
+
+    // look-back: heads in the tiles before this one
+    unsigned sum = 0;
+    const int first = (int)(tile & ~(unsigned)(kEmitSuper - 1));
+    unsigned v[kEmitSuper / 64];
+#pragma unroll
+    for (int u = 0; u < kEmitSuper / 64; ++u) {
+      const int j = (int)tile - 1 - lane - 64 * u;
+      v[u] = j >= first ? ld_agent(&A.agg[j]) : kReady;
+    }
+#pragma unroll
+    for (int u = 0; u < kEmitSuper / 64; ++u) {
+      const int j = (int)tile - 1 - lane - 64 * u;
+      if (j >= first) v[u] = wait_ready(&A.agg[j], v[u], A.abort_flag, A.err);
+      sum += v[u] & kCount;
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off);
+    if (lane == 0) {
+      if (first > 0) {
+        const unsigned* p = &A.pre[first / kEmitSuper - 1];
+        sum += wait_ready(p, ld_agent(p), A.abort_flag, A.err) & kCount;
+      }
+      if ((tile & (kEmitSuper - 1)) == kEmitSuper - 1) st_agent(&A.pre[tile / kEmitSuper], ((sum + total) & kCount) | kReady);
+      tmp[21] = sum;
+      tmp[22] = ld_agent(A.abort_flag);
+    }
+  }
+  __syncthreads();
+  if (tmp[22]) return;  // a tile gave up waiting: segment numbers are not trustworthy, write nothing
+  const unsigned first_seg = tmp[21];
+
+#pragma unroll
+  for (int it = 0; it < kEmitIters; ++it) {
+    const long long p = base + it * kAuxThreads + tid;
+    if (p < n) {
+      const bool head = (heads >> it) & 1u;
+      const int seg = (int)(first_seg + counts[it * kAuxWaves + w] + below[it] + (head ? 1u : 0u)) - 1;
+      A.seg_of_pos[p] = seg;
+      if (head) {
+        A.uniq[seg] = (long long)key[it];
+        A.seg_start[seg] = (int)p;
+      }
+      if (A.inverse) A.inverse[A.order[p]] = seg;
+      if (A.pair_seg && ((singles >> it) & 1u)) A.pair_seg[A.order[p]] = seg | (int)0x80000000;  // sign bit + segment number
+      if (p == n - 1) {  // the last position closes the list
+        A.seg_start[seg + 1] = (int)n;
+        *A.n_uniq = seg + 1 - ((unsigned long long)key[it] >= A.n_rows ? 1 : 0);  // ids outside the table are not counted
+      }
+    }
+  }
+}
+
+// ---- host side ----------------------------------------------------------------------------------
+static unsigned key_bits(size_t n_values) {
   unsigned bits = 1;
-  while (bits < 32 && (1ull << bits) < n_rows) ++bits;
+  while (bits < 32 && (1ull << bits) < n_values) ++bits;
   return bits;
 }
 
-// rocPRIM ships no tuned radix-sort configuration for gfx950 and falls back to 8-bit digits; measured
-// on MI355X, one-sweep passes over 9-bit digits (10-bit when that saves a whole pass) sort the plan's
-// (id, pair) list 1.2-2.4x faster: 27-bit ids of 4M pairs in 3 passes instead of 4, 20-bit ids in 2.
-// Above 4096 pairs the one-sweep path is used instead of rocPRIM's merge sort (its default up to 1M).
-using Sort9 = rocprim::radix_sort_config<
-    rocprim::default_config, rocprim::default_config,
-    rocprim::radix_sort_onesweep_config<rocprim::kernel_config<1024, 8>, rocprim::kernel_config<1024, 8>, 9,
-                                        rocprim::block_radix_rank_algorithm::match>,
-    4096>;
-using Sort10 = rocprim::radix_sort_config<
-    rocprim::default_config, rocprim::default_config,
-    rocprim::radix_sort_onesweep_config<rocprim::kernel_config<1024, 4>, rocprim::kernel_config<1024, 4>, 10,
-                                        rocprim::block_radix_rank_algorithm::match>,
-    4096>;
-
-static bool ten_bit_digits(unsigned bits) { return (bits + 9) / 10 < (bits + 8) / 9; }
-
-static hipError_t sort_pairs(void* temp, size_t& temp_bytes, unsigned* keys, unsigned* keys_out, int* order, size_t n,
-                             unsigned bits, hipStream_t st) {
-  if (ten_bit_digits(bits))
-    return rocprim::radix_sort_pairs<Sort10>(temp, temp_bytes, keys, keys_out, rocprim::counting_iterator<int>(0), order,
-                                             n, 0, bits, st);
-  return rocprim::radix_sort_pairs<Sort9>(temp, temp_bytes, keys, keys_out, rocprim::counting_iterator<int>(0), order, n,
-                                          0, bits, st);
+// LDS bytes a workgroup may use on the current device (gfx950: 160 KiB); 64 KiB when it cannot be asked.
+static size_t lds_limit() {
+  static std::mutex mu;
+  static size_t per_device[64] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 64 * 1024;
+  std::lock_guard<std::mutex> lock(mu);
+  if (!per_device[dev]) {
+    int v = 0;
+    if (hipDeviceGetAttribute(&v, hipDeviceAttributeMaxSharedMemoryPerBlock, dev) != hipSuccess || v <= 0) v = 64 * 1024;
+    per_device[dev] = (size_t)v;
+  }
+  return per_device[dev];
 }
 
-struct PlanScratch {
-  size_t keys_off, heads_off, first_off, temp_off, temp_bytes, total;
-  int spans;
+// Wavefronts per workgroup of the radix passes.  Measured on MI355X (4M pairs, 27-bit ids): 16 wavefronts
+// with 16 elements per thread, one workgroup per CU, 36 us per pass; smaller workgroups or tiles are
+// slower (47-56 us), the cost per tile being dominated by the look-back and the workgroup-wide steps.
+constexpr int kSortWaves = 16;
+
+struct PlanLayout {
+  int passes, dbits, bins, nw, rounds, tiles, units[3], chain, hist_blocks, emit_tiles, emit_supers;
+  size_t stage_bytes, pass_lds;
+  size_t a_off, b_off, bh_off, count_off, zero_off, zero_words, total;
+  // inside the zeroed region (in words from zero_off)
+  size_t level_w[3], pre_w, eagg_w, epre_w, ticket_w, abort_w;
 };
 
-static hipError_t plan_scratch(size_t n, size_t n_rows, PlanScratch* s) {
-  size_t sort_bytes = 0;
-  unsigned* kp = nullptr;
-  int* ip = nullptr;
-  hipError_t e = sort_pairs(nullptr, sort_bytes, kp, kp, ip, n, key_bits(n_rows), (hipStream_t)0);
-  if (e != hipSuccess) return e;
+static PlanLayout plan_layout(size_t n, size_t n_rows) {
   auto up = [](size_t x) { return (x + 255) & ~(size_t)255; };
-  s->spans = (int)((n + kPlanSpan - 1) / kPlanSpan);
-  s->keys_off = 0;
-  s->heads_off = up(n * sizeof(unsigned));
-  s->first_off = s->heads_off + up((size_t)s->spans * sizeof(unsigned));
-  s->temp_off = s->first_off + up((size_t)s->spans * sizeof(unsigned));
-  s->temp_bytes = up(sort_bytes);
-  s->total = s->temp_off + s->temp_bytes;
-  return hipSuccess;
+  PlanLayout L{};
+  const unsigned bits = key_bits(n_rows + 1);  // + the key of ids outside the table
+  L.passes = (int)((bits + kSortMaxDigitBits - 1) / kSortMaxDigitBits);
+  L.dbits = (int)((bits + L.passes - 1) / L.passes);
+  L.bins = 1 << L.dbits;
+  L.nw = kSortWaves;
+  const size_t nt = (size_t)L.nw * 64;
+  // elements per thread: enough tiles to fill the chip (one workgroup per CU), tiles as large as the LDS allows
+  const size_t fixed_lds = (size_t)(2 * L.bins + 32) * sizeof(unsigned);
+  const size_t counters = (size_t)L.nw * L.bins * sizeof(unsigned);
+  const size_t per_cu = 16 / (size_t)L.nw;  // workgroups that share a CU's LDS
+  size_t max_rounds = (lds_limit() / per_cu - fixed_lds - 1024) / (nt * 8);
+  if (max_rounds > (size_t)kSortMaxRounds) max_rounds = kSortMaxRounds;
+  if (max_rounds < 1) max_rounds = 1;
+  size_t rounds = (n + nt * 256 * per_cu - 1) / (nt * 256 * per_cu);
+  if (rounds < 1) rounds = 1;
+  if (rounds > max_rounds) rounds = max_rounds;
+  L.rounds = (int)rounds;
+  const size_t tile = rounds * nt;
+  L.tiles = (int)((n + tile - 1) / tile);
+  L.units[0] = L.tiles;
+  L.units[1] = (L.tiles + kGroup - 1) / kGroup;
+  L.units[2] = (L.units[1] + kGroup - 1) / kGroup;
+  L.chain = (L.tiles + 4095) / 4096;
+  L.stage_bytes = tile * 8 > counters ? tile * 8 : counters;
+  L.pass_lds = L.stage_bytes + fixed_lds;
+  L.hist_blocks = (int)((n + (size_t)kAuxThreads * kHistBatch - 1) / ((size_t)kAuxThreads * kHistBatch));
+  if (L.hist_blocks > kHistBlocks) L.hist_blocks = kHistBlocks;
+  L.emit_tiles = (int)((n + kEmitTile - 1) / kEmitTile);
+  L.emit_supers = (L.emit_tiles + kEmitSuper - 1) / kEmitSuper;
+  L.a_off = 0;
+  L.b_off = up(n * 8);
+  L.bh_off = L.b_off + (L.passes > 2 ? up(n * 8) : 0);
+  L.count_off = L.bh_off + up((size_t)L.hist_blocks * L.passes * L.bins * 4);
+  L.zero_off = L.count_off + up((size_t)L.passes * L.bins * 4);
+  size_t wds = 0;
+  for (int l = 0; l < 3; ++l) {
+    L.level_w[l] = wds;
+    wds += (size_t)L.passes * L.units[l] * L.bins;
+  }
+  L.pre_w = wds;    wds += (size_t)L.passes * L.chain * L.bins;
+  L.eagg_w = wds;   wds += (size_t)L.emit_tiles;
+  L.epre_w = wds;   wds += (size_t)L.emit_supers;
+  L.ticket_w = wds; wds += (size_t)L.passes + 1;
+  L.abort_w = wds;  wds += 1;
+  L.zero_words = wds;
+  L.total = L.zero_off + up(wds * 4);
+  return L;
+}
+
+template <int NW, int MAXR, bool IN_IDX, bool OUT_SPLIT>
+static void launch_pass(hipStream_t st, const PlanLayout& L, const SortPassArgs& A) {
+  auto kernel = sort_pass_kernel<NW, MAXR, IN_IDX, OUT_SPLIT>;
+  // More than 64 KiB of dynamic LDS: said once per kernel and device (not again under a later stream
+  // capture); a runtime that does not know the attribute leaves it to the launch to accept or refuse the size.
+  if (L.pass_lds > 64 * 1024) {
+    static std::mutex mu;
+    static bool told[64] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < 64) {
+      std::lock_guard<std::mutex> lock(mu);
+      if (!told[dev]) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  (int)lds_limit());
+        (void)hipGetLastError();
+        told[dev] = true;
+      }
+    }
+  }
+  hipLaunchKernelGGL(kernel, dim3((unsigned)L.tiles), dim3(NW * 64), L.pass_lds, st, A);
+}
+
+template <int NW, int MAXR>
+static void launch_pass_r(hipStream_t st, const PlanLayout& L, const SortPassArgs& A, bool first, bool last) {
+  if (first && last) launch_pass<NW, MAXR, true, true>(st, L, A);
+  else if (first) launch_pass<NW, MAXR, true, false>(st, L, A);
+  else if (last) launch_pass<NW, MAXR, false, true>(st, L, A);
+  else launch_pass<NW, MAXR, false, false>(st, L, A);
+}
+template <int NW>
+static void launch_pass_nw(hipStream_t st, const PlanLayout& L, const SortPassArgs& A, bool first, bool last) {
+  if (L.rounds <= 8) launch_pass_r<NW, 8>(st, L, A, first, last);
+  else launch_pass_r<NW, 16>(st, L, A, first, last);
 }
 
 }  // namespace smx
@@ -188,10 +659,9 @@ static hipError_t plan_scratch(size_t n, size_t n_rows, PlanScratch* s) {
 extern "C" {
 
 size_t smx_plan_workspace_bytes(size_t n_pairs, size_t n_rows) {
-  smx::PlanScratch s;
   if (n_pairs == 0) return 256;
-  if (smx::plan_scratch(n_pairs, n_rows, &s) != hipSuccess) return 0;
-  return s.total;
+  if (n_pairs > 0x7fffffffull || n_rows == 0 || n_rows > 0xffffffffull) return 0;
+  return smx::plan_layout(n_pairs, n_rows).total;
 }
 
 int smx_plan_build(void* stream, const int64_t* idx, size_t n_pairs, size_t n_rows, void* workspace,
@@ -201,34 +671,71 @@ int smx_plan_build(void* stream, const int64_t* idx, size_t n_pairs, size_t n_ro
   if (!idx || !order || !sorted_ids || !seg_of_pos || !uniq || !seg_start || !n_uniq || !workspace)
     return fail(SMX_ERR_ARG, "null pointer in plan build");
   if (n_pairs == 0 || n_pairs > 0x7fffffffull) return fail(SMX_ERR_SHAPE, "pair count %zu out of range", n_pairs);
-  if (n_rows == 0 || n_rows > 0x100000000ull) return fail(SMX_ERR_SHAPE, "entity count %zu needs ids wider than 32 bits", n_rows);
-  PlanScratch s;
-  if (plan_scratch(n_pairs, n_rows, &s) != hipSuccess) return fail(SMX_ERR_HIP, "rocprim size query failed");
-  if (workspace_bytes < s.total)
-    return fail(SMX_ERR_WORKSPACE, "plan workspace too small: %zu < %zu", workspace_bytes, s.total);
+  if (n_rows == 0 || n_rows > 0xffffffffull) return fail(SMX_ERR_SHAPE, "entity count %zu needs ids wider than 32 bits", n_rows);
+  const PlanLayout L = plan_layout(n_pairs, n_rows);
+  if (workspace_bytes < L.total)
+    return fail(SMX_ERR_WORKSPACE, "plan workspace too small: %zu < %zu", workspace_bytes, L.total);
   if (reinterpret_cast<uintptr_t>(workspace) & 255u) return fail(SMX_ERR_ARG, "workspace must be 256-byte aligned");
+  if (L.pass_lds > lds_limit())
+    return fail(SMX_ERR_HIP, "a radix pass needs %zu bytes of LDS per workgroup, the device allows %zu", L.pass_lds, lds_limit());
   hipStream_t st = as_stream(stream);
   char* ws = static_cast<char*>(workspace);
-  unsigned* keys = reinterpret_cast<unsigned*>(ws + s.keys_off);
-  unsigned* span_heads = reinterpret_cast<unsigned*>(ws + s.heads_off);
-  unsigned* span_first = reinterpret_cast<unsigned*>(ws + s.first_off);
-  void* temp = ws + s.temp_off;
+  unsigned long long* buf_a = reinterpret_cast<unsigned long long*>(ws + L.a_off);
+  unsigned long long* buf_b = reinterpret_cast<unsigned long long*>(ws + L.b_off);
+  unsigned* block_hist = reinterpret_cast<unsigned*>(ws + L.bh_off);
+  unsigned* digit_count = reinterpret_cast<unsigned*>(ws + L.count_off);
+  unsigned* zeroed = reinterpret_cast<unsigned*>(ws + L.zero_off);
   const int n = (int)n_pairs;
-  const unsigned blocks = (unsigned)((n_pairs + 255) / 256);
 
-  hipLaunchKernelGGL(plan_keys_kernel, dim3(blocks), dim3(256), 0, st, reinterpret_cast<const long long*>(idx), keys,
-                     pair_seg, n, (unsigned long long)n_rows, err_flag);
-  size_t tb = s.temp_bytes;
-  hipError_t e = sort_pairs(temp, tb, keys, reinterpret_cast<unsigned*>(sorted_ids), order, n_pairs, key_bits(n_rows), st);
-  if (e != hipSuccess) return fail(SMX_ERR_HIP, "radix sort: %s", hipGetErrorString(e));
-  hipLaunchKernelGGL(plan_count_kernel, dim3((unsigned)s.spans), dim3(256), 0, st, sorted_ids, n, span_heads);
-  hipLaunchKernelGGL(plan_offsets_kernel, dim3(1), dim3(1024), 0, st, span_heads, span_first, s.spans, n_uniq, seg_start,
-                     n);
-  hipLaunchKernelGGL(plan_emit_kernel, dim3((unsigned)s.spans), dim3(256), 0, st, sorted_ids, order, span_first,
-                     seg_of_pos, reinterpret_cast<long long*>(uniq), seg_start, reinterpret_cast<long long*>(inverse),
-                     pair_seg, n);
+  hipLaunchKernelGGL(sort_hist_kernel, dim3((unsigned)L.hist_blocks), dim3(kAuxThreads),
+                     (size_t)L.passes * L.bins * sizeof(unsigned), st, reinterpret_cast<const long long*>(idx), n,
+                     (unsigned long long)n_rows, L.passes, L.dbits, block_hist, zeroed, L.zero_words, pair_seg, err_flag);
+  hipLaunchKernelGGL(sort_sum_kernel, dim3((unsigned)(L.passes * ((L.bins + 63) / 64))), dim3(kAuxThreads), 0, st, block_hist,
+                     L.hist_blocks, L.passes, L.dbits, digit_count);
+  for (int s = 0; s < L.passes; ++s) {
+    SortPassArgs A{};
+    const bool first = s == 0, last = s == L.passes - 1;
+    // the packed buffers are used in turn; the last pass writes the plan's two arrays
+    A.idx = reinterpret_cast<const long long*>(idx);
+    A.in = (s % 2 == 1) ? buf_a : buf_b;
+    A.out = (s % 2 == 0) ? buf_a : buf_b;
+    A.out_keys = reinterpret_cast<unsigned*>(sorted_ids);
+    A.out_vals = order;
+    A.n = n;
+    A.rounds = L.rounds;
+    A.shift = s * L.dbits;
+    A.dbits = L.dbits;
+    A.stage_bytes = L.stage_bytes;
+    A.digit_count = digit_count + (size_t)s * L.bins;
+    for (int l = 0; l < 3; ++l) A.level[l] = zeroed + L.level_w[l] + (size_t)s * L.units[l] * L.bins;
+    A.pre = zeroed + L.pre_w + (size_t)s * L.chain * L.bins;
+    A.ticket = zeroed + L.ticket_w + s;
+    A.abort_flag = zeroed + L.abort_w;
+    A.n_rows = (unsigned long long)n_rows;
+    A.err = err_flag;
+    launch_pass_nw<kSortWaves>(st, L, A, first, last);
+    if (int rc = check_launch("radix pass")) return rc;
+  }
+  EmitArgs E{};
+  E.sorted_ids = reinterpret_cast<const unsigned*>(sorted_ids);
+  E.order = order;
+  E.n = n;
+  E.n_rows = (unsigned long long)n_rows;
+  E.seg_of_pos = seg_of_pos;
+  E.uniq = reinterpret_cast<long long*>(uniq);
+  E.seg_start = seg_start;
+  E.inverse = reinterpret_cast<long long*>(inverse);
+  E.pair_seg = pair_seg;
+  E.n_uniq = n_uniq;
+  E.agg = zeroed + L.eagg_w;
+  E.pre = zeroed + L.epre_w;
+  E.ticket = zeroed + L.ticket_w + L.passes;
+  E.abort_flag = zeroed + L.abort_w;
+  E.err = err_flag;
+  hipLaunchKernelGGL(plan_emit_kernel, dim3((unsigned)L.emit_tiles), dim3(kAuxThreads), 0, st, E);
   return check_launch("plan build");
 }
+
 
 }  // extern "C"
 

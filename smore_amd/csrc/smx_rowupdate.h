@@ -45,6 +45,14 @@ inline AdamConsts make_adam_consts(const smx_opt_params* a) {
   return c;
 }
 
+// The two constants that change from step to step (learning rate and Adam's bias corrections), as a
+// caller may keep them in device memory: { -lr / (1 - beta1^step), 1 / sqrt(1 - beta2^step) }.
+inline void step_consts(const smx_opt_params* a, float out[2]) {
+  const AdamConsts c = make_adam_consts(a);
+  out[0] = c.step_size;
+  out[1] = c.inv_sqrt_bc2;
+}
+
 // Square root and reciprocal of the update's denominator as the single hardware instructions (1 ulp
 // each) instead of the correctly rounded sequences (about ten instructions each): the step they scale
 // is added to a weight hundreds of times its size, so the weight changes by far less than one ulp of
@@ -90,6 +98,7 @@ struct RowSink {
   int adam_on;    // OptKind; 0 = no optimizer (name kept from the Adam-only version)
   int squeeze;
   AdamConsts a;
+  const float* step_dev;  // null, or device memory holding { step_size, inv_sqrt_bc2 } that replace a's
   ScoreParams p;
   int ncol;       // columns per half row (model sources) or per row (gradient rows)
 };
@@ -197,6 +206,10 @@ __device__ __forceinline__ void finish_row(const RowSink& A, int lane, unsigned 
   }
   if (ADAM_STATIC || A.adam_on) {
     const int kind = A.adam_on;
+    // per-step constants: from the launch arguments, or read now from the caller's device buffer (so that a
+    // captured launch follows the learning-rate schedule and the step counter between replays)
+    const float step_size = A.step_dev ? A.step_dev[0] : A.a.step_size;
+    const float inv_sqrt_bc2 = A.step_dev ? A.step_dev[1] : A.a.inv_sqrt_bc2;
     float* pw = A.table + (size_t)row_id * row_len;
     float* pm = A.m + (size_t)row_id * row_len;
     float* pv = A.v + (size_t)row_id * row_len;
@@ -234,15 +247,15 @@ __device__ __forceinline__ void finish_row(const RowSink& A, int lane, unsigned 
             if (kind == kOptAdam) {
               mn[x] = __builtin_fmaf(m0.h[h][it].v[x], A.a.beta1, g * A.a.omb1);
               vn[x] = __builtin_fmaf(v_old, A.a.beta2, gg * A.a.omb2);
-              const float denom = __builtin_fmaf(hw_sqrt(vn[x]), A.a.inv_sqrt_bc2, A.a.eps);
-              wn[x] = __builtin_fmaf(A.a.step_size * mn[x], hw_rcp(denom), w.h[h][it].v[x]);
+              const float denom = __builtin_fmaf(hw_sqrt(vn[x]), inv_sqrt_bc2, A.a.eps);
+              wn[x] = __builtin_fmaf(step_size * mn[x], hw_rcp(denom), w.h[h][it].v[x]);
             } else if (kind == kOptSgd) {
               mn[x] = vn[x] = 0.f;
-              wn[x] = __builtin_fmaf(A.a.step_size, g, w.h[h][it].v[x]);
+              wn[x] = __builtin_fmaf(step_size, g, w.h[h][it].v[x]);
             } else {
               mn[x] = 0.f;
               vn[x] = kind == kOptAdagrad ? v_old + gg : __builtin_fmaf(v_old, A.a.beta2, gg * A.a.omb2);
-              wn[x] = __builtin_fmaf(A.a.step_size * g, hw_rcp(hw_sqrt(vn[x]) + A.a.eps), w.h[h][it].v[x]);
+              wn[x] = __builtin_fmaf(step_size * g, hw_rcp(hw_sqrt(vn[x]) + A.a.eps), w.h[h][it].v[x]);
             }
             v_new_row = vn[x];
           }

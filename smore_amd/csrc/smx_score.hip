@@ -96,6 +96,7 @@ static void fill_sink(ScoreArgs* A, float* table, float* m, float* v, float* mer
   A->sink.adam_on = adam ? adam->kind : 0;
   A->sink.squeeze = (adam && adam->squeeze) ? 1 : 0;
   if (adam) A->sink.a = make_adam_consts(adam);
+  A->sink.step_dev = adam ? adam->step_consts_dev : nullptr;
   A->sink.p = A->p;
   A->sink.ncol = A->ncol;
 }

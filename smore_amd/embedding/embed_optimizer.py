@@ -108,6 +108,7 @@ class EmbeddingOptimizer(ABC):
         if sp_embed.embedding.device.type != "cuda":
             raise _lib.SmxError("the entity table must live on the GPU (no CPU-table mode in this build)")
         self.err_flag = fused.new_error_flag(sp_embed.embedding.device)
+        self.check_ids_every_step = True
         self.prepare_state()
 
     # -- hooks of the concrete optimizer
@@ -179,14 +180,26 @@ class EmbeddingOptimizer(ABC):
 
     def check_ids(self):
         """Raises if any lookup since the last check met an id outside the table (synchronises)."""
-        if int(self.err_flag.item()) != 0:
+        code = int(self.err_flag.item())
+        if code != 0:
             self.err_flag.zero_()
+            if code == 2:
+                raise _lib.SmxError("the segment plan of this step is invalid (a sort workgroup gave up waiting)")
             raise IndexError("entity id out of range in a sparse lookup")
 
     def apply_grad(self, lr):
+        """Unique-merge, segment sum and row update of everything recorded since zero_grad().  Pairs whose id
+        lies outside the table never reach a row (the plan keeps them apart); with check_ids_every_step
+        (default) the step then ends with IndexError, as table[idx] does in the reference
+        (embed_rw.py:74-75) -- one 4-byte read back per step, after the update has been enqueued."""
         self.step += 1  # counts calls, also those without gradients (embed_optimizer.py:156)
         if not self.grad_list and not self.fused_list:
             return
+        self._apply_grad(lr)
+        if self.check_ids_every_step:
+            self.check_ids()
+
+    def _apply_grad(self, lr):
         n_rows = self.sparse_embed.num_rows
         with torch.no_grad():
             if len(self.fused_list) == 1 and not self.grad_list:

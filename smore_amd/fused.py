@@ -177,17 +177,31 @@ def build_plan(idx, n_rows, want_inverse=False, err_flag=None):
     return plan
 
 
-def adam_params(lr, step, beta1=0.9, beta2=0.999, eps=1e-8, squeeze=False):
-    return _lib.OptParams(lr, beta1, beta2, eps, int(step), _lib.OPT_KINDS["adam"], int(bool(squeeze)))
+def adam_params(lr, step, beta1=0.9, beta2=0.999, eps=1e-8, squeeze=False, step_consts=None):
+    """step_consts: device tensor of two floats kept up to date with set_step_consts(); the kernels then take
+    the learning rate and the bias corrections from it at run time (needed when the launch is replayed
+    from a HIP graph: its by-value arguments are frozen at capture)."""
+    return _lib.OptParams(lr, beta1, beta2, eps, int(step), _lib.OPT_KINDS["adam"], int(bool(squeeze)),
+                          _ptr(step_consts))
 
 
-def opt_params(kind, lr, step=1, squeeze=False, eps=1e-8, alpha=0.99):
+def opt_params(kind, lr, step=1, squeeze=False, eps=1e-8, alpha=0.99, step_consts=None):
     """Parameters of a row optimizer: kind in {adam, sgd, adagrad, rmsprop} (see smx_opt_params)."""
     if kind == "adam":
-        return adam_params(lr, step, eps=eps, squeeze=squeeze)
+        return adam_params(lr, step, eps=eps, squeeze=squeeze, step_consts=step_consts)
     if kind not in _lib.OPT_KINDS:
         raise _lib.SmxError(f"unknown optimizer {kind}")
-    return _lib.OptParams(lr, 0.0, alpha, eps, int(step), _lib.OPT_KINDS[kind], int(bool(squeeze)))
+    return _lib.OptParams(lr, 0.0, alpha, eps, int(step), _lib.OPT_KINDS[kind], int(bool(squeeze)), _ptr(step_consts))
+
+
+def set_step_consts(buf, opt):
+    """Writes the per-step constants of `opt` (its lr and step) into the two-float device tensor `buf`, in
+    stream order (a 8-byte copy from pinned memory)."""
+    host = (ctypes.c_float * 2)()
+    _lib.call("smx_opt_step_consts", ctypes.byref(opt), host)
+    pinned = torch.tensor([host[0], host[1]], dtype=torch.float32).pin_memory()
+    buf.copy_(pinned, non_blocking=True)
+    return buf
 
 
 def _check_state(table, m, v, opt):

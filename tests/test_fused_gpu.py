@@ -281,6 +281,59 @@ def test_out_of_range_id_sets_the_flag():
     assert err.item() == 1
 
 
+@pytest.mark.parametrize("n_pairs_shape", [(6, 40), (40, 1024)])
+def test_out_of_range_ids_update_no_row(n_pairs_shape):
+    """Pairs whose id lies outside the table are kept out of the plan's segments: n_uniq / uniq are those of the
+    valid ids, no row -- row 0 least of all -- is updated for them, and the rows of the valid ids get what the
+    oracle gives when the bad pairs contribute nothing."""
+    from smore_amd import fused
+    b, k = n_pairs_shape
+    n, dim, lr = 3000, 64, 1e-3
+    rng = np.random.default_rng(seed("bad ids", b, k))
+    table, q1, q2, idx, gs = make_problem("box", n, b, k, dim, rng, zipf=1.05)
+    idx = np.maximum(idx, 1)                                   # row 0 is named by no valid pair
+    bad = rng.random((b, k)) < 0.03
+    bad[0, 0] = bad[-1, -1] = True
+    idx_bad = idx.copy()
+    idx_bad[bad] = rng.choice([-1, n, n + 7, 1 << 40, -(1 << 35)], size=int(bad.sum()))
+    t_q1, t_q2, t_gs = dev(q1), dev(q2), dev(gs)
+    t_idx = torch.tensor(idx_bad, device="cuda")
+    params = fused.score_params(24.0, 0.02)
+    err = fused.new_error_flag("cuda")
+    plan = fused.build_plan(t_idx, n, want_inverse=True, err_flag=err)
+    assert err.item() == 1
+    uniq = np.unique(idx[~bad])
+    assert plan.n_uniq == uniq.size and np.array_equal(plan.uniq.cpu().numpy(), uniq)
+    inv = plan.inverse.cpu().numpy().reshape(b, k)
+    assert np.array_equal(inv[~bad], np.searchsorted(uniq, idx[~bad])) and (inv[bad] == uniq.size).all()
+    assert not (plan.pair_seg.cpu().numpy().reshape(b, k)[bad] < 0).any()
+    # the oracle's step on the valid pairs: bad pairs moved onto a valid id of their query with zero upstream gradient
+    idx_ref, gs_ref = idx_bad.copy(), gs.copy()
+    idx_ref[bad] = np.broadcast_to(uniq[:1], (b, k))[bad]
+    gs_ref[bad] = 0.0
+    w_o, m_o, v_o = table.copy(), np.zeros_like(table), np.zeros_like(table)
+    orc.train_step("box", w_o, m_o, v_o, idx_ref, q1[:, None], q2[:, None], gs_ref, 24.0, 0.02, lr, 1)
+    touched = np.zeros(n, bool)
+    touched[uniq] = True
+    for one_call in (False, True):
+        t_table = dev(table)
+        t_m, t_v = torch.zeros_like(t_table), torch.zeros_like(t_table)
+        codes = fused.new_codes("box", t_table, t_idx, t_q1)
+        score = fused.score_forward("box", t_table, t_idx, t_q1, t_q2, params, err, codes=codes)
+        if one_call:
+            fused.score_backward_fused("box", plan, t_table, t_idx, t_q1, t_q2, score, t_gs, params, m=t_m, v=t_v,
+                                       adam=fused.adam_params(lr, 1), codes=codes)
+        else:
+            fused.score_backward_entity("box", plan, t_table, t_q1, t_q2, score, t_gs, params, m=t_m, v=t_v,
+                                        adam=fused.adam_params(lr, 1))
+        w, m, v = (x.cpu().numpy() for x in (t_table, t_m, t_v))
+        assert np.array_equal(w[~touched], table[~touched].astype(np.float32)), "a row without a valid pair changed"
+        assert not m[~touched].any() and not v[~touched].any()
+        # (the row that collected the moved pairs in the oracle got zero gradient from them: nothing was added)
+        assert_close(m[touched], m_o[touched], 5 * REL_F32, "first moment of the valid rows")
+        assert_close(v[touched], v_o[touched], 5 * REL_F32, "second moment of the valid rows")
+
+
 def test_entity_pass_is_deterministic():
     from smore_amd import fused
     rng = np.random.default_rng(5)
