@@ -228,8 +228,8 @@ def measure_ceilings(device, row_bytes, full=False):
     stream = ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
     for name, kind, moved in kinds:
         def launch():
-            _lib.call("smx_probe_bandwidth", kind, stream, ctypes.c_void_p(a.data_ptr()), ctypes.c_void_p(b.data_ptr()),
-                      nbytes, row_bytes, n_reads, ctypes.c_void_p(sink.data_ptr()))
+            _lib.probe_bandwidth(kind, stream, ctypes.c_void_p(a.data_ptr()), ctypes.c_void_p(b.data_ptr()),
+                                 nbytes, row_bytes, n_reads, ctypes.c_void_p(sink.data_ptr()))
         launch()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
@@ -392,12 +392,12 @@ def main():
     if cfg["adam"] and step.codes is not None:
         # the same backward with its kernels one after the other on one stream (the library's profiling
         # switch): the figure the per-kernel durations of a rocprofv3 trace of that mode add up to
-        os.environ["SMX_SERIAL_BACKWARD"] = "1"
+        _lib.call("smx_set_option", _lib.OPTION_SERIAL_BACKWARD, 1)
         ev2 = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(5)]
         for e in ev2:
             step.run(e)
         torch.cuda.synchronize()
-        del os.environ["SMX_SERIAL_BACKWARD"]
+        _lib.call("smx_set_option", _lib.OPTION_SERIAL_BACKWARD, 0)
         out["roofline"]["one_stream_avg_ms"] = sum(e[2].elapsed_time(e[3]) for e in ev2) / len(ev2)
     # what plain kernels sustain on this GPU for the step's access shapes, measured now with the library's
     # probes (after the timed region); a step that writes w, m, v back is a copy-like mix of reads and writes

@@ -53,6 +53,13 @@ extern "C" {
 int smx_version(void);
 const char* smx_last_error(void);
 
+/* Process-wide switches (thread-safe; take effect for calls made afterwards).
+ *   SMX_OPTION_SERIAL_BACKWARD  != 0: smx_score_backward_fused / smx_score_backward_entity keep all their
+ *                               kernels on the caller's stream instead of running the entity pass on the
+ *                               library's second stream -- same results, for per-kernel profiling. */
+#define SMX_OPTION_SERIAL_BACKWARD 1
+int smx_set_option(int option, int value);
+
 /* kind id for a dist_name string ("l1", "box_out", ...), -1 if unknown.
  * Replaces the string chain of ext_cuda_kernel.cu:25-49 (which prints and
  * silently does nothing for an unknown name; here the caller gets -1). */
@@ -222,8 +229,8 @@ int smx_opt_step_consts(const smx_opt_params* opt, float* out2);
  * With them, an optimizer, no merged output and a step of a million pairs or more whose queries
  * exceed one L2, the call finishes ids that occur once in a pair-ordered kernel on `stream` and
  * reduces the others on the library's second stream beside it (joined to `stream` before return);
- * the rows get the same bits either way.  (Environment: SMX_SERIAL_BACKWARD=1 keeps this call and
- * smx_score_backward_fused on the caller's stream alone -- for per-kernel profiling.) */
+ * the rows get the same bits either way (smx_set_option(SMX_OPTION_SERIAL_BACKWARD, 1) keeps this call
+ * and smx_score_backward_fused on the caller's stream alone). */
 size_t smx_entity_workspace_bytes(size_t n_pairs, size_t row_len);
 int smx_score_backward_entity(int model, void* stream, const smx_plan_view* plan, float* table,
                               size_t n_rows, const float* q1, const float* q2, const float* score,
@@ -315,23 +322,6 @@ int smx_rank_scan(int model, void* stream, const float* table, size_t n_rows, co
                   const float* q2, size_t B, size_t dim, const smx_score_params* params,
                   const int64_t* ans_id, const uint64_t* ans_key, const int32_t* ans_count, size_t A,
                   int64_t* filtered_rank, void* workspace, size_t workspace_bytes);
-
-/* ---- bandwidth probes (measurement only) --------------------------------------------------------
- * No counterpart in the reference.  One launch of a kernel that does nothing but move memory in one of
- * the access shapes of this path, for bench.py to time: what the box sustains, next to the nominal peak.
- *   READ_NT / READ   stream `bytes` of a (non-temporal / plain loads)
- *   COPY             a -> b          UPDATE  a = 2 a in place          FILL  a = constant
- *   ROWS / ROWS_NT   n_reads rows of row_bytes (16..1024, multiple of 16) at pseudo-random positions of a
- * sink: one device float the read probes may write (keeps their loads alive); never meaningful. */
-#define SMX_PROBE_READ_NT 0
-#define SMX_PROBE_READ 1
-#define SMX_PROBE_COPY 2
-#define SMX_PROBE_UPDATE 3
-#define SMX_PROBE_FILL 4
-#define SMX_PROBE_ROWS 5
-#define SMX_PROBE_ROWS_NT 6
-int smx_probe_bandwidth(int kind, void* stream, void* a, void* b, size_t bytes, size_t row_bytes,
-                        size_t n_reads, float* sink);
 
 /* Plain row lookup out[k,:] = table[idx[k],:] (smore/common/embedding/embed_rw.py:74-75, the GPU
  * branch of EmbeddingReadOnly.read) for callers that need the rows themselves. */

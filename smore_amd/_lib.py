@@ -29,8 +29,7 @@ SIGNATURES = {
     "smx_dist_forward_f64": (_i, _DENSE_FWD),
     "smx_dist_backward_f32": (_i, _DENSE_BWD),
     "smx_dist_backward_f64": (_i, _DENSE_BWD),
-    # kind, stream, a, b, bytes, row_bytes, n_reads, sink
-    "smx_probe_bandwidth": (_i, [_i, _vp, _vp, _vp, _sz, _sz, _sz, _vp]),
+    "smx_set_option": (_i, [_i, _i]),
     "smx_score_codes_bytes": (_sz, [_i, _sz, _sz]),
     # model, stream, table, n_rows, idx, q1, q2, score, B, K, dim, params, err_flag, codes, codes_bytes
     "smx_score_forward": (_i, [_i, _vp, _vp, _sz, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _vp, _vp, _vp, _sz]),
@@ -88,7 +87,11 @@ class PlanView(ctypes.Structure):
     _fields_ = [("order", _vp), ("sorted_ids", _vp), ("seg_of_pos", _vp), ("seg_start", _vp), ("uniq", _vp),
                 ("n_uniq", _vp), ("pair_seg", _vp), ("n_pairs", _sz)]
 
+OPTION_SERIAL_BACKWARD = 1
+
 _lib = None
+_probe = None
+PROBE_PATH = os.path.join(_HERE, "libsmx_probe.so")
 
 
 class SmxError(RuntimeError):
@@ -120,3 +123,19 @@ def check(rc):
 
 def call(name, *args):
     check(getattr(load(), name)(*args))
+
+
+def probe_bandwidth(kind, stream, a, b, nbytes, row_bytes, n_reads, sink):
+    """smx_probe_bandwidth of libsmx_probe.so (include/smx_probe.h): the benchmark's bandwidth probes."""
+    global _probe
+    if _probe is None:
+        if not os.path.exists(PROBE_PATH):
+            raise SmxError(f"{PROBE_PATH} is missing: build it with `make -C smore_amd/csrc`")
+        lib = ctypes.CDLL(PROBE_PATH)
+        lib.smx_probe_bandwidth.restype = _i
+        lib.smx_probe_bandwidth.argtypes = [_i, _vp, _vp, _vp, _sz, _sz, _sz, _vp]
+        lib.smx_probe_last_error.restype = _c.c_char_p
+        _probe = lib
+    rc = _probe.smx_probe_bandwidth(kind, stream, a, b, nbytes, row_bytes, n_reads, sink)
+    if rc != 0:
+        raise SmxError(f"smx_probe status {rc}: {_probe.smx_probe_last_error().decode('utf-8', 'replace')}")

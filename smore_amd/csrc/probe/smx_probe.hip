@@ -2,9 +2,32 @@
 // kernels that do nothing else.  bench.py reports the figures next to the step's achieved rate, so the
 // fraction of the 8 TB/s nominal peak can be read against what a plain kernel reaches on the same box.
 // Every probe keeps eight 16-byte loads (or stores) per lane in flight on a persistent grid.
-#include "smx_common.h"
+// Built into a library of its own (libsmx_probe.so): measurement only, not part of the drop-in ABI.
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+
+#include "../../../include/smx_probe.h"
 
 namespace smx {
+
+static thread_local char g_probe_err[256] = "";
+static int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_probe_err, sizeof(g_probe_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+static int check_launch(const char* what) {
+  const hipError_t e = hipGetLastError();
+  return e == hipSuccess ? 0 : fail(4, "%s: %s", what, hipGetErrorString(e));
+}
+static hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
+static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+constexpr int SMX_ERR_KIND = 1, SMX_ERR_SHAPE = 2, SMX_ERR_ARG = 3;
 
 typedef float probe_vec4 __attribute__((ext_vector_type(4)));
 constexpr int kProbeUnroll = 8;
@@ -75,6 +98,8 @@ __global__ __launch_bounds__(256) void probe_rows_kernel(const probe_vec4* __res
 }  // namespace smx
 
 extern "C" {
+
+const char* smx_probe_last_error(void) { return smx::g_probe_err; }
 
 int smx_probe_bandwidth(int kind, void* stream, void* a, void* b, size_t bytes, size_t row_bytes, size_t n_reads,
                         float* sink) {

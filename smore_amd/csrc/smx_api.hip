@@ -1,4 +1,5 @@
 // Version, error text and name lookup of the C ABI.
+#include <atomic>
 #include <cstring>
 
 #include "smx_common.h"
@@ -22,11 +23,22 @@ int check_launch(const char* what) {
   return SMX_OK;
 }
 
+static std::atomic<int> g_serial_backward{0};
+bool serial_backward() { return g_serial_backward.load(std::memory_order_relaxed) != 0; }
+
 }  // namespace smx
 
 extern "C" {
 
-int smx_version(void) { return 1; }
+int smx_version(void) { return 2; }
+
+int smx_set_option(int option, int value) {
+  if (option == SMX_OPTION_SERIAL_BACKWARD) {
+    smx::g_serial_backward.store(value ? 1 : 0, std::memory_order_relaxed);
+    return SMX_OK;
+  }
+  return smx::fail(SMX_ERR_ARG, "unknown option %d", option);
+}
 
 const char* smx_last_error(void) { return smx::g_err; }
 

@@ -19,6 +19,9 @@ int fail(int code, const char* fmt, ...);
 // Checks the launch that just happened on this thread.
 int check_launch(const char* what);
 
+// smx_set_option(SMX_OPTION_SERIAL_BACKWARD, ..): the backward keeps to the caller's stream
+bool serial_backward();
+
 inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }

@@ -25,6 +25,8 @@
 // derivative is linear in the upstream coefficient, so coefficients are summed
 // first.
 #pragma once
+#include <mutex>
+
 #include "smx_common.h"
 #include "smx_models.h"
 #include "smx_rowupdate.h"
@@ -473,19 +475,22 @@ __global__ __launch_bounds__(NW * 64) void entity_fixup_kernel(EntityArgs A) {
   }
 }
 
-// Workgroups of 256 threads of `kernel` the current device keeps resident (asked once per kernel).
+// Workgroups of 256 threads of `kernel` the current device keeps resident (asked once per kernel and device).
 template <class K>
 unsigned resident_blocks(K kernel) {
-  static unsigned cached = 0;  // one value per instantiation, i.e. per kernel
-  if (cached == 0) {
-    int dev = 0, cus = 0, per_cu = 0;
-    if (hipGetDevice(&dev) != hipSuccess ||
-        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+  static std::mutex mu;                 // one table per instantiation, i.e. per kernel
+  static unsigned cached[64] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256u * 8u;
+  std::lock_guard<std::mutex> lock(mu);
+  if (cached[dev] == 0) {
+    int cus = 0, per_cu = 0;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
         hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, 256, 0) != hipSuccess || cus <= 0 || per_cu <= 0)
       return 256u * 8u;
-    cached = (unsigned)cus * (unsigned)per_cu;
+    cached[dev] = (unsigned)cus * (unsigned)per_cu;
   }
-  return cached;
+  return cached[dev];
 }
 
 template <int SRC, int VEC, int NIT, bool REG>

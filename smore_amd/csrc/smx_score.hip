@@ -16,7 +16,6 @@
 // quarter of the tile's rows, two batches of rows in flight at a time.  backward: one workgroup per
 // query walks all K negatives, wavefront partial sums are combined through LDS
 // in wavefront order, so the gradient has a fixed summation order.
-#include <cstdlib>
 #include <mutex>
 
 #include "smx_score_impl.h"
@@ -220,7 +219,7 @@ int smx_score_backward_entity(int model, void* stream, const smx_plan_view* plan
                      queries_beyond_l2(model, B, dim) && B * K >= ((size_t)1 << 20) && plan->n_pairs == B * K &&
                      workspace && !(reinterpret_cast<uintptr_t>(workspace) & 255u) &&
                      workspace_bytes >= entity_ws_bytes(B * K, dim * model_mul(model)) &&
-                     !std::getenv("SMX_SERIAL_BACKWARD");
+                     !serial_backward();
   if (split) {
     ScoreArgs A;
     int vec, nit;
@@ -316,8 +315,8 @@ int smx_score_backward_fused(int model, void* stream, const smx_plan_view* plan,
       codes = A.codes;
     }
   }
-  // (SMX_SERIAL_BACKWARD=1 keeps everything on the caller's stream, for per-kernel profiling)
-  if (fwd_codes && adam && B * K >= ((size_t)1 << 20) && !std::getenv("SMX_SERIAL_BACKWARD")) {
+  // (the serial-backward option keeps everything on the caller's stream, for per-kernel profiling)
+  if (fwd_codes && adam && B * K >= ((size_t)1 << 20) && !serial_backward()) {
     // With the forward's codes the entity pass does not depend on the query-gradient kernel and the two
     // touch disjoint rows; one is bound by instruction issue for much of its time, the other by memory
     // latency, so they run side by side: the entity pass on a second stream of the same device, forked

@@ -675,9 +675,12 @@ int launch_score(hipStream_t st, const ScoreArgs& A, bool forward) {
     }
     return launch_forward_reg<M, VEC, NIT, false>(st, A);
   }
-  // wavefronts per query: as many as the LDS combine buffer allows
+  // wavefronts per query: as many as 64 KiB of LDS allow -- the staged query and one partial-sum row per
+  // wavefront, the wavefronts' 1 KiB pair slabs and, where the kernel writes sign codes, their code stages
   const size_t per_wave = (size_t)model_nq(M) * A.ncol * VEC * sizeof(float);
-  const int nw = 9 * per_wave <= 60 * 1024 ? 8 : (5 * per_wave <= 60 * 1024 ? 4 : 2);
+  const size_t extra = kSlabDwords * sizeof(unsigned) + (model_coded(M) ? (size_t)kStagePairs * NIT * 64 : 0);
+  auto fits = [&](size_t n) { return (n + 1) * per_wave + n * extra <= 64 * 1024; };
+  const int nw = fits(8) ? 8 : (fits(4) ? 4 : 2);
   if constexpr (M == mBetaKL) {
     if (reg) {
       if (nw == 8) return launch_backward_query_reg<M, VEC, NIT, 8, true>(st, A);

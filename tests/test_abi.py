@@ -9,8 +9,8 @@ import pytest
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
-def _declared():
-    text = open(os.path.join(ROOT, "include", "smore_amd.h")).read()
+def _declared(header="smore_amd.h"):
+    text = open(os.path.join(ROOT, "include", header)).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(smx_[a-z0-9_]+)\s*\(", text)))
 
@@ -27,6 +27,17 @@ def test_header_symbols_are_exported_and_bound():
     assert sorted(_lib.SIGNATURES) == names
 
 
+def test_probe_library_exports_its_header():
+    """The benchmark's bandwidth probes live in a library of their own, outside the drop-in ABI."""
+    from smore_amd import _lib
+    if not os.path.exists(_lib.PROBE_PATH):
+        pytest.fail("libsmx_probe.so is not built (run __graft_entry__.build())")
+    lib = ctypes.CDLL(_lib.PROBE_PATH)
+    for n in _declared("smx_probe.h"):
+        assert hasattr(lib, n), f"{n} declared in smx_probe.h but not exported"
+    assert not any("probe" in n for n in _declared())
+
+
 def test_host_only_entry_points():
     from smore_amd import _lib
     lib = _lib.load()
@@ -34,6 +45,12 @@ def test_host_only_entry_points():
     assert lib.smx_kind_from_name(b"box_out") == 2
     assert lib.smx_kind_from_name(b"beta_fisher_approx") == 9
     assert lib.smx_kind_from_name(b"nope") == -1
+    assert lib.smx_set_option(_lib.OPTION_SERIAL_BACKWARD, 0) == 0 and lib.smx_set_option(99, 1) != 0
+    import ctypes as c
+    opt = _lib.OptParams(1e-3, 0.9, 0.999, 1e-8, 2, _lib.OPT_KINDS["adam"], 0, None)
+    out = (c.c_float * 2)()
+    assert lib.smx_opt_step_consts(c.byref(opt), out) == 0
+    assert abs(out[0] + 1e-3 / (1 - 0.9 ** 2)) < 1e-9 and abs(out[1] - (1 - 0.999 ** 2) ** -0.5) < 1e-4
 
 
 def test_missing_library_fails_loudly(monkeypatch):

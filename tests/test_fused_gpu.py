@@ -37,6 +37,12 @@ def make_problem(model, n, b, k, dim, rng, zipf=None, scale=0.07):
     return f32(table), f32(q1), None if q2 is None else f32(q2), idx.astype(np.int64), f32(gs)
 
 
+def _serial_backward(on):
+    """smx_set_option(SMX_OPTION_SERIAL_BACKWARD): every kernel of the backward on the caller's stream."""
+    from smore_amd import _lib
+    _lib.call("smx_set_option", _lib.OPTION_SERIAL_BACKWARD, int(on))
+
+
 def dev(a, dtype=torch.float32):
     return None if a is None else torch.tensor(a, dtype=dtype, device="cuda")
 
@@ -637,6 +643,10 @@ def test_fused_entity_pass_with_every_optimizer(kind, squeeze):
     (64, 2, 3, 2048),    # the widest row the fused path takes (8 float4 columns per lane)
     (64, 2, 3, 252),     # widest unaligned-friendly scalar row is 256; 252 is float4-aligned
     (30, 2, 5, 255),     # scalar columns, four per lane
+    (40, 2, 70, 800),    # two-query models: eight wavefronts' rows + slabs would pass 64 KiB of LDS here
+    (40, 2, 70, 848),
+    (40, 2, 70, 1600),   # the same band for one-query models
+    (40, 2, 70, 1704),
 ])
 def test_fused_edge_shapes(shape):
     n, b, k, dim = shape
@@ -681,7 +691,7 @@ def test_unsupported_rows_are_refused_not_mangled():
         fused.build_plan(torch.zeros(0, dtype=torch.int64, device="cuda"), 10)
 
 
-def test_second_stream_backward_gives_the_bits_of_the_serial_one(monkeypatch):
+def test_second_stream_backward_gives_the_bits_of_the_serial_one():
     """Steps of a million pairs or more with the forward's codes and an optimizer run the entity pass on
     the library's second stream beside the query-gradient kernel.  Same kernels, same data, disjoint
     rows: the results must be bit-identical to the one-stream order, and repeatable."""
@@ -700,11 +710,8 @@ def test_second_stream_backward_gives_the_bits_of_the_serial_one(monkeypatch):
     codes = fused.new_codes("box", table, idx, q1)
     score = fused.score_forward("box", table, idx, q1, q2, params, codes=codes)
     results = []
-    for serial in ("1", None, None):
-        if serial:
-            monkeypatch.setenv("SMX_SERIAL_BACKWARD", serial)
-        else:
-            monkeypatch.delenv("SMX_SERIAL_BACKWARD", raising=False)
+    for serial in (1, 0, 0):
+        _serial_backward(serial)
         w, m, v = table.clone(), torch.zeros_like(table), torch.zeros_like(table)
         g1, g2 = fused.score_backward_fused("box", plan, w, idx, q1, q2, score, gs, params, m=m, v=v,
                                             adam=fused.adam_params(1e-4, 1), codes=codes)
@@ -717,7 +724,7 @@ def test_second_stream_backward_gives_the_bits_of_the_serial_one(monkeypatch):
     assert abs(touched - plan.n_uniq) <= int((gs == 0).sum().item())
 
 
-def test_deferred_entity_pass_matches_the_one_call_backward(monkeypatch):
+def test_deferred_entity_pass_matches_the_one_call_backward():
     """The autograd flow takes the query gradients first and updates the rows later, in
     score_backward_entity.  For large steps with the forward's codes that call hands the one-pair
     segments to the pair-ordered kernel and runs the entity pass beside it: table, m and v must come
@@ -741,16 +748,13 @@ def test_deferred_entity_pass_matches_the_one_call_backward(monkeypatch):
             v_shape = (n, 1) if squeeze else (n, dim)
             return table.clone(), torch.zeros_like(table), torch.zeros(v_shape, device="cuda")
         opt = fused.adam_params(1e-4, 1, squeeze=squeeze)
-        monkeypatch.delenv("SMX_SERIAL_BACKWARD", raising=False)
+        _serial_backward(0)
         w0, m0, v0 = state()
         g1, g2 = fused.score_backward_fused("box", plan, w0, idx, q1, q2, score, gs, params, m=m0, v=v0, adam=opt,
                                             codes=codes)
         outcomes = []
-        for serial in (None, "1", None):
-            if serial:
-                monkeypatch.setenv("SMX_SERIAL_BACKWARD", serial)
-            else:
-                monkeypatch.delenv("SMX_SERIAL_BACKWARD", raising=False)
+        for serial in (0, 1, 0):
+            _serial_backward(serial)
             w, m, v = state()
             d1, d2 = fused.score_backward_query("box", table, idx, q1, q2, score, gs, params, codes=codes)
             fused.score_backward_entity("box", plan, w, q1, q2, score, gs, params, m=m, v=v, adam=opt, codes=codes)

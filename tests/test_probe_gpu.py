@@ -10,9 +10,9 @@ pytestmark = pytest.mark.gpu
 def _run(kind, a, b, row_bytes=800, n_reads=1000):
     from smore_amd import _lib
     sink = torch.zeros(1, device="cuda")
-    _lib.call("smx_probe_bandwidth", kind, ctypes.c_void_p(torch.cuda.current_stream().cuda_stream),
-              ctypes.c_void_p(a.data_ptr()), None if b is None else ctypes.c_void_p(b.data_ptr()),
-              a.numel() * a.element_size(), row_bytes, n_reads, ctypes.c_void_p(sink.data_ptr()))
+    _lib.probe_bandwidth(kind, ctypes.c_void_p(torch.cuda.current_stream().cuda_stream),
+                         ctypes.c_void_p(a.data_ptr()), None if b is None else ctypes.c_void_p(b.data_ptr()),
+                         a.numel() * a.element_size(), row_bytes, n_reads, ctypes.c_void_p(sink.data_ptr()))
     torch.cuda.synchronize()
 
 
