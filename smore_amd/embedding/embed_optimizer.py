@@ -15,6 +15,7 @@ import torch
 import torch.nn as nn
 
 from .. import _lib, fused
+from .lazy_rows import LazyRows
 from .sparse_embed import SparseEmbedding
 
 
@@ -109,6 +110,9 @@ class EmbeddingOptimizer(ABC):
             raise _lib.SmxError("the entity table must live on the GPU (no CPU-table mode in this build)")
         self.err_flag = fused.new_error_flag(sp_embed.embedding.device)
         self.check_ids_every_step = True
+        self._flag_host = torch.zeros(1, dtype=torch.int32, pin_memory=True)   # where the flag of a step lands
+        self._flag_event = None                                                # set while such a copy is under way
+        self.lazy_lookup = True
         self.prepare_state()
 
     # -- hooks of the concrete optimizer
@@ -142,12 +146,47 @@ class EmbeddingOptimizer(ABC):
         self.has_grad_list.append(fwd_idx)
 
     def forward(self, indices, name=None):
+        """What sp_embed(indices, name) returns while this optimizer is attached (embed_optimizer.py:150-153).
+        With lazy_lookup (default) that is a LazyRows handle: model code that only views it, regularizes it and
+        hands it to the distance operators of ext_ops gets the gather-fused scorer without knowing; any other use
+        turns it into the looked-up rows.  lazy_lookup = False: the rows at once, as in the reference."""
         if indices is None:
             mat = self.sparse_embed.embedding
-        else:
-            mat = EmbedLookupFunc.apply(self, self.dummy_tensor, indices, name)
+            mat.job_handle = self.sparse_embed.dummy_job
+            return mat
+        if self.lazy_lookup:
+            return LazyRows(self, indices, name)
+        return self.lookup_rows(indices, name)
+
+    def lookup_rows(self, indices, name=None):
+        """rows = table[indices], shaped indices.shape + (row,), through the autograd node that records the
+        gradient rows for apply_grad (EmbedLookupFunc, embed_optimizer.py:51-66)."""
+        mat = EmbedLookupFunc.apply(self, self.dummy_tensor, indices, name)
+        if indices.dim() != 1:
+            mat = mat.view(tuple(indices.shape) + (mat.shape[-1],))
         mat.job_handle = self.sparse_embed.dummy_job
         return mat
+
+    def score_lazy(self, model, rows, queries, gamma, cen):
+        """Logits gamma - dist(rows, queries) for a LazyRows handle [Be, K, row] against query tensors [B, 1, D]
+        (-> [B, K]) or [B, U, 1, D] (-> [B, U, K], one slice per union branch as the dense operators return it),
+        in one launch of the fused scorer.  None when this is not a layout the fused scorer takes."""
+        q = queries[0]
+        if q.dim() == 4:
+            bq, nc, dim = q.shape[0], q.shape[2], q.shape[3]
+        else:
+            bq, nc, dim = q.shape
+        be, k, row = rows.shape
+        mul = 2 if model in fused.TWO_HALVES else 1
+        n_q = 1 if model in fused.ONE_QUERY else 2
+        if (nc != 1 or be not in (1, bq) or row != dim * mul or len(queries) != n_q or
+                (rows.reg is not None and model != "beta_kl") or rows.ids.numel() != be * k):
+            return None
+        if any(t.dtype != torch.float32 or t.device != rows.device for t in queries):
+            return None
+        q2 = queries[1] if n_q == 2 else None
+        logit = self._score_branches(model, rows.ids.reshape(be, k), q, q2, gamma, cen, rows.reg)
+        return logit if q.dim() == 4 else logit[:, 0]
 
     def score_negatives(self, model, ids, q1, q2=None, gamma=0.0, cen=0.0, regularizer=None):
         """Gather-fused logits [B,K]; q1/q2 are [B,dim] or [B,1,dim] and receive gradients.
@@ -156,6 +195,11 @@ class EmbeddingOptimizer(ABC):
         Union queries: q1/q2 of shape [B,U,dim] or [B,U,1,dim] (the merged branch embeddings of
         kg_reasoning.py:326) give max over the U branches of each branch's logit, as the last line of
         every custom_cal_logit does (box.py:163, vec.py:89, rotate.py:141, beta.py:307)."""
+        logit = self._score_branches(model, ids, q1, q2, gamma, cen, regularizer)
+        return torch.max(logit, dim=1)[0] if logit.shape[1] > 1 else logit[:, 0]
+
+    def _score_branches(self, model, ids, q1, q2, gamma, cen, regularizer):
+        """[B, branches, K] logits of every union branch of every query against that query's negatives."""
         table = self.sparse_embed.embedding
         b = q1.shape[0]
         dim = q1.shape[-1]
@@ -174,30 +218,48 @@ class EmbeddingOptimizer(ABC):
         q2c = None if q2 is None else q2.reshape(b * branches, dim).contiguous()
         params = fused.score_params(gamma, cen, regularizer)
         logit = _FusedScoreFunc.apply(self, self.dummy_tensor, model, ids, params, q1c, q2c)
-        if branches > 1:
-            logit = torch.max(logit.view(b, branches, -1), dim=1)[0]
-        return logit
+        return logit.view(b, branches, -1)
+
+    def _raise_for(self, code):
+        if code == 2:
+            raise _lib.SmxError("the segment plan of this step is invalid (a sort workgroup gave up waiting)")
+        if code != 0:
+            raise IndexError("entity id out of range in a sparse lookup")
 
     def check_ids(self):
         """Raises if any lookup since the last check met an id outside the table (synchronises)."""
+        self._flag_event = None
         code = int(self.err_flag.item())
         if code != 0:
             self.err_flag.zero_()
-            if code == 2:
-                raise _lib.SmxError("the segment plan of this step is invalid (a sort workgroup gave up waiting)")
-            raise IndexError("entity id out of range in a sparse lookup")
+        self._raise_for(code)
+
+    def _check_ids_one_step_late(self):
+        """The per-step check without draining the queue: this step's flag is copied to pinned host memory behind
+        the update, and looked at when the next step gets here -- by then the copy has long finished, so the host
+        keeps running ahead of the device."""
+        if self._flag_event is not None:
+            self._flag_event.synchronize()
+            self._flag_event = None
+            code = int(self._flag_host[0])
+            if code != 0:
+                self.err_flag.zero_()
+                self._raise_for(code)
+        self._flag_host.copy_(self.err_flag, non_blocking=True)
+        self._flag_event = torch.cuda.Event()
+        self._flag_event.record()
 
     def apply_grad(self, lr):
         """Unique-merge, segment sum and row update of everything recorded since zero_grad().  Pairs whose id
-        lies outside the table never reach a row (the plan keeps them apart); with check_ids_every_step
-        (default) the step then ends with IndexError, as table[idx] does in the reference
-        (embed_rw.py:74-75) -- one 4-byte read back per step, after the update has been enqueued."""
+        lies outside the table never reach a row (the plan keeps them apart), and the lookup that met one raises
+        IndexError as table[idx] does in the reference (embed_rw.py:74-75) -- with check_ids_every_step (default)
+        from the apply_grad of the following step, so that no step waits for the device; check_ids() asks at once."""
         self.step += 1  # counts calls, also those without gradients (embed_optimizer.py:156)
         if not self.grad_list and not self.fused_list:
             return
         self._apply_grad(lr)
         if self.check_ids_every_step:
-            self.check_ids()
+            self._check_ids_one_step_late()
 
     def _apply_grad(self, lr):
         n_rows = self.sparse_embed.num_rows

@@ -1,0 +1,386 @@
+"""Rows of the entity table that are looked up only when something needs their values.
+
+Unchanged SMORE model code computes a step's negative logits as (smore/models/kg_reasoning.py:301-307,349-355)
+    rows  = self.entity_embedding(negative_sample.view(-1), "negative_entity")      # sparse lookup
+    rows  = self.entity_regularizer(rows.view(batch_size, negative_size, -1))        # identity, or clamp(rows + 1, .05, 1e9)
+    logit = self.cal_logit(rows, None, query_embedding)                              # custom_cal_logit of the model
+and custom_cal_logit (models/box.py:157-164, vec.py:85-90, rotate.py:137-142, beta.py:303-308) is
+    gamma - dist(rows, query)            [box: gamma - box_dist_out(..) - cen * box_dist_in(..)]   then max over dim 1.
+With an EmbeddingOptimizer attached, the lookup returns a `LazyRows` handle instead of a [B*K, row] tensor.
+The handle understands exactly what that call sequence does to it -- `.view`, `.unsqueeze`, `+ base_add`,
+`torch.clamp` -- and the distance operators of smore_amd.torchext.ext_ops, given a handle, return a `LazyLogit`:
+a running affine expression  const + sum coef * dist  that scalar arithmetic extends.  The first operation that
+needs values (torch.max in custom_cal_logit) evaluates the expression; when it has the shape of one of the
+models' logits it becomes ONE launch of the gather-fused scorer (smx_score_forward) on the ids, and its autograd
+node hands the entity gradient to the optimizer's fused entity pass.  Anything else -- an expression the fused
+scorer has no model for, or any other use of the rows (cal_reg, indexing, printing) -- falls back to the plain
+lookup (EmbedLookupFunc) and the dense operators, with the reference's results.
+"""
+import numbers
+import weakref
+
+import torch
+
+from .. import _lib
+
+_FUSED_MODEL = {"l1": "l1", "l2": "l2", "rotate": "rotate", "beta_kl": "beta_kl"}
+
+
+def _is_lazy(x):
+    return isinstance(x, (LazyRows, LazyLogit))
+
+
+def _resolve(x):
+    """Replaces every lazy object in a (possibly nested) argument by its tensor."""
+    if _is_lazy(x):
+        return x.materialize()
+    if isinstance(x, (list, tuple)):
+        return type(x)(_resolve(v) for v in x)
+    if isinstance(x, dict):
+        return {k: _resolve(v) for k, v in x.items()}
+    return x
+
+
+def _func_name(func):
+    return getattr(func, "__name__", "")
+
+
+_scalar_cache = {}     # id(tensor) -> (weak reference to that tensor, its version when read, value)
+
+
+def _scalar(x):
+    """Python float of a scalar operand: a number, or a one-element tensor that needs no gradient (the margin
+    gamma is nn.Parameter(torch.Tensor([gamma]), requires_grad=False), models/kg_reasoning.py:97-100).  The value
+    of such a tensor is read from the device once per version of the tensor, not once per step; the entry holds a
+    weak reference, so it can never answer for another tensor that later gets the same id.  None: not a scalar."""
+    if isinstance(x, bool):
+        return None
+    if isinstance(x, numbers.Real):
+        return float(x)
+    if isinstance(x, torch.Tensor) and x.numel() == 1 and not x.requires_grad and not _is_lazy(x):
+        hit = _scalar_cache.get(id(x))
+        if hit is None or hit[0]() is not x or hit[1] != x._version:
+            key = id(x)
+            ref = weakref.ref(x, lambda _, key=key: _scalar_cache.pop(key, None))
+            hit = (ref, x._version, float(x.detach().reshape(()).item()))
+            _scalar_cache[key] = hit
+        return hit[2]
+    return None
+
+
+class _Delegating:
+    """Everything a handle does not know about is done by the tensor it stands for."""
+
+    def materialize(self):
+        raise NotImplementedError
+
+    @classmethod
+    def __torch_function__(cls, func, types, args=(), kwargs=None):
+        kwargs = kwargs or {}
+        handled = cls._try_lazy(func, args, kwargs)
+        if handled is not NotImplemented:
+            return handled
+        return func(*_resolve(args), **_resolve(kwargs))
+
+    @classmethod
+    def _try_lazy(cls, func, args, kwargs):
+        return NotImplemented
+
+    def __getattr__(self, name):
+        if name.startswith("__") and name.endswith("__"):
+            raise AttributeError(name)
+        return getattr(self.materialize(), name)
+
+    def __getitem__(self, key):
+        return self.materialize()[key]
+
+    def __len__(self):
+        return self.shape[0]
+
+    def __iter__(self):
+        return iter(self.materialize())
+
+    def __repr__(self):
+        return f"{type(self).__name__}(shape={tuple(self.shape)})"
+
+
+def _binary(name, reflected=False):
+    def op(self, other):
+        a, b = self.materialize(), _resolve(other)
+        return getattr(torch, name)(b, a) if reflected else getattr(torch, name)(a, b)
+    return op
+
+
+class LazyRows(_Delegating):
+    """rows-of(table, ids): logical shape ids.shape + (row,), optionally viewed / unsqueezed, optionally carrying the
+    entity prologue clamp(rows + add, lo, hi) of smore/common/modules.py:29-36."""
+
+    def __init__(self, opt, ids, name, shape=None, reg=None, pending_add=None, root=None):
+        self.opt, self.ids, self.name = opt, ids, name
+        row = opt.sparse_embed.embedding.shape[1]
+        self.shape = torch.Size(tuple(ids.shape) + (row,)) if shape is None else torch.Size(shape)
+        self.reg = reg                    # (add, lo, hi) once the clamp has been seen
+        self.pending_add = pending_add    # `rows + c` that has not met its clamp yet
+        self.root = root if root is not None else self
+        self.job_handle = opt.sparse_embed.dummy_job
+        if root is None:
+            self._looked_up = None        # the plain lookup, made at most once per handle family
+
+    # -- what the model code asks of a tensor before any value is needed
+    device = property(lambda self: self.opt.sparse_embed.embedding.device)
+    dtype = property(lambda self: self.opt.sparse_embed.embedding.dtype)
+    requires_grad = True
+    is_cuda = True
+
+    def dim(self):
+        return len(self.shape)
+
+    ndim = property(dim)
+
+    def size(self, d=None):
+        return self.shape if d is None else self.shape[d]
+
+    def numel(self):
+        return self.shape.numel()
+
+    def is_contiguous(self):
+        return True
+
+    def contiguous(self):
+        return self
+
+    def _like(self, shape):
+        return LazyRows(self.opt, self.ids, self.name, shape, self.reg, self.pending_add, self.root)
+
+    def view(self, *shape):
+        if len(shape) == 1 and isinstance(shape[0], (tuple, list, torch.Size)):
+            shape = tuple(shape[0])
+        shape = list(shape)
+        if shape.count(-1) > 1 or any(not isinstance(s, int) for s in shape):
+            return self.materialize().view(*shape)
+        total = self.shape.numel()
+        known = 1
+        for s in shape:
+            known *= s if s != -1 else 1
+        if -1 in shape:
+            if known == 0 or total % known:
+                raise RuntimeError(f"shape {shape} is invalid for input of size {total}")
+            shape[shape.index(-1)] = total // known
+        elif known != total:
+            raise RuntimeError(f"shape {shape} is invalid for input of size {total}")
+        if shape[-1] != self.shape[-1]:          # rows are split or joined: values are needed
+            return self.materialize().view(*shape)
+        return self._like(shape)
+
+    reshape = view
+
+    def unsqueeze(self, d):
+        n = len(self.shape)
+        d = d + n + 1 if d < 0 else d
+        if d > n - 1:                            # a new last dimension is no longer a stack of rows
+            return self.materialize().unsqueeze(d)
+        return self._like(tuple(self.shape[:d]) + (1,) + tuple(self.shape[d:]))
+
+    def __add__(self, other):
+        c = _scalar(other)
+        if c is None or self.reg is not None or self.pending_add is not None:
+            return torch.add(self.materialize(), _resolve(other))
+        out = self._like(self.shape)
+        out.pending_add = c
+        return out
+
+    __radd__ = __add__
+    __sub__ = _binary("sub")
+    __rsub__ = _binary("sub", True)
+    __mul__ = _binary("mul")
+    __rmul__ = _binary("mul", True)
+    __truediv__ = _binary("div")
+    __rtruediv__ = _binary("div", True)
+    __matmul__ = _binary("matmul")
+    __pow__ = _binary("pow")
+
+    def __neg__(self):
+        return -self.materialize()
+
+    @classmethod
+    def _try_lazy(cls, func, args, kwargs):
+        name = _func_name(func)
+        if name == "clamp" and args and isinstance(args[0], LazyRows):
+            x = args[0]
+            lo = kwargs.get("min", args[1] if len(args) > 1 else None)
+            hi = kwargs.get("max", args[2] if len(args) > 2 else None)
+            lo, hi = _scalar(lo), _scalar(hi)
+            if x.reg is None and lo is not None and hi is not None:
+                out = x._like(x.shape)
+                out.reg = (x.pending_add or 0.0, lo, hi)
+                out.pending_add = None
+                return out
+        if name in ("add", "__add__", "__radd__") and len(args) == 2 and not kwargs:
+            rows, other = (args[0], args[1]) if isinstance(args[0], LazyRows) else (args[1], args[0])
+            if isinstance(rows, LazyRows) and _scalar(other) is not None:
+                return rows.__add__(other)
+        return NotImplemented
+
+    def materialize(self):
+        """The plain lookup (one per handle family, through the optimizer's autograd node), then whatever views
+        and prologue this handle carries, as torch operations."""
+        root = self.root
+        if root._looked_up is None:
+            root._looked_up = self.opt.lookup_rows(self.ids, self.name)
+        rows = root._looked_up.view(self.shape)
+        if self.pending_add is not None:
+            rows = rows + self.pending_add
+        if self.reg is not None:
+            rows = torch.clamp(rows + self.reg[0], self.reg[1], self.reg[2])
+        return rows
+
+
+class _Dist:
+    """dist(kind, rows handle, query tensors), not yet evaluated."""
+
+    def __init__(self, kind, rows, queries):
+        self.kind, self.rows, self.queries = kind, rows, tuple(queries)
+
+    def same_operands(self, other):
+        return (self.rows.root is other.rows.root and self.rows.shape == other.rows.shape and
+                self.rows.reg == other.rows.reg and self.rows.pending_add == other.rows.pending_add and
+                len(self.queries) == len(other.queries) and all(a is b for a, b in zip(self.queries, other.queries)))
+
+    def out_shape(self):
+        q, e = self.queries[0], self.rows
+        if q.dim() == 4:
+            return torch.Size((max(e.shape[0], q.shape[0]), q.shape[1], max(e.shape[1], q.shape[2])))
+        return torch.Size((max(e.shape[0], q.shape[0]), max(e.shape[1], q.shape[1])))
+
+    def dense(self):
+        from ..torchext.dist_func import _base
+        rows = self.rows.materialize().contiguous()
+        if self.kind == "l2":
+            return torch.sqrt(_base.apply_dist("l2", rows, *self.queries))
+        return _base.apply_dist(self.kind, rows, *self.queries)
+
+
+class LazyLogit(_Delegating):
+    """const + sum coef_i * dist_i over unevaluated distances; scalar arithmetic keeps it lazy."""
+
+    def __init__(self, const, terms):
+        self.const, self.terms = float(const), list(terms)
+        self._value = None
+
+    @staticmethod
+    def of(kind, rows, queries):
+        return LazyLogit(0.0, [(1.0, _Dist(kind, rows, queries))])
+
+    shape = property(lambda self: self.terms[0][1].out_shape())
+    device = property(lambda self: self.terms[0][1].rows.device)
+    dtype = torch.float32
+
+    def dim(self):
+        return len(self.shape)
+
+    def size(self, d=None):
+        return self.shape if d is None else self.shape[d]
+
+    # -- arithmetic that keeps the expression lazy
+    def _scaled(self, c):
+        return LazyLogit(self.const * c, [(k * c, d) for k, d in self.terms])
+
+    def _plus(self, other, sign):
+        if isinstance(other, LazyLogit):
+            return LazyLogit(self.const + sign * other.const, self.terms + [(sign * k, d) for k, d in other.terms])
+        c = _scalar(other)
+        if c is None:
+            return NotImplemented
+        return LazyLogit(self.const + sign * c, self.terms)
+
+    def __neg__(self):
+        return self._scaled(-1.0)
+
+    def __add__(self, other):
+        out = self._plus(other, 1.0)
+        return torch.add(self.materialize(), _resolve(other)) if out is NotImplemented else out
+
+    __radd__ = __add__
+
+    def __sub__(self, other):
+        out = self._plus(other, -1.0)
+        return torch.sub(self.materialize(), _resolve(other)) if out is NotImplemented else out
+
+    def __rsub__(self, other):
+        out = self._scaled(-1.0)._plus(other, 1.0)
+        return torch.sub(_resolve(other), self.materialize()) if out is NotImplemented else out
+
+    def __mul__(self, other):
+        c = _scalar(other)
+        return torch.mul(self.materialize(), _resolve(other)) if c is None else self._scaled(c)
+
+    __rmul__ = __mul__
+
+    def __truediv__(self, other):
+        c = _scalar(other)
+        return torch.div(self.materialize(), _resolve(other)) if c is None or c == 0.0 else self._scaled(1.0 / c)
+
+    @classmethod
+    def _try_lazy(cls, func, args, kwargs):
+        name = _func_name(func)
+        if len(args) == 2 and not kwargs:
+            a, b = args
+            if name in ("rsub", "__rsub__"):            # other - input
+                a, b, name = b, a, "sub"
+            lazy_first = isinstance(a, LazyLogit)
+            if name in ("add", "__add__", "__radd__"):
+                return a.__add__(b) if lazy_first else b.__add__(a)
+            if name in ("sub", "subtract", "__sub__"):
+                return a.__sub__(b) if lazy_first else b.__rsub__(a)
+            if name in ("mul", "multiply", "__mul__", "__rmul__"):
+                return a.__mul__(b) if lazy_first else b.__mul__(a)
+        if name in ("neg", "negative", "__neg__") and len(args) == 1 and not kwargs:
+            return -args[0]
+        return NotImplemented
+
+    # -- evaluation
+    def _fusable(self):
+        """(model, cen) when the expression is one of the logits the fused scorer computes, else None."""
+        if len(self.terms) == 1:
+            k, d = self.terms[0]
+            if k == -1.0 and d.kind in _FUSED_MODEL:
+                return _FUSED_MODEL[d.kind], 0.0
+            if k == -1.0 and d.kind == "box_out":
+                return "box", 0.0
+        if len(self.terms) == 2:
+            (k0, d0), (k1, d1) = self.terms
+            if d0.kind == "box_in":
+                (k0, d0), (k1, d1) = (k1, d1), (k0, d0)
+            if d0.kind == "box_out" and d1.kind == "box_in" and k0 == -1.0 and d0.same_operands(d1):
+                return "box", -k1
+        return None
+
+    def materialize(self):
+        if self._value is not None:
+            return self._value
+        fused = self._fusable()
+        value = None
+        if fused is not None:
+            model, cen = fused
+            d = self.terms[0][1]
+            value = d.rows.opt.score_lazy(model, d.rows, d.queries, self.const, cen)
+        if value is None:      # not a shape the fused scorer takes: plain lookup + dense operators
+            value = self.const
+            for k, d in self.terms:
+                value = value + k * d.dense()
+        self._value = value
+        return value
+
+
+def lazy_dist(kind, entity_embed, *queries):
+    """What an operator of ext_ops returns for a LazyRows entity argument."""
+    if kind not in ("l1", "l2", "rotate", "beta_kl", "box_out", "box_in"):
+        return None
+    if any(_is_lazy(q) or not isinstance(q, torch.Tensor) for q in queries):
+        return None
+    if entity_embed.dim() != 3 or entity_embed.pending_add is not None:
+        return None
+    q = queries[0]
+    if q.dim() not in (3, 4) or any(x.shape != q.shape for x in queries[1:]):
+        return None
+    return LazyLogit.of(kind, entity_embed, queries)

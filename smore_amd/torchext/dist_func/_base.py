@@ -15,6 +15,7 @@ the per-operator Functions of smore/common/torchext/dist_func/*.py:
 import torch
 
 from ... import extlib_hip as extlib
+from ...embedding.lazy_rows import LazyRows, lazy_dist
 
 TWO_HALVES = ("rotate", "complex", "beta_kl", "beta_l2", "beta_fisher_approx")
 
@@ -57,7 +58,14 @@ class DistFunction(torch.autograd.Function):
 
 
 def apply_dist(kind, entity_embed, *queries):
-    """3-D or (query) 4-D front end shared by every operator."""
+    """3-D or (query) 4-D front end shared by every operator.  An entity argument that is a lazy lookup handle
+    (what sp_embed(ids) returns while an EmbeddingOptimizer is attached) gives a lazy distance: the table rows are
+    then read by the gather-fused scorer when the logit is needed, never as a [B,K,row] tensor."""
+    if isinstance(entity_embed, LazyRows):
+        lazy = lazy_dist(kind, entity_embed, *queries) if kind != "l2" else None   # "l2" here is the squared distance
+        if lazy is not None:
+            return lazy
+        entity_embed = entity_embed.materialize().contiguous()
     first = queries[0]
     if entity_embed.dim() != first.dim():
         assert first.dim() == 4

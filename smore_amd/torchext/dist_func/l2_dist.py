@@ -5,6 +5,7 @@ here, outside the Function, so autograd supplies g / (2 sqrt(d2)) -- infinite
 at d2 == 0, exactly as in the reference (l2_dist.py:59,62)."""
 import torch
 
+from ...embedding.lazy_rows import LazyRows, lazy_dist
 from ._base import apply_dist
 
 
@@ -13,6 +14,10 @@ def l2_sqr_dist(entity_embed, center_embed):
 
 
 def l2_dist(entity_embed, center_embed):
+    if isinstance(entity_embed, LazyRows):     # a lazy lookup: the fused scorer has the rooted distance as a model
+        lazy = lazy_dist("l2", entity_embed, center_embed)
+        if lazy is not None:
+            return lazy
     return torch.sqrt(l2_sqr_dist(entity_embed, center_embed))
 
 

@@ -1,0 +1,283 @@
+"""Unchanged model code on the fused path.
+
+The classes below are a few-line restatement, written for this test, of how SMORE's models reach the scoring
+path: the lookup / view / regularizer / cal_logit sequence of KGReasoning.forward (kg_reasoning.py:298-307,
+340-355) and the four custom_cal_logit bodies (box.py:157-164, vec.py:85-90, rotate.py:137-142, beta.py:303-308).
+They call only sp_embed(ids, name), tensor methods and ext_ops -- no score_negatives -- and must get, through the
+lazy lookup handle, the gather-fused scorer, with logits, query gradients and Adam state equal to the float64
+oracle's."""
+import types
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle as orc
+from tests.util import REL_F32, assert_adam_weights, assert_close
+
+pytestmark = pytest.mark.gpu
+
+
+class Reasoner(torch.nn.Module):
+    def __init__(self, entity_embedding, gamma):
+        super().__init__()
+        self.entity_embedding = entity_embedding
+        self.gamma = torch.nn.Parameter(torch.Tensor([gamma]), requires_grad=False)
+
+    def entity_regularizer(self, embedding):
+        return embedding
+
+    def forward(self, positive_sample, negative_sample, query_embedding):
+        all_positive = self.entity_embedding(positive_sample, "positive_entity")
+        batch_size, negative_size = negative_sample.shape
+        all_negative = self.entity_embedding(negative_sample.view(-1), "negative_entity")
+        all_positive.job_handle.sync()
+        all_positive = self.entity_regularizer(all_positive)
+        positive_logits = self.cal_logit(all_positive.unsqueeze(1), None, query_embedding)
+        all_negative.job_handle.sync()
+        all_negative = self.entity_regularizer(all_negative.view(batch_size, negative_size, -1))
+        negative_logits = self.cal_logit(all_negative, None, query_embedding)
+        return positive_logits, negative_logits
+
+
+class Box(Reasoner):
+    cen = 0.02
+
+    def cal_logit(self, entity_embedding, entity_feat, query_embedding):
+        from smore_amd.torchext.ext_ops import box_dist_in, box_dist_out
+        assert entity_feat is None
+        center, offset = query_embedding
+        d1 = box_dist_out(entity_embedding, center, offset)
+        d2 = box_dist_in(entity_embedding, center, offset)
+        logit = self.gamma - d1 - self.cen * d2
+        return torch.max(logit, dim=1)[0]
+
+
+class Vec(Reasoner):
+    def __init__(self, entity_embedding, gamma, mode):
+        super().__init__(entity_embedding, gamma)
+        from smore_amd.torchext import ext_ops
+        self.dist_func = getattr(ext_ops, mode + "_dist")
+
+    def cal_logit(self, entity_embedding, entity_feat, query_embedding):
+        assert entity_feat is None
+        logit = self.gamma - self.dist_func(entity_embedding, query_embedding[0])
+        return torch.max(logit, dim=1)[0]
+
+
+class Rotate(Reasoner):
+    def cal_logit(self, entity_embedding, entity_feat, query_embedding):
+        from smore_amd.torchext.ext_ops import rotate_dist
+        assert entity_feat is None
+        re, im = query_embedding
+        logit = self.gamma - rotate_dist(entity_embedding, re, im)
+        return torch.max(logit, dim=1)[0]
+
+
+class Beta(Reasoner):
+    def entity_regularizer(self, embedding):      # Regularizer(1, 0.05, 1e9), beta.py:210, modules.py:29-36
+        return torch.clamp(embedding + 1.0, 0.05, 1e9)
+
+    def cal_logit(self, entity_embedding, entity_feat, query_embedding):
+        from smore_amd.torchext.ext_ops import BetaDist, beta_kl
+        assert entity_feat is None
+        logit = self.gamma - beta_kl(entity_embedding, BetaDist(*query_embedding))
+        return torch.max(logit, dim=1)[0]
+
+
+CASES = {
+    # name: (class, extra ctor args, fused model, queries per branch, row / dim, gamma, cen)
+    "box": (Box, (), "box", 2, 1, 24.0, 0.02),
+    "l1": (Vec, ("l1",), "l1", 1, 1, 12.0, 0.0),
+    "l2": (Vec, ("l2",), "l2", 1, 1, 12.0, 0.0),
+    "rotate": (Rotate, (), "rotate", 2, 2, 9.0, 0.0),
+    "beta": (Beta, (), "beta_kl", 2, 2, 60.0, 0.0),
+}
+
+
+def _table_and_queries(name, n, d, b, u, rng):
+    mul = CASES[name][4]
+    n_q = CASES[name][3]
+    if name == "beta":
+        table = rng.standard_normal((n, 2 * d)) * 1.5           # raw values; the regularizer clamps some
+        pos = lambda *s: np.clip(1 + rng.standard_normal(s), 0.05, 1e9)
+        qs = [pos(b, u, 1, d) for _ in range(n_q)]
+    else:
+        table = rng.uniform(-0.07, 0.07, (n, mul * d))
+        qs = [rng.uniform(-0.07, 0.07, (b, u, 1, d)) for _ in range(n_q)]
+        if name == "box":
+            qs[1] = np.abs(qs[1])
+    f32 = lambda a: a.astype(np.float32).astype(np.float64)
+    return f32(table), [f32(q) for q in qs]
+
+
+def _oracle_branch_logits(name, table, ids, qs, gamma, cen):
+    """[B,U,K] float64 logits and the rows they were computed from."""
+    model = CASES[name][2]
+    b, k = ids.shape
+    src = orc.regularizer(table) if name == "beta" else table
+    rows = orc.gather(src, ids).reshape(b, k, -1)
+    u = qs[0].shape[1]
+    logit = np.stack([orc.score_forward(model, rows, qs[0][:, j], qs[1][:, j] if len(qs) > 1 else None, gamma, cen)
+                      for j in range(u)], axis=1)
+    return logit, rows
+
+
+def _oracle_grads(name, table, ids, qs, rows, logit, gout, cen):
+    """Upstream gradient gout [B,K] on max over branches -> (entity gradient rows [B*K,row], [query grads])."""
+    model = CASES[name][2]
+    b, k = ids.shape
+    u = logit.shape[1]
+    win = np.argmax(logit, axis=1)                                        # first maximum, as torch.max
+    g_rows = np.zeros((b, k, rows.shape[-1]))
+    g_qs = [np.zeros_like(q) for q in qs]
+    for j in range(u):
+        gj = np.where(win == j, gout, 0.0)
+        gr, g1, g2 = orc.score_backward(model, gj, rows, qs[0][:, j], qs[1][:, j] if len(qs) > 1 else None, cen)
+        g_rows += gr
+        g_qs[0][:, j] = g1
+        if len(qs) > 1:
+            g_qs[1][:, j] = g2
+    g_rows = g_rows.reshape(b * k, -1)
+    if name == "beta":
+        raw = orc.gather(table, ids)
+        g_rows = g_rows * ((raw + 1 >= 0.05) & (raw + 1 <= 1e9))
+    return g_rows, g_qs
+
+
+@pytest.mark.parametrize("name", list(CASES))
+@pytest.mark.parametrize("branches", [1, 2])
+def test_model_code_without_score_negatives_matches_oracle(name, branches):
+    from smore_amd.embedding.embed_optimizer import AdamEmbedOptimizer
+    from smore_amd.embedding.sparse_embed import SparseEmbedding
+    cls, extra, model, n_q, mul, gamma, cen = CASES[name]
+    n, d, b, k, lr = 400, 32, 6, 24, 1e-3
+    rng = np.random.default_rng(11 + branches)
+    table, qs = _table_and_queries(name, n, d, b, branches, rng)
+    emb = SparseEmbedding(n, mul * d).cuda()
+    with torch.no_grad():
+        emb.embedding.copy_(torch.tensor(table, dtype=torch.float32))
+    opt = AdamEmbedOptimizer(types.SimpleNamespace(optim_mode="(aggr,adam,gpu,False,5)", share_optim_stats=True), emb, 0)
+    net = cls(emb, gamma, *extra).cuda()
+    t_qs = [torch.tensor(q, dtype=torch.float32, device="cuda", requires_grad=True) for q in qs]
+    w, m, v = table.copy(), np.zeros_like(table), np.zeros_like(table)
+    for step in (1, 2):
+        pos = rng.integers(0, n, b)
+        neg = rng.integers(0, n // 4, (b, k))                             # repeated ids: real segments
+        gp = rng.standard_normal((b, 1)).astype(np.float32).astype(np.float64)
+        gn = rng.standard_normal((b, k)).astype(np.float32).astype(np.float64)
+        opt.zero_grad()
+        for t in t_qs:
+            t.grad = None
+        lp, ln = net(torch.tensor(pos, device="cuda"), torch.tensor(neg, device="cuda"), t_qs)
+        assert lp.shape == (b, 1) and ln.shape == (b, k)
+        ((lp * torch.tensor(gp, dtype=torch.float32, device="cuda")).sum() +
+         (ln * torch.tensor(gn, dtype=torch.float32, device="cuda")).sum()).backward()
+        assert len(opt.fused_list) == 2 and not opt.grad_list, "both lookups must have stayed on the fused scorer"
+        opt.apply_grad(lr)
+
+        o_lp, rows_p = _oracle_branch_logits(name, w, pos.reshape(b, 1), qs, gamma, cen)
+        o_ln, rows_n = _oracle_branch_logits(name, w, neg, qs, gamma, cen)
+        assert_close(lp.detach().cpu().numpy(), o_lp.max(axis=1), REL_F32, f"{name} positive logits, step {step}")
+        assert_close(ln.detach().cpu().numpy(), o_ln.max(axis=1), REL_F32, f"{name} negative logits, step {step}")
+        gr_p, gq_p = _oracle_grads(name, w, pos.reshape(b, 1), qs, rows_p, o_lp, gp, cen)
+        gr_n, gq_n = _oracle_grads(name, w, neg, qs, rows_n, o_ln, gn, cen)
+        for t, a, c in zip(t_qs, gq_p, gq_n):
+            assert_close(t.grad.cpu().numpy(), a + c, REL_F32, f"{name} query gradient, step {step}")
+        all_idx = np.concatenate([pos.reshape(-1), neg.reshape(-1)])
+        uniq, inverse, _, _ = orc.merge_indices(all_idx)
+        merged = orc.merge_grads(np.concatenate([gr_p, gr_n]), inverse, uniq.size)
+        w_before = w.copy()
+        orc.adam_rows(w, m, v, uniq, merged, lr, step)
+        got = emb.embedding.detach().cpu().numpy().astype(np.float64)
+        touched = np.zeros(n, bool)
+        touched[uniq] = True
+        assert np.array_equal(got[~touched], w_before[~touched]), "rows outside the step must keep their bits"
+        assert_close(emb.state_sum_fo.cpu().numpy()[touched], m[touched], REL_F32, f"{name} first moment, step {step}")
+        assert_close(emb.state_sum_sq.cpu().numpy()[touched], v[touched], REL_F32, f"{name} second moment, step {step}")
+        assert_adam_weights(got, w, merged, uniq, lr, f"{name} weights, step {step}")
+        w = got.copy()   # continue from the device's fp32 weights so that step 2 compares one step, not two
+        m = emb.state_sum_fo.cpu().numpy().astype(np.float64)
+        v = emb.state_sum_sq.cpu().numpy().astype(np.float64)
+
+
+def test_negatives_only_step_is_the_one_record_fast_path():
+    """The cfg5 call shape: negatives only.  The lazy route must leave exactly one fused record (plan + fused
+    entity pass, no gradient rows) and give the bits of the explicit score_negatives call."""
+    from smore_amd.embedding.embed_optimizer import AdamEmbedOptimizer
+    from smore_amd.embedding.sparse_embed import SparseEmbedding
+    n, d, b, k, lr = 3000, 200, 16, 64, 1e-4
+    rng = np.random.default_rng(5)
+    neg = torch.tensor(np.minimum(rng.zipf(1.3, (b, k)) - 1, n - 1), device="cuda")
+    cn = rng.uniform(-0.07, 0.07, (b, 1, 1, d)).astype(np.float32)
+    on = np.abs(rng.uniform(-0.07, 0.07, (b, 1, 1, d))).astype(np.float32)
+    gn = torch.tensor(rng.standard_normal((b, k)).astype(np.float32), device="cuda")
+
+    def run(lazy):
+        torch.manual_seed(3)
+        emb = SparseEmbedding(n, d).cuda()
+        emb.init_params(-0.07, 0.07)
+        opt = AdamEmbedOptimizer(types.SimpleNamespace(optim_mode="(aggr,adam,gpu,False,5)", share_optim_stats=True), emb, 0)
+        net = Box(emb, 24.0).cuda()
+        c = torch.tensor(cn, device="cuda", requires_grad=True)
+        o = torch.tensor(on, device="cuda", requires_grad=True)
+        for _ in range(2):
+            opt.zero_grad()
+            c.grad = o.grad = None
+            if lazy:
+                rows = emb(neg.view(-1), "negative_entity")
+                rows.job_handle.sync()
+                ln = net.cal_logit(net.entity_regularizer(rows.view(b, k, -1)), None, [c, o])
+            else:
+                ln = opt.score_negatives("box", neg, c, o, gamma=24.0, cen=0.02)
+            (ln * gn).sum().backward()
+            assert len(opt.fused_list) == 1 and not opt.grad_list
+            opt.apply_grad(lr)
+        return [x.detach().cpu() for x in (ln, c.grad, o.grad, emb.embedding, emb.state_sum_fo, emb.state_sum_sq)]
+
+    for a, r in zip(run(True), run(False)):
+        assert torch.equal(a, r)
+
+
+def test_shared_negatives_and_other_uses_of_the_rows():
+    """--share_negative: negative_sample is [1,K] (online_sampler.py:155-157), so batch_size = 1 in the model code
+    and the operators broadcast the K rows over the B queries.  cal_reg (kg_reasoning.py:149-152) also wants the
+    rows' values: the handle then looks them up once, and the step merges the two records."""
+    from smore_amd.embedding.embed_optimizer import AdamEmbedOptimizer
+    from smore_amd.embedding.sparse_embed import SparseEmbedding
+    n, d, b, k, lr = 300, 16, 5, 12, 1e-3
+    rng = np.random.default_rng(8)
+    table = rng.uniform(-0.07, 0.07, (n, d)).astype(np.float32).astype(np.float64)
+    q = rng.uniform(-0.07, 0.07, (b, 1, 1, d)).astype(np.float32).astype(np.float64)
+    neg = rng.integers(0, n, (1, k))
+    gn = rng.standard_normal((b, k)).astype(np.float32).astype(np.float64)
+    emb = SparseEmbedding(n, d).cuda()
+    with torch.no_grad():
+        emb.embedding.copy_(torch.tensor(table, dtype=torch.float32))
+    opt = AdamEmbedOptimizer(types.SimpleNamespace(optim_mode="(aggr,adam,gpu,False,5)", share_optim_stats=True), emb, 0)
+    net = Vec(emb, 12.0, "l1").cuda()
+    tq = torch.tensor(q, dtype=torch.float32, device="cuda", requires_grad=True)
+    opt.zero_grad()
+    t_neg = torch.tensor(neg, device="cuda")
+    rows = emb(t_neg.view(-1), "negative_entity")
+    ln = net.cal_logit(rows.view(1, k, -1), None, [tq])
+    assert ln.shape == (b, k)
+    reg = torch.norm(rows, p=3) ** 3
+    ((ln * torch.tensor(gn, dtype=torch.float32, device="cuda")).sum() + 0.5 * reg).backward()
+    assert len(opt.fused_list) == 1 and len(opt.grad_list) == 1
+    opt.apply_grad(lr)
+
+    ids_full = np.broadcast_to(neg, (b, k))
+    o_rows = orc.gather(table, ids_full).reshape(b, k, d)
+    assert_close(ln.detach().cpu().numpy(), orc.score_forward("l1", o_rows, q[:, 0], None, 12.0), REL_F32, "logits")
+    g_rows, g_q, _ = orc.score_backward("l1", gn, o_rows, q[:, 0], None)
+    assert_close(tq.grad.cpu().numpy()[:, 0], g_q, REL_F32, "query gradient")
+    r = orc.gather(table, neg)
+    g_reg = 0.5 * 3.0 * np.abs(r) * r                                       # d/dx |x|^3 = 3 |x| x
+    all_idx = np.concatenate([ids_full.reshape(-1), neg.reshape(-1)])
+    uniq, inverse, _, _ = orc.merge_indices(all_idx)
+    merged = orc.merge_grads(np.concatenate([g_rows.reshape(b * k, d), g_reg]), inverse, uniq.size)
+    w, m, v = table.copy(), np.zeros_like(table), np.zeros_like(table)
+    orc.adam_rows(w, m, v, uniq, merged, lr, 1)
+    assert_close(emb.state_sum_fo.cpu().numpy()[uniq], m[uniq], REL_F32, "first moment")
+    assert_adam_weights(emb.embedding.detach().cpu().numpy(), w, merged, uniq, lr, "weights")

@@ -20,6 +20,7 @@ def _setup(n, d, seed):
     emb.init_params(-0.07, 0.07)
     args = types.SimpleNamespace(optim_mode="(aggr,adam,gpu,False,5)", share_optim_stats=True)
     opt = AdamEmbedOptimizer(args, emb, 0)
+    opt.lazy_lookup = False    # these tests use sp_embed(ids) for the plain lookup + dense operators (the lazy route: test_dropin_gpu.py)
     return emb, opt
 
 
@@ -276,6 +277,27 @@ def test_out_of_range_lookup_is_reported():
     emb(torch.tensor([1, 25], device="cuda"), "x")
     with pytest.raises(IndexError):
         opt.check_ids()
+
+
+def test_out_of_range_id_in_a_step_raises_from_the_next_apply_grad():
+    """The per-step check does not wait for the device: the flag of step n is read when step n+1 reaches
+    apply_grad.  The bad pair itself updates no row (its key sorts behind every real segment)."""
+    emb, opt = _setup(20, 8, 9)
+    c = torch.zeros(2, 1, 8, device="cuda", requires_grad=True)
+    o = torch.ones(2, 1, 8, device="cuda", requires_grad=True)
+    w0 = emb.embedding.detach().clone()
+    for step, ids in enumerate(([[1, 25], [2, 3]], [[4, 5], [6, 7]])):
+        opt.zero_grad()
+        ln = opt.score_negatives("box", torch.tensor(ids, device="cuda"), c, o, gamma=1.0, cen=0.02)
+        ln.sum().backward()
+        if step == 0:
+            opt.apply_grad(1e-3)
+        else:
+            with pytest.raises(IndexError):
+                opt.apply_grad(1e-3)
+    changed = (emb.embedding.detach() != w0).any(dim=1).nonzero().flatten().tolist()
+    assert changed == [1, 2, 3, 4, 5, 6, 7]
+    opt.check_ids()       # the flag was cleared when the error was raised
 
 
 def test_state_buffers_are_in_the_state_dict():
