@@ -244,8 +244,12 @@ int smx_score_backward_entity(int model, void* stream, const smx_plan_view* plan
  * smx_score_backward_entity would do -- except that rows of ids occurring once in the step are
  * finished by the query-gradient kernel itself, which already holds the query in registers and has
  * just read the entity row; the entity pass then skips them.  The plan must have been built with
- * pair_seg.  Same results as the two separate calls up to fp32 rounding (the one-pair rows are computed
- * by a different kernel, so a multiply-add may be contracted differently).
+ * pair_seg.  Against the two separate calls: query gradients and the w, m, v rows of the sign-coded models
+ * (box, l1) are the same bits -- same decisions, same +-c terms, same order, and the row update is written
+ * with explicit fused multiply-adds, so it does not depend on the kernel that runs it.  For l2, rotate and
+ * beta_kl the gradient of a one-pair row is formed by the query-gradient kernel instead of the entity pass,
+ * whose multiply-adds the compiler contracts differently: merged gradient rows agree to a few units of the
+ * last place (the tests bound the difference by 1e-6 relative).
  * workspace: smx_fused_workspace_bytes (below).  No counterpart as one function in the reference:
  * it stands for dist_backward (extlib_cuda.cpp:230-262) + EmbedLookupFunc.backward +
  * EmbeddingOptimizer.apply_grad (embed_optimizer.py:63-66,155-163). */

@@ -27,3 +27,20 @@ def pytest_collection_modifyitems(config, items):
     for item in items:
         if "gpu" in item.keywords:
             item.add_marker(skip)
+
+
+def pytest_terminal_summary(terminalreporter, exitstatus, config):
+    """Tolerance headroom: worst err/bound of every tensor compared through tests.util.assert_close in this
+    run, against the bound in force and against the purely elementwise relative bound."""
+    from tests import util
+    if not util.HEADROOM:
+        return
+    terminalreporter.section("tolerance headroom (worst err/bound per compared tensor)")
+    rows = sorted(util.HEADROOM.items(), key=lambda kv: -kv[1][0])
+    for (test, what), (with_floor, pure) in rows:
+        terminalreporter.write_line(f"{with_floor:9.3g} {pure:9.3g}  {test} :: {what}")
+    out_dir = os.path.join(ROOT, "gpurun_out")
+    if os.path.isdir(out_dir):
+        import json
+        with open(os.path.join(out_dir, "headroom.json"), "w") as f:
+            json.dump([[t, w, a, b] for (t, w), (a, b) in rows], f, indent=0)

@@ -13,7 +13,7 @@ import pytest
 import torch
 
 from oracle import oracle as orc
-from tests.util import REL_F32, assert_adam_weights, assert_close
+from tests.util import REL_F32, assert_adam_weights, assert_close, oracle_union_grads, oracle_union_logits
 
 pytestmark = pytest.mark.gpu
 
@@ -112,37 +112,11 @@ def _table_and_queries(name, n, d, b, u, rng):
 
 
 def _oracle_branch_logits(name, table, ids, qs, gamma, cen):
-    """[B,U,K] float64 logits and the rows they were computed from."""
-    model = CASES[name][2]
-    b, k = ids.shape
-    src = orc.regularizer(table) if name == "beta" else table
-    rows = orc.gather(src, ids).reshape(b, k, -1)
-    u = qs[0].shape[1]
-    logit = np.stack([orc.score_forward(model, rows, qs[0][:, j], qs[1][:, j] if len(qs) > 1 else None, gamma, cen)
-                      for j in range(u)], axis=1)
-    return logit, rows
+    return oracle_union_logits(CASES[name][2], table, ids, qs, gamma, cen, regularizer=name == "beta")
 
 
 def _oracle_grads(name, table, ids, qs, rows, logit, gout, cen):
-    """Upstream gradient gout [B,K] on max over branches -> (entity gradient rows [B*K,row], [query grads])."""
-    model = CASES[name][2]
-    b, k = ids.shape
-    u = logit.shape[1]
-    win = np.argmax(logit, axis=1)                                        # first maximum, as torch.max
-    g_rows = np.zeros((b, k, rows.shape[-1]))
-    g_qs = [np.zeros_like(q) for q in qs]
-    for j in range(u):
-        gj = np.where(win == j, gout, 0.0)
-        gr, g1, g2 = orc.score_backward(model, gj, rows, qs[0][:, j], qs[1][:, j] if len(qs) > 1 else None, cen)
-        g_rows += gr
-        g_qs[0][:, j] = g1
-        if len(qs) > 1:
-            g_qs[1][:, j] = g2
-    g_rows = g_rows.reshape(b * k, -1)
-    if name == "beta":
-        raw = orc.gather(table, ids)
-        g_rows = g_rows * ((raw + 1 >= 0.05) & (raw + 1 <= 1e9))
-    return g_rows, g_qs
+    return oracle_union_grads(CASES[name][2], table, ids, qs, rows, logit, gout, cen, regularizer=name == "beta")
 
 
 @pytest.mark.parametrize("name", list(CASES))

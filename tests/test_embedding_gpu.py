@@ -7,7 +7,8 @@ import pytest
 import torch
 
 from oracle import oracle as orc
-from tests.util import REL_F32, assert_close
+from tests.util import (REL_F32, assert_adam_weights, assert_close, oracle_adam_step, oracle_union_grads,
+                        oracle_union_logits)
 
 pytestmark = pytest.mark.gpu
 
@@ -144,6 +145,7 @@ def test_shared_negatives_with_mask_match_the_dense_operators():
 
     def run(fused_neg):
         emb, opt = _setup(n, d, 7)
+        w0.append(emb.embedding.detach().cpu().numpy().astype(np.float64))
         c = torch.tensor(cn, device="cuda", requires_grad=True)
         o = torch.tensor(on, device="cuda", requires_grad=True)
         neg = torch.tensor(neg_n, device="cuda")
@@ -160,11 +162,28 @@ def test_shared_negatives_with_mask_match_the_dense_operators():
         return (ln.detach().cpu().numpy(), c.grad.cpu().numpy(), o.grad.cpu().numpy(), emb.state_sum_fo.cpu().numpy(),
                 emb.embedding.detach().cpu().numpy())
 
+    w0 = []
     a, r = run(True), run(False)
     for x, y, what in zip(a[:4], r[:4], ("logits", "center grad", "offset grad", "first moment")):
         assert_close(x, y, 5 * REL_F32, what)
     # masked-out pairs still touch their rows: every listed id has moved (momentum), nothing else has
     assert np.abs(a[4] - r[4]).max() < 2 * lr
+    # the float64 oracle as the third party: every query scores the K shared rows, the mask multiplies the
+    # upstream gradient, masked pairs stay in the merge (their rows are touched with a zero term)
+    assert np.array_equal(w0[0], w0[1])
+    ids = np.broadcast_to(neg_n, (b, k))
+    qs = [cn.astype(np.float64)[:, None], on.astype(np.float64)[:, None]]
+    logit, rows = oracle_union_logits("box", w0[0], ids, qs, 24.0, 0.02)
+    g_rows, g_qs = oracle_union_grads("box", w0[0], ids, qs, rows, logit, (mask_n * gn_n).astype(np.float64), 0.02)
+    w, m, _, uniq, merged = oracle_adam_step(w0[0], [ids], [g_rows], lr, 1)
+    for got, route in ((a, "fused"), (r, "dense")):
+        assert_close(got[0], logit[:, 0], REL_F32, f"shared negatives, {route}: logits vs oracle")
+        assert_close(got[1], g_qs[0][:, 0], REL_F32, f"shared negatives, {route}: center grad vs oracle")
+        assert_close(got[2], g_qs[1][:, 0], REL_F32, f"shared negatives, {route}: offset grad vs oracle")
+        assert_close(got[3][uniq], m[uniq], REL_F32, f"shared negatives, {route}: first moment vs oracle")
+        assert_adam_weights(got[4], w, merged, uniq, lr, f"shared negatives, {route}: weights vs oracle")
+        untouched = np.setdiff1d(np.arange(n), uniq)
+        assert np.array_equal(got[4][untouched], w0[0][untouched].astype(np.float32))
 
 
 @pytest.mark.parametrize("model", ["box", "l1", "rotate"])
@@ -182,6 +201,7 @@ def test_union_branches_take_the_max_like_custom_cal_logit(model):
 
     def run(fused_neg):
         emb, opt = _setup(n, row, 7)
+        w0.append(emb.embedding.detach().cpu().numpy().astype(np.float64))
         q1 = torch.tensor(q1n, device="cuda", requires_grad=True)
         q2 = torch.tensor(q2n, device="cuda", requires_grad=True) if model != "l1" else None
         neg = torch.tensor(neg_n, device="cuda")
@@ -203,12 +223,26 @@ def test_union_branches_take_the_max_like_custom_cal_logit(model):
         opt.apply_grad(lr)
         opt.check_ids()
         grads = [q1.grad.cpu().numpy()] + ([q2.grad.cpu().numpy()] if q2 is not None else [])
-        return [ln.detach().cpu().numpy()] + grads + [emb.state_sum_fo.cpu().numpy()]
+        return [ln.detach().cpu().numpy()] + grads + [emb.state_sum_fo.cpu().numpy(), emb.embedding.detach().cpu().numpy()]
 
+    w0 = []
     a, r = run(True), run(False)
-    for x, y in zip(a, r):
+    for x, y in zip(a[:-1], r[:-1]):
         assert_close(x, y, 5 * REL_F32, model)
     assert np.abs(a[1]).sum() > 0
+    # the float64 oracle as the third party: per-branch logits, max over branches, gradient to the first maximal
+    # branch only, one Adam step on the merged rows
+    qs = [q1n.astype(np.float64)] + ([q2n.astype(np.float64)] if model != "l1" else [])
+    logit, rows = oracle_union_logits(model, w0[0], neg_n, qs, 24.0, 0.02)
+    assert len(np.unique(np.argmax(logit, axis=1))) > 1, "the case must have more than one winning branch"
+    g_rows, g_qs = oracle_union_grads(model, w0[0], neg_n, qs, rows, logit, gn_n.astype(np.float64), 0.02)
+    w, m, _, uniq, merged = oracle_adam_step(w0[0], [neg_n], [g_rows], lr, 1)
+    for got, route in ((a, "fused"), (r, "dense")):
+        assert_close(got[0], logit.max(axis=1), REL_F32, f"union {model}, {route}: logits vs oracle")
+        for t, want in zip(got[1:], g_qs):
+            assert_close(t, want, REL_F32, f"union {model}, {route}: query grad vs oracle")
+        assert_close(got[-2][uniq], m[uniq], REL_F32, f"union {model}, {route}: first moment vs oracle")
+        assert_adam_weights(got[-1], w, merged, uniq, lr, f"union {model}, {route}: weights vs oracle")
 
 
 def test_positives_as_column_zero_of_the_fused_call():
@@ -226,6 +260,7 @@ def test_positives_as_column_zero_of_the_fused_call():
 
     def run(one_call):
         emb, opt = _setup(n, d, 7)
+        w0.append(emb.embedding.detach().cpu().numpy().astype(np.float64))
         c = torch.tensor(cn, device="cuda", requires_grad=True)
         o = torch.tensor(on, device="cuda", requires_grad=True)
         pos, neg = torch.tensor(pos_n, device="cuda"), torch.tensor(neg_n, device="cuda")
@@ -243,10 +278,27 @@ def test_positives_as_column_zero_of_the_fused_call():
         return [x.detach().cpu().numpy() for x in (lp, ln, c.grad, o.grad, emb.state_sum_fo, emb.state_sum_sq)] + \
             [emb.embedding.detach().cpu().numpy()]
 
+    w0 = []
     a, r = run(True), run(False)
     for x, y, what in zip(a[:6], r[:6], ("positive logit", "negative logits", "center grad", "offset grad", "m", "v")):
         assert_close(x, y, 5 * REL_F32, what)
     assert np.abs(a[6] - r[6]).max() < 2 * lr
+    # the float64 oracle as the third party: positives and negatives are two index streams into one merge
+    # (embed_optimizer.py:155-163); the entity that is both gets one row update from the sum of both gradients
+    ids = np.concatenate([pos_n, neg_n], axis=1)
+    qs = [cn.astype(np.float64)[:, None], on.astype(np.float64)[:, None]]
+    gout = np.concatenate([gp, gn], axis=1).astype(np.float64)
+    logit, rows = oracle_union_logits("box", w0[0], ids, qs, 24.0, 0.02)
+    g_rows, g_qs = oracle_union_grads("box", w0[0], ids, qs, rows, logit, gout, 0.02)
+    w, m, v, uniq, merged = oracle_adam_step(w0[0], [ids], [g_rows], lr, 1)
+    for got, route in ((a, "one call"), (r, "two records")):
+        assert_close(got[0], logit[:, 0, :1], REL_F32, f"positives, {route}: positive logit vs oracle")
+        assert_close(got[1], logit[:, 0, 1:], REL_F32, f"positives, {route}: negative logits vs oracle")
+        assert_close(got[2], g_qs[0][:, 0], REL_F32, f"positives, {route}: center grad vs oracle")
+        assert_close(got[3], g_qs[1][:, 0], REL_F32, f"positives, {route}: offset grad vs oracle")
+        assert_close(got[4][uniq], m[uniq], REL_F32, f"positives, {route}: first moment vs oracle")
+        assert_close(got[5][uniq], v[uniq], REL_F32, f"positives, {route}: second moment vs oracle")
+        assert_adam_weights(got[6], w, merged, uniq, lr, f"positives, {route}: weights vs oracle")
 
 
 def test_step_counter_and_empty_steps():

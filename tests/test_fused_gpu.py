@@ -6,7 +6,7 @@ import pytest
 import torch
 
 from oracle import oracle as orc
-from tests.util import REL_F32, assert_close, seed
+from tests.util import REL_F32, assert_close, record_headroom, seed
 
 pytestmark = pytest.mark.gpu
 
@@ -63,7 +63,8 @@ def run_case(model, n, b, k, dim, zipf=None, cen=0.02, adam_steps=2, lr=1e-3):
     o_q1 = q1[:, None, :]
     o_q2 = None if q2 is None else q2[:, None, :]
     want = orc.score_forward(model, rows, o_q1, o_q2, gamma, cen)
-    assert_close(score.cpu().numpy(), want, REL_F32, f"{model} score")
+    # no RMS floor for the scores of the models whose distance is a sum of non-negative terms: every element to 1e-5
+    assert_close(score.cpu().numpy(), want, REL_F32, f"{model} score", rms_floor=model == "beta_kl")
     assert err.item() == 0
 
     # dense layout (idx = None) gives the same scores bit for bit
@@ -140,12 +141,14 @@ def run_case(model, n, b, k, dim, zipf=None, cen=0.02, adam_steps=2, lr=1e-3):
             assert torch.equal(got[torch.tensor(~touched, device="cuda")], ref[torch.tensor(~touched, device="cuda")])
         assert_close(t_table.cpu().numpy()[touched], w_s[touched], REL_F32, f"{model} Adam step {step}: w")
         assert_close(t_m.cpu().numpy()[touched], m_s[touched], REL_F32, f"{model} Adam step {step}: m")
-        assert_close(t_v.cpu().numpy()[touched], v_s[touched], REL_F32, f"{model} Adam step {step}: v")
+        assert_close(t_v.cpu().numpy()[touched], v_s[touched], REL_F32, f"{model} Adam step {step}: v", rms_floor=False)
         orc.train_step(model, w_o, m_o, v_o, idx, o_q1, o_q2, gs, gamma, cen, lr, step)
     got_w = t_table.cpu().numpy()
     err = np.abs(got_w - w_o)[touched]
     tol = REL_F32 * np.maximum(np.abs(w_o[touched]), np.sqrt(np.mean(w_o[touched] ** 2)))
     assert (err > tol).mean() < 1e-3 and err.max() < 2 * lr * adam_steps, (err.max(), (err > tol).mean())
+    record_headroom(f"{model} w trajectory: share of elements outside 1e-5 / 1e-3, worst error / (2 lr steps)",
+                    (err > tol).mean() / 1e-3, err.max() / (2 * lr * adam_steps))
     assert_close(t_m.cpu().numpy()[touched], m_o[touched], 5 * REL_F32, f"{model} m trajectory")
     assert np.array_equal(got_w[~touched], table[~touched].astype(np.float32)), "untouched rows must stay bit-identical"
     assert not t_m.cpu().numpy()[~touched].any() and not t_v.cpu().numpy()[~touched].any()

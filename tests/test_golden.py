@@ -58,7 +58,7 @@ def test_hip_path_reproduces_fixture(path):
     assert np.array_equal(plan.order.cpu().numpy(), d["order"])
     assert np.array_equal(plan.seg_start[: u + 1].cpu().numpy(), d["seg_start"])
     score = fused.score_forward(model, table, idx, q1, q2, params)
-    assert_close(score.cpu().numpy(), d["score"], REL_F32, "score")
+    assert_close(score.cpu().numpy(), d["score"], REL_F32, "score", rms_floor=False)
     gq1, gq2 = fused.score_backward_query(model, table, idx, q1, q2, score, gs, params)
     assert_close(gq1.cpu().numpy(), d["gq1"], REL_F32, "gq1")
     if q2 is not None:
@@ -89,7 +89,7 @@ def test_timed_path_reproduces_the_box_fixture():
     plan = fused.build_plan(idx, table.shape[0])
     codes = fused.new_codes("box", table, idx, q1)
     score = fused.score_forward("box", table, idx, q1, q2, params, codes=codes)
-    assert_close(score.cpu().numpy(), d["score"], REL_F32, "score")
+    assert_close(score.cpu().numpy(), d["score"], REL_F32, "score", rms_floor=False)
     merged = torch.empty((plan.n_uniq, table.shape[1]), device="cuda")
     gq1, gq2 = fused.score_backward_fused("box", plan, table, idx, q1, q2, score, gs, params, merged=merged, codes=codes)
     assert_close(gq1.cpu().numpy(), d["gq1"], REL_F32, "gq1")
