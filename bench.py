@@ -21,12 +21,41 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E bandwidth
 
-# Traffic of the backward call per launch in bytes (L2<->fabric, reads + writes), measured with two
-# `rocprofv3 --pmc` runs (FETCH_SIZE, WRITE_SIZE) and scaled by what the same counters read for a plain
-# row copy of known size (`bench.py --calibrate-copy`: FETCH_SIZE x1.942, WRITE_SIZE x0.986).  A counter
-# cannot be read from inside this process, so the figures are those of the profile summary
-# pmc_traffic_<workload>.md kept with the other rocprofv3 summaries; workloads not profiled report null.
-MEASURED_BACKWARD_TRAFFIC = {"cfg5-box-adam-86m-zipf1.1": 4.82e9}
+PROFILES = os.path.join(ROOT, "profiles")
+CSRC = os.path.join(ROOT, "smore_amd", "csrc")
+
+
+def kernel_source_digest():
+    """Identifies the kernel sources a profile summary was taken with: sha256 over the .hip / .h files of the
+    library (names and contents, sorted; the probe library is not part of it)."""
+    import hashlib
+    h = hashlib.sha256()
+    for name in sorted(os.listdir(CSRC)):
+        if name.endswith((".hip", ".h")):
+            h.update(name.encode())
+            with open(os.path.join(CSRC, name), "rb") as f:
+                h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+def measured_traffic(workload):
+    """HBM-side traffic per launch of this workload's kernels (L2 <-> fabric, reads + writes, bytes), as measured
+    with two `rocprofv3 --pmc` runs (FETCH_SIZE, WRITE_SIZE), each scaled by what the same counter reads for a
+    plain row copy of known size (`bench.py --calibrate-copy`).  A counter cannot be read from inside this
+    process: the figures are those of the committed summary profiles/pmc_traffic_<workload>.md, whose last line
+    is a JSON object {"sources": digest, "commit": ..., "kernels": {name: [read, write]}}.  None when there is no
+    summary, or when it was taken with other kernel sources than the ones in this tree."""
+    path = os.path.join(PROFILES, f"pmc_traffic_{workload}.md")
+    try:
+        with open(path) as f:
+            lines = [ln for ln in f.read().splitlines() if ln.startswith("traffic_json: ")]
+        rec = json.loads(lines[-1][len("traffic_json: "):])
+    except (OSError, IndexError, ValueError):
+        return None
+    if rec.get("sources") != kernel_source_digest():
+        return None
+    return rec
+
 
 CONFIGS = {
     1: dict(name="cfg1-l2-15k", model="l2", n=15_000, dim=200, b=512, k=128, r=0.07, gamma=12.0, cen=0.0,
@@ -105,14 +134,31 @@ def algorithmic_bytes(cfg, n_uniq, streaming=False):
     return total
 
 
-def backward_bytes(cfg, n_uniq):
+def backward_bytes(cfg, n_uniq, from_codes=False):
     """Algorithmic bytes of the backward call (query gradients + entity pass): the backward share of the step
     model above -- every distinct row once, Adam's read + write of w, m, v (or, without optimizer, the merged
-    gradient rows written), the upstream gradient of every pair, queries read and their gradients written."""
+    gradient rows written), the upstream gradient of every pair, queries read and their gradients written.
+    from_codes: the backward works from the forward's sign codes and reads no entity row for the derivative, so
+    the row read of the model is not compulsory for it (with an optimizer it is the same read as Adam's)."""
     p = cfg["b"] * cfg["k"]
     de = row_len(cfg)
-    rows = 4 * de * n_uniq + (6 * 4 * de * n_uniq if cfg["adam"] else 4 * de * n_uniq)
+    rows = (0 if from_codes else 4 * de * n_uniq) + (6 * 4 * de * n_uniq if cfg["adam"] else 4 * de * n_uniq)
     return rows + 4 * p + 2 * 4 * cfg["b"] * cfg["dim"] * n_query_tensors(cfg)
+
+
+def backward_kernel_bytes(cfg, n_uniq, n_one_pair, from_codes):
+    """The same model split over the two halves of the backward call.  The query-gradient kernel: upstream
+    gradient of every pair, queries read and gradients written, the distinct rows when it recomputes from them,
+    and the optimizer's read + write (or the merged row written) of the ids that occur once, which it finishes.
+    The entity pass (segment, tile and fix-up kernels): the rows of all other ids, and the upstream gradient of
+    their pairs a second time."""
+    p = cfg["b"] * cfg["k"]
+    de = row_len(cfg)
+    per_row = 6 * 4 * de if cfg["adam"] else 4 * de
+    query = ((0 if from_codes else 4 * de * n_uniq) + per_row * n_one_pair + 4 * p +
+             2 * 4 * cfg["b"] * cfg["dim"] * n_query_tensors(cfg))
+    entity = per_row * (n_uniq - n_one_pair) + 4 * (p - n_one_pair)
+    return query, entity
 
 
 class Step:
@@ -358,8 +404,45 @@ def main():
     pairs = cfg["b"] * cfg["k"]
     algo = algorithmic_bytes(cfg, n_uniq)
     algo_stream = algorithmic_bytes(cfg, n_uniq, streaming=True)
-    ent_bytes = backward_bytes(cfg, n_uniq)
-    ent_gbps = ent_bytes / (phase_ms["backward"] * 1e-3) / 1e9
+    from_codes = step.codes is not None
+    n_one_pair = int((step.plan.pair_seg < 0).sum().item())     # ids that occur once in the step
+    seg_len = step.plan.seg_start[1: n_uniq + 1] - step.plan.seg_start[:n_uniq]
+    n_short = int(((seg_len > 1) & (seg_len <= 64)).sum().item())   # finished by entity_segment_kernel
+    n_long = n_uniq - n_one_pair - n_short                           # entity_tile_kernel + entity_fixup_kernel
+    call_bytes = backward_bytes(cfg, n_uniq, from_codes)
+    q_bytes, e_bytes = backward_kernel_bytes(cfg, n_uniq, n_one_pair, from_codes)
+
+    def timed_backward(parts, serial, reps=5):
+        """Average event-bracketed duration (ms) of the backward call with only `parts` of it running (the
+        library's measuring switch; 3 = the whole call).  Run after the timed region: a call with one half
+        leaves an incomplete step behind."""
+        _lib.call("smx_set_option", _lib.OPTION_SERIAL_BACKWARD, 1 if serial else 0)
+        _lib.call("smx_set_option", _lib.OPTION_BACKWARD_PARTS, parts)
+        try:
+            evs = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(reps)]
+            for e in evs:
+                step.run(e)
+            torch.cuda.synchronize()
+        finally:
+            _lib.call("smx_set_option", _lib.OPTION_BACKWARD_PARTS, 3)
+            _lib.call("smx_set_option", _lib.OPTION_SERIAL_BACKWARD, 0)
+        return sum(e[2].elapsed_time(e[3]) for e in evs) / reps
+
+    query_alone_ms = timed_backward(1, True)     # the dominant kernel by itself, on the stream it is launched on
+    entity_alone_ms = timed_backward(2, True)
+    one_stream_ms = timed_backward(3, True)
+    gbps = lambda nbytes, ms: nbytes / (ms * 1e-3) / 1e9
+    prof = measured_traffic(cfg["name"])
+    traffic = {k: sum(v) for k, v in prof["kernels"].items()} if prof else {}
+    q_traffic = next((v for k, v in traffic.items() if "score_backward_query" in k), None)
+    e_traffic = sum(v for k, v in traffic.items() if "entity_" in k) if traffic else None
+    dominant = ("score_backward_query_kernel: query gradients of every pair" +
+                (" from the sign codes the forward saved" if from_codes else " recomputed from the gathered rows") +
+                ("; it also finishes the ids that occur once (" +
+                 ("optimizer update of their w, m, v rows" if cfg["adam"] else "their merged gradient rows") + ")"))
+    # cfg4: Beta-KL evaluates 12 special-function values per (pair, feature); the kernel is bound by VALU issue,
+    # not by memory (profiles/pmc_valu_cfg4-betakl-1m.md); the GB/s figure is still reported against the HBM peak
+    bound = "valu" if cfg["model"] == "beta_kl" else "hbm"
 
     out = {
         "metric": "scored (query,neg) pairs/sec fwd+bwd+opt; achieved HBM GB/s vs peak",
@@ -371,15 +454,35 @@ def main():
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": cfg["name"], "model": None, "N": cfg["n"], "row_len": row_len(cfg), "B": cfg["b"],
                    "K": cfg["k"], "ids": "zipf(1.1)" if cfg["zipf"] else "uniform", "optimizer": "sparse adam" if
-                   cfg["adam"] else None, "seed": seed, "distinct_ids": n_uniq},
+                   cfg["adam"] else None, "seed": seed, "distinct_ids": n_uniq, "one_pair_ids": n_one_pair,
+                   "ids_with_2_to_64_pairs": n_short, "ids_with_more_pairs": n_long},
         "roofline": {
-            "bound": "hbm",
-            "kernel": "backward (one C-ABI call, smx_score_backward_fused = score_backward_query_kernel + "
-                      "entity_segment_kernel + entity_tile_kernel + entity_fixup_kernel): query gradients, segmented "
-                      "entity gradient" + (" + fused sparse Adam" if cfg["adam"] else " (merged rows)") +
-                      ("; works from the sign codes the forward saved" if step.codes is not None else ""),
-            "achieved": ent_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": ent_gbps / HBM_PEAK_GBPS,
-            "traffic": MEASURED_BACKWARD_TRAFFIC.get(cfg["name"]) if step.codes is not None else None, "algorithmic_bytes": ent_bytes, "avg_ms": phase_ms["backward"],
+            "bound": bound,
+            "kernel": dominant,
+            "achieved": gbps(q_bytes, query_alone_ms), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+            "frac": gbps(q_bytes, query_alone_ms) / HBM_PEAK_GBPS,
+            "traffic": q_traffic, "algorithmic_bytes": q_bytes, "avg_ms": query_alone_ms,
+            "units_per_launch": {"pairs": pairs, "queries": cfg["b"], "one_pair_rows": n_one_pair,
+                                 "distinct_rows_read": 0 if from_codes else n_uniq},
+            "kernels": [
+                {"name": "score_backward_query_kernel", "algorithmic_bytes": q_bytes, "avg_ms_alone": query_alone_ms,
+                 "achieved": gbps(q_bytes, query_alone_ms), "traffic": q_traffic},
+                {"name": "entity pass: entity_segment_kernel + entity_tile_kernel + entity_fixup_kernel",
+                 "algorithmic_bytes": e_bytes, "avg_ms_alone": entity_alone_ms, "achieved": gbps(e_bytes, entity_alone_ms),
+                 "traffic": e_traffic, "rows": n_uniq - n_one_pair, "pairs": pairs - n_one_pair},
+            ],
+            "call": {
+                "what": "smx_score_backward_fused, the whole backward as bench.py times it (query-gradient kernel on "
+                        "the caller's stream, entity pass beside it on the library's second stream where that pays)",
+                "algorithmic_bytes": call_bytes,
+                "algorithmic_bytes_with_row_read": backward_bytes(cfg, n_uniq, False),
+                "avg_ms": phase_ms["backward"], "one_stream_avg_ms": one_stream_ms,
+                "achieved": gbps(call_bytes, phase_ms["backward"]),
+                "frac": gbps(call_bytes, phase_ms["backward"]) / HBM_PEAK_GBPS,
+                "traffic": (q_traffic + e_traffic) if q_traffic is not None and e_traffic is not None else None,
+            },
+            "traffic_source": (f"profiles/pmc_traffic_{cfg['name']}.md (commit {prof.get('commit')})" if prof else
+                               "no PMC summary for these kernel sources"),
         },
         "step_hbm": {
             "algorithmic_bytes": algo, "achieved_GBps": algo / (ms_per_step * 1e-3) / 1e9,
@@ -389,22 +492,14 @@ def main():
         },
         "phase_ms": phase_ms,
     }
-    if cfg["adam"] and step.codes is not None:
-        # the same backward with its kernels one after the other on one stream (the library's profiling
-        # switch): the figure the per-kernel durations of a rocprofv3 trace of that mode add up to
-        _lib.call("smx_set_option", _lib.OPTION_SERIAL_BACKWARD, 1)
-        ev2 = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(5)]
-        for e in ev2:
-            step.run(e)
-        torch.cuda.synchronize()
-        _lib.call("smx_set_option", _lib.OPTION_SERIAL_BACKWARD, 0)
-        out["roofline"]["one_stream_avg_ms"] = sum(e[2].elapsed_time(e[3]) for e in ev2) / len(ev2)
     # what plain kernels sustain on this GPU for the step's access shapes, measured now with the library's
     # probes (after the timed region); a step that writes w, m, v back is a copy-like mix of reads and writes
     try:
         out["measured_ceilings"] = measure_ceilings(device, 4 * row_len(cfg))
         out["step_hbm"]["frac_of_measured_copy"] = out["step_hbm"]["achieved_GBps"] / out["measured_ceilings"]["copy_GBps"]
-        out["roofline"]["frac_of_measured_copy"] = ent_gbps / out["measured_ceilings"]["copy_GBps"]
+        out["roofline"]["frac_of_measured_copy"] = out["roofline"]["achieved"] / out["measured_ceilings"]["copy_GBps"]
+        out["roofline"]["call"]["frac_of_measured_copy"] = (out["roofline"]["call"]["achieved"] /
+                                                            out["measured_ceilings"]["copy_GBps"])
     except torch.OutOfMemoryError:  # no room left for the two 4 GiB probe buffers: the step's figures stand alone
         out["measured_ceilings"] = None
     del out["config"]["model"]

@@ -88,6 +88,7 @@ class PlanView(ctypes.Structure):
                 ("n_uniq", _vp), ("pair_seg", _vp), ("n_pairs", _sz)]
 
 OPTION_SERIAL_BACKWARD = 1
+OPTION_BACKWARD_PARTS = 2     # bit 0: query-gradient kernel, bit 1: entity pass (3 = both, the default)
 
 _lib = None
 _probe = None

@@ -21,6 +21,8 @@ int check_launch(const char* what);
 
 // smx_set_option(SMX_OPTION_SERIAL_BACKWARD, ..): the backward keeps to the caller's stream
 bool serial_backward();
+// smx_set_option(SMX_OPTION_BACKWARD_PARTS, ..): bit 0 query-gradient kernel, bit 1 entity pass
+int backward_parts();
 
 inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
 

@@ -330,8 +330,9 @@ int smx_score_backward_fused(int model, void* stream, const smx_plan_view* plan,
     std::lock_guard<std::mutex> one_call(side->in_use);
     if (hipEventRecord(side->fork, st) != hipSuccess || hipStreamWaitEvent(side->stream, side->fork, 0) != hipSuccess)
       return fail(SMX_ERR_HIP, "fork to the side stream failed");
-    int rc = dispatch_model(model, st, A, vec, nit, false);
-    if (rc == SMX_OK)
+    const int parts = backward_parts();
+    int rc = (parts & 1) ? dispatch_model(model, st, A, vec, nit, false) : SMX_OK;
+    if (rc == SMX_OK && (parts & 2))
       rc = entity_backward(model, side->stream, plan, table, n_rows, q1, q2, score, gscore, B, K, dim, params, merged, m,
                            v, adam, workspace, workspace_bytes, singles_here ? 1 : 0, codes, vec, nit);
     // join even after a failed launch, so that the caller's stream never runs ahead of the side stream
@@ -339,7 +340,10 @@ int smx_score_backward_fused(int model, void* stream, const smx_plan_view* plan,
       return fail(SMX_ERR_HIP, "join with the side stream failed");
     return rc;
   }
-  if (int rc = dispatch_model(model, as_stream(stream), A, vec, nit, false)) return rc;
+  const int parts = backward_parts();
+  if (parts & 1)
+    if (int rc = dispatch_model(model, as_stream(stream), A, vec, nit, false)) return rc;
+  if (!(parts & 2)) return SMX_OK;
   return entity_backward(model, stream, plan, table, n_rows, q1, q2, score, gscore, B, K, dim, params, merged, m, v,
                          adam, workspace, workspace_bytes, singles_here ? 1 : 0, codes, vec, nit);
 }

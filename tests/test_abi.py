@@ -46,6 +46,7 @@ def test_host_only_entry_points():
     assert lib.smx_kind_from_name(b"beta_fisher_approx") == 9
     assert lib.smx_kind_from_name(b"nope") == -1
     assert lib.smx_set_option(_lib.OPTION_SERIAL_BACKWARD, 0) == 0 and lib.smx_set_option(99, 1) != 0
+    assert lib.smx_set_option(_lib.OPTION_BACKWARD_PARTS, 3) == 0 and lib.smx_set_option(_lib.OPTION_BACKWARD_PARTS, 0) != 0
     import ctypes as c
     opt = _lib.OptParams(1e-3, 0.9, 0.999, 1e-8, 2, _lib.OPT_KINDS["adam"], 0, None)
     out = (c.c_float * 2)()

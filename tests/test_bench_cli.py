@@ -24,6 +24,31 @@ def test_byte_models_of_the_headline_workload():
     back = bench.backward_bytes(cfg, u)
     assert back == 4 * de * u + 24 * de * u + 4 * p + 8 * cfg["b"] * cfg["dim"] * 2
     assert bench.algorithmic_bytes(cfg, u, streaming=True) > step
+    # working from the forward's sign codes, the backward reads no entity row for the derivative
+    assert bench.backward_bytes(cfg, u, from_codes=True) == back - 4 * de * u
+    # the two halves of the call: ids that occur once are finished by the query-gradient kernel
+    u1 = 606000
+    q, e = bench.backward_kernel_bytes(cfg, u, u1, True)
+    assert q == 24 * de * u1 + 4 * p + 8 * cfg["b"] * cfg["dim"] * 2 and e == 24 * de * (u - u1) + 4 * (p - u1)
+    assert q + e == bench.backward_bytes(cfg, u, from_codes=True) + 4 * (p - u1)
+    q, e = bench.backward_kernel_bytes(bench.CONFIGS[3], 1000, 900, False)      # rotate: rows re-read, merged rows written
+    assert q == 4 * 1000 * 1000 + 4 * 1000 * 900 + 4 * 1024 * 1024 + 8 * 1024 * 500 * 2 and e == 4 * 1000 * 100 + 4 * (1024 * 1024 - 900)
+
+
+def test_measured_traffic_is_tied_to_the_kernel_sources(tmp_path, monkeypatch):
+    """bench.py quotes PMC traffic only from a summary taken with the kernel sources of this tree."""
+    sys.path.insert(0, str(ROOT))
+    import bench
+    digest = bench.kernel_source_digest()
+    assert len(digest) == 16 and digest == bench.kernel_source_digest()
+    monkeypatch.setattr(bench, "PROFILES", str(tmp_path))
+    assert bench.measured_traffic("w") is None
+    rec = {"sources": digest, "commit": "abc", "kernels": {"k": [1.0, 2.0]}}
+    (tmp_path / "pmc_traffic_w.md").write_text("# text\n\ntraffic_json: " + json.dumps(rec) + "\n")
+    assert bench.measured_traffic("w") == rec
+    rec["sources"] = "0" * 16
+    (tmp_path / "pmc_traffic_w.md").write_text("traffic_json: " + json.dumps(rec) + "\n")
+    assert bench.measured_traffic("w") is None
 
 
 def test_product_path_has_no_cpu_fallback():
