@@ -244,6 +244,31 @@ int smx_score_backward_entity(int model, void* stream, const smx_plan_view* plan
                               const smx_opt_params* adam, void* workspace, size_t workspace_bytes,
                               const void* fwd_codes, size_t fwd_codes_bytes);
 
+/* The same pass over several index streams that share one query batch -- a step's positives [B,1] and
+ * negatives [B,K] scored against the same query embeddings (kg_reasoning.py:340-355), each by its own
+ * smx_score_forward call.  Replaces what the reference does with several (indices, gradient rows) records in
+ * apply_grad (embed_optimizer.py:155-163): concatenate, merge_grad_indices (:39-42), merge_grad_list (:45-48),
+ * one update_step per entity (:208-252) -- without materialising gradient rows.
+ * plan: built by smx_plan_build over the concatenation [ids of source 0 (B*K_0) | ids of source 1 (B*K_1) | ..];
+ * pair j of source s (query j / K_s) is pair B*(K_0 + .. + K_s-1) + j of the plan.  Every source brings the
+ * score its forward produced, the upstream gradient, and its sign codes (all sources or none); q1, q2, B, dim,
+ * params are common to all.  An entity that occurs in several sources gets ONE update from the sum of all its
+ * pairs' gradients, summed in plan order (source by source, pairs ascending).  n_src == 1 is
+ * smx_score_backward_entity.  workspace: smx_entity_workspace_bytes(total pairs, dim*mul). */
+#define SMX_MAX_PAIR_SOURCES 4
+typedef struct smx_pair_source {
+  const float* score;      /* [B, K] */
+  const float* gscore;     /* [B, K] */
+  const void* fwd_codes;   /* may be NULL */
+  size_t fwd_codes_bytes;
+  size_t K;
+} smx_pair_source;
+int smx_score_backward_entity_multi(int model, void* stream, const smx_plan_view* plan, float* table,
+                                    size_t n_rows, const float* q1, const float* q2,
+                                    const smx_pair_source* src, size_t n_src, size_t B, size_t dim,
+                                    const smx_score_params* params, float* merged, float* m, float* v,
+                                    const smx_opt_params* adam, void* workspace, size_t workspace_bytes);
+
 /* Everything after the loss in one call: query gradients, and every entity row of the step finished
  * (merged gradient row and/or lazy Adam on w, m, v), as smx_score_backward_query followed by
  * smx_score_backward_entity would do -- except that rows of ids occurring once in the step are

@@ -47,6 +47,9 @@ SIGNATURES = {
     # fwd_codes, bytes
     "smx_score_backward_entity": (_i, [_i, _vp, _vp, _vp, _sz, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _vp, _vp, _vp, _vp,
                                        _vp, _vp, _sz, _vp, _sz]),
+    # model, stream, plan, table, n_rows, q1, q2, src[], n_src, B, dim, params, merged, m, v, adam, ws, ws_bytes
+    "smx_score_backward_entity_multi": (_i, [_i, _vp, _vp, _vp, _sz, _vp, _vp, _vp, _sz, _sz, _sz, _vp, _vp, _vp, _vp,
+                                             _vp, _vp, _sz]),
     # model, stream, plan, table, n_rows, idx, q1, q2, score, gscore, gq1, gq2, B, K, dim, params, merged, m, v,
     # adam, ws, ws_bytes, fwd_codes, fwd_codes_bytes
     "smx_score_backward_fused": (_i, [_i, _vp, _vp, _vp, _sz, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _vp,
@@ -87,6 +90,14 @@ class PlanView(ctypes.Structure):
     _fields_ = [("order", _vp), ("sorted_ids", _vp), ("seg_of_pos", _vp), ("seg_start", _vp), ("uniq", _vp),
                 ("n_uniq", _vp), ("pair_seg", _vp), ("n_pairs", _sz)]
 
+
+
+class PairSource(ctypes.Structure):
+    """smx_pair_source of include/smore_amd.h."""
+    _fields_ = [("score", _vp), ("gscore", _vp), ("fwd_codes", _vp), ("fwd_codes_bytes", _sz), ("K", _sz)]
+
+
+MAX_PAIR_SOURCES = 4
 OPTION_SERIAL_BACKWARD = 1
 OPTION_BACKWARD_PARTS = 2     # bit 0: query-gradient kernel, bit 1: entity pass (3 = both, the default)
 

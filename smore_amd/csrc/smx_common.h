@@ -24,6 +24,18 @@ bool serial_backward();
 // smx_set_option(SMX_OPTION_BACKWARD_PARTS, ..): bit 0 query-gradient kernel, bit 1 entity pass
 int backward_parts();
 
+constexpr int kMaxSources = 4;  // index streams one entity pass can reduce together (SMX_MAX_PAIR_SOURCES)
+
+// Several index streams behind one segment plan: source i holds pairs [B * (K_0 + .. + K_i-1), + B * K_i) of the
+// plan, with its own score / upstream gradient / sign-code arrays; all sources share the query tensors.
+struct PairSources {
+  int n;
+  const float* score[kMaxSources];
+  const float* gscore[kMaxSources];
+  const unsigned char* codes[kMaxSources];
+  size_t K[kMaxSources];
+};
+
 inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }

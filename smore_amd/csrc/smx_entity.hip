@@ -96,7 +96,7 @@ int entity_backward(int model, void* stream, const smx_plan_view* plan, float* t
                     const float* q2, const float* score, const float* gscore, size_t B, size_t K, size_t dim,
                     const smx_score_params* params, float* merged, float* m, float* v, const smx_opt_params* adam,
                     void* workspace, size_t workspace_bytes, int skip_single, const unsigned char* codes, int codes_vec,
-                    int codes_nit);
+                    int codes_nit, const PairSources* multi = nullptr);
 
 static int fill_adam(EntityArgs* A, float* m, float* v, const smx_opt_params* opt) {
   A->adam_on = 0;
@@ -146,9 +146,9 @@ int entity_backward(int model, void* stream, const smx_plan_view* plan, float* t
                     const float* q2, const float* score, const float* gscore, size_t B, size_t K, size_t dim,
                     const smx_score_params* params, float* merged, float* m, float* v, const smx_opt_params* adam,
                     void* workspace, size_t workspace_bytes, int skip_single, const unsigned char* codes, int codes_vec,
-                    int codes_nit) {
+                    int codes_nit, const PairSources* multi) {
   if (model < 0 || model >= mNumModels) return fail(SMX_ERR_KIND, "unknown score model %d", model);
-  if (!table || !q1 || !score || !gscore || !params || (model_nq(model) == 2 && !q2))
+  if (!table || !q1 || (!multi && (!score || !gscore)) || !params || (model_nq(model) == 2 && !q2))
     return fail(SMX_ERR_ARG, "null pointer");
   if (B == 0 || K == 0 || dim == 0 || n_rows == 0) return fail(SMX_ERR_SHAPE, "empty dimension");
   if (params->reg_on && model != mBetaKL)
@@ -158,6 +158,23 @@ int entity_backward(int model, void* stream, const smx_plan_view* plan, float* t
   const size_t row_len = dim * model_mul(model);
   if (int rc = fill_plan(&A, plan, workspace, workspace_bytes, row_len)) return rc;
   if (plan->n_pairs != B * K) return fail(SMX_ERR_SHAPE, "plan holds %zu pairs, call has %zu", plan->n_pairs, B * K);
+  if (multi) {  // K is then the sum of the sources' K (checked by the caller): pairs of source s start at B * (K_0 + .. + K_s-1)
+    if (multi->n < 2 || multi->n > kMaxSources) return fail(SMX_ERR_ARG, "2 to %d pair sources", kMaxSources);
+    A.n_src = multi->n;
+    size_t first = 0;
+    for (int i = 0; i < multi->n; ++i) {
+      if (!multi->score[i] || !multi->gscore[i] || multi->K[i] == 0) return fail(SMX_ERR_ARG, "incomplete pair source %d", i);
+      if ((codes != nullptr) != (multi->codes[i] != nullptr)) return fail(SMX_ERR_ARG, "sign codes for some pair sources only");
+      A.first[i] = (int)first;
+      A.src_score[i] = multi->score[i];
+      A.src_gscore[i] = multi->gscore[i];
+      A.src_codes[i] = multi->codes[i];
+      A.src_K[i] = (int)multi->K[i];
+      first += B * multi->K[i];
+    }
+    if (first != B * K) return fail(SMX_ERR_SHAPE, "pair sources hold %zu pairs, plan %zu", first, B * K);
+    for (int i = multi->n; i <= kMaxSources; ++i) A.first[i] = (int)first;
+  }
   if (int rc = fill_adam(&A, m, v, adam)) return rc;
   const bool vec4 = dim % 4 == 0 && aligned16(table) && aligned16(q1) && (!q2 || aligned16(q2)) &&
                     (!merged || aligned16(merged)) && (!m || aligned16(m)) && (!v || (adam && adam->squeeze) || aligned16(v));

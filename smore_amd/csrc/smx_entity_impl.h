@@ -59,6 +59,16 @@ struct EntityArgs : RowSink {
   int skip_single;  // segments of one pair were already finished by the query-backward kernel
   // sign codes written by the query-backward kernel, [n_pairs][NIT*64] bytes, or null (CODED kernels)
   const unsigned char* codes;
+  // several index streams in one plan (positives + negatives of one query batch, embed_optimizer.py:155-163):
+  // n_src > 1, and pair p of the plan with first[s] <= p < first[s+1] is pair (p - first[s]) of source s, which
+  // has its own score / gscore / codes arrays and its own K; all sources share q1, q2.  n_src <= 1: the single
+  // source described by score, gscore, codes and K above.
+  int n_src;
+  int first[kMaxSources + 1];
+  const float* src_score[kMaxSources];
+  const float* src_gscore[kMaxSources];
+  const unsigned char* src_codes[kMaxSources];
+  int src_K[kMaxSources];
 };
 
 template <int SRC>
@@ -123,7 +133,19 @@ __device__ __forceinline__ void request_runs(const EntityArgs& A, int lane, cons
   for (int r = 0; r < R; ++r) {
     if (r < rs.n) {
       if constexpr (CODED) {
-        const unsigned char* pc = A.codes + (size_t)rs.pair[r] * (NIT * 64) + lane;
+        const unsigned char* cbase = A.codes;
+        int cpair = rs.pair[r];  // wave-uniform
+        if (A.n_src > 1) {
+          cbase = A.src_codes[0];
+#pragma unroll
+          for (int s = 1; s < kMaxSources; ++s) {
+            if (s < A.n_src && rs.pair[r] >= A.first[s]) {
+              cbase = A.src_codes[s];
+              cpair = rs.pair[r] - A.first[s];
+            }
+          }
+        }
+        const unsigned char* pc = cbase + (size_t)cpair * (NIT * 64) + lane;
 #pragma unroll
         for (int it = 0; it < NIT; ++it) rr.code[r][it] = pc[64 * it];
       } else if constexpr (SRC == kSrcRows) {
@@ -192,8 +214,25 @@ __device__ __forceinline__ void load_window(const EntityArgs& A, int lane, int b
   } else {
     const int pair = my_pair = A.order[pos];
     float c1;
-    ModelOps<SRC>::coef(A.gscore[pair], A.score[pair], A.p, my_c, c1);
-    my_key = pair / A.K;
+    if (A.n_src > 1) {  // uniform: which index stream the pair came from, and its number inside that stream
+      int local = pair, K = A.src_K[0];
+      const float* gs = A.src_gscore[0];
+      const float* sc = A.src_score[0];
+#pragma unroll
+      for (int s = 1; s < kMaxSources; ++s) {
+        if (s < A.n_src && pair >= A.first[s]) {
+          local = pair - A.first[s];
+          K = A.src_K[s];
+          gs = A.src_gscore[s];
+          sc = A.src_score[s];
+        }
+      }
+      ModelOps<SRC>::coef(gs[local], sc[local], A.p, my_c, c1);
+      my_key = local / K;
+    } else {
+      ModelOps<SRC>::coef(A.gscore[pair], A.score[pair], A.p, my_c, c1);
+      my_key = pair / A.K;
+    }
   }
 }
 

@@ -33,7 +33,7 @@ int entity_backward(int model, void* stream, const smx_plan_view* plan, float* t
                     const float* q2, const float* score, const float* gscore, size_t B, size_t K, size_t dim,
                     const smx_score_params* params, float* merged, float* m, float* v, const smx_opt_params* adam,
                     void* workspace, size_t workspace_bytes, int skip_single, const unsigned char* codes, int codes_vec,
-                    int codes_nit);
+                    int codes_nit, const PairSources* multi = nullptr);
 size_t entity_ws_bytes(size_t n_pairs, size_t row_len);
 size_t code_bytes_per_pair(size_t dim);
 
@@ -250,6 +250,92 @@ int smx_score_backward_entity(int model, void* stream, const smx_plan_view* plan
   }
   return entity_backward(model, stream, plan, table, n_rows, q1, q2, score, gscore, B, K, dim, params, merged, m, v,
                          adam, workspace, workspace_bytes, 0, codes, codes_vec, codes_nit);
+}
+
+int smx_score_backward_entity_multi(int model, void* stream, const smx_plan_view* plan, float* table, size_t n_rows,
+                                    const float* q1, const float* q2, const smx_pair_source* src, size_t n_src,
+                                    size_t B, size_t dim, const smx_score_params* params, float* merged, float* m,
+                                    float* v, const smx_opt_params* adam, void* workspace, size_t workspace_bytes) {
+  using namespace smx;
+  if (!src || n_src == 0 || n_src > (size_t)kMaxSources)
+    return fail(SMX_ERR_ARG, "1 to %d pair sources", kMaxSources);
+  if (n_src == 1)
+    return smx_score_backward_entity(model, stream, plan, table, n_rows, q1, q2, src[0].score, src[0].gscore, B,
+                                     src[0].K, dim, params, merged, m, v, adam, workspace, workspace_bytes,
+                                     src[0].fwd_codes, src[0].fwd_codes_bytes);
+  if (model < 0 || model >= mNumModels) return fail(SMX_ERR_KIND, "unknown score model %d", model);
+  PairSources S{};
+  S.n = (int)n_src;
+  size_t k_sum = 0;
+  const bool coded = src[0].fwd_codes != nullptr;
+  int codes_vec = 0, codes_nit = 0;
+  if (coded) {
+    if (!model_coded(model) || code_bytes_per_pair(dim) > 2 * 64) return fail(SMX_ERR_ARG, "this model has no sign codes");
+    codes_vec = dim % 4 == 0 ? 4 : 1;
+    codes_nit = (int)(code_bytes_per_pair(dim) / 64);
+  }
+  for (size_t i = 0; i < n_src; ++i) {
+    if (!src[i].score || !src[i].gscore || src[i].K == 0) return fail(SMX_ERR_ARG, "incomplete pair source %zu", i);
+    if ((src[i].fwd_codes != nullptr) != coded) return fail(SMX_ERR_ARG, "sign codes for some pair sources only");
+    if (coded) {
+      if (src[i].fwd_codes_bytes != B * src[i].K * code_bytes_per_pair(dim))
+        return fail(SMX_ERR_ARG, "codes buffer of source %zu is not smx_score_codes_bytes() long", i);
+      if (reinterpret_cast<uintptr_t>(src[i].fwd_codes) & 15u) return fail(SMX_ERR_ARG, "codes must be 16-byte aligned");
+    }
+    S.score[i] = src[i].score;
+    S.gscore[i] = src[i].gscore;
+    S.codes[i] = static_cast<const unsigned char*>(src[i].fwd_codes);
+    S.K[i] = src[i].K;
+    k_sum += src[i].K;
+  }
+  if (B == 0 || B * k_sum > 0x7fffffffull) return fail(SMX_ERR_SHAPE, "pair count out of range");
+  if (!plan || plan->n_pairs != B * k_sum)
+    return fail(SMX_ERR_SHAPE, "the plan must hold the %zu pairs of all sources", B * k_sum);
+  // the same division of work as smx_score_backward_entity: ids that occur once in the whole step go through
+  // the pair-ordered kernel, one launch per source, while the entity pass reduces the others beside it
+  const bool split = coded && adam && !merged && plan->pair_seg && plan->uniq && plan->order && plan->sorted_ids &&
+                     plan->seg_of_pos && plan->seg_start && plan->n_uniq && queries_beyond_l2(model, B, dim) &&
+                     B * k_sum >= ((size_t)1 << 20) && workspace && !(reinterpret_cast<uintptr_t>(workspace) & 255u) &&
+                     workspace_bytes >= entity_ws_bytes(B * k_sum, dim * model_mul(model)) && !serial_backward();
+  if (split) {
+    if (const char* msg = check_opt_params(adam, m, v)) return fail(SMX_ERR_ARG, "%s", msg);
+    ScoreArgs A[kMaxSources];
+    bool fits = true;
+    size_t first = 0;
+    for (size_t i = 0; i < n_src && fits; ++i) {
+      int vec, nit;
+      if (int rc = fill_args(&A[i], &vec, &nit, model, table, n_rows, nullptr, q1, q2, B, src[i].K, dim, params, nullptr, m))
+        return rc;
+      fits = vec == codes_vec && nit == codes_nit && !(vec == 4 && v && !adam->squeeze && !aligned16(v));
+      A[i].n_rows = n_rows;
+      A[i].score = src[i].score;
+      A[i].gscore = src[i].gscore;
+      A[i].codes_in = S.codes[i];
+      A[i].pair_seg = plan->pair_seg + first;
+      A[i].uniq = reinterpret_cast<const long long*>(plan->uniq);
+      fill_sink(&A[i], table, m, v, nullptr, adam);
+      first += B * src[i].K;
+    }
+    if (fits) {
+      SideStream* side = side_stream();
+      if (!side) return fail(SMX_ERR_HIP, "cannot create the side stream");
+      hipStream_t st = as_stream(stream);
+      std::lock_guard<std::mutex> one_call(side->in_use);
+      if (hipEventRecord(side->fork, st) != hipSuccess || hipStreamWaitEvent(side->stream, side->fork, 0) != hipSuccess)
+        return fail(SMX_ERR_HIP, "fork to the side stream failed");
+      int rc = SMX_OK;
+      for (size_t i = 0; i < n_src && rc == SMX_OK; ++i)
+        rc = dispatch_model(model, st, A[i], codes_vec, codes_nit, false);  // gq1 == null: one-pair segments only
+      if (rc == SMX_OK)
+        rc = entity_backward(model, side->stream, plan, table, n_rows, q1, q2, nullptr, nullptr, B, k_sum, dim, params,
+                             nullptr, m, v, adam, workspace, workspace_bytes, 1, S.codes[0], codes_vec, codes_nit, &S);
+      if (hipEventRecord(side->join, side->stream) != hipSuccess || hipStreamWaitEvent(st, side->join, 0) != hipSuccess)
+        return fail(SMX_ERR_HIP, "join with the side stream failed");
+      return rc;
+    }
+  }
+  return entity_backward(model, stream, plan, table, n_rows, q1, q2, nullptr, nullptr, B, k_sum, dim, params, merged, m, v,
+                         adam, workspace, workspace_bytes, 0, S.codes[0], codes_vec, codes_nit, &S);
 }
 
 int smx_score_backward_fused(int model, void* stream, const smx_plan_view* plan, float* table, size_t n_rows,

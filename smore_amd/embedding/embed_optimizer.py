@@ -128,6 +128,10 @@ class EmbeddingOptimizer(ABC):
     def update_fused(self, plan, rec, lr):
         """Same for one fused record whose entity gradient is recomputed on the fly."""
 
+    @abstractmethod
+    def update_fused_multi(self, plan, recs, lr):
+        """Same for several fused records of one query batch; plan covers their ids in the order of recs."""
+
     # -- protocol of the training loop
     def zero_grad(self):
         self.grad_list, self.fused_list, self.has_grad_list = [], [], []
@@ -142,7 +146,7 @@ class EmbeddingOptimizer(ABC):
 
     def accumulate_fused(self, model, ids, q1, q2, score, gscore, params, fwd_idx, codes=None):
         self.fused_list.append(dict(model=model, ids=ids, q1=q1, q2=q2, score=score, gscore=gscore, params=params,
-                                    codes=codes))
+                                    codes=codes, fwd_idx=fwd_idx))
         self.has_grad_list.append(fwd_idx)
 
     def forward(self, indices, name=None):
@@ -269,6 +273,14 @@ class EmbeddingOptimizer(ABC):
                 plan = fused.build_plan(rec["ids"], n_rows, err_flag=self.err_flag)
                 self.update_fused(plan, rec, lr)
                 return
+            if not self.grad_list and self._one_query_batch(self.fused_list):
+                # positives and negatives of one query batch (kg_reasoning.py:340-355): one plan over all their
+                # ids, one entity pass that reads each record's own scores / upstream gradients / sign codes
+                recs = sorted(self.fused_list, key=lambda r: r["fwd_idx"])   # forward order, whatever autograd's was
+                flat = torch.cat([r["ids"].reshape(-1) for r in recs], dim=0)
+                plan = fused.build_plan(flat, n_rows, err_flag=self.err_flag)
+                self.update_fused_multi(plan, recs, lr)
+                return
             idx_list = [i.reshape(-1).to(self.sparse_embed.device) for i, _ in self.grad_list]
             grad_list = [g.reshape(g.shape[0] if g.dim() == 2 else -1, g.shape[-1]).contiguous().float()
                          for _, g in self.grad_list]
@@ -285,6 +297,27 @@ class EmbeddingOptimizer(ABC):
             rows = grad_list[0] if len(grad_list) == 1 else torch.cat(grad_list, dim=0)
             plan = fused.build_plan(flat, n_rows, err_flag=self.err_flag)
             self.update_from_plan(plan, rows.contiguous(), lr)
+
+
+    @staticmethod
+    def _one_query_batch(recs):
+        """True when the fused records can share one entity pass: same model and score parameters, the same
+        query tensors (same memory, shape and version), sign codes for all or none, few enough of them."""
+        if not 2 <= len(recs) <= _lib.MAX_PAIR_SOURCES:
+            return False
+        first = recs[0]
+
+        def same_tensor(a, b):
+            if a is None or b is None:
+                return a is b
+            return a.data_ptr() == b.data_ptr() and a.shape == b.shape and a._version == b._version
+
+        def same_params(a, b):
+            return all(getattr(a, f) == getattr(b, f) for f, _ in a._fields_)
+
+        return all(r["model"] == first["model"] and same_params(r["params"], first["params"]) and
+                   same_tensor(r["q1"], first["q1"]) and same_tensor(r["q2"], first["q2"]) and
+                   (r["codes"] is None) == (first["codes"] is None) for r in recs[1:])
 
 
 class _RowOptimizer(EmbeddingOptimizer):
@@ -318,6 +351,13 @@ class _RowOptimizer(EmbeddingOptimizer):
         m, v = self._state()
         fused.rows_backward(plan, grad_rows, table=self.sparse_embed.embedding.detach(), m=m, v=v,
                             adam=self._params(lr))
+
+    def update_fused_multi(self, plan, recs, lr):
+        m, v = self._state()
+        first = recs[0]
+        fused.score_backward_entity_multi(first["model"], plan, self.sparse_embed.embedding.detach(), first["q1"],
+                                          first["q2"], [(r["score"], r["gscore"], r["codes"]) for r in recs],
+                                          first["params"], m=m, v=v, adam=self._params(lr))
 
     def update_fused(self, plan, rec, lr):
         m, v = self._state()

@@ -237,6 +237,38 @@ def score_backward_entity(model, plan, table, q1, q2, score, gscore, params, mer
                   _ptr(codes), 0 if codes is None else codes.numel())
 
 
+def score_backward_entity_multi(model, plan, table, q1, q2, sources, params, merged=None, m=None, v=None, adam=None):
+    """score_backward_entity for several index streams of one query batch (see smx_score_backward_entity_multi).
+    sources: list of (score [B,K_s], gscore [B,K_s], codes or None); plan: built over the concatenation of the
+    streams' flattened ids in the same order."""
+    b, dim = q1.shape[0], q1.shape[-1]
+    if model not in MODELS:
+        raise _lib.SmxError(f"unknown score model {model}")
+    if not 1 <= len(sources) <= _lib.MAX_PAIR_SOURCES:
+        raise _lib.SmxError(f"1 to {_lib.MAX_PAIR_SOURCES} pair sources")
+    for t, name in ((table, "table"), (q1, "q1"), (q2, "q2"), (merged, "merged"), (m, "m"), (v, "v")):
+        _f32(t, name)
+    arr = (_lib.PairSource * len(sources))()
+    for i, (score, gscore, codes) in enumerate(sources):
+        _f32(score, "score")
+        _f32(gscore, "gscore")
+        if score.numel() % b or gscore.shape != score.shape:
+            raise _lib.SmxError("score and gscore of a source must both be [B, K]")
+        arr[i] = _lib.PairSource(_ptr(score), _ptr(gscore), _ptr(codes), 0 if codes is None else codes.numel(),
+                                 score.numel() // b)
+    row_len = table.shape[1]
+    _check_state(table, m, v, adam)
+    if merged is not None and (merged.dim() != 2 or merged.shape[1] != row_len):
+        raise _lib.SmxError("merged must be [n_uniq or more, row]")
+    with torch.cuda.device(table.device):
+        ws = _workspace(_lib.load().smx_entity_workspace_bytes(plan.n_pairs, row_len), table.device)
+        view = plan.view()
+        _lib.call("smx_score_backward_entity_multi", MODELS[model], _stream(table), ctypes.byref(view), _ptr(table),
+                  table.shape[0], _ptr(q1), _ptr(q2), ctypes.cast(arr, ctypes.c_void_p), len(sources), b, dim,
+                  ctypes.byref(params), _ptr(merged), _ptr(m), _ptr(v), None if adam is None else ctypes.byref(adam),
+                  _ptr(ws), ws.numel())
+
+
 def score_backward_fused(model, plan, table, idx, q1, q2, score, gscore, params, merged=None, m=None, v=None,
                          adam=None, sign_codes=True, codes=None):
     """Query gradients and all entity rows of the step in one call (see smx_score_backward_fused).

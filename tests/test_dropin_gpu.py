@@ -121,9 +121,14 @@ def _oracle_grads(name, table, ids, qs, rows, logit, gout, cen):
 
 @pytest.mark.parametrize("name", list(CASES))
 @pytest.mark.parametrize("branches", [1, 2])
-def test_model_code_without_score_negatives_matches_oracle(name, branches):
+def test_model_code_without_score_negatives_matches_oracle(name, branches, monkeypatch):
+    from smore_amd import fused
     from smore_amd.embedding.embed_optimizer import AdamEmbedOptimizer
     from smore_amd.embedding.sparse_embed import SparseEmbedding
+
+    def no_gradient_rows(*a, **k):
+        raise AssertionError("positives + negatives of one query batch must not go through materialised gradient rows")
+    monkeypatch.setattr(fused, "rows_backward", no_gradient_rows)
     cls, extra, model, n_q, mul, gamma, cen = CASES[name]
     n, d, b, k, lr = 400, 32, 6, 24, 1e-3
     rng = np.random.default_rng(11 + branches)

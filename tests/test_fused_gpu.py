@@ -825,3 +825,103 @@ def test_l1_codes_written_by_the_query_gradient_kernel():
         out.append((merged.cpu().numpy(), g1.cpu().numpy()))
     assert np.array_equal(out[0][0], out[1][0])
     assert_close(out[1][1], out[0][1], 1e-6, "gq1")
+
+
+@pytest.mark.parametrize("model", ["box", "l1", "l2", "rotate", "beta_kl"])
+def test_entity_pass_over_several_index_streams(model):
+    """smx_score_backward_entity_multi: three index streams of one query batch (K = 1, 7, 20; the first is what a
+    positive lookup looks like) behind one plan.  Merged rows against the oracle's unique-merge + scatter-sum over
+    the concatenated streams (embed_optimizer.py:39-48,155-163), then one Adam step per entity."""
+    from smore_amd import fused
+    n, b, dim, ks, lr = 150, 9, 24, (1, 7, 20), 1e-3
+    rng = np.random.default_rng(seed("multi", model))
+    table, q1, q2, _, _ = make_problem(model, n, b, 1, dim, rng)
+    gamma, cen = GAMMA[model], 0.02
+    params = fused.score_params(gamma, cen)
+    t_table, t_q1, t_q2 = dev(table), dev(q1), dev(q2)
+    o_q1 = q1[:, None, :]
+    o_q2 = None if q2 is None else q2[:, None, :]
+    ids, sources, o_rows = [], [], []
+    for k in ks:
+        idx = rng.integers(0, n, (b, k))
+        idx[0, 0] = 5                                   # an entity present in every stream
+        gs = rng.standard_normal((b, k)).astype(np.float32).astype(np.float64)
+        t_idx = torch.tensor(idx, device="cuda")
+        codes = fused.new_codes(model, t_table, t_idx, t_q1)
+        score = fused.score_forward(model, t_table, t_idx, t_q1, t_q2, params, codes=codes)
+        sources.append((score, dev(gs), codes))
+        ids.append(idx)
+        rows = orc.gather(table, idx).reshape(b, k, -1)
+        g_rows, _, _ = orc.score_backward(model, gs, rows, o_q1, o_q2, cen)
+        o_rows.append(g_rows.reshape(b * k, -1))
+    flat = np.concatenate([i.reshape(-1) for i in ids])
+    plan = fused.build_plan(torch.tensor(flat, device="cuda"), n, want_inverse=True)
+    uniq, inverse, _, _ = orc.merge_indices(flat)
+    o_merged = orc.merge_grads(np.concatenate(o_rows), inverse, uniq.size)
+    o_abs = orc.merge_grads(np.abs(np.concatenate(o_rows)), inverse, uniq.size)
+    merged = torch.full((uniq.size, table.shape[1]), float("nan"), device="cuda")
+    fused.score_backward_entity_multi(model, plan, t_table, t_q1, t_q2, sources, params, merged=merged)
+    assert_close(merged.cpu().numpy(), o_merged, REL_F32, f"{model} merged over three streams", sum_abs=o_abs)
+    # the optimizer step from the same pass, checked from the device's own merged rows
+    t_m, t_v = torch.zeros_like(t_table), torch.zeros_like(t_table)
+    w_s, m_s, v_s = table.copy(), np.zeros_like(table), np.zeros_like(table)
+    orc.adam_rows(w_s, m_s, v_s, uniq, merged.cpu().numpy().astype(np.float64), lr, 1)
+    fused.score_backward_entity_multi(model, plan, t_table, t_q1, t_q2, sources, params, m=t_m, v=t_v,
+                                      adam=fused.adam_params(lr, 1))
+    touched = np.zeros(n, bool)
+    touched[uniq] = True
+    assert_close(t_table.cpu().numpy()[touched], w_s[touched], REL_F32, f"{model} w over three streams")
+    assert_close(t_m.cpu().numpy()[touched], m_s[touched], REL_F32, f"{model} m over three streams")
+    assert_close(t_v.cpu().numpy()[touched], v_s[touched], REL_F32, f"{model} v over three streams", rms_floor=False)
+    assert np.array_equal(t_table.cpu().numpy()[~touched], table[~touched].astype(np.float32))
+    # one source through the same entry point is the single-stream call
+    one = torch.full((plan.n_uniq, table.shape[1]), float("nan"), device="cuda")
+    t_idx = torch.tensor(ids[2], device="cuda")
+    plan1 = fused.build_plan(t_idx, n)
+    a = torch.full((plan1.n_uniq, table.shape[1]), float("nan"), device="cuda")
+    b_ = torch.full_like(a, float("nan"))
+    fused.score_backward_entity_multi(model, plan1, dev(table), t_q1, t_q2, sources[2:], params, merged=a)
+    fused.score_backward_entity(model, plan1, dev(table), t_q1, t_q2, sources[2][0], sources[2][1], params, merged=b_,
+                                codes=sources[2][2])
+    assert torch.equal(a, b_)
+
+
+def test_several_index_streams_at_a_size_that_forks():
+    """Two streams (K = 1 and 300) of 4096 box queries, Adam: more than a million pairs and queries beyond one L2,
+    so ids that occur once go through the pair-ordered kernel (one launch per stream) beside the entity pass.
+    Against the same pairs laid out as one [B, 301] stream: the same rows are touched, the same values up to the
+    order of summation."""
+    from smore_amd import fused
+    n, b, dim, lr = 400_000, 4096, 200, 1e-3
+    g = torch.Generator(device="cuda").manual_seed(3)
+    table = torch.empty((n, dim), device="cuda").uniform_(-0.07, 0.07, generator=g)
+    q1 = torch.empty((b, dim), device="cuda").uniform_(-0.07, 0.07, generator=g)
+    q2 = torch.empty((b, dim), device="cuda").uniform_(-0.07, 0.07, generator=g).abs_()
+    pos = torch.randint(0, n, (b, 1), device="cuda", generator=g)
+    neg = torch.randint(0, n, (b, 300), device="cuda", generator=g)
+    gp = torch.randn((b, 1), device="cuda", generator=g)
+    gn = torch.randn((b, 300), device="cuda", generator=g)
+    params = fused.score_params(24.0, 0.02)
+
+    def run(streams):
+        w, m, v = table.clone(), torch.zeros_like(table), torch.zeros_like(table)
+        sources = []
+        for ids, gs in streams:
+            codes = fused.new_codes("box", w, ids, q1)
+            assert codes is not None
+            sources.append((fused.score_forward("box", w, ids, q1, q2, params, codes=codes), gs.contiguous(), codes))
+        plan = fused.build_plan(torch.cat([ids.reshape(-1) for ids, _ in streams]), n)
+        fused.score_backward_entity_multi("box", plan, w, q1, q2, sources, params, m=m, v=v, adam=fused.adam_params(lr, 1))
+        return w, m, v, plan
+
+    w2, m2, v2, plan2 = run([(pos, gp), (neg, gn)])
+    w1, m1, v1, plan1 = run([(torch.cat([pos, neg], dim=1), torch.cat([gp, gn], dim=1))])
+    assert plan1.n_uniq == plan2.n_uniq and torch.equal(plan1.uniq, plan2.uniq)
+    assert (plan2.pair_seg < 0).sum().item() > 30_000, "the case must have one-pair ids"
+    touched = torch.zeros(n, dtype=torch.bool, device="cuda")
+    touched[plan2.uniq] = True
+    assert torch.equal(w2[~touched], table[~touched]) and not bool(m2[~touched].any())
+    assert_close(m2[touched].cpu().numpy(), m1[touched].cpu().numpy(), REL_F32, "m, two streams vs one")
+    assert_close(v2[touched].cpu().numpy(), v1[touched].cpu().numpy(), REL_F32, "v, two streams vs one")
+    assert float((w2 - w1).abs().max()) <= 2 * lr
+    assert float(((w2 - w1).abs() > 1e-5 * 0.07).float().mean()) < 1e-4
