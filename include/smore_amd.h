@@ -49,6 +49,8 @@ extern "C" {
 #define SMX_MODEL_BOX 2     /* gamma - d_out - cen * d_in          models/box.py:157-164 */
 #define SMX_MODEL_ROTATE 3  /* gamma - sum sqrt(dre^2 + dim^2)     models/rotate.py:137-142 */
 #define SMX_MODEL_BETA_KL 4 /* gamma - sum KL(Beta(e) || Beta(q))  models/beta.py:303-308 */
+#define SMX_MODEL_COMPLEX 5 /* gamma + sum (e_re q_re + e_im q_im)  models/complex.py:140-148 (gamma = 0 there) */
+#define SMX_MODEL_DISTMULT 6 /* gamma + sum e q                     models/distmult.py, distmult_sim (gamma = 0 there) */
 
 int smx_version(void);
 const char* smx_last_error(void);

@@ -28,7 +28,7 @@ function is pinned by an independent check in tests/test_oracle_pinning.py:
                             first step; squeeze variant by closed form
   sgd / adagrad / rmsprop   torch.optim.SGD / Adagrad / RMSprop(alpha=0.99) when
                             every row is touched; squeeze variants by closed form
-  score / train_step        composition only (gamma - dist, chain rule of sqrt)
+  score / train_step        composition only (gamma - dist, gamma + similarity, chain rule of sqrt)
 """
 import ctypes
 import os
@@ -256,7 +256,8 @@ def filtered_ranks(scores, easy, hard):
 
 # ---- composition: the score of each model and one training step -------------------------------
 
-MODELS = ("l1", "l2", "box", "rotate", "beta_kl")
+MODELS = ("l1", "l2", "box", "rotate", "beta_kl", "complex", "distmult")
+SIMILARITY = ("complex", "distmult")
 
 
 def score_forward(model, rows, q1, q2=None, gamma=0.0, cen=0.0, dtype=np.float64):
@@ -267,6 +268,8 @@ def score_forward(model, rows, q1, q2=None, gamma=0.0, cen=0.0, dtype=np.float64
         d = dist_forward("box_out", rows, q1, q2, dtype) + cen * dist_forward("box_in", rows, q1, q2, dtype)
     elif model == "l2":
         d = np.sqrt(dist_forward("l2", rows, q1, None, dtype))
+    elif model in SIMILARITY:   # models/complex.py:140-148, distmult.py: the logit is the similarity itself
+        return (gamma + dist_forward(model, rows, q1, q2, dtype)).astype(dtype)
     else:
         d = dist_forward(model, rows, q1, q2, dtype)
     return (gamma - d).astype(dtype)
@@ -283,6 +286,8 @@ def score_backward(model, gscore, rows, q1, q2=None, cen=0.0, dtype=np.float64):
         d2 = dist_forward("l2", rows, q1, None, dtype)
         g = -gscore / (2.0 * np.sqrt(d2))
         return dist_backward("l2", g.astype(dtype), rows, q1, None, dtype)
+    if model in SIMILARITY:
+        return dist_backward(model, gscore, rows, q1, q2, dtype)
     return dist_backward(model, -gscore, rows, q1, q2, dtype)
 
 

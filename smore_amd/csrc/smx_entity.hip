@@ -35,6 +35,8 @@ extern template int entity_dispatch<mL2>(hipStream_t, const EntityArgs&, int, in
 extern template int entity_dispatch<mBox>(hipStream_t, const EntityArgs&, int, int);
 extern template int entity_dispatch<mRotate>(hipStream_t, const EntityArgs&, int, int);
 extern template int entity_dispatch<mBetaKL>(hipStream_t, const EntityArgs&, int, int);
+extern template int entity_dispatch<mComplex>(hipStream_t, const EntityArgs&, int, int);
+extern template int entity_dispatch<mDistmult>(hipStream_t, const EntityArgs&, int, int);
 extern template int entity_dispatch<kSrcRows>(hipStream_t, const EntityArgs&, int, int);
 
 constexpr int kTile = 256;      // sorted positions per tile of the long-segment pass
@@ -205,6 +207,8 @@ int entity_backward(int model, void* stream, const smx_plan_view* plan, float* t
     case mBox: return entity_dispatch<mBox>(st, A, vec, nit);
     case mRotate: return entity_dispatch<mRotate>(st, A, vec, nit);
     case mBetaKL: return entity_dispatch<mBetaKL>(st, A, vec, nit);
+    case mComplex: return entity_dispatch<mComplex>(st, A, vec, nit);
+    case mDistmult: return entity_dispatch<mDistmult>(st, A, vec, nit);
   }
   return fail(SMX_ERR_KIND, "unknown score model %d", model);
 }

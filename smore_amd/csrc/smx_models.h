@@ -7,6 +7,8 @@
 //   BOX        gamma - d_out - cen * d_in               smore/models/box.py:157-164
 //   ROTATE     gamma - sum sqrt(dre^2 + dim^2 + 1e-20)  smore/models/rotate.py:137-142
 //   BETA_KL    gamma - sum KL(Beta(e) || Beta(q))       smore/models/beta.py:303-308
+//   COMPLEX    gamma + sum (e_re q_re + e_im q_im)      smore/models/complex.py:140-148 (a similarity; gamma = 0 there)
+//   DISTMULT   gamma + sum e q                          smore/models/distmult.py (distmult_sim; gamma = 0 there)
 //
 // A model exposes
 //   fwd(e1,e2,q,acc0,acc1)      add one feature's term(s) to the lane's accumulators
@@ -23,10 +25,10 @@
 
 namespace smx {
 
-enum Model : int { mL1 = 0, mL2 = 1, mBox = 2, mRotate = 3, mBetaKL = 4, mNumModels = 5 };
+enum Model : int { mL1 = 0, mL2 = 1, mBox = 2, mRotate = 3, mBetaKL = 4, mComplex = 5, mDistmult = 6, mNumModels = 7 };
 
-__host__ __device__ constexpr int model_mul(int m) { return (m == mRotate || m == mBetaKL) ? 2 : 1; }
-__host__ __device__ constexpr int model_nq(int m) { return (m == mL1 || m == mL2) ? 1 : 2; }
+__host__ __device__ constexpr int model_mul(int m) { return (m == mRotate || m == mBetaKL || m == mComplex) ? 2 : 1; }
+__host__ __device__ constexpr int model_nq(int m) { return (m == mL1 || m == mL2 || m == mDistmult) ? 1 : 2; }
 // models whose entity derivative can be kept as sign codes (ModelOps<M>::bwd_q_coded / bwd_e_coded)
 __host__ __device__ constexpr bool model_coded(int m) { return m == mBox || m == mL1; }
 
@@ -341,6 +343,52 @@ template <> struct ModelOps<mBetaKL> {
     digamma3(e1, e2, pa, pb, ps);
     g1 += c0 * (q.k - pa + ps);
     g2 += c0 * (q.l - pb + ps);
+  }
+};
+
+// ComplEx and DistMult score by similarity, not distance (dist_kernel.h:187-204, 324-349): the logit grows
+// with the inner product, so the upstream coefficient keeps its sign.
+template <> struct ModelOps<mComplex> {
+  using Q = QPair;  // a = re, b = im
+  static __device__ __forceinline__ Q prep(float q1, float q2) { return {q1, q2}; }
+  static __device__ __forceinline__ void fwd(float e1, float e2, const Q& q, float& a0, float&) {
+    a0 += Term<kComplex, float>::fwd(e1, e2, q.a, q.b);
+  }
+  static __device__ __forceinline__ float fold(float a0, float, const ScoreParams&) { return a0; }
+  static __device__ __forceinline__ float score(float folded, const ScoreParams& p) { return p.gamma + folded; }
+  static __device__ __forceinline__ void coef(float g, float, const ScoreParams&, float& c0, float& c1) {
+    c0 = g;
+    c1 = 0.f;
+  }
+  static __device__ __forceinline__ void bwd_e(float c0, float, float e1, float e2, const Q& q, float& ge1, float& ge2) {
+    float s1 = 0, s2 = 0;
+    Term<kComplex, float>::bwd(c0, e1, e2, q.a, q.b, ge1, ge2, s1, s2);
+  }
+  static __device__ __forceinline__ void bwd_q(float c0, float, float e1, float e2, const Q& q, float& g1, float& g2) {
+    float s1 = 0, s2 = 0;
+    Term<kComplex, float>::bwd(c0, e1, e2, q.a, q.b, s1, s2, g1, g2);
+  }
+};
+
+template <> struct ModelOps<mDistmult> {
+  using Q = QPair;
+  static __device__ __forceinline__ Q prep(float q1, float) { return {q1, 0.f}; }
+  static __device__ __forceinline__ void fwd(float e1, float, const Q& q, float& a0, float&) {
+    a0 += Term<kDistmult, float>::fwd(e1, 0.f, q.a, 0.f);
+  }
+  static __device__ __forceinline__ float fold(float a0, float, const ScoreParams&) { return a0; }
+  static __device__ __forceinline__ float score(float folded, const ScoreParams& p) { return p.gamma + folded; }
+  static __device__ __forceinline__ void coef(float g, float, const ScoreParams&, float& c0, float& c1) {
+    c0 = g;
+    c1 = 0.f;
+  }
+  static __device__ __forceinline__ void bwd_e(float c0, float, float e1, float, const Q& q, float& ge1, float&) {
+    float s1 = 0, s2 = 0, s3 = 0;
+    Term<kDistmult, float>::bwd(c0, e1, 0.f, q.a, 0.f, ge1, s1, s2, s3);
+  }
+  static __device__ __forceinline__ void bwd_q(float c0, float, float e1, float, const Q& q, float& gq1, float&) {
+    float s1 = 0, s2 = 0, s3 = 0;
+    Term<kDistmult, float>::bwd(c0, e1, 0.f, q.a, 0.f, s1, s2, gq1, s3);
   }
 };
 

@@ -8,6 +8,8 @@ extern template int rank_dispatch<mL2>(hipStream_t, const RankArgs&, int, int, b
 extern template int rank_dispatch<mBox>(hipStream_t, const RankArgs&, int, int, bool);
 extern template int rank_dispatch<mRotate>(hipStream_t, const RankArgs&, int, int, bool);
 extern template int rank_dispatch<mBetaKL>(hipStream_t, const RankArgs&, int, int, bool);
+extern template int rank_dispatch<mComplex>(hipStream_t, const RankArgs&, int, int, bool);
+extern template int rank_dispatch<mDistmult>(hipStream_t, const RankArgs&, int, int, bool);
 
 constexpr size_t kRankMaxAnswers = 2048;  // per query; bins and keys of a pass live in LDS (per query of the pass 2049 x 4 + 2048 x 8 bytes)
 
@@ -53,6 +55,8 @@ static int rank_run(int model, hipStream_t st, const RankArgs& R, int vec, int n
     case mBox: return rank_dispatch<mBox>(st, R, vec, nit, keys_only);
     case mRotate: return rank_dispatch<mRotate>(st, R, vec, nit, keys_only);
     case mBetaKL: return rank_dispatch<mBetaKL>(st, R, vec, nit, keys_only);
+    case mComplex: return rank_dispatch<mComplex>(st, R, vec, nit, keys_only);
+    case mDistmult: return rank_dispatch<mDistmult>(st, R, vec, nit, keys_only);
   }
   return fail(SMX_ERR_KIND, "unknown score model %d", model);
 }

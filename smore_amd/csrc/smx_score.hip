@@ -27,6 +27,8 @@ extern template int score_dispatch<mL2>(hipStream_t, const ScoreArgs&, int, int,
 extern template int score_dispatch<mBox>(hipStream_t, const ScoreArgs&, int, int, bool);
 extern template int score_dispatch<mRotate>(hipStream_t, const ScoreArgs&, int, int, bool);
 extern template int score_dispatch<mBetaKL>(hipStream_t, const ScoreArgs&, int, int, bool);
+extern template int score_dispatch<mComplex>(hipStream_t, const ScoreArgs&, int, int, bool);
+extern template int score_dispatch<mDistmult>(hipStream_t, const ScoreArgs&, int, int, bool);
 
 // defined in smx_entity.hip
 int entity_backward(int model, void* stream, const smx_plan_view* plan, float* table, size_t n_rows, const float* q1,
@@ -82,6 +84,8 @@ static int dispatch_model(int model, hipStream_t st, const ScoreArgs& A, int vec
     case mBox: return score_dispatch<mBox>(st, A, vec, nit, forward);
     case mRotate: return score_dispatch<mRotate>(st, A, vec, nit, forward);
     case mBetaKL: return score_dispatch<mBetaKL>(st, A, vec, nit, forward);
+    case mComplex: return score_dispatch<mComplex>(st, A, vec, nit, forward);
+    case mDistmult: return score_dispatch<mDistmult>(st, A, vec, nit, forward);
   }
   return fail(SMX_ERR_KIND, "unknown score model %d", model);
 }

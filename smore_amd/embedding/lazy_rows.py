@@ -23,7 +23,8 @@ import torch
 
 from .. import _lib
 
-_FUSED_MODEL = {"l1": "l1", "l2": "l2", "rotate": "rotate", "beta_kl": "beta_kl"}
+_FUSED_MODEL = {"l1": "l1", "l2": "l2", "rotate": "rotate", "beta_kl": "beta_kl"}   # logit = const - dist
+_FUSED_SIMILARITY = ("complex", "distmult")                                          # logit = const + similarity
 
 
 def _is_lazy(x):
@@ -347,6 +348,8 @@ class LazyLogit(_Delegating):
                 return _FUSED_MODEL[d.kind], 0.0
             if k == -1.0 and d.kind == "box_out":
                 return "box", 0.0
+            if k == 1.0 and d.kind in _FUSED_SIMILARITY:        # models/complex.py:140-148: the similarity is the logit
+                return d.kind, 0.0
         if len(self.terms) == 2:
             (k0, d0), (k1, d1) = self.terms
             if d0.kind == "box_in":
@@ -374,7 +377,7 @@ class LazyLogit(_Delegating):
 
 def lazy_dist(kind, entity_embed, *queries):
     """What an operator of ext_ops returns for a LazyRows entity argument."""
-    if kind not in ("l1", "l2", "rotate", "beta_kl", "box_out", "box_in"):
+    if kind not in ("l1", "l2", "rotate", "beta_kl", "box_out", "box_in", "complex", "distmult"):
         return None
     if any(_is_lazy(q) or not isinstance(q, torch.Tensor) for q in queries):
         return None

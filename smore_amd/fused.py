@@ -13,9 +13,10 @@ import torch
 
 from . import _lib
 
-MODELS = {"l1": 0, "l2": 1, "box": 2, "rotate": 3, "beta_kl": 4}
-TWO_HALVES = ("rotate", "beta_kl")
-ONE_QUERY = ("l1", "l2")
+MODELS = {"l1": 0, "l2": 1, "box": 2, "rotate": 3, "beta_kl": 4, "complex": 5, "distmult": 6}
+TWO_HALVES = ("rotate", "beta_kl", "complex")
+ONE_QUERY = ("l1", "l2", "distmult")
+SIMILARITY = ("complex", "distmult")     # logit = gamma + sim; the others: gamma - distance
 
 
 def _stream(t):

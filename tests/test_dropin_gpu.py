@@ -2,7 +2,8 @@
 
 The classes below are a few-line restatement, written for this test, of how SMORE's models reach the scoring
 path: the lookup / view / regularizer / cal_logit sequence of KGReasoning.forward (kg_reasoning.py:298-307,
-340-355) and the four custom_cal_logit bodies (box.py:157-164, vec.py:85-90, rotate.py:137-142, beta.py:303-308).
+340-355) and the custom_cal_logit bodies (box.py:157-164, vec.py:85-90, rotate.py:137-142, beta.py:303-308,
+complex.py:140-148, distmult.py).
 They call only sp_embed(ids, name), tensor methods and ext_ops -- no score_negatives -- and must get, through the
 lazy lookup handle, the gather-fused scorer, with logits, query gradients and Adam state equal to the float64
 oracle's."""
@@ -85,6 +86,23 @@ class Beta(Reasoner):
         return torch.max(logit, dim=1)[0]
 
 
+class Complex(Reasoner):                           # complex.py:140-148 without its optional normalisation
+    def cal_logit(self, entity_embedding, entity_feat, query_embedding):
+        from smore_amd.torchext.ext_ops import complex_sim
+        assert entity_feat is None
+        re, im = query_embedding
+        logit = complex_sim(entity_embedding, re, im)
+        return torch.max(logit, dim=1)[0]
+
+
+class Distmult(Reasoner):
+    def cal_logit(self, entity_embedding, entity_feat, query_embedding):
+        from smore_amd.torchext.ext_ops import distmult_sim
+        assert entity_feat is None
+        logit = distmult_sim(entity_embedding, query_embedding[0])
+        return torch.max(logit, dim=1)[0]
+
+
 CASES = {
     # name: (class, extra ctor args, fused model, queries per branch, row / dim, gamma, cen)
     "box": (Box, (), "box", 2, 1, 24.0, 0.02),
@@ -92,6 +110,8 @@ CASES = {
     "l2": (Vec, ("l2",), "l2", 1, 1, 12.0, 0.0),
     "rotate": (Rotate, (), "rotate", 2, 2, 9.0, 0.0),
     "beta": (Beta, (), "beta_kl", 2, 2, 60.0, 0.0),
+    "complex": (Complex, (), "complex", 2, 2, 0.0, 0.0),
+    "distmult": (Distmult, (), "distmult", 1, 1, 0.0, 0.0),
 }
 
 

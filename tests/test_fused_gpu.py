@@ -10,12 +10,12 @@ from tests.util import REL_F32, assert_close, record_headroom, seed
 
 pytestmark = pytest.mark.gpu
 
-GAMMA = {"l1": 12.0, "l2": 12.0, "box": 24.0, "rotate": 9.0, "beta_kl": 60.0}
+GAMMA = {"l1": 12.0, "l2": 12.0, "box": 24.0, "rotate": 9.0, "beta_kl": 60.0, "complex": 0.0, "distmult": 0.0}
 
 
 def make_problem(model, n, b, k, dim, rng, zipf=None, scale=0.07):
     """Table, queries, ids and upstream gradient of one step, as fp32-representable float64."""
-    mul = 2 if model in ("rotate", "beta_kl") else 1
+    mul = 2 if model in ("rotate", "beta_kl", "complex") else 1
     f32 = lambda x: x.astype(np.float32).astype(np.float64)
     if model == "beta_kl":
         def beta(*s):
@@ -25,7 +25,7 @@ def make_problem(model, n, b, k, dim, rng, zipf=None, scale=0.07):
     else:
         table = rng.uniform(-scale, scale, (n, dim * mul))
         q1 = rng.uniform(-scale, scale, (b, dim))
-        q2 = None if model in ("l1", "l2") else rng.uniform(-scale, scale, (b, dim))
+        q2 = None if model in ("l1", "l2", "distmult") else rng.uniform(-scale, scale, (b, dim))
         if model == "box":
             q2 = np.abs(q2)
     if zipf is None:
@@ -64,7 +64,8 @@ def run_case(model, n, b, k, dim, zipf=None, cen=0.02, adam_steps=2, lr=1e-3):
     o_q2 = None if q2 is None else q2[:, None, :]
     want = orc.score_forward(model, rows, o_q1, o_q2, gamma, cen)
     # no RMS floor for the scores of the models whose distance is a sum of non-negative terms: every element to 1e-5
-    assert_close(score.cpu().numpy(), want, REL_F32, f"{model} score", rms_floor=model == "beta_kl")
+    # (a KL divergence or an inner product is a sum of signed terms)
+    assert_close(score.cpu().numpy(), want, REL_F32, f"{model} score", rms_floor=model in ("beta_kl", "complex", "distmult"))
     assert err.item() == 0
 
     # dense layout (idx = None) gives the same scores bit for bit
@@ -827,7 +828,7 @@ def test_l1_codes_written_by_the_query_gradient_kernel():
     assert_close(out[1][1], out[0][1], 1e-6, "gq1")
 
 
-@pytest.mark.parametrize("model", ["box", "l1", "l2", "rotate", "beta_kl"])
+@pytest.mark.parametrize("model", ["box", "l1", "l2", "rotate", "beta_kl", "complex", "distmult"])
 def test_entity_pass_over_several_index_streams(model):
     """smx_score_backward_entity_multi: three index streams of one query batch (K = 1, 7, 20; the first is what a
     positive lookup looks like) behind one plan.  Merged rows against the oracle's unique-merge + scatter-sum over
