@@ -104,6 +104,11 @@ class EmbeddingOptimizer(ABC):
             mode = tuple(x.strip() for x in mode.strip("()").split(","))
         self.optim_mode = mode
         self.optimizer_name = mode[1]
+        # mode[2] is where the reference keeps the optimizer statistics ('gpu' or 'cpu'); here they always live in
+        # HBM beside the table, so 'cpu' (what the reference's Freebase scripts pass) is accepted and means the same
+        self.optimizer_device = str(mode[2]).strip("'\" ") if len(mode) > 2 else "gpu"
+        if self.optimizer_device not in ("gpu", "cpu"):
+            raise _lib.SmxError(f"optimizer device must be 'gpu' or 'cpu', got {self.optimizer_device!r}")
         self.squeeze = str(mode[3]).lower() in ("true", "1") if len(mode) > 3 else False
         self.share_optim_stats = getattr(args, "share_optim_stats", True)
         if sp_embed.embedding.device.type != "cuda":
@@ -114,6 +119,23 @@ class EmbeddingOptimizer(ABC):
         self._flag_event = None                                                # set while such a copy is under way
         self.lazy_lookup = True
         self.prepare_state()
+
+    # -- set-up protocol of the trainer (embed_optimizer.py:71-75, 102-110; called as
+    #    get_optim_class(args).prepare_optimizers(args, sparse_embeds) before the workers start)
+    @classmethod
+    def prepare_embed(cls, args, optim_mode, embed, fn_register):
+        """Registers this optimizer's state tensors for `embed` through fn_register(name, tensor)."""
+
+    @classmethod
+    def prepare_optimizers(cls, args, list_sparse_embeds):
+        if not getattr(args, "share_optim_stats", True):
+            return
+        mode = args.optim_mode
+        if isinstance(mode, str):
+            mode = tuple(x.strip() for x in mode.strip("()").split(","))
+        for e in list_sparse_embeds:
+            assert isinstance(e, SparseEmbedding)
+            cls.prepare_embed(args, mode, e, e.register_tensor)
 
     # -- hooks of the concrete optimizer
     @abstractmethod
@@ -329,14 +351,20 @@ class _RowOptimizer(EmbeddingOptimizer):
     second_moment = None   # buffer name of the squared-gradient state, [N,row] or [N,1] with squeeze
     eps = 1e-8             # common/consts.py:20
 
+    @classmethod
+    def prepare_embed(cls, args, optim_mode, embed, fn_register):
+        """State buffers under the reference's names (embed_optimizer.py:190-197, 257-262, 314-320), zero-filled,
+        on the table's device; optim_mode[3] asks for one second-moment value per row."""
+        table = embed.embedding.detach()
+        squeeze = str(optim_mode[3]).lower() in ("true", "1") if len(optim_mode) > 3 else False
+        if cls.first_moment and not hasattr(embed, cls.first_moment):
+            fn_register(cls.first_moment, torch.zeros_like(table))
+        if cls.second_moment and not hasattr(embed, cls.second_moment):
+            shape = (table.shape[0], 1) if squeeze else tuple(table.shape)
+            fn_register(cls.second_moment, torch.zeros(shape, dtype=table.dtype, device=table.device))
+
     def prepare_state(self):
-        emb = self.sparse_embed
-        table = emb.embedding.detach()
-        if self.first_moment and not hasattr(emb, self.first_moment):
-            emb.register_tensor(self.first_moment, torch.zeros_like(table))
-        if self.second_moment and not hasattr(emb, self.second_moment):
-            shape = (table.shape[0], 1) if self.squeeze else tuple(table.shape)
-            emb.register_tensor(self.second_moment, torch.zeros(shape, dtype=table.dtype, device=table.device))
+        self.prepare_embed(self.args, self.optim_mode, self.sparse_embed, self.sparse_embed.register_tensor)
 
     def _state(self):
         emb = self.sparse_embed

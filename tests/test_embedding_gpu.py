@@ -352,6 +352,26 @@ def test_out_of_range_id_in_a_step_raises_from_the_next_apply_grad():
     opt.check_ids()       # the flag was cleared when the error was raised
 
 
+def test_trainer_set_up_protocol_and_cpu_statistics_mode():
+    """get_optim_class(args).prepare_optimizers(args, embeds) before the optimizer objects exist (the trainer's
+    order, embed_optimizer.py:102-110), the reference scripts' optim_mode with 'cpu' statistics and a squeezed
+    second moment, and a lookup with [B,K] ids keeping its shape."""
+    from smore_amd.embedding.embed_optimizer import AdamEmbedOptimizer, get_optim_class
+    from smore_amd.embedding.sparse_embed import SparseEmbedding
+    emb = SparseEmbedding(30, 8).cuda()
+    args = types.SimpleNamespace(optim_mode="(aggr, adam, cpu, True, 5)", share_optim_stats=True)
+    cls = get_optim_class(args)
+    assert cls is AdamEmbedOptimizer
+    cls.prepare_optimizers(args, [emb])
+    assert emb.state_sum_fo.shape == (30, 8) and emb.state_sum_sq.shape == (30, 1) and emb.state_sum_sq.is_cuda
+    fo = emb.state_sum_fo
+    opt = cls(args, emb, 0)
+    assert emb.state_sum_fo is fo and opt.squeeze and opt.optimizer_device == "cpu"
+    opt.lazy_lookup = False
+    rows = emb(torch.tensor([[1, 2, 3], [4, 5, 6]], device="cuda"), "x")
+    assert rows.shape == (2, 3, 8) and torch.equal(rows[1, 2], emb.embedding.detach()[6])
+
+
 def test_state_buffers_are_in_the_state_dict():
     emb, _ = _setup(20, 8, 11)
     sd = emb.state_dict()

@@ -38,7 +38,8 @@ def test_integer_valued_l1_ranks_are_exact_ties_included():
         assert got[i][1].cpu().numpy().tolist() == want_e.tolist()
 
 
-@pytest.mark.parametrize("model,dim", [("box", 200), ("l2", 64), ("rotate", 100), ("beta_kl", 40), ("box", 30)])
+@pytest.mark.parametrize("model,dim", [("box", 200), ("l2", 64), ("rotate", 100), ("beta_kl", 40), ("box", 30), ("complex", 48),
+                                       ("distmult", 64)])
 def test_ranks_lie_in_the_interval_fp32_allows(model, dim):
     """Random floats: an entity whose logit is within fp32 error of an answer's may fall on either side;
     every rank must lie between the counts with the tolerance subtracted and added."""
