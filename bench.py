@@ -339,6 +339,12 @@ def main():
     ap.add_argument("--no-sign-codes", action="store_true",
                     help="box: do not save sign codes in the forward; the backward re-reads entity and query rows")
     ap.add_argument("--seed", type=int, default=None)
+    ap.add_argument("--profile-run", action="store_true",
+                    help="only warm-up and timed steps (no kernel-by-kernel timing, bandwidth probes or CPU baseline "
+                         "afterwards): what a rocprofv3 run of this script should see")
+    ap.add_argument("--serial-backward", action="store_true",
+                    help="keep every kernel of the backward on one stream (the library's profiling switch), so that "
+                         "a kernel trace shows each kernel's duration by itself")
     ap.add_argument("--rank-scan", action="store_true",
                     help="time the all-entity evaluation scan (filtered ranks of 16 answers per query) on the "
                          "config's table instead of the training step; prints its own JSON line")
@@ -382,6 +388,8 @@ def main():
         rank_scan_bench(cfg, device, seed, args.steps, args.warmup, args.rank_queries)
         return
 
+    if args.serial_backward:
+        _lib.call("smx_set_option", _lib.OPTION_SERIAL_BACKWARD, 1)
     table, q1, q2, idx, gscore = make_inputs(cfg, device, seed)
     step = Step(cfg, table, q1, q2, idx, gscore, sign_codes=not args.no_sign_codes)
     for _ in range(args.warmup):
@@ -428,6 +436,14 @@ def main():
             _lib.call("smx_set_option", _lib.OPTION_SERIAL_BACKWARD, 0)
         return sum(e[2].elapsed_time(e[3]) for e in evs) / reps
 
+    if args.profile_run:
+        print(json.dumps({"workload": cfg["name"], "profile_run": True, "serial_backward": args.serial_backward,
+                          "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step, "phase_ms": phase_ms,
+                          "distinct_ids": n_uniq, "one_pair_ids": n_one_pair, "ids_with_2_to_64_pairs": n_short,
+                          "ids_with_more_pairs": n_long, "pairs": pairs, "algorithmic_bytes_step": algo,
+                          "algorithmic_bytes_query_kernel": q_bytes, "algorithmic_bytes_entity_pass": e_bytes,
+                          "algorithmic_bytes_backward_call": call_bytes, "sources": kernel_source_digest()}))
+        return
     query_alone_ms = timed_backward(1, True)     # the dominant kernel by itself, on the stream it is launched on
     entity_alone_ms = timed_backward(2, True)
     one_stream_ms = timed_backward(3, True)
