@@ -342,6 +342,9 @@ def main():
     ap.add_argument("--profile-run", action="store_true",
                     help="only warm-up and timed steps (no kernel-by-kernel timing, bandwidth probes or CPU baseline "
                          "afterwards): what a rocprofv3 run of this script should see")
+    ap.add_argument("--backward-parts", type=int, default=3, choices=(1, 2, 3),
+                    help="with --profile-run: run only the query-gradient kernel (1) or only the entity pass (2) of the "
+                         "backward call (the library's measuring switch); the steps are then incomplete")
     ap.add_argument("--serial-backward", action="store_true",
                     help="keep every kernel of the backward on one stream (the library's profiling switch), so that "
                          "a kernel trace shows each kernel's duration by itself")
@@ -390,6 +393,10 @@ def main():
 
     if args.serial_backward:
         _lib.call("smx_set_option", _lib.OPTION_SERIAL_BACKWARD, 1)
+    if args.backward_parts != 3:
+        if not args.profile_run:
+            sys.exit("--backward-parts is for --profile-run")
+        _lib.call("smx_set_option", _lib.OPTION_BACKWARD_PARTS, args.backward_parts)
     table, q1, q2, idx, gscore = make_inputs(cfg, device, seed)
     step = Step(cfg, table, q1, q2, idx, gscore, sign_codes=not args.no_sign_codes)
     for _ in range(args.warmup):
@@ -420,21 +427,22 @@ def main():
     call_bytes = backward_bytes(cfg, n_uniq, from_codes)
     q_bytes, e_bytes = backward_kernel_bytes(cfg, n_uniq, n_one_pair, from_codes)
 
-    def timed_backward(parts, serial, reps=5):
+    def timed_backward(parts, serial, reps=10, lead=3):
         """Average event-bracketed duration (ms) of the backward call with only `parts` of it running (the
         library's measuring switch; 3 = the whole call).  Run after the timed region: a call with one half
-        leaves an incomplete step behind."""
+        leaves an incomplete step behind.  The first `lead` steps are not counted: they let the host get ahead of
+        the device again, so that no bracket contains the device waiting for a launch."""
         _lib.call("smx_set_option", _lib.OPTION_SERIAL_BACKWARD, 1 if serial else 0)
         _lib.call("smx_set_option", _lib.OPTION_BACKWARD_PARTS, parts)
         try:
-            evs = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(reps)]
+            evs = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(lead + reps)]
             for e in evs:
                 step.run(e)
             torch.cuda.synchronize()
         finally:
             _lib.call("smx_set_option", _lib.OPTION_BACKWARD_PARTS, 3)
             _lib.call("smx_set_option", _lib.OPTION_SERIAL_BACKWARD, 0)
-        return sum(e[2].elapsed_time(e[3]) for e in evs) / reps
+        return sum(e[2].elapsed_time(e[3]) for e in evs[lead:]) / reps
 
     if args.profile_run:
         print(json.dumps({"workload": cfg["name"], "profile_run": True, "serial_backward": args.serial_backward,

@@ -121,8 +121,8 @@ def run_case(model, n, b, k, dim, zipf=None, cen=0.02, adam_steps=2, lr=1e-3):
     # fused Adam, several steps so m and v are non-trivial.  Adam divides by sqrt(v): where a summed
     # gradient cancels to ~eps its update is ill-conditioned, so (a) the Adam arithmetic is checked step
     # by step from the device's own state and merged gradient, to the 1e-5 bar, and (b) the end-to-end
-    # trajectory against the float64 oracle is checked to 1e-5 on all but a sliver of such elements,
-    # which must still be within two learning-rate steps (an Adam step is at most lr long, in either direction).
+    # trajectory against the float64 oracle is checked to 1e-5 on all but a sliver of such elements (at most 2 in
+    # 10,000), which must still be within a tenth of a learning-rate step per step taken.
     w_o, m_o, v_o = table.copy(), np.zeros_like(table), np.zeros_like(table)
     t_m, t_v = torch.zeros_like(t_table), torch.zeros_like(t_table)
     touched = np.zeros(n, bool)
@@ -147,9 +147,10 @@ def run_case(model, n, b, k, dim, zipf=None, cen=0.02, adam_steps=2, lr=1e-3):
     got_w = t_table.cpu().numpy()
     err = np.abs(got_w - w_o)[touched]
     tol = REL_F32 * np.maximum(np.abs(w_o[touched]), np.sqrt(np.mean(w_o[touched] ** 2)))
-    assert (err > tol).mean() < 1e-3 and err.max() < 2 * lr * adam_steps, (err.max(), (err > tol).mean())
-    record_headroom(f"{model} w trajectory: share of elements outside 1e-5 / 1e-3, worst error / (2 lr steps)",
-                    (err > tol).mean() / 1e-3, err.max() / (2 * lr * adam_steps))
+    # (worst seen over every case of this file: a share of 1.6e-5 and 0.003 lr per step)
+    assert (err > tol).mean() < 2e-4 and err.max() < 0.1 * lr * adam_steps, (err.max(), (err > tol).mean())
+    record_headroom(f"{model} w trajectory: share of elements outside 1e-5 / 2e-4, worst error / (0.1 lr steps)",
+                    (err > tol).mean() / 2e-4, err.max() / (0.1 * lr * adam_steps))
     assert_close(t_m.cpu().numpy()[touched], m_o[touched], 5 * REL_F32, f"{model} m trajectory")
     assert np.array_equal(got_w[~touched], table[~touched].astype(np.float32)), "untouched rows must stay bit-identical"
     assert not t_m.cpu().numpy()[~touched].any() and not t_v.cpu().numpy()[~touched].any()

@@ -7,7 +7,7 @@ import numpy as np
 import pytest
 
 from oracle import oracle as orc
-from tests.util import REL_F32, assert_close
+from tests.util import REL_F32, assert_close, record_headroom
 
 GOLDEN = sorted(glob.glob(os.path.join(os.path.dirname(__file__), "golden", "step_*.npz")))  # one per score model
 
@@ -73,7 +73,10 @@ def test_hip_path_reproduces_fixture(path):
                                     adam=fused.adam_params(float(d["lr"]), step))
     assert_close(m.cpu().numpy(), d["m_after"], 5 * REL_F32, "m after two steps")
     err = np.abs(table.cpu().numpy() - d["w_after"])
-    assert err.max() < 2 * float(d["lr"]) and (err > 1e-5 * np.maximum(np.abs(d["w_after"]), 0.04)).mean() < 0.01
+    share = (err > 1e-5 * np.maximum(np.abs(d["w_after"]), 0.04)).mean()
+    record_headroom("w after two steps: share of elements outside 1e-5 / 1e-2, worst error / (2 lr)", share / 0.01,
+                    err.max() / (2 * float(d["lr"])))
+    assert err.max() < 2 * float(d["lr"]) and share < 0.01
 
 
 @pytest.mark.gpu
@@ -102,7 +105,10 @@ def test_timed_path_reproduces_the_box_fixture():
                                    adam=fused.adam_params(float(d["lr"]), step), codes=codes)
     assert_close(m.cpu().numpy(), d["m_after"], 5 * REL_F32, "m after two steps")
     err = np.abs(table.cpu().numpy() - d["w_after"])
-    assert err.max() < 2 * float(d["lr"]) and (err > 1e-5 * np.maximum(np.abs(d["w_after"]), 0.04)).mean() < 0.01
+    share = (err > 1e-5 * np.maximum(np.abs(d["w_after"]), 0.04)).mean()
+    record_headroom("w after two steps: share of elements outside 1e-5 / 1e-2, worst error / (2 lr)", share / 0.01,
+                    err.max() / (2 * float(d["lr"])))
+    assert err.max() < 2 * float(d["lr"]) and share < 0.01
 
 
 def _golden(name):
