@@ -140,6 +140,8 @@ static int fill_args(ScoreArgs* A, int* vec, int* nit, int model, const float* t
   A->K = (int)K;
   A->ncol = (int)ncol;
   A->n_rows = idx ? n_rows : B * K;
+  A->id_bits = 1;
+  while (A->id_bits < 32 && ((A->n_rows - 1) >> A->id_bits) != 0) ++A->id_bits;
   A->p = ScoreParams{params->gamma, params->cen, params->reg_on, params->reg_add, params->reg_lo, params->reg_hi};
   return SMX_OK;
 }

@@ -35,6 +35,7 @@ struct ScoreArgs {
   float* gq1;
   float* gq2;
   int B, K, ncol;
+  int id_bits;           // significant bits of n_rows - 1 (at most 32): what the forward compares to find equal ids
   unsigned long long n_rows;
   ScoreParams p;
   int* err;
@@ -240,7 +241,14 @@ __device__ __forceinline__ void flush_codes(const unsigned char* stage, unsigned
   }
 }
 
-template <int M, int VEC, int NIT, int RIF, bool REG, bool CODED = false>
+// DEDUP: a wavefront scores each DISTINCT entity among its (up to 64) pairs once.  With skewed ids a query's
+// negatives repeat the hot entities many times (Zipf 1.1: ~51 distinct among 64 consecutive negatives), every
+// repeat costs the same instructions as the first occurrence although its row comes from the cache, and at such
+// shapes the kernel is bound by instruction issue.  The lanes find equal ids with one ballot per id bit, the
+// first lane of each group represents it, the representatives' rows are streamed, and every pair then takes
+// its score (and its code bytes, from the wavefront's LDS stage) from its representative: the same bits as
+// without de-duplication, pair by pair.
+template <int M, int VEC, int NIT, int RIF, bool REG, bool CODED = false, bool DEDUP = false>
 __global__ __launch_bounds__(256) void score_forward_kernel(ScoreArgs A, int tiles, int tile_k) {
   const float* __restrict__ table = A.table;
   const long long* __restrict__ idx = A.idx;
@@ -274,6 +282,27 @@ __global__ __launch_bounds__(256) void score_forward_kernel(ScoreArgs A, int til
   if (cnt <= 0) return;
   unsigned* slab = reinterpret_cast<unsigned*>(lds + model_nq(M) * dim) + wave * kSlabDwords;
   stage_pairs(slab, lane, table, pb, 0.f, 0.f);
+  int n_stream = cnt;        // rows this wavefront streams
+  int my_slot = lane;        // position among them of the row my pair's score comes from
+  if constexpr (DEDUP) {
+    const unsigned long long live = __ballot(lane < cnt);
+    const unsigned long long same = match_key(pb.row, A.id_bits, live) | (1ull << lane);
+    int rep = __builtin_ctzll(same);  // lowest lane with my id (ids that differ only above bit 31: checked below)
+    if (__shfl((int)pb.off_lo, rep) != (int)pb.off_lo || __shfl((int)pb.off_hi, rep) != (int)pb.off_hi) rep = lane;
+    const unsigned long long reps = __ballot(rep == lane && lane < cnt);
+    n_stream = __popcll(reps);
+    const int my_rank = (int)lanes_below_in(reps);   // for a representative: its position among the streamed rows
+    my_slot = __shfl(my_rank, rep);
+    // the slab holds every lane's own row address (stage_pairs, fenced); the representatives now move theirs to
+    // the front, in lane order.  rank <= lane, ranks are distinct, nobody reads in this phase, and the entries
+    // from n_stream on keep a valid address for the unconditional loads of the row loop
+    if (rep == lane && lane < cnt) {
+      const unsigned long long addr =
+          (unsigned long long)(table + (((unsigned long long)pb.off_hi << 32) | pb.off_lo));
+      *reinterpret_cast<uint2*>(slab + 4 * my_rank) = make_uint2((unsigned)addr, (unsigned)(addr >> 32));
+    }
+    slab_fence();
+  }
 
   float neg_thr[NIT][VEC];
   if constexpr (CODED) {
@@ -283,9 +312,11 @@ __global__ __launch_bounds__(256) void score_forward_kernel(ScoreArgs A, int til
       for (int v = 0; v < VEC; ++v) neg_thr[it][v] = ModelOps<M>::neg_threshold(q[it][v]);
   }
   float* out = score + (size_t)b * K + kw0;
+  constexpr int kStaged = DEDUP ? 64 : kStagePairs;  // pairs whose code bytes the wavefront's stage holds
   unsigned char* stage =
-      reinterpret_cast<unsigned char*>(lds + model_nq(M) * dim + 4 * kSlabDwords) + wave * (kStagePairs * NIT * 64);
-  stream_batch<MUL, VEC, NIT, RIF>(slab, cnt, dim, ncol, lane,
+      reinterpret_cast<unsigned char*>(lds + model_nq(M) * dim + 4 * kSlabDwords) + wave * (kStaged * NIT * 64);
+  float my_score = 0.f;  // DEDUP: lane j keeps the score of streamed row j
+  stream_batch<MUL, VEC, NIT, RIF>(slab, n_stream, dim, ncol, lane,
                                    [&](int j, const Pack<VEC>(&e1)[NIT], const Pack<VEC>(&e2)[NIT]) {
     // lanes past the row end hold a copy of the last column: they compute along and are dropped here.
     // The logit is linear in the accumulators: fold them per lane, reduce once.
@@ -297,7 +328,7 @@ __global__ __launch_bounds__(256) void score_forward_kernel(ScoreArgs A, int til
         unsigned code = 0;
 #pragma unroll
         for (int v = 0; v < VEC; ++v) ModelOps<M>::fwd_coded(e1[it].v[v], q[it][v], neg_thr[it][v], a0, a1, code);
-        stage[(j & (kStagePairs - 1)) * (NIT * 64) + 64 * it + lane] = (unsigned char)code;
+        stage[(j & (kStaged - 1)) * (NIT * 64) + 64 * it + lane] = (unsigned char)code;
       } else {
 #pragma unroll
         for (int v = 0; v < VEC; ++v) {
@@ -310,9 +341,34 @@ __global__ __launch_bounds__(256) void score_forward_kernel(ScoreArgs A, int til
       mine += lane + 64 * it < ncol ? f : 0.f;
     }
     const float folded = wave_sum_last_f32(mine);
-    if (lane == 63) out[j] = ModelOps<M>::score(folded, p);
-    if constexpr (CODED) flush_codes<NIT>(stage, A.codes, (size_t)b * K + kw0, j, cnt, lane);
+    if constexpr (DEDUP) {
+      const float s = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(ModelOps<M>::score(folded, p)), 63));
+      my_score = lane == j ? s : my_score;
+    } else {
+      if (lane == 63) out[j] = ModelOps<M>::score(folded, p);
+      if constexpr (CODED) flush_codes<NIT>(stage, A.codes, (size_t)b * K + kw0, j, cnt, lane);
+    }
   });
+  if constexpr (DEDUP) {
+    // every pair takes what its representative produced: the score from the lane that kept it ...
+    const float s = __shfl(my_score, my_slot);
+    if (lane < cnt) out[lane] = s;
+    if constexpr (CODED) {
+      // ... and its NIT x 64 code bytes from the representative's row of the stage, 16 bytes per lane and turn;
+      // the wavefront's pairs are contiguous in the code array
+      slab_fence();
+      typedef unsigned vec4u __attribute__((ext_vector_type(4)));
+      constexpr int kPer = NIT * 4;  // 16-byte pieces per pair
+      vec4u* dst = reinterpret_cast<vec4u*>(A.codes + ((size_t)b * K + kw0) * (size_t)(NIT * 64));
+      for (int c0 = 0; c0 < cnt * kPer; c0 += 64) {
+        const int c = c0 + lane;
+        const int pair = min(c / kPer, cnt - 1);
+        const int src_row = __shfl(my_slot, pair);
+        if (c < cnt * kPer)
+          __builtin_nontemporal_store(reinterpret_cast<const vec4u*>(stage + src_row * (NIT * 64))[c % kPer], dst + c);
+      }
+    }
+  }
   if (__ballot(bad != 0) != 0ull && err && lane == 0) *err = 1;
 }
 
@@ -604,15 +660,26 @@ int launch_forward_reg(hipStream_t st, const ScoreArgs& A) {
   while (tile_k > 4 * RIF && (B * ((K + tile_k - 1) / tile_k) < 8192 || (size_t)tile_k / 2 >= K)) tile_k /= 2;
   const int tiles = (int)((K + tile_k - 1) / tile_k);
   const size_t lds = ((size_t)model_nq(M) * A.ncol * VEC + 4 * kSlabDwords) * sizeof(float);
+  // ids given (not the dense layout, whose rows are all different): score each distinct entity of a
+  // wavefront's batch once
+  const bool dedup = A.idx != nullptr;
   if constexpr (model_coded(M) && !REG) {
     if (A.codes) {
-      hipLaunchKernelGGL((score_forward_kernel<M, VEC, NIT, RIF, REG, true>), dim3((unsigned)(B * tiles)), dim3(256),
-                         lds + 4 * kStagePairs * NIT * 64, st, A, tiles, tile_k);
+      if (dedup)
+        hipLaunchKernelGGL((score_forward_kernel<M, VEC, NIT, RIF, REG, true, true>), dim3((unsigned)(B * tiles)),
+                           dim3(256), lds + 4 * 64 * NIT * 64, st, A, tiles, tile_k);
+      else
+        hipLaunchKernelGGL((score_forward_kernel<M, VEC, NIT, RIF, REG, true>), dim3((unsigned)(B * tiles)), dim3(256),
+                           lds + 4 * kStagePairs * NIT * 64, st, A, tiles, tile_k);
       return check_launch("score forward (coded)");
     }
   }
-  hipLaunchKernelGGL((score_forward_kernel<M, VEC, NIT, RIF, REG>), dim3((unsigned)(B * tiles)), dim3(256), lds, st, A,
-                     tiles, tile_k);
+  if (dedup)
+    hipLaunchKernelGGL((score_forward_kernel<M, VEC, NIT, RIF, REG, false, true>), dim3((unsigned)(B * tiles)),
+                       dim3(256), lds, st, A, tiles, tile_k);
+  else
+    hipLaunchKernelGGL((score_forward_kernel<M, VEC, NIT, RIF, REG>), dim3((unsigned)(B * tiles)), dim3(256), lds, st, A,
+                       tiles, tile_k);
   return check_launch("score forward");
 }
 

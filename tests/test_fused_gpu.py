@@ -927,3 +927,50 @@ def test_several_index_streams_at_a_size_that_forks():
     assert_close(v2[touched].cpu().numpy(), v1[touched].cpu().numpy(), REL_F32, "v, two streams vs one")
     assert float((w2 - w1).abs().max()) <= 2 * lr
     assert float(((w2 - w1).abs() > 1e-5 * 0.07).float().mean()) < 1e-4
+
+
+@pytest.mark.parametrize("model,dim", [("box", 200), ("box", 400), ("l1", 30), ("l2", 64), ("rotate", 48), ("beta_kl", 20)])
+def test_forward_scores_each_distinct_entity_of_a_wavefront_once(model, dim):
+    """The forward de-duplicates ids inside a wavefront's batch of up to 64 negatives: every pair must still get
+    the bits it would get alone.  Queries whose negatives are all one entity, all distinct, drawn from three
+    entities, and a last batch of 6 pairs (K = 70); scores against the dense layout (rows given pair by pair, no
+    ids, no de-duplication) bit for bit and against the oracle; sign codes (box, l1) through the backward that
+    reads them against the backward that recomputes from the rows, bit for bit."""
+    from smore_amd import fused
+    rng = np.random.default_rng(seed("dedup", model, dim))
+    n, b, k = 90, 5, 70
+    table, q1, q2, idx, gs = make_problem(model, n, b, k, dim, rng)
+    idx[0, :] = 7
+    idx[1, :] = np.arange(k) % n
+    idx[2, :] = rng.choice([3, 4, 88], size=k)
+    idx[3, :64] = 11                                   # the first batch all equal, the short last batch distinct
+    idx[3, 64:] = np.arange(6) + 20
+    gamma = GAMMA[model]
+    params = fused.score_params(gamma, 0.02)
+    t_table, t_q1, t_q2, t_gs = dev(table), dev(q1), dev(q2), dev(gs)
+    t_idx = torch.tensor(idx, device="cuda")
+    score = fused.score_forward(model, t_table, t_idx, t_q1, t_q2, params)
+    rows = orc.gather(table, idx).reshape(b, k, -1)
+    dense = fused.score_forward(model, dev(rows.reshape(b * k, -1)), None, t_q1, t_q2, params)
+    assert torch.equal(score, dense)
+    want = orc.score_forward(model, rows, q1[:, None], None if q2 is None else q2[:, None], gamma, 0.02)
+    assert_close(score.cpu().numpy(), want, REL_F32, f"{model} score with repeated ids", rms_floor=model == "beta_kl")
+    assert bool((score[0] == score[0, 0]).all()) and bool((score[3, :64] == score[3, 0]).all())
+    codes = fused.new_codes(model, t_table, t_idx, t_q1)
+    if model in ("box", "l1"):
+        assert codes is not None
+        score_c = fused.score_forward(model, t_table, t_idx, t_q1, t_q2, params, codes=codes)
+        assert torch.equal(score_c, score)
+        per_pair = codes.view(b, k, -1)
+        assert torch.equal(per_pair[0], per_pair[0, :1].expand(k, -1)), "repeats must carry their representative's codes"
+        plan = fused.build_plan(t_idx, n)
+        got = {}
+        for use in (True, False):
+            merged = torch.full((plan.n_uniq, table.shape[1]), float("nan"), device="cuda")
+            g1, g2 = fused.score_backward_fused(model, plan, t_table, t_idx, t_q1, t_q2, score, t_gs, params,
+                                                merged=merged, sign_codes=False, codes=codes if use else None)
+            got[use] = (merged, g1, g2)
+        assert torch.equal(got[True][0], got[False][0])
+        assert_close(got[True][1].cpu().numpy(), got[False][1].cpu().numpy(), 1e-6, "gq1 from the forward's codes")
+    else:
+        assert codes is None
