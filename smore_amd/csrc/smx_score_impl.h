@@ -315,7 +315,6 @@ __global__ __launch_bounds__(256) void score_forward_kernel(ScoreArgs A, int til
   constexpr int kStaged = DEDUP ? 64 : kStagePairs;  // pairs whose code bytes the wavefront's stage holds
   unsigned char* stage =
       reinterpret_cast<unsigned char*>(lds + model_nq(M) * dim + 4 * kSlabDwords) + wave * (kStaged * NIT * 64);
-  float my_score = 0.f;  // DEDUP: lane j keeps the score of streamed row j
   stream_batch<MUL, VEC, NIT, RIF>(slab, n_stream, dim, ncol, lane,
                                    [&](int j, const Pack<VEC>(&e1)[NIT], const Pack<VEC>(&e2)[NIT]) {
     // lanes past the row end hold a copy of the last column: they compute along and are dropped here.
@@ -342,17 +341,18 @@ __global__ __launch_bounds__(256) void score_forward_kernel(ScoreArgs A, int til
     }
     const float folded = wave_sum_last_f32(mine);
     if constexpr (DEDUP) {
-      const float s = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(ModelOps<M>::score(folded, p)), 63));
-      my_score = lane == j ? s : my_score;
+      // the score of streamed row j waits in the third word of slab entry j (free in the forward; the entry's
+      // address words were consumed when the row was requested): one LDS store instead of vector selects
+      if (lane == 63) slab[4 * j + 2] = __float_as_uint(ModelOps<M>::score(folded, p));
     } else {
       if (lane == 63) out[j] = ModelOps<M>::score(folded, p);
       if constexpr (CODED) flush_codes<NIT>(stage, A.codes, (size_t)b * K + kw0, j, cnt, lane);
     }
   });
   if constexpr (DEDUP) {
-    // every pair takes what its representative produced: the score from the lane that kept it ...
-    const float s = __shfl(my_score, my_slot);
-    if (lane < cnt) out[lane] = s;
+    // every pair takes what its representative produced: the score from the representative's slab entry ...
+    slab_fence();
+    if (lane < cnt) out[lane] = __uint_as_float(slab[4 * my_slot + 2]);
     if constexpr (CODED) {
       // ... and its NIT x 64 code bytes from the representative's row of the stage, 16 bytes per lane and turn;
       // the wavefront's pairs are contiguous in the code array
