@@ -14,7 +14,8 @@ import pytest
 import torch
 
 from oracle import oracle as orc
-from tests.util import REL_F32, assert_adam_weights, assert_close, oracle_union_grads, oracle_union_logits
+from tests.util import (REL_F32, assert_adam_weights, assert_close, oracle_adam_step, oracle_union_grads,
+                        oracle_union_logits)
 
 pytestmark = pytest.mark.gpu
 
@@ -280,3 +281,52 @@ def test_shared_negatives_and_other_uses_of_the_rows():
     orc.adam_rows(w, m, v, uniq, merged, lr, 1)
     assert_close(emb.state_sum_fo.cpu().numpy()[uniq], m[uniq], REL_F32, "first moment")
     assert_adam_weights(emb.embedding.detach().cpu().numpy(), w, merged, uniq, lr, "weights")
+
+
+def test_inverse_query_call_sequence_runs_on_the_reverse_layout():
+    """Inverse ('<') queries, kg_reasoning.py:306-336: the TAIL entity is looked up and becomes the 'entity' operand
+    [B,1,D] (embed_reverse_query, :252-255), while the negatives go through the relation projection
+    (cal_reverse_logit, :257-263; vec.py:58-60: rows + relation) and arrive as the 'query' operand [B,1,K,D].
+    Arithmetic on the negatives' handle needs their values, and the distance has nothing to gather-fuse: both
+    lookups fall back to rows, the operator runs on its reverse-layout kernels, and apply_grad merges the two
+    gradient-row records.  Logits, relation gradient and the Adam step against the float64 oracle."""
+    from smore_amd.embedding.embed_optimizer import AdamEmbedOptimizer
+    from smore_amd.embedding.sparse_embed import SparseEmbedding
+    from smore_amd.torchext.ext_ops import l1_dist
+    n, d, b, k, lr = 300, 32, 6, 20, 1e-3
+    rng = np.random.default_rng(31)
+    table = rng.uniform(-0.07, 0.07, (n, d)).astype(np.float32).astype(np.float64)
+    rel = rng.uniform(-0.07, 0.07, (b, d)).astype(np.float32).astype(np.float64)
+    tail, neg = rng.integers(0, n, b), rng.integers(0, n // 3, (b, k))
+    gn = rng.standard_normal((b, k)).astype(np.float32).astype(np.float64)
+    emb = SparseEmbedding(n, d).cuda()
+    with torch.no_grad():
+        emb.embedding.copy_(torch.tensor(table, dtype=torch.float32))
+    opt = AdamEmbedOptimizer(types.SimpleNamespace(optim_mode="(aggr,adam,gpu,False,5)", share_optim_stats=True), emb, 0)
+    t_rel = torch.tensor(rel, dtype=torch.float32, device="cuda", requires_grad=True)
+    gamma = torch.nn.Parameter(torch.Tensor([12.0]).cuda(), requires_grad=False)
+
+    opt.zero_grad()
+    all_negative = emb(torch.tensor(neg, device="cuda").view(-1), "negative_entity")
+    inv_query_embed = emb(torch.tensor(tail, device="cuda")).unsqueeze(1)                  # embed_reverse_query
+    all_negative.job_handle.sync()
+    embedding = [all_negative.view(b, k, -1)]
+    embedding = [embedding[0] + t_rel.unsqueeze(1)]                                          # relation_projection
+    query_embedding = [e.unsqueeze(1) for e in embedding]
+    logit = gamma - l1_dist(inv_query_embed, query_embedding[0])                             # custom_cal_logit, vec.py:85-90
+    logit = torch.max(logit, dim=1)[0]
+    assert logit.shape == (b, k)
+    (logit * torch.tensor(gn, dtype=torch.float32, device="cuda")).sum().backward()
+    assert len(opt.grad_list) == 2 and not opt.fused_list
+    opt.apply_grad(lr)
+
+    # oracle: dist(entity = tail rows [B,1,D], query = negatives + relation [B,K,D]) -> [B,K]
+    e = orc.gather(table, tail).reshape(b, 1, d)
+    q = orc.gather(table, neg).reshape(b, k, d) + rel[:, None, :]
+    want = 12.0 - orc.dist_forward("l1", e, q)
+    assert_close(logit.detach().cpu().numpy(), want, REL_F32, "inverse-query logits")
+    g_e, g_q, _ = orc.dist_backward("l1", -gn, e, q)
+    assert_close(t_rel.grad.cpu().numpy(), g_q.sum(axis=1), REL_F32, "relation gradient")
+    w, m, v, uniq, merged = oracle_adam_step(table, [tail, neg], [g_e.reshape(b, d), g_q.reshape(b * k, d)], lr, 1)
+    assert_close(emb.state_sum_fo.cpu().numpy()[uniq], m[uniq], REL_F32, "inverse query: first moment")
+    assert_adam_weights(emb.embedding.detach().cpu().numpy(), w, merged, uniq, lr, "inverse query: weights")
