@@ -54,6 +54,29 @@ def test_host_only_entry_points():
     assert abs(out[0] + 1e-3 / (1 - 0.9 ** 2)) < 1e-9 and abs(out[1] - (1 - 0.999 ** 2) ** -0.5) < 1e-4
 
 
+def test_multi_stream_entity_pass_refuses_bad_source_lists():
+    """Argument checks of smx_score_backward_entity_multi happen before any launch: they can run without a GPU."""
+    from smore_amd import _lib
+    import ctypes as c
+    lib = _lib.load()
+    params = _lib.ScoreParams(24.0, 0.02, 0, 0.0, 0.0, 0.0)
+    plan = _lib.PlanView(None, None, None, None, None, None, None, 40)
+    src = (_lib.PairSource * 5)()
+    fake = c.c_void_p(256)          # never dereferenced: every case below is refused on the host
+    for i in range(5):
+        src[i] = _lib.PairSource(fake, fake, None, 0, 4)
+    call = lambda n_src, b=2: lib.smx_score_backward_entity_multi(
+        2, None, c.byref(plan), fake, 100, fake, fake, c.cast(src, c.c_void_p), n_src, b, 8, c.byref(params), fake, None,
+        None, None, fake, 1 << 20)
+    assert call(0) != 0 and call(5) != 0
+    assert b"pair sources" in lib.smx_last_error()
+    assert call(2, b=7) != 0 and b"pairs" in lib.smx_last_error()          # 2 sources x 7 x 4 pairs, the plan holds 40
+    src[1] = _lib.PairSource(fake, fake, fake, 64, 4)                       # sign codes for one source only
+    assert call(2, b=5) != 0 and b"sign codes" in lib.smx_last_error()
+    src[1] = _lib.PairSource(fake, None, None, 0, 4)
+    assert call(2, b=5) != 0 and b"incomplete" in lib.smx_last_error()
+
+
 def test_missing_library_fails_loudly(monkeypatch):
     from smore_amd import _lib
     monkeypatch.setattr(_lib, "_lib", None)
