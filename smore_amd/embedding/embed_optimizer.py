@@ -60,11 +60,12 @@ class _FusedScoreFunc(torch.autograd.Function):
     autograd but recorded with the optimizer, which reduces it per entity in apply_grad."""
 
     @staticmethod
-    def forward(ctx, embed_opt, dummy_tensor, model, ids, params, q1, q2):
+    def forward(ctx, embed_opt, dummy_tensor, model, ids, params, q1, q2, for_training=True):
         table = embed_opt.sparse_embed.embedding.detach()
         with torch.no_grad():
-            # box: the forward leaves 2-bit sign codes from which both backward passes work (None otherwise)
-            codes = fused.new_codes(model, table, ids, q1) if table.shape[1] % 4 == 0 else None
+            # box, l1: the forward leaves 2-bit sign codes from which both backward passes work (None otherwise;
+            # none either when no backward will follow, e.g. scoring sampled negatives under torch.no_grad())
+            codes = fused.new_codes(model, table, ids, q1) if for_training and table.shape[1] % 4 == 0 else None
             score = fused.score_forward(model, table, ids, q1, q2, params, embed_opt.err_flag, codes=codes)
         ctx.embed_opt, ctx.model, ctx.ids, ctx.params, ctx.codes = embed_opt, model, ids, params, codes
         ctx.save_for_backward(q1.detach(), q2.detach() if q2 is not None else None, score)
@@ -82,7 +83,7 @@ class _FusedScoreFunc(torch.autograd.Function):
             gq1, gq2 = fused.score_backward_query(ctx.model, table, ctx.ids, q1, q2, score, gscore, ctx.params,
                                                   codes=ctx.codes)
         opt.accumulate_fused(ctx.model, ctx.ids, q1, q2, score, gscore, ctx.params, ctx.idx_fwd, ctx.codes)
-        return None, None, None, None, None, gq1, gq2
+        return None, None, None, None, None, gq1, gq2, None
 
 
 class EmbeddingOptimizer(ABC):
@@ -243,7 +244,7 @@ class EmbeddingOptimizer(ABC):
         q1c = q1.reshape(b * branches, dim).contiguous()
         q2c = None if q2 is None else q2.reshape(b * branches, dim).contiguous()
         params = fused.score_params(gamma, cen, regularizer)
-        logit = _FusedScoreFunc.apply(self, self.dummy_tensor, model, ids, params, q1c, q2c)
+        logit = _FusedScoreFunc.apply(self, self.dummy_tensor, model, ids, params, q1c, q2c, torch.is_grad_enabled())
         return logit.view(b, branches, -1)
 
     def _raise_for(self, code):

@@ -372,6 +372,26 @@ def test_trainer_set_up_protocol_and_cpu_statistics_mode():
     assert rows.shape == (2, 3, 8) and torch.equal(rows[1, 2], emb.embedding.detach()[6])
 
 
+def test_scoring_without_gradients_saves_no_codes_and_leaves_no_record(monkeypatch):
+    """Evaluation on sampled negatives (train_process.py:103-108) runs the model code under torch.no_grad():
+    same logits, no sign-code buffer, nothing for apply_grad."""
+    from smore_amd import fused
+    emb, opt = _setup(60, 16, 13)
+    c = torch.rand(4, 1, 16, device="cuda") * 0.1
+    o = torch.rand(4, 1, 16, device="cuda") * 0.1
+    ids = torch.randint(0, 60, (4, 9), device="cuda")
+    opt.zero_grad()
+    want = opt.score_negatives("box", ids, c, o, gamma=24.0, cen=0.02)
+    made = []
+    real = fused.new_codes
+    monkeypatch.setattr(fused, "new_codes", lambda *a, **k: made.append(1) or real(*a, **k))
+    with torch.no_grad():
+        got = opt.score_negatives("box", ids, c, o, gamma=24.0, cen=0.02)
+    assert torch.equal(got, want) and not made and not got.requires_grad
+    opt.zero_grad()
+    opt.apply_grad(1e-3)
+
+
 def test_state_buffers_are_in_the_state_dict():
     emb, _ = _setup(20, 8, 11)
     sd = emb.state_dict()
