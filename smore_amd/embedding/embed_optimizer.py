@@ -97,6 +97,7 @@ class EmbeddingOptimizer(ABC):
         sp_embed.fwd_delegate = self.forward
         self.dummy_tensor = nn.Parameter(torch.randn(1, 1))
         self.grad_list, self.fused_list, self.has_grad_list = [], [], []
+        self.pending_scores = []    # LazyScores of this step that nothing has needed yet
         self.n_fwd = 0
         self.step = 0
         self.gpu_id = gpu_id
@@ -158,6 +159,7 @@ class EmbeddingOptimizer(ABC):
     # -- protocol of the training loop
     def zero_grad(self):
         self.grad_list, self.fused_list, self.has_grad_list = [], [], []
+        self.pending_scores = []
         self.n_fwd = 0
 
     def share_memory(self):
@@ -194,10 +196,10 @@ class EmbeddingOptimizer(ABC):
         mat.job_handle = self.sparse_embed.dummy_job
         return mat
 
-    def score_lazy(self, model, rows, queries, gamma, cen):
-        """Logits gamma - dist(rows, queries) for a LazyRows handle [Be, K, row] against query tensors [B, 1, D]
-        (-> [B, K]) or [B, U, 1, D] (-> [B, U, K], one slice per union branch as the dense operators return it),
-        in one launch of the fused scorer.  None when this is not a layout the fused scorer takes."""
+    def lazy_request(self, model, rows, queries, gamma, cen):
+        """What one launch of the fused scorer needs for gamma - dist(rows, queries) with a LazyRows handle
+        [Be, K, row] against query tensors [B, 1, D] or [B, U, 1, D]: a dict, or None when this is not a layout the
+        fused scorer takes."""
         q = queries[0]
         if q.dim() == 4:
             bq, nc, dim = q.shape[0], q.shape[2], q.shape[3]
@@ -211,9 +213,43 @@ class EmbeddingOptimizer(ABC):
             return None
         if any(t.dtype != torch.float32 or t.device != rows.device for t in queries):
             return None
-        q2 = queries[1] if n_q == 2 else None
-        logit = self._score_branches(model, rows.ids.reshape(be, k), q, q2, gamma, cen, rows.reg)
-        return logit if q.dim() == 4 else logit[:, 0]
+        return dict(model=model, ids=rows.ids.reshape(be, k), q1=q, q2=queries[1] if n_q == 2 else None, gamma=gamma,
+                    cen=cen, reg=rows.reg, b=bq)
+
+    def score_lazy(self, model, rows, queries, gamma, cen):
+        """Those logits in one launch of the fused scorer: [B, K], or [B, U, K] for 4-D queries (one slice per
+        union branch, as the dense operators return it).  None when this is not a layout the fused scorer takes."""
+        r = self.lazy_request(model, rows, queries, gamma, cen)
+        if r is None:
+            return None
+        logit = self._score_branches(model, r["ids"], r["q1"], r["q2"], gamma, cen, r["reg"])
+        return logit if r["q1"].dim() == 4 else logit[:, 0]
+
+    def evaluate_pending(self, wanted):
+        """Computes `wanted` (a LazyScores) together with every other pending one of this step that can share its
+        launch: same model, margin, parameters, prologue and query tensors.  Their ids go side by side."""
+        w = wanted.request
+
+        def same(a, b):     # the same memory read the same way (the very tensor, or an equal view of it)
+            if a is None or b is None:
+                return a is b
+            return a is b or (a.data_ptr() == b.data_ptr() and a.shape == b.shape and a.stride() == b.stride() and
+                              a._version == b._version and a.requires_grad == b.requires_grad)
+
+        group = [p for p in self.pending_scores if p._value is None and p.request["model"] == w["model"] and
+                 p.request["gamma"] == w["gamma"] and p.request["cen"] == w["cen"] and p.request["reg"] == w["reg"] and
+                 same(p.request["q1"], w["q1"]) and same(p.request["q2"], w["q2"])]
+        if not any(p is wanted for p in group):
+            group.append(wanted)
+        ids = [p.request["ids"].to(self.sparse_embed.embedding.device) for p in group]
+        if len(group) > 1:      # ids shared by the batch ([1, K]) stand beside per-query ones as [B, K]
+            ids = [i.expand(w["b"], i.shape[1]) if i.shape[0] == 1 else i for i in ids]
+        all_ids = ids[0] if len(ids) == 1 else torch.cat(ids, dim=1)
+        logit = self._score_branches(w["model"], all_ids, w["q1"], w["q2"], w["gamma"], w["cen"], w["reg"])[:, 0]
+        parts = [logit] if len(ids) == 1 else torch.split(logit, [i.shape[1] for i in ids], dim=1)
+        for p, part in zip(group, parts):
+            p._value = part
+        self.pending_scores = [p for p in self.pending_scores if p._value is None]
 
     def score_negatives(self, model, ids, q1, q2=None, gamma=0.0, cen=0.0, regularizer=None):
         """Gather-fused logits [B,K]; q1/q2 are [B,dim] or [B,1,dim] and receive gradients.
@@ -282,6 +318,7 @@ class EmbeddingOptimizer(ABC):
         IndexError as table[idx] does in the reference (embed_rw.py:74-75) -- with check_ids_every_step (default)
         from the apply_grad of the following step, so that no step waits for the device; check_ids() asks at once."""
         self.step += 1  # counts calls, also those without gradients (embed_optimizer.py:156)
+        self.pending_scores = []    # logits that nothing used have no gradient and must not ride along later
         if not self.grad_list and not self.fused_list:
             return
         self._apply_grad(lr)

@@ -28,7 +28,7 @@ _FUSED_SIMILARITY = ("complex", "distmult")                                     
 
 
 def _is_lazy(x):
-    return isinstance(x, (LazyRows, LazyLogit))
+    return isinstance(x, _Delegating)
 
 
 def _resolve(x):
@@ -69,8 +69,44 @@ def _scalar(x):
     return None
 
 
+def _binary(name, reflected=False):
+    def op(self, other):
+        a, b = self.materialize(), _resolve(other)
+        return getattr(torch, name)(b, a) if reflected else getattr(torch, name)(a, b)
+    return op
+
+
 class _Delegating:
     """Everything a handle does not know about is done by the tensor it stands for."""
+
+    # Python's operators do not go through __getattr__: the defaults compute on the tensor (subclasses keep the
+    # ones they can do lazily)
+    __add__ = _binary("add")
+    __radd__ = _binary("add", True)
+    __sub__ = _binary("sub")
+    __rsub__ = _binary("sub", True)
+    __mul__ = _binary("mul")
+    __rmul__ = _binary("mul", True)
+    __truediv__ = _binary("div")
+    __rtruediv__ = _binary("div", True)
+    __matmul__ = _binary("matmul")
+    __pow__ = _binary("pow")
+    __lt__ = _binary("lt")
+    __le__ = _binary("le")
+    __gt__ = _binary("gt")
+    __ge__ = _binary("ge")
+
+    def __neg__(self):
+        return -self.materialize()
+
+    def __abs__(self):
+        return abs(self.materialize())
+
+    def __float__(self):
+        return float(self.materialize())
+
+    def __bool__(self):
+        return bool(self.materialize())
 
     def materialize(self):
         raise NotImplementedError
@@ -103,13 +139,6 @@ class _Delegating:
 
     def __repr__(self):
         return f"{type(self).__name__}(shape={tuple(self.shape)})"
-
-
-def _binary(name, reflected=False):
-    def op(self, other):
-        a, b = self.materialize(), _resolve(other)
-        return getattr(torch, name)(b, a) if reflected else getattr(torch, name)(a, b)
-    return op
 
 
 class LazyRows(_Delegating):
@@ -191,17 +220,6 @@ class LazyRows(_Delegating):
         return out
 
     __radd__ = __add__
-    __sub__ = _binary("sub")
-    __rsub__ = _binary("sub", True)
-    __mul__ = _binary("mul")
-    __rmul__ = _binary("mul", True)
-    __truediv__ = _binary("div")
-    __rtruediv__ = _binary("div", True)
-    __matmul__ = _binary("matmul")
-    __pow__ = _binary("pow")
-
-    def __neg__(self):
-        return -self.materialize()
 
     @classmethod
     def _try_lazy(cls, func, args, kwargs):
@@ -337,6 +355,17 @@ class LazyLogit(_Delegating):
                 return a.__mul__(b) if lazy_first else b.__mul__(a)
         if name in ("neg", "negative", "__neg__") and len(args) == 1 and not kwargs:
             return -args[0]
+        if name == "max" and args and isinstance(args[0], LazyLogit):
+            # torch.max(logit, dim=1) of custom_cal_logit: with ONE union branch the maximum is that branch, and
+            # the logits can wait until something needs their values -- by then the step's other lookups against
+            # the same queries (positives, negatives) have been scored too and all go into one launch
+            dim = kwargs.get("dim", args[1] if len(args) > 1 else None)
+            self = args[0]
+            if (dim == 1 and len(args) <= 2 and set(kwargs) <= {"dim"} and self._value is None and
+                    len(self.shape) == 3 and self.shape[1] == 1 and self._fusable() is not None):
+                scores = LazyScores(self)
+                if scores.request is not None:
+                    return _MaxResult(scores, _LazyZeros(scores.shape, scores.device))
         return NotImplemented
 
     # -- evaluation
@@ -373,6 +402,58 @@ class LazyLogit(_Delegating):
                 value = value + k * d.dense()
         self._value = value
         return value
+
+
+class _MaxResult(tuple):
+    """(values, indices) as torch.max(x, dim) returns them."""
+
+    def __new__(cls, values, indices):
+        return super().__new__(cls, (values, indices))
+
+    values = property(lambda self: self[0])
+    indices = property(lambda self: self[1])
+
+
+class _LazyZeros(_Delegating):
+    """Indices of a maximum over a dimension of size one: zeros, made only if somebody looks."""
+
+    def __init__(self, shape, device):
+        self.shape, self.device, self.dtype = torch.Size(shape), device, torch.int64
+
+    def materialize(self):
+        return torch.zeros(self.shape, dtype=torch.int64, device=self.device)
+
+
+class LazyScores(_Delegating):
+    """Logits [B, K] of one lookup against one branch of queries, not yet computed.  The optimizer keeps the
+    step's pending ones; the first that is needed evaluates all that share its model, margin, parameters and
+    query tensors in one launch of the fused scorer (ids side by side, [B, K_1 + K_2 + ..]), so that the step
+    leaves one record with the optimizer, as if the caller had concatenated positives and negatives itself."""
+
+    def __init__(self, logit):
+        self.logit = logit
+        self._value = None
+        d = logit.terms[0][1]
+        self.opt = d.rows.opt
+        model, cen = logit._fusable()
+        self.request = self.opt.lazy_request(model, d.rows, d.queries, logit.const, cen)   # None: not a fused layout
+        if self.request is not None:
+            self.opt.pending_scores.append(self)
+
+    shape = property(lambda self: torch.Size((self.logit.shape[0], self.logit.shape[2])))
+    device = property(lambda self: self.logit.device)
+    dtype = torch.float32
+
+    def dim(self):
+        return 2
+
+    def size(self, d=None):
+        return self.shape if d is None else self.shape[d]
+
+    def materialize(self):
+        if self._value is None:
+            self.opt.evaluate_pending(self)
+        return self._value
 
 
 def lazy_dist(kind, entity_embed, *queries):

@@ -12,24 +12,33 @@ from smore_amd.torchext import ext_ops
 
 
 class RecordingOptimizer:
-    """Stands where EmbeddingOptimizer stands for a LazyRows handle."""
+    """Stands where EmbeddingOptimizer stands for a LazyRows handle: the real request / batching logic, with the
+    launch of the fused scorer replaced by textbook torch expressions and a record of what was asked."""
+    from smore_amd.embedding.embed_optimizer import EmbeddingOptimizer as _Real
+    lazy_request = _Real.lazy_request
+    score_lazy = _Real.score_lazy
+    evaluate_pending = _Real.evaluate_pending
 
     def __init__(self, n, row):
         g = torch.Generator().manual_seed(5)
         table = torch.rand((n, row), generator=g) * 2 - 0.5
         self.sparse_embed = types.SimpleNamespace(embedding=table, dummy_job=types.SimpleNamespace(sync=lambda: None))
-        self.scored, self.looked_up = [], []
+        self.scored, self.looked_up, self.pending_scores = [], [], []
 
     def lookup_rows(self, ids, name=None):
         self.looked_up.append(name)
         return self.sparse_embed.embedding[ids]
 
-    def score_lazy(self, model, rows, queries, gamma, cen):
-        self.scored.append((model, tuple(rows.shape), gamma, cen, rows.reg))
-        e = self.sparse_embed.embedding[rows.ids.reshape(-1)].view(rows.shape)
-        if rows.reg is not None:
-            e = torch.clamp(e + rows.reg[0], rows.reg[1], rows.reg[2])
-        return gamma - _textbook(model, e, queries, cen)
+    def _score_branches(self, model, ids, q1, q2, gamma, cen, reg):
+        """[B, U, K] logits, as the real optimizer's launch returns them."""
+        self.scored.append((model, tuple(ids.shape), gamma, cen, reg))
+        e = self.sparse_embed.embedding[ids]
+        if reg is not None:
+            e = torch.clamp(e + reg[0], reg[1], reg[2])
+        if q1.dim() == 3:
+            q1, q2 = q1.unsqueeze(1), None if q2 is None else q2.unsqueeze(1)
+        sign = 1.0 if model in ("complex", "distmult") else -1.0
+        return gamma + sign * _textbook(model, e, (q1, q2), cen)
 
 
 def _textbook(model, e, queries, cen):
@@ -70,7 +79,7 @@ def test_box_logit_of_the_model_code_is_one_fused_request():
     logit = gamma - d1 - 0.02 * d2
     assert isinstance(logit, LazyLogit) and logit.shape == (b, u, k) and not opt.scored
     out = torch.max(logit, dim=1)[0]
-    assert opt.scored == [("box", (b, k, d), 24.0, 0.02, None)] and not opt.looked_up
+    assert opt.scored == [("box", (b, k), 24.0, 0.02, None)] and not opt.looked_up
     e = opt.sparse_embed.embedding[ids]
     want = torch.max(24.0 - _textbook("box", e, (c, o), 0.02), dim=1)[0]
     assert torch.allclose(out, want, rtol=0, atol=1e-5)
@@ -87,7 +96,10 @@ def test_one_distance_models(op, model, n_q):
     rows = LazyRows(opt, ids, "positive_entity").unsqueeze(1)
     logit = 12.0 - getattr(ext_ops, op)(rows, *q)
     out = torch.max(logit, dim=1)[0]
-    assert opt.scored == [(model, (b, 1, d * mul), 12.0, 0.0, None)]
+    assert not opt.scored, "one branch: the logits wait until somebody needs them"
+    assert out.shape == (b, 1) and out.dim() == 2
+    assert torch.allclose(out, (12.0 - _textbook(model, opt.sparse_embed.embedding[ids].unsqueeze(1), q, 0.0))[:, 0], rtol=0, atol=1e-5)
+    assert opt.scored == [(model, (b, 1), 12.0, 0.0, None)]
     e = opt.sparse_embed.embedding[ids].unsqueeze(1)
     assert torch.allclose(out, (12.0 - _textbook(model, e, q, 0.0))[:, 0], rtol=0, atol=1e-5)
 
@@ -154,3 +166,40 @@ def test_scalar_tensor_values_are_not_confused_between_tensors():
     assert (gamma - ext_ops.l1_dist(rows, q)).const == 1.0
     gamma.fill_(2.0)
     assert (gamma - ext_ops.l1_dist(rows, q)).const == 2.0
+
+
+def test_positives_and_negatives_of_one_query_batch_share_one_launch():
+    """kg_reasoning.py:340-355: positives [B] and negatives [B,K] are scored against the same query tensors by two
+    cal_logit calls.  With one union branch both logits stay pending after torch.max; the first use evaluates both
+    in one request with the ids side by side, and each gets its own columns."""
+    n, d, b, k = 60, 8, 4, 6
+    opt = RecordingOptimizer(n, d)
+    gen = torch.Generator().manual_seed(2)
+    pos, neg = torch.randint(0, n, (b,), generator=gen), torch.randint(0, n, (b, k), generator=gen)
+    c, o = _queries(b, 1, d, 2, 12)
+    gamma = torch.nn.Parameter(torch.tensor([24.0]), requires_grad=False)
+
+    def cal_logit(rows):
+        logit = gamma - ext_ops.box_dist_out(rows, c, o) - 0.02 * ext_ops.box_dist_in(rows, c, o)
+        return torch.max(logit, dim=1)[0]
+
+    lp = cal_logit(LazyRows(opt, pos, "positive_entity").unsqueeze(1))
+    ln = cal_logit(LazyRows(opt, neg.view(-1), "negative_entity").view(b, k, -1))
+    assert not opt.scored and len(opt.pending_scores) == 2 and lp.shape == (b, 1) and ln.shape == (b, k)
+    loss = -torch.nn.functional.logsigmoid(lp).mean() - torch.nn.functional.logsigmoid(-ln).mean()
+    assert opt.scored == [("box", (b, 1 + k), 24.0, 0.02, None)] and not opt.pending_scores and not opt.looked_up
+    table = opt.sparse_embed.embedding
+    want_p = (24.0 - _textbook("box", table[pos].unsqueeze(1), (c, o), 0.02))[:, 0]
+    want_n = (24.0 - _textbook("box", table[neg], (c, o), 0.02))[:, 0]
+    assert torch.allclose(lp.materialize(), want_p, atol=1e-5) and torch.allclose(ln.materialize(), want_n, atol=1e-5)
+    want = -torch.nn.functional.logsigmoid(want_p).mean() - torch.nn.functional.logsigmoid(-want_n).mean()
+    assert torch.allclose(loss, want, atol=1e-6)
+    # other queries, another margin or several branches do not join
+    c2, o2 = _queries(b, 1, d, 2, 13)
+    other = torch.max(24.0 - ext_ops.box_dist_out(LazyRows(opt, neg.view(-1), None).view(b, k, -1), c2, o2), dim=1)[0]
+    again = cal_logit(LazyRows(opt, pos, None).unsqueeze(1))
+    assert len(opt.pending_scores) == 2
+    float(again.sum())
+    assert opt.scored[-1] == ("box", (b, 1), 24.0, 0.02, None) and len(opt.pending_scores) == 1
+    values, indices = torch.max(24.0 - ext_ops.l1_dist(LazyRows(opt, pos, None).unsqueeze(1), c), dim=1)
+    assert indices.shape == (b, 1) and int(indices.sum()) == 0
