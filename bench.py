@@ -180,7 +180,9 @@ class Step:
         self.codes = fused.new_codes(cfg["model"], table, idx, q1) if sign_codes else None
         self.plan = None
 
-    def run(self, events=None):
+    def run(self, events=None, step_consts=None):
+        """step_consts: two-float device tensor the optimizer kernels read lr / bias corrections from (a captured
+        step is replayed with frozen by-value arguments, so the advancing step counter has to come from memory)."""
         f, cfg = self.fused, self.cfg
         mark = (lambda i: events[i].record()) if events is not None else (lambda i: None)
         self.step_no += 1
@@ -192,16 +194,62 @@ class Step:
         mark(2)
         if cfg["adam"]:
             gq = f.score_backward_fused(cfg["model"], plan, self.table, self.idx, self.q1, self.q2, score, self.gscore,
-                                        self.params, m=self.m, v=self.v, adam=f.adam_params(cfg["lr"], self.step_no),
+                                        self.params, m=self.m, v=self.v,
+                                        adam=f.adam_params(cfg["lr"], self.step_no, step_consts=step_consts),
                                         codes=self.codes)
         else:
-            if self.merged is None:
-                self.merged = self.torch.empty((plan.n_uniq, self.table.shape[1]), device=self.table.device)
+            if self.merged is None:     # one row per distinct id; no more of those than pairs or table rows
+                self.merged = self.torch.empty((min(self.idx.numel(), cfg["n"]), self.table.shape[1]),
+                                               device=self.table.device)
             gq = f.score_backward_fused(cfg["model"], plan, self.table, self.idx, self.q1, self.q2, score, self.gscore,
                                         self.params, merged=self.merged, codes=self.codes)
         mark(3)
         self.plan = plan
         return score, gq
+
+
+def time_graph_replays(step, steps, warmup):
+    """The same step captured once in a HIP graph (torch.cuda.CUDAGraph: plan, forward, backward + optimizer, the
+    library's second stream included) and replayed: ms per step over `steps` replays after `warmup` untimed ones.
+    The optimizer's per-step constants come from a two-float device buffer that is rewritten before every
+    replay (an 8-byte device copy from a table staged beforehand), so the step counter advances as in the
+    eager loop."""
+    import ctypes
+    import torch
+    from smore_amd import _lib, fused
+    cfg, dev = step.cfg, step.table.device
+    consts, staged = None, None
+    if cfg["adam"]:
+        host = (ctypes.c_float * 2)()
+        rows = []
+        for i in range(warmup + steps):
+            opt = fused.adam_params(cfg["lr"], step.step_no + 1 + i)
+            _lib.call("smx_opt_step_consts", ctypes.byref(opt), host)
+            rows.append([host[0], host[1]])
+        staged = torch.tensor(rows, dtype=torch.float32, device=dev)
+        consts = staged[0].clone()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step.run(step_consts=consts)
+    torch.cuda.synchronize()
+
+    def replay(i):
+        if consts is not None:
+            consts.copy_(staged[i])
+        graph.replay()
+    for i in range(warmup):
+        replay(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        replay(warmup + i)
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / steps
+    if step.err.item() != 0:
+        sys.exit("a replayed step reported an error")
+    step.step_no += warmup + steps
+    return ms
 
 
 def cpu_baseline(cfg, seed):
@@ -345,6 +393,9 @@ def main():
     ap.add_argument("--backward-parts", type=int, default=3, choices=(1, 2, 3),
                     help="with --profile-run: run only the query-gradient kernel (1) or only the entity pass (2) of the "
                          "backward call (the library's measuring switch); the steps are then incomplete")
+    ap.add_argument("--graph", action="store_true",
+                    help="also capture the whole step (plan, forward, backward + optimizer, second stream included) "
+                         "in a HIP graph and time its replays; reported as graph_replay next to the eager figures")
     ap.add_argument("--serial-backward", action="store_true",
                     help="keep every kernel of the backward on one stream (the library's profiling switch), so that "
                          "a kernel trace shows each kernel's duration by itself")
@@ -427,6 +478,8 @@ def main():
     call_bytes = backward_bytes(cfg, n_uniq, from_codes)
     q_bytes, e_bytes = backward_kernel_bytes(cfg, n_uniq, n_one_pair, from_codes)
 
+    graph_ms = time_graph_replays(step, args.steps, args.warmup) if args.graph else None
+
     def timed_backward(parts, serial, reps=10, lead=3):
         """Average event-bracketed duration (ms) of the backward call with only `parts` of it running (the
         library's measuring switch; 3 = the whole call).  Run after the timed region: a call with one half
@@ -447,6 +500,7 @@ def main():
     if args.profile_run:
         print(json.dumps({"workload": cfg["name"], "profile_run": True, "serial_backward": args.serial_backward,
                           "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step, "phase_ms": phase_ms,
+                          "graph_replay_ms_per_step": graph_ms,
                           "distinct_ids": n_uniq, "one_pair_ids": n_one_pair, "ids_with_2_to_64_pairs": n_short,
                           "ids_with_more_pairs": n_long, "pairs": pairs, "algorithmic_bytes_step": algo,
                           "algorithmic_bytes_query_kernel": q_bytes, "algorithmic_bytes_entity_pass": e_bytes,
@@ -516,6 +570,9 @@ def main():
         },
         "phase_ms": phase_ms,
     }
+    if graph_ms is not None:
+        out["graph_replay"] = {"ms_per_step": graph_ms, "value": pairs / (graph_ms * 1e-3), "unit": "pairs/s",
+                               "frac_of_peak": algo / (graph_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS}
     # what plain kernels sustain on this GPU for the step's access shapes, measured now with the library's
     # probes (after the timed region); a step that writes w, m, v back is a copy-like mix of reads and writes
     try:
