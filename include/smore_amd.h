@@ -256,7 +256,13 @@ int smx_score_backward_entity(int model, void* stream, const smx_plan_view* plan
  * score its forward produced, the upstream gradient, and its sign codes (all sources or none); q1, q2, B, dim,
  * params are common to all.  An entity that occurs in several sources gets ONE update from the sum of all its
  * pairs' gradients, summed in plan order (source by source, pairs ascending).  n_src == 1 is
- * smx_score_backward_entity.  workspace: smx_entity_workspace_bytes(total pairs, dim*mul). */
+ * smx_score_backward_entity.
+ * grad_rows (may be NULL): [n_grad_rows, dim*mul] gradient rows that autograd has materialised for the step's
+ * plain lookups -- the anchor entities every query starts from (models/box.py:137), which reach the optimizer
+ * as (indices, gradient rows) records of their own (embed_optimizer.py:63-66, 146-148).  Their ids are the last
+ * n_grad_rows entries of the plan's concatenation; a row is added to its entity's gradient after the model's own
+ * part is complete (clamp mask of the entity prologue included), so that such an entity too gets ONE update.
+ * workspace: smx_entity_workspace_bytes(plan->n_pairs, dim*mul). */
 #define SMX_MAX_PAIR_SOURCES 4
 typedef struct smx_pair_source {
   const float* score;      /* [B, K] */
@@ -269,7 +275,8 @@ int smx_score_backward_entity_multi(int model, void* stream, const smx_plan_view
                                     size_t n_rows, const float* q1, const float* q2,
                                     const smx_pair_source* src, size_t n_src, size_t B, size_t dim,
                                     const smx_score_params* params, float* merged, float* m, float* v,
-                                    const smx_opt_params* adam, void* workspace, size_t workspace_bytes);
+                                    const smx_opt_params* adam, void* workspace, size_t workspace_bytes,
+                                    const float* grad_rows, size_t n_grad_rows);
 
 /* Everything after the loss in one call: query gradients, and every entity row of the step finished
  * (merged gradient row and/or lazy Adam on w, m, v), as smx_score_backward_query followed by

@@ -49,7 +49,7 @@ SIGNATURES = {
                                        _vp, _vp, _sz, _vp, _sz]),
     # model, stream, plan, table, n_rows, q1, q2, src[], n_src, B, dim, params, merged, m, v, adam, ws, ws_bytes
     "smx_score_backward_entity_multi": (_i, [_i, _vp, _vp, _vp, _sz, _vp, _vp, _vp, _sz, _sz, _sz, _vp, _vp, _vp, _vp,
-                                             _vp, _vp, _sz]),
+                                             _vp, _vp, _sz, _vp, _sz]),
     # model, stream, plan, table, n_rows, idx, q1, q2, score, gscore, gq1, gq2, B, K, dim, params, merged, m, v,
     # adam, ws, ws_bytes, fwd_codes, fwd_codes_bytes
     "smx_score_backward_fused": (_i, [_i, _vp, _vp, _vp, _sz, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _vp,

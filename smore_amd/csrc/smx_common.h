@@ -34,6 +34,10 @@ struct PairSources {
   const float* gscore[kMaxSources];
   const unsigned char* codes[kMaxSources];
   size_t K[kMaxSources];
+  // behind the pairs of all sources the plan may hold n_grad more entries whose gradient autograd has already
+  // materialised as a row each (plain lookups of the step: anchor entities): grad_rows[n_grad, row]
+  const float* grad_rows;
+  size_t n_grad;
 };
 
 inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }

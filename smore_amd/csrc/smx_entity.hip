@@ -85,6 +85,7 @@ static int fill_plan(EntityArgs* A, const smx_plan_view* plan, void* workspace, 
   A->uniq = reinterpret_cast<const long long*>(plan->uniq);
   A->n_uniq = plan->n_uniq;
   A->n_pairs = (int)plan->n_pairs;
+  A->rows_first = (int)plan->n_pairs;  // no gradient rows of plain lookups behind the model's pairs
   A->tile = kTile;
   A->short_max = kShortMax;
   char* ws = static_cast<char*>(workspace);
@@ -159,9 +160,16 @@ int entity_backward(int model, void* stream, const smx_plan_view* plan, float* t
   EntityArgs A{};
   const size_t row_len = dim * model_mul(model);
   if (int rc = fill_plan(&A, plan, workspace, workspace_bytes, row_len)) return rc;
-  if (plan->n_pairs != B * K) return fail(SMX_ERR_SHAPE, "plan holds %zu pairs, call has %zu", plan->n_pairs, B * K);
+  const size_t n_grad = multi ? multi->n_grad : 0;
+  if (plan->n_pairs != B * K + n_grad)
+    return fail(SMX_ERR_SHAPE, "plan holds %zu pairs, call has %zu", plan->n_pairs, B * K + n_grad);
+  if (n_grad) {
+    if (!multi->grad_rows) return fail(SMX_ERR_ARG, "null gradient rows");
+    A.grad_rows = multi->grad_rows;
+    A.rows_first = (int)(B * K);
+  }
   if (multi) {  // K is then the sum of the sources' K (checked by the caller): pairs of source s start at B * (K_0 + .. + K_s-1)
-    if (multi->n < 2 || multi->n > kMaxSources) return fail(SMX_ERR_ARG, "2 to %d pair sources", kMaxSources);
+    if (multi->n < 1 || multi->n > kMaxSources) return fail(SMX_ERR_ARG, "1 to %d pair sources", kMaxSources);
     A.n_src = multi->n;
     size_t first = 0;
     for (int i = 0; i < multi->n; ++i) {
@@ -179,7 +187,8 @@ int entity_backward(int model, void* stream, const smx_plan_view* plan, float* t
   }
   if (int rc = fill_adam(&A, m, v, adam)) return rc;
   const bool vec4 = dim % 4 == 0 && aligned16(table) && aligned16(q1) && (!q2 || aligned16(q2)) &&
-                    (!merged || aligned16(merged)) && (!m || aligned16(m)) && (!v || (adam && adam->squeeze) || aligned16(v));
+                    (!merged || aligned16(merged)) && (!m || aligned16(m)) && (!v || (adam && adam->squeeze) || aligned16(v)) &&
+                    (!n_grad || aligned16(multi->grad_rows));
   const int vec = vec4 ? 4 : 1;
   const size_t ncol = dim / vec;
   if (ncol > 512) return fail(SMX_ERR_SHAPE, "dim %zu not supported by the fused path", dim);
@@ -191,6 +200,11 @@ int entity_backward(int model, void* stream, const smx_plan_view* plan, float* t
   A.score = score;
   A.gscore = gscore;
   A.K = (int)K;
+  if (multi && multi->n == 1) {  // one index stream (+ gradient rows): the single-source fields describe it
+    A.n_src = 0;
+    A.score = multi->score[0];
+    A.gscore = multi->gscore[0];
+  }
   A.p = ScoreParams{params->gamma, params->cen, params->reg_on, params->reg_add, params->reg_lo, params->reg_hi};
   A.table = table;
   A.merged = merged;

@@ -69,6 +69,10 @@ struct EntityArgs : RowSink {
   const float* src_gscore[kMaxSources];
   const unsigned char* src_codes[kMaxSources];
   int src_K[kMaxSources];
+  // Plain lookups of the same step (anchor entities, box.py:137) whose gradient autograd has materialised:
+  // plan pairs from rows_first on are rows of grad_rows, [n_pairs - rows_first, row].  They sort behind the model
+  // pairs of their segment and are added when the segment's row is finished.  rows_first == n_pairs: none.
+  int rows_first;
 };
 
 template <int SRC>
@@ -203,7 +207,8 @@ __device__ __forceinline__ void apply_runs(const EntityArgs& A, const RunSet<R>&
   }
 }
 
-// One sorted position per lane: the window [base, base+64) of the per-position inputs.
+// One sorted position per lane: the window [base, base+64) of the per-position inputs.  A position that holds
+// a gradient row of a plain lookup comes back with my_pair = ~(its row number) < 0 and a zero coefficient.
 template <int SRC>
 __device__ __forceinline__ void load_window(const EntityArgs& A, int lane, int base, int& my_key, float& my_c,
                                             int& my_pair) {
@@ -212,7 +217,10 @@ __device__ __forceinline__ void load_window(const EntityArgs& A, int lane, int b
     my_key = my_pair = A.order[pos];
     my_c = 0.f;
   } else {
-    const int pair = my_pair = A.order[pos];
+    const int plan_pair = A.order[pos];
+    const bool is_row = plan_pair >= A.rows_first;
+    const int pair = is_row ? 0 : plan_pair;  // a pair whose inputs exist
+    my_pair = pair;
     float c1;
     if (A.n_src > 1) {  // uniform: which index stream the pair came from, and its number inside that stream
       int local = pair, K = A.src_K[0];
@@ -233,7 +241,56 @@ __device__ __forceinline__ void load_window(const EntityArgs& A, int lane, int b
       ModelOps<SRC>::coef(A.gscore[pair], A.score[pair], A.p, my_c, c1);
       my_key = pair / A.K;
     }
+    if (is_row) {
+      my_c = 0.f;
+      my_pair = ~(plan_pair - A.rows_first);
+    }
   }
+}
+
+// Lanes [j, j_end) of a window: how many of them hold gradient rows (they are the last ones of their segment).
+__device__ __forceinline__ int rows_in_window(int my_pair, int j, int j_end) {
+  const unsigned long long upto = j_end >= 64 ? ~0ull : ((1ull << j_end) - 1ull);
+  const unsigned long long from = j >= 64 ? 0ull : ~((1ull << j) - 1ull);
+  return __builtin_popcountll(__ballot(my_pair < 0) & upto & from);
+}
+
+// g += gradient row r of the plain lookups
+template <int MUL, int VEC, int NIT>
+__device__ __forceinline__ void add_grad_row(const EntityArgs& A, int lane, int r, float (&g1)[NIT][VEC],
+                                             float (&g2)[NIT][VEC]) {
+  const int half = A.ncol * VEC;
+  const float* pg = A.grad_rows + (size_t)r * half * MUL;
+#pragma unroll
+  for (int it = 0; it < NIT; ++it) {
+    const int c = min(lane + 64 * it, A.ncol - 1);
+    const Pack2<VEC> a = ld<VEC, true>(pg, c);
+#pragma unroll
+    for (int x = 0; x < VEC; ++x) g1[it][x] += a.v[x];
+    if constexpr (MUL == 2) {
+      const Pack2<VEC> b = ld<VEC, true>(pg + half, c);
+#pragma unroll
+      for (int x = 0; x < VEC; ++x) g2[it][x] += b.v[x];
+    }
+  }
+}
+
+// The gradient rows at the end of segment [s0, s1), found from the plan (for the kernels that no longer hold the
+// segment's window): added in ascending plan order.
+template <int MUL, int VEC, int NIT>
+__device__ __forceinline__ void add_segment_grad_rows(const EntityArgs& A, int lane, int s0, int s1,
+                                                      float (&g1)[NIT][VEC], float (&g2)[NIT][VEC]) {
+  int first = s1;
+  for (int hi = s1; hi > s0; hi -= 64) {
+    const int lo = max(s0, hi - 64);
+    const int pos = lo + lane;
+    const bool is_row = pos < hi && A.order[pos] >= A.rows_first;
+    const unsigned long long mk = __ballot(is_row);
+    if (mk == 0ull) break;
+    first = lo + __builtin_ctzll(mk);
+    if (__builtin_popcountll(mk) < hi - lo) break;
+  }
+  for (int pos = first; pos < s1; ++pos) add_grad_row<MUL, VEC, NIT>(A, lane, uniform(A.order[pos]) - A.rows_first, g1, g2);
 }
 
 template <int SRC, int VEC, int NIT>
@@ -280,6 +337,7 @@ __global__ __launch_bounds__(256) void entity_segment_kernel(EntityArgs A) {
   const int n_waves = gridDim.x * 4;
   const int n_chunks = (A.n_pairs + 63) / 64;
   const int n_valid = *A.n_uniq;  // a last segment beyond this one holds the pairs whose id is outside the table: skipped
+  const bool mixed = SRC != kSrcRows && A.rows_first < A.n_pairs;  // the plan also holds gradient rows of plain lookups
 
   for (int chunk = blockIdx.x * 4 + wave; chunk < n_chunks; chunk += n_waves) {
     const int base = chunk * 64;
@@ -289,9 +347,10 @@ __global__ __launch_bounds__(256) void entity_segment_kernel(EntityArgs A) {
     const int my_s0 = A.seg_start[my_seg];
     const int my_s1 = A.seg_start[my_seg + 1];
     const int my_len = my_s1 - my_s0;
+    bool done_elsewhere = A.skip_single && my_len == 1;  // by the pair-ordered kernel -- unless the one pair is a gradient row
+    if (SRC != kSrcRows && mixed && done_elsewhere) done_elsewhere = A.order[pos] < A.rows_first;
     unsigned long long todo =
-        __ballot(lane < n_here && my_s0 == pos && my_len <= A.short_max && !(A.skip_single && my_len == 1) &&
-                 my_seg < n_valid);
+        __ballot(lane < n_here && my_s0 == pos && my_len <= A.short_max && !done_elsewhere && my_seg < n_valid);
     if (todo == 0ull) continue;
     const int my_id = A.sorted_ids[pos];
 
@@ -315,7 +374,8 @@ __global__ __launch_bounds__(256) void entity_segment_kernel(EntityArgs A) {
       float g1[NIT][VEC], g2[NIT][VEC];
       zero_acc<VEC, NIT>(g1, g2);
       int j = s0 - win_base;
-      const int j_end = s1 - win_base;
+      const int j_all = s1 - win_base;
+      const int j_end = mixed ? j_all - rows_in_window(my_pair, j, j_all) : j_all;  // the model's pairs come first
       RunSet<R> rs;
       RunRows<SRC, VEC, NIT, R> rr;
       collect_runs<SRC, R, CODED>(rs, j, j_end, my_key, my_c, my_pair);
@@ -327,7 +387,13 @@ __global__ __launch_bounds__(256) void entity_segment_kernel(EntityArgs A) {
         request_runs<SRC, VEC, NIT, R, CODED>(A, lane, rs, rr);
         apply_runs<SRC, VEC, NIT, REG, R, CODED>(A, rs, rr, cur.e, g1, g2);
       }
-      finish_row<SRC, VEC, NIT, REG>(A, lane, row_id, seg, g1, g2, cur.e, cur.m, cur.v);
+      auto grad_rows_of_segment = [&](float (&a1)[NIT][VEC], float (&a2)[NIT][VEC]) {
+        if constexpr (SRC != kSrcRows) {
+          for (int jj = j_end; jj < j_all; ++jj)  // uniform bounds; empty unless the step has plain lookups
+            add_grad_row<MUL, VEC, NIT>(A, lane, ~__builtin_amdgcn_readlane(my_pair, jj), a1, a2);
+        }
+      };
+      finish_row<SRC, VEC, NIT, REG>(A, lane, row_id, seg, g1, g2, cur.e, cur.m, cur.v, grad_rows_of_segment);
     };
     auto pop = [&]() {  // lane of the next short segment start in the chunk, -1 when none is left
       if (todo == 0ull) return -1;
@@ -365,6 +431,7 @@ __global__ __launch_bounds__(256) void entity_tile_kernel(EntityArgs A) {
   if (p0 >= A.n_pairs) return;  // whole wavefront leaves; no workgroup barrier is used below
   const int p1 = min(A.n_pairs, p0 + A.tile);
   const int n_valid = *A.n_uniq;  // the segment of ids outside the table, if there is one, is number n_valid: skipped
+  const bool mixed = SRC != kSrcRows && A.rows_first < A.n_pairs;  // the plan also holds gradient rows of plain lookups
   {  // does a long segment that came in from the left end inside this tile?  The fix-up pass finishes it.
     const int sg = A.seg_of_pos[p0];
     const int b0 = A.seg_start[sg], b1 = A.seg_start[sg + 1];
@@ -401,7 +468,8 @@ __global__ __launch_bounds__(256) void entity_tile_kernel(EntityArgs A) {
         float my_c;
         load_window<SRC>(A, lane, base, my_key, my_c, my_pair);
         int j = 0;
-        const int j_end = min(64, end - base);
+        int j_end = min(64, end - base);
+        if (mixed) j_end -= rows_in_window(my_pair, 0, j_end);  // gradient rows wait for the row's finish
         while (j < j_end) {
           RunSet<R> rs;
           RunRows<SRC, VEC, NIT, R> rr;
@@ -410,9 +478,12 @@ __global__ __launch_bounds__(256) void entity_tile_kernel(EntityArgs A) {
           apply_runs<SRC, VEC, NIT, REG, R, CODED>(A, rs, rr, st.e, g1, g2);
         }
       }
-      if (whole)
-        finish_row<SRC, VEC, NIT, REG>(A, lane, row_id, seg, g1, g2, st.e, st.m, st.v);
-      else if (s1 > p1)
+      if (whole) {
+        auto grad_rows_of_segment = [&](float (&a1)[NIT][VEC], float (&a2)[NIT][VEC]) {
+          if (mixed) add_segment_grad_rows<MUL, VEC, NIT>(A, lane, s0, s1, a1, a2);
+        };
+        finish_row<SRC, VEC, NIT, REG>(A, lane, row_id, seg, g1, g2, st.e, st.m, st.v, grad_rows_of_segment);
+      } else if (s1 > p1)
         store_partial<SRC, VEC, NIT>(A, A.tail, t, lane, g1, g2);
       else
         store_partial<SRC, VEC, NIT>(A, A.head, t, lane, g1, g2);
@@ -510,7 +581,11 @@ __global__ __launch_bounds__(NW * 64) void entity_fixup_kernel(EntityArgs A) {
     if (A.adam_on == kOptAdam) load_row<MUL, VEC, NIT, true>(m0, A.m + (size_t)row_id * row_len, half, A.ncol, lane);
     if (A.adam_on && A.adam_on != kOptSgd && !A.squeeze)
       load_row<MUL, VEC, NIT, true>(v0, A.v + (size_t)row_id * row_len, half, A.ncol, lane);
-    finish_row<SRC, VEC, NIT, REG>(A, lane, row_id, seg, g1, g2, e, m0, v0);
+    auto grad_rows_of_segment = [&](float (&a1)[NIT][VEC], float (&a2)[NIT][VEC]) {
+      if (SRC != kSrcRows && A.rows_first < A.n_pairs)
+        add_segment_grad_rows<MUL, VEC, NIT>(A, lane, s0, A.seg_start[seg + 1], a1, a2);
+    };
+    finish_row<SRC, VEC, NIT, REG>(A, lane, row_id, seg, g1, g2, e, m0, v0, grad_rows_of_segment);
   }
 }
 

@@ -159,18 +159,23 @@ __device__ __forceinline__ void load_row(RowRegs<MUL, VEC, NIT>& r, const float*
     for (int it = 0; it < NIT; ++it) r.h[h][it] = ld<VEC, STREAM>(base + h * half, min(lane + 64 * it, ncol - 1));
 }
 
-// Coefficient on the second accumulator (BOX: inside distance) from the first.
+// finish_row's default for `extra`: nothing to add
+struct NoExtraRows {
+  template <class G> __device__ __forceinline__ void operator()(G&, G&) const {}
+};
+
 // Finishes one entity row: clamp mask, merged-gradient store, Adam.  g1/g2 are the lane's columns of
 // the summed gradient of the first / second half row; w, m0, v0 the row's current weights and moments
 // (w is always valid for the model sources -- it is the entity row the gradient was computed from).
 // ADAM_STATIC: the caller knows at compile time that Adam is on (its m0 / v0 are loaded); otherwise the
-// run-time flag A.adam_on decides.
-template <int SRC, int VEC, int NIT, bool REG, bool ADAM_STATIC = false>
+// run-time flag A.adam_on decides.  extra(g1, g2): adds what reaches the row from outside the score model
+// (gradient rows of the step's plain lookups) once the model's own gradient is complete, clamp mask included.
+template <int SRC, int VEC, int NIT, bool REG, bool ADAM_STATIC = false, class Extra = NoExtraRows>
 __device__ __forceinline__ void finish_row(const RowSink& A, int lane, unsigned row_id, int seg,
                                            float (&g1)[NIT][VEC], float (&g2)[NIT][VEC],
                                            const RowRegs<src_mul(SRC), VEC, NIT>& w,
                                            const RowRegs<src_mul(SRC), VEC, NIT>& m0,
-                                           const RowRegs<src_mul(SRC), VEC, NIT>& v0) {
+                                           const RowRegs<src_mul(SRC), VEC, NIT>& v0, Extra&& extra = Extra()) {
   constexpr int MUL = src_mul(SRC);
   const int half = A.ncol * VEC;
   const size_t row_len = (size_t)half * MUL;
@@ -193,6 +198,7 @@ __device__ __forceinline__ void finish_row(const RowSink& A, int lane, unsigned 
         if (MUL == 2) g2[it][x] = reg_mask(w.h[MUL - 1][it].v[x], g2[it][x], A.p);
       }
   }
+  extra(g1, g2);
   if (A.merged) {
     float* out = A.merged + (size_t)seg * row_len;
 #pragma unroll

@@ -261,11 +261,13 @@ int smx_score_backward_entity(int model, void* stream, const smx_plan_view* plan
 int smx_score_backward_entity_multi(int model, void* stream, const smx_plan_view* plan, float* table, size_t n_rows,
                                     const float* q1, const float* q2, const smx_pair_source* src, size_t n_src,
                                     size_t B, size_t dim, const smx_score_params* params, float* merged, float* m,
-                                    float* v, const smx_opt_params* adam, void* workspace, size_t workspace_bytes) {
+                                    float* v, const smx_opt_params* adam, void* workspace, size_t workspace_bytes,
+                                    const float* grad_rows, size_t n_grad_rows) {
   using namespace smx;
   if (!src || n_src == 0 || n_src > (size_t)kMaxSources)
     return fail(SMX_ERR_ARG, "1 to %d pair sources", kMaxSources);
-  if (n_src == 1)
+  if ((grad_rows != nullptr) != (n_grad_rows != 0)) return fail(SMX_ERR_ARG, "gradient rows and their count must come together");
+  if (n_src == 1 && !grad_rows)
     return smx_score_backward_entity(model, stream, plan, table, n_rows, q1, q2, src[0].score, src[0].gscore, B,
                                      src[0].K, dim, params, merged, m, v, adam, workspace, workspace_bytes,
                                      src[0].fwd_codes, src[0].fwd_codes_bytes);
@@ -294,15 +296,20 @@ int smx_score_backward_entity_multi(int model, void* stream, const smx_plan_view
     S.K[i] = src[i].K;
     k_sum += src[i].K;
   }
-  if (B == 0 || B * k_sum > 0x7fffffffull) return fail(SMX_ERR_SHAPE, "pair count out of range");
-  if (!plan || plan->n_pairs != B * k_sum)
-    return fail(SMX_ERR_SHAPE, "the plan must hold the %zu pairs of all sources", B * k_sum);
+  S.grad_rows = grad_rows;
+  S.n_grad = n_grad_rows;
+  const size_t n_all = B * k_sum + n_grad_rows;
+  if (B == 0 || n_all > 0x7fffffffull) return fail(SMX_ERR_SHAPE, "pair count out of range");
+  if (!plan || plan->n_pairs != n_all)
+    return fail(SMX_ERR_SHAPE, "the plan must hold the %zu pairs of all sources and the %zu gradient rows", B * k_sum,
+                n_grad_rows);
   // the same division of work as smx_score_backward_entity: ids that occur once in the whole step go through
   // the pair-ordered kernel, one launch per source, while the entity pass reduces the others beside it
   const bool split = coded && adam && !merged && plan->pair_seg && plan->uniq && plan->order && plan->sorted_ids &&
                      plan->seg_of_pos && plan->seg_start && plan->n_uniq && queries_beyond_l2(model, B, dim) &&
                      B * k_sum >= ((size_t)1 << 20) && workspace && !(reinterpret_cast<uintptr_t>(workspace) & 255u) &&
-                     workspace_bytes >= entity_ws_bytes(B * k_sum, dim * model_mul(model)) && !serial_backward();
+                     workspace_bytes >= entity_ws_bytes(n_all, dim * model_mul(model)) && !serial_backward() &&
+                     (!grad_rows || aligned16(grad_rows));
   if (split) {
     if (const char* msg = check_opt_params(adam, m, v)) return fail(SMX_ERR_ARG, "%s", msg);
     ScoreArgs A[kMaxSources];

@@ -153,8 +153,9 @@ class EmbeddingOptimizer(ABC):
         """Same for one fused record whose entity gradient is recomputed on the fly."""
 
     @abstractmethod
-    def update_fused_multi(self, plan, recs, lr):
-        """Same for several fused records of one query batch; plan covers their ids in the order of recs."""
+    def update_fused_multi(self, plan, recs, lr, grad_rows=None):
+        """Same for several fused records of one query batch; plan covers their ids in the order of recs, then
+        the ids of grad_rows (gradient rows of the step's plain lookups), when there are any."""
 
     # -- protocol of the training loop
     def zero_grad(self):
@@ -333,17 +334,23 @@ class EmbeddingOptimizer(ABC):
                 plan = fused.build_plan(rec["ids"], n_rows, err_flag=self.err_flag)
                 self.update_fused(plan, rec, lr)
                 return
-            if not self.grad_list and self._one_query_batch(self.fused_list):
-                # positives and negatives of one query batch (kg_reasoning.py:340-355): one plan over all their
-                # ids, one entity pass that reads each record's own scores / upstream gradients / sign codes
-                recs = sorted(self.fused_list, key=lambda r: r["fwd_idx"])   # forward order, whatever autograd's was
-                flat = torch.cat([r["ids"].reshape(-1) for r in recs], dim=0)
-                plan = fused.build_plan(flat, n_rows, err_flag=self.err_flag)
-                self.update_fused_multi(plan, recs, lr)
-                return
             idx_list = [i.reshape(-1).to(self.sparse_embed.device) for i, _ in self.grad_list]
             grad_list = [g.reshape(g.shape[0] if g.dim() == 2 else -1, g.shape[-1]).contiguous().float()
                          for _, g in self.grad_list]
+            if self.fused_list and (len(self.fused_list) == 1 or self._one_query_batch(self.fused_list)):
+                # positives and negatives of one query batch (kg_reasoning.py:340-355): one plan over all their
+                # ids, one entity pass that reads each record's own scores / upstream gradients / sign codes.
+                # The step's plain lookups -- the anchor entities every query starts from (box.py:137), whose
+                # gradient rows autograd has materialised -- go behind them in the same plan: such a row is
+                # added to its entity's gradient when the entity's row is finished.
+                recs = sorted(self.fused_list, key=lambda r: r["fwd_idx"])   # forward order, whatever autograd's was
+                flat = torch.cat([r["ids"].reshape(-1) for r in recs] + idx_list, dim=0)
+                rows = None
+                if grad_list:
+                    rows = grad_list[0] if len(grad_list) == 1 else torch.cat(grad_list, dim=0)
+                plan = fused.build_plan(flat, n_rows, err_flag=self.err_flag)
+                self.update_fused_multi(plan, recs, lr, grad_rows=rows)
+                return
             table = self.sparse_embed.embedding.detach()
             for rec in self.fused_list:  # reduce each fused record to (distinct ids, summed rows) first
                 plan = fused.build_plan(rec["ids"], n_rows, err_flag=self.err_flag)
@@ -418,12 +425,12 @@ class _RowOptimizer(EmbeddingOptimizer):
         fused.rows_backward(plan, grad_rows, table=self.sparse_embed.embedding.detach(), m=m, v=v,
                             adam=self._params(lr))
 
-    def update_fused_multi(self, plan, recs, lr):
+    def update_fused_multi(self, plan, recs, lr, grad_rows=None):
         m, v = self._state()
         first = recs[0]
         fused.score_backward_entity_multi(first["model"], plan, self.sparse_embed.embedding.detach(), first["q1"],
                                           first["q2"], [(r["score"], r["gscore"], r["codes"]) for r in recs],
-                                          first["params"], m=m, v=v, adam=self._params(lr))
+                                          first["params"], m=m, v=v, adam=self._params(lr), grad_rows=grad_rows)
 
     def update_fused(self, plan, rec, lr):
         m, v = self._state()

@@ -238,10 +238,12 @@ def score_backward_entity(model, plan, table, q1, q2, score, gscore, params, mer
                   _ptr(codes), 0 if codes is None else codes.numel())
 
 
-def score_backward_entity_multi(model, plan, table, q1, q2, sources, params, merged=None, m=None, v=None, adam=None):
+def score_backward_entity_multi(model, plan, table, q1, q2, sources, params, merged=None, m=None, v=None, adam=None,
+                                grad_rows=None):
     """score_backward_entity for several index streams of one query batch (see smx_score_backward_entity_multi).
     sources: list of (score [B,K_s], gscore [B,K_s], codes or None); plan: built over the concatenation of the
-    streams' flattened ids in the same order."""
+    streams' flattened ids in the same order.  grad_rows [n, row]: materialised gradient rows of the step's plain
+    lookups, whose ids are the last n entries of that concatenation."""
     b, dim = q1.shape[0], q1.shape[-1]
     if model not in MODELS:
         raise _lib.SmxError(f"unknown score model {model}")
@@ -261,13 +263,19 @@ def score_backward_entity_multi(model, plan, table, q1, q2, sources, params, mer
     _check_state(table, m, v, adam)
     if merged is not None and (merged.dim() != 2 or merged.shape[1] != row_len):
         raise _lib.SmxError("merged must be [n_uniq or more, row]")
+    n_grad = 0
+    if grad_rows is not None:
+        _f32(grad_rows, "grad_rows")
+        if grad_rows.dim() != 2 or grad_rows.shape[1] != row_len or grad_rows.shape[0] == 0:
+            raise _lib.SmxError("grad_rows must be [n >= 1, row]")
+        n_grad = grad_rows.shape[0]
     with torch.cuda.device(table.device):
         ws = _workspace(_lib.load().smx_entity_workspace_bytes(plan.n_pairs, row_len), table.device)
         view = plan.view()
         _lib.call("smx_score_backward_entity_multi", MODELS[model], _stream(table), ctypes.byref(view), _ptr(table),
                   table.shape[0], _ptr(q1), _ptr(q2), ctypes.cast(arr, ctypes.c_void_p), len(sources), b, dim,
                   ctypes.byref(params), _ptr(merged), _ptr(m), _ptr(v), None if adam is None else ctypes.byref(adam),
-                  _ptr(ws), ws.numel())
+                  _ptr(ws), ws.numel(), _ptr(grad_rows), n_grad)
 
 
 def score_backward_fused(model, plan, table, idx, q1, q2, score, gscore, params, merged=None, m=None, v=None,

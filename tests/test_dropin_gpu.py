@@ -332,3 +332,96 @@ def test_inverse_query_call_sequence_runs_on_the_reverse_layout():
     w, m, v, uniq, merged = oracle_adam_step(table, [tail, neg], [g_e.reshape(b, d), g_q.reshape(b * k, d)], lr, 1)
     assert_close(emb.state_sum_fo.cpu().numpy()[uniq], m[uniq], REL_F32, "inverse query: first moment")
     assert_adam_weights(emb.embedding.detach().cpu().numpy(), w, merged, uniq, lr, "inverse query: weights")
+
+
+@pytest.mark.parametrize("name", list(CASES))
+def test_anchor_lookups_join_the_fused_records_in_one_update(name, monkeypatch):
+    """Every query of the reference starts from the embedding of its anchor entities: a plain lookup in
+    embed_query (box.py:137 and siblings) whose rows feed the query side, so that autograd hands the optimizer
+    gradient ROWS for them (embed_optimizer.py:63-66) next to the fused record of positives + negatives.  A
+    restated 1p query: queries = f(anchor rows, relation tensors).  The step must stay on the fused entity pass
+    (no gradient rows materialised for the scored pairs, one plan, one update per entity -- also for entities
+    that are anchor and negative at once); logits, relation gradients and Adam state against the oracle."""
+    from smore_amd import fused
+    from smore_amd.embedding.embed_optimizer import AdamEmbedOptimizer
+    from smore_amd.embedding.sparse_embed import SparseEmbedding
+
+    def no_gradient_rows(*a, **k):
+        raise AssertionError("the scored pairs must not go through materialised gradient rows")
+    monkeypatch.setattr(fused, "rows_backward", no_gradient_rows)
+    cls, extra, model, n_q, mul, gamma, cen = CASES[name]
+    n, d, b, k, lr = 300, 32, 6, 24, 1e-3
+    rng = np.random.default_rng(23)
+    f32 = lambda a: np.asarray(a).astype(np.float32).astype(np.float64)
+    table, _ = _table_and_queries(name, n, d, b, 1, rng)
+    if name == "beta":
+        rel = [f32(rng.uniform(0.5, 1.5, (b, d))) for _ in range(2)]           # positive scales keep alpha, beta > 0
+    else:
+        rel = [f32(rng.uniform(-0.07, 0.07, (b, d))) for _ in range(n_q)]
+        if name == "box":
+            rel[1] = np.abs(rel[1])
+    emb = SparseEmbedding(n, mul * d).cuda()
+    with torch.no_grad():
+        emb.embedding.copy_(torch.tensor(table, dtype=torch.float32))
+    opt = AdamEmbedOptimizer(types.SimpleNamespace(optim_mode="(aggr,adam,gpu,False,5)", share_optim_stats=True), emb, 0)
+    net = cls(emb, gamma, *extra).cuda()
+    t_rel = [torch.tensor(r, dtype=torch.float32, device="cuda", requires_grad=True) for r in rel]
+
+    def embed_query(rows, rels, lib):
+        """rows [B, mul*d] -> the model's query tensors [B, d] each (lib = torch or numpy)."""
+        if name == "beta":
+            rows = lib.clip(rows + 1.0, 0.05, 1e9) if lib is np else torch.clamp(rows + 1.0, 0.05, 1e9)
+            return [rows[:, :d] * rels[0], rows[:, d:] * rels[1]]
+        if mul == 2:
+            return [rows[:, :d] + rels[0], rows[:, d:] + rels[1]]
+        return [rows + rels[0]] + list(rels[1:])
+
+    w, m, v = table.copy(), np.zeros_like(table), np.zeros_like(table)
+    for step in (1, 2):
+        pos = rng.integers(0, n, b)
+        neg = rng.integers(0, n // 4, (b, k))
+        anchor = rng.integers(0, n // 4, b)                                    # some anchors are negatives too
+        anchor[0], anchor[1] = neg[0, 0], anchor[0]
+        gp, gn = f32(rng.standard_normal((b, 1))), f32(rng.standard_normal((b, k)))
+        opt.zero_grad()
+        for t in t_rel:
+            t.grad = None
+        a_rows = emb(torch.tensor(anchor, device="cuda"), "anchor")
+        a_rows.job_handle.sync()
+        t_qs = [q.view(b, 1, 1, d) for q in embed_query(a_rows, t_rel, torch)]
+        lp, ln = net(torch.tensor(pos, device="cuda"), torch.tensor(neg, device="cuda"), t_qs)
+        ((lp * torch.tensor(gp, dtype=torch.float32, device="cuda")).sum() +
+         (ln * torch.tensor(gn, dtype=torch.float32, device="cuda")).sum()).backward()
+        assert len(opt.fused_list) == 1 and len(opt.grad_list) == 1
+        opt.apply_grad(lr)
+
+        qs = [q.reshape(b, 1, 1, d) for q in embed_query(orc.gather(w, anchor), rel, np)]
+        o_lp, rows_p = _oracle_branch_logits(name, w, pos.reshape(b, 1), qs, gamma, cen)
+        o_ln, rows_n = _oracle_branch_logits(name, w, neg, qs, gamma, cen)
+        assert_close(lp.detach().cpu().numpy(), o_lp[:, 0], REL_F32, f"{name} positive logits, step {step}")
+        assert_close(ln.detach().cpu().numpy(), o_ln[:, 0], REL_F32, f"{name} negative logits, step {step}")
+        gr_p, gq_p = _oracle_grads(name, w, pos.reshape(b, 1), qs, rows_p, o_lp, gp, cen)
+        gr_n, gq_n = _oracle_grads(name, w, neg, qs, rows_n, o_ln, gn, cen)
+        gq = [(a + c).reshape(b, d) for a, c in zip(gq_p, gq_n)]              # d loss / d query tensors
+        raw = orc.gather(w, anchor)
+        if name == "beta":
+            reg = np.clip(raw + 1.0, 0.05, 1e9)
+            mask = (raw + 1 >= 0.05) & (raw + 1 <= 1e9)
+            g_anchor = np.concatenate([gq[0] * rel[0], gq[1] * rel[1]], axis=1) * mask
+            g_rel = [gq[0] * reg[:, :d], gq[1] * reg[:, d:]]
+        elif mul == 2:
+            g_anchor, g_rel = np.concatenate(gq, axis=1), gq
+        else:
+            g_anchor, g_rel = gq[0], gq
+        for t, want in zip(t_rel, g_rel):
+            assert_close(t.grad.cpu().numpy(), want, REL_F32, f"{name} relation gradient, step {step}")
+        w_before = w.copy()
+        w, m, v, uniq, merged = oracle_adam_step(w, [pos, neg, anchor], [gr_p, gr_n, g_anchor], lr, step, m, v)
+        got = emb.embedding.detach().cpu().numpy().astype(np.float64)
+        touched = np.zeros(n, bool)
+        touched[uniq] = True
+        assert np.array_equal(got[~touched], w_before[~touched]), "rows outside the step must keep their bits"
+        assert_close(emb.state_sum_fo.cpu().numpy()[touched], m[touched], REL_F32, f"{name} first moment, step {step}")
+        assert_close(emb.state_sum_sq.cpu().numpy()[touched], v[touched], REL_F32, f"{name} second moment, step {step}")
+        assert_adam_weights(got, w, merged, uniq, lr, f"{name} weights, step {step}")
+        w = got.copy()   # continue from the device's fp32 weights so that step 2 compares one step, not two

@@ -974,3 +974,95 @@ def test_forward_scores_each_distinct_entity_of_a_wavefront_once(model, dim):
         assert_close(got[True][1].cpu().numpy(), got[False][1].cpu().numpy(), 1e-6, "gq1 from the forward's codes")
     else:
         assert codes is None
+
+
+@pytest.mark.parametrize("model,ks", [("box", (12,)), ("box", (1, 20)), ("l1", (1, 7)), ("l2", (5,)), ("rotate", (1, 9)),
+                                      ("beta_kl", (1, 6)), ("complex", (4,)), ("distmult", (1, 3))])
+def test_entity_pass_with_gradient_rows_of_plain_lookups(model, ks):
+    """The step's plain lookups (anchor entities, models/box.py:137) hand the optimizer materialised gradient rows
+    (embed_optimizer.py:63-66); they go behind the fused streams in one plan, and an entity named by both gets one
+    update from the sum (embed_optimizer.py:155-163).  Rows for ids the streams also hold, for ids only the lookup
+    holds, an id looked up 3 times, and one looked up 150 times (a segment longer than a tile, finished by the
+    fix-up kernel).  Merged rows and the Adam step against the oracle's merge of the concatenation."""
+    from smore_amd import fused
+    n, b, dim, lr = 700, 9, 24, 1e-3
+    rng = np.random.default_rng(seed("plain lookups", model, ks))
+    table, q1, q2, _, _ = make_problem(model, n, b, 1, dim, rng)
+    gamma, cen = GAMMA[model], 0.02
+    params = fused.score_params(gamma, cen)
+    t_table, t_q1, t_q2 = dev(table), dev(q1), dev(q2)
+    o_q1 = q1[:, None, :]
+    o_q2 = None if q2 is None else q2[:, None, :]
+    ids, sources, o_rows = [], [], []
+    for k in ks:
+        idx = rng.integers(0, n // 2, (b, k))             # the upper half of the table is the lookup's alone
+        idx[0, 0] = 5
+        gs = rng.standard_normal((b, k)).astype(np.float32).astype(np.float64)
+        t_idx = torch.tensor(idx, device="cuda")
+        codes = fused.new_codes(model, t_table, t_idx, t_q1)
+        score = fused.score_forward(model, t_table, t_idx, t_q1, t_q2, params, codes=codes)
+        sources.append((score, dev(gs), codes))
+        ids.append(idx.reshape(-1))
+        rows = orc.gather(table, idx).reshape(b, k, -1)
+        g_rows, _, _ = orc.score_backward(model, gs, rows, o_q1, o_q2, cen)
+        o_rows.append(g_rows.reshape(b * k, -1))
+    in_streams = np.unique(np.concatenate(ids))
+    looked_up = np.concatenate([in_streams[:6], [5, 5, 5], rng.integers(n // 2, n, 10), np.full(150, 17),
+                                np.full(150, n - 1)])
+    rng.shuffle(looked_up)
+    extra = rng.standard_normal((looked_up.size, table.shape[1])).astype(np.float32).astype(np.float64)
+    flat = np.concatenate(ids + [looked_up])
+    plan = fused.build_plan(torch.tensor(flat, device="cuda"), n, want_inverse=True)
+    uniq, inverse, _, _ = orc.merge_indices(flat)
+    all_rows = np.concatenate(o_rows + [extra])
+    o_merged = orc.merge_grads(all_rows, inverse, uniq.size)
+    o_abs = orc.merge_grads(np.abs(all_rows), inverse, uniq.size)
+    merged = torch.full((uniq.size, table.shape[1]), float("nan"), device="cuda")
+    fused.score_backward_entity_multi(model, plan, t_table, t_q1, t_q2, sources, params, merged=merged,
+                                      grad_rows=dev(extra))
+    assert_close(merged.cpu().numpy(), o_merged, REL_F32, f"{model} merged, streams + lookup rows", sum_abs=o_abs)
+    t_m, t_v = torch.zeros_like(t_table), torch.zeros_like(t_table)
+    w_s, m_s, v_s = table.copy(), np.zeros_like(table), np.zeros_like(table)
+    orc.adam_rows(w_s, m_s, v_s, uniq, merged.cpu().numpy().astype(np.float64), lr, 1)
+    fused.score_backward_entity_multi(model, plan, t_table, t_q1, t_q2, sources, params, m=t_m, v=t_v,
+                                      adam=fused.adam_params(lr, 1), grad_rows=dev(extra))
+    touched = np.zeros(n, bool)
+    touched[uniq] = True
+    assert touched[n - 1] and touched[17]
+    assert_close(t_table.cpu().numpy()[touched], w_s[touched], REL_F32, f"{model} w, streams + lookup rows")
+    assert_close(t_m.cpu().numpy()[touched], m_s[touched], REL_F32, f"{model} m, streams + lookup rows")
+    assert_close(t_v.cpu().numpy()[touched], v_s[touched], REL_F32, f"{model} v, streams + lookup rows", rms_floor=False)
+    assert np.array_equal(t_table.cpu().numpy()[~touched], table[~touched].astype(np.float32))
+
+
+def test_gradient_rows_pass_the_clamp_mask_of_the_entity_prologue():
+    """BetaE's prologue clamp(x + 1, 0.05, 1e9) masks the MODEL's gradient where the clamp is active
+    (models/beta.py regularizer); the rows of a plain lookup are gradients with respect to the stored values
+    already and are added after the mask."""
+    from smore_amd import fused
+    rng = np.random.default_rng(78)
+    n, b, k, dim = 300, 6, 20, 24
+    raw = (rng.standard_normal((n, 2 * dim)) * 1.5).astype(np.float32).astype(np.float64)
+    f = lambda *s: np.clip(1 + rng.standard_normal(s), 0.05, 1e9).astype(np.float32).astype(np.float64)
+    qa, qb = f(b, dim), f(b, dim)
+    idx = rng.integers(0, n, (b, k))
+    gs = rng.standard_normal((b, k)).astype(np.float32).astype(np.float64)
+    params = fused.score_params(60.0, 0.0, regularizer=(1.0, 0.05, 1e9))
+    t_raw, t_qa, t_qb = dev(raw), dev(qa), dev(qb)
+    t_idx = torch.tensor(idx, device="cuda")
+    score = fused.score_forward("beta_kl", t_raw, t_idx, t_qa, t_qb, params)
+    rows = orc.gather(orc.regularizer(raw), idx).reshape(b, k, -1)
+    g_rows, _, _ = orc.score_backward("beta_kl", gs, rows, qa[:, None], qb[:, None])
+    looked_up = np.concatenate([idx[0, :5], idx[1, :3], [idx[0, 0]] * 2])
+    extra = rng.standard_normal((looked_up.size, 2 * dim)).astype(np.float32).astype(np.float64)
+    flat = np.concatenate([idx.reshape(-1), looked_up])
+    plan = fused.build_plan(torch.tensor(flat, device="cuda"), n, want_inverse=True)
+    uniq, inverse, _, _ = orc.merge_indices(flat)
+    mask = ((raw + 1 >= 0.05) & (raw + 1 <= 1e9))
+    assert not mask[looked_up].all(), "the looked-up rows must hit the clamp somewhere"
+    model_rows = g_rows.reshape(b * k, -1) * mask[idx.reshape(-1)]
+    o_merged = orc.merge_grads(np.concatenate([model_rows, extra]), inverse, uniq.size)
+    merged = torch.empty((uniq.size, 2 * dim), device="cuda")
+    fused.score_backward_entity_multi("beta_kl", plan, t_raw, t_qa, t_qb, [(score, dev(gs), None)], params,
+                                      merged=merged, grad_rows=dev(extra))
+    assert_close(merged.cpu().numpy(), o_merged, REL_F32, "masked model gradient + unmasked lookup rows")
