@@ -255,22 +255,36 @@ __device__ __forceinline__ int rows_in_window(int my_pair, int j, int j_end) {
   return __builtin_popcountll(__ballot(my_pair < 0) & upto & from);
 }
 
-// g += gradient row r of the plain lookups
-template <int MUL, int VEC, int NIT>
-__device__ __forceinline__ void add_grad_row(const EntityArgs& A, int lane, int r, float (&g1)[NIT][VEC],
-                                             float (&g2)[NIT][VEC]) {
+// g += the gradient rows of the plain lookups whose numbers lanes [j0, j1) of `row_of_lane` hold, in lane order;
+// kAhead rows are requested before the first is added.
+template <int MUL, int VEC, int NIT, int kAhead = 4>
+__device__ __forceinline__ void add_grad_rows(const EntityArgs& A, int lane, int row_of_lane, int j0, int j1,
+                                              float (&g1)[NIT][VEC], float (&g2)[NIT][VEC]) {
   const int half = A.ncol * VEC;
-  const float* pg = A.grad_rows + (size_t)r * half * MUL;
+  for (int j = j0; j < j1; j += kAhead) {  // uniform bounds
+    Pack2<VEC> a[kAhead][NIT], b[kAhead][NIT];
 #pragma unroll
-  for (int it = 0; it < NIT; ++it) {
-    const int c = min(lane + 64 * it, A.ncol - 1);
-    const Pack2<VEC> a = ld<VEC, true>(pg, c);
+    for (int u = 0; u < kAhead; ++u) {
+      const int r = __builtin_amdgcn_readlane(row_of_lane, min(j + u, j1 - 1));
+      const float* pg = A.grad_rows + (size_t)r * half * MUL;
 #pragma unroll
-    for (int x = 0; x < VEC; ++x) g1[it][x] += a.v[x];
-    if constexpr (MUL == 2) {
-      const Pack2<VEC> b = ld<VEC, true>(pg + half, c);
+      for (int it = 0; it < NIT; ++it) {
+        const int c = min(lane + 64 * it, A.ncol - 1);
+        a[u][it] = ld<VEC, true>(pg, c);
+        if constexpr (MUL == 2) b[u][it] = ld<VEC, true>(pg + half, c);
+      }
+    }
 #pragma unroll
-      for (int x = 0; x < VEC; ++x) g2[it][x] += b.v[x];
+    for (int u = 0; u < kAhead; ++u) {
+      if (j + u < j1) {
+#pragma unroll
+        for (int it = 0; it < NIT; ++it)
+#pragma unroll
+          for (int x = 0; x < VEC; ++x) {
+            g1[it][x] += a[u][it].v[x];
+            if constexpr (MUL == 2) g2[it][x] += b[u][it].v[x];
+          }
+      }
     }
   }
 }
@@ -290,7 +304,12 @@ __device__ __forceinline__ void add_segment_grad_rows(const EntityArgs& A, int l
     first = lo + __builtin_ctzll(mk);
     if (__builtin_popcountll(mk) < hi - lo) break;
   }
-  for (int pos = first; pos < s1; ++pos) add_grad_row<MUL, VEC, NIT>(A, lane, uniform(A.order[pos]) - A.rows_first, g1, g2);
+  for (int base = first; base < s1; base += 64) {
+    const int n_here = min(64, s1 - base);
+    const int row_of_lane = A.order[base + min(lane, n_here - 1)] - A.rows_first;
+    // (a popular entity is the anchor of hundreds of queries of a batch: more rows in flight for these)
+    add_grad_rows<MUL, VEC, NIT, (MUL * NIT <= 2 ? 8 : 4)>(A, lane, row_of_lane, 0, n_here, g1, g2);
+  }
 }
 
 template <int SRC, int VEC, int NIT>
@@ -389,8 +408,7 @@ __global__ __launch_bounds__(256) void entity_segment_kernel(EntityArgs A) {
       }
       auto grad_rows_of_segment = [&](float (&a1)[NIT][VEC], float (&a2)[NIT][VEC]) {
         if constexpr (SRC != kSrcRows) {
-          for (int jj = j_end; jj < j_all; ++jj)  // uniform bounds; empty unless the step has plain lookups
-            add_grad_row<MUL, VEC, NIT>(A, lane, ~__builtin_amdgcn_readlane(my_pair, jj), a1, a2);
+          if (j_end < j_all) add_grad_rows<MUL, VEC, NIT>(A, lane, ~my_pair, j_end, j_all, a1, a2);  // plain lookups only
         }
       };
       finish_row<SRC, VEC, NIT, REG>(A, lane, row_id, seg, g1, g2, cur.e, cur.m, cur.v, grad_rows_of_segment);

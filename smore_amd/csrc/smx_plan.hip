@@ -14,7 +14,7 @@
 // also the tie-break, so inside a segment pairs stay in ascending pair order and every later
 // reduction over a segment has one fixed summation order.
 //
-// A radix pass handles a tile of up to 16384 elements per workgroup of 1024 threads: elements are
+// A radix pass handles a tile of up to 18432 elements per workgroup of 1024 threads: elements are
 // kept in registers, ranked per wavefront with ballot matching (stable: lane order inside a round,
 // rounds in order, wavefronts in order), the tile's digit counts are published and the counts of
 // the tiles before it are read back ("look-back"; tiles take their number from a ticket counter,
@@ -32,7 +32,7 @@
 
 namespace smx {
 
-constexpr int kSortMaxRounds = 16;          // elements per thread and tile
+constexpr int kSortMaxRounds = 18;          // elements per thread and tile
 constexpr int kSortMaxDigitBits = 10;
 constexpr int kGroup = 16;                  // look-back fan-in: tiles per group, groups per super-block, ...
 constexpr unsigned kReady = 0x80000000u;    // published words: flag | 31-bit count
@@ -650,8 +650,12 @@ static void launch_pass_r(hipStream_t st, const PlanLayout& L, const SortPassArg
 }
 template <int NW>
 static void launch_pass_nw(hipStream_t st, const PlanLayout& L, const SortPassArgs& A, bool first, bool last) {
+  // (a step of B x (1 + K) pairs -- positives beside the negatives -- lies just beyond 256 tiles of 16 elements
+  // per thread and still fits one tile per CU with 17: the third form saves such steps a second round of
+  // workgroups, 51 -> 37 us per pass at 4.2 M pairs, at the price of a few spilled registers)
   if (L.rounds <= 8) launch_pass_r<NW, 8>(st, L, A, first, last);
-  else launch_pass_r<NW, 16>(st, L, A, first, last);
+  else if (L.rounds <= 16) launch_pass_r<NW, 16>(st, L, A, first, last);
+  else launch_pass_r<NW, kSortMaxRounds>(st, L, A, first, last);
 }
 
 }  // namespace smx

@@ -181,3 +181,29 @@ def test_full_size_workload(cfg_id):
             assert_close(table[eid].cpu().numpy(), wn[0], REL_F32, f"step 2 weights of entity {eid}")
             assert_close(v[eid].cpu().numpy(), vn[0], REL_F32, f"step 2 second moment of entity {eid}",
                          sum_abs=np.full_like(w1, 1e-12), rms_floor=False)
+
+
+@pytest.mark.parametrize("n_pairs", [4096 * 1025, 4096 * 1025 + 4096, 18 * 1024 * 256 + 5, 6_000_000])
+def test_plan_at_pair_counts_beyond_256_tiles_of_16_rounds(n_pairs):
+    """A step that scores positives beside the negatives holds B x (1 + K) pairs (kg_reasoning.py:340-355), with
+    anchors B more: just past the 4,194,304 the radix passes cover with 16 elements per thread and one tile per CU.
+    They then take 17 or 18 per thread; beyond that, more tiles.  Integer invariants against torch, bit-exact."""
+    from smore_amd import fused
+    n = 86_054_151
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(n_pairs % 1000)
+    ids = bench.zipf_ids(n, (n_pairs,), 1.1, gen, torch.device("cuda"))
+    plan = fused.build_plan(ids, n, want_inverse=True)
+    uniq_t, inverse_t = torch.unique(ids, return_inverse=True)
+    assert plan.n_uniq == uniq_t.numel() and torch.equal(plan.uniq, uniq_t)
+    assert torch.equal(plan.inverse, inverse_t)
+    assert torch.equal(ids[plan.order.long()], plan.sorted_ids.long())
+    assert bool((plan.sorted_ids[1:] >= plan.sorted_ids[:-1]).all())
+    order = plan.order.long()
+    same_seg = plan.sorted_ids[1:] == plan.sorted_ids[:-1]
+    assert bool((order[1:][same_seg] > order[:-1][same_seg]).all()), "pairs inside a segment must stay in pair order"
+    counts = torch.bincount(inverse_t, minlength=uniq_t.numel())
+    seg = plan.seg_start[: plan.n_uniq + 1].long()
+    assert torch.equal(seg[1:] - seg[:-1], counts)
+    alone = plan.pair_seg < 0
+    assert int(alone.sum().item()) == int((counts == 1).sum().item())
