@@ -301,6 +301,86 @@ def cpu_baseline(cfg, seed):
     }
 
 
+def cpu_baseline_torch(cfg, seed):
+    """The reference's CPU-capable arithmetic restated with torch on the host cores: the `--logit_impl native`
+    expressions (models/vec.py, box.py, rotate.py, beta.py native_cal_logit), autograd's backward, then the sparse
+    optimizer's data flow with torch index operations (embed_optimizer.py:39-48 unique + scatter-sum, :208-252
+    lazy Adam).  Bounded sample: fewer queries and rows than the workload, same K, row length and id distribution."""
+    import torch
+    cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+    torch.set_num_threads(cores)
+    gen = torch.Generator().manual_seed(seed)
+    n, b = min(cfg["n"], 2_000_000), min(cfg["b"], 128)
+    k, dim, rl, model = cfg["k"], cfg["dim"], row_len(cfg), cfg["model"]
+    if model == "beta_kl":
+        beta = lambda *s: torch.clamp(1 + torch.nn.functional.elu(torch.randn(s, generator=gen)), 0.05, 1e9)
+        table, q1, q2 = beta(n, rl), beta(b, 1, dim), beta(b, 1, dim)
+    else:
+        r = cfg["r"]
+        table = torch.empty((n, rl)).uniform_(-r, r, generator=gen)
+        q1 = torch.empty((b, 1, dim)).uniform_(-r, r, generator=gen)
+        q2 = torch.empty((b, 1, dim)).uniform_(-r, r, generator=gen).abs_() if n_query_tensors(cfg) == 2 else None
+    if cfg["zipf"] is None:
+        idx = torch.randint(0, n, (b, k), generator=gen)
+    else:
+        w = torch.arange(1, n + 1, dtype=torch.float64).pow_(-cfg["zipf"])
+        cdf = torch.cumsum(w, 0)
+        cdf /= cdf[-1].clone()
+        idx = torch.searchsorted(cdf, torch.rand((b, k), dtype=torch.float64, generator=gen)).clamp_(max=n - 1)
+    gs = torch.randn((b, k), generator=gen)
+    m, v = (torch.zeros_like(table), torch.zeros_like(table)) if cfg["adam"] else (None, None)
+    q1.requires_grad_(True)
+    if q2 is not None:
+        q2.requires_grad_(True)
+    gamma, cen, lr = cfg["gamma"], cfg["cen"], cfg.get("lr", 0.0)
+
+    def step(t):
+        rows = table[idx.view(-1)].view(b, k, rl).requires_grad_(True)
+        if model == "l1":
+            logit = gamma - torch.norm(rows - q1, p=1, dim=-1)
+        elif model == "l2":
+            logit = gamma - torch.norm(rows - q1, p=2, dim=-1)
+        elif model == "box":
+            delta = (rows - q1).abs()
+            logit = gamma - torch.norm(torch.relu(delta - q2), p=1, dim=-1) - \
+                cen * torch.norm(torch.min(delta, q2), p=1, dim=-1)
+        elif model == "rotate":
+            re, im = torch.chunk(rows, 2, dim=-1)
+            logit = gamma - torch.sqrt((re - q1) ** 2 + (im - q2) ** 2).sum(dim=-1)
+        else:
+            ea, eb = torch.chunk(rows, 2, dim=-1)
+            kld = torch.distributions.kl._kl_beta_beta(torch.distributions.Beta(ea, eb), torch.distributions.Beta(q1, q2))
+            logit = gamma - torch.norm(kld, p=1, dim=-1)
+        logit.backward(gs)
+        uniq, inverse = torch.unique(idx.view(-1), return_inverse=True)
+        merged = torch.zeros((uniq.numel(), rl)).index_add_(0, inverse, rows.grad.view(-1, rl))
+        if cfg["adam"]:
+            m_rows = m[uniq].mul_(0.9).add_(merged, alpha=0.1)
+            v_rows = v[uniq].mul_(0.999).addcmul_(merged, merged, value=0.001)
+            bc1, bc2 = 1 - 0.9 ** t, 1 - 0.999 ** t
+            upd = m_rows / (v_rows.sqrt() / bc2 ** 0.5 + 1e-8)
+            table.index_add_(0, uniq, upd, alpha=-lr / bc1)
+            m.index_copy_(0, uniq, m_rows)
+            v.index_copy_(0, uniq, v_rows)
+        q1.grad = None
+        if q2 is not None:
+            q2.grad = None
+
+    step(1)
+    times = []
+    for t in range(2, 5):
+        t0 = time.perf_counter()
+        step(t)
+        times.append(time.perf_counter() - t0)
+    best = sorted(times)[len(times) // 2]
+    return {
+        "value": b * k / best, "unit": "pairs/s", "cores": cores, "kind": "port",
+        "sample": f"torch {torch.__version__.split('+')[0]} on the host, native logit expressions + autograd + unique / "
+                  f"index_add_ / lazy Adam with index operations, same model/K/D/id distribution, B={b}, N={n}, "
+                  f"median of {len(times)} steps of {best * 1e3:.0f} ms",
+    }
+
+
 def measure_ceilings(device, row_bytes, full=False):
     """What plain kernels sustain on this GPU (GB/s of bytes moved, reads + writes), from the library's
     probe kernels on two 4 GiB scratch buffers: streaming read, copy, and rows of the workload's length
@@ -586,6 +666,7 @@ def main():
     del out["config"]["model"]
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(cfg, seed)
+        out["cpu_baseline_torch"] = cpu_baseline_torch(cfg, seed)
     print(json.dumps(out))
 
 
