@@ -425,3 +425,50 @@ def test_anchor_lookups_join_the_fused_records_in_one_update(name, monkeypatch):
         assert_close(emb.state_sum_sq.cpu().numpy()[touched], v[touched], REL_F32, f"{name} second moment, step {step}")
         assert_adam_weights(got, w, merged, uniq, lr, f"{name} weights, step {step}")
         w = got.copy()   # continue from the device's fp32 weights so that step 2 compares one step, not two
+
+
+def test_shared_negatives_beside_positives_share_one_record():
+    """--share_negative (online_sampler.py:155-157): negatives [1,K] for the whole batch, positives [B] per query,
+    both scored by unchanged model code against one branch of queries.  They wait for the loss together and
+    leave ONE record [B, 1 + K]; the is_negative_mat mask of train_process.py:195-196 multiplies the negative
+    logits.  Logits, query gradient and the Adam step against the oracle."""
+    from smore_amd.embedding.embed_optimizer import AdamEmbedOptimizer
+    from smore_amd.embedding.sparse_embed import SparseEmbedding
+    n, d, b, k, lr = 300, 16, 5, 12, 1e-3
+    rng = np.random.default_rng(9)
+    f32 = lambda a: np.asarray(a).astype(np.float32).astype(np.float64)
+    table = f32(rng.uniform(-0.07, 0.07, (n, d)))
+    q = f32(rng.uniform(-0.07, 0.07, (b, 1, 1, d)))
+    pos, neg = rng.integers(0, n, b), rng.integers(0, n, (1, k))
+    pos[0] = neg[0, 0]                                                       # a positive that is also a shared negative
+    mask = (rng.random((b, k)) < 0.8).astype(np.float64)
+    gp, gn = f32(rng.standard_normal((b, 1))), f32(rng.standard_normal((b, k)))
+    emb = SparseEmbedding(n, d).cuda()
+    with torch.no_grad():
+        emb.embedding.copy_(torch.tensor(table, dtype=torch.float32))
+    opt = AdamEmbedOptimizer(types.SimpleNamespace(optim_mode="(aggr,adam,gpu,False,5)", share_optim_stats=True), emb, 0)
+    net = Vec(emb, 12.0, "l1").cuda()
+    tq = torch.tensor(q, dtype=torch.float32, device="cuda", requires_grad=True)
+    dev = lambda a: torch.tensor(a, dtype=torch.float32, device="cuda")
+    opt.zero_grad()
+    p_rows = emb(torch.tensor(pos, device="cuda"), "positive_entity")
+    n_rows = emb(torch.tensor(neg, device="cuda").view(-1), "negative_entity")
+    p_rows.job_handle.sync()
+    lp = net.cal_logit(p_rows.unsqueeze(1), None, [tq])
+    n_rows.job_handle.sync()
+    ln = net.cal_logit(n_rows.view(1, k, -1), None, [tq])
+    ln = ln * dev(mask)
+    ((lp * dev(gp)).sum() + (ln * dev(gn)).sum()).backward()
+    assert len(opt.fused_list) == 1 and not opt.grad_list
+    opt.apply_grad(lr)
+
+    ids = np.concatenate([pos.reshape(b, 1), np.broadcast_to(neg, (b, k))], axis=1)
+    rows = orc.gather(table, ids).reshape(b, 1 + k, d)
+    want = orc.score_forward("l1", rows, q[:, 0], None, 12.0)
+    assert_close(lp.detach().cpu().numpy(), want[:, :1], REL_F32, "positive logits")
+    assert_close(ln.detach().cpu().numpy(), want[:, 1:] * mask, REL_F32, "masked shared-negative logits")
+    g_rows, g_q, _ = orc.score_backward("l1", np.concatenate([gp, gn * mask], axis=1), rows, q[:, 0], None)
+    assert_close(tq.grad.cpu().numpy()[:, 0], g_q, REL_F32, "query gradient")
+    w, m, v, uniq, merged = oracle_adam_step(table, [ids], [g_rows.reshape(b * (1 + k), d)], lr, 1)
+    assert_close(emb.state_sum_fo.cpu().numpy()[uniq], m[uniq], REL_F32, "first moment")
+    assert_adam_weights(emb.embedding.detach().cpu().numpy(), w, merged, uniq, lr, "weights")

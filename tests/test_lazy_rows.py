@@ -203,3 +203,26 @@ def test_positives_and_negatives_of_one_query_batch_share_one_launch():
     assert opt.scored[-1] == ("box", (b, 1), 24.0, 0.02, None) and len(opt.pending_scores) == 1
     values, indices = torch.max(24.0 - ext_ops.l1_dist(LazyRows(opt, pos, None).unsqueeze(1), c), dim=1)
     assert indices.shape == (b, 1) and int(indices.sum()) == 0
+
+
+def test_shared_negatives_wait_beside_per_query_positives():
+    """--share_negative gives negative ids [1,K] (online_sampler.py:155-157) next to positives [B]: in one request
+    the shared ids stand beside the per-query ones as [B, 1 + K]; alone they stay [1, K]."""
+    n, d, b, k = 50, 8, 5, 7
+    opt = RecordingOptimizer(n, d)
+    gen = torch.Generator().manual_seed(4)
+    pos, neg = torch.randint(0, n, (b,), generator=gen), torch.randint(0, n, (1, k), generator=gen)
+    (q,) = _queries(b, 1, d, 1, 21)
+    cal_logit = lambda rows: torch.max(12.0 - ext_ops.l1_dist(rows, q), dim=1)[0]
+    lp = cal_logit(LazyRows(opt, pos, "positive_entity").unsqueeze(1))
+    ln = cal_logit(LazyRows(opt, neg.view(-1), "negative_entity").view(1, k, -1))
+    assert lp.shape == (b, 1) and ln.shape == (b, k)
+    total = lp.sum() + ln.sum()
+    assert opt.scored == [("l1", (b, 1 + k), 12.0, 0.0, None)]
+    table = opt.sparse_embed.embedding
+    want = (12.0 - _textbook("l1", table[pos].unsqueeze(1), (q,), 0.0)).sum() + \
+        (12.0 - _textbook("l1", table[neg].expand(b, k, d), (q,), 0.0)).sum()
+    assert torch.allclose(total, want, atol=1e-4)
+    alone = cal_logit(LazyRows(opt, neg.view(-1), "negative_entity").view(1, k, -1))
+    float(alone.sum())
+    assert opt.scored[-1] == ("l1", (1, k), 12.0, 0.0, None)
