@@ -246,10 +246,16 @@ class EmbeddingOptimizer(ABC):
         if len(group) > 1:      # ids shared by the batch ([1, K]) stand beside per-query ones as [B, K]
             ids = [i.expand(w["b"], i.shape[1]) if i.shape[0] == 1 else i for i in ids]
         all_ids = ids[0] if len(ids) == 1 else torch.cat(ids, dim=1)
-        logit = self._score_branches(w["model"], all_ids, w["q1"], w["q2"], w["gamma"], w["cen"], w["reg"])[:, 0]
-        parts = [logit] if len(ids) == 1 else torch.split(logit, [i.shape[1] for i in ids], dim=1)
-        for p, part in zip(group, parts):
-            p._value = part
+        logit = self._score_branches(w["model"], all_ids, w["q1"], w["q2"], w["gamma"], w["cen"], w["reg"])
+        if logit.shape[1] == 1:
+            values, index = logit[:, 0], None
+        else:                   # union branches: the first maximal one, as torch.max(logit, dim=1) in the model code
+            values, index = torch.max(logit, dim=1)
+        sizes = [i.shape[1] for i in ids]
+        parts = [values] if len(ids) == 1 else torch.split(values, sizes, dim=1)
+        iparts = [index] * len(ids) if (index is None or len(ids) == 1) else torch.split(index, sizes, dim=1)
+        for p, part, ipart in zip(group, parts, iparts):
+            p._value, p._index = part, ipart
         self.pending_scores = [p for p in self.pending_scores if p._value is None]
 
     def score_negatives(self, model, ids, q1, q2=None, gamma=0.0, cen=0.0, regularizer=None):

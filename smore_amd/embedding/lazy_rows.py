@@ -356,16 +356,16 @@ class LazyLogit(_Delegating):
         if name in ("neg", "negative", "__neg__") and len(args) == 1 and not kwargs:
             return -args[0]
         if name == "max" and args and isinstance(args[0], LazyLogit):
-            # torch.max(logit, dim=1) of custom_cal_logit: with ONE union branch the maximum is that branch, and
-            # the logits can wait until something needs their values -- by then the step's other lookups against
-            # the same queries (positives, negatives) have been scored too and all go into one launch
+            # torch.max(logit, dim=1) of custom_cal_logit, the maximum over the union branches: the logits can wait
+            # until something needs their values -- by then the step's other lookups against the same queries
+            # (positives, negatives) have asked too, and all of them go into one launch
             dim = kwargs.get("dim", args[1] if len(args) > 1 else None)
             self = args[0]
             if (dim == 1 and len(args) <= 2 and set(kwargs) <= {"dim"} and self._value is None and
-                    len(self.shape) == 3 and self.shape[1] == 1 and self._fusable() is not None):
+                    len(self.shape) == 3 and self._fusable() is not None):
                 scores = LazyScores(self)
                 if scores.request is not None:
-                    return _MaxResult(scores, _LazyZeros(scores.shape, scores.device))
+                    return _MaxResult(scores, _LazyIndices(scores))
         return NotImplemented
 
     # -- evaluation
@@ -414,25 +414,34 @@ class _MaxResult(tuple):
     indices = property(lambda self: self[1])
 
 
-class _LazyZeros(_Delegating):
-    """Indices of a maximum over a dimension of size one: zeros, made only if somebody looks."""
+class _LazyIndices(_Delegating):
+    """Which branch held the maximum: known once the scores are, made only if somebody looks."""
 
-    def __init__(self, shape, device):
-        self.shape, self.device, self.dtype = torch.Size(shape), device, torch.int64
+    def __init__(self, scores):
+        self.scores = scores
+        self.dtype = torch.int64
+
+    shape = property(lambda self: self.scores.shape)
+    device = property(lambda self: self.scores.device)
 
     def materialize(self):
-        return torch.zeros(self.shape, dtype=torch.int64, device=self.device)
+        self.scores.materialize()
+        if self.scores._index is None:      # one branch
+            self.scores._index = torch.zeros(self.shape, dtype=torch.int64, device=self.device)
+        return self.scores._index
 
 
 class LazyScores(_Delegating):
-    """Logits [B, K] of one lookup against one branch of queries, not yet computed.  The optimizer keeps the
-    step's pending ones; the first that is needed evaluates all that share its model, margin, parameters and
-    query tensors in one launch of the fused scorer (ids side by side, [B, K_1 + K_2 + ..]), so that the step
-    leaves one record with the optimizer, as if the caller had concatenated positives and negatives itself."""
+    """Logits [B, K] of one lookup against the queries (the maximum over their union branches), not yet computed.
+    The optimizer keeps the step's pending ones; the first that is needed evaluates all that share its model,
+    margin, parameters and query tensors in one launch of the fused scorer (ids side by side,
+    [B, K_1 + K_2 + ..]), so that the step leaves one record with the optimizer, as if the caller had concatenated
+    positives and negatives itself."""
 
     def __init__(self, logit):
         self.logit = logit
         self._value = None
+        self._index = None      # branch of the maximum, [B, K]; None while there is one branch only
         d = logit.terms[0][1]
         self.opt = d.rows.opt
         model, cen = logit._fusable()

@@ -173,9 +173,8 @@ def test_model_code_without_score_negatives_matches_oracle(name, branches, monke
         assert lp.shape == (b, 1) and ln.shape == (b, k)
         ((lp * torch.tensor(gp, dtype=torch.float32, device="cuda")).sum() +
          (ln * torch.tensor(gn, dtype=torch.float32, device="cuda")).sum()).backward()
-        # one branch: both lookups wait for their first use and share one launch; a union scores each at its max
-        assert len(opt.fused_list) == (1 if branches == 1 else 2) and not opt.grad_list, \
-            "both lookups must have stayed on the fused scorer"
+        # both lookups wait for their first use (the maximum over union branches included) and share one launch
+        assert len(opt.fused_list) == 1 and not opt.grad_list, "both lookups must have stayed on the fused scorer"
         opt.apply_grad(lr)
 
         o_lp, rows_p = _oracle_branch_logits(name, w, pos.reshape(b, 1), qs, gamma, cen)

@@ -78,11 +78,13 @@ def test_box_logit_of_the_model_code_is_one_fused_request():
     d2 = ext_ops.box_dist_in(rows, c, o)
     logit = gamma - d1 - 0.02 * d2
     assert isinstance(logit, LazyLogit) and logit.shape == (b, u, k) and not opt.scored
-    out = torch.max(logit, dim=1)[0]
-    assert opt.scored == [("box", (b, k), 24.0, 0.02, None)] and not opt.looked_up
+    out, which = torch.max(logit, dim=1)
+    assert out.shape == (b, k) and not opt.scored, "the maximum over the branches waits for its first use"
     e = opt.sparse_embed.embedding[ids]
-    want = torch.max(24.0 - _textbook("box", e, (c, o), 0.02), dim=1)[0]
+    want, want_which = torch.max(24.0 - _textbook("box", e, (c, o), 0.02), dim=1)
     assert torch.allclose(out, want, rtol=0, atol=1e-5)
+    assert opt.scored == [("box", (b, k), 24.0, 0.02, None)] and not opt.looked_up
+    assert torch.equal(which.materialize(), want_which)
 
 
 @pytest.mark.parametrize("op,model,n_q", [("l1_dist", "l1", 1), ("l2_dist", "l2", 1), ("rotate_dist", "rotate", 2)])
