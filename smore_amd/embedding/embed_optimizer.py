@@ -255,7 +255,9 @@ class EmbeddingOptimizer(ABC):
         parts = [values] if len(ids) == 1 else torch.split(values, sizes, dim=1)
         iparts = [index] * len(ids) if (index is None or len(ids) == 1) else torch.split(index, sizes, dim=1)
         for p, part, ipart in zip(group, parts, iparts):
-            p._value, p._index = part, ipart
+            # (each caller gets a tensor of its own layout, as torch.max would have returned it: .view() works)
+            p._value = part.contiguous()
+            p._index = None if ipart is None else ipart.contiguous()
         self.pending_scores = [p for p in self.pending_scores if p._value is None]
 
     def score_negatives(self, model, ids, q1, q2=None, gamma=0.0, cen=0.0, regularizer=None):

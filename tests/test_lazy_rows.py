@@ -228,3 +228,38 @@ def test_shared_negatives_wait_beside_per_query_positives():
     alone = cal_logit(LazyRows(opt, neg.view(-1), "negative_entity").view(1, k, -1))
     float(alone.sum())
     assert opt.scored[-1] == ("l1", (1, k), 12.0, 0.0, None)
+
+
+def test_pending_scores_behave_as_the_tensor_they_stand_for():
+    """What training and evaluation code does with the logits (train_process.py:112-128, 194-213): arithmetic from
+    both sides, comparison, indexing, iteration, cat / stack / argsort / softmax, views and reductions."""
+    n, d, b, k = 60, 8, 4, 6
+    opt = RecordingOptimizer(n, d)
+    gen = torch.Generator().manual_seed(2)
+    pos, neg = torch.randint(0, n, (b,), generator=gen), torch.randint(0, n, (b, k), generator=gen)
+    c, o = _queries(b, 1, d, 2, 12)
+    cal = lambda rows: torch.max(24.0 - ext_ops.box_dist_out(rows, c, o) - 0.02 * ext_ops.box_dist_in(rows, c, o), dim=1)[0]
+    fresh = lambda: (cal(LazyRows(opt, pos, None).unsqueeze(1)), cal(LazyRows(opt, neg.view(-1), None).view(b, k, -1)))
+    table = opt.sparse_embed.embedding
+    want_p = (24.0 - _textbook("box", table[pos].unsqueeze(1), (c, o), 0.02))[:, 0]
+    want_n = (24.0 - _textbook("box", table[neg], (c, o), 0.02))[:, 0]
+    uses = [
+        lambda lp, ln: (torch.cat([lp, ln], dim=1), torch.cat([want_p, want_n], dim=1)),
+        lambda lp, ln: (torch.stack([ln, ln]), torch.stack([want_n, want_n])),
+        lambda lp, ln: (torch.nn.functional.logsigmoid(lp).squeeze(dim=1), torch.nn.functional.logsigmoid(want_p).squeeze(dim=1)),
+        lambda lp, ln: ((ln > 20).sum(), (want_n > 20).sum()),
+        lambda lp, ln: (torch.argsort(ln, dim=1, descending=True), torch.argsort(want_n, dim=1, descending=True)),
+        lambda lp, ln: (ln[1], want_n[1]),
+        lambda lp, ln: (torch.stack(list(ln)), want_n),
+        lambda lp, ln: (torch.softmax(ln * 0.5, dim=1).detach() * torch.nn.functional.logsigmoid(-ln),
+                        torch.softmax(want_n * 0.5, dim=1) * torch.nn.functional.logsigmoid(-want_n)),
+        lambda lp, ln: (torch.ones(b, k) * ln + (1.0 - ln) / 2, want_n + (1.0 - want_n) / 2),
+        lambda lp, ln: (ln.view(-1), want_n.reshape(-1)),
+        lambda lp, ln: (ln.t().sum(dim=0) + lp.mean(), want_n.sum(dim=1) + want_p.mean()),
+    ]
+    for use in uses:
+        got, want = use(*fresh())
+        assert got.shape == want.shape and torch.allclose(got.float(), want.float(), atol=1e-4)
+    lp, ln = fresh()
+    assert len(ln) == b and ln.size(1) == k and ln.dim() == 2 and ln.numel() == b * k and ln.dtype == torch.float32
+    assert abs(float(lp.sum()) - float(want_p.sum())) < 1e-3
