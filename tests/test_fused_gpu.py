@@ -976,17 +976,20 @@ def test_forward_scores_each_distinct_entity_of_a_wavefront_once(model, dim):
         assert codes is None
 
 
-@pytest.mark.parametrize("model,ks", [("box", (12,)), ("box", (1, 20)), ("l1", (1, 7)), ("l2", (5,)), ("rotate", (1, 9)),
-                                      ("beta_kl", (1, 6)), ("complex", (4,)), ("distmult", (1, 3))])
-def test_entity_pass_with_gradient_rows_of_plain_lookups(model, ks):
+@pytest.mark.parametrize("model,ks,dim", [("box", (12,), 24), ("box", (1, 20), 24), ("l1", (1, 7), 24), ("l2", (5,), 24),
+                                          ("rotate", (1, 9), 24), ("beta_kl", (1, 6), 24), ("complex", (4,), 24),
+                                          ("distmult", (1, 3), 24),
+                                          # single-float columns, and rows of several column groups per lane
+                                          ("l1", (1, 7), 30), ("box", (3,), 520), ("rotate", (2,), 130), ("box", (1, 4), 200)])
+def test_entity_pass_with_gradient_rows_of_plain_lookups(model, ks, dim):
     """The step's plain lookups (anchor entities, models/box.py:137) hand the optimizer materialised gradient rows
     (embed_optimizer.py:63-66); they go behind the fused streams in one plan, and an entity named by both gets one
     update from the sum (embed_optimizer.py:155-163).  Rows for ids the streams also hold, for ids only the lookup
     holds, an id looked up 3 times, and one looked up 150 times (a segment longer than a tile, finished by the
     fix-up kernel).  Merged rows and the Adam step against the oracle's merge of the concatenation."""
     from smore_amd import fused
-    n, b, dim, lr = 700, 9, 24, 1e-3
-    rng = np.random.default_rng(seed("plain lookups", model, ks))
+    n, b, lr = 700, 9, 1e-3
+    rng = np.random.default_rng(seed("plain lookups", model, ks, dim))
     table, q1, q2, _, _ = make_problem(model, n, b, 1, dim, rng)
     gamma, cen = GAMMA[model], 0.02
     params = fused.score_params(gamma, cen)
@@ -1066,3 +1069,43 @@ def test_gradient_rows_pass_the_clamp_mask_of_the_entity_prologue():
     fused.score_backward_entity_multi("beta_kl", plan, t_raw, t_qa, t_qb, [(score, dev(gs), None)], params,
                                       merged=merged, grad_rows=dev(extra))
     assert_close(merged.cpu().numpy(), o_merged, REL_F32, "masked model gradient + unmasked lookup rows")
+
+
+@pytest.mark.parametrize("kind,squeeze", [("adam", True), ("sgd", False), ("adagrad", False), ("adagrad", True),
+                                          ("rmsprop", False)])
+def test_gradient_rows_reach_every_row_optimizer(kind, squeeze):
+    """The rows of plain lookups are part of the gradient every optimizer of embed_optimizer.py sees (SGD :166-178,
+    RMSprop :255-309, AdaGrad :312-349, Adam with the squeezed second moment :226-229): the update from the fused
+    pass must equal the update from the materialised route (merged rows of the same call -> smx_rows_backward)."""
+    from smore_amd import fused
+    n, b, k, dim, lr = 400, 8, 16, 64, 1e-2
+    rng = np.random.default_rng(seed("rows and optimizers", kind, squeeze))
+    table, q1, q2, idx, gs = make_problem("box", n, b, k, dim, rng)
+    params = fused.score_params(24.0, 0.02)
+    t_q1, t_q2 = dev(q1), dev(q2)
+    looked_up = np.concatenate([idx[0, :4], rng.integers(0, n, 12), np.full(70, int(idx[1, 0]))])
+    extra = dev(rng.standard_normal((looked_up.size, dim)))
+    flat = torch.tensor(np.concatenate([idx.reshape(-1), looked_up]), device="cuda")
+    plan = fused.build_plan(flat, n)
+    uniq_plan = fused.build_plan(plan.uniq, n)                      # the merged rows as one gradient row per entity
+    out = {}
+    for route in ("fused", "rows"):
+        w = dev(table)
+        m = torch.zeros_like(w) if kind == "adam" else None
+        v = None if kind == "sgd" else (torch.full((n,), 0.01, device="cuda") if squeeze else torch.full_like(w, 0.01))
+        t_idx = torch.tensor(idx, device="cuda")
+        codes = fused.new_codes("box", w, t_idx, t_q1)
+        score = fused.score_forward("box", w, t_idx, t_q1, t_q2, params, codes=codes)
+        opt = fused.opt_params(kind, lr, step=3, squeeze=squeeze)
+        if route == "fused":
+            fused.score_backward_entity_multi("box", plan, w, t_q1, t_q2, [(score, dev(gs), codes)], params, m=m, v=v,
+                                              adam=opt, grad_rows=extra)
+        else:
+            merged = torch.empty((plan.n_uniq, dim), device="cuda")
+            fused.score_backward_entity_multi("box", plan, w, t_q1, t_q2, [(score, dev(gs), codes)], params,
+                                              merged=merged, grad_rows=extra)
+            fused.rows_backward(uniq_plan, merged, table=w, m=m, v=v, adam=opt)
+        out[route] = (w, m, v)
+    for name, a, c in zip("wmv", out["fused"], out["rows"]):
+        if a is not None:
+            assert torch.equal(a, c), f"{kind}: {name} differs between the fused pass and the materialised route"
