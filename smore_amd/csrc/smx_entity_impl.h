@@ -73,6 +73,7 @@ struct EntityArgs : RowSink {
   // plan pairs from rows_first on are rows of grad_rows, [n_pairs - rows_first, row].  They sort behind the model
   // pairs of their segment and are added when the segment's row is finished.  rows_first == n_pairs: none.
   int rows_first;
+  int share_rows;  // fix-up kernel: its LDS has room for one more row per wavefront, they share a segment's gradient rows
 };
 
 template <int SRC>
@@ -289,11 +290,9 @@ __device__ __forceinline__ void add_grad_rows(const EntityArgs& A, int lane, int
   }
 }
 
-// The gradient rows at the end of segment [s0, s1), found from the plan (for the kernels that no longer hold the
-// segment's window): added in ascending plan order.
-template <int MUL, int VEC, int NIT>
-__device__ __forceinline__ void add_segment_grad_rows(const EntityArgs& A, int lane, int s0, int s1,
-                                                      float (&g1)[NIT][VEC], float (&g2)[NIT][VEC]) {
+// First plan position of the gradient rows at the end of segment [s0, s1) (s1 when it has none), found from the
+// plan by the kernels that no longer hold the segment's window.
+__device__ __forceinline__ int first_grad_row_of_segment(const EntityArgs& A, int lane, int s0, int s1) {
   int first = s1;
   for (int hi = s1; hi > s0; hi -= 64) {
     const int lo = max(s0, hi - 64);
@@ -304,10 +303,18 @@ __device__ __forceinline__ void add_segment_grad_rows(const EntityArgs& A, int l
     first = lo + __builtin_ctzll(mk);
     if (__builtin_popcountll(mk) < hi - lo) break;
   }
-  for (int base = first; base < s1; base += 64) {
+  return first;
+}
+
+// g += the gradient rows at plan positions [first, s1), 64 at a time; of those stretches this caller takes
+// number `part`, `part + parts`, ..  (a popular entity is the anchor of hundreds of queries of a batch: the
+// wavefronts of a workgroup share them, and each keeps several rows in flight).  Ascending plan order per caller.
+template <int MUL, int VEC, int NIT>
+__device__ __forceinline__ void add_segment_grad_rows(const EntityArgs& A, int lane, int first, int s1, int part,
+                                                      int parts, float (&g1)[NIT][VEC], float (&g2)[NIT][VEC]) {
+  for (int base = first + part * 64; base < s1; base += parts * 64) {
     const int n_here = min(64, s1 - base);
     const int row_of_lane = A.order[base + min(lane, n_here - 1)] - A.rows_first;
-    // (a popular entity is the anchor of hundreds of queries of a batch: more rows in flight for these)
     add_grad_rows<MUL, VEC, NIT, (MUL * NIT <= 2 ? 8 : 4)>(A, lane, row_of_lane, 0, n_here, g1, g2);
   }
 }
@@ -498,7 +505,8 @@ __global__ __launch_bounds__(256) void entity_tile_kernel(EntityArgs A) {
       }
       if (whole) {
         auto grad_rows_of_segment = [&](float (&a1)[NIT][VEC], float (&a2)[NIT][VEC]) {
-          if (mixed) add_segment_grad_rows<MUL, VEC, NIT>(A, lane, s0, s1, a1, a2);
+          if (mixed)
+            add_segment_grad_rows<MUL, VEC, NIT>(A, lane, first_grad_row_of_segment(A, lane, s0, s1), s1, 0, 1, a1, a2);
         };
         finish_row<SRC, VEC, NIT, REG>(A, lane, row_id, seg, g1, g2, st.e, st.m, st.v, grad_rows_of_segment);
       } else if (s1 > p1)
@@ -577,8 +585,23 @@ __global__ __launch_bounds__(NW * 64) void entity_fixup_kernel(EntityArgs A) {
       g1[it][x] = s1;
       g2[it][x] = MUL == 2 ? s2 : 0.f;
     }
+  // The segment's gradient rows of plain lookups are not part of the model's accumulators (they join after the
+  // model hook and the clamp mask): with room in the LDS every wavefront sums a share of them, else the first does
+  // all of them.  A.share_rows is uniform.
+  const bool mixed = SRC != kSrcRows && A.rows_first < A.n_pairs;
+  float h1[NIT][VEC], h2[NIT][VEC];
+  zero_acc<VEC, NIT>(h1, h2);
+  if (mixed && (A.share_rows || wave == 0)) {
+    const int seg_end = A.seg_start[seg + 1];
+    const int first = first_grad_row_of_segment(A, lane, s0, seg_end);
+    add_segment_grad_rows<MUL, VEC, NIT>(A, lane, first, seg_end, A.share_rows ? wave : 0, A.share_rows ? NW : 1, h1, h2);
+  }
+  float* lds_rows = lds + (size_t)(NW - 1) * row_len;   // [NW - 1] rows, only there with A.share_rows
   // combine the wavefront sums in wavefront order
-  if (wave > 0) store_partial<SRC, VEC, NIT>(A, lds, wave - 1, lane, g1, g2);
+  if (wave > 0) {
+    store_partial<SRC, VEC, NIT>(A, lds, wave - 1, lane, g1, g2);
+    if (mixed && A.share_rows) store_partial<SRC, VEC, NIT>(A, lds_rows, wave - 1, lane, h1, h2);
+  }
   __syncthreads();
   if (wave == 0) {
     for (int w = 1; w < NW; ++w) {
@@ -592,6 +615,19 @@ __global__ __launch_bounds__(NW * 64) void entity_fixup_kernel(EntityArgs A) {
           if (MUL == 2) g2[it][x] += o.h[MUL - 1][it].v[x];
         }
     }
+    if (mixed && A.share_rows) {
+      for (int w = 1; w < NW; ++w) {
+        RowRegs<MUL, VEC, NIT> o;
+        load_row<MUL, VEC, NIT>(o, lds_rows + (size_t)(w - 1) * row_len, half, A.ncol, lane);
+#pragma unroll
+        for (int it = 0; it < NIT; ++it)
+#pragma unroll
+          for (int x = 0; x < VEC; ++x) {
+            h1[it][x] += o.h[0][it].v[x];
+            if (MUL == 2) h2[it][x] += o.h[MUL - 1][it].v[x];
+          }
+      }
+    }
     const unsigned row_id = (unsigned)A.sorted_ids[p0];
     RowRegs<MUL, VEC, NIT> e, m0, v0;
     if (REG || A.adam_on || SRC == mBetaKL)
@@ -600,8 +636,15 @@ __global__ __launch_bounds__(NW * 64) void entity_fixup_kernel(EntityArgs A) {
     if (A.adam_on && A.adam_on != kOptSgd && !A.squeeze)
       load_row<MUL, VEC, NIT, true>(v0, A.v + (size_t)row_id * row_len, half, A.ncol, lane);
     auto grad_rows_of_segment = [&](float (&a1)[NIT][VEC], float (&a2)[NIT][VEC]) {
-      if (SRC != kSrcRows && A.rows_first < A.n_pairs)
-        add_segment_grad_rows<MUL, VEC, NIT>(A, lane, s0, A.seg_start[seg + 1], a1, a2);
+      if (mixed) {
+#pragma unroll
+        for (int it = 0; it < NIT; ++it)
+#pragma unroll
+          for (int x = 0; x < VEC; ++x) {
+            a1[it][x] += h1[it][x];
+            if (MUL == 2) a2[it][x] += h2[it][x];
+          }
+      }
     };
     finish_row<SRC, VEC, NIT, REG>(A, lane, row_id, seg, g1, g2, e, m0, v0, grad_rows_of_segment);
   }
@@ -645,10 +688,17 @@ int launch_entity_reg(hipStream_t st, const EntityArgs& A) {
     hipLaunchKernelGGL((entity_tile_kernel<SRC, VEC, NIT, REG>), dim3((tiles + 3) / 4), dim3(256), 0, st, A);
   }
   const size_t row_bytes = (size_t)A.ncol * VEC * src_mul(SRC) * sizeof(float);
-  if (7 * row_bytes <= 60 * 1024)
-    hipLaunchKernelGGL((entity_fixup_kernel<SRC, VEC, NIT, 8, REG>), dim3(tiles), dim3(8 * 64), 7 * row_bytes, st, A);
-  else
-    hipLaunchKernelGGL((entity_fixup_kernel<SRC, VEC, NIT, 4, REG>), dim3(tiles), dim3(4 * 64), 3 * row_bytes, st, A);
+  const bool mixed = SRC != kSrcRows && A.rows_first < A.n_pairs;
+  EntityArgs F = A;
+  if (7 * row_bytes <= 60 * 1024) {
+    F.share_rows = mixed && 14 * row_bytes <= 60 * 1024;
+    hipLaunchKernelGGL((entity_fixup_kernel<SRC, VEC, NIT, 8, REG>), dim3(tiles), dim3(8 * 64),
+                       (F.share_rows ? 14 : 7) * row_bytes, st, F);
+  } else {
+    F.share_rows = mixed && 6 * row_bytes <= 60 * 1024;
+    hipLaunchKernelGGL((entity_fixup_kernel<SRC, VEC, NIT, 4, REG>), dim3(tiles), dim3(4 * 64),
+                       (F.share_rows ? 6 : 3) * row_bytes, st, F);
+  }
   return check_launch("entity backward");
 }
 

@@ -980,7 +980,9 @@ def test_forward_scores_each_distinct_entity_of_a_wavefront_once(model, dim):
                                           ("rotate", (1, 9), 24), ("beta_kl", (1, 6), 24), ("complex", (4,), 24),
                                           ("distmult", (1, 3), 24),
                                           # single-float columns, and rows of several column groups per lane
-                                          ("l1", (1, 7), 30), ("box", (3,), 520), ("rotate", (2,), 130), ("box", (1, 4), 200)])
+                                          ("l1", (1, 7), 30), ("box", (3,), 520), ("rotate", (2,), 130), ("box", (1, 4), 200),
+                                          # rows too long for the fix-up kernel's wavefronts to share the lookup rows
+                                          ("rotate", (2,), 600)])
 def test_entity_pass_with_gradient_rows_of_plain_lookups(model, ks, dim):
     """The step's plain lookups (anchor entities, models/box.py:137) hand the optimizer materialised gradient rows
     (embed_optimizer.py:63-66); they go behind the fused streams in one plan, and an entity named by both gets one
