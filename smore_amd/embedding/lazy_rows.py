@@ -21,7 +21,6 @@ import weakref
 
 import torch
 
-from .. import _lib
 
 _FUSED_MODEL = {"l1": "l1", "l2": "l2", "rotate": "rotate", "beta_kl": "beta_kl"}   # logit = const - dist
 _FUSED_SIMILARITY = ("complex", "distmult")                                          # logit = const + similarity
