@@ -97,7 +97,7 @@ class EmbeddingOptimizer(ABC):
         sp_embed.fwd_delegate = self.forward
         self.dummy_tensor = nn.Parameter(torch.randn(1, 1))
         self.grad_list, self.fused_list, self.has_grad_list = [], [], []
-        self.pending_scores = []    # LazyScores of this step that nothing has needed yet
+        self.pending_scores = []    # weak references to the LazyScores of this step that nothing has needed yet
         self.n_fwd = 0
         self.step = 0
         self.gpu_id = gpu_id
@@ -237,7 +237,8 @@ class EmbeddingOptimizer(ABC):
             return a is b or (a.data_ptr() == b.data_ptr() and a.shape == b.shape and a.stride() == b.stride() and
                               a._version == b._version and a.requires_grad == b.requires_grad)
 
-        group = [p for p in self.pending_scores if p._value is None and p.request["model"] == w["model"] and
+        alive = [p for p in (r() for r in self.pending_scores) if p is not None and p._value is None]
+        group = [p for p in alive if p.request["model"] == w["model"] and
                  p.request["gamma"] == w["gamma"] and p.request["cen"] == w["cen"] and p.request["reg"] == w["reg"] and
                  same(p.request["q1"], w["q1"]) and same(p.request["q2"], w["q2"])]
         if not any(p is wanted for p in group):
@@ -258,7 +259,7 @@ class EmbeddingOptimizer(ABC):
             # (each caller gets a tensor of its own layout, as torch.max would have returned it: .view() works)
             p._value = part.contiguous()
             p._index = None if ipart is None else ipart.contiguous()
-        self.pending_scores = [p for p in self.pending_scores if p._value is None]
+        self.pending_scores = [r for r in self.pending_scores if r() is not None and r()._value is None]
 
     def score_negatives(self, model, ids, q1, q2=None, gamma=0.0, cen=0.0, regularizer=None):
         """Gather-fused logits [B,K]; q1/q2 are [B,dim] or [B,1,dim] and receive gradients.

@@ -446,7 +446,7 @@ class LazyScores(_Delegating):
         model, cen = logit._fusable()
         self.request = self.opt.lazy_request(model, d.rows, d.queries, logit.const, cen)   # None: not a fused layout
         if self.request is not None:
-            self.opt.pending_scores.append(self)
+            self.opt.pending_scores.append(weakref.ref(self))   # a placeholder nobody holds any more is never scored
 
     shape = property(lambda self: torch.Size((self.logit.shape[0], self.logit.shape[2])))
     device = property(lambda self: self.logit.device)

@@ -263,3 +263,21 @@ def test_pending_scores_behave_as_the_tensor_they_stand_for():
     lp, ln = fresh()
     assert len(ln) == b and ln.size(1) == k and ln.dim() == 2 and ln.numel() == b * k and ln.dtype == torch.float32
     assert abs(float(lp.sum()) - float(want_p.sum())) < 1e-3
+
+
+def test_a_placeholder_nobody_holds_is_never_scored():
+    """An evaluation loop that ignores one of the two logits (train_process.py:112-128 takes the negative ones only)
+    must not leave work or memory behind: the optimizer holds pending scores by weak reference."""
+    import gc
+    n, d, b, k = 40, 8, 3, 5
+    opt = RecordingOptimizer(n, d)
+    (q,) = _queries(b, 1, d, 1, 31)
+    ids = torch.randint(0, n, (b, k), generator=torch.Generator().manual_seed(6))
+    cal = lambda rows: torch.max(12.0 - ext_ops.l1_dist(rows, q), dim=1)[0]
+    for _ in range(3):
+        dropped = cal(LazyRows(opt, ids[:, 0], None).unsqueeze(1))
+        del dropped
+    gc.collect()
+    kept = cal(LazyRows(opt, ids.view(-1), None).view(b, k, -1))
+    float(kept.sum())
+    assert opt.scored == [("l1", (b, k), 12.0, 0.0, None)] and not opt.pending_scores
