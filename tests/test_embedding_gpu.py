@@ -472,3 +472,40 @@ def test_row_optimizers_match_oracle(name, squeeze):
         assert_close(state.cpu().numpy(), v, 2e-5, f"{name} second moment")
     if name == "adam":
         assert_close(emb.state_sum_fo.cpu().numpy(), m, 2e-5, "adam first moment")
+
+
+def test_fused_records_of_two_query_batches_and_a_plain_lookup_in_one_step():
+    """Two score_negatives calls against DIFFERENT query tensors cannot share one entity pass: each record is
+    reduced to per-entity gradient rows, merged with the plain lookup's rows (embed_optimizer.py:155-163) and
+    applied as one update per entity.  Against the oracle's merge of all three index streams."""
+    n, d, b, k, lr = 300, 32, 6, 10, 1e-3
+    rng = np.random.default_rng(12)
+    f32 = lambda a: np.asarray(a).astype(np.float32).astype(np.float64)
+    emb, opt = _setup(n, d, 9)
+    table = emb.embedding.detach().cpu().numpy().astype(np.float64)
+    qa, qb = f32(rng.uniform(-0.07, 0.07, (b, d))), f32(rng.uniform(-0.07, 0.07, (b, d)))
+    ids_a, ids_b = rng.integers(0, n // 3, (b, k)), rng.integers(0, n // 3, (b, k))
+    looked = rng.integers(0, n // 3, b)
+    ga, gb = f32(rng.standard_normal((b, k))), f32(rng.standard_normal((b, k)))
+    gl = f32(rng.standard_normal((b, d)))
+    dev = lambda a: torch.tensor(a, dtype=torch.float32, device="cuda")
+    ta, tb = dev(qa).requires_grad_(), dev(qb).requires_grad_()
+    opt.zero_grad()
+    la = opt.score_negatives("l1", torch.tensor(ids_a, device="cuda"), ta, None, gamma=12.0)
+    lb = opt.score_negatives("l1", torch.tensor(ids_b, device="cuda"), tb, None, gamma=12.0)
+    rows = emb(torch.tensor(looked, device="cuda"), "anchor")
+    ((la * dev(ga)).sum() + (lb * dev(gb)).sum() + (rows * dev(gl)).sum()).backward()
+    assert len(opt.fused_list) == 2 and len(opt.grad_list) == 1
+    opt.apply_grad(lr)
+    opt.check_ids()
+    grads = []
+    for ids, q, g, t, logit in ((ids_a, qa, ga, ta, la), (ids_b, qb, gb, tb, lb)):
+        e = orc.gather(table, ids).reshape(b, k, d)
+        assert_close(logit.detach().cpu().numpy(), orc.score_forward("l1", e, q[:, None], None, 12.0), REL_F32, "logits")
+        g_rows, g_q, _ = orc.score_backward("l1", g, e, q[:, None], None)
+        assert_close(t.grad.cpu().numpy(), g_q[:, 0], REL_F32, "query gradient")
+        grads.append(g_rows.reshape(b * k, d))
+    w, m, v, uniq, merged = oracle_adam_step(table, [ids_a, ids_b, looked], grads + [gl], lr, 1)
+    assert_close(emb.state_sum_fo.cpu().numpy()[uniq], m[uniq], REL_F32, "first moment")
+    assert_close(emb.state_sum_sq.cpu().numpy()[uniq], v[uniq], REL_F32, "second moment", rms_floor=False)
+    assert_adam_weights(emb.embedding.detach().cpu().numpy(), w, merged, uniq, lr, "weights")
