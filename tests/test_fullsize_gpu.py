@@ -207,3 +207,26 @@ def test_plan_at_pair_counts_beyond_256_tiles_of_16_rounds(n_pairs):
     assert torch.equal(seg[1:] - seg[:-1], counts)
     alone = plan.pair_seg < 0
     assert int(alone.sum().item()) == int((counts == 1).sum().item())
+
+
+def test_plan_around_the_tile_geometry_boundaries():
+    """Pair counts on both sides of every change of the radix passes' geometry near one tile per CU (16, 17, 18
+    elements per thread, then a second round of tiles), uniform 27-bit ids: sorted order, stability and segment
+    table against torch's stable sort."""
+    from smore_amd import fused
+    n = 86_054_151
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(99)
+    per = 1024 * 256
+    for n_pairs in (16 * per - 1, 16 * per, 16 * per + 1, 17 * per, 17 * per + 1, 18 * per - 1, 18 * per, 18 * per + 1,
+                    18 * per + 18 * 1024, 19 * per + 7):
+        ids = torch.randint(0, n, (n_pairs,), device="cuda", generator=gen)
+        ids[: n_pairs // 50] = ids[0]                                  # one long segment as well
+        plan = fused.build_plan(ids, n)
+        want_ids, want_order = torch.sort(ids, stable=True)
+        assert torch.equal(plan.sorted_ids.long(), want_ids), n_pairs
+        assert torch.equal(plan.order.long(), want_order), n_pairs
+        heads = torch.ones(n_pairs, dtype=torch.bool, device="cuda")
+        heads[1:] = want_ids[1:] != want_ids[:-1]
+        assert plan.n_uniq == int(heads.sum().item())
+        assert torch.equal(plan.seg_start[: plan.n_uniq].long(), torch.nonzero(heads).reshape(-1))
