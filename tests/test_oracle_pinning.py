@@ -436,6 +436,43 @@ def test_score_backward_matches_autograd_l2_and_box():
     assert np.allclose(go, to.grad.numpy(), rtol=1e-11, atol=1e-14)
 
 
+def test_similarity_and_two_half_scores_match_autograd_of_the_closed_forms():
+    """score_forward / score_backward for the models the two tests above leave open: ComplEx and DistMult, whose
+    logit is gamma + similarity (models/complex.py:140-148; naive_complex_sim, complex_dist.py:67-70;
+    naive_innerprod, distmult_dist.py:66-68) -- a flipped sign on the coefficient would pass every distance
+    test -- RotatE (naive_rotate_dist, rotate_dist.py:68-75) and Beta-KL (torch.distributions' _kl_beta_beta,
+    beta.py:298)."""
+    rng = np.random.default_rng(16)
+    b, k, d = 3, 5, 6
+    gs = rng.standard_normal((b, k))
+    t = lambda x: torch.tensor(x, requires_grad=True)
+
+    def check(model, rows, q1, q2, gamma, closed_form):
+        tr, t1 = t(rows), t(q1)
+        t2 = None if q2 is None else t(q2)
+        s = closed_form(tr, t1, t2)
+        assert np.allclose(orc.score_forward(model, rows, q1, q2, gamma), s.detach().numpy(), rtol=1e-11, atol=1e-13), model
+        (s * torch.from_numpy(gs)).sum().backward()
+        gr, g1, g2 = orc.score_backward(model, gs, rows, q1, q2)
+        assert np.allclose(gr, tr.grad.numpy(), rtol=1e-9, atol=1e-12), model
+        assert np.allclose(g1, t1.grad.numpy(), rtol=1e-9, atol=1e-12), model
+        if q2 is not None:
+            assert np.allclose(g2, t2.grad.numpy(), rtol=1e-9, atol=1e-12), model
+
+    rows2 = rng.standard_normal((b, k, 2 * d))
+    re, im = rng.standard_normal((b, 1, d)), rng.standard_normal((b, 1, d))
+    check("complex", rows2, re, im, 3.0, lambda e, a, c: 3.0 + (e[..., :d] * a + e[..., d:] * c).sum(-1))
+    check("rotate", rows2, re, im, 9.0,
+          lambda e, a, c: 9.0 - torch.sqrt((e[..., :d] - a) ** 2 + (e[..., d:] - c) ** 2).sum(-1))
+    rows1, q = rng.standard_normal((b, k, d)), rng.standard_normal((b, 1, d))
+    check("distmult", rows1, q, None, 2.0, lambda e, a, c: 2.0 + (e * a).sum(-1))
+    pos = lambda *sh: np.clip(1 + rng.standard_normal(sh), 0.05, 1e9)
+    rows_b, qa, qb = pos(b, k, 2 * d), pos(b, 1, d), pos(b, 1, d)
+    kl = torch.distributions.kl._kl_beta_beta
+    check("beta_kl", rows_b, qa, qb, 60.0,
+          lambda e, a, c: 60.0 - kl(torch.distributions.Beta(e[..., :d], e[..., d:]), torch.distributions.Beta(a, c)).sum(-1))
+
+
 def test_train_step_equals_dense_autograd_pipeline():
     """gather -> score -> backward -> merge -> Adam equals autograd through table[idx]
     followed by a dense Adam restricted to the touched rows."""
