@@ -252,6 +252,84 @@ def time_graph_replays(step, steps, warmup):
     return ms
 
 
+def dropin_bench(cfg, device, seed, steps, warmup):
+    """The step as SMORE's own code reaches it (box workloads): SparseEmbedding + AdamEmbedOptimizer, the lookup /
+    view / cal_logit sequence of KGReasoning.forward (kg_reasoning.py:298-307, 340-355) with box.py:157-164 as the
+    logit, the sample loss of train_process.py:197-213 (uniform weights), loss.backward(), apply_grad(lr).
+    Three flows -- negatives only; + the positive lookup; + an anchor lookup whose rows make the query centers
+    (a 1p query: center = anchor + relation, box.py:137) -- each with the lazy lookup handle and with plain lookups
+    (lazy_lookup = False: the reference's data flow, materialised [B*K, row] rows and gradient rows), and the
+    explicit score_negatives call.  Prints one JSON line of ms per step."""
+    import types
+    import torch
+    import torch.nn.functional as F
+    from smore_amd.embedding.embed_optimizer import AdamEmbedOptimizer
+    from smore_amd.embedding.sparse_embed import SparseEmbedding
+    from smore_amd.torchext.ext_ops import box_dist_in, box_dist_out
+    if cfg["model"] != "box":
+        sys.exit("--dropin restates the box model's code path: use --config 2 or 5")
+    table, q1, q2, idx, _ = make_inputs(cfg, device, seed)
+    b, k = idx.shape
+    emb = SparseEmbedding(8, cfg["dim"])
+    emb.embedding = torch.nn.Parameter(table, requires_grad=True)
+    emb.num_rows = cfg["n"]
+    opt = AdamEmbedOptimizer(types.SimpleNamespace(optim_mode="(aggr,adam,gpu,False,5)", share_optim_stats=True), emb, 0)
+    gamma = torch.nn.Parameter(torch.tensor([cfg["gamma"]], device=device), requires_grad=False)
+    rel_c, rel_o = q1.clone().requires_grad_(True), q2.clone().requires_grad_(True)
+    pos, anchor = idx[:, 0].contiguous(), idx[:, 1].contiguous()
+    lr = cfg.get("lr", 1e-4)
+
+    def cal_logit(entity_embedding, center, offset):        # box.py:157-164
+        d1 = box_dist_out(entity_embedding, center, offset)
+        d2 = box_dist_in(entity_embedding, center, offset)
+        return torch.max(gamma - d1 - cfg["cen"] * d2, dim=1)[0]
+
+    def step(flow, explicit=False):
+        opt.zero_grad()
+        rel_c.grad = rel_o.grad = None
+        center = rel_c
+        if flow == "anchor+positive+negatives":
+            a = emb(anchor, "anchor")
+            a.job_handle.sync()
+            center = a + rel_c
+        center, offset = center.view(b, 1, 1, -1), rel_o.view(b, 1, 1, -1)
+        positive_logit = None
+        if flow != "negatives":
+            p_rows = emb(pos, "positive_entity")
+        n_rows = None if explicit else emb(idx.view(-1), "negative_entity")
+        if flow != "negatives":
+            p_rows.job_handle.sync()
+            positive_logit = cal_logit(p_rows.unsqueeze(1), center, offset)
+        if explicit:
+            negative_logit = opt.score_negatives("box", idx, center, offset, gamma=cfg["gamma"], cen=cfg["cen"])
+        else:
+            n_rows.job_handle.sync()
+            negative_logit = cal_logit(n_rows.view(b, k, -1), center, offset)
+        loss = -F.logsigmoid(-negative_logit).mean(dim=1).mean()
+        if positive_logit is not None:
+            loss = loss - F.logsigmoid(positive_logit).squeeze(dim=1).mean()
+        (loss / 2).backward()
+        opt.apply_grad(lr)
+
+    out = {}
+    routes = [("explicit score_negatives", True, "negatives", True)]
+    for flow in ("negatives", "positive+negatives", "anchor+positive+negatives"):
+        routes += [(f"lazy handle, {flow}", True, flow, False), (f"plain lookups, {flow}", False, flow, False)]
+    for name, lazy, flow, explicit in routes:
+        opt.lazy_lookup = lazy
+        for _ in range(warmup):
+            step(flow, explicit)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            step(flow, explicit)
+        torch.cuda.synchronize()
+        out[name] = (time.perf_counter() - t0) * 1e3 / steps
+    opt.check_ids()
+    print(json.dumps({"workload": cfg["name"], "dropin_ms_per_step": out, "steps": steps, "warmup": warmup,
+                      "pairs_per_step": b * k}))
+
+
 def cpu_baseline(cfg, seed):
     """Times the CPU oracle (fp32 build, OpenMP) on a bounded sample of the same workload: same row length,
     K, id distribution and optimizer, fewer queries and -- for the 86M-row table -- fewer rows."""
@@ -484,6 +562,9 @@ def main():
                          "config's table instead of the training step; prints its own JSON line")
     ap.add_argument("--rank-queries", type=int, default=1,
                     help="queries per call of the evaluation scan (the reference evaluates one query at a time)")
+    ap.add_argument("--dropin", action="store_true",
+                    help="time the step as SMORE's model code and training loop reach it (lookup handle, cal_logit, "
+                         "sample loss, backward, apply_grad) beside the reference's data flow, instead of the three C calls")
     ap.add_argument("--ceilings", action="store_true",
                     help="run only the bandwidth probes (read, copy, update, fill, random rows of the config's row "
                          "length, plain and non-temporal) and print them as one JSON line")
@@ -520,6 +601,9 @@ def main():
         return
     if args.rank_scan:
         rank_scan_bench(cfg, device, seed, args.steps, args.warmup, args.rank_queries)
+        return
+    if args.dropin:
+        dropin_bench(cfg, device, seed, args.steps, args.warmup)
         return
 
     if args.serial_backward:
