@@ -266,6 +266,7 @@ def dropin_bench(cfg, device, seed, steps, warmup):
     from smore_amd.embedding.embed_optimizer import AdamEmbedOptimizer
     from smore_amd.embedding.sparse_embed import SparseEmbedding
     from smore_amd.torchext.ext_ops import box_dist_in, box_dist_out
+    from smore_amd.training import sample_loss
     if cfg["model"] != "box":
         sys.exit("--dropin restates the box model's code path: use --config 2 or 5")
     table, q1, q2, idx, _ = make_inputs(cfg, device, seed)
@@ -284,7 +285,7 @@ def dropin_bench(cfg, device, seed, steps, warmup):
         d2 = box_dist_in(entity_embedding, center, offset)
         return torch.max(gamma - d1 - cfg["cen"] * d2, dim=1)[0]
 
-    def step(flow, explicit=False):
+    def step(flow, explicit=False, fused_loss=False):
         opt.zero_grad()
         rel_c.grad = rel_o.grad = None
         center = rel_c
@@ -305,24 +306,29 @@ def dropin_bench(cfg, device, seed, steps, warmup):
         else:
             n_rows.job_handle.sync()
             negative_logit = cal_logit(n_rows.view(b, k, -1), center, offset)
-        loss = -F.logsigmoid(-negative_logit).mean(dim=1).mean()
-        if positive_logit is not None:
-            loss = loss - F.logsigmoid(positive_logit).squeeze(dim=1).mean()
-        (loss / 2).backward()
+        if fused_loss:      # smore_amd.training.sample_loss: the same loss as one launch (needs both logits)
+            loss, _, _ = sample_loss(positive_logit, negative_logit)
+            loss.backward()
+        else:
+            loss = -F.logsigmoid(-negative_logit).mean(dim=1).mean()
+            if positive_logit is not None:
+                loss = loss - F.logsigmoid(positive_logit).squeeze(dim=1).mean()
+            (loss / 2).backward()
         opt.apply_grad(lr)
 
     out = {}
-    routes = [("explicit score_negatives", True, "negatives", True)]
+    routes = [("explicit score_negatives", True, "negatives", True, False)]
     for flow in ("negatives", "positive+negatives", "anchor+positive+negatives"):
-        routes += [(f"lazy handle, {flow}", True, flow, False), (f"plain lookups, {flow}", False, flow, False)]
-    for name, lazy, flow, explicit in routes:
+        routes += [(f"lazy handle, {flow}", True, flow, False, False), (f"plain lookups, {flow}", False, flow, False, False)]
+    routes.append(("lazy handle + fused sample loss, anchor+positive+negatives", True, "anchor+positive+negatives", False, True))
+    for name, lazy, flow, explicit, fused_loss in routes:
         opt.lazy_lookup = lazy
         for _ in range(warmup):
-            step(flow, explicit)
+            step(flow, explicit, fused_loss)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         for _ in range(steps):
-            step(flow, explicit)
+            step(flow, explicit, fused_loss)
         torch.cuda.synchronize()
         out[name] = (time.perf_counter() - t0) * 1e3 / steps
     opt.check_ids()

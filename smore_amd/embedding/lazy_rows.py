@@ -150,10 +150,12 @@ class LazyRows(_Delegating):
         self.shape = torch.Size(tuple(ids.shape) + (row,)) if shape is None else torch.Size(shape)
         self.reg = reg                    # (add, lo, hi) once the clamp has been seen
         self.pending_add = pending_add    # `rows + c` that has not met its clamp yet
-        self.root = root if root is not None else self
+        self._root = root                 # None: this handle is the family's first (no reference to itself: the
         self.job_handle = opt.sparse_embed.dummy_job
-        if root is None:
+        if root is None:                  # rows it may hold must go when the last user lets go, not at a later GC pass)
             self._looked_up = None        # the plain lookup, made at most once per handle family
+
+    root = property(lambda self: self if self._root is None else self._root)
 
     # -- what the model code asks of a tensor before any value is needed
     device = property(lambda self: self.opt.sparse_embed.embedding.device)

@@ -281,3 +281,33 @@ def test_a_placeholder_nobody_holds_is_never_scored():
     kept = cal(LazyRows(opt, ids.view(-1), None).view(b, k, -1))
     float(kept.sum())
     assert opt.scored == [("l1", (b, k), 12.0, 0.0, None)] and not opt.pending_scores
+
+
+def test_handles_leave_no_reference_cycles():
+    """A handle family can hold gigabytes (the ids, the looked-up rows): everything must go when the model code
+    lets go of it, by reference count, not at some later pass of the cycle collector."""
+    import gc
+    n, d, b, k = 60, 8, 4, 6
+    opt = RecordingOptimizer(n, d)
+    c, o = _queries(b, 1, d, 2, 12)
+    ids = torch.randint(0, n, (b, k), generator=torch.Generator().manual_seed(3))
+
+    def fused_use():
+        rows = LazyRows(opt, ids.view(-1), None)
+        rows.job_handle.sync()
+        rows = rows.view(b, k, -1)
+        values, which = torch.max(24.0 - ext_ops.box_dist_out(rows, c, o) - 0.02 * ext_ops.box_dist_in(rows, c, o), dim=1)
+        return float(values.sum()) + float(which.sum())
+
+    def plain_use():
+        rows = LazyRows(opt, ids.view(-1), None).view(b, k, -1)
+        return float(torch.norm(rows + 1.0, p=3))
+
+    gc.collect()
+    gc.disable()
+    try:
+        for use in (fused_use, plain_use):
+            use()
+            assert gc.collect() == 0, use.__name__
+    finally:
+        gc.enable()
