@@ -15,7 +15,7 @@ the per-operator Functions of smore/common/torchext/dist_func/*.py:
 import torch
 
 from ... import extlib_hip as extlib
-from ...embedding.lazy_rows import LazyRows, lazy_dist
+from ...embedding.lazy_rows import LazyRows, _is_lazy, lazy_dist
 
 TWO_HALVES = ("rotate", "complex", "beta_kl", "beta_l2", "beta_fisher_approx")
 
@@ -66,6 +66,8 @@ def apply_dist(kind, entity_embed, *queries):
         if lazy is not None:
             return lazy
         entity_embed = entity_embed.materialize().contiguous()
+    # a lookup handle (or a pending score) on the query side has nothing to fuse: the operator gets its values
+    queries = [q.materialize() if _is_lazy(q) else q for q in queries]
     first = queries[0]
     if entity_embed.dim() != first.dim():
         assert first.dim() == 4

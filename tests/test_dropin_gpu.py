@@ -471,3 +471,35 @@ def test_shared_negatives_beside_positives_share_one_record():
     w, m, v, uniq, merged = oracle_adam_step(table, [ids], [g_rows.reshape(b * (1 + k), d)], lr, 1)
     assert_close(emb.state_sum_fo.cpu().numpy()[uniq], m[uniq], REL_F32, "first moment")
     assert_adam_weights(emb.embedding.detach().cpu().numpy(), w, merged, uniq, lr, "weights")
+
+
+def test_a_lookup_handle_as_the_query_operand():
+    """Negatives handed to the operator as its QUERY operand without any arithmetic first (the reverse layout with
+    an identity projection): the handle stands for its rows, the operator runs on its reverse-layout kernels and
+    the lookup's gradient rows reach the optimizer."""
+    from smore_amd.embedding.embed_optimizer import AdamEmbedOptimizer
+    from smore_amd.embedding.sparse_embed import SparseEmbedding
+    from smore_amd.torchext.ext_ops import l1_dist
+    n, d, b, k, lr = 200, 16, 4, 9, 1e-3
+    rng = np.random.default_rng(41)
+    table = rng.uniform(-0.07, 0.07, (n, d)).astype(np.float32).astype(np.float64)
+    tail, neg = rng.integers(0, n, b), rng.integers(0, n, (b, k))
+    gn = rng.standard_normal((b, k)).astype(np.float32).astype(np.float64)
+    emb = SparseEmbedding(n, d).cuda()
+    with torch.no_grad():
+        emb.embedding.copy_(torch.tensor(table, dtype=torch.float32))
+    opt = AdamEmbedOptimizer(types.SimpleNamespace(optim_mode="(aggr,adam,gpu,False,5)", share_optim_stats=True), emb, 0)
+    opt.zero_grad()
+    entity = emb(torch.tensor(tail, device="cuda")).unsqueeze(1)
+    queries = emb(torch.tensor(neg, device="cuda").view(-1), "negative_entity").view(b, k, -1)
+    logit = 12.0 - l1_dist(entity, queries)
+    assert logit.shape == (b, k)
+    (logit * torch.tensor(gn, dtype=torch.float32, device="cuda")).sum().backward()
+    assert len(opt.grad_list) == 2 and not opt.fused_list
+    opt.apply_grad(lr)
+    e, q = orc.gather(table, tail).reshape(b, 1, d), orc.gather(table, neg).reshape(b, k, d)
+    assert_close(logit.detach().cpu().numpy(), 12.0 - orc.dist_forward("l1", e, q), REL_F32, "logits, handle as query")
+    g_e, g_q, _ = orc.dist_backward("l1", -gn, e, q)
+    w, m, v, uniq, merged = oracle_adam_step(table, [tail, neg], [g_e.reshape(b, d), g_q.reshape(b * k, d)], lr, 1)
+    assert_close(emb.state_sum_fo.cpu().numpy()[uniq], m[uniq], REL_F32, "first moment, handle as query")
+    assert_adam_weights(emb.embedding.detach().cpu().numpy(), w, merged, uniq, lr, "weights, handle as query")

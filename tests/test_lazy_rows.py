@@ -311,3 +311,23 @@ def test_handles_leave_no_reference_cycles():
             assert gc.collect() == 0, use.__name__
     finally:
         gc.enable()
+
+
+def test_a_handle_on_the_query_side_is_looked_up():
+    """The reverse layout of inverse queries hands the negatives to the operator as the QUERY operand
+    (kg_reasoning.py:257-263): a handle there has nothing to fuse and stands for its rows."""
+    n, d, b, k = 30, 8, 3, 4
+    opt = RecordingOptimizer(n, d)
+    gen = torch.Generator().manual_seed(8)
+    tail, neg = torch.randint(0, n, (b,), generator=gen), torch.randint(0, n, (b, k), generator=gen)
+    table = opt.sparse_embed.embedding
+    entity = table[tail].unsqueeze(1).contiguous()                                   # [B,1,D] tensor
+    queries = LazyRows(opt, neg.view(-1), "negative_entity").view(b, k, -1)         # [B,K,D] handle
+    want = _textbook("l1", entity, (table[neg],), 0.0)
+    try:
+        got = ext_ops.l1_dist(entity, queries)
+    except Exception as e:                                                          # no GPU here: the dense operator needs the library's kernels
+        assert "materialize" not in str(e) and "LazyRows" not in str(e), e
+        assert opt.looked_up == ["negative_entity"]
+        return
+    assert torch.allclose(got, want, atol=1e-5)
