@@ -1111,3 +1111,48 @@ def test_gradient_rows_reach_every_row_optimizer(kind, squeeze):
     for name, a, c in zip("wmv", out["fused"], out["rows"]):
         if a is not None:
             assert torch.equal(a, c), f"{kind}: {name} differs between the fused pass and the materialised route"
+
+
+def test_gradient_rows_at_a_size_that_forks():
+    """4096 box queries x 300 negatives + 4096 looked-up rows, Adam: the step is large enough for the pair-ordered
+    kernel (ids that occur once among the scored pairs) beside the entity pass on the second stream.  An id that is
+    scored once AND looked up is no one-pair segment and must get both parts.  Against the materialised route
+    (merged rows of the same call -> smx_rows_backward), bit for bit."""
+    from smore_amd import fused
+    n, b, k, dim, lr = 4_000_000, 4096, 300, 200, 1e-3
+    g = torch.Generator(device="cuda").manual_seed(5)
+    table = torch.empty((n, dim), device="cuda").uniform_(-0.07, 0.07, generator=g)
+    q1 = torch.empty((b, dim), device="cuda").uniform_(-0.07, 0.07, generator=g)
+    q2 = torch.empty((b, dim), device="cuda").uniform_(-0.07, 0.07, generator=g).abs_()
+    idx = torch.randint(0, n, (b, k), device="cuda", generator=g)
+    gs = torch.randn((b, k), device="cuda", generator=g)
+    looked_up = torch.cat([idx[:, 0], torch.randint(0, n, (b // 2,), device="cuda", generator=g),
+                           torch.full((300,), int(idx[0, 1]), device="cuda")])
+    extra = torch.randn((looked_up.numel(), dim), device="cuda", generator=g)
+    params = fused.score_params(24.0, 0.02)
+    flat = torch.cat([idx.reshape(-1), looked_up])
+    plan = fused.build_plan(flat, n)
+    counts = torch.bincount(flat, minlength=n)
+    assert int(((counts == 1)[idx.reshape(-1)]).sum().item()) > 30_000, "the case must have one-pair ids among the scored pairs"
+    assert int((counts[idx[:, 0]] == 2).sum().item()) > 1000, "and ids scored once that are also looked up"
+    uniq_plan = fused.build_plan(plan.uniq, n)
+    out = {}
+    for route in ("fused", "rows"):
+        w, m, v = table.clone(), torch.zeros_like(table), torch.zeros_like(table)
+        codes = fused.new_codes("box", w, idx, q1)
+        score = fused.score_forward("box", w, idx, q1, q2, params, codes=codes)
+        opt = fused.adam_params(lr, 2)
+        if route == "fused":
+            fused.score_backward_entity_multi("box", plan, w, q1, q2, [(score, gs, codes)], params, m=m, v=v, adam=opt,
+                                              grad_rows=extra)
+        else:
+            merged = torch.empty((plan.n_uniq, dim), device="cuda")
+            fused.score_backward_entity_multi("box", plan, w, q1, q2, [(score, gs, codes)], params, merged=merged,
+                                              grad_rows=extra)
+            fused.rows_backward(uniq_plan, merged, table=w, m=m, v=v, adam=opt)
+        out[route] = (w, m, v)
+    for name, a, c in zip("wmv", out["fused"], out["rows"]):
+        assert torch.equal(a, c), f"{name} differs between the forking fused pass and the materialised route"
+    touched = torch.zeros(n, dtype=torch.bool, device="cuda")
+    touched[plan.uniq] = True
+    assert torch.equal(out["fused"][0][~touched], table[~touched])
