@@ -180,9 +180,11 @@ class Step:
         self.codes = fused.new_codes(cfg["model"], table, idx, q1) if sign_codes else None
         self.plan = None
 
-    def run(self, events=None, step_consts=None):
+    def run(self, events=None, step_consts=None, measure_parts=None):
         """step_consts: two-float device tensor the optimizer kernels read lr / bias corrections from (a captured
-        step is replayed with frozen by-value arguments, so the advancing step counter has to come from memory)."""
+        step is replayed with frozen by-value arguments, so the advancing step counter has to come from memory).
+        measure_parts (1 or 2): launch only one half of the backward call, through the library's measuring entry
+        point (include/smx_measure.h); the step is then incomplete."""
         f, cfg = self.fused, self.cfg
         mark = (lambda i: events[i].record()) if events is not None else (lambda i: None)
         self.step_no += 1
@@ -196,13 +198,14 @@ class Step:
             gq = f.score_backward_fused(cfg["model"], plan, self.table, self.idx, self.q1, self.q2, score, self.gscore,
                                         self.params, m=self.m, v=self.v,
                                         adam=f.adam_params(cfg["lr"], self.step_no, step_consts=step_consts),
-                                        codes=self.codes)
+                                        codes=self.codes, measure_parts=measure_parts)
         else:
             if self.merged is None:     # one row per distinct id; no more of those than pairs or table rows
                 self.merged = self.torch.empty((min(self.idx.numel(), cfg["n"]), self.table.shape[1]),
                                                device=self.table.device)
             gq = f.score_backward_fused(cfg["model"], plan, self.table, self.idx, self.q1, self.q2, score, self.gscore,
-                                        self.params, merged=self.merged, codes=self.codes)
+                                        self.params, merged=self.merged, codes=self.codes,
+                                        measure_parts=measure_parts)
         mark(3)
         self.plan = plan
         return score, gq
@@ -544,8 +547,8 @@ def rank_scan_bench(cfg, device, seed, steps, warmup, nq):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--config", type=int, default=5, choices=sorted(CONFIGS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-sign-codes", action="store_true",
@@ -556,7 +559,7 @@ def main():
                          "afterwards): what a rocprofv3 run of this script should see")
     ap.add_argument("--backward-parts", type=int, default=3, choices=(1, 2, 3),
                     help="with --profile-run: run only the query-gradient kernel (1) or only the entity pass (2) of the "
-                         "backward call (the library's measuring switch); the steps are then incomplete")
+                         "backward call (the library's measuring entry point); the steps are then incomplete")
     ap.add_argument("--graph", action="store_true",
                     help="also capture the whole step (plan, forward, backward + optimizer, second stream included) "
                          "in a HIP graph and time its replays; reported as graph_replay next to the eager figures")
@@ -614,10 +617,9 @@ def main():
 
     if args.serial_backward:
         _lib.call("smx_set_option", _lib.OPTION_SERIAL_BACKWARD, 1)
-    if args.backward_parts != 3:
-        if not args.profile_run:
-            sys.exit("--backward-parts is for --profile-run")
-        _lib.call("smx_set_option", _lib.OPTION_BACKWARD_PARTS, args.backward_parts)
+    if args.backward_parts != 3 and not args.profile_run:
+        sys.exit("--backward-parts is for --profile-run")
+    parts = None if args.backward_parts == 3 else args.backward_parts
     table, q1, q2, idx, gscore = make_inputs(cfg, device, seed)
     step = Step(cfg, table, q1, q2, idx, gscore, sign_codes=not args.no_sign_codes)
     for _ in range(args.warmup):
@@ -631,12 +633,18 @@ def main():
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for s in range(args.steps):
-        step.run(ev[s])
+        step.run(ev[s], measure_parts=parts)
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
+    if step.err.item() != 0:
+        sys.exit("a timed step reported an error (id out of range, or an invalid segment plan)")
 
     phase_ms = {name: sum(e[i].elapsed_time(e[i + 1]) for e in ev) / args.steps for i, name in enumerate(Step.PHASES)}
     ms_per_step = wall * 1e3 / args.steps
+    # spread of the steps' own device times (first to last event of a step), next to the wall-clock mean
+    per_step = sorted(e[0].elapsed_time(e[3]) for e in ev)
+    step_ms_events = {"median": per_step[len(per_step) // 2], "min": per_step[0], "max": per_step[-1],
+                      "p10": per_step[len(per_step) // 10], "p90": per_step[(9 * len(per_step)) // 10]}
     pairs = cfg["b"] * cfg["k"]
     algo = algorithmic_bytes(cfg, n_uniq)
     algo_stream = algorithmic_bytes(cfg, n_uniq, streaming=True)
@@ -652,25 +660,23 @@ def main():
 
     def timed_backward(parts, serial, reps=10, lead=3):
         """Average event-bracketed duration (ms) of the backward call with only `parts` of it running (the
-        library's measuring switch; 3 = the whole call).  Run after the timed region: a call with one half
+        library's measuring entry point; 3 = the whole call).  Run after the timed region: a call with one half
         leaves an incomplete step behind.  The first `lead` steps are not counted: they let the host get ahead of
         the device again, so that no bracket contains the device waiting for a launch."""
         _lib.call("smx_set_option", _lib.OPTION_SERIAL_BACKWARD, 1 if serial else 0)
-        _lib.call("smx_set_option", _lib.OPTION_BACKWARD_PARTS, parts)
         try:
             evs = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(lead + reps)]
             for e in evs:
-                step.run(e)
+                step.run(e, measure_parts=None if parts == 3 else parts)
             torch.cuda.synchronize()
         finally:
-            _lib.call("smx_set_option", _lib.OPTION_BACKWARD_PARTS, 3)
             _lib.call("smx_set_option", _lib.OPTION_SERIAL_BACKWARD, 0)
         return sum(e[2].elapsed_time(e[3]) for e in evs[lead:]) / reps
 
     if args.profile_run:
         print(json.dumps({"workload": cfg["name"], "profile_run": True, "serial_backward": args.serial_backward,
                           "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step, "phase_ms": phase_ms,
-                          "graph_replay_ms_per_step": graph_ms,
+                          "step_ms_events": step_ms_events, "graph_replay_ms_per_step": graph_ms,
                           "distinct_ids": n_uniq, "one_pair_ids": n_one_pair, "ids_with_2_to_64_pairs": n_short,
                           "ids_with_more_pairs": n_long, "pairs": pairs, "algorithmic_bytes_step": algo,
                           "algorithmic_bytes_query_kernel": q_bytes, "algorithmic_bytes_entity_pass": e_bytes,
@@ -739,6 +745,7 @@ def main():
             "streaming_GBps": algo_stream / (ms_per_step * 1e-3) / 1e9,
         },
         "phase_ms": phase_ms,
+        "step_ms_events": step_ms_events,
     }
     if graph_ms is not None:
         out["graph_replay"] = {"ms_per_step": graph_ms, "value": pairs / (graph_ms * 1e-3), "unit": "pairs/s",

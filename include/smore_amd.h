@@ -55,16 +55,11 @@ extern "C" {
 int smx_version(void);
 const char* smx_last_error(void);
 
-/* Process-wide switches (thread-safe; take effect for calls made afterwards).
+/* Process-wide switches (thread-safe; take effect for calls made afterwards).  None changes a result.
  *   SMX_OPTION_SERIAL_BACKWARD  != 0: smx_score_backward_fused / smx_score_backward_entity keep all their
  *                               kernels on the caller's stream instead of running the entity pass on the
- *                               library's second stream -- same results, for per-kernel profiling.
- *   SMX_OPTION_BACKWARD_PARTS   which halves of smx_score_backward_fused run: bit 0 the query-gradient kernel
- *                               (with the rows of ids that occur once), bit 1 the entity pass; default 3.
- *                               A measuring switch: with 1 or 2 a harness can bracket one half with events
- *                               by itself; the step such a call leaves is incomplete. */
+ *                               library's second stream -- same results, for per-kernel profiling. */
 #define SMX_OPTION_SERIAL_BACKWARD 1
-#define SMX_OPTION_BACKWARD_PARTS 2
 int smx_set_option(int option, int value);
 
 /* kind id for a dist_name string ("l1", "box_out", ...), -1 if unknown.

@@ -1,0 +1,31 @@
+/*
+ * smx_measure -- entry points of libsmore_amd.so that exist for measurement only.  Not part of the drop-in C ABI
+ * of smore_amd.h: no caller of the scoring path needs them, and what they leave behind is not a training step.
+ */
+#ifndef SMX_MEASURE_H
+#define SMX_MEASURE_H
+
+#include "smore_amd.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* No counterpart in the reference.  smx_score_backward_fused with only some of its kernels launched, so that a
+ * harness can bracket one half of the call with events by itself:
+ *   parts bit 0   the query-gradient kernel (with the rows of ids that occur once)
+ *   parts bit 1   the entity pass (segment, tile and fix-up kernels)
+ * parts = 3 is smx_score_backward_fused.  With 1 or 2 the step is INCOMPLETE: rows of the other half are not
+ * updated and, with 2, the query gradients are not written.  The choice is an argument of the call: nothing is
+ * remembered, no other call or caller is affected. */
+int smx_measure_backward_fused(int parts, int model, void* stream, const smx_plan_view* plan, float* table,
+                               size_t n_rows, const int64_t* idx, const float* q1, const float* q2,
+                               const float* score, const float* gscore, float* gq1, float* gq2, size_t B, size_t K,
+                               size_t dim, const smx_score_params* params, float* merged, float* m, float* v,
+                               const smx_opt_params* adam, void* workspace, size_t workspace_bytes,
+                               const void* fwd_codes, size_t fwd_codes_bytes);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SMX_MEASURE_H */

@@ -99,7 +99,6 @@ class PairSource(ctypes.Structure):
 
 MAX_PAIR_SOURCES = 4
 OPTION_SERIAL_BACKWARD = 1
-OPTION_BACKWARD_PARTS = 2     # bit 0: query-gradient kernel, bit 1: entity pass (3 = both, the default)
 
 _lib = None
 _probe = None
@@ -108,6 +107,13 @@ PROBE_PATH = os.path.join(_HERE, "libsmx_probe.so")
 
 class SmxError(RuntimeError):
     pass
+
+
+# measurement-only entry points of the same library (include/smx_measure.h), not part of the drop-in ABI
+MEASURE_SIGNATURES = {
+    # parts, then the arguments of smx_score_backward_fused
+    "smx_measure_backward_fused": (_i, [_i] + SIGNATURES["smx_score_backward_fused"][1]),
+}
 
 
 def load():
@@ -119,10 +125,11 @@ def load():
                 f"{LIB_PATH} is missing: build it with `python -c 'import __graft_entry__ as g; g.build()'` "
                 "or `make -C smore_amd/csrc`. There is no fallback path.")
         lib = ctypes.CDLL(LIB_PATH)
-        for name, (res, args) in SIGNATURES.items():
-            fn = getattr(lib, name)
-            fn.restype = res
-            fn.argtypes = args
+        for table in (SIGNATURES, MEASURE_SIGNATURES):
+            for name, (res, args) in table.items():
+                fn = getattr(lib, name)
+                fn.restype = res
+                fn.argtypes = args
         _lib = lib
     return _lib
 

@@ -25,8 +25,6 @@ int check_launch(const char* what) {
 
 static std::atomic<int> g_serial_backward{0};
 bool serial_backward() { return g_serial_backward.load(std::memory_order_relaxed) != 0; }
-static std::atomic<int> g_backward_parts{3};
-int backward_parts() { return g_backward_parts.load(std::memory_order_relaxed); }
 
 }  // namespace smx
 
@@ -37,11 +35,6 @@ int smx_version(void) { return 2; }
 int smx_set_option(int option, int value) {
   if (option == SMX_OPTION_SERIAL_BACKWARD) {
     smx::g_serial_backward.store(value ? 1 : 0, std::memory_order_relaxed);
-    return SMX_OK;
-  }
-  if (option == SMX_OPTION_BACKWARD_PARTS) {
-    if (value < 1 || value > 3) return smx::fail(SMX_ERR_ARG, "backward parts must be 1, 2 or 3");
-    smx::g_backward_parts.store(value, std::memory_order_relaxed);
     return SMX_OK;
   }
   return smx::fail(SMX_ERR_ARG, "unknown option %d", option);

@@ -21,8 +21,6 @@ int check_launch(const char* what);
 
 // smx_set_option(SMX_OPTION_SERIAL_BACKWARD, ..): the backward keeps to the caller's stream
 bool serial_backward();
-// smx_set_option(SMX_OPTION_BACKWARD_PARTS, ..): bit 0 query-gradient kernel, bit 1 entity pass
-int backward_parts();
 
 constexpr int kMaxSources = 4;  // index streams one entity pass can reduce together (SMX_MAX_PAIR_SOURCES)
 

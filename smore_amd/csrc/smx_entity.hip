@@ -39,14 +39,12 @@ extern template int entity_dispatch<mComplex>(hipStream_t, const EntityArgs&, in
 extern template int entity_dispatch<mDistmult>(hipStream_t, const EntityArgs&, int, int);
 extern template int entity_dispatch<kSrcRows>(hipStream_t, const EntityArgs&, int, int);
 
-constexpr int kTile = 256;      // sorted positions per tile of the long-segment pass
-constexpr int kShortMax = 64;   // longest segment one wavefront finishes on its own
-
 static size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
 
 struct EntityScratch {
   size_t tail_off, head_off, fix_off, total;
 };
+constexpr size_t kFixHeader = 64;  // ints in front of the fix-up list; the first is the list's length
 
 static EntityScratch entity_scratch(size_t n_pairs, size_t row_len) {
   const size_t tiles = (n_pairs + kTile - 1) / kTile;
@@ -54,7 +52,7 @@ static EntityScratch entity_scratch(size_t n_pairs, size_t row_len) {
   s.tail_off = 0;
   s.head_off = align256(tiles * row_len * sizeof(float));
   s.fix_off = s.head_off + align256(tiles * row_len * sizeof(float));
-  s.total = s.fix_off + align256(tiles);
+  s.total = s.fix_off + align256((tiles + kFixHeader) * sizeof(int));
   return s;
 }
 
@@ -91,7 +89,8 @@ static int fill_plan(EntityArgs* A, const smx_plan_view* plan, void* workspace, 
   char* ws = static_cast<char*>(workspace);
   A->tail = reinterpret_cast<float*>(ws + sc.tail_off);
   A->head = reinterpret_cast<float*>(ws + sc.head_off);
-  A->fix = reinterpret_cast<unsigned char*>(ws + sc.fix_off);
+  A->fix_count = reinterpret_cast<int*>(ws + sc.fix_off);
+  A->fix_list = A->fix_count + kFixHeader;
   return SMX_OK;
 }
 

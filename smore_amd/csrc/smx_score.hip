@@ -18,6 +18,7 @@
 // in wavefront order, so the gradient has a fixed summation order.
 #include <mutex>
 
+#include "../../include/smx_measure.h"
 #include "smx_score_impl.h"
 
 namespace smx {
@@ -351,13 +352,17 @@ int smx_score_backward_entity_multi(int model, void* stream, const smx_plan_view
                          adam, workspace, workspace_bytes, 0, S.codes[0], codes_vec, codes_nit, &S);
 }
 
-int smx_score_backward_fused(int model, void* stream, const smx_plan_view* plan, float* table, size_t n_rows,
-                             const int64_t* idx, const float* q1, const float* q2, const float* score,
-                             const float* gscore, float* gq1, float* gq2, size_t B, size_t K, size_t dim,
-                             const smx_score_params* params, float* merged, float* m, float* v,
-                             const smx_opt_params* adam, void* workspace, size_t workspace_bytes,
-                             const void* fwd_codes, size_t fwd_codes_bytes) {
-  using namespace smx;
+}  // extern "C"
+
+namespace smx {
+
+// parts: bit 0 the query-gradient kernel, bit 1 the entity pass (3 for every caller but the measuring entry point)
+static int backward_fused(int parts, int model, void* stream, const smx_plan_view* plan, float* table, size_t n_rows,
+                          const int64_t* idx, const float* q1, const float* q2, const float* score,
+                          const float* gscore, float* gq1, float* gq2, size_t B, size_t K, size_t dim,
+                          const smx_score_params* params, float* merged, float* m, float* v,
+                          const smx_opt_params* adam, void* workspace, size_t workspace_bytes,
+                          const void* fwd_codes, size_t fwd_codes_bytes) {
   ScoreArgs A;
   int vec, nit;
   if (!idx) return fail(SMX_ERR_ARG, "the fused backward needs the id tensor");
@@ -429,7 +434,6 @@ int smx_score_backward_fused(int model, void* stream, const smx_plan_view* plan,
     std::lock_guard<std::mutex> one_call(side->in_use);
     if (hipEventRecord(side->fork, st) != hipSuccess || hipStreamWaitEvent(side->stream, side->fork, 0) != hipSuccess)
       return fail(SMX_ERR_HIP, "fork to the side stream failed");
-    const int parts = backward_parts();
     int rc = (parts & 1) ? dispatch_model(model, st, A, vec, nit, false) : SMX_OK;
     if (rc == SMX_OK && (parts & 2))
       rc = entity_backward(model, side->stream, plan, table, n_rows, q1, q2, score, gscore, B, K, dim, params, merged, m,
@@ -439,12 +443,36 @@ int smx_score_backward_fused(int model, void* stream, const smx_plan_view* plan,
       return fail(SMX_ERR_HIP, "join with the side stream failed");
     return rc;
   }
-  const int parts = backward_parts();
   if (parts & 1)
     if (int rc = dispatch_model(model, as_stream(stream), A, vec, nit, false)) return rc;
   if (!(parts & 2)) return SMX_OK;
   return entity_backward(model, stream, plan, table, n_rows, q1, q2, score, gscore, B, K, dim, params, merged, m, v,
                          adam, workspace, workspace_bytes, singles_here ? 1 : 0, codes, vec, nit);
+}
+
+}  // namespace smx
+
+extern "C" {
+
+int smx_score_backward_fused(int model, void* stream, const smx_plan_view* plan, float* table, size_t n_rows,
+                             const int64_t* idx, const float* q1, const float* q2, const float* score,
+                             const float* gscore, float* gq1, float* gq2, size_t B, size_t K, size_t dim,
+                             const smx_score_params* params, float* merged, float* m, float* v,
+                             const smx_opt_params* adam, void* workspace, size_t workspace_bytes,
+                             const void* fwd_codes, size_t fwd_codes_bytes) {
+  return smx::backward_fused(3, model, stream, plan, table, n_rows, idx, q1, q2, score, gscore, gq1, gq2, B, K, dim, params,
+                             merged, m, v, adam, workspace, workspace_bytes, fwd_codes, fwd_codes_bytes);
+}
+
+int smx_measure_backward_fused(int parts, int model, void* stream, const smx_plan_view* plan, float* table, size_t n_rows,
+                               const int64_t* idx, const float* q1, const float* q2, const float* score,
+                               const float* gscore, float* gq1, float* gq2, size_t B, size_t K, size_t dim,
+                               const smx_score_params* params, float* merged, float* m, float* v,
+                               const smx_opt_params* adam, void* workspace, size_t workspace_bytes,
+                               const void* fwd_codes, size_t fwd_codes_bytes) {
+  if (parts < 1 || parts > 3) return smx::fail(SMX_ERR_ARG, "backward parts must be 1, 2 or 3");
+  return smx::backward_fused(parts, model, stream, plan, table, n_rows, idx, q1, q2, score, gscore, gq1, gq2, B, K, dim,
+                             params, merged, m, v, adam, workspace, workspace_bytes, fwd_codes, fwd_codes_bytes);
 }
 
 }  // extern "C"

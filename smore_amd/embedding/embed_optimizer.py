@@ -9,6 +9,7 @@ building the [B,K,row] tensor.  Everything after loss.backward() -- unique-merge
 (embed_optimizer.py:39-42), segment sum of gradient rows (:45-48) and the lazy Adam update
 (:208-252) -- runs as the segment plan and the fused entity pass of libsmore_amd.so.
 """
+import warnings
 from abc import ABC, abstractmethod
 
 import torch
@@ -117,9 +118,14 @@ class EmbeddingOptimizer(ABC):
             raise _lib.SmxError("the entity table must live on the GPU (no CPU-table mode in this build)")
         self.err_flag = fused.new_error_flag(sp_embed.embedding.device)
         self.check_ids_every_step = True
+        self.check_ids_synchronously = False   # True: every apply_grad waits for the device and raises for its own step
         self._flag_host = torch.zeros(1, dtype=torch.int32, pin_memory=True)   # where the flag of a step lands
         self._flag_event = None                                                # set while such a copy is under way
         self.lazy_lookup = True
+        self.stats = self._new_stats()
+        self._warned_fallback = False
+        # saving the table (state_dict of the SparseEmbedding) is one of the moments a pending id error must surface
+        sp_embed.register_state_dict_pre_hook(lambda module, prefix, keep_vars: self.poll_pending_id_check())
         self.prepare_state()
 
     # -- set-up protocol of the trainer (embed_optimizer.py:71-75, 102-110; called as
@@ -157,11 +163,31 @@ class EmbeddingOptimizer(ABC):
         """Same for several fused records of one query batch; plan covers their ids in the order of recs, then
         the ids of grad_rows (gradient rows of the step's plain lookups), when there are any."""
 
+    # -- what happened since zero_grad(): how the step's lookups were served
+    @staticmethod
+    def _new_stats():
+        """fused_launches: launches of the gather-fused scorer.  materialized_lookups: plain lookups made for a lazy
+        handle (anchors and other uses of the rows themselves; also every fallback).  dense_fallbacks: logits of a
+        handle that were evaluated by lookup + dense operators because the fused scorer has no form for them.
+        per_record_merges: fused records that apply_grad had to reduce to gradient rows one by one."""
+        return dict(fused_launches=0, materialized_lookups=0, dense_fallbacks=0, per_record_merges=0)
+
+    def note_dense_fallback(self, what):
+        """Called by the lazy handle when a logit leaves the fused path; says so once per optimizer."""
+        self.stats["dense_fallbacks"] += 1
+        if not self._warned_fallback:
+            self._warned_fallback = True
+            warnings.warn(f"smore_amd: {what} is evaluated by plain lookup + dense operators, not by the gather-fused "
+                          "scorer (correct results, several times the memory traffic); EmbeddingOptimizer.stats counts "
+                          "such steps", RuntimeWarning, stacklevel=3)
+
     # -- protocol of the training loop
     def zero_grad(self):
+        self.poll_pending_id_check()
         self.grad_list, self.fused_list, self.has_grad_list = [], [], []
         self.pending_scores = []
         self.n_fwd = 0
+        self.stats = self._new_stats()
 
     def share_memory(self):
         pass  # state is device memory of one process
@@ -188,9 +214,11 @@ class EmbeddingOptimizer(ABC):
             return LazyRows(self, indices, name)
         return self.lookup_rows(indices, name)
 
-    def lookup_rows(self, indices, name=None):
+    def lookup_rows(self, indices, name=None, for_handle=False):
         """rows = table[indices], shaped indices.shape + (row,), through the autograd node that records the
         gradient rows for apply_grad (EmbedLookupFunc, embed_optimizer.py:51-66)."""
+        if for_handle:
+            self.stats["materialized_lookups"] += 1
         mat = EmbedLookupFunc.apply(self, self.dummy_tensor, indices, name)
         if indices.dim() != 1:
             mat = mat.view(tuple(indices.shape) + (mat.shape[-1],))
@@ -290,6 +318,7 @@ class EmbeddingOptimizer(ABC):
         q1c = q1.reshape(b * branches, dim).contiguous()
         q2c = None if q2 is None else q2.reshape(b * branches, dim).contiguous()
         params = fused.score_params(gamma, cen, regularizer)
+        self.stats["fused_launches"] += 1
         logit = _FusedScoreFunc.apply(self, self.dummy_tensor, model, ids, params, q1c, q2c, torch.is_grad_enabled())
         return logit.view(b, branches, -1)
 
@@ -307,10 +336,10 @@ class EmbeddingOptimizer(ABC):
             self.err_flag.zero_()
         self._raise_for(code)
 
-    def _check_ids_one_step_late(self):
-        """The per-step check without draining the queue: this step's flag is copied to pinned host memory behind
-        the update, and looked at when the next step gets here -- by then the copy has long finished, so the host
-        keeps running ahead of the device."""
+    def poll_pending_id_check(self):
+        """Looks at the flag a finished step left in pinned host memory, if one is waiting (see
+        _check_ids_one_step_late), and raises for it.  Called wherever the next step, or the end of training, passes
+        by: apply_grad (also one that has nothing to apply), zero_grad, saving the table's state_dict."""
         if self._flag_event is not None:
             self._flag_event.synchronize()
             self._flag_event = None
@@ -318,6 +347,14 @@ class EmbeddingOptimizer(ABC):
             if code != 0:
                 self.err_flag.zero_()
                 self._raise_for(code)
+
+    def _check_ids_one_step_late(self):
+        """The per-step check without draining the queue: this step's flag is copied to pinned host memory behind
+        the update, and looked at when the next step gets here -- by then the copy has long finished, so the host
+        keeps running ahead of the device.  The step that met the bad id has by then scored row 0 in its place: its
+        loss and the gradients of the dense parameters are those of a wrong lookup (no table row was updated for
+        the bad id).  check_ids() after the step, or check_ids_synchronously = True, fails before anything uses them."""
+        self.poll_pending_id_check()
         self._flag_host.copy_(self.err_flag, non_blocking=True)
         self._flag_event = torch.cuda.Event()
         self._flag_event.record()
@@ -330,9 +367,12 @@ class EmbeddingOptimizer(ABC):
         self.step += 1  # counts calls, also those without gradients (embed_optimizer.py:156)
         self.pending_scores = []    # logits that nothing used have no gradient and must not ride along later
         if not self.grad_list and not self.fused_list:
+            self.poll_pending_id_check()
             return
         self._apply_grad(lr)
-        if self.check_ids_every_step:
+        if self.check_ids_synchronously:
+            self.check_ids()
+        elif self.check_ids_every_step:
             self._check_ids_one_step_late()
 
     def _apply_grad(self, lr):
@@ -361,6 +401,7 @@ class EmbeddingOptimizer(ABC):
                 self.update_fused_multi(plan, recs, lr, grad_rows=rows)
                 return
             table = self.sparse_embed.embedding.detach()
+            self.stats["per_record_merges"] += len(self.fused_list)
             for rec in self.fused_list:  # reduce each fused record to (distinct ids, summed rows) first
                 plan = fused.build_plan(rec["ids"], n_rows, err_flag=self.err_flag)
                 merged = torch.empty((plan.n_uniq, table.shape[1]), dtype=torch.float32, device=table.device)

@@ -88,12 +88,38 @@ class _Delegating:
     __rmul__ = _binary("mul", True)
     __truediv__ = _binary("div")
     __rtruediv__ = _binary("div", True)
+    __floordiv__ = _binary("floor_divide")
+    __rfloordiv__ = _binary("floor_divide", True)
+    __mod__ = _binary("remainder")
+    __rmod__ = _binary("remainder", True)
     __matmul__ = _binary("matmul")
+    __rmatmul__ = _binary("matmul", True)
     __pow__ = _binary("pow")
+    __rpow__ = _binary("pow", True)
+    __and__ = _binary("bitwise_and")
+    __rand__ = _binary("bitwise_and", True)
+    __or__ = _binary("bitwise_or")
+    __ror__ = _binary("bitwise_or", True)
+    __xor__ = _binary("bitwise_xor")
+    __rxor__ = _binary("bitwise_xor", True)
     __lt__ = _binary("lt")
     __le__ = _binary("le")
     __gt__ = _binary("gt")
     __ge__ = _binary("ge")
+    # comparisons give a tensor, as they do for the tensor the handle stands for (object identity otherwise);
+    # a class that defines __eq__ loses the inherited __hash__: handles stay hashable by identity
+    __eq__ = _binary("eq")
+    __ne__ = _binary("ne")
+    __hash__ = object.__hash__
+
+    def __setitem__(self, key, value):
+        self.materialize()[key] = _resolve(value)
+
+    def __invert__(self):
+        return ~self.materialize()
+
+    def __pos__(self):
+        return +self.materialize()
 
     def __neg__(self):
         return -self.materialize()
@@ -246,7 +272,7 @@ class LazyRows(_Delegating):
         and prologue this handle carries, as torch operations."""
         root = self.root
         if root._looked_up is None:
-            root._looked_up = self.opt.lookup_rows(self.ids, self.name)
+            root._looked_up = self.opt.lookup_rows(self.ids, self.name, for_handle=True)
         rows = root._looked_up.view(self.shape)
         if self.pending_add is not None:
             rows = rows + self.pending_add
@@ -398,6 +424,10 @@ class LazyLogit(_Delegating):
             d = self.terms[0][1]
             value = d.rows.opt.score_lazy(model, d.rows, d.queries, self.const, cen)
         if value is None:      # not a shape the fused scorer takes: plain lookup + dense operators
+            note = getattr(self.terms[0][1].rows.opt, "note_dense_fallback", None)
+            if note is not None:
+                note("a logit of " + " / ".join(sorted({d.kind for _, d in self.terms})) +
+                     f" on rows {tuple(self.terms[0][1].rows.shape)}")
             value = self.const
             for k, d in self.terms:
                 value = value + k * d.dense()

@@ -279,12 +279,14 @@ def score_backward_entity_multi(model, plan, table, q1, q2, sources, params, mer
 
 
 def score_backward_fused(model, plan, table, idx, q1, q2, score, gscore, params, merged=None, m=None, v=None,
-                         adam=None, sign_codes=True, codes=None):
+                         adam=None, sign_codes=True, codes=None, measure_parts=None):
     """Query gradients and all entity rows of the step in one call (see smx_score_backward_fused).
     Returns (gq1, gq2); merged / table, m, v are written in place as in score_backward_entity.
     codes: the buffer score_forward filled for these pairs (table and queries unchanged since).
     sign_codes=False gives the call only the entity pass's own workspace, which keeps the box model on
-    the path that re-reads the query rows (same results; for tests and comparison)."""
+    the path that re-reads the query rows (same results; for tests and comparison).
+    measure_parts (1 or 2; benchmarks only): launch one half of the call through the measuring entry point
+    smx_measure_backward_fused (include/smx_measure.h); the step such a call leaves is incomplete."""
     b, k, dim = _dims(model, table, idx, q1, q2)
     for t, name in ((score, "score"), (gscore, "gscore"), (merged, "merged"), (m, "m"), (v, "v")):
         _f32(t, name)
@@ -301,7 +303,8 @@ def score_backward_fused(model, plan, table, idx, q1, q2, score, gscore, params,
             _lib.load().smx_entity_workspace_bytes(plan.n_pairs, table.shape[1])
         ws = _workspace(ws_bytes, table.device)
         view = plan.view()
-        _lib.call("smx_score_backward_fused", MODELS[model], _stream(table), ctypes.byref(view), _ptr(table),
+        entry = ("smx_score_backward_fused",) if measure_parts is None else ("smx_measure_backward_fused", measure_parts)
+        _lib.call(*entry, MODELS[model], _stream(table), ctypes.byref(view), _ptr(table),
                   table.shape[0], _ptr(idx), _ptr(q1), _ptr(q2), _ptr(score), _ptr(gscore), _ptr(gq1), _ptr(gq2),
                   b, k, dim, ctypes.byref(params), _ptr(merged), _ptr(m), _ptr(v),
                   None if adam is None else ctypes.byref(adam), _ptr(ws), ws.numel(),

@@ -27,6 +27,17 @@ def test_header_symbols_are_exported_and_bound():
     assert sorted(_lib.SIGNATURES) == names
 
 
+def test_measuring_entry_points_stay_out_of_the_drop_in_header():
+    """include/smx_measure.h: exported by the same library, bound by the ctypes table of their own, absent from
+    smore_amd.h."""
+    from smore_amd import _lib
+    names = _declared("smx_measure.h")
+    assert names == sorted(_lib.MEASURE_SIGNATURES) and not set(names) & set(_declared())
+    lib = ctypes.CDLL(_lib.LIB_PATH)
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in smx_measure.h but not exported"
+
+
 def test_probe_library_exports_its_header():
     """The benchmark's bandwidth probes live in a library of their own, outside the drop-in ABI."""
     from smore_amd import _lib
@@ -46,7 +57,7 @@ def test_host_only_entry_points():
     assert lib.smx_kind_from_name(b"beta_fisher_approx") == 9
     assert lib.smx_kind_from_name(b"nope") == -1
     assert lib.smx_set_option(_lib.OPTION_SERIAL_BACKWARD, 0) == 0 and lib.smx_set_option(99, 1) != 0
-    assert lib.smx_set_option(_lib.OPTION_BACKWARD_PARTS, 3) == 0 and lib.smx_set_option(_lib.OPTION_BACKWARD_PARTS, 0) != 0
+    assert lib.smx_set_option(2, 1) != 0, "the drop-in ABI has no switch that leaves a partial step behind"
     import ctypes as c
     opt = _lib.OptParams(1e-3, 0.9, 0.999, 1e-8, 2, _lib.OPT_KINDS["adam"], 0, None)
     out = (c.c_float * 2)()

@@ -25,7 +25,7 @@ class RecordingOptimizer:
         self.sparse_embed = types.SimpleNamespace(embedding=table, dummy_job=types.SimpleNamespace(sync=lambda: None))
         self.scored, self.looked_up, self.pending_scores = [], [], []
 
-    def lookup_rows(self, ids, name=None):
+    def lookup_rows(self, ids, name=None, for_handle=False):
         self.looked_up.append(name)
         return self.sparse_embed.embedding[ids]
 
@@ -331,3 +331,29 @@ def test_a_handle_on_the_query_side_is_looked_up():
         assert opt.looked_up == ["negative_entity"]
         return
     assert torch.allclose(got, want, atol=1e-5)
+
+
+def test_comparisons_and_the_rarer_operators_give_what_the_tensor_gives():
+    """`rows == 0`, `logit != x` with a Python scalar must be elementwise tensors, not object identity; the
+    operators a handle has no lazy form for (%, **, &, item assignment) compute on the rows it stands for."""
+    n, d, b, k = 20, 4, 2, 3
+    opt = RecordingOptimizer(n, d)
+    ids = torch.randint(0, n, (b * k,), generator=torch.Generator().manual_seed(11))
+    rows = LazyRows(opt, ids, "negative_entity")
+    table = opt.sparse_embed.embedding
+    want = table[ids]
+    assert torch.equal(rows == 0, want == 0) and torch.equal(rows != 0.25, want != 0.25)
+    assert torch.equal(0.0 == rows, want == 0.0) and torch.equal(rows == want, torch.ones_like(want, dtype=torch.bool))
+    assert torch.equal(rows % 0.3, want % 0.3) and torch.equal(2.0 ** rows, 2.0 ** want)
+    assert torch.equal(rows // 0.3, want // 0.3) and torch.equal(+rows, want)
+    assert torch.equal((rows > 0) & (rows < 1), (want > 0) & (want < 1))
+    assert torch.equal((rows > 0) | (rows < -1), (want > 0) | (want < -1))
+    assert isinstance(hash(rows), int) and len({rows: 1}) == 1        # still usable as a dictionary key
+    (c,) = _queries(b, 1, d, 1, 12)
+    logit = 12.0 - ext_ops.l1_dist(LazyRows(opt, ids, None).view(b, k, -1), c)
+    value = logit.materialize()
+    assert torch.equal(logit == value, torch.ones_like(value, dtype=torch.bool))
+    assert torch.equal(logit != 12.0, value != 12.0)
+    copy = LazyRows(opt, ids, None)
+    copy[0] = 0.0                                                       # writes into the looked-up rows
+    assert float(copy.materialize()[0].abs().sum()) == 0.0
