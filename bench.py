@@ -68,6 +68,11 @@ CONFIGS = {
             zipf=None, adam=False),
     5: dict(name="cfg5-box-adam-86m-zipf1.1", model="box", n=86_054_151, dim=200, b=4096, k=1024, r=0.07, gamma=24.0,
             cen=0.02, zipf=1.1, adam=True, lr=1e-4),
+    # not one of BASELINE.json's configurations: the layout the reference's own training scripts run
+    # (training/box_scripts/train_freebase.sh: -n 1024 -d 400 --share_negative, optim_mode (aggr,adam,cpu,True,5)):
+    # K negatives shared by the batch, one positive per query, is_negative_mat mask, squeezed second moment
+    6: dict(name="cfg6-box-shared-negatives-20m", model="box", n=20_000_000, dim=400, b=512, k=1024, r=0.035, gamma=24.0,
+            cen=0.02, zipf=None, adam=True, lr=5e-5, shared=True),
 }
 
 
@@ -337,6 +342,109 @@ def dropin_bench(cfg, device, seed, steps, warmup):
     opt.check_ids()
     print(json.dumps({"workload": cfg["name"], "dropin_ms_per_step": out, "steps": steps, "warmup": warmup,
                       "pairs_per_step": b * k}))
+
+
+class SharedStep:
+    """One step of the shared-negative layout through the C calls: plan over [B positive ids | K shared ids],
+    positives scored per query, the K shared negatives scored by every query, query gradients of both, one gradient
+    row per shared list position (sum over all queries), then one entity pass over the plan that reduces the
+    positives' pairs and those rows and applies Adam (second moment one value per row)."""
+    PHASES = ("plan", "forward", "backward")
+
+    def __init__(self, cfg, table, q1, q2, pos, neg, gpos, gneg):
+        import torch
+        from smore_amd import fused
+        self.fused, self.torch, self.cfg = fused, torch, cfg
+        self.table, self.q1, self.q2, self.pos, self.neg, self.gpos, self.gneg = table, q1, q2, pos, neg, gpos, gneg
+        self.params = fused.score_params(cfg["gamma"], cfg["cen"])
+        self.m = torch.zeros_like(table)
+        self.v = torch.zeros(table.shape[0], device=table.device)
+        self.err = fused.new_error_flag(table.device)
+        self.all_ids = torch.cat([pos.reshape(-1), neg.reshape(-1)])
+        self.codes = fused.new_codes(cfg["model"], table, pos, q1)
+        self.step_no = 0
+        self.plan = None
+
+    def run(self, events=None, step_consts=None):
+        f, cfg = self.fused, self.cfg
+        mark = (lambda i: events[i].record()) if events is not None else (lambda i: None)
+        self.step_no += 1
+        mark(0)
+        plan = f.build_plan(self.all_ids, cfg["n"], err_flag=self.err)
+        mark(1)
+        sp = f.score_forward(cfg["model"], self.table, self.pos, self.q1, self.q2, self.params, self.err, codes=self.codes)
+        sn = f.score_forward_shared(cfg["model"], self.table, self.neg, self.q1, self.q2, self.params, self.err)
+        mark(2)
+        gp = f.score_backward_query(cfg["model"], self.table, self.pos, self.q1, self.q2, sp, self.gpos, self.params,
+                                    codes=self.codes)
+        gn = f.score_backward_query_shared(cfg["model"], self.table, self.neg, self.q1, self.q2, sn, self.gneg, self.params)
+        rows = f.score_backward_entity_shared(cfg["model"], self.table, self.neg, self.q1, self.q2, sn, self.gneg,
+                                              self.params)
+        f.score_backward_entity_multi(cfg["model"], plan, self.table, self.q1, self.q2, [(sp, self.gpos, self.codes)],
+                                      self.params, m=self.m, v=self.v,
+                                      adam=f.adam_params(cfg["lr"], self.step_no, squeeze=True, step_consts=step_consts),
+                                      grad_rows=rows)
+        mark(3)
+        self.plan = plan
+        return sn, (gp, gn)
+
+
+def shared_step_bench(cfg, device, seed, steps, warmup, graph):
+    """bench.py --config 6: the shared-negative step (see SharedStep), eager and replayed from a HIP graph."""
+    import torch
+    gen = torch.Generator(device=device)
+    gen.manual_seed(seed)
+    n, dim, b, k, r = cfg["n"], cfg["dim"], cfg["b"], cfg["k"], cfg["r"]
+    table = torch.empty((n, dim), device=device).uniform_(-r, r, generator=gen)
+    q1 = torch.empty((b, dim), device=device).uniform_(-r, r, generator=gen)
+    q2 = torch.empty((b, dim), device=device).uniform_(-r, r, generator=gen).abs_()
+    pos = torch.randint(0, n, (b, 1), device=device, generator=gen)
+    neg = torch.randint(0, n, (k,), device=device, generator=gen)
+    mask = (torch.rand((b, k), device=device, generator=gen) > 0.01).float()      # is_negative_mat
+    gneg = torch.randn((b, k), device=device, generator=gen) * mask
+    gpos = torch.randn((b, 1), device=device, generator=gen)
+    step = SharedStep(cfg, table, q1, q2, pos, neg, gpos, gneg)
+    for _ in range(warmup):
+        step.run()
+    torch.cuda.synchronize()
+    if step.err.item() != 0:
+        sys.exit("a warm-up step reported an error")
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(steps)]
+    t0 = time.perf_counter()
+    for s in range(steps):
+        step.run(ev[s])
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    if step.err.item() != 0:
+        sys.exit("a timed step reported an error")
+    ms = wall * 1e3 / steps
+    phase_ms = {name: sum(e[i].elapsed_time(e[i + 1]) for e in ev) / steps for i, name in enumerate(SharedStep.PHASES)}
+    per_step = sorted(e[0].elapsed_time(e[3]) for e in ev)
+    pairs = b * (k + 1)
+    n_uniq = step.plan.n_uniq
+    rl = dim
+    # compulsory traffic: every distinct row once forward and once backward, the optimizer's read + write of w and m
+    # (v is one float per row), ids, scores and upstream gradients of every pair, queries read twice and written once
+    algo = 4 * rl * 2 * n_uniq + 4 * 4 * rl * n_uniq + 8 * n_uniq + (k + b) * 8 + pairs * 8 + 3 * 4 * b * dim * 2
+    graph_ms = time_graph_replays(step, steps, warmup) if graph else None
+    out = {
+        "metric": "scored (query,neg) pairs/sec fwd+bwd+opt; achieved HBM GB/s vs peak",
+        "value": pairs / (ms * 1e-3), "unit": "pairs/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+        "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": cfg["name"], "N": n, "row_len": rl, "B": b, "K": k, "ids": "K negatives shared by the batch "
+                   "(uniform) + one positive per query", "mask": "is_negative_mat folded into the upstream gradient",
+                   "optimizer": "sparse adam, squeezed second moment", "seed": seed, "distinct_ids": n_uniq},
+        "phase_ms": phase_ms,
+        "step_ms_events": {"median": per_step[len(per_step) // 2], "min": per_step[0], "max": per_step[-1]},
+        "step_hbm": {"algorithmic_bytes": algo, "achieved_GBps": algo / (ms * 1e-3) / 1e9,
+                     "frac_of_peak": algo / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+                     "note": "the step touches K + B rows: it is bound by kernel latencies and VALU work on L2-resident "
+                             "operands, not by HBM"},
+    }
+    if graph_ms is not None:
+        out["graph_replay"] = {"ms_per_step": graph_ms, "value": pairs / (graph_ms * 1e-3), "unit": "pairs/s"}
+    print(json.dumps(out))
 
 
 def cpu_baseline(cfg, seed):
@@ -613,6 +721,9 @@ def main():
         return
     if args.dropin:
         dropin_bench(cfg, device, seed, args.steps, args.warmup)
+        return
+    if cfg.get("shared"):
+        shared_step_bench(cfg, device, seed, args.steps, args.warmup, args.graph)
         return
 
     if args.serial_backward:

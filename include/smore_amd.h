@@ -164,7 +164,10 @@ int smx_score_backward_query(int model, void* stream, const float* table, size_t
  * Ids outside [0, n_rows) set *err_flag = 1 and sort behind every valid id as one last segment that is not
  * counted in n_uniq, is skipped by the entity pass and is never a one-pair segment: no row is updated for
  * them (inverse[] holds n_uniq for such pairs).  *err_flag = 2: a workgroup of the sort gave up waiting for
- * another one (bounded wait, never seen in practice); the plan must then not be used. */
+ * another one (bounded wait, never seen in practice); *n_uniq is then -1, and every entry point that is handed
+ * such a plan does nothing (its kernels look at n_uniq before anything else of the plan).
+ * Up to 4096 ids are sorted by one workgroup in one launch (the ids of a step whose negatives are shared by the
+ * batch: K + B + anchors); the workspace is not used then. */
 size_t smx_plan_workspace_bytes(size_t n_pairs, size_t n_rows);
 int smx_plan_build(void* stream, const int64_t* idx, size_t n_pairs, size_t n_rows, void* workspace,
                    size_t workspace_bytes, int32_t* order, int32_t* sorted_ids, int32_t* seg_of_pos,
@@ -309,6 +312,40 @@ int smx_score_backward_fused(int model, void* stream, const smx_plan_view* plan,
 int smx_rows_backward(void* stream, const smx_plan_view* plan, const float* grad_rows,
                       size_t row_len, float* merged, float* table, float* m, float* v,
                       const smx_opt_params* adam, void* workspace, size_t workspace_bytes);
+
+/* ---- negatives shared by the whole batch ------------------------------------------------------
+ * Every training script of the reference runs with --share_negative: the sampler draws ONE list of K negative
+ * ids per batch (smore/cpp_sampler/online_sampler.py:155-157), the model looks those K rows up once and scores
+ * them against every query -- entity [1,K,row] against query [B,1,dim] (smore/models/kg_reasoning.py:349-355) --
+ * and is_negative_mat masks the pairs that are true answers (smore/training/train_process.py:195-196; the mask
+ * multiplies the logits, so it reaches the backward folded into gscore).  These entry points are the gather-fused
+ * forms of that layout: ids [K] int64, score / gscore [B,K]; nothing of size B*K is built besides the logits.
+ *   smx_score_forward_shared          score[b,k] = logit(table[ids[k]], q[b])       (as smx_score_forward)
+ *   smx_score_backward_query_shared   gq1, gq2 [B,dim]                              (as smx_score_backward_query)
+ *   smx_score_backward_entity_shared  the gradient of list position k is the sum over all B queries of
+ *                                     d(gscore[b,k] * score[b,k]) / d row, summed in a fixed order (b ascending
+ *                                     per wavefront, wavefronts in order), then
+ *     plan == NULL: written to grad_rows[k,:] ([K, dim*mul]; the model's hook and the clamp mask of the entity
+ *                   prologue applied -- what autograd hands EmbedLookupFunc.backward for the [1,K,row] lookup,
+ *                   embed_optimizer.py:63-66).  The caller merges these rows with the step's other index streams:
+ *                   grad_rows of smx_score_backward_entity_multi, or smx_rows_backward.
+ *     plan != NULL: a plan built by smx_plan_build over exactly these K ids.  One result per DISTINCT id (a list
+ *                   that holds an id twice sums both positions): merged[u,:] and / or the optimizer update of
+ *                   table, m, v in place, as smx_score_backward_entity.
+ * Replaces dist_forward / dist_backward in the [1,K] x [B,1] layout (common_kernel.h:33-123) plus gather,
+ * merge_grad_* and update_step as listed at smx_score_backward_entity. */
+int smx_score_forward_shared(int model, void* stream, const float* table, size_t n_rows, const int64_t* ids,
+                             const float* q1, const float* q2, float* score, size_t B, size_t K, size_t dim,
+                             const smx_score_params* params, int* err_flag);
+int smx_score_backward_query_shared(int model, void* stream, const float* table, size_t n_rows, const int64_t* ids,
+                                    const float* q1, const float* q2, const float* score, const float* gscore,
+                                    float* gq1, float* gq2, size_t B, size_t K, size_t dim,
+                                    const smx_score_params* params);
+int smx_score_backward_entity_shared(int model, void* stream, float* table, size_t n_rows, const int64_t* ids,
+                                     const float* q1, const float* q2, const float* score, const float* gscore,
+                                     size_t B, size_t K, size_t dim, const smx_score_params* params,
+                                     const smx_plan_view* plan, float* grad_rows, float* merged, float* m, float* v,
+                                     const smx_opt_params* adam);
 
 /* ---- sample loss ---------------------------------------------------------------------------
  * The loss between the scoring forward and its backward (smore/training/train_process.py:194-213)

@@ -25,6 +25,19 @@ int smx_measure_backward_fused(int parts, int model, void* stream, const smx_pla
                                const smx_opt_params* adam, void* workspace, size_t workspace_bytes,
                                const void* fwd_codes, size_t fwd_codes_bytes);
 
+/* No counterpart in the reference.  smx_plan_build with the two knobs a test needs to see a plan give up while
+ * every kernel still ends normally:
+ *   spin_limit    polls a workgroup of the sort makes before it stops waiting for another one (the library
+ *                 uses 2^22); 0 makes a workgroup give up the first time it would have to wait
+ *   force_abort   != 0: the build starts with its "a workgroup gave up" word already set, so every pass leaves
+ *                 without writing (also for inputs small enough for the one-workgroup build)
+ * A build that gave up leaves *err_flag = 2 and *n_uniq = -1; the kernels that read a plan look at n_uniq first
+ * and do nothing for such a plan. */
+int smx_measure_plan_build(void* stream, const int64_t* idx, size_t n_pairs, size_t n_rows, void* workspace,
+                           size_t workspace_bytes, int32_t* order, int32_t* sorted_ids, int32_t* seg_of_pos,
+                           int64_t* uniq, int32_t* seg_start, int64_t* inverse, int32_t* pair_seg, int32_t* n_uniq,
+                           int* err_flag, unsigned spin_limit, int force_abort);
+
 #ifdef __cplusplus
 }
 #endif

@@ -36,6 +36,13 @@ SIGNATURES = {
     # model, stream, table, n_rows, idx, q1, q2, score, gscore, gq1, gq2, B, K, dim, params, fwd_codes, bytes
     "smx_score_backward_query": (_i, [_i, _vp, _vp, _sz, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _vp, _vp,
                                       _sz]),
+    # model, stream, table, n_rows, ids, q1, q2, score, B, K, dim, params, err_flag
+    "smx_score_forward_shared": (_i, [_i, _vp, _vp, _sz, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _vp, _vp]),
+    # model, stream, table, n_rows, ids, q1, q2, score, gscore, gq1, gq2, B, K, dim, params
+    "smx_score_backward_query_shared": (_i, [_i, _vp, _vp, _sz, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _vp]),
+    # model, stream, table, n_rows, ids, q1, q2, score, gscore, B, K, dim, params, plan, grad_rows, merged, m, v, adam
+    "smx_score_backward_entity_shared": (_i, [_i, _vp, _vp, _sz, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _vp, _vp, _vp,
+                                              _vp, _vp, _vp, _vp]),
     "smx_plan_workspace_bytes": (_sz, [_sz, _sz]),
     # stream, idx, n_pairs, n_rows, ws, ws_bytes, order, sorted_ids, seg_of_pos, uniq, seg_start, inverse, pair_seg,
     # n_uniq, err
@@ -113,6 +120,8 @@ class SmxError(RuntimeError):
 MEASURE_SIGNATURES = {
     # parts, then the arguments of smx_score_backward_fused
     "smx_measure_backward_fused": (_i, [_i] + SIGNATURES["smx_score_backward_fused"][1]),
+    # the arguments of smx_plan_build, then spin_limit, force_abort
+    "smx_measure_plan_build": (_i, SIGNATURES["smx_plan_build"][1] + [_c.c_uint, _i]),
 }
 
 

@@ -343,6 +343,7 @@ __global__ __launch_bounds__(256) void entity_segment_kernel(EntityArgs A) {
   const int n_waves = gridDim.x * 4;
   const int n_chunks = (A.n_pairs + 63) / 64;
   const int n_valid = *A.n_uniq;  // a last segment beyond this one holds the pairs whose id is outside the table: skipped
+  if (n_valid < 0) return;  // the plan's build gave up: nothing of it may be read
   const bool mixed = SRC != kSrcRows && A.rows_first < A.n_pairs;  // the plan also holds gradient rows of plain lookups
 
   for (int chunk = blockIdx.x * 4 + wave; chunk < n_chunks; chunk += n_waves) {
@@ -436,6 +437,7 @@ __global__ __launch_bounds__(256) void entity_tile_kernel(EntityArgs A) {
   if (p0 >= A.n_pairs) return;  // whole wavefront leaves; no workgroup barrier is used below
   const int p1 = min(A.n_pairs, p0 + A.tile);
   const int n_valid = *A.n_uniq;  // the segment of ids outside the table, if there is one, is number n_valid: skipped
+  if (n_valid < 0) return;  // the plan's build gave up: nothing of it may be read
   const bool mixed = SRC != kSrcRows && A.rows_first < A.n_pairs;  // the plan also holds gradient rows of plain lookups
   {  // does a long segment that came in from the left end inside this tile?  The fix-up pass finishes it.
     const int sg = A.seg_of_pos[p0];
@@ -791,6 +793,7 @@ __global__ __launch_bounds__(256) void entity_segment_coded_kernel(EntityArgs A)
   const int n_waves = gridDim.x * 4;
   const int n_chunks = (A.n_pairs + 63) / 64;
   const int n_valid = *A.n_uniq;  // a last segment beyond this one holds the pairs whose id is outside the table: skipped
+  if (n_valid < 0) return;  // the plan's build gave up: nothing of it may be read
   const bool mixed = A.rows_first < A.n_pairs;  // the plan also holds gradient rows of plain lookups
 
   for (int chunk = blockIdx.x * 4 + wave; chunk < n_chunks; chunk += n_waves) {
@@ -887,6 +890,7 @@ __global__ __launch_bounds__(256, 4) void entity_tile_coded_kernel(EntityArgs A)
   if (p0 >= A.n_pairs) return;  // whole wavefront leaves; no workgroup barrier is used below
   const int p1 = min(A.n_pairs, p0 + kTile);
   const int n_valid = *A.n_uniq;  // the segment of ids outside the table, if there is one, is number n_valid: skipped
+  if (n_valid < 0) return;  // the plan's build gave up: nothing of it may be read
   const bool mixed = A.rows_first < A.n_pairs;
 
   int sg[TW], b0[TW], b1[TW], id[TW];

@@ -28,6 +28,7 @@
 #include <cstring>
 #include <mutex>
 
+#include "../../include/smx_measure.h"
 #include "smx_common.h"
 
 namespace smx {
@@ -54,13 +55,14 @@ __device__ __forceinline__ void st_agent(unsigned* p, unsigned v) {
 }
 
 // Waits until the word at p carries the ready flag; v is what was last read there.  Bounded: after
-// kSpinLimit polls the caller gets a ready word with count 0 and the plan is marked invalid.
-__device__ __forceinline__ unsigned wait_ready(const unsigned* p, unsigned v, unsigned* abort_flag, int* err) {
+// spin_limit polls the caller gets a ready word with count 0 and the plan is marked invalid.
+__device__ __forceinline__ unsigned wait_ready(const unsigned* p, unsigned v, unsigned* abort_flag, int* err,
+                                               unsigned spin_limit) {
   unsigned spins = 0;
   while (!(v & kReady)) {
     __builtin_amdgcn_s_sleep(1);
     v = ld_agent(p);
-    if (++spins > kSpinLimit) {
+    if (++spins > spin_limit) {
       st_agent(abort_flag, 1u);
       if (err) *err = 2;
       return kReady;
@@ -136,14 +138,18 @@ __global__ __launch_bounds__(kAuxThreads) void sort_hist_kernel(const long long*
                                                                 unsigned long long n_rows, int passes, int dbits,
                                                                 unsigned* __restrict__ block_hist,
                                                                 unsigned* __restrict__ zero_from, size_t zero_words,
-                                                                int* __restrict__ pair_seg, int* err) {
+                                                                int* __restrict__ pair_seg, int* err,
+                                                                unsigned* abort_word, unsigned abort_init,
+                                                                int* __restrict__ n_uniq) {
   extern __shared__ unsigned lds_hist[];  // [passes][bins]
   const int bins = 1 << dbits;
   const unsigned mask = (unsigned)bins - 1u;
   const int lane = threadIdx.x & 63;
   for (int i = threadIdx.x; i < passes * bins; i += kAuxThreads) lds_hist[i] = 0;
   for (size_t i = (size_t)blockIdx.x * kAuxThreads + threadIdx.x; i < zero_words; i += (size_t)gridDim.x * kAuxThreads)
-    zero_from[i] = 0;
+    zero_from[i] = &zero_from[i] == abort_word ? abort_init : 0u;  // (abort_init != 0: a test asks for a plan that gives up)
+  // n_uniq ends as the smallest value anybody writes: the number of distinct ids, or -1 from a workgroup that gave up
+  if (blockIdx.x == 0 && threadIdx.x == 0) *n_uniq = 0x7fffffff;
   __syncthreads();
   int bad = 0;
   const size_t span = (size_t)kAuxThreads * kHistBatch;
@@ -232,6 +238,7 @@ struct SortPassArgs {
   unsigned* abort_flag;
   unsigned long long n_rows;
   int* err;
+  unsigned spin_limit;
 };
 
 // Digits are owned by threads: thread t owns digit t (and t + threads when there are more digits
@@ -349,7 +356,7 @@ __global__ __launch_bounds__(NW * 64, (MAXR <= 8 ? 8 : 4)) void sort_pass_kernel
         unsigned here = 0;
 #pragma unroll
         for (int j = 0; j < kGroup - 1; ++j) {
-          if (first + j < unit) v[j] = wait_ready(tab + (size_t)(first + j) * bins, v[j], A.abort_flag, A.err);
+          if (first + j < unit) v[j] = wait_ready(tab + (size_t)(first + j) * bins, v[j], A.abort_flag, A.err, A.spin_limit);
           here += v[j] & kCount;
         }
         before += here;
@@ -363,7 +370,7 @@ __global__ __launch_bounds__(NW * 64, (MAXR <= 8 ? 8 : 4)) void sort_pass_kernel
       }
       if (tile >= 4096u) {
         const unsigned* p = &A.pre[(size_t)(tile / 4096u - 1) * bins + d];
-        before += wait_ready(p, ld_agent(p), A.abort_flag, A.err) & kCount;
+        before += wait_ready(p, ld_agent(p), A.abort_flag, A.err, A.spin_limit) & kCount;
       }
       if ((tile & 4095u) == 4095u) st_agent(&A.pre[(size_t)(tile / 4096u) * bins + d], ((before + mine[u]) & kCount) | kReady);
       local_base[d] = lb[u];
@@ -424,6 +431,7 @@ struct EmitArgs {
   unsigned* ticket;
   unsigned* abort_flag;
   int* err;
+  unsigned spin_limit;
 };
 
 // Consecutive lanes own consecutive sorted positions (kEmitIters rows of 1024 per tile).  Segment
@@ -492,7 +500,7 @@ __global__ __launch_bounds__(kAuxThreads) void plan_emit_kernel(EmitArgs A) {
 #pragma unroll
     for (int u = 0; u < kEmitSuper / 64; ++u) {
       const int j = (int)tile - 1 - lane - 64 * u;
-      if (j >= first) v[u] = wait_ready(&A.agg[j], v[u], A.abort_flag, A.err);
+      if (j >= first) v[u] = wait_ready(&A.agg[j], v[u], A.abort_flag, A.err, A.spin_limit);
       sum += v[u] & kCount;
     }
 #pragma unroll
@@ -500,7 +508,7 @@ __global__ __launch_bounds__(kAuxThreads) void plan_emit_kernel(EmitArgs A) {
     if (lane == 0) {
       if (first > 0) {
         const unsigned* p = &A.pre[first / kEmitSuper - 1];
-        sum += wait_ready(p, ld_agent(p), A.abort_flag, A.err) & kCount;
+        sum += wait_ready(p, ld_agent(p), A.abort_flag, A.err, A.spin_limit) & kCount;
       }
       if ((tile & (kEmitSuper - 1)) == kEmitSuper - 1) st_agent(&A.pre[tile / kEmitSuper], ((sum + total) & kCount) | kReady);
       tmp[21] = sum;
@@ -508,7 +516,13 @@ __global__ __launch_bounds__(kAuxThreads) void plan_emit_kernel(EmitArgs A) {
     }
   }
   __syncthreads();
-  if (tmp[22]) return;  // a tile gave up waiting: segment numbers are not trustworthy, write nothing
+  if (tmp[22]) {  // a tile gave up waiting: segment numbers are not trustworthy, write nothing but "no plan"
+    if (tid == 0) {
+      atomicMin(A.n_uniq, -1);  // every kernel that reads the plan looks at this first and leaves
+      if (A.err) *A.err = 2;
+    }
+    return;
+  }
   const unsigned first_seg = tmp[21];
 
 #pragma unroll
@@ -526,9 +540,77 @@ __global__ __launch_bounds__(kAuxThreads) void plan_emit_kernel(EmitArgs A) {
       if (A.pair_seg && ((singles >> it) & 1u)) A.pair_seg[A.order[p]] = seg | (int)0x80000000;  // sign bit + segment number
       if (p == n - 1) {  // the last position closes the list
         A.seg_start[seg + 1] = (int)n;
-        *A.n_uniq = seg + 1 - ((unsigned long long)key[it] >= A.n_rows ? 1 : 0);  // ids outside the table are not counted
+        atomicMin(A.n_uniq, seg + 1 - ((unsigned long long)key[it] >= A.n_rows ? 1 : 0));  // ids outside the table are not counted
       }
     }
+  }
+}
+
+
+// ---- small inputs: the whole plan in one launch ---------------------------------------------------
+// A step whose negatives are shared by the batch sorts K + B (+ anchors) ids, a couple of thousand: six dependent
+// launches would cost more than the work.  One workgroup sorts (id, position) as 64-bit keys in LDS (bitonic
+// network; the keys are distinct, so the order is the stable order by id) and writes every array of the plan.
+constexpr int kSmallPlanMax = 4096;
+
+__global__ __launch_bounds__(kAuxThreads) void plan_small_kernel(const long long* __restrict__ idx, int n, int n_pow2,
+                                                                 unsigned long long n_rows, int* __restrict__ order,
+                                                                 unsigned* __restrict__ sorted_ids,
+                                                                 int* __restrict__ seg_of_pos, long long* __restrict__ uniq,
+                                                                 int* __restrict__ seg_start, long long* __restrict__ inverse,
+                                                                 int* __restrict__ pair_seg, int* __restrict__ n_uniq,
+                                                                 int* err) {
+  extern __shared__ unsigned long long small_keys[];  // [n_pow2]
+  __shared__ unsigned tmp[32];
+  const int tid = threadIdx.x;
+  int bad = 0;
+  for (int i = tid; i < n_pow2; i += kAuxThreads)
+    small_keys[i] = i < n ? (((unsigned long long)clamp_id(idx[i], n_rows, bad) << 32) | (unsigned)i) : ~0ull;
+  if (bad && err) *err = 1;
+  __syncthreads();
+  for (int k = 2; k <= n_pow2; k <<= 1) {
+    for (int j = k >> 1; j > 0; j >>= 1) {
+      for (int t = tid; t < n_pow2 / 2; t += kAuxThreads) {
+        const int i = ((t & ~(j - 1)) << 1) | (t & (j - 1));  // the t-th index whose bit j is clear
+        const unsigned long long a = small_keys[i], b = small_keys[i | j];
+        const bool up = (i & k) == 0;
+        if ((a > b) == up) {
+          small_keys[i] = b;
+          small_keys[i | j] = a;
+        }
+      }
+      __syncthreads();
+    }
+  }
+  // segment heads and numbers, 1024 sorted positions at a time
+  unsigned carry = 0;
+  for (int base = 0; base < n; base += kAuxThreads) {
+    const int p = base + tid;
+    const bool in = p < n;
+    const unsigned long long el = in ? small_keys[p] : 0ull;
+    const unsigned key = (unsigned)(el >> 32);
+    const int pair = (int)(unsigned)el;
+    const bool head = in && (p == 0 || (unsigned)(small_keys[p - 1] >> 32) != key);
+    const bool last_of_seg = in && (p == n - 1 || (unsigned)(small_keys[p + 1] >> 32) != key);
+    unsigned total = 0;
+    const unsigned before = block_excl_scan<kAuxWaves>(head ? 1u : 0u, tmp, &total);
+    if (in) {
+      const int seg = (int)(carry + before + (head ? 1u : 0u)) - 1;
+      order[p] = pair;
+      sorted_ids[p] = key;
+      seg_of_pos[p] = seg;
+      if (head) {
+        uniq[seg] = (long long)key;
+        seg_start[seg] = p;
+      }
+      if (inverse) inverse[pair] = seg;
+      if (pair_seg) pair_seg[pair] = (head && last_of_seg && (unsigned long long)key < n_rows) ? (seg | (int)0x80000000) : 0;
+      if (p == n - 1) {
+        seg_start[seg + 1] = n;
+        *n_uniq = seg + 1 - ((unsigned long long)key >= n_rows ? 1 : 0);  // ids outside the table are not counted
+      }
+    }
+    carry += total;
   }
 }
 
@@ -668,14 +750,29 @@ size_t smx_plan_workspace_bytes(size_t n_pairs, size_t n_rows) {
   return smx::plan_layout(n_pairs, n_rows).total;
 }
 
-int smx_plan_build(void* stream, const int64_t* idx, size_t n_pairs, size_t n_rows, void* workspace,
-                   size_t workspace_bytes, int32_t* order, int32_t* sorted_ids, int32_t* seg_of_pos, int64_t* uniq,
-                   int32_t* seg_start, int64_t* inverse, int32_t* pair_seg, int32_t* n_uniq, int* err_flag) {
-  using namespace smx;
+}  // extern "C"
+
+namespace smx {
+
+// spin_limit, force_abort: kSpinLimit and 0 for every caller but the measuring entry point
+static int plan_build(void* stream, const int64_t* idx, size_t n_pairs, size_t n_rows, void* workspace,
+                      size_t workspace_bytes, int32_t* order, int32_t* sorted_ids, int32_t* seg_of_pos, int64_t* uniq,
+                      int32_t* seg_start, int64_t* inverse, int32_t* pair_seg, int32_t* n_uniq, int* err_flag,
+                      unsigned spin_limit, int force_abort) {
   if (!idx || !order || !sorted_ids || !seg_of_pos || !uniq || !seg_start || !n_uniq || !workspace)
     return fail(SMX_ERR_ARG, "null pointer in plan build");
   if (n_pairs == 0 || n_pairs > 0x7fffffffull) return fail(SMX_ERR_SHAPE, "pair count %zu out of range", n_pairs);
   if (n_rows == 0 || n_rows > 0xffffffffull) return fail(SMX_ERR_SHAPE, "entity count %zu needs ids wider than 32 bits", n_rows);
+  if (n_pairs <= (size_t)kSmallPlanMax && !force_abort) {
+    int n_pow2 = 64;
+    while ((size_t)n_pow2 < n_pairs) n_pow2 *= 2;
+    hipLaunchKernelGGL(plan_small_kernel, dim3(1), dim3(kAuxThreads), (size_t)n_pow2 * sizeof(unsigned long long),
+                       as_stream(stream), reinterpret_cast<const long long*>(idx), (int)n_pairs, n_pow2,
+                       (unsigned long long)n_rows, order, reinterpret_cast<unsigned*>(sorted_ids), seg_of_pos,
+                       reinterpret_cast<long long*>(uniq), seg_start, reinterpret_cast<long long*>(inverse), pair_seg,
+                       n_uniq, err_flag);
+    return check_launch("plan build (one workgroup)");
+  }
   const PlanLayout L = plan_layout(n_pairs, n_rows);
   if (workspace_bytes < L.total)
     return fail(SMX_ERR_WORKSPACE, "plan workspace too small: %zu < %zu", workspace_bytes, L.total);
@@ -693,7 +790,8 @@ int smx_plan_build(void* stream, const int64_t* idx, size_t n_pairs, size_t n_ro
 
   hipLaunchKernelGGL(sort_hist_kernel, dim3((unsigned)L.hist_blocks), dim3(kAuxThreads),
                      (size_t)L.passes * L.bins * sizeof(unsigned), st, reinterpret_cast<const long long*>(idx), n,
-                     (unsigned long long)n_rows, L.passes, L.dbits, block_hist, zeroed, L.zero_words, pair_seg, err_flag);
+                     (unsigned long long)n_rows, L.passes, L.dbits, block_hist, zeroed, L.zero_words, pair_seg, err_flag,
+                     zeroed + L.abort_w, force_abort ? 1u : 0u, n_uniq);
   hipLaunchKernelGGL(sort_sum_kernel, dim3((unsigned)(L.passes * ((L.bins + 63) / 64))), dim3(kAuxThreads), 0, st, block_hist,
                      L.hist_blocks, L.passes, L.dbits, digit_count);
   for (int s = 0; s < L.passes; ++s) {
@@ -717,6 +815,7 @@ int smx_plan_build(void* stream, const int64_t* idx, size_t n_pairs, size_t n_ro
     A.abort_flag = zeroed + L.abort_w;
     A.n_rows = (unsigned long long)n_rows;
     A.err = err_flag;
+    A.spin_limit = spin_limit;
     launch_pass_nw<kSortWaves>(st, L, A, first, last);
     if (int rc = check_launch("radix pass")) return rc;
   }
@@ -736,8 +835,28 @@ int smx_plan_build(void* stream, const int64_t* idx, size_t n_pairs, size_t n_ro
   E.ticket = zeroed + L.ticket_w + L.passes;
   E.abort_flag = zeroed + L.abort_w;
   E.err = err_flag;
+  E.spin_limit = spin_limit;
   hipLaunchKernelGGL(plan_emit_kernel, dim3((unsigned)L.emit_tiles), dim3(kAuxThreads), 0, st, E);
   return check_launch("plan build");
+}
+
+}  // namespace smx
+
+extern "C" {
+
+int smx_plan_build(void* stream, const int64_t* idx, size_t n_pairs, size_t n_rows, void* workspace,
+                   size_t workspace_bytes, int32_t* order, int32_t* sorted_ids, int32_t* seg_of_pos, int64_t* uniq,
+                   int32_t* seg_start, int64_t* inverse, int32_t* pair_seg, int32_t* n_uniq, int* err_flag) {
+  return smx::plan_build(stream, idx, n_pairs, n_rows, workspace, workspace_bytes, order, sorted_ids, seg_of_pos, uniq,
+                         seg_start, inverse, pair_seg, n_uniq, err_flag, smx::kSpinLimit, 0);
+}
+
+int smx_measure_plan_build(void* stream, const int64_t* idx, size_t n_pairs, size_t n_rows, void* workspace,
+                           size_t workspace_bytes, int32_t* order, int32_t* sorted_ids, int32_t* seg_of_pos,
+                           int64_t* uniq, int32_t* seg_start, int64_t* inverse, int32_t* pair_seg, int32_t* n_uniq,
+                           int* err_flag, unsigned spin_limit, int force_abort) {
+  return smx::plan_build(stream, idx, n_pairs, n_rows, workspace, workspace_bytes, order, sorted_ids, seg_of_pos, uniq,
+                         seg_start, inverse, pair_seg, n_uniq, err_flag, spin_limit, force_abort);
 }
 
 

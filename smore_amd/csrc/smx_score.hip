@@ -197,6 +197,39 @@ int smx_score_backward_query(int model, void* stream, const float* table, size_t
   return dispatch_model(model, as_stream(stream), A, vec, nit, false);
 }
 
+int smx_score_forward_shared(int model, void* stream, const float* table, size_t n_rows, const int64_t* ids,
+                             const float* q1, const float* q2, float* score, size_t B, size_t K, size_t dim,
+                             const smx_score_params* params, int* err_flag) {
+  using namespace smx;
+  ScoreArgs A;
+  int vec, nit;
+  if (!ids) return fail(SMX_ERR_ARG, "null id list");
+  if (int rc = fill_args(&A, &vec, &nit, model, table, n_rows, ids, q1, q2, B, K, dim, params, nullptr, nullptr)) return rc;
+  if (!score) return fail(SMX_ERR_ARG, "null score pointer");
+  A.ids_shared = 1;
+  A.score_out = score;
+  A.err = err_flag;
+  return dispatch_model(model, as_stream(stream), A, vec, nit, true);
+}
+
+int smx_score_backward_query_shared(int model, void* stream, const float* table, size_t n_rows, const int64_t* ids,
+                                    const float* q1, const float* q2, const float* score, const float* gscore,
+                                    float* gq1, float* gq2, size_t B, size_t K, size_t dim,
+                                    const smx_score_params* params) {
+  using namespace smx;
+  ScoreArgs A;
+  int vec, nit;
+  if (!ids) return fail(SMX_ERR_ARG, "null id list");
+  if (int rc = fill_args(&A, &vec, &nit, model, table, n_rows, ids, q1, q2, B, K, dim, params, nullptr, nullptr)) return rc;
+  if (!score || !gscore || !gq1 || (model_nq(model) == 2 && !gq2)) return fail(SMX_ERR_ARG, "null pointer");
+  A.ids_shared = 1;
+  A.score = score;
+  A.gscore = gscore;
+  A.gq1 = gq1;
+  A.gq2 = gq2;
+  return dispatch_model(model, as_stream(stream), A, vec, nit, false);
+}
+
 int smx_score_backward_entity(int model, void* stream, const smx_plan_view* plan, float* table, size_t n_rows,
                               const float* q1, const float* q2, const float* score, const float* gscore, size_t B,
                               size_t K, size_t dim, const smx_score_params* params, float* merged, float* m, float* v,

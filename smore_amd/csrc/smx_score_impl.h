@@ -35,6 +35,7 @@ struct ScoreArgs {
   float* gq1;
   float* gq2;
   int B, K, ncol;
+  int ids_shared;        // idx holds K ids that every query scores (--share_negative, online_sampler.py:155-157), not B*K
   int id_bits;           // significant bits of n_rows - 1 (at most 32): what the forward compares to find equal ids
   unsigned long long n_rows;
   ScoreParams p;
@@ -274,7 +275,7 @@ __global__ __launch_bounds__(256) void score_forward_kernel(ScoreArgs A, int til
   const int cnt = min(per_wave, K - kw0);
   int bad = 0;
   PairBatch pb{0u, 0u};
-  if (cnt > 0) pb = load_pair_batch(idx, (size_t)b * K + kw0, cnt, lane, row_len, n_rows, bad);
+  if (cnt > 0) pb = load_pair_batch(idx, (A.ids_shared ? (size_t)0 : (size_t)b * K) + kw0, cnt, lane, row_len, n_rows, bad);
 
   stage_query<M>(lds, q1, q2, b, dim);
   typename ModelOps<M>::Q q[NIT][VEC];
@@ -440,7 +441,7 @@ __global__ __launch_bounds__(NW * 64) void score_backward_query_kernel(ScoreArgs
     }
     PairBatch pb;
     if constexpr (GQ) {
-      pb = load_pair_batch(idx, first, cnt, lane, row_len, n_rows, bad);
+      pb = load_pair_batch(idx, A.ids_shared ? (size_t)kb : first, cnt, lane, row_len, n_rows, bad);
     } else {
       if (singles == 0ull) continue;  // wave-uniform
       const unsigned long long row = my_ps < 0 ? (unsigned long long)A.uniq[my_ps & 0x7fffffff] : 0ull;
@@ -662,7 +663,8 @@ int launch_forward_reg(hipStream_t st, const ScoreArgs& A) {
   const size_t lds = ((size_t)model_nq(M) * A.ncol * VEC + 4 * kSlabDwords) * sizeof(float);
   // ids given (not the dense layout, whose rows are all different): score each distinct entity of a
   // wavefront's batch once
-  const bool dedup = A.idx != nullptr;
+  // (not for a list of ids shared by the batch: a sampler's K negatives hardly ever repeat)
+  const bool dedup = A.idx != nullptr && !A.ids_shared;
   if constexpr (model_coded(M) && !REG) {
     if (A.codes) {
       if (dedup)

@@ -63,11 +63,17 @@ class _FusedScoreFunc(torch.autograd.Function):
     @staticmethod
     def forward(ctx, embed_opt, dummy_tensor, model, ids, params, q1, q2, for_training=True):
         table = embed_opt.sparse_embed.embedding.detach()
+        # ids [1, K] against more than one query: negatives shared by the batch (--share_negative); they stay K ids
+        ctx.shared = ids.shape[0] == 1 and q1.shape[0] > 1
         with torch.no_grad():
-            # box, l1: the forward leaves 2-bit sign codes from which both backward passes work (None otherwise;
-            # none either when no backward will follow, e.g. scoring sampled negatives under torch.no_grad())
-            codes = fused.new_codes(model, table, ids, q1) if for_training and table.shape[1] % 4 == 0 else None
-            score = fused.score_forward(model, table, ids, q1, q2, params, embed_opt.err_flag, codes=codes)
+            if ctx.shared:
+                codes = None
+                score = fused.score_forward_shared(model, table, ids.reshape(-1), q1, q2, params, embed_opt.err_flag)
+            else:
+                # box, l1: the forward leaves 2-bit sign codes from which both backward passes work (None otherwise;
+                # none either when no backward will follow, e.g. scoring sampled negatives under torch.no_grad())
+                codes = fused.new_codes(model, table, ids, q1) if for_training and table.shape[1] % 4 == 0 else None
+                score = fused.score_forward(model, table, ids, q1, q2, params, embed_opt.err_flag, codes=codes)
         ctx.embed_opt, ctx.model, ctx.ids, ctx.params, ctx.codes = embed_opt, model, ids, params, codes
         ctx.save_for_backward(q1.detach(), q2.detach() if q2 is not None else None, score)
         ctx.idx_fwd = embed_opt.n_fwd
@@ -81,9 +87,14 @@ class _FusedScoreFunc(torch.autograd.Function):
         table = opt.sparse_embed.embedding.detach()
         with torch.no_grad():
             gscore = gscore.contiguous()
-            gq1, gq2 = fused.score_backward_query(ctx.model, table, ctx.ids, q1, q2, score, gscore, ctx.params,
-                                                  codes=ctx.codes)
-        opt.accumulate_fused(ctx.model, ctx.ids, q1, q2, score, gscore, ctx.params, ctx.idx_fwd, ctx.codes)
+            if ctx.shared:
+                gq1, gq2 = fused.score_backward_query_shared(ctx.model, table, ctx.ids.reshape(-1), q1, q2, score,
+                                                             gscore, ctx.params)
+            else:
+                gq1, gq2 = fused.score_backward_query(ctx.model, table, ctx.ids, q1, q2, score, gscore, ctx.params,
+                                                      codes=ctx.codes)
+        opt.accumulate_fused(ctx.model, ctx.ids, q1, q2, score, gscore, ctx.params, ctx.idx_fwd, ctx.codes,
+                             shared=ctx.shared)
         return None, None, None, None, None, gq1, gq2, None
 
 
@@ -159,6 +170,10 @@ class EmbeddingOptimizer(ABC):
         """Same for one fused record whose entity gradient is recomputed on the fly."""
 
     @abstractmethod
+    def update_shared(self, plan, rec, lr):
+        """Same for one fused record whose K ids are shared by all its queries; plan covers those K ids."""
+
+    @abstractmethod
     def update_fused_multi(self, plan, recs, lr, grad_rows=None):
         """Same for several fused records of one query batch; plan covers their ids in the order of recs, then
         the ids of grad_rows (gradient rows of the step's plain lookups), when there are any."""
@@ -196,9 +211,9 @@ class EmbeddingOptimizer(ABC):
         self.grad_list.append((indices, grad_submat))
         self.has_grad_list.append(fwd_idx)
 
-    def accumulate_fused(self, model, ids, q1, q2, score, gscore, params, fwd_idx, codes=None):
+    def accumulate_fused(self, model, ids, q1, q2, score, gscore, params, fwd_idx, codes=None, shared=False):
         self.fused_list.append(dict(model=model, ids=ids, q1=q1, q2=q2, score=score, gscore=gscore, params=params,
-                                    codes=codes, fwd_idx=fwd_idx))
+                                    codes=codes, fwd_idx=fwd_idx, shared=shared))
         self.has_grad_list.append(fwd_idx)
 
     def forward(self, indices, name=None):
@@ -271,22 +286,28 @@ class EmbeddingOptimizer(ABC):
                  same(p.request["q1"], w["q1"]) and same(p.request["q2"], w["q2"])]
         if not any(p is wanted for p in group):
             group.append(wanted)
-        ids = [p.request["ids"].to(self.sparse_embed.embedding.device) for p in group]
-        if len(group) > 1:      # ids shared by the batch ([1, K]) stand beside per-query ones as [B, K]
-            ids = [i.expand(w["b"], i.shape[1]) if i.shape[0] == 1 else i for i in ids]
-        all_ids = ids[0] if len(ids) == 1 else torch.cat(ids, dim=1)
-        logit = self._score_branches(w["model"], all_ids, w["q1"], w["q2"], w["gamma"], w["cen"], w["reg"])
-        if logit.shape[1] == 1:
-            values, index = logit[:, 0], None
-        else:                   # union branches: the first maximal one, as torch.max(logit, dim=1) in the model code
-            values, index = torch.max(logit, dim=1)
-        sizes = [i.shape[1] for i in ids]
-        parts = [values] if len(ids) == 1 else torch.split(values, sizes, dim=1)
-        iparts = [index] * len(ids) if (index is None or len(ids) == 1) else torch.split(index, sizes, dim=1)
-        for p, part, ipart in zip(group, parts, iparts):
-            # (each caller gets a tensor of its own layout, as torch.max would have returned it: .view() works)
-            p._value = part.contiguous()
-            p._index = None if ipart is None else ipart.contiguous()
+        dev = self.sparse_embed.embedding.device
+        # ids shared by the batch ([1, K], --share_negative) go into a launch of their own, K ids long; the per-query
+        # ones ([B, K_i]) stand side by side in another
+        shared = [p for p in group if p.request["ids"].shape[0] == 1 and w["b"] > 1]
+        own = [p for p in group if not (p.request["ids"].shape[0] == 1 and w["b"] > 1)]
+        for part in (own, shared):
+            if not part:
+                continue
+            ids = [p.request["ids"].to(dev) for p in part]
+            all_ids = ids[0] if len(ids) == 1 else torch.cat(ids, dim=1)
+            logit = self._score_branches(w["model"], all_ids, w["q1"], w["q2"], w["gamma"], w["cen"], w["reg"])
+            if logit.shape[1] == 1:
+                values, index = logit[:, 0], None
+            else:               # union branches: the first maximal one, as torch.max(logit, dim=1) in the model code
+                values, index = torch.max(logit, dim=1)
+            sizes = [i.shape[1] for i in ids]
+            parts = [values] if len(ids) == 1 else torch.split(values, sizes, dim=1)
+            iparts = [index] * len(ids) if (index is None or len(ids) == 1) else torch.split(index, sizes, dim=1)
+            for p, val, ipart in zip(part, parts, iparts):
+                # (each caller gets a tensor of its own layout, as torch.max would have returned it: .view() works)
+                p._value = val.contiguous()
+                p._index = None if ipart is None else ipart.contiguous()
         self.pending_scores = [r for r in self.pending_scores if r() is not None and r()._value is None]
 
     def score_negatives(self, model, ids, q1, q2=None, gamma=0.0, cen=0.0, regularizer=None):
@@ -310,9 +331,11 @@ class EmbeddingOptimizer(ABC):
         ids = ids.to(table.device)
         if ids.dim() != 2:
             raise _lib.SmxError("ids must be [B,K] or [1,K]")
-        if ids.shape[0] == 1 and b > 1:
-            ids = ids.expand(b, ids.shape[1])
-        if branches > 1:  # every branch of a query scores that query's negatives
+        if ids.shape[0] == 1 and b * branches > 1:
+            pass                # shared by the batch: every query row (every branch of every query) scores the same K ids
+        elif ids.shape[0] != b:
+            raise _lib.SmxError("ids must be [B,K] or [1,K]")
+        elif branches > 1:      # every branch of a query scores that query's negatives
             ids = ids.repeat_interleave(branches, dim=0)
         ids = ids.contiguous()
         q1c = q1.reshape(b * branches, dim).contiguous()
@@ -377,11 +400,15 @@ class EmbeddingOptimizer(ABC):
 
     def _apply_grad(self, lr):
         n_rows = self.sparse_embed.num_rows
+        table = self.sparse_embed.embedding.detach()
         with torch.no_grad():
             if len(self.fused_list) == 1 and not self.grad_list:
                 rec = self.fused_list[0]
                 plan = fused.build_plan(rec["ids"], n_rows, err_flag=self.err_flag)
-                self.update_fused(plan, rec, lr)
+                if rec["shared"]:
+                    self.update_shared(plan, rec, lr)
+                else:
+                    self.update_fused(plan, rec, lr)
                 return
             idx_list = [i.reshape(-1).to(self.sparse_embed.device) for i, _ in self.grad_list]
             grad_list = [g.reshape(g.shape[0] if g.dim() == 2 else -1, g.shape[-1]).contiguous().float()
@@ -389,24 +416,48 @@ class EmbeddingOptimizer(ABC):
             if self.fused_list and (len(self.fused_list) == 1 or self._one_query_batch(self.fused_list)):
                 # positives and negatives of one query batch (kg_reasoning.py:340-355): one plan over all their
                 # ids, one entity pass that reads each record's own scores / upstream gradients / sign codes.
-                # The step's plain lookups -- the anchor entities every query starts from (box.py:137), whose
-                # gradient rows autograd has materialised -- go behind them in the same plan: such a row is
-                # added to its entity's gradient when the entity's row is finished.
+                # Negatives shared by the batch bring one gradient row per list position (each the sum over all
+                # queries, formed by one workgroup per row) instead of B x K pairs.  Those rows, and the rows of the
+                # step's plain lookups -- the anchor entities every query starts from (box.py:137), whose gradient
+                # autograd has materialised -- go behind the pairs in the same plan: such a row is added to its
+                # entity's gradient when the entity's row is finished.
                 recs = sorted(self.fused_list, key=lambda r: r["fwd_idx"])   # forward order, whatever autograd's was
-                flat = torch.cat([r["ids"].reshape(-1) for r in recs] + idx_list, dim=0)
+                own = [r for r in recs if not r["shared"]]
+                shared = [r for r in recs if r["shared"]]
+                n_shared = sum(r["ids"].numel() for r in shared)
+                n_lookup = sum(g.shape[0] for g in grad_list)
                 rows = None
-                if grad_list:
+                if n_shared:
+                    rows = torch.empty((n_shared + n_lookup, table.shape[1]), dtype=torch.float32, device=table.device)
+                    at = 0
+                    for r in shared:
+                        k = r["ids"].numel()
+                        fused.score_backward_entity_shared(r["model"], table, r["ids"].reshape(-1), r["q1"], r["q2"],
+                                                           r["score"], r["gscore"], r["params"], grad_rows=rows[at:at + k])
+                        at += k
+                    for g in grad_list:
+                        rows[at:at + g.shape[0]].copy_(g)
+                        at += g.shape[0]
+                elif grad_list:
                     rows = grad_list[0] if len(grad_list) == 1 else torch.cat(grad_list, dim=0)
+                flat = torch.cat([r["ids"].reshape(-1) for r in own] + [r["ids"].reshape(-1) for r in shared] + idx_list,
+                                 dim=0)
                 plan = fused.build_plan(flat, n_rows, err_flag=self.err_flag)
-                self.update_fused_multi(plan, recs, lr, grad_rows=rows)
+                if own:
+                    self.update_fused_multi(plan, own, lr, grad_rows=rows)
+                else:
+                    self.update_from_plan(plan, rows, lr)
                 return
-            table = self.sparse_embed.embedding.detach()
             self.stats["per_record_merges"] += len(self.fused_list)
             for rec in self.fused_list:  # reduce each fused record to (distinct ids, summed rows) first
                 plan = fused.build_plan(rec["ids"], n_rows, err_flag=self.err_flag)
                 merged = torch.empty((plan.n_uniq, table.shape[1]), dtype=torch.float32, device=table.device)
-                fused.score_backward_entity(rec["model"], plan, table, rec["q1"], rec["q2"], rec["score"],
-                                            rec["gscore"], rec["params"], merged=merged, codes=rec["codes"])
+                if rec["shared"]:
+                    fused.score_backward_entity_shared(rec["model"], table, rec["ids"].reshape(-1), rec["q1"], rec["q2"],
+                                                       rec["score"], rec["gscore"], rec["params"], plan=plan, merged=merged)
+                else:
+                    fused.score_backward_entity(rec["model"], plan, table, rec["q1"], rec["q2"], rec["score"],
+                                                rec["gscore"], rec["params"], merged=merged, codes=rec["codes"])
                 idx_list.append(plan.uniq)
                 grad_list.append(merged)
             # (a single record is used as it is: torch.cat would copy its gradient rows)
@@ -415,12 +466,13 @@ class EmbeddingOptimizer(ABC):
             plan = fused.build_plan(flat, n_rows, err_flag=self.err_flag)
             self.update_from_plan(plan, rows.contiguous(), lr)
 
-
     @staticmethod
     def _one_query_batch(recs):
         """True when the fused records can share one entity pass: same model and score parameters, the same
-        query tensors (same memory, shape and version), sign codes for all or none, few enough of them."""
-        if not 2 <= len(recs) <= _lib.MAX_PAIR_SOURCES:
+        query tensors (same memory, shape and version), sign codes for all per-query records or for none, few
+        enough of those."""
+        own = [r for r in recs if not r["shared"]]
+        if len(recs) < 2 or len(own) > _lib.MAX_PAIR_SOURCES:
             return False
         first = recs[0]
 
@@ -432,9 +484,9 @@ class EmbeddingOptimizer(ABC):
         def same_params(a, b):
             return all(getattr(a, f) == getattr(b, f) for f, _ in a._fields_)
 
-        return all(r["model"] == first["model"] and same_params(r["params"], first["params"]) and
-                   same_tensor(r["q1"], first["q1"]) and same_tensor(r["q2"], first["q2"]) and
-                   (r["codes"] is None) == (first["codes"] is None) for r in recs[1:])
+        return (all(r["model"] == first["model"] and same_params(r["params"], first["params"]) and
+                    same_tensor(r["q1"], first["q1"]) and same_tensor(r["q2"], first["q2"]) for r in recs[1:]) and
+                all((r["codes"] is None) == (own[0]["codes"] is None) for r in own[1:]))
 
 
 class _RowOptimizer(EmbeddingOptimizer):
@@ -481,6 +533,12 @@ class _RowOptimizer(EmbeddingOptimizer):
         fused.score_backward_entity_multi(first["model"], plan, self.sparse_embed.embedding.detach(), first["q1"],
                                           first["q2"], [(r["score"], r["gscore"], r["codes"]) for r in recs],
                                           first["params"], m=m, v=v, adam=self._params(lr), grad_rows=grad_rows)
+
+    def update_shared(self, plan, rec, lr):
+        m, v = self._state()
+        fused.score_backward_entity_shared(rec["model"], self.sparse_embed.embedding.detach(), rec["ids"].reshape(-1),
+                                           rec["q1"], rec["q2"], rec["score"], rec["gscore"], rec["params"], plan=plan,
+                                           m=m, v=v, adam=self._params(lr))
 
     def update_fused(self, plan, rec, lr):
         m, v = self._state()

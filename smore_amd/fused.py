@@ -110,6 +110,80 @@ def score_backward_query(model, table, idx, q1, q2, score, gscore, params, codes
     return gq1, gq2
 
 
+def _shared_dims(model, table, ids, q1, q2):
+    if model not in MODELS:
+        raise _lib.SmxError(f"unknown score model {model}")
+    _f32(table, "table")
+    _f32(q1, "q1")
+    _f32(q2, "q2")
+    if (q2 is None) != (model in ONE_QUERY):
+        raise _lib.SmxError(f"model {model} takes {'one' if model in ONE_QUERY else 'two'} query tensor(s)")
+    mul = 2 if model in TWO_HALVES else 1
+    b, dim = q1.shape[0], q1.shape[-1]
+    if q1.numel() != b * dim or (q2 is not None and q2.shape != q1.shape):
+        raise _lib.SmxError("query tensors must be [B, dim] (or [B, 1, dim])")
+    if table.dim() != 2 or table.shape[1] != dim * mul:
+        raise _lib.SmxError(f"table row length {tuple(table.shape)} does not match dim {dim} x {mul}")
+    if ids.dtype != torch.int64 or not ids.is_contiguous() or ids.device != table.device or ids.numel() == 0:
+        raise _lib.SmxError("shared ids must be a contiguous int64 tensor [K] (or [1, K]) on the table's device")
+    return b, ids.numel(), dim
+
+
+def score_forward_shared(model, table, ids, q1, q2, params, err_flag=None):
+    """logit[b,k] = gamma - dist(table[ids[k]], q[b]) for K ids that every query scores (--share_negative)."""
+    b, k, dim = _shared_dims(model, table, ids, q1, q2)
+    score = torch.empty((b, k), dtype=torch.float32, device=table.device)
+    with torch.cuda.device(table.device):
+        _lib.call("smx_score_forward_shared", MODELS[model], _stream(table), _ptr(table), table.shape[0], _ptr(ids),
+                  _ptr(q1), _ptr(q2), _ptr(score), b, k, dim, ctypes.byref(params), _ptr(err_flag))
+    return score
+
+
+def score_backward_query_shared(model, table, ids, q1, q2, score, gscore, params):
+    """Gradients of sum(gscore * score) w.r.t. q1 (and q2) for shared ids."""
+    b, k, dim = _shared_dims(model, table, ids, q1, q2)
+    _f32(score, "score")
+    _f32(gscore, "gscore")
+    gq1 = torch.empty_like(q1)
+    gq2 = None if q2 is None else torch.empty_like(q2)
+    with torch.cuda.device(table.device):
+        _lib.call("smx_score_backward_query_shared", MODELS[model], _stream(table), _ptr(table), table.shape[0],
+                  _ptr(ids), _ptr(q1), _ptr(q2), _ptr(score), _ptr(gscore), _ptr(gq1), _ptr(gq2), b, k, dim,
+                  ctypes.byref(params))
+    return gq1, gq2
+
+
+def score_backward_entity_shared(model, table, ids, q1, q2, score, gscore, params, plan=None, grad_rows=None,
+                                 merged=None, m=None, v=None, adam=None):
+    """Entity side of shared ids (see smx_score_backward_entity_shared).  plan None: returns (and fills) grad_rows
+    [K, row], one gradient row per list position.  plan (built over exactly these ids): merged rows per distinct id
+    and / or the optimizer update of table, m, v in place."""
+    b, k, dim = _shared_dims(model, table, ids, q1, q2)
+    for t, name in ((score, "score"), (gscore, "gscore"), (grad_rows, "grad_rows"), (merged, "merged"), (m, "m"), (v, "v")):
+        _f32(t, name)
+    if score.shape != (b, k) or gscore.shape != (b, k):
+        raise _lib.SmxError("score and gscore must be [B, K]")
+    row_len = table.shape[1]
+    if plan is None:
+        if grad_rows is None:
+            grad_rows = torch.empty((k, row_len), dtype=torch.float32, device=table.device)
+        elif grad_rows.shape != (k, row_len):
+            raise _lib.SmxError("grad_rows must be [K, row]")
+    else:
+        if plan.n_pairs != k:
+            raise _lib.SmxError("the plan must be built over the shared ids")
+        _check_state(table, m, v, adam)
+        if merged is not None and (merged.dim() != 2 or merged.shape[1] != row_len):
+            raise _lib.SmxError("merged must be [n_uniq or more, row]")
+    with torch.cuda.device(table.device):
+        view = None if plan is None else plan.view()
+        _lib.call("smx_score_backward_entity_shared", MODELS[model], _stream(table), _ptr(table), table.shape[0],
+                  _ptr(ids), _ptr(q1), _ptr(q2), _ptr(score), _ptr(gscore), b, k, dim, ctypes.byref(params),
+                  None if view is None else ctypes.byref(view), _ptr(grad_rows), _ptr(merged), _ptr(m), _ptr(v),
+                  None if adam is None else ctypes.byref(adam))
+    return grad_rows
+
+
 def gather_rows(table, idx, err_flag=None):
     """rows = table[idx] (idx any shape, flattened) -> [idx.numel(), row]."""
     _f32(table, "table")
@@ -144,7 +218,10 @@ class SegmentPlan:
     def n_uniq(self):
         """Number of distinct ids (first use synchronises with the device)."""
         if self._n_uniq is None:
-            self._n_uniq = int(self.n_uniq_dev.item())
+            n = int(self.n_uniq_dev.item())
+            if n < 0:
+                raise _lib.SmxError("the segment plan is invalid (a sort workgroup gave up waiting)")
+            self._n_uniq = n
         return self._n_uniq
 
     @property
@@ -160,8 +237,9 @@ def _workspace(nbytes, device):
     return torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)
 
 
-def build_plan(idx, n_rows, want_inverse=False, err_flag=None):
-    """Sorts the pairs of idx (any shape, int64, device) by entity id; see SegmentPlan."""
+def build_plan(idx, n_rows, want_inverse=False, err_flag=None, measure=None):
+    """Sorts the pairs of idx (any shape, int64, device) by entity id; see SegmentPlan.
+    measure (tests only): (spin_limit, force_abort) for smx_measure_plan_build (include/smx_measure.h)."""
     if idx.dtype != torch.int64 or idx.device.type != "cuda":
         raise _lib.SmxError("idx must be an int64 device tensor")
     flat = idx.reshape(-1).contiguous()
@@ -172,9 +250,10 @@ def build_plan(idx, n_rows, want_inverse=False, err_flag=None):
         if nbytes == 0:
             raise _lib.SmxError("smx_plan_workspace_bytes failed")
         ws = _workspace(nbytes, flat.device)
-        _lib.call("smx_plan_build", _stream(flat), _ptr(flat), n, n_rows, _ptr(ws), ws.numel(), _ptr(plan.order),
+        entry, extra = ("smx_plan_build", ()) if measure is None else ("smx_measure_plan_build", tuple(measure))
+        _lib.call(entry, _stream(flat), _ptr(flat), n, n_rows, _ptr(ws), ws.numel(), _ptr(plan.order),
                   _ptr(plan.sorted_ids), _ptr(plan.seg_of_pos), _ptr(plan.uniq_buf), _ptr(plan.seg_start),
-                  _ptr(plan.inverse), _ptr(plan.pair_seg), _ptr(plan.n_uniq_dev), _ptr(err_flag))
+                  _ptr(plan.inverse), _ptr(plan.pair_seg), _ptr(plan.n_uniq_dev), _ptr(err_flag), *extra)
     return plan
 
 

@@ -426,11 +426,13 @@ def test_anchor_lookups_join_the_fused_records_in_one_update(name, monkeypatch):
         w = got.copy()   # continue from the device's fp32 weights so that step 2 compares one step, not two
 
 
-def test_shared_negatives_beside_positives_share_one_record():
+def test_shared_negatives_beside_positives_share_one_update():
     """--share_negative (online_sampler.py:155-157): negatives [1,K] for the whole batch, positives [B] per query,
-    both scored by unchanged model code against one branch of queries.  They wait for the loss together and
-    leave ONE record [B, 1 + K]; the is_negative_mat mask of train_process.py:195-196 multiplies the negative
-    logits.  Logits, query gradient and the Adam step against the oracle."""
+    both scored by unchanged model code against one branch of queries.  They leave two records with the optimizer
+    -- the positives' B pairs and the K shared ids, which are never expanded to [B, K] -- and apply_grad reduces
+    both behind ONE plan (an entity that is positive and shared negative gets one update); the is_negative_mat mask
+    of train_process.py:195-196 multiplies the negative logits.  Logits, query gradient and the Adam step against
+    the oracle."""
     from smore_amd.embedding.embed_optimizer import AdamEmbedOptimizer
     from smore_amd.embedding.sparse_embed import SparseEmbedding
     n, d, b, k, lr = 300, 16, 5, 12, 1e-3
@@ -458,8 +460,10 @@ def test_shared_negatives_beside_positives_share_one_record():
     ln = net.cal_logit(n_rows.view(1, k, -1), None, [tq])
     ln = ln * dev(mask)
     ((lp * dev(gp)).sum() + (ln * dev(gn)).sum()).backward()
-    assert len(opt.fused_list) == 1 and not opt.grad_list
+    assert sorted(tuple(r["ids"].shape) for r in opt.fused_list) == [(1, k), (b, 1)] and not opt.grad_list
+    assert opt.stats["materialized_lookups"] == 0 and opt.stats["dense_fallbacks"] == 0
     opt.apply_grad(lr)
+    assert opt.stats["per_record_merges"] == 0
 
     ids = np.concatenate([pos.reshape(b, 1), np.broadcast_to(neg, (b, k))], axis=1)
     rows = orc.gather(table, ids).reshape(b, 1 + k, d)

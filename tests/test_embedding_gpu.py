@@ -331,25 +331,40 @@ def test_out_of_range_lookup_is_reported():
         opt.check_ids()
 
 
-def test_out_of_range_id_in_a_step_raises_from_the_next_apply_grad():
-    """The per-step check does not wait for the device: the flag of step n is read when step n+1 reaches
-    apply_grad.  The bad pair itself updates no row (its key sorts behind every real segment)."""
+def test_out_of_range_id_in_a_step_raises_when_the_next_step_begins():
+    """The per-step check does not wait for the device: the flag of step n is read where step n+1 first passes by
+    -- its zero_grad (or an apply_grad without gradients, or saving the table).  The bad pair itself updates no row
+    (its key sorts behind every real segment)."""
     emb, opt = _setup(20, 8, 9)
     c = torch.zeros(2, 1, 8, device="cuda", requires_grad=True)
     o = torch.ones(2, 1, 8, device="cuda", requires_grad=True)
     w0 = emb.embedding.detach().clone()
-    for step, ids in enumerate(([[1, 25], [2, 3]], [[4, 5], [6, 7]])):
-        opt.zero_grad()
+
+    def step(ids):
         ln = opt.score_negatives("box", torch.tensor(ids, device="cuda"), c, o, gamma=1.0, cen=0.02)
         ln.sum().backward()
-        if step == 0:
-            opt.apply_grad(1e-3)
-        else:
-            with pytest.raises(IndexError):
-                opt.apply_grad(1e-3)
+        opt.apply_grad(1e-3)
+
+    opt.zero_grad()
+    step([[1, 25], [2, 3]])
+    with pytest.raises(IndexError):
+        opt.zero_grad()
+    opt.zero_grad()       # the flag was cleared when the error was raised
+    step([[4, 5], [6, 7]])
     changed = (emb.embedding.detach() != w0).any(dim=1).nonzero().flatten().tolist()
     assert changed == [1, 2, 3, 4, 5, 6, 7]
-    opt.check_ids()       # the flag was cleared when the error was raised
+    opt.check_ids()
+    # the other places a waiting flag is looked at: an apply_grad with nothing to apply, and saving the table
+    for look in (lambda: opt.apply_grad(1e-3), lambda: emb.state_dict()):
+        opt.zero_grad()
+        step([[1, 2], [3, 99]])
+        with pytest.raises(IndexError):
+            look()
+    # check_ids_synchronously: the step that met the id fails itself
+    opt.check_ids_synchronously = True
+    opt.zero_grad()
+    with pytest.raises(IndexError):
+        step([[1, 2], [3, 99]])
 
 
 def test_trainer_set_up_protocol_and_cpu_statistics_mode():

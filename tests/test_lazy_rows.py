@@ -208,8 +208,9 @@ def test_positives_and_negatives_of_one_query_batch_share_one_launch():
 
 
 def test_shared_negatives_wait_beside_per_query_positives():
-    """--share_negative gives negative ids [1,K] (online_sampler.py:155-157) next to positives [B]: in one request
-    the shared ids stand beside the per-query ones as [B, 1 + K]; alone they stay [1, K]."""
+    """--share_negative gives negative ids [1,K] (online_sampler.py:155-157) next to positives [B]: both wait for
+    the first use, then the per-query ids go into one launch and the shared ids, still K of them, into another
+    (never expanded to [B, K])."""
     n, d, b, k = 50, 8, 5, 7
     opt = RecordingOptimizer(n, d)
     gen = torch.Generator().manual_seed(4)
@@ -220,7 +221,7 @@ def test_shared_negatives_wait_beside_per_query_positives():
     ln = cal_logit(LazyRows(opt, neg.view(-1), "negative_entity").view(1, k, -1))
     assert lp.shape == (b, 1) and ln.shape == (b, k)
     total = lp.sum() + ln.sum()
-    assert opt.scored == [("l1", (b, 1 + k), 12.0, 0.0, None)]
+    assert opt.scored == [("l1", (b, 1), 12.0, 0.0, None), ("l1", (1, k), 12.0, 0.0, None)]
     table = opt.sparse_embed.embedding
     want = (12.0 - _textbook("l1", table[pos].unsqueeze(1), (q,), 0.0)).sum() + \
         (12.0 - _textbook("l1", table[neg].expand(b, k, d), (q,), 0.0)).sum()

@@ -1,0 +1,255 @@
+"""Negatives shared by the whole batch (--share_negative: ids [K] scored by every query, the is_negative_mat mask
+of train_process.py:195-196 folded into the upstream gradient) through the C ABI, against the CPU oracle; the
+one-workgroup segment plan those steps use; and a plan whose build gives up."""
+import types
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle as orc
+from tests.test_fused_gpu import GAMMA, dev, make_problem
+from tests.util import (REL_F32, assert_adam_weights, assert_close, oracle_adam_step, oracle_union_grads,
+                        oracle_union_logits, seed)
+
+pytestmark = pytest.mark.gpu
+
+SHAPES = [("box", 300, 9, 40, 48), ("l1", 200, 5, 17, 200), ("l2", 150, 6, 33, 36), ("rotate", 120, 7, 20, 500),
+          ("beta_kl", 100, 4, 24, 400), ("complex", 90, 3, 10, 64), ("distmult", 90, 8, 65, 30), ("box", 500, 70, 130, 400)]
+
+
+def _shared_problem(model, n, b, k, dim):
+    rng = np.random.default_rng(seed("shared", model, n, b, k, dim))
+    table, q1, q2, _, gs = make_problem(model, n, b, k, dim, rng)
+    ids = rng.integers(0, n, k)
+    ids[k // 2] = ids[0]                 # the list holds one entity twice: one update from both positions
+    mask = (rng.random((b, k)) > 0.2).astype(np.float64)   # is_negative_mat: true answers among the negatives drop out
+    return table, q1, q2, ids.astype(np.int64), gs * mask
+
+
+@pytest.mark.parametrize("model,n,b,k,dim", SHAPES)
+def test_shared_negatives_match_oracle_and_the_per_query_kernels(model, n, b, k, dim):
+    from smore_amd import fused
+    table, q1, q2, ids, gs = _shared_problem(model, n, b, k, dim)
+    reg = (1.0, 0.05, 1e9) if model == "beta_kl" else None      # BetaE's entity prologue rides along
+    cen = 0.02
+    params = fused.score_params(GAMMA[model], cen, reg)
+    if reg is not None:
+        table = table - 1.0 + np.where(np.arange(table.shape[1]) % 7 == 0, -0.99, 0.0)   # some values under the clamp
+        table = table.astype(np.float32).astype(np.float64)
+    t_table, t_q1, t_q2, t_gs = dev(table), dev(q1), dev(q2), dev(gs)
+    t_ids = torch.tensor(ids, device="cuda")
+    err = fused.new_error_flag("cuda")
+
+    score = fused.score_forward_shared(model, t_table, t_ids, t_q1, t_q2, params, err)
+    idx_full = np.broadcast_to(ids[None, :], (b, k))
+    qs = [q1[:, None, None, :]] + ([] if q2 is None else [q2[:, None, None, :]])
+    logit, rows = oracle_union_logits(model, table, idx_full, qs, GAMMA[model], cen, regularizer=reg is not None)
+    assert_close(score.cpu().numpy(), logit[:, 0], REL_F32, f"{model} shared score",
+                 rms_floor=model in ("beta_kl", "complex", "distmult"))
+    # the same kernel as the per-query layout, the ids addressed without the query number: same bits
+    t_full = torch.tensor(np.ascontiguousarray(idx_full), device="cuda")
+    assert torch.equal(score, fused.score_forward(model, t_table, t_full, t_q1, t_q2, params, err))
+    assert err.item() == 0
+
+    gq1, gq2 = fused.score_backward_query_shared(model, t_table, t_ids, t_q1, t_q2, score, t_gs, params)
+    g_rows, g_qs = oracle_union_grads(model, table, idx_full, qs, rows, logit, gs, cen, regularizer=reg is not None)
+    q_abs = None if model == "beta_kl" else np.abs(gs).sum(axis=1)[:, None] * np.ones((1, dim))
+    assert_close(gq1.cpu().numpy(), g_qs[0][:, 0, 0], REL_F32, f"{model} shared gq1", sum_abs=q_abs)
+    if q2 is not None:
+        assert_close(gq2.cpu().numpy(), g_qs[1][:, 0, 0], REL_F32, f"{model} shared gq2", sum_abs=q_abs)
+    f1, f2 = fused.score_backward_query(model, t_table, t_full, t_q1, t_q2, score, t_gs, params)
+    assert torch.equal(f1, gq1) and (f2 is None or torch.equal(f2, gq2))
+
+    # one gradient row per list position: the sum over all queries
+    want_rows = g_rows.reshape(b, k, -1).sum(axis=0)
+    abs_rows = np.abs(g_rows).reshape(b, k, -1).sum(axis=0)
+    got_rows = fused.score_backward_entity_shared(model, t_table, t_ids, t_q1, t_q2, score, t_gs, params)
+    assert_close(got_rows.cpu().numpy(), want_rows, REL_F32, f"{model} shared gradient rows", sum_abs=abs_rows)
+    assert torch.equal(t_table, dev(table)), "the table must not change without an optimizer"
+
+    # with the plan of the K ids: one merged row / one Adam update per distinct id
+    plan = fused.build_plan(t_ids, n, err_flag=err)
+    uniq, inverse, _, _ = orc.merge_indices(ids)
+    assert plan.n_uniq == uniq.size and np.array_equal(plan.uniq.cpu().numpy(), uniq)
+    merged = torch.full((uniq.size, table.shape[1]), float("nan"), device="cuda")
+    fused.score_backward_entity_shared(model, t_table, t_ids, t_q1, t_q2, score, t_gs, params, plan=plan, merged=merged)
+    o_merged = orc.merge_grads(want_rows, inverse, uniq.size)
+    assert_close(merged.cpu().numpy(), o_merged, REL_F32, f"{model} shared merged rows",
+                 sum_abs=orc.merge_grads(abs_rows, inverse, uniq.size))
+    lr = 1e-3
+    t_m, t_v = torch.zeros_like(t_table), torch.zeros_like(t_table)
+    fused.score_backward_entity_shared(model, t_table, t_ids, t_q1, t_q2, score, t_gs, params, plan=plan, m=t_m, v=t_v,
+                                       adam=fused.adam_params(lr, 1))
+    w, m, v, uniq2, merged2 = oracle_adam_step(table, [ids], [want_rows], lr, 1)
+    assert_close(t_m.cpu().numpy()[uniq], m[uniq], REL_F32, f"{model} shared first moment",
+                 sum_abs=0.1 * orc.merge_grads(abs_rows, inverse, uniq.size))
+    assert_adam_weights(t_table.cpu().numpy(), w, merged2, uniq, lr, f"{model} shared weights")
+    untouched = np.setdiff1d(np.arange(n), uniq)
+    assert np.array_equal(t_table.cpu().numpy()[untouched], table[untouched].astype(np.float32))
+    assert err.item() == 0
+
+
+def test_shared_negatives_next_to_positives_and_anchors_in_one_step():
+    """The step every shipped training script runs (kg_reasoning.py:298-355 with --share_negative): an anchor lookup
+    feeds the query, positives [B] and shared negatives [1,K] are scored against it, one apply_grad.  The shared ids
+    stay K ids all the way (no [B,K] id tensor exists), an entity that is anchor, positive and negative at once gets
+    ONE update; against the float64 oracle."""
+    from smore_amd.embedding.embed_optimizer import AdamEmbedOptimizer
+    from smore_amd.embedding.sparse_embed import SparseEmbedding
+    from smore_amd.torchext.ext_ops import box_dist_in, box_dist_out
+    n, d, b, k, lr, gamma, cen = 60, 48, 9, 21, 1e-3, 24.0, 0.02
+    rng = np.random.default_rng(5)
+    torch.manual_seed(3)
+    emb = SparseEmbedding(n, d).cuda()
+    emb.init_params(-0.07, 0.07)
+    opt = AdamEmbedOptimizer(types.SimpleNamespace(optim_mode="(aggr,adam,gpu,False,5)", share_optim_stats=True), emb, 0)
+    w0 = emb.embedding.detach().cpu().numpy().astype(np.float64)
+    anchor_n, pos_n, neg_n = rng.integers(0, n, b), rng.integers(0, n, b), rng.integers(0, n, (1, k))
+    rel_n = rng.uniform(-0.07, 0.07, (b, d)).astype(np.float32)
+    off_n = np.abs(rng.uniform(-0.07, 0.07, (b, d))).astype(np.float32)
+    mask_n = (rng.random((b, k)) > 0.3).astype(np.float32)
+    gp_n, gn_n = rng.standard_normal((b, 1)).astype(np.float32), rng.standard_normal((b, k)).astype(np.float32)
+    rel = torch.tensor(rel_n, device="cuda", requires_grad=True)
+    off = torch.tensor(off_n, device="cuda", requires_grad=True)
+    g = torch.nn.Parameter(torch.tensor([gamma], device="cuda"), requires_grad=False)
+    anchor, pos, neg = (torch.tensor(x, device="cuda") for x in (anchor_n, pos_n, neg_n))
+
+    def cal_logit(rows, center, offset):        # box.py:157-164
+        return torch.max(g - box_dist_out(rows, center, offset) - cen * box_dist_in(rows, center, offset), dim=1)[0]
+
+    opt.zero_grad()
+    a = emb(anchor, "anchor")
+    center = (a + rel).view(b, 1, 1, -1)
+    offset = off.view(b, 1, 1, -1)
+    lp = cal_logit(emb(pos, "positive_entity").unsqueeze(1), center, offset)
+    ln = cal_logit(emb(neg.view(-1), "negative_entity").view(1, k, -1), center, offset)
+    assert lp.shape == (b, 1) and ln.shape == (b, k)
+    ((ln * torch.tensor(mask_n, device="cuda")) * torch.tensor(gn_n, device="cuda")).sum().backward(retain_graph=True)
+    (lp * torch.tensor(gp_n, device="cuda")).sum().backward()
+    assert opt.stats["fused_launches"] == 2 and opt.stats["dense_fallbacks"] == 0
+    assert opt.stats["materialized_lookups"] == 1, "only the anchor rows are looked up"
+    assert [tuple(r["ids"].shape) for r in sorted(opt.fused_list, key=lambda r: r["fwd_idx"])] == [(b, 1), (1, k)]
+    opt.apply_grad(lr)
+    opt.check_ids()
+    assert opt.stats["per_record_merges"] == 0
+
+    # oracle: queries from the anchors, both logits, every gradient row, one merge
+    c64 = (w0[anchor_n] + rel_n.astype(np.float32).astype(np.float64)).astype(np.float32).astype(np.float64)
+    qs = [c64[:, None, None, :], off_n.astype(np.float64)[:, None, None, :]]
+    ids_n = np.broadcast_to(neg_n, (b, k))
+    logit_n, rows_n = oracle_union_logits("box", w0, ids_n, qs, gamma, cen)
+    logit_p, rows_p = oracle_union_logits("box", w0, pos_n[:, None], qs, gamma, cen)
+    assert_close(ln.detach().cpu().numpy(), logit_n[:, 0], REL_F32, "shared step: negative logits")
+    assert_close(lp.detach().cpu().numpy(), logit_p[:, 0], REL_F32, "shared step: positive logits")
+    gr_n, gq_n = oracle_union_grads("box", w0, ids_n, qs, rows_n, logit_n, (mask_n * gn_n).astype(np.float64), cen)
+    gr_p, gq_p = oracle_union_grads("box", w0, pos_n[:, None], qs, rows_p, logit_p, gp_n.astype(np.float64), cen)
+    g_center = (gq_n[0] + gq_p[0])[:, 0, 0]
+    assert_close(rel.grad.cpu().numpy(), g_center, REL_F32, "shared step: relation gradient",
+                 sum_abs=(np.abs(mask_n * gn_n).sum(axis=1) + np.abs(gp_n[:, 0]))[:, None] * np.ones((1, d)))
+    w, m, _, uniq, merged = oracle_adam_step(w0, [pos_n, ids_n, anchor_n], [gr_p, gr_n, g_center], lr, 1)
+    assert_close(emb.state_sum_fo.cpu().numpy()[uniq], m[uniq], REL_F32, "shared step: first moment")
+    assert_adam_weights(emb.embedding.detach().cpu().numpy(), w, merged, uniq, lr, "shared step: weights")
+    untouched = np.setdiff1d(np.arange(n), uniq)
+    assert np.array_equal(emb.embedding.detach().cpu().numpy()[untouched], w0[untouched].astype(np.float32))
+
+
+@pytest.mark.parametrize("n_ids", [1, 2, 63, 64, 65, 1000, 2049, 4096, 4097])
+def test_small_plans_are_the_bits_of_numpy(n_ids):
+    """Up to 4096 ids are sorted by one workgroup in one launch; 4097 take the radix passes.  Same contract."""
+    from smore_amd import fused
+    rng = np.random.default_rng(n_ids)
+    n_rows = 50 if n_ids > 10 else 3
+    idx = rng.integers(0, n_rows, n_ids).astype(np.int64)
+    if n_ids >= 63:
+        idx[[5, n_ids - 1]] = [n_rows + 7, -3]           # ids outside the table: flagged, kept out of every segment
+    err = fused.new_error_flag("cuda")
+    plan = fused.build_plan(torch.tensor(idx, device="cuda"), n_rows, want_inverse=True, err_flag=err)
+    bad = (idx < 0) | (idx >= n_rows)
+    key = np.where(bad, n_rows, idx)
+    order = np.argsort(key, kind="stable")
+    uniq = np.unique(key[~bad])
+    assert err.item() == (1 if bad.any() else 0)
+    assert plan.n_uniq == uniq.size and np.array_equal(plan.uniq.cpu().numpy(), uniq)
+    assert np.array_equal(plan.order.cpu().numpy(), order)
+    assert np.array_equal(plan.sorted_ids.cpu().numpy().astype(np.int64) & 0xffffffff, key[order])
+    seg_of_pos = np.cumsum(np.r_[0, np.diff(key[order]) != 0])
+    assert np.array_equal(plan.seg_of_pos.cpu().numpy(), seg_of_pos)
+    n_seg = seg_of_pos[-1] + 1
+    starts = np.r_[np.flatnonzero(np.r_[1, np.diff(key[order]) != 0]), n_ids]
+    assert np.array_equal(plan.seg_start[: n_seg + 1].cpu().numpy(), starts)
+    inverse = np.empty(n_ids, dtype=np.int64)
+    inverse[order] = seg_of_pos
+    assert np.array_equal(plan.inverse.cpu().numpy(), inverse)
+    counts = np.bincount(key, minlength=n_rows + 1)
+    alone = (counts[key] == 1) & ~bad
+    ps = plan.pair_seg.cpu().numpy()
+    assert np.array_equal(ps < 0, alone) and np.array_equal(ps[alone] & 0x7fffffff, inverse[alone])
+    assert np.all(ps[~alone] == 0)
+
+
+def test_a_plan_that_gives_up_is_marked_on_the_device_and_nothing_reads_it():
+    """The bounded waits of the sort: a build that starts with its give-up word set leaves err = 2 and n_uniq = -1
+    with every kernel ending normally; the entity pass, the one-call backward and the shared entity pass, handed
+    that plan, touch no row; the Python handle refuses to hand out its sizes.  With a wait limit of zero polls a
+    build either completes correctly or gives up the same way."""
+    from smore_amd import _lib, fused
+    rng = np.random.default_rng(0)
+    n, b, k, dim = 5000, 40, 300, 32
+    table, q1, q2, idx, gs = make_problem("box", n, b, k, dim, rng)
+    t_idx = torch.tensor(idx, device="cuda")
+    t_table, t_q1, t_q2, t_gs = dev(table), dev(q1), dev(q2), dev(gs)
+    params = fused.score_params(24.0, 0.02)
+    err = fused.new_error_flag("cuda")
+    score = fused.score_forward("box", t_table, t_idx, t_q1, t_q2, params, err)
+    plan = fused.build_plan(t_idx, n, err_flag=err, measure=(1 << 22, 1))
+    torch.cuda.synchronize()
+    assert err.item() == 2 and plan.n_uniq_dev.item() == -1
+    with pytest.raises(_lib.SmxError):
+        plan.n_uniq
+    before = t_table.clone()
+    m, v = torch.zeros_like(t_table), torch.zeros_like(t_table)
+    adam = fused.adam_params(1e-3, 1)
+    fused.score_backward_entity("box", plan, t_table, t_q1, t_q2, score, t_gs, params, m=m, v=v, adam=adam)
+    fused.score_backward_fused("box", plan, t_table, t_idx, t_q1, t_q2, score, t_gs, params, m=m, v=v, adam=adam)
+    fused.rows_backward(plan, torch.zeros((b * k, dim), device="cuda"), table=t_table, m=m, v=v, adam=adam)
+    torch.cuda.synchronize()
+    assert torch.equal(t_table, before) and not m.any() and not v.any()
+    err.zero_()
+    small = fused.build_plan(t_idx[0, :100].contiguous(), n, err_flag=err, measure=(1 << 22, 1))
+    assert err.item() == 2 and small.n_uniq_dev.item() == -1
+    fused.score_backward_entity_shared("box", t_table, t_idx[0, :100].contiguous(), t_q1, t_q2, score[:, :100].contiguous(),
+                                       t_gs[:, :100].contiguous(), params, plan=small, m=m, v=v, adam=adam)
+    torch.cuda.synchronize()
+    assert torch.equal(t_table, before)
+    # a wait limit of zero polls: whichever way it ends, it ends, and it says which
+    err.zero_()
+    plan0 = fused.build_plan(t_idx, n, want_inverse=True, err_flag=err, measure=(0, 0))
+    torch.cuda.synchronize()
+    if err.item() == 0:
+        uniq, inverse, order, _ = orc.merge_indices(idx)
+        assert plan0.n_uniq == uniq.size and np.array_equal(plan0.order.cpu().numpy().astype(np.int64), order)
+    else:
+        assert err.item() == 2 and plan0.n_uniq_dev.item() == -1
+
+
+def test_apply_grad_raises_for_a_plan_that_gave_up(monkeypatch):
+    """The optimizer finds err = 2 at its next check and says what happened."""
+    from smore_amd import _lib, fused
+    from smore_amd.embedding.embed_optimizer import AdamEmbedOptimizer
+    from smore_amd.embedding.sparse_embed import SparseEmbedding
+    emb = SparseEmbedding(5000, 16).cuda()
+    emb.init_params(-0.07, 0.07)
+    opt = AdamEmbedOptimizer(types.SimpleNamespace(optim_mode="(aggr,adam,gpu,False,5)", share_optim_stats=True), emb, 0)
+    real = fused.build_plan
+    monkeypatch.setattr(fused, "build_plan", lambda idx, n_rows, want_inverse=False, err_flag=None:
+                        real(idx, n_rows, want_inverse, err_flag, measure=(1 << 22, 1)))
+    before = emb.embedding.detach().clone()
+    q = torch.rand((6, 16), device="cuda", requires_grad=True)
+    ids = torch.randint(0, 5000, (6, 900), device="cuda")
+    opt.zero_grad()
+    opt.score_negatives("l1", ids, q, gamma=12.0).sum().backward()
+    opt.apply_grad(1e-3)
+    with pytest.raises(_lib.SmxError, match="plan"):
+        opt.check_ids()
+    assert torch.equal(emb.embedding.detach(), before)
