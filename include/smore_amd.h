@@ -398,6 +398,22 @@ int smx_rank_scan(int model, void* stream, const float* table, size_t n_rows, co
                   const int64_t* ans_id, const uint64_t* ans_key, const int32_t* ans_count, size_t A,
                   int64_t* filtered_rank, void* workspace, size_t workspace_bytes);
 
+/* Evaluation against sampled candidates: the branch of test_step_mp taken when the evaluation set brings its own
+ * negatives (smore/training/train_process.py:118-128, 141-147).  cand [B, C] int64: per query its candidates, the
+ * first n_hard[b] of them its hard answers, -1 = padding.  As the reference does, a padding slot is scored as
+ * entity 0 and -1e6 is added to its logit (:119-120, :123).
+ *   logit [B, C]     (may be NULL) the biased logits, negative_logit of :123
+ *   ranking [B, C]   position of candidate j in argsort(logit, descending) (:124-128); equal logits: the lower
+ *                    candidate position first
+ *   hard_rank [B, H] filtered rank, 1-based, of hard answer j < n_hard[b] in the order given: ranking[j] minus
+ *                    the number of the query's hard answers ranked before it, plus 1 (:141-145); 0 in unused slots
+ * One workgroup per query: scores, ranks by counting, no sort.  At most 4096 candidates per query, H <= C.
+ * A candidate id other than -1 outside [0, n_rows) sets *err_flag (may be NULL) and is scored as entity 0. */
+int smx_rank_candidates(int model, void* stream, const float* table, size_t n_rows, const float* q1,
+                        const float* q2, size_t B, size_t dim, const smx_score_params* params,
+                        const int64_t* cand, size_t C, const int32_t* n_hard, size_t H, float* logit,
+                        int64_t* ranking, int64_t* hard_rank, int* err_flag);
+
 /* Plain row lookup out[k,:] = table[idx[k],:] (smore/common/embedding/embed_rw.py:74-75, the GPU
  * branch of EmbeddingReadOnly.read) for callers that need the rows themselves. */
 int smx_gather_rows(void* stream, const float* table, size_t n_rows, size_t row_len,

@@ -254,6 +254,23 @@ def filtered_ranks(scores, easy, hard):
     return filt[len(easy):], filt[: len(easy)]
 
 
+def candidate_ranks(logit, neg, n_hard):
+    """Evaluation against sampled candidates, train_process.py:118-128 and 141-147.  logit [C]: the logits of one
+    query's candidates neg [C] (padding -1 scored as entity 0, :120); the bias -1e6 is added where neg == -1 (:119,
+    :123); ranking = position in the descending argsort of the biased logits (equal logits: lower position first);
+    the first n_hard candidates are the hard answers, and the filtered rank of one is its position minus the
+    number of hard answers before it, plus 1.  Returns (biased logits, ranking [C], filtered ranks [n_hard] in the
+    order given)."""
+    logit = np.asarray(logit)
+    biased = logit + np.where(np.asarray(neg) == -1, logit.dtype.type(-1e6), logit.dtype.type(0))
+    order = np.argsort(-biased, kind="stable")
+    ranking = np.empty(biased.shape[0], dtype=np.int64)
+    ranking[order] = np.arange(biased.shape[0])
+    pos = ranking[:n_hard]
+    before = (pos[None, :] < pos[:, None]).sum(axis=1) if n_hard else pos
+    return biased, ranking, pos - before + 1
+
+
 # ---- composition: the score of each model and one training step -------------------------------
 
 MODELS = ("l1", "l2", "box", "rotate", "beta_kl", "complex", "distmult")

@@ -67,6 +67,8 @@ SIGNATURES = {
     "smx_rank_answer_keys": (_i, [_i, _vp, _vp, _sz, _vp, _vp, _sz, _sz, _vp, _vp, _vp, _sz, _vp, _vp]),
     # model, stream, table, n_rows, q1, q2, B, dim, params, ans_id, ans_key, ans_count, A, rank, ws, ws_bytes
     "smx_rank_scan": (_i, [_i, _vp, _vp, _sz, _vp, _vp, _sz, _sz, _vp, _vp, _vp, _vp, _sz, _vp, _vp, _sz]),
+    # model, stream, table, n_rows, q1, q2, B, dim, params, cand, C, n_hard, H, logit, ranking, hard_rank, err
+    "smx_rank_candidates": (_i, [_i, _vp, _vp, _sz, _vp, _vp, _sz, _sz, _vp, _vp, _sz, _vp, _sz, _vp, _vp, _vp, _vp]),
     "smx_sample_loss_workspace_bytes": (_sz, [_sz]),
     # stream, pos, neg, mask, weight, B, K, temperature, scale, out_loss, gpos, gneg, ws, ws_bytes
     "smx_sample_loss": (_i, [_vp, _vp, _vp, _vp, _vp, _sz, _sz, ctypes.c_double, ctypes.c_double, _vp, _vp, _vp, _vp, _sz]),

@@ -86,6 +86,8 @@ static int fill_plan(EntityArgs* A, const smx_plan_view* plan, void* workspace, 
   A->rows_first = (int)plan->n_pairs;  // no gradient rows of plain lookups behind the model's pairs
   A->tile = kTile;
   A->short_max = kShortMax;
+  A->chunk = 64;  // enough wavefronts to fill the chip also for a short list
+  while (A->chunk > 1 && plan->n_pairs / (size_t)A->chunk < 4096) A->chunk /= 2;
   char* ws = static_cast<char*>(workspace);
   A->tail = reinterpret_cast<float*>(ws + sc.tail_off);
   A->head = reinterpret_cast<float*>(ws + sc.head_off);

@@ -46,6 +46,9 @@ struct EntityArgs : RowSink {
   const int* n_uniq;
   int n_pairs;
   int tile;        // sorted positions per tile of the long-segment pass, multiple of 64
+  int chunk;       // sorted positions a wavefront of the short-segment pass owns per turn: 64, or a smaller power of
+                   // two for a short list (a step whose negatives are shared sorts a couple of thousand ids: with 64
+                   // positions per wavefront two dozen wavefronts would finish their segments one after the other)
   int short_max;   // segments of at most this many pairs are finished by one wavefront
   // source: score model
   const float* q1;
@@ -341,14 +344,14 @@ __global__ __launch_bounds__(256) void entity_segment_kernel(EntityArgs A) {
   const int lane = threadIdx.x & 63;
   const int wave = uniform(threadIdx.x >> 6);
   const int n_waves = gridDim.x * 4;
-  const int n_chunks = (A.n_pairs + 63) / 64;
+  const int n_chunks = (A.n_pairs + A.chunk - 1) / A.chunk;
   const int n_valid = *A.n_uniq;  // a last segment beyond this one holds the pairs whose id is outside the table: skipped
   if (n_valid < 0) return;  // the plan's build gave up: nothing of it may be read
   const bool mixed = SRC != kSrcRows && A.rows_first < A.n_pairs;  // the plan also holds gradient rows of plain lookups
 
   for (int chunk = blockIdx.x * 4 + wave; chunk < n_chunks; chunk += n_waves) {
-    const int base = chunk * 64;
-    const int n_here = min(64, A.n_pairs - base);
+    const int base = chunk * A.chunk;  // the window is 64 positions wide whatever the chunk: a segment that starts in
+    const int n_here = min(64, A.n_pairs - base);  // the chunk usually ends inside it
     const int pos = base + min(lane, n_here - 1);
     const int my_seg = A.seg_of_pos[pos];
     const int my_s0 = A.seg_start[my_seg];
@@ -356,8 +359,8 @@ __global__ __launch_bounds__(256) void entity_segment_kernel(EntityArgs A) {
     const int my_len = my_s1 - my_s0;
     bool done_elsewhere = A.skip_single && my_len == 1;  // by the pair-ordered kernel -- unless the one pair is a gradient row
     if (SRC != kSrcRows && mixed && done_elsewhere) done_elsewhere = A.order[pos] < A.rows_first;
-    unsigned long long todo =
-        __ballot(lane < n_here && my_s0 == pos && my_len <= A.short_max && !done_elsewhere && my_seg < n_valid);
+    unsigned long long todo = __ballot(lane < n_here && lane < A.chunk && my_s0 == pos && my_len <= A.short_max &&
+                                       !done_elsewhere && my_seg < n_valid);
     if (todo == 0ull) continue;
     const int my_id = A.sorted_ids[pos];
 
@@ -791,14 +794,14 @@ __global__ __launch_bounds__(256) void entity_segment_coded_kernel(EntityArgs A)
   const int wave = uniform(threadIdx.x >> 6);
   unsigned char* slab = code_lds + wave * (64 * NIT * 64);
   const int n_waves = gridDim.x * 4;
-  const int n_chunks = (A.n_pairs + 63) / 64;
+  const int n_chunks = (A.n_pairs + A.chunk - 1) / A.chunk;
   const int n_valid = *A.n_uniq;  // a last segment beyond this one holds the pairs whose id is outside the table: skipped
   if (n_valid < 0) return;  // the plan's build gave up: nothing of it may be read
   const bool mixed = A.rows_first < A.n_pairs;  // the plan also holds gradient rows of plain lookups
 
   for (int chunk = blockIdx.x * 4 + wave; chunk < n_chunks; chunk += n_waves) {
-    const int base = chunk * 64;
-    const int n_here = min(64, A.n_pairs - base);
+    const int base = chunk * A.chunk;  // the window is 64 positions wide whatever the chunk: a segment that starts in
+    const int n_here = min(64, A.n_pairs - base);  // the chunk usually ends inside it
     const int pos = base + min(lane, n_here - 1);
     const int my_seg = A.seg_of_pos[pos];
     const int my_plan_pair = A.order[pos];
@@ -809,13 +812,13 @@ __global__ __launch_bounds__(256) void entity_segment_coded_kernel(EntityArgs A)
     // a one-pair segment was finished by the pair-ordered kernel -- unless its one pair is a gradient row
     const bool done_elsewhere = A.skip_single && my_len == 1 && !(mixed && my_plan_pair >= A.rows_first);
     const bool mine = lane < n_here && my_len <= A.short_max && !done_elsewhere && my_seg < n_valid;
-    unsigned long long todo = __ballot(mine && my_s0 == pos);
+    unsigned long long todo = __ballot(mine && my_s0 == pos && lane < A.chunk);
     if (todo == 0ull) continue;
 
     int win_base = base;
     unsigned win_id = my_id;
     // the lanes of segments that started before the chunk belong to another wavefront's work
-    CodedLane cur = resolve_coded_lane<SRC, NIT>(A, my_plan_pair, mine && my_s0 >= base);
+    CodedLane cur = resolve_coded_lane<SRC, NIT>(A, my_plan_pair, mine && my_s0 >= base && my_s0 < base + A.chunk);
     {
       const bool head = starts_run(lane, cur, win_id);
       code_vec4 cd[NIT * 4];
@@ -1010,7 +1013,7 @@ int launch_entity_reg(hipStream_t st, const EntityArgs& A) {
   const unsigned tiles = (unsigned)((A.n_pairs + A.tile - 1) / A.tile);
   // short segments: a fixed grid of wavefronts strides over the segment list (its length lives on the device)
   // (as many workgroups as the chip holds at once: a second wave of workgroups would run half empty)
-  const unsigned want_blocks = (unsigned)((A.n_pairs + 255) / 256);
+  const unsigned want_blocks = (unsigned)(((A.n_pairs + A.chunk - 1) / A.chunk + 3) / 4);
   bool coded = false;
   // (sign codes exist for rows of up to two column groups)
   if constexpr (SRC != kSrcRows && model_coded(SRC) && !REG && NIT <= 2) coded = A.codes != nullptr;

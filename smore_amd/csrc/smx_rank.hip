@@ -3,14 +3,15 @@
 
 namespace smx {
 
-extern template int rank_dispatch<mL1>(hipStream_t, const RankArgs&, int, int, bool);
-extern template int rank_dispatch<mL2>(hipStream_t, const RankArgs&, int, int, bool);
-extern template int rank_dispatch<mBox>(hipStream_t, const RankArgs&, int, int, bool);
-extern template int rank_dispatch<mRotate>(hipStream_t, const RankArgs&, int, int, bool);
-extern template int rank_dispatch<mBetaKL>(hipStream_t, const RankArgs&, int, int, bool);
-extern template int rank_dispatch<mComplex>(hipStream_t, const RankArgs&, int, int, bool);
-extern template int rank_dispatch<mDistmult>(hipStream_t, const RankArgs&, int, int, bool);
+extern template int rank_dispatch<mL1>(hipStream_t, const RankArgs&, int, int, int);
+extern template int rank_dispatch<mL2>(hipStream_t, const RankArgs&, int, int, int);
+extern template int rank_dispatch<mBox>(hipStream_t, const RankArgs&, int, int, int);
+extern template int rank_dispatch<mRotate>(hipStream_t, const RankArgs&, int, int, int);
+extern template int rank_dispatch<mBetaKL>(hipStream_t, const RankArgs&, int, int, int);
+extern template int rank_dispatch<mComplex>(hipStream_t, const RankArgs&, int, int, int);
+extern template int rank_dispatch<mDistmult>(hipStream_t, const RankArgs&, int, int, int);
 
+constexpr size_t kRankMaxCandidates = 4096;  // per query: their keys live in LDS
 constexpr size_t kRankMaxAnswers = 2048;  // per query; bins and keys of a pass live in LDS (per query of the pass 2049 x 4 + 2048 x 8 bytes)
 
 static size_t rank_ws_bytes(size_t B, size_t A) { return (B * (A + 1) * sizeof(unsigned) + 255) & ~(size_t)255; }
@@ -48,7 +49,7 @@ static int rank_common(RankArgs* R, int* vec, int* nit, int model, const float* 
   return SMX_OK;
 }
 
-static int rank_run(int model, hipStream_t st, const RankArgs& R, int vec, int nit, bool keys_only) {
+static int rank_run(int model, hipStream_t st, const RankArgs& R, int vec, int nit, int keys_only) {
   switch (model) {
     case mL1: return rank_dispatch<mL1>(st, R, vec, nit, keys_only);
     case mL2: return rank_dispatch<mL2>(st, R, vec, nit, keys_only);
@@ -77,7 +78,7 @@ int smx_rank_answer_keys(int model, void* stream, const float* table, size_t n_r
   if (!ans_score || !ans_key) return fail(SMX_ERR_ARG, "null output pointer");
   R.score_out = ans_score;
   R.key_out = reinterpret_cast<unsigned long long*>(ans_key);
-  return rank_run(model, as_stream(stream), R, vec, nit, true);
+  return rank_run(model, as_stream(stream), R, vec, nit, kRankKeys);
 }
 
 int smx_rank_scan(int model, void* stream, const float* table, size_t n_rows, const float* q1, const float* q2, size_t B,
@@ -93,7 +94,33 @@ int smx_rank_scan(int model, void* stream, const float* table, size_t n_rows, co
   R.ans_key = reinterpret_cast<const unsigned long long*>(ans_key);
   R.bins = static_cast<unsigned*>(workspace);
   R.rank_out = reinterpret_cast<long long*>(filtered_rank);
-  return rank_run(model, as_stream(stream), R, vec, nit, false);
+  return rank_run(model, as_stream(stream), R, vec, nit, kRankScan);
+}
+
+int smx_rank_candidates(int model, void* stream, const float* table, size_t n_rows, const float* q1, const float* q2,
+                        size_t B, size_t dim, const smx_score_params* params, const int64_t* cand, size_t C,
+                        const int32_t* n_hard, size_t H, float* logit, int64_t* ranking, int64_t* hard_rank,
+                        int* err_flag) {
+  using namespace smx;
+  RankArgs R;
+  int vec, nit;
+  if (!cand || !n_hard || !ranking || !hard_rank) return fail(SMX_ERR_ARG, "null pointer");
+  if (C == 0 || C > kRankMaxCandidates) return fail(SMX_ERR_SHAPE, "1 to %zu candidates per query", kRankMaxCandidates);
+  if (H == 0 || H > C) return fail(SMX_ERR_SHAPE, "between 1 and C hard-answer slots");
+  // (the shape checks shared with the all-entity scan; its answer arguments are not used here)
+  if (int rc = rank_common(&R, &vec, &nit, model, table, n_rows, q1, q2, B, dim, params, cand, n_hard, 1)) return rc;
+  if (B * C > 0x7fffffffull) return fail(SMX_ERR_SHAPE, "too many candidates in one call");
+  R.ans_id = nullptr;
+  R.ans_count = nullptr;
+  R.cand = reinterpret_cast<const long long*>(cand);
+  R.C = (int)C;
+  R.H = (int)H;
+  R.n_hard = n_hard;
+  R.cand_logit = logit;
+  R.cand_rank = reinterpret_cast<long long*>(ranking);
+  R.hard_rank = reinterpret_cast<long long*>(hard_rank);
+  R.err = err_flag;
+  return rank_run(model, as_stream(stream), R, vec, nit, kRankCandidates);
 }
 
 }  // extern "C"

@@ -37,7 +37,17 @@ struct RankArgs {
   int A;
   unsigned* bins;                    // [B, A + 1]
   long long* rank_out;               // [B, A]
+  // ranking among sampled candidates (rank_candidates_kernel)
+  const long long* cand;             // [B, C], -1 = padding
+  int C, H;
+  const int* n_hard;                 // [B]: the first n_hard[b] candidates of query b are its hard answers
+  float* cand_logit;                 // [B, C] or null
+  long long* cand_rank;              // [B, C]
+  long long* hard_rank;              // [B, H]
+  int* err;
 };
+
+enum RankMode : int { kRankScan = 0, kRankKeys = 1, kRankCandidates = 2 };
 
 __device__ __forceinline__ unsigned sortable_bits(float s) {
   const unsigned u = __float_as_uint(s);
@@ -247,6 +257,67 @@ __global__ __launch_bounds__(256) void rank_scan_kernel(RankArgs A) {
   }
 }
 
+// Evaluation against sampled candidates (the branch of smore/training/train_process.py:118-128 taken when the
+// evaluation set brings its own negatives): one workgroup per query scores the query's C candidates -- padding
+// (-1) is scored as entity 0 with a bias of -1e6 added to the logit, exactly as the reference does -- and ranks
+// them among themselves: ranking[j] = number of candidates ordered before candidate j by descending biased
+// logit, i.e. the position `argsort(descending)` gives it (equal logits: the lower position first, one of the
+// orders an unstable argsort may produce).  The first n_hard candidates are the hard answers; their filtered
+// ranks (rank - number of hard answers ranked before it + 1, :141-145) come out as well.
+// LDS: keys [C] (64-bit), ranks of the hard answers [H].
+constexpr int kCandThreads = 1024;
+
+template <int M, int VEC, int NIT, bool REG>
+__global__ __launch_bounds__(kCandThreads) void rank_candidates_kernel(RankArgs A) {
+  constexpr int MUL = model_mul(M);
+  extern __shared__ unsigned long long cand_keys[];  // [C], then int ranks [H]
+  int* hard_ranks = reinterpret_cast<int*>(cand_keys + A.C);
+  const int b = blockIdx.x;
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int dim = A.ncol * VEC;
+  typename ModelOps<M>::Q q[NIT][VEC];
+  load_rank_query<M, VEC, NIT>(A.q1, A.q2, b, dim, A.ncol, lane, q);
+  int bad = 0;
+  for (int j = wave; j < A.C; j += kCandThreads / 64) {  // uniform per wavefront
+    const long long raw = A.cand[(size_t)b * A.C + j];
+    const bool pad = raw == -1;
+    unsigned long long id = pad ? 0ull : (unsigned long long)raw;
+    if (id >= A.n_rows) {
+      bad = 1;
+      id = 0;
+    }
+    float e1[NIT][VEC], e2[NIT][VEC];
+    load_entity<VEC, NIT, MUL>(A.table + id * (size_t)dim * MUL, dim, A.ncol, lane, e1, e2);
+    const float s = row_score<M, VEC, NIT, REG>(e1, e2, q, A.ncol, lane, A.p) + (pad ? -1e6f : 0.f);
+    if (lane == 63) {
+      if (A.cand_logit) A.cand_logit[(size_t)b * A.C + j] = s;
+      cand_keys[j] = ((unsigned long long)sortable_bits(s) << 32) | (unsigned)(~(unsigned)j);
+    }
+  }
+  if (bad && A.err && lane == 0) *A.err = 1;
+  __syncthreads();
+  const int n_hard = min(A.n_hard[b], min(A.H, A.C));
+  for (int j = threadIdx.x; j < A.C; j += kCandThreads) {
+    const unsigned long long mine = cand_keys[j];
+    int before = 0;
+    for (int i = 0; i < A.C; ++i) before += cand_keys[i] > mine ? 1 : 0;  // every thread reads the same key: a broadcast
+    A.cand_rank[(size_t)b * A.C + j] = before;
+    if (j < n_hard) hard_ranks[j] = before;
+  }
+  __syncthreads();
+  for (int j = threadIdx.x; j < A.H; j += kCandThreads) {
+    long long out = 0;
+    if (j < n_hard) {
+      const int mine = hard_ranks[j];
+      int ahead = 0;
+      for (int i = 0; i < n_hard; ++i) ahead += hard_ranks[i] < mine ? 1 : 0;
+      out = (long long)(mine - ahead + 1);
+    }
+    A.hard_rank[(size_t)b * A.H + j] = out;
+  }
+}
+
 static __global__ __launch_bounds__(256) void rank_clear_kernel(unsigned* bins, size_t n) {
   const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
   if (i < n) bins[i] = 0u;
@@ -267,8 +338,13 @@ static __global__ __launch_bounds__(256) void rank_finish_kernel(RankArgs A) {
 }
 
 template <int M, int VEC, int NIT, bool REG>
-int launch_rank_reg(hipStream_t st, RankArgs A, bool keys_only) {
-  if (keys_only) {
+int launch_rank_reg(hipStream_t st, RankArgs A, int mode) {
+  if (mode == kRankCandidates) {
+    const size_t lds = (size_t)A.C * sizeof(unsigned long long) + (size_t)A.H * sizeof(int);
+    hipLaunchKernelGGL((rank_candidates_kernel<M, VEC, NIT, REG>), dim3((unsigned)A.B), dim3(kCandThreads), lds, st, A);
+    return check_launch("rank candidates");
+  }
+  if (mode == kRankKeys) {
     const unsigned blocks = (unsigned)(((size_t)A.B * A.A + 3) / 4);
     hipLaunchKernelGGL((rank_answer_keys_kernel<M, VEC, NIT, REG>), dim3(blocks), dim3(256), 0, st, A);
     return check_launch("rank answer keys");
@@ -319,28 +395,28 @@ int launch_rank_reg(hipStream_t st, RankArgs A, bool keys_only) {
 }
 
 template <int M, int VEC, int NIT>
-int launch_rank(hipStream_t st, const RankArgs& A, bool keys_only) {
+int launch_rank(hipStream_t st, const RankArgs& A, int mode) {
   if constexpr (M == mBetaKL) {
-    if (A.p.reg_on) return launch_rank_reg<M, VEC, NIT, true>(st, A, keys_only);
+    if (A.p.reg_on) return launch_rank_reg<M, VEC, NIT, true>(st, A, mode);
   }
-  return launch_rank_reg<M, VEC, NIT, false>(st, A, keys_only);
+  return launch_rank_reg<M, VEC, NIT, false>(st, A, mode);
 }
 
 // Instantiated once per model in its own translation unit (smx_rank_inst_*.hip).
 template <int M>
-int rank_dispatch(hipStream_t st, const RankArgs& A, int vec, int nit, bool keys_only) {
+int rank_dispatch(hipStream_t st, const RankArgs& A, int vec, int nit, int mode) {
   if (vec == 4) {
     switch (nit) {
-      case 1: return launch_rank<M, 4, 1>(st, A, keys_only);
-      case 2: return launch_rank<M, 4, 2>(st, A, keys_only);
-      case 4: return launch_rank<M, 4, 4>(st, A, keys_only);
-      default: return launch_rank<M, 4, 8>(st, A, keys_only);
+      case 1: return launch_rank<M, 4, 1>(st, A, mode);
+      case 2: return launch_rank<M, 4, 2>(st, A, mode);
+      case 4: return launch_rank<M, 4, 4>(st, A, mode);
+      default: return launch_rank<M, 4, 8>(st, A, mode);
     }
   }
   switch (nit) {
-    case 1: return launch_rank<M, 1, 1>(st, A, keys_only);
-    case 2: return launch_rank<M, 1, 2>(st, A, keys_only);
-    default: return launch_rank<M, 1, 4>(st, A, keys_only);
+    case 1: return launch_rank<M, 1, 1>(st, A, mode);
+    case 2: return launch_rank<M, 1, 2>(st, A, mode);
+    default: return launch_rank<M, 1, 4>(st, A, mode);
   }
 }
 

@@ -3,5 +3,5 @@
 #include "smx_rank_impl.h"
 
 namespace smx {
-template int rank_dispatch<mDistmult>(hipStream_t, const RankArgs&, int, int, bool);
+template int rank_dispatch<mDistmult>(hipStream_t, const RankArgs&, int, int, int);
 }

@@ -60,6 +60,36 @@ def filtered_ranks(model, table, q1, q2, params, easy_answers, hard_answers):
     return out
 
 
+def candidate_ranks(model, table, q1, q2, params, negative_sample, n_hard, err_flag=None):
+    """The other branch of test_step_mp (train_process.py:118-128, 141-147): the evaluation set brings its own
+    candidates.  negative_sample [B, C] int64 on the table's device, -1 = padding; the first n_hard[b] candidates
+    of query b are its hard answers (n_hard: sequence or int tensor of B counts).  Returns (negative_logit [B, C]
+    with the -1e6 bias on the padding, ranking [B, C] int64, filtered ranks of the hard answers [B, max n_hard]
+    int64, 0 in unused slots) -- one launch, no argsort."""
+    b = q1.shape[0]
+    if negative_sample.dim() != 2 or negative_sample.shape[0] != b or negative_sample.dtype != torch.int64:
+        raise _lib.SmxError("negative_sample must be int64 [B, C]")
+    dev = table.device
+    cand = negative_sample.to(dev).contiguous()
+    counts = torch.as_tensor(n_hard, dtype=torch.int32).reshape(-1)
+    if counts.numel() != b or int(counts.min()) < 0 or int(counts.max()) > cand.shape[1]:
+        raise _lib.SmxError("one hard-answer count per query, between 0 and C")
+    h = max(1, int(counts.max()))
+    counts = counts.to(dev)
+    q1c = q1.reshape(b, -1).contiguous()
+    q2c = None if q2 is None else q2.reshape(b, -1).contiguous()
+    _, _, dim = _dims(model, table, cand, q1c, q2c)
+    c = cand.shape[1]
+    logit = torch.empty((b, c), dtype=torch.float32, device=dev)
+    ranking = torch.empty((b, c), dtype=torch.int64, device=dev)
+    hard = torch.empty((b, h), dtype=torch.int64, device=dev)
+    with torch.cuda.device(dev):
+        _lib.call("smx_rank_candidates", MODELS[model], _stream(table), _ptr(table), table.shape[0], _ptr(q1c), _ptr(q2c),
+                  b, dim, ctypes.byref(params), _ptr(cand), c, _ptr(counts), h, _ptr(logit), _ptr(ranking), _ptr(hard),
+                  _ptr(err_flag))
+    return logit, ranking, hard
+
+
 def ranking_metrics(hard_ranks):
     """MRR, HITS1/3/10 and HITS1max of one query from the filtered ranks of its hard answers
     (train_process.py:146-152); an empty tensor gives zeros, as the reference does for a query whose

@@ -84,9 +84,32 @@ def make_ranking(seed):
                         scores=scores, hard_ranks=np.array(hr), easy_ranks=np.array(er))
 
 
+def make_candidates(seed):
+    """Sampled-candidate evaluation on an integer-valued L1 problem (exact in any precision): padding, ties, a hard
+    answer that is not the best candidate."""
+    rng = np.random.default_rng(seed)
+    n, d, b, c = 200, 8, 3, 40
+    table = rng.integers(-3, 4, (n, d)).astype(np.float64)
+    q1 = rng.integers(-3, 4, (b, d)).astype(np.float64)
+    neg = rng.integers(0, n, (b, c)).astype(np.int64)
+    neg[0, 30:] = -1
+    neg[1, [5, 6]] = neg[1, 0]          # the same entity three times: equal logits
+    neg[2, 0] = -1                      # the answer is not among the candidates (train_process.py:137)
+    n_hard = np.array([3, 2, 1], dtype=np.int32)
+    rows = table[np.where(neg == -1, 0, neg)]
+    logit = orc.score_forward("l1", rows, q1[:, None], None, GAMMA["l1"], 0.0).astype(np.float32)
+    out = [orc.candidate_ranks(logit[i], neg[i], int(n_hard[i])) for i in range(b)]
+    hard = np.zeros((b, 3), dtype=np.int64)
+    for i, (_, _, f) in enumerate(out):
+        hard[i, : f.size] = f
+    np.savez_compressed(os.path.join(HERE, "candidates.npz"), table=table, q1=q1, neg=neg, n_hard=n_hard, gamma=GAMMA["l1"],
+                        logit=np.stack([o[0] for o in out]), ranking=np.stack([o[1] for o in out]), hard_ranks=hard)
+
+
 if __name__ == "__main__":
     for i, model in enumerate(GAMMA):
         make(model, 100 + i)
     make_loss(200)
     make_ranking(300)
+    make_candidates(400)
     print("wrote", sorted(f for f in os.listdir(HERE) if f.endswith(".npz")))

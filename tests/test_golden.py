@@ -125,6 +125,13 @@ def test_oracle_reproduces_loss_and_ranking_fixtures():
     for i in range(r["q1"].shape[0]):
         h, e = orc.filtered_ranks(r["scores"][i], r["easy"][i].tolist(), r["hard"][i].tolist())
         assert np.array_equal(h, r["hard_ranks"][i]) and np.array_equal(e, r["easy_ranks"][i])
+    c = _golden("candidates.npz")
+    for i in range(c["q1"].shape[0]):
+        rows = c["table"][np.where(c["neg"][i] == -1, 0, c["neg"][i])]
+        logit = orc.score_forward("l1", rows[None], c["q1"][i][None, None], None, float(c["gamma"]), 0.0)[0].astype(np.float32)
+        biased, ranking, filt = orc.candidate_ranks(logit, c["neg"][i], int(c["n_hard"][i]))
+        assert np.array_equal(biased, c["logit"][i]) and np.array_equal(ranking, c["ranking"][i])
+        assert np.array_equal(filt, c["hard_ranks"][i][: filt.size])
 
 
 @pytest.mark.gpu
@@ -149,3 +156,9 @@ def test_hip_path_reproduces_loss_and_ranking_fixtures():
     for i, (h, e) in enumerate(got):
         assert h.cpu().numpy().tolist() == r["hard_ranks"][i].tolist()
         assert e.cpu().numpy().tolist() == r["easy_ranks"][i].tolist()
+    c = _golden("candidates.npz")
+    from smore_amd.evaluation import candidate_ranks
+    logit, ranking, hard = candidate_ranks("l1", dev(c["table"]), dev(c["q1"]), None, fused.score_params(float(c["gamma"])),
+                                           torch.tensor(c["neg"], device="cuda"), c["n_hard"])
+    assert np.array_equal(logit.cpu().numpy(), c["logit"]) and np.array_equal(ranking.cpu().numpy(), c["ranking"])
+    assert np.array_equal(hard.cpu().numpy(), c["hard_ranks"])

@@ -572,3 +572,30 @@ def test_filtered_ranks_follow_the_evaluation_loop():
     assert h.tolist() == [5] and e.size == 0
     h, _ = orc.filtered_ranks(tied, [1], [4, 0])
     assert h.tolist() == [3, 1]      # position 4, two answers (ids 0 and 1) before it
+
+
+def test_candidate_ranks_follow_the_sampled_negatives_branch():
+    """orc.candidate_ranks against the tensor recipe of train_process.py:118-128, 141-147 restated with torch
+    (where / bias, argsort, scatter of arange, ranking[:num_hard], sort, minus arange, +1) on tie-free logits, and
+    the tie rule by hand."""
+    rng = np.random.default_rng(29)
+    c, n_hard = 300, 6
+    neg = rng.integers(0, 1000, c)
+    neg[[40, 41, 299]] = -1
+    logit = (rng.permutation(c).astype(np.float32) * np.float32(0.37) - np.float32(20.0))
+    biased, ranking, filt = orc.candidate_ranks(logit, neg, n_hard)
+    t_neg = torch.tensor(neg)[None]
+    bias = torch.where(t_neg == -1, -1e6, 0.)
+    negative_logit = torch.tensor(logit)[None] + bias.to(torch.float32)
+    assert np.array_equal(biased, negative_logit[0].numpy())
+    argsort = torch.argsort(negative_logit, dim=1, descending=True)
+    rk = argsort.clone().to(torch.float)
+    rk = rk.scatter_(1, argsort, torch.arange(c).to(torch.float).repeat(1, 1))
+    assert np.array_equal(ranking, rk[0].to(torch.int64).numpy())
+    cur, _ = torch.sort(rk[0, :n_hard])
+    cur = cur - torch.arange(n_hard).to(torch.float) + 1
+    assert sorted(filt.tolist()) == cur.to(torch.int64).tolist()
+    assert ranking[40] > ranking[(neg != -1)].max() and ranking[41] == ranking[40] + 1    # padding last, in position order
+    # equal logits: the lower position first
+    _, r, f = orc.candidate_ranks(np.zeros(5, np.float32), np.array([3, 3, -1, 3, 3]), 2)
+    assert r.tolist() == [0, 1, 4, 2, 3] and f.tolist() == [1, 1]

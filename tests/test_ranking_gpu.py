@@ -5,6 +5,7 @@ import torch
 
 from oracle import oracle as orc
 from tests.test_fused_gpu import GAMMA, dev, make_problem
+from tests.util import REL_F32, assert_close
 
 pytestmark = pytest.mark.gpu
 
@@ -124,3 +125,44 @@ def test_ranking_argument_errors():
         filtered_ranks("l1", t, q, None, p, [[]], [[1], [2]])
     with pytest.raises(_lib.SmxError, match="answers per query"):
         filtered_ranks("l1", torch.zeros(4000, 8, device="cuda"), q, None, p, [[]], [list(range(2049))])
+
+
+@pytest.mark.parametrize("model,dim", [("box", 64), ("rotate", 40), ("beta_kl", 36), ("l2", 200), ("distmult", 30)])
+def test_sampled_candidates_follow_the_reference_recipe(model, dim):
+    """The sampled-negatives branch of test_step_mp (train_process.py:118-128, 141-147): -1 padding scored as entity
+    0 with the -1e6 bias, ranking among the candidates, filtered ranks of the leading hard answers.  The logits
+    against the float64 oracle; ranking and filtered ranks exactly the oracle's recipe applied to the device's own
+    fp32 logits (two logits within rounding of each other may legitimately swap between precisions)."""
+    from smore_amd import fused
+    from smore_amd.evaluation import candidate_ranks
+    from tests.test_fused_gpu import GAMMA, make_problem
+    rng = np.random.default_rng(dim)
+    n, b, c = 500, 5, 333
+    table, q1, q2, _, _ = make_problem(model, n, b, 1, dim, rng)
+    neg = rng.integers(0, n, (b, c)).astype(np.int64)
+    neg[0, 100:] = -1
+    neg[1, 0] = -1
+    neg[2, 7] = neg[2, 3]
+    n_hard = np.array([4, 1, 9, 0, 333], dtype=np.int32)
+    dev = lambda a: None if a is None else torch.tensor(a, dtype=torch.float32, device="cuda")
+    params = fused.score_params(GAMMA[model], 0.02)
+    err = fused.new_error_flag("cuda")
+    logit, ranking, hard = candidate_ranks(model, dev(table), dev(q1), dev(q2), params, torch.tensor(neg, device="cuda"),
+                                           n_hard, err)
+    assert err.item() == 0
+    rows = table[np.where(neg == -1, 0, neg)]
+    want = orc.score_forward(model, rows, q1[:, None], None if q2 is None else q2[:, None], GAMMA[model], 0.02)
+    want = want + np.where(neg == -1, -1e6, 0.0)
+    assert_close(logit.cpu().numpy(), want, REL_F32, f"{model} candidate logits")
+    got_logit = logit.cpu().numpy()
+    for i in range(b):
+        _, rk, filt = orc.candidate_ranks(np.where(neg[i] == -1, got_logit[i] + np.float32(1e6), got_logit[i]), neg[i],
+                                          int(n_hard[i]))
+        # (the bias is already in the device's logits; candidate_ranks adds it again to the un-biased copy: for a
+        # padded slot fl(fl(x - 1e6) + 1e6) - 1e6 keeps the order among padded slots, which hold one value anyway)
+        assert np.array_equal(ranking[i].cpu().numpy(), rk), f"{model} ranking of query {i}"
+        assert np.array_equal(hard[i, : filt.size].cpu().numpy(), filt) and not hard[i, filt.size:].any()
+    bad = torch.tensor(neg, device="cuda")
+    bad[3, 5] = n + 4
+    candidate_ranks(model, dev(table), dev(q1), dev(q2), params, bad, n_hard, err)
+    assert err.item() == 1
