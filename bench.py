@@ -260,14 +260,21 @@ def time_graph_replays(step, steps, warmup):
     return ms
 
 
-def dropin_bench(cfg, device, seed, steps, warmup):
+DROPIN_ROUTES = [("explicit score_negatives", True, "negatives", True, False)]
+for _flow in ("negatives", "positive+negatives", "anchor+positive+negatives"):
+    DROPIN_ROUTES += [(f"lazy handle, {_flow}", True, _flow, False, False), (f"plain lookups, {_flow}", False, _flow, False, False)]
+DROPIN_ROUTES.append(("lazy handle + fused sample loss, anchor+positive+negatives", True, "anchor+positive+negatives", False, True))
+
+
+def dropin_flows(cfg, table, q1, q2, idx, steps, warmup, m=None, v=None, only=None):
     """The step as SMORE's own code reaches it (box workloads): SparseEmbedding + AdamEmbedOptimizer, the lookup /
     view / cal_logit sequence of KGReasoning.forward (kg_reasoning.py:298-307, 340-355) with box.py:157-164 as the
     logit, the sample loss of train_process.py:197-213 (uniform weights), loss.backward(), apply_grad(lr).
     Three flows -- negatives only; + the positive lookup; + an anchor lookup whose rows make the query centers
     (a 1p query: center = anchor + relation, box.py:137) -- each with the lazy lookup handle and with plain lookups
     (lazy_lookup = False: the reference's data flow, materialised [B*K, row] rows and gradient rows), and the
-    explicit score_negatives call.  Prints one JSON line of ms per step."""
+    explicit score_negatives call.  m, v: existing Adam state tables to continue from (else new ones are made);
+    only: names of the routes to time (default all).  Returns {route: ms per step}."""
     import types
     import torch
     import torch.nn.functional as F
@@ -275,13 +282,14 @@ def dropin_bench(cfg, device, seed, steps, warmup):
     from smore_amd.embedding.sparse_embed import SparseEmbedding
     from smore_amd.torchext.ext_ops import box_dist_in, box_dist_out
     from smore_amd.training import sample_loss
-    if cfg["model"] != "box":
-        sys.exit("--dropin restates the box model's code path: use --config 2 or 5")
-    table, q1, q2, idx, _ = make_inputs(cfg, device, seed)
+    device = table.device
     b, k = idx.shape
     emb = SparseEmbedding(8, cfg["dim"])
     emb.embedding = torch.nn.Parameter(table, requires_grad=True)
     emb.num_rows = cfg["n"]
+    if m is not None:
+        emb.register_buffer("state_sum_fo", m)
+        emb.register_buffer("state_sum_sq", v)
     opt = AdamEmbedOptimizer(types.SimpleNamespace(optim_mode="(aggr,adam,gpu,False,5)", share_optim_stats=True), emb, 0)
     gamma = torch.nn.Parameter(torch.tensor([cfg["gamma"]], device=device), requires_grad=False)
     rel_c, rel_o = q1.clone().requires_grad_(True), q2.clone().requires_grad_(True)
@@ -325,11 +333,9 @@ def dropin_bench(cfg, device, seed, steps, warmup):
         opt.apply_grad(lr)
 
     out = {}
-    routes = [("explicit score_negatives", True, "negatives", True, False)]
-    for flow in ("negatives", "positive+negatives", "anchor+positive+negatives"):
-        routes += [(f"lazy handle, {flow}", True, flow, False, False), (f"plain lookups, {flow}", False, flow, False, False)]
-    routes.append(("lazy handle + fused sample loss, anchor+positive+negatives", True, "anchor+positive+negatives", False, True))
-    for name, lazy, flow, explicit, fused_loss in routes:
+    for name, lazy, flow, explicit, fused_loss in DROPIN_ROUTES:
+        if only is not None and name not in only:
+            continue
         opt.lazy_lookup = lazy
         for _ in range(warmup):
             step(flow, explicit, fused_loss)
@@ -339,9 +345,20 @@ def dropin_bench(cfg, device, seed, steps, warmup):
             step(flow, explicit, fused_loss)
         torch.cuda.synchronize()
         out[name] = (time.perf_counter() - t0) * 1e3 / steps
+        if lazy and (opt.stats["dense_fallbacks"] or opt.stats["per_record_merges"]):
+            sys.exit(f"drop-in route {name!r} left the fused path: {opt.stats}")
     opt.check_ids()
+    return out
+
+
+def dropin_bench(cfg, device, seed, steps, warmup):
+    """bench.py --dropin: every route of dropin_flows on freshly made inputs; prints one JSON line of ms per step."""
+    if cfg["model"] != "box":
+        sys.exit("--dropin restates the box model's code path: use --config 2 or 5")
+    table, q1, q2, idx, _ = make_inputs(cfg, device, seed)
+    out = dropin_flows(cfg, table, q1, q2, idx, steps, warmup)
     print(json.dumps({"workload": cfg["name"], "dropin_ms_per_step": out, "steps": steps, "warmup": warmup,
-                      "pairs_per_step": b * k}))
+                      "pairs_per_step": idx.numel()}))
 
 
 class SharedStep:
@@ -855,12 +872,24 @@ def main():
             "streaming_bytes": algo_stream,
             "streaming_GBps": algo_stream / (ms_per_step * 1e-3) / 1e9,
         },
+        # secondary figure for the workloads without an optimizer: the step has to write one merged gradient row per
+        # distinct id (what apply_grad would consume), which the compulsory-traffic model above does not charge
+        **({} if cfg["adam"] else {"step_hbm_with_merged_rows": {
+            "algorithmic_bytes": algo + 4 * row_len(cfg) * n_uniq,
+            "achieved_GBps": (algo + 4 * row_len(cfg) * n_uniq) / (ms_per_step * 1e-3) / 1e9,
+            "frac_of_peak": (algo + 4 * row_len(cfg) * n_uniq) / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS}}),
         "phase_ms": phase_ms,
         "step_ms_events": step_ms_events,
     }
     if graph_ms is not None:
         out["graph_replay"] = {"ms_per_step": graph_ms, "value": pairs / (graph_ms * 1e-3), "unit": "pairs/s",
                                "frac_of_peak": algo / (graph_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS}
+    # the same step as unchanged SMORE model code reaches it (lookup handle, cal_logit, sample loss, backward,
+    # apply_grad), continuing on the same table and optimizer state: two routes of `bench.py --dropin`
+    if cfg["model"] == "box" and cfg["adam"]:
+        out["dropin_ms_per_step"] = dropin_flows(
+            cfg, table, q1, q2, idx, min(args.steps, 50), args.warmup, m=step.m, v=step.v,
+            only=("lazy handle, negatives", "lazy handle, anchor+positive+negatives"))
     # what plain kernels sustain on this GPU for the step's access shapes, measured now with the library's
     # probes (after the timed region); a step that writes w, m, v back is a copy-like mix of reads and writes
     try:

@@ -268,6 +268,7 @@ typedef struct smx_pair_source {
   const void* fwd_codes;   /* may be NULL */
   size_t fwd_codes_bytes;
   size_t K;
+  const uint8_t* winner;   /* [B, K] union queries only (smx_score_backward_entity_union), else NULL */
 } smx_pair_source;
 int smx_score_backward_entity_multi(int model, void* stream, const smx_plan_view* plan, float* table,
                                     size_t n_rows, const float* q1, const float* q2,
@@ -275,6 +276,35 @@ int smx_score_backward_entity_multi(int model, void* stream, const smx_plan_view
                                     const smx_score_params* params, float* merged, float* m, float* v,
                                     const smx_opt_params* adam, void* workspace, size_t workspace_bytes,
                                     const float* grad_rows, size_t n_grad_rows);
+
+/* ---- union queries ---------------------------------------------------------------------------
+ * A query in disjunctive normal form has U branch embeddings (smore/models/kg_reasoning.py:326), and the last line
+ * of every custom_cal_logit takes the maximum of the branches' logits (box.py:163, vec.py:89, rotate.py:141,
+ * beta.py:307).  q1, q2 are [B, U, dim] (branch rows of one query adjacent), idx [B, K] as for one branch.
+ *   smx_score_forward_union         score[b,k] = max_u logit(table[idx[b,k]], q[b,u]); winner[b,k] = the first
+ *                                   branch that holds the maximum (values / indices of torch.max(logit, dim=1)).
+ *                                   workspace: smx_union_workspace_bytes(B, U, K), every branch's logits.
+ *   smx_score_backward_query_union  gq1, gq2 [B, U, dim]: a branch row gets the gradient of the pairs it won
+ *                                   (autograd of torch.max), summed in pair order; it streams those pairs only.
+ *   smx_score_backward_entity_union smx_score_backward_entity_multi for such queries: every source brings its
+ *                                   winner array, a pair's entity gradient is taken against the branch that won
+ *                                   it, and the plan is built over the B*K pairs of each source, not over B*U*K.
+ *                                   No sign codes with union queries (pass fwd_codes = NULL).
+ * Replaces the same reference functions as the one-branch entry points, plus torch.max and its backward. */
+size_t smx_union_workspace_bytes(size_t B, size_t U, size_t K);
+int smx_score_forward_union(int model, void* stream, const float* table, size_t n_rows, const int64_t* idx,
+                            const float* q1, const float* q2, float* score, uint8_t* winner, size_t B, size_t U,
+                            size_t K, size_t dim, const smx_score_params* params, int* err_flag, void* workspace,
+                            size_t workspace_bytes);
+int smx_score_backward_query_union(int model, void* stream, const float* table, size_t n_rows, const int64_t* idx,
+                                   const float* q1, const float* q2, const float* score, const float* gscore,
+                                   const uint8_t* winner, float* gq1, float* gq2, size_t B, size_t U, size_t K,
+                                   size_t dim, const smx_score_params* params);
+int smx_score_backward_entity_union(int model, void* stream, const smx_plan_view* plan, float* table,
+                                    size_t n_rows, const float* q1, const float* q2, const smx_pair_source* src,
+                                    size_t n_src, size_t B, size_t U, size_t dim, const smx_score_params* params,
+                                    float* merged, float* m, float* v, const smx_opt_params* adam, void* workspace,
+                                    size_t workspace_bytes, const float* grad_rows, size_t n_grad_rows);
 
 /* Everything after the loss in one call: query gradients, and every entity row of the step finished
  * (merged gradient row and/or lazy Adam on w, m, v), as smx_score_backward_query followed by

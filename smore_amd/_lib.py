@@ -43,6 +43,16 @@ SIGNATURES = {
     # model, stream, table, n_rows, ids, q1, q2, score, gscore, B, K, dim, params, plan, grad_rows, merged, m, v, adam
     "smx_score_backward_entity_shared": (_i, [_i, _vp, _vp, _sz, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _vp, _vp, _vp,
                                               _vp, _vp, _vp, _vp]),
+    "smx_union_workspace_bytes": (_sz, [_sz, _sz, _sz]),
+    # model, stream, table, n_rows, idx, q1, q2, score, winner, B, U, K, dim, params, err_flag, ws, ws_bytes
+    "smx_score_forward_union": (_i, [_i, _vp, _vp, _sz, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _vp, _vp, _vp, _sz]),
+    # model, stream, table, n_rows, idx, q1, q2, score, gscore, winner, gq1, gq2, B, U, K, dim, params
+    "smx_score_backward_query_union": (_i, [_i, _vp, _vp, _sz, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz,
+                                            _vp]),
+    # model, stream, plan, table, n_rows, q1, q2, src[], n_src, B, U, dim, params, merged, m, v, adam, ws, ws_bytes,
+    # grad_rows, n_grad_rows
+    "smx_score_backward_entity_union": (_i, [_i, _vp, _vp, _vp, _sz, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _vp, _vp, _vp, _vp,
+                                             _vp, _vp, _sz, _vp, _sz]),
     "smx_plan_workspace_bytes": (_sz, [_sz, _sz]),
     # stream, idx, n_pairs, n_rows, ws, ws_bytes, order, sorted_ids, seg_of_pos, uniq, seg_start, inverse, pair_seg,
     # n_uniq, err
@@ -103,7 +113,8 @@ class PlanView(ctypes.Structure):
 
 class PairSource(ctypes.Structure):
     """smx_pair_source of include/smore_amd.h."""
-    _fields_ = [("score", _vp), ("gscore", _vp), ("fwd_codes", _vp), ("fwd_codes_bytes", _sz), ("K", _sz)]
+    _fields_ = [("score", _vp), ("gscore", _vp), ("fwd_codes", _vp), ("fwd_codes_bytes", _sz), ("K", _sz),
+                ("winner", _vp)]
 
 
 MAX_PAIR_SOURCES = 4

@@ -32,6 +32,10 @@ struct PairSources {
   const float* gscore[kMaxSources];
   const unsigned char* codes[kMaxSources];
   size_t K[kMaxSources];
+  // union queries: U branch rows per query in q1 / q2, and per source the branch that gave each pair's logit
+  // (null when U == 1)
+  const unsigned char* winner[kMaxSources];
+  size_t U;
   // behind the pairs of all sources the plan may hold n_grad more entries whose gradient autograd has already
   // materialised as a row each (plain lookups of the step: anchor entities): grad_rows[n_grad, row]
   const float* grad_rows;

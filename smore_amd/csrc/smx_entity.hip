@@ -181,6 +181,7 @@ int entity_backward(int model, void* stream, const smx_plan_view* plan, float* t
       A.src_gscore[i] = multi->gscore[i];
       A.src_codes[i] = multi->codes[i];
       A.src_K[i] = (int)multi->K[i];
+      A.src_winner[i] = multi->winner[i];
       first += B * multi->K[i];
     }
     if (first != B * K) return fail(SMX_ERR_SHAPE, "pair sources hold %zu pairs, plan %zu", first, B * K);
@@ -201,10 +202,18 @@ int entity_backward(int model, void* stream, const smx_plan_view* plan, float* t
   A.score = score;
   A.gscore = gscore;
   A.K = (int)K;
+  A.U = 1;
+  if (multi && multi->U > 1) {
+    if (codes) return fail(SMX_ERR_ARG, "union queries have no sign codes");
+    for (int i = 0; i < multi->n; ++i)
+      if (!multi->winner[i]) return fail(SMX_ERR_ARG, "union queries: pair source %d has no winner array", i);
+    A.U = (int)multi->U;
+  }
   if (multi && multi->n == 1) {  // one index stream (+ gradient rows): the single-source fields describe it
     A.n_src = 0;
     A.score = multi->score[0];
     A.gscore = multi->gscore[0];
+    A.winner = multi->winner[0];
   }
   A.p = ScoreParams{params->gamma, params->cen, params->reg_on, params->reg_add, params->reg_lo, params->reg_hi};
   A.table = table;

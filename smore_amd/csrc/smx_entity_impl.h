@@ -75,6 +75,11 @@ struct EntityArgs : RowSink {
   const float* src_gscore[kMaxSources];
   const unsigned char* src_codes[kMaxSources];
   int src_K[kMaxSources];
+  // Union queries: q1 / q2 hold U branch rows per query; a pair's gradient is taken against the branch that gave
+  // its logit (the first maximal one, as torch.max routes it): winner[pair], per source.  U == 1: no such array.
+  int U;
+  const unsigned char* winner;
+  const unsigned char* src_winner[kMaxSources];
   // Plain lookups of the same step (anchor entities, box.py:137) whose gradient autograd has materialised:
   // plan pairs from rows_first on are rows of grad_rows, [n_pairs - rows_first, row].  They sort behind the model
   // pairs of their segment and are added when the segment's row is finished.  rows_first == n_pairs: none.
@@ -210,6 +215,7 @@ __device__ __forceinline__ void load_window(const EntityArgs& A, int lane, int b
       int local = pair, K = A.src_K[0];
       const float* gs = A.src_gscore[0];
       const float* sc = A.src_score[0];
+      const unsigned char* win = A.src_winner[0];
 #pragma unroll
       for (int s = 1; s < kMaxSources; ++s) {
         if (s < A.n_src && pair >= A.first[s]) {
@@ -217,13 +223,16 @@ __device__ __forceinline__ void load_window(const EntityArgs& A, int lane, int b
           K = A.src_K[s];
           gs = A.src_gscore[s];
           sc = A.src_score[s];
+          win = A.src_winner[s];
         }
       }
       ModelOps<SRC>::coef(gs[local], sc[local], A.p, my_c, c1);
       my_key = local / K;
+      if (A.U > 1) my_key = my_key * A.U + win[local];  // the query row of the branch that won the pair
     } else {
       ModelOps<SRC>::coef(A.gscore[pair], A.score[pair], A.p, my_c, c1);
       my_key = pair / A.K;
+      if (A.U > 1) my_key = my_key * A.U + A.winner[pair];
     }
     if (is_row) {
       my_c = 0.f;

@@ -141,10 +141,31 @@ static int fill_args(ScoreArgs* A, int* vec, int* nit, int model, const float* t
   A->K = (int)K;
   A->ncol = (int)ncol;
   A->n_rows = idx ? n_rows : B * K;
+  A->U = 1;
   A->id_bits = 1;
   while (A->id_bits < 32 && ((A->n_rows - 1) >> A->id_bits) != 0) ++A->id_bits;
   A->p = ScoreParams{params->gamma, params->cen, params->reg_on, params->reg_add, params->reg_lo, params->reg_hi};
   return SMX_OK;
+}
+
+// score[b,k] = max over the branches u of branch[b*U+u, k], winner[b,k] = the first branch that holds it -- what
+// torch.max(logit, dim=1) returns as values and indices in the custom_cal_logit bodies (box.py:163).
+__global__ __launch_bounds__(256) void union_max_kernel(const float* __restrict__ branch, float* __restrict__ score,
+                                                        unsigned char* __restrict__ winner, int U, int K, size_t n) {
+  const size_t p = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (p >= n) return;
+  const size_t b = p / K, k = p - b * K;
+  float best = branch[(b * U) * K + k];
+  int at = 0;
+  for (int u = 1; u < U; ++u) {
+    const float s = branch[(b * U + u) * K + k];
+    if (s > best || (s != s && best == best)) {  // torch.max: a NaN wins, and the first of equals stays
+      best = s;
+      at = u;
+    }
+  }
+  score[p] = best;
+  winner[p] = (unsigned char)at;
 }
 
 }  // namespace smx
@@ -230,6 +251,54 @@ int smx_score_backward_query_shared(int model, void* stream, const float* table,
   return dispatch_model(model, as_stream(stream), A, vec, nit, false);
 }
 
+size_t smx_union_workspace_bytes(size_t B, size_t U, size_t K) { return (B * U * K * sizeof(float) + 255) & ~(size_t)255; }
+
+int smx_score_forward_union(int model, void* stream, const float* table, size_t n_rows, const int64_t* idx,
+                            const float* q1, const float* q2, float* score, uint8_t* winner, size_t B, size_t U,
+                            size_t K, size_t dim, const smx_score_params* params, int* err_flag, void* workspace,
+                            size_t workspace_bytes) {
+  using namespace smx;
+  ScoreArgs A;
+  int vec, nit;
+  if (!idx) return fail(SMX_ERR_ARG, "null id tensor");
+  if (U == 0 || U > 255) return fail(SMX_ERR_SHAPE, "1 to 255 union branches");
+  if (B > 0x7fffffffull / U) return fail(SMX_ERR_SHAPE, "too many branch rows");
+  if (int rc = fill_args(&A, &vec, &nit, model, table, n_rows, idx, q1, q2, B * U, K, dim, params, nullptr, nullptr)) return rc;
+  if (!score || !winner) return fail(SMX_ERR_ARG, "null output pointer");
+  if (!workspace || (reinterpret_cast<uintptr_t>(workspace) & 15u) || workspace_bytes < smx_union_workspace_bytes(B, U, K))
+    return fail(SMX_ERR_WORKSPACE, "the union forward needs smx_union_workspace_bytes() of 16-byte aligned workspace");
+  A.U = (int)U;
+  A.score_out = static_cast<float*>(workspace);  // [B*U, K]: every branch's logits
+  A.err = err_flag;
+  hipStream_t st = as_stream(stream);
+  if (int rc = dispatch_model(model, st, A, vec, nit, true)) return rc;
+  const size_t n = B * K;
+  hipLaunchKernelGGL(union_max_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, A.score_out, score, winner,
+                     (int)U, (int)K, n);
+  return check_launch("union maximum");
+}
+
+int smx_score_backward_query_union(int model, void* stream, const float* table, size_t n_rows, const int64_t* idx,
+                                   const float* q1, const float* q2, const float* score, const float* gscore,
+                                   const uint8_t* winner, float* gq1, float* gq2, size_t B, size_t U, size_t K,
+                                   size_t dim, const smx_score_params* params) {
+  using namespace smx;
+  ScoreArgs A;
+  int vec, nit;
+  if (!idx) return fail(SMX_ERR_ARG, "null id tensor");
+  if (U == 0 || U > 255) return fail(SMX_ERR_SHAPE, "1 to 255 union branches");
+  if (B > 0x7fffffffull / U) return fail(SMX_ERR_SHAPE, "too many branch rows");
+  if (int rc = fill_args(&A, &vec, &nit, model, table, n_rows, idx, q1, q2, B * U, K, dim, params, nullptr, nullptr)) return rc;
+  if (!score || !gscore || !winner || !gq1 || (model_nq(model) == 2 && !gq2)) return fail(SMX_ERR_ARG, "null pointer");
+  A.U = (int)U;
+  A.winner = winner;
+  A.score = score;
+  A.gscore = gscore;
+  A.gq1 = gq1;
+  A.gq2 = gq2;
+  return dispatch_model(model, as_stream(stream), A, vec, nit, false);
+}
+
 int smx_score_backward_entity(int model, void* stream, const smx_plan_view* plan, float* table, size_t n_rows,
                               const float* q1, const float* q2, const float* score, const float* gscore, size_t B,
                               size_t K, size_t dim, const smx_score_params* params, float* merged, float* m, float* v,
@@ -292,16 +361,21 @@ int smx_score_backward_entity(int model, void* stream, const smx_plan_view* plan
                          adam, workspace, workspace_bytes, 0, codes, codes_vec, codes_nit);
 }
 
-int smx_score_backward_entity_multi(int model, void* stream, const smx_plan_view* plan, float* table, size_t n_rows,
-                                    const float* q1, const float* q2, const smx_pair_source* src, size_t n_src,
-                                    size_t B, size_t dim, const smx_score_params* params, float* merged, float* m,
-                                    float* v, const smx_opt_params* adam, void* workspace, size_t workspace_bytes,
-                                    const float* grad_rows, size_t n_grad_rows) {
-  using namespace smx;
+}  // extern "C"
+
+namespace smx {
+
+// U: branch rows per query in q1 / q2 (union queries); 1 for every caller but smx_score_backward_entity_union
+static int entity_multi(int model, void* stream, const smx_plan_view* plan, float* table, size_t n_rows,
+                        const float* q1, const float* q2, const smx_pair_source* src, size_t n_src,
+                        size_t B, size_t U, size_t dim, const smx_score_params* params, float* merged, float* m,
+                        float* v, const smx_opt_params* adam, void* workspace, size_t workspace_bytes,
+                        const float* grad_rows, size_t n_grad_rows) {
   if (!src || n_src == 0 || n_src > (size_t)kMaxSources)
     return fail(SMX_ERR_ARG, "1 to %d pair sources", kMaxSources);
   if ((grad_rows != nullptr) != (n_grad_rows != 0)) return fail(SMX_ERR_ARG, "gradient rows and their count must come together");
-  if (n_src == 1 && !grad_rows)
+  if (U == 0 || U > 255) return fail(SMX_ERR_SHAPE, "1 to 255 union branches");
+  if (n_src == 1 && !grad_rows && U == 1)
     return smx_score_backward_entity(model, stream, plan, table, n_rows, q1, q2, src[0].score, src[0].gscore, B,
                                      src[0].K, dim, params, merged, m, v, adam, workspace, workspace_bytes,
                                      src[0].fwd_codes, src[0].fwd_codes_bytes);
@@ -328,8 +402,12 @@ int smx_score_backward_entity_multi(int model, void* stream, const smx_plan_view
     S.gscore[i] = src[i].gscore;
     S.codes[i] = static_cast<const unsigned char*>(src[i].fwd_codes);
     S.K[i] = src[i].K;
+    S.winner[i] = src[i].winner;
+    if (U > 1 && !src[i].winner) return fail(SMX_ERR_ARG, "union queries: pair source %zu has no winner array", i);
     k_sum += src[i].K;
   }
+  S.U = U;
+  if (U > 1 && coded) return fail(SMX_ERR_ARG, "union queries have no sign codes");
   S.grad_rows = grad_rows;
   S.n_grad = n_grad_rows;
   const size_t n_all = B * k_sum + n_grad_rows;
@@ -383,6 +461,28 @@ int smx_score_backward_entity_multi(int model, void* stream, const smx_plan_view
   }
   return entity_backward(model, stream, plan, table, n_rows, q1, q2, nullptr, nullptr, B, k_sum, dim, params, merged, m, v,
                          adam, workspace, workspace_bytes, 0, S.codes[0], codes_vec, codes_nit, &S);
+}
+
+}  // namespace smx
+
+extern "C" {
+
+int smx_score_backward_entity_multi(int model, void* stream, const smx_plan_view* plan, float* table, size_t n_rows,
+                                    const float* q1, const float* q2, const smx_pair_source* src, size_t n_src,
+                                    size_t B, size_t dim, const smx_score_params* params, float* merged, float* m,
+                                    float* v, const smx_opt_params* adam, void* workspace, size_t workspace_bytes,
+                                    const float* grad_rows, size_t n_grad_rows) {
+  return smx::entity_multi(model, stream, plan, table, n_rows, q1, q2, src, n_src, B, 1, dim, params, merged, m, v, adam,
+                           workspace, workspace_bytes, grad_rows, n_grad_rows);
+}
+
+int smx_score_backward_entity_union(int model, void* stream, const smx_plan_view* plan, float* table, size_t n_rows,
+                                    const float* q1, const float* q2, const smx_pair_source* src, size_t n_src,
+                                    size_t B, size_t U, size_t dim, const smx_score_params* params, float* merged,
+                                    float* m, float* v, const smx_opt_params* adam, void* workspace,
+                                    size_t workspace_bytes, const float* grad_rows, size_t n_grad_rows) {
+  return smx::entity_multi(model, stream, plan, table, n_rows, q1, q2, src, n_src, B, U, dim, params, merged, m, v, adam,
+                           workspace, workspace_bytes, grad_rows, n_grad_rows);
 }
 
 }  // extern "C"

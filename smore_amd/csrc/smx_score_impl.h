@@ -36,6 +36,10 @@ struct ScoreArgs {
   float* gq2;
   int B, K, ncol;
   int ids_shared;        // idx holds K ids that every query scores (--share_negative, online_sampler.py:155-157), not B*K
+  // Union queries (kg_reasoning.py:326, box.py:163): q1 / q2 hold U branch rows per query, [B*U, dim]; a kernel's
+  // "query" is then one branch row, number bq = b * U + u, which scores the ids of query b.
+  int U;                 // branches per query (1: none of this)
+  const unsigned char* winner;  // query backward, [B, K]: the branch that gave the pair's logit; a branch row sums its own pairs only
   int id_bits;           // significant bits of n_rows - 1 (at most 32): what the forward compares to find equal ids
   unsigned long long n_rows;
   ScoreParams p;
@@ -275,7 +279,8 @@ __global__ __launch_bounds__(256) void score_forward_kernel(ScoreArgs A, int til
   const int cnt = min(per_wave, K - kw0);
   int bad = 0;
   PairBatch pb{0u, 0u};
-  if (cnt > 0) pb = load_pair_batch(idx, (A.ids_shared ? (size_t)0 : (size_t)b * K) + kw0, cnt, lane, row_len, n_rows, bad);
+  if (cnt > 0)
+    pb = load_pair_batch(idx, (A.ids_shared ? (size_t)0 : (size_t)(b / A.U) * K) + kw0, cnt, lane, row_len, n_rows, bad);
 
   stage_query<M>(lds, q1, q2, b, dim);
   typename ModelOps<M>::Q q[NIT][VEC];
@@ -431,7 +436,7 @@ __global__ __launch_bounds__(NW * 64) void score_backward_query_kernel(ScoreArgs
   int bad = 0;
   for (int kb = kw0; kb < kw1; kb += 64) {
     const int cnt = min(64, kw1 - kb);
-    const size_t first = (size_t)b * K + kb;
+    const size_t first = (size_t)(b / A.U) * K + kb;  // pairs belong to queries, a union's branch rows share them
     const size_t mine = first + min(lane, cnt - 1);
     int my_ps = 0;
     unsigned long long singles = 0ull;  // pairs of the batch that are a segment of their own
@@ -510,8 +515,24 @@ __global__ __launch_bounds__(NW * 64) void score_backward_query_kernel(ScoreArgs
       }
     } else {
     stage_pairs(slab, lane, table, pb, my_c0, my_c1);
+    int n_stream = cnt;
+    if constexpr (SINGLES == 0 && CODES == 0) {
+      if (A.winner) {  // uniform: a branch row of a union query streams the pairs it won, moved to the front of the slab
+        const bool keep = lane < cnt && A.winner[mine] == (unsigned char)(b - (b / A.U) * A.U);
+        const unsigned long long won = __ballot(keep);
+        n_stream = __popcll(won);
+        if (keep) {
+          const unsigned long long addr =
+              (unsigned long long)(table + (((unsigned long long)pb.off_hi << 32) | pb.off_lo));
+          *reinterpret_cast<uint4*>(slab + 4 * lanes_below_in(won)) =
+              make_uint4((unsigned)addr, (unsigned)(addr >> 32), __float_as_uint(my_c0), __float_as_uint(my_c1));
+        }
+        slab_fence();
+      }
+    }
     // lanes past the row end hold a copy of the last column: what they accumulate is never stored
-    stream_batch<MUL, VEC, NIT, RIF>(slab, cnt, dim, ncol, lane,
+    if (n_stream > 0)
+    stream_batch<MUL, VEC, NIT, RIF>(slab, n_stream, dim, ncol, lane,
                                      [&](int j, const Pack<VEC>(&e1)[NIT], const Pack<VEC>(&e2)[NIT]) {
       float2 c = slab_coef(slab, j);
       if constexpr (M == mL2)

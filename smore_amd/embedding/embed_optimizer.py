@@ -61,14 +61,22 @@ class _FusedScoreFunc(torch.autograd.Function):
     autograd but recorded with the optimizer, which reduces it per entity in apply_grad."""
 
     @staticmethod
-    def forward(ctx, embed_opt, dummy_tensor, model, ids, params, q1, q2, for_training=True):
+    def forward(ctx, embed_opt, dummy_tensor, model, ids, params, q1, q2, for_training=True, branches=1):
+        """q1 / q2 [B * branches, dim].  ids [1, K] against more than one query row: negatives shared by the batch
+        (--share_negative), they stay K ids and every row scores them: returns [B * branches, K].  Else ids [B, K];
+        with branches > 1 (union queries) the result is the maximum over a query's branch rows, [B, K], and the
+        second output says which branch held it ([B, K] int64; empty for one branch)."""
         table = embed_opt.sparse_embed.embedding.detach()
-        # ids [1, K] against more than one query: negatives shared by the batch (--share_negative); they stay K ids
         ctx.shared = ids.shape[0] == 1 and q1.shape[0] > 1
+        ctx.branches = 1 if ctx.shared else branches
+        ctx.winner = None
         with torch.no_grad():
             if ctx.shared:
                 codes = None
                 score = fused.score_forward_shared(model, table, ids.reshape(-1), q1, q2, params, embed_opt.err_flag)
+            elif branches > 1:
+                codes = None
+                score, ctx.winner = fused.score_forward_union(model, table, ids, q1, q2, params, branches, embed_opt.err_flag)
             else:
                 # box, l1: the forward leaves 2-bit sign codes from which both backward passes work (None otherwise;
                 # none either when no backward will follow, e.g. scoring sampled negatives under torch.no_grad())
@@ -78,10 +86,12 @@ class _FusedScoreFunc(torch.autograd.Function):
         ctx.save_for_backward(q1.detach(), q2.detach() if q2 is not None else None, score)
         ctx.idx_fwd = embed_opt.n_fwd
         embed_opt.n_fwd += 1
-        return score
+        index = ctx.winner.long() if ctx.winner is not None else torch.empty(0, dtype=torch.int64, device=score.device)
+        ctx.mark_non_differentiable(index)
+        return score, index
 
     @staticmethod
-    def backward(ctx, gscore):
+    def backward(ctx, gscore, _gindex):
         q1, q2, score = ctx.saved_tensors
         opt = ctx.embed_opt
         table = opt.sparse_embed.embedding.detach()
@@ -90,12 +100,15 @@ class _FusedScoreFunc(torch.autograd.Function):
             if ctx.shared:
                 gq1, gq2 = fused.score_backward_query_shared(ctx.model, table, ctx.ids.reshape(-1), q1, q2, score,
                                                              gscore, ctx.params)
+            elif ctx.winner is not None:
+                gq1, gq2 = fused.score_backward_query_union(ctx.model, table, ctx.ids, q1, q2, score, gscore, ctx.winner,
+                                                            ctx.params, ctx.branches)
             else:
                 gq1, gq2 = fused.score_backward_query(ctx.model, table, ctx.ids, q1, q2, score, gscore, ctx.params,
                                                       codes=ctx.codes)
         opt.accumulate_fused(ctx.model, ctx.ids, q1, q2, score, gscore, ctx.params, ctx.idx_fwd, ctx.codes,
-                             shared=ctx.shared)
-        return None, None, None, None, None, gq1, gq2, None
+                             shared=ctx.shared, winner=ctx.winner, branches=ctx.branches)
+        return None, None, None, None, None, gq1, gq2, None, None
 
 
 class EmbeddingOptimizer(ABC):
@@ -198,7 +211,7 @@ class EmbeddingOptimizer(ABC):
 
     # -- protocol of the training loop
     def zero_grad(self):
-        self.poll_pending_id_check()
+        self.poll_pending_id_check(wait=False)   # (never waits for the device: the next step must be free to run ahead)
         self.grad_list, self.fused_list, self.has_grad_list = [], [], []
         self.pending_scores = []
         self.n_fwd = 0
@@ -211,9 +224,10 @@ class EmbeddingOptimizer(ABC):
         self.grad_list.append((indices, grad_submat))
         self.has_grad_list.append(fwd_idx)
 
-    def accumulate_fused(self, model, ids, q1, q2, score, gscore, params, fwd_idx, codes=None, shared=False):
+    def accumulate_fused(self, model, ids, q1, q2, score, gscore, params, fwd_idx, codes=None, shared=False,
+                         winner=None, branches=1):
         self.fused_list.append(dict(model=model, ids=ids, q1=q1, q2=q2, score=score, gscore=gscore, params=params,
-                                    codes=codes, fwd_idx=fwd_idx, shared=shared))
+                                    codes=codes, fwd_idx=fwd_idx, shared=shared, winner=winner, branches=branches))
         self.has_grad_list.append(fwd_idx)
 
     def forward(self, indices, name=None):
@@ -267,6 +281,8 @@ class EmbeddingOptimizer(ABC):
         if r is None:
             return None
         logit = self._score_branches(model, r["ids"], r["q1"], r["q2"], gamma, cen, r["reg"])
+        if logit is None:
+            return None
         return logit if r["q1"].dim() == 4 else logit[:, 0]
 
     def evaluate_pending(self, wanted):
@@ -296,11 +312,8 @@ class EmbeddingOptimizer(ABC):
                 continue
             ids = [p.request["ids"].to(dev) for p in part]
             all_ids = ids[0] if len(ids) == 1 else torch.cat(ids, dim=1)
-            logit = self._score_branches(w["model"], all_ids, w["q1"], w["q2"], w["gamma"], w["cen"], w["reg"])
-            if logit.shape[1] == 1:
-                values, index = logit[:, 0], None
-            else:               # union branches: the first maximal one, as torch.max(logit, dim=1) in the model code
-                values, index = torch.max(logit, dim=1)
+            # (union branches: the first maximal one, as torch.max(logit, dim=1) in the model code)
+            values, index = self._score_max(w["model"], all_ids, w["q1"], w["q2"], w["gamma"], w["cen"], w["reg"])
             sizes = [i.shape[1] for i in ids]
             parts = [values] if len(ids) == 1 else torch.split(values, sizes, dim=1)
             iparts = [index] * len(ids) if (index is None or len(ids) == 1) else torch.split(index, sizes, dim=1)
@@ -317,11 +330,12 @@ class EmbeddingOptimizer(ABC):
         Union queries: q1/q2 of shape [B,U,dim] or [B,U,1,dim] (the merged branch embeddings of
         kg_reasoning.py:326) give max over the U branches of each branch's logit, as the last line of
         every custom_cal_logit does (box.py:163, vec.py:89, rotate.py:141, beta.py:307)."""
-        logit = self._score_branches(model, ids, q1, q2, gamma, cen, regularizer)
-        return torch.max(logit, dim=1)[0] if logit.shape[1] > 1 else logit[:, 0]
+        return self._score_max(model, ids, q1, q2, gamma, cen, regularizer)[0]
 
-    def _score_branches(self, model, ids, q1, q2, gamma, cen, regularizer):
-        """[B, branches, K] logits of every union branch of every query against that query's negatives."""
+    def _launch(self, model, ids, q1, q2, gamma, cen, regularizer):
+        """One launch of the fused scorer.  Returns (b, branches, shared, scores, index): scores [B * branches, K]
+        for one branch or for ids shared by the batch, else (union queries with their own ids) the maximum over the
+        branches [B, K] with index [B, K], the branch that held it."""
         table = self.sparse_embed.embedding
         b = q1.shape[0]
         dim = q1.shape[-1]
@@ -331,19 +345,38 @@ class EmbeddingOptimizer(ABC):
         ids = ids.to(table.device)
         if ids.dim() != 2:
             raise _lib.SmxError("ids must be [B,K] or [1,K]")
-        if ids.shape[0] == 1 and b * branches > 1:
-            pass                # shared by the batch: every query row (every branch of every query) scores the same K ids
-        elif ids.shape[0] != b:
+        shared = ids.shape[0] == 1 and b * branches > 1     # every query row (every branch of every query) scores the same K ids
+        if not shared and ids.shape[0] != b:
             raise _lib.SmxError("ids must be [B,K] or [1,K]")
-        elif branches > 1:      # every branch of a query scores that query's negatives
-            ids = ids.repeat_interleave(branches, dim=0)
-        ids = ids.contiguous()
         q1c = q1.reshape(b * branches, dim).contiguous()
         q2c = None if q2 is None else q2.reshape(b * branches, dim).contiguous()
         params = fused.score_params(gamma, cen, regularizer)
         self.stats["fused_launches"] += 1
-        logit = _FusedScoreFunc.apply(self, self.dummy_tensor, model, ids, params, q1c, q2c, torch.is_grad_enabled())
-        return logit.view(b, branches, -1)
+        scores, index = _FusedScoreFunc.apply(self, self.dummy_tensor, model, ids.contiguous(), params, q1c, q2c,
+                                              torch.is_grad_enabled(), branches)
+        return b, branches, shared, scores, index
+
+    def _score_max(self, model, ids, q1, q2, gamma, cen, regularizer):
+        """(values [B, K], index [B, K] or None): the maximum over the union branches of each branch's logit and the
+        first branch that holds it, as torch.max(logit, dim=1) of the custom_cal_logit bodies; one branch: the logits
+        and None.  Queries with their own ids take the maximum inside the scorer; for ids shared by the batch the
+        branch rows are scored like queries and torch.max runs on [B, U, K]."""
+        b, branches, shared, scores, index = self._launch(model, ids, q1, q2, gamma, cen, regularizer)
+        if branches == 1:
+            return scores, None
+        if shared:
+            return torch.max(scores.view(b, branches, -1), dim=1)
+        return scores, index
+
+    def _score_branches(self, model, ids, q1, q2, gamma, cen, regularizer):
+        """[B, branches, K] logits of every union branch of every query, for code that wants them before the maximum;
+        None for union queries with their own ids, whose branches meet inside the scorer."""
+        b = q1.shape[0]
+        branches = q1.numel() // (b * q1.shape[-1])
+        if branches > 1 and not (ids.dim() == 2 and ids.shape[0] == 1):
+            return None
+        b, branches, shared, scores, _ = self._launch(model, ids, q1, q2, gamma, cen, regularizer)
+        return scores.view(b, branches, -1)
 
     def _raise_for(self, code):
         if code == 2:
@@ -359,11 +392,14 @@ class EmbeddingOptimizer(ABC):
             self.err_flag.zero_()
         self._raise_for(code)
 
-    def poll_pending_id_check(self):
+    def poll_pending_id_check(self, wait=True):
         """Looks at the flag a finished step left in pinned host memory, if one is waiting (see
         _check_ids_one_step_late), and raises for it.  Called wherever the next step, or the end of training, passes
-        by: apply_grad (also one that has nothing to apply), zero_grad, saving the table's state_dict."""
+        by: zero_grad (only if the copy has already landed), the start of apply_grad -- also of one that has nothing
+        to apply --, saving the table's state_dict."""
         if self._flag_event is not None:
+            if not wait and not self._flag_event.query():
+                return
             self._flag_event.synchronize()
             self._flag_event = None
             code = int(self._flag_host[0])
@@ -373,11 +409,11 @@ class EmbeddingOptimizer(ABC):
 
     def _check_ids_one_step_late(self):
         """The per-step check without draining the queue: this step's flag is copied to pinned host memory behind
-        the update, and looked at when the next step gets here -- by then the copy has long finished, so the host
-        keeps running ahead of the device.  The step that met the bad id has by then scored row 0 in its place: its
-        loss and the gradients of the dense parameters are those of a wrong lookup (no table row was updated for
-        the bad id).  check_ids() after the step, or check_ids_synchronously = True, fails before anything uses them."""
-        self.poll_pending_id_check()
+        the update, and looked at when the next step reaches its apply_grad (before that update is applied) -- by
+        then the copy has long finished, so the host keeps running ahead of the device.  The step that met the bad id
+        has by then scored row 0 in its place: its loss and the gradients of the dense parameters are those of a wrong
+        lookup (no table row was updated for the bad id).  check_ids() after the step, or check_ids_synchronously =
+        True, fails before anything uses them."""
         self._flag_host.copy_(self.err_flag, non_blocking=True)
         self._flag_event = torch.cuda.Event()
         self._flag_event.record()
@@ -389,8 +425,8 @@ class EmbeddingOptimizer(ABC):
         from the apply_grad of the following step, so that no step waits for the device; check_ids() asks at once."""
         self.step += 1  # counts calls, also those without gradients (embed_optimizer.py:156)
         self.pending_scores = []    # logits that nothing used have no gradient and must not ride along later
+        self.poll_pending_id_check()    # the previous step's flag, before this step's update is applied
         if not self.grad_list and not self.fused_list:
-            self.poll_pending_id_check()
             return
         self._apply_grad(lr)
         if self.check_ids_synchronously:
@@ -456,8 +492,7 @@ class EmbeddingOptimizer(ABC):
                     fused.score_backward_entity_shared(rec["model"], table, rec["ids"].reshape(-1), rec["q1"], rec["q2"],
                                                        rec["score"], rec["gscore"], rec["params"], plan=plan, merged=merged)
                 else:
-                    fused.score_backward_entity(rec["model"], plan, table, rec["q1"], rec["q2"], rec["score"],
-                                                rec["gscore"], rec["params"], merged=merged, codes=rec["codes"])
+                    self._entity_pass(plan, [rec], merged=merged)
                 idx_list.append(plan.uniq)
                 grad_list.append(merged)
             # (a single record is used as it is: torch.cat would copy its gradient rows)
@@ -465,6 +500,21 @@ class EmbeddingOptimizer(ABC):
             rows = grad_list[0] if len(grad_list) == 1 else torch.cat(grad_list, dim=0)
             plan = fused.build_plan(flat, n_rows, err_flag=self.err_flag)
             self.update_from_plan(plan, rows.contiguous(), lr)
+
+    def _entity_pass(self, plan, recs, merged=None, m=None, v=None, adam=None, grad_rows=None):
+        """The fused entity pass over the plan of the records' ids (per-query records of one query batch, in the
+        order of the plan), then grad_rows: merged rows and / or the optimizer update."""
+        table = self.sparse_embed.embedding.detach()
+        first = recs[0]
+        if len(recs) == 1 and grad_rows is None and first["branches"] == 1:
+            fused.score_backward_entity(first["model"], plan, table, first["q1"], first["q2"], first["score"],
+                                        first["gscore"], first["params"], merged=merged, m=m, v=v, adam=adam,
+                                        codes=first["codes"])
+            return
+        sources = [(r["score"], r["gscore"], r["codes"]) + ((r["winner"],) if first["branches"] > 1 else ()) for r in recs]
+        fused.score_backward_entity_multi(first["model"], plan, table, first["q1"], first["q2"], sources, first["params"],
+                                          merged=merged, m=m, v=v, adam=adam, grad_rows=grad_rows,
+                                          branches=first["branches"])
 
     @staticmethod
     def _one_query_batch(recs):
@@ -529,10 +579,7 @@ class _RowOptimizer(EmbeddingOptimizer):
 
     def update_fused_multi(self, plan, recs, lr, grad_rows=None):
         m, v = self._state()
-        first = recs[0]
-        fused.score_backward_entity_multi(first["model"], plan, self.sparse_embed.embedding.detach(), first["q1"],
-                                          first["q2"], [(r["score"], r["gscore"], r["codes"]) for r in recs],
-                                          first["params"], m=m, v=v, adam=self._params(lr), grad_rows=grad_rows)
+        self._entity_pass(plan, recs, m=m, v=v, adam=self._params(lr), grad_rows=grad_rows)
 
     def update_shared(self, plan, rec, lr):
         m, v = self._state()
@@ -542,9 +589,7 @@ class _RowOptimizer(EmbeddingOptimizer):
 
     def update_fused(self, plan, rec, lr):
         m, v = self._state()
-        fused.score_backward_entity(rec["model"], plan, self.sparse_embed.embedding.detach(), rec["q1"], rec["q2"],
-                                    rec["score"], rec["gscore"], rec["params"], m=m, v=v, adam=self._params(lr),
-                                    codes=rec["codes"])
+        self._entity_pass(plan, [rec], m=m, v=v, adam=self._params(lr))
 
 
 class AdamEmbedOptimizer(_RowOptimizer):

@@ -317,13 +317,54 @@ def score_backward_entity(model, plan, table, q1, q2, score, gscore, params, mer
                   _ptr(codes), 0 if codes is None else codes.numel())
 
 
+def score_forward_union(model, table, idx, q1, q2, params, branches, err_flag=None):
+    """Union queries: q1 / q2 [B * branches, dim] (a query's branch rows adjacent), idx [B, K].  Returns
+    (score [B, K] = the maximum over the branches, winner [B, K] uint8 = the first branch that holds it)."""
+    if model not in MODELS:
+        raise _lib.SmxError(f"unknown score model {model}")
+    _f32(table, "table")
+    _f32(q1, "q1")
+    _f32(q2, "q2")
+    dim = q1.shape[-1]
+    bu = q1.numel() // dim
+    if bu % branches or idx.dim() != 2 or idx.shape[0] * branches != bu or idx.dtype != torch.int64 or \
+            not idx.is_contiguous() or idx.device != table.device:
+        raise _lib.SmxError("union scoring takes idx [B, K] int64 and query tensors [B * branches, dim]")
+    b, k = idx.shape
+    score = torch.empty((b, k), dtype=torch.float32, device=table.device)
+    winner = torch.empty((b, k), dtype=torch.uint8, device=table.device)
+    with torch.cuda.device(table.device):
+        ws = _workspace(_lib.load().smx_union_workspace_bytes(b, branches, k), table.device)
+        _lib.call("smx_score_forward_union", MODELS[model], _stream(table), _ptr(table), table.shape[0], _ptr(idx),
+                  _ptr(q1), _ptr(q2), _ptr(score), _ptr(winner), b, branches, k, dim, ctypes.byref(params),
+                  _ptr(err_flag), _ptr(ws), ws.numel())
+    return score, winner
+
+
+def score_backward_query_union(model, table, idx, q1, q2, score, gscore, winner, params, branches):
+    """Gradients of sum(gscore * score) w.r.t. the branch rows q1 (and q2), [B * branches, dim]."""
+    _f32(score, "score")
+    _f32(gscore, "gscore")
+    b, k = idx.shape
+    dim = q1.shape[-1]
+    gq1 = torch.empty_like(q1)
+    gq2 = None if q2 is None else torch.empty_like(q2)
+    with torch.cuda.device(table.device):
+        _lib.call("smx_score_backward_query_union", MODELS[model], _stream(table), _ptr(table), table.shape[0], _ptr(idx),
+                  _ptr(q1), _ptr(q2), _ptr(score), _ptr(gscore), _ptr(winner), _ptr(gq1), _ptr(gq2), b, branches, k,
+                  dim, ctypes.byref(params))
+    return gq1, gq2
+
+
 def score_backward_entity_multi(model, plan, table, q1, q2, sources, params, merged=None, m=None, v=None, adam=None,
-                                grad_rows=None):
+                                grad_rows=None, branches=1):
     """score_backward_entity for several index streams of one query batch (see smx_score_backward_entity_multi).
-    sources: list of (score [B,K_s], gscore [B,K_s], codes or None); plan: built over the concatenation of the
-    streams' flattened ids in the same order.  grad_rows [n, row]: materialised gradient rows of the step's plain
-    lookups, whose ids are the last n entries of that concatenation."""
-    b, dim = q1.shape[0], q1.shape[-1]
+    sources: list of (score [B,K_s], gscore [B,K_s], codes or None[, winner]); plan: built over the concatenation of
+    the streams' flattened ids in the same order.  grad_rows [n, row]: materialised gradient rows of the step's plain
+    lookups, whose ids are the last n entries of that concatenation.  branches > 1: union queries, q1 / q2 are
+    [B * branches, dim] and every source brings its winner array (smx_score_backward_entity_union)."""
+    dim = q1.shape[-1]
+    b = q1.numel() // (dim * branches)
     if model not in MODELS:
         raise _lib.SmxError(f"unknown score model {model}")
     if not 1 <= len(sources) <= _lib.MAX_PAIR_SOURCES:
@@ -331,13 +372,17 @@ def score_backward_entity_multi(model, plan, table, q1, q2, sources, params, mer
     for t, name in ((table, "table"), (q1, "q1"), (q2, "q2"), (merged, "merged"), (m, "m"), (v, "v")):
         _f32(t, name)
     arr = (_lib.PairSource * len(sources))()
-    for i, (score, gscore, codes) in enumerate(sources):
+    for i, src in enumerate(sources):
+        score, gscore, codes = src[:3]
+        winner = src[3] if len(src) > 3 else None
         _f32(score, "score")
         _f32(gscore, "gscore")
         if score.numel() % b or gscore.shape != score.shape:
             raise _lib.SmxError("score and gscore of a source must both be [B, K]")
+        if (branches > 1) != (winner is not None):
+            raise _lib.SmxError("union queries, and only they, bring a winner array per source")
         arr[i] = _lib.PairSource(_ptr(score), _ptr(gscore), _ptr(codes), 0 if codes is None else codes.numel(),
-                                 score.numel() // b)
+                                 score.numel() // b, _ptr(winner))
     row_len = table.shape[1]
     _check_state(table, m, v, adam)
     if merged is not None and (merged.dim() != 2 or merged.shape[1] != row_len):
@@ -351,10 +396,16 @@ def score_backward_entity_multi(model, plan, table, q1, q2, sources, params, mer
     with torch.cuda.device(table.device):
         ws = _workspace(_lib.load().smx_entity_workspace_bytes(plan.n_pairs, row_len), table.device)
         view = plan.view()
-        _lib.call("smx_score_backward_entity_multi", MODELS[model], _stream(table), ctypes.byref(view), _ptr(table),
-                  table.shape[0], _ptr(q1), _ptr(q2), ctypes.cast(arr, ctypes.c_void_p), len(sources), b, dim,
-                  ctypes.byref(params), _ptr(merged), _ptr(m), _ptr(v), None if adam is None else ctypes.byref(adam),
-                  _ptr(ws), ws.numel(), _ptr(grad_rows), n_grad)
+        if branches > 1:
+            _lib.call("smx_score_backward_entity_union", MODELS[model], _stream(table), ctypes.byref(view), _ptr(table),
+                      table.shape[0], _ptr(q1), _ptr(q2), ctypes.cast(arr, ctypes.c_void_p), len(sources), b, branches,
+                      dim, ctypes.byref(params), _ptr(merged), _ptr(m), _ptr(v),
+                      None if adam is None else ctypes.byref(adam), _ptr(ws), ws.numel(), _ptr(grad_rows), n_grad)
+        else:
+            _lib.call("smx_score_backward_entity_multi", MODELS[model], _stream(table), ctypes.byref(view), _ptr(table),
+                      table.shape[0], _ptr(q1), _ptr(q2), ctypes.cast(arr, ctypes.c_void_p), len(sources), b, dim,
+                      ctypes.byref(params), _ptr(merged), _ptr(m), _ptr(v),
+                      None if adam is None else ctypes.byref(adam), _ptr(ws), ws.numel(), _ptr(grad_rows), n_grad)
 
 
 def score_backward_fused(model, plan, table, idx, q1, q2, score, gscore, params, merged=None, m=None, v=None,

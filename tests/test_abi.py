@@ -75,18 +75,18 @@ def test_multi_stream_entity_pass_refuses_bad_source_lists():
     src = (_lib.PairSource * 5)()
     fake = c.c_void_p(256)          # never dereferenced: every case below is refused on the host
     for i in range(5):
-        src[i] = _lib.PairSource(fake, fake, None, 0, 4)
+        src[i] = _lib.PairSource(fake, fake, None, 0, 4, None)
     call = lambda n_src, b=2, rows=None, n_rows=0: lib.smx_score_backward_entity_multi(
         2, None, c.byref(plan), fake, 100, fake, fake, c.cast(src, c.c_void_p), n_src, b, 8, c.byref(params), fake, None,
         None, None, fake, 1 << 20, rows, n_rows)
     assert call(0) != 0 and call(5) != 0
     assert b"pair sources" in lib.smx_last_error()
     assert call(2, b=7) != 0 and b"pairs" in lib.smx_last_error()          # 2 sources x 7 x 4 pairs, the plan holds 40
-    src[1] = _lib.PairSource(fake, fake, fake, 64, 4)                       # sign codes for one source only
+    src[1] = _lib.PairSource(fake, fake, fake, 64, 4, None)                       # sign codes for one source only
     assert call(2, b=5) != 0 and b"sign codes" in lib.smx_last_error()
-    src[1] = _lib.PairSource(fake, None, None, 0, 4)
+    src[1] = _lib.PairSource(fake, None, None, 0, 4, None)
     assert call(2, b=5) != 0 and b"incomplete" in lib.smx_last_error()
-    src[1] = _lib.PairSource(fake, fake, None, 0, 4)
+    src[1] = _lib.PairSource(fake, fake, None, 0, 4, None)
     assert call(2, b=5, rows=fake, n_rows=0) != 0 and b"gradient rows" in lib.smx_last_error()
     assert call(2, b=5, rows=None, n_rows=3) != 0 and b"gradient rows" in lib.smx_last_error()
     assert call(2, b=5, rows=fake, n_rows=3) != 0 and b"gradient rows" in lib.smx_last_error()   # the plan holds 40, not 43

@@ -332,9 +332,10 @@ def test_out_of_range_lookup_is_reported():
 
 
 def test_out_of_range_id_in_a_step_raises_when_the_next_step_begins():
-    """The per-step check does not wait for the device: the flag of step n is read where step n+1 first passes by
-    -- its zero_grad (or an apply_grad without gradients, or saving the table).  The bad pair itself updates no row
-    (its key sorts behind every real segment)."""
+    """The per-step check does not wait for the device: the flag of step n is read where step n+1 passes by -- its
+    zero_grad if the flag has landed by then, its apply_grad at the latest (before that update is applied; also an
+    apply_grad without gradients), or saving the table.  The bad pair itself updates no row (its key sorts behind
+    every real segment)."""
     emb, opt = _setup(20, 8, 9)
     c = torch.zeros(2, 1, 8, device="cuda", requires_grad=True)
     o = torch.ones(2, 1, 8, device="cuda", requires_grad=True)
@@ -349,6 +350,9 @@ def test_out_of_range_id_in_a_step_raises_when_the_next_step_begins():
     step([[1, 25], [2, 3]])
     with pytest.raises(IndexError):
         opt.zero_grad()
+        step([[4, 5], [6, 7]])
+    changed = (emb.embedding.detach() != w0).any(dim=1).nonzero().flatten().tolist()
+    assert changed == [1, 2, 3], "the step that finds the flag raised is not applied"
     opt.zero_grad()       # the flag was cleared when the error was raised
     step([[4, 5], [6, 7]])
     changed = (emb.embedding.detach() != w0).any(dim=1).nonzero().flatten().tolist()

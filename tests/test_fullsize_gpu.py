@@ -5,6 +5,8 @@ random subsample of queries and of touched entities, and (b) through size-indepe
 bit-exact integer invariants of the segment plan, untouched rows staying bit-identical (row
 checksums), exact linearity of the backward in the upstream gradient (scaling by 2 is exact in
 fp32), and run-to-run determinism."""
+import gc
+
 import numpy as np
 import pytest
 import torch
@@ -47,6 +49,8 @@ def test_full_size_workload(cfg_id):
     from smore_amd import fused
     cfg = bench.CONFIGS[cfg_id]
     dev = torch.device("cuda:0")
+    gc.collect()
+    torch.cuda.empty_cache()    # what an earlier test of this size has released is still held by the caching allocator
     free, _ = torch.cuda.mem_get_info()
     need = cfg["n"] * bench.row_len(cfg) * 4 * (3 if cfg["adam"] else 1) + (4 << 30)
     if free < need:
@@ -230,3 +234,100 @@ def test_plan_around_the_tile_geometry_boundaries():
         heads[1:] = want_ids[1:] != want_ids[:-1]
         assert plan.n_uniq == int(heads.sum().item())
         assert torch.equal(plan.seg_start[: plan.n_uniq].long(), torch.nonzero(heads).reshape(-1))
+
+
+def test_full_size_dropin_flow():
+    """The 86M-entity step as SMORE's own code reaches it: lookup handles for positives and negatives, the box
+    model's cal_logit (box.py:157-164) on them, backward, apply_grad -- nothing but the reference's call sequence
+    (kg_reasoning.py:298-307, 340-355; train_process.py:172-220).  No lookup may be materialised and no logit may
+    leave the fused scorer; logits, relation gradients and the Adam state of sampled entities (the three hottest
+    included) against the float64 oracle; rows outside the touched set bit-identical."""
+    import types
+    from smore_amd.embedding.embed_optimizer import AdamEmbedOptimizer
+    from smore_amd.embedding.sparse_embed import SparseEmbedding
+    from smore_amd.torchext.ext_ops import box_dist_in, box_dist_out
+    cfg = bench.CONFIGS[5]
+    dev = torch.device("cuda:0")
+    gc.collect()
+    torch.cuda.empty_cache()    # what an earlier test of this size has released is still held by the caching allocator
+    free, _ = torch.cuda.mem_get_info()
+    need = cfg["n"] * bench.row_len(cfg) * 4 * 3 + (6 << 30)
+    if free < need:
+        pytest.skip(f"needs {need >> 30} GiB of HBM, {free >> 30} free")
+    table, q1, q2, idx, gs = bench.make_inputs(cfg, dev, 20245)
+    n, b, k, lr = cfg["n"], cfg["b"], cfg["k"], cfg["lr"]
+    rng = np.random.default_rng(55)
+    emb = SparseEmbedding(8, cfg["dim"])
+    emb.embedding = torch.nn.Parameter(table, requires_grad=True)
+    emb.num_rows = n
+    opt = AdamEmbedOptimizer(types.SimpleNamespace(optim_mode="(aggr,adam,gpu,False,5)", share_optim_stats=True), emb, 0)
+    gamma = torch.nn.Parameter(torch.tensor([cfg["gamma"]], device=dev), requires_grad=False)
+    rel_c, rel_o = q1.clone().requires_grad_(True), q2.clone().requires_grad_(True)
+    pos = idx[:, 7].contiguous()
+    gp = gs[:, :1].contiguous()
+
+    def cal_logit(rows, center, offset):
+        return torch.max(gamma - box_dist_out(rows, center, offset) - cfg["cen"] * box_dist_in(rows, center, offset), dim=1)[0]
+
+    ids_all = torch.cat([pos[:, None], idx], dim=1)
+    gs_all = torch.cat([gp, gs], dim=1)
+    uniq = torch.unique(ids_all)
+    sample = np.unique(np.concatenate([rng.choice(uniq.numel(), size=40, replace=False), np.arange(3)]))
+    sample_ids = uniq[torch.as_tensor(sample, device=dev)].tolist()
+    w_before = {e: table[e].clone() for e in sample_ids}
+    row_sum_before = table.detach().sum(dim=1)
+    qs = np.sort(rng.choice(b, size=16, replace=False))           # queries whose logits and gradients the oracle checks
+    qs_t = torch.as_tensor(qs, device=dev)
+    rows_q = table.detach()[ids_all[qs_t]].cpu().numpy().astype(np.float64)      # [16, 1 + K, row], before the update
+
+    opt.zero_grad()
+    center, offset = rel_c.view(b, 1, 1, -1), rel_o.view(b, 1, 1, -1)
+    p_rows = emb(pos, "positive_entity")
+    n_rows = emb(idx.view(-1), "negative_entity")
+    lp = cal_logit(p_rows.unsqueeze(1), center, offset)
+    ln = cal_logit(n_rows.view(b, k, -1), center, offset)
+    ((lp * gp).sum() + (ln * gs).sum()).backward()
+    assert opt.stats == dict(fused_launches=1, materialized_lookups=0, dense_fallbacks=0, per_record_merges=0)
+    opt.apply_grad(lr)
+    opt.check_ids()
+    assert opt.stats["per_record_merges"] == 0 and opt.stats["materialized_lookups"] == 0
+
+    got_logit = torch.cat([lp, ln], dim=1).detach()
+
+    # entity side: first moment and weights of the sampled entities from their saved rows, all their pairs
+    flat_ids = ids_all.reshape(-1)
+    m = emb.state_sum_fo
+    hottest = 0
+    for e in sample_ids:
+        pairs = (flat_ids == e).nonzero().flatten()
+        hottest = max(hottest, pairs.numel())
+        want, sum_abs = _oracle_segment_gradient("box", w_before[e], q1, q2, pairs, k + 1, gs_all, cfg["cen"])
+        got_m = m[e].cpu().numpy().astype(np.float64)
+        assert_close(got_m, 0.1 * want, REL_F32, f"drop-in flow: first moment of entity {e}", sum_abs=0.1 * sum_abs)
+        w0 = w_before[e].cpu().numpy().astype(np.float64)
+        wn, mn, vn = w0[None].copy(), np.zeros((1, w0.size)), np.zeros((1, w0.size))
+        orc.adam_rows(wn, mn, vn, np.array([0]), (got_m / 0.1)[None], lr, 1)
+        assert_close(table[e].detach().cpu().numpy(), wn[0], REL_F32, f"drop-in flow: weights of entity {e}")
+        # this entity's logits, from its saved row, for up to 64 of its pairs
+        part = pairs[:64]
+        pb = (part // (k + 1)).cpu().numpy()
+        erow = np.broadcast_to(w0, (part.numel(), 1, w0.size))
+        a1 = q1[torch.as_tensor(pb, device=dev)].cpu().numpy().astype(np.float64)[:, None]
+        a2 = q2[torch.as_tensor(pb, device=dev)].cpu().numpy().astype(np.float64)[:, None]
+        want_logit = orc.score_forward("box", np.ascontiguousarray(erow), a1, a2, cfg["gamma"], cfg["cen"])[:, 0]
+        assert_close(got_logit.reshape(-1)[part].cpu().numpy(), want_logit, REL_F32, f"drop-in flow: logits of entity {e}",
+                     rms_floor=False)
+    assert hottest > 100000, hottest
+
+    # logits and relation gradients of the sampled queries
+    oq1 = q1[qs_t].cpu().numpy().astype(np.float64)[:, None]
+    oq2 = q2[qs_t].cpu().numpy().astype(np.float64)[:, None]
+    assert_close(got_logit[qs_t].cpu().numpy(), orc.score_forward("box", rows_q, oq1, oq2, cfg["gamma"], cfg["cen"]),
+                 REL_F32, "drop-in flow: logits of sampled queries", rms_floor=False)
+    _, o1, o2 = orc.score_backward("box", gs_all[qs_t].cpu().numpy().astype(np.float64), rows_q, oq1, oq2, cfg["cen"])
+    assert_close(rel_c.grad[qs_t].cpu().numpy(), o1[:, 0], REL_F32, "drop-in flow: center gradient of sampled queries")
+    assert_close(rel_o.grad[qs_t].cpu().numpy(), o2[:, 0], REL_F32, "drop-in flow: offset gradient of sampled queries")
+
+    # touched-row set: only rows of the step's ids may have changed
+    changed = (table.detach().sum(dim=1) != row_sum_before).nonzero().flatten()
+    assert bool(torch.isin(changed, uniq).all()), "a row outside the touched set changed"

@@ -29,6 +29,10 @@ class RecordingOptimizer:
         self.looked_up.append(name)
         return self.sparse_embed.embedding[ids]
 
+    def _score_max(self, model, ids, q1, q2, gamma, cen, reg):
+        logit = self._score_branches(model, ids, q1, q2, gamma, cen, reg)
+        return (logit[:, 0], None) if logit.shape[1] == 1 else torch.max(logit, dim=1)
+
     def _score_branches(self, model, ids, q1, q2, gamma, cen, reg):
         """[B, U, K] logits, as the real optimizer's launch returns them."""
         self.scored.append((model, tuple(ids.shape), gamma, cen, reg))
