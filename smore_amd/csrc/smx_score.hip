@@ -40,6 +40,16 @@ int entity_backward(int model, void* stream, const smx_plan_view* plan, float* t
 size_t entity_ws_bytes(size_t n_pairs, size_t row_len);
 size_t code_bytes_per_pair(size_t dim);
 
+// defined in smx_beta_shared.hip
+bool beta_shared_fits(size_t dim, const void* table, const void* q1, const void* q2, const void* workspace,
+                      size_t workspace_bytes, size_t K, bool forward);
+int beta_shared_forward(hipStream_t st, const float* table, size_t n_rows, const long long* ids, const float* q1,
+                        const float* q2, float* score, size_t B, size_t K, size_t dim, const ScoreParams& p, int* err,
+                        float* terms);
+int beta_shared_backward_query(hipStream_t st, const float* table, size_t n_rows, const long long* ids, const float* q1,
+                               const float* q2, const float* gscore, float* gq1, float* gq2, size_t B, size_t K,
+                               size_t dim, const ScoreParams& p, float* terms);
+
 // One extra stream and two events per device, created at first use and kept for the life of the process.
 struct SideStream {
   hipStream_t stream = nullptr;
@@ -218,15 +228,23 @@ int smx_score_backward_query(int model, void* stream, const float* table, size_t
   return dispatch_model(model, as_stream(stream), A, vec, nit, false);
 }
 
+size_t smx_shared_workspace_bytes(int model, size_t K, size_t dim) {
+  return model == smx::mBetaKL ? ((K * 6 * dim * sizeof(float) + 255) & ~(size_t)255) : 0;
+}
+
 int smx_score_forward_shared(int model, void* stream, const float* table, size_t n_rows, const int64_t* ids,
                              const float* q1, const float* q2, float* score, size_t B, size_t K, size_t dim,
-                             const smx_score_params* params, int* err_flag) {
+                             const smx_score_params* params, int* err_flag, void* workspace, size_t workspace_bytes) {
   using namespace smx;
   ScoreArgs A;
   int vec, nit;
   if (!ids) return fail(SMX_ERR_ARG, "null id list");
   if (int rc = fill_args(&A, &vec, &nit, model, table, n_rows, ids, q1, q2, B, K, dim, params, nullptr, nullptr)) return rc;
   if (!score) return fail(SMX_ERR_ARG, "null score pointer");
+  // BetaE: the entity side of the divergence once per shared row (needs the workspace for the rows' terms)
+  if (model == mBetaKL && beta_shared_fits(dim, table, q1, q2, workspace, workspace_bytes, K, true))
+    return beta_shared_forward(as_stream(stream), table, n_rows, reinterpret_cast<const long long*>(ids), q1, q2, score, B,
+                               K, dim, A.p, err_flag, static_cast<float*>(workspace));
   A.ids_shared = 1;
   A.score_out = score;
   A.err = err_flag;
@@ -236,13 +254,17 @@ int smx_score_forward_shared(int model, void* stream, const float* table, size_t
 int smx_score_backward_query_shared(int model, void* stream, const float* table, size_t n_rows, const int64_t* ids,
                                     const float* q1, const float* q2, const float* score, const float* gscore,
                                     float* gq1, float* gq2, size_t B, size_t K, size_t dim,
-                                    const smx_score_params* params) {
+                                    const smx_score_params* params, void* workspace, size_t workspace_bytes) {
   using namespace smx;
   ScoreArgs A;
   int vec, nit;
   if (!ids) return fail(SMX_ERR_ARG, "null id list");
   if (int rc = fill_args(&A, &vec, &nit, model, table, n_rows, ids, q1, q2, B, K, dim, params, nullptr, nullptr)) return rc;
   if (!score || !gscore || !gq1 || (model_nq(model) == 2 && !gq2)) return fail(SMX_ERR_ARG, "null pointer");
+  if (model == mBetaKL && aligned16(gq1) && aligned16(gq2) &&
+      beta_shared_fits(dim, table, q1, q2, workspace, workspace_bytes, K, false))
+    return beta_shared_backward_query(as_stream(stream), table, n_rows, reinterpret_cast<const long long*>(ids), q1, q2,
+                                      gscore, gq1, gq2, B, K, dim, A.p, static_cast<float*>(workspace));
   A.ids_shared = 1;
   A.score = score;
   A.gscore = gscore;

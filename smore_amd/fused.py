@@ -129,17 +129,25 @@ def _shared_dims(model, table, ids, q1, q2):
     return b, ids.numel(), dim
 
 
-def score_forward_shared(model, table, ids, q1, q2, params, err_flag=None):
-    """logit[b,k] = gamma - dist(table[ids[k]], q[b]) for K ids that every query scores (--share_negative)."""
+def _shared_workspace(model, k, dim, device, use):
+    nbytes = _lib.load().smx_shared_workspace_bytes(MODELS[model], k, dim) if use else 0
+    return _workspace(nbytes, device) if nbytes else None
+
+
+def score_forward_shared(model, table, ids, q1, q2, params, err_flag=None, per_row_terms=True):
+    """logit[b,k] = gamma - dist(table[ids[k]], q[b]) for K ids that every query scores (--share_negative).
+    per_row_terms=False keeps beta_kl on the per-pair kernels (no workspace for the rows' terms; for comparison)."""
     b, k, dim = _shared_dims(model, table, ids, q1, q2)
     score = torch.empty((b, k), dtype=torch.float32, device=table.device)
     with torch.cuda.device(table.device):
+        ws = _shared_workspace(model, k, dim, table.device, per_row_terms)
         _lib.call("smx_score_forward_shared", MODELS[model], _stream(table), _ptr(table), table.shape[0], _ptr(ids),
-                  _ptr(q1), _ptr(q2), _ptr(score), b, k, dim, ctypes.byref(params), _ptr(err_flag))
+                  _ptr(q1), _ptr(q2), _ptr(score), b, k, dim, ctypes.byref(params), _ptr(err_flag), _ptr(ws),
+                  0 if ws is None else ws.numel())
     return score
 
 
-def score_backward_query_shared(model, table, ids, q1, q2, score, gscore, params):
+def score_backward_query_shared(model, table, ids, q1, q2, score, gscore, params, per_row_terms=True):
     """Gradients of sum(gscore * score) w.r.t. q1 (and q2) for shared ids."""
     b, k, dim = _shared_dims(model, table, ids, q1, q2)
     _f32(score, "score")
@@ -147,9 +155,10 @@ def score_backward_query_shared(model, table, ids, q1, q2, score, gscore, params
     gq1 = torch.empty_like(q1)
     gq2 = None if q2 is None else torch.empty_like(q2)
     with torch.cuda.device(table.device):
+        ws = _shared_workspace(model, k, dim, table.device, per_row_terms)
         _lib.call("smx_score_backward_query_shared", MODELS[model], _stream(table), _ptr(table), table.shape[0],
                   _ptr(ids), _ptr(q1), _ptr(q2), _ptr(score), _ptr(gscore), _ptr(gq1), _ptr(gq2), b, k, dim,
-                  ctypes.byref(params))
+                  ctypes.byref(params), _ptr(ws), 0 if ws is None else ws.numel())
     return gq1, gq2
 
 

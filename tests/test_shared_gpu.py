@@ -15,7 +15,8 @@ from tests.util import (REL_F32, assert_adam_weights, assert_close, oracle_adam_
 pytestmark = pytest.mark.gpu
 
 SHAPES = [("box", 300, 9, 40, 48), ("l1", 200, 5, 17, 200), ("l2", 150, 6, 33, 36), ("rotate", 120, 7, 20, 500),
-          ("beta_kl", 100, 4, 24, 400), ("complex", 90, 3, 10, 64), ("distmult", 90, 8, 65, 30), ("box", 500, 70, 130, 400)]
+          ("beta_kl", 100, 4, 24, 400), ("beta_kl", 300, 19, 131, 64), ("beta_kl", 50, 3, 70, 516), ("beta_kl", 40, 9, 5, 30),
+          ("complex", 90, 3, 10, 64), ("distmult", 90, 8, 65, 30), ("box", 500, 70, 130, 400)]
 
 
 def _shared_problem(model, n, b, k, dim):
@@ -49,7 +50,12 @@ def test_shared_negatives_match_oracle_and_the_per_query_kernels(model, n, b, k,
                  rms_floor=model in ("beta_kl", "complex", "distmult"))
     # the same kernel as the per-query layout, the ids addressed without the query number: same bits
     t_full = torch.tensor(np.ascontiguousarray(idx_full), device="cuda")
-    assert torch.equal(score, fused.score_forward(model, t_table, t_full, t_q1, t_q2, params, err))
+    per_pair = fused.score_forward_shared(model, t_table, t_ids, t_q1, t_q2, params, err, per_row_terms=False)
+    assert torch.equal(per_pair, fused.score_forward(model, t_table, t_full, t_q1, t_q2, params, err))
+    if model == "beta_kl":      # the entity-side terms once per row: the same expression, another kernel's contractions
+        assert_close(score.cpu().numpy(), per_pair.cpu().numpy(), 2e-6, "beta_kl shared score, per-row terms vs per-pair kernel")
+    else:
+        assert torch.equal(score, per_pair)
     assert err.item() == 0
 
     gq1, gq2 = fused.score_backward_query_shared(model, t_table, t_ids, t_q1, t_q2, score, t_gs, params)
@@ -59,7 +65,13 @@ def test_shared_negatives_match_oracle_and_the_per_query_kernels(model, n, b, k,
     if q2 is not None:
         assert_close(gq2.cpu().numpy(), g_qs[1][:, 0, 0], REL_F32, f"{model} shared gq2", sum_abs=q_abs)
     f1, f2 = fused.score_backward_query(model, t_table, t_full, t_q1, t_q2, score, t_gs, params)
-    assert torch.equal(f1, gq1) and (f2 is None or torch.equal(f2, gq2))
+    p1, p2 = fused.score_backward_query_shared(model, t_table, t_ids, t_q1, t_q2, score, t_gs, params, per_row_terms=False)
+    assert torch.equal(f1, p1) and (f2 is None or torch.equal(f2, p2))
+    if model == "beta_kl":
+        assert_close(gq1.cpu().numpy(), p1.cpu().numpy(), 2e-6, "beta_kl shared gq1, per-row terms vs per-pair kernel")
+        assert_close(gq2.cpu().numpy(), p2.cpu().numpy(), 2e-6, "beta_kl shared gq2, per-row terms vs per-pair kernel")
+    else:
+        assert torch.equal(gq1, p1) and (gq2 is None or torch.equal(gq2, p2))
 
     # one gradient row per list position: the sum over all queries
     want_rows = g_rows.reshape(b, k, -1).sum(axis=0)

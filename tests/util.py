@@ -20,16 +20,17 @@ def seed(*parts):
 
 
 # Worst err/bound of every comparison made through assert_close, per (test, label with numbers replaced by #):
-# [ratio against the bound in force, ratio against the purely elementwise bound rel * |ref|].  The second is the
-# headroom a tensor would have without the RMS floor (inf where a reference element is 0 and the result is not).
+# [ratio against the bound in force, ratio against the purely elementwise bound rel * |ref|, elements compared,
+# elements outside the elementwise bound].  The second is the headroom a tensor would have without the RMS floor
+# (inf where a reference element is 0 and the result is not); the last two say how many elements need the floor.
 HEADROOM = {}
 
 
-def record_headroom(what, with_floor, pure):
+def record_headroom(what, with_floor, pure, n=0, n_over=0):
     test = os.environ.get("PYTEST_CURRENT_TEST", "").split(" ")[0].split("::")[-1]
     key = (test, re.sub(r"\d+", "#", what))
-    old = HEADROOM.get(key, (0.0, 0.0))
-    HEADROOM[key] = (max(old[0], with_floor), max(old[1], pure))
+    old = HEADROOM.get(key, (0.0, 0.0, 0, 0))
+    HEADROOM[key] = (max(old[0], with_floor), max(old[1], pure), old[2] + n, old[3] + n_over)
 
 
 def assert_close(got, ref, rel, what="", sum_abs=None, rms_floor=True):
@@ -47,8 +48,9 @@ def assert_close(got, ref, rel, what="", sum_abs=None, rms_floor=True):
     err = np.abs(got - ref)
     ratio = err / bound
     worst = float(ratio.max()) if ratio.size else 0.0
-    pure = float((err / (rel * np.abs(ref) + 1e-300 + extra)).max()) if ratio.size else 0.0
-    record_headroom(what, worst, pure)
+    pure_ratio = err / (rel * np.abs(ref) + 1e-300 + extra)
+    pure = float(pure_ratio.max()) if ratio.size else 0.0
+    record_headroom(what, worst, pure, int(ratio.size), int((pure_ratio > 1.0).sum()))
     if worst > 1.0:
         k = np.argmax(ratio)
         raise AssertionError(
