@@ -4,9 +4,10 @@
 // i.e. torch.unique(ids, return_inverse=True), which the reference runs on the
 // host CPU, with a device pipeline of six kernel launches and nothing else (no
 // library sort, no memset: the whole build can be recorded into a HIP graph):
-//   hist    one read of the ids: range check, digit histograms of every radix pass per workgroup,
+//   hist    one read of the ids: range check, digit histograms of every radix pass per tile of the passes,
 //           zero fill of the tables the later kernels count in
-//   sum     digit counts of every pass over the whole input
+//   sum     digit counts of every pass over the whole input; for the first pass also per tile the
+//           counts of the tiles before it
 //   pass    x (key bits / digit bits): stable LSD radix pass over (id, pair) as one 64-bit element
 //   emit    segment heads, segment numbers, uniq, seg_start, inverse, pair_seg, n_uniq
 // The sort is written for this shape: keys are entity ids (only the bits an id below n_rows can
@@ -16,11 +17,12 @@
 //
 // A radix pass handles a tile of up to 18432 elements per workgroup of 1024 threads: elements are
 // kept in registers, ranked per wavefront with ballot matching (stable: lane order inside a round,
-// rounds in order, wavefronts in order), the tile's digit counts are published and the counts of
-// the tiles before it are read back ("look-back"; tiles take their number from a ticket counter,
-// so a tile only ever waits for tiles that are already running), the tile is reordered in LDS and
-// written out in digit runs.  Waiting is bounded: a tile that would wait too long gives up, marks
-// the plan invalid (*err_flag = 2) and every kernel still ends.
+// rounds in order, wavefronts in order), the tile is reordered in LDS and written out in digit runs.
+// Where a digit's run starts in the output depends on the tiles before: the first pass reads that from
+// the sum kernel's table; in the later passes a tile publishes its digit counts and reads back the counts
+// of the tiles before it ("look-back"; tiles take their number from a ticket counter, so a tile only ever
+// waits for tiles that are already running).  Waiting is bounded: a tile that would wait too long gives
+// up, marks the plan invalid (*err_flag = 2, n_uniq = -1) and every kernel still ends.
 //
 // An id outside [0, n_rows) sets *err_flag = 1 and gets the key n_rows: such pairs sort behind
 // every valid id, form a last segment of their own that is not counted in n_uniq and that the
@@ -41,8 +43,7 @@ constexpr unsigned kCount = 0x7fffffffu;
 constexpr unsigned kSpinLimit = 1u << 22;   // polls before a waiting tile gives up
 constexpr int kAuxThreads = 1024;           // workgroup size of the hist, sum and emit kernels
 constexpr int kAuxWaves = kAuxThreads / 64;
-constexpr int kHistBlocks = 256;
-constexpr int kHistBatch = 8;               // ids a thread of the hist kernel requests at a time
+constexpr int kHistBatch = 6;               // ids a thread of the hist kernel requests at a time
 constexpr int kEmitIters = 16;              // sorted positions per thread of the emit kernel
 constexpr int kEmitTile = kAuxThreads * kEmitIters;
 constexpr int kEmitSuper = 256;             // emit tiles whose head counts one wavefront reads back at once
@@ -55,9 +56,9 @@ __device__ __forceinline__ void st_agent(unsigned* p, unsigned v) {
 }
 
 // Waits until the word at p carries the ready flag; v is what was last read there.  Bounded: after
-// spin_limit polls the caller gets a ready word with count 0 and the plan is marked invalid.
+// spin_limit polls the caller gets a ready word with count 0, gave_up is set and the plan is marked invalid.
 __device__ __forceinline__ unsigned wait_ready(const unsigned* p, unsigned v, unsigned* abort_flag, int* err,
-                                               unsigned spin_limit) {
+                                               unsigned spin_limit, unsigned& gave_up) {
   unsigned spins = 0;
   while (!(v & kReady)) {
     __builtin_amdgcn_s_sleep(1);
@@ -65,6 +66,7 @@ __device__ __forceinline__ unsigned wait_ready(const unsigned* p, unsigned v, un
     if (++spins > spin_limit) {
       st_agent(abort_flag, 1u);
       if (err) *err = 2;
+      gave_up = 1u;
       return kReady;
     }
   }
@@ -131,10 +133,23 @@ __device__ __forceinline__ unsigned lanes_below(unsigned long long m) {
 }
 
 // ---- hist -------------------------------------------------------------------------------------
-// block_hist[block][pass][digit]: how many ids of the block's share have that digit in that pass.
+// block_hist[tile][pass][digit]: how many ids of a tile of the radix passes (tile_len consecutive ids, one
+// workgroup each) have that digit in that pass.  The first pass takes its tiles' counts from here and needs no
+// look-back; the later passes need the counts of the whole input only (their tiles hold other elements).
 // Ids are skewed (a few entities collect most pairs, and the high digits of small ids are all zero):
 // lanes that share the first lane's digit are counted with one LDS atomic for all of them.
-__global__ __launch_bounds__(kAuxThreads) void sort_hist_kernel(const long long* __restrict__ idx, int n,
+__device__ __forceinline__ void count_digit(unsigned* hist, unsigned d, bool valid, int lane) {
+  const unsigned long long live = __ballot(valid);
+  if (live == 0ull) return;  // uniform
+  const unsigned d0 = (unsigned)__builtin_amdgcn_readlane((int)d, __builtin_ctzll(live));
+  const unsigned long long like_first = __ballot(valid && d == d0);
+  if (valid) {
+    if (d != d0) atomicAdd(&hist[d], 1u);
+    else if (lane == __builtin_ctzll(like_first)) atomicAdd(&hist[d], (unsigned)__popcll(like_first));
+  }
+}
+
+__global__ __launch_bounds__(kAuxThreads) void sort_hist_kernel(const long long* __restrict__ idx, int n, int tile_len,
                                                                 unsigned long long n_rows, int passes, int dbits,
                                                                 unsigned* __restrict__ block_hist,
                                                                 unsigned* __restrict__ zero_from, size_t zero_words,
@@ -152,30 +167,21 @@ __global__ __launch_bounds__(kAuxThreads) void sort_hist_kernel(const long long*
   if (blockIdx.x == 0 && threadIdx.x == 0) *n_uniq = 0x7fffffff;
   __syncthreads();
   int bad = 0;
-  const size_t span = (size_t)kAuxThreads * kHistBatch;
-  for (size_t base = (size_t)blockIdx.x * span; base < (size_t)n; base += (size_t)gridDim.x * span) {
+  const size_t tile_base = (size_t)blockIdx.x * tile_len;
+  const size_t tile_end = tile_base + tile_len < (size_t)n ? tile_base + tile_len : (size_t)n;
+  for (size_t base = tile_base; base < tile_end; base += (size_t)kAuxThreads * kHistBatch) {
     long long id[kHistBatch];
 #pragma unroll
     for (int u = 0; u < kHistBatch; ++u) {  // all requests of the batch before the first use
       const size_t p = base + (size_t)u * kAuxThreads + threadIdx.x;
-      id[u] = p < (size_t)n ? idx[p] : 0;
+      id[u] = p < tile_end ? idx[p] : 0;
     }
 #pragma unroll
     for (int u = 0; u < kHistBatch; ++u) {
       const size_t p = base + (size_t)u * kAuxThreads + threadIdx.x;
-      const bool valid = p < (size_t)n;
+      const bool valid = p < tile_end;
       const unsigned key = clamp_id(id[u], n_rows, bad);
-      for (int s = 0; s < passes; ++s) {
-        const unsigned d = (key >> (s * dbits)) & mask;
-        const unsigned long long live = __ballot(valid);
-        if (live == 0ull) break;  // uniform
-        const unsigned d0 = (unsigned)__builtin_amdgcn_readlane((int)d, __builtin_ctzll(live));
-        const unsigned long long like_first = __ballot(valid && d == d0);
-        if (valid) {
-          if (d != d0) atomicAdd(&lds_hist[s * bins + d], 1u);
-          else if (lane == __builtin_ctzll(like_first)) atomicAdd(&lds_hist[s * bins + d], (unsigned)__popcll(like_first));
-        }
-      }
+      for (int s = 0; s < passes; ++s) count_digit(lds_hist + s * bins, (key >> (s * dbits)) & mask, valid, lane);
       if (valid && pair_seg) pair_seg[p] = 0;  // "not alone"; the emit kernel overwrites the entries of one-pair segments
     }
   }
@@ -185,37 +191,53 @@ __global__ __launch_bounds__(kAuxThreads) void sort_hist_kernel(const long long*
     block_hist[(size_t)blockIdx.x * passes * bins + i] = lds_hist[i];
 }
 
-// digit_count[pass][digit] = sum over the hist workgroups; one workgroup per (pass, 64 digits), its
-// sixteen wavefronts share the hist workgroups among them, so every thread has a few independent loads.
+// digit_count[pass][digit] = sum over the tiles; one workgroup per (pass, 64 digits), its sixteen wavefronts take
+// one stretch of the tiles each.  For the first pass the running sum is kept as well:
+// tile_before[tile][digit] = ids with that digit in the tiles before it.
 __global__ __launch_bounds__(kAuxThreads) void sort_sum_kernel(const unsigned* __restrict__ block_hist, int blocks,
                                                                int passes, int dbits,
-                                                               unsigned* __restrict__ digit_count) {
+                                                               unsigned* __restrict__ digit_count,
+                                                               unsigned* __restrict__ tile_before) {
   __shared__ unsigned part[kAuxWaves][64];
   const int bins = 1 << dbits;
   const int groups = (bins + 63) / 64;
   const int s = blockIdx.x / groups;
-  const int d = (blockIdx.x - s * groups) * 64 + (threadIdx.x & 63);
+  const int lane = threadIdx.x & 63;
+  const int d = (blockIdx.x - s * groups) * 64 + lane;
   const int w = threadIdx.x >> 6;
+  const int per_wave = (blocks + kAuxWaves - 1) / kAuxWaves;
+  const int b_lo = w * per_wave, b_hi = min(blocks, b_lo + per_wave);
+  const unsigned* src = block_hist + (size_t)s * bins + (d < bins ? d : 0);
+  const size_t stride = (size_t)passes * bins;
   unsigned sum = 0;
-  if (d < bins) {
-    for (int b0 = w; b0 < blocks; b0 += kAuxWaves * 8) {
-      unsigned v[8];
+  for (int b0 = b_lo; b0 < b_hi; b0 += 8) {
+    unsigned v[8];
 #pragma unroll
-      for (int u = 0; u < 8; ++u) {
-        const int b = b0 + u * kAuxWaves;
-        v[u] = b < blocks ? block_hist[((size_t)b * passes + s) * bins + d] : 0u;
-      }
+    for (int u = 0; u < 8; ++u) v[u] = b0 + u < b_hi ? src[(size_t)(b0 + u) * stride] : 0u;
 #pragma unroll
-      for (int u = 0; u < 8; ++u) sum += v[u];
-    }
+    for (int u = 0; u < 8; ++u) sum += v[u];
   }
-  part[w][threadIdx.x & 63] = sum;
+  part[w][lane] = sum;
   __syncthreads();
-  if (w == 0 && d < bins) {
-    unsigned all = 0;
+  unsigned before = 0, all = 0;
 #pragma unroll
-    for (int i = 0; i < kAuxWaves; ++i) all += part[i][threadIdx.x];
-    digit_count[s * bins + d] = all;
+  for (int i = 0; i < kAuxWaves; ++i) {
+    const unsigned t = part[i][lane];
+    before += i < w ? t : 0u;
+    all += t;
+  }
+  if (d >= bins) return;
+  if (w == 0) digit_count[s * bins + d] = all;
+  if (s != 0) return;
+  for (int b0 = b_lo; b0 < b_hi; b0 += 8) {
+    unsigned v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = b0 + u < b_hi ? src[(size_t)(b0 + u) * stride] : 0u;
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      if (b0 + u < b_hi) tile_before[(size_t)(b0 + u) * bins + d] = before;
+      before += v[u];
+    }
   }
 }
 
@@ -231,7 +253,8 @@ struct SortPassArgs {
   int shift, dbits;
   size_t stage_bytes;               // LDS bytes of the region shared by the per-wavefront counters and the staged tile
   const unsigned* digit_count;      // [bins] of this pass: elements per digit in the whole input
-  // look-back tables, each word = ready flag | count per digit:
+  const unsigned* tile_before;      // IN_IDX: [tiles][bins] elements per digit in the tiles before each (from the sum kernel)
+  // look-back tables of the other passes, each word = ready flag | count per digit:
   unsigned* level[3];               // [tiles / 16^l][bins], l = 0: one tile, 1: a group of 16 tiles, 2: 256 tiles
   unsigned* pre;                    // [tiles / 4096][bins]: everything up to the end of a stretch of 4096 tiles
   unsigned* ticket;
@@ -319,7 +342,7 @@ __global__ __launch_bounds__(NW * 64, (MAXR <= 8 ? 8 : 4)) void sort_pass_kernel
         run += t;
       }
       mine[u] = run;
-      st_agent(&A.level[0][(size_t)tile * bins + d], run | kReady);
+      if constexpr (!IN_IDX) st_agent(&A.level[0][(size_t)tile * bins + d], run | kReady);
     }
   }
   // position of a digit's first element inside the reordered tile, and in the whole output
@@ -336,50 +359,57 @@ __global__ __launch_bounds__(NW * 64, (MAXR <= 8 ? 8 : 4)) void sort_pass_kernel
     }
   }
 
-  // 4. look-back: elements with a digit in the tiles before this one.  Tiles form groups of 16, groups
-  // form super-blocks of 16 groups, and so on: a thread fetches, per level, at most 15 independent words
-  // (the units of that level before its own inside the next-larger unit), and the last tile of a unit
-  // publishes the unit's total as soon as it has it.  Beyond 4096 tiles a chain of prefixes takes over.
+  // 4. elements with a digit in the tiles before this one.  The first pass has them from the sum kernel.  The
+  // others look back: tiles form groups of 16, groups form blocks of 16 groups, and so on; a thread fetches,
+  // per level, at most 15 independent words (the units of that level before its own inside the next-larger
+  // unit), and the last tile of a unit publishes the unit's total as soon as it has it.  Beyond 4096 tiles a
+  // chain of prefixes takes over.
 #pragma unroll
   for (int u = 0; u < PER; ++u) {
     const int d = tid + u * NT;
     if (d < bins) {
       unsigned before = 0;
-      unsigned unit = tile;  // my unit's number at this level
+      [[maybe_unused]] unsigned gave_up = 0;  // (the mark on the device is what counts here)
+      if constexpr (IN_IDX) {
+        before = A.tile_before[(size_t)tile * bins + d];
+      } else {
+        unsigned unit = tile;  // my unit's number at this level
 #pragma unroll
-      for (int l = 0; l < 3; ++l) {
-        const unsigned first = unit & ~(unsigned)(kGroup - 1);
-        const unsigned* tab = A.level[l] + d;
-        unsigned v[kGroup - 1];
+        for (int l = 0; l < 3; ++l) {
+          const unsigned first = unit & ~(unsigned)(kGroup - 1);
+          const unsigned* tab = A.level[l] + d;
+          unsigned v[kGroup - 1];
 #pragma unroll
-        for (int j = 0; j < kGroup - 1; ++j) v[j] = first + j < unit ? ld_agent(tab + (size_t)(first + j) * bins) : kReady;
-        unsigned here = 0;
+          for (int j = 0; j < kGroup - 1; ++j) v[j] = first + j < unit ? ld_agent(tab + (size_t)(first + j) * bins) : kReady;
+          unsigned here = 0;
 #pragma unroll
-        for (int j = 0; j < kGroup - 1; ++j) {
-          if (first + j < unit) v[j] = wait_ready(tab + (size_t)(first + j) * bins, v[j], A.abort_flag, A.err, A.spin_limit);
-          here += v[j] & kCount;
+          for (int j = 0; j < kGroup - 1; ++j) {
+            if (first + j < unit) v[j] = wait_ready(tab + (size_t)(first + j) * bins, v[j], A.abort_flag, A.err, A.spin_limit, gave_up);
+            here += v[j] & kCount;
+          }
+          before += here;
+          // the last tile of a unit of the next level publishes that unit's total: everything before me
+          // inside it (levels up to here) plus my own count
+          const unsigned span = 1u << (4 * (l + 1));
+          if ((tile & (span - 1)) == span - 1) {
+            if (l < 2) st_agent(A.level[l + 1] + (size_t)(tile / span) * bins + d, ((before + mine[u]) & kCount) | kReady);
+          }
+          unit >>= 4;
         }
-        before += here;
-        // the last tile of a unit of the next level publishes that unit's total: everything before me
-        // inside it (levels up to here) plus my own count
-        const unsigned span = 1u << (4 * (l + 1));
-        if ((tile & (span - 1)) == span - 1) {
-          if (l < 2) st_agent(A.level[l + 1] + (size_t)(tile / span) * bins + d, ((before + mine[u]) & kCount) | kReady);
+        if (tile >= 4096u) {
+          const unsigned* p = &A.pre[(size_t)(tile / 4096u - 1) * bins + d];
+          before += wait_ready(p, ld_agent(p), A.abort_flag, A.err, A.spin_limit, gave_up) & kCount;
         }
-        unit >>= 4;
+        if ((tile & 4095u) == 4095u) st_agent(&A.pre[(size_t)(tile / 4096u) * bins + d], ((before + mine[u]) & kCount) | kReady);
       }
-      if (tile >= 4096u) {
-        const unsigned* p = &A.pre[(size_t)(tile / 4096u - 1) * bins + d];
-        before += wait_ready(p, ld_agent(p), A.abort_flag, A.err, A.spin_limit) & kCount;
-      }
-      if ((tile & 4095u) == 4095u) st_agent(&A.pre[(size_t)(tile / 4096u) * bins + d], ((before + mine[u]) & kCount) | kReady);
       local_base[d] = lb[u];
       run_base[d] = db[u] + before - lb[u];  // + position in the reordered tile = global position
     }
   }
-  if (tid == 0) tmp[21] = ld_agent(A.abort_flag);
+  // (A tile that gave up waiting has taken the missing counts as zero: its positions are wrong but inside the
+  // output, like those of the tiles that read what it publishes; the emit kernel sees the mark and declares the
+  // plan invalid, so nobody reads the result.)
   __syncthreads();
-  if (tmp[21]) return;  // a tile gave up waiting: positions are not trustworthy, write nothing
 
   // 5. position of every element in the tile reordered by digit
 #pragma unroll
@@ -490,6 +520,7 @@ __global__ __launch_bounds__(kAuxThreads) void plan_emit_kernel(EmitArgs A) {
 
     // look-back: heads in the tiles before this one
     unsigned sum = 0;
+    [[maybe_unused]] unsigned gave_up = 0;  // (the mark on the device is what counts here)
     const int first = (int)(tile & ~(unsigned)(kEmitSuper - 1));
     unsigned v[kEmitSuper / 64];
 #pragma unroll
@@ -500,7 +531,7 @@ __global__ __launch_bounds__(kAuxThreads) void plan_emit_kernel(EmitArgs A) {
 #pragma unroll
     for (int u = 0; u < kEmitSuper / 64; ++u) {
       const int j = (int)tile - 1 - lane - 64 * u;
-      if (j >= first) v[u] = wait_ready(&A.agg[j], v[u], A.abort_flag, A.err, A.spin_limit);
+      if (j >= first) v[u] = wait_ready(&A.agg[j], v[u], A.abort_flag, A.err, A.spin_limit, gave_up);
       sum += v[u] & kCount;
     }
 #pragma unroll
@@ -508,7 +539,7 @@ __global__ __launch_bounds__(kAuxThreads) void plan_emit_kernel(EmitArgs A) {
     if (lane == 0) {
       if (first > 0) {
         const unsigned* p = &A.pre[first / kEmitSuper - 1];
-        sum += wait_ready(p, ld_agent(p), A.abort_flag, A.err, A.spin_limit) & kCount;
+        sum += wait_ready(p, ld_agent(p), A.abort_flag, A.err, A.spin_limit, gave_up) & kCount;
       }
       if ((tile & (kEmitSuper - 1)) == kEmitSuper - 1) st_agent(&A.pre[tile / kEmitSuper], ((sum + total) & kCount) | kReady);
       tmp[21] = sum;
@@ -645,7 +676,7 @@ constexpr int kSortWaves = 16;
 struct PlanLayout {
   int passes, dbits, bins, nw, rounds, tiles, units[3], chain, hist_blocks, emit_tiles, emit_supers;
   size_t stage_bytes, pass_lds;
-  size_t a_off, b_off, bh_off, count_off, zero_off, zero_words, total;
+  size_t a_off, b_off, bh_off, count_off, tb_off, zero_off, zero_words, total;
   // inside the zeroed region (in words from zero_off)
   size_t level_w[3], pre_w, eagg_w, epre_w, ticket_w, abort_w;
 };
@@ -678,15 +709,15 @@ static PlanLayout plan_layout(size_t n, size_t n_rows) {
   L.chain = (L.tiles + 4095) / 4096;
   L.stage_bytes = tile * 8 > counters ? tile * 8 : counters;
   L.pass_lds = L.stage_bytes + fixed_lds;
-  L.hist_blocks = (int)((n + (size_t)kAuxThreads * kHistBatch - 1) / ((size_t)kAuxThreads * kHistBatch));
-  if (L.hist_blocks > kHistBlocks) L.hist_blocks = kHistBlocks;
+  L.hist_blocks = L.tiles;  // the hist kernel counts per tile of the radix passes
   L.emit_tiles = (int)((n + kEmitTile - 1) / kEmitTile);
   L.emit_supers = (L.emit_tiles + kEmitSuper - 1) / kEmitSuper;
   L.a_off = 0;
   L.b_off = up(n * 8);
   L.bh_off = L.b_off + (L.passes > 2 ? up(n * 8) : 0);
   L.count_off = L.bh_off + up((size_t)L.hist_blocks * L.passes * L.bins * 4);
-  L.zero_off = L.count_off + up((size_t)L.passes * L.bins * 4);
+  L.tb_off = L.count_off + up((size_t)L.passes * L.bins * 4);
+  L.zero_off = L.tb_off + up((size_t)L.tiles * L.bins * 4);
   size_t wds = 0;
   for (int l = 0; l < 3; ++l) {
     L.level_w[l] = wds;
@@ -786,15 +817,17 @@ static int plan_build(void* stream, const int64_t* idx, size_t n_pairs, size_t n
   unsigned long long* buf_b = reinterpret_cast<unsigned long long*>(ws + L.b_off);
   unsigned* block_hist = reinterpret_cast<unsigned*>(ws + L.bh_off);
   unsigned* digit_count = reinterpret_cast<unsigned*>(ws + L.count_off);
+  unsigned* tile_before = reinterpret_cast<unsigned*>(ws + L.tb_off);
   unsigned* zeroed = reinterpret_cast<unsigned*>(ws + L.zero_off);
   const int n = (int)n_pairs;
 
   hipLaunchKernelGGL(sort_hist_kernel, dim3((unsigned)L.hist_blocks), dim3(kAuxThreads),
                      (size_t)L.passes * L.bins * sizeof(unsigned), st, reinterpret_cast<const long long*>(idx), n,
-                     (unsigned long long)n_rows, L.passes, L.dbits, block_hist, zeroed, L.zero_words, pair_seg, err_flag,
+                     L.rounds * L.nw * 64, (unsigned long long)n_rows, L.passes, L.dbits, block_hist, zeroed, L.zero_words, pair_seg,
+                     err_flag,
                      zeroed + L.abort_w, force_abort ? 1u : 0u, n_uniq);
   hipLaunchKernelGGL(sort_sum_kernel, dim3((unsigned)(L.passes * ((L.bins + 63) / 64))), dim3(kAuxThreads), 0, st, block_hist,
-                     L.hist_blocks, L.passes, L.dbits, digit_count);
+                     L.hist_blocks, L.passes, L.dbits, digit_count, tile_before);
   for (int s = 0; s < L.passes; ++s) {
     SortPassArgs A{};
     const bool first = s == 0, last = s == L.passes - 1;
@@ -810,6 +843,7 @@ static int plan_build(void* stream, const int64_t* idx, size_t n_pairs, size_t n
     A.dbits = L.dbits;
     A.stage_bytes = L.stage_bytes;
     A.digit_count = digit_count + (size_t)s * L.bins;
+    A.tile_before = tile_before;
     for (int l = 0; l < 3; ++l) A.level[l] = zeroed + L.level_w[l] + (size_t)s * L.units[l] * L.bins;
     A.pre = zeroed + L.pre_w + (size_t)s * L.chain * L.bins;
     A.ticket = zeroed + L.ticket_w + s;

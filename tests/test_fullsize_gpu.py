@@ -236,6 +236,26 @@ def test_plan_around_the_tile_geometry_boundaries():
         assert torch.equal(plan.seg_start[: plan.n_uniq].long(), torch.nonzero(heads).reshape(-1))
 
 
+def test_plan_beyond_4096_tiles():
+    """More than 4096 tiles of 18 elements per thread: the look-back's three levels end and the chain of prefixes
+    over stretches of 4096 tiles takes over.  Sorted order, stability and segment table against torch's stable sort."""
+    from smore_amd import fused
+    n = 86_054_151
+    n_pairs = 4096 * 18 * 1024 + 3 * 18 * 1024 + 77
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(4097)
+    ids = torch.randint(0, n, (n_pairs,), device="cuda", generator=gen)
+    ids[: n_pairs // 64] = ids[0]
+    plan = fused.build_plan(ids, n)
+    want_ids, want_order = torch.sort(ids, stable=True)
+    assert torch.equal(plan.sorted_ids.long(), want_ids)
+    assert torch.equal(plan.order.long(), want_order)
+    heads = torch.ones(n_pairs, dtype=torch.bool, device="cuda")
+    heads[1:] = want_ids[1:] != want_ids[:-1]
+    assert plan.n_uniq == int(heads.sum().item())
+    assert torch.equal(plan.seg_start[: plan.n_uniq].long(), torch.nonzero(heads).reshape(-1))
+
+
 def test_full_size_dropin_flow():
     """The 86M-entity step as SMORE's own code reaches it: lookup handles for positives and negatives, the box
     model's cal_logit (box.py:157-164) on them, backward, apply_grad -- nothing but the reference's call sequence
