@@ -467,6 +467,7 @@ def shared_step_bench(cfg, device, seed, steps, warmup, graph):
     }
     if graph_ms is not None:
         out["graph_replay"] = {"ms_per_step": graph_ms, "value": pairs / (graph_ms * 1e-3), "unit": "pairs/s"}
+    out["sources"] = kernel_source_digest()
     print(json.dumps(out))
 
 
