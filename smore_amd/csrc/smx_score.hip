@@ -20,6 +20,7 @@
 
 #include "../../include/smx_measure.h"
 #include "smx_score_impl.h"
+#include "smx_shared_fwd_impl.h"
 
 namespace smx {
 
@@ -39,6 +40,14 @@ int entity_backward(int model, void* stream, const smx_plan_view* plan, float* t
                     int codes_nit, const PairSources* multi = nullptr);
 size_t entity_ws_bytes(size_t n_pairs, size_t row_len);
 size_t code_bytes_per_pair(size_t dim);
+
+// instantiated in smx_shared_inst_*.hip
+extern template int shared_forward_dispatch<mL1>(hipStream_t, const SharedFwdArgs&, int);
+extern template int shared_forward_dispatch<mL2>(hipStream_t, const SharedFwdArgs&, int);
+extern template int shared_forward_dispatch<mBox>(hipStream_t, const SharedFwdArgs&, int);
+extern template int shared_forward_dispatch<mRotate>(hipStream_t, const SharedFwdArgs&, int);
+extern template int shared_forward_dispatch<mComplex>(hipStream_t, const SharedFwdArgs&, int);
+extern template int shared_forward_dispatch<mDistmult>(hipStream_t, const SharedFwdArgs&, int);
 
 // defined in smx_beta_shared.hip
 bool beta_shared_fits(size_t dim, const void* table, const void* q1, const void* q2, const void* workspace,
@@ -245,6 +254,19 @@ int smx_score_forward_shared(int model, void* stream, const float* table, size_t
   if (model == mBetaKL && beta_shared_fits(dim, table, q1, q2, workspace, workspace_bytes, K, true))
     return beta_shared_forward(as_stream(stream), table, n_rows, reinterpret_cast<const long long*>(ids), q1, q2, score, B,
                                K, dim, A.p, err_flag, static_cast<float*>(workspace));
+  if (shared_forward_fits(model, vec, nit)) {  // rows staged in LDS for eight queries at a time
+    const SharedFwdArgs S{table, reinterpret_cast<const long long*>(ids), q1, q2, score, (int)B, (int)K, A.ncol, n_rows, A.p,
+                          err_flag};
+    hipStream_t st = as_stream(stream);
+    switch (model) {
+      case mL1: return shared_forward_dispatch<mL1>(st, S, nit);
+      case mL2: return shared_forward_dispatch<mL2>(st, S, nit);
+      case mBox: return shared_forward_dispatch<mBox>(st, S, nit);
+      case mRotate: return shared_forward_dispatch<mRotate>(st, S, nit);
+      case mComplex: return shared_forward_dispatch<mComplex>(st, S, nit);
+      case mDistmult: return shared_forward_dispatch<mDistmult>(st, S, nit);
+    }
+  }
   A.ids_shared = 1;
   A.score_out = score;
   A.err = err_flag;
