@@ -105,6 +105,32 @@ def test_shared_negatives_match_oracle_and_the_per_query_kernels(model, n, b, k,
     assert err.item() == 0
 
 
+@pytest.mark.parametrize("model,dim", [("box", 400), ("rotate", 100), ("beta_kl", 64), ("l2", 30)])
+def test_an_id_outside_the_table_in_the_shared_list_is_flagged_and_scored_as_row_0(model, dim):
+    """Every scorer of the library reads row 0 for an id outside [0, n) and raises the caller's flag
+    (the reference fails at the lookup itself, embed_rw.py:74-75); the shared forms included, for lists
+    shorter and longer than a workgroup's stretch and batches that do not fill a workgroup."""
+    from smore_amd import fused
+    n, b = 60, 11
+    for k in (3, 64, 131):
+        rng = np.random.default_rng(seed("shared-bad", model, dim, k))
+        table, q1, q2, _, _ = make_problem(model, n, b, k, dim, rng)
+        ids = rng.integers(0, n, k).astype(np.int64)
+        bad = ids.copy()
+        bad[k // 3] = n + 5
+        bad[k - 1] = -2
+        ids[k // 3] = 0
+        ids[k - 1] = 0
+        params = fused.score_params(GAMMA[model], 0.02)
+        t_table, t_q1, t_q2 = dev(table), dev(q1), dev(q2)
+        err = fused.new_error_flag("cuda")
+        want = fused.score_forward_shared(model, t_table, torch.tensor(ids, device="cuda"), t_q1, t_q2, params, err)
+        assert err.item() == 0
+        got = fused.score_forward_shared(model, t_table, torch.tensor(bad, device="cuda"), t_q1, t_q2, params, err)
+        assert err.item() == 1
+        assert torch.equal(got, want)
+
+
 def test_shared_negatives_next_to_positives_and_anchors_in_one_step():
     """The step every shipped training script runs (kg_reasoning.py:298-355 with --share_negative): an anchor lookup
     feeds the query, positives [B] and shared negatives [1,K] are scored against it, one apply_grad.  The shared ids
