@@ -36,7 +36,7 @@ SIGNATURES = {
     # model, stream, table, n_rows, idx, q1, q2, score, gscore, gq1, gq2, B, K, dim, params, fwd_codes, bytes
     "smx_score_backward_query": (_i, [_i, _vp, _vp, _sz, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _vp, _vp,
                                       _sz]),
-    "smx_shared_workspace_bytes": (_sz, [_i, _sz, _sz]),
+    "smx_shared_workspace_bytes": (_sz, [_i, _sz, _sz, _sz]),
     # model, stream, table, n_rows, ids, q1, q2, score, B, K, dim, params, err_flag, ws, ws_bytes
     "smx_score_forward_shared": (_i, [_i, _vp, _vp, _sz, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _vp, _vp, _vp, _sz]),
     # model, stream, table, n_rows, ids, q1, q2, score, gscore, gq1, gq2, B, K, dim, params, ws, ws_bytes

@@ -1,18 +1,23 @@
-// BetaE with negatives shared by the batch: the entity side of the KL divergence once per row.
+// BetaE with negatives shared by the batch: the entity side of the KL divergence once per row, the pairs as a
+// matrix product.
 //
 // KL(Beta(e) || Beta(q)) per feature (smore/common/torchext/dist_kernel.h:207-266) is
 //   [lgG(qa)+lgG(qb)-lgG(sq)] + [lgG(se)-lgG(ea)-lgG(eb)] + (ea-qa) psi(ea) + (eb-qb) psi(eb) + (sq-se) psi(se):
 // three digammas and a log-beta of the ENTITY per (pair, feature), which is what makes the per-query kernels
 // instruction-bound (smore/models/beta.py:303-308 through beta_dist.py).  With --share_negative
-// (smore/cpp_sampler/online_sampler.py:155-157) the same K rows meet all B queries, so those entity terms are
-// evaluated once per row into a side table -- K x dim evaluations instead of B x K x dim -- and a pair costs a
-// handful of multiply-adds per feature on them.  The side table is several times the size of the rows, so it
-// is reused from LDS: a workgroup stages a few rows' terms, and each of its wavefronts, holding one query in
-// registers, scores that query against all of them.
-//   forward:         score[b,k] = gamma - sum_d KL         (same per-feature expression and summation order
-//                                                           as the per-query kernel: ModelOps<mBetaKL>::fwd)
-//   query backward:  gqa[b,d] = sum_k c[b,k] ((psi(qa)-psi(sq)) - psi(ea_k) + psi(se_k)), same with b
-//                                                          (ModelOps<mBetaKL>::bwd_q), rows in ascending order
+// (smore/cpp_sampler/online_sampler.py:155-157) the same K rows meet all B queries.  Regrouped by what each
+// term depends on,
+//   KL[b,k] = Qk[b] + Ek[k] + sum_d qa[b,d] T[k,d] + sum_d qb[b,d] T[k,D+d]
+//     T[k,d] = psi(se)-psi(ea),  T[k,D+d] = psi(se)-psi(eb)                       (one row of 2D floats per shared row)
+//     Ek[k]  = sum_d [lgG(se)-lgG(ea)-lgG(eb)] + ea psi(ea) + eb psi(eb) - se psi(se)
+//     Qk[b]  = sum_d lgG(qa)+lgG(qb)-lgG(sq)
+// the special functions are evaluated K x D + B x D times instead of B x K x D, and what is left per pair is an
+// inner product over 2D features with an operand shared along each axis: a matrix product [B, 2D] x [2D, K], the one
+// shape on this path that the matrix cores fit (v_mfma_f32_32x32x2_f32: fp32 operands, fp32 accumulation in a fixed
+// order).  The query backward is the other product with the same table,
+//   gqa[b,d] = (psi(qa)-psi(sq)) sum_k c[b,k] + sum_k c[b,k] T[k,d]            (c = -upstream gradient; same with b),
+// i.e. [B, K] x [K, 2D].  The sums are those of ModelOps<mBetaKL>::fwd / bwd_q taken in another order: the four
+// groups are summed separately, which costs some of the tolerance's headroom (measured in the tests), not the bar.
 // The entity side of the backward needs no special functions per pair at all (sums of c (e - q), one trigamma
 // hook per finished row): it is shared_entity_kernel of smx_shared_impl.h as it stands.
 #include "smx_common.h"
@@ -21,22 +26,14 @@
 
 namespace smx {
 
-constexpr int kBsFwdWaves = 8;    // queries per workgroup of the forward (one per wavefront)
-constexpr int kBsBwdWaves = 4;    // queries per workgroup of the query backward
-constexpr int kBsFwdTile = 4;     // rows whose six term vectors are staged in LDS per turn (forward)
-constexpr int kBsBwdTile = 8;     // rows whose three digamma vectors are staged per turn (query backward)
-constexpr int kBsFwdChunk = 64;   // rows per workgroup of the forward
-constexpr int kBsMaxDim = 512;    // two float4 columns per lane at most
+typedef float facc16 __attribute__((ext_vector_type(16)));
 
-typedef float bvec4 __attribute__((ext_vector_type(4)));
-
-// terms of row ids[k]: forward {ea, eb, lgB(e), psi(ea), psi(eb), psi(se)} x dim, backward {psi(ea), psi(eb), psi(se)} x dim
-// (ea, eb after the entity prologue clamp(x + add, lo, hi) when it is on); one wavefront per row.
+// ---- the terms of the shared rows: T [K][2D], then (forward) Ek [K]; one wavefront per row ------------------
 template <bool FWD>
 __global__ __launch_bounds__(256) void beta_row_terms_kernel(const float* __restrict__ table,
                                                              const long long* __restrict__ ids, int K, int dim,
                                                              unsigned long long n_rows, ScoreParams p,
-                                                             float* __restrict__ terms, int* err) {
+                                                             float* __restrict__ T, float* __restrict__ Ek, int* err) {
   const int lane = threadIdx.x & 63;
   const int k = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (k >= K) return;
@@ -46,206 +43,242 @@ __global__ __launch_bounds__(256) void beta_row_terms_kernel(const float* __rest
     row = 0;
   }
   const float* e = table + (size_t)row * 2 * dim;
-  constexpr int NV = FWD ? 6 : 3;
-  float* out = terms + (size_t)k * NV * dim;
+  float* out = T + (size_t)k * 2 * dim;
+  float mine = 0.f;
   for (int d = lane; d < dim; d += 64) {
     const float ea = reg_apply(e[d], p), eb = reg_apply(e[dim + d], p);
     float lb, pa, pb, ps;
     if constexpr (FWD) {
       beta_terms(ea, eb, lb, pa, pb, ps);
-      out[d] = ea;
-      out[dim + d] = eb;
-      out[2 * dim + d] = lb;
-      out[3 * dim + d] = pa;
-      out[4 * dim + d] = pb;
-      out[5 * dim + d] = ps;
+      mine += (lb + ea * pa) + (eb * pb - (ea + eb) * ps);
     } else {
       digamma3(ea, eb, pa, pb, ps);
-      out[d] = pa;
-      out[dim + d] = pb;
-      out[2 * dim + d] = ps;
     }
+    out[d] = ps - pa;
+    out[dim + d] = ps - pb;
+  }
+  if constexpr (FWD) {
+    const float total = wave_sum_last_f32(mine);
+    if (lane == 63) Ek[k] = total;
   }
 }
 
-template <int NIT, bool FWD>
-__device__ __forceinline__ void load_beta_query(const float* __restrict__ q1, const float* __restrict__ q2, int b, int dim,
-                                                int ncol, int lane, QBeta (&q)[NIT][4]) {
+// Qk [B]: one wavefront per query
+__global__ __launch_bounds__(256) void beta_query_terms_kernel(const float* __restrict__ q1, const float* __restrict__ q2,
+                                                               int B, int dim, float* __restrict__ Qk) {
+  const int lane = threadIdx.x & 63;
+  const int b = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (b >= B) return;
+  float mine = 0.f;
+  for (int d = lane; d < dim; d += 64) mine += ModelOps<mBetaKL>::prep_fwd(q1[(size_t)b * dim + d], q2[(size_t)b * dim + d]).k;
+  const float total = wave_sum_last_f32(mine);
+  if (lane == 63) Qk[b] = total;
+}
+
+// ---- the matrix products ------------------------------------------------------------------------------------
+// A 32 x 32 tile of the result is formed by walking the inner dimension two at a time with
+// v_mfma_f32_32x32x2_f32.  Operand layout of the instruction: lane l supplies A[l % 32][l / 32] and B[l / 32][l % 32];
+// of the 16 accumulators of lane l, number r is the element (8 (r / 4) + 4 (l / 32) + r % 4, l % 32).
+__device__ __forceinline__ int acc_row(int r, int lane) { return 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3); }
+
+// The four wavefronts of a workgroup share one tile: each walks a quarter of the inner dimension, the partial tiles
+// are added through LDS in wavefront order, the first wavefront finishes (a tile alone would leave a SIMD one
+// wavefront whose loads nothing hides).
+__device__ __forceinline__ void combine_tiles(facc16& acc, float* part, int wave, int lane) {
+  if (wave > 0) {
 #pragma unroll
-  for (int it = 0; it < NIT; ++it) {
-    const int c = min(lane + 64 * it, ncol - 1);
+    for (int r = 0; r < 16; ++r) part[((wave - 1) * 16 + r) * 64 + lane] = acc[r];
+  }
+  __syncthreads();
+  if (wave == 0) {
 #pragma unroll
-    for (int v = 0; v < 4; ++v) {
-      const float a = q1[(size_t)b * dim + c * 4 + v], bb = q2[(size_t)b * dim + c * 4 + v];
-      q[it][v] = FWD ? ModelOps<mBetaKL>::prep_fwd(a, bb) : ModelOps<mBetaKL>::prep_bwd_q(a, bb);
-    }
+    for (int w = 1; w < 4; ++w)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[r] += part[((w - 1) * 16 + r) * 64 + lane];
   }
 }
 
-// grid (ceil(B / 8), ceil(K / 64)); LDS: kBsFwdTile rows x 6 x dim floats
-template <int NIT>
-__global__ __launch_bounds__(kBsFwdWaves * 64) void beta_shared_forward_kernel(const float* __restrict__ terms,
-                                                                               const float* __restrict__ q1,
-                                                                               const float* __restrict__ q2,
-                                                                               float* __restrict__ score, int B, int K,
-                                                                               int dim, ScoreParams p) {
-  extern __shared__ __align__(16) float tile[];
+// score[b,k] = gamma - (Qk[b] + Ek[k] + sum_j q[b,j] T[k,j]), j over the 2D features ([q1 | q2] against a row of T).
+// Both operands have the inner dimension contiguous: a lane reads two neighbouring features per load and feeds
+// them to two instructions (instruction t of a group of four features takes feature 4 g + 2 (l / 32) + t).
+// Wavefronts 0, 1: the two halves of the q1 part; 2, 3: of the q2 part.
+__global__ __launch_bounds__(256) void beta_shared_forward_gemm_kernel(const float* __restrict__ T,
+                                                                       const float* __restrict__ Ek,
+                                                                       const float* __restrict__ Qk,
+                                                                       const float* __restrict__ q1,
+                                                                       const float* __restrict__ q2,
+                                                                       float* __restrict__ score, int B, int K, int dim,
+                                                                       float gamma) {
+  __shared__ float part[3 * 16 * 64];
   const int lane = threadIdx.x & 63;
   const int wave = uniform(threadIdx.x >> 6);
-  const int ncol = dim / 4;
-  const int b_raw = blockIdx.x * kBsFwdWaves + wave;
-  const int b = min(b_raw, B - 1);  // a wavefront past the last query computes along (it takes part in the barriers)
-  const int k0 = blockIdx.y * kBsFwdChunk, k1 = min(K, k0 + kBsFwdChunk);
-  QBeta q[NIT][4];
-  load_beta_query<NIT, true>(q1, q2, b, dim, ncol, lane, q);
-  // a thread's share of a tile travels through registers: the next tile is requested before this one is used
-  constexpr int kPer = (kBsFwdTile * 6 * (kBsMaxDim / 4) + kBsFwdWaves * 64 - 1) / (kBsFwdWaves * 64);
-  bvec4 next[kPer];
-  auto request = [&](int kt) {
-    const int n4 = min(kBsFwdTile, k1 - kt) * 6 * ncol;
-    const bvec4* src = reinterpret_cast<const bvec4*>(terms + (size_t)kt * 6 * dim);
+  const int tiles_k = (K + 31) / 32;
+  const int tile = blockIdx.x;
+  const int b0 = (tile / tiles_k) * 32, k0 = (tile % tiles_k) * 32;
+  const int half = lane >> 5, col = lane & 31;
+  const int my_b = min(b0 + col, B - 1), my_k = min(k0 + col, K - 1);  // rows past the end repeat the last one; never stored
+  facc16 acc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+  {
+    const int seg = wave >> 1;
+    const float2* a = reinterpret_cast<const float2*>((seg ? q2 : q1) + (size_t)my_b * dim) + half;
+    const float2* t = reinterpret_cast<const float2*>(T + (size_t)my_k * 2 * dim + (size_t)seg * dim) + half;
+    // four groups at a time, the next four requested before these are used (requests past the end repeat the last group)
+    const int G = dim / 4;
+    const int g_lo = (wave & 1) ? G / 2 : 0, g_hi = (wave & 1) ? G : G / 2;
+    float2 av[4], tv[4], an[4], tn[4];
 #pragma unroll
-    for (int u = 0; u < kPer; ++u) {
-      const int i = threadIdx.x + u * kBsFwdWaves * 64;
-      if (i < n4) next[u] = src[i];
+    for (int u = 0; u < 4; ++u) {
+      av[u] = a[2 * min(g_lo + u, G - 1)];
+      tv[u] = t[2 * min(g_lo + u, G - 1)];
     }
-  };
-  request(k0);
-  for (int kt = k0; kt < k1; kt += kBsFwdTile) {
-    const int rows_here = min(kBsFwdTile, k1 - kt);
-    __syncthreads();  // the previous rows have been used by every wavefront
+    for (int g = g_lo; g < g_hi; g += 4) {
 #pragma unroll
-    for (int u = 0; u < kPer; ++u) {
-      const int i = threadIdx.x + u * kBsFwdWaves * 64;
-      if (i < rows_here * 6 * ncol) reinterpret_cast<bvec4*>(tile)[i] = next[u];
-    }
-    __syncthreads();
-    if (kt + kBsFwdTile < k1) request(kt + kBsFwdTile);
-    for (int r = 0; r < rows_here; ++r) {
-      const bvec4* t = reinterpret_cast<const bvec4*>(tile + (size_t)r * 6 * dim);
-      float mine = 0.f;
-#pragma unroll
-      for (int it = 0; it < NIT; ++it) {
-        const int c = min(lane + 64 * it, ncol - 1);
-        const bvec4 ea = t[c], eb = t[ncol + c], lb = t[2 * ncol + c], pa = t[3 * ncol + c], pb = t[4 * ncol + c],
-                    ps = t[5 * ncol + c];
-        float a0 = 0.f;
-#pragma unroll
-        for (int v = 0; v < 4; ++v)
-          a0 += (q[it][v].k + lb[v]) + (ea[v] - q[it][v].a) * pa[v] + (eb[v] - q[it][v].b) * pb[v] +
-                ((q[it][v].a + q[it][v].b) - (ea[v] + eb[v])) * ps[v];
-        mine += lane + 64 * it < ncol ? a0 : 0.f;
+      for (int u = 0; u < 4; ++u) {
+        an[u] = a[2 * min(g + 4 + u, G - 1)];
+        tn[u] = t[2 * min(g + 4 + u, G - 1)];
       }
-      const float folded = wave_sum_last_f32(mine);
-      if (lane == 63 && b_raw < B) score[(size_t)b * K + kt + r] = p.gamma - folded;
-    }
-  }
-}
-
-// Every workgroup walks all K rows (a query's gradient is one sum over them, rows ascending) for 4 / NIT queries: a
-// query's columns are independent sums, so with two column groups two wavefronts share a query, one group each,
-// and the grid is twice as long.  grid ceil(B * NIT / 4).  LDS: kBsBwdTile rows x 3 x dim floats
-template <int NIT>
-__global__ __launch_bounds__(kBsBwdWaves * 64) void beta_shared_backward_query_kernel(
-    const float* __restrict__ terms, const float* __restrict__ q1, const float* __restrict__ q2,
-    const float* __restrict__ gscore, float* __restrict__ gq1, float* __restrict__ gq2, int B, int K, int dim) {
-  extern __shared__ __align__(16) float tile[];
-  constexpr int kQueries = kBsBwdWaves / NIT;
-  const int lane = threadIdx.x & 63;
-  const int wave = uniform(threadIdx.x >> 6);
-  const int ncol = dim / 4;
-  const int b_raw = blockIdx.x * kQueries + wave / NIT;
-  const int b = min(b_raw, B - 1);  // a wavefront past the last query computes along (it takes part in the barriers)
-  const int my_col = lane + 64 * (wave % NIT);
-  const int c = min(my_col, ncol - 1);
-  QBeta q[4];
-  float g1[4], g2[4];
 #pragma unroll
-  for (int v = 0; v < 4; ++v) {
-    q[v] = ModelOps<mBetaKL>::prep_bwd_q(q1[(size_t)b * dim + c * 4 + v], q2[(size_t)b * dim + c * 4 + v]);
-    g1[v] = g2[v] = 0.f;
-  }
-  // a thread's share of a tile travels through registers: the next tile is requested before this one is used
-  // (64 is a multiple of the tile, so tiles never straddle a batch of upstream gradients)
-  static_assert(64 % kBsBwdTile == 0, "tiles must not straddle a batch of 64 rows");
-  constexpr int kPer = (kBsBwdTile * 3 * (kBsMaxDim / 4) + kBsBwdWaves * 64 - 1) / (kBsBwdWaves * 64);
-  bvec4 next[kPer];
-  auto request = [&](int kt) {
-    const int n4 = min(kBsBwdTile, K - kt) * 3 * ncol;
-    const bvec4* src = reinterpret_cast<const bvec4*>(terms + (size_t)kt * 3 * dim);
-#pragma unroll
-    for (int u = 0; u < kPer; ++u) {
-      const int i = threadIdx.x + u * kBsBwdWaves * 64;
-      if (i < n4) next[u] = src[i];
-    }
-  };
-  request(0);
-  for (int k64 = 0; k64 < K; k64 += 64) {
-    const int n64 = min(64, K - k64);
-    const float my_c0 = -gscore[(size_t)b * K + k64 + min(lane, n64 - 1)];  // d(gamma - KL) / d KL times the upstream gradient
-    for (int kt = 0; kt < n64; kt += kBsBwdTile) {
-      const int rows_here = min(kBsBwdTile, n64 - kt);
-      __syncthreads();
-#pragma unroll
-      for (int u = 0; u < kPer; ++u) {
-        const int i = threadIdx.x + u * kBsBwdWaves * 64;
-        if (i < rows_here * 3 * ncol) reinterpret_cast<bvec4*>(tile)[i] = next[u];
-      }
-      __syncthreads();
-      if (k64 + kt + kBsBwdTile < K) request(k64 + kt + kBsBwdTile);
-      for (int r = 0; r < rows_here; ++r) {
-        const float c0 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(my_c0), kt + r));
-        const bvec4* t = reinterpret_cast<const bvec4*>(tile + (size_t)r * 3 * dim);
-        const bvec4 pa = t[c], pb = t[ncol + c], ps = t[2 * ncol + c];
-#pragma unroll
-        for (int v = 0; v < 4; ++v) {
-          g1[v] += c0 * (q[v].k - pa[v] + ps[v]);
-          g2[v] += c0 * (q[v].l - pb[v] + ps[v]);
+      for (int u = 0; u < 4; ++u) {
+        if (g + u < g_hi) {  // uniform
+          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av[u].x, tv[u].x, acc, 0, 0, 0);
+          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av[u].y, tv[u].y, acc, 0, 0, 0);
         }
       }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        av[u] = an[u];
+        tv[u] = tn[u];
+      }
     }
   }
-  if (b_raw >= B || my_col >= ncol) return;
-  reinterpret_cast<bvec4*>(gq1 + (size_t)b * dim)[c] = bvec4{g1[0], g1[1], g1[2], g1[3]};
-  reinterpret_cast<bvec4*>(gq2 + (size_t)b * dim)[c] = bvec4{g2[0], g2[1], g2[2], g2[3]};
+  combine_tiles(acc, part, wave, lane);
+  const int k = k0 + col;
+  if (wave != 0 || k >= K) return;
+  const float ek = Ek[k];
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int b = b0 + acc_row(r, lane);
+    if (b < B) score[(size_t)b * K + k] = gamma - ((Qk[b] + ek) + acc[r]);
+  }
 }
 
-// Whether the call can take these kernels: float4 columns, two per lane at most, aligned operands, room for the terms.
+// gq[b,n] = kq[b,n] sum_k c[b,k] + sum_k c[b,k] T[k,n], n over the 2D features (n < D: gq1 with kq = psi(qa)-psi(sq),
+// else gq2 with psi(qb)-psi(sq)), c = -gscore.  The lanes of a tile's A operand also add up what they load: the
+// row sums of c come for free.  Each of the four wavefronts walks a quarter of the list.
+__global__ __launch_bounds__(256) void beta_shared_backward_query_gemm_kernel(const float* __restrict__ T,
+                                                                              const float* __restrict__ q1,
+                                                                              const float* __restrict__ q2,
+                                                                              const float* __restrict__ gscore,
+                                                                              float* __restrict__ gq1,
+                                                                              float* __restrict__ gq2, int B, int K,
+                                                                              int dim) {
+  __shared__ float part[3 * 16 * 64];
+  __shared__ float part_c[3 * 64];
+  const int lane = threadIdx.x & 63;
+  const int wave = uniform(threadIdx.x >> 6);
+  const int tiles_n = (2 * dim + 31) / 32;
+  const int tile = blockIdx.x;
+  const int b0 = (tile / tiles_n) * 32, n0 = (tile % tiles_n) * 32;
+  const int half = lane >> 5, col = lane & 31;
+  const int my_b = min(b0 + col, B - 1);
+  const int my_n = min(n0 + col, 2 * dim - 1);
+  const float* a = gscore + (size_t)my_b * K;
+  const float* t = T + my_n;
+  facc16 acc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+  float c_sum = 0.f;
+  // this wavefront's stretch of the list, a multiple of eight rows: four instructions take eight rows, lanes 0-31
+  // supplying rows kk .. kk+3 and lanes 32-63 rows kk+4 .. kk+7 (one 16-byte load of coefficients per lane when the
+  // rows of gscore are 16-byte aligned).  The next eight are requested before these are used; a request past the
+  // end of the stretch repeats the list's last row with coefficient 0
+  const int per = ((K + 31) / 32) * 8;
+  const int k_lo = wave * per, k_hi = min(K, k_lo + per);
+  const size_t ld = (size_t)2 * dim;
+  const bool wide = (K & 3) == 0 && (reinterpret_cast<unsigned long long>(gscore) & 15ull) == 0ull;
+  float cv[4], tv[4], cn[4], tn[4];
+  auto request = [&](float (&c)[4], float (&tt)[4], int kk0) {
+    const int k4 = kk0 + 4 * half;
+    if (wide && k4 + 3 < k_hi) {  // (k_hi is a multiple of 4 here: all four rows or none)
+      const float4 g = *reinterpret_cast<const float4*>(a + k4);
+      c[0] = -g.x;
+      c[1] = -g.y;
+      c[2] = -g.z;
+      c[3] = -g.w;
+    } else {
+#pragma unroll
+      for (int u = 0; u < 4; ++u) c[u] = k4 + u < k_hi ? -a[min(k4 + u, K - 1)] : 0.f;
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) tt[u] = t[(size_t)min(k4 + u, K - 1) * ld];
+  };
+  request(cv, tv, k_lo);
+  for (int kk = k_lo; kk < k_hi; kk += 8) {
+    request(cn, tn, kk + 8);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      if (kk + u < k_hi) {  // uniform (rows kk+4+u past the end carry coefficient 0)
+        c_sum += cv[u];
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(cv[u], tv[u], acc, 0, 0, 0);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      cv[u] = cn[u];
+      tv[u] = tn[u];
+    }
+  }
+  c_sum += __shfl_xor(c_sum, 32);  // row my_b: both halves of every eight rows
+  if (wave > 0) part_c[(wave - 1) * 64 + lane] = c_sum;
+  combine_tiles(acc, part, wave, lane);
+  if (wave != 0) return;
+#pragma unroll
+  for (int w = 1; w < 4; ++w) c_sum += part_c[(w - 1) * 64 + lane];
+  const int n = n0 + col;
+  const int d = n < dim ? n : n - dim;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int row = acc_row(r, lane);
+    const float s = __shfl(c_sum, row);
+    const int b = b0 + row;
+    if (b < B && n < 2 * dim) {
+      const QBeta q = ModelOps<mBetaKL>::prep_bwd_q(q1[(size_t)b * dim + d], q2[(size_t)b * dim + d]);
+      float* out = n < dim ? gq1 : gq2;
+      out[(size_t)b * dim + d] = (n < dim ? q.k : q.l) * s + acc[r];
+    }
+  }
+}
+
+// Whether the call can take these kernels: float4-aligned operands and room for T, Ek and Qk in the workspace.
 bool beta_shared_fits(size_t dim, const void* table, const void* q1, const void* q2, const void* workspace,
-                      size_t workspace_bytes, size_t K, bool forward) {
-  if (dim % 4 != 0 || dim > (size_t)kBsMaxDim || !workspace) return false;
+                      size_t workspace_bytes, size_t B, size_t K) {
+  if (dim % 4 != 0 || !workspace) return false;
   if (!aligned16(table) || !aligned16(q1) || !aligned16(q2) || !aligned16(workspace)) return false;
-  return workspace_bytes >= K * (forward ? 6 : 3) * dim * sizeof(float);
+  return workspace_bytes >= (K * (2 * dim + 1) + B) * sizeof(float);
 }
 
 int beta_shared_forward(hipStream_t st, const float* table, size_t n_rows, const long long* ids, const float* q1,
                         const float* q2, float* score, size_t B, size_t K, size_t dim, const ScoreParams& p, int* err,
-                        float* terms) {
+                        float* workspace) {
+  float* T = workspace;
+  float* Ek = T + K * 2 * dim;
+  float* Qk = Ek + K;
   hipLaunchKernelGGL(beta_row_terms_kernel<true>, dim3((unsigned)((K + 3) / 4)), dim3(256), 0, st, table, ids, (int)K,
-                     (int)dim, (unsigned long long)n_rows, p, terms, err);
-  const dim3 grid((unsigned)((B + kBsFwdWaves - 1) / kBsFwdWaves), (unsigned)((K + kBsFwdChunk - 1) / kBsFwdChunk));
-  const size_t lds = (size_t)kBsFwdTile * 6 * dim * sizeof(float);
-  if (dim <= 256)
-    hipLaunchKernelGGL(beta_shared_forward_kernel<1>, grid, dim3(kBsFwdWaves * 64), lds, st, terms, q1, q2, score, (int)B,
-                       (int)K, (int)dim, p);
-  else
-    hipLaunchKernelGGL(beta_shared_forward_kernel<2>, grid, dim3(kBsFwdWaves * 64), lds, st, terms, q1, q2, score, (int)B,
-                       (int)K, (int)dim, p);
+                     (int)dim, (unsigned long long)n_rows, p, T, Ek, err);
+  hipLaunchKernelGGL(beta_query_terms_kernel, dim3((unsigned)((B + 3) / 4)), dim3(256), 0, st, q1, q2, (int)B, (int)dim, Qk);
+  const size_t tiles = ((B + 31) / 32) * ((K + 31) / 32);
+  hipLaunchKernelGGL(beta_shared_forward_gemm_kernel, dim3((unsigned)tiles), dim3(256), 0, st, T, Ek, Qk, q1, q2,
+                     score, (int)B, (int)K, (int)dim, p.gamma);
   return check_launch("score forward (shared negatives, beta_kl)");
 }
 
 int beta_shared_backward_query(hipStream_t st, const float* table, size_t n_rows, const long long* ids, const float* q1,
                                const float* q2, const float* gscore, float* gq1, float* gq2, size_t B, size_t K,
-                               size_t dim, const ScoreParams& p, float* terms) {
+                               size_t dim, const ScoreParams& p, float* workspace) {
+  float* T = workspace;
   hipLaunchKernelGGL(beta_row_terms_kernel<false>, dim3((unsigned)((K + 3) / 4)), dim3(256), 0, st, table, ids, (int)K,
-                     (int)dim, (unsigned long long)n_rows, p, terms, nullptr);
-  const size_t lds = (size_t)kBsBwdTile * 3 * dim * sizeof(float);
-  if (dim <= 256)
-    hipLaunchKernelGGL(beta_shared_backward_query_kernel<1>, dim3((unsigned)((B + kBsBwdWaves - 1) / kBsBwdWaves)),
-                       dim3(kBsBwdWaves * 64), lds, st, terms, q1, q2, gscore, gq1, gq2, (int)B, (int)K, (int)dim);
-  else
-    hipLaunchKernelGGL(beta_shared_backward_query_kernel<2>, dim3((unsigned)((2 * B + kBsBwdWaves - 1) / kBsBwdWaves)),
-                       dim3(kBsBwdWaves * 64), lds, st, terms, q1, q2, gscore, gq1, gq2, (int)B, (int)K, (int)dim);
+                     (int)dim, (unsigned long long)n_rows, p, T, nullptr, nullptr);
+  const size_t tiles = ((B + 31) / 32) * ((2 * dim + 31) / 32);
+  hipLaunchKernelGGL(beta_shared_backward_query_gemm_kernel, dim3((unsigned)tiles), dim3(256), 0, st, T, q1, q2,
+                     gscore, gq1, gq2, (int)B, (int)K, (int)dim);
   return check_launch("score backward (query, shared negatives, beta_kl)");
 }
 

@@ -51,7 +51,7 @@ extern template int shared_forward_dispatch<mDistmult>(hipStream_t, const Shared
 
 // defined in smx_beta_shared.hip
 bool beta_shared_fits(size_t dim, const void* table, const void* q1, const void* q2, const void* workspace,
-                      size_t workspace_bytes, size_t K, bool forward);
+                      size_t workspace_bytes, size_t B, size_t K);
 int beta_shared_forward(hipStream_t st, const float* table, size_t n_rows, const long long* ids, const float* q1,
                         const float* q2, float* score, size_t B, size_t K, size_t dim, const ScoreParams& p, int* err,
                         float* terms);
@@ -237,8 +237,8 @@ int smx_score_backward_query(int model, void* stream, const float* table, size_t
   return dispatch_model(model, as_stream(stream), A, vec, nit, false);
 }
 
-size_t smx_shared_workspace_bytes(int model, size_t K, size_t dim) {
-  return model == smx::mBetaKL ? ((K * 6 * dim * sizeof(float) + 255) & ~(size_t)255) : 0;
+size_t smx_shared_workspace_bytes(int model, size_t B, size_t K, size_t dim) {
+  return model == smx::mBetaKL ? (((K * (2 * dim + 1) + B) * sizeof(float) + 255) & ~(size_t)255) : 0;
 }
 
 int smx_score_forward_shared(int model, void* stream, const float* table, size_t n_rows, const int64_t* ids,
@@ -251,7 +251,7 @@ int smx_score_forward_shared(int model, void* stream, const float* table, size_t
   if (int rc = fill_args(&A, &vec, &nit, model, table, n_rows, ids, q1, q2, B, K, dim, params, nullptr, nullptr)) return rc;
   if (!score) return fail(SMX_ERR_ARG, "null score pointer");
   // BetaE: the entity side of the divergence once per shared row (needs the workspace for the rows' terms)
-  if (model == mBetaKL && beta_shared_fits(dim, table, q1, q2, workspace, workspace_bytes, K, true))
+  if (model == mBetaKL && beta_shared_fits(dim, table, q1, q2, workspace, workspace_bytes, B, K))
     return beta_shared_forward(as_stream(stream), table, n_rows, reinterpret_cast<const long long*>(ids), q1, q2, score, B,
                                K, dim, A.p, err_flag, static_cast<float*>(workspace));
   if (shared_forward_fits(model, vec, nit)) {  // rows staged in LDS for eight queries at a time
@@ -284,7 +284,7 @@ int smx_score_backward_query_shared(int model, void* stream, const float* table,
   if (int rc = fill_args(&A, &vec, &nit, model, table, n_rows, ids, q1, q2, B, K, dim, params, nullptr, nullptr)) return rc;
   if (!score || !gscore || !gq1 || (model_nq(model) == 2 && !gq2)) return fail(SMX_ERR_ARG, "null pointer");
   if (model == mBetaKL && aligned16(gq1) && aligned16(gq2) &&
-      beta_shared_fits(dim, table, q1, q2, workspace, workspace_bytes, K, false))
+      beta_shared_fits(dim, table, q1, q2, workspace, workspace_bytes, B, K))
     return beta_shared_backward_query(as_stream(stream), table, n_rows, reinterpret_cast<const long long*>(ids), q1, q2,
                                       gscore, gq1, gq2, B, K, dim, A.p, static_cast<float*>(workspace));
   A.ids_shared = 1;

@@ -129,8 +129,8 @@ def _shared_dims(model, table, ids, q1, q2):
     return b, ids.numel(), dim
 
 
-def _shared_workspace(model, k, dim, device, use):
-    nbytes = _lib.load().smx_shared_workspace_bytes(MODELS[model], k, dim) if use else 0
+def _shared_workspace(model, b, k, dim, device, use):
+    nbytes = _lib.load().smx_shared_workspace_bytes(MODELS[model], b, k, dim) if use else 0
     return _workspace(nbytes, device) if nbytes else None
 
 
@@ -140,7 +140,7 @@ def score_forward_shared(model, table, ids, q1, q2, params, err_flag=None, per_r
     b, k, dim = _shared_dims(model, table, ids, q1, q2)
     score = torch.empty((b, k), dtype=torch.float32, device=table.device)
     with torch.cuda.device(table.device):
-        ws = _shared_workspace(model, k, dim, table.device, per_row_terms)
+        ws = _shared_workspace(model, b, k, dim, table.device, per_row_terms)
         _lib.call("smx_score_forward_shared", MODELS[model], _stream(table), _ptr(table), table.shape[0], _ptr(ids),
                   _ptr(q1), _ptr(q2), _ptr(score), b, k, dim, ctypes.byref(params), _ptr(err_flag), _ptr(ws),
                   0 if ws is None else ws.numel())
@@ -155,7 +155,7 @@ def score_backward_query_shared(model, table, ids, q1, q2, score, gscore, params
     gq1 = torch.empty_like(q1)
     gq2 = None if q2 is None else torch.empty_like(q2)
     with torch.cuda.device(table.device):
-        ws = _shared_workspace(model, k, dim, table.device, per_row_terms)
+        ws = _shared_workspace(model, b, k, dim, table.device, per_row_terms)
         _lib.call("smx_score_backward_query_shared", MODELS[model], _stream(table), _ptr(table), table.shape[0],
                   _ptr(ids), _ptr(q1), _ptr(q2), _ptr(score), _ptr(gscore), _ptr(gq1), _ptr(gq2), b, k, dim,
                   ctypes.byref(params), _ptr(ws), 0 if ws is None else ws.numel())

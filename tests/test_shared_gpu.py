@@ -56,7 +56,9 @@ def test_shared_negatives_match_oracle_and_the_per_query_kernels(model, n, b, k,
     if model in ("l1", "box"):
         assert torch.equal(score, per_pair)
     else:
-        assert_close(score.cpu().numpy(), per_pair.cpu().numpy(), 2e-6, f"{model} shared score, shared-list kernel vs per-pair kernel")
+        # (beta_kl's shared form sums the divergence's four groups of terms separately: a looser bar between the two)
+        assert_close(score.cpu().numpy(), per_pair.cpu().numpy(), 5e-6 if model == "beta_kl" else 2e-6,
+                     f"{model} shared score, shared-list kernel vs per-pair kernel")
     if model == "beta_kl":      # without the workspace: the per-query kernel with the ids addressed without the query number
         assert torch.equal(per_pair, fused.score_forward_shared(model, t_table, t_ids, t_q1, t_q2, params, err, per_row_terms=False))
     assert err.item() == 0
@@ -71,8 +73,8 @@ def test_shared_negatives_match_oracle_and_the_per_query_kernels(model, n, b, k,
     p1, p2 = fused.score_backward_query_shared(model, t_table, t_ids, t_q1, t_q2, score, t_gs, params, per_row_terms=False)
     assert torch.equal(f1, p1) and (f2 is None or torch.equal(f2, p2))
     if model == "beta_kl":
-        assert_close(gq1.cpu().numpy(), p1.cpu().numpy(), 2e-6, "beta_kl shared gq1, per-row terms vs per-pair kernel")
-        assert_close(gq2.cpu().numpy(), p2.cpu().numpy(), 2e-6, "beta_kl shared gq2, per-row terms vs per-pair kernel")
+        assert_close(gq1.cpu().numpy(), p1.cpu().numpy(), 5e-6, "beta_kl shared gq1, per-row terms vs per-pair kernel")
+        assert_close(gq2.cpu().numpy(), p2.cpu().numpy(), 5e-6, "beta_kl shared gq2, per-row terms vs per-pair kernel")
     else:
         assert torch.equal(gq1, p1) and (gq2 is None or torch.equal(gq2, p2))
 
