@@ -362,13 +362,14 @@ int smx_rows_backward(void* stream, const smx_plan_view* plan, const float* grad
  *     plan != NULL: a plan built by smx_plan_build over exactly these K ids.  One result per DISTINCT id (a list
  *                   that holds an id twice sums both positions): merged[u,:] and / or the optimizer update of
  *                   table, m, v in place, as smx_score_backward_entity.
- * workspace of the forward and the query backward (may be NULL): smx_shared_workspace_bytes(model, B, K, dim)
+ * workspace of the three calls (may be NULL): smx_shared_workspace_bytes(model, B, K, dim)
  * bytes, 16-byte aligned; 0 for every model but BETA_KL.  Given it (and rows of 16-byte aligned floats, dim a
  * multiple of 4), BetaE's entity-side terms -- three digammas and a log-beta per feature, dist_kernel.h:212-221 --
  * are evaluated once per shared row into the workspace instead of once per pair, and the pairs are a matrix product
  * on them (fp32 matrix instructions, fixed summation order); without it the per-pair kernels run (same results to
- * rounding: the product sums the divergence's four groups of terms separately).  Each call fills the workspace
- * itself: nothing is carried from one call to the next.
+ * rounding: the product sums the divergence's four groups of terms separately); the entity side forms its sums
+ * over the queries as a product too ([K,B] x [B,2 dim]) and finishes them row by row as before.  Each call fills the
+ * workspace itself: nothing is carried from one call to the next.
  * Replaces dist_forward / dist_backward in the [1,K] x [B,1] layout (common_kernel.h:33-123) plus gather,
  * merge_grad_* and update_step as listed at smx_score_backward_entity. */
 size_t smx_shared_workspace_bytes(int model, size_t B, size_t K, size_t dim);
@@ -384,7 +385,7 @@ int smx_score_backward_entity_shared(int model, void* stream, float* table, size
                                      const float* q1, const float* q2, const float* score, const float* gscore,
                                      size_t B, size_t K, size_t dim, const smx_score_params* params,
                                      const smx_plan_view* plan, float* grad_rows, float* merged, float* m, float* v,
-                                     const smx_opt_params* adam);
+                                     const smx_opt_params* adam, void* workspace, size_t workspace_bytes);
 
 /* ---- sample loss ---------------------------------------------------------------------------
  * The loss between the scoring forward and its backward (smore/training/train_process.py:194-213)

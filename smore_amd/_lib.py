@@ -44,7 +44,7 @@ SIGNATURES = {
                                              _vp, _sz]),
     # model, stream, table, n_rows, ids, q1, q2, score, gscore, B, K, dim, params, plan, grad_rows, merged, m, v, adam
     "smx_score_backward_entity_shared": (_i, [_i, _vp, _vp, _sz, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _vp, _vp, _vp,
-                                              _vp, _vp, _vp, _vp]),
+                                              _vp, _vp, _vp, _vp, _vp, _sz]),
     "smx_union_workspace_bytes": (_sz, [_sz, _sz, _sz]),
     # model, stream, table, n_rows, idx, q1, q2, score, winner, B, U, K, dim, params, err_flag, ws, ws_bytes
     "smx_score_forward_union": (_i, [_i, _vp, _vp, _sz, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _vp, _vp, _vp, _sz]),

@@ -247,6 +247,75 @@ __global__ __launch_bounds__(256) void beta_shared_backward_query_gemm_kernel(co
   }
 }
 
+// Entity side: ModelOps<mBetaKL>::bwd_e sums c (ea - qa) and c (eb - qb) over the queries, i.e. for list position k
+//   S1[k,d] = ea[k,d] C[k] - R[k,d],  S2[k,d] = eb[k,d] C[k] - R[k,D+d],  C[k] = sum_b c[b,k],  R = c^T [K,B] x [q1 | q2] [B,2D]:
+// this kernel leaves R [K][2D] and C [K] in the workspace, and shared_entity_kernel turns them into the gradient row
+// (the trigamma hook, the clamp mask, the optimizer) as it does with the sums it forms itself.  Both operands
+// are read along their contiguous dimension (lane l: c[b + l / 32][k0 + l % 32] and q[b + l / 32][n0 + l % 32]);
+// each of the four wavefronts walks a quarter of the queries.
+__global__ __launch_bounds__(256) void beta_shared_entity_gemm_kernel(const float* __restrict__ q1,
+                                                                      const float* __restrict__ q2,
+                                                                      const float* __restrict__ gscore,
+                                                                      float* __restrict__ R, float* __restrict__ C, int B,
+                                                                      int K, int dim) {
+  __shared__ float part[3 * 16 * 64];
+  __shared__ float part_c[3 * 64];
+  const int lane = threadIdx.x & 63;
+  const int wave = uniform(threadIdx.x >> 6);
+  const int tiles_n = (2 * dim + 31) / 32;
+  const int tile = blockIdx.x;
+  const int k0 = (tile / tiles_n) * 32, n0 = (tile % tiles_n) * 32;
+  const int half = lane >> 5, col = lane & 31;
+  const int my_k = min(k0 + col, K - 1);
+  const int my_n = min(n0 + col, 2 * dim - 1);
+  const float* a = gscore + my_k;
+  const float* t = my_n < dim ? q1 + my_n : q2 + (my_n - dim);
+  facc16 acc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+  float c_sum = 0.f;
+  const int per = ((B + 31) / 32) * 8;  // a multiple of eight queries: four instructions
+  const int b_lo = wave * per, b_hi = min(B, b_lo + per);
+  float cv[4], tv[4], cn[4], tn[4];
+  auto request = [&](float (&c)[4], float (&tt)[4], int bb0) {
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int b = bb0 + 2 * u + half;
+      const int bc = min(b, B - 1);
+      c[u] = b < b_hi ? -a[(size_t)bc * K] : 0.f;
+      tt[u] = t[(size_t)bc * dim];
+    }
+  };
+  request(cv, tv, b_lo);
+  for (int bb = b_lo; bb < b_hi; bb += 8) {
+    request(cn, tn, bb + 8);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      if (bb + 2 * u < b_hi) {  // uniform (an odd query past the end carries coefficient 0)
+        c_sum += cv[u];
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(cv[u], tv[u], acc, 0, 0, 0);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      cv[u] = cn[u];
+      tv[u] = tn[u];
+    }
+  }
+  c_sum += __shfl_xor(c_sum, 32);  // list position my_k: even queries of the stretch + odd ones
+  if (wave > 0) part_c[(wave - 1) * 64 + lane] = c_sum;
+  combine_tiles(acc, part, wave, lane);
+  if (wave != 0) return;
+#pragma unroll
+  for (int w = 1; w < 4; ++w) c_sum += part_c[(w - 1) * 64 + lane];
+  if (n0 == 0 && half == 0 && k0 + col < K) C[k0 + col] = c_sum;
+  const int n = n0 + col;
+  if (n >= 2 * dim) return;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int k = k0 + acc_row(r, lane);
+    if (k < K) R[(size_t)k * 2 * dim + n] = acc[r];
+  }
+}
+
 // Whether the call can take these kernels: float4-aligned operands and room for T, Ek and Qk in the workspace.
 bool beta_shared_fits(size_t dim, const void* table, const void* q1, const void* q2, const void* workspace,
                       size_t workspace_bytes, size_t B, size_t K) {
@@ -280,6 +349,15 @@ int beta_shared_backward_query(hipStream_t st, const float* table, size_t n_rows
   hipLaunchKernelGGL(beta_shared_backward_query_gemm_kernel, dim3((unsigned)tiles), dim3(256), 0, st, T, q1, q2,
                      gscore, gq1, gq2, (int)B, (int)K, (int)dim);
   return check_launch("score backward (query, shared negatives, beta_kl)");
+}
+
+// R [K][2D] and C [K] for the entity side (see beta_shared_entity_gemm_kernel); workspace: K (2 dim + 1) floats
+int beta_shared_entity_sums(hipStream_t st, const float* q1, const float* q2, const float* gscore, size_t B, size_t K,
+                            size_t dim, float* workspace) {
+  const size_t tiles = ((K + 31) / 32) * ((2 * dim + 31) / 32);
+  hipLaunchKernelGGL(beta_shared_entity_gemm_kernel, dim3((unsigned)tiles), dim3(256), 0, st, q1, q2, gscore, workspace,
+                     workspace + K * 2 * dim, (int)B, (int)K, (int)dim);
+  return check_launch("entity backward (shared negatives, beta_kl sums)");
 }
 
 }  // namespace smx

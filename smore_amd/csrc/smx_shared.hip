@@ -11,6 +11,10 @@ extern template int shared_entity_dispatch<mBetaKL>(hipStream_t, const SharedArg
 extern template int shared_entity_dispatch<mComplex>(hipStream_t, const SharedArgs&, int, int);
 extern template int shared_entity_dispatch<mDistmult>(hipStream_t, const SharedArgs&, int, int);
 
+// defined in smx_beta_shared.hip
+int beta_shared_entity_sums(hipStream_t st, const float* q1, const float* q2, const float* gscore, size_t B, size_t K,
+                            size_t dim, float* workspace);
+
 }  // namespace smx
 
 extern "C" int smx_score_backward_entity_shared(int model, void* stream, float* table, size_t n_rows, const int64_t* ids,
@@ -18,7 +22,7 @@ extern "C" int smx_score_backward_entity_shared(int model, void* stream, float* 
                                                 const float* gscore, size_t B, size_t K, size_t dim,
                                                 const smx_score_params* params, const smx_plan_view* plan,
                                                 float* grad_rows, float* merged, float* m, float* v,
-                                                const smx_opt_params* adam) {
+                                                const smx_opt_params* adam, void* workspace, size_t workspace_bytes) {
   using namespace smx;
   if (model < 0 || model >= mNumModels) return fail(SMX_ERR_KIND, "unknown score model %d", model);
   if (!table || !ids || !q1 || !score || !gscore || !params || (model_nq(model) == 2 && !q2))
@@ -78,6 +82,14 @@ extern "C" int smx_score_backward_entity_shared(int model, void* stream, float* 
   A.table = table;
   A.ncol = (int)ncol;
   hipStream_t st = as_stream(stream);
+  // BetaE: the sums over the queries as a matrix product into the workspace, finished row by row below
+  if (model == mBetaKL && vec == 4 && workspace && aligned16(workspace) &&
+      workspace_bytes >= K * (2 * dim + 1) * sizeof(float)) {
+    float* ws = static_cast<float*>(workspace);
+    if (int rc = beta_shared_entity_sums(st, q1, q2, gscore, B, K, dim, ws)) return rc;
+    A.sums_r = ws;
+    A.sums_c = ws + K * 2 * dim;
+  }
   switch (model) {
     case mL1: return shared_entity_dispatch<mL1>(st, A, vec, nit);
     case mL2: return shared_entity_dispatch<mL2>(st, A, vec, nit);

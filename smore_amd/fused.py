@@ -163,7 +163,7 @@ def score_backward_query_shared(model, table, ids, q1, q2, score, gscore, params
 
 
 def score_backward_entity_shared(model, table, ids, q1, q2, score, gscore, params, plan=None, grad_rows=None,
-                                 merged=None, m=None, v=None, adam=None):
+                                 merged=None, m=None, v=None, adam=None, per_row_terms=True):
     """Entity side of shared ids (see smx_score_backward_entity_shared).  plan None: returns (and fills) grad_rows
     [K, row], one gradient row per list position.  plan (built over exactly these ids): merged rows per distinct id
     and / or the optimizer update of table, m, v in place."""
@@ -186,10 +186,11 @@ def score_backward_entity_shared(model, table, ids, q1, q2, score, gscore, param
             raise _lib.SmxError("merged must be [n_uniq or more, row]")
     with torch.cuda.device(table.device):
         view = None if plan is None else plan.view()
+        ws = _shared_workspace(model, b, k, dim, table.device, per_row_terms)
         _lib.call("smx_score_backward_entity_shared", MODELS[model], _stream(table), _ptr(table), table.shape[0],
                   _ptr(ids), _ptr(q1), _ptr(q2), _ptr(score), _ptr(gscore), b, k, dim, ctypes.byref(params),
                   None if view is None else ctypes.byref(view), _ptr(grad_rows), _ptr(merged), _ptr(m), _ptr(v),
-                  None if adam is None else ctypes.byref(adam))
+                  None if adam is None else ctypes.byref(adam), _ptr(ws), 0 if ws is None else ws.numel())
     return grad_rows
 
 

@@ -83,6 +83,9 @@ def test_shared_negatives_match_oracle_and_the_per_query_kernels(model, n, b, k,
     abs_rows = np.abs(g_rows).reshape(b, k, -1).sum(axis=0)
     got_rows = fused.score_backward_entity_shared(model, t_table, t_ids, t_q1, t_q2, score, t_gs, params)
     assert_close(got_rows.cpu().numpy(), want_rows, REL_F32, f"{model} shared gradient rows", sum_abs=abs_rows)
+    if model == "beta_kl":      # the sums over the queries formed by the kernel itself instead of as a matrix product
+        own = fused.score_backward_entity_shared(model, t_table, t_ids, t_q1, t_q2, score, t_gs, params, per_row_terms=False)
+        assert_close(own.cpu().numpy(), want_rows, REL_F32, "beta_kl shared gradient rows, sums in the kernel", sum_abs=abs_rows)
     assert torch.equal(t_table, dev(table)), "the table must not change without an optimizer"
 
     # with the plan of the K ids: one merged row / one Adam update per distinct id
