@@ -49,15 +49,16 @@ extern template int shared_forward_dispatch<mRotate>(hipStream_t, const SharedFw
 extern template int shared_forward_dispatch<mComplex>(hipStream_t, const SharedFwdArgs&, int);
 extern template int shared_forward_dispatch<mDistmult>(hipStream_t, const SharedFwdArgs&, int);
 
-// defined in smx_beta_shared.hip
-bool beta_shared_fits(size_t dim, const void* table, const void* q1, const void* q2, const void* workspace,
-                      size_t workspace_bytes, size_t B, size_t K);
-int beta_shared_forward(hipStream_t st, const float* table, size_t n_rows, const long long* ids, const float* q1,
-                        const float* q2, float* score, size_t B, size_t K, size_t dim, const ScoreParams& p, int* err,
-                        float* terms);
-int beta_shared_backward_query(hipStream_t st, const float* table, size_t n_rows, const long long* ids, const float* q1,
-                               const float* q2, const float* gscore, float* gq1, float* gq2, size_t B, size_t K,
-                               size_t dim, const ScoreParams& p, float* terms);
+// defined in smx_shared_gemm.hip: shared negatives of beta_kl, complex and distmult as matrix products
+size_t shared_gemm_workspace_floats(int model, size_t B, size_t K, size_t dim, bool entity);
+bool shared_gemm_fits(int model, size_t dim, const void* table, const void* q1, const void* q2, const void* workspace,
+                      size_t workspace_bytes, size_t B, size_t K, bool entity);
+int shared_gemm_forward(int model, hipStream_t st, const float* table, size_t n_rows, const long long* ids,
+                        const float* q1, const float* q2, float* score, size_t B, size_t K, size_t dim,
+                        const ScoreParams& p, int* err, float* workspace);
+int shared_gemm_backward_query(int model, hipStream_t st, const float* table, size_t n_rows, const long long* ids,
+                               const float* q1, const float* q2, const float* gscore, float* gq1, float* gq2, size_t B,
+                               size_t K, size_t dim, const ScoreParams& p, float* workspace);
 
 // One extra stream and two events per device, created at first use and kept for the life of the process.
 struct SideStream {
@@ -238,7 +239,11 @@ int smx_score_backward_query(int model, void* stream, const float* table, size_t
 }
 
 size_t smx_shared_workspace_bytes(int model, size_t B, size_t K, size_t dim) {
-  return model == smx::mBetaKL ? (((K * (2 * dim + 1) + B) * sizeof(float) + 255) & ~(size_t)255) : 0;
+  if (model < 0 || model >= smx::mNumModels) return 0;
+  const size_t a = smx::shared_gemm_workspace_floats(model, B, K, dim, false);
+  const size_t b = smx::shared_gemm_workspace_floats(model, B, K, dim, true);
+  const size_t n = a > b ? a : b;
+  return n ? ((n * sizeof(float) + 255) & ~(size_t)255) : 0;
 }
 
 int smx_score_forward_shared(int model, void* stream, const float* table, size_t n_rows, const int64_t* ids,
@@ -250,10 +255,11 @@ int smx_score_forward_shared(int model, void* stream, const float* table, size_t
   if (!ids) return fail(SMX_ERR_ARG, "null id list");
   if (int rc = fill_args(&A, &vec, &nit, model, table, n_rows, ids, q1, q2, B, K, dim, params, nullptr, nullptr)) return rc;
   if (!score) return fail(SMX_ERR_ARG, "null score pointer");
-  // BetaE: the entity side of the divergence once per shared row (needs the workspace for the rows' terms)
-  if (model == mBetaKL && beta_shared_fits(dim, table, q1, q2, workspace, workspace_bytes, B, K))
-    return beta_shared_forward(as_stream(stream), table, n_rows, reinterpret_cast<const long long*>(ids), q1, q2, score, B,
-                               K, dim, A.p, err_flag, static_cast<float*>(workspace));
+  // BetaE (the entity side of the divergence once per shared row: needs the workspace), ComplEx, DistMult: the pairs
+  // as a matrix product
+  if (shared_gemm_fits(model, dim, table, q1, q2, workspace, workspace_bytes, B, K, false))
+    return shared_gemm_forward(model, as_stream(stream), table, n_rows, reinterpret_cast<const long long*>(ids), q1, q2,
+                               score, B, K, dim, A.p, err_flag, static_cast<float*>(workspace));
   if (shared_forward_fits(model, vec, nit)) {  // rows staged in LDS for eight queries at a time
     const SharedFwdArgs S{table, reinterpret_cast<const long long*>(ids), q1, q2, score, (int)B, (int)K, A.ncol, n_rows, A.p,
                           err_flag};
@@ -283,10 +289,9 @@ int smx_score_backward_query_shared(int model, void* stream, const float* table,
   if (!ids) return fail(SMX_ERR_ARG, "null id list");
   if (int rc = fill_args(&A, &vec, &nit, model, table, n_rows, ids, q1, q2, B, K, dim, params, nullptr, nullptr)) return rc;
   if (!score || !gscore || !gq1 || (model_nq(model) == 2 && !gq2)) return fail(SMX_ERR_ARG, "null pointer");
-  if (model == mBetaKL && aligned16(gq1) && aligned16(gq2) &&
-      beta_shared_fits(dim, table, q1, q2, workspace, workspace_bytes, B, K))
-    return beta_shared_backward_query(as_stream(stream), table, n_rows, reinterpret_cast<const long long*>(ids), q1, q2,
-                                      gscore, gq1, gq2, B, K, dim, A.p, static_cast<float*>(workspace));
+  if (shared_gemm_fits(model, dim, table, q1, q2, workspace, workspace_bytes, B, K, false))
+    return shared_gemm_backward_query(model, as_stream(stream), table, n_rows, reinterpret_cast<const long long*>(ids), q1,
+                                      q2, gscore, gq1, gq2, B, K, dim, A.p, static_cast<float*>(workspace));
   A.ids_shared = 1;
   A.score = score;
   A.gscore = gscore;

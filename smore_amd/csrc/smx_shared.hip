@@ -11,9 +11,11 @@ extern template int shared_entity_dispatch<mBetaKL>(hipStream_t, const SharedArg
 extern template int shared_entity_dispatch<mComplex>(hipStream_t, const SharedArgs&, int, int);
 extern template int shared_entity_dispatch<mDistmult>(hipStream_t, const SharedArgs&, int, int);
 
-// defined in smx_beta_shared.hip
-int beta_shared_entity_sums(hipStream_t st, const float* q1, const float* q2, const float* gscore, size_t B, size_t K,
-                            size_t dim, float* workspace);
+// defined in smx_shared_gemm.hip
+bool shared_gemm_fits(int model, size_t dim, const void* table, const void* q1, const void* q2, const void* workspace,
+                      size_t workspace_bytes, size_t B, size_t K, bool entity);
+int shared_gemm_entity_sums(int model, hipStream_t st, const float* q1, const float* q2, const float* gscore, size_t B,
+                            size_t K, size_t dim, float* workspace);
 
 }  // namespace smx
 
@@ -82,13 +84,12 @@ extern "C" int smx_score_backward_entity_shared(int model, void* stream, float* 
   A.table = table;
   A.ncol = (int)ncol;
   hipStream_t st = as_stream(stream);
-  // BetaE: the sums over the queries as a matrix product into the workspace, finished row by row below
-  if (model == mBetaKL && vec == 4 && workspace && aligned16(workspace) &&
-      workspace_bytes >= K * (2 * dim + 1) * sizeof(float)) {
+  // BetaE, ComplEx, DistMult: the sums over the queries as a matrix product into the workspace, finished row by row below
+  if (vec == 4 && shared_gemm_fits(model, dim, table, q1, q2, workspace, workspace_bytes, B, K, true)) {
     float* ws = static_cast<float*>(workspace);
-    if (int rc = beta_shared_entity_sums(st, q1, q2, gscore, B, K, dim, ws)) return rc;
+    if (int rc = shared_gemm_entity_sums(model, st, q1, q2, gscore, B, K, dim, ws)) return rc;
     A.sums_r = ws;
-    A.sums_c = ws + K * 2 * dim;
+    A.sums_c = ws + K * (size_t)model_nq(model) * dim;
   }
   switch (model) {
     case mL1: return shared_entity_dispatch<mL1>(st, A, vec, nit);

@@ -40,8 +40,8 @@ struct SharedArgs : RowSink {
   const int* seg_start;
   const long long* uniq;
   const int* n_uniq;
-  // beta_kl only: the sums over the queries come from a matrix product (R [K][2 dim] and C [K], see
-  // smx_beta_shared.hip) instead of being formed here
+  // beta_kl, complex, distmult: the sums over the queries come from a matrix product (R [K][nq dim] and, beta_kl,
+  // C [K], see smx_shared_gemm.hip) instead of being formed here
   const float* sums_r;
   const float* sums_c;
 };
@@ -81,25 +81,30 @@ __global__ __launch_bounds__(NW * 64) void shared_entity_kernel(SharedArgs A) {
     for (int x = 0; x < VEC; ++x) g1[it][x] = g2[it][x] = 0.f;
 
   bool have_sums = false;
-  if constexpr (M == mBetaKL && VEC == 4) {
-    if (A.sums_r) {  // uniform: S1 = ea C - R, S2 = eb C - R' per list position; the first wavefront alone has work
+  if constexpr ((M == mBetaKL || M == mComplex || M == mDistmult) && VEC == 4) {
+    if (A.sums_r) {  // uniform: the sums over the queries are there; the first wavefront alone has work
       have_sums = true;
       if (wave == 0) {
         for (int mi = m0; mi < m1; ++mi) {
           const int k = A.by_segment ? A.order[mi] : mi;
-          const float c = A.sums_c[k];
-          const float4* r = reinterpret_cast<const float4*>(A.sums_r + (size_t)k * 2 * half);
+          const float4* r = reinterpret_cast<const float4*>(A.sums_r + (size_t)k * NQ * half);
+          const float c = M == mBetaKL ? A.sums_c[k] : 0.f;
 #pragma unroll
           for (int it = 0; it < NIT; ++it) {
             const int col = min(lane + 64 * it, A.ncol - 1);
-            const float4 r1 = r[col], r2 = r[A.ncol + col];
+            const float4 r1 = r[col], r2 = NQ == 2 ? r[A.ncol + col] : r1;
             const float r1v[4] = {r1.x, r1.y, r1.z, r1.w}, r2v[4] = {r2.x, r2.y, r2.z, r2.w};
 #pragma unroll
             for (int x = 0; x < VEC; ++x) {
-              const float x1 = REG ? reg_apply(e.h[0][it].v[x], A.p) : e.h[0][it].v[x];
-              const float x2 = REG ? reg_apply(e.h[MUL - 1][it].v[x], A.p) : e.h[MUL - 1][it].v[x];
-              g1[it][x] += x1 * c - r1v[x];
-              g2[it][x] += x2 * c - r2v[x];
+              if constexpr (M == mBetaKL) {  // S1 = ea C - R, S2 = eb C - R'
+                const float x1 = REG ? reg_apply(e.h[0][it].v[x], A.p) : e.h[0][it].v[x];
+                const float x2 = REG ? reg_apply(e.h[MUL - 1][it].v[x], A.p) : e.h[MUL - 1][it].v[x];
+                g1[it][x] += x1 * c - r1v[x];
+                g2[it][x] += x2 * c - r2v[x];
+              } else {                       // the gradient row itself: sum_b g q
+                g1[it][x] += r1v[x];
+                if (MUL == 2) g2[it][x] += r2v[x];
+              }
             }
           }
         }
