@@ -193,6 +193,12 @@ template <int M, int VEC, int NIT, bool REG>
 int launch_shared_entity_reg(hipStream_t st, const SharedArgs& A) {
   const size_t row_bytes = (size_t)A.ncol * VEC * model_mul(M) * sizeof(float);
   // one workgroup per list position; with a plan the workgroups beyond the number of distinct ids leave at once
+  if constexpr ((M == mBetaKL || M == mComplex || M == mDistmult) && VEC == 4) {
+    if (A.sums_r) {  // the sums over the queries are there: one wavefront per row finishes it
+      hipLaunchKernelGGL((shared_entity_kernel<M, VEC, NIT, 1, REG>), dim3((unsigned)A.K), dim3(64), 0, st, A);
+      return check_launch("entity backward (shared negatives, rows from the sums)");
+    }
+  }
   if (7 * row_bytes <= 60 * 1024)
     hipLaunchKernelGGL((shared_entity_kernel<M, VEC, NIT, 8, REG>), dim3((unsigned)A.K), dim3(8 * 64), 7 * row_bytes, st, A);
   else
