@@ -39,7 +39,7 @@ def pytest_terminal_summary(terminalreporter, exitstatus, config):
     terminalreporter.section("tolerance headroom (worst err/bound per compared tensor)")
     rows = sorted(util.HEADROOM.items(), key=lambda kv: -kv[1][0])
     terminalreporter.write_line(f"{len(rows)} tensors compared; the 40 with the least headroom (all of them: "
-                                "gpurun_out/headroom.json when that folder exists)")
+                                "headroom.json in the folder SMX_TEST_REPORT_DIR names, when set)")
     n_all = sum(r[1][2] for r in rows)
     n_over = sum(r[1][3] for r in rows)
     terminalreporter.write_line(f"{n_over} of {n_all} compared elements ({n_over / max(n_all, 1):.2e}) lie outside the plain "
@@ -57,8 +57,8 @@ def pytest_terminal_summary(terminalreporter, exitstatus, config):
     terminalreporter.write_line("  in force  elementwise  outside/elements  test :: tensor")
     for (test, what), (with_floor, pure, n, over) in rows[:40]:
         terminalreporter.write_line(f"{with_floor:9.3g} {pure:9.3g}  {over:>7d}/{n:<9d} {test} :: {what}")
-    out_dir = os.path.join(ROOT, "gpurun_out")
-    if os.path.isdir(out_dir):
+    out_dir = os.environ.get("SMX_TEST_REPORT_DIR")
+    if out_dir and os.path.isdir(out_dir):
         import json
         with open(os.path.join(out_dir, "headroom.json"), "w") as f:
             json.dump([[t, w, a, b, n, over] for (t, w), (a, b, n, over) in rows], f, indent=0)
