@@ -17,7 +17,10 @@ pytestmark = pytest.mark.gpu
 SHAPES = [("box", 300, 9, 40, 48), ("l1", 200, 5, 17, 200), ("l2", 150, 6, 33, 36), ("rotate", 120, 7, 20, 500),
           ("beta_kl", 100, 4, 24, 400), ("beta_kl", 300, 19, 131, 64), ("beta_kl", 50, 3, 70, 516), ("beta_kl", 40, 9, 5, 30),
           ("complex", 90, 3, 10, 64), ("distmult", 90, 8, 65, 30), ("box", 500, 70, 130, 400),
-          ("complex", 150, 33, 45, 200), ("distmult", 120, 37, 70, 100), ("distmult", 300, 64, 96, 64)]
+          ("complex", 150, 33, 45, 200), ("distmult", 120, 37, 70, 100), ("distmult", 300, 64, 96, 64),
+          # edges of the matrix-product kernels: one query, one list position, a row of one float4, tiles cut on both axes
+          ("beta_kl", 20, 1, 1, 4), ("complex", 30, 2, 1, 8), ("distmult", 30, 1, 3, 12), ("beta_kl", 90, 65, 33, 36),
+          ("complex", 70, 32, 64, 16), ("distmult", 50, 31, 257, 4)]
 
 
 def _shared_problem(model, n, b, k, dim):
