@@ -65,6 +65,22 @@ def test_host_only_entry_points():
     assert abs(out[0] + 1e-3 / (1 - 0.9 ** 2)) < 1e-9 and abs(out[1] - (1 - 0.999 ** 2) ** -0.5) < 1e-4
 
 
+def test_workspace_sizes_of_the_shared_negative_calls():
+    """smx_shared_workspace_bytes (host only): nothing for the distance models; the matrix-product models need the
+    entity side's sums [K, n_q dim], BetaE also its per-row terms [K, 2 dim + 1] and per-query terms [B]."""
+    from smore_amd import _lib
+    from smore_amd.fused import MODELS
+    lib = _lib.load()
+    b, k, d = 512, 1024, 400
+    up = lambda n: (4 * n + 255) // 256 * 256
+    for model in ("l1", "l2", "box", "rotate"):
+        assert lib.smx_shared_workspace_bytes(MODELS[model], b, k, d) == 0
+    assert lib.smx_shared_workspace_bytes(MODELS["distmult"], b, k, d) == up(k * d)
+    assert lib.smx_shared_workspace_bytes(MODELS["complex"], b, k, d) == up(k * 2 * d)
+    assert lib.smx_shared_workspace_bytes(MODELS["beta_kl"], b, k, d) == up(k * (2 * d + 1) + b)
+    assert lib.smx_shared_workspace_bytes(99, b, k, d) == 0
+
+
 def test_multi_stream_entity_pass_refuses_bad_source_lists():
     """Argument checks of smx_score_backward_entity_multi happen before any launch: they can run without a GPU."""
     from smore_amd import _lib
