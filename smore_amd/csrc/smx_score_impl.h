@@ -246,13 +246,19 @@ __device__ __forceinline__ void flush_codes(const unsigned char* stage, unsigned
   }
 }
 
-// DEDUP: a wavefront scores each DISTINCT entity among its (up to 64) pairs once.  With skewed ids a query's
-// negatives repeat the hot entities many times (Zipf 1.1: ~51 distinct among 64 consecutive negatives), every
-// repeat costs the same instructions as the first occurrence although its row comes from the cache, and at such
-// shapes the kernel is bound by instruction issue.  The lanes find equal ids with one ballot per id bit, the
-// first lane of each group represents it, the representatives' rows are streamed, and every pair then takes
-// its score (and its code bytes, from the wavefront's LDS stage) from its representative: the same bits as
-// without de-duplication, pair by pair.
+// DEDUP: a workgroup scores each DISTINCT entity among the (up to 256) pairs of its tile once.  With skewed ids a
+// query's negatives repeat the hot entities many times (Zipf 1.1: ~175 distinct among 256 consecutive negatives,
+// ~51 among 64), every repeat costs the same instructions as the first occurrence although its row comes from
+// the cache, and at such shapes the kernel is bound by instruction issue.  The lanes enter their ids into a small
+// hash table in LDS; whoever enters an id first puts its row on the tile's list of representatives; the list is
+// dealt out to the four wavefronts in equal parts and streamed; every pair then takes its score (and its code
+// bytes, from the tile's LDS stage) from its representative: the same bits as without de-duplication, pair by
+// pair, whichever wavefront happened to score the row.
+constexpr int kDedupSlots = 512;   // hash table entries for the 256 ids of a tile
+constexpr unsigned kDedupEmpty = 0xffffffffu;  // (no id: the table has at most 2^32 - 1 rows)
+// LDS bytes of the de-duplication tables: ids and list positions of the slots, row addresses and scores of the list
+constexpr size_t kDedupLds = kDedupSlots * 8 + 256 * 8 + 256 * 4 + 16;
+
 template <int M, int VEC, int NIT, int RIF, bool REG, bool CODED = false, bool DEDUP = false>
 __global__ __launch_bounds__(256) void score_forward_kernel(ScoreArgs A, int tiles, int tile_k) {
   const float* __restrict__ table = A.table;
@@ -282,32 +288,65 @@ __global__ __launch_bounds__(256) void score_forward_kernel(ScoreArgs A, int til
   if (cnt > 0)
     pb = load_pair_batch(idx, (A.ids_shared ? (size_t)0 : (size_t)(b / A.U) * K) + kw0, cnt, lane, row_len, n_rows, bad);
 
-  stage_query<M>(lds, q1, q2, b, dim);
+  // LDS: query | per-wavefront pair slabs | code stage (per wavefront; one for the tile with DEDUP) | DEDUP tables
+  unsigned* slab = reinterpret_cast<unsigned*>(lds + model_nq(M) * dim) + wave * kSlabDwords;
+  constexpr int kStaged = DEDUP ? 256 : kStagePairs;  // pairs whose code bytes a stage holds
+  unsigned char* stage_base = reinterpret_cast<unsigned char*>(lds + model_nq(M) * dim + 4 * kSlabDwords);
+  unsigned char* stage = DEDUP ? stage_base : stage_base + wave * (kStaged * NIT * 64);
+  unsigned char* after_stage = stage_base + (CODED ? (size_t)(DEDUP ? 1 : 4) * kStaged * NIT * 64 : 0);
+  unsigned* slot_id = reinterpret_cast<unsigned*>(after_stage);                   // [kDedupSlots]
+  int* slot_pos = reinterpret_cast<int*>(slot_id + kDedupSlots);                   // [kDedupSlots]
+  uint2* rep_addr = reinterpret_cast<uint2*>(slot_pos + kDedupSlots);              // [256]
+  float* rep_score = reinterpret_cast<float*>(rep_addr + 256);                     // [256]
+  int* rep_count = reinterpret_cast<int*>(rep_score + 256);
+  if constexpr (DEDUP) {
+    for (int i = threadIdx.x; i < kDedupSlots; i += 256) slot_id[i] = kDedupEmpty;
+    if (threadIdx.x == 0) *rep_count = 0;
+  }
+
+  stage_query<M>(lds, q1, q2, b, dim);  // (ends with a barrier: the tables are cleared)
   typename ModelOps<M>::Q q[NIT][VEC];
   load_query_regs<M, VEC, NIT, true>(lds, dim, ncol, lane, q);
-  if (cnt <= 0) return;
-  unsigned* slab = reinterpret_cast<unsigned*>(lds + model_nq(M) * dim) + wave * kSlabDwords;
-  stage_pairs(slab, lane, table, pb, 0.f, 0.f);
+  if constexpr (!DEDUP) {
+    if (cnt <= 0) return;
+  }
   int n_stream = cnt;        // rows this wavefront streams
-  int my_slot = lane;        // position among them of the row my pair's score comes from
+  int first_rep = 0;         // DEDUP: position on the tile's list of the first of them
+  int my_pos = lane;         // DEDUP: position on the list of the row my pair's score comes from
   if constexpr (DEDUP) {
-    const unsigned long long live = __ballot(lane < cnt);
-    const unsigned long long same = match_key(pb.row, A.id_bits, live) | (1ull << lane);
-    int rep = __builtin_ctzll(same);  // lowest lane with my id (ids that differ only above bit 31: checked below)
-    if (__shfl((int)pb.off_lo, rep) != (int)pb.off_lo || __shfl((int)pb.off_hi, rep) != (int)pb.off_hi) rep = lane;
-    const unsigned long long reps = __ballot(rep == lane && lane < cnt);
-    n_stream = __popcll(reps);
-    const int my_rank = (int)lanes_below_in(reps);   // for a representative: its position among the streamed rows
-    my_slot = __shfl(my_rank, rep);
-    // the slab holds every lane's own row address (stage_pairs, fenced); the representatives now move theirs to
-    // the front, in lane order.  rank <= lane, ranks are distinct, nobody reads in this phase, and the entries
-    // from n_stream on keep a valid address for the unconditional loads of the row loop
-    if (rep == lane && lane < cnt) {
-      const unsigned long long addr =
-          (unsigned long long)(table + (((unsigned long long)pb.off_hi << 32) | pb.off_lo));
-      *reinterpret_cast<uint2*>(slab + 4 * my_rank) = make_uint2((unsigned)addr, (unsigned)(addr >> 32));
+    if (lane < cnt) {
+      const unsigned key = pb.row;
+      unsigned s = (key * 2654435761u) >> 23;  // 9 bits
+      bool first = false;
+      while (true) {
+        const unsigned old = atomicCAS(&slot_id[s], kDedupEmpty, key);
+        first = old == kDedupEmpty;
+        if (first || old == key) break;
+        s = (s + 1) & (kDedupSlots - 1);
+      }
+      if (first) {
+        const int pos = atomicAdd(rep_count, 1);
+        slot_pos[s] = pos;
+        const unsigned long long addr =
+            (unsigned long long)(table + (((unsigned long long)pb.off_hi << 32) | pb.off_lo));
+        rep_addr[pos] = make_uint2((unsigned)addr, (unsigned)(addr >> 32));
+      }
+      my_pos = (int)s;  // the slot for now; its list position once everybody has entered
     }
-    slab_fence();
+    __syncthreads();
+    if (lane < cnt) my_pos = slot_pos[my_pos];
+    const int n_reps = *rep_count;
+    const int share = (n_reps + 3) / 4;  // <= 64
+    first_rep = wave * share;
+    n_stream = max(0, min(share, n_reps - first_rep));
+    // this wavefront's part of the list goes into its slab (entries past its end repeat the last: the row loop's
+    // loads are unconditional)
+    if (n_stream > 0) {
+      *reinterpret_cast<uint2*>(slab + 4 * lane) = rep_addr[first_rep + min(lane, n_stream - 1)];
+      slab_fence();
+    }
+  } else {
+    stage_pairs(slab, lane, table, pb, 0.f, 0.f);
   }
 
   float neg_thr[NIT][VEC];
@@ -318,9 +357,7 @@ __global__ __launch_bounds__(256) void score_forward_kernel(ScoreArgs A, int til
       for (int v = 0; v < VEC; ++v) neg_thr[it][v] = ModelOps<M>::neg_threshold(q[it][v]);
   }
   float* out = score + (size_t)b * K + kw0;
-  constexpr int kStaged = DEDUP ? 64 : kStagePairs;  // pairs whose code bytes the wavefront's stage holds
-  unsigned char* stage =
-      reinterpret_cast<unsigned char*>(lds + model_nq(M) * dim + 4 * kSlabDwords) + wave * (kStaged * NIT * 64);
+  if (n_stream > 0)
   stream_batch<MUL, VEC, NIT, RIF>(slab, n_stream, dim, ncol, lane,
                                    [&](int j, const Pack<VEC>(&e1)[NIT], const Pack<VEC>(&e2)[NIT]) {
     // lanes past the row end hold a copy of the last column: they compute along and are dropped here.
@@ -333,7 +370,7 @@ __global__ __launch_bounds__(256) void score_forward_kernel(ScoreArgs A, int til
         unsigned code = 0;
 #pragma unroll
         for (int v = 0; v < VEC; ++v) ModelOps<M>::fwd_coded(e1[it].v[v], q[it][v], neg_thr[it][v], a0, a1, code);
-        stage[(j & (kStaged - 1)) * (NIT * 64) + 64 * it + lane] = (unsigned char)code;
+        stage[((DEDUP ? first_rep + j : j) & (kStaged - 1)) * (NIT * 64) + 64 * it + lane] = (unsigned char)code;
       } else {
 #pragma unroll
         for (int v = 0; v < VEC; ++v) {
@@ -347,31 +384,30 @@ __global__ __launch_bounds__(256) void score_forward_kernel(ScoreArgs A, int til
     }
     const float folded = wave_sum_last_f32(mine);
     if constexpr (DEDUP) {
-      // the score of streamed row j waits in the third word of slab entry j (free in the forward; the entry's
-      // address words were consumed when the row was requested): one LDS store instead of vector selects
-      if (lane == 63) slab[4 * j + 2] = __float_as_uint(ModelOps<M>::score(folded, p));
+      if (lane == 63) rep_score[first_rep + j] = ModelOps<M>::score(folded, p);
     } else {
       if (lane == 63) out[j] = ModelOps<M>::score(folded, p);
       if constexpr (CODED) flush_codes<NIT>(stage, A.codes, (size_t)b * K + kw0, j, cnt, lane);
     }
   });
   if constexpr (DEDUP) {
-    // every pair takes what its representative produced: the score from the representative's slab entry ...
-    slab_fence();
-    if (lane < cnt) out[lane] = __uint_as_float(slab[4 * my_slot + 2]);
+    // every pair takes what its representative produced: the score from the tile's list ...
+    __syncthreads();
+    if (lane < cnt) out[lane] = rep_score[my_pos];
     if constexpr (CODED) {
       // ... and its NIT x 64 code bytes from the representative's row of the stage, 16 bytes per lane and turn;
       // the wavefront's pairs are contiguous in the code array
-      slab_fence();
-      typedef unsigned vec4u __attribute__((ext_vector_type(4)));
-      constexpr int kPer = NIT * 4;  // 16-byte pieces per pair
-      vec4u* dst = reinterpret_cast<vec4u*>(A.codes + ((size_t)b * K + kw0) * (size_t)(NIT * 64));
-      for (int c0 = 0; c0 < cnt * kPer; c0 += 64) {
-        const int c = c0 + lane;
-        const int pair = min(c / kPer, cnt - 1);
-        const int src_row = __shfl(my_slot, pair);
-        if (c < cnt * kPer)
-          __builtin_nontemporal_store(reinterpret_cast<const vec4u*>(stage + src_row * (NIT * 64))[c % kPer], dst + c);
+      if (cnt > 0) {
+        typedef unsigned vec4u __attribute__((ext_vector_type(4)));
+        constexpr int kPer = NIT * 4;  // 16-byte pieces per pair
+        vec4u* dst = reinterpret_cast<vec4u*>(A.codes + ((size_t)b * K + kw0) * (size_t)(NIT * 64));
+        for (int c0 = 0; c0 < cnt * kPer; c0 += 64) {
+          const int c = c0 + lane;
+          const int pair = min(c / kPer, cnt - 1);
+          const int src_row = __shfl(my_pos, pair);
+          if (c < cnt * kPer)
+            __builtin_nontemporal_store(reinterpret_cast<const vec4u*>(stage + src_row * (NIT * 64))[c % kPer], dst + c);
+        }
       }
     }
   }
@@ -683,14 +719,14 @@ int launch_forward_reg(hipStream_t st, const ScoreArgs& A) {
   const int tiles = (int)((K + tile_k - 1) / tile_k);
   const size_t lds = ((size_t)model_nq(M) * A.ncol * VEC + 4 * kSlabDwords) * sizeof(float);
   // ids given (not the dense layout, whose rows are all different): score each distinct entity of a
-  // wavefront's batch once
+  // tile once
   // (not for a list of ids shared by the batch: a sampler's K negatives hardly ever repeat)
   const bool dedup = A.idx != nullptr && !A.ids_shared;
   if constexpr (model_coded(M) && !REG) {
     if (A.codes) {
       if (dedup)
         hipLaunchKernelGGL((score_forward_kernel<M, VEC, NIT, RIF, REG, true, true>), dim3((unsigned)(B * tiles)),
-                           dim3(256), lds + 4 * 64 * NIT * 64, st, A, tiles, tile_k);
+                           dim3(256), lds + 256 * NIT * 64 + kDedupLds, st, A, tiles, tile_k);
       else
         hipLaunchKernelGGL((score_forward_kernel<M, VEC, NIT, RIF, REG, true>), dim3((unsigned)(B * tiles)), dim3(256),
                            lds + 4 * kStagePairs * NIT * 64, st, A, tiles, tile_k);
@@ -699,7 +735,7 @@ int launch_forward_reg(hipStream_t st, const ScoreArgs& A) {
   }
   if (dedup)
     hipLaunchKernelGGL((score_forward_kernel<M, VEC, NIT, RIF, REG, false, true>), dim3((unsigned)(B * tiles)),
-                       dim3(256), lds, st, A, tiles, tile_k);
+                       dim3(256), lds + kDedupLds, st, A, tiles, tile_k);
   else
     hipLaunchKernelGGL((score_forward_kernel<M, VEC, NIT, RIF, REG>), dim3((unsigned)(B * tiles)), dim3(256), lds, st, A,
                        tiles, tile_k);

@@ -930,8 +930,8 @@ def test_several_index_streams_at_a_size_that_forks():
 
 
 @pytest.mark.parametrize("model,dim", [("box", 200), ("box", 400), ("l1", 30), ("l2", 64), ("rotate", 48), ("beta_kl", 20)])
-def test_forward_scores_each_distinct_entity_of_a_wavefront_once(model, dim):
-    """The forward de-duplicates ids inside a wavefront's batch of up to 64 negatives: every pair must still get
+def test_forward_scores_each_distinct_entity_of_a_tile_once(model, dim):
+    """The forward de-duplicates ids inside a workgroup's tile of negatives: every pair must still get
     the bits it would get alone.  Queries whose negatives are all one entity, all distinct, drawn from three
     entities, and a last batch of 6 pairs (K = 70); scores against the dense layout (rows given pair by pair, no
     ids, no de-duplication) bit for bit and against the oracle; sign codes (box, l1) through the backward that
@@ -974,6 +974,47 @@ def test_forward_scores_each_distinct_entity_of_a_wavefront_once(model, dim):
         assert_close(got[True][1].cpu().numpy(), got[False][1].cpu().numpy(), 1e-6, "gq1 from the forward's codes")
     else:
         assert codes is None
+
+
+@pytest.mark.parametrize("model,dim,n", [("box", 16, 3000), ("l2", 8, 200), ("box", 200, 100_000)])
+def test_forward_de_duplication_over_full_tiles(model, dim, n):
+    """2 M pairs, so that the forward takes tiles of 256 negatives (four wavefronts share one hash table and one list
+    of distinct entities): skewed ids from a small table -- every tile holds repeats inside and across its
+    wavefronts, and ids that collide in the table's slots.  Scores against the dense layout (rows given pair by pair,
+    nothing to de-duplicate) bit for bit; the sign codes of repeats must be their representative's; the
+    query gradient from those codes against the recomputing backward."""
+    from smore_amd import fused
+    rng = np.random.default_rng(seed("dedup-tiles", model, dim, n))
+    b, k = 2048, 1024
+    table = rng.uniform(-0.07, 0.07, (n, dim)).astype(np.float32)
+    q1 = rng.uniform(-0.07, 0.07, (b, dim)).astype(np.float32)
+    q2 = np.abs(rng.uniform(-0.07, 0.07, (b, dim))).astype(np.float32) if model == "box" else None
+    idx = np.minimum((rng.pareto(0.9, (b, k)) * 3).astype(np.int64), n - 1)
+    idx[5, :] = 17                                     # a query whose negatives are one entity
+    idx[6, :] = (np.arange(k) * 7) % n                 # ... and one without repeats inside a tile
+    t_table, t_q1, t_q2 = torch.tensor(table, device="cuda"), torch.tensor(q1, device="cuda"), None if q2 is None else torch.tensor(q2, device="cuda")
+    t_idx = torch.tensor(idx, device="cuda")
+    params = fused.score_params(GAMMA[model], 0.02)
+    err = fused.new_error_flag("cuda")
+    score = fused.score_forward(model, t_table, t_idx, t_q1, t_q2, params, err)
+    dense = torch.empty_like(score)
+    for b0 in range(0, b, 256):                        # the dense layout in slices: [256 * K, dim] rows at a time
+        rows = t_table[t_idx[b0:b0 + 256].reshape(-1)]
+        dense[b0:b0 + 256] = fused.score_forward(model, rows, None, t_q1[b0:b0 + 256], None if t_q2 is None else t_q2[b0:b0 + 256], params)
+    assert torch.equal(score, dense)
+    assert err.item() == 0
+    codes = fused.new_codes(model, t_table, t_idx, t_q1)
+    if codes is not None:
+        score_c = fused.score_forward(model, t_table, t_idx, t_q1, t_q2, params, codes=codes)
+        assert torch.equal(score_c, score)
+        per_pair = codes.view(b, k, -1)
+        assert torch.equal(per_pair[5], per_pair[5, :1].expand(k, -1)), "repeats must carry their representative's codes"
+        same = t_idx[:64, 1:] == t_idx[:64, :-1]       # neighbours with one id: one code record
+        assert torch.equal(per_pair[:64, 1:][same], per_pair[:64, :-1][same])
+        gs = torch.randn((b, k), device="cuda", generator=torch.Generator(device="cuda").manual_seed(3))
+        from_codes = fused.score_backward_query(model, t_table, t_idx, t_q1, t_q2, score, gs, params, codes=codes)
+        recomputed = fused.score_backward_query(model, t_table, t_idx, t_q1, t_q2, score, gs, params)
+        assert_close(from_codes[0].cpu().numpy(), recomputed[0].cpu().numpy(), 1e-6, "gq1 from the forward's codes, full tiles")
 
 
 @pytest.mark.parametrize("model,ks,dim", [("box", (12,), 24), ("box", (1, 20), 24), ("l1", (1, 7), 24), ("l2", (5,), 24),
