@@ -250,14 +250,15 @@ __device__ __forceinline__ void flush_codes(const unsigned char* stage, unsigned
 // query's negatives repeat the hot entities many times (Zipf 1.1: ~175 distinct among 256 consecutive negatives,
 // ~51 among 64), every repeat costs the same instructions as the first occurrence although its row comes from
 // the cache, and at such shapes the kernel is bound by instruction issue.  The lanes enter their ids into a small
-// hash table in LDS; whoever enters an id first puts its row on the tile's list of representatives; the list is
-// dealt out to the four wavefronts in equal parts and streamed; every pair then takes its score (and its code
-// bytes, from the tile's LDS stage) from its representative: the same bits as without de-duplication, pair by
-// pair, whichever wavefront happened to score the row.
+// hash table in LDS; the first pair of the tile with an id puts its row on the tile's list of representatives; the
+// list (in pair order) is dealt out to the four wavefronts in equal parts and streamed; every pair then takes its
+// score (and its code bytes, from the tile's LDS stage) from its representative: the same bits as without
+// de-duplication, pair by pair.
 constexpr int kDedupSlots = 512;   // hash table entries for the 256 ids of a tile
 constexpr unsigned kDedupEmpty = 0xffffffffu;  // (no id: the table has at most 2^32 - 1 rows)
-// LDS bytes of the de-duplication tables: ids and list positions of the slots, row addresses and scores of the list
-constexpr size_t kDedupLds = kDedupSlots * 8 + 256 * 8 + 256 * 4 + 16;
+// LDS bytes of the de-duplication tables: ids, first pairs and list positions of the slots, row addresses and
+// scores of the list, representatives per wavefront
+constexpr size_t kDedupLds = kDedupSlots * 12 + 256 * 8 + 256 * 4 + 16;
 
 template <int M, int VEC, int NIT, int RIF, bool REG, bool CODED = false, bool DEDUP = false>
 __global__ __launch_bounds__(256) void score_forward_kernel(ScoreArgs A, int tiles, int tile_k) {
@@ -298,10 +299,13 @@ __global__ __launch_bounds__(256) void score_forward_kernel(ScoreArgs A, int til
   int* slot_pos = reinterpret_cast<int*>(slot_id + kDedupSlots);                   // [kDedupSlots]
   uint2* rep_addr = reinterpret_cast<uint2*>(slot_pos + kDedupSlots);              // [256]
   float* rep_score = reinterpret_cast<float*>(rep_addr + 256);                     // [256]
-  int* rep_count = reinterpret_cast<int*>(rep_score + 256);
+  int* slot_first = reinterpret_cast<int*>(rep_score + 256);                        // [kDedupSlots]
+  int* wave_reps = slot_first + kDedupSlots;                                        // [4]
   if constexpr (DEDUP) {
-    for (int i = threadIdx.x; i < kDedupSlots; i += 256) slot_id[i] = kDedupEmpty;
-    if (threadIdx.x == 0) *rep_count = 0;
+    for (int i = threadIdx.x; i < kDedupSlots; i += 256) {
+      slot_id[i] = kDedupEmpty;
+      slot_first[i] = 0x7fffffff;
+    }
   }
 
   stage_query<M>(lds, q1, q2, b, dim);  // (ends with a barrier: the tables are cleared)
@@ -314,28 +318,42 @@ __global__ __launch_bounds__(256) void score_forward_kernel(ScoreArgs A, int til
   int first_rep = 0;         // DEDUP: position on the tile's list of the first of them
   int my_pos = lane;         // DEDUP: position on the list of the row my pair's score comes from
   if constexpr (DEDUP) {
+    // The representative of an id is its first pair of the tile, and the list holds the representatives in pair
+    // order: which wavefront scores which row is then the same in every run (a row's bits may depend on where it
+    // stands in a wavefront's stream, through the contraction of multiply-adds in the unrolled row loop).
+    const int pair_in_tile = wave * per_wave + lane;
+    unsigned s = 0;
     if (lane < cnt) {
       const unsigned key = pb.row;
-      unsigned s = (key * 2654435761u) >> 23;  // 9 bits
-      bool first = false;
+      s = (key * 2654435761u) >> 23;  // 9 bits
       while (true) {
         const unsigned old = atomicCAS(&slot_id[s], kDedupEmpty, key);
-        first = old == kDedupEmpty;
-        if (first || old == key) break;
+        if (old == kDedupEmpty || old == key) break;
         s = (s + 1) & (kDedupSlots - 1);
       }
-      if (first) {
-        const int pos = atomicAdd(rep_count, 1);
-        slot_pos[s] = pos;
-        const unsigned long long addr =
-            (unsigned long long)(table + (((unsigned long long)pb.off_hi << 32) | pb.off_lo));
-        rep_addr[pos] = make_uint2((unsigned)addr, (unsigned)(addr >> 32));
-      }
-      my_pos = (int)s;  // the slot for now; its list position once everybody has entered
+      atomicMin(&slot_first[s], pair_in_tile);
     }
     __syncthreads();
-    if (lane < cnt) my_pos = slot_pos[my_pos];
-    const int n_reps = *rep_count;
+    const bool is_rep = lane < cnt && slot_first[s] == pair_in_tile;
+    const unsigned long long reps = __ballot(is_rep);
+    if (lane == 0) wave_reps[wave] = __popcll(reps);
+    __syncthreads();
+    int before = 0, n_reps = 0;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const int c = wave_reps[w];
+      before += w < wave ? c : 0;
+      n_reps += c;
+    }
+    if (is_rep) {
+      const int pos = before + (int)lanes_below_in(reps);
+      slot_pos[s] = pos;
+      const unsigned long long addr =
+          (unsigned long long)(table + (((unsigned long long)pb.off_hi << 32) | pb.off_lo));
+      rep_addr[pos] = make_uint2((unsigned)addr, (unsigned)(addr >> 32));
+    }
+    __syncthreads();
+    if (lane < cnt) my_pos = slot_pos[s];
     const int share = (n_reps + 3) / 4;  // <= 64
     first_rep = wave * share;
     n_stream = max(0, min(share, n_reps - first_rep));
