@@ -105,7 +105,9 @@ int smx_dist_backward_f64(int kind, void* stream, const double* gout, const doub
  * An id outside [0, n_rows) sets *err_flag (device int, may be NULL) to 1 and
  * row 0 is read in its place for the score and the query gradient; the caller
  * decides when to look at the flag.  No table row is ever updated for such a
- * pair (see smx_plan_build). */
+ * pair (see smx_plan_build).  With an id list, n_rows is at most 2^32 - 1
+ * (SMX_ERR_SHAPE beyond: ids are told apart by their low 32 bits, as in the
+ * segment plan). */
 typedef struct smx_score_params {
   float gamma;   /* margin: logit = gamma - distance */
   float cen;     /* BOX: weight of the inside distance */

@@ -139,6 +139,8 @@ static int fill_args(ScoreArgs* A, int* vec, int* nit, int model, const float* t
   if (B == 0 || K == 0 || dim == 0) return fail(SMX_ERR_SHAPE, "empty dimension");
   if (B > 0x7fffffffull || K > 0x7fffffffull || B * K > 0x7fffffffull)
     return fail(SMX_ERR_SHAPE, "more than 2^31-1 pairs in one call");
+  if (idx && n_rows > 0xffffffffull)  // the kernels tell ids apart by their low 32 bits, as the segment plan does
+    return fail(SMX_ERR_SHAPE, "entity count %zu needs ids wider than 32 bits", n_rows);
   if (params->reg_on && model != mBetaKL)
     return fail(SMX_ERR_ARG, "the entity clamp prologue exists for the beta_kl model only");
   const bool vec4 = dim % 4 == 0 && aligned16(table) && aligned16(q1) && (model_nq(model) == 1 || aligned16(q2)) &&
@@ -159,8 +161,6 @@ static int fill_args(ScoreArgs* A, int* vec, int* nit, int model, const float* t
   A->ncol = (int)ncol;
   A->n_rows = idx ? n_rows : B * K;
   A->U = 1;
-  A->id_bits = 1;
-  while (A->id_bits < 32 && ((A->n_rows - 1) >> A->id_bits) != 0) ++A->id_bits;
   A->p = ScoreParams{params->gamma, params->cen, params->reg_on, params->reg_add, params->reg_lo, params->reg_hi};
   return SMX_OK;
 }

@@ -40,7 +40,6 @@ struct ScoreArgs {
   // "query" is then one branch row, number bq = b * U + u, which scores the ids of query b.
   int U;                 // branches per query (1: none of this)
   const unsigned char* winner;  // query backward, [B, K]: the branch that gave the pair's logit; a branch row sums its own pairs only
-  int id_bits;           // significant bits of n_rows - 1 (at most 32): what the forward compares to find equal ids
   unsigned long long n_rows;
   ScoreParams p;
   int* err;

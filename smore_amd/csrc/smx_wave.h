@@ -44,18 +44,6 @@ __device__ __forceinline__ float wave_sum_last_f32(float v) {
   return v;
 }
 
-// Lanes of the wavefront (among those of `live`) whose low `bits` bits of `key` equal this lane's: one ballot
-// per bit, combined with a three-input bit operation per half (same & ~(has ^ mine)).  `bits` is wave-uniform.
-__device__ __forceinline__ unsigned long long match_key(unsigned key, int bits, unsigned long long live) {
-  unsigned lo = (unsigned)live, hi = (unsigned)(live >> 32);
-  for (int b = 0; b < bits; ++b) {
-    const unsigned mine = (unsigned)__builtin_amdgcn_sbfe((int)key, b, 1);  // 0 or ~0
-    const unsigned long long has = __ballot(mine != 0u);
-    lo = __builtin_amdgcn_bitop3_b32(lo, (unsigned)has, mine, 0x90);
-    hi = __builtin_amdgcn_bitop3_b32(hi, (unsigned)(has >> 32), mine, 0x90);
-  }
-  return ((unsigned long long)hi << 32) | lo;
-}
 // Number of set bits of m at lanes below this one.
 __device__ __forceinline__ unsigned lanes_below_in(unsigned long long m) {
   return __builtin_amdgcn_mbcnt_hi((unsigned)(m >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)m, 0u));

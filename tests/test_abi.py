@@ -108,6 +108,17 @@ def test_multi_stream_entity_pass_refuses_bad_source_lists():
     assert call(2, b=5, rows=fake, n_rows=3) != 0 and b"gradient rows" in lib.smx_last_error()   # the plan holds 40, not 43
 
 
+def test_scorer_refuses_tables_whose_ids_need_more_than_32_bits():
+    """The forward finds equal ids of a tile by their low 32 bits: a table with more rows is refused on the host."""
+    from smore_amd import _lib
+    import ctypes as c
+    lib = _lib.load()
+    params = _lib.ScoreParams(24.0, 0.02, 0, 0.0, 0.0, 0.0)
+    fake = c.c_void_p(256)          # never dereferenced
+    rc = lib.smx_score_forward(2, None, fake, 1 << 32, fake, fake, fake, fake, 2, 4, 8, c.byref(params), None, None, 0)
+    assert rc != 0 and b"wider than 32 bits" in lib.smx_last_error()
+
+
 def test_missing_library_fails_loudly(monkeypatch):
     from smore_amd import _lib
     monkeypatch.setattr(_lib, "_lib", None)
