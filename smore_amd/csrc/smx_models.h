@@ -110,7 +110,7 @@ template <> struct ModelOps<mL1> {
     a0 += fabsf(d);
     code = push2(code, __ballot(!(d > 0.f)), 0ull);
   }
-  static __device__ __forceinline__ void bwd_q_coded(float c0, float, float e1, const Q& q, float& gq1, float&,
+  static __device__ __forceinline__ void bwd_q_coded(float c0, float, float e1, const Q& q, float, float& gq1, float&,
                                                      unsigned& code) {
     const float d = e1 - q.a;
     const bool pos = d > 0.f;
@@ -185,16 +185,17 @@ template <> struct ModelOps<mBox> {
     c0 = -g;
     c1 = -p.cen * g;
   }
-  // gradient of the entity feature; the center's is its negative
-  // Written as three selects on three compares: that is what the hardware does in one instruction each
-  // (v_cmp + v_cndmask with a sign modifier).  |d| >= o decides the same as |d| - o >= 0 for finite
-  // operands (a difference of two distinct floats never rounds to zero).
+  // gradient of the entity feature; the center's is its negative:
+  //   outside (|d| >= o) ? (d > 0 ? c0 : -c0) : (d >= 0 ? c1 : -c1)
+  // The two sign rules differ at d == 0 only, and there "outside" means o <= 0: so the sign is  d > t  with
+  // t = 0 where o <= 0 and the largest negative float where o > 0 (d > t is then d >= 0), which is -o clamped
+  // to [t_min, 0] -- one v_med3 instead of a second compare and a select.
   static __device__ __forceinline__ float de(float c0, float c1, float e1, const Q& q, bool& outside) {
     const float d = e1 - q.a;
     outside = fabsf(d) >= q.b;
-    const float r_out = d > 0.f ? c0 : -c0;
-    const float r_in = d >= 0.f ? c1 : -c1;
-    return outside ? r_out : r_in;
+    const float mag = outside ? c0 : c1;
+    const float t = __builtin_amdgcn_fmed3f(-q.b, __uint_as_float(0x80000001u), 0.f);
+    return d > t ? mag : -mag;
   }
   static __device__ __forceinline__ void bwd_e(float c0, float c1, float e1, float, const Q& q, float& ge1, float&) {
     bool outside;
@@ -206,6 +207,17 @@ template <> struct ModelOps<mBox> {
     gc -= de(c0, c1, e1, q, outside);
     go += outside ? c0 : 0.f;
   }
+  // The same for a kernel that keeps the query in registers: the sign decision of de() is one compare against
+  // the feature's neg_threshold (below), which such a kernel computes once per query instead of two compares
+  // and a select per pair.  Same decisions for finite operands, same +-c terms, same bits.
+  static __device__ __forceinline__ void bwd_q_thr(float c0, float c1, float e1, const Q& q, float neg_thr, float& gc,
+                                                   float& go) {
+    const float d = e1 - q.a;
+    const bool outside = fabsf(d) >= q.b;
+    const float mag = outside ? c0 : c1;
+    gc -= d < neg_thr ? -mag : mag;
+    go += outside ? c0 : 0.f;
+  }
   static __device__ __forceinline__ void finish_q(const Q& q, float&, float& go, const ScoreParams& p) {
     go *= (q.b > 0.f ? p.cen : -p.cen) - 1.0f;
   }
@@ -215,17 +227,15 @@ template <> struct ModelOps<mBox> {
   // The kernels that make these decisions anyway (forward, or the query-gradient kernel) can leave
   // them behind, one byte per four features; the entity pass then sums  +-c  straight from the codes
   // and needs neither the query rows nor the comparisons -- same decisions, same bits.
-  // As bwd_q, and pushes this feature's two bits onto `code`.
-  static __device__ __forceinline__ void bwd_q_coded(float c0, float c1, float e1, const Q& q, float& gc, float& go,
-                                                     unsigned& code) {
+  // As bwd_q_thr, and pushes this feature's two bits onto `code`.
+  static __device__ __forceinline__ void bwd_q_coded(float c0, float c1, float e1, const Q& q, float neg_thr, float& gc,
+                                                     float& go, unsigned& code) {
     const float d = e1 - q.a;
-    const bool outside = fabsf(d) >= q.b, gt = d > 0.f, ge = d >= 0.f;
-    const float r_out = gt ? c0 : -c0;
-    const float r_in = ge ? c1 : -c1;
-    gc -= outside ? r_out : r_in;
+    const bool outside = fabsf(d) >= q.b, neg = d < neg_thr;
+    const float mag = outside ? c0 : c1;
+    gc -= neg ? -mag : mag;
     go += outside ? c0 : 0.f;
-    const unsigned long long T = __ballot(outside), GT = __ballot(gt), GE = __ballot(ge);
-    code = push2(code, ~((T & GT) | (~T & GE)), T);
+    code = push2(code, __ballot(neg), __ballot(outside));
   }
   // As fwd, and pushes this feature's two bits onto `code`: the forward pass
   // can leave the codes too, and then the whole backward works from them without the entity rows.

@@ -473,10 +473,14 @@ __global__ __launch_bounds__(NW * 64) void score_backward_query_kernel(ScoreArgs
   load_query_regs<M, VEC, NIT, false>(lds, dim, ncol, lane, q);
 
   float g1[NIT][VEC], g2[NIT][VEC];
+  [[maybe_unused]] float neg_thr[NIT][VEC];  // sign-coded models, when this kernel makes the comparisons itself
 #pragma unroll
   for (int it = 0; it < NIT; ++it)
 #pragma unroll
-    for (int v = 0; v < VEC; ++v) g1[it][v] = g2[it][v] = 0.f;
+    for (int v = 0; v < VEC; ++v) {
+      g1[it][v] = g2[it][v] = 0.f;
+      if constexpr (model_coded(M)) neg_thr[it][v] = ModelOps<M>::neg_threshold(q[it][v]);
+    }
   // LDS: query | per-wavefront partial sums | per-wavefront pair slabs
   unsigned* slab = reinterpret_cast<unsigned*>(lds + (NW + 1) * NQ * dim) + wave * kSlabDwords;
   unsigned char* stage =
@@ -599,7 +603,7 @@ __global__ __launch_bounds__(NW * 64) void score_backward_query_kernel(ScoreArgs
           unsigned code = 0;
 #pragma unroll
           for (int v = 0; v < VEC; ++v)
-            ModelOps<M>::bwd_q_coded(c.x, c.y, e1[it].v[v], q[it][v], g1[it][v], g2[it][v], code);
+            ModelOps<M>::bwd_q_coded(c.x, c.y, e1[it].v[v], q[it][v], neg_thr[it][v], g1[it][v], g2[it][v], code);
           mine_b[64 * it] = (unsigned char)code;
         }
         flush_codes<NIT>(stage, A.codes, first, j, cnt, lane);
@@ -610,7 +614,8 @@ __global__ __launch_bounds__(NW * 64) void score_backward_query_kernel(ScoreArgs
           for (int v = 0; v < VEC; ++v) {
             const float x1 = REG ? reg_apply(e1[it].v[v], p) : e1[it].v[v];
             const float x2 = MUL == 2 ? (REG ? reg_apply(e2[it].v[v], p) : e2[it].v[v]) : 0.f;
-            ModelOps<M>::bwd_q(c.x, c.y, x1, x2, q[it][v], g1[it][v], g2[it][v]);
+            if constexpr (M == mBox) ModelOps<M>::bwd_q_thr(c.x, c.y, x1, q[it][v], neg_thr[it][v], g1[it][v], g2[it][v]);
+            else ModelOps<M>::bwd_q(c.x, c.y, x1, x2, q[it][v], g1[it][v], g2[it][v]);
           }
         }
       }

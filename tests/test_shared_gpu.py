@@ -20,7 +20,11 @@ SHAPES = [("box", 300, 9, 40, 48), ("l1", 200, 5, 17, 200), ("l2", 150, 6, 33, 3
           ("complex", 150, 33, 45, 200), ("distmult", 120, 37, 70, 100), ("distmult", 300, 64, 96, 64),
           # edges of the matrix-product kernels: one query, one list position, a row of one float4, tiles cut on both axes
           ("beta_kl", 20, 1, 1, 4), ("complex", 30, 2, 1, 8), ("distmult", 30, 1, 3, 12), ("beta_kl", 90, 65, 33, 36),
-          ("complex", 70, 32, 64, 16), ("distmult", 50, 31, 257, 4)]
+          ("complex", 70, 32, 64, 16), ("distmult", 50, 31, 257, 4),
+          # lists of 512 and more ids under 64 and more queries: the entity side takes two rows per workgroup (an odd
+          # number of positions and of distinct ids, ids that hold several positions beside ids that hold one)
+          ("box", 700, 70, 513, 200), ("box", 2000, 64, 512, 400), ("l1", 800, 65, 515, 64), ("l2", 700, 66, 600, 100),
+          ("rotate", 900, 64, 512, 100)]
 
 
 def _shared_problem(model, n, b, k, dim):
