@@ -389,8 +389,10 @@ def score_backward_entity_multi(model, plan, table, q1, q2, sources, params, mer
         _f32(gscore, "gscore")
         if score.numel() % b or gscore.shape != score.shape:
             raise _lib.SmxError("score and gscore of a source must both be [B, K]")
-        if (branches > 1) != (winner is not None):
-            raise _lib.SmxError("union queries, and only they, bring a winner array per source")
+        if branches > 1 and winner is None:
+            raise _lib.SmxError("union queries bring a winner array per source")
+        if branches == 1:
+            winner = None       # a union of one branch is a plain query: its winner array holds zeros
         arr[i] = _lib.PairSource(_ptr(score), _ptr(gscore), _ptr(codes), 0 if codes is None else codes.numel(),
                                  score.numel() // b, _ptr(winner))
     row_len = table.shape[1]

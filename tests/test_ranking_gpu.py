@@ -40,7 +40,7 @@ def test_integer_valued_l1_ranks_are_exact_ties_included():
 
 
 @pytest.mark.parametrize("model,dim", [("box", 200), ("l2", 64), ("rotate", 100), ("beta_kl", 40), ("box", 30), ("complex", 48),
-                                       ("distmult", 64)])
+                                       ("distmult", 64), ("beta_kl", 30)])
 def test_ranks_lie_in_the_interval_fp32_allows(model, dim):
     """Random floats: an entity whose logit is within fp32 error of an answer's may fall on either side;
     every rank must lie between the counts with the tolerance subtracted and added."""
@@ -72,7 +72,8 @@ def test_ranks_lie_in_the_interval_fp32_allows(model, dim):
         m = ranking_metrics(got[i][0])
         if hard[i]:
             rr = got[i][0].cpu().numpy().astype(np.float64)
-            assert abs(m["MRR"] - (1 / rr).mean()) < 1e-6 and m["HITS10"] == (rr <= 10).mean()
+            # (the metrics are fp32 means, as in the reference: train_process.py:150-154)
+            assert abs(m["MRR"] - (1 / rr).mean()) < 1e-6 and abs(m["HITS10"] - (rr <= 10).mean()) < 1e-6
         else:
             assert m == dict(MRR=0.0, HITS1=0.0, HITS3=0.0, HITS10=0.0, HITS1max=0.0)
 

@@ -14,7 +14,8 @@ pytestmark = pytest.mark.gpu
 
 @pytest.mark.parametrize("model,n,b,u,k,dim", [("box", 300, 6, 2, 70, 48), ("l1", 100, 5, 3, 33, 200), ("rotate", 80, 4, 2, 20, 500),
                                               ("beta_kl", 90, 3, 2, 24, 64), ("l2", 120, 7, 4, 65, 36),
-                                              ("distmult", 60, 2, 2, 9, 30)])
+                                              ("distmult", 60, 2, 2, 9, 30),
+                                              ("box", 200, 5, 1, 40, 48)])    # one branch: a plain query through the union calls
 def test_union_forward_and_both_backwards_match_oracle(model, n, b, u, k, dim):
     from smore_amd import fused
     rng = np.random.default_rng(seed("union", model, n, b, u, k, dim))
