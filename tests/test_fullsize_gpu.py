@@ -222,7 +222,9 @@ def test_plan_around_the_tile_geometry_boundaries():
     gen = torch.Generator(device="cuda")
     gen.manual_seed(99)
     per = 1024 * 256
-    for n_pairs in (16 * per - 1, 16 * per, 16 * per + 1, 17 * per, 17 * per + 1, 18 * per - 1, 18 * per, 18 * per + 1,
+    # (and of the emit kernel's: one sorted position per thread up to 2^18 positions, four up to 2^20, sixteen beyond)
+    for n_pairs in (4097, per - 1, per, per + 1, 4 * per - 1, 4 * per, 4 * per + 1,
+                    16 * per - 1, 16 * per, 16 * per + 1, 17 * per, 17 * per + 1, 18 * per - 1, 18 * per, 18 * per + 1,
                     18 * per + 18 * 1024, 19 * per + 7):
         ids = torch.randint(0, n, (n_pairs,), device="cuda", generator=gen)
         ids[: n_pairs // 50] = ids[0]                                  # one long segment as well
