@@ -271,6 +271,8 @@ typedef struct smx_pair_source {
   size_t fwd_codes_bytes;
   size_t K;
   const uint8_t* winner;   /* [B, K] union queries only (smx_score_backward_entity_union), else NULL */
+  size_t q_first;          /* first query (row of q1 / q2; with union queries: group of U rows) of this source */
+  size_t n_queries;        /* queries of this source; 0 = B, all of them */
 } smx_pair_source;
 int smx_score_backward_entity_multi(int model, void* stream, const smx_plan_view* plan, float* table,
                                     size_t n_rows, const float* q1, const float* q2,

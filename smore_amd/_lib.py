@@ -116,7 +116,7 @@ class PlanView(ctypes.Structure):
 class PairSource(ctypes.Structure):
     """smx_pair_source of include/smore_amd.h."""
     _fields_ = [("score", _vp), ("gscore", _vp), ("fwd_codes", _vp), ("fwd_codes_bytes", _sz), ("K", _sz),
-                ("winner", _vp)]
+                ("winner", _vp), ("q_first", _sz), ("n_queries", _sz)]
 
 
 MAX_PAIR_SOURCES = 4

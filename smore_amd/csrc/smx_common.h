@@ -32,6 +32,8 @@ struct PairSources {
   const float* gscore[kMaxSources];
   const unsigned char* codes[kMaxSources];
   size_t K[kMaxSources];
+  size_t B[kMaxSources];        // queries of the source, and the row of q1 / q2 (group of U rows) where they start
+  size_t q_first[kMaxSources];
   // union queries: U branch rows per query in q1 / q2, and per source the branch that gave each pair's logit
   // (null when U == 1)
   const unsigned char* winner[kMaxSources];

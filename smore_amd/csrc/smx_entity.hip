@@ -162,30 +162,37 @@ int entity_backward(int model, void* stream, const smx_plan_view* plan, float* t
   const size_t row_len = dim * model_mul(model);
   if (int rc = fill_plan(&A, plan, workspace, workspace_bytes, row_len)) return rc;
   const size_t n_grad = multi ? multi->n_grad : 0;
-  if (plan->n_pairs != B * K + n_grad)
-    return fail(SMX_ERR_SHAPE, "plan holds %zu pairs, call has %zu", plan->n_pairs, B * K + n_grad);
-  if (n_grad) {
-    if (!multi->grad_rows) return fail(SMX_ERR_ARG, "null gradient rows");
-    A.grad_rows = multi->grad_rows;
-    A.rows_first = (int)(B * K);
-  }
-  if (multi) {  // K is then the sum of the sources' K (checked by the caller): pairs of source s start at B * (K_0 + .. + K_s-1)
+  // the model's pairs: B * K, or what the sources hold (a source has its own K and, when the sources belong to
+  // different query batches, its own stretch of the B query rows)
+  size_t n_model = B * K;
+  if (multi) {
     if (multi->n < 1 || multi->n > kMaxSources) return fail(SMX_ERR_ARG, "1 to %d pair sources", kMaxSources);
     A.n_src = multi->n;
     size_t first = 0;
     for (int i = 0; i < multi->n; ++i) {
       if (!multi->score[i] || !multi->gscore[i] || multi->K[i] == 0) return fail(SMX_ERR_ARG, "incomplete pair source %d", i);
       if ((codes != nullptr) != (multi->codes[i] != nullptr)) return fail(SMX_ERR_ARG, "sign codes for some pair sources only");
+      if (multi->B[i] == 0 || multi->q_first[i] + multi->B[i] > B)
+        return fail(SMX_ERR_SHAPE, "pair source %d: queries %zu .. %zu of %zu", i, multi->q_first[i],
+                    multi->q_first[i] + multi->B[i], B);
       A.first[i] = (int)first;
       A.src_score[i] = multi->score[i];
       A.src_gscore[i] = multi->gscore[i];
       A.src_codes[i] = multi->codes[i];
       A.src_K[i] = (int)multi->K[i];
+      A.src_q0[i] = (int)multi->q_first[i];
       A.src_winner[i] = multi->winner[i];
-      first += B * multi->K[i];
+      first += multi->B[i] * multi->K[i];
     }
-    if (first != B * K) return fail(SMX_ERR_SHAPE, "pair sources hold %zu pairs, plan %zu", first, B * K);
     for (int i = multi->n; i <= kMaxSources; ++i) A.first[i] = (int)first;
+    n_model = first;
+  }
+  if (plan->n_pairs != n_model + n_grad)
+    return fail(SMX_ERR_SHAPE, "plan holds %zu pairs, call has %zu", plan->n_pairs, n_model + n_grad);
+  if (n_grad) {
+    if (!multi->grad_rows) return fail(SMX_ERR_ARG, "null gradient rows");
+    A.grad_rows = multi->grad_rows;
+    A.rows_first = (int)n_model;
   }
   if (int rc = fill_adam(&A, m, v, adam)) return rc;
   const bool vec4 = dim % 4 == 0 && aligned16(table) && aligned16(q1) && (!q2 || aligned16(q2)) &&
@@ -210,6 +217,7 @@ int entity_backward(int model, void* stream, const smx_plan_view* plan, float* t
     A.U = (int)multi->U;
   }
   if (multi && multi->n == 1) {  // one index stream (+ gradient rows): the single-source fields describe it
+    if (multi->q_first[0] != 0) return fail(SMX_ERR_ARG, "a single pair source starts at the first query");
     A.n_src = 0;
     A.score = multi->score[0];
     A.gscore = multi->gscore[0];

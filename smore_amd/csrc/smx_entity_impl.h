@@ -67,10 +67,12 @@ struct EntityArgs : RowSink {
   const unsigned char* codes;
   // several index streams in one plan (positives + negatives of one query batch, embed_optimizer.py:155-163):
   // n_src > 1, and pair p of the plan with first[s] <= p < first[s+1] is pair (p - first[s]) of source s, which
-  // has its own score / gscore / codes arrays and its own K; all sources share q1, q2.  n_src <= 1: the single
-  // source described by score, gscore, codes and K above.
+  // has its own score / gscore / codes arrays and its own K; its queries are rows src_q0[s] .. of q1, q2 (all
+  // sources the same rows when they belong to one query batch).  n_src <= 1: the single source described by
+  // score, gscore, codes and K above.
   int n_src;
   int first[kMaxSources + 1];
+  int src_q0[kMaxSources];
   const float* src_score[kMaxSources];
   const float* src_gscore[kMaxSources];
   const unsigned char* src_codes[kMaxSources];
@@ -212,7 +214,7 @@ __device__ __forceinline__ void load_window(const EntityArgs& A, int lane, int b
     my_pair = pair;
     float c1;
     if (A.n_src > 1) {  // uniform: which index stream the pair came from, and its number inside that stream
-      int local = pair, K = A.src_K[0];
+      int local = pair, K = A.src_K[0], q0 = A.src_q0[0];
       const float* gs = A.src_gscore[0];
       const float* sc = A.src_score[0];
       const unsigned char* win = A.src_winner[0];
@@ -221,13 +223,14 @@ __device__ __forceinline__ void load_window(const EntityArgs& A, int lane, int b
         if (s < A.n_src && pair >= A.first[s]) {
           local = pair - A.first[s];
           K = A.src_K[s];
+          q0 = A.src_q0[s];
           gs = A.src_gscore[s];
           sc = A.src_score[s];
           win = A.src_winner[s];
         }
       }
       ModelOps<SRC>::coef(gs[local], sc[local], A.p, my_c, c1);
-      my_key = local / K;
+      my_key = q0 + local / K;
       if (A.U > 1) my_key = my_key * A.U + win[local];  // the query row of the branch that won the pair
     } else {
       ModelOps<SRC>::coef(A.gscore[pair], A.score[pair], A.p, my_c, c1);
@@ -678,12 +681,13 @@ __device__ __forceinline__ CodedLane resolve_coded_lane(const EntityArgs& A, int
   if (!want) return L;
   const bool is_row = plan_pair >= A.rows_first;
   const int pair = is_row ? 0 : plan_pair;  // a pair whose inputs exist
-  int local = pair, K = A.K;
+  int local = pair, K = A.K, q0 = 0;
   const float* gs = A.gscore;
   const float* sc = A.score;
   const unsigned char* cb = A.codes;
   if (A.n_src > 1) {  // uniform: which index stream the pair came from, and its number inside that stream
     K = A.src_K[0];
+    q0 = A.src_q0[0];
     gs = A.src_gscore[0];
     sc = A.src_score[0];
     cb = A.src_codes[0];
@@ -692,6 +696,7 @@ __device__ __forceinline__ CodedLane resolve_coded_lane(const EntityArgs& A, int
       if (s < A.n_src && pair >= A.first[s]) {
         local = pair - A.first[s];
         K = A.src_K[s];
+        q0 = A.src_q0[s];
         gs = A.src_gscore[s];
         sc = A.src_score[s];
         cb = A.src_codes[s];
@@ -700,7 +705,7 @@ __device__ __forceinline__ CodedLane resolve_coded_lane(const EntityArgs& A, int
   }
   float c1;
   ModelOps<SRC>::coef(gs[local], sc[local], A.p, L.c, c1);
-  L.key = local / K;
+  L.key = q0 + local / K;
   L.pair = pair;
   L.code = cb + (size_t)local * (NIT * 64);
   if (is_row) {

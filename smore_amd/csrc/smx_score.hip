@@ -418,6 +418,8 @@ static int entity_multi(int model, void* stream, const smx_plan_view* plan, floa
     return fail(SMX_ERR_ARG, "1 to %d pair sources", kMaxSources);
   if ((grad_rows != nullptr) != (n_grad_rows != 0)) return fail(SMX_ERR_ARG, "gradient rows and their count must come together");
   if (U == 0 || U > 255) return fail(SMX_ERR_SHAPE, "1 to 255 union branches");
+  if (n_src == 1 && (src[0].q_first != 0 || (src[0].n_queries != 0 && src[0].n_queries != B)))
+    return fail(SMX_ERR_ARG, "a single pair source covers all B queries");
   if (n_src == 1 && !grad_rows && U == 1)
     return smx_score_backward_entity(model, stream, plan, table, n_rows, q1, q2, src[0].score, src[0].gscore, B,
                                      src[0].K, dim, params, merged, m, v, adam, workspace, workspace_bytes,
@@ -425,7 +427,7 @@ static int entity_multi(int model, void* stream, const smx_plan_view* plan, floa
   if (model < 0 || model >= mNumModels) return fail(SMX_ERR_KIND, "unknown score model %d", model);
   PairSources S{};
   S.n = (int)n_src;
-  size_t k_sum = 0;
+  size_t k_sum = 0, n_model = 0;
   const bool coded = src[0].fwd_codes != nullptr;
   int codes_vec = 0, codes_nit = 0;
   if (coded) {
@@ -437,7 +439,7 @@ static int entity_multi(int model, void* stream, const smx_plan_view* plan, floa
     if (!src[i].score || !src[i].gscore || src[i].K == 0) return fail(SMX_ERR_ARG, "incomplete pair source %zu", i);
     if ((src[i].fwd_codes != nullptr) != coded) return fail(SMX_ERR_ARG, "sign codes for some pair sources only");
     if (coded) {
-      if (src[i].fwd_codes_bytes != B * src[i].K * code_bytes_per_pair(dim))
+      if (src[i].fwd_codes_bytes != (src[i].n_queries ? src[i].n_queries : B) * src[i].K * code_bytes_per_pair(dim))
         return fail(SMX_ERR_ARG, "codes buffer of source %zu is not smx_score_codes_bytes() long", i);
       if (reinterpret_cast<uintptr_t>(src[i].fwd_codes) & 15u) return fail(SMX_ERR_ARG, "codes must be 16-byte aligned");
     }
@@ -445,24 +447,29 @@ static int entity_multi(int model, void* stream, const smx_plan_view* plan, floa
     S.gscore[i] = src[i].gscore;
     S.codes[i] = static_cast<const unsigned char*>(src[i].fwd_codes);
     S.K[i] = src[i].K;
+    S.B[i] = src[i].n_queries ? src[i].n_queries : B;
+    S.q_first[i] = src[i].q_first;
+    if (S.q_first[i] + S.B[i] > B)
+      return fail(SMX_ERR_SHAPE, "pair source %zu: queries %zu .. %zu of %zu", i, S.q_first[i], S.q_first[i] + S.B[i], B);
     S.winner[i] = src[i].winner;
     if (U > 1 && !src[i].winner) return fail(SMX_ERR_ARG, "union queries: pair source %zu has no winner array", i);
     k_sum += src[i].K;
+    n_model += S.B[i] * src[i].K;
   }
   S.U = U;
   if (U > 1 && coded) return fail(SMX_ERR_ARG, "union queries have no sign codes");
   S.grad_rows = grad_rows;
   S.n_grad = n_grad_rows;
-  const size_t n_all = B * k_sum + n_grad_rows;
+  const size_t n_all = n_model + n_grad_rows;
   if (B == 0 || n_all > 0x7fffffffull) return fail(SMX_ERR_SHAPE, "pair count out of range");
   if (!plan || plan->n_pairs != n_all)
-    return fail(SMX_ERR_SHAPE, "the plan must hold the %zu pairs of all sources and the %zu gradient rows", B * k_sum,
+    return fail(SMX_ERR_SHAPE, "the plan must hold the %zu pairs of all sources and the %zu gradient rows", n_model,
                 n_grad_rows);
   // the same division of work as smx_score_backward_entity: ids that occur once in the whole step go through
   // the pair-ordered kernel, one launch per source, while the entity pass reduces the others beside it
   const bool split = coded && adam && !merged && plan->pair_seg && plan->uniq && plan->order && plan->sorted_ids &&
                      plan->seg_of_pos && plan->seg_start && plan->n_uniq && queries_beyond_l2(model, B, dim) &&
-                     B * k_sum >= ((size_t)1 << 20) && workspace && !(reinterpret_cast<uintptr_t>(workspace) & 255u) &&
+                     n_model >= ((size_t)1 << 20) && workspace && !(reinterpret_cast<uintptr_t>(workspace) & 255u) &&
                      workspace_bytes >= entity_ws_bytes(n_all, dim * model_mul(model)) && !serial_backward() &&
                      (!grad_rows || aligned16(grad_rows));
   if (split) {
@@ -472,7 +479,11 @@ static int entity_multi(int model, void* stream, const smx_plan_view* plan, floa
     size_t first = 0;
     for (size_t i = 0; i < n_src && fits; ++i) {
       int vec, nit;
-      if (int rc = fill_args(&A[i], &vec, &nit, model, table, n_rows, nullptr, q1, q2, B, src[i].K, dim, params, nullptr, m))
+      // (the one-pair kernel numbers a source's queries from its own first row)
+      const float* s_q1 = q1 + S.q_first[i] * dim;
+      const float* s_q2 = q2 ? q2 + S.q_first[i] * dim : nullptr;
+      if (int rc = fill_args(&A[i], &vec, &nit, model, table, n_rows, nullptr, s_q1, s_q2, S.B[i], src[i].K, dim, params,
+                             nullptr, m))
         return rc;
       fits = vec == codes_vec && nit == codes_nit && !(vec == 4 && v && !adam->squeeze && !aligned16(v));
       A[i].n_rows = n_rows;
@@ -482,7 +493,7 @@ static int entity_multi(int model, void* stream, const smx_plan_view* plan, floa
       A[i].pair_seg = plan->pair_seg + first;
       A[i].uniq = reinterpret_cast<const long long*>(plan->uniq);
       fill_sink(&A[i], table, m, v, nullptr, adam);
-      first += B * src[i].K;
+      first += S.B[i] * src[i].K;
     }
     if (fits) {
       SideStream* side = side_stream();

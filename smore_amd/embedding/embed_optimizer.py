@@ -449,9 +449,10 @@ class EmbeddingOptimizer(ABC):
             idx_list = [i.reshape(-1).to(self.sparse_embed.device) for i, _ in self.grad_list]
             grad_list = [g.reshape(g.shape[0] if g.dim() == 2 else -1, g.shape[-1]).contiguous().float()
                          for _, g in self.grad_list]
-            if self.fused_list and (len(self.fused_list) == 1 or self._one_query_batch(self.fused_list)):
-                # positives and negatives of one query batch (kg_reasoning.py:340-355): one plan over all their
-                # ids, one entity pass that reads each record's own scores / upstream gradients / sign codes.
+            if self.fused_list and (len(self.fused_list) == 1 or self._one_entity_pass(self.fused_list)):
+                # positives and negatives of one query batch (kg_reasoning.py:340-355), or records of several batches
+                # scored in one step: one plan over all their ids, one entity pass that reads each record's own
+                # scores / upstream gradients / sign codes against its own queries.
                 # Negatives shared by the batch bring one gradient row per list position (each the sum over all
                 # queries, formed by one workgroup per row) instead of B x K pairs.  Those rows, and the rows of the
                 # step's plain lookups -- the anchor entities every query starts from (box.py:137), whose gradient
@@ -511,31 +512,55 @@ class EmbeddingOptimizer(ABC):
                                         first["gscore"], first["params"], merged=merged, m=m, v=v, adam=adam,
                                         codes=first["codes"])
             return
-        sources = [(r["score"], r["gscore"], r["codes"]) + ((r["winner"],) if first["branches"] > 1 else ()) for r in recs]
-        fused.score_backward_entity_multi(first["model"], plan, table, first["q1"], first["q2"], sources, first["params"],
+        # records of one query batch share its tensors; those of several batches (several forward calls in one step)
+        # get the batches one after the other and each record its stretch of them
+        batches, starts = [], []
+        for r in recs:
+            for i, b in enumerate(batches):
+                if self._same_tensor(r["q1"], b["q1"]) and self._same_tensor(r["q2"], b["q2"]):
+                    starts.append(i)
+                    break
+            else:
+                batches.append(r)
+                starts.append(len(batches) - 1)
+        if len(batches) == 1:
+            q1, q2 = first["q1"], first["q2"]
+            sources = [(r["score"], r["gscore"], r["codes"]) + ((r["winner"],) if first["branches"] > 1 else ())
+                       for r in recs]
+        else:
+            dim = first["q1"].shape[-1]
+            rows = [b["q1"].numel() // (dim * first["branches"]) for b in batches]
+            offs = [sum(rows[:i]) for i in range(len(rows))]
+            q1 = torch.cat([b["q1"].reshape(-1, dim) for b in batches], dim=0)
+            q2 = None if first["q2"] is None else torch.cat([b["q2"].reshape(-1, dim) for b in batches], dim=0)
+            sources = [(r["score"], r["gscore"], r["codes"], r["winner"] if first["branches"] > 1 else None,
+                        offs[starts[i]], rows[starts[i]]) for i, r in enumerate(recs)]
+        fused.score_backward_entity_multi(first["model"], plan, table, q1, q2, sources, first["params"],
                                           merged=merged, m=m, v=v, adam=adam, grad_rows=grad_rows,
                                           branches=first["branches"])
 
     @staticmethod
-    def _one_query_batch(recs):
-        """True when the fused records can share one entity pass: same model and score parameters, the same
-        query tensors (same memory, shape and version), sign codes for all per-query records or for none, few
-        enough of those."""
+    def _same_tensor(a, b):
+        if a is None or b is None:
+            return a is b
+        return a.data_ptr() == b.data_ptr() and a.shape == b.shape and a._version == b._version
+
+    @staticmethod
+    def _one_entity_pass(recs):
+        """True when the fused records can share one entity pass: same model, score parameters and number of union
+        branches, sign codes for all per-query records or for none, few enough of those.  Their query batches may
+        differ (records of several forward calls in one step, embed_optimizer.py:155-163 of the reference)."""
         own = [r for r in recs if not r["shared"]]
         if len(recs) < 2 or len(own) > _lib.MAX_PAIR_SOURCES:
             return False
         first = recs[0]
 
-        def same_tensor(a, b):
-            if a is None or b is None:
-                return a is b
-            return a.data_ptr() == b.data_ptr() and a.shape == b.shape and a._version == b._version
-
         def same_params(a, b):
             return all(getattr(a, f) == getattr(b, f) for f, _ in a._fields_)
 
         return (all(r["model"] == first["model"] and same_params(r["params"], first["params"]) and
-                    same_tensor(r["q1"], first["q1"]) and same_tensor(r["q2"], first["q2"]) for r in recs[1:]) and
+                    r["branches"] == first["branches"] and (r["q2"] is None) == (first["q2"] is None) and
+                    r["q1"].shape[-1] == first["q1"].shape[-1] for r in recs[1:]) and
                 all((r["codes"] is None) == (own[0]["codes"] is None) for r in own[1:]))
 
 

@@ -369,10 +369,12 @@ def score_backward_query_union(model, table, idx, q1, q2, score, gscore, winner,
 def score_backward_entity_multi(model, plan, table, q1, q2, sources, params, merged=None, m=None, v=None, adam=None,
                                 grad_rows=None, branches=1):
     """score_backward_entity for several index streams of one query batch (see smx_score_backward_entity_multi).
-    sources: list of (score [B,K_s], gscore [B,K_s], codes or None[, winner]); plan: built over the concatenation of
-    the streams' flattened ids in the same order.  grad_rows [n, row]: materialised gradient rows of the step's plain
-    lookups, whose ids are the last n entries of that concatenation.  branches > 1: union queries, q1 / q2 are
-    [B * branches, dim] and every source brings its winner array (smx_score_backward_entity_union)."""
+    sources: list of (score [B,K_s], gscore [B,K_s], codes or None[, winner[, q_first, n_queries]]); plan: built over
+    the concatenation of the streams' flattened ids in the same order.  grad_rows [n, row]: materialised gradient rows
+    of the step's plain lookups, whose ids are the last n entries of that concatenation.  branches > 1: union queries,
+    q1 / q2 are [B * branches, dim] and every source brings its winner array (smx_score_backward_entity_union).
+    Sources of different query batches: q1 / q2 hold the batches one after the other and a source names its stretch
+    of queries with q_first and n_queries (its score is then [n_queries, K_s])."""
     dim = q1.shape[-1]
     b = q1.numel() // (dim * branches)
     if model not in MODELS:
@@ -385,16 +387,19 @@ def score_backward_entity_multi(model, plan, table, q1, q2, sources, params, mer
     for i, src in enumerate(sources):
         score, gscore, codes = src[:3]
         winner = src[3] if len(src) > 3 else None
+        q_first, n_q = (int(src[4]), int(src[5])) if len(src) > 5 else (0, b)
         _f32(score, "score")
         _f32(gscore, "gscore")
-        if score.numel() % b or gscore.shape != score.shape:
-            raise _lib.SmxError("score and gscore of a source must both be [B, K]")
+        if n_q < 1 or q_first < 0 or q_first + n_q > b:
+            raise _lib.SmxError(f"a source's queries {q_first} .. {q_first + n_q} of {b}")
+        if score.numel() % n_q or gscore.shape != score.shape:
+            raise _lib.SmxError("score and gscore of a source must both be [its queries, K]")
         if branches > 1 and winner is None:
             raise _lib.SmxError("union queries bring a winner array per source")
         if branches == 1:
             winner = None       # a union of one branch is a plain query: its winner array holds zeros
         arr[i] = _lib.PairSource(_ptr(score), _ptr(gscore), _ptr(codes), 0 if codes is None else codes.numel(),
-                                 score.numel() // b, _ptr(winner))
+                                 score.numel() // n_q, _ptr(winner), q_first, 0 if n_q == b else n_q)
     row_len = table.shape[1]
     _check_state(table, m, v, adam)
     if merged is not None and (merged.dim() != 2 or merged.shape[1] != row_len):

@@ -493,10 +493,13 @@ def test_row_optimizers_match_oracle(name, squeeze):
         assert_close(emb.state_sum_fo.cpu().numpy(), m, 2e-5, "adam first moment")
 
 
-def test_fused_records_of_two_query_batches_and_a_plain_lookup_in_one_step():
-    """Two score_negatives calls against DIFFERENT query tensors cannot share one entity pass: each record is
-    reduced to per-entity gradient rows, merged with the plain lookup's rows (embed_optimizer.py:155-163) and
-    applied as one update per entity.  Against the oracle's merge of all three index streams."""
+@pytest.mark.parametrize("gamma_b", [12.0, 9.0])
+def test_fused_records_of_two_query_batches_and_a_plain_lookup_in_one_step(gamma_b):
+    """Two score_negatives calls against DIFFERENT query tensors: their records still share one plan and one entity
+    pass (each source reads its own stretch of the query rows, laid one batch after the other), together with the
+    plain lookup's gradient rows (embed_optimizer.py:155-163), and every entity gets one update.  Against the
+    oracle's merge of all three index streams.  Records scored with different margins (second case) cannot share a
+    pass: each is reduced to per-entity gradient rows first and those are merged."""
     n, d, b, k, lr = 300, 32, 6, 10, 1e-3
     rng = np.random.default_rng(12)
     f32 = lambda a: np.asarray(a).astype(np.float32).astype(np.float64)
@@ -511,16 +514,17 @@ def test_fused_records_of_two_query_batches_and_a_plain_lookup_in_one_step():
     ta, tb = dev(qa).requires_grad_(), dev(qb).requires_grad_()
     opt.zero_grad()
     la = opt.score_negatives("l1", torch.tensor(ids_a, device="cuda"), ta, None, gamma=12.0)
-    lb = opt.score_negatives("l1", torch.tensor(ids_b, device="cuda"), tb, None, gamma=12.0)
+    lb = opt.score_negatives("l1", torch.tensor(ids_b, device="cuda"), tb, None, gamma=gamma_b)
     rows = emb(torch.tensor(looked, device="cuda"), "anchor")
     ((la * dev(ga)).sum() + (lb * dev(gb)).sum() + (rows * dev(gl)).sum()).backward()
     assert len(opt.fused_list) == 2 and len(opt.grad_list) == 1
     opt.apply_grad(lr)
     opt.check_ids()
+    assert opt.stats["per_record_merges"] == (0 if gamma_b == 12.0 else 2)
     grads = []
-    for ids, q, g, t, logit in ((ids_a, qa, ga, ta, la), (ids_b, qb, gb, tb, lb)):
+    for ids, q, g, t, logit, gamma in ((ids_a, qa, ga, ta, la, 12.0), (ids_b, qb, gb, tb, lb, gamma_b)):
         e = orc.gather(table, ids).reshape(b, k, d)
-        assert_close(logit.detach().cpu().numpy(), orc.score_forward("l1", e, q[:, None], None, 12.0), REL_F32, "logits")
+        assert_close(logit.detach().cpu().numpy(), orc.score_forward("l1", e, q[:, None], None, gamma), REL_F32, "logits")
         g_rows, g_q, _ = orc.score_backward("l1", g, e, q[:, None], None)
         assert_close(t.grad.cpu().numpy(), g_q[:, 0], REL_F32, "query gradient")
         grads.append(g_rows.reshape(b * k, d))

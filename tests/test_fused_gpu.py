@@ -888,6 +888,63 @@ def test_entity_pass_over_several_index_streams(model):
     assert torch.equal(a, b_)
 
 
+@pytest.mark.parametrize("model", ["box", "l1", "l2", "rotate", "beta_kl", "distmult"])
+def test_entity_pass_over_streams_of_different_query_batches(model):
+    """Records of several forward calls in one step (the reference merges them like any others,
+    embed_optimizer.py:155-163): three streams of three query batches (B = 5, 3, 8; K = 7, 20, 1) whose query rows lie
+    one after the other, each source naming its stretch; the second and third batch share entities with the first.
+    Merged rows against the oracle's unique-merge + scatter-sum, then one Adam step."""
+    from smore_amd import fused
+    n, dim, lr = 120, 24, 1e-3
+    shapes = ((5, 7), (3, 20), (8, 1))
+    rng = np.random.default_rng(seed("multi-batch", model))
+    b_all = sum(b for b, _ in shapes)
+    table, q1, q2, _, _ = make_problem(model, n, b_all, 1, dim, rng)
+    gamma, cen = GAMMA[model], 0.02
+    params = fused.score_params(gamma, cen)
+    t_table, t_q1, t_q2 = dev(table), dev(q1), dev(q2)
+    ids, sources, o_rows, at = [], [], [], 0
+    for b, k in shapes:
+        idx = rng.integers(0, n, (b, k))
+        idx[0, 0] = 5                                   # an entity present in every stream
+        gs = rng.standard_normal((b, k)).astype(np.float32).astype(np.float64)
+        t_idx = torch.tensor(idx, device="cuda")
+        s_q1 = t_q1[at:at + b]
+        s_q2 = None if t_q2 is None else t_q2[at:at + b]
+        codes = fused.new_codes(model, t_table, t_idx, s_q1)
+        score = fused.score_forward(model, t_table, t_idx, s_q1, s_q2, params, codes=codes)
+        sources.append((score, dev(gs), codes, None, at, b))
+        ids.append(idx)
+        rows = orc.gather(table, idx).reshape(b, k, -1)
+        g_rows, _, _ = orc.score_backward(model, gs, rows, q1[at:at + b, None, :],
+                                          None if q2 is None else q2[at:at + b, None, :], cen)
+        o_rows.append(g_rows.reshape(b * k, -1))
+        at += b
+    flat = np.concatenate([i.reshape(-1) for i in ids])
+    plan = fused.build_plan(torch.tensor(flat, device="cuda"), n, want_inverse=True)
+    uniq, inverse, _, _ = orc.merge_indices(flat)
+    o_merged = orc.merge_grads(np.concatenate(o_rows), inverse, uniq.size)
+    o_abs = orc.merge_grads(np.abs(np.concatenate(o_rows)), inverse, uniq.size)
+    merged = torch.full((uniq.size, table.shape[1]), float("nan"), device="cuda")
+    fused.score_backward_entity_multi(model, plan, t_table, t_q1, t_q2, sources, params, merged=merged)
+    assert_close(merged.cpu().numpy(), o_merged, REL_F32, f"{model} merged over three query batches", sum_abs=o_abs)
+    t_m, t_v = torch.zeros_like(t_table), torch.zeros_like(t_table)
+    w_s, m_s, v_s = table.copy(), np.zeros_like(table), np.zeros_like(table)
+    orc.adam_rows(w_s, m_s, v_s, uniq, merged.cpu().numpy().astype(np.float64), lr, 1)
+    fused.score_backward_entity_multi(model, plan, t_table, t_q1, t_q2, sources, params, m=t_m, v=t_v,
+                                      adam=fused.adam_params(lr, 1))
+    touched = np.zeros(n, bool)
+    touched[uniq] = True
+    assert_close(t_table.cpu().numpy()[touched], w_s[touched], REL_F32, f"{model} w over three query batches")
+    assert_close(t_m.cpu().numpy()[touched], m_s[touched], REL_F32, f"{model} m over three query batches")
+    assert np.array_equal(t_table.cpu().numpy()[~touched], table[~touched].astype(np.float32))
+    # a stretch of queries that does not exist is refused
+    bad = list(sources)
+    bad[2] = sources[2][:4] + (b_all - 3, 8)
+    with pytest.raises(Exception):
+        fused.score_backward_entity_multi(model, plan, t_table, t_q1, t_q2, bad, params, merged=merged)
+
+
 def test_several_index_streams_at_a_size_that_forks():
     """Two streams (K = 1 and 300) of 4096 box queries, Adam: more than a million pairs and queries beyond one L2,
     so ids that occur once go through the pair-ordered kernel (one launch per stream) beside the entity pass.
@@ -905,18 +962,24 @@ def test_several_index_streams_at_a_size_that_forks():
     gn = torch.randn((b, 300), device="cuda", generator=g)
     params = fused.score_params(24.0, 0.02)
 
-    def run(streams):
+    def run(streams, batches=False):
         w, m, v = table.clone(), torch.zeros_like(table), torch.zeros_like(table)
         sources = []
-        for ids, gs in streams:
+        for i, (ids, gs) in enumerate(streams):
             codes = fused.new_codes("box", w, ids, q1)
             assert codes is not None
-            sources.append((fused.score_forward("box", w, ids, q1, q2, params, codes=codes), gs.contiguous(), codes))
+            src = (fused.score_forward("box", w, ids, q1, q2, params, codes=codes), gs.contiguous(), codes)
+            # batches: every stream has a query batch of its own (here: copies), the later stream's rows first
+            sources.append(src + (None, (len(streams) - 1 - i) * b, b) if batches else src)
         plan = fused.build_plan(torch.cat([ids.reshape(-1) for ids, _ in streams]), n)
-        fused.score_backward_entity_multi("box", plan, w, q1, q2, sources, params, m=m, v=v, adam=fused.adam_params(lr, 1))
+        reps = len(streams) if batches else 1
+        fused.score_backward_entity_multi("box", plan, w, q1.repeat(reps, 1), q2.repeat(reps, 1), sources, params, m=m,
+                                          v=v, adam=fused.adam_params(lr, 1))
         return w, m, v, plan
 
     w2, m2, v2, plan2 = run([(pos, gp), (neg, gn)])
+    w3, m3, v3, _ = run([(pos, gp), (neg, gn)], batches=True)
+    assert torch.equal(w3, w2) and torch.equal(m3, m2) and torch.equal(v3, v2), "a query batch per stream: the same bits"
     w1, m1, v1, plan1 = run([(torch.cat([pos, neg], dim=1), torch.cat([gp, gn], dim=1))])
     assert plan1.n_uniq == plan2.n_uniq and torch.equal(plan1.uniq, plan2.uniq)
     assert (plan2.pair_seg < 0).sum().item() > 30_000, "the case must have one-pair ids"
