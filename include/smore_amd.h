@@ -458,6 +458,26 @@ int smx_rank_candidates(int model, void* stream, const float* table, size_t n_ro
                         const int64_t* cand, size_t C, const int32_t* n_hard, size_t H, float* logit,
                         int64_t* ranking, int64_t* hard_rank, int* err_flag);
 
+/* The three evaluation calls for union queries: q1, q2 are [B, U, dim] (the U branch rows of a query adjacent, as
+ * for smx_score_forward_union), and an entity's logit is the maximum over the branches -- the last line of every
+ * custom_cal_logit (smore/models/box.py:163, vec.py:89, rotate.py:141, beta.py:307), which the evaluation loop
+ * reaches through the same model call as training (train_process.py:112-123).  Everything else as above; the
+ * ranks are those of the maximum logits, not the best of the branches' ranks.  U <= 4 (the scan keeps a query's
+ * branch rows in registers: rows of more than 512 floats -- 256 for the two-halves models -- allow U <= 2).
+ * U == 1 is the plain call. */
+int smx_rank_answer_keys_union(int model, void* stream, const float* table, size_t n_rows, const float* q1,
+                               const float* q2, size_t B, size_t U, size_t dim, const smx_score_params* params,
+                               const int64_t* ans_id, const int32_t* ans_count, size_t A, float* ans_score,
+                               uint64_t* ans_key);
+int smx_rank_scan_union(int model, void* stream, const float* table, size_t n_rows, const float* q1,
+                        const float* q2, size_t B, size_t U, size_t dim, const smx_score_params* params,
+                        const int64_t* ans_id, const uint64_t* ans_key, const int32_t* ans_count, size_t A,
+                        int64_t* filtered_rank, void* workspace, size_t workspace_bytes);
+int smx_rank_candidates_union(int model, void* stream, const float* table, size_t n_rows, const float* q1,
+                              const float* q2, size_t B, size_t U, size_t dim, const smx_score_params* params,
+                              const int64_t* cand, size_t C, const int32_t* n_hard, size_t H, float* logit,
+                              int64_t* ranking, int64_t* hard_rank, int* err_flag);
+
 /* Plain row lookup out[k,:] = table[idx[k],:] (smore/common/embedding/embed_rw.py:74-75, the GPU
  * branch of EmbeddingReadOnly.read) for callers that need the rows themselves. */
 int smx_gather_rows(void* stream, const float* table, size_t n_rows, size_t row_len,

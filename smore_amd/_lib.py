@@ -81,6 +81,11 @@ SIGNATURES = {
     "smx_rank_scan": (_i, [_i, _vp, _vp, _sz, _vp, _vp, _sz, _sz, _vp, _vp, _vp, _vp, _sz, _vp, _vp, _sz]),
     # model, stream, table, n_rows, q1, q2, B, dim, params, cand, C, n_hard, H, logit, ranking, hard_rank, err
     "smx_rank_candidates": (_i, [_i, _vp, _vp, _sz, _vp, _vp, _sz, _sz, _vp, _vp, _sz, _vp, _sz, _vp, _vp, _vp, _vp]),
+    # the same three with U (branch rows per query) behind B
+    "smx_rank_answer_keys_union": (_i, [_i, _vp, _vp, _sz, _vp, _vp, _sz, _sz, _sz, _vp, _vp, _vp, _sz, _vp, _vp]),
+    "smx_rank_scan_union": (_i, [_i, _vp, _vp, _sz, _vp, _vp, _sz, _sz, _sz, _vp, _vp, _vp, _vp, _sz, _vp, _vp, _sz]),
+    "smx_rank_candidates_union": (_i, [_i, _vp, _vp, _sz, _vp, _vp, _sz, _sz, _sz, _vp, _vp, _sz, _vp, _sz, _vp, _vp, _vp,
+                                       _vp]),
     "smx_sample_loss_workspace_bytes": (_sz, [_sz]),
     # stream, pos, neg, mask, weight, B, K, temperature, scale, out_loss, gpos, gneg, ws, ws_bytes
     "smx_sample_loss": (_i, [_vp, _vp, _vp, _vp, _vp, _sz, _sz, ctypes.c_double, ctypes.c_double, _vp, _vp, _vp, _vp, _sz]),

@@ -17,12 +17,14 @@ constexpr size_t kRankMaxAnswers = 2048;  // per query; bins and keys of a pass 
 static size_t rank_ws_bytes(size_t B, size_t A) { return (B * (A + 1) * sizeof(unsigned) + 255) & ~(size_t)255; }
 
 static int rank_common(RankArgs* R, int* vec, int* nit, int model, const float* table, size_t n_rows, const float* q1,
-                       const float* q2, size_t B, size_t dim, const smx_score_params* params, const int64_t* ans_id,
-                       const int32_t* ans_count, size_t A) {
+                       const float* q2, size_t B, size_t U, size_t dim, const smx_score_params* params,
+                       const int64_t* ans_id, const int32_t* ans_count, size_t A) {
   if (model < 0 || model >= mNumModels) return fail(SMX_ERR_KIND, "unknown score model %d", model);
   if (!table || !q1 || !params || !ans_id || !ans_count || (model_nq(model) == 2 && !q2))
     return fail(SMX_ERR_ARG, "null pointer");
   if (B == 0 || dim == 0 || n_rows == 0 || A == 0) return fail(SMX_ERR_SHAPE, "empty dimension");
+  if (U == 0 || U > (size_t)kRankQueries) return fail(SMX_ERR_SHAPE, "1 to %d union branches", kRankQueries);
+  if (B * U > 0x7fffffffull) return fail(SMX_ERR_SHAPE, "too many query rows");
   if (n_rows > 0xfffffff8ull) return fail(SMX_ERR_SHAPE, "entity count %zu needs ids wider than 32 bits", n_rows);
   if (A > kRankMaxAnswers) return fail(SMX_ERR_SHAPE, "at most %zu answers per query", kRankMaxAnswers);
   if (B > 0x7fffffffull / (A + 1)) return fail(SMX_ERR_SHAPE, "too many queries");
@@ -40,6 +42,7 @@ static int rank_common(RankArgs* R, int* vec, int* nit, int model, const float* 
   R->q1 = q1;
   R->q2 = q2;
   R->B = (int)B;
+  R->U = (int)U;
   R->ncol = (int)ncol;
   R->n_rows = n_rows;
   R->p = ScoreParams{params->gamma, params->cen, params->reg_on, params->reg_add, params->reg_lo, params->reg_hi};
@@ -68,26 +71,35 @@ extern "C" {
 
 size_t smx_rank_workspace_bytes(size_t B, size_t A) { return smx::rank_ws_bytes(B, A); }
 
-int smx_rank_answer_keys(int model, void* stream, const float* table, size_t n_rows, const float* q1, const float* q2,
-                         size_t B, size_t dim, const smx_score_params* params, const int64_t* ans_id,
-                         const int32_t* ans_count, size_t A, float* ans_score, uint64_t* ans_key) {
+int smx_rank_answer_keys_union(int model, void* stream, const float* table, size_t n_rows, const float* q1,
+                               const float* q2, size_t B, size_t U, size_t dim, const smx_score_params* params,
+                               const int64_t* ans_id, const int32_t* ans_count, size_t A, float* ans_score,
+                               uint64_t* ans_key) {
   using namespace smx;
   RankArgs R;
   int vec, nit;
-  if (int rc = rank_common(&R, &vec, &nit, model, table, n_rows, q1, q2, B, dim, params, ans_id, ans_count, A)) return rc;
+  if (int rc = rank_common(&R, &vec, &nit, model, table, n_rows, q1, q2, B, U, dim, params, ans_id, ans_count, A)) return rc;
   if (!ans_score || !ans_key) return fail(SMX_ERR_ARG, "null output pointer");
   R.score_out = ans_score;
   R.key_out = reinterpret_cast<unsigned long long*>(ans_key);
   return rank_run(model, as_stream(stream), R, vec, nit, kRankKeys);
 }
 
-int smx_rank_scan(int model, void* stream, const float* table, size_t n_rows, const float* q1, const float* q2, size_t B,
-                  size_t dim, const smx_score_params* params, const int64_t* ans_id, const uint64_t* ans_key,
-                  const int32_t* ans_count, size_t A, int64_t* filtered_rank, void* workspace, size_t workspace_bytes) {
+int smx_rank_answer_keys(int model, void* stream, const float* table, size_t n_rows, const float* q1, const float* q2,
+                         size_t B, size_t dim, const smx_score_params* params, const int64_t* ans_id,
+                         const int32_t* ans_count, size_t A, float* ans_score, uint64_t* ans_key) {
+  return smx_rank_answer_keys_union(model, stream, table, n_rows, q1, q2, B, 1, dim, params, ans_id, ans_count, A,
+                                    ans_score, ans_key);
+}
+
+int smx_rank_scan_union(int model, void* stream, const float* table, size_t n_rows, const float* q1, const float* q2,
+                        size_t B, size_t U, size_t dim, const smx_score_params* params, const int64_t* ans_id,
+                        const uint64_t* ans_key, const int32_t* ans_count, size_t A, int64_t* filtered_rank,
+                        void* workspace, size_t workspace_bytes) {
   using namespace smx;
   RankArgs R;
   int vec, nit;
-  if (int rc = rank_common(&R, &vec, &nit, model, table, n_rows, q1, q2, B, dim, params, ans_id, ans_count, A)) return rc;
+  if (int rc = rank_common(&R, &vec, &nit, model, table, n_rows, q1, q2, B, U, dim, params, ans_id, ans_count, A)) return rc;
   if (!ans_key || !filtered_rank || !workspace) return fail(SMX_ERR_ARG, "null pointer");
   if (workspace_bytes < rank_ws_bytes(B, A))
     return fail(SMX_ERR_WORKSPACE, "rank workspace too small: %zu < %zu", workspace_bytes, rank_ws_bytes(B, A));
@@ -97,10 +109,17 @@ int smx_rank_scan(int model, void* stream, const float* table, size_t n_rows, co
   return rank_run(model, as_stream(stream), R, vec, nit, kRankScan);
 }
 
-int smx_rank_candidates(int model, void* stream, const float* table, size_t n_rows, const float* q1, const float* q2,
-                        size_t B, size_t dim, const smx_score_params* params, const int64_t* cand, size_t C,
-                        const int32_t* n_hard, size_t H, float* logit, int64_t* ranking, int64_t* hard_rank,
-                        int* err_flag) {
+int smx_rank_scan(int model, void* stream, const float* table, size_t n_rows, const float* q1, const float* q2, size_t B,
+                  size_t dim, const smx_score_params* params, const int64_t* ans_id, const uint64_t* ans_key,
+                  const int32_t* ans_count, size_t A, int64_t* filtered_rank, void* workspace, size_t workspace_bytes) {
+  return smx_rank_scan_union(model, stream, table, n_rows, q1, q2, B, 1, dim, params, ans_id, ans_key, ans_count, A,
+                             filtered_rank, workspace, workspace_bytes);
+}
+
+int smx_rank_candidates_union(int model, void* stream, const float* table, size_t n_rows, const float* q1,
+                              const float* q2, size_t B, size_t U, size_t dim, const smx_score_params* params,
+                              const int64_t* cand, size_t C, const int32_t* n_hard, size_t H, float* logit,
+                              int64_t* ranking, int64_t* hard_rank, int* err_flag) {
   using namespace smx;
   RankArgs R;
   int vec, nit;
@@ -108,7 +127,7 @@ int smx_rank_candidates(int model, void* stream, const float* table, size_t n_ro
   if (C == 0 || C > kRankMaxCandidates) return fail(SMX_ERR_SHAPE, "1 to %zu candidates per query", kRankMaxCandidates);
   if (H == 0 || H > C) return fail(SMX_ERR_SHAPE, "between 1 and C hard-answer slots");
   // (the shape checks shared with the all-entity scan; its answer arguments are not used here)
-  if (int rc = rank_common(&R, &vec, &nit, model, table, n_rows, q1, q2, B, dim, params, cand, n_hard, 1)) return rc;
+  if (int rc = rank_common(&R, &vec, &nit, model, table, n_rows, q1, q2, B, U, dim, params, cand, n_hard, 1)) return rc;
   if (B * C > 0x7fffffffull) return fail(SMX_ERR_SHAPE, "too many candidates in one call");
   R.ans_id = nullptr;
   R.ans_count = nullptr;
@@ -121,6 +140,14 @@ int smx_rank_candidates(int model, void* stream, const float* table, size_t n_ro
   R.hard_rank = reinterpret_cast<long long*>(hard_rank);
   R.err = err_flag;
   return rank_run(model, as_stream(stream), R, vec, nit, kRankCandidates);
+}
+
+int smx_rank_candidates(int model, void* stream, const float* table, size_t n_rows, const float* q1, const float* q2,
+                        size_t B, size_t dim, const smx_score_params* params, const int64_t* cand, size_t C,
+                        const int32_t* n_hard, size_t H, float* logit, int64_t* ranking, int64_t* hard_rank,
+                        int* err_flag) {
+  return smx_rank_candidates_union(model, stream, table, n_rows, q1, q2, B, 1, dim, params, cand, C, n_hard, H, logit,
+                                   ranking, hard_rank, err_flag);
 }
 
 }  // extern "C"

@@ -25,6 +25,8 @@ struct RankArgs {
   const float* q1;
   const float* q2;
   int b0, B;            // queries [b0, b0 + NB) of B are handled by this launch (NB: see rank_scan_kernel)
+  int U;                // union queries: q1 / q2 hold U branch rows per query, a logit is the maximum over them
+                        // (the last line of every custom_cal_logit, smore/models/box.py:163); 1 otherwise
   int ncol;
   unsigned long long n_rows;
   ScoreParams p;
@@ -56,6 +58,9 @@ __device__ __forceinline__ unsigned sortable_bits(float s) {
 __device__ __forceinline__ unsigned long long rank_key(float score, unsigned long long id) {
   return ((unsigned long long)sortable_bits(score) << 32) | (unsigned)(~(unsigned)id);
 }
+
+// Whether branch logit s replaces the best so far: torch.max over the branch axis (a NaN wins, the first of equals stays).
+__device__ __forceinline__ bool union_takes(float s, float best) { return s > best || (s != s && best == best); }
 
 // Score of one row against one staged query; the value is valid in lane 63.
 template <int M, int VEC, int NIT, bool REG>
@@ -132,19 +137,26 @@ __global__ __launch_bounds__(256) void rank_answer_keys_kernel(RankArgs A) {
   unsigned long long id = valid ? (unsigned long long)A.ans_id[slot] : 0ull;
   if (id >= A.n_rows) id = 0;  // the host wrapper has already refused such ids
   typename ModelOps<M>::Q q[NIT][VEC];
-  load_rank_query<M, VEC, NIT>(A.q1, A.q2, b, dim, A.ncol, lane, q);
   float e1[NIT][VEC], e2[NIT][VEC];
   load_entity<VEC, NIT, MUL>(A.table + id * (size_t)dim * MUL, dim, A.ncol, lane, e1, e2);
-  const float s = row_score<M, VEC, NIT, REG>(e1, e2, q, A.ncol, lane, A.p);
+  float s = 0.f;
+  for (int u = 0; u < A.U; ++u) {  // uniform
+    load_rank_query<M, VEC, NIT>(A.q1, A.q2, b * A.U + u, dim, A.ncol, lane, q);
+    const float su = row_score<M, VEC, NIT, REG>(e1, e2, q, A.ncol, lane, A.p);
+    if (u == 0 || union_takes(su, s)) s = su;
+  }
   if (lane == 63) {
     A.score_out[slot] = valid ? s : 0.f;
     A.key_out[slot] = valid ? rank_key(s, id) : 0ull;  // key 0 sorts last and is never counted
   }
 }
 
-// The scan for NB (1, 2 or 4) queries.  LDS: bins [NB][A + 1], keys [NB][A].
-template <int M, int VEC, int NIT, bool REG, int NB>
+// The scan for NB (1, 2 or 4) queries -- or, UNION, for ONE query whose NB register sets hold its branch rows (a
+// set past the last branch repeats it): an entity's logit is then the maximum over the sets, and there is one list
+// of answers.  LDS: bins [NL][A + 1], keys [NL][A] with NL = the number of answer lists (NB, or 1).
+template <int M, int VEC, int NIT, bool REG, int NB, bool UNION = false>
 __global__ __launch_bounds__(256) void rank_scan_kernel(RankArgs A) {
+  constexpr int NL = UNION ? 1 : NB;
   constexpr int MUL = model_mul(M);
   constexpr int RIF = NIT * MUL <= 2 ? 4 : (NIT * MUL <= 4 ? 2 : 1);
   extern __shared__ unsigned lds_bins[];  // bins [NB][A + 1], then (8-byte aligned) the answers' keys [NB][A]
@@ -153,9 +165,9 @@ __global__ __launch_bounds__(256) void rank_scan_kernel(RankArgs A) {
   const int dim = A.ncol * VEC;
   const size_t row_len = (size_t)dim * MUL;
   const int A1 = A.A + 1;
-  unsigned long long* lds_keys = reinterpret_cast<unsigned long long*>(lds_bins + ((NB * A1 + 1) & ~1));
-  for (int i = threadIdx.x; i < NB * A1; i += 256) lds_bins[i] = 0u;
-  for (int i = threadIdx.x; i < NB * A.A; i += 256) {
+  unsigned long long* lds_keys = reinterpret_cast<unsigned long long*>(lds_bins + ((NL * A1 + 1) & ~1));
+  for (int i = threadIdx.x; i < NL * A1; i += 256) lds_bins[i] = 0u;
+  for (int i = threadIdx.x; i < NL * A.A; i += 256) {
     const int x = i / A.A, j = i - x * A.A;
     const int b = min(A.b0 + x, A.B - 1);
     lds_keys[i] = j < A.ans_count[b] ? A.ans_key[(size_t)b * A.A + j] : 0ull;
@@ -163,23 +175,25 @@ __global__ __launch_bounds__(256) void rank_scan_kernel(RankArgs A) {
   __syncthreads();
 
   typename ModelOps<M>::Q q[NB][NIT][VEC];
-  int count[NB], qb[NB];
+  int count[NL], qb[NL];
 #pragma unroll
-  for (int x = 0; x < NB; ++x) {
+  for (int x = 0; x < NL; ++x) {
     qb[x] = min(A.b0 + x, A.B - 1);  // a pass past the last query repeats it; its histogram is dropped
     count[x] = min(max(A.ans_count[qb[x]], 0), A.A);  // a count beyond the slots would index past the LDS arrays
-    load_rank_query<M, VEC, NIT>(A.q1, A.q2, qb[x], dim, A.ncol, lane, q[x]);
   }
+#pragma unroll
+  for (int x = 0; x < NB; ++x)
+    load_rank_query<M, VEC, NIT>(A.q1, A.q2, UNION ? qb[0] * A.U + min(x, A.U - 1) : qb[x], dim, A.ncol, lane, q[x]);
   const int chunks = (A.A + 63) / 64;
   // The first 64 answers' keys stay in registers (most queries have no more); further chunks come from LDS.
   // live[x]: lanes that hold one of them.  my_id[x]: that answer's entity id.
-  unsigned long long first_keys[NB], live[NB];
-  unsigned my_id[NB];
+  unsigned long long first_keys[NL], live[NL];
+  unsigned my_id[NL];
   // tally[x], lane L: rows so far that beat exactly L of query x's answers (the common cases: L = 0 is
   // every entity ranked below all answers).  Rows that beat 64 or more go to the LDS histogram directly.
-  unsigned tally[NB];
+  unsigned tally[NL];
 #pragma unroll
-  for (int x = 0; x < NB; ++x) {
+  for (int x = 0; x < NL; ++x) {
     first_keys[x] = lane < count[x] ? lds_keys[x * A.A + lane] : 0ull;
     live[x] = count[x] >= 64 ? ~0ull : ((1ull << count[x]) - 1ull);
     my_id[x] = (unsigned)~(unsigned)first_keys[x];
@@ -209,9 +223,17 @@ __global__ __launch_bounds__(256) void rank_scan_kernel(RankArgs A) {
     for (int r = 0; r < RIF; ++r) {
       const unsigned id = g * RIF + r;  // entity id of the row
 #pragma unroll
-      for (int x = 0; x < NB; ++x) {
+      for (int x = 0; x < NL; ++x) {
         const float s = row_score<M, VEC, NIT, REG>(x1[r], x2[r], q[x], A.ncol, lane, A.p);
-        const float su = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(s), 63));
+        float su = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(s), 63));
+        if constexpr (UNION) {
+#pragma unroll
+          for (int u = 1; u < NB; ++u) {
+            const float t = row_score<M, VEC, NIT, REG>(x1[r], x2[r], q[u], A.ncol, lane, A.p);
+            const float tu = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(t), 63));
+            if (union_takes(tu, su)) su = tu;
+          }
+        }
         const unsigned long long key = rank_key(su, id);
         int not_beaten = __popcll(__ballot(!(key > first_keys[x])) & live[x]);
         bool skip = id >= n_rows32 || (__ballot(my_id[x] == id) & live[x]) != 0ull;  // past the end, or an answer
@@ -243,11 +265,11 @@ __global__ __launch_bounds__(256) void rank_scan_kernel(RankArgs A) {
     }
   }
 #pragma unroll
-  for (int x = 0; x < NB; ++x)
+  for (int x = 0; x < NL; ++x)
     if (lane <= count[x] && tally[x] != 0u) atomicAdd(&lds_bins[x * A1 + (count[x] - lane)], tally[x]);
   __syncthreads();
 #pragma unroll
-  for (int x = 0; x < NB; ++x) {
+  for (int x = 0; x < NL; ++x) {
     if (A.b0 + x < A.B) {
       for (int i = threadIdx.x; i < A1; i += 256) {
         const unsigned v = lds_bins[x * A1 + i];
@@ -277,7 +299,7 @@ __global__ __launch_bounds__(kCandThreads) void rank_candidates_kernel(RankArgs 
   const int wave = threadIdx.x >> 6;
   const int dim = A.ncol * VEC;
   typename ModelOps<M>::Q q[NIT][VEC];
-  load_rank_query<M, VEC, NIT>(A.q1, A.q2, b, dim, A.ncol, lane, q);
+  load_rank_query<M, VEC, NIT>(A.q1, A.q2, b * A.U, dim, A.ncol, lane, q);  // (the first branch, or the only one)
   int bad = 0;
   for (int j = wave; j < A.C; j += kCandThreads / 64) {  // uniform per wavefront
     const long long raw = A.cand[(size_t)b * A.C + j];
@@ -289,7 +311,14 @@ __global__ __launch_bounds__(kCandThreads) void rank_candidates_kernel(RankArgs 
     }
     float e1[NIT][VEC], e2[NIT][VEC];
     load_entity<VEC, NIT, MUL>(A.table + id * (size_t)dim * MUL, dim, A.ncol, lane, e1, e2);
-    const float s = row_score<M, VEC, NIT, REG>(e1, e2, q, A.ncol, lane, A.p) + (pad ? -1e6f : 0.f);
+    float s = row_score<M, VEC, NIT, REG>(e1, e2, q, A.ncol, lane, A.p);
+    for (int u = 1; u < A.U; ++u) {  // uniform: the other branches of a union query, fetched again per candidate
+      typename ModelOps<M>::Q qu[NIT][VEC];
+      load_rank_query<M, VEC, NIT>(A.q1, A.q2, b * A.U + u, dim, A.ncol, lane, qu);
+      const float su = row_score<M, VEC, NIT, REG>(e1, e2, qu, A.ncol, lane, A.p);
+      if (union_takes(su, s)) s = su;
+    }
+    s += pad ? -1e6f : 0.f;
     if (lane == 63) {
       if (A.cand_logit) A.cand_logit[(size_t)b * A.C + j] = s;
       cand_keys[j] = ((unsigned long long)sortable_bits(s) << 32) | (unsigned)(~(unsigned)j);
@@ -368,6 +397,23 @@ int launch_rank_reg(hipStream_t st, RankArgs A, int mode) {
   // to issue-bound between one and two.  Four when the rows are short enough for four queries' registers
   // and the answers' keys and histograms of four queries fit 48 KB of LDS.
   constexpr bool kFourFit = NIT * model_mul(M) <= 2;
+  if (A.U > 1) {  // union queries: one query per pass, its branch rows in the register sets
+    if (A.U > 2 && !kFourFit)
+      return fail(SMX_ERR_SHAPE, "union queries of %d branches over rows this long are not supported by the scan (2 at most)", A.U);
+    for (int b0 = 0; b0 < A.B; ++b0) {
+      A.b0 = b0;
+      const size_t lds = lds_bytes(1);
+      if (A.U == 2) {
+        hipLaunchKernelGGL((rank_scan_kernel<M, VEC, NIT, REG, 2, true>),
+                           dim3(grid_for(rank_scan_kernel<M, VEC, NIT, REG, 2, true>, lds)), dim3(256), lds, st, A);
+      } else if constexpr (kFourFit) {
+        hipLaunchKernelGGL((rank_scan_kernel<M, VEC, NIT, REG, 4, true>),
+                           dim3(grid_for(rank_scan_kernel<M, VEC, NIT, REG, 4, true>, lds)), dim3(256), lds, st, A);
+      }
+    }
+    hipLaunchKernelGGL(rank_finish_kernel, dim3((unsigned)A.B), dim3(256), 0, st, A);
+    return check_launch("rank scan (union queries)");
+  }
   for (int b0 = 0; b0 < A.B;) {
     A.b0 = b0;
     const int left = A.B - b0;

@@ -167,3 +167,116 @@ def test_sampled_candidates_follow_the_reference_recipe(model, dim):
     bad[3, 5] = n + 4
     candidate_ranks(model, dev(table), dev(q1), dev(q2), params, bad, n_hard, err)
     assert err.item() == 1
+
+
+def _union_scores64(model, table, q1, q2, cen, u):
+    """float64 logits of union queries: q1 / q2 [B, U, dim], the maximum over the branches (box.py:163), [B, N]"""
+    b = q1.shape[0]
+    per = [_scores64(model, table, q1[:, j], None if q2 is None else q2[:, j], cen) for j in range(u)]
+    return np.max(np.stack(per, axis=1), axis=1).reshape(b, -1)
+
+
+@pytest.mark.parametrize("u", [2, 3, 4])
+def test_union_queries_rank_exactly_by_the_maximum_over_branches(u):
+    """Integer coordinates (every fp32 sum exact, many ties): the filtered ranks of a union query are those of
+    max_u logit_u in the stable descending order -- not the best of the branches' own ranks."""
+    from smore_amd import fused
+    from smore_amd.evaluation import filtered_ranks
+    rng = np.random.default_rng(u)
+    n, d, b = 4000, 16, 5
+    table = rng.integers(-3, 4, (n, d)).astype(np.float64)
+    q1 = rng.integers(-3, 4, (b, u, d)).astype(np.float64)
+    q1[1, 1] = q1[1, 0]                                   # two equal branches
+    easy = [[3, 77, 3000], [], [11], [5], [1, 2]]
+    hard = [[9, 2500, 3999, 0], [123], list(range(100, 180)), list(range(200, 270)), [42]]
+    params = fused.score_params(GAMMA["l1"], 0.0)
+    got = filtered_ranks("l1", dev(table), dev(q1), None, params, easy, hard, branches=u)
+    scores = _union_scores64("l1", table, q1, None, 0.0, u)
+    differs = 0
+    for i in range(b):
+        want_h, want_e = orc.filtered_ranks(scores[i], easy[i], hard[i])
+        assert got[i][0].cpu().numpy().tolist() == want_h.tolist()
+        assert got[i][1].cpu().numpy().tolist() == want_e.tolist()
+        best_branch = np.min([orc.filtered_ranks(_scores64("l1", table, q1[i:i + 1, j], None, 0.0)[0], easy[i], hard[i])[0]
+                              for j in range(u)], axis=0)
+        differs += int((best_branch != want_h).any())
+    assert differs > 0, "the case must tell the rank of the maximum from the best rank of a branch"
+
+
+@pytest.mark.parametrize("model,dim,u", [("box", 200, 2), ("rotate", 100, 2), ("beta_kl", 40, 2), ("l2", 64, 3), ("distmult", 64, 4),
+                                         ("box", 400, 2), ("l1", 30, 3)])
+def test_union_ranks_lie_in_the_interval_fp32_allows(model, dim, u):
+    """Random floats, union queries: every rank between the counts with the fp32 tolerance subtracted and added;
+    the answers' logits against the float64 maximum over the branches."""
+    from smore_amd import fused
+    from smore_amd.evaluation import filtered_ranks
+    rng = np.random.default_rng(dim + u)
+    n, b = 6000, 3
+    table, q1, q2, _, _ = make_problem(model, n, b * u, 1, dim, rng)
+    q1 = q1.reshape(b, u, dim)
+    q2 = None if q2 is None else q2.reshape(b, u, dim)
+    easy = [rng.choice(n, size=s, replace=False).tolist() for s in (0, 3, 10)]
+    hard = []
+    for e, s in zip(easy, (1, 5, 70)):
+        pool = np.setdiff1d(np.arange(n), np.array(e, dtype=np.int64))
+        hard.append(rng.choice(pool, size=s, replace=False).tolist())
+    params = fused.score_params(GAMMA[model], 0.02)
+    got = filtered_ranks(model, dev(table), dev(q1), dev(q2), params, easy, hard, branches=u)
+    scores = _union_scores64(model, table, q1, q2, 0.02, u)
+    for i in range(b):
+        is_ans = np.zeros(n, bool)
+        is_ans[easy[i] + hard[i]] = True
+        tol = 2e-5 * max(1.0, np.abs(scores[i]).max())
+        others = np.sort(scores[i][~is_ans])
+        for ids, ranks in ((hard[i], got[i][0]), (easy[i], got[i][1])):
+            for a, ra in zip(ids, ranks.cpu().numpy()):
+                lo = 1 + (others.size - np.searchsorted(others, scores[i][a] + tol, side="right"))
+                hi = 1 + (others.size - np.searchsorted(others, scores[i][a] - tol, side="left"))
+                assert lo <= ra <= hi, (model, i, a, ra, lo, hi)
+
+
+def test_union_of_many_branches_over_long_rows_is_refused():
+    from smore_amd import _lib, fused
+    from smore_amd.evaluation import filtered_ranks
+    rng = np.random.default_rng(1)
+    table, q1, q2, _, _ = make_problem("rotate", 50, 3, 1, 400, rng)       # rows of 800 floats: two branches at most
+    params = fused.score_params(GAMMA["rotate"], 0.02)
+    with pytest.raises(_lib.SmxError):
+        filtered_ranks("rotate", dev(table), dev(q1.reshape(1, 3, 400)), dev(q2.reshape(1, 3, 400)), params, [[1]], [[2]],
+                       branches=3)
+    five = dev(rng.uniform(-0.07, 0.07, (1, 5, 400)))                       # more branches than the scan has register sets
+    with pytest.raises(_lib.SmxError):
+        filtered_ranks("l1", dev(table[:, :400]), five, None, fused.score_params(GAMMA["l1"], 0.0), [[1]], [[2]], branches=5)
+
+
+@pytest.mark.parametrize("model,dim,u", [("box", 64, 2), ("rotate", 40, 3), ("l2", 200, 2)])
+def test_sampled_candidates_of_union_queries(model, dim, u):
+    """smx_rank_candidates_union: the candidates' logits are the maximum over the branches (then the -1e6 bias on the
+    padding); ranking and filtered ranks are the oracle's recipe on the device's own logits."""
+    from smore_amd import fused
+    from smore_amd.evaluation import candidate_ranks
+    rng = np.random.default_rng(dim * u)
+    n, b, c = 400, 4, 150
+    table, q1, q2, _, _ = make_problem(model, n, b * u, 1, dim, rng)
+    q1 = q1.reshape(b, u, dim)
+    q2 = None if q2 is None else q2.reshape(b, u, dim)
+    neg = rng.integers(0, n, (b, c)).astype(np.int64)
+    neg[0, 100:] = -1
+    neg[1, 0] = -1
+    n_hard = np.array([4, 1, 9, 0], dtype=np.int32)
+    params = fused.score_params(GAMMA[model], 0.02)
+    err = fused.new_error_flag("cuda")
+    logit, ranking, hard = candidate_ranks(model, dev(table), dev(q1), dev(q2), params, torch.tensor(neg, device="cuda"),
+                                           n_hard, err, branches=u)
+    assert err.item() == 0
+    rows = table[np.where(neg == -1, 0, neg)]
+    per = [orc.score_forward(model, rows, q1[:, j, None], None if q2 is None else q2[:, j, None], GAMMA[model], 0.02)
+           for j in range(u)]
+    want = np.max(np.stack(per, axis=0), axis=0) + np.where(neg == -1, -1e6, 0.0)
+    assert_close(logit.cpu().numpy(), want, REL_F32, f"{model} union candidate logits")
+    got_logit = logit.cpu().numpy()
+    for i in range(b):
+        _, rk, filt = orc.candidate_ranks(np.where(neg[i] == -1, got_logit[i] + np.float32(1e6), got_logit[i]), neg[i],
+                                          int(n_hard[i]))
+        assert np.array_equal(ranking[i].cpu().numpy(), rk), f"{model} ranking of query {i}"
+        assert np.array_equal(hard[i, : filt.size].cpu().numpy(), filt) and not hard[i, filt.size:].any()
