@@ -462,7 +462,11 @@ __global__ __launch_bounds__(NW * 64) void score_backward_query_kernel(ScoreArgs
   constexpr int MUL = model_mul(M);
   constexpr int NQ = model_nq(M);
   extern __shared__ float lds[];
-  const int b = blockIdx.x;
+  // Queries are taken last to first: the forward walks them first to last, and what it touched last -- the sign
+  // codes it wrote, the rows it read -- is what the memory-side cache still holds when this kernel starts
+  // (86 M x 200 box workload: backward 0.92 -> 0.91 ms; the kernel by itself, with nothing of a forward left in
+  // that cache, takes 0.71 ms instead of 0.63).
+  const int b = (int)(gridDim.x - 1u - blockIdx.x);
   const int lane = threadIdx.x & 63;
   const int wave = uniform(threadIdx.x >> 6);
   const int dim = ncol * VEC;
