@@ -889,15 +889,14 @@ def test_entity_pass_over_several_index_streams(model):
 
 
 @pytest.mark.parametrize("model", ["box", "l1", "l2", "rotate", "beta_kl", "distmult"])
-def test_entity_pass_over_streams_of_different_query_batches(model):
+def test_entity_pass_over_streams_of_different_query_batches(model, shapes=((5, 7), (3, 20), (8, 1)), dim=24, n=120):
     """Records of several forward calls in one step (the reference merges them like any others,
     embed_optimizer.py:155-163): three streams of three query batches (B = 5, 3, 8; K = 7, 20, 1) whose query rows lie
     one after the other, each source naming its stretch; the second and third batch share entities with the first.
     Merged rows against the oracle's unique-merge + scatter-sum, then one Adam step."""
     from smore_amd import fused
-    n, dim, lr = 120, 24, 1e-3
-    shapes = ((5, 7), (3, 20), (8, 1))
-    rng = np.random.default_rng(seed("multi-batch", model))
+    lr = 1e-3
+    rng = np.random.default_rng(seed("multi-batch", model, dim, n, *[x for s in shapes for x in s]))
     b_all = sum(b for b, _ in shapes)
     table, q1, q2, _, _ = make_problem(model, n, b_all, 1, dim, rng)
     gamma, cen = GAMMA[model], 0.02
@@ -906,7 +905,7 @@ def test_entity_pass_over_streams_of_different_query_batches(model):
     ids, sources, o_rows, at = [], [], [], 0
     for b, k in shapes:
         idx = rng.integers(0, n, (b, k))
-        idx[0, 0] = 5                                   # an entity present in every stream
+        idx[0, 0] = min(5, n - 1)                       # an entity present in every stream
         gs = rng.standard_normal((b, k)).astype(np.float32).astype(np.float64)
         t_idx = torch.tensor(idx, device="cuda")
         s_q1 = t_q1[at:at + b]
@@ -940,7 +939,7 @@ def test_entity_pass_over_streams_of_different_query_batches(model):
     assert np.array_equal(t_table.cpu().numpy()[~touched], table[~touched].astype(np.float32))
     # a stretch of queries that does not exist is refused
     bad = list(sources)
-    bad[2] = sources[2][:4] + (b_all - 3, 8)
+    bad[-1] = sources[-1][:4] + (b_all - shapes[-1][0] + 1, shapes[-1][0])
     with pytest.raises(Exception):
         fused.score_backward_entity_multi(model, plan, t_table, t_q1, t_q2, bad, params, merged=merged)
 
