@@ -45,6 +45,7 @@ size_t code_bytes_per_pair(size_t dim);
 extern template int shared_forward_dispatch<mL1>(hipStream_t, const SharedFwdArgs&, int);
 extern template int shared_forward_dispatch<mL2>(hipStream_t, const SharedFwdArgs&, int);
 extern template int shared_forward_dispatch<mBox>(hipStream_t, const SharedFwdArgs&, int);
+extern template int shared_forward_dispatch<mRotate>(hipStream_t, const SharedFwdArgs&, int);
 
 // defined in smx_shared_gemm.hip: shared negatives of beta_kl, complex and distmult as matrix products
 size_t shared_gemm_workspace_floats(int model, size_t B, size_t K, size_t dim, bool entity);
@@ -265,6 +266,7 @@ int smx_score_forward_shared(int model, void* stream, const float* table, size_t
       case mL1: return shared_forward_dispatch<mL1>(st, S, nit);
       case mL2: return shared_forward_dispatch<mL2>(st, S, nit);
       case mBox: return shared_forward_dispatch<mBox>(st, S, nit);
+      case mRotate: return shared_forward_dispatch<mRotate>(st, S, nit);
     }
   }
   A.ids_shared = 1;

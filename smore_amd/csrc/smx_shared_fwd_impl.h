@@ -7,7 +7,7 @@
 // the next tile is requested into registers before the current tile is used.  Per pair the arithmetic is that
 // of score_forward_kernel (same accumulation per lane, same reduction), so scores are the same bits.
 //
-// For l1, l2 and box (the inner-product models and BetaE are matrix products for a shared list,
+// For l1, l2, box and rotate (the inner-product models and BetaE are matrix products for a shared list,
 // smx_shared_gemm.hip) and rows of 16-byte aligned float4 columns, up to 128 columns per half (two per lane);
 // other shapes use the id-driven kernels with the shared list.
 #pragma once
@@ -128,9 +128,8 @@ int shared_forward_dispatch(hipStream_t st, const SharedFwdArgs& A, int nit) {
 }
 
 // Whether a call has the shape these kernels are written for.
-// (rotate, whose pairs cost a square root per feature, gains nothing from the staging: measured 9 % slower.)
 inline bool shared_forward_fits(int model, int vec, int nit) {
-  return (model == mL1 || model == mL2 || model == mBox) && vec == 4 && nit <= 2;
+  return (model == mL1 || model == mL2 || model == mBox || model == mRotate) && vec == 4 && nit <= 2;
 }
 
 }  // namespace smx
