@@ -51,7 +51,8 @@ constexpr int shared_rows_ahead(int nit, int nq) { return nit * nq <= 2 ? 4 : (n
 
 // RW: rows per workgroup.  With two, every query row a wavefront fetches meets both of them: half the requests
 // to the L2 per pair, which is what bounds this kernel once the B x K pairs are many (B = 512, K = 1024, 400-float
-// box rows: 1.7 GB of query rows through the L2 in 76 us with one row per workgroup).  A row's sum has the same
+// box rows: 1.7 GB of query rows through the L2 in 76 us with one row per workgroup, 62 us with two; rotate rows of
+// 800 floats: 105 -> 89 us).  A row's sum has the same
 // terms in the same order for either value.
 template <int M, int VEC, int NIT, int NW, bool REG, int RW>
 __global__ __launch_bounds__(NW * 64) void shared_entity_kernel(SharedArgs A) {
@@ -237,7 +238,9 @@ int launch_shared_entity_reg(hipStream_t st, const SharedArgs& A) {
     }
   }
   // two rows per workgroup where their registers fit beside the queries in flight and enough workgroups remain
-  if constexpr (VEC == 4 && NIT * model_mul(M) <= 2) {
+  // (not BetaE, whose special-function terms need the registers: it spills with two rows; its shared lists are
+  // matrix products anyway)
+  if constexpr (VEC == 4 && NIT * model_mul(M) <= 4 && M != mBetaKL) {
     if (A.K >= 512 && A.B >= 64 && 14 * row_bytes <= 60 * 1024) {
       hipLaunchKernelGGL((shared_entity_kernel<M, VEC, NIT, 8, REG, 2>), dim3((unsigned)((A.K + 1) / 2)), dim3(8 * 64),
                          14 * row_bytes, st, A);

@@ -24,7 +24,7 @@ SHAPES = [("box", 300, 9, 40, 48), ("l1", 200, 5, 17, 200), ("l2", 150, 6, 33, 3
           # lists of 512 and more ids under 64 and more queries: the entity side takes two rows per workgroup (an odd
           # number of positions and of distinct ids, ids that hold several positions beside ids that hold one)
           ("box", 700, 70, 513, 200), ("box", 2000, 64, 512, 400), ("l1", 800, 65, 515, 64), ("l2", 700, 66, 600, 100),
-          ("rotate", 900, 64, 512, 100)]
+          ("rotate", 900, 64, 512, 100), ("rotate", 1200, 64, 512, 400), ("beta_kl", 700, 64, 520, 260)]
 
 
 def _shared_problem(model, n, b, k, dim):
