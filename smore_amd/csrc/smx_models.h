@@ -132,7 +132,10 @@ template <> struct ModelOps<mL2> {
     a0 += Term<kL2, float>::fwd(e1, 0.f, q.a, 0.f);
   }
   static __device__ __forceinline__ float fold(float a0, float, const ScoreParams&) { return a0; }
-  static __device__ __forceinline__ float score(float folded, const ScoreParams& p) { return p.gamma - sqrtf(folded); }
+  // (the root as the hardware instruction, one ulp: the correctly rounded sqrtf is a third of this model's forward)
+  static __device__ __forceinline__ float score(float folded, const ScoreParams& p) {
+    return p.gamma - __builtin_amdgcn_sqrtf(folded);
+  }
   // d(gamma - sqrt(d2)) / d d2 = -1 / (2 sqrt(d2)): the kernels multiply this upstream part by the
   // pair's own 1 / (2 sqrt(d2)), see l2_pair_coef.  At d2 == 0 the coefficient is infinite, as autograd
   // of torch.sqrt makes it in the reference.

@@ -64,7 +64,7 @@ __device__ __forceinline__ float hw_rcp(float x) { return __builtin_amdgcn_rcpf(
 // L2 only.  score = gamma - sqrt(d2), so d score / d d2 = -1 / (2 sqrt(d2)).  The reference divides by the
 // square root autograd saved (l2_dist.py:59,62); recovering it as gamma - score would add half an ulp of
 // gamma to the distance, a relative error of 5e-7 / distance.  The backward kernels hold the pair's entity
-// row and query in registers anyway, so they sum d2 again, in the forward's order, and divide by its root.
+// row and query in registers anyway, so they sum d2 again, in the forward's order, and multiply by its reciprocal root.
 // c_raw: the upstream part of the coefficient (-gscore).  e(it, v), q(it, v): the lane's features.
 template <int VEC, int NIT, class GetE, class GetQ>
 __device__ __forceinline__ float l2_pair_coef(float c_raw, int ncol, int lane, GetE&& e, GetQ&& q) {
@@ -77,7 +77,7 @@ __device__ __forceinline__ float l2_pair_coef(float c_raw, int ncol, int lane, G
     mine += lane + 64 * it < ncol ? a0 : 0.f;
   }
   const float d2 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(wave_sum_last_f32(mine)), 63));
-  return c_raw / (2.0f * sqrtf(d2));
+  return c_raw * (0.5f * __builtin_amdgcn_rsqf(d2));  // (one ulp; infinite at d2 == 0 like the division)
 }
 
 // 0 when the parameters are usable, else a message for the caller
