@@ -139,9 +139,11 @@ __device__ __forceinline__ const float* shared_row(const GemmArgs& A, int k, int
 }
 
 // score[b,k] = gamma -/+ (... + sum_j q[b,j] row_k[j]), j over the nq * dim features ([q1 | q2] against a row).
-// Both operands have the inner dimension contiguous: a lane reads two neighbouring features per load and feeds
-// them to two instructions (instruction t of a group of four features takes feature 4 g + 2 (l / 32) + t).
-// The groups of four features are dealt out to the four wavefronts in contiguous quarters.
+// Both operands have the inner dimension contiguous, so a lane's operand values lie along its own row: it reads
+// four neighbouring features per 16-byte load and feeds them to four instructions (8-byte loads for two
+// instructions took 26 us where this takes 21, ComplEx at B = 512, K = 1024, D = 400: the loads of a wavefront touch
+// 64 different lines either way).  The units of eight features are dealt out to the four wavefronts in contiguous
+// quarters.
 template <bool BETA>
 __global__ __launch_bounds__(256) void shared_forward_gemm_kernel(GemmArgs A) {
   __shared__ float part[3 * 16 * 64];
@@ -154,28 +156,36 @@ __global__ __launch_bounds__(256) void shared_forward_gemm_kernel(GemmArgs A) {
   const int half = lane >> 5, col = lane & 31;
   const int my_b = min(b0 + col, B - 1), my_k = min(k0 + col, K - 1);  // rows past the end repeat the last one; never stored
   int bad = 0;
-  const float2* t = reinterpret_cast<const float2*>(shared_row<BETA>(A, my_k, bad)) + half;
-  const float2* a1 = reinterpret_cast<const float2*>(A.q1 + (size_t)my_b * dim) + half;
-  const float2* a2 = A.nq == 2 ? reinterpret_cast<const float2*>(A.q2 + (size_t)my_b * dim) + half : a1;
+  // a unit of eight features: lanes 0-31 supply features 8 u .. 8 u + 3 of their row, lanes 32-63 features
+  // 8 u + 4 .. 8 u + 7, one 16-byte load each; instruction s of the unit's four takes element s of both
+  const float* t_row = shared_row<BETA>(A, my_k, bad);
+  const float* a1_row = A.q1 + (size_t)my_b * dim;
+  const float* a2_row = A.nq == 2 ? A.q2 + (size_t)my_b * dim : a1_row;
   if (bad && A.err) *A.err = 1;
-  const int G = dim / 4;               // groups per query tensor
-  const int GT = A.nq * G;             // groups of the inner dimension
-  const int per = (GT + 3) / 4;
-  const int g_lo = wave * per, g_hi = min(GT, g_lo + per);
-  auto ld_a = [&](int gi) {
-    const int g = min(gi, GT - 1);
-    return g < G ? a1[2 * g] : a2[2 * (g - G)];
+  const int J = A.nq * dim;            // the inner dimension, a multiple of four
+  const int UT = (J + 7) / 8;          // units
+  const int per = (UT + 3) / 4;
+  const int u_lo = wave * per, u_hi = min(UT, u_lo + per);
+  typedef float f4 __attribute__((ext_vector_type(4)));
+  const f4 zero4 = {0.f, 0.f, 0.f, 0.f};
+  auto ld_a = [&](int ui) -> f4 {
+    const int f = 8 * min(ui, UT - 1) + 4 * half;
+    if (f >= J) return zero4;  // the second half of a last unit of four features
+    return *reinterpret_cast<const f4*>(f < dim ? a1_row + f : a2_row + (f - dim));
   };
-  auto ld_t = [&](int gi) { return t[2 * min(gi, GT - 1)]; };
+  auto ld_t = [&](int ui) -> f4 {
+    const int f = 8 * min(ui, UT - 1) + 4 * half;
+    return f >= J ? zero4 : *reinterpret_cast<const f4*>(t_row + f);
+  };
   facc16 acc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-  // four groups at a time, the next four requested before these are used (requests past the end repeat the last group)
-  float2 av[4], tv[4], an[4], tn[4];
+  // four units at a time, the next four requested before these are used (requests past the end repeat the last unit)
+  f4 av[4], tv[4], an[4], tn[4];
 #pragma unroll
   for (int u = 0; u < 4; ++u) {
-    av[u] = ld_a(g_lo + u);
-    tv[u] = ld_t(g_lo + u);
+    av[u] = ld_a(u_lo + u);
+    tv[u] = ld_t(u_lo + u);
   }
-  for (int g = g_lo; g < g_hi; g += 4) {
+  for (int g = u_lo; g < u_hi; g += 4) {
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       an[u] = ld_a(g + 4 + u);
@@ -183,9 +193,9 @@ __global__ __launch_bounds__(256) void shared_forward_gemm_kernel(GemmArgs A) {
     }
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
-      if (g + u < g_hi) {  // uniform
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av[u].x, tv[u].x, acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av[u].y, tv[u].y, acc, 0, 0, 0);
+      if (g + u < u_hi) {  // uniform
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av[u][e], tv[u][e], acc, 0, 0, 0);
       }
     }
 #pragma unroll
