@@ -28,6 +28,10 @@ function is pinned by an independent check in tests/test_oracle_pinning.py:
                             first step; squeeze variant by closed form
   sgd / adagrad / rmsprop   torch.optim.SGD / Adagrad / RMSprop(alpha=0.99) when
                             every row is touched; squeeze variants by closed form
+  unit_halves (+backward)   torch.nn.functional.normalize (the routine the reference calls) and
+                            its autograd on each half, unit length of the result, orthogonality
+                            of the gradient to the row, central finite differences, the
+                            below-eps branch by hand
   score / train_step        composition only (gamma - dist, gamma + similarity, chain rule of sqrt)
 """
 import ctypes
@@ -158,6 +162,38 @@ def regularizer(x, base_add=1.0, lo=0.05, hi=1e9, dtype=np.float64):
     return out
 
 
+def unit_halves(rows, dtype=np.float64, eps=1e-12):
+    """Each half of the last axis scaled to unit L2 length, x / max(|x|, eps): what ComplexReasoning does to an
+    entity row before complex_sim when its mode names 'norm' (models/complex.py:142-146; embed_norm = Normalizer,
+    common/modules.py:38-40 = F.normalize(p=2, dim=-1), whose eps is 1e-12)."""
+    rows = np.asarray(rows, dtype=dtype)
+    h = rows.shape[-1] // 2
+    out = np.empty_like(rows)
+    for sl in (slice(0, h), slice(h, 2 * h)):
+        x = rows[..., sl]
+        n = np.maximum(np.sqrt((x * x).sum(axis=-1, keepdims=True)), dtype(eps))
+        out[..., sl] = x / n
+    return out
+
+
+def unit_halves_backward(rows, gout, dtype=np.float64, eps=1e-12):
+    """Gradient w.r.t. rows of sum(gout * unit_halves(rows)): per half (g - x_n (x_n . g)) / |x| where |x| > eps,
+    g / eps below (the denominator is then the constant eps)."""
+    rows = np.asarray(rows, dtype=dtype)
+    gout = np.asarray(gout, dtype=dtype)
+    h = rows.shape[-1] // 2
+    out = np.empty_like(rows)
+    for sl in (slice(0, h), slice(h, 2 * h)):
+        x, g = rows[..., sl], gout[..., sl]
+        n = np.sqrt((x * x).sum(axis=-1, keepdims=True))
+        live = n > eps
+        safe = np.where(live, n, dtype(1.0))
+        xn = x / safe
+        proj = (g - xn * (xn * g).sum(axis=-1, keepdims=True)) / safe
+        out[..., sl] = np.where(live, proj, g / dtype(eps))
+    return out
+
+
 def merge_indices(idx):
     """Returns (uniq[U], inverse[P], order[P], seg_start[U+1]).
 
@@ -277,10 +313,14 @@ MODELS = ("l1", "l2", "box", "rotate", "beta_kl", "complex", "distmult")
 SIMILARITY = ("complex", "distmult")
 
 
-def score_forward(model, rows, q1, q2=None, gamma=0.0, cen=0.0, dtype=np.float64):
+def score_forward(model, rows, q1, q2=None, gamma=0.0, cen=0.0, dtype=np.float64, norm=False):
     """rows [B,K,De], q [B,1,D] -> logit [B,K] as the custom_cal_logit bodies compute it
     (models/vec.py:85-90, box.py:157-164, rotate.py:137-142, beta.py:303-308) with one
-    union branch; l2 takes the square root outside the operator (dist_func/l2_dist.py:59-62)."""
+    union branch; l2 takes the square root outside the operator (dist_func/l2_dist.py:59-62).
+    norm (complex only): the halves of every entity row at unit length first (complex.py:142-146)."""
+    if norm:
+        assert model == "complex"
+        rows = unit_halves(rows, dtype)
     if model == "box":
         d = dist_forward("box_out", rows, q1, q2, dtype) + cen * dist_forward("box_in", rows, q1, q2, dtype)
     elif model == "l2":
@@ -292,9 +332,13 @@ def score_forward(model, rows, q1, q2=None, gamma=0.0, cen=0.0, dtype=np.float64
     return (gamma - d).astype(dtype)
 
 
-def score_backward(model, gscore, rows, q1, q2=None, cen=0.0, dtype=np.float64):
+def score_backward(model, gscore, rows, q1, q2=None, cen=0.0, dtype=np.float64, norm=False):
     """Gradients of sum(gscore * score) w.r.t. rows, q1, q2."""
     gscore = np.asarray(gscore, dtype=dtype)
+    if norm:
+        assert model == "complex"
+        gn, gq1, gq2 = dist_backward(model, gscore, unit_halves(rows, dtype), q1, q2, dtype)
+        return unit_halves_backward(rows, gn, dtype), gq1, gq2
     if model == "box":
         a = dist_backward("box_out", -gscore, rows, q1, q2, dtype)
         b = dist_backward("box_in", -cen * gscore, rows, q1, q2, dtype)
@@ -309,14 +353,14 @@ def score_backward(model, gscore, rows, q1, q2=None, cen=0.0, dtype=np.float64):
 
 
 def train_step(model, table, m, v, idx, q1, q2, gscore, gamma, cen, lr, step, dtype=np.float64,
-               squeeze=False, apply_adam=True):
+               squeeze=False, apply_adam=True, norm=False):
     """One pass in the order of training/train_process.py:172-220 with the loss replaced by
     a given upstream gradient: gather, score, backward, unique-merge, segment sum, lazy Adam.
     table/m/v are updated in place.  Returns a dict of everything in between."""
     b, k = idx.shape
     rows = gather(table, idx, dtype).reshape(b, k, -1)
-    score = score_forward(model, rows, q1, q2, gamma, cen, dtype)
-    grows, gq1, gq2 = score_backward(model, gscore, rows, q1, q2, cen, dtype)
+    score = score_forward(model, rows, q1, q2, gamma, cen, dtype, norm)
+    grows, gq1, gq2 = score_backward(model, gscore, rows, q1, q2, cen, dtype, norm)
     uniq, inverse, order, seg_start = merge_indices(idx)
     merged = merge_grads(grows.reshape(b * k, -1), inverse, uniq.size, dtype)
     if apply_adam:

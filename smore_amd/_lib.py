@@ -99,7 +99,8 @@ SIGNATURES = {
 
 class ScoreParams(ctypes.Structure):
     """smx_score_params of include/smore_amd.h."""
-    _fields_ = [("gamma", _f), ("cen", _f), ("reg_on", _i), ("reg_add", _f), ("reg_lo", _f), ("reg_hi", _f)]
+    _fields_ = [("gamma", _f), ("cen", _f), ("reg_on", _i), ("reg_add", _f), ("reg_lo", _f), ("reg_hi", _f),
+                ("norm_on", _i)]
 
 
 OPT_KINDS = {"adam": 1, "sgd": 2, "adagrad": 3, "rmsprop": 4}

@@ -155,8 +155,7 @@ int entity_backward(int model, void* stream, const smx_plan_view* plan, float* t
   if (!table || !q1 || (!multi && (!score || !gscore)) || !params || (model_nq(model) == 2 && !q2))
     return fail(SMX_ERR_ARG, "null pointer");
   if (B == 0 || K == 0 || dim == 0 || n_rows == 0) return fail(SMX_ERR_SHAPE, "empty dimension");
-  if (params->reg_on && model != mBetaKL)
-    return fail(SMX_ERR_ARG, "the entity clamp prologue exists for the beta_kl model only");
+  if (const char* why = params_refused(model, params)) return fail(SMX_ERR_ARG, "%s", why);
   if (!merged && !adam) return fail(SMX_ERR_ARG, "nothing to do: neither merged gradient nor an optimizer requested");
   EntityArgs A{};
   const size_t row_len = dim * model_mul(model);
@@ -223,7 +222,7 @@ int entity_backward(int model, void* stream, const smx_plan_view* plan, float* t
     A.gscore = multi->gscore[0];
     A.winner = multi->winner[0];
   }
-  A.p = ScoreParams{params->gamma, params->cen, params->reg_on, params->reg_add, params->reg_lo, params->reg_hi};
+  A.p = to_params(params);
   A.table = table;
   A.merged = merged;
   A.ncol = (int)ncol;

@@ -21,6 +21,7 @@
 // (smore/common/modules.py:29-36 applied at smore/models/kg_reasoning.py:352);
 // its backward passes gradient where lo <= e + add <= hi.
 #pragma once
+#include "../../include/smore_amd.h"
 #include "smx_functors.h"
 
 namespace smx {
@@ -37,7 +38,14 @@ struct ScoreParams {
   float cen;      // weight of the inside distance (BOX only)
   int reg_on;     // entity prologue on/off
   float reg_add, reg_lo, reg_hi;
+  int norm_on;    // COMPLEX: unit-length halves (the kernels' REG instantiation stands for it there)
 };
+
+inline ScoreParams to_params(const smx_score_params* c) {
+  return ScoreParams{c->gamma, c->cen, c->reg_on, c->reg_add, c->reg_lo, c->reg_hi, c->norm_on ? 1 : 0};
+}
+// the entity-side options a model does not have: nullptr, or what to tell the caller
+inline const char* params_refused(int model, const smx_score_params* c);
 
 __device__ __forceinline__ float reg_apply(float e, const ScoreParams& p) {
   if (!p.reg_on) return e;
@@ -48,6 +56,12 @@ __device__ __forceinline__ float reg_mask(float e_raw, float g, const ScoreParam
   if (!p.reg_on) return g;
   const float v = e_raw + p.reg_add;
   return (v >= p.reg_lo && v <= p.reg_hi) ? g : 0.0f;
+}
+
+inline const char* params_refused(int model, const smx_score_params* c) {
+  if (c->reg_on && model != mBetaKL) return "the entity clamp prologue exists for the beta_kl model only";
+  if (c->norm_on && model != mComplex) return "unit-length row halves exist for the complex model only";
+  return nullptr;
 }
 
 // per-feature query registers kept by a lane for the whole tile
@@ -382,6 +396,19 @@ template <> struct ModelOps<mComplex> {
     Term<kComplex, float>::bwd(c0, e1, e2, q.a, q.b, s1, s2, g1, g2);
   }
 };
+
+// ComplEx with unit-length halves (complex.py:142-146 when the model's mode names 'norm', complex.py:87-89;
+// embed_norm = F.normalize(p = 2, dim = -1), modules.py:38-40):
+//   logit = gamma + (re . q_re) / max(|re|, eps) + (im . q_im) / max(|im|, eps),   eps = 1e-12
+//   d logit / d q_re = re / max(|re|, eps)
+//   d logit / d re   = (q_re - re_n (re_n . q_re)) / |re|   with re_n = re / |re|    (q_re / eps below eps)
+// The scaling belongs to the entity, not to the pair: summed over an entity's pairs the gradient is the plain ComplEx
+// gradient G = sum c q pushed through the scaling once, g_re = (G_re - re_n (re_n . G_re)) / |re|.  The entity
+// kernels therefore accumulate G as they do for plain ComplEx, and the function that finishes a row applies the
+// projection.  In the kernels the REG instantiation of the ComplEx model stands for this form.
+constexpr float kNormEps = 1e-12f;
+__host__ __device__ constexpr bool model_norm(int m, bool reg) { return m == mComplex && reg; }
+__device__ __forceinline__ float inv_norm(float sumsq) { return 1.f / fmaxf(__builtin_sqrtf(sumsq), kNormEps); }
 
 template <> struct ModelOps<mDistmult> {
   using Q = QPair;

@@ -28,8 +28,8 @@ static int rank_common(RankArgs* R, int* vec, int* nit, int model, const float* 
   if (n_rows > 0xfffffff8ull) return fail(SMX_ERR_SHAPE, "entity count %zu needs ids wider than 32 bits", n_rows);
   if (A > kRankMaxAnswers) return fail(SMX_ERR_SHAPE, "at most %zu answers per query", kRankMaxAnswers);
   if (B > 0x7fffffffull / (A + 1)) return fail(SMX_ERR_SHAPE, "too many queries");
-  if (params->reg_on && model != mBetaKL)
-    return fail(SMX_ERR_ARG, "the entity clamp prologue exists for the beta_kl model only");
+  if (const char* why = params_refused(model, params)) return fail(SMX_ERR_ARG, "%s", why);
+  if (params->norm_on) return fail(SMX_ERR_ARG, "the ranking kernels have no unit-length form of the complex model");
   const bool vec4 = dim % 4 == 0 && aligned16(table) && aligned16(q1) && (model_nq(model) == 1 || aligned16(q2));
   *vec = vec4 ? 4 : 1;
   const size_t ncol = dim / *vec;
@@ -45,7 +45,7 @@ static int rank_common(RankArgs* R, int* vec, int* nit, int model, const float* 
   R->U = (int)U;
   R->ncol = (int)ncol;
   R->n_rows = n_rows;
-  R->p = ScoreParams{params->gamma, params->cen, params->reg_on, params->reg_add, params->reg_lo, params->reg_hi};
+  R->p = to_params(params);
   R->ans_id = reinterpret_cast<const long long*>(ans_id);
   R->ans_count = ans_count;
   R->A = (int)A;

@@ -80,6 +80,53 @@ __device__ __forceinline__ float l2_pair_coef(float c_raw, int ncol, int lane, G
   return c_raw * (0.5f * __builtin_amdgcn_rsqf(d2));  // (one ulp; infinite at d2 == 0 like the division)
 }
 
+// ComplEx with unit-length halves, query backward: the pair's upstream coefficient over the two lengths of its row.
+template <int VEC, int NIT, class GetE1, class GetE2>
+__device__ __forceinline__ float2 norm_pair_coef(float c_raw, int ncol, int lane, GetE1&& e1, GetE2&& e2) {
+  float s1 = 0.f, s2 = 0.f;
+#pragma unroll
+  for (int it = 0; it < NIT; ++it) {
+    float a = 0.f, b = 0.f;
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) {
+      a = __builtin_fmaf(e1(it, v), e1(it, v), a);
+      b = __builtin_fmaf(e2(it, v), e2(it, v), b);
+    }
+    const bool in = lane + 64 * it < ncol;
+    s1 += in ? a : 0.f;
+    s2 += in ? b : 0.f;
+  }
+  return make_float2(c_raw * inv_norm(wave_sum_f32(s1)), c_raw * inv_norm(wave_sum_f32(s2)));
+}
+
+// ... entity side: the summed plain gradient g of one half row w pushed through w / max(|w|, eps)
+template <int VEC, int NIT, class GetW>
+__device__ __forceinline__ void norm_project(float (&g)[NIT][VEC], int ncol, int lane, GetW&& w) {
+  float sq = 0.f, dot = 0.f;
+#pragma unroll
+  for (int it = 0; it < NIT; ++it) {
+    float a = 0.f, b = 0.f;
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) {
+      a = __builtin_fmaf(w(it, v), w(it, v), a);
+      b = __builtin_fmaf(w(it, v), g[it][v], b);
+    }
+    const bool in = lane + 64 * it < ncol;
+    sq += in ? a : 0.f;
+    dot += in ? b : 0.f;
+  }
+  sq = wave_sum_f32(sq);
+  dot = wave_sum_f32(dot);
+  const float len = __builtin_sqrtf(sq);
+  const bool live = len > kNormEps;  // below eps the scaling is the constant 1 / eps
+  const float inv = live ? 1.f / len : 1.f / kNormEps;
+  const float k = live ? dot * inv * inv : 0.f;
+#pragma unroll
+  for (int it = 0; it < NIT; ++it)
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) g[it][v] = (g[it][v] - w(it, v) * k) * inv;
+}
+
 // 0 when the parameters are usable, else a message for the caller
 inline const char* check_opt_params(const smx_opt_params* a, const void* m, const void* v) {
   if (a->kind < SMX_OPT_ADAM || a->kind > SMX_OPT_RMSPROP) return "unknown optimizer kind";
@@ -188,6 +235,10 @@ __device__ __forceinline__ void finish_row(const RowSink& A, int lane, unsigned 
         const float x2 = MUL == 2 ? (REG ? reg_apply(w.h[MUL - 1][it].v[x], A.p) : w.h[MUL - 1][it].v[x]) : 0.f;
         finish_entity_grad<SRC>(x1, x2, g1[it][x], g2[it][x]);
       }
+    if constexpr (model_norm(SRC, REG)) {
+      norm_project<VEC, NIT>(g1, A.ncol, lane, [&](int it, int x) { return w.h[0][it].v[x]; });
+      norm_project<VEC, NIT>(g2, A.ncol, lane, [&](int it, int x) { return w.h[MUL - 1][it].v[x]; });
+    }
   }
   if (REG) {
 #pragma unroll

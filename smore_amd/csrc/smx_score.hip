@@ -48,9 +48,9 @@ extern template int shared_forward_dispatch<mBox>(hipStream_t, const SharedFwdAr
 extern template int shared_forward_dispatch<mRotate>(hipStream_t, const SharedFwdArgs&, int);
 
 // defined in smx_shared_gemm.hip: shared negatives of beta_kl, complex and distmult as matrix products
-size_t shared_gemm_workspace_floats(int model, size_t B, size_t K, size_t dim, bool entity);
+size_t shared_gemm_workspace_floats(int model, size_t B, size_t K, size_t dim, bool entity, bool norm);
 bool shared_gemm_fits(int model, size_t dim, const void* table, const void* q1, const void* q2, const void* workspace,
-                      size_t workspace_bytes, size_t B, size_t K, bool entity);
+                      size_t workspace_bytes, size_t B, size_t K, bool entity, bool norm);
 int shared_gemm_forward(int model, hipStream_t st, const float* table, size_t n_rows, const long long* ids,
                         const float* q1, const float* q2, float* score, size_t B, size_t K, size_t dim,
                         const ScoreParams& p, int* err, float* workspace);
@@ -142,8 +142,7 @@ static int fill_args(ScoreArgs* A, int* vec, int* nit, int model, const float* t
     return fail(SMX_ERR_SHAPE, "more than 2^31-1 pairs in one call");
   if (idx && n_rows > 0xffffffffull)  // the kernels tell ids apart by their low 32 bits, as the segment plan does
     return fail(SMX_ERR_SHAPE, "entity count %zu needs ids wider than 32 bits", n_rows);
-  if (params->reg_on && model != mBetaKL)
-    return fail(SMX_ERR_ARG, "the entity clamp prologue exists for the beta_kl model only");
+  if (const char* why = params_refused(model, params)) return fail(SMX_ERR_ARG, "%s", why);
   const bool vec4 = dim % 4 == 0 && aligned16(table) && aligned16(q1) && (model_nq(model) == 1 || aligned16(q2)) &&
                     aligned16(extra_a) && aligned16(extra_b);
   *vec = vec4 ? 4 : 1;
@@ -162,7 +161,7 @@ static int fill_args(ScoreArgs* A, int* vec, int* nit, int model, const float* t
   A->ncol = (int)ncol;
   A->n_rows = idx ? n_rows : B * K;
   A->U = 1;
-  A->p = ScoreParams{params->gamma, params->cen, params->reg_on, params->reg_add, params->reg_lo, params->reg_hi};
+  A->p = to_params(params);
   return SMX_OK;
 }
 
@@ -238,8 +237,8 @@ int smx_score_backward_query(int model, void* stream, const float* table, size_t
 
 size_t smx_shared_workspace_bytes(int model, size_t B, size_t K, size_t dim) {
   if (model < 0 || model >= smx::mNumModels) return 0;
-  const size_t a = smx::shared_gemm_workspace_floats(model, B, K, dim, false);
-  const size_t b = smx::shared_gemm_workspace_floats(model, B, K, dim, true);
+  const size_t a = smx::shared_gemm_workspace_floats(model, B, K, dim, false, true);
+  const size_t b = smx::shared_gemm_workspace_floats(model, B, K, dim, true, true);
   const size_t n = a > b ? a : b;
   return n ? ((n * sizeof(float) + 255) & ~(size_t)255) : 0;
 }
@@ -255,7 +254,7 @@ int smx_score_forward_shared(int model, void* stream, const float* table, size_t
   if (!score) return fail(SMX_ERR_ARG, "null score pointer");
   // BetaE (the entity side of the divergence once per shared row: needs the workspace), ComplEx, DistMult: the pairs
   // as a matrix product
-  if (shared_gemm_fits(model, dim, table, q1, q2, workspace, workspace_bytes, B, K, false))
+  if (shared_gemm_fits(model, dim, table, q1, q2, workspace, workspace_bytes, B, K, false, A.p.norm_on != 0))
     return shared_gemm_forward(model, as_stream(stream), table, n_rows, reinterpret_cast<const long long*>(ids), q1, q2,
                                score, B, K, dim, A.p, err_flag, static_cast<float*>(workspace));
   if (shared_forward_fits(model, vec, nit)) {  // rows staged in LDS for eight queries at a time
@@ -285,7 +284,7 @@ int smx_score_backward_query_shared(int model, void* stream, const float* table,
   if (!ids) return fail(SMX_ERR_ARG, "null id list");
   if (int rc = fill_args(&A, &vec, &nit, model, table, n_rows, ids, q1, q2, B, K, dim, params, nullptr, nullptr)) return rc;
   if (!score || !gscore || !gq1 || (model_nq(model) == 2 && !gq2)) return fail(SMX_ERR_ARG, "null pointer");
-  if (shared_gemm_fits(model, dim, table, q1, q2, workspace, workspace_bytes, B, K, false))
+  if (shared_gemm_fits(model, dim, table, q1, q2, workspace, workspace_bytes, B, K, false, A.p.norm_on != 0))
     return shared_gemm_backward_query(model, as_stream(stream), table, n_rows, reinterpret_cast<const long long*>(ids), q1,
                                       q2, gscore, gq1, gq2, B, K, dim, A.p, static_cast<float*>(workspace));
   A.ids_shared = 1;

@@ -378,6 +378,37 @@ __global__ __launch_bounds__(256) void score_forward_kernel(ScoreArgs A, int til
   stream_batch<MUL, VEC, NIT, RIF>(slab, n_stream, dim, ncol, lane,
                                    [&](int j, const Pack<VEC>(&e1)[NIT], const Pack<VEC>(&e2)[NIT]) {
     // lanes past the row end hold a copy of the last column: they compute along and are dropped here.
+    if constexpr (model_norm(M, REG)) {
+      // unit-length halves: the two inner products and the two squared lengths are summed separately
+      float dot1 = 0.f, dot2 = 0.f, sq1 = 0.f, sq2 = 0.f;
+#pragma unroll
+      for (int it = 0; it < NIT; ++it) {
+        float a = 0.f, b2 = 0.f, c = 0.f, d = 0.f;
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) {
+          a = __builtin_fmaf(e1[it].v[v], q[it][v].a, a);
+          b2 = __builtin_fmaf(e2[it].v[v], q[it][v].b, b2);
+          c = __builtin_fmaf(e1[it].v[v], e1[it].v[v], c);
+          d = __builtin_fmaf(e2[it].v[v], e2[it].v[v], d);
+        }
+        const bool in = lane + 64 * it < ncol;
+        dot1 += in ? a : 0.f;
+        dot2 += in ? b2 : 0.f;
+        sq1 += in ? c : 0.f;
+        sq2 += in ? d : 0.f;
+      }
+      dot1 = wave_sum_last_f32(dot1);
+      dot2 = wave_sum_last_f32(dot2);
+      sq1 = wave_sum_last_f32(sq1);
+      sq2 = wave_sum_last_f32(sq2);
+      const float s = p.gamma + (dot1 * inv_norm(sq1) + dot2 * inv_norm(sq2));
+      if constexpr (DEDUP) {
+        if (lane == 63) rep_score[first_rep + j] = s;
+      } else {
+        if (lane == 63) out[j] = s;
+      }
+      return;
+    }
     // The logit is linear in the accumulators: fold them per lane, reduce once.
     float mine = 0.f;
 #pragma unroll
@@ -596,9 +627,13 @@ __global__ __launch_bounds__(NW * 64) void score_backward_query_kernel(ScoreArgs
     stream_batch<MUL, VEC, NIT, RIF>(slab, n_stream, dim, ncol, lane,
                                      [&](int j, const Pack<VEC>(&e1)[NIT], const Pack<VEC>(&e2)[NIT]) {
       float2 c = slab_coef(slab, j);
+      [[maybe_unused]] const float c_raw = c.x;
       if constexpr (M == mL2)
         c.x = l2_pair_coef<VEC, NIT>(c.x, ncol, lane, [&](int it, int v) { return e1[it].v[v]; },
                                      [&](int it, int v) { return q[it][v].a; });
+      if constexpr (model_norm(M, REG))  // d logit / d q = e / |e| per half: the upstream coefficient over the lengths
+        c = norm_pair_coef<VEC, NIT>(c_raw, ncol, lane, [&](int it, int v) { return e1[it].v[v]; },
+                                     [&](int it, int v) { return e2[it].v[v]; });
       if constexpr (CODES == 1) {
         // the pair's code bytes go to the wavefront's LDS stage, see flush_codes
         unsigned char* mine_b = stage + (j & (kStagePairs - 1)) * (NIT * 64) + lane;
@@ -618,8 +653,14 @@ __global__ __launch_bounds__(NW * 64) void score_backward_query_kernel(ScoreArgs
           for (int v = 0; v < VEC; ++v) {
             const float x1 = REG ? reg_apply(e1[it].v[v], p) : e1[it].v[v];
             const float x2 = MUL == 2 ? (REG ? reg_apply(e2[it].v[v], p) : e2[it].v[v]) : 0.f;
-            if constexpr (M == mBox) ModelOps<M>::bwd_q_thr(c.x, c.y, x1, q[it][v], neg_thr[it][v], g1[it][v], g2[it][v]);
-            else ModelOps<M>::bwd_q(c.x, c.y, x1, x2, q[it][v], g1[it][v], g2[it][v]);
+            if constexpr (M == mBox) {
+              ModelOps<M>::bwd_q_thr(c.x, c.y, x1, q[it][v], neg_thr[it][v], g1[it][v], g2[it][v]);
+            } else if constexpr (model_norm(M, REG)) {
+              g1[it][v] = __builtin_fmaf(c.x, x1, g1[it][v]);
+              g2[it][v] = __builtin_fmaf(c.y, x2, g2[it][v]);
+            } else {
+              ModelOps<M>::bwd_q(c.x, c.y, x1, x2, q[it][v], g1[it][v], g2[it][v]);
+            }
           }
         }
       }
@@ -636,7 +677,7 @@ __global__ __launch_bounds__(NW * 64) void score_backward_query_kernel(ScoreArgs
               ge1[it][v] = ge2[it][v] = 0.f;
               const float x1 = REG ? reg_apply(e1[it].v[v], p) : e1[it].v[v];
               const float x2 = MUL == 2 ? (REG ? reg_apply(e2[it].v[v], p) : e2[it].v[v]) : 0.f;
-              ModelOps<M>::bwd_e(c.x, c.y, x1, x2, q[it][v], ge1[it][v], ge2[it][v]);
+              ModelOps<M>::bwd_e(model_norm(M, REG) ? c_raw : c.x, c.y, x1, x2, q[it][v], ge1[it][v], ge2[it][v]);
             }
           const int seg = __builtin_amdgcn_readlane(my_ps, j) & 0x7fffffff;
           const unsigned row = (unsigned)__builtin_amdgcn_readlane((int)pb.row, j);
@@ -820,9 +861,9 @@ int launch_backward_query_reg(hipStream_t st, const ScoreArgs& A) {
 
 template <int M, int VEC, int NIT>
 int launch_score(hipStream_t st, const ScoreArgs& A, bool forward) {
-  const bool reg = M == mBetaKL && A.p.reg_on;
+  const bool reg = (M == mBetaKL && A.p.reg_on) || (M == mComplex && A.p.norm_on);
   if (forward) {
-    if constexpr (M == mBetaKL) {
+    if constexpr (M == mBetaKL || M == mComplex) {
       if (reg) return launch_forward_reg<M, VEC, NIT, true>(st, A);
     }
     return launch_forward_reg<M, VEC, NIT, false>(st, A);
@@ -833,7 +874,7 @@ int launch_score(hipStream_t st, const ScoreArgs& A, bool forward) {
   const size_t extra = kSlabDwords * sizeof(unsigned) + (model_coded(M) ? (size_t)kStagePairs * NIT * 64 : 0);
   auto fits = [&](size_t n) { return (n + 1) * per_wave + n * extra <= 64 * 1024; };
   const int nw = fits(8) ? 8 : (fits(4) ? 4 : 2);
-  if constexpr (M == mBetaKL) {
+  if constexpr (M == mBetaKL || M == mComplex) {
     if (reg) {
       if (nw == 8) return launch_backward_query_reg<M, VEC, NIT, 8, true>(st, A);
       if (nw == 4) return launch_backward_query_reg<M, VEC, NIT, 4, true>(st, A);

@@ -13,7 +13,7 @@ extern template int shared_entity_dispatch<mDistmult>(hipStream_t, const SharedA
 
 // defined in smx_shared_gemm.hip
 bool shared_gemm_fits(int model, size_t dim, const void* table, const void* q1, const void* q2, const void* workspace,
-                      size_t workspace_bytes, size_t B, size_t K, bool entity);
+                      size_t workspace_bytes, size_t B, size_t K, bool entity, bool norm);
 int shared_gemm_entity_sums(int model, hipStream_t st, const float* q1, const float* q2, const float* gscore, size_t B,
                             size_t K, size_t dim, float* workspace);
 
@@ -32,8 +32,7 @@ extern "C" int smx_score_backward_entity_shared(int model, void* stream, float* 
   if (B == 0 || K == 0 || dim == 0 || n_rows == 0) return fail(SMX_ERR_SHAPE, "empty dimension");
   if (B > 0x7fffffffull || K > 0x7fffffffull || B * K > 0x7fffffffull)
     return fail(SMX_ERR_SHAPE, "more than 2^31-1 pairs in one call");
-  if (params->reg_on && model != mBetaKL)
-    return fail(SMX_ERR_ARG, "the entity clamp prologue exists for the beta_kl model only");
+  if (const char* why = params_refused(model, params)) return fail(SMX_ERR_ARG, "%s", why);
   SharedArgs A{};
   if (plan) {
     if (grad_rows) return fail(SMX_ERR_ARG, "gradient rows per list position are the output of the call without a plan");
@@ -80,12 +79,12 @@ extern "C" int smx_score_backward_entity_shared(int model, void* stream, float* 
   A.B = (int)B;
   A.K = (int)K;
   A.n_rows = n_rows;
-  A.p = ScoreParams{params->gamma, params->cen, params->reg_on, params->reg_add, params->reg_lo, params->reg_hi};
+  A.p = to_params(params);
   A.table = table;
   A.ncol = (int)ncol;
   hipStream_t st = as_stream(stream);
   // BetaE, ComplEx, DistMult: the sums over the queries as a matrix product into the workspace, finished row by row below
-  if (vec == 4 && shared_gemm_fits(model, dim, table, q1, q2, workspace, workspace_bytes, B, K, true)) {
+  if (vec == 4 && shared_gemm_fits(model, dim, table, q1, q2, workspace, workspace_bytes, B, K, true, false)) {
     float* ws = static_cast<float*>(workspace);
     if (int rc = shared_gemm_entity_sums(model, st, q1, q2, gscore, B, K, dim, ws)) return rc;
     A.sums_r = ws;

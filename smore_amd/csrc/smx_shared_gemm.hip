@@ -110,7 +110,7 @@ __device__ __forceinline__ void combine_tiles(facc16& acc, float* part, int wave
 // the table found through the list's ids; nq = query tensors (the inner dimension is nq * dim features).
 struct GemmArgs {
   const float* rows;       // T [K][2 dim] (BETA) or the table
-  const long long* ids;    // [K] (not BETA)
+  const long long* ids;    // [K] (not BETA); null: `rows` holds the K rows themselves, in list order
   unsigned long long n_rows;
   const float* q1;
   const float* q2;
@@ -129,6 +129,7 @@ __device__ __forceinline__ const float* shared_row(const GemmArgs& A, int k, int
   if constexpr (BETA) {
     return A.rows + (size_t)k * 2 * A.dim;
   } else {
+    if (!A.ids) return A.rows + (size_t)k * A.nq * A.dim;  // uniform
     long long row = A.ids[k];
     if ((unsigned long long)row >= A.n_rows) {  // remember it, read row 0 instead (as every scorer of the library does)
       bad = 1;
@@ -366,22 +367,50 @@ __global__ __launch_bounds__(256) void shared_entity_gemm_kernel(GemmArgs A) {
   }
 }
 
+// ---- ComplEx with unit-length halves: the K rows of the list, scaled, as the products' second operand ----------
+// En [K][2 dim]: row k = [re / max(|re|, eps) | im / max(|im|, eps)] of table row ids[k]; one wavefront per row.
+__global__ __launch_bounds__(256) void unit_rows_kernel(const float* __restrict__ table, const long long* __restrict__ ids,
+                                                        int K, int dim, unsigned long long n_rows,
+                                                        float* __restrict__ En, int* err) {
+  const int lane = threadIdx.x & 63;
+  const int k = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (k >= K) return;
+  long long row = ids[k];
+  if ((unsigned long long)row >= n_rows) {
+    if (err && lane == 0) *err = 1;
+    row = 0;
+  }
+  const float* e = table + (size_t)row * 2 * dim;
+  float* out = En + (size_t)k * 2 * dim;
+  float s1 = 0.f, s2 = 0.f;
+  for (int d = lane; d < dim; d += 64) {
+    s1 = __builtin_fmaf(e[d], e[d], s1);
+    s2 = __builtin_fmaf(e[dim + d], e[dim + d], s2);
+  }
+  const float i1 = inv_norm(wave_sum_f32(s1)), i2 = inv_norm(wave_sum_f32(s2));
+  for (int d = lane; d < dim; d += 64) {
+    out[d] = e[d] * i1;
+    out[dim + d] = e[dim + d] * i2;
+  }
+}
+
 // ---- host side ----------------------------------------------------------------------------------------------
 static bool is_inner(int model) { return model == mComplex || model == mDistmult; }
 
 // floats of workspace a call of the model needs: forward / query backward, and the entity side
-size_t shared_gemm_workspace_floats(int model, size_t B, size_t K, size_t dim, bool entity) {
+// (norm: ComplEx with unit-length halves, whose scaled rows stand in the workspace for the first two)
+size_t shared_gemm_workspace_floats(int model, size_t B, size_t K, size_t dim, bool entity, bool norm) {
   if (model == mBetaKL) return entity ? K * (2 * dim + 1) : K * (2 * dim + 1) + B;
-  if (is_inner(model)) return entity ? K * (size_t)model_nq(model) * dim : 0;
+  if (is_inner(model)) return entity || norm ? K * (size_t)model_nq(model) * dim : 0;
   return 0;
 }
 
 // Whether the call can take these kernels: a model with a product form, float4-aligned operands, room in the workspace.
 bool shared_gemm_fits(int model, size_t dim, const void* table, const void* q1, const void* q2, const void* workspace,
-                      size_t workspace_bytes, size_t B, size_t K, bool entity) {
+                      size_t workspace_bytes, size_t B, size_t K, bool entity, bool norm) {
   if (model != mBetaKL && !is_inner(model)) return false;
   if (dim % 4 != 0 || !aligned16(table) || !aligned16(q1) || (model_nq(model) == 2 && !aligned16(q2))) return false;
-  const size_t need = shared_gemm_workspace_floats(model, B, K, dim, entity) * sizeof(float);
+  const size_t need = shared_gemm_workspace_floats(model, B, K, dim, entity, norm) * sizeof(float);
   if (need == 0) return true;
   return workspace && aligned16(workspace) && workspace_bytes >= need;
 }
@@ -422,6 +451,12 @@ int shared_gemm_forward(int model, hipStream_t st, const float* table, size_t n_
     A.Qk = Qk;
     hipLaunchKernelGGL(shared_forward_gemm_kernel<true>, dim3(tiles), dim3(256), 0, st, A);
   } else {
+    if (p.norm_on) {
+      hipLaunchKernelGGL(unit_rows_kernel, dim3((unsigned)((K + 3) / 4)), dim3(256), 0, st, table, ids, (int)K, (int)dim,
+                         (unsigned long long)n_rows, workspace, err);
+      A.rows = workspace;
+      A.ids = nullptr;
+    }
     hipLaunchKernelGGL(shared_forward_gemm_kernel<false>, dim3(tiles), dim3(256), 0, st, A);
   }
   return check_launch("score forward (shared negatives, matrix product)");
@@ -441,6 +476,12 @@ int shared_gemm_backward_query(int model, hipStream_t st, const float* table, si
     A.rows = T;
     hipLaunchKernelGGL(shared_backward_query_gemm_kernel<true>, dim3(tiles), dim3(256), 0, st, A);
   } else {
+    if (p.norm_on) {  // (scaled again rather than kept: the entity side of the previous step has used the workspace since)
+      hipLaunchKernelGGL(unit_rows_kernel, dim3((unsigned)((K + 3) / 4)), dim3(256), 0, st, table, ids, (int)K, (int)dim,
+                         (unsigned long long)n_rows, workspace, nullptr);
+      A.rows = workspace;
+      A.ids = nullptr;
+    }
     hipLaunchKernelGGL(shared_backward_query_gemm_kernel<false>, dim3(tiles), dim3(256), 0, st, A);
   }
   return check_launch("score backward (query, shared negatives, matrix product)");

@@ -256,8 +256,8 @@ int launch_shared_entity_reg(hipStream_t st, const SharedArgs& A) {
 
 template <int M, int VEC, int NIT>
 int launch_shared_entity(hipStream_t st, const SharedArgs& A) {
-  if constexpr (M == mBetaKL) {
-    if (A.p.reg_on) return launch_shared_entity_reg<M, VEC, NIT, true>(st, A);
+  if constexpr (M == mBetaKL || M == mComplex) {
+    if (M == mBetaKL ? A.p.reg_on : A.p.norm_on) return launch_shared_entity_reg<M, VEC, NIT, true>(st, A);
   }
   return launch_shared_entity_reg<M, VEC, NIT, false>(st, A);
 }

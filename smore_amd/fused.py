@@ -34,12 +34,13 @@ def _f32(t, name):
         raise _lib.SmxError(f"{name} must be a contiguous fp32 device tensor")
 
 
-def score_params(gamma, cen=0.0, regularizer=None):
-    """regularizer: None or (base_add, min_val, max_val) as in smore/common/modules.py:29-36."""
+def score_params(gamma, cen=0.0, regularizer=None, norm=False):
+    """regularizer: None or (base_add, min_val, max_val) as in smore/common/modules.py:29-36.
+    norm (complex): the halves of every entity row at unit length, smore/models/complex.py:142-146."""
     if regularizer is None:
-        return _lib.ScoreParams(gamma, cen, 0, 0.0, 0.0, 0.0)
+        return _lib.ScoreParams(gamma, cen, 0, 0.0, 0.0, 0.0, 1 if norm else 0)
     add, lo, hi = regularizer
-    return _lib.ScoreParams(gamma, cen, 1, add, lo, hi)
+    return _lib.ScoreParams(gamma, cen, 1, add, lo, hi, 1 if norm else 0)
 
 
 def new_error_flag(device):

@@ -10,7 +10,8 @@ from tests.util import REL_F32, assert_close, record_headroom, seed
 
 pytestmark = pytest.mark.gpu
 
-GAMMA = {"l1": 12.0, "l2": 12.0, "box": 24.0, "rotate": 9.0, "beta_kl": 60.0, "complex": 0.0, "distmult": 0.0}
+GAMMA = {"l1": 12.0, "l2": 12.0, "box": 24.0, "rotate": 9.0, "beta_kl": 60.0, "complex": 0.0, "distmult": 0.0,
+         "complex_norm": 0.0}   # complex with unit-length row halves (complex.py:142-146)
 
 
 def make_problem(model, n, b, k, dim, rng, zipf=None, scale=0.07):
@@ -50,9 +51,11 @@ def dev(a, dtype=torch.float32):
 def run_case(model, n, b, k, dim, zipf=None, cen=0.02, adam_steps=2, lr=1e-3):
     from smore_amd import fused
     rng = np.random.default_rng(seed(model, n, b, k, dim, zipf))
-    table, q1, q2, idx, gs = make_problem(model, n, b, k, dim, rng, zipf)
     gamma = GAMMA[model]
-    params = fused.score_params(gamma, cen)
+    norm = model == "complex_norm"
+    model = "complex" if norm else model
+    table, q1, q2, idx, gs = make_problem(model, n, b, k, dim, rng, zipf)
+    params = fused.score_params(gamma, cen, norm=norm)
     t_table, t_q1, t_q2, t_gs = dev(table), dev(q1), dev(q2), dev(gs)
     t_idx = torch.tensor(idx, device="cuda")
     err = fused.new_error_flag("cuda")
@@ -62,7 +65,7 @@ def run_case(model, n, b, k, dim, zipf=None, cen=0.02, adam_steps=2, lr=1e-3):
     rows = orc.gather(table, idx).reshape(b, k, -1)
     o_q1 = q1[:, None, :]
     o_q2 = None if q2 is None else q2[:, None, :]
-    want = orc.score_forward(model, rows, o_q1, o_q2, gamma, cen)
+    want = orc.score_forward(model, rows, o_q1, o_q2, gamma, cen, norm=norm)
     # no RMS floor for the scores of the models whose distance is a sum of non-negative terms: every element to 1e-5
     # (a KL divergence or an inner product is a sum of signed terms)
     assert_close(score.cpu().numpy(), want, REL_F32, f"{model} score", rms_floor=model in ("beta_kl", "complex", "distmult"))
@@ -75,7 +78,7 @@ def run_case(model, n, b, k, dim, zipf=None, cen=0.02, adam_steps=2, lr=1e-3):
 
     # query backward
     gq1, gq2 = fused.score_backward_query(model, t_table, t_idx, t_q1, t_q2, score, t_gs, params)
-    o_rows, o_g1, o_g2 = orc.score_backward(model, gs, rows, o_q1, o_q2, cen)
+    o_rows, o_g1, o_g2 = orc.score_backward(model, gs, rows, o_q1, o_q2, cen, norm=norm)
     # a query gradient is a sum over K signed terms of size <= |g_k| (unit-bounded derivatives of l1, l2, box,
     # rotate): when it cancels, one fp32 ulp of sum |g_k| is the floor of any summation order
     q_abs = None if model == "beta_kl" else np.abs(gs).sum(axis=1)[:, None] * np.ones((1, dim))
@@ -143,7 +146,7 @@ def run_case(model, n, b, k, dim, zipf=None, cen=0.02, adam_steps=2, lr=1e-3):
         assert_close(t_table.cpu().numpy()[touched], w_s[touched], REL_F32, f"{model} Adam step {step}: w")
         assert_close(t_m.cpu().numpy()[touched], m_s[touched], REL_F32, f"{model} Adam step {step}: m")
         assert_close(t_v.cpu().numpy()[touched], v_s[touched], REL_F32, f"{model} Adam step {step}: v", rms_floor=False)
-        orc.train_step(model, w_o, m_o, v_o, idx, o_q1, o_q2, gs, gamma, cen, lr, step)
+        orc.train_step(model, w_o, m_o, v_o, idx, o_q1, o_q2, gs, gamma, cen, lr, step, norm=norm)
     got_w = t_table.cpu().numpy()
     err = np.abs(got_w - w_o)[touched]
     tol = REL_F32 * np.maximum(np.abs(w_o[touched]), np.sqrt(np.mean(w_o[touched] ** 2)))

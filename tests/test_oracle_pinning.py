@@ -473,6 +473,59 @@ def test_similarity_and_two_half_scores_match_autograd_of_the_closed_forms():
           lambda e, a, c: 60.0 - kl(torch.distributions.Beta(e[..., :d], e[..., d:]), torch.distributions.Beta(a, c)).sum(-1))
 
 
+def test_unit_halves_is_f_normalize_per_half_and_its_backward_is_autograd():
+    """unit_halves / unit_halves_backward and the `norm` form of the ComplEx score (models/complex.py:142-146 with
+    embed_norm = F.normalize, common/modules.py:38-40).  torch's own normalize is the routine the reference calls;
+    the properties below catch what a comparison of two implementations of the same formula would not: a result
+    that is not of unit length, a gradient with a component along the row (the dropped projection term), a
+    wrong power of the length (finite differences)."""
+    rng = np.random.default_rng(31)
+    b, k, d = 3, 4, 5
+    rows = rng.standard_normal((b, k, 2 * d)) * rng.uniform(0.1, 5.0, (b, k, 1))
+    un = orc.unit_halves(rows)
+    assert np.allclose((un[..., :d] ** 2).sum(-1), 1.0, atol=1e-14) and np.allclose((un[..., d:] ** 2).sum(-1), 1.0, atol=1e-14)
+    tr = torch.tensor(rows, requires_grad=True)
+    F = torch.nn.functional
+    tn = torch.cat((F.normalize(tr[..., :d], p=2, dim=-1), F.normalize(tr[..., d:], p=2, dim=-1)), dim=-1)
+    assert np.allclose(un, tn.detach().numpy(), rtol=1e-14, atol=0)
+    g = rng.standard_normal(rows.shape)
+    (tn * torch.from_numpy(g)).sum().backward()
+    gb = orc.unit_halves_backward(rows, g)
+    assert np.allclose(gb, tr.grad.numpy(), rtol=1e-11, atol=1e-13)
+    # scaling a row does not change the result: the gradient has no component along it
+    assert np.abs((gb[..., :d] * rows[..., :d]).sum(-1)).max() < 1e-12
+    assert np.abs((gb[..., d:] * rows[..., d:]).sum(-1)).max() < 1e-12
+    # central finite differences of sum(g * unit_halves(rows))
+    f = lambda x: (g * orc.unit_halves(x)).sum()
+    h = 1e-6
+    for pos in [(0, 0, 0), (1, 2, d - 1), (2, 3, d), (0, 1, 2 * d - 1)]:
+        hi, lo = rows.copy(), rows.copy()
+        hi[pos] += h
+        lo[pos] -= h
+        assert abs((f(hi) - f(lo)) / (2 * h) - gb[pos]) < 1e-7 * max(1.0, abs(gb[pos]))
+    # a half shorter than eps is divided by eps, and so is its gradient (the clamp's constant branch)
+    tiny = np.zeros((1, 1, 4))
+    tiny[0, 0, :2] = [3e-13, 4e-13]          # length 5e-13 < 1e-12
+    tiny[0, 0, 2:] = [3.0, 4.0]
+    assert np.allclose(orc.unit_halves(tiny)[0, 0], [0.3, 0.4, 0.6, 0.8], rtol=1e-12)
+    gt = orc.unit_halves_backward(tiny, np.ones((1, 1, 4)))[0, 0]
+    assert np.allclose(gt[:2], [1e12, 1e12]) and np.allclose(gt[2:], [(1 - 0.6 * 1.4) / 5, (1 - 0.8 * 1.4) / 5], rtol=1e-12)
+    # the ComplEx logit over the scaled rows, and its three gradients, against autograd of the model's lines
+    re, im = rng.standard_normal((b, 1, d)), rng.standard_normal((b, 1, d))
+    gs = rng.standard_normal((b, k))
+    tr = torch.tensor(rows, requires_grad=True)
+    t1, t2 = torch.tensor(re, requires_grad=True), torch.tensor(im, requires_grad=True)
+    e_re, e_im = torch.chunk(tr, 2, dim=-1)
+    ent = torch.cat((F.normalize(e_re, p=2, dim=-1), F.normalize(e_im, p=2, dim=-1)), dim=-1)
+    s = 0.5 + (ent[..., :d] * t1 + ent[..., d:] * t2).sum(-1)
+    assert np.allclose(orc.score_forward("complex", rows, re, im, 0.5, norm=True), s.detach().numpy(), rtol=1e-12, atol=1e-14)
+    (s * torch.from_numpy(gs)).sum().backward()
+    gr, g1, g2 = orc.score_backward("complex", gs, rows, re, im, norm=True)
+    assert np.allclose(gr, tr.grad.numpy(), rtol=1e-10, atol=1e-13)
+    assert np.allclose(g1, t1.grad.numpy(), rtol=1e-10, atol=1e-13)
+    assert np.allclose(g2, t2.grad.numpy(), rtol=1e-10, atol=1e-13)
+
+
 def test_train_step_equals_dense_autograd_pipeline():
     """gather -> score -> backward -> merge -> Adam equals autograd through table[idx]
     followed by a dense Adam restricted to the touched rows."""

@@ -24,7 +24,10 @@ SHAPES = [("box", 300, 9, 40, 48), ("l1", 200, 5, 17, 200), ("l2", 150, 6, 33, 3
           # lists of 512 and more ids under 64 and more queries: the entity side takes two rows per workgroup (an odd
           # number of positions and of distinct ids, ids that hold several positions beside ids that hold one)
           ("box", 700, 70, 513, 200), ("box", 2000, 64, 512, 400), ("l1", 800, 65, 515, 64), ("l2", 700, 66, 600, 100),
-          ("rotate", 900, 64, 512, 100), ("rotate", 1200, 64, 512, 400), ("beta_kl", 700, 64, 520, 260)]
+          ("rotate", 900, 64, 512, 100), ("rotate", 1200, 64, 512, 400), ("beta_kl", 700, 64, 520, 260),
+          # complex with unit-length row halves (complex.py:142-146): scaled rows in the workspace as the products' operand
+          ("complex_norm", 90, 3, 10, 64), ("complex_norm", 150, 33, 45, 200), ("complex_norm", 30, 2, 1, 8),
+          ("complex_norm", 70, 32, 64, 16), ("complex_norm", 400, 70, 300, 400), ("complex_norm", 60, 5, 40, 30)]
 
 
 def _shared_problem(model, n, b, k, dim):
@@ -39,10 +42,12 @@ def _shared_problem(model, n, b, k, dim):
 @pytest.mark.parametrize("model,n,b,k,dim", SHAPES)
 def test_shared_negatives_match_oracle_and_the_per_query_kernels(model, n, b, k, dim):
     from smore_amd import fused
+    norm = model == "complex_norm"
+    model = "complex" if norm else model
     table, q1, q2, ids, gs = _shared_problem(model, n, b, k, dim)
     reg = (1.0, 0.05, 1e9) if model == "beta_kl" else None      # BetaE's entity prologue rides along
     cen = 0.02
-    params = fused.score_params(GAMMA[model], cen, reg)
+    params = fused.score_params(GAMMA[model], cen, reg, norm=norm)
     if reg is not None:
         table = table - 1.0 + np.where(np.arange(table.shape[1]) % 7 == 0, -0.99, 0.0)   # some values under the clamp
         table = table.astype(np.float32).astype(np.float64)
@@ -53,7 +58,7 @@ def test_shared_negatives_match_oracle_and_the_per_query_kernels(model, n, b, k,
     score = fused.score_forward_shared(model, t_table, t_ids, t_q1, t_q2, params, err)
     idx_full = np.broadcast_to(ids[None, :], (b, k))
     qs = [q1[:, None, None, :]] + ([] if q2 is None else [q2[:, None, None, :]])
-    logit, rows = oracle_union_logits(model, table, idx_full, qs, GAMMA[model], cen, regularizer=reg is not None)
+    logit, rows = oracle_union_logits(model, table, idx_full, qs, GAMMA[model], cen, regularizer=reg is not None, norm=norm)
     assert_close(score.cpu().numpy(), logit[:, 0], REL_F32, f"{model} shared score",
                  rms_floor=model in ("beta_kl", "complex", "distmult"))
     # against the per-query layout (the same ids repeated for every query).  The kernel written for the shared list
@@ -73,7 +78,7 @@ def test_shared_negatives_match_oracle_and_the_per_query_kernels(model, n, b, k,
     assert err.item() == 0
 
     gq1, gq2 = fused.score_backward_query_shared(model, t_table, t_ids, t_q1, t_q2, score, t_gs, params)
-    g_rows, g_qs = oracle_union_grads(model, table, idx_full, qs, rows, logit, gs, cen, regularizer=reg is not None)
+    g_rows, g_qs = oracle_union_grads(model, table, idx_full, qs, rows, logit, gs, cen, regularizer=reg is not None, norm=norm)
     q_abs = None if model == "beta_kl" else np.abs(gs).sum(axis=1)[:, None] * np.ones((1, dim))
     assert_close(gq1.cpu().numpy(), g_qs[0][:, 0, 0], REL_F32, f"{model} shared gq1", sum_abs=q_abs)
     if q2 is not None:
@@ -86,9 +91,9 @@ def test_shared_negatives_match_oracle_and_the_per_query_kernels(model, n, b, k,
             assert_close(p2.cpu().numpy(), f2.cpu().numpy(), 5e-6, f"{model} shared gq2, matrix product vs per-pair kernel", sum_abs=q_abs)
     else:
         assert torch.equal(f1, p1) and (f2 is None or torch.equal(f2, p2))
-    if model == "beta_kl":
-        assert_close(gq1.cpu().numpy(), p1.cpu().numpy(), 5e-6, "beta_kl shared gq1, per-row terms vs per-pair kernel")
-        assert_close(gq2.cpu().numpy(), p2.cpu().numpy(), 5e-6, "beta_kl shared gq2, per-row terms vs per-pair kernel")
+    if model == "beta_kl" or norm:   # (unit-length complex without workspace: the per-query kernel, not a matrix product)
+        assert_close(gq1.cpu().numpy(), p1.cpu().numpy(), 5e-6, f"{model} shared gq1, per-row terms vs per-pair kernel", sum_abs=q_abs)
+        assert_close(gq2.cpu().numpy(), p2.cpu().numpy(), 5e-6, f"{model} shared gq2, per-row terms vs per-pair kernel", sum_abs=q_abs)
     else:
         assert torch.equal(gq1, p1) and (gq2 is None or torch.equal(gq2, p2))
 

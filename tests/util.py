@@ -95,19 +95,20 @@ def make_inputs(kind, be, ne, bc, nc, dim, rng, scale=1.0):
     return e, q1, q2
 
 
-def oracle_union_logits(model, table, ids, qs, gamma, cen, regularizer=False):
+def oracle_union_logits(model, table, ids, qs, gamma, cen, regularizer=False, norm=False):
     """Float64 logits [B,U,K] of ids [B,K] against union-branch queries qs = [q1 (, q2)], each [B,U,1,D], as the
     custom_cal_logit bodies compute them before their max over dim 1 (box.py:157-164 and siblings), plus the
     gathered (regularized) rows [B,K,row] they were computed from."""
     b, k = ids.shape
     src = orc.regularizer(table) if regularizer else table
     rows = orc.gather(src, ids).reshape(b, k, -1)
-    logit = np.stack([orc.score_forward(model, rows, qs[0][:, j], qs[1][:, j] if len(qs) > 1 else None, gamma, cen)
+    logit = np.stack([orc.score_forward(model, rows, qs[0][:, j], qs[1][:, j] if len(qs) > 1 else None, gamma, cen,
+                                        norm=norm)
                       for j in range(qs[0].shape[1])], axis=1)
     return logit, rows
 
 
-def oracle_union_grads(model, table, ids, qs, rows, logit, gout, cen, regularizer=False):
+def oracle_union_grads(model, table, ids, qs, rows, logit, gout, cen, regularizer=False, norm=False):
     """Backward of sum(gout * max over branches of logit): gradient rows [B*K,row] w.r.t. the table rows of the
     pairs and [d/dq1 (, d/dq2)] shaped like qs.  The first maximal branch takes the gradient, as torch.max does;
     with the regularizer clamp(x + 1, 0.05, 1e9) the row gradient is masked where the clamp is active."""
@@ -117,7 +118,7 @@ def oracle_union_grads(model, table, ids, qs, rows, logit, gout, cen, regularize
     g_qs = [np.zeros_like(q) for q in qs]
     for j in range(logit.shape[1]):
         gj = np.where(win == j, gout, 0.0)
-        gr, g1, g2 = orc.score_backward(model, gj, rows, qs[0][:, j], qs[1][:, j] if len(qs) > 1 else None, cen)
+        gr, g1, g2 = orc.score_backward(model, gj, rows, qs[0][:, j], qs[1][:, j] if len(qs) > 1 else None, cen, norm=norm)
         g_rows += gr
         g_qs[0][:, j] = g1
         if len(qs) > 1:
