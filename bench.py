@@ -657,7 +657,10 @@ def shared_kernels_bench(device, seed, steps, warmup):
         return (time.perf_counter() - t0) * 1e3 / steps
 
     out = {}
-    for model in ("box", "l1", "rotate", "beta_kl", "complex", "distmult"):
+    for label in ("box", "l1", "rotate", "beta_kl", "complex", "complex_norm", "distmult"):
+        # complex_norm: complex with the halves of every entity row at unit length (the 'norm' mode of the
+        # reference's ComplEx scripts)
+        model = "complex" if label == "complex_norm" else label
         mul = 2 if model in ("rotate", "beta_kl", "complex") else 1
         if model == "beta_kl":
             def make(*shape):
@@ -671,9 +674,9 @@ def shared_kernels_bench(device, seed, steps, warmup):
         ids = torch.randint(0, n, (k,), device=device, generator=gen)
         full = ids[None, :].expand(b, k).contiguous()
         gs = torch.randn((b, k), device=device, generator=gen)
-        params = fused.score_params(24.0, 0.02)
+        params = fused.score_params(24.0, 0.02, norm=label == "complex_norm")
         score = fused.score_forward_shared(model, table, ids, q1, q2, params)
-        out[model] = {
+        out[label] = {
             "shared_list": {
                 "forward": timed(lambda: fused.score_forward_shared(model, table, ids, q1, q2, params)),
                 "query_backward": timed(lambda: fused.score_backward_query_shared(model, table, ids, q1, q2, score, gs, params)),

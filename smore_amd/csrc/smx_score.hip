@@ -56,7 +56,7 @@ int shared_gemm_forward(int model, hipStream_t st, const float* table, size_t n_
                         const ScoreParams& p, int* err, float* workspace);
 int shared_gemm_backward_query(int model, hipStream_t st, const float* table, size_t n_rows, const long long* ids,
                                const float* q1, const float* q2, const float* gscore, float* gq1, float* gq2, size_t B,
-                               size_t K, size_t dim, const ScoreParams& p, float* workspace);
+                               size_t K, size_t dim, const ScoreParams& p, float* workspace, size_t workspace_bytes);
 
 // One extra stream and two events per device, created at first use and kept for the life of the process.
 struct SideStream {
@@ -286,7 +286,7 @@ int smx_score_backward_query_shared(int model, void* stream, const float* table,
   if (!score || !gscore || !gq1 || (model_nq(model) == 2 && !gq2)) return fail(SMX_ERR_ARG, "null pointer");
   if (shared_gemm_fits(model, dim, table, q1, q2, workspace, workspace_bytes, B, K, false, A.p.norm_on != 0))
     return shared_gemm_backward_query(model, as_stream(stream), table, n_rows, reinterpret_cast<const long long*>(ids), q1,
-                                      q2, gscore, gq1, gq2, B, K, dim, A.p, static_cast<float*>(workspace));
+                                      q2, gscore, gq1, gq2, B, K, dim, A.p, static_cast<float*>(workspace), workspace_bytes);
   A.ids_shared = 1;
   A.score = score;
   A.gscore = gscore;

@@ -8,7 +8,8 @@ and custom_cal_logit (models/box.py:157-164, vec.py:85-90, rotate.py:137-142, be
     gamma - dist(rows, query)            [box: gamma - box_dist_out(..) - cen * box_dist_in(..)]   then max over dim 1.
 With an EmbeddingOptimizer attached, the lookup returns a `LazyRows` handle instead of a [B*K, row] tensor.
 The handle understands exactly what that call sequence does to it -- `.view`, `.unsqueeze`, `+ base_add`,
-`torch.clamp` -- and the distance operators of smore_amd.torchext.ext_ops, given a handle, return a `LazyLogit`:
+`torch.clamp`, and ComplEx's `torch.chunk(rows, 2, dim=-1)` / `F.normalize` of each half / `torch.cat` of the two
+(models/complex.py:142-146 in its 'norm' mode) -- and the distance operators of smore_amd.torchext.ext_ops, given a handle, return a `LazyLogit`:
 a running affine expression  const + sum coef * dist  that scalar arithmetic extends.  The first operation that
 needs values (torch.max in custom_cal_logit) evaluates the expression; when it has the shape of one of the
 models' logits it becomes ONE launch of the gather-fused scorer (smx_score_forward) on the ids, and its autograd
@@ -24,6 +25,7 @@ import torch
 
 _FUSED_MODEL = {"l1": "l1", "l2": "l2", "rotate": "rotate", "beta_kl": "beta_kl"}   # logit = const - dist
 _FUSED_SIMILARITY = ("complex", "distmult")                                          # logit = const + similarity
+UNIT_HALVES = "unit_halves"     # LazyRows.reg of ComplEx rows whose halves were scaled to unit length
 
 
 def _is_lazy(x):
@@ -168,7 +170,8 @@ class _Delegating:
 
 class LazyRows(_Delegating):
     """rows-of(table, ids): logical shape ids.shape + (row,), optionally viewed / unsqueezed, optionally carrying the
-    entity prologue clamp(rows + add, lo, hi) of smore/common/modules.py:29-36."""
+    entity prologue clamp(rows + add, lo, hi) of smore/common/modules.py:29-36 (reg = (add, lo, hi)) or ComplEx's
+    unit-length halves (reg = UNIT_HALVES)."""
 
     def __init__(self, opt, ids, name, shape=None, reg=None, pending_add=None, root=None):
         self.opt, self.ids, self.name = opt, ids, name
@@ -261,6 +264,13 @@ class LazyRows(_Delegating):
                 out.reg = (x.pending_add or 0.0, lo, hi)
                 out.pending_add = None
                 return out
+        if name == "chunk" and args and isinstance(args[0], LazyRows):
+            x = args[0]
+            chunks = kwargs.get("chunks", args[1] if len(args) > 1 else None)
+            dim = kwargs.get("dim", args[2] if len(args) > 2 else 0)
+            if (chunks == 2 and dim in (-1, x.dim() - 1) and x.dim() == 3 and x.reg is None and
+                    x.pending_add is None and x.shape[-1] % 2 == 0):
+                return _LazyHalf(x, 0), _LazyHalf(x, 1)
         if name in ("add", "__add__", "__radd__") and len(args) == 2 and not kwargs:
             rows, other = (args[0], args[1]) if isinstance(args[0], LazyRows) else (args[1], args[0])
             if isinstance(rows, LazyRows) and _scalar(other) is not None:
@@ -276,9 +286,60 @@ class LazyRows(_Delegating):
         rows = root._looked_up.view(self.shape)
         if self.pending_add is not None:
             rows = rows + self.pending_add
-        if self.reg is not None:
+        if self.reg == UNIT_HALVES:
+            re, im = torch.chunk(rows, 2, dim=-1)
+            norm = torch.nn.functional.normalize
+            rows = torch.cat((norm(re, p=2, dim=-1), norm(im, p=2, dim=-1)), dim=-1)
+        elif self.reg is not None:
             rows = torch.clamp(rows + self.reg[0], self.reg[1], self.reg[2])
         return rows
+
+
+class _LazyHalf(_Delegating):
+    """One of the two halves torch.chunk(rows, 2, dim=-1) returns for a LazyRows handle [Be, K, row], optionally
+    scaled to unit length by F.normalize(half, p=2, dim=-1).  torch.cat of both halves of one handle, in order and
+    both scaled, is that handle again with reg = UNIT_HALVES; of both unscaled, the handle itself."""
+
+    def __init__(self, rows, which, unit=False):
+        self.rows, self.which, self.unit = rows, which, unit
+        self.shape = torch.Size(tuple(rows.shape[:-1]) + (rows.shape[-1] // 2,))
+
+    device = property(lambda self: self.rows.device)
+    dtype = property(lambda self: self.rows.dtype)
+    requires_grad = True
+    is_cuda = True
+
+    def dim(self):
+        return len(self.shape)
+
+    ndim = property(dim)
+
+    def size(self, d=None):
+        return self.shape if d is None else self.shape[d]
+
+    @classmethod
+    def _try_lazy(cls, func, args, kwargs):
+        name = _func_name(func)
+        if name == "normalize" and args and isinstance(args[0], _LazyHalf) and len(args) == 1:
+            x = args[0]
+            if (not x.unit and kwargs.get("p", 2.0) == 2 and kwargs.get("dim", 1) in (-1, x.dim() - 1) and
+                    kwargs.get("eps", 1e-12) == 1e-12 and kwargs.get("out") is None):
+                return _LazyHalf(x.rows, x.which, True)
+        if name == "cat" and args and isinstance(args[0], (tuple, list)) and len(args[0]) == 2:
+            a, b = args[0]
+            dim = kwargs.get("dim", args[1] if len(args) > 1 else 0)
+            if (isinstance(a, _LazyHalf) and isinstance(b, _LazyHalf) and a.rows is b.rows and a.which == 0 and
+                    b.which == 1 and a.unit == b.unit and dim in (-1, a.dim() - 1) and kwargs.get("out") is None):
+                if not a.unit:
+                    return a.rows
+                out = a.rows._like(a.rows.shape)
+                out.reg = UNIT_HALVES
+                return out
+        return NotImplemented
+
+    def materialize(self):
+        half = torch.chunk(self.rows.materialize(), 2, dim=-1)[self.which]
+        return torch.nn.functional.normalize(half, p=2, dim=-1) if self.unit else half
 
 
 class _Dist:

@@ -36,7 +36,10 @@ def _f32(t, name):
 
 def score_params(gamma, cen=0.0, regularizer=None, norm=False):
     """regularizer: None or (base_add, min_val, max_val) as in smore/common/modules.py:29-36.
-    norm (complex): the halves of every entity row at unit length, smore/models/complex.py:142-146."""
+    norm (complex), also spelled regularizer = "unit_halves": the halves of every entity row at unit length,
+    smore/models/complex.py:142-146."""
+    if regularizer == "unit_halves":
+        regularizer, norm = None, True
     if regularizer is None:
         return _lib.ScoreParams(gamma, cen, 0, 0.0, 0.0, 0.0, 1 if norm else 0)
     add, lo, hi = regularizer

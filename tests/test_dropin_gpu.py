@@ -96,6 +96,25 @@ class Complex(Reasoner):                           # complex.py:140-148 without 
         return torch.max(logit, dim=1)[0]
 
 
+class ComplexNorm(Reasoner):       # complex.py:140-148 in its 'norm' mode (complex.py:87-89; Normalizer, modules.py:38-40)
+    need_norm = True
+
+    @staticmethod
+    def embed_norm(embedding):
+        return torch.nn.functional.normalize(embedding, p=2, dim=-1)
+
+    def cal_logit(self, entity_embedding, entity_feat, query_embedding):
+        from smore_amd.torchext.ext_ops import complex_sim
+        assert entity_feat is None
+        query_re_embedding, query_im_embedding = query_embedding
+        if self.need_norm:
+            entity_re_embedding, entity_im_embedding = torch.chunk(entity_embedding, 2, dim=-1)
+            entity_re_embedding, entity_im_embedding = self.embed_norm(entity_re_embedding), self.embed_norm(entity_im_embedding)
+            entity_embedding = torch.cat((entity_re_embedding, entity_im_embedding), dim=-1).contiguous()
+        logit = complex_sim(entity_embedding, query_re_embedding, query_im_embedding)
+        return torch.max(logit, dim=1)[0]
+
+
 class Distmult(Reasoner):
     def cal_logit(self, entity_embedding, entity_feat, query_embedding):
         from smore_amd.torchext.ext_ops import distmult_sim
@@ -113,6 +132,7 @@ CASES = {
     "beta": (Beta, (), "beta_kl", 2, 2, 60.0, 0.0),
     "complex": (Complex, (), "complex", 2, 2, 0.0, 0.0),
     "distmult": (Distmult, (), "distmult", 1, 1, 0.0, 0.0),
+    "complex_norm": (ComplexNorm, (), "complex", 2, 2, 0.0, 0.0),
 }
 
 
@@ -133,11 +153,13 @@ def _table_and_queries(name, n, d, b, u, rng):
 
 
 def _oracle_branch_logits(name, table, ids, qs, gamma, cen):
-    return oracle_union_logits(CASES[name][2], table, ids, qs, gamma, cen, regularizer=name == "beta")
+    return oracle_union_logits(CASES[name][2], table, ids, qs, gamma, cen, regularizer=name == "beta",
+                               norm=name == "complex_norm")
 
 
 def _oracle_grads(name, table, ids, qs, rows, logit, gout, cen):
-    return oracle_union_grads(CASES[name][2], table, ids, qs, rows, logit, gout, cen, regularizer=name == "beta")
+    return oracle_union_grads(CASES[name][2], table, ids, qs, rows, logit, gout, cen, regularizer=name == "beta",
+                              norm=name == "complex_norm")
 
 
 @pytest.mark.parametrize("name", list(CASES))
@@ -278,6 +300,54 @@ def test_shared_negatives_and_other_uses_of_the_rows():
     all_idx = np.concatenate([ids_full.reshape(-1), neg.reshape(-1)])
     uniq, inverse, _, _ = orc.merge_indices(all_idx)
     merged = orc.merge_grads(np.concatenate([g_rows.reshape(b * k, d), g_reg]), inverse, uniq.size)
+    w, m, v = table.copy(), np.zeros_like(table), np.zeros_like(table)
+    orc.adam_rows(w, m, v, uniq, merged, lr, 1)
+    assert_close(emb.state_sum_fo.cpu().numpy()[uniq], m[uniq], REL_F32, "first moment")
+    assert_adam_weights(emb.embedding.detach().cpu().numpy(), w, merged, uniq, lr, "weights")
+
+
+def test_complex_norm_step_with_shared_negatives_stays_fused():
+    """The layout of the reference's ComplEx scripts (complex_scripts/train_*.sh: -complexm '(Mean,True,norm)' with
+    --share_negative): negatives [1,K] and positives [B] through the unchanged custom_cal_logit of the 'norm' mode.
+    No lookup is materialised, the K ids and the B positives meet in one plan, and logits, query gradients and the
+    Adam step are the float64 oracle's."""
+    from smore_amd.embedding.embed_optimizer import AdamEmbedOptimizer
+    from smore_amd.embedding.sparse_embed import SparseEmbedding
+    n, d, b, k, lr = 500, 48, 9, 70, 1e-3
+    rng = np.random.default_rng(77)
+    table, qs = _table_and_queries("complex_norm", n, d, b, 1, rng)
+    emb = SparseEmbedding(n, 2 * d).cuda()
+    with torch.no_grad():
+        emb.embedding.copy_(torch.tensor(table, dtype=torch.float32))
+    opt = AdamEmbedOptimizer(types.SimpleNamespace(optim_mode="(aggr,adam,gpu,False,5)", share_optim_stats=True), emb, 0)
+    net = ComplexNorm(emb, 0.0).cuda()
+    t_qs = [torch.tensor(q, dtype=torch.float32, device="cuda", requires_grad=True) for q in qs]
+    pos = rng.integers(0, n, b)
+    neg = rng.integers(0, n // 4, (1, k))
+    neg[0, 5] = pos[2]                                   # an entity that is a positive and a shared negative at once
+    gp = rng.standard_normal((b, 1)).astype(np.float32).astype(np.float64)
+    gn = rng.standard_normal((b, k)).astype(np.float32).astype(np.float64)
+    opt.zero_grad()
+    lp, ln = net(torch.tensor(pos, device="cuda"), torch.tensor(neg, device="cuda"), t_qs)
+    assert lp.shape == (b, 1) and ln.shape == (b, k)
+    ((lp * torch.tensor(gp, dtype=torch.float32, device="cuda")).sum() +
+     (ln * torch.tensor(gn, dtype=torch.float32, device="cuda")).sum()).backward()
+    assert len(opt.fused_list) == 2 and not opt.grad_list and opt.stats["materialized_lookups"] == 0
+    assert opt.stats["dense_fallbacks"] == 0
+    opt.apply_grad(lr)
+
+    neg_full = np.broadcast_to(neg, (b, k))
+    o_lp, rows_p = _oracle_branch_logits("complex_norm", table, pos.reshape(b, 1), qs, 0.0, 0.0)
+    o_ln, rows_n = _oracle_branch_logits("complex_norm", table, neg_full, qs, 0.0, 0.0)
+    assert_close(lp.detach().cpu().numpy(), o_lp[:, 0], REL_F32, "positive logits")
+    assert_close(ln.detach().cpu().numpy(), o_ln[:, 0], REL_F32, "negative logits")
+    gr_p, gq_p = _oracle_grads("complex_norm", table, pos.reshape(b, 1), qs, rows_p, o_lp, gp, 0.0)
+    gr_n, gq_n = _oracle_grads("complex_norm", table, neg_full, qs, rows_n, o_ln, gn, 0.0)
+    for t, a, c in zip(t_qs, gq_p, gq_n):
+        assert_close(t.grad.cpu().numpy(), a + c, REL_F32, "query gradient")
+    all_idx = np.concatenate([pos.reshape(-1), neg_full.reshape(-1)])
+    uniq, inverse, _, _ = orc.merge_indices(all_idx)
+    merged = orc.merge_grads(np.concatenate([gr_p, gr_n]), inverse, uniq.size)
     w, m, v = table.copy(), np.zeros_like(table), np.zeros_like(table)
     orc.adam_rows(w, m, v, uniq, merged, lr, 1)
     assert_close(emb.state_sum_fo.cpu().numpy()[uniq], m[uniq], REL_F32, "first moment")

@@ -37,7 +37,10 @@ class RecordingOptimizer:
         """[B, U, K] logits, as the real optimizer's launch returns them."""
         self.scored.append((model, tuple(ids.shape), gamma, cen, reg))
         e = self.sparse_embed.embedding[ids]
-        if reg is not None:
+        if reg == "unit_halves":
+            re, im = torch.chunk(e, 2, dim=-1)
+            e = torch.cat((re / re.norm(dim=-1, keepdim=True), im / im.norm(dim=-1, keepdim=True)), dim=-1)
+        elif reg is not None:
             e = torch.clamp(e + reg[0], reg[1], reg[2])
         if q1.dim() == 3:
             q1, q2 = q1.unsqueeze(1), None if q2 is None else q2.unsqueeze(1)
@@ -59,6 +62,9 @@ def _textbook(model, e, queries, cen):
     if model == "rotate":
         re, im = torch.chunk(e, 2, dim=-1)
         return torch.sqrt((re - queries[0]) ** 2 + (im - queries[1]) ** 2).sum(-1)
+    if model == "complex":
+        re, im = torch.chunk(e, 2, dim=-1)
+        return (re * queries[0] + im * queries[1]).sum(-1)
     raise AssertionError(model)
 
 
@@ -126,6 +132,73 @@ def test_regularizer_becomes_the_prologue_only_for_beta():
     opt1 = RecordingOptimizer(n, d)
     r1 = torch.clamp(LazyRows(opt1, ids, None).view(b, k, -1) + 1.0, 0.05, 1e9)
     assert isinstance(ext_ops.l1_dist(r1, _queries(b, 1, d, 1, 6)[0]), LazyLogit)
+
+
+class _Normalizer:                  # common/modules.py:38-40
+    def __call__(self, embedding):
+        return torch.nn.functional.normalize(embedding, p=2, dim=-1)
+
+
+def _complex_logit(embed_norm, entity_embedding, query_embedding):
+    """custom_cal_logit of models/complex.py:140-148 in its 'norm' mode."""
+    query_re_embedding, query_im_embedding = query_embedding
+    entity_re_embedding, entity_im_embedding = torch.chunk(entity_embedding, 2, dim=-1)
+    entity_re_embedding, entity_im_embedding = embed_norm(entity_re_embedding), embed_norm(entity_im_embedding)
+    entity_embedding = torch.cat((entity_re_embedding, entity_im_embedding), dim=-1).contiguous()
+    logit = ext_ops.complex_sim(entity_embedding, query_re_embedding, query_im_embedding)
+    return entity_embedding, torch.max(logit, dim=1)[0]
+
+
+@pytest.mark.parametrize("branches", [1, 2])
+def test_unit_length_halves_of_complex_stay_on_the_handle(branches):
+    """chunk / F.normalize / cat of models/complex.py:142-146: the rows are never looked up, the scorer gets ONE
+    request for the complex model with the unit-length option, and the value is that of the torch expression."""
+    n, d, b, k = 40, 6, 3, 5
+    opt = RecordingOptimizer(n, 2 * d)
+    ids = torch.randint(0, n, (b * k,), generator=torch.Generator().manual_seed(9))
+    qs = _queries(b, branches, d, 2, 12)
+    handle = LazyRows(opt, ids, "negative_entity").view(b, k, -1)
+    ent, logit = _complex_logit(_Normalizer(), handle, qs)
+    assert isinstance(ent, LazyRows) and ent.reg == "unit_halves"
+    rows = opt.sparse_embed.embedding[ids].view(b, k, -1)
+    F = torch.nn.functional
+    re, im = torch.chunk(rows, 2, dim=-1)
+    want = torch.max((F.normalize(re, p=2, dim=-1).unsqueeze(1) * qs[0] + F.normalize(im, p=2, dim=-1).unsqueeze(1) * qs[1]).sum(-1), dim=1)[0]
+    torch.testing.assert_close(logit + 0.0, want, rtol=1e-6, atol=1e-6)       # (the first use scores the placeholder)
+    assert opt.looked_up == [] and opt.scored == [("complex", (b, k), 0.0, 0.0, "unit_halves")]
+    # the values the handle stands for, when something else asks for them
+    assert torch.equal(ent.materialize(), torch.cat((F.normalize(re, p=2, dim=-1), F.normalize(im, p=2, dim=-1)), dim=-1))
+
+
+def test_halves_put_to_any_other_use_become_tensors():
+    n, d, b, k = 40, 6, 3, 5
+    F = torch.nn.functional
+    ids = torch.randint(0, n, (b * k,), generator=torch.Generator().manual_seed(10))
+    opt = RecordingOptimizer(n, 2 * d)
+    rows = opt.sparse_embed.embedding[ids].view(b, k, -1)
+    re, im = torch.chunk(rows, 2, dim=-1)
+    handle = LazyRows(opt, ids, None).view(b, k, -1)
+    h_re, h_im = torch.chunk(handle, 2, dim=-1)
+    assert h_re.shape == re.shape and h_im.dim() == 3 and opt.looked_up == []
+    # Identity in the place of the normalizer (complex.py:91): the two halves put together are the handle again
+    assert torch.cat((h_re, h_im), dim=-1) is handle
+    # the halves the other way round, another norm, another axis, one half alone, arithmetic: the tensor's results
+    assert torch.equal(torch.cat((h_im, h_re), dim=-1), torch.cat((im, re), dim=-1))
+    assert torch.equal(F.normalize(h_re, p=1, dim=-1), F.normalize(re, p=1, dim=-1))
+    assert torch.equal(F.normalize(h_re, p=2, dim=1), F.normalize(re, p=2, dim=1))
+    assert torch.equal(torch.cat((F.normalize(h_re, p=2, dim=-1), h_im), dim=-1), torch.cat((F.normalize(re, p=2, dim=-1), im), dim=-1))
+    assert torch.equal(F.normalize(h_im, p=2, dim=-1) * 2.0, F.normalize(im, p=2, dim=-1) * 2.0)
+    assert torch.equal(h_re + 1.0, re + 1.0) and torch.equal(h_im[0], im[0])
+    assert len(opt.looked_up) == 1, "one lookup per handle family"
+    # three chunks, or chunks along another axis, are no halves
+    three = torch.chunk(LazyRows(opt, ids, None).view(b, k, -1), 3, dim=-1)
+    assert all(isinstance(t, torch.Tensor) for t in three) and torch.equal(three[1], torch.chunk(rows, 3, dim=-1)[1])
+    # unit-length halves under a model that has no such form: dense route, right values
+    ent = torch.cat((F.normalize(h_re, p=2, dim=-1), F.normalize(h_im, p=2, dim=-1)), dim=-1)
+    q = _queries(b, 1, 2 * d, 1, 3)[0]
+    lazy = 12.0 - ext_ops.l1_dist(ent, q)
+    assert lazy._fusable() == ("l1", 0.0)      # the expression has the model's form; the request is what is refused:
+    assert opt.lazy_request("l1", ent, (q,), 12.0, 0.0) is None and opt.score_lazy("l1", ent, (q,), 12.0, 0.0) is None
 
 
 def test_other_uses_fall_back_to_one_lookup():
