@@ -405,6 +405,14 @@ __global__ __launch_bounds__(256) void list_rows_kernel(const float* __restrict_
 }
 
 // ---- host side ----------------------------------------------------------------------------------------------
+// out [K][width] = table rows ids[k], width a multiple of four floats, everything 16-byte aligned
+int shared_list_rows(hipStream_t st, const float* table, size_t n_rows, const long long* ids, size_t K, size_t width,
+                     float* out) {
+  hipLaunchKernelGGL(list_rows_kernel<false>, dim3((unsigned)((K + 3) / 4)), dim3(256), 0, st, table, ids, (int)K, 0,
+                     (int)width, (unsigned long long)n_rows, out, nullptr);
+  return check_launch("rows of the shared list, side by side");
+}
+
 static bool is_inner(int model) { return model == mComplex || model == mDistmult; }
 
 // floats of workspace a call of the model needs: forward / query backward, and the entity side

@@ -129,6 +129,42 @@ def test_shared_negatives_match_oracle_and_the_per_query_kernels(model, n, b, k,
     assert err.item() == 0
 
 
+@pytest.mark.parametrize("model", ["box", "l1", "l2", "rotate"])
+def test_query_backward_of_a_list_scattered_over_a_table_of_many_gigabytes(model):
+    """From 8 GiB of table on, the query backward of the distance models first copies the list's K rows side by side
+    (each query's workgroup reads all of them; scattered over that much memory every read is a page of its own).
+    Same bits as the kernel reading the table, and the float64 oracle's gradient."""
+    import gc
+    from smore_amd import fused
+    mul = 2 if model == "rotate" else 1
+    b, k, dim = 40, 200, 200
+    n = ((8 << 30) // (mul * dim * 4)) + 1000
+    rng = np.random.default_rng(seed("far apart", model))
+    ids = rng.choice(n, k, replace=False)
+    ids[7] = ids[3]
+    rows, q1, q2, _, gs = make_problem(model, k, b, k, dim, rng)      # rows [k, row]: row j of the list
+    rows[7] = rows[3]
+    table = torch.empty((n, mul * dim), device="cuda")               # only the list's rows are ever read
+    t_ids = torch.tensor(ids, device="cuda")
+    table[t_ids] = dev(rows)
+    t_q1, t_q2, t_gs = dev(q1), dev(q2), dev(gs)
+    params = fused.score_params(GAMMA[model], 0.02)
+    score = fused.score_forward_shared(model, table, t_ids, t_q1, t_q2, params)
+    g1, g2 = fused.score_backward_query_shared(model, table, t_ids, t_q1, t_q2, score, t_gs, params)
+    p1, p2 = fused.score_backward_query_shared(model, table, t_ids, t_q1, t_q2, score, t_gs, params, per_row_terms=False)
+    assert torch.equal(g1, p1) and (g2 is None or torch.equal(g2, p2))
+    o_rows = np.broadcast_to(rows[None], (b, k, rows.shape[1]))
+    o_q1, o_q2 = q1[:, None, :], None if q2 is None else q2[:, None, :]
+    _, w1, w2 = orc.score_backward(model, gs, o_rows, o_q1, o_q2, 0.02)
+    q_abs = np.abs(gs).sum(axis=1)[:, None] * np.ones((1, dim))
+    assert_close(g1.cpu().numpy(), w1[:, 0], REL_F32, f"{model} gq1, list copied side by side", sum_abs=q_abs)
+    if q2 is not None:
+        assert_close(g2.cpu().numpy(), w2[:, 0], REL_F32, f"{model} gq2, list copied side by side", sum_abs=q_abs)
+    del table
+    gc.collect()
+    torch.cuda.empty_cache()
+
+
 @pytest.mark.parametrize("model,dim", [("box", 400), ("rotate", 100), ("beta_kl", 64), ("l2", 30)])
 def test_an_id_outside_the_table_in_the_shared_list_is_flagged_and_scored_as_row_0(model, dim):
     """Every scorer of the library reads row 0 for an id outside [0, n) and raises the caller's flag
