@@ -117,7 +117,7 @@ typedef struct smx_score_params {
   float reg_hi;
   int norm_on;   /* COMPLEX: each half of an entity row (re, im) is scaled to unit L2 length before it is scored
                   * (complex.py:142-146 with the 'norm' mode of complex.py:87-89: F.normalize, eps 1e-12), and the
-                  * entity gradient is taken through that scaling.  The ranking calls refuse it (SMX_ERR_ARG). */
+                  * entity gradient is taken through that scaling. */
 } smx_score_params;
 
 /* Sign codes (optional, what autograd would call a saved tensor).  For the box model (and, with one
@@ -370,7 +370,12 @@ int smx_rows_backward(void* stream, const smx_plan_view* plan, const float* grad
  *                   that holds an id twice sums both positions): merged[u,:] and / or the optimizer update of
  *                   table, m, v in place, as smx_score_backward_entity.
  * workspace of the three calls (may be NULL): smx_shared_workspace_bytes(model, B, K, dim)
- * bytes, 16-byte aligned; 0 for every model but BETA_KL.  Given it (and rows of 16-byte aligned floats, dim a
+ * bytes, 16-byte aligned.  Every model: room for the list's K rows side by side -- the query backward copies them
+ * there first when the table spans 8 GiB or more (every query's workgroup reads all K rows; out of that much memory
+ * each read is a page of its own), and always for the matrix products of COMPLEX and DISTMULT, whose entity side
+ * also keeps its sums [K, n_q dim] there; COMPLEX with norm_on: the K rows scaled to unit-length halves as the
+ * products' operand (without workspace the per-pair kernels run).
+ * BETA_KL: given it (and rows of 16-byte aligned floats, dim a
  * multiple of 4), BetaE's entity-side terms -- three digammas and a log-beta per feature, dist_kernel.h:212-221 --
  * are evaluated once per shared row into the workspace instead of once per pair, and the pairs are a matrix product
  * on them (fp32 matrix instructions, fixed summation order); without it the per-pair kernels run (same results to

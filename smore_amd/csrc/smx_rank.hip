@@ -29,7 +29,6 @@ static int rank_common(RankArgs* R, int* vec, int* nit, int model, const float* 
   if (A > kRankMaxAnswers) return fail(SMX_ERR_SHAPE, "at most %zu answers per query", kRankMaxAnswers);
   if (B > 0x7fffffffull / (A + 1)) return fail(SMX_ERR_SHAPE, "too many queries");
   if (const char* why = params_refused(model, params)) return fail(SMX_ERR_ARG, "%s", why);
-  if (params->norm_on) return fail(SMX_ERR_ARG, "the ranking kernels have no unit-length form of the complex model");
   const bool vec4 = dim % 4 == 0 && aligned16(table) && aligned16(q1) && (model_nq(model) == 1 || aligned16(q2));
   *vec = vec4 ? 4 : 1;
   const size_t ncol = dim / *vec;

@@ -84,6 +84,35 @@ __device__ __forceinline__ float row_score(const float (&e1)[NIT][VEC], const fl
   return ModelOps<M>::score(wave_sum_last_f32(mine), p);
 }
 
+// ComplEx with unit-length halves (REG stands for it there): the row's halves scaled in the lanes' registers, once
+// per row however many queries score it.
+template <int M, int VEC, int NIT, bool REG>
+__device__ __forceinline__ void unit_row(float (&e1)[NIT][VEC], float (&e2)[NIT][VEC], int ncol, int lane) {
+  if constexpr (model_norm(M, REG)) {
+    float s1 = 0.f, s2 = 0.f;
+#pragma unroll
+    for (int it = 0; it < NIT; ++it) {
+      float a = 0.f, b = 0.f;
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) {
+        a = __builtin_fmaf(e1[it][v], e1[it][v], a);
+        b = __builtin_fmaf(e2[it][v], e2[it][v], b);
+      }
+      const bool in = lane + 64 * it < ncol;
+      s1 += in ? a : 0.f;
+      s2 += in ? b : 0.f;
+    }
+    const float i1 = inv_norm(wave_sum_f32(s1)), i2 = inv_norm(wave_sum_f32(s2));
+#pragma unroll
+    for (int it = 0; it < NIT; ++it)
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) {
+        e1[it][v] *= i1;
+        e2[it][v] *= i2;
+      }
+  }
+}
+
 // STREAM: the row is read once in a pass over the whole table (non-temporal load).
 template <int VEC, int NIT, int MUL, bool STREAM = false>
 __device__ __forceinline__ void load_entity(const float* __restrict__ row, int dim, int ncol, int lane,
@@ -139,6 +168,7 @@ __global__ __launch_bounds__(256) void rank_answer_keys_kernel(RankArgs A) {
   typename ModelOps<M>::Q q[NIT][VEC];
   float e1[NIT][VEC], e2[NIT][VEC];
   load_entity<VEC, NIT, MUL>(A.table + id * (size_t)dim * MUL, dim, A.ncol, lane, e1, e2);
+  unit_row<M, VEC, NIT, REG>(e1, e2, A.ncol, lane);
   float s = 0.f;
   for (int u = 0; u < A.U; ++u) {  // uniform
     load_rank_query<M, VEC, NIT>(A.q1, A.q2, b * A.U + u, dim, A.ncol, lane, q);
@@ -222,14 +252,23 @@ __global__ __launch_bounds__(256) void rank_scan_kernel(RankArgs A) {
 #pragma unroll
     for (int r = 0; r < RIF; ++r) {
       const unsigned id = g * RIF + r;  // entity id of the row
+      float u1[NIT][VEC], u2[NIT][VEC];  // (the row itself unless the model scales it)
+#pragma unroll
+      for (int it = 0; it < NIT; ++it)
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) {
+          u1[it][v] = x1[r][it][v];
+          u2[it][v] = MUL == 2 ? x2[r][it][v] : 0.f;
+        }
+      unit_row<M, VEC, NIT, REG>(u1, u2, A.ncol, lane);
 #pragma unroll
       for (int x = 0; x < NL; ++x) {
-        const float s = row_score<M, VEC, NIT, REG>(x1[r], x2[r], q[x], A.ncol, lane, A.p);
+        const float s = row_score<M, VEC, NIT, REG>(u1, u2, q[x], A.ncol, lane, A.p);
         float su = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(s), 63));
         if constexpr (UNION) {
 #pragma unroll
           for (int u = 1; u < NB; ++u) {
-            const float t = row_score<M, VEC, NIT, REG>(x1[r], x2[r], q[u], A.ncol, lane, A.p);
+            const float t = row_score<M, VEC, NIT, REG>(u1, u2, q[u], A.ncol, lane, A.p);
             const float tu = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(t), 63));
             if (union_takes(tu, su)) su = tu;
           }
@@ -311,6 +350,7 @@ __global__ __launch_bounds__(kCandThreads) void rank_candidates_kernel(RankArgs 
     }
     float e1[NIT][VEC], e2[NIT][VEC];
     load_entity<VEC, NIT, MUL>(A.table + id * (size_t)dim * MUL, dim, A.ncol, lane, e1, e2);
+    unit_row<M, VEC, NIT, REG>(e1, e2, A.ncol, lane);
     float s = row_score<M, VEC, NIT, REG>(e1, e2, q, A.ncol, lane, A.p);
     for (int u = 1; u < A.U; ++u) {  // uniform: the other branches of a union query, fetched again per candidate
       typename ModelOps<M>::Q qu[NIT][VEC];
@@ -442,8 +482,8 @@ int launch_rank_reg(hipStream_t st, RankArgs A, int mode) {
 
 template <int M, int VEC, int NIT>
 int launch_rank(hipStream_t st, const RankArgs& A, int mode) {
-  if constexpr (M == mBetaKL) {
-    if (A.p.reg_on) return launch_rank_reg<M, VEC, NIT, true>(st, A, mode);
+  if constexpr (M == mBetaKL || M == mComplex) {
+    if (M == mBetaKL ? A.p.reg_on : A.p.norm_on) return launch_rank_reg<M, VEC, NIT, true>(st, A, mode);
   }
   return launch_rank_reg<M, VEC, NIT, false>(st, A, mode);
 }

@@ -66,15 +66,16 @@ def test_host_only_entry_points():
 
 
 def test_workspace_sizes_of_the_shared_negative_calls():
-    """smx_shared_workspace_bytes (host only): nothing for the distance models; the matrix-product models need the
-    entity side's sums [K, n_q dim], BetaE also its per-row terms [K, 2 dim + 1] and per-query terms [B]."""
+    """smx_shared_workspace_bytes (host only): the list's rows side by side [K, row] for every model (the query
+    backward's copy; the same size as the entity side's sums [K, n_q dim] of the matrix-product models and as
+    ComplEx's unit-length rows); BetaE its per-row terms [K, 2 dim + 1] and per-query terms [B]."""
     from smore_amd import _lib
     from smore_amd.fused import MODELS
     lib = _lib.load()
     b, k, d = 512, 1024, 400
     up = lambda n: (4 * n + 255) // 256 * 256
-    for model in ("l1", "l2", "box", "rotate"):
-        assert lib.smx_shared_workspace_bytes(MODELS[model], b, k, d) == 0
+    for model, mul in (("l1", 1), ("l2", 1), ("box", 1), ("rotate", 2)):
+        assert lib.smx_shared_workspace_bytes(MODELS[model], b, k, d) == up(k * mul * d)
     assert lib.smx_shared_workspace_bytes(MODELS["distmult"], b, k, d) == up(k * d)
     assert lib.smx_shared_workspace_bytes(MODELS["complex"], b, k, d) == up(k * 2 * d)
     assert lib.smx_shared_workspace_bytes(MODELS["beta_kl"], b, k, d) == up(k * (2 * d + 1) + b)
@@ -120,8 +121,8 @@ def test_scorer_refuses_tables_whose_ids_need_more_than_32_bits():
 
 
 def test_entity_side_options_are_refused_where_a_model_has_none():
-    """The clamp prologue belongs to beta_kl and unit-length row halves to complex (complex.py:142-146); the ranking
-    scans have no unit-length form.  All of it is decided on the host, before any launch."""
+    """The clamp prologue belongs to beta_kl and unit-length row halves to complex (complex.py:142-146); decided
+    on the host, before any launch."""
     from smore_amd import _lib
     import ctypes as c
     lib = _lib.load()
@@ -130,9 +131,9 @@ def test_entity_side_options_are_refused_where_a_model_has_none():
                                                       c.byref(params), None, None, 0)
     assert fwd(2, _lib.ScoreParams(24.0, 0.02, 0, 0.0, 0.0, 0.0, 1)) != 0 and b"complex model only" in lib.smx_last_error()
     assert fwd(5, _lib.ScoreParams(0.0, 0.0, 1, 1.0, 0.05, 1e9, 0)) != 0 and b"beta_kl model only" in lib.smx_last_error()
-    params = _lib.ScoreParams(0.0, 0.0, 0, 0.0, 0.0, 0.0, 1)
-    rc = lib.smx_rank_answer_keys(5, None, fake, 100, fake, fake, 2, 8, c.byref(params), fake, fake, 4, fake, fake)
-    assert rc != 0 and b"unit-length" in lib.smx_last_error()
+    params = _lib.ScoreParams(24.0, 0.02, 0, 0.0, 0.0, 0.0, 1)
+    rc = lib.smx_rank_answer_keys(2, None, fake, 100, fake, fake, 2, 8, c.byref(params), fake, fake, 4, fake, fake)
+    assert rc != 0 and b"complex model only" in lib.smx_last_error()
     assert c.sizeof(_lib.ScoreParams) == 28      # seven four-byte fields, as the header declares them
 
 

@@ -10,11 +10,16 @@ from tests.util import REL_F32, assert_close
 pytestmark = pytest.mark.gpu
 
 
-def _scores64(model, table, q1, q2, cen):
+def _alias(model):
+    """complex_norm: the complex model with the halves of every entity row at unit length (complex.py:142-146)"""
+    return ("complex", True) if model == "complex_norm" else (model, False)
+
+
+def _scores64(model, table, q1, q2, cen, norm=False):
     """float64 logits of every entity for every query, [B, N]"""
     b = q1.shape[0]
     rows = np.broadcast_to(table[None], (b,) + table.shape)
-    return orc.score_forward(model, rows, q1[:, None], None if q2 is None else q2[:, None], GAMMA[model], cen)
+    return orc.score_forward(model, rows, q1[:, None], None if q2 is None else q2[:, None], GAMMA[model], cen, norm=norm)
 
 
 def test_integer_valued_l1_ranks_are_exact_ties_included():
@@ -40,7 +45,7 @@ def test_integer_valued_l1_ranks_are_exact_ties_included():
 
 
 @pytest.mark.parametrize("model,dim", [("box", 200), ("l2", 64), ("rotate", 100), ("beta_kl", 40), ("box", 30), ("complex", 48),
-                                       ("distmult", 64), ("beta_kl", 30)])
+                                       ("distmult", 64), ("beta_kl", 30), ("complex_norm", 48), ("complex_norm", 200)])
 def test_ranks_lie_in_the_interval_fp32_allows(model, dim):
     """Random floats: an entity whose logit is within fp32 error of an answer's may fall on either side;
     every rank must lie between the counts with the tolerance subtracted and added."""
@@ -48,15 +53,16 @@ def test_ranks_lie_in_the_interval_fp32_allows(model, dim):
     from smore_amd.evaluation import filtered_ranks, ranking_metrics
     rng = np.random.default_rng(dim)
     n, b = 20000, 5
+    model, norm = _alias(model)
     table, q1, q2, _, _ = make_problem(model, n, b, 1, dim, rng)
     easy = [rng.choice(n, size=s, replace=False).tolist() for s in (0, 3, 10, 1, 64)]
     hard = []
     for e, s in zip(easy, (1, 5, 70, 0, 130)):
         pool = np.setdiff1d(np.arange(n), np.array(e, dtype=np.int64))
         hard.append(rng.choice(pool, size=s, replace=False).tolist())
-    params = fused.score_params(GAMMA[model], 0.02)
+    params = fused.score_params(GAMMA[model], 0.02, norm=norm)
     got = filtered_ranks(model, dev(table), dev(q1), dev(q2), params, easy, hard)
-    scores = _scores64(model, table, q1, q2, 0.02)
+    scores = _scores64(model, table, q1, q2, 0.02, norm)
     for i in range(b):
         is_ans = np.zeros(n, bool)
         is_ans[easy[i] + hard[i]] = True
@@ -128,7 +134,8 @@ def test_ranking_argument_errors():
         filtered_ranks("l1", torch.zeros(4000, 8, device="cuda"), q, None, p, [[]], [list(range(2049))])
 
 
-@pytest.mark.parametrize("model,dim", [("box", 64), ("rotate", 40), ("beta_kl", 36), ("l2", 200), ("distmult", 30)])
+@pytest.mark.parametrize("model,dim", [("box", 64), ("rotate", 40), ("beta_kl", 36), ("l2", 200), ("distmult", 30),
+                                       ("complex_norm", 52)])
 def test_sampled_candidates_follow_the_reference_recipe(model, dim):
     """The sampled-negatives branch of test_step_mp (train_process.py:118-128, 141-147): -1 padding scored as entity
     0 with the -1e6 bias, ranking among the candidates, filtered ranks of the leading hard answers.  The logits
@@ -139,6 +146,7 @@ def test_sampled_candidates_follow_the_reference_recipe(model, dim):
     from tests.test_fused_gpu import GAMMA, make_problem
     rng = np.random.default_rng(dim)
     n, b, c = 500, 5, 333
+    model, norm = _alias(model)
     table, q1, q2, _, _ = make_problem(model, n, b, 1, dim, rng)
     neg = rng.integers(0, n, (b, c)).astype(np.int64)
     neg[0, 100:] = -1
@@ -146,13 +154,13 @@ def test_sampled_candidates_follow_the_reference_recipe(model, dim):
     neg[2, 7] = neg[2, 3]
     n_hard = np.array([4, 1, 9, 0, 333], dtype=np.int32)
     dev = lambda a: None if a is None else torch.tensor(a, dtype=torch.float32, device="cuda")
-    params = fused.score_params(GAMMA[model], 0.02)
+    params = fused.score_params(GAMMA[model], 0.02, norm=norm)
     err = fused.new_error_flag("cuda")
     logit, ranking, hard = candidate_ranks(model, dev(table), dev(q1), dev(q2), params, torch.tensor(neg, device="cuda"),
                                            n_hard, err)
     assert err.item() == 0
     rows = table[np.where(neg == -1, 0, neg)]
-    want = orc.score_forward(model, rows, q1[:, None], None if q2 is None else q2[:, None], GAMMA[model], 0.02)
+    want = orc.score_forward(model, rows, q1[:, None], None if q2 is None else q2[:, None], GAMMA[model], 0.02, norm=norm)
     want = want + np.where(neg == -1, -1e6, 0.0)
     assert_close(logit.cpu().numpy(), want, REL_F32, f"{model} candidate logits")
     got_logit = logit.cpu().numpy()
@@ -169,10 +177,10 @@ def test_sampled_candidates_follow_the_reference_recipe(model, dim):
     assert err.item() == 1
 
 
-def _union_scores64(model, table, q1, q2, cen, u):
+def _union_scores64(model, table, q1, q2, cen, u, norm=False):
     """float64 logits of union queries: q1 / q2 [B, U, dim], the maximum over the branches (box.py:163), [B, N]"""
     b = q1.shape[0]
-    per = [_scores64(model, table, q1[:, j], None if q2 is None else q2[:, j], cen) for j in range(u)]
+    per = [_scores64(model, table, q1[:, j], None if q2 is None else q2[:, j], cen, norm) for j in range(u)]
     return np.max(np.stack(per, axis=1), axis=1).reshape(b, -1)
 
 
@@ -204,7 +212,7 @@ def test_union_queries_rank_exactly_by_the_maximum_over_branches(u):
 
 
 @pytest.mark.parametrize("model,dim,u", [("box", 200, 2), ("rotate", 100, 2), ("beta_kl", 40, 2), ("l2", 64, 3), ("distmult", 64, 4),
-                                         ("box", 400, 2), ("l1", 30, 3)])
+                                         ("box", 400, 2), ("l1", 30, 3), ("complex_norm", 48, 2), ("complex_norm", 100, 3)])
 def test_union_ranks_lie_in_the_interval_fp32_allows(model, dim, u):
     """Random floats, union queries: every rank between the counts with the fp32 tolerance subtracted and added;
     the answers' logits against the float64 maximum over the branches."""
@@ -212,6 +220,7 @@ def test_union_ranks_lie_in_the_interval_fp32_allows(model, dim, u):
     from smore_amd.evaluation import filtered_ranks
     rng = np.random.default_rng(dim + u)
     n, b = 6000, 3
+    model, norm = _alias(model)
     table, q1, q2, _, _ = make_problem(model, n, b * u, 1, dim, rng)
     q1 = q1.reshape(b, u, dim)
     q2 = None if q2 is None else q2.reshape(b, u, dim)
@@ -220,9 +229,9 @@ def test_union_ranks_lie_in_the_interval_fp32_allows(model, dim, u):
     for e, s in zip(easy, (1, 5, 70)):
         pool = np.setdiff1d(np.arange(n), np.array(e, dtype=np.int64))
         hard.append(rng.choice(pool, size=s, replace=False).tolist())
-    params = fused.score_params(GAMMA[model], 0.02)
+    params = fused.score_params(GAMMA[model], 0.02, norm=norm)
     got = filtered_ranks(model, dev(table), dev(q1), dev(q2), params, easy, hard, branches=u)
-    scores = _union_scores64(model, table, q1, q2, 0.02, u)
+    scores = _union_scores64(model, table, q1, q2, 0.02, u, norm)
     for i in range(b):
         is_ans = np.zeros(n, bool)
         is_ans[easy[i] + hard[i]] = True
