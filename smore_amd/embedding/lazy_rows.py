@@ -16,6 +16,15 @@ models' logits it becomes ONE launch of the gather-fused scorer (smx_score_forwa
 node hands the entity gradient to the optimizer's fused entity pass.  Anything else -- an expression the fused
 scorer has no model for, or any other use of the rows (cal_reg, indexing, printing) -- falls back to the plain
 lookup (EmbedLookupFunc) and the dense operators, with the reference's results.
+
+The native_cal_logit bodies (--logit_impl native, the default: config.py:119) write the same logits with torch
+operators on the rows: box.py:147-155, vec.py:78-83, rotate.py:125-135, distmult.py:126-133, and the per-query
+branch of complex.py:169-177.  Their intermediates on a handle are
+`_LazyExpr` nodes (rows.unsqueeze(1) - center, its abs, relu(abs - offset), min(abs, offset), the stacked halves'
+modulus, the products with the queries); torch.norm(.., p=1, dim=-1) or .sum(dim=-1) of the right node is the same
+`LazyLogit` term the ext_ops call would have returned.  The fused scorer then computes them with ITS conventions where the two forms differ on a
+set of measure zero: the subgradients at |e - c| = 0 and = offset are those of the CUDA functors
+(dist_kernel.h:141), not autograd's of abs / relu / min, and RotatE's modulus carries the functor's 1e-20.
 """
 import numbers
 import weakref
@@ -251,9 +260,25 @@ class LazyRows(_Delegating):
 
     __radd__ = __add__
 
+    def __sub__(self, other):          # rows.unsqueeze(1) - center of the native_cal_logit bodies
+        node = _LazyExpr.delta(self, other)
+        return torch.sub(self.materialize(), _resolve(other)) if node is None else node
+
+    def __mul__(self, other):          # query * rows.unsqueeze(1), distmult.py:131
+        node = _LazyExpr.prod(self, other)
+        return torch.mul(self.materialize(), _resolve(other)) if node is None else node
+
+    __rmul__ = __mul__
+
     @classmethod
     def _try_lazy(cls, func, args, kwargs):
         name = _func_name(func)
+        if name in ("mul", "multiply", "__mul__", "__rmul__") and len(args) == 2 and not kwargs:
+            rows, other = (args[0], args[1]) if isinstance(args[0], LazyRows) else (args[1], args[0])
+            if isinstance(rows, LazyRows):
+                node = _LazyExpr.prod(rows, other)
+                if node is not None:
+                    return node
         if name == "clamp" and args and isinstance(args[0], LazyRows):
             x = args[0]
             lo = kwargs.get("min", args[1] if len(args) > 1 else None)
@@ -268,8 +293,8 @@ class LazyRows(_Delegating):
             x = args[0]
             chunks = kwargs.get("chunks", args[1] if len(args) > 1 else None)
             dim = kwargs.get("dim", args[2] if len(args) > 2 else 0)
-            if (chunks == 2 and dim in (-1, x.dim() - 1) and x.dim() == 3 and x.reg is None and
-                    x.pending_add is None and x.shape[-1] % 2 == 0):
+            if (chunks == 2 and dim in (-1, x.dim() - 1) and (x.dim() == 3 or (x.dim() == 4 and x.shape[1] == 1)) and
+                    x.reg is None and x.pending_add is None and x.shape[-1] % 2 == 0):
                 return _LazyHalf(x, 0), _LazyHalf(x, 1)
         if name in ("add", "__add__", "__radd__") and len(args) == 2 and not kwargs:
             rows, other = (args[0], args[1]) if isinstance(args[0], LazyRows) else (args[1], args[0])
@@ -325,6 +350,12 @@ class _LazyHalf(_Delegating):
             if (not x.unit and kwargs.get("p", 2.0) == 2 and kwargs.get("dim", 1) in (-1, x.dim() - 1) and
                     kwargs.get("eps", 1e-12) == 1e-12 and kwargs.get("out") is None):
                 return _LazyHalf(x.rows, x.which, True)
+        if name in ("mul", "multiply", "__mul__", "__rmul__") and len(args) == 2 and not kwargs:
+            half, other = (args[0], args[1]) if isinstance(args[0], _LazyHalf) else (args[1], args[0])
+            if isinstance(half, _LazyHalf):
+                node = _LazyExpr.prod(half, other)
+                if node is not None:
+                    return node
         if name == "cat" and args and isinstance(args[0], (tuple, list)) and len(args[0]) == 2:
             a, b = args[0]
             dim = kwargs.get("dim", args[1] if len(args) > 1 else 0)
@@ -337,9 +368,177 @@ class _LazyHalf(_Delegating):
                 return out
         return NotImplemented
 
+    def __sub__(self, other):          # entity_re_embedding - query_re_embedding of rotate.py:129-130
+        node = _LazyExpr.delta(self, other)
+        return torch.sub(self.materialize(), _resolve(other)) if node is None else node
+
+    def __mul__(self, other):          # entity_re_embedding * query_re_embedding of complex.py:176
+        node = _LazyExpr.prod(self, other)
+        return torch.mul(self.materialize(), _resolve(other)) if node is None else node
+
+    __rmul__ = __mul__
+
     def materialize(self):
         half = torch.chunk(self.rows.materialize(), 2, dim=-1)[self.which]
         return torch.nn.functional.normalize(half, p=2, dim=-1) if self.unit else half
+
+
+class _LazyExpr(_Delegating):
+    """An intermediate of a native_cal_logit body on a handle: `op` applied to rows [Be, 1, K, w] (a 4-D handle, or
+    one half of it) and the query tensors [B, U, 1, w] in `queries`; logical shape [B, U, K, w].
+      delta     rows - c                      box.py:150, vec.py:80, rotate.py:129-130 (half = 0 / 1)
+      absdelta  |rows - c|                    box.py:150
+      excess    |rows - c| - o                box.py:151
+      box_out   relu(|rows - c| - o)          box.py:151
+      box_in    min(|rows - c|, o)            box.py:152
+      stack     stack([re - q_re, im - q_im], dim=0)     rotate.py:131
+      modulus   its norm over dim 0                      rotate.py:132
+      prod      rows * q                      distmult.py:131; one half (possibly at unit length): complex.py:176
+      cprod     re * q_re + im * q_im         complex.py:176
+    The value, if something else asks for it, is the torch expression itself."""
+
+    def __init__(self, op, rows, queries, shape, compute, half=None, unit=False):
+        self.op, self.rows, self.queries, self.half, self.unit = op, rows, tuple(queries), half, unit
+        self.shape = torch.Size(shape)
+        self._compute, self._value = compute, None
+
+    device = property(lambda self: self.rows.device)
+    dtype = property(lambda self: self.rows.dtype)
+    requires_grad = True
+    is_cuda = True
+
+    def dim(self):
+        return len(self.shape)
+
+    ndim = property(dim)
+
+    def size(self, d=None):
+        return self.shape if d is None else self.shape[d]
+
+    def materialize(self):
+        if self._value is None:
+            self._value = self._compute()
+        return self._value
+
+    @staticmethod
+    def _query(t, like):
+        """Whether t is a plain query tensor [B, U, 1, w] for rows / another query tensor `like`."""
+        return (isinstance(t, torch.Tensor) and not _is_lazy(t) and t.dim() == 4 and t.shape[2] == 1 and
+                t.shape[3] == like.shape[3] and t.dtype == like.dtype and t.device == like.device)
+
+    @staticmethod
+    def _binary_with_query(op, source, q, compute, unit_ok):
+        """op(source, q) for a 4-D handle [Be, 1, K, w] or one of its halves; None when it is not that shape."""
+        if isinstance(source, LazyRows):
+            handle, half, unit = source, None, False
+        elif isinstance(source, _LazyHalf) and (unit_ok or not source.unit):
+            handle, half, unit = source.rows, source.which, source.unit
+        else:
+            return None
+        if (handle.dim() != 4 or handle.shape[1] != 1 or handle.reg is not None or handle.pending_add is not None or
+                not _LazyExpr._query(q, source) or q.shape[0] not in (1, handle.shape[0]) and handle.shape[0] != 1):
+            return None
+        rows = handle._like((handle.shape[0], handle.shape[2], handle.shape[3]))
+        shape = (max(q.shape[0], handle.shape[0]), q.shape[1], handle.shape[2], q.shape[3])
+        return _LazyExpr(op, rows, (q,), shape, compute, half, unit)
+
+    @staticmethod
+    def delta(source, q):
+        return _LazyExpr._binary_with_query("delta", source, q, lambda: source.materialize() - q, False)
+
+    @staticmethod
+    def prod(source, q):
+        return _LazyExpr._binary_with_query("prod", source, q, lambda: source.materialize() * q, True)
+
+    def __add__(self, other):
+        if (self.op == "prod" and isinstance(other, _LazyExpr) and other.op == "prod" and self.half == 0 and
+                other.half == 1 and self._same_rows(other) and self.unit == other.unit and self.shape == other.shape):
+            return _LazyExpr("cprod", self.rows, self.queries + other.queries, self.shape,
+                             lambda: self.materialize() + other.materialize(), None, self.unit)
+        return torch.add(self.materialize(), _resolve(other))
+
+    def _same_rows(self, other):
+        return self.rows.root is other.rows.root and self.rows.shape == other.rows.shape
+
+    def _follow(self, op, queries, compute):
+        return _LazyExpr(op, self.rows, queries, self.shape, compute, self.half)
+
+    # -- the steps of the bodies
+    def abs(self):
+        if self.op == "delta" and self.half is None:
+            return self._follow("absdelta", self.queries, lambda: self.materialize().abs())
+        return self.materialize().abs()
+
+    __abs__ = abs
+
+    def __sub__(self, other):
+        if self.op == "absdelta" and self._query(other, self.queries[0]) and other.shape == self.queries[0].shape:
+            return self._follow("excess", self.queries + (other,), lambda: self.materialize() - other)
+        return torch.sub(self.materialize(), _resolve(other))
+
+    def norm(self, p="fro", dim=None, keepdim=False, dtype=None):
+        out = self._norm(p, dim, keepdim, dtype)
+        return self.materialize().norm(p=p, dim=dim, keepdim=keepdim, dtype=dtype) if out is None else out
+
+    def _norm(self, p, dim, keepdim, dtype):
+        if keepdim or dtype is not None:
+            return None
+        if self.op == "stack" and p in ("fro", 2, 2.0) and dim == 0:
+            shape = tuple(self.shape[1:])
+            return _LazyExpr("modulus", self.rows, self.queries, shape, lambda: self.materialize().norm(dim=0))
+        if p in (1, 1.0) and dim in (-1, self.dim() - 1):
+            if self.op in ("box_out", "box_in"):
+                return lazy_dist(self.op, self.rows, *self.queries)
+            if self.op == "delta" and self.half is None:
+                return lazy_dist("l1", self.rows, *self.queries)
+        return None
+
+    def sum(self, dim=None, keepdim=False, dtype=None):
+        if dim in (-1, self.dim() - 1) and not keepdim and dtype is None:
+            out = None
+            if self.op == "modulus":
+                out = lazy_dist("rotate", self.rows, *self.queries)
+            elif self.op == "prod" and self.half is None:
+                out = lazy_dist("distmult", self.rows, *self.queries)
+            elif self.op == "cprod":
+                rows = self.rows
+                if self.unit:
+                    rows = rows._like(rows.shape)
+                    rows.reg = UNIT_HALVES
+                out = lazy_dist("complex", rows, *self.queries)
+            if out is not None:
+                return out
+        return self.materialize().sum(dim=dim, keepdim=keepdim, dtype=dtype)
+
+    @classmethod
+    def _try_lazy(cls, func, args, kwargs):
+        name = _func_name(func)
+        x = args[0] if args else None
+        if name == "abs" and isinstance(x, _LazyExpr) and len(args) == 1 and not kwargs:
+            return x.abs()
+        if name == "relu" and isinstance(x, _LazyExpr) and len(args) == 1 and not kwargs.get("inplace", False):
+            if x.op == "excess":
+                return x._follow("box_out", x.queries, lambda: torch.relu(x.materialize()))
+        if name in ("min", "minimum") and len(args) == 2 and not kwargs and isinstance(x, _LazyExpr):
+            o = args[1]
+            if x.op == "absdelta" and cls._query(o, x.queries[0]) and o.shape == x.queries[0].shape:
+                return x._follow("box_in", x.queries + (o,), lambda: torch.min(x.materialize(), o))
+        if name == "norm" and isinstance(x, _LazyExpr) and len(args) == 1:
+            out = x._norm(kwargs.get("p", "fro"), kwargs.get("dim"), kwargs.get("keepdim", False), kwargs.get("dtype"))
+            if out is not None and kwargs.get("out") is None:
+                return out
+        if name == "sum" and isinstance(x, _LazyExpr) and len(args) <= 2 and set(kwargs) <= {"dim"}:
+            return x.sum(dim=kwargs.get("dim", args[1] if len(args) > 1 else None))
+        if name in ("add", "__add__") and len(args) == 2 and not kwargs and isinstance(x, _LazyExpr):
+            return x.__add__(args[1])
+        if name == "stack" and isinstance(x, (list, tuple)) and len(x) == 2 and kwargs.get("out") is None:
+            a, b = x
+            dim = kwargs.get("dim", args[1] if len(args) > 1 else 0)
+            if (isinstance(a, _LazyExpr) and isinstance(b, _LazyExpr) and a.op == b.op == "delta" and a.half == 0 and
+                    b.half == 1 and a._same_rows(b) and a.shape == b.shape and dim == 0):
+                return _LazyExpr("stack", a.rows, a.queries + b.queries, (2,) + tuple(a.shape),
+                                 lambda: torch.stack([a.materialize(), b.materialize()], dim=0))
+        return NotImplemented
 
 
 class _Dist:

@@ -115,6 +115,73 @@ class ComplexNorm(Reasoner):       # complex.py:140-148 in its 'norm' mode (comp
         return torch.max(logit, dim=1)[0]
 
 
+class BoxNative(Reasoner):         # native_cal_logit, box.py:147-155 (--logit_impl native, the scripts' default)
+    cen = 0.02
+
+    def cal_logit(self, entity_embedding, entity_feat, query_embedding):
+        F = torch.nn.functional
+        assert entity_feat is None
+        query_center_embedding, query_offset_embedding = query_embedding
+        delta = (entity_embedding.unsqueeze(1) - query_center_embedding).abs()
+        distance_out = F.relu(delta - query_offset_embedding)
+        distance_in = torch.min(delta, query_offset_embedding)
+        logit = self.gamma - torch.norm(distance_out, p=1, dim=-1) - self.cen * torch.norm(distance_in, p=1, dim=-1)
+        logit = torch.max(logit, dim=1)[0]
+        return logit
+
+
+class VecNative(Reasoner):         # native_cal_logit, vec.py:78-83
+    def cal_logit(self, entity_embedding, entity_feat, query_embedding):
+        assert entity_feat is None
+        distance = entity_embedding.unsqueeze(1) - query_embedding[0]
+        logit = self.gamma - torch.norm(distance, p=1, dim=-1)
+        logit = torch.max(logit, dim=1)[0]
+        return logit
+
+
+class RotateNative(Reasoner):      # native_cal_logit, rotate.py:125-135
+    def cal_logit(self, entity_embedding, entity_feat, query_embedding):
+        assert entity_feat is None
+        query_re_embedding, query_im_embedding = query_embedding
+        entity_re_embedding, entity_im_embedding = torch.chunk(entity_embedding.unsqueeze(1), 2, dim=-1)
+        re_distance = entity_re_embedding - query_re_embedding
+        im_distance = entity_im_embedding - query_im_embedding
+        distance = torch.stack([re_distance, im_distance], dim=0)
+        distance = distance.norm(dim=0)
+        logit = self.gamma - distance.sum(dim=-1)
+        logit = torch.max(logit, dim=1)[0]
+        return logit
+
+
+class DistmultNative(Reasoner):    # native_cal_logit, distmult.py:126-133 (the model's only form), without 'norm'
+    def cal_logit(self, entity_embedding, entity_feat, query_embedding):
+        assert entity_feat is None
+        entity_embedding = entity_embedding.unsqueeze(1)
+        logit = (query_embedding[0] * entity_embedding).sum(-1)
+        logit = torch.max(logit, dim=1)[0]
+        return logit
+
+
+class ComplexNative(Reasoner):     # native_cal_logit, complex.py:169-177: rows of the queries' own batch
+    need_norm = False
+    embed_norm = staticmethod(ComplexNorm.embed_norm)
+
+    def cal_logit(self, entity_embedding, entity_feat, query_embedding):
+        assert entity_feat is None
+        query_re_embedding, query_im_embedding = query_embedding
+        entity_re_embedding, entity_im_embedding = torch.chunk(entity_embedding.unsqueeze(1), 2, dim=-1)
+        if self.need_norm:
+            entity_re_embedding, entity_im_embedding = self.embed_norm(entity_re_embedding), self.embed_norm(entity_im_embedding)
+        assert entity_re_embedding.shape[0] == query_re_embedding.shape[0]
+        logit = (entity_re_embedding * query_re_embedding + entity_im_embedding * query_im_embedding).sum(dim=-1)
+        logit = torch.max(logit, dim=1)[0]
+        return logit
+
+
+class ComplexNativeNorm(ComplexNative):
+    need_norm = True
+
+
 class Distmult(Reasoner):
     def cal_logit(self, entity_embedding, entity_feat, query_embedding):
         from smore_amd.torchext.ext_ops import distmult_sim
@@ -133,6 +200,12 @@ CASES = {
     "complex": (Complex, (), "complex", 2, 2, 0.0, 0.0),
     "distmult": (Distmult, (), "distmult", 1, 1, 0.0, 0.0),
     "complex_norm": (ComplexNorm, (), "complex", 2, 2, 0.0, 0.0),
+    "box_native": (BoxNative, (), "box", 2, 1, 24.0, 0.02),
+    "l1_native": (VecNative, (), "l1", 1, 1, 12.0, 0.0),
+    "rotate_native": (RotateNative, (), "rotate", 2, 2, 9.0, 0.0),
+    "distmult_native": (DistmultNative, (), "distmult", 1, 1, 0.0, 0.0),
+    "complex_native": (ComplexNative, (), "complex", 2, 2, 0.0, 0.0),
+    "complex_norm_native": (ComplexNativeNorm, (), "complex", 2, 2, 0.0, 0.0),
 }
 
 
@@ -146,7 +219,7 @@ def _table_and_queries(name, n, d, b, u, rng):
     else:
         table = rng.uniform(-0.07, 0.07, (n, mul * d))
         qs = [rng.uniform(-0.07, 0.07, (b, u, 1, d)) for _ in range(n_q)]
-        if name == "box":
+        if name in ("box", "box_native"):
             qs[1] = np.abs(qs[1])
     f32 = lambda a: a.astype(np.float32).astype(np.float64)
     return f32(table), [f32(q) for q in qs]
@@ -154,12 +227,12 @@ def _table_and_queries(name, n, d, b, u, rng):
 
 def _oracle_branch_logits(name, table, ids, qs, gamma, cen):
     return oracle_union_logits(CASES[name][2], table, ids, qs, gamma, cen, regularizer=name == "beta",
-                               norm=name == "complex_norm")
+                               norm=name.startswith("complex_norm"))
 
 
 def _oracle_grads(name, table, ids, qs, rows, logit, gout, cen):
     return oracle_union_grads(CASES[name][2], table, ids, qs, rows, logit, gout, cen, regularizer=name == "beta",
-                              norm=name == "complex_norm")
+                              norm=name.startswith("complex_norm"))
 
 
 @pytest.mark.parametrize("name", list(CASES))
@@ -352,6 +425,44 @@ def test_complex_norm_step_with_shared_negatives_stays_fused():
     orc.adam_rows(w, m, v, uniq, merged, lr, 1)
     assert_close(emb.state_sum_fo.cpu().numpy()[uniq], m[uniq], REL_F32, "first moment")
     assert_adam_weights(emb.embedding.detach().cpu().numpy(), w, merged, uniq, lr, "weights")
+
+
+@pytest.mark.parametrize("native,custom,mul,n_q", [(BoxNative, Box, 1, 2), (VecNative, None, 1, 1), (RotateNative, Rotate, 2, 2)])
+def test_native_bodies_with_shared_negatives_give_the_bits_of_the_ext_ops_form(native, custom, mul, n_q):
+    """--share_negative with --logit_impl native (what 31 of the reference's 40 scripts run): the torch-operator
+    body on a [1, K] handle asks the fused scorer for exactly what the ext_ops body asks -- same launches, same
+    bits in logits, query gradients, table and optimizer state, and no lookup materialised."""
+    from smore_amd.embedding.embed_optimizer import AdamEmbedOptimizer
+    from smore_amd.embedding.sparse_embed import SparseEmbedding
+    n, d, b, k, lr = 400, 40, 7, 90, 1e-3
+    rng = np.random.default_rng(41)
+    table = rng.uniform(-0.07, 0.07, (n, mul * d)).astype(np.float32)
+    qs = [rng.uniform(-0.07, 0.07, (b, 1, 1, d)).astype(np.float32) for _ in range(n_q)]
+    if native is BoxNative:
+        qs[1] = np.abs(qs[1])
+    pos, neg = rng.integers(0, n, b), rng.integers(0, n // 3, (1, k))
+    gp = rng.standard_normal((b, 1)).astype(np.float32)
+    gn = rng.standard_normal((b, k)).astype(np.float32)
+
+    def run(cls, *extra):
+        emb = SparseEmbedding(n, mul * d).cuda()
+        with torch.no_grad():
+            emb.embedding.copy_(torch.tensor(table))
+        opt = AdamEmbedOptimizer(types.SimpleNamespace(optim_mode="(aggr,adam,gpu,False,5)", share_optim_stats=True), emb, 0)
+        net = cls(emb, 12.0, *extra).cuda()
+        t_qs = [torch.tensor(q, device="cuda", requires_grad=True) for q in qs]
+        opt.zero_grad()
+        lp, ln = net(torch.tensor(pos, device="cuda"), torch.tensor(neg, device="cuda"), t_qs)
+        assert lp.shape == (b, 1) and ln.shape == (b, k)
+        ((lp * torch.tensor(gp, device="cuda")).sum() + (ln * torch.tensor(gn, device="cuda")).sum()).backward()
+        assert not opt.grad_list and opt.stats["materialized_lookups"] == 0 and opt.stats["dense_fallbacks"] == 0
+        opt.apply_grad(lr)
+        return [x.detach().cpu() for x in (lp, ln, *[t.grad for t in t_qs], emb.embedding, emb.state_sum_fo, emb.state_sum_sq)]
+
+    got = run(native)
+    want = run(custom) if custom is not None else run(Vec, "l1")
+    for a, r in zip(got, want):
+        assert torch.equal(a, r)
 
 
 def test_inverse_query_call_sequence_runs_on_the_reverse_layout():

@@ -65,6 +65,8 @@ def _textbook(model, e, queries, cen):
     if model == "complex":
         re, im = torch.chunk(e, 2, dim=-1)
         return (re * queries[0] + im * queries[1]).sum(-1)
+    if model == "distmult":
+        return (e * queries[0]).sum(-1)
     raise AssertionError(model)
 
 
@@ -199,6 +201,117 @@ def test_halves_put_to_any_other_use_become_tensors():
     lazy = 12.0 - ext_ops.l1_dist(ent, q)
     assert lazy._fusable() == ("l1", 0.0)      # the expression has the model's form; the request is what is refused:
     assert opt.lazy_request("l1", ent, (q,), 12.0, 0.0) is None and opt.score_lazy("l1", ent, (q,), 12.0, 0.0) is None
+
+
+def _native_box(gamma, cen, entity_embedding, query_embedding):
+    """native_cal_logit of models/box.py:147-155"""
+    F = torch.nn.functional
+    query_center_embedding, query_offset_embedding = query_embedding
+    delta = (entity_embedding.unsqueeze(1) - query_center_embedding).abs()
+    distance_out = F.relu(delta - query_offset_embedding)
+    distance_in = torch.min(delta, query_offset_embedding)
+    logit = gamma - torch.norm(distance_out, p=1, dim=-1) - cen * torch.norm(distance_in, p=1, dim=-1)
+    return torch.max(logit, dim=1)[0]
+
+
+def _native_vec(gamma, cen, entity_embedding, query_embedding):
+    """native_cal_logit of models/vec.py:78-83"""
+    distance = entity_embedding.unsqueeze(1) - query_embedding[0]
+    logit = gamma - torch.norm(distance, p=1, dim=-1)
+    return torch.max(logit, dim=1)[0]
+
+
+def _native_rotate(gamma, cen, entity_embedding, query_embedding):
+    """native_cal_logit of models/rotate.py:125-135"""
+    query_re_embedding, query_im_embedding = query_embedding
+    entity_re_embedding, entity_im_embedding = torch.chunk(entity_embedding.unsqueeze(1), 2, dim=-1)
+    re_distance = entity_re_embedding - query_re_embedding
+    im_distance = entity_im_embedding - query_im_embedding
+    distance = torch.stack([re_distance, im_distance], dim=0)
+    distance = distance.norm(dim=0)
+    logit = gamma - distance.sum(dim=-1)
+    return torch.max(logit, dim=1)[0]
+
+
+def _native_distmult(gamma, cen, entity_embedding, query_embedding):
+    """native_cal_logit of models/distmult.py:126-133 (no 'norm')"""
+    entity_embedding = entity_embedding.unsqueeze(1)
+    logit = (query_embedding[0] * entity_embedding).sum(-1)
+    return torch.max(logit, dim=1)[0]
+
+
+def _native_complex(gamma, cen, entity_embedding, query_embedding, embed_norm=None):
+    """native_cal_logit of models/complex.py:169-177, the branch for rows of the queries' own batch"""
+    query_re_embedding, query_im_embedding = query_embedding
+    entity_re_embedding, entity_im_embedding = torch.chunk(entity_embedding.unsqueeze(1), 2, dim=-1)
+    if embed_norm is not None:
+        entity_re_embedding, entity_im_embedding = embed_norm(entity_re_embedding), embed_norm(entity_im_embedding)
+    assert entity_re_embedding.shape[0] == query_re_embedding.shape[0]
+    logit = (entity_re_embedding * query_re_embedding + entity_im_embedding * query_im_embedding).sum(dim=-1)
+    return torch.max(logit, dim=1)[0]
+
+
+def _native_complex_norm(gamma, cen, entity_embedding, query_embedding):
+    return _native_complex(gamma, cen, entity_embedding, query_embedding, _Normalizer())
+
+
+@pytest.mark.parametrize("body,model,reg", [(_native_distmult, "distmult", None), (_native_complex, "complex", None),
+                                            (_native_complex_norm, "complex", "unit_halves")])
+@pytest.mark.parametrize("branches", [1, 2])
+def test_native_similarity_bodies_become_one_fused_request(body, model, reg, branches):
+    n, d, b, k = 40, 6, 3, 5
+    mul = 2 if model == "complex" else 1
+    opt = RecordingOptimizer(n, mul * d)
+    ids = torch.randint(0, n, (b * k,), generator=torch.Generator().manual_seed(31))
+    qs = _queries(b, branches, d, mul, 32)
+    logit = body(None, 0.0, LazyRows(opt, ids, "negative_entity").view(b, k, -1), qs)
+    want = body(None, 0.0, opt.sparse_embed.embedding[ids].view(b, k, -1), qs)
+    torch.testing.assert_close(logit + 0.0, want, rtol=1e-5, atol=1e-6)
+    assert opt.looked_up == [] and opt.scored == [(model, (b, k), 0.0, 0.0, reg)]
+
+
+@pytest.mark.parametrize("body,model,n_q,mul,cen", [(_native_box, "box", 2, 1, 0.02), (_native_vec, "l1", 1, 1, 0.0),
+                                                      (_native_rotate, "rotate", 2, 2, 0.0)])
+@pytest.mark.parametrize("branches", [1, 2])
+@pytest.mark.parametrize("shared", [False, True])
+def test_native_cal_logit_bodies_become_one_fused_request(body, model, n_q, mul, cen, branches, shared):
+    """The torch-operator form of the logits (--logit_impl native): no lookup, one request with the model, margin
+    and coefficient the ext_ops form gives, and the value of the torch expression on the rows."""
+    n, d, b, k = 40, 6, 3, 5
+    be = 1 if shared else b
+    opt = RecordingOptimizer(n, mul * d)
+    ids = torch.randint(0, n, (be * k,), generator=torch.Generator().manual_seed(21))
+    qs = _queries(b, branches, d, n_q, 22)
+    gamma = torch.nn.Parameter(torch.Tensor([12.0]), requires_grad=False)
+    logit = body(gamma, cen, LazyRows(opt, ids, "negative_entity").view(be, k, -1), qs)
+    want = body(gamma, cen, opt.sparse_embed.embedding[ids].view(be, k, -1), qs)
+    torch.testing.assert_close(logit + 0.0, want, rtol=1e-5, atol=1e-6)        # (the first use scores the placeholder)
+    assert opt.looked_up == [] and opt.scored == [(model, (be, k), 12.0, cen, None)]
+
+
+def test_native_intermediates_put_to_other_uses_are_the_tensors_they_stand_for():
+    n, d, b, k = 40, 6, 3, 5
+    F = torch.nn.functional
+    opt = RecordingOptimizer(n, d)
+    ids = torch.randint(0, n, (b * k,), generator=torch.Generator().manual_seed(23))
+    c, o = _queries(b, 2, d, 2, 24)
+    other = _queries(b, 2, d, 1, 25)[0]
+    rows = opt.sparse_embed.embedding[ids].view(b, k, -1)
+    handle = LazyRows(opt, ids, None).view(b, k, -1)
+    delta = (handle.unsqueeze(1) - c).abs()
+    t_delta = (rows.unsqueeze(1) - c).abs()
+    assert delta.shape == t_delta.shape and opt.looked_up == []
+    assert torch.equal(delta * 2.0, t_delta * 2.0)
+    assert torch.equal(F.relu(delta - o) + 1.0, F.relu(t_delta - o) + 1.0)
+    assert torch.equal(torch.min(delta, o).sum(-1), torch.min(t_delta, o).sum(-1))
+    assert torch.equal(torch.norm(F.relu(delta - o), p=2, dim=-1), torch.norm(F.relu(t_delta - o), p=2, dim=-1))
+    assert torch.equal(torch.norm(delta, p=1, dim=-1), torch.norm(t_delta, p=1, dim=-1))      # |e - c| has no model
+    assert torch.equal((handle.unsqueeze(1) - c).abs() - 0.5, t_delta - 0.5)                  # a scalar is no offset
+    assert torch.equal(handle.unsqueeze(1) - c[0, 0, 0], rows.unsqueeze(1) - c[0, 0, 0])      # a 1-D operand is no query
+    assert len(opt.looked_up) == 1 and opt.scored == []
+    # box_out and box_in with different offsets: two terms that do not share their operands
+    logit = 24.0 - torch.norm(F.relu(delta - o), p=1, dim=-1) - 0.02 * torch.norm(torch.min(delta, other), p=1, dim=-1)
+    assert logit._fusable() is None
 
 
 def test_other_uses_fall_back_to_one_lookup():
