@@ -412,6 +412,35 @@ class SharedStep:
         return sn, (gp, gn)
 
 
+def timing_events(steps, per_step=4):
+    """Timing events for `steps` steps, each recorded once already, so that whatever the runtime sets up at an
+    event's first use happens before the timed region."""
+    import torch
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(per_step)] for _ in range(steps)]
+    for row in ev:
+        for e in row:
+            e.record()
+    torch.cuda.synchronize()
+    return ev
+
+
+class no_collector_pauses:
+    """The timed loops run with Python's cyclic collector off, as timeit does: a full collection of this process's
+    heap takes 30-60 ms, and the thousand event objects of a long run are what makes one due in the middle of the
+    loop (seen as one 40 ms gap between two launches of a 0.2 ms step)."""
+
+    def __enter__(self):
+        import gc
+        self.was_on = gc.isenabled()
+        gc.collect()
+        gc.disable()
+
+    def __exit__(self, *exc):
+        import gc
+        if self.was_on:
+            gc.enable()
+
+
 def shared_step_bench(cfg, device, seed, steps, warmup, graph):
     """bench.py --config 6: the shared-negative step (see SharedStep), eager and replayed from a HIP graph."""
     import torch
@@ -432,17 +461,19 @@ def shared_step_bench(cfg, device, seed, steps, warmup, graph):
     torch.cuda.synchronize()
     if step.err.item() != 0:
         sys.exit("a warm-up step reported an error")
-    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(steps)]
-    t0 = time.perf_counter()
-    for s in range(steps):
-        step.run(ev[s])
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
+    ev = timing_events(steps)
+    with no_collector_pauses():
+        t0 = time.perf_counter()
+        for s in range(steps):
+            step.run(ev[s])
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
     if step.err.item() != 0:
         sys.exit("a timed step reported an error")
     ms = wall * 1e3 / steps
     phase_ms = {name: sum(e[i].elapsed_time(e[i + 1]) for e in ev) / steps for i, name in enumerate(SharedStep.PHASES)}
-    per_step = sorted(e[0].elapsed_time(e[3]) for e in ev)
+    in_order = [e[0].elapsed_time(e[3]) for e in ev]
+    per_step = sorted(in_order)
     pairs = b * (k + 1)
     n_uniq = step.plan.n_uniq
     rl = dim
@@ -459,7 +490,8 @@ def shared_step_bench(cfg, device, seed, steps, warmup, graph):
                    "(uniform) + one positive per query", "mask": "is_negative_mat folded into the upstream gradient",
                    "optimizer": "sparse adam, squeezed second moment", "seed": seed, "distinct_ids": n_uniq},
         "phase_ms": phase_ms,
-        "step_ms_events": {"median": per_step[len(per_step) // 2], "min": per_step[0], "max": per_step[-1]},
+        "step_ms_events": {"median": per_step[len(per_step) // 2], "min": per_step[0], "max": per_step[-1],
+                           "slowest_step": in_order.index(per_step[-1])},
         "step_hbm": {"algorithmic_bytes": algo, "achieved_GBps": algo / (ms * 1e-3) / 1e9,
                      "frac_of_peak": algo / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
                      "note": "the step touches K + B rows: it is bound by kernel latencies and VALU work on L2-resident "
@@ -823,13 +855,13 @@ def main():
     if step.err.item() != 0:
         sys.exit("entity id out of range in the synthetic batch")
 
-    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(args.steps)]
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for s in range(args.steps):
-        step.run(ev[s], measure_parts=parts)
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
+    ev = timing_events(args.steps)
+    with no_collector_pauses():
+        t0 = time.perf_counter()
+        for s in range(args.steps):
+            step.run(ev[s], measure_parts=parts)
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
     if step.err.item() != 0:
         sys.exit("a timed step reported an error (id out of range, or an invalid segment plan)")
 
