@@ -357,8 +357,82 @@ def dropin_flows(cfg, table, q1, q2, idx, steps, warmup, m=None, v=None, only=No
     return out
 
 
+def dropin_shared_bench(cfg, device, seed, steps, warmup):
+    """bench.py --dropin --config 6: the step of the reference's own training scripts (box model, K negatives shared
+    by the batch, one positive per query, Adam with one second-moment value per row) as its code reaches it --
+    lookups, cal_logit in its ext_ops form (box.py:157-164, --logit_impl custom) and in its torch-operator form
+    (box.py:147-155, --logit_impl native, the default), sample loss with the is_negative_mat mask
+    (train_process.py:194-213), backward, apply_grad -- with the lazy lookup handle and with plain lookups
+    (lazy_lookup = False: the reference's data flow; the native body then builds the [B, 1, K, D] intermediates)."""
+    import types
+    import torch
+    import torch.nn.functional as F
+    from smore_amd.embedding.embed_optimizer import AdamEmbedOptimizer
+    from smore_amd.embedding.sparse_embed import SparseEmbedding
+    from smore_amd.torchext.ext_ops import box_dist_in, box_dist_out
+    gen = torch.Generator(device=device)
+    gen.manual_seed(seed)
+    n, dim, b, k, r = cfg["n"], cfg["dim"], cfg["b"], cfg["k"], cfg["r"]
+    emb = SparseEmbedding(8, dim)
+    emb.embedding = torch.nn.Parameter(torch.empty((n, dim), device=device).uniform_(-r, r, generator=gen), requires_grad=True)
+    emb.num_rows = n
+    opt = AdamEmbedOptimizer(types.SimpleNamespace(optim_mode="(aggr,adam,gpu,True,5)", share_optim_stats=True), emb, 0)
+    gamma = torch.nn.Parameter(torch.tensor([cfg["gamma"]], device=device), requires_grad=False)
+    center = torch.empty((b, 1, 1, dim), device=device).uniform_(-r, r, generator=gen).requires_grad_(True)
+    offset = torch.empty((b, 1, 1, dim), device=device).uniform_(-r, r, generator=gen).abs_().requires_grad_(True)
+    pos = torch.randint(0, n, (b,), device=device, generator=gen)
+    neg = torch.randint(0, n, (1, k), device=device, generator=gen)
+    mask = (torch.rand((b, k), device=device, generator=gen) > 0.01).float()      # is_negative_mat
+
+    def custom(entity_embedding):                            # box.py:157-164
+        d1 = box_dist_out(entity_embedding, center, offset)
+        d2 = box_dist_in(entity_embedding, center, offset)
+        return torch.max(gamma - d1 - cfg["cen"] * d2, dim=1)[0]
+
+    def native(entity_embedding):                            # box.py:147-155
+        delta = (entity_embedding.unsqueeze(1) - center).abs()
+        distance_out = F.relu(delta - offset)
+        distance_in = torch.min(delta, offset)
+        logit = gamma - torch.norm(distance_out, p=1, dim=-1) - cfg["cen"] * torch.norm(distance_in, p=1, dim=-1)
+        return torch.max(logit, dim=1)[0]
+
+    def step(cal_logit):
+        opt.zero_grad()
+        center.grad = offset.grad = None
+        p_rows = emb(pos, "positive_entity")
+        n_rows = emb(neg.view(-1), "negative_entity")
+        p_rows.job_handle.sync()
+        positive_logit = cal_logit(p_rows.unsqueeze(1))
+        n_rows.job_handle.sync()
+        negative_logit = cal_logit(n_rows.view(1, k, -1)) * mask
+        loss = -F.logsigmoid(-negative_logit).mean(dim=1).mean() - F.logsigmoid(positive_logit).squeeze(dim=1).mean()
+        (loss / 2).backward()
+        opt.apply_grad(cfg["lr"])
+
+    out = {}
+    with no_collector_pauses():
+        for name, lazy, body in (("lazy handle, ext_ops body", True, custom), ("lazy handle, torch-operator body", True, native),
+                                 ("plain lookups, ext_ops body", False, custom), ("plain lookups, torch-operator body", False, native)):
+            opt.lazy_lookup = lazy
+            for _ in range(warmup):
+                step(body)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(steps):
+                step(body)
+            torch.cuda.synchronize()
+            out[name] = (time.perf_counter() - t0) * 1e3 / steps
+            if lazy and (opt.stats["dense_fallbacks"] or opt.stats["per_record_merges"] or opt.stats["materialized_lookups"]):
+                sys.exit(f"drop-in route {name!r} left the fused path: {opt.stats}")
+    opt.check_ids()
+    print(json.dumps({"workload": cfg["name"], "dropin_ms_per_step": out, "steps": steps, "warmup": warmup,
+                      "pairs_per_step": b * (k + 1)}))
+
+
 def dropin_bench(cfg, device, seed, steps, warmup):
     """bench.py --dropin: every route of dropin_flows on freshly made inputs; prints one JSON line of ms per step."""
+    if cfg.get("shared"):
+        return dropin_shared_bench(cfg, device, seed, steps, warmup)
     if cfg["model"] != "box":
         sys.exit("--dropin restates the box model's code path: use --config 2 or 5")
     table, q1, q2, idx, _ = make_inputs(cfg, device, seed)

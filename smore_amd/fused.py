@@ -19,8 +19,36 @@ ONE_QUERY = ("l1", "l2", "distmult")
 SIMILARITY = ("complex", "distmult")     # logit = gamma + sim; the others: gamma - distance
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream(t):
+    """The caller's current HIP stream on t's device, as an integer handle."""
+    index = t.device.index
+    if _raw_stream is not None and index is not None:      # (no Stream object built per call)
+        return _raw_stream(index)
     return torch.cuda.current_stream(t.device).cuda_stream
+
+
+class _Here:
+    """`with _on(device):` when that device is already the current one: nothing to switch, nothing to restore."""
+
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_here = _Here()
+
+
+def _on(device):
+    """torch.cuda.device(device), or nothing where the device is current already (the common case: a dozen library
+    calls per step would otherwise each switch to the device they are on)."""
+    if device.index is not None and torch.cuda.current_device() == device.index:
+        return _here
+    return torch.cuda.device(device)
 
 
 def _ptr(t):
@@ -93,7 +121,7 @@ def score_forward(model, table, idx, q1, q2, params, err_flag=None, codes=None):
     codes: buffer from new_codes() that receives the step's sign codes."""
     b, k, dim = _dims(model, table, idx, q1, q2)
     score = torch.empty((b, k), dtype=torch.float32, device=table.device)
-    with torch.cuda.device(table.device):
+    with _on(table.device):
         _lib.call("smx_score_forward", MODELS[model], _stream(table), _ptr(table), table.shape[0], _ptr(idx),
                   _ptr(q1), _ptr(q2), _ptr(score), b, k, dim, ctypes.byref(params), _ptr(err_flag),
                   _ptr(codes), 0 if codes is None else codes.numel())
@@ -107,7 +135,7 @@ def score_backward_query(model, table, idx, q1, q2, score, gscore, params, codes
     _f32(gscore, "gscore")
     gq1 = torch.empty_like(q1)
     gq2 = None if q2 is None else torch.empty_like(q2)
-    with torch.cuda.device(table.device):
+    with _on(table.device):
         _lib.call("smx_score_backward_query", MODELS[model], _stream(table), _ptr(table), table.shape[0], _ptr(idx),
                   _ptr(q1), _ptr(q2), _ptr(score), _ptr(gscore), _ptr(gq1), _ptr(gq2), b, k, dim,
                   ctypes.byref(params), _ptr(codes), 0 if codes is None else codes.numel())
@@ -143,7 +171,7 @@ def score_forward_shared(model, table, ids, q1, q2, params, err_flag=None, per_r
     per_row_terms=False keeps beta_kl on the per-pair kernels (no workspace for the rows' terms; for comparison)."""
     b, k, dim = _shared_dims(model, table, ids, q1, q2)
     score = torch.empty((b, k), dtype=torch.float32, device=table.device)
-    with torch.cuda.device(table.device):
+    with _on(table.device):
         ws = _shared_workspace(model, b, k, dim, table.device, per_row_terms)
         _lib.call("smx_score_forward_shared", MODELS[model], _stream(table), _ptr(table), table.shape[0], _ptr(ids),
                   _ptr(q1), _ptr(q2), _ptr(score), b, k, dim, ctypes.byref(params), _ptr(err_flag), _ptr(ws),
@@ -158,7 +186,7 @@ def score_backward_query_shared(model, table, ids, q1, q2, score, gscore, params
     _f32(gscore, "gscore")
     gq1 = torch.empty_like(q1)
     gq2 = None if q2 is None else torch.empty_like(q2)
-    with torch.cuda.device(table.device):
+    with _on(table.device):
         ws = _shared_workspace(model, b, k, dim, table.device, per_row_terms)
         _lib.call("smx_score_backward_query_shared", MODELS[model], _stream(table), _ptr(table), table.shape[0],
                   _ptr(ids), _ptr(q1), _ptr(q2), _ptr(score), _ptr(gscore), _ptr(gq1), _ptr(gq2), b, k, dim,
@@ -188,7 +216,7 @@ def score_backward_entity_shared(model, table, ids, q1, q2, score, gscore, param
         _check_state(table, m, v, adam)
         if merged is not None and (merged.dim() != 2 or merged.shape[1] != row_len):
             raise _lib.SmxError("merged must be [n_uniq or more, row]")
-    with torch.cuda.device(table.device):
+    with _on(table.device):
         view = None if plan is None else plan.view()
         ws = _shared_workspace(model, b, k, dim, table.device, per_row_terms)
         _lib.call("smx_score_backward_entity_shared", MODELS[model], _stream(table), _ptr(table), table.shape[0],
@@ -206,7 +234,7 @@ def gather_rows(table, idx, err_flag=None):
     flat = idx.reshape(-1).contiguous()
     out = torch.empty((flat.numel(), table.shape[1]), dtype=torch.float32, device=table.device)
     if flat.numel():
-        with torch.cuda.device(table.device):
+        with _on(table.device):
             _lib.call("smx_gather_rows", _stream(table), _ptr(table), table.shape[0], table.shape[1], _ptr(flat),
                       flat.numel(), _ptr(out), _ptr(err_flag))
     return out
@@ -259,7 +287,7 @@ def build_plan(idx, n_rows, want_inverse=False, err_flag=None, measure=None):
     flat = idx.reshape(-1).contiguous()
     n = flat.numel()
     plan = SegmentPlan(n, n_rows, flat.device, want_inverse)
-    with torch.cuda.device(flat.device):
+    with _on(flat.device):
         nbytes = _lib.load().smx_plan_workspace_bytes(n, n_rows)
         if nbytes == 0:
             raise _lib.SmxError("smx_plan_workspace_bytes failed")
@@ -322,7 +350,7 @@ def score_backward_entity(model, plan, table, q1, q2, score, gscore, params, mer
     _check_state(table, m, v, adam)
     if merged is not None and (merged.dim() != 2 or merged.shape[1] != row_len):
         raise _lib.SmxError("merged must be [n_uniq or more, row]")
-    with torch.cuda.device(table.device):
+    with _on(table.device):
         ws = _workspace(_lib.load().smx_entity_workspace_bytes(plan.n_pairs, row_len), table.device)
         view = plan.view()
         _lib.call("smx_score_backward_entity", MODELS[model], _stream(table), ctypes.byref(view), _ptr(table),
@@ -347,7 +375,7 @@ def score_forward_union(model, table, idx, q1, q2, params, branches, err_flag=No
     b, k = idx.shape
     score = torch.empty((b, k), dtype=torch.float32, device=table.device)
     winner = torch.empty((b, k), dtype=torch.uint8, device=table.device)
-    with torch.cuda.device(table.device):
+    with _on(table.device):
         ws = _workspace(_lib.load().smx_union_workspace_bytes(b, branches, k), table.device)
         _lib.call("smx_score_forward_union", MODELS[model], _stream(table), _ptr(table), table.shape[0], _ptr(idx),
                   _ptr(q1), _ptr(q2), _ptr(score), _ptr(winner), b, branches, k, dim, ctypes.byref(params),
@@ -363,7 +391,7 @@ def score_backward_query_union(model, table, idx, q1, q2, score, gscore, winner,
     dim = q1.shape[-1]
     gq1 = torch.empty_like(q1)
     gq2 = None if q2 is None else torch.empty_like(q2)
-    with torch.cuda.device(table.device):
+    with _on(table.device):
         _lib.call("smx_score_backward_query_union", MODELS[model], _stream(table), _ptr(table), table.shape[0], _ptr(idx),
                   _ptr(q1), _ptr(q2), _ptr(score), _ptr(gscore), _ptr(winner), _ptr(gq1), _ptr(gq2), b, branches, k,
                   dim, ctypes.byref(params))
@@ -414,7 +442,7 @@ def score_backward_entity_multi(model, plan, table, q1, q2, sources, params, mer
         if grad_rows.dim() != 2 or grad_rows.shape[1] != row_len or grad_rows.shape[0] == 0:
             raise _lib.SmxError("grad_rows must be [n >= 1, row]")
         n_grad = grad_rows.shape[0]
-    with torch.cuda.device(table.device):
+    with _on(table.device):
         ws = _workspace(_lib.load().smx_entity_workspace_bytes(plan.n_pairs, row_len), table.device)
         view = plan.view()
         if branches > 1:
@@ -448,7 +476,7 @@ def score_backward_fused(model, plan, table, idx, q1, q2, score, gscore, params,
         raise _lib.SmxError("merged must be [n_uniq or more, row]")
     gq1 = torch.empty_like(q1)
     gq2 = None if q2 is None else torch.empty_like(q2)
-    with torch.cuda.device(table.device):
+    with _on(table.device):
         ws_bytes = _lib.load().smx_fused_workspace_bytes(MODELS[model], plan.n_pairs, dim) \
             if sign_codes and codes is None else \
             _lib.load().smx_entity_workspace_bytes(plan.n_pairs, table.shape[1])
@@ -472,7 +500,7 @@ def rows_backward(plan, grad_rows, merged=None, table=None, m=None, v=None, adam
     row_len = grad_rows.shape[1]
     if table is not None:
         _check_state(table, m, v, adam)
-    with torch.cuda.device(grad_rows.device):
+    with _on(grad_rows.device):
         ws = _workspace(_lib.load().smx_entity_workspace_bytes(plan.n_pairs, row_len), grad_rows.device)
         view = plan.view()
         _lib.call("smx_rows_backward", _stream(grad_rows), ctypes.byref(view), _ptr(grad_rows), row_len, _ptr(merged),
