@@ -117,7 +117,8 @@ typedef struct smx_score_params {
   float reg_hi;
   int norm_on;   /* COMPLEX: each half of an entity row (re, im) is scaled to unit L2 length before it is scored
                   * (complex.py:142-146 with the 'norm' mode of complex.py:87-89: F.normalize, eps 1e-12), and the
-                  * entity gradient is taken through that scaling. */
+                  * entity gradient is taken through that scaling.  DISTMULT: the same with the whole row
+                  * (distmult.py:85-87,129-130).  Other models refuse it (SMX_ERR_ARG). */
 } smx_score_params;
 
 /* Sign codes (optional, what autograd would call a saved tensor).  For the box model (and, with one

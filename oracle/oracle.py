@@ -162,28 +162,29 @@ def regularizer(x, base_add=1.0, lo=0.05, hi=1e9, dtype=np.float64):
     return out
 
 
-def unit_halves(rows, dtype=np.float64, eps=1e-12):
+def unit_halves(rows, dtype=np.float64, eps=1e-12, halves=2):
     """Each half of the last axis scaled to unit L2 length, x / max(|x|, eps): what ComplexReasoning does to an
     entity row before complex_sim when its mode names 'norm' (models/complex.py:142-146; embed_norm = Normalizer,
-    common/modules.py:38-40 = F.normalize(p=2, dim=-1), whose eps is 1e-12)."""
+    common/modules.py:38-40 = F.normalize(p=2, dim=-1), whose eps is 1e-12).  halves = 1: the whole row, DistMult's
+    'norm' mode (models/distmult.py:129-130)."""
     rows = np.asarray(rows, dtype=dtype)
-    h = rows.shape[-1] // 2
+    h = rows.shape[-1] // halves
     out = np.empty_like(rows)
-    for sl in (slice(0, h), slice(h, 2 * h)):
+    for sl in [slice(i * h, (i + 1) * h) for i in range(halves)]:
         x = rows[..., sl]
         n = np.maximum(np.sqrt((x * x).sum(axis=-1, keepdims=True)), dtype(eps))
         out[..., sl] = x / n
     return out
 
 
-def unit_halves_backward(rows, gout, dtype=np.float64, eps=1e-12):
+def unit_halves_backward(rows, gout, dtype=np.float64, eps=1e-12, halves=2):
     """Gradient w.r.t. rows of sum(gout * unit_halves(rows)): per half (g - x_n (x_n . g)) / |x| where |x| > eps,
     g / eps below (the denominator is then the constant eps)."""
     rows = np.asarray(rows, dtype=dtype)
     gout = np.asarray(gout, dtype=dtype)
-    h = rows.shape[-1] // 2
+    h = rows.shape[-1] // halves
     out = np.empty_like(rows)
-    for sl in (slice(0, h), slice(h, 2 * h)):
+    for sl in [slice(i * h, (i + 1) * h) for i in range(halves)]:
         x, g = rows[..., sl], gout[..., sl]
         n = np.sqrt((x * x).sum(axis=-1, keepdims=True))
         live = n > eps
@@ -317,10 +318,11 @@ def score_forward(model, rows, q1, q2=None, gamma=0.0, cen=0.0, dtype=np.float64
     """rows [B,K,De], q [B,1,D] -> logit [B,K] as the custom_cal_logit bodies compute it
     (models/vec.py:85-90, box.py:157-164, rotate.py:137-142, beta.py:303-308) with one
     union branch; l2 takes the square root outside the operator (dist_func/l2_dist.py:59-62).
-    norm (complex only): the halves of every entity row at unit length first (complex.py:142-146)."""
+    norm (complex: the halves of every entity row at unit length first, complex.py:142-146; distmult: the whole
+    row, distmult.py:129-130)."""
     if norm:
-        assert model == "complex"
-        rows = unit_halves(rows, dtype)
+        assert model in SIMILARITY
+        rows = unit_halves(rows, dtype, halves=2 if model == "complex" else 1)
     if model == "box":
         d = dist_forward("box_out", rows, q1, q2, dtype) + cen * dist_forward("box_in", rows, q1, q2, dtype)
     elif model == "l2":
@@ -336,9 +338,10 @@ def score_backward(model, gscore, rows, q1, q2=None, cen=0.0, dtype=np.float64, 
     """Gradients of sum(gscore * score) w.r.t. rows, q1, q2."""
     gscore = np.asarray(gscore, dtype=dtype)
     if norm:
-        assert model == "complex"
-        gn, gq1, gq2 = dist_backward(model, gscore, unit_halves(rows, dtype), q1, q2, dtype)
-        return unit_halves_backward(rows, gn, dtype), gq1, gq2
+        assert model in SIMILARITY
+        halves = 2 if model == "complex" else 1
+        gn, gq1, gq2 = dist_backward(model, gscore, unit_halves(rows, dtype, halves=halves), q1, q2, dtype)
+        return unit_halves_backward(rows, gn, dtype, halves=halves), gq1, gq2
     if model == "box":
         a = dist_backward("box_out", -gscore, rows, q1, q2, dtype)
         b = dist_backward("box_in", -cen * gscore, rows, q1, q2, dtype)

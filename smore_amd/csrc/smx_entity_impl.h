@@ -1063,7 +1063,7 @@ int launch_entity_reg(hipStream_t st, const EntityArgs& A) {
 
 template <int SRC, int VEC, int NIT>
 int launch_entity(hipStream_t st, const EntityArgs& A) {
-  if constexpr (SRC == mBetaKL || SRC == mComplex) {
+  if constexpr (SRC == mBetaKL || SRC == mComplex || SRC == mDistmult) {
     if (SRC == mBetaKL ? A.p.reg_on : A.p.norm_on) return launch_entity_reg<SRC, VEC, NIT, true>(st, A);
   }
   return launch_entity_reg<SRC, VEC, NIT, false>(st, A);

@@ -38,7 +38,7 @@ struct ScoreParams {
   float cen;      // weight of the inside distance (BOX only)
   int reg_on;     // entity prologue on/off
   float reg_add, reg_lo, reg_hi;
-  int norm_on;    // COMPLEX: unit-length halves (the kernels' REG instantiation stands for it there)
+  int norm_on;    // COMPLEX, DISTMULT: unit-length halves / rows (the kernels' REG instantiation stands for it there)
 };
 
 inline ScoreParams to_params(const smx_score_params* c) {
@@ -60,7 +60,8 @@ __device__ __forceinline__ float reg_mask(float e_raw, float g, const ScoreParam
 
 inline const char* params_refused(int model, const smx_score_params* c) {
   if (c->reg_on && model != mBetaKL) return "the entity clamp prologue exists for the beta_kl model only";
-  if (c->norm_on && model != mComplex) return "unit-length row halves exist for the complex model only";
+  if (c->norm_on && model != mComplex && model != mDistmult)
+    return "unit-length rows exist for the complex and distmult models only";
   return nullptr;
 }
 
@@ -406,8 +407,10 @@ template <> struct ModelOps<mComplex> {
 // gradient G = sum c q pushed through the scaling once, g_re = (G_re - re_n (re_n . G_re)) / |re|.  The entity
 // kernels therefore accumulate G as they do for plain ComplEx, and the function that finishes a row applies the
 // projection.  In the kernels the REG instantiation of the ComplEx model stands for this form.
+// DistMult's 'norm' mode (distmult.py:85-87,129-130) is the same with the whole row as its only half:
+//   logit = gamma + (e . q) / max(|e|, eps).
 constexpr float kNormEps = 1e-12f;
-__host__ __device__ constexpr bool model_norm(int m, bool reg) { return m == mComplex && reg; }
+__host__ __device__ constexpr bool model_norm(int m, bool reg) { return (m == mComplex || m == mDistmult) && reg; }
 __device__ __forceinline__ float inv_norm(float sumsq) { return 1.f / fmaxf(__builtin_sqrtf(sumsq), kNormEps); }
 
 template <> struct ModelOps<mDistmult> {

@@ -96,19 +96,20 @@ __device__ __forceinline__ void unit_row(float (&e1)[NIT][VEC], float (&e2)[NIT]
 #pragma unroll
       for (int v = 0; v < VEC; ++v) {
         a = __builtin_fmaf(e1[it][v], e1[it][v], a);
-        b = __builtin_fmaf(e2[it][v], e2[it][v], b);
+        if constexpr (model_mul(M) == 2) b = __builtin_fmaf(e2[it][v], e2[it][v], b);
       }
       const bool in = lane + 64 * it < ncol;
       s1 += in ? a : 0.f;
       s2 += in ? b : 0.f;
     }
-    const float i1 = inv_norm(wave_sum_f32(s1)), i2 = inv_norm(wave_sum_f32(s2));
+    const float i1 = inv_norm(wave_sum_f32(s1));
+    const float i2 = model_mul(M) == 2 ? inv_norm(wave_sum_f32(s2)) : 0.f;
 #pragma unroll
     for (int it = 0; it < NIT; ++it)
 #pragma unroll
       for (int v = 0; v < VEC; ++v) {
         e1[it][v] *= i1;
-        e2[it][v] *= i2;
+        if constexpr (model_mul(M) == 2) e2[it][v] *= i2;
       }
   }
 }
@@ -482,7 +483,7 @@ int launch_rank_reg(hipStream_t st, RankArgs A, int mode) {
 
 template <int M, int VEC, int NIT>
 int launch_rank(hipStream_t st, const RankArgs& A, int mode) {
-  if constexpr (M == mBetaKL || M == mComplex) {
+  if constexpr (M == mBetaKL || M == mComplex || M == mDistmult) {
     if (M == mBetaKL ? A.p.reg_on : A.p.norm_on) return launch_rank_reg<M, VEC, NIT, true>(st, A, mode);
   }
   return launch_rank_reg<M, VEC, NIT, false>(st, A, mode);

@@ -81,7 +81,7 @@ __device__ __forceinline__ float l2_pair_coef(float c_raw, int ncol, int lane, G
 }
 
 // ComplEx with unit-length halves, query backward: the pair's upstream coefficient over the two lengths of its row.
-template <int VEC, int NIT, class GetE1, class GetE2>
+template <int VEC, int NIT, int MUL, class GetE1, class GetE2>
 __device__ __forceinline__ float2 norm_pair_coef(float c_raw, int ncol, int lane, GetE1&& e1, GetE2&& e2) {
   float s1 = 0.f, s2 = 0.f;
 #pragma unroll
@@ -90,13 +90,15 @@ __device__ __forceinline__ float2 norm_pair_coef(float c_raw, int ncol, int lane
 #pragma unroll
     for (int v = 0; v < VEC; ++v) {
       a = __builtin_fmaf(e1(it, v), e1(it, v), a);
-      b = __builtin_fmaf(e2(it, v), e2(it, v), b);
+      if constexpr (MUL == 2) b = __builtin_fmaf(e2(it, v), e2(it, v), b);
     }
     const bool in = lane + 64 * it < ncol;
     s1 += in ? a : 0.f;
     s2 += in ? b : 0.f;
   }
-  return make_float2(c_raw * inv_norm(wave_sum_f32(s1)), c_raw * inv_norm(wave_sum_f32(s2)));
+  const float c1 = c_raw * inv_norm(wave_sum_f32(s1));
+  if constexpr (MUL == 1) return make_float2(c1, 0.f);  // (DistMult: the row is its only half)
+  return make_float2(c1, c_raw * inv_norm(wave_sum_f32(s2)));
 }
 
 // ... entity side: the summed plain gradient g of one half row w pushed through w / max(|w|, eps)
@@ -237,7 +239,7 @@ __device__ __forceinline__ void finish_row(const RowSink& A, int lane, unsigned 
       }
     if constexpr (model_norm(SRC, REG)) {
       norm_project<VEC, NIT>(g1, A.ncol, lane, [&](int it, int x) { return w.h[0][it].v[x]; });
-      norm_project<VEC, NIT>(g2, A.ncol, lane, [&](int it, int x) { return w.h[MUL - 1][it].v[x]; });
+      if constexpr (MUL == 2) norm_project<VEC, NIT>(g2, A.ncol, lane, [&](int it, int x) { return w.h[MUL - 1][it].v[x]; });
     }
   }
   if (REG) {

@@ -387,9 +387,11 @@ __global__ __launch_bounds__(256) void score_forward_kernel(ScoreArgs A, int til
 #pragma unroll
         for (int v = 0; v < VEC; ++v) {
           a = __builtin_fmaf(e1[it].v[v], q[it][v].a, a);
-          b2 = __builtin_fmaf(e2[it].v[v], q[it][v].b, b2);
           c = __builtin_fmaf(e1[it].v[v], e1[it].v[v], c);
-          d = __builtin_fmaf(e2[it].v[v], e2[it].v[v], d);
+          if constexpr (MUL == 2) {
+            b2 = __builtin_fmaf(e2[it].v[v], q[it][v].b, b2);
+            d = __builtin_fmaf(e2[it].v[v], e2[it].v[v], d);
+          }
         }
         const bool in = lane + 64 * it < ncol;
         dot1 += in ? a : 0.f;
@@ -398,10 +400,14 @@ __global__ __launch_bounds__(256) void score_forward_kernel(ScoreArgs A, int til
         sq2 += in ? d : 0.f;
       }
       dot1 = wave_sum_last_f32(dot1);
-      dot2 = wave_sum_last_f32(dot2);
       sq1 = wave_sum_last_f32(sq1);
-      sq2 = wave_sum_last_f32(sq2);
-      const float s = p.gamma + (dot1 * inv_norm(sq1) + dot2 * inv_norm(sq2));
+      float s = dot1 * inv_norm(sq1);
+      if constexpr (MUL == 2) {
+        dot2 = wave_sum_last_f32(dot2);
+        sq2 = wave_sum_last_f32(sq2);
+        s += dot2 * inv_norm(sq2);
+      }
+      s += p.gamma;
       if constexpr (DEDUP) {
         if (lane == 63) rep_score[first_rep + j] = s;
       } else {
@@ -632,8 +638,8 @@ __global__ __launch_bounds__(NW * 64) void score_backward_query_kernel(ScoreArgs
         c.x = l2_pair_coef<VEC, NIT>(c.x, ncol, lane, [&](int it, int v) { return e1[it].v[v]; },
                                      [&](int it, int v) { return q[it][v].a; });
       if constexpr (model_norm(M, REG))  // d logit / d q = e / |e| per half: the upstream coefficient over the lengths
-        c = norm_pair_coef<VEC, NIT>(c_raw, ncol, lane, [&](int it, int v) { return e1[it].v[v]; },
-                                     [&](int it, int v) { return e2[it].v[v]; });
+        c = norm_pair_coef<VEC, NIT, MUL>(c_raw, ncol, lane, [&](int it, int v) { return e1[it].v[v]; },
+                                          [&](int it, int v) { return e2[it].v[v]; });
       if constexpr (CODES == 1) {
         // the pair's code bytes go to the wavefront's LDS stage, see flush_codes
         unsigned char* mine_b = stage + (j & (kStagePairs - 1)) * (NIT * 64) + lane;
@@ -657,7 +663,7 @@ __global__ __launch_bounds__(NW * 64) void score_backward_query_kernel(ScoreArgs
               ModelOps<M>::bwd_q_thr(c.x, c.y, x1, q[it][v], neg_thr[it][v], g1[it][v], g2[it][v]);
             } else if constexpr (model_norm(M, REG)) {
               g1[it][v] = __builtin_fmaf(c.x, x1, g1[it][v]);
-              g2[it][v] = __builtin_fmaf(c.y, x2, g2[it][v]);
+              if constexpr (MUL == 2) g2[it][v] = __builtin_fmaf(c.y, x2, g2[it][v]);
             } else {
               ModelOps<M>::bwd_q(c.x, c.y, x1, x2, q[it][v], g1[it][v], g2[it][v]);
             }
@@ -861,9 +867,9 @@ int launch_backward_query_reg(hipStream_t st, const ScoreArgs& A) {
 
 template <int M, int VEC, int NIT>
 int launch_score(hipStream_t st, const ScoreArgs& A, bool forward) {
-  const bool reg = (M == mBetaKL && A.p.reg_on) || (M == mComplex && A.p.norm_on);
+  const bool reg = (M == mBetaKL && A.p.reg_on) || ((M == mComplex || M == mDistmult) && A.p.norm_on);
   if (forward) {
-    if constexpr (M == mBetaKL || M == mComplex) {
+    if constexpr (M == mBetaKL || M == mComplex || M == mDistmult) {
       if (reg) return launch_forward_reg<M, VEC, NIT, true>(st, A);
     }
     return launch_forward_reg<M, VEC, NIT, false>(st, A);
@@ -874,7 +880,7 @@ int launch_score(hipStream_t st, const ScoreArgs& A, bool forward) {
   const size_t extra = kSlabDwords * sizeof(unsigned) + (model_coded(M) ? (size_t)kStagePairs * NIT * 64 : 0);
   auto fits = [&](size_t n) { return (n + 1) * per_wave + n * extra <= 64 * 1024; };
   const int nw = fits(8) ? 8 : (fits(4) ? 4 : 2);
-  if constexpr (M == mBetaKL || M == mComplex) {
+  if constexpr (M == mBetaKL || M == mComplex || M == mDistmult) {
     if (reg) {
       if (nw == 8) return launch_backward_query_reg<M, VEC, NIT, 8, true>(st, A);
       if (nw == 4) return launch_backward_query_reg<M, VEC, NIT, 4, true>(st, A);

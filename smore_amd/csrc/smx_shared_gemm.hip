@@ -369,7 +369,8 @@ __global__ __launch_bounds__(256) void shared_entity_gemm_kernel(GemmArgs A) {
 
 // ---- the K rows of the list side by side, as the products' second operand -------------------------------------
 // UNIT (ComplEx with unit-length halves, width = 2 dim): out [K][2 dim], row k = [re / max(|re|, eps) |
-// im / max(|im|, eps)] of table row ids[k]; one wavefront per row.
+// im / max(|im|, eps)] of table row ids[k]; DistMult with unit-length rows, width = dim: e / max(|e|, eps).  One
+// wavefront per row.
 // Not UNIT: out [K][width], row k = table row ids[k] as it is.  The query backward reads 128-byte pieces of all K
 // rows in each of its tiles: from K rows scattered over a table of gigabytes that is K address translations and
 // K cache lines of different pages per tile, from the copy it is one stretch of memory that stays in L2.
@@ -392,15 +393,16 @@ __global__ __launch_bounds__(256) void list_rows_kernel(const float* __restrict_
     for (int c = lane; c < width / 4; c += 64) reinterpret_cast<f4*>(out)[c] = reinterpret_cast<const f4*>(e)[c];
     return;
   }
+  const bool two = width == 2 * dim;  // ComplEx; DistMult: the row is its only half
   float s1 = 0.f, s2 = 0.f;
   for (int d = lane; d < dim; d += 64) {
     s1 = __builtin_fmaf(e[d], e[d], s1);
-    s2 = __builtin_fmaf(e[dim + d], e[dim + d], s2);
+    if (two) s2 = __builtin_fmaf(e[dim + d], e[dim + d], s2);
   }
   const float i1 = inv_norm(wave_sum_f32(s1)), i2 = inv_norm(wave_sum_f32(s2));
   for (int d = lane; d < dim; d += 64) {
     out[d] = e[d] * i1;
-    out[dim + d] = e[dim + d] * i2;
+    if (two) out[dim + d] = e[dim + d] * i2;
   }
 }
 
@@ -471,7 +473,7 @@ int shared_gemm_forward(int model, hipStream_t st, const float* table, size_t n_
   } else {
     if (p.norm_on) {
       hipLaunchKernelGGL(list_rows_kernel<true>, dim3((unsigned)((K + 3) / 4)), dim3(256), 0, st, table, ids, (int)K,
-                         (int)dim, 2 * (int)dim, (unsigned long long)n_rows, workspace, err);
+                         (int)dim, model_nq(model) * (int)dim, (unsigned long long)n_rows, workspace, err);
       A.rows = workspace;
       A.ids = nullptr;
     }

@@ -256,7 +256,7 @@ int launch_shared_entity_reg(hipStream_t st, const SharedArgs& A) {
 
 template <int M, int VEC, int NIT>
 int launch_shared_entity(hipStream_t st, const SharedArgs& A) {
-  if constexpr (M == mBetaKL || M == mComplex) {
+  if constexpr (M == mBetaKL || M == mComplex || M == mDistmult) {
     if (M == mBetaKL ? A.p.reg_on : A.p.norm_on) return launch_shared_entity_reg<M, VEC, NIT, true>(st, A);
   }
   return launch_shared_entity_reg<M, VEC, NIT, false>(st, A);

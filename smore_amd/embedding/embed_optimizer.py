@@ -16,7 +16,9 @@ import torch
 import torch.nn as nn
 
 from .. import _lib, fused
-from .lazy_rows import UNIT_HALVES, LazyRows
+from .lazy_rows import UNIT_HALVES, UNIT_ROW, LazyRows
+
+_REG_MODEL = {UNIT_HALVES: "complex", UNIT_ROW: "distmult"}     # the one model each unit-length marker belongs to
 from .sparse_embed import SparseEmbedding
 
 
@@ -267,7 +269,7 @@ class EmbeddingOptimizer(ABC):
         mul = 2 if model in fused.TWO_HALVES else 1
         n_q = 1 if model in fused.ONE_QUERY else 2
         if (nc != 1 or be not in (1, bq) or row != dim * mul or len(queries) != n_q or
-                (rows.reg is not None and model != ("complex" if rows.reg == UNIT_HALVES else "beta_kl")) or
+                (rows.reg is not None and model != _REG_MODEL.get(rows.reg if isinstance(rows.reg, str) else "", "beta_kl")) or
                 rows.ids.numel() != be * k):
             return None
         if any(t.dtype != torch.float32 or t.device != rows.device for t in queries):

@@ -35,6 +35,7 @@ import torch
 _FUSED_MODEL = {"l1": "l1", "l2": "l2", "rotate": "rotate", "beta_kl": "beta_kl"}   # logit = const - dist
 _FUSED_SIMILARITY = ("complex", "distmult")                                          # logit = const + similarity
 UNIT_HALVES = "unit_halves"     # LazyRows.reg of ComplEx rows whose halves were scaled to unit length
+UNIT_ROW = "unit_row"           # ... of rows scaled to unit length as a whole (DistMult's 'norm' mode)
 
 
 def _is_lazy(x):
@@ -289,6 +290,14 @@ class LazyRows(_Delegating):
                 out.reg = (x.pending_add or 0.0, lo, hi)
                 out.pending_add = None
                 return out
+        if name == "normalize" and len(args) == 1 and isinstance(args[0], LazyRows):      # distmult.py:129-130
+            x = args[0]
+            if (x.reg is None and x.pending_add is None and kwargs.get("p", 2.0) == 2 and
+                    kwargs.get("dim", 1) in (-1, x.dim() - 1) and kwargs.get("eps", 1e-12) == 1e-12 and
+                    kwargs.get("out") is None):
+                out = x._like(x.shape)
+                out.reg = UNIT_ROW
+                return out
         if name == "chunk" and args and isinstance(args[0], LazyRows):
             x = args[0]
             chunks = kwargs.get("chunks", args[1] if len(args) > 1 else None)
@@ -315,6 +324,8 @@ class LazyRows(_Delegating):
             re, im = torch.chunk(rows, 2, dim=-1)
             norm = torch.nn.functional.normalize
             rows = torch.cat((norm(re, p=2, dim=-1), norm(im, p=2, dim=-1)), dim=-1)
+        elif self.reg == UNIT_ROW:
+            rows = torch.nn.functional.normalize(rows, p=2, dim=-1)
         elif self.reg is not None:
             rows = torch.clamp(rows + self.reg[0], self.reg[1], self.reg[2])
         return rows
@@ -430,15 +441,16 @@ class _LazyExpr(_Delegating):
     def _binary_with_query(op, source, q, compute, unit_ok):
         """op(source, q) for a 4-D handle [Be, 1, K, w] or one of its halves; None when it is not that shape."""
         if isinstance(source, LazyRows):
-            handle, half, unit = source, None, False
+            handle, half, unit = source, None, source.reg == UNIT_ROW
         elif isinstance(source, _LazyHalf) and (unit_ok or not source.unit):
             handle, half, unit = source.rows, source.which, source.unit
         else:
             return None
-        if (handle.dim() != 4 or handle.shape[1] != 1 or handle.reg is not None or handle.pending_add is not None or
+        plain = handle.reg is None or (half is None and unit and unit_ok)
+        if (handle.dim() != 4 or handle.shape[1] != 1 or not plain or handle.pending_add is not None or
                 not _LazyExpr._query(q, source) or q.shape[0] not in (1, handle.shape[0]) and handle.shape[0] != 1):
             return None
-        rows = handle._like((handle.shape[0], handle.shape[2], handle.shape[3]))
+        rows = handle._like((handle.shape[0], handle.shape[2], handle.shape[3]))   # (keeps the handle's reg)
         shape = (max(q.shape[0], handle.shape[0]), q.shape[1], handle.shape[2], q.shape[3])
         return _LazyExpr(op, rows, (q,), shape, compute, half, unit)
 

@@ -65,8 +65,10 @@ def _f32(t, name):
 def score_params(gamma, cen=0.0, regularizer=None, norm=False):
     """regularizer: None or (base_add, min_val, max_val) as in smore/common/modules.py:29-36.
     norm (complex), also spelled regularizer = "unit_halves": the halves of every entity row at unit length,
-    smore/models/complex.py:142-146."""
-    if regularizer == "unit_halves":
+    smore/models/complex.py:142-146; (distmult), also regularizer = "unit_row": the whole row, distmult.py:129-130."""
+    if isinstance(regularizer, str):
+        if regularizer not in ("unit_halves", "unit_row"):
+            raise _lib.SmxError(f"unknown entity option {regularizer!r}")
         regularizer, norm = None, True
     if regularizer is None:
         return _lib.ScoreParams(gamma, cen, 0, 0.0, 0.0, 0.0, 1 if norm else 0)

@@ -121,7 +121,7 @@ def test_scorer_refuses_tables_whose_ids_need_more_than_32_bits():
 
 
 def test_entity_side_options_are_refused_where_a_model_has_none():
-    """The clamp prologue belongs to beta_kl and unit-length row halves to complex (complex.py:142-146); decided
+    """The clamp prologue belongs to beta_kl, unit-length rows to complex and distmult (complex.py:142-146); decided
     on the host, before any launch."""
     from smore_amd import _lib
     import ctypes as c
@@ -129,11 +129,11 @@ def test_entity_side_options_are_refused_where_a_model_has_none():
     fake = c.c_void_p(256)          # never dereferenced
     fwd = lambda model, params: lib.smx_score_forward(model, None, fake, 100, fake, fake, fake, fake, 2, 4, 8,
                                                       c.byref(params), None, None, 0)
-    assert fwd(2, _lib.ScoreParams(24.0, 0.02, 0, 0.0, 0.0, 0.0, 1)) != 0 and b"complex model only" in lib.smx_last_error()
+    assert fwd(2, _lib.ScoreParams(24.0, 0.02, 0, 0.0, 0.0, 0.0, 1)) != 0 and b"complex and distmult models only" in lib.smx_last_error()
     assert fwd(5, _lib.ScoreParams(0.0, 0.0, 1, 1.0, 0.05, 1e9, 0)) != 0 and b"beta_kl model only" in lib.smx_last_error()
     params = _lib.ScoreParams(24.0, 0.02, 0, 0.0, 0.0, 0.0, 1)
     rc = lib.smx_rank_answer_keys(2, None, fake, 100, fake, fake, 2, 8, c.byref(params), fake, fake, 4, fake, fake)
-    assert rc != 0 and b"complex model only" in lib.smx_last_error()
+    assert rc != 0 and b"complex and distmult models only" in lib.smx_last_error()
     assert c.sizeof(_lib.ScoreParams) == 28      # seven four-byte fields, as the header declares them
 
 

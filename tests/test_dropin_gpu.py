@@ -153,13 +153,25 @@ class RotateNative(Reasoner):      # native_cal_logit, rotate.py:125-135
         return logit
 
 
-class DistmultNative(Reasoner):    # native_cal_logit, distmult.py:126-133 (the model's only form), without 'norm'
+class DistmultNative(Reasoner):    # native_cal_logit, distmult.py:126-133 (the model's only form)
+    need_norm = False
+
+    @staticmethod
+    def embed_norm(embedding):     # Normalizer, modules.py:38-40
+        return torch.nn.functional.normalize(embedding, p=2, dim=-1)
+
     def cal_logit(self, entity_embedding, entity_feat, query_embedding):
         assert entity_feat is None
         entity_embedding = entity_embedding.unsqueeze(1)
+        if self.need_norm:
+            entity_embedding = self.embed_norm(entity_embedding)
         logit = (query_embedding[0] * entity_embedding).sum(-1)
         logit = torch.max(logit, dim=1)[0]
         return logit
+
+
+class DistmultNativeNorm(DistmultNative):      # -distmultm '(Mean,True,norm)', three of the reference's scripts
+    need_norm = True
 
 
 class ComplexNative(Reasoner):     # native_cal_logit, complex.py:169-177: rows of the queries' own batch
@@ -206,6 +218,7 @@ CASES = {
     "distmult_native": (DistmultNative, (), "distmult", 1, 1, 0.0, 0.0),
     "complex_native": (ComplexNative, (), "complex", 2, 2, 0.0, 0.0),
     "complex_norm_native": (ComplexNativeNorm, (), "complex", 2, 2, 0.0, 0.0),
+    "distmult_norm_native": (DistmultNativeNorm, (), "distmult", 1, 1, 0.0, 0.0),
 }
 
 
@@ -227,12 +240,12 @@ def _table_and_queries(name, n, d, b, u, rng):
 
 def _oracle_branch_logits(name, table, ids, qs, gamma, cen):
     return oracle_union_logits(CASES[name][2], table, ids, qs, gamma, cen, regularizer=name == "beta",
-                               norm=name.startswith("complex_norm"))
+                               norm="_norm" in name)
 
 
 def _oracle_grads(name, table, ids, qs, rows, logit, gout, cen):
     return oracle_union_grads(CASES[name][2], table, ids, qs, rows, logit, gout, cen, regularizer=name == "beta",
-                              norm=name.startswith("complex_norm"))
+                              norm="_norm" in name)
 
 
 @pytest.mark.parametrize("name", list(CASES))

@@ -11,7 +11,8 @@ from tests.util import REL_F32, assert_close, record_headroom, seed
 pytestmark = pytest.mark.gpu
 
 GAMMA = {"l1": 12.0, "l2": 12.0, "box": 24.0, "rotate": 9.0, "beta_kl": 60.0, "complex": 0.0, "distmult": 0.0,
-         "complex_norm": 0.0}   # complex with unit-length row halves (complex.py:142-146)
+         "complex_norm": 0.0,   # complex with unit-length row halves (complex.py:142-146)
+         "distmult_norm": 0.0}  # distmult with unit-length rows (distmult.py:129-130)
 
 
 def make_problem(model, n, b, k, dim, rng, zipf=None, scale=0.07):
@@ -52,8 +53,8 @@ def run_case(model, n, b, k, dim, zipf=None, cen=0.02, adam_steps=2, lr=1e-3):
     from smore_amd import fused
     rng = np.random.default_rng(seed(model, n, b, k, dim, zipf))
     gamma = GAMMA[model]
-    norm = model == "complex_norm"
-    model = "complex" if norm else model
+    norm = model.endswith("_norm")
+    model = model[:-5] if norm else model
     table, q1, q2, idx, gs = make_problem(model, n, b, k, dim, rng, zipf)
     params = fused.score_params(gamma, cen, norm=norm)
     t_table, t_q1, t_q2, t_gs = dev(table), dev(q1), dev(q2), dev(gs)

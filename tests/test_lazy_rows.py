@@ -40,6 +40,8 @@ class RecordingOptimizer:
         if reg == "unit_halves":
             re, im = torch.chunk(e, 2, dim=-1)
             e = torch.cat((re / re.norm(dim=-1, keepdim=True), im / im.norm(dim=-1, keepdim=True)), dim=-1)
+        elif reg == "unit_row":
+            e = e / e.norm(dim=-1, keepdim=True)
         elif reg is not None:
             e = torch.clamp(e + reg[0], reg[1], reg[2])
         if q1.dim() == 3:
@@ -233,11 +235,17 @@ def _native_rotate(gamma, cen, entity_embedding, query_embedding):
     return torch.max(logit, dim=1)[0]
 
 
-def _native_distmult(gamma, cen, entity_embedding, query_embedding):
-    """native_cal_logit of models/distmult.py:126-133 (no 'norm')"""
+def _native_distmult(gamma, cen, entity_embedding, query_embedding, embed_norm=None):
+    """native_cal_logit of models/distmult.py:126-133"""
     entity_embedding = entity_embedding.unsqueeze(1)
+    if embed_norm is not None:
+        entity_embedding = embed_norm(entity_embedding)
     logit = (query_embedding[0] * entity_embedding).sum(-1)
     return torch.max(logit, dim=1)[0]
+
+
+def _native_distmult_norm(gamma, cen, entity_embedding, query_embedding):
+    return _native_distmult(gamma, cen, entity_embedding, query_embedding, _Normalizer())
 
 
 def _native_complex(gamma, cen, entity_embedding, query_embedding, embed_norm=None):
@@ -256,7 +264,8 @@ def _native_complex_norm(gamma, cen, entity_embedding, query_embedding):
 
 
 @pytest.mark.parametrize("body,model,reg", [(_native_distmult, "distmult", None), (_native_complex, "complex", None),
-                                            (_native_complex_norm, "complex", "unit_halves")])
+                                            (_native_complex_norm, "complex", "unit_halves"),
+                                            (_native_distmult_norm, "distmult", "unit_row")])
 @pytest.mark.parametrize("branches", [1, 2])
 def test_native_similarity_bodies_become_one_fused_request(body, model, reg, branches):
     n, d, b, k = 40, 6, 3, 5

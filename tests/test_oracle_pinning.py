@@ -510,6 +510,21 @@ def test_unit_halves_is_f_normalize_per_half_and_its_backward_is_autograd():
     assert np.allclose(orc.unit_halves(tiny)[0, 0], [0.3, 0.4, 0.6, 0.8], rtol=1e-12)
     gt = orc.unit_halves_backward(tiny, np.ones((1, 1, 4)))[0, 0]
     assert np.allclose(gt[:2], [1e12, 1e12]) and np.allclose(gt[2:], [(1 - 0.6 * 1.4) / 5, (1 - 0.8 * 1.4) / 5], rtol=1e-12)
+    # one half = the whole row (DistMult's 'norm' mode, distmult.py:129-130): F.normalize of the row and its autograd
+    tw = torch.tensor(rows, requires_grad=True)
+    whole = F.normalize(tw, p=2, dim=-1)
+    assert np.allclose(orc.unit_halves(rows, halves=1), whole.detach().numpy(), rtol=1e-14, atol=0)
+    (whole * torch.from_numpy(g)).sum().backward()
+    assert np.allclose(orc.unit_halves_backward(rows, g, halves=1), tw.grad.numpy(), rtol=1e-11, atol=1e-13)
+    qd = rng.standard_normal((b, 1, 2 * d))
+    td = torch.tensor(qd, requires_grad=True)
+    tw.grad = None
+    sd = (F.normalize(tw, p=2, dim=-1) * td).sum(-1)
+    gsd = rng.standard_normal((b, k))
+    assert np.allclose(orc.score_forward("distmult", rows, qd, None, 0.0, norm=True), sd.detach().numpy(), rtol=1e-12, atol=1e-14)
+    (sd * torch.from_numpy(gsd)).sum().backward()
+    grd, gqd, _ = orc.score_backward("distmult", gsd, rows, qd, None, norm=True)
+    assert np.allclose(grd, tw.grad.numpy(), rtol=1e-10, atol=1e-13) and np.allclose(gqd, td.grad.numpy(), rtol=1e-10, atol=1e-13)
     # the ComplEx logit over the scaled rows, and its three gradients, against autograd of the model's lines
     re, im = rng.standard_normal((b, 1, d)), rng.standard_normal((b, 1, d))
     gs = rng.standard_normal((b, k))

@@ -11,8 +11,9 @@ pytestmark = pytest.mark.gpu
 
 
 def _alias(model):
-    """complex_norm: the complex model with the halves of every entity row at unit length (complex.py:142-146)"""
-    return ("complex", True) if model == "complex_norm" else (model, False)
+    """complex_norm / distmult_norm: the model with the halves of every entity row / the whole row at unit length
+    (complex.py:142-146, distmult.py:129-130)"""
+    return (model[:-5], True) if model.endswith("_norm") else (model, False)
 
 
 def _scores64(model, table, q1, q2, cen, norm=False):
@@ -45,7 +46,8 @@ def test_integer_valued_l1_ranks_are_exact_ties_included():
 
 
 @pytest.mark.parametrize("model,dim", [("box", 200), ("l2", 64), ("rotate", 100), ("beta_kl", 40), ("box", 30), ("complex", 48),
-                                       ("distmult", 64), ("beta_kl", 30), ("complex_norm", 48), ("complex_norm", 200)])
+                                       ("distmult", 64), ("beta_kl", 30), ("complex_norm", 48), ("complex_norm", 200),
+                                       ("distmult_norm", 64), ("distmult_norm", 30)])
 def test_ranks_lie_in_the_interval_fp32_allows(model, dim):
     """Random floats: an entity whose logit is within fp32 error of an answer's may fall on either side;
     every rank must lie between the counts with the tolerance subtracted and added."""
@@ -135,7 +137,7 @@ def test_ranking_argument_errors():
 
 
 @pytest.mark.parametrize("model,dim", [("box", 64), ("rotate", 40), ("beta_kl", 36), ("l2", 200), ("distmult", 30),
-                                       ("complex_norm", 52)])
+                                       ("complex_norm", 52), ("distmult_norm", 44)])
 def test_sampled_candidates_follow_the_reference_recipe(model, dim):
     """The sampled-negatives branch of test_step_mp (train_process.py:118-128, 141-147): -1 padding scored as entity
     0 with the -1e6 bias, ranking among the candidates, filtered ranks of the leading hard answers.  The logits
@@ -212,7 +214,8 @@ def test_union_queries_rank_exactly_by_the_maximum_over_branches(u):
 
 
 @pytest.mark.parametrize("model,dim,u", [("box", 200, 2), ("rotate", 100, 2), ("beta_kl", 40, 2), ("l2", 64, 3), ("distmult", 64, 4),
-                                         ("box", 400, 2), ("l1", 30, 3), ("complex_norm", 48, 2), ("complex_norm", 100, 3)])
+                                         ("box", 400, 2), ("l1", 30, 3), ("complex_norm", 48, 2), ("complex_norm", 100, 3),
+                                         ("distmult_norm", 64, 4)])
 def test_union_ranks_lie_in_the_interval_fp32_allows(model, dim, u):
     """Random floats, union queries: every rank between the counts with the fp32 tolerance subtracted and added;
     the answers' logits against the float64 maximum over the branches."""

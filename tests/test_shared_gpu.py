@@ -27,7 +27,9 @@ SHAPES = [("box", 300, 9, 40, 48), ("l1", 200, 5, 17, 200), ("l2", 150, 6, 33, 3
           ("rotate", 900, 64, 512, 100), ("rotate", 1200, 64, 512, 400), ("beta_kl", 700, 64, 520, 260),
           # complex with unit-length row halves (complex.py:142-146): scaled rows in the workspace as the products' operand
           ("complex_norm", 90, 3, 10, 64), ("complex_norm", 150, 33, 45, 200), ("complex_norm", 30, 2, 1, 8),
-          ("complex_norm", 70, 32, 64, 16), ("complex_norm", 400, 70, 300, 400), ("complex_norm", 60, 5, 40, 30)]
+          ("complex_norm", 70, 32, 64, 16), ("complex_norm", 400, 70, 300, 400), ("complex_norm", 60, 5, 40, 30),
+          ("distmult_norm", 90, 8, 65, 32), ("distmult_norm", 300, 64, 96, 64), ("distmult_norm", 50, 31, 257, 4),
+          ("distmult_norm", 400, 70, 300, 400), ("distmult_norm", 60, 5, 40, 30), ("distmult_norm", 30, 1, 3, 12)]
 
 
 def _shared_problem(model, n, b, k, dim):
@@ -42,8 +44,8 @@ def _shared_problem(model, n, b, k, dim):
 @pytest.mark.parametrize("model,n,b,k,dim", SHAPES)
 def test_shared_negatives_match_oracle_and_the_per_query_kernels(model, n, b, k, dim):
     from smore_amd import fused
-    norm = model == "complex_norm"
-    model = "complex" if norm else model
+    norm = model.endswith("_norm")
+    model = model[:-5] if norm else model
     table, q1, q2, ids, gs = _shared_problem(model, n, b, k, dim)
     reg = (1.0, 0.05, 1e9) if model == "beta_kl" else None      # BetaE's entity prologue rides along
     cen = 0.02
@@ -93,7 +95,8 @@ def test_shared_negatives_match_oracle_and_the_per_query_kernels(model, n, b, k,
         assert torch.equal(f1, p1) and (f2 is None or torch.equal(f2, p2))
     if model == "beta_kl" or norm:   # (unit-length complex without workspace: the per-query kernel, not a matrix product)
         assert_close(gq1.cpu().numpy(), p1.cpu().numpy(), 5e-6, f"{model} shared gq1, per-row terms vs per-pair kernel", sum_abs=q_abs)
-        assert_close(gq2.cpu().numpy(), p2.cpu().numpy(), 5e-6, f"{model} shared gq2, per-row terms vs per-pair kernel", sum_abs=q_abs)
+        if gq2 is not None:
+            assert_close(gq2.cpu().numpy(), p2.cpu().numpy(), 5e-6, f"{model} shared gq2, per-row terms vs per-pair kernel", sum_abs=q_abs)
     else:
         assert torch.equal(gq1, p1) and (gq2 is None or torch.equal(gq2, p2))
 
