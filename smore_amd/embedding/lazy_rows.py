@@ -18,8 +18,8 @@ scorer has no model for, or any other use of the rows (cal_reg, indexing, printi
 lookup (EmbedLookupFunc) and the dense operators, with the reference's results.
 
 The native_cal_logit bodies (--logit_impl native, the default: config.py:119) write the same logits with torch
-operators on the rows: box.py:147-155, vec.py:78-83, rotate.py:125-135, distmult.py:126-133, and the per-query
-branch of complex.py:169-177.  Their intermediates on a handle are
+operators on the rows: box.py:147-155, vec.py:78-83, rotate.py:125-135, distmult.py:126-133, the per-query
+branch of complex.py:169-177, and beta.py:293-301 (torch's own Beta-Beta KL routine on the halves: `_Sym`).  Their intermediates on a handle are
 `_LazyExpr` nodes (rows.unsqueeze(1) - center, its abs, relu(abs - offset), min(abs, offset), the stacked halves'
 modulus, the products with the queries); torch.norm(.., p=1, dim=-1) or .sum(dim=-1) of the right node is the same
 `LazyLogit` term the ext_ops call would have returned.  The fused scorer then computes them with ITS conventions where the two forms differ on a
@@ -302,9 +302,10 @@ class LazyRows(_Delegating):
             x = args[0]
             chunks = kwargs.get("chunks", args[1] if len(args) > 1 else None)
             dim = kwargs.get("dim", args[2] if len(args) > 2 else 0)
-            if (chunks == 2 and dim in (-1, x.dim() - 1) and (x.dim() == 3 or (x.dim() == 4 and x.shape[1] == 1)) and
-                    x.reg is None and x.pending_add is None and x.shape[-1] % 2 == 0):
-                return _LazyHalf(x, 0), _LazyHalf(x, 1)
+            if (chunks == 2 and dim in (-1, x.dim() - 1) and x.pending_add is None and x.shape[-1] % 2 == 0 and
+                    ((x.dim() == 3 and x.reg is None) or
+                     (x.dim() == 4 and x.shape[1] == 1 and (x.reg is None or isinstance(x.reg, tuple))))):
+                return _LazyHalf(x, 0), _LazyHalf(x, 1)    # (4-D with the clamp prologue: beta.py:295)
         if name in ("add", "__add__", "__radd__") and len(args) == 2 and not kwargs:
             rows, other = (args[0], args[1]) if isinstance(args[0], LazyRows) else (args[1], args[0])
             if isinstance(rows, LazyRows) and _scalar(other) is not None:
@@ -358,8 +359,9 @@ class _LazyHalf(_Delegating):
         name = _func_name(func)
         if name == "normalize" and args and isinstance(args[0], _LazyHalf) and len(args) == 1:
             x = args[0]
-            if (not x.unit and kwargs.get("p", 2.0) == 2 and kwargs.get("dim", 1) in (-1, x.dim() - 1) and
-                    kwargs.get("eps", 1e-12) == 1e-12 and kwargs.get("out") is None):
+            if (not x.unit and x.rows.reg is None and kwargs.get("p", 2.0) == 2 and
+                    kwargs.get("dim", 1) in (-1, x.dim() - 1) and kwargs.get("eps", 1e-12) == 1e-12 and
+                    kwargs.get("out") is None):
                 return _LazyHalf(x.rows, x.which, True)
         if name in ("mul", "multiply", "__mul__", "__rmul__") and len(args) == 2 and not kwargs:
             half, other = (args[0], args[1]) if isinstance(args[0], _LazyHalf) else (args[1], args[0])
@@ -367,6 +369,10 @@ class _LazyHalf(_Delegating):
                 node = _LazyExpr.prod(half, other)
                 if node is not None:
                     return node
+        if name in ("digamma", "lgamma") and len(args) == 1 and not kwargs and isinstance(args[0], _LazyHalf):
+            node = _Sym.make(name, args[0])
+            if node is not None:
+                return node
         if name == "cat" and args and isinstance(args[0], (tuple, list)) and len(args[0]) == 2:
             a, b = args[0]
             dim = kwargs.get("dim", args[1] if len(args) > 1 else 0)
@@ -381,6 +387,8 @@ class _LazyHalf(_Delegating):
 
     def __sub__(self, other):          # entity_re_embedding - query_re_embedding of rotate.py:129-130
         node = _LazyExpr.delta(self, other)
+        if node is None:
+            node = _Sym.make("sub", self, other)
         return torch.sub(self.materialize(), _resolve(other)) if node is None else node
 
     def __mul__(self, other):          # entity_re_embedding * query_re_embedding of complex.py:176
@@ -389,9 +397,235 @@ class _LazyHalf(_Delegating):
 
     __rmul__ = __mul__
 
+    def __add__(self, other):          # p.concentration1 + p.concentration0 of torch's Beta KL (beta.py:298)
+        node = _Sym.make("add", self, other)
+        return torch.add(self.materialize(), _resolve(other)) if node is None else node
+
+    def lgamma(self):
+        node = _Sym.make("lgamma", self)
+        return self.materialize().lgamma() if node is None else node
+
+    def digamma(self):
+        node = _Sym.make("digamma", self)
+        return self.materialize().digamma() if node is None else node
+
     def materialize(self):
         half = torch.chunk(self.rows.materialize(), 2, dim=-1)[self.which]
         return torch.nn.functional.normalize(half, p=2, dim=-1) if self.unit else half
+
+
+class _Sym(_Delegating):
+    """A node of the expression torch's Beta-Beta KL routine builds from the two halves of a 4-D handle
+    (native_cal_logit of beta.py:293-301 hands it BetaDist(alpha half, beta half) and BetaDist(*query)):
+    add / sub / mul of nodes, halves and plain tensors, lgamma and digamma of nodes and halves.  Nothing is
+    computed while the expression grows; torch.norm(.., p=1, dim=-1) of the finished one asks `beta_kl_operands`
+    whether it IS that routine's expression of these halves and two query tensors, and if so becomes the same
+    LazyLogit term ext_ops.beta_kl returns.  Any other use evaluates the expression with torch, node by node."""
+
+    _BINARY = {"add": torch.add, "sub": torch.sub, "mul": torch.mul}
+    _UNARY = {"lgamma": torch.lgamma, "digamma": torch.digamma}
+
+    def __init__(self, op, args, handle, shape):
+        self.op, self.args, self.handle = op, tuple(args), handle
+        self.shape = torch.Size(shape)
+        self._value = None
+
+    device = property(lambda self: self.handle.device)
+    dtype = property(lambda self: self.handle.dtype)
+    requires_grad = True
+    is_cuda = True
+
+    def dim(self):
+        return len(self.shape)
+
+    ndim = property(dim)
+
+    def size(self, d=None):
+        return self.shape if d is None else self.shape[d]
+
+    @staticmethod
+    def _handle_of(x):
+        if isinstance(x, _Sym):
+            return x.handle
+        if isinstance(x, _LazyHalf) and not x.unit and x.dim() == 4:
+            return x.rows
+        return None
+
+    @staticmethod
+    def make(op, *args):
+        """The node op(args), or None when an operand is neither a node, a half of the same 4-D handle nor a plain
+        tensor of the handle's dtype and device."""
+        handle = None
+        for a in args:
+            h = _Sym._handle_of(a)
+            if h is not None:
+                if handle is not None and h is not handle:
+                    return None
+                handle = h
+            elif not (isinstance(a, torch.Tensor) and not _is_lazy(a) and a.dim() == 4):
+                return None
+        if handle is None or any(isinstance(a, torch.Tensor) and (a.dtype != handle.dtype or a.device != handle.device)
+                                 for a in args):
+            return None
+        try:
+            shape = torch.broadcast_shapes(*[tuple(a.shape) for a in args])
+        except RuntimeError:
+            return None
+        return _Sym(op, args, handle, shape)
+
+    def materialize(self):
+        if self._value is None:
+            vals = [_resolve(a) for a in self.args]
+            self._value = (self._BINARY.get(self.op) or self._UNARY[self.op])(*vals)
+        return self._value
+
+    def _binary(self, op, other, reflected=False):
+        node = _Sym.make(op, other, self) if reflected else _Sym.make(op, self, other)
+        if node is not None:
+            return node
+        a, b = (_resolve(other), self.materialize()) if reflected else (self.materialize(), _resolve(other))
+        return self._BINARY[op](a, b)
+
+    def __add__(self, other):
+        return self._binary("add", other)
+
+    def __radd__(self, other):
+        return self._binary("add", other, True)
+
+    def __sub__(self, other):
+        return self._binary("sub", other)
+
+    def __rsub__(self, other):
+        return self._binary("sub", other, True)
+
+    def __mul__(self, other):
+        return self._binary("mul", other)
+
+    def __rmul__(self, other):
+        return self._binary("mul", other, True)
+
+    def lgamma(self):
+        return _Sym.make("lgamma", self)
+
+    def digamma(self):
+        return _Sym.make("digamma", self)
+
+    def norm(self, p="fro", dim=None, keepdim=False, dtype=None):
+        out = self._l1(p, dim, keepdim, dtype)
+        return self.materialize().norm(p=p, dim=dim, keepdim=keepdim, dtype=dtype) if out is None else out
+
+    def _l1(self, p, dim, keepdim, dtype):
+        if p in (1, 1.0) and dim in (-1, self.dim() - 1) and not keepdim and dtype is None:
+            found = beta_kl_operands(self)
+            if found is not None:
+                return lazy_dist("beta_kl", *found)
+        return None
+
+    @classmethod
+    def _try_lazy(cls, func, args, kwargs):
+        name = _func_name(func)
+        if len(args) == 2 and not kwargs:
+            a, b = args
+            op = {"add": "add", "__add__": "add", "__radd__": "add", "sub": "sub", "subtract": "sub", "__sub__": "sub",
+                  "mul": "mul", "multiply": "mul", "__mul__": "mul", "__rmul__": "mul"}.get(name)
+            if name in ("rsub", "__rsub__"):
+                a, b, op = b, a, "sub"
+            if op is not None:
+                node = _Sym.make(op, a, b)
+                if node is not None:
+                    return node
+        if name in cls._UNARY and len(args) == 1 and not kwargs:
+            node = _Sym.make(name, args[0])
+            if node is not None:
+                return node
+        if name == "norm" and len(args) == 1 and isinstance(args[0], _Sym) and kwargs.get("out") is None:
+            out = args[0]._l1(kwargs.get("p", "fro"), kwargs.get("dim"), kwargs.get("keepdim", False), kwargs.get("dtype"))
+            if out is not None:
+                return out
+        return NotImplemented
+
+
+def _same_source(a, b):
+    """Whether two tensors are the same value of the same autograd graph: one object, or one output of one node."""
+    if a is b:
+        return True
+    return (isinstance(a, torch.Tensor) and isinstance(b, torch.Tensor) and a.grad_fn is not None and
+            a.grad_fn is b.grad_fn and a.output_nr == b.output_nr)
+
+
+def _made_by(t, node_name, *inputs):
+    """Whether autograd recorded tensor t as node_name(inputs) -- each input a tensor, or a nested (node_name,
+    inputs...) tuple for an intermediate that nothing else holds."""
+    fn = t if not isinstance(t, torch.Tensor) else t.grad_fn
+    if fn is None or fn.name() != node_name or len(fn.next_functions) < len(inputs):
+        return False
+    for (nxt, nr), want in zip(fn.next_functions, inputs):
+        if isinstance(want, tuple):
+            if nxt is None or not _made_by(nxt, *want):
+                return False
+        elif want.grad_fn is not None:
+            if nxt is not want.grad_fn or nr != want.output_nr:
+                return False
+        elif nxt is None or getattr(nxt, "variable", None) is not want:     # a leaf that requires grad
+            return False
+    return True
+
+
+def beta_kl_operands(expr):
+    """(rows, qa, qb) when `expr` is, node for node, what torch.distributions.kl._kl_beta_beta(p, q) builds for
+    p = BetaDist(alpha half, beta half) of one 4-D handle and q = BetaDist(qa, qb):
+        sp = a + b;  sq = qa + qb
+        t1 = qa.lgamma() + qb.lgamma() + sp.lgamma();  t2 = a.lgamma() + b.lgamma() + sq.lgamma()
+        t3 = (a - qa) * digamma(a);  t4 = (b - qb) * digamma(b);  t5 = (sq - sp) * digamma(sp)
+        t1 - t2 + t3 + t4 + t5
+    The query-side operands are plain tensors when they reach the expression; that they are lgamma(qa) + lgamma(qb),
+    lgamma(qa + qb) and qa + qb of the very qa and qb the halves meet in t3 and t4 is read off the autograd graph
+    torch recorded for them (queries that carry no graph -- evaluation under no_grad -- are not recognised).
+    None otherwise."""
+    def node(x, op, n):
+        return x.args if isinstance(x, _Sym) and x.op == op and len(x.args) == n else None
+
+    def half(x, which):
+        return isinstance(x, _LazyHalf) and x.which == which and not x.unit and x.rows is expr.handle
+
+    def is_sp(x):
+        args = node(x, "add", 2)
+        return args is not None and half(args[0], 0) and half(args[1], 1)
+
+    def unary(x, op, inner):
+        args = node(x, op, 1)
+        return args is not None and inner(args[0])
+
+    plain = lambda t: isinstance(t, torch.Tensor) and not _is_lazy(t)
+    try:
+        s4, t5 = node(expr, "add", 2)
+        s3, t4 = node(s4, "add", 2)
+        s2, t3 = node(s3, "add", 2)
+        t1, t2 = node(s2, "sub", 2)
+        x, lg_sp = node(t1, "add", 2)                     # (lgamma(qa) + lgamma(qb)) + lgamma(sp)
+        lg_ab, y = node(t2, "add", 2)                     # (lgamma(a) + lgamma(b)) + lgamma(sq)
+        lg_a, lg_b = node(lg_ab, "add", 2)
+        d_a, psi_a = node(t3, "mul", 2)
+        d_b, psi_b = node(t4, "mul", 2)
+        d_s, psi_s = node(t5, "mul", 2)
+        a0, qa = node(d_a, "sub", 2)
+        b0, qb = node(d_b, "sub", 2)
+        sq, sp2 = node(d_s, "sub", 2)
+    except TypeError:                                      # some node was not of the expected kind
+        return None
+    a_is = lambda v: half(v, 0)
+    b_is = lambda v: half(v, 1)
+    if not (unary(lg_sp, "lgamma", is_sp) and unary(lg_a, "lgamma", a_is) and unary(lg_b, "lgamma", b_is) and
+            unary(psi_a, "digamma", a_is) and unary(psi_b, "digamma", b_is) and unary(psi_s, "digamma", is_sp) and
+            a_is(a0) and b_is(b0) and is_sp(sp2) and all(plain(t) for t in (x, y, qa, qb, sq))):
+        return None
+    if qa.shape != qb.shape or not _LazyExpr._query(qa, a0) or not _LazyExpr._query(qb, b0):
+        return None
+    if not (_made_by(sq, "AddBackward0", qa, qb) and _made_by(y, "LgammaBackward0", ("AddBackward0", qa, qb)) and
+            _made_by(x, "AddBackward0", ("LgammaBackward0", qa), ("LgammaBackward0", qb))):
+        return None
+    handle = expr.handle
+    return handle._like((handle.shape[0], handle.shape[2], handle.shape[3])), qa, qb
 
 
 class _LazyExpr(_Delegating):

@@ -87,6 +87,20 @@ class Beta(Reasoner):
         return torch.max(logit, dim=1)[0]
 
 
+class BetaNative(Beta):            # native_cal_logit, beta.py:293-301: torch's own Beta-Beta KL routine on the halves
+    def cal_logit(self, entity_embedding, entity_feat, query_embedding):
+        import torch.distributions.kl as torch_kl
+        from smore_amd.torchext.ext_ops import BetaDist
+        assert entity_feat is None
+        alpha_embedding, beta_embedding = torch.chunk(entity_embedding.unsqueeze(1), 2, dim=-1)
+        entity_dist = BetaDist(alpha_embedding, beta_embedding)
+        query_dist = BetaDist(*query_embedding)
+        kld = torch_kl._kl_beta_beta(entity_dist, query_dist)
+        logit = self.gamma - torch.norm(kld, p=1, dim=-1)
+        logit = torch.max(logit, dim=1)[0]
+        return logit
+
+
 class Complex(Reasoner):                           # complex.py:140-148 without its optional normalisation
     def cal_logit(self, entity_embedding, entity_feat, query_embedding):
         from smore_amd.torchext.ext_ops import complex_sim
@@ -219,13 +233,14 @@ CASES = {
     "complex_native": (ComplexNative, (), "complex", 2, 2, 0.0, 0.0),
     "complex_norm_native": (ComplexNativeNorm, (), "complex", 2, 2, 0.0, 0.0),
     "distmult_norm_native": (DistmultNativeNorm, (), "distmult", 1, 1, 0.0, 0.0),
+    "beta_native": (BetaNative, (), "beta_kl", 2, 2, 60.0, 0.0),
 }
 
 
 def _table_and_queries(name, n, d, b, u, rng):
     mul = CASES[name][4]
     n_q = CASES[name][3]
-    if name == "beta":
+    if name.startswith("beta"):
         table = rng.standard_normal((n, 2 * d)) * 1.5           # raw values; the regularizer clamps some
         pos = lambda *s: np.clip(1 + rng.standard_normal(s), 0.05, 1e9)
         qs = [pos(b, u, 1, d) for _ in range(n_q)]
@@ -239,12 +254,12 @@ def _table_and_queries(name, n, d, b, u, rng):
 
 
 def _oracle_branch_logits(name, table, ids, qs, gamma, cen):
-    return oracle_union_logits(CASES[name][2], table, ids, qs, gamma, cen, regularizer=name == "beta",
+    return oracle_union_logits(CASES[name][2], table, ids, qs, gamma, cen, regularizer=name.startswith("beta"),
                                norm="_norm" in name)
 
 
 def _oracle_grads(name, table, ids, qs, rows, logit, gout, cen):
-    return oracle_union_grads(CASES[name][2], table, ids, qs, rows, logit, gout, cen, regularizer=name == "beta",
+    return oracle_union_grads(CASES[name][2], table, ids, qs, rows, logit, gout, cen, regularizer=name.startswith("beta"),
                               norm="_norm" in name)
 
 
@@ -547,11 +562,11 @@ def test_anchor_lookups_join_the_fused_records_in_one_update(name, monkeypatch):
     rng = np.random.default_rng(23)
     f32 = lambda a: np.asarray(a).astype(np.float32).astype(np.float64)
     table, _ = _table_and_queries(name, n, d, b, 1, rng)
-    if name == "beta":
+    if name.startswith("beta"):
         rel = [f32(rng.uniform(0.5, 1.5, (b, d))) for _ in range(2)]           # positive scales keep alpha, beta > 0
     else:
         rel = [f32(rng.uniform(-0.07, 0.07, (b, d))) for _ in range(n_q)]
-        if name == "box":
+        if name in ("box", "box_native"):
             rel[1] = np.abs(rel[1])
     emb = SparseEmbedding(n, mul * d).cuda()
     with torch.no_grad():
@@ -562,7 +577,7 @@ def test_anchor_lookups_join_the_fused_records_in_one_update(name, monkeypatch):
 
     def embed_query(rows, rels, lib):
         """rows [B, mul*d] -> the model's query tensors [B, d] each (lib = torch or numpy)."""
-        if name == "beta":
+        if name.startswith("beta"):
             rows = lib.clip(rows + 1.0, 0.05, 1e9) if lib is np else torch.clamp(rows + 1.0, 0.05, 1e9)
             return [rows[:, :d] * rels[0], rows[:, d:] * rels[1]]
         if mul == 2:
@@ -597,7 +612,7 @@ def test_anchor_lookups_join_the_fused_records_in_one_update(name, monkeypatch):
         gr_n, gq_n = _oracle_grads(name, w, neg, qs, rows_n, o_ln, gn, cen)
         gq = [(a + c).reshape(b, d) for a, c in zip(gq_p, gq_n)]              # d loss / d query tensors
         raw = orc.gather(w, anchor)
-        if name == "beta":
+        if name.startswith("beta"):
             reg = np.clip(raw + 1.0, 0.05, 1e9)
             mask = (raw + 1 >= 0.05) & (raw + 1 <= 1e9)
             g_anchor = np.concatenate([gq[0] * rel[0], gq[1] * rel[1]], axis=1) * mask

@@ -69,6 +69,11 @@ def _textbook(model, e, queries, cen):
         return (re * queries[0] + im * queries[1]).sum(-1)
     if model == "distmult":
         return (e * queries[0]).sum(-1)
+    if model == "beta_kl":
+        ea, eb = torch.chunk(e, 2, dim=-1)
+        D = torch.distributions
+        ea, eb, qa, qb = torch.broadcast_tensors(ea, eb, queries[0], queries[1])
+        return D.kl.kl_divergence(D.Beta(ea, eb), D.Beta(qa, qb)).sum(-1)
     raise AssertionError(model)
 
 
@@ -296,6 +301,76 @@ def test_native_cal_logit_bodies_become_one_fused_request(body, model, n_q, mul,
     want = body(gamma, cen, opt.sparse_embed.embedding[ids].view(be, k, -1), qs)
     torch.testing.assert_close(logit + 0.0, want, rtol=1e-5, atol=1e-6)        # (the first use scores the placeholder)
     assert opt.looked_up == [] and opt.scored == [(model, (be, k), 12.0, cen, None)]
+
+
+def _native_beta(gamma, entity_embedding, query_embedding):
+    """native_cal_logit of models/beta.py:293-301"""
+    import torch.distributions.kl as torch_kl
+    alpha_embedding, beta_embedding = torch.chunk(entity_embedding.unsqueeze(1), 2, dim=-1)
+    entity_dist = ext_ops.BetaDist(alpha_embedding, beta_embedding)
+    query_dist = ext_ops.BetaDist(*query_embedding)
+    kld = torch_kl._kl_beta_beta(entity_dist, query_dist)
+    logit = gamma - torch.norm(kld, p=1, dim=-1)
+    return torch.max(logit, dim=1)[0]
+
+
+@pytest.mark.parametrize("leaf_queries", [True, False])
+@pytest.mark.parametrize("branches", [1, 2])
+def test_native_beta_body_is_recognised_node_for_node(leaf_queries, branches):
+    """torch's own Beta-Beta KL routine on the halves of the regularized handle: one request for beta_kl with the
+    clamp prologue; the query-side operands are identified through the autograd graph (leaves, and two outputs of one
+    chunk node as the query nets produce them)."""
+    n, d, b, k = 40, 5, 3, 4
+    opt = RecordingOptimizer(n, 2 * d)
+    ids = torch.randint(0, n, (b * k,), generator=torch.Generator().manual_seed(41))
+    g = torch.Generator().manual_seed(42)
+    if leaf_queries:
+        qs = [(torch.rand((b, branches, 1, d), generator=g) + 0.1).requires_grad_(True) for _ in range(2)]
+    else:
+        both = (torch.rand((b, branches, 1, 2 * d), generator=g) + 0.1).requires_grad_(True)
+        qs = list(torch.chunk(both * 1.0, 2, dim=-1))
+    gamma = torch.nn.Parameter(torch.Tensor([60.0]), requires_grad=False)
+    reg = lambda x: torch.clamp(x + 1.0, 0.05, 1e9)                       # Regularizer(1, 0.05, 1e9), beta.py:210
+    logit = _native_beta(gamma, reg(LazyRows(opt, ids, "negative_entity").view(b, k, -1)), qs)
+    want = _native_beta(gamma, reg(opt.sparse_embed.embedding[ids].view(b, k, -1)), qs)
+    torch.testing.assert_close(logit + 0.0, want.detach(), rtol=1e-5, atol=1e-5)
+    assert opt.looked_up == [] and opt.scored == [("beta_kl", (b, k), 60.0, 0.0, (1.0, 0.05, 1e9))]
+
+
+def test_expressions_that_only_resemble_the_beta_routine_are_evaluated_by_torch():
+    """Another tensor in the place of lgamma(qa + qb), queries without a graph, a swapped pair of halves: no request,
+    the torch value."""
+    import torch.distributions.kl as torch_kl
+    n, d, b, k = 40, 5, 3, 4
+    ids = torch.randint(0, n, (b * k,), generator=torch.Generator().manual_seed(43))
+    g = torch.Generator().manual_seed(44)
+    reg = lambda x: torch.clamp(x + 1.0, 0.05, 1e9)
+    qa, qb = [(torch.rand((b, 1, 1, d), generator=g) + 0.1).requires_grad_(True) for _ in range(2)]
+
+    def kl_with(p1, p0, q1, q0, y=None):          # torch's routine with its lgamma(sq) replaceable
+        sp, sq = p1 + p0, q1 + q0
+        t1 = q1.lgamma() + q0.lgamma() + sp.lgamma()
+        t2 = p1.lgamma() + p0.lgamma() + (sq.lgamma() if y is None else y)
+        return t1 - t2 + (p1 - q1) * torch.digamma(p1) + (p0 - q0) * torch.digamma(p0) + (sq - sp) * torch.digamma(sp)
+
+    cases = {"other tensor": lambda a, c: kl_with(a, c, qa, qb, y=(qa * qb).lgamma()),
+             "no graph": lambda a, c: kl_with(a, c, qa.detach(), qb.detach()),
+             "halves swapped": lambda a, c: kl_with(c, a, qa, qb),
+             "queries swapped in one term": lambda a, c: kl_with(a, c, qa, qb) + ((a - qb) * torch.digamma(a) - (a - qa) * torch.digamma(a))}
+    for name, f in cases.items():
+        opt = RecordingOptimizer(n, 2 * d)
+        rows = reg(opt.sparse_embed.embedding[ids].view(b, k, -1)).unsqueeze(1)
+        handle = reg(LazyRows(opt, ids, None).view(b, k, -1)).unsqueeze(1)
+        got = torch.norm(f(*torch.chunk(handle, 2, dim=-1)), p=1, dim=-1)
+        want = torch.norm(f(*torch.chunk(rows, 2, dim=-1)), p=1, dim=-1)
+        assert isinstance(got, torch.Tensor) and opt.scored == [], name
+        torch.testing.assert_close(got, want, rtol=1e-6, atol=1e-6)
+    # and the routine itself on these operands is recognised
+    opt = RecordingOptimizer(n, 2 * d)
+    handle = reg(LazyRows(opt, ids, None).view(b, k, -1)).unsqueeze(1)
+    a, c = torch.chunk(handle, 2, dim=-1)
+    kld = torch_kl._kl_beta_beta(ext_ops.BetaDist(a, c), ext_ops.BetaDist(qa, qb))
+    assert not isinstance(torch.norm(kld, p=1, dim=-1), torch.Tensor)
 
 
 def test_native_intermediates_put_to_other_uses_are_the_tensors_they_stand_for():
