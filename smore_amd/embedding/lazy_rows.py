@@ -516,7 +516,10 @@ class _Sym(_Delegating):
 
     def _l1(self, p, dim, keepdim, dtype):
         if p in (1, 1.0) and dim in (-1, self.dim() - 1) and not keepdim and dtype is None:
-            found = beta_kl_operands(self)
+            try:
+                found = beta_kl_operands(self)
+            except (AttributeError, TypeError, ValueError, RuntimeError):   # an autograd graph of a shape this code
+                found = None                                                # does not know: torch evaluates the expression
             if found is not None:
                 return lazy_dist("beta_kl", *found)
         return None
