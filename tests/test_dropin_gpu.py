@@ -493,6 +493,77 @@ def test_native_bodies_with_shared_negatives_give_the_bits_of_the_ext_ops_form(n
         assert torch.equal(a, r)
 
 
+@pytest.mark.parametrize("need_norm", [False, True])
+def test_complex_native_body_with_shared_negatives_takes_its_matrix_product_branch(need_norm):
+    """What every ComplEx script of the reference runs: native_cal_logit (complex.py:169-187) with --share_negative.
+    The positives [B] meet the queries' own batch and stay on the fused scorer; the shared negatives [1, K] take the
+    model's torch.mm branch, for which the halves' values are needed: one plain lookup of K rows, torch's matrix
+    products, gradient rows.  apply_grad merges the fused record and the rows in one plan.  Against the oracle."""
+    from smore_amd.embedding.embed_optimizer import AdamEmbedOptimizer
+    from smore_amd.embedding.sparse_embed import SparseEmbedding
+    F = torch.nn.functional
+    n, d, b, k, lr = 300, 24, 6, 40, 1e-3
+    rng = np.random.default_rng(91)
+    name = "complex_norm" if need_norm else "complex"
+    table, qs = _table_and_queries(name, n, d, b, 1, rng)
+    emb = SparseEmbedding(n, 2 * d).cuda()
+    with torch.no_grad():
+        emb.embedding.copy_(torch.tensor(table, dtype=torch.float32))
+    opt = AdamEmbedOptimizer(types.SimpleNamespace(optim_mode="(aggr,adam,gpu,False,5)", share_optim_stats=True), emb, 0)
+    embed_norm = (lambda x: F.normalize(x, p=2, dim=-1)) if need_norm else (lambda x: x)
+
+    def native_cal_logit(entity_embedding, query_embedding):            # complex.py:169-187
+        query_re_embedding, query_im_embedding = query_embedding
+        entity_re_embedding, entity_im_embedding = torch.chunk(entity_embedding.unsqueeze(1), 2, dim=-1)
+        if need_norm:
+            entity_re_embedding, entity_im_embedding = embed_norm(entity_re_embedding), embed_norm(entity_im_embedding)
+        if entity_re_embedding.shape[0] == query_re_embedding.shape[0]:
+            logit = (entity_re_embedding * query_re_embedding + entity_im_embedding * query_im_embedding).sum(dim=-1)
+            logit = torch.max(logit, dim=1)[0]
+        else:
+            bsize = query_re_embedding.shape[0]
+            nent = entity_re_embedding.shape[2]
+            embed_dim = query_re_embedding.shape[-1]
+            entity_re_embedding = entity_re_embedding.view(nent, embed_dim)
+            entity_im_embedding = entity_im_embedding.view(nent, embed_dim)
+            query_re_embedding = query_re_embedding.view(bsize, embed_dim)
+            query_im_embedding = query_im_embedding.view(bsize, embed_dim)
+            logit = torch.mm(query_re_embedding, entity_re_embedding.t()) + torch.mm(query_im_embedding, entity_im_embedding.t())
+        return logit
+
+    t_qs = [torch.tensor(q, dtype=torch.float32, device="cuda", requires_grad=True) for q in qs]
+    pos, neg = rng.integers(0, n, b), rng.integers(0, n // 3, (1, k))
+    neg[0, 4] = pos[1]
+    gp = rng.standard_normal((b, 1)).astype(np.float32).astype(np.float64)
+    gn = rng.standard_normal((b, k)).astype(np.float32).astype(np.float64)
+    opt.zero_grad()
+    p_rows = emb(torch.tensor(pos, device="cuda"), "positive_entity")
+    n_rows = emb(torch.tensor(neg, device="cuda").view(-1), "negative_entity")
+    lp = native_cal_logit(p_rows.unsqueeze(1), t_qs)
+    ln = native_cal_logit(n_rows.view(1, k, -1), t_qs)
+    assert lp.shape == (b, 1) and ln.shape == (b, k)
+    ((lp * torch.tensor(gp, dtype=torch.float32, device="cuda")).sum() +
+     (ln * torch.tensor(gn, dtype=torch.float32, device="cuda")).sum()).backward()
+    assert len(opt.fused_list) == 1 and len(opt.grad_list) == 1 and opt.stats["materialized_lookups"] == 1
+    opt.apply_grad(lr)
+
+    neg_full = np.broadcast_to(neg, (b, k))
+    o_lp, rows_p = _oracle_branch_logits(name, table, pos.reshape(b, 1), qs, 0.0, 0.0)
+    o_ln, rows_n = _oracle_branch_logits(name, table, neg_full, qs, 0.0, 0.0)
+    assert_close(lp.detach().cpu().numpy(), o_lp[:, 0], REL_F32, "positive logits")
+    assert_close(ln.detach().cpu().numpy(), o_ln[:, 0], REL_F32, "negative logits")
+    gr_p, gq_p = _oracle_grads(name, table, pos.reshape(b, 1), qs, rows_p, o_lp, gp, 0.0)
+    gr_n, gq_n = _oracle_grads(name, table, neg_full, qs, rows_n, o_ln, gn, 0.0)
+    for t, a, c in zip(t_qs, gq_p, gq_n):
+        assert_close(t.grad.cpu().numpy(), a + c, REL_F32, "query gradient")
+    uniq, inverse, _, _ = orc.merge_indices(np.concatenate([pos.reshape(-1), neg_full.reshape(-1)]))
+    merged = orc.merge_grads(np.concatenate([gr_p, gr_n]), inverse, uniq.size)
+    w, m, v = table.copy(), np.zeros_like(table), np.zeros_like(table)
+    orc.adam_rows(w, m, v, uniq, merged, lr, 1)
+    assert_close(emb.state_sum_fo.cpu().numpy()[uniq], m[uniq], REL_F32, "first moment")
+    assert_adam_weights(emb.embedding.detach().cpu().numpy(), w, merged, uniq, lr, "weights")
+
+
 def test_inverse_query_call_sequence_runs_on_the_reverse_layout():
     """Inverse ('<') queries, kg_reasoning.py:306-336: the TAIL entity is looked up and becomes the 'entity' operand
     [B,1,D] (embed_reverse_query, :252-255), while the negatives go through the relation projection
