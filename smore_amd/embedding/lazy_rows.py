@@ -18,8 +18,9 @@ scorer has no model for, or any other use of the rows (cal_reg, indexing, printi
 lookup (EmbedLookupFunc) and the dense operators, with the reference's results.
 
 The native_cal_logit bodies (--logit_impl native, the default: config.py:119) write the same logits with torch
-operators on the rows: box.py:147-155, vec.py:78-83, rotate.py:125-135, distmult.py:126-133, the per-query
-branch of complex.py:169-177, and beta.py:293-301 (torch's own Beta-Beta KL routine on the halves: `_Sym`).  Their intermediates on a handle are
+operators on the rows: box.py:147-155, vec.py:78-83, rotate.py:125-135, distmult.py:126-133, both branches
+of complex.py:169-186 (`_LazyMat` for the shared negatives' torch.mm), and beta.py:293-301 (torch's own Beta-Beta
+KL routine on the halves: `_Sym`).  Their intermediates on a handle are
 `_LazyExpr` nodes (rows.unsqueeze(1) - center, its abs, relu(abs - offset), min(abs, offset), the stacked halves'
 modulus, the products with the queries); torch.norm(.., p=1, dim=-1) or .sum(dim=-1) of the right node is the same
 `LazyLogit` term the ext_ops call would have returned.  The fused scorer then computes them with ITS conventions where the two forms differ on a
@@ -401,6 +402,14 @@ class _LazyHalf(_Delegating):
         node = _Sym.make("add", self, other)
         return torch.add(self.materialize(), _resolve(other)) if node is None else node
 
+    def view(self, *shape):            # entity_re_embedding.view(nent, embed_dim) of complex.py:181-182
+        if len(shape) == 1 and isinstance(shape[0], (tuple, list, torch.Size)):
+            shape = tuple(shape[0])
+        if (self.dim() == 4 and tuple(self.shape[:2]) == (1, 1) and tuple(shape) == tuple(self.shape[2:]) and
+                self.rows.pending_add is None and (self.rows.reg is None or self.unit)):
+            return _LazyMat(self, False)
+        return self.materialize().view(*shape)
+
     def lgamma(self):
         node = _Sym.make("lgamma", self)
         return self.materialize().lgamma() if node is None else node
@@ -412,6 +421,74 @@ class _LazyHalf(_Delegating):
     def materialize(self):
         half = torch.chunk(self.rows.materialize(), 2, dim=-1)[self.which]
         return torch.nn.functional.normalize(half, p=2, dim=-1) if self.unit else half
+
+
+class _LazyMat(_Delegating):
+    """The shared-negative branch of ComplEx's native_cal_logit (complex.py:178-186): one half of a [1, 1, K, 2h]
+    handle viewed as the matrix [K, h] (`product` None, `transposed` False), its transpose [h, K], and
+    torch.mm(query [B, h], that transpose) -> [B, K] (`product` = the query matrix).  The sum of the two halves'
+    products is the ComplEx logit of the K shared rows against every query: the LazyLogit term of ext_ops.complex_sim,
+    its single branch taken."""
+
+    def __init__(self, half, transposed, product=None):
+        self.half, self.transposed, self.product = half, transposed, product
+        k, h = half.shape[2], half.shape[3]
+        self.shape = torch.Size((product.shape[0], k) if product is not None else ((h, k) if transposed else (k, h)))
+
+    device = property(lambda self: self.half.device)
+    dtype = property(lambda self: self.half.dtype)
+    requires_grad = True
+    is_cuda = True
+
+    def dim(self):
+        return 2
+
+    ndim = property(dim)
+
+    def size(self, d=None):
+        return self.shape if d is None else self.shape[d]
+
+    def t(self):
+        if self.product is None:
+            return _LazyMat(self.half, not self.transposed)
+        return self.materialize().t()
+
+    def materialize(self):
+        k, h = self.half.shape[2], self.half.shape[3]
+        m = self.half.materialize().view(k, h)
+        if self.product is not None:
+            return torch.mm(self.product, m.t())
+        return m.t() if self.transposed else m
+
+    def __add__(self, other):
+        a, b = self, other
+        if (isinstance(b, _LazyMat) and a.product is not None and b.product is not None and a.half.which == 0 and
+                b.half.which == 1 and a.half.rows is b.half.rows and a.half.unit == b.half.unit and
+                a.product.shape == b.product.shape):
+            handle = a.half.rows                                   # [1, 1, K, 2h]
+            rows = handle._like((1, handle.shape[2], handle.shape[3]))
+            if a.half.unit:
+                rows.reg = UNIT_HALVES
+            bq, h = a.product.shape
+            term = lazy_dist("complex", rows, a.product.view(bq, 1, 1, h), b.product.view(bq, 1, 1, h))
+            if term is not None:
+                return torch.max(term, dim=1)[0]                   # one branch: [B, 1, K] -> [B, K]
+        return torch.add(self.materialize(), _resolve(other))
+
+    @classmethod
+    def _try_lazy(cls, func, args, kwargs):
+        name = _func_name(func)
+        if name == "mm" and len(args) == 2 and not kwargs:
+            q, m = args
+            if (isinstance(m, _LazyMat) and m.product is None and m.transposed and isinstance(q, torch.Tensor) and
+                    not _is_lazy(q) and q.dim() == 2 and q.shape[1] == m.shape[0] and q.dtype == m.dtype and
+                    q.device == m.device):
+                return _LazyMat(m.half, True, q)
+        if name in ("add", "__add__") and len(args) == 2 and not kwargs and isinstance(args[0], _LazyMat):
+            return args[0].__add__(args[1])
+        if name == "t" and len(args) == 1 and isinstance(args[0], _LazyMat):
+            return args[0].t()
+        return NotImplemented
 
 
 class _Sym(_Delegating):

@@ -496,9 +496,9 @@ def test_native_bodies_with_shared_negatives_give_the_bits_of_the_ext_ops_form(n
 @pytest.mark.parametrize("need_norm", [False, True])
 def test_complex_native_body_with_shared_negatives_takes_its_matrix_product_branch(need_norm):
     """What every ComplEx script of the reference runs: native_cal_logit (complex.py:169-187) with --share_negative.
-    The positives [B] meet the queries' own batch and stay on the fused scorer; the shared negatives [1, K] take the
-    model's torch.mm branch, for which the halves' values are needed: one plain lookup of K rows, torch's matrix
-    products, gradient rows.  apply_grad merges the fused record and the rows in one plan.  Against the oracle."""
+    The positives [B] meet the queries' own batch; the shared negatives [1, K] take the model's torch.mm branch (the
+    halves viewed as matrices, transposed, multiplied by the query matrices, added).  The handle follows both: no
+    lookup is materialised and the step leaves the two fused records of the ext_ops form.  Against the oracle."""
     from smore_amd.embedding.embed_optimizer import AdamEmbedOptimizer
     from smore_amd.embedding.sparse_embed import SparseEmbedding
     F = torch.nn.functional
@@ -544,7 +544,8 @@ def test_complex_native_body_with_shared_negatives_takes_its_matrix_product_bran
     assert lp.shape == (b, 1) and ln.shape == (b, k)
     ((lp * torch.tensor(gp, dtype=torch.float32, device="cuda")).sum() +
      (ln * torch.tensor(gn, dtype=torch.float32, device="cuda")).sum()).backward()
-    assert len(opt.fused_list) == 1 and len(opt.grad_list) == 1 and opt.stats["materialized_lookups"] == 1
+    assert len(opt.fused_list) == 2 and not opt.grad_list and opt.stats["materialized_lookups"] == 0
+    assert opt.stats["dense_fallbacks"] == 0
     opt.apply_grad(lr)
 
     neg_full = np.broadcast_to(neg, (b, k))

@@ -373,6 +373,40 @@ def test_expressions_that_only_resemble_the_beta_routine_are_evaluated_by_torch(
     assert not isinstance(torch.norm(kld, p=1, dim=-1), torch.Tensor)
 
 
+@pytest.mark.parametrize("norm", [False, True])
+def test_complex_matrix_product_branch_for_shared_negatives(norm):
+    """complex.py:178-186: halves of the [1, K] rows viewed as [K, h], transposed, torch.mm with the query matrices,
+    added -- one request for the K shared ids; the pieces put to other uses are torch's values."""
+    n, d, b, k = 40, 6, 3, 5
+    opt = RecordingOptimizer(n, 2 * d)
+    ids = torch.randint(0, n, (k,), generator=torch.Generator().manual_seed(51))
+    q_re, q_im = _queries(b, 1, d, 2, 52)
+    embed_norm = _Normalizer() if norm else (lambda x: x)
+
+    def branch(entity_embedding):
+        re, im = torch.chunk(entity_embedding.unsqueeze(1), 2, dim=-1)
+        re, im = embed_norm(re), embed_norm(im)
+        assert re.shape[0] != q_re.shape[0]
+        re, im = re.view(k, d), im.view(k, d)
+        return torch.mm(q_re.view(b, d), re.t()) + torch.mm(q_im.view(b, d), im.t())
+
+    logit = branch(LazyRows(opt, ids, "negative_entity").view(1, k, -1))
+    want = branch(opt.sparse_embed.embedding[ids].view(1, k, -1))
+    assert tuple(logit.shape) == (b, k)
+    torch.testing.assert_close(logit + 0.0, want, rtol=1e-5, atol=1e-6)
+    assert opt.looked_up == [] and opt.scored == [("complex", (1, k), 0.0, 0.0, "unit_halves" if norm else None)]
+    # pieces on their own
+    opt2 = RecordingOptimizer(n, 2 * d)
+    rows = opt2.sparse_embed.embedding[ids].view(1, 1, k, -1)
+    h_re, h_im = torch.chunk(LazyRows(opt2, ids, None).view(1, k, -1).unsqueeze(1), 2, dim=-1)
+    t_re, t_im = torch.chunk(rows, 2, dim=-1)
+    assert torch.equal(h_re.view(k, d).t() * 1.0, t_re.view(k, d).t())
+    assert torch.equal(torch.mm(q_re.view(b, d), h_re.view(k, d).t()) * 1.0, torch.mm(q_re.view(b, d), t_re.view(k, d).t()))
+    assert torch.equal(torch.mm(q_re.view(b, d), h_re.view(k, d).t()) + torch.mm(q_im.view(b, d), h_re.view(k, d).t()),
+                       torch.mm(q_re.view(b, d), t_re.view(k, d).t()) + torch.mm(q_im.view(b, d), t_re.view(k, d).t()))
+    assert torch.equal(h_im.view(k, d) * 1.0, t_im.view(k, d)) and opt2.scored == []
+
+
 def test_native_intermediates_put_to_other_uses_are_the_tensors_they_stand_for():
     n, d, b, k = 40, 6, 3, 5
     F = torch.nn.functional
