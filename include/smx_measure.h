@@ -25,6 +25,13 @@ int smx_measure_backward_fused(int parts, int model, void* stream, const smx_pla
                                const smx_opt_params* adam, void* workspace, size_t workspace_bytes,
                                const void* fwd_codes, size_t fwd_codes_bytes);
 
+/* No counterpart in the reference.  Two HIP events (hipEvent_t, created with timing) that the NEXT
+ * smx_score_backward_fused / smx_measure_backward_fused call of this host thread records on the caller's stream
+ * immediately before and after its query-gradient kernel, so that a harness can time that kernel in its place
+ * inside the call (the entity pass still follows it) instead of bracketing a call that launches nothing else.
+ * The events are used once; NULL, NULL clears a pair that was set and not used. */
+int smx_measure_query_kernel_events(void* before, void* after);
+
 /* No counterpart in the reference.  smx_plan_build with the two knobs a test needs to see a plan give up while
  * every kernel still ends normally:
  *   spin_limit    polls a workgroup of the sort makes before it stops waiting for another one (the library

@@ -143,6 +143,7 @@ MEASURE_SIGNATURES = {
     "smx_measure_backward_fused": (_i, [_i] + SIGNATURES["smx_score_backward_fused"][1]),
     # the arguments of smx_plan_build, then spin_limit, force_abort
     "smx_measure_plan_build": (_i, SIGNATURES["smx_plan_build"][1] + [_c.c_uint, _i]),
+    "smx_measure_query_kernel_events": (_i, [_vp, _vp]),
 }
 
 

@@ -565,6 +565,18 @@ int smx_score_backward_entity_union(int model, void* stream, const smx_plan_view
 namespace smx {
 
 // parts: bit 0 the query-gradient kernel, bit 1 the entity pass (3 for every caller but the measuring entry point)
+// smx_measure_query_kernel_events: the pair the next backward call of this thread records around its query kernel
+static thread_local hipEvent_t g_query_before = nullptr, g_query_after = nullptr;
+
+static int dispatch_query_kernel(int model, hipStream_t st, const ScoreArgs& A, int vec, int nit) {
+  hipEvent_t before = g_query_before, after = g_query_after;
+  g_query_before = g_query_after = nullptr;
+  if (before && hipEventRecord(before, st) != hipSuccess) return fail(SMX_ERR_HIP, "cannot record the measuring event");
+  const int rc = dispatch_model(model, st, A, vec, nit, false);
+  if (after && hipEventRecord(after, st) != hipSuccess) return fail(SMX_ERR_HIP, "cannot record the measuring event");
+  return rc;
+}
+
 static int backward_fused(int parts, int model, void* stream, const smx_plan_view* plan, float* table, size_t n_rows,
                           const int64_t* idx, const float* q1, const float* q2, const float* score,
                           const float* gscore, float* gq1, float* gq2, size_t B, size_t K, size_t dim,
@@ -642,7 +654,7 @@ static int backward_fused(int parts, int model, void* stream, const smx_plan_vie
     std::lock_guard<std::mutex> one_call(side->in_use);
     if (hipEventRecord(side->fork, st) != hipSuccess || hipStreamWaitEvent(side->stream, side->fork, 0) != hipSuccess)
       return fail(SMX_ERR_HIP, "fork to the side stream failed");
-    int rc = (parts & 1) ? dispatch_model(model, st, A, vec, nit, false) : SMX_OK;
+    int rc = (parts & 1) ? dispatch_query_kernel(model, st, A, vec, nit) : SMX_OK;
     if (rc == SMX_OK && (parts & 2))
       rc = entity_backward(model, side->stream, plan, table, n_rows, q1, q2, score, gscore, B, K, dim, params, merged, m,
                            v, adam, workspace, workspace_bytes, singles_here ? 1 : 0, codes, vec, nit);
@@ -652,7 +664,7 @@ static int backward_fused(int parts, int model, void* stream, const smx_plan_vie
     return rc;
   }
   if (parts & 1)
-    if (int rc = dispatch_model(model, as_stream(stream), A, vec, nit, false)) return rc;
+    if (int rc = dispatch_query_kernel(model, as_stream(stream), A, vec, nit)) return rc;
   if (!(parts & 2)) return SMX_OK;
   return entity_backward(model, stream, plan, table, n_rows, q1, q2, score, gscore, B, K, dim, params, merged, m, v,
                          adam, workspace, workspace_bytes, singles_here ? 1 : 0, codes, vec, nit);
@@ -670,6 +682,13 @@ int smx_score_backward_fused(int model, void* stream, const smx_plan_view* plan,
                              const void* fwd_codes, size_t fwd_codes_bytes) {
   return smx::backward_fused(3, model, stream, plan, table, n_rows, idx, q1, q2, score, gscore, gq1, gq2, B, K, dim, params,
                              merged, m, v, adam, workspace, workspace_bytes, fwd_codes, fwd_codes_bytes);
+}
+
+int smx_measure_query_kernel_events(void* before, void* after) {
+  if ((before == nullptr) != (after == nullptr)) return smx::fail(SMX_ERR_ARG, "two events, or none");
+  smx::g_query_before = static_cast<hipEvent_t>(before);
+  smx::g_query_after = static_cast<hipEvent_t>(after);
+  return SMX_OK;
 }
 
 int smx_measure_backward_fused(int parts, int model, void* stream, const smx_plan_view* plan, float* table, size_t n_rows,
