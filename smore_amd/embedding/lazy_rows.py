@@ -660,7 +660,7 @@ def beta_kl_operands(expr):
         t1 - t2 + t3 + t4 + t5
     The query-side operands are plain tensors when they reach the expression; that they are lgamma(qa) + lgamma(qb),
     lgamma(qa + qb) and qa + qb of the very qa and qb the halves meet in t3 and t4 is read off the autograd graph
-    torch recorded for them (queries that carry no graph -- evaluation under no_grad -- are not recognised).
+    torch recorded for them; where nothing carries a graph (evaluation under no_grad) they are compared by value.
     None otherwise."""
     def node(x, op, n):
         return x.args if isinstance(x, _Sym) and x.op == op and len(x.args) == n else None
@@ -701,8 +701,13 @@ def beta_kl_operands(expr):
         return None
     if qa.shape != qb.shape or not _LazyExpr._query(qa, a0) or not _LazyExpr._query(qb, b0):
         return None
-    if not (_made_by(sq, "AddBackward0", qa, qb) and _made_by(y, "LgammaBackward0", ("AddBackward0", qa, qb)) and
-            _made_by(x, "AddBackward0", ("LgammaBackward0", qa), ("LgammaBackward0", qb))):
+    if all(t.grad_fn is None and not t.requires_grad for t in (x, y, qa, qb, sq)):
+        # no graph at all (evaluation under torch.no_grad()): the operands are compared by value instead -- three
+        # small elementwise kernels and one wait for the device, nothing next to scoring every entity
+        if not (torch.equal(sq, qa + qb) and torch.equal(y, sq.lgamma()) and torch.equal(x, qa.lgamma() + qb.lgamma())):
+            return None
+    elif not (_made_by(sq, "AddBackward0", qa, qb) and _made_by(y, "LgammaBackward0", ("AddBackward0", qa, qb)) and
+              _made_by(x, "AddBackward0", ("LgammaBackward0", qa), ("LgammaBackward0", qb))):
         return None
     handle = expr.handle
     return handle._like((handle.shape[0], handle.shape[2], handle.shape[3])), qa, qb

@@ -354,7 +354,8 @@ def test_expressions_that_only_resemble_the_beta_routine_are_evaluated_by_torch(
         return t1 - t2 + (p1 - q1) * torch.digamma(p1) + (p0 - q0) * torch.digamma(p0) + (sq - sp) * torch.digamma(sp)
 
     cases = {"other tensor": lambda a, c: kl_with(a, c, qa, qb, y=(qa * qb).lgamma()),
-             "no graph": lambda a, c: kl_with(a, c, qa.detach(), qb.detach()),
+             "no graph, other tensor": lambda a, c: kl_with(a, c, qa.detach(), qb.detach(), y=(qa * qb).detach().lgamma()),
+             "graph on one side only": lambda a, c: kl_with(a, c, qa, qb.detach()),
              "halves swapped": lambda a, c: kl_with(c, a, qa, qb),
              "queries swapped in one term": lambda a, c: kl_with(a, c, qa, qb) + ((a - qb) * torch.digamma(a) - (a - qa) * torch.digamma(a))}
     for name, f in cases.items():
@@ -371,6 +372,11 @@ def test_expressions_that_only_resemble_the_beta_routine_are_evaluated_by_torch(
     a, c = torch.chunk(handle, 2, dim=-1)
     kld = torch_kl._kl_beta_beta(ext_ops.BetaDist(a, c), ext_ops.BetaDist(qa, qb))
     assert not isinstance(torch.norm(kld, p=1, dim=-1), torch.Tensor)
+    # ... and under no_grad, where the query-side operands are compared by value
+    with torch.no_grad():
+        a, c = torch.chunk(reg(LazyRows(opt, ids, None).view(b, k, -1)).unsqueeze(1), 2, dim=-1)
+        kld = torch_kl._kl_beta_beta(ext_ops.BetaDist(a, c), ext_ops.BetaDist(qa.detach(), qb.detach()))
+        assert not isinstance(torch.norm(kld, p=1, dim=-1), torch.Tensor)
 
 
 @pytest.mark.parametrize("norm", [False, True])
